@@ -1,0 +1,142 @@
+/*
+ * C ABI of libmedvision_hip.so -- MI355X (gfx950) kernels for MedVision's trilinear-sampling
+ * operator family.  One entry point per function that the reference registers in its pybind11
+ * module `medvision._C` for this path (/root/reference/medvision/csrc/vision.cpp:26-77).
+ *
+ * Conventions (all entry points):
+ *   - every pointer is a DEVICE pointer to a dense, contiguous NC(D)HW tensor of element type
+ *     `dtype` (mv_dtype); shapes are passed as plain ints;
+ *   - `rois` are float32 [num_rois, cols] -- except when dtype == MV_F64, then float64 -- with the
+ *     reference's column layouts (5 | 7 | 6 | 10 columns);
+ *   - coordinates are computed in fp64 and interpolation weights / accumulation in fp32 (fp64 for
+ *     MV_F64) regardless of the storage type;
+ *   - `stream` is a hipStream_t (NULL = the null stream); launches are asynchronous, nothing
+ *     synchronises;
+ *   - return value 0 = success, otherwise an mv_status; mv_last_error() gives the message of the
+ *     last failure on the calling thread.  No entry point allocates device memory: scratch is
+ *     passed in as `workspace` (size queried with the matching *_workspace_bytes function).
+ */
+#ifndef MEDVISION_HIP_H
+#define MEDVISION_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum { MV_F32 = 0, MV_F16 = 1, MV_BF16 = 2, MV_F64 = 3 } mv_dtype;
+typedef enum { MV_OK = 0, MV_INVALID_ARGUMENT = 1, MV_HIP_ERROR = 2 } mv_status;
+
+const char *mv_last_error(void);
+int mv_version(void);
+
+/* ---- RoIAlign, plain boxes --------------------------------------------------------------
+ * replaces roi_align_2d_forward / roi_align_2d_backward   csrc/roi_align_2d.h (vision.cpp:31-34)
+ *          roi_align_3d_forward / roi_align_3d_backward   csrc/roi_align_3d.h:71,98 (vision.cpp:36-39)
+ * input  [batch, channels, (depth,) height, width], rois [num_rois, 5 | 7], output
+ * [num_rois, channels, (out_d,) out_h, out_w].  order: 0 nearest, 1 linear.
+ * backward ACCUMULATES into grad_input (callers pass a zero-filled buffer, like the reference's
+ * Python wrapper ops/roi_align_nd.py:139 does).  For MV_F16 / MV_BF16 the backward needs an fp32
+ * workspace of mv_roi_align_backward_workspace_bytes(); other dtypes accept NULL.            */
+int mv_roi_align_2d_forward(const void *input, const void *rois, void *output, int dtype,
+                            int batch, int channels, int height, int width, int num_rois,
+                            int out_h, int out_w, float spatial_scale, int sampling_ratio,
+                            int order, void *stream);
+int mv_roi_align_2d_backward(const void *grad_output, const void *rois, void *grad_input,
+                             int dtype, int batch, int channels, int height, int width,
+                             int num_rois, int out_h, int out_w, float spatial_scale,
+                             int sampling_ratio, int order, void *workspace, void *stream);
+int mv_roi_align_3d_forward(const void *input, const void *rois, void *output, int dtype,
+                            int batch, int channels, int depth, int height, int width,
+                            int num_rois, int out_d, int out_h, int out_w, float spatial_scale,
+                            int sampling_ratio, int order, void *stream);
+int mv_roi_align_3d_backward(const void *grad_output, const void *rois, void *grad_input,
+                             int dtype, int batch, int channels, int depth, int height, int width,
+                             int num_rois, int out_d, int out_h, int out_w, float spatial_scale,
+                             int sampling_ratio, int order, void *workspace, void *stream);
+
+/* ---- RoIAlignRotated ---------------------------------------------------------------------
+ * replaces roi_align_rotated_2d_forward/backward  csrc/roi_align_rotated_2d.h (vision.cpp:41-44)
+ *          roi_align_rotated_3d_forward/backward  csrc/roi_align_rotated_3d.h:71,98 (vision.cpp:45-48)
+ * rois [num_rois, 6] = (b, cx, cy, w, h, theta) or [num_rois, 10] = (b, cx, cy, cz, w, h, d,
+ * angle_x, angle_y, angle_z), radians.                                                        */
+int mv_roi_align_rotated_2d_forward(const void *input, const void *rois, void *output, int dtype,
+                                    int batch, int channels, int height, int width, int num_rois,
+                                    int out_h, int out_w, float spatial_scale, int sampling_ratio,
+                                    int aligned, int order, void *stream);
+int mv_roi_align_rotated_2d_backward(const void *grad_output, const void *rois, void *grad_input,
+                                     int dtype, int batch, int channels, int height, int width,
+                                     int num_rois, int out_h, int out_w, float spatial_scale,
+                                     int sampling_ratio, int aligned, int order, void *workspace,
+                                     void *stream);
+int mv_roi_align_rotated_3d_forward(const void *input, const void *rois, void *output, int dtype,
+                                    int batch, int channels, int depth, int height, int width,
+                                    int num_rois, int out_d, int out_h, int out_w,
+                                    float spatial_scale, int sampling_ratio, int aligned,
+                                    int order, void *stream);
+int mv_roi_align_rotated_3d_backward(const void *grad_output, const void *rois, void *grad_input,
+                                     int dtype, int batch, int channels, int depth, int height,
+                                     int width, int num_rois, int out_d, int out_h, int out_w,
+                                     float spatial_scale, int sampling_ratio, int aligned,
+                                     int order, void *workspace, void *stream);
+size_t mv_roi_align_backward_workspace_bytes(int dtype, int batch, int channels, int depth,
+                                             int height, int width);
+
+/* ---- affine resampling engine (forward only) ----------------------------------------------
+ * replaces affine_2d  csrc/affine_2d.h (vision.cpp:74), affine_3d  csrc/affine_3d.h:40 (vision.cpp:75)
+ * Same arguments and results as the rotated forward for order 0 / 1 (the reference kernel text
+ * is identical, csrc/cuda_aug/affine_3d_cuda_kernel.cuh:14-120).  order 3 is rejected with
+ * MV_INVALID_ARGUMENT.                                                                        */
+int mv_affine_2d(const void *input, const void *rois, void *output, int dtype, int batch,
+                 int channels, int height, int width, int num_rois, int out_h, int out_w,
+                 float spatial_scale, int sampling_ratio, int aligned, int order, void *stream);
+int mv_affine_3d(const void *input, const void *rois, void *output, int dtype, int batch,
+                 int channels, int depth, int height, int width, int num_rois, int out_d,
+                 int out_h, int out_w, float spatial_scale, int sampling_ratio, int aligned,
+                 int order, void *stream);
+
+/* ---- deformable convolution 3-D -----------------------------------------------------------
+ * replaces deform_conv_3d_forward / _backward                 csrc/deform_conv_3d.h:48,87
+ *          modulated_deform_conv_3d_forward / _backward       csrc/modulated_deform_conv_3d.h:61,89
+ * One shape record serves v1 (mask == NULL) and v2.  Layouts: input [B,Cin,D,H,W], offset
+ * [B, dg*3*K, Do,Ho,Wo] (channel 3k+0 = depth, +1 = height, +2 = width displacement of tap k),
+ * mask [B, dg*K, Do,Ho,Wo], weight [Cout, Cin/groups, kd,kh,kw], bias [Cout] or NULL, output
+ * [B,Cout,Do,Ho,Wo] with Do = (D + 2*pad_d - (dil_d*(kd-1)+1)) / stride_d + 1 etc.
+ * The backward accumulates into grad_weight / grad_bias / grad_input and overwrites
+ * grad_offset / grad_mask; grad_mask and grad_bias may be NULL.                               */
+typedef struct {
+  int batch, in_channels, depth, height, width;
+  int out_channels, kernel_d, kernel_h, kernel_w;
+  int stride_d, stride_h, stride_w;
+  int pad_d, pad_h, pad_w;
+  int dil_d, dil_h, dil_w;
+  int groups, deformable_groups;
+} mv_dcn3d_shape;
+
+int mv_dcn3d_output_dims(const mv_dcn3d_shape *shape, int *out_d, int *out_h, int *out_w);
+size_t mv_dcn3d_forward_workspace_bytes(const mv_dcn3d_shape *shape, int dtype);
+size_t mv_dcn3d_backward_workspace_bytes(const mv_dcn3d_shape *shape, int dtype);
+int mv_dcn3d_forward(const void *input, const void *offset, const void *mask, const void *weight,
+                     const void *bias, void *output, const mv_dcn3d_shape *shape, int dtype,
+                     void *workspace, void *stream);
+int mv_dcn3d_backward(const void *input, const void *offset, const void *mask, const void *weight,
+                      const void *grad_output, void *grad_input, void *grad_offset,
+                      void *grad_mask, void *grad_weight, void *grad_bias,
+                      const mv_dcn3d_shape *shape, int dtype, void *workspace, void *stream);
+
+/* ---- displacement-field warp (elastic engine) -----------------------------------------------
+ * replaces deform_2d / deform_3d  csrc/deform_2d.h, csrc/deform_3d.h:27 (vision.cpp:71-72) for the
+ * way the reference calls them (ops/cuda_fun_tools.py:94-167: 1x1x1 kernel, identity weight,
+ * zero bias): out[b,c,q] = S(img[b,c], q + off[b,:,q]) on the open interval (-1, size), else 0.
+ * img/out [B,C,(D,)H,W], offset [B, 2|3, (D,)H,W] (3-D: 0 = depth, 1 = height, 2 = width).       */
+int mv_deform_warp_2d(const void *img, const void *offset, void *output, int dtype, int batch,
+                      int channels, int height, int width, int order, void *stream);
+int mv_deform_warp_3d(const void *img, const void *offset, void *output, int dtype, int batch,
+                      int channels, int depth, int height, int width, int order, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MEDVISION_HIP_H */

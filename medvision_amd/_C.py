@@ -1,0 +1,365 @@
+"""Drop-in for the reference's pybind11 module ``medvision._C`` on the sampling path.
+
+Function names, argument order and error behaviour follow ``medvision/csrc/vision.cpp:26-77`` and
+the dispatch headers it includes; the work is done by ``libmedvision_hip.so`` through its C ABI.
+Deliberate differences from the reference binding:
+
+* rois may have any float dtype; they are cast once to fp32 (fp64 for double features) instead of
+  having to match the feature dtype (reference reads ``rois.data<scalar_t>()``,
+  csrc/cuda/roi_align_3d_cuda.cu:17);
+* kernels run on the current torch stream of the feature tensor's device (the reference RoI
+  launchers use the legacy default stream, csrc/cuda/roi_align_3d_cuda.cu:20-21);
+* output / gradient buffers must be contiguous (the reference silently writes into a temporary
+  when they are not, csrc/cuda/roi_align_3d_cuda.cu:18);
+* bfloat16 is accepted in addition to double / float / half.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+
+
+def _require_cuda(t, what):
+    if not t.is_cuda:
+        raise RuntimeError(f"{what} is not implemented on CPU")
+
+
+def _prep_rois(rois, features, cols):
+    if rois.dim() != 2 or rois.size(1) != cols:
+        raise RuntimeError(f"wrong roi size! size_rois should be {cols}")
+    want = torch.float64 if features.dtype == torch.float64 else torch.float32
+    return rois.to(device=features.device, dtype=want).contiguous()
+
+
+def _require_contiguous(t, name):
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} tensor has to be contiguous")
+
+
+def _roi_forward(fn_name, what, ndim, cols, input, rois, output, out_sizes, spatial_scale,
+                 sampling_ratio, extra):
+    _require_cuda(input, what)
+    lib = _lib.load()
+    _require_contiguous(output, "output")
+    if output.dtype != input.dtype:
+        raise RuntimeError("output dtype must match input dtype")
+    feats = input.contiguous()
+    r = _prep_rois(rois, feats, cols)
+    dims = list(feats.shape)
+    if len(dims) != ndim + 2:
+        raise RuntimeError(f"expected a {ndim + 2}-d feature tensor, got {len(dims)}-d")
+    want_shape = (r.size(0), dims[1], *out_sizes)
+    if tuple(output.shape) != want_shape:
+        raise RuntimeError(f"output has shape {tuple(output.shape)}, expected {want_shape}")
+    with torch.cuda.device(feats.device):
+        _lib.check(getattr(lib, fn_name)(
+            _lib.ptr(feats), _lib.ptr(r), _lib.ptr(output), _lib.dtype_code(feats), *dims,
+            r.size(0), *out_sizes, float(spatial_scale), int(sampling_ratio), *extra,
+            _lib.stream_of(feats)))
+
+
+def _roi_backward(fn_name, what, ndim, cols, top_grad, rois, bottom_grad, out_sizes,
+                  spatial_scale, sampling_ratio, extra):
+    _require_cuda(top_grad, what)
+    lib = _lib.load()
+    _require_contiguous(bottom_grad, "bottom_grad")
+    if bottom_grad.dtype != top_grad.dtype:
+        raise RuntimeError("bottom_grad dtype must match top_grad dtype")
+    g = top_grad.contiguous()
+    r = _prep_rois(rois, g, cols)
+    dims = list(bottom_grad.shape)
+    if len(dims) != ndim + 2:
+        raise RuntimeError(f"expected a {ndim + 2}-d gradient buffer, got {len(dims)}-d")
+    want_shape = (r.size(0), dims[1], *out_sizes)
+    if tuple(g.shape) != want_shape:
+        raise RuntimeError(f"top_grad has shape {tuple(g.shape)}, expected {want_shape}")
+    code = _lib.dtype_code(g)
+    d5 = dims if ndim == 3 else [dims[0], dims[1], 1, dims[2], dims[3]]
+    ws_bytes = lib.mv_roi_align_backward_workspace_bytes(code, *d5)
+    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=g.device) if ws_bytes else None
+    with torch.cuda.device(g.device):
+        _lib.check(getattr(lib, fn_name)(
+            _lib.ptr(g), _lib.ptr(r), _lib.ptr(bottom_grad), code, *dims, r.size(0), *out_sizes,
+            float(spatial_scale), int(sampling_ratio), *extra, _lib.ptr(ws), _lib.stream_of(g)))
+
+
+# ---- csrc/roi_align_2d.h, csrc/roi_align_3d.h:71-117 ------------------------------------
+def roi_align_2d_forward(input, rois, output, out_h, out_w, spatial_scale, sampling_ratio, order):
+    _roi_forward("mv_roi_align_2d_forward", "RoIAlign", 2, 5, input, rois, output,
+                 (out_h, out_w), spatial_scale, sampling_ratio, (int(order),))
+
+
+def roi_align_2d_backward(top_grad, rois, bottom_grad, out_h, out_w, spatial_scale,
+                          sampling_ratio, order):
+    _roi_backward("mv_roi_align_2d_backward", "RoIAlign", 2, 5, top_grad, rois, bottom_grad,
+                  (out_h, out_w), spatial_scale, sampling_ratio, (int(order),))
+
+
+def roi_align_3d_forward(input, rois, output, out_d, out_h, out_w, spatial_scale, sampling_ratio,
+                         order):
+    _roi_forward("mv_roi_align_3d_forward", "RoIAlign", 3, 7, input, rois, output,
+                 (out_d, out_h, out_w), spatial_scale, sampling_ratio, (int(order),))
+
+
+def roi_align_3d_backward(top_grad, rois, bottom_grad, out_d, out_h, out_w, spatial_scale,
+                          sampling_ratio, order):
+    _roi_backward("mv_roi_align_3d_backward", "RoIAlign", 3, 7, top_grad, rois, bottom_grad,
+                  (out_d, out_h, out_w), spatial_scale, sampling_ratio, (int(order),))
+
+
+# ---- csrc/roi_align_rotated_2d.h, csrc/roi_align_rotated_3d.h:71-117 ----------------------
+def roi_align_rotated_2d_forward(input, rois, output, out_h, out_w, spatial_scale,
+                                 sampling_ratio, aligned, order):
+    _roi_forward("mv_roi_align_rotated_2d_forward", "RoIAlignRotated", 2, 6, input, rois, output,
+                 (out_h, out_w), spatial_scale, sampling_ratio, (int(bool(aligned)), int(order)))
+
+
+def roi_align_rotated_2d_backward(top_grad, rois, bottom_grad, out_h, out_w, spatial_scale,
+                                  sampling_ratio, aligned, order):
+    _roi_backward("mv_roi_align_rotated_2d_backward", "RoIAlignRotated", 2, 6, top_grad, rois,
+                  bottom_grad, (out_h, out_w), spatial_scale, sampling_ratio,
+                  (int(bool(aligned)), int(order)))
+
+
+def roi_align_rotated_3d_forward(input, rois, output, out_d, out_h, out_w, spatial_scale,
+                                 sampling_ratio, aligned, order):
+    _roi_forward("mv_roi_align_rotated_3d_forward", "RoIAlignRotated", 3, 10, input, rois, output,
+                 (out_d, out_h, out_w), spatial_scale, sampling_ratio,
+                 (int(bool(aligned)), int(order)))
+
+
+def roi_align_rotated_3d_backward(top_grad, rois, bottom_grad, out_d, out_h, out_w, spatial_scale,
+                                  sampling_ratio, aligned, order):
+    _roi_backward("mv_roi_align_rotated_3d_backward", "RoIAlignRotated", 3, 10, top_grad, rois,
+                  bottom_grad, (out_d, out_h, out_w), spatial_scale, sampling_ratio,
+                  (int(bool(aligned)), int(order)))
+
+
+# ---- csrc/affine_2d.h, csrc/affine_3d.h:40-65 ---------------------------------------------
+def affine_2d(input, rois, output, out_h, out_w, spatial_scale, sampling_ratio, aligned, order):
+    _roi_forward("mv_affine_2d", "affine", 2, 6, input, rois, output, (out_h, out_w),
+                 spatial_scale, sampling_ratio, (int(bool(aligned)), int(order)))
+
+
+def affine_3d(input, rois, output, out_d, out_h, out_w, spatial_scale, sampling_ratio, aligned,
+              order):
+    _roi_forward("mv_affine_3d", "affine", 3, 10, input, rois, output, (out_d, out_h, out_w),
+                 spatial_scale, sampling_ratio, (int(bool(aligned)), int(order)))
+
+
+# ---- deformable convolution 3-D -----------------------------------------------------------
+def _dcn_shape(input, weight, kernel, stride, pad, dil, group, deformable_group):
+    _require_contiguous(input, "input")
+    _require_contiguous(weight, "weight")
+    B, C, D, H, W = input.shape
+    Cout, ck, kd_, kh_, kw_ = weight.shape
+    kd, kh, kw = kernel
+    if (kd_, kh_, kw_) != (kd, kh, kw):
+        raise RuntimeError("Input shape and kernel shape wont match: (%d x %d x %d vs %d x %d x %d)."
+                           % (kh, kw, kd, kh_, kw_, kd_))
+    if C != ck * group:
+        raise RuntimeError("Input shape and kernel channels wont match: (%d vs %d)." % (C, ck * group))
+    if C % group or Cout % group:
+        raise RuntimeError("channels(%d) and channels_out(%d) must divide group(%d)" % (C, Cout, group))
+    if C % deformable_group:
+        raise RuntimeError("channels(%d) must divide deformable_group(%d)" % (C, deformable_group))
+    return _lib.DcnShape(B, C, D, H, W, Cout, kd, kh, kw, *stride, *pad, *dil, group,
+                         deformable_group)
+
+
+def _dcn_out_dims(lib, shape):
+    od, oh, ow = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    _lib.check(lib.mv_dcn3d_output_dims(ctypes.byref(shape), ctypes.byref(od), ctypes.byref(oh),
+                                        ctypes.byref(ow)))
+    return od.value, oh.value, ow.value
+
+
+def _dcn_check_aux(shape, dims, offset, mask, K):
+    B, dg = shape.batch, shape.deformable_groups
+    if tuple(offset.shape) != (B, dg * 3 * K, *dims):
+        raise RuntimeError(f"offset has shape {tuple(offset.shape)}, expected {(B, dg * 3 * K, *dims)}")
+    if mask is not None and tuple(mask.shape) != (B, dg * K, *dims):
+        raise RuntimeError(f"mask has shape {tuple(mask.shape)}, expected {(B, dg * K, *dims)}")
+
+
+def _dcn_forward(input, offset, mask, weight, bias, output, shape):
+    lib = _lib.load()
+    dims = _dcn_out_dims(lib, shape)
+    K = shape.kernel_d * shape.kernel_h * shape.kernel_w
+    offset = offset.to(input.dtype).contiguous()
+    mask = mask.to(input.dtype).contiguous() if mask is not None else None
+    _dcn_check_aux(shape, dims, offset, mask, K)
+    if weight.dtype != input.dtype or (bias is not None and bias.dtype != input.dtype):
+        raise RuntimeError("input, weight and bias must share one dtype")
+    code = _lib.dtype_code(input)
+    nbytes = lib.mv_dcn3d_forward_workspace_bytes(ctypes.byref(shape), code)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=input.device) if nbytes else None
+    with torch.cuda.device(input.device):
+        _lib.check(lib.mv_dcn3d_forward(
+            _lib.ptr(input), _lib.ptr(offset), _lib.ptr(mask), _lib.ptr(weight), _lib.ptr(bias),
+            _lib.ptr(output), ctypes.byref(shape), code, _lib.ptr(ws), _lib.stream_of(input)))
+
+
+def _dcn_backward(input, offset, mask, weight, grad_output, gi, goff, gmask, gw, gb, shape):
+    lib = _lib.load()
+    dims = _dcn_out_dims(lib, shape)
+    K = shape.kernel_d * shape.kernel_h * shape.kernel_w
+    offset = offset.to(input.dtype).contiguous()
+    mask = mask.to(input.dtype).contiguous() if mask is not None else None
+    _dcn_check_aux(shape, dims, offset, mask, K)
+    grad_output = grad_output.to(input.dtype).contiguous()
+    if tuple(grad_output.shape) != (shape.batch, shape.out_channels, *dims):
+        raise RuntimeError("Input shape and grad_out shape wont match: (%s vs %s)."
+                           % ((shape.batch, shape.out_channels, *dims), tuple(grad_output.shape)))
+    for t, n in ((gi, "grad_input"), (goff, "grad_offset"), (gw, "grad_weight")):
+        _require_contiguous(t, n)
+    code = _lib.dtype_code(input)
+    nbytes = lib.mv_dcn3d_backward_workspace_bytes(ctypes.byref(shape), code)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=input.device) if nbytes else None
+    with torch.cuda.device(input.device):
+        _lib.check(lib.mv_dcn3d_backward(
+            _lib.ptr(input), _lib.ptr(offset), _lib.ptr(mask), _lib.ptr(weight),
+            _lib.ptr(grad_output), _lib.ptr(gi), _lib.ptr(goff), _lib.ptr(gmask), _lib.ptr(gw),
+            _lib.ptr(gb), ctypes.byref(shape), code, _lib.ptr(ws), _lib.stream_of(input)))
+
+
+# csrc/deform_conv_3d.h:48-129 (host: csrc/cuda/deform_conv_3d_cuda.cu:110-376)
+def deform_conv_3d_forward(input, weight, bias, offset, kernel_d, kernel_h, kernel_w, stride_d,
+                           stride_h, stride_w, pad_d, pad_h, pad_w, dilation_d, dilation_h,
+                           dilation_w, group, deformable_group, im2col_step):
+    if not input.is_cuda:
+        raise RuntimeError("Not implemented on the CPU")
+    batch = input.size(0)
+    step = min(batch, im2col_step)
+    if batch % step != 0:
+        raise RuntimeError("batch(%d) must divide im2col_step(%d)" % (batch, step))
+    shape = _dcn_shape(input, weight, (kernel_d, kernel_h, kernel_w), (stride_d, stride_h, stride_w),
+                       (pad_d, pad_h, pad_w), (dilation_d, dilation_h, dilation_w), group,
+                       deformable_group)
+    dims = _dcn_out_dims(_lib.load(), shape)
+    output = torch.empty((batch, weight.size(0), *dims), dtype=input.dtype, device=input.device)
+    _dcn_forward(input, offset, None, weight, bias.contiguous(), output, shape)
+    return output
+
+
+def deform_conv_3d_backward(input, weight, bias, offset, grad_output, kernel_d, kernel_h, kernel_w,
+                            stride_d, stride_h, stride_w, pad_d, pad_h, pad_w, dilation_d,
+                            dilation_h, dilation_w, group, deformable_group, im2col_step):
+    if not input.is_cuda:
+        raise RuntimeError("Not implemented on the CPU")
+    batch = input.size(0)
+    step = min(batch, im2col_step)
+    if batch % step != 0:
+        raise RuntimeError("batch(%d) must divide im2col_step(%d)" % (batch, step))
+    shape = _dcn_shape(input, weight, (kernel_d, kernel_h, kernel_w), (stride_d, stride_h, stride_w),
+                       (pad_d, pad_h, pad_w), (dilation_d, dilation_h, dilation_w), group,
+                       deformable_group)
+    gi, goff = torch.zeros_like(input), torch.zeros_like(offset, dtype=input.dtype)
+    gw, gb = torch.zeros_like(weight), torch.zeros_like(bias)
+    _dcn_backward(input, offset, None, weight, grad_output, gi, goff, None, gw, gb, shape)
+    return [gi, goff, gw, gb]
+
+
+# csrc/modulated_deform_conv_3d.h:61-117 (host: csrc/cuda/modulated_deform_conv_3d_cuda.cu:137-396)
+def modulated_deform_conv_3d_forward(input, weight, bias, ones, offset, mask, output, columns,
+                                     kernel_d, kernel_h, kernel_w, stride_d, stride_h, stride_w,
+                                     pad_d, pad_h, pad_w, dilation_d, dilation_h, dilation_w,
+                                     group, deformable_group, with_bias):
+    """``ones`` and ``columns`` are scratch handles of the reference and are ignored."""
+    if not input.is_cuda:
+        raise RuntimeError("Not implemented on the CPU")
+    shape = _dcn_shape(input, weight, (kernel_d, kernel_h, kernel_w), (stride_d, stride_h, stride_w),
+                       (pad_d, pad_h, pad_w), (dilation_d, dilation_h, dilation_w), group,
+                       deformable_group)
+    dims = _dcn_out_dims(_lib.load(), shape)
+    want = (input.size(0), weight.size(0), *dims)
+    if output.numel() != torch.Size(want).numel() or not output.is_contiguous():
+        raise RuntimeError(f"output must be a contiguous tensor of shape {want}")
+    if output.dtype != input.dtype:
+        raise RuntimeError("output dtype must match input dtype")
+    _dcn_forward(input, offset, mask, weight, bias.contiguous() if with_bias else None, output, shape)
+
+
+def modulated_deform_conv_3d_backward(input, weight, bias, ones, offset, mask, columns, grad_input,
+                                      grad_weight, grad_bias, grad_offset, grad_mask, grad_output,
+                                      kernel_d, kernel_h, kernel_w, stride_d, stride_h, stride_w,
+                                      pad_d, pad_h, pad_w, dilation_d, dilation_h, dilation_w,
+                                      group, deformable_group, with_bias):
+    """Writes the analytic gradients of the forward.  The reference's 3-D v2 backward launches its
+    col2im over a truncated index range and writes the mask gradient with a 2-D channel index
+    (csrc/cuda/modulated_deform_conv_3d_cuda.cu:64, ..._kernel.cuh:410-411); those two defects
+    are not reproduced."""
+    if not input.is_cuda:
+        raise RuntimeError("Not implemented on the CPU")
+    shape = _dcn_shape(input, weight, (kernel_d, kernel_h, kernel_w), (stride_d, stride_h, stride_w),
+                       (pad_d, pad_h, pad_w), (dilation_d, dilation_h, dilation_w), group,
+                       deformable_group)
+    for t in (grad_input, grad_weight, grad_offset, grad_mask):
+        if t.dtype != input.dtype:
+            raise RuntimeError("gradient buffers must have the dtype of input")
+    _require_contiguous(grad_mask, "grad_mask")
+    _dcn_backward(input, offset, mask, weight, grad_output, grad_input, grad_offset, grad_mask,
+                  grad_weight, grad_bias if with_bias else None, shape)
+
+
+# csrc/deform_2d.h, csrc/deform_3d.h:27-65 as used by ops/cuda_fun_tools.py:94-167
+def _deform(fn_name, ndim, input, weight, bias, offset, kernel, stride, pad, dil, group,
+            deformable_group, order):
+    if not input.is_cuda:
+        raise RuntimeError("Not implemented on the CPU")
+    C = input.size(1)
+    eye = torch.eye(C, dtype=weight.dtype, device=weight.device).reshape(C, C, *([1] * ndim))
+    if (any(k != 1 for k in kernel) or any(s != 1 for s in stride) or any(p != 0 for p in pad)
+            or group != 1 or deformable_group != 1 or tuple(weight.shape) != tuple(eye.shape)
+            or not torch.equal(weight, eye) or bool((bias != 0).any())):
+        raise RuntimeError("deform_%dd supports the displacement-field warp only: 1x1 kernel, "
+                           "stride 1, no padding, identity weight, zero bias" % ndim)
+    if order not in (0, 1):
+        raise RuntimeError(f"order {order} is not implemented")
+    _require_contiguous(input, "input")
+    offset = offset.to(device=input.device, dtype=input.dtype).contiguous()
+    if tuple(offset.shape) != (input.size(0), ndim, *input.shape[2:]):
+        raise RuntimeError("offset must have shape [B, %d, *spatial]" % ndim)
+    out = torch.empty_like(input)
+    with torch.cuda.device(input.device):
+        _lib.check(getattr(_lib.load(), fn_name)(
+            _lib.ptr(input), _lib.ptr(offset), _lib.ptr(out), _lib.dtype_code(input),
+            *input.shape, int(order), _lib.stream_of(input)))
+    return out
+
+
+def deform_2d(input, weight, bias, offset, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w,
+              dilation_h, dilation_w, group, deformable_group, im2col_step, order):
+    return _deform("mv_deform_warp_2d", 2, input, weight, bias, offset, (kernel_h, kernel_w),
+                   (stride_h, stride_w), (pad_h, pad_w), (dilation_h, dilation_w), group,
+                   deformable_group, order)
+
+
+def deform_3d(input, weight, bias, offset, kernel_d, kernel_h, kernel_w, stride_d, stride_h,
+              stride_w, pad_d, pad_h, pad_w, dilation_d, dilation_h, dilation_w, group,
+              deformable_group, im2col_step, order):
+    return _deform("mv_deform_warp_3d", 3, input, weight, bias, offset,
+                   (kernel_d, kernel_h, kernel_w), (stride_d, stride_h, stride_w),
+                   (pad_d, pad_h, pad_w), (dilation_d, dilation_h, dilation_w), group,
+                   deformable_group, order)
+
+
+def deform_warp(img, offset, order=1):
+    """Direct entry to the warp kernel (no identity weight to build or verify)."""
+    ndim = img.dim() - 2
+    if not img.is_cuda:
+        raise RuntimeError("Not implemented on the CPU")
+    img = img.contiguous()
+    offset = offset.to(device=img.device, dtype=img.dtype).contiguous()
+    if tuple(offset.shape) != (img.size(0), ndim, *img.shape[2:]):
+        raise RuntimeError("offset must have shape [B, %d, *spatial]" % ndim)
+    if order not in (0, 1):
+        raise RuntimeError(f"order {order} is not implemented")
+    out = torch.empty_like(img)
+    fn = "mv_deform_warp_2d" if ndim == 2 else "mv_deform_warp_3d"
+    with torch.cuda.device(img.device):
+        _lib.check(getattr(_lib.load(), fn)(
+            _lib.ptr(img), _lib.ptr(offset), _lib.ptr(out), _lib.dtype_code(img), *img.shape,
+            int(order), _lib.stream_of(img)))
+    return out

@@ -1,0 +1,328 @@
+// 3-D deformable convolution (DCNv1 when mask == nullptr, DCNv2 otherwise): general-shape
+// kernels for every dtype / group configuration, plus the entry points that choose between them
+// and the matrix-core forward for 16-bit tensors (dcn3d_mfma.hip).
+//
+// Nothing here materialises the reference's column matrix: the trilinear gather feeds the weight
+// contraction directly, and the 8 corner offsets / weights of a (tap, position) pair are computed
+// once and reused for all channels of the deformable group.
+#include "dcn_common.hpp"
+
+namespace mv {
+
+constexpr int kDcnThreads = 128;
+constexpr int kOutTile = 32;  // output channels accumulated per thread in the general forward
+
+// ---- forward: thread = (output position, tile of <= 32 output channels of one group) --------
+template <typename T>
+__global__ __launch_bounds__(kDcnThreads) void dcn_forward_kernel(
+    const T *__restrict__ x, const T *__restrict__ off, const T *__restrict__ mask,
+    const T *__restrict__ wt, const T *__restrict__ bias, T *__restrict__ y, const DcnDims s) {
+  using A = typename Acc<T>::type;
+  const long q = blockIdx.x * static_cast<long>(kDcnThreads) + threadIdx.x;
+  const int tiles_per_group = (s.opg + kOutTile - 1) / kOutTile;
+  const int grp = blockIdx.y / tiles_per_group, tile = blockIdx.y % tiles_per_group;
+  const int b = blockIdx.z;
+  if (q >= s.Q) return;
+  const int ow = q % s.Wo, oh = (q / s.Wo) % s.Ho, od = q / (static_cast<long>(s.Wo) * s.Ho);
+  const int o_begin = grp * s.opg + tile * kOutTile;
+  const int o_count = min(kOutTile, grp * s.opg + s.opg - o_begin);
+  A acc[kOutTile];
+#pragma unroll
+  for (int i = 0; i < kOutTile; i++) acc[i] = A(0);
+  const int c_begin = grp * s.cpg, c_end = c_begin + s.cpg;
+  for (int dgi = c_begin / s.cpd; dgi <= (c_end - 1) / s.cpd; dgi++) {
+    const int c_lo = max(c_begin, dgi * s.cpd), c_hi = min(c_end, (dgi + 1) * s.cpd);
+    const T *off_bg = off + (static_cast<long>(b) * s.dg + dgi) * 3 * s.K * s.Q;
+    const T *mask_bg = mask ? mask + (static_cast<long>(b) * s.dg + dgi) * s.K * s.Q : nullptr;
+    for (int k = 0; k < s.K; k++) {
+      double pd, ph, pw;
+      dcn_position(s, off_bg, k, od, oh, ow, q, pd, ph, pw);
+      ZTaps<A> t;
+      zero_pad_taps(s, pd, ph, pw, t);
+      if (!t.ok) continue;
+      const A m = mask_bg ? load(mask_bg + static_cast<long>(k) * s.Q + q) : A(1);
+      for (int c = c_lo; c < c_hi; c++) {
+        const A col = zsample<T, A>(x + (static_cast<long>(b) * s.Cin + c) * s.P, t) * m;
+        const T *wrow = wt + (static_cast<long>(o_begin) * s.cpg + (c - c_begin)) * s.K + k;
+#pragma unroll
+        for (int i = 0; i < kOutTile; i++)
+          if (i < o_count) acc[i] += load(wrow + static_cast<long>(i) * s.cpg * s.K) * col;
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kOutTile; i++)
+    if (i < o_count) {
+      const int o = o_begin + i;
+      y[(static_cast<long>(b) * s.Cout + o) * s.Q + q] =
+          store_cast<T>(acc[i] + (bias ? load(bias + o) : A(0)));
+    }
+}
+
+// ---- backward 1: thread = (b, dgi, k, q): grad wrt input (atomic scatter), offset and mask ---
+//   gcol[c] = sum_o Wt[o,c_l,k] * gy[b,o,q];  gx += gcol*m*w_corner;  goff_a = sum_c gcol*m*dZ/dp_a;
+//   gm = sum_c gcol*Z.   G = accumulation element type of gx (T, or float for 16-bit T).
+template <typename T, typename G>
+__global__ __launch_bounds__(kDcnThreads) void dcn_backward_data_kernel(
+    const T *__restrict__ x, const T *__restrict__ off, const T *__restrict__ mask,
+    const T *__restrict__ wt, const T *__restrict__ gy, G *__restrict__ gx, T *__restrict__ goff,
+    T *__restrict__ gmask, const DcnDims s) {
+  using A = typename Acc<T>::type;
+  const long q = blockIdx.x * static_cast<long>(kDcnThreads) + threadIdx.x;
+  const int k = blockIdx.y % s.K, dgi = blockIdx.y / s.K;
+  const int b = blockIdx.z;
+  if (q >= s.Q) return;
+  const int ow = q % s.Wo, oh = (q / s.Wo) % s.Ho, od = q / (static_cast<long>(s.Wo) * s.Ho);
+  const long bg = static_cast<long>(b) * s.dg + dgi;
+  double pd, ph, pw;
+  dcn_position(s, off + bg * 3 * s.K * s.Q, k, od, oh, ow, q, pd, ph, pw);
+  ZTaps<A> t;
+  zero_pad_taps(s, pd, ph, pw, t);
+  A go_d = A(0), go_h = A(0), go_w = A(0), gm = A(0);
+  if (t.ok) {
+    const A m = mask ? load(mask + (bg * s.K + k) * s.Q + q) : A(1);
+    for (int c = dgi * s.cpd; c < (dgi + 1) * s.cpd; c++) {
+      const int grp = c / s.cpg, cl = c % s.cpg;
+      A gcol = A(0);
+      const T *wcol = wt + (static_cast<long>(grp) * s.opg * s.cpg + cl) * s.K + k;
+      const T *gyo = gy + (static_cast<long>(b) * s.Cout + grp * s.opg) * s.Q + q;
+      for (int o = 0; o < s.opg; o++)
+        gcol += load(wcol + static_cast<long>(o) * s.cpg * s.K) * load(gyo + o * s.Q);
+      const T *plane = x + (static_cast<long>(b) * s.Cin + c) * s.P;
+      G *gplane = gx + (static_cast<long>(b) * s.Cin + c) * s.P;
+      A v[8];
+      A val = A(0);
+#pragma unroll
+      for (int n = 0; n < 8; n++) {
+        v[n] = t.off[n] >= 0 ? load(plane + t.off[n]) : A(0);
+        val += t.w[n] * v[n];
+        if (t.off[n] >= 0) atomic_add(gplane + t.off[n], static_cast<G>(t.w[n] * gcol * m));
+      }
+      gm += gcol * val;
+      const A hd = A(1) - t.fd, hh = A(1) - t.fh, hw = A(1) - t.fw;
+      // d/dp of the trilinear blend: the differentiated axis contributes -1 (low) / +1 (high)
+      const A dd = hh * (hw * (v[4] - v[0]) + t.fw * (v[5] - v[1])) +
+                   t.fh * (hw * (v[6] - v[2]) + t.fw * (v[7] - v[3]));
+      const A dh = hd * (hw * (v[2] - v[0]) + t.fw * (v[3] - v[1])) +
+                   t.fd * (hw * (v[6] - v[4]) + t.fw * (v[7] - v[5]));
+      const A dw = hd * (hh * (v[1] - v[0]) + t.fh * (v[3] - v[2])) +
+                   t.fd * (hh * (v[5] - v[4]) + t.fh * (v[7] - v[6]));
+      go_d += dd * gcol * m; go_h += dh * gcol * m; go_w += dw * gcol * m;
+    }
+  }
+  T *o = goff + (bg * 3 * s.K + 3 * k) * s.Q + q;
+  o[0] = store_cast<T>(go_d); o[s.Q] = store_cast<T>(go_h); o[2 * s.Q] = store_cast<T>(go_w);
+  if (gmask) gmask[(bg * s.K + k) * s.Q + q] = store_cast<T>(gm);
+}
+
+// ---- backward 2: grad wrt weight.  workgroup = (input channel c, tap k, slab of positions) ----
+// every thread rebuilds col[c,k,q] for its positions, multiplies with gy[b,o,q] for the <= 32
+// output channels of the tile, the workgroup reduces and adds one value per (o,c,k) atomically.
+constexpr int kGwThreads = 256;
+constexpr int kGwPositions = 4096;
+
+template <typename T, typename G>
+__global__ __launch_bounds__(kGwThreads) void dcn_backward_weight_kernel(
+    const T *__restrict__ x, const T *__restrict__ off, const T *__restrict__ mask,
+    const T *__restrict__ gy, G *__restrict__ gw, const DcnDims s, const int slabs) {
+  using A = typename Acc<T>::type;
+  const int k = blockIdx.x % s.K, c = blockIdx.x / s.K;
+  const int tiles = (s.opg + kOutTile - 1) / kOutTile;
+  const int tile = blockIdx.y % tiles, slab = blockIdx.y / tiles;
+  const int b = blockIdx.z;
+  const int grp = c / s.cpg, cl = c % s.cpg, dgi = c / s.cpd;
+  const int o_begin = grp * s.opg + tile * kOutTile;
+  const int o_count = min(kOutTile, grp * s.opg + s.opg - o_begin);
+  const long bg = static_cast<long>(b) * s.dg + dgi;
+  const T *plane = x + (static_cast<long>(b) * s.Cin + c) * s.P;
+  A acc[kOutTile];
+#pragma unroll
+  for (int i = 0; i < kOutTile; i++) acc[i] = A(0);
+  const long q_end = min(static_cast<long>(slab + 1) * kGwPositions, s.Q);
+  for (long q = static_cast<long>(slab) * kGwPositions + threadIdx.x; q < q_end; q += kGwThreads) {
+    const int ow = q % s.Wo, oh = (q / s.Wo) % s.Ho, od = q / (static_cast<long>(s.Wo) * s.Ho);
+    double pd, ph, pw;
+    dcn_position(s, off + bg * 3 * s.K * s.Q, k, od, oh, ow, q, pd, ph, pw);
+    ZTaps<A> t;
+    zero_pad_taps(s, pd, ph, pw, t);
+    if (!t.ok) continue;
+    const A m = mask ? load(mask + (bg * s.K + k) * s.Q + q) : A(1);
+    const A col = zsample<T, A>(plane, t) * m;
+    const T *gyo = gy + (static_cast<long>(b) * s.Cout + o_begin) * s.Q + q;
+#pragma unroll
+    for (int i = 0; i < kOutTile; i++)
+      if (i < o_count) acc[i] += col * load(gyo + i * s.Q);
+  }
+  __shared__ A part[kGwThreads / kWave][kOutTile];
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+#pragma unroll
+  for (int i = 0; i < kOutTile; i++) {
+    A v = acc[i];
+    for (int d = kWave / 2; d > 0; d >>= 1) v += __shfl_down(v, d, kWave);
+    if (lane == 0) part[wave][i] = v;
+  }
+  __syncthreads();
+  if (threadIdx.x < o_count) {
+    A v = A(0);
+    for (int w = 0; w < kGwThreads / kWave; w++) v += part[w][threadIdx.x];
+    atomic_add(gw + (static_cast<long>(o_begin + threadIdx.x) * s.cpg + cl) * s.K + k,
+               static_cast<G>(v));
+  }
+  (void)slabs;
+}
+
+// ---- backward 3: grad wrt bias: workgroup = (o, b) --------------------------------------------
+template <typename T, typename G>
+__global__ __launch_bounds__(256) void dcn_backward_bias_kernel(const T *__restrict__ gy,
+                                                                G *__restrict__ gb,
+                                                                const DcnDims s) {
+  using A = typename Acc<T>::type;
+  const int o = blockIdx.x, b = blockIdx.y;
+  const T *src = gy + (static_cast<long>(b) * s.Cout + o) * s.Q;
+  A v = A(0);
+  for (long q = threadIdx.x; q < s.Q; q += 256) v += load(src + q);
+  __shared__ A part[4];
+  for (int d = kWave / 2; d > 0; d >>= 1) v += __shfl_down(v, d, kWave);
+  if (threadIdx.x % kWave == 0) part[threadIdx.x / kWave] = v;
+  __syncthreads();
+  if (threadIdx.x == 0) atomic_add(gb + o, static_cast<G>(part[0] + part[1] + part[2] + part[3]));
+}
+
+__global__ void dcn_fill_zero_kernel(float *p, long n) {
+  for (long i = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; i < n;
+       i += static_cast<long>(gridDim.x) * blockDim.x)
+    p[i] = 0.f;
+}
+
+template <typename T>
+__global__ void dcn_add_from_f32_kernel(T *dst, const float *src, long n) {
+  for (long i = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; i < n;
+       i += static_cast<long>(gridDim.x) * blockDim.x)
+    dst[i] = store_cast<T>(load(dst + i) + src[i]);
+}
+
+// matrix-core forward for 16-bit tensors (dcn3d_mfma.hip)
+bool dcn_mfma_supported(const DcnDims &s, int dtype);
+size_t dcn_mfma_workspace_bytes(const DcnDims &s, int dtype);
+int dcn_mfma_forward(const void *x, const void *off, const void *mask, const void *wt,
+                     const void *bias, void *y, const DcnDims &s, int dtype, void *workspace,
+                     hipStream_t stream);
+
+static inline int blocks_for(long n, int per_block, int cap) {
+  return static_cast<int>(std::min<long>((n + per_block - 1) / per_block, cap));
+}
+
+}  // namespace mv
+
+using namespace mv;
+
+extern "C" {
+
+int mv_dcn3d_output_dims(const mv_dcn3d_shape *shape, int *out_d, int *out_h, int *out_w) {
+  DcnDims s;
+  int st = make_dcn_dims(s, shape);
+  if (st) return st;
+  *out_d = s.Do; *out_h = s.Ho; *out_w = s.Wo;
+  return MV_OK;
+}
+
+size_t mv_dcn3d_forward_workspace_bytes(const mv_dcn3d_shape *shape, int dtype) {
+  DcnDims s;
+  if (make_dcn_dims(s, shape)) return 0;
+  return dcn_mfma_supported(s, dtype) ? dcn_mfma_workspace_bytes(s, dtype) : 0;
+}
+
+size_t mv_dcn3d_backward_workspace_bytes(const mv_dcn3d_shape *shape, int dtype) {
+  DcnDims s;
+  if (make_dcn_dims(s, shape)) return 0;
+  if (dtype != MV_F16 && dtype != MV_BF16) return 0;
+  // fp32 accumulators for grad_input, grad_weight, grad_bias
+  const size_t n = static_cast<size_t>(s.B) * s.Cin * s.P + static_cast<size_t>(s.Cout) * s.cpg * s.K + s.Cout;
+  return n * sizeof(float);
+}
+
+int mv_dcn3d_forward(const void *input, const void *offset, const void *mask, const void *weight,
+                     const void *bias, void *output, const mv_dcn3d_shape *shape, int dtype,
+                     void *workspace, void *stream) {
+  DcnDims s;
+  int st = make_dcn_dims(s, shape);
+  if (st) return st;
+  MV_REQUIRE(input && offset && weight && output, "null pointer argument");
+  hipStream_t hs = static_cast<hipStream_t>(stream);
+  if (dcn_mfma_supported(s, dtype)) {
+    MV_REQUIRE(workspace, "this shape needs a workspace of mv_dcn3d_forward_workspace_bytes()");
+    return dcn_mfma_forward(input, offset, mask, weight, bias, output, s, dtype, workspace, hs);
+  }
+  const long qb = (s.Q + kDcnThreads - 1) / kDcnThreads;
+  const long yb = static_cast<long>(s.groups) * ((s.opg + kOutTile - 1) / kOutTile);
+  MV_REQUIRE(qb < (1L << 31) && yb <= 65535 && s.B <= 65535, "grid too large");
+  const dim3 grid(static_cast<unsigned>(qb), static_cast<unsigned>(yb), s.B), block(kDcnThreads);
+  MV_DISPATCH(dtype, {
+    hipLaunchKernelGGL((dcn_forward_kernel<T>), grid, block, 0, hs, static_cast<const T *>(input),
+                       static_cast<const T *>(offset), static_cast<const T *>(mask),
+                       static_cast<const T *>(weight), static_cast<const T *>(bias),
+                       static_cast<T *>(output), s);
+  });
+  return check_launch("dcn_forward_kernel");
+}
+
+int mv_dcn3d_backward(const void *input, const void *offset, const void *mask, const void *weight,
+                      const void *grad_output, void *grad_input, void *grad_offset,
+                      void *grad_mask, void *grad_weight, void *grad_bias,
+                      const mv_dcn3d_shape *shape, int dtype, void *workspace, void *stream) {
+  DcnDims s;
+  int st = make_dcn_dims(s, shape);
+  if (st) return st;
+  MV_REQUIRE(input && offset && weight && grad_output && grad_input && grad_offset && grad_weight,
+             "null pointer argument");
+  MV_REQUIRE((mask == nullptr) == (grad_mask == nullptr) || grad_mask == nullptr,
+             "grad_mask given without mask");
+  const bool narrow = dtype == MV_F16 || dtype == MV_BF16;
+  MV_REQUIRE(!narrow || workspace, "16-bit backward needs an fp32 workspace");
+  hipStream_t hs = static_cast<hipStream_t>(stream);
+  const long n_gx = static_cast<long>(s.B) * s.Cin * s.P, n_gw = static_cast<long>(s.Cout) * s.cpg * s.K;
+  float *ws = static_cast<float *>(workspace);
+  if (narrow) {
+    const long n = n_gx + n_gw + s.Cout;
+    hipLaunchKernelGGL(dcn_fill_zero_kernel, dim3(blocks_for(n, 1024, 65536)), dim3(256), 0, hs, ws, n);
+  }
+  const long qb = (s.Q + kDcnThreads - 1) / kDcnThreads;
+  const long kb = static_cast<long>(s.dg) * s.K;
+  const int tiles = (s.opg + kOutTile - 1) / kOutTile;
+  const int slabs = static_cast<int>((s.Q + kGwPositions - 1) / kGwPositions);
+  MV_REQUIRE(qb < (1L << 31) && kb <= 65535 && s.B <= 65535 &&
+                 static_cast<long>(tiles) * slabs <= 65535 &&
+                 static_cast<long>(s.Cin) * s.K < (1L << 31), "grid too large");
+  MV_DISPATCH(dtype, {
+    using G = typename std::conditional<(sizeof(T) == 2), float, T>::type;
+    G *gx = narrow ? reinterpret_cast<G *>(ws) : static_cast<G *>(grad_input);
+    G *gw = narrow ? reinterpret_cast<G *>(ws + n_gx) : static_cast<G *>(grad_weight);
+    G *gb = narrow ? reinterpret_cast<G *>(ws + n_gx + n_gw) : static_cast<G *>(grad_bias);
+    hipLaunchKernelGGL((dcn_backward_data_kernel<T, G>),
+                       dim3(static_cast<unsigned>(qb), static_cast<unsigned>(kb), s.B),
+                       dim3(kDcnThreads), 0, hs, static_cast<const T *>(input),
+                       static_cast<const T *>(offset), static_cast<const T *>(mask),
+                       static_cast<const T *>(weight), static_cast<const T *>(grad_output), gx,
+                       static_cast<T *>(grad_offset), static_cast<T *>(grad_mask), s);
+    hipLaunchKernelGGL((dcn_backward_weight_kernel<T, G>),
+                       dim3(static_cast<unsigned>(s.Cin * s.K), static_cast<unsigned>(tiles * slabs), s.B),
+                       dim3(kGwThreads), 0, hs, static_cast<const T *>(input),
+                       static_cast<const T *>(offset), static_cast<const T *>(mask),
+                       static_cast<const T *>(grad_output), gw, s, slabs);
+    if (grad_bias)
+      hipLaunchKernelGGL((dcn_backward_bias_kernel<T, G>), dim3(s.Cout, s.B), dim3(256), 0, hs,
+                         static_cast<const T *>(grad_output), gb, s);
+    if (sizeof(T) == 2) {
+      hipLaunchKernelGGL((dcn_add_from_f32_kernel<T>), dim3(blocks_for(n_gx, 1024, 65536)), dim3(256),
+                         0, hs, static_cast<T *>(grad_input), ws, n_gx);
+      hipLaunchKernelGGL((dcn_add_from_f32_kernel<T>), dim3(blocks_for(n_gw, 1024, 65536)), dim3(256),
+                         0, hs, static_cast<T *>(grad_weight), ws + n_gx, n_gw);
+      if (grad_bias)
+        hipLaunchKernelGGL((dcn_add_from_f32_kernel<T>), dim3(1), dim3(256), 0, hs,
+                           static_cast<T *>(grad_bias), ws + n_gx + n_gw, static_cast<long>(s.Cout));
+    }
+  });
+  return check_launch("dcn3d backward");
+}
+
+}  // extern "C"

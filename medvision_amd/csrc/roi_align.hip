@@ -1,0 +1,310 @@
+// RoIAlign / RoIAlignRotated 2-D and 3-D, forward and backward: general-shape kernels.
+//
+// Work decomposition: one workgroup = (one roi, one chunk of kChunk consecutive output elements
+// of that roi in [C, od, oh, ow] order).  Lane 0 turns the roi row into the sample-grid geometry
+// (fp64, 3 sincos) once per workgroup and shares it through LDS, so the per-element work is only
+// the sample loop.  Consecutive lanes own consecutive pw, so output stores (forward) and
+// grad_output loads (backward) are coalesced along W.
+#include "common.hpp"
+#include "roi_geometry.hpp"
+#include "sampling.hpp"
+
+namespace mv {
+
+constexpr int kRoiThreads = 256;
+constexpr int kRoiChunk = kRoiThreads * 4;
+
+template <typename T, typename RT, bool ROT>
+__global__ __launch_bounds__(kRoiThreads) void roi_forward_kernel(const T *__restrict__ feat,
+                                                                  const RT *__restrict__ rois,
+                                                                  T *__restrict__ out,
+                                                                  const RoiProblem p) {
+  using A = typename Acc<T>::type;
+  __shared__ RoiGeom g;
+  const unsigned n = blockIdx.x / p.chunks, chunk = blockIdx.x % p.chunks;
+  if (threadIdx.x == 0) build_geom(g, rois + static_cast<long>(n) * roi_columns(p.ndim, p.rotated), p);
+  __syncthreads();
+  const unsigned begin = chunk * kRoiChunk;
+  const unsigned end = min(begin + kRoiChunk, p.per_roi);
+  const long plane = static_cast<long>(p.D) * p.H * p.W;
+  const int gz = p.ndim == 3 ? g.grid[2] : 1, gy = g.grid[1], gx = g.grid[0];
+  for (unsigned e = begin + threadIdx.x; e < end; e += kRoiThreads) {
+    const unsigned pw = e % p.ow, t1 = e / p.ow;
+    const unsigned ph = t1 % p.oh, t2 = t1 / p.oh;
+    const unsigned pd = t2 % p.od, c = t2 / p.od;
+    A acc = A(0);
+    if (g.batch >= 0) {
+      const T *src = feat + (static_cast<long>(g.batch) * p.C + c) * plane;
+      for (int iz = 0; iz < gz; iz++) {
+        const double z = p.ndim == 3 ? local_coord(g, 2, pd, iz) : 0.0;
+        for (int iy = 0; iy < gy; iy++) {
+          const double y = local_coord(g, 1, ph, iy);
+          for (int ix = 0; ix < gx; ix++) {
+            const double x = local_coord(g, 0, pw, ix);
+            double rx = x, ry = y, rz = z;
+            if (ROT) {
+              rx = g.rot[0] * x + g.rot[1] * y + g.rot[2] * z + g.centre[0];
+              ry = g.rot[3] * x + g.rot[4] * y + g.rot[5] * z + g.centre[1];
+              rz = p.ndim == 3 ? g.rot[6] * x + g.rot[7] * y + g.rot[8] * z + g.centre[2] : 0.0;
+            }
+            acc += sample_clamped<T>(src, p.D, p.H, p.W, rz, ry, rx, p.order);
+          }
+        }
+      }
+    }
+    out[static_cast<long>(n) * p.per_roi + e] = store_cast<T>(acc / static_cast<A>(g.count));
+  }
+}
+
+// G = element type of the accumulation buffer (T itself for fp32/fp64, float for 16-bit T).
+template <typename T, typename G, typename RT, bool ROT>
+__global__ __launch_bounds__(kRoiThreads) void roi_backward_kernel(const T *__restrict__ gout,
+                                                                   const RT *__restrict__ rois,
+                                                                   G *__restrict__ gin,
+                                                                   const RoiProblem p) {
+  using A = typename Acc<T>::type;
+  __shared__ RoiGeom g;
+  const unsigned n = blockIdx.x / p.chunks, chunk = blockIdx.x % p.chunks;
+  if (threadIdx.x == 0) build_geom(g, rois + static_cast<long>(n) * roi_columns(p.ndim, p.rotated), p);
+  __syncthreads();
+  if (g.batch < 0) return;
+  const unsigned begin = chunk * kRoiChunk;
+  const unsigned end = min(begin + kRoiChunk, p.per_roi);
+  const long plane = static_cast<long>(p.D) * p.H * p.W;
+  const int gz = p.ndim == 3 ? g.grid[2] : 1, gy = g.grid[1], gx = g.grid[0];
+  for (unsigned e = begin + threadIdx.x; e < end; e += kRoiThreads) {
+    const unsigned pw = e % p.ow, t1 = e / p.ow;
+    const unsigned ph = t1 % p.oh, t2 = t1 / p.oh;
+    const unsigned pd = t2 % p.od, c = t2 / p.od;
+    const A top = load(gout + static_cast<long>(n) * p.per_roi + e) / static_cast<A>(g.count);
+    G *dst = gin + (static_cast<long>(g.batch) * p.C + c) * plane;
+    for (int iz = 0; iz < gz; iz++) {
+      const double z = p.ndim == 3 ? local_coord(g, 2, pd, iz) : 0.0;
+      for (int iy = 0; iy < gy; iy++) {
+        const double y = local_coord(g, 1, ph, iy);
+        for (int ix = 0; ix < gx; ix++) {
+          const double x = local_coord(g, 0, pw, ix);
+          double rx = x, ry = y, rz = z;
+          if (ROT) {
+            rx = g.rot[0] * x + g.rot[1] * y + g.rot[2] * z + g.centre[0];
+            ry = g.rot[3] * x + g.rot[4] * y + g.rot[5] * z + g.centre[1];
+            rz = p.ndim == 3 ? g.rot[6] * x + g.rot[7] * y + g.rot[8] * z + g.centre[2] : 0.0;
+          }
+          Corners<A> cw;
+          if (!clamped_corners<A>(p.D, p.H, p.W, rz, ry, rx, p.order, cw)) continue;
+#pragma unroll
+          for (int k = 0; k < 8; k++)
+            if (cw.w[k] != A(0)) atomic_add(dst + cw.idx[k], static_cast<G>(top * cw.w[k]));
+        }
+      }
+    }
+  }
+}
+
+__global__ void fill_zero_kernel(float *p, long n) {
+  for (long i = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; i < n;
+       i += static_cast<long>(gridDim.x) * blockDim.x)
+    p[i] = 0.f;
+}
+
+template <typename T>
+__global__ void add_from_f32_kernel(T *dst, const float *src, long n) {
+  for (long i = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; i < n;
+       i += static_cast<long>(gridDim.x) * blockDim.x)
+    dst[i] = store_cast<T>(load(dst + i) + src[i]);
+}
+
+static int make_problem(RoiProblem &p, int ndim, int rotated, int batch, int channels, int depth,
+                        int height, int width, int num_rois, int out_d, int out_h, int out_w,
+                        float spatial_scale, int sampling_ratio, int aligned, int order) {
+  MV_REQUIRE(batch > 0 && channels > 0 && depth > 0 && height > 0 && width > 0,
+             "feature dims must be positive (got %d,%d,%d,%d,%d)", batch, channels, depth, height, width);
+  MV_REQUIRE(num_rois >= 0, "num_rois must be >= 0");
+  MV_REQUIRE(out_d > 0 && out_h > 0 && out_w > 0, "output size must be positive");
+  MV_REQUIRE(order == 0 || order == 1, "only support order = 0 (nearest) or 1 (linear), got %d", order);
+  const long per_roi = static_cast<long>(channels) * out_d * out_h * out_w;
+  MV_REQUIRE(per_roi < (1L << 31), "channels*out_d*out_h*out_w must be < 2^31");
+  const long chunks = (per_roi + kRoiChunk - 1) / kRoiChunk;
+  MV_REQUIRE(chunks * static_cast<long>(num_rois) < (1L << 31), "too many workgroups");
+  p.ndim = ndim; p.rotated = rotated;
+  p.N = batch; p.C = channels; p.D = depth; p.H = height; p.W = width; p.R = num_rois;
+  p.od = out_d; p.oh = out_h; p.ow = out_w;
+  p.scale = static_cast<double>(spatial_scale);
+  p.sampling_ratio = sampling_ratio; p.aligned = aligned; p.order = order;
+  p.per_roi = static_cast<unsigned>(per_roi);
+  p.chunks = static_cast<unsigned>(chunks);
+  return MV_OK;
+}
+
+int roi_forward(const void *input, const void *rois, void *output, int dtype, int ndim,
+                int rotated, int batch, int channels, int depth, int height, int width,
+                int num_rois, int out_d, int out_h, int out_w, float spatial_scale,
+                int sampling_ratio, int aligned, int order, void *stream) {
+  RoiProblem p;
+  int st = make_problem(p, ndim, rotated, batch, channels, depth, height, width, num_rois, out_d,
+                        out_h, out_w, spatial_scale, sampling_ratio, aligned, order);
+  if (st) return st;
+  if (num_rois == 0) return MV_OK;
+  MV_REQUIRE(input && rois && output, "null pointer argument");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(p.chunks * num_rois), block(kRoiThreads);
+  MV_DISPATCH(dtype, {
+    using RT = typename std::conditional<std::is_same<T, double>::value, double, float>::type;
+    if (rotated)
+      hipLaunchKernelGGL((roi_forward_kernel<T, RT, true>), grid, block, 0, s,
+                         static_cast<const T *>(input), static_cast<const RT *>(rois),
+                         static_cast<T *>(output), p);
+    else
+      hipLaunchKernelGGL((roi_forward_kernel<T, RT, false>), grid, block, 0, s,
+                         static_cast<const T *>(input), static_cast<const RT *>(rois),
+                         static_cast<T *>(output), p);
+  });
+  return check_launch("roi_forward_kernel");
+}
+
+int roi_backward(const void *grad_output, const void *rois, void *grad_input, int dtype, int ndim,
+                 int rotated, int batch, int channels, int depth, int height, int width,
+                 int num_rois, int out_d, int out_h, int out_w, float spatial_scale,
+                 int sampling_ratio, int aligned, int order, void *workspace, void *stream) {
+  RoiProblem p;
+  int st = make_problem(p, ndim, rotated, batch, channels, depth, height, width, num_rois, out_d,
+                        out_h, out_w, spatial_scale, sampling_ratio, aligned, order);
+  if (st) return st;
+  if (num_rois == 0) return MV_OK;
+  MV_REQUIRE(grad_output && rois && grad_input, "null pointer argument");
+  const bool narrow = dtype == MV_F16 || dtype == MV_BF16;
+  MV_REQUIRE(!narrow || workspace, "16-bit backward needs an fp32 workspace");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(p.chunks * num_rois), block(kRoiThreads);
+  const long total = static_cast<long>(batch) * channels * depth * height * width;
+  const int fill_blocks = static_cast<int>(std::min<long>((total + 1023) / 1024, 65536));
+  if (narrow) {
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(fill_blocks), dim3(256), 0, s,
+                       static_cast<float *>(workspace), total);
+  }
+  MV_DISPATCH(dtype, {
+    using RT = typename std::conditional<std::is_same<T, double>::value, double, float>::type;
+    using G = typename std::conditional<(sizeof(T) == 2), float, T>::type;
+    G *acc = narrow ? static_cast<G *>(workspace) : static_cast<G *>(grad_input);
+    if (rotated)
+      hipLaunchKernelGGL((roi_backward_kernel<T, G, RT, true>), grid, block, 0, s,
+                         static_cast<const T *>(grad_output), static_cast<const RT *>(rois), acc, p);
+    else
+      hipLaunchKernelGGL((roi_backward_kernel<T, G, RT, false>), grid, block, 0, s,
+                         static_cast<const T *>(grad_output), static_cast<const RT *>(rois), acc, p);
+    if (sizeof(T) == 2)
+      hipLaunchKernelGGL((add_from_f32_kernel<T>), dim3(fill_blocks), dim3(256), 0, s,
+                         static_cast<T *>(grad_input), static_cast<const float *>(workspace), total);
+  });
+  return check_launch("roi_backward_kernel");
+}
+
+}  // namespace mv
+
+// ---------------------------------------------------------------------------------------------
+// C ABI
+// ---------------------------------------------------------------------------------------------
+using mv::roi_backward;
+using mv::roi_forward;
+
+extern "C" {
+
+int mv_roi_align_2d_forward(const void *input, const void *rois, void *output, int dtype,
+                            int batch, int channels, int height, int width, int num_rois,
+                            int out_h, int out_w, float spatial_scale, int sampling_ratio,
+                            int order, void *stream) {
+  return roi_forward(input, rois, output, dtype, 2, 0, batch, channels, 1, height, width, num_rois,
+                     1, out_h, out_w, spatial_scale, sampling_ratio, 1, order, stream);
+}
+
+int mv_roi_align_2d_backward(const void *grad_output, const void *rois, void *grad_input,
+                             int dtype, int batch, int channels, int height, int width,
+                             int num_rois, int out_h, int out_w, float spatial_scale,
+                             int sampling_ratio, int order, void *workspace, void *stream) {
+  return roi_backward(grad_output, rois, grad_input, dtype, 2, 0, batch, channels, 1, height,
+                      width, num_rois, 1, out_h, out_w, spatial_scale, sampling_ratio, 1, order,
+                      workspace, stream);
+}
+
+int mv_roi_align_3d_forward(const void *input, const void *rois, void *output, int dtype,
+                            int batch, int channels, int depth, int height, int width,
+                            int num_rois, int out_d, int out_h, int out_w, float spatial_scale,
+                            int sampling_ratio, int order, void *stream) {
+  return roi_forward(input, rois, output, dtype, 3, 0, batch, channels, depth, height, width,
+                     num_rois, out_d, out_h, out_w, spatial_scale, sampling_ratio, 1, order, stream);
+}
+
+int mv_roi_align_3d_backward(const void *grad_output, const void *rois, void *grad_input,
+                             int dtype, int batch, int channels, int depth, int height, int width,
+                             int num_rois, int out_d, int out_h, int out_w, float spatial_scale,
+                             int sampling_ratio, int order, void *workspace, void *stream) {
+  return roi_backward(grad_output, rois, grad_input, dtype, 3, 0, batch, channels, depth, height,
+                      width, num_rois, out_d, out_h, out_w, spatial_scale, sampling_ratio, 1,
+                      order, workspace, stream);
+}
+
+int mv_roi_align_rotated_2d_forward(const void *input, const void *rois, void *output, int dtype,
+                                    int batch, int channels, int height, int width, int num_rois,
+                                    int out_h, int out_w, float spatial_scale, int sampling_ratio,
+                                    int aligned, int order, void *stream) {
+  return roi_forward(input, rois, output, dtype, 2, 1, batch, channels, 1, height, width, num_rois,
+                     1, out_h, out_w, spatial_scale, sampling_ratio, aligned, order, stream);
+}
+
+int mv_roi_align_rotated_2d_backward(const void *grad_output, const void *rois, void *grad_input,
+                                     int dtype, int batch, int channels, int height, int width,
+                                     int num_rois, int out_h, int out_w, float spatial_scale,
+                                     int sampling_ratio, int aligned, int order, void *workspace,
+                                     void *stream) {
+  return roi_backward(grad_output, rois, grad_input, dtype, 2, 1, batch, channels, 1, height,
+                      width, num_rois, 1, out_h, out_w, spatial_scale, sampling_ratio, aligned,
+                      order, workspace, stream);
+}
+
+int mv_roi_align_rotated_3d_forward(const void *input, const void *rois, void *output, int dtype,
+                                    int batch, int channels, int depth, int height, int width,
+                                    int num_rois, int out_d, int out_h, int out_w,
+                                    float spatial_scale, int sampling_ratio, int aligned,
+                                    int order, void *stream) {
+  return roi_forward(input, rois, output, dtype, 3, 1, batch, channels, depth, height, width,
+                     num_rois, out_d, out_h, out_w, spatial_scale, sampling_ratio, aligned, order,
+                     stream);
+}
+
+int mv_roi_align_rotated_3d_backward(const void *grad_output, const void *rois, void *grad_input,
+                                     int dtype, int batch, int channels, int depth, int height,
+                                     int width, int num_rois, int out_d, int out_h, int out_w,
+                                     float spatial_scale, int sampling_ratio, int aligned,
+                                     int order, void *workspace, void *stream) {
+  return roi_backward(grad_output, rois, grad_input, dtype, 3, 1, batch, channels, depth, height,
+                      width, num_rois, out_d, out_h, out_w, spatial_scale, sampling_ratio, aligned,
+                      order, workspace, stream);
+}
+
+size_t mv_roi_align_backward_workspace_bytes(int dtype, int batch, int channels, int depth,
+                                             int height, int width) {
+  if (dtype != MV_F16 && dtype != MV_BF16) return 0;
+  return sizeof(float) * static_cast<size_t>(batch) * channels * depth * height * width;
+}
+
+int mv_affine_2d(const void *input, const void *rois, void *output, int dtype, int batch,
+                 int channels, int height, int width, int num_rois, int out_h, int out_w,
+                 float spatial_scale, int sampling_ratio, int aligned, int order, void *stream) {
+  if (order == 3)
+    return mv::fail(MV_INVALID_ARGUMENT, "affine_2d: order 3 (cubic) is not implemented");
+  return roi_forward(input, rois, output, dtype, 2, 1, batch, channels, 1, height, width, num_rois,
+                     1, out_h, out_w, spatial_scale, sampling_ratio, aligned, order, stream);
+}
+
+int mv_affine_3d(const void *input, const void *rois, void *output, int dtype, int batch,
+                 int channels, int depth, int height, int width, int num_rois, int out_d,
+                 int out_h, int out_w, float spatial_scale, int sampling_ratio, int aligned,
+                 int order, void *stream) {
+  if (order == 3)
+    return mv::fail(MV_INVALID_ARGUMENT, "affine_3d: order 3 (cubic) is not implemented");
+  return roi_forward(input, rois, output, dtype, 3, 1, batch, channels, depth, height, width,
+                     num_rois, out_d, out_h, out_w, spatial_scale, sampling_ratio, aligned, order,
+                     stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,88 @@
+// Device-side samplers shared by the RoI, warp and DCN kernels.
+//
+// Coordinates are carried in fp64 (full-rate on CDNA and accurate enough that the position of a
+// sample relative to the floor / 0.5-tie / [-1,S] discontinuities agrees with an fp64 evaluation);
+// interpolation weights and sums use the arithmetic type A (fp32, or fp64 for double tensors).
+#pragma once
+#include "common.hpp"
+
+namespace mv {
+
+// Border-replicating tap on one axis (reference: csrc/cuda/interpolation_helpers_3d.h:12-48):
+// outside the closed interval [-1, size] the sample is void; negatives snap to 0; a base index
+// at or beyond size-1 collapses both taps onto size-1.
+template <typename A>
+__device__ __forceinline__ bool clamped_tap(double v, int size, int &lo, int &hi, A &frac) {
+  if (v < -1.0 || v > static_cast<double>(size)) return false;
+  v = v <= 0.0 ? 0.0 : v;
+  const int base = static_cast<int>(v);
+  if (base >= size - 1) {
+    lo = hi = size - 1;
+    frac = A(0);
+  } else {
+    lo = base;
+    hi = base + 1;
+    frac = static_cast<A>(v - static_cast<double>(base));
+  }
+  return true;
+}
+
+// Eight-corner description of one sample; `w` follows the z-major corner order
+// (z0y0x0, z0y0x1, z0y1x0, ...).  For order 0 exactly one weight is 1: per axis the low index
+// wins when 1 - frac >= 0.5 (csrc/cuda/interpolation_helpers_3d.h:186-194).
+template <typename A> struct Corners {
+  long idx[8];
+  A w[8];
+};
+
+template <typename A>
+__device__ __forceinline__ bool clamped_corners(int D, int H, int W, double z, double y, double x,
+                                                int order, Corners<A> &c) {
+  int z0, z1, y0, y1, x0, x1;
+  A lz, ly, lx;
+  if (!clamped_tap(z, D, z0, z1, lz) || !clamped_tap(y, H, y0, y1, ly) ||
+      !clamped_tap(x, W, x0, x1, lx))
+    return false;
+  if (order == 0) {
+    lz = (A(1) - lz >= A(0.5)) ? A(0) : A(1);
+    ly = (A(1) - ly >= A(0.5)) ? A(0) : A(1);
+    lx = (A(1) - lx >= A(0.5)) ? A(0) : A(1);
+  }
+  const A hz = A(1) - lz, hy = A(1) - ly, hx = A(1) - lx;
+  const long r00 = (static_cast<long>(z0) * H + y0) * W, r01 = (static_cast<long>(z0) * H + y1) * W;
+  const long r10 = (static_cast<long>(z1) * H + y0) * W, r11 = (static_cast<long>(z1) * H + y1) * W;
+  c.idx[0] = r00 + x0; c.idx[1] = r00 + x1; c.idx[2] = r01 + x0; c.idx[3] = r01 + x1;
+  c.idx[4] = r10 + x0; c.idx[5] = r10 + x1; c.idx[6] = r11 + x0; c.idx[7] = r11 + x1;
+  c.w[0] = hz * hy * hx; c.w[1] = hz * hy * lx; c.w[2] = hz * ly * hx; c.w[3] = hz * ly * lx;
+  c.w[4] = lz * hy * hx; c.w[5] = lz * hy * lx; c.w[6] = lz * ly * hx; c.w[7] = lz * ly * lx;
+  return true;
+}
+
+template <typename T>
+__device__ __forceinline__ typename Acc<T>::type sample_clamped(const T *plane, int D, int H,
+                                                                int W, double z, double y,
+                                                                double x, int order) {
+  using A = typename Acc<T>::type;
+  int z0, z1, y0, y1, x0, x1;
+  A lz, ly, lx;
+  if (!clamped_tap(z, D, z0, z1, lz) || !clamped_tap(y, H, y0, y1, ly) ||
+      !clamped_tap(x, W, x0, x1, lx))
+    return A(0);
+  if (order == 0) {
+    const int zi = (A(1) - lz >= A(0.5)) ? z0 : z1;
+    const int yi = (A(1) - ly >= A(0.5)) ? y0 : y1;
+    const int xi = (A(1) - lx >= A(0.5)) ? x0 : x1;
+    return load(plane + (static_cast<long>(zi) * H + yi) * W + xi);
+  }
+  const A hz = A(1) - lz, hy = A(1) - ly, hx = A(1) - lx;
+  const T *r00 = plane + (static_cast<long>(z0) * H + y0) * W;
+  const T *r01 = plane + (static_cast<long>(z0) * H + y1) * W;
+  const T *r10 = plane + (static_cast<long>(z1) * H + y0) * W;
+  const T *r11 = plane + (static_cast<long>(z1) * H + y1) * W;
+  const A v1 = load(r00 + x0), v2 = load(r00 + x1), v3 = load(r01 + x0), v4 = load(r01 + x1);
+  const A v5 = load(r10 + x0), v6 = load(r10 + x1), v7 = load(r11 + x0), v8 = load(r11 + x1);
+  return hz * (hy * (hx * v1 + lx * v2) + ly * (hx * v3 + lx * v4)) +
+         lz * (hy * (hx * v5 + lx * v6) + ly * (hx * v7 + lx * v8));
+}
+
+}  // namespace mv

@@ -1,0 +1,153 @@
+"""GPU parity of the 3-D deformable convolutions (DCNv1 / DCNv2) and the displacement-field warp
+against the fp64 oracle, through the drop-in modules and the `_C` shim."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from parity import BWD_TOL, FWD_TOL, assert_close
+import workloads as wl
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import medvision_amd.ops as ops_
+    from medvision_amd import _lib
+    _lib.load()
+    return ops_
+
+
+def _to(dev, *ts):
+    return [None if t is None else t.to(dev) for t in ts]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("modulated,groups,dg,stride,pad,dil", [
+    (True, 1, 1, 1, 1, 1), (True, 2, 2, 2, 1, 1), (False, 1, 2, 1, 2, 2), (False, 2, 1, 1, 0, 1)])
+def test_functions_vs_oracle(ops, oracle, dtype, modulated, groups, dg, stride, pad, dil):
+    from medvision_amd.ops.deform_conv_3d import deform_conv
+    from medvision_amd.ops.modulated_deform_conv_3d import modulated_deform_conv
+    g = wl.gen(40 + groups + 2 * dg + stride)
+    x, off, mask, w, b = wl.dcn_inputs(g, 2, 4, 6, (6, 7, 8), 3, dg, groups, dtype, stride, pad, dil,
+                                       modulated)
+    xs, offs, ms, ws, bs = [None if t is None else t.to(DEV).requires_grad_(True)
+                            for t in (x, off, mask, w, b)]
+    if modulated:
+        y = modulated_deform_conv(xs, offs, ms, ws, bs, stride, pad, dil, groups, dg)
+    else:
+        y = deform_conv(xs, offs, ws, bs, stride, pad, dil, groups, dg, 64)
+    want = oracle.dcn3d_forward(x, off, mask, w, b, stride, pad, dil, groups, dg)
+    assert y.dtype == dtype
+    assert_close(y, want, FWD_TOL[dtype], "forward")
+    gy = torch.randn(y.shape, generator=g).to(dtype)
+    y.backward(gy.to(DEV))
+    gx, goff, gm, gw, gb = oracle.dcn3d_backward(x, off, mask, w, gy, True, stride, pad, dil, groups, dg)
+    tol = BWD_TOL[dtype]
+    assert_close(xs.grad, gx, tol, "grad input")
+    assert_close(offs.grad, goff, tol, "grad offset")
+    assert_close(ws.grad, gw, tol, "grad weight")
+    assert_close(bs.grad, gb, tol, "grad bias")
+    if modulated:
+        assert_close(ms.grad, gm, tol, "grad mask")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_config4_reduced_vs_oracle(ops, oracle, dtype):
+    """BASELINE config 4 channel / kernel geometry (Cin 32, Cout 64, 3^3, pad 1, dg 1,
+    offsets N(0,2), sigmoid mask) on a 12x12x16 volume so the CPU oracle finishes in seconds."""
+    from medvision_amd.ops.modulated_deform_conv_3d import modulated_deform_conv
+    g = wl.gen(3)
+    x, off, mask, w, b = wl.dcn_inputs(g, 2, 32, 64, (12, 12, 16), 3, 1, 1, dtype)
+    xs, offs, ms, ws, bs = _to(DEV, x, off, mask, w, b)
+    y = modulated_deform_conv(xs, offs, ms, ws, bs, 1, 1, 1, 1, 1)
+    want = oracle.dcn3d_forward(x, off, mask, w, b, 1, 1, 1, 1, 1)
+    assert_close(y, want, FWD_TOL[dtype], "config 4 forward")
+
+
+def test_config4_full_size_properties(ops):
+    """Full config-4 shape [2,32,48^3] -> Cout 64: zero offsets and unit mask reduce DCN to a plain
+    convolution (checked against torch's conv3d), and the op is linear in the mask."""
+    from medvision_amd.ops.modulated_deform_conv_3d import modulated_deform_conv
+    g = wl.gen(5)
+    x, off, mask, w, b = wl.dcn_inputs(g, 2, 32, 64, (48, 48, 48), 3, 1, 1, torch.float16)
+    xs, offs, ms, ws, bs = _to(DEV, x, off, mask, w, b)
+    y0 = modulated_deform_conv(xs, torch.zeros_like(offs), torch.ones_like(ms), ws, bs, 1, 1, 1, 1, 1)
+    ref = F.conv3d(xs.float(), ws.float(), bs.float(), 1, 1)
+    assert_close(y0, ref, FWD_TOL[torch.float16], "zero-offset == conv3d")
+    y1 = modulated_deform_conv(xs, offs, ms, ws, None, 1, 1, 1, 1, 1)
+    y2 = modulated_deform_conv(xs, offs, ms * 0.5, ws, None, 1, 1, 1, 1, 1)
+    assert_close(y2.float() * 2, y1.float(), 4e-3, "mask linearity")
+
+
+def test_modules_state_dict_and_autocast_training(ops):
+    """Mirrors the reference's smoke script (test/ops_test_dcn.py:41-65): Adam steps under autocast
+    with a GradScaler on a 1x3x5^3 input; here the loss must also go down."""
+    torch.manual_seed(0)
+    x = torch.rand(1, 3, 5, 5, 5, device=DEV)
+    target = torch.ones(1, 7, 5, 5, 5, device=DEV)
+    for cls, keys in ((ops.ModulatedDeformConv3dPack, {"weight", "bias", "conv_offset_mask.weight", "conv_offset_mask.bias"}),
+                      (ops.DeformConv3dPack, {"weight", "bias", "conv_offset.weight", "conv_offset.bias"})):
+        dcn = cls(in_channels=3, out_channels=7, kernel_size=3, stride=1, padding=1).to(DEV)
+        assert set(dcn.state_dict().keys()) == keys
+        opt = torch.optim.Adam(dcn.parameters(), lr=0.01)
+        scaler = torch.amp.GradScaler("cuda")
+        losses = []
+        for _ in range(20):
+            with torch.autocast("cuda", dtype=torch.float16):
+                out = dcn(x)
+                loss = F.binary_cross_entropy_with_logits(out.float(), target)
+            opt.zero_grad()
+            scaler.scale(loss).backward()
+            scaler.step(opt)
+            scaler.update()
+            losses.append(float(loss))
+        assert out.shape == (1, 7, 5, 5, 5)
+        assert losses[-1] < losses[0]
+    # zero-initialised offset branch: the pack equals a plain convolution at initialisation
+    dcn = ops.ModulatedDeformConv3dPack(3, 7, 3, stride=1, padding=1).to(DEV)
+    want = 0.5 * F.conv3d(x, dcn.weight, None, 1, 1) + dcn.bias.view(1, -1, 1, 1, 1)  # sigmoid(0) = .5
+    assert_close(dcn(x), want, 1e-5, "pack at init")
+
+
+def test_dcn_errors(ops):
+    from medvision_amd import _C
+    x = torch.randn(2, 4, 5, 5, 5, device=DEV)
+    w = torch.randn(6, 4, 3, 3, 3, device=DEV)
+    off = torch.zeros(2, 81, 5, 5, 5, device=DEV)
+    b = torch.zeros(6, device=DEV)
+    args = (3, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        _C.deform_conv_3d_forward(x.transpose(3, 4), w, b, off, *args, 64)
+    with pytest.raises(RuntimeError, match="kernel channels wont match"):
+        _C.deform_conv_3d_forward(x, w[:, :3].contiguous(), b, off, *args, 64)
+    with pytest.raises(RuntimeError, match="kernel shape wont match"):
+        _C.deform_conv_3d_forward(x, w, b, off, 3, 3, 2, *args[3:], 64)
+    with pytest.raises(RuntimeError, match="must divide im2col_step"):
+        _C.deform_conv_3d_forward(x.repeat(2, 1, 1, 1, 1)[:3].contiguous(), w, b,
+                                  off.repeat(2, 1, 1, 1, 1)[:3].contiguous(), *args, 2)
+    with pytest.raises(RuntimeError, match="Not implemented on the CPU"):
+        _C.deform_conv_3d_forward(x.cpu(), w.cpu(), b.cpu(), off.cpu(), *args, 64)
+    with pytest.raises(RuntimeError, match="offset has shape"):
+        _C.deform_conv_3d_forward(x, w, b, off[:, :80].contiguous(), *args, 64)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("order", [0, 1])
+def test_warp_vs_oracle(ops, oracle, dtype, order):
+    g = wl.gen(8)
+    img = torch.randn(2, 3, 10, 12, 14, generator=g).to(dtype)
+    off = (torch.randn(2, 3, 10, 12, 14, generator=g) * 3).to(dtype)
+    got = ops.apply_offset_3d(img.to(DEV), off.to(DEV), order)
+    assert_close(got, oracle.deform_warp(img, off, order), FWD_TOL[dtype], "warp 3d")
+    img2 = torch.randn(2, 3, 20, 24, generator=g).to(dtype)
+    off2 = (torch.randn(2, 2, 20, 24, generator=g) * 3).to(dtype)
+    got = ops.apply_offset_2d(img2.to(DEV), off2.to(DEV), order)
+    assert_close(got, oracle.deform_warp(img2, off2, order), FWD_TOL[dtype], "warp 2d")
+    # the reference's calling convention (identity weight through `_C.deform_3d`) gives the same
+    from medvision_amd import _C
+    eye = torch.eye(3, device=DEV, dtype=dtype).reshape(3, 3, 1, 1, 1)
+    same = _C.deform_3d(img.to(DEV), eye, torch.zeros(3, device=DEV, dtype=dtype), off.to(DEV),
+                        1, 1, 1, 1, 1, 1, 0, 0, 0, 1, 1, 1, 1, 1, 64, order)
+    assert torch.equal(same, ops.apply_offset_3d(img.to(DEV), off.to(DEV), order))

@@ -1,0 +1,218 @@
+"""GPU parity of RoIAlign / RoIAlignRotated / affine (through medvision_amd.ops -> _C -> C ABI)
+against the fp64 oracle on the same seeded inputs, plus the reference test-script's crop
+identities and size-independent properties at the benchmark's full sizes."""
+import math
+
+import pytest
+import torch
+
+from parity import BWD_TOL, FWD_TOL, assert_close, rel_err
+import workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.float16, torch.bfloat16, torch.float64]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import medvision_amd.ops as ops_
+    from medvision_amd import _lib
+    _lib.load()
+    return ops_
+
+
+def _random_case(ndim, rotated, seed, R=12):
+    g = wl.gen(seed)
+    size = (9, 12, 14)[3 - ndim:]
+    feat = torch.randn(2, 5, *size, generator=g)
+    ext = torch.tensor(size[::-1], dtype=torch.float32)
+    cols = {(2, False): 5, (3, False): 7, (2, True): 6, (3, True): 10}[(ndim, rotated)]
+    rois = torch.zeros(R, cols)
+    rois[:, 0] = torch.randint(0, 2, (R,), generator=g)
+    if rotated:
+        rois[:, 1:1 + ndim] = torch.rand(R, ndim, generator=g) * ext * 2.0
+        rois[:, 1 + ndim:1 + 2 * ndim] = (torch.rand(R, ndim, generator=g) * 0.9 + 0.05) * ext * 2.4
+        rois[:, 1 + 2 * ndim:] = (torch.rand(R, cols - 1 - 2 * ndim, generator=g) - 0.5) * 2.0
+        rois[0, 1 + ndim:1 + 2 * ndim] = 0.3
+    else:
+        lo = (torch.rand(R, ndim, generator=g) * 1.2 - 0.2) * ext * 2.0
+        rois[:, 1:1 + ndim] = lo
+        rois[:, 1 + ndim:] = lo + torch.rand(R, ndim, generator=g) * ext * 1.6
+        rois[0, 1 + ndim:] = rois[0, 1:1 + ndim] + 0.4
+    return feat, rois
+
+
+def _module(ops, ndim, rotated, out_size, scale, sr, aligned):
+    if rotated:
+        return ops.RoIAlignRotated(out_size, scale, sr, aligned)
+    return ops.RoIAlign(out_size, scale, sr)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("ndim,rotated", [(2, False), (3, False), (2, True), (3, True)])
+@pytest.mark.parametrize("sr,aligned,order", [(2, True, 1), (0, False, 1), (1, True, 0), (-1, True, 1)])
+def test_forward_backward_vs_oracle(ops, oracle, dtype, ndim, rotated, sr, aligned, order):
+    feat, rois = _random_case(ndim, rotated, seed=100 * ndim + 10 * rotated + sr + 3)
+    feat = feat.to(dtype)
+    out_size = (3, 4, 5)[3 - ndim:]
+    mod = _module(ops, ndim, rotated, out_size, 0.5, sr, aligned)
+    fg = feat.to(DEV).requires_grad_(True)
+    out = mod(fg, rois.to(DEV), order=order)
+    eff_sr = 1 if order == 0 else sr
+    want = oracle.roi_align_forward(feat, rois, out_size, 0.5, eff_sr, aligned, order, rotated)
+    assert out.dtype == dtype and out.shape == want.shape
+    assert_close(out, want, FWD_TOL[dtype], "forward")
+    gy = torch.randn(out.shape, generator=wl.gen(7)).to(dtype)
+    out.backward(gy.to(DEV))
+    gwant = oracle.roi_align_backward(gy, rois, feat.shape, 0.5, eff_sr, aligned, order, rotated)
+    assert fg.grad.dtype == dtype
+    assert_close(fg.grad, gwant, BWD_TOL[dtype], "backward")
+
+
+def test_reference_crop_identities(ops):
+    """Known answers of the reference's own script (test/ops_test_RoIAlign.py:68,86,121,124,131)."""
+    g = wl.gen(0)
+    img = torch.randn(2, 1, 400, 440, generator=g).to(DEV)
+    rois = torch.tensor([[0, 161.5, 111.5, 417.5, 367.5]] * 3).to(DEV)
+    out = ops.RoIAlign((256, 256), 1.0, 1)(img, rois)
+    assert torch.equal(out[2, 0], img[0, 0, 112:368, 162:418])
+    out = ops.RoIAlign((256, 256), 1.0, 1)(img.half(), rois.half())   # the script runs in fp16
+    assert torch.equal(out[0, 0], img.half()[0, 0, 112:368, 162:418])
+    rr = torch.tensor([[0, 290., 240., 256., 256., 0.0]]).to(DEV)
+    out = ops.RoIAlignRotated((256, 256), 1.0, 1)(img, rr)
+    assert torch.equal(out[0, 0], img[0, 0, 112:368, 162:418])
+    vol = torch.randn(1, 1, 95, 192, 190, generator=g).to(DEV)
+    r3 = torch.tensor([[0, 9.5, 9.5, 59.5, 187.5, 187.5, 89.5]]).to(DEV)
+    out = ops.RoIAlign((30, 178, 178), 1.0, 1)(vol, r3)
+    assert torch.equal(out[0, 0], vol[0, 0, 60:90, 10:188, 10:188])
+    rr3 = torch.tensor([[0, 99., 99., 75., 178, 178, 30, 0, 0, 0]]).to(DEV)
+    for order in (0, 1):
+        out = ops.RoIAlignRotated((30, 178, 178), 1.0, 1)(vol, rr3, order=order)
+        assert torch.equal(out[0, 0], vol[0, 0, 60:90, 10:188, 10:188])
+
+
+def test_edge_cases_and_errors(ops):
+    feat = torch.randn(2, 3, 6, 7, 8, device=DEV)
+    empty = ops.RoIAlignRotated((2, 2, 2), 1.0, 2)(feat, torch.zeros(0, 10, device=DEV))
+    assert empty.shape == (0, 3, 2, 2, 2)
+    # batch index outside [0, N): zeros instead of an out-of-bounds read
+    bad = torch.tensor([[5, 4., 3., 3., 4., 4., 4., 0, 0, 0], [-1, 4., 3., 3., 4., 4., 4., 0, 0, 0]], device=DEV)
+    assert float(ops.RoIAlignRotated((2, 2, 2), 1.0, 2)(feat, bad).abs().max()) == 0.0
+    with pytest.raises(RuntimeError, match="size_rois should be 10"):
+        ops.RoIAlignRotated((2, 2, 2), 1.0, 2)(feat, torch.zeros(1, 7, device=DEV))
+    with pytest.raises(RuntimeError, match="size_rois should be 7"):
+        ops.RoIAlign((2, 2, 2), 1.0, 2)(feat, torch.zeros(1, 10, device=DEV))
+    with pytest.raises(RuntimeError, match="size_rois should be 5"):
+        ops.RoIAlign((2, 2), 1.0, 2)(feat[:, :, 0], torch.zeros(1, 7, device=DEV))
+    with pytest.raises(RuntimeError, match="not implemented on CPU"):
+        ops.RoIAlign((2, 2, 2), 1.0, 2)(feat.cpu(), torch.zeros(1, 7))
+    with pytest.raises(AssertionError):
+        ops.RoIAlign((2, 2, 2), 1.0, 2)(feat, torch.zeros(1, 7, device=DEV), order=3)
+    # non-contiguous features are accepted (made contiguous), result unchanged
+    r = torch.tensor([[1, 1., 1., 1., 6., 5., 4.]], device=DEV)
+    a = ops.RoIAlign((2, 2, 2), 1.0, 2)(feat, r)
+    b = ops.RoIAlign((2, 2, 2), 1.0, 2)(feat.transpose(3, 4).contiguous().transpose(3, 4), r)
+    assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_config2_affine_resampling_full_size(ops, oracle, dtype):
+    """BASELINE config 2: [4,1,128^3] -> 128^3, one rotated full-volume roi per sample, sr=1."""
+    g = wl.gen(1)
+    vol = torch.randn(4, 1, 128, 128, 128, generator=g).to(dtype)
+    rois = wl.affine_rois(g, 4, (128, 128, 128))
+    got = ops.affine_3d(vol.to(DEV), rois.to(DEV), (128, 128, 128), 1.0, 1, True, 1)
+    want = oracle.roi_align_forward(vol, rois, (128, 128, 128), 1.0, 1, True, 1, True)
+    assert_close(got, want, FWD_TOL[dtype], "config 2 forward")
+    same = ops.RoIAlignRotated((128, 128, 128), 1.0, 1, True)(vol.to(DEV), rois.to(DEV))
+    assert torch.equal(same, got)
+    # identity roi -> exact copy; nearest on the identity roi too
+    ident = torch.tensor([[b, 64, 64, 64, 128, 128, 128, 0, 0, 0] for b in range(4)], dtype=torch.float32)
+    for order in (0, 1):
+        out = ops.affine_3d(vol.to(DEV), ident.to(DEV), (128, 128, 128), 1.0, 1, True, order)
+        assert torch.equal(out.cpu(), vol)
+    # nearest under rotation: every output is one of the input values of its sample or 0
+    out0 = ops.affine_3d(vol.to(DEV), rois.to(DEV), (128, 128, 128), 1.0, 1, True, 0)
+    want0 = oracle.roi_align_forward(vol, rois, (128, 128, 128), 1.0, 1, True, 0, True)
+    mism = (out0.cpu().double() != want0).float().mean()
+    assert float(mism) < 1e-6, f"nearest mismatches: {float(mism):.2e}"
+
+
+def test_config2_backward_adjoint_full_size(ops, oracle):
+    g = wl.gen(11)
+    vol = torch.randn(4, 1, 128, 128, 128, generator=g)
+    rois = wl.affine_rois(g, 4, (128, 128, 128))
+    x = vol.to(DEV).requires_grad_(True)
+    y = ops.RoIAlignRotated((128, 128, 128), 1.0, 1, True)(x, rois.to(DEV))
+    gy = torch.randn(y.shape, generator=g)
+    y.backward(gy.to(DEV))
+    lhs = float((y.detach().double() * gy.to(DEV).double()).sum())
+    rhs = float((x.detach().double() * x.grad.double()).sum())
+    assert abs(lhs - rhs) <= 1e-5 * max(abs(lhs), 1.0)
+    gwant = oracle.roi_align_backward(gy, rois, vol.shape, 1.0, 1, True, 1, True)
+    assert_close(x.grad, gwant, BWD_TOL[torch.float32], "config 2 backward")
+
+
+def test_config3_resize_and_crops(ops, oracle):
+    """BASELINE config 3 at reduced size: CT-like fp16 volume, resize then rotated 3-D crops."""
+    g = wl.gen(2)
+    vol = wl.ct_like(g, (2, 1, 64, 128, 128))
+    full = torch.tensor([[b, 64, 64, 32, 128, 128, 64, 0, 0, 0] for b in range(2)], dtype=torch.float32)
+    small = ops.affine_3d(vol.to(DEV), full.to(DEV), (40, 64, 64), 1.0, 1, True, 1)
+    want = oracle.roi_align_forward(vol, full, (40, 64, 64), 1.0, 1, True, 1, True)
+    assert_close(small, want, FWD_TOL[torch.float16], "resize")
+    crops = []
+    for b in range(2):
+        for _ in range(8):
+            c = torch.rand(3, generator=g) * torch.tensor([64 - 24., 64 - 24., 40 - 24.]) + 12
+            ang = (float(torch.rand(1, generator=g)) * 2 - 1) * math.radians(15)
+            crops.append([b, *c.tolist(), 24, 24, 24, 0, 0, ang])
+    crops = torch.tensor(crops)
+    got = ops.affine_3d(small, crops.to(DEV), (24, 24, 24), 1.0, 1, True, 1)
+    want = oracle.roi_align_forward(small, crops, (24, 24, 24), 1.0, 1, True, 1, True)
+    assert_close(got, want, FWD_TOL[torch.float16], "crops")
+    # segmentation-style call: nearest, values stay in the input's value set
+    seg = (vol > 0).to(torch.float16)
+    got = ops.affine_3d(seg.to(DEV), crops.to(DEV), (24, 24, 24), 1.0, 1, True, 0)
+    assert set(got.unique().tolist()) <= {0.0, 1.0}
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_config5_detection_head_reduced(ops, oracle, dtype):
+    """BASELINE config 5 shape family (log-uniform extents, scale 0.25, 7^3, sr=2), reduced."""
+    g = wl.gen(4)
+    feat = torch.randn(2, 16, 12, 48, 48, generator=g).to(dtype)
+    rois = wl.roi3d_detection(g, 200, 2, (192, 192, 48), (2.0, 48.0), log_uniform=True)
+    x = feat.to(DEV).requires_grad_(True)
+    out = ops.RoIAlign((7, 7, 7), 0.25, 2)(x, rois.to(DEV))
+    want = oracle.roi_align_forward(feat, rois, (7, 7, 7), 0.25, 2)
+    assert_close(out, want, FWD_TOL[dtype], "forward")
+    gy = torch.randn(out.shape, generator=g).to(dtype)
+    out.backward(gy.to(DEV))
+    gwant = oracle.roi_align_backward(gy, rois, feat.shape, 0.25, 2)
+    assert_close(x.grad, gwant, BWD_TOL[dtype], "backward")
+
+
+def test_config1_rois_on_gpu(ops, oracle):
+    """BASELINE config 1 inputs (fp32 [2,16,32,64,64], 128 rois, 7^3, sr=2) through RoIAlign3D."""
+    g = wl.gen(0)
+    feat = torch.randn(2, 16, 32, 64, 64, generator=g)
+    rois = wl.roi3d_detection(g, 128, 2, (64, 64, 32), (4.0, 24.0))
+    out = ops.RoIAlign((7, 7, 7), 1.0, 2)(feat.to(DEV), rois.to(DEV))
+    want = oracle.roi_align_forward(feat, rois, (7, 7, 7), 1.0, 2)
+    assert_close(out, want, FWD_TOL[torch.float32], "config 1")
+
+
+def test_non_default_stream_and_determinism(ops):
+    g = wl.gen(3)
+    vol = torch.randn(1, 2, 32, 32, 32, generator=g).to(DEV)
+    rois = wl.affine_rois(g, 1, (32, 32, 32)).to(DEV)
+    ref = ops.affine_3d(vol, rois, (32, 32, 32), 1.0, 2, True, 1)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        again = ops.affine_3d(vol, rois, (32, 32, 32), 1.0, 2, True, 1)
+    s.synchronize()
+    assert torch.equal(ref, again)
