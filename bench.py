@@ -1,0 +1,157 @@
+#!/usr/bin/env python
+"""Benchmark of the trilinear-sampling hot path on one MI355X.
+
+A "step" is one RoIAlignRotated3D forward over one batch of BASELINE config 2 (fp16 volume
+[4,1,128^3] -> 128^3, one rotated full-volume roi per sample, sampling_ratio 1), inputs resident in
+HBM.  ``value`` is output Gvox/s.  Inputs/outputs rotate over ``--copies`` buffer sets (default 16,
+~540 MB) so that consecutive steps are not served from the 256 MB Infinity Cache.  The same JSON
+line carries the roofline of that kernel, the DCNv2-3D forward figure of config 4 (``dcn``) and the
+CPU baseline (the fp64 oracle timed on the host cores, bounded sample).
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
+MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense fp16/bf16
+
+
+def _events_ms(fn, steps, warmup):
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(steps):
+        fn(i)
+    stop.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return start.elapsed_time(stop) / steps, wall_ms / steps
+
+
+def bench_affine(args, dtype=torch.float16):
+    import medvision_amd.ops as ops
+    import workloads as wl
+    dev = "cuda:0"
+    g = wl.gen(1)
+    B, S = 4, 128
+    vols = [torch.randn(B, 1, S, S, S, generator=g).to(dtype).to(dev) for _ in range(args.copies)]
+    rois = [wl.affine_rois(g, B, (S, S, S)).to(dev) for _ in range(args.copies)]
+    outs = [torch.empty(B, 1, S, S, S, dtype=dtype, device=dev) for _ in range(args.copies)]
+    from medvision_amd import _C
+
+    def step(i):
+        j = i % args.copies
+        _C.roi_align_rotated_3d_forward(vols[j], rois[j], outs[j], S, S, S, 1.0, 1, True, 1)
+
+    ms, wall_ms = _events_ms(step, args.steps, args.warmup)
+    vox = B * S ** 3
+    esz = torch.finfo(dtype).bits // 8
+    alg_bytes = 2 * vox * esz            # read every input voxel once + write every output voxel
+    return {"ms": ms, "wall_ms": wall_ms, "gvox_s": vox / ms / 1e6, "gbps": alg_bytes / ms / 1e6,
+            "alg_bytes": alg_bytes, "vox": vox}
+
+
+def bench_dcn(args, dtype=torch.float16):
+    import workloads as wl
+    from medvision_amd.ops.modulated_deform_conv_3d import modulated_deform_conv
+    dev = "cuda:0"
+    g = wl.gen(3)
+    x, off, mask, w, b = [t.to(dev) for t in wl.dcn_inputs(g, 2, 32, 64, (48, 48, 48), 3, 1, 1, dtype)]
+
+    def step(i):
+        with torch.no_grad():
+            modulated_deform_conv(x, off, mask, w, b, 1, 1, 1, 1, 1)
+
+    ms, _ = _events_ms(step, max(3, args.steps // 10), max(1, args.warmup // 5))
+    flops = 2 * 2 * 64 * 32 * 27 * 48 ** 3
+    return {"ms": ms, "tflops": flops / ms / 1e9, "flops": flops}
+
+
+def cpu_baseline(args):
+    """fp64 oracle (C, OpenMP) on the benchmark's config-2 inputs: 2 of the 4 samples, median of 3."""
+    import oracle
+    import workloads as wl
+    oracle.build()
+    cores = min(os.cpu_count() or 1, 16)
+    oracle.set_threads(cores)
+    g = wl.gen(1)
+    B, S = 2, 128
+    vol = torch.randn(B, 1, S, S, S, generator=g).half()
+    rois = wl.affine_rois(g, B, (S, S, S))
+    times = []
+    for _ in range(4):
+        t0 = time.perf_counter()
+        oracle.roi_align_forward(vol, rois, (S, S, S), 1.0, 1, True, 1, True)
+        times.append(time.perf_counter() - t0)
+    t = sorted(times[1:])[1]
+    return {"value": B * S ** 3 / t / 1e9, "unit": "Gvox/s", "cores": cores, "kind": "port",
+            "sample": f"{B} of 4 samples of config 2 (fp16 [.,1,128^3] -> 128^3), fp64 oracle, "
+                      f"median of 3 after 1 warm-up, {t * 1e3:.0f} ms"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--copies", type=int, default=16)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-dcn", action="store_true", help="skip the DCN leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    from medvision_amd import _lib
+    _lib.load()
+
+    a16 = bench_affine(args, torch.float16)
+    a32 = bench_affine(args, torch.float32)
+    line = {
+        "metric": "RoIAlignRotated3D output throughput (fp16 [4,1,128^3] -> 128^3, sr=1)",
+        "value": round(a16["gvox_s"], 3), "unit": "Gvox/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(a16["ms"], 6), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16 storage, f32 interpolation, f64 coordinates",
+        "data": "synthetic",
+        "config": {"workload": "BASELINE config 2: RoIAlignRotated3D as RandomAffine resampling, "
+                               "volume fp16 [4,1,128,128,128] N(0,1), one full-volume roi per sample, "
+                               "angles U(+-30deg), scale U(0.8,1.2), shift +-10 vox, out 128^3, "
+                               "sampling_ratio 1, aligned, order 1",
+                   "buffer_sets": args.copies},
+        "roofline": {"bound": "hbm", "achieved": round(a16["gbps"], 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(a16["gbps"] / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "roi_forward", "algorithmic_bytes_per_launch": a16["alg_bytes"],
+                     "avg_launch_us": round(a16["ms"] * 1e3, 3)},
+        "fp32": {"gvox_s": round(a32["gvox_s"], 3), "gbps": round(a32["gbps"], 1),
+                 "ms_per_step": round(a32["ms"], 6),
+                 "frac": round(a32["gbps"] / HBM_PEAK_GBPS, 4)},
+    }
+    if not args.no_dcn:
+        d = bench_dcn(args)
+        line["dcn"] = {"metric": "DCNv2-3D forward (fp16 [2,32,48^3], 3^3, Cout 64)",
+                       "value": round(d["tflops"], 3), "unit": "TFLOP/s",
+                       "ms_per_step": round(d["ms"], 6),
+                       "roofline": {"bound": "mfma", "achieved": round(d["tflops"], 3),
+                                    "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                    "frac": round(d["tflops"] / MFMA_F16_PEAK_TFLOPS, 5),
+                                    "traffic": None, "flops_per_launch": d["flops"]}}
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(args)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
