@@ -1,13 +1,263 @@
 // Matrix-core (MFMA) forward of the 3-D deformable convolution for fp16 / bf16 tensors.
+//
+//   y[b, o, q] = sum_{k, c} Wt[o, c, k] * col[c, k, q] + bias[o],
+//   col[c, k, q] = mask[k, q] * Z(x[b, c], p(k, q))           (zero-padded trilinear sample)
+//
+// is a GEMM whose B operand (the column matrix, Cin*K x positions) is never written to memory:
+// every wavefront owns 32 output positions and builds the 16 x 32 B fragment of one (tap, 16
+// channel) slice directly in registers, then issues v_mfma_f32_32x32x16_{f16,bf16} against the
+// weight fragments of up to MT 32-row blocks of output channels, accumulating in fp32.
+//
+// Data layout chosen for the gather, not for the GEMM:
+//   * x is first transposed to channels-last [B, D*H*W, Cin] (workspace).  The MFMA B fragment
+//     gives lane l the 8 consecutive K rows (l / 32) * 8 .. + 7 of column l % 32, so with
+//     channels-last storage ONE 16-byte load per trilinear corner brings exactly the 8 channels a
+//     lane needs: 8 loads + 64 mixed-precision FMAs per lane produce its part of the fragment;
+//   * the 8 corner offsets / weights (x mask) of a (tap, position) are computed once per lane and
+//     reused for every channel slice of the deformable group (positions are exact in fp32 for
+//     16-bit offsets);
+//   * weights are re-laid out once per call into A-fragment order [group][tap][slice][row block]
+//     [lane][8] (workspace) so that a fragment is one coalesced 16-byte load per lane (L2 hits).
+// The sampling gather, not the matrix core, bounds this kernel: per (tap, position) 8 corners x
+// Cin channels are fetched, 8 x more bytes than the fragment holds.
 #include "dcn_common.hpp"
 
 namespace mv {
 
-bool dcn_mfma_supported(const DcnDims &, int) { return false; }
-size_t dcn_mfma_workspace_bytes(const DcnDims &, int) { return 0; }
-int dcn_mfma_forward(const void *, const void *, const void *, const void *, const void *, void *,
-                     const DcnDims &, int, void *, hipStream_t) {
-  return fail(MV_INVALID_ARGUMENT, "matrix-core DCN forward is not available for this shape");
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+template <typename T> struct Mfma;
+template <> struct Mfma<__half> {
+  using frag = half8_t;
+  static __device__ __forceinline__ float16_t run(frag a, frag b, float16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float lo(unsigned w) {
+    return __half2float(__ushort_as_half(static_cast<unsigned short>(w & 0xffffu)));
+  }
+  static __device__ __forceinline__ float hi(unsigned w) {
+    return __half2float(__ushort_as_half(static_cast<unsigned short>(w >> 16)));
+  }
+  static __device__ __forceinline__ unsigned pack(float a, float b) {
+    return static_cast<unsigned>(__half_as_ushort(__float2half_rn(a))) |
+           (static_cast<unsigned>(__half_as_ushort(__float2half_rn(b))) << 16);
+  }
+};
+template <> struct Mfma<__hip_bfloat16> {
+  using frag = bf16x8_t;
+  static __device__ __forceinline__ float16_t run(frag a, frag b, float16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float lo(unsigned w) { return __uint_as_float(w << 16); }
+  static __device__ __forceinline__ float hi(unsigned w) { return __uint_as_float(w & 0xffff0000u); }
+  static __device__ __forceinline__ unsigned pack(float a, float b) {
+    // round to nearest even on the upper 16 bits
+    const unsigned ua = __float_as_uint(a), ub = __float_as_uint(b);
+    const unsigned ra = (ua + 0x7fffu + ((ua >> 16) & 1u)) >> 16;
+    const unsigned rb = (ub + 0x7fffu + ((ub >> 16) & 1u)) & 0xffff0000u;
+    return ra | rb;
+  }
+};
+
+// x [B, Cin, P] -> xt [B, P, Cin]; one workgroup moves 64 positions of all channels through LDS
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_channels_last_kernel(const T *__restrict__ x,
+                                                                T *__restrict__ xt, int Cin,
+                                                                long P) {
+  extern __shared__ unsigned short stage[];  // [64][Cin + 2]
+  const int b = blockIdx.y;
+  const long p0 = static_cast<long>(blockIdx.x) * 64;
+  const int pitch = Cin + 2;
+  const unsigned short *src = reinterpret_cast<const unsigned short *>(x) + static_cast<long>(b) * Cin * P;
+  unsigned short *dst = reinterpret_cast<unsigned short *>(xt) + (static_cast<long>(b) * P + p0) * Cin;
+  const int lp = threadIdx.x % 64;
+  for (int c = threadIdx.x / 64; c < Cin; c += 4)
+    if (p0 + lp < P) stage[lp * pitch + c] = src[static_cast<long>(c) * P + p0 + lp];
+  __syncthreads();
+  const long count = min(static_cast<long>(64), P - p0) * Cin;
+  for (long i = threadIdx.x; i < count; i += 256) {
+    const int pp = static_cast<int>(i / Cin), c = static_cast<int>(i % Cin);
+    dst[i] = stage[pp * pitch + c];
+  }
+}
+
+// weight [Cout, cpg, K] -> A fragments [group][tap][slice][row block][lane][8]
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_weight_fragments_kernel(const T *__restrict__ wt,
+                                                                   T *__restrict__ wf,
+                                                                   const DcnDims s) {
+  const int slices = s.cpg / 16, blocks = s.opg / 32;
+  const long total = static_cast<long>(s.groups) * s.K * slices * blocks * 64;
+  const long id = blockIdx.x * 256L + threadIdx.x;
+  if (id >= total) return;
+  const int lane = id % 64;
+  long r = id / 64;
+  const int mb = r % blocks; r /= blocks;
+  const int cc = r % slices; r /= slices;
+  const int k = r % s.K;
+  const int g = static_cast<int>(r / s.K);
+  const int o = g * s.opg + mb * 32 + lane % 32;
+  const int cl = cc * 16 + (lane / 32) * 8;
+  for (int i = 0; i < 8; i++) wf[id * 8 + i] = wt[(static_cast<long>(o) * s.cpg + cl + i) * s.K + k];
+}
+
+template <typename T, int MT>
+__global__ __launch_bounds__(256) void dcn_forward_mfma_kernel(
+    const T *__restrict__ xt, const T *__restrict__ off, const T *__restrict__ mask,
+    const T *__restrict__ wf, const T *__restrict__ bias, T *__restrict__ y, const DcnDims s) {
+  using M = Mfma<T>;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int n = lane % 32, h = lane / 32;
+  const long q0 = (static_cast<long>(blockIdx.x) * 4 + wave) * 32;
+  if (q0 >= s.Q) return;  // whole wave idle (no barriers in this kernel)
+  const long q = q0 + n;
+  const bool live = q < s.Q;
+  const long qc = live ? q : s.Q - 1;
+  const int slices = s.cpg / 16, blocks = s.opg / 32;
+  const int chunks = (blocks + MT - 1) / MT;
+  const int g = blockIdx.y / chunks, mb0 = (blockIdx.y % chunks) * MT;
+  const int b = blockIdx.z;
+  const int ow = qc % s.Wo, oh = (qc / s.Wo) % s.Ho, od = qc / (static_cast<long>(s.Wo) * s.Ho);
+  const int bd = od * s.sd - s.pd, bh = oh * s.sh - s.ph, bw = ow * s.sw - s.pw;
+  const T *xb = xt + static_cast<long>(b) * s.P * s.Cin;
+
+  float16_t acc[MT];
+#pragma unroll
+  for (int m = 0; m < MT; m++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[m][r] = 0.f;
+
+  for (int k = 0; k < s.K; k++) {
+    const int ki = k / (s.kh * s.kw), kj = (k / s.kw) % s.kh, kk = k % s.kw;
+    int prev_dgi = -1;
+    int coff[8];
+    float cw[8];
+    for (int cc = 0; cc < slices; cc++) {
+      const int c0 = g * s.cpg + cc * 16;
+      const int dgi = c0 / s.cpd;
+      if (dgi != prev_dgi) {
+        prev_dgi = dgi;
+        const long bg = static_cast<long>(b) * s.dg + dgi;
+        const T *o = off + (bg * 3 * s.K + 3 * k) * s.Q + qc;
+        const float pd = static_cast<float>(bd + ki * s.dd) + load(o);
+        const float ph = static_cast<float>(bh + kj * s.dh) + load(o + s.Q);
+        const float pw = static_cast<float>(bw + kk * s.dw) + load(o + 2 * s.Q);
+        const float m = mask ? load(mask + (bg * s.K + k) * s.Q + qc) : 1.f;
+        const bool ok = pd > -1.f && ph > -1.f && pw > -1.f && pd < s.D && ph < s.H && pw < s.W;
+        const float fd = floorf(pd), fh = floorf(ph), fw = floorf(pw);
+        const int d0 = static_cast<int>(fd), h0 = static_cast<int>(fh), w0 = static_cast<int>(fw);
+        const float ld = pd - fd, lh = ph - fh, lw = pw - fw;
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+          const int a = c >> 2, bb = (c >> 1) & 1, e = c & 1;
+          const int zd = d0 + a, zh = h0 + bb, zw = w0 + e;
+          const bool in = ok && zd >= 0 && zd < s.D && zh >= 0 && zh < s.H && zw >= 0 && zw < s.W;
+          coff[c] = in ? (zd * s.H + zh) * s.W + zw : -1;
+          cw[c] = m * (a ? ld : 1.f - ld) * (bb ? lh : 1.f - lh) * (e ? lw : 1.f - lw);
+        }
+      }
+      // this lane's 8 channels of the slice: c0 + h*8 .. + 7
+      float v[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) v[i] = 0.f;
+      uint4 raw[8];
+#pragma unroll
+      for (int c = 0; c < 8; c++) {
+        raw[c] = make_uint4(0u, 0u, 0u, 0u);
+        if (coff[c] >= 0)
+          raw[c] = *reinterpret_cast<const uint4 *>(xb + static_cast<long>(coff[c]) * s.Cin + c0 + h * 8);
+      }
+#pragma unroll
+      for (int c = 0; c < 8; c++) {
+        const float w = cw[c];
+        v[0] += w * M::lo(raw[c].x); v[1] += w * M::hi(raw[c].x);
+        v[2] += w * M::lo(raw[c].y); v[3] += w * M::hi(raw[c].y);
+        v[4] += w * M::lo(raw[c].z); v[5] += w * M::hi(raw[c].z);
+        v[6] += w * M::lo(raw[c].w); v[7] += w * M::hi(raw[c].w);
+      }
+      union { uint4 u; typename M::frag f; } bfrag;
+      bfrag.u = make_uint4(M::pack(v[0], v[1]), M::pack(v[2], v[3]), M::pack(v[4], v[5]), M::pack(v[6], v[7]));
+      const T *wfk = wf + ((((static_cast<long>(g) * s.K + k) * slices + cc) * blocks + mb0) * 64 + lane) * 8;
+#pragma unroll
+      for (int m = 0; m < MT; m++) {
+        if (mb0 + m < blocks) {
+          union { uint4 u; typename M::frag f; } afrag;
+          afrag.u = *reinterpret_cast<const uint4 *>(wfk + static_cast<long>(m) * 64 * 8);
+          acc[m] = M::run(afrag.f, bfrag.f, acc[m]);
+        }
+      }
+    }
+  }
+  if (!live) return;
+#pragma unroll
+  for (int m = 0; m < MT; m++) {
+    if (mb0 + m >= blocks) continue;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      // 32x32 accumulator layout: register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32
+      const int o = g * s.opg + (mb0 + m) * 32 + (r / 4) * 8 + h * 4 + (r % 4);
+      const float val = acc[m][r] + (bias ? load(bias + o) : 0.f);
+      y[(static_cast<long>(b) * s.Cout + o) * s.Q + q] = store_cast<T>(val);
+    }
+  }
+}
+
+static size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+
+bool dcn_mfma_supported(const DcnDims &s, int dtype) {
+  if (dtype != MV_F16 && dtype != MV_BF16) return false;
+  if (s.cpg % 16 || s.opg % 32 || s.cpd % 16) return false;
+  if (s.Cin > 4096 || s.B > 65535) return false;
+  if (static_cast<long>(s.P) * s.Cin >= (1L << 40)) return false;
+  return true;
+}
+
+size_t dcn_mfma_workspace_bytes(const DcnDims &s, int dtype) {
+  (void)dtype;
+  const size_t xt = static_cast<size_t>(s.B) * s.P * s.Cin * 2;
+  const size_t wf = static_cast<size_t>(s.Cout) * s.cpg * s.K * 2;
+  return align256(xt) + align256(wf);
+}
+
+template <typename T>
+static int dcn_mfma_run(const void *x, const void *off, const void *mask, const void *wt,
+                        const void *bias, void *y, const DcnDims &s, void *workspace,
+                        hipStream_t stream) {
+  T *xt = static_cast<T *>(workspace);
+  T *wf = reinterpret_cast<T *>(static_cast<char *>(workspace) +
+                                align256(static_cast<size_t>(s.B) * s.P * s.Cin * 2));
+  const long pblocks = (s.P + 63) / 64;
+  MV_REQUIRE(pblocks < (1L << 31), "volume too large");
+  hipLaunchKernelGGL((dcn_channels_last_kernel<T>), dim3(static_cast<unsigned>(pblocks), s.B), dim3(256),
+                     64 * (s.Cin + 2) * sizeof(unsigned short), stream, static_cast<const T *>(x), xt,
+                     s.Cin, s.P);
+  const long frag_lanes = static_cast<long>(s.groups) * s.K * (s.cpg / 16) * (s.opg / 32) * 64;
+  hipLaunchKernelGGL((dcn_weight_fragments_kernel<T>), dim3(static_cast<unsigned>((frag_lanes + 255) / 256)),
+                     dim3(256), 0, stream, static_cast<const T *>(wt), wf, s);
+  const int blocks = s.opg / 32;
+  const int mt = blocks >= 4 ? 4 : (blocks >= 2 ? 2 : 1);
+  const int chunks = (blocks + mt - 1) / mt;
+  const long qblocks = (s.Q + 127) / 128;
+  MV_REQUIRE(qblocks < (1L << 31) && static_cast<long>(s.groups) * chunks <= 65535, "grid too large");
+  const dim3 grid(static_cast<unsigned>(qblocks), s.groups * chunks, s.B), block(256);
+#define MV_LAUNCH_MFMA(MTV)                                                                      \
+  hipLaunchKernelGGL((dcn_forward_mfma_kernel<T, MTV>), grid, block, 0, stream, xt,              \
+                     static_cast<const T *>(off), static_cast<const T *>(mask), wf,              \
+                     static_cast<const T *>(bias), static_cast<T *>(y), s)
+  if (mt == 4) MV_LAUNCH_MFMA(4);
+  else if (mt == 2) MV_LAUNCH_MFMA(2);
+  else MV_LAUNCH_MFMA(1);
+#undef MV_LAUNCH_MFMA
+  return check_launch("dcn_forward_mfma_kernel");
+}
+
+int dcn_mfma_forward(const void *x, const void *off, const void *mask, const void *wt,
+                     const void *bias, void *y, const DcnDims &s, int dtype, void *workspace,
+                     hipStream_t stream) {
+  if (dtype == MV_F16) return dcn_mfma_run<__half>(x, off, mask, wt, bias, y, s, workspace, stream);
+  return dcn_mfma_run<__hip_bfloat16>(x, off, mask, wt, bias, y, s, workspace, stream);
 }
 
 }  // namespace mv

@@ -66,6 +66,26 @@ def test_config4_reduced_vs_oracle(ops, oracle, dtype):
     assert_close(y, want, FWD_TOL[dtype], "config 4 forward")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("modulated,groups,dg,stride,pad,dil,cin,cout", [
+    (True, 2, 2, 1, 1, 1, 64, 128), (False, 1, 2, 2, 1, 2, 32, 32), (True, 1, 1, 1, 0, 1, 16, 160)])
+def test_matrix_core_path_vs_oracle(ops, oracle, dtype, modulated, groups, dg, stride, pad, dil, cin, cout):
+    """Shapes that take the MFMA forward (channels per group % 16 == 0, outputs per group % 32 == 0)
+    with groups, deformable groups, stride, dilation and a ragged last position tile."""
+    from medvision_amd.ops.deform_conv_3d import deform_conv
+    from medvision_amd.ops.modulated_deform_conv_3d import modulated_deform_conv
+    g = wl.gen(60 + groups + dg)
+    x, off, mask, w, b = wl.dcn_inputs(g, 2, cin, cout, (7, 9, 11), 3, dg, groups, dtype, stride, pad, dil,
+                                       modulated)
+    xs, offs, ms, ws, bs = _to(DEV, x, off, mask, w, b)
+    if modulated:
+        y = modulated_deform_conv(xs, offs, ms, ws, bs, stride, pad, dil, groups, dg)
+    else:
+        y = deform_conv(xs, offs, ws, bs, stride, pad, dil, groups, dg, 64)
+    want = oracle.dcn3d_forward(x, off, mask, w, b, stride, pad, dil, groups, dg)
+    assert_close(y, want, FWD_TOL[dtype], "mfma forward")
+
+
 def test_config4_full_size_properties(ops):
     """Full config-4 shape [2,32,48^3] -> Cout 64: zero offsets and unit mask reduce DCN to a plain
     convolution (checked against torch's conv3d), and the op is linear in the mask."""
