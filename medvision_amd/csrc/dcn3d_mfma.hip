@@ -129,63 +129,74 @@ __global__ __launch_bounds__(256) void dcn_forward_mfma_kernel(
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[m][r] = 0.f;
 
-  for (int k = 0; k < s.K; k++) {
-    const int ki = k / (s.kh * s.kw), kj = (k / s.kw) % s.kh, kk = k % s.kw;
-    int prev_dgi = -1;
-    int coff[8];
-    float cw[8];
-    for (int cc = 0; cc < slices; cc++) {
-      const int c0 = g * s.cpg + cc * 16;
-      const int dgi = c0 / s.cpd;
-      if (dgi != prev_dgi) {
-        prev_dgi = dgi;
-        const long bg = static_cast<long>(b) * s.dg + dgi;
-        const T *o = off + (bg * 3 * s.K + 3 * k) * s.Q + qc;
-        const float pd = static_cast<float>(bd + ki * s.dd) + load(o);
-        const float ph = static_cast<float>(bh + kj * s.dh) + load(o + s.Q);
-        const float pw = static_cast<float>(bw + kk * s.dw) + load(o + 2 * s.Q);
-        const float m = mask ? load(mask + (bg * s.K + k) * s.Q + qc) : 1.f;
-        const bool ok = pd > -1.f && ph > -1.f && pw > -1.f && pd < s.D && ph < s.H && pw < s.W;
-        const float fd = floorf(pd), fh = floorf(ph), fw = floorf(pw);
-        const int d0 = static_cast<int>(fd), h0 = static_cast<int>(fh), w0 = static_cast<int>(fw);
-        const float ld = pd - fd, lh = ph - fh, lw = pw - fw;
+  // deformable groups that intersect this convolution group's channels, and the 16-channel
+  // slices of each (cpd % 16 == 0, so a slice never straddles two deformable groups)
+  const int dg_first = g * s.cpg / s.cpd, dg_last = (g * s.cpg + s.cpg - 1) / s.cpd;
+  const unsigned cin = s.Cin;
+  const T *wfg = wf + ((static_cast<long>(g) * s.K * slices) * blocks + mb0) * 512 + lane * 8;
+  for (int dgi = dg_first; dgi <= dg_last; dgi++) {
+    const int c_lo = max(g * s.cpg, dgi * s.cpd), c_hi = min(g * s.cpg + s.cpg, (dgi + 1) * s.cpd);
+    const int cc_lo = (c_lo - g * s.cpg) / 16, cc_hi = (c_hi - g * s.cpg) / 16;
+    const long bg = static_cast<long>(b) * s.dg + dgi;
+    const T *o = off + bg * 3 * s.K * s.Q + qc;
+    const T *mk = mask ? mask + bg * s.K * s.Q + qc : nullptr;
+    int ki = 0, kj = 0, kk = 0;
+    for (int k = 0; k < s.K; k++) {
+      const float pd = static_cast<float>(bd + ki * s.dd) + load(o);
+      const float ph = static_cast<float>(bh + kj * s.dh) + load(o + s.Q);
+      const float pw = static_cast<float>(bw + kk * s.dw) + load(o + 2 * s.Q);
+      const float m = mk ? load(mk) : 1.f;
+      o += 3 * s.Q;
+      if (mk) mk += s.Q;
+      if (++kk == s.kw) { kk = 0; if (++kj == s.kh) { kj = 0; ++ki; } }
+      const bool ok = pd > -1.f && ph > -1.f && pw > -1.f && pd < s.D && ph < s.H && pw < s.W;
+      const float fd = floorf(pd), fh = floorf(ph), fw = floorf(pw);
+      const int d0 = static_cast<int>(fd), h0 = static_cast<int>(fh), w0 = static_cast<int>(fw);
+      const float ld = pd - fd, lh = ph - fh, lw = pw - fw;
+      unsigned coff[8];  // element offset of the corner's channel vector in xt, ~0u = outside
+      float cw[8];
+#pragma unroll
+      for (int c = 0; c < 8; c++) {
+        const int a = c >> 2, bb = (c >> 1) & 1, e = c & 1;
+        const int zd = d0 + a, zh = h0 + bb, zw = w0 + e;
+        const bool in = ok && zd >= 0 && zd < s.D && zh >= 0 && zh < s.H && zw >= 0 && zw < s.W;
+        coff[c] = in ? static_cast<unsigned>((zd * s.H + zh) * s.W + zw) * cin + h * 8 : ~0u;
+        cw[c] = m * (a ? ld : 1.f - ld) * (bb ? lh : 1.f - lh) * (e ? lw : 1.f - lw);
+      }
+      for (int cc = cc_lo; cc < cc_hi; cc++) {
+        const unsigned c0 = g * s.cpg + cc * 16;
+        // this lane's 8 channels of the slice: c0 + h*8 .. + 7
+        uint4 raw[8];
 #pragma unroll
         for (int c = 0; c < 8; c++) {
-          const int a = c >> 2, bb = (c >> 1) & 1, e = c & 1;
-          const int zd = d0 + a, zh = h0 + bb, zw = w0 + e;
-          const bool in = ok && zd >= 0 && zd < s.D && zh >= 0 && zh < s.H && zw >= 0 && zw < s.W;
-          coff[c] = in ? (zd * s.H + zh) * s.W + zw : -1;
-          cw[c] = m * (a ? ld : 1.f - ld) * (bb ? lh : 1.f - lh) * (e ? lw : 1.f - lw);
+          raw[c] = make_uint4(0u, 0u, 0u, 0u);
+          if (coff[c] != ~0u) raw[c] = *reinterpret_cast<const uint4 *>(xb + (coff[c] + c0));
         }
-      }
-      // this lane's 8 channels of the slice: c0 + h*8 .. + 7
-      float v[8];
+        const T *wfk = wfg + (static_cast<long>(k) * slices + cc) * blocks * 512;
+        uint4 araw[MT];
 #pragma unroll
-      for (int i = 0; i < 8; i++) v[i] = 0.f;
-      uint4 raw[8];
+        for (int mm = 0; mm < MT; mm++)
+          if (mb0 + mm < blocks) araw[mm] = *reinterpret_cast<const uint4 *>(wfk + mm * 512);
+        float v[8];
 #pragma unroll
-      for (int c = 0; c < 8; c++) {
-        raw[c] = make_uint4(0u, 0u, 0u, 0u);
-        if (coff[c] >= 0)
-          raw[c] = *reinterpret_cast<const uint4 *>(xb + static_cast<long>(coff[c]) * s.Cin + c0 + h * 8);
-      }
+        for (int i = 0; i < 8; i++) v[i] = 0.f;
 #pragma unroll
-      for (int c = 0; c < 8; c++) {
-        const float w = cw[c];
-        v[0] += w * M::lo(raw[c].x); v[1] += w * M::hi(raw[c].x);
-        v[2] += w * M::lo(raw[c].y); v[3] += w * M::hi(raw[c].y);
-        v[4] += w * M::lo(raw[c].z); v[5] += w * M::hi(raw[c].z);
-        v[6] += w * M::lo(raw[c].w); v[7] += w * M::hi(raw[c].w);
-      }
-      union { uint4 u; typename M::frag f; } bfrag;
-      bfrag.u = make_uint4(M::pack(v[0], v[1]), M::pack(v[2], v[3]), M::pack(v[4], v[5]), M::pack(v[6], v[7]));
-      const T *wfk = wf + ((((static_cast<long>(g) * s.K + k) * slices + cc) * blocks + mb0) * 64 + lane) * 8;
+        for (int c = 0; c < 8; c++) {
+          const float w = cw[c];
+          v[0] += w * M::lo(raw[c].x); v[1] += w * M::hi(raw[c].x);
+          v[2] += w * M::lo(raw[c].y); v[3] += w * M::hi(raw[c].y);
+          v[4] += w * M::lo(raw[c].z); v[5] += w * M::hi(raw[c].z);
+          v[6] += w * M::lo(raw[c].w); v[7] += w * M::hi(raw[c].w);
+        }
+        union { uint4 u; typename M::frag f; } bfrag;
+        bfrag.u = make_uint4(M::pack(v[0], v[1]), M::pack(v[2], v[3]), M::pack(v[4], v[5]), M::pack(v[6], v[7]));
 #pragma unroll
-      for (int m = 0; m < MT; m++) {
-        if (mb0 + m < blocks) {
-          union { uint4 u; typename M::frag f; } afrag;
-          afrag.u = *reinterpret_cast<const uint4 *>(wfk + static_cast<long>(m) * 64 * 8);
-          acc[m] = M::run(afrag.f, bfrag.f, acc[m]);
+        for (int mm = 0; mm < MT; mm++) {
+          if (mb0 + mm < blocks) {
+            union { uint4 u; typename M::frag f; } afrag;
+            afrag.u = araw[mm];
+            acc[mm] = M::run(afrag.f, bfrag.f, acc[mm]);
+          }
         }
       }
     }
@@ -210,7 +221,7 @@ bool dcn_mfma_supported(const DcnDims &s, int dtype) {
   if (dtype != MV_F16 && dtype != MV_BF16) return false;
   if (s.cpg % 16 || s.opg % 32 || s.cpd % 16) return false;
   if (s.Cin > 4096 || s.B > 65535) return false;
-  if (static_cast<long>(s.P) * s.Cin >= (1L << 40)) return false;
+  if (static_cast<long>(s.P) * s.Cin >= (1L << 31)) return false;  // 32-bit element offsets
   return true;
 }
 
