@@ -80,25 +80,74 @@ def bench_dcn(args, dtype=torch.float16):
 
 
 def cpu_baseline(args):
-    """fp64 oracle (C, OpenMP) on the benchmark's config-2 inputs: 2 of the 4 samples, median of 3."""
+    """fp64 oracle (C, OpenMP) on the benchmark's config-2 inputs (all 4 samples), repeated until
+    about 12 s of wall time have been spent; the median pass is reported."""
     import oracle
     import workloads as wl
     oracle.build()
     cores = min(os.cpu_count() or 1, 16)
     oracle.set_threads(cores)
     g = wl.gen(1)
-    B, S = 2, 128
+    B, S = 4, 128
     vol = torch.randn(B, 1, S, S, S, generator=g).half()
     rois = wl.affine_rois(g, B, (S, S, S))
-    times = []
-    for _ in range(4):
+    oracle.roi_align_forward(vol, rois, (S, S, S), 1.0, 1, True, 1, True)   # warm-up
+    times, t_start = [], time.perf_counter()
+    while time.perf_counter() - t_start < args.cpu_seconds and len(times) < 200:
         t0 = time.perf_counter()
         oracle.roi_align_forward(vol, rois, (S, S, S), 1.0, 1, True, 1, True)
         times.append(time.perf_counter() - t0)
-    t = sorted(times[1:])[1]
-    return {"value": B * S ** 3 / t / 1e9, "unit": "Gvox/s", "cores": cores, "kind": "port",
-            "sample": f"{B} of 4 samples of config 2 (fp16 [.,1,128^3] -> 128^3), fp64 oracle, "
-                      f"median of 3 after 1 warm-up, {t * 1e3:.0f} ms"}
+    t = sorted(times)[len(times) // 2]
+    return {"value": round(B * S ** 3 / t / 1e9, 4), "unit": "Gvox/s", "cores": cores, "kind": "port",
+            "sample": f"config 2 (fp16 [4,1,128^3] -> 128^3) through the fp64 C oracle, OpenMP x{cores}, "
+                      f"median of {len(times)} passes after 1 warm-up ({t * 1e3:.0f} ms per pass)"}
+
+
+def cpu_reference_paths(args):
+    """The reference's own CPU paths, restated (baseline only, no parity claim): the torch-function
+    RoIAlign on config 1 and the aug_cpu affine steps (scipy.ndimage) on one 128^3 volume."""
+    import numpy as np
+    import workloads as wl
+    from oracle.torchfun_roi_align import torchfun_roi_align
+    res = {"threads": torch.get_num_threads()}
+    g = wl.gen(0)
+    feat = torch.randn(2, 16, 32, 64, 64, generator=g)
+    rois = wl.roi3d_detection(g, 128, 2, (64, 64, 32), (4.0, 24.0))
+    torchfun_roi_align(feat, rois[:8], (7, 7, 7), 1.0)
+    ts = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        out = torchfun_roi_align(feat, rois, (7, 7, 7), 1.0)
+        ts.append(time.perf_counter() - t0)
+    t = sorted(ts)[1]
+    res["torchfun_roialign_config1"] = {"ms": round(t * 1e3, 2), "outputs_per_s": round(out.numel() / t, 1)}
+    try:
+        from scipy import ndimage as ndi
+        vol = np.random.default_rng(0).standard_normal((1, 128, 128, 128)).astype(np.float32)
+        steps = {
+            "rotate_order1": lambda: ndi.rotate(vol, 20.0, axes=(3, 2), reshape=False, order=1),
+            "shift_order1": lambda: ndi.shift(vol, (0, 5.5, -3.2, 7.1), order=1),
+            "zoom_order1": lambda: ndi.zoom(vol, (1, 1.1, 1.1, 1.1), order=1),
+            "resize_zoom_order2": lambda: ndi.zoom(vol, (1, 0.625, 0.5, 0.5), order=2),
+        }
+        for name, fn in steps.items():
+            t0 = time.perf_counter()
+            o = fn()
+            dt = time.perf_counter() - t0
+            res["scipy_" + name] = {"ms": round(dt * 1e3, 1), "gvox_s": round(o.size / dt / 1e9, 5)}
+    except Exception as e:  # scipy missing on the box
+        res["scipy"] = f"unavailable: {e}"
+    return res
+
+
+def copy_calibration(args):
+    """Plain device copy of known size, for scaling the FETCH_SIZE / WRITE_SIZE counters."""
+    n = 4 * 128 ** 3
+    src = [torch.randn(n, device="cuda:0").half() for _ in range(args.copies)]
+    dst = [torch.empty(n, dtype=torch.float16, device="cuda:0") for _ in range(args.copies)]
+    ms, _ = _events_ms(lambda i: dst[i % args.copies].copy_(src[i % args.copies]), args.steps, args.warmup)
+    print(json.dumps({"copy_bytes_read": 2 * n, "copy_bytes_written": 2 * n, "ms": ms,
+                      "gbps": 4 * n / ms / 1e6}))
 
 
 def main():
@@ -109,6 +158,9 @@ def main():
     ap.add_argument("--copies", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-dcn", action="store_true", help="skip the DCN leg")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="wall time spent on the CPU oracle")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run a device copy of 4*128^3 fp16 elements (counter calibration)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -116,6 +168,9 @@ def main():
         sys.exit("bench.py needs a GPU")
     from medvision_amd import _lib
     _lib.load()
+    if args.copy_calibration:
+        copy_calibration(args)
+        return
 
     a16 = bench_affine(args, torch.float16)
     a32 = bench_affine(args, torch.float32)
@@ -133,7 +188,7 @@ def main():
                    "buffer_sets": args.copies},
         "roofline": {"bound": "hbm", "achieved": round(a16["gbps"], 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(a16["gbps"] / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "roi_forward", "algorithmic_bytes_per_launch": a16["alg_bytes"],
+                     "kernel": "roi_plan_kernel + roi_resample_kernel", "algorithmic_bytes_per_launch": a16["alg_bytes"],
                      "avg_launch_us": round(a16["ms"] * 1e3, 3)},
         "fp32": {"gvox_s": round(a32["gvox_s"], 3), "gbps": round(a32["gbps"], 1),
                  "ms_per_step": round(a32["ms"], 6),
@@ -150,6 +205,10 @@ def main():
                                     "traffic": None, "flops_per_launch": d["flops"]}}
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(args)
+        line["cpu_reference_paths"] = cpu_reference_paths(args)
+    traffic = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(traffic):   # HBM bytes per launch measured with rocprofv3 --pmc (see profiles/)
+        line["roofline"]["traffic"] = json.load(open(traffic)).get("roi_resample_fp16_config2")
     print(json.dumps(line))
 
 
