@@ -118,6 +118,12 @@ __global__ void add_from_f32_kernel(T *dst, const float *src, long n) {
 int roi_forward_tiled(const void *input, const void *rois, void *output, int dtype,
                       const RoiProblem &p, void *workspace, size_t *need, hipStream_t s);
 
+// roi_pool.hip: separable LDS kernels for plain boxes with small outputs; -1 when not applicable
+int roi_pool_forward(const void *input, const void *rois, void *output, int dtype,
+                     const RoiProblem &p, hipStream_t s);
+int roi_pool_backward(const void *grad_output, const void *rois, void *acc, int dtype,
+                      const RoiProblem &p, hipStream_t s);
+
 static int make_problem(RoiProblem &p, int ndim, int rotated, int batch, int channels, int depth,
                         int height, int width, int num_rois, int out_d, int out_h, int out_w,
                         float spatial_scale, int sampling_ratio, int aligned, int order) {
@@ -154,6 +160,8 @@ int roi_forward(const void *input, const void *rois, void *output, int dtype, in
   {
     const int tiled = roi_forward_tiled(input, rois, output, dtype, p, workspace, nullptr, s);
     if (tiled >= 0) return tiled;
+    const int pooled = roi_pool_forward(input, rois, output, dtype, p, s);
+    if (pooled >= 0) return pooled;
   }
   const dim3 grid(p.chunks * num_rois), block(kRoiThreads);
   MV_DISPATCH(dtype, {
@@ -190,11 +198,15 @@ int roi_backward(const void *grad_output, const void *rois, void *grad_input, in
     hipLaunchKernelGGL(fill_zero_kernel, dim3(fill_blocks), dim3(256), 0, s,
                        static_cast<float *>(workspace), total);
   }
+  const int pooled = roi_pool_backward(grad_output, rois, narrow ? workspace : grad_input, dtype, p, s);
+  if (pooled > 0) return pooled;
   MV_DISPATCH(dtype, {
     using RT = typename std::conditional<std::is_same<T, double>::value, double, float>::type;
     using G = typename std::conditional<(sizeof(T) == 2), float, T>::type;
     G *acc = narrow ? static_cast<G *>(workspace) : static_cast<G *>(grad_input);
-    if (rotated)
+    if (pooled == 0) {
+      // gradient already accumulated by the pooled kernel
+    } else if (rotated)
       hipLaunchKernelGGL((roi_backward_kernel<T, G, RT, true>), grid, block, 0, s,
                          static_cast<const T *>(grad_output), static_cast<const RT *>(rois), acc, p);
     else

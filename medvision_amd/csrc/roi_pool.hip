@@ -1,0 +1,363 @@
+// RoIAlign for plain (axis-aligned) boxes with SMALL outputs per roi (detection heads: thousands of
+// rois, 7x7x7 cells, hundreds of channels), forward and backward.
+//
+// For an axis-aligned box the sample coordinates are separable: x depends only on (pw, ix), y on
+// (ph, iy), z on (pd, iz).  Each axis therefore has a short tap table (cells * grid entries of
+// {low index, high index, two weights}; validity and the 1/grid factor folded into the weights)
+// and the pooled output is the source sub-box contracted with three small sparse matrices:
+//     out[pd,ph,pw] = sum_z Wz[pd,z] sum_y Wy[ph,y] sum_x Wx[pw,x] * box[z,y,x]
+// One workgroup = (roi, chunk of channels).  It builds the tables, copies the roi's source sub-box
+// of its channels into LDS (every feature voxel is read once per roi instead of once per sample
+// corner), runs the three contractions through LDS and writes the outputs with coalesced stores.
+// The backward runs the transposed contractions and adds the sub-box gradient to global memory:
+// one atomic per touched feature voxel and (roi, channel) instead of one per sample corner
+// (config 5: ~64 instead of 21 952).
+// rois whose sub-box or tables exceed the LDS budget are handled in the same workgroup by a plain
+// per-output gather / scatter.
+#include "common.hpp"
+#include "roi_geometry.hpp"
+#include "sampling.hpp"
+
+namespace mv {
+
+constexpr int kPoolThreads = 256;
+constexpr int kPoolEntries = 64;               // tap-table entries per axis (cells * grid)
+constexpr int kPoolLdsBytes = 40 * 1024;       // staged data + intermediates of one channel chunk
+
+// i / d for 0 <= i < 2^21 and 0 < d < 2^12, with inv = 1.0f / d (exact: the product is at least
+// 0.5 / d away from an integer and its rounding error is below that)
+__device__ __forceinline__ int fdiv(int i, float inv) { return static_cast<int>((static_cast<float>(i) + 0.5f) * inv); }
+
+struct AxisTaps {
+  int lo[kPoolEntries], hi[kPoolEntries];      // box-relative tap indices
+  float wlo[kPoolEntries], whi[kPoolEntries];  // weights (0 for void samples), include 1 / grid
+  int box_lo, box_hi;                          // inclusive source range covered by valid taps
+  int entries, grid;
+};
+
+struct PoolShared {
+  RoiGeom g;
+  AxisTaps ax[3];  // x, y, z
+  int staged;      // 1: LDS path, 0: per-output gather, -1: every output is zero
+  int chunk;       // channels per LDS pass
+};
+
+// Builds geometry and tap tables for roi `roi`; all threads must call it (contains barriers).
+template <typename RT>
+__device__ inline void pool_setup(PoolShared &sh, const RT *roi, const RoiProblem &p, size_t elem_bytes) {
+  if (threadIdx.x == 0) {
+    const double sn[3] = {0, 0, 0}, cs[3] = {1, 1, 1};
+    build_geom(sh.g, roi, p, sn, cs);
+    const int cells[3] = {p.ow, p.oh, p.od};
+    for (int a = 0; a < 3; a++) {
+      sh.ax[a].grid = a < p.ndim ? sh.g.grid[a] : 1;
+      sh.ax[a].entries = cells[a] * max(sh.ax[a].grid, 0);
+      sh.ax[a].box_lo = 1 << 30;
+      sh.ax[a].box_hi = -1;
+    }
+    sh.staged = 1;
+    if (sh.g.batch < 0) sh.staged = -1;
+    for (int a = 0; a < 3; a++) {
+      if (sh.ax[a].entries > kPoolEntries) sh.staged = min(sh.staged, 0);
+      if (sh.ax[a].entries <= 0) sh.staged = -1;  // empty sampling grid: outputs are zero
+    }
+  }
+  __syncthreads();
+  if (sh.staged <= 0) return;
+  const int size[3] = {p.W, p.H, p.D};
+  for (int e = threadIdx.x; e < 3 * kPoolEntries; e += kPoolThreads) {
+    const int a = e / kPoolEntries, i = e % kPoolEntries;
+    AxisTaps &t = sh.ax[a];
+    if (i >= t.entries) continue;
+    const int cell = i / t.grid, sub = i % t.grid;
+    const double v = a < p.ndim ? local_coord(sh.g, a, cell, sub) : 0.0;
+    int lo, hi;
+    float frac;
+    const bool ok = clamped_tap<float>(v, size[a], lo, hi, frac);
+    if (p.order == 0) frac = (1.f - frac >= 0.5f) ? 0.f : 1.f;
+    const float inv = 1.f / static_cast<float>(t.grid);
+    t.lo[i] = ok ? lo : -1;
+    t.hi[i] = ok ? hi : -1;
+    t.wlo[i] = ok ? (1.f - frac) * inv : 0.f;
+    t.whi[i] = ok ? frac * inv : 0.f;
+    if (ok) {
+      atomicMin(&t.box_lo, lo);
+      atomicMax(&t.box_hi, hi);
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    long vol = 1;
+    for (int a = 0; a < 3; a++) {
+      if (sh.ax[a].box_hi < 0) { sh.staged = -1; break; }  // no valid sample on this axis
+      vol *= sh.ax[a].box_hi - sh.ax[a].box_lo + 1;
+    }
+    if (sh.staged == 1) {
+      const long nz = sh.ax[2].box_hi - sh.ax[2].box_lo + 1, ny = sh.ax[1].box_hi - sh.ax[1].box_lo + 1;
+      const long per_channel = vol * static_cast<long>(elem_bytes) + (nz * ny * p.ow + nz * p.oh * p.ow) * 4 + 16;
+      const long chunk = kPoolLdsBytes / per_channel;
+      if (chunk < 1) sh.staged = 0;
+      sh.chunk = static_cast<int>(min(chunk, 64L));
+    }
+  }
+  __syncthreads();
+  if (sh.staged != 1) return;
+  for (int e = threadIdx.x; e < 3 * kPoolEntries; e += kPoolThreads) {  // make indices box-relative
+    const int a = e / kPoolEntries, i = e % kPoolEntries;
+    AxisTaps &t = sh.ax[a];
+    if (i >= t.entries) continue;
+    t.lo[i] = t.lo[i] < 0 ? 0 : t.lo[i] - t.box_lo;
+    t.hi[i] = t.hi[i] < 0 ? 0 : t.hi[i] - t.box_lo;
+  }
+  __syncthreads();
+}
+
+template <typename T, typename RT>
+__global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
+    const T *__restrict__ feat, const RT *__restrict__ rois, T *__restrict__ out, const RoiProblem p,
+    const int channels_per_block) {
+  __shared__ PoolShared sh;
+  __shared__ __attribute__((aligned(16))) unsigned char lds[kPoolLdsBytes];
+  const unsigned n = blockIdx.x;
+  const int c_begin = blockIdx.y * channels_per_block, c_end = min(c_begin + channels_per_block, p.C);
+  pool_setup(sh, rois + static_cast<long>(n) * roi_columns(p.ndim, 0), p, sizeof(T));
+  const int cells = p.od * p.oh * p.ow;
+  const long plane = static_cast<long>(p.D) * p.H * p.W;
+  T *dst = out + (static_cast<long>(n) * p.C + c_begin) * cells;
+  const int total = (c_end - c_begin) * cells;
+  if (sh.staged < 0) {
+    for (int i = threadIdx.x; i < total; i += kPoolThreads) dst[i] = store_cast<T>(0.f);
+    return;
+  }
+  const T *src = feat + (static_cast<long>(sh.g.batch) * p.C + c_begin) * plane;
+  if (sh.staged == 0) {  // per-output gather
+    const int gz = p.ndim == 3 ? sh.g.grid[2] : 1, gy = sh.g.grid[1], gx = sh.g.grid[0];
+    for (int i = threadIdx.x; i < total; i += kPoolThreads) {
+      const int pw = i % p.ow, ph = (i / p.ow) % p.oh, pd = (i / (p.ow * p.oh)) % p.od, c = i / cells;
+      float acc = 0.f;
+      for (int iz = 0; iz < gz; iz++) {
+        const double z = p.ndim == 3 ? local_coord(sh.g, 2, pd, iz) : 0.0;
+        for (int iy = 0; iy < gy; iy++) {
+          const double y = local_coord(sh.g, 1, ph, iy);
+          for (int ix = 0; ix < gx; ix++)
+            acc += sample_clamped<T>(src + c * plane, p.D, p.H, p.W, z, y, local_coord(sh.g, 0, pw, ix), p.order);
+        }
+      }
+      dst[i] = store_cast<T>(acc / static_cast<float>(sh.g.count));
+    }
+    return;
+  }
+  const AxisTaps &tx = sh.ax[0], &ty = sh.ax[1], &tz = sh.ax[2];
+  const int nx = tx.box_hi - tx.box_lo + 1, ny = ty.box_hi - ty.box_lo + 1, nz = tz.box_hi - tz.box_lo + 1;
+  const int vol = nx * ny * nz;
+  const int gx = tx.grid, gy = ty.grid, gz = tz.grid;
+  const int ohw = p.oh * p.ow;
+  const float inv_vol = 1.f / vol, inv_nxy = 1.f / (nx * ny), inv_nx = 1.f / nx, inv_ow = 1.f / p.ow,
+              inv_ohw = 1.f / ohw, inv_cells = 1.f / cells;
+  for (int cb = c_begin; cb < c_end; cb += sh.chunk) {
+    const int cs = min(sh.chunk, c_end - cb);
+    T *box = reinterpret_cast<T *>(lds);                                            // [cs][nz][ny][nx]
+    float *t1 = reinterpret_cast<float *>(lds + ((static_cast<size_t>(cs) * vol * sizeof(T) + 15) / 16) * 16);  // [cs][nz][ny][ow]
+    float *t2 = t1 + cs * nz * ny * p.ow;                                           // [cs][nz][oh][ow]
+    const T *corner = src + static_cast<long>(cb - c_begin) * plane +
+                      (static_cast<long>(tz.box_lo) * p.H + ty.box_lo) * p.W + tx.box_lo;
+    for (int i = threadIdx.x; i < cs * vol; i += kPoolThreads) {
+      const int c = fdiv(i, inv_vol), r0 = i - c * vol, z = fdiv(r0, inv_nxy), r1 = r0 - z * nx * ny;
+      const int y = fdiv(r1, inv_nx), x = r1 - y * nx;
+      box[i] = corner[c * plane + (static_cast<long>(z) * p.H + y) * p.W + x];
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < cs * nz * ny * p.ow; i += kPoolThreads) {  // contract x
+      const int row = fdiv(i, inv_ow), pw = i - row * p.ow;                 // row = (c, z, y)
+      const T *r = box + row * nx;
+      float acc = 0.f;
+      for (int s = 0; s < gx; s++) {
+        const int e = pw * gx + s;
+        acc += tx.wlo[e] * load(r + tx.lo[e]) + tx.whi[e] * load(r + tx.hi[e]);
+      }
+      t1[i] = acc;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < cs * nz * p.oh * p.ow; i += kPoolThreads) {  // contract y
+      const int cz = fdiv(i, inv_ohw), hw = i - cz * ohw, ph = fdiv(hw, inv_ow), pw = hw - ph * p.ow;  // cz = (c, z)
+      const float *r = t1 + cz * ny * p.ow + pw;
+      float acc = 0.f;
+      for (int s = 0; s < gy; s++) {
+        const int e = ph * gy + s;
+        acc += ty.wlo[e] * r[ty.lo[e] * p.ow] + ty.whi[e] * r[ty.hi[e] * p.ow];
+      }
+      t2[i] = acc;
+    }
+    __syncthreads();
+    T *o = dst + static_cast<long>(cb - c_begin) * cells;
+    for (int i = threadIdx.x; i < cs * cells; i += kPoolThreads) {  // contract z, store
+      const int c = fdiv(i, inv_cells), r0 = i - c * cells, pd = fdiv(r0, inv_ohw), hw = r0 - pd * ohw;
+      const float *r = t2 + c * nz * ohw + hw;
+      float acc = 0.f;
+      for (int s = 0; s < gz; s++) {
+        const int e = pd * gz + s;
+        acc += tz.wlo[e] * r[tz.lo[e] * ohw] + tz.whi[e] * r[tz.hi[e] * ohw];
+      }
+      o[i] = store_cast<T>(acc);
+    }
+    __syncthreads();
+  }
+}
+
+// G = element type of the accumulation buffer (T for fp32, float for 16-bit T).
+template <typename T, typename G, typename RT>
+__global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
+    const T *__restrict__ gout, const RT *__restrict__ rois, G *__restrict__ gin, const RoiProblem p,
+    const int channels_per_block) {
+  __shared__ PoolShared sh;
+  __shared__ __attribute__((aligned(16))) unsigned char lds[kPoolLdsBytes];
+  const unsigned n = blockIdx.x;
+  const int c_begin = blockIdx.y * channels_per_block, c_end = min(c_begin + channels_per_block, p.C);
+  // intermediates are fp32 here, so size the chunk with 4-byte box elements
+  pool_setup(sh, rois + static_cast<long>(n) * roi_columns(p.ndim, 0), p, sizeof(float));
+  if (sh.staged < 0) return;
+  const int cells = p.od * p.oh * p.ow;
+  const long plane = static_cast<long>(p.D) * p.H * p.W;
+  const T *src = gout + (static_cast<long>(n) * p.C + c_begin) * cells;
+  G *dst = gin + (static_cast<long>(sh.g.batch) * p.C + c_begin) * plane;
+  if (sh.staged == 0) {  // per-output scatter
+    const int total = (c_end - c_begin) * cells;
+    const int gz = p.ndim == 3 ? sh.g.grid[2] : 1, gy = sh.g.grid[1], gx = sh.g.grid[0];
+    for (int i = threadIdx.x; i < total; i += kPoolThreads) {
+      const int pw = i % p.ow, ph = (i / p.ow) % p.oh, pd = (i / (p.ow * p.oh)) % p.od, c = i / cells;
+      const float top = load(src + i) / static_cast<float>(sh.g.count);
+      for (int iz = 0; iz < gz; iz++) {
+        const double z = p.ndim == 3 ? local_coord(sh.g, 2, pd, iz) : 0.0;
+        for (int iy = 0; iy < gy; iy++) {
+          const double y = local_coord(sh.g, 1, ph, iy);
+          for (int ix = 0; ix < gx; ix++) {
+            Corners<float> cw;
+            if (!clamped_corners<float>(p.D, p.H, p.W, z, y, local_coord(sh.g, 0, pw, ix), p.order, cw)) continue;
+#pragma unroll
+            for (int k = 0; k < 8; k++)
+              if (cw.w[k] != 0.f) atomic_add(dst + c * plane + cw.idx[k], static_cast<G>(top * cw.w[k]));
+          }
+        }
+      }
+    }
+    return;
+  }
+  const AxisTaps &tx = sh.ax[0], &ty = sh.ax[1], &tz = sh.ax[2];
+  const int nx = tx.box_hi - tx.box_lo + 1, ny = ty.box_hi - ty.box_lo + 1, nz = tz.box_hi - tz.box_lo + 1;
+  const int vol = nx * ny * nz;
+  const int ohw = p.oh * p.ow;
+  const float inv_vol = 1.f / vol, inv_nxy = 1.f / (nx * ny), inv_nx = 1.f / nx, inv_ow = 1.f / p.ow,
+              inv_ohw = 1.f / ohw, inv_nzohw = 1.f / (nz * ohw), inv_nyow = 1.f / (ny * p.ow);
+  for (int cb = c_begin; cb < c_end; cb += sh.chunk) {
+    const int cs = min(sh.chunk, c_end - cb);
+    float *gbox = reinterpret_cast<float *>(lds);    // [cs][nz][ny][nx]
+    float *t1 = gbox + cs * vol;                     // [cs][nz][ny][ow]
+    float *t2 = t1 + cs * nz * ny * p.ow;            // [cs][nz][oh][ow]
+    const T *go = src + static_cast<long>(cb - c_begin) * cells;
+    for (int i = threadIdx.x; i < cs * nz * ohw; i += kPoolThreads) {  // transpose of "contract z"
+      const int c = fdiv(i, inv_nzohw), r0 = i - c * nz * ohw, z = fdiv(r0, inv_ohw), hw = r0 - z * ohw;
+      const T *r = go + c * cells + hw;
+      float acc = 0.f;
+      for (int e = 0; e < tz.entries; e++) {
+        const float w = (tz.lo[e] == z ? tz.wlo[e] : 0.f) + (tz.hi[e] == z ? tz.whi[e] : 0.f);
+        if (w != 0.f) acc += w * load(r + (e / tz.grid) * ohw);
+      }
+      t2[i] = acc;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < cs * nz * ny * p.ow; i += kPoolThreads) {  // transpose of "contract y"
+      const int cz = fdiv(i, inv_nyow), r0 = i - cz * ny * p.ow, y = fdiv(r0, inv_ow), pw = r0 - y * p.ow;
+      const float *r = t2 + cz * ohw + pw;
+      float acc = 0.f;
+      for (int e = 0; e < ty.entries; e++) {
+        const float w = (ty.lo[e] == y ? ty.wlo[e] : 0.f) + (ty.hi[e] == y ? ty.whi[e] : 0.f);
+        if (w != 0.f) acc += w * r[(e / ty.grid) * p.ow];
+      }
+      t1[i] = acc;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < cs * vol; i += kPoolThreads) {  // transpose of "contract x"
+      const int row = fdiv(i, inv_nx), x = i - row * nx;
+      const float *r = t1 + row * p.ow;
+      float acc = 0.f;
+      for (int e = 0; e < tx.entries; e++) {
+        const float w = (tx.lo[e] == x ? tx.wlo[e] : 0.f) + (tx.hi[e] == x ? tx.whi[e] : 0.f);
+        if (w != 0.f) acc += w * r[e / tx.grid];
+      }
+      gbox[i] = acc;
+    }
+    __syncthreads();
+    G *corner = dst + static_cast<long>(cb - c_begin) * plane +
+                (static_cast<long>(tz.box_lo) * p.H + ty.box_lo) * p.W + tx.box_lo;
+    for (int i = threadIdx.x; i < cs * vol; i += kPoolThreads) {
+      const float v = gbox[i];
+      if (v == 0.f) continue;
+      const int c = fdiv(i, inv_vol), r0 = i - c * vol, z = fdiv(r0, inv_nxy), r1 = r0 - z * nx * ny;
+      const int y = fdiv(r1, inv_nx), x = r1 - y * nx;
+      atomic_add(corner + c * plane + (static_cast<long>(z) * p.H + y) * p.W + x, static_cast<G>(v));
+    }
+    __syncthreads();
+  }
+}
+
+static bool pool_applies(int dtype, const RoiProblem &p) {
+  if (p.rotated || dtype == MV_F64) return false;
+  const long cells = static_cast<long>(p.od) * p.oh * p.ow;
+  if (cells > 1024 || p.od > 16 || p.oh > 16 || p.ow > 16) return false;
+  if (p.sampling_ratio > 4) return false;
+  return p.R <= 0x7fffffff;
+}
+
+// Returns -1 when the pooled kernels do not apply.
+int roi_pool_forward(const void *input, const void *rois, void *output, int dtype,
+                     const RoiProblem &p, hipStream_t s) {
+  if (!pool_applies(dtype, p)) return -1;
+  const int cpb = 32;
+  const long cblocks = (p.C + cpb - 1) / cpb;
+  if (cblocks > 65535) return -1;
+  const dim3 grid(p.R, static_cast<unsigned>(cblocks)), block(kPoolThreads);
+  const float *r = static_cast<const float *>(rois);
+  switch (dtype) {
+    case MV_F32:
+      hipLaunchKernelGGL((roi_pool_forward_kernel<float, float>), grid, block, 0, s,
+                         static_cast<const float *>(input), r, static_cast<float *>(output), p, cpb);
+      break;
+    case MV_F16:
+      hipLaunchKernelGGL((roi_pool_forward_kernel<__half, float>), grid, block, 0, s,
+                         static_cast<const __half *>(input), r, static_cast<__half *>(output), p, cpb);
+      break;
+    default:
+      hipLaunchKernelGGL((roi_pool_forward_kernel<__hip_bfloat16, float>), grid, block, 0, s,
+                         static_cast<const __hip_bfloat16 *>(input), r,
+                         static_cast<__hip_bfloat16 *>(output), p, cpb);
+  }
+  return check_launch("roi_pool_forward_kernel");
+}
+
+// `acc` is the accumulation buffer: grad_input itself for fp32, the fp32 workspace for 16-bit.
+int roi_pool_backward(const void *grad_output, const void *rois, void *acc, int dtype,
+                      const RoiProblem &p, hipStream_t s) {
+  if (!pool_applies(dtype, p)) return -1;
+  const int cpb = 32;
+  const long cblocks = (p.C + cpb - 1) / cpb;
+  if (cblocks > 65535) return -1;
+  const dim3 grid(p.R, static_cast<unsigned>(cblocks)), block(kPoolThreads);
+  const float *r = static_cast<const float *>(rois);
+  switch (dtype) {
+    case MV_F32:
+      hipLaunchKernelGGL((roi_pool_backward_kernel<float, float, float>), grid, block, 0, s,
+                         static_cast<const float *>(grad_output), r, static_cast<float *>(acc), p, cpb);
+      break;
+    case MV_F16:
+      hipLaunchKernelGGL((roi_pool_backward_kernel<__half, float, float>), grid, block, 0, s,
+                         static_cast<const __half *>(grad_output), r, static_cast<float *>(acc), p, cpb);
+      break;
+    default:
+      hipLaunchKernelGGL((roi_pool_backward_kernel<__hip_bfloat16, float, float>), grid, block, 0, s,
+                         static_cast<const __hip_bfloat16 *>(grad_output), r, static_cast<float *>(acc),
+                         p, cpb);
+  }
+  return check_launch("roi_pool_backward_kernel");
+}
+
+}  // namespace mv
