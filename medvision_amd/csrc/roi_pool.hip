@@ -31,6 +31,7 @@ __device__ __forceinline__ int fdiv(int i, float inv) { return static_cast<int>(
 struct AxisTaps {
   int lo[kPoolEntries], hi[kPoolEntries];      // box-relative tap indices
   float wlo[kPoolEntries], whi[kPoolEntries];  // weights (0 for void samples), include 1 / grid
+  int first[kPoolEntries + 4];                 // first[i] = first entry whose low tap is >= i (box-relative)
   int box_lo, box_hi;                          // inclusive source range covered by valid taps
   int entries, grid;
 };
@@ -73,11 +74,11 @@ __device__ inline void pool_setup(PoolShared &sh, const RT *roi, const RoiProble
     const double v = a < p.ndim ? local_coord(sh.g, a, cell, sub) : 0.0;
     int lo, hi;
     float frac;
-    const bool ok = clamped_tap<float>(v, size[a], lo, hi, frac);
-    if (p.order == 0) frac = (1.f - frac >= 0.5f) ? 0.f : 1.f;
+    const bool ok = clamped_tap<float>(v, size[a], lo, hi, frac, p.order);
     const float inv = 1.f / static_cast<float>(t.grid);
-    t.lo[i] = ok ? lo : -1;
-    t.hi[i] = ok ? hi : -1;
+    // void samples keep weight 0; park them at the matching end so that `lo` stays monotonic
+    t.lo[i] = ok ? lo : (v > 0.0 ? -2 : -1);
+    t.hi[i] = t.lo[i] < 0 ? t.lo[i] : hi;
     t.wlo[i] = ok ? (1.f - frac) * inv : 0.f;
     t.whi[i] = ok ? frac * inv : 0.f;
     if (ok) {
@@ -106,8 +107,18 @@ __device__ inline void pool_setup(PoolShared &sh, const RT *roi, const RoiProble
     const int a = e / kPoolEntries, i = e % kPoolEntries;
     AxisTaps &t = sh.ax[a];
     if (i >= t.entries) continue;
-    t.lo[i] = t.lo[i] < 0 ? 0 : t.lo[i] - t.box_lo;
-    t.hi[i] = t.hi[i] < 0 ? 0 : t.hi[i] - t.box_lo;
+    const int top = t.box_hi - t.box_lo;
+    t.lo[i] = t.lo[i] == -1 ? 0 : (t.lo[i] == -2 ? top : t.lo[i] - t.box_lo);
+    t.hi[i] = t.hi[i] == -1 ? 0 : (t.hi[i] == -2 ? top : t.hi[i] - t.box_lo);
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < 3 * (kPoolEntries + 4); e += kPoolThreads) {  // entry ranges per source index
+    const int a = e / (kPoolEntries + 4), i = e % (kPoolEntries + 4);
+    AxisTaps &t = sh.ax[a];
+    if (i > t.box_hi - t.box_lo + 1) continue;
+    int f = 0;
+    while (f < t.entries && t.lo[f] < i) f++;
+    t.first[i] = f;
   }
   __syncthreads();
 }
@@ -246,21 +257,27 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
   const int nx = tx.box_hi - tx.box_lo + 1, ny = ty.box_hi - ty.box_lo + 1, nz = tz.box_hi - tz.box_lo + 1;
   const int vol = nx * ny * nz;
   const int ohw = p.oh * p.ow;
+  const int gx = tx.grid, gy = ty.grid, gz = tz.grid;
   const float inv_vol = 1.f / vol, inv_nxy = 1.f / (nx * ny), inv_nx = 1.f / nx, inv_ow = 1.f / p.ow,
-              inv_ohw = 1.f / ohw, inv_nzohw = 1.f / (nz * ohw), inv_nyow = 1.f / (ny * p.ow);
+              inv_ohw = 1.f / ohw, inv_nzohw = 1.f / (nz * ohw), inv_nyow = 1.f / (ny * p.ow),
+              inv_gx = 1.f / gx, inv_gy = 1.f / gy, inv_gz = 1.f / gz;
   for (int cb = c_begin; cb < c_end; cb += sh.chunk) {
     const int cs = min(sh.chunk, c_end - cb);
     float *gbox = reinterpret_cast<float *>(lds);    // [cs][nz][ny][nx]
     float *t1 = gbox + cs * vol;                     // [cs][nz][ny][ow]
     float *t2 = t1 + cs * nz * ny * p.ow;            // [cs][nz][oh][ow]
     const T *go = src + static_cast<long>(cb - c_begin) * cells;
+    // Transposed contractions as gathers.  Entries are sorted by coordinate, so the entries whose
+    // low tap is source index i form the range [first[i], first[i+1]) and those whose high tap is
+    // i are the low-tap entries of i - 1 (a clamped edge entry has lo == hi and zero high weight).
     for (int i = threadIdx.x; i < cs * nz * ohw; i += kPoolThreads) {  // transpose of "contract z"
       const int c = fdiv(i, inv_nzohw), r0 = i - c * nz * ohw, z = fdiv(r0, inv_ohw), hw = r0 - z * ohw;
       const T *r = go + c * cells + hw;
+      const int mid = tz.first[z], e0 = z > 0 ? tz.first[z - 1] : mid, e1 = tz.first[z + 1];
       float acc = 0.f;
-      for (int e = 0; e < tz.entries; e++) {
-        const float w = (tz.lo[e] == z ? tz.wlo[e] : 0.f) + (tz.hi[e] == z ? tz.whi[e] : 0.f);
-        if (w != 0.f) acc += w * load(r + (e / tz.grid) * ohw);
+      for (int e = e0; e < e1; e++) {
+        const float w = e < mid ? (tz.hi[e] == z ? tz.whi[e] : 0.f) : tz.wlo[e];
+        acc += w * load(r + fdiv(e, inv_gz) * ohw);
       }
       t2[i] = acc;
     }
@@ -268,10 +285,11 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
     for (int i = threadIdx.x; i < cs * nz * ny * p.ow; i += kPoolThreads) {  // transpose of "contract y"
       const int cz = fdiv(i, inv_nyow), r0 = i - cz * ny * p.ow, y = fdiv(r0, inv_ow), pw = r0 - y * p.ow;
       const float *r = t2 + cz * ohw + pw;
+      const int mid = ty.first[y], e0 = y > 0 ? ty.first[y - 1] : mid, e1 = ty.first[y + 1];
       float acc = 0.f;
-      for (int e = 0; e < ty.entries; e++) {
-        const float w = (ty.lo[e] == y ? ty.wlo[e] : 0.f) + (ty.hi[e] == y ? ty.whi[e] : 0.f);
-        if (w != 0.f) acc += w * r[(e / ty.grid) * p.ow];
+      for (int e = e0; e < e1; e++) {
+        const float w = e < mid ? (ty.hi[e] == y ? ty.whi[e] : 0.f) : ty.wlo[e];
+        acc += w * r[fdiv(e, inv_gy) * p.ow];
       }
       t1[i] = acc;
     }
@@ -279,10 +297,11 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
     for (int i = threadIdx.x; i < cs * vol; i += kPoolThreads) {  // transpose of "contract x"
       const int row = fdiv(i, inv_nx), x = i - row * nx;
       const float *r = t1 + row * p.ow;
+      const int mid = tx.first[x], e0 = x > 0 ? tx.first[x - 1] : mid, e1 = tx.first[x + 1];
       float acc = 0.f;
-      for (int e = 0; e < tx.entries; e++) {
-        const float w = (tx.lo[e] == x ? tx.wlo[e] : 0.f) + (tx.hi[e] == x ? tx.whi[e] : 0.f);
-        if (w != 0.f) acc += w * r[e / tx.grid];
+      for (int e = e0; e < e1; e++) {
+        const float w = e < mid ? (tx.hi[e] == x ? tx.whi[e] : 0.f) : tx.wlo[e];
+        acc += w * r[fdiv(e, inv_gx)];
       }
       gbox[i] = acc;
     }

@@ -163,8 +163,8 @@ __device__ __forceinline__ float staged_sample(const T *__restrict__ tile, CT rx
     rz = clamp_ct(rz, b.cmin[2], b.cmax[2]);
   }
   const CT flx = floor(rx), fly = floor(ry), flz = floor(rz);
-  const float wx = static_cast<float>(rx - flx), wy = static_cast<float>(ry - fly),
-              wz = static_cast<float>(rz - flz);
+  const CT dx_ = rx - flx, dy_ = ry - fly, dz_ = rz - flz;
+  const float wx = static_cast<float>(dx_), wy = static_cast<float>(dy_), wz = static_cast<float>(dz_);
   int ix = static_cast<int>(flx), iy = static_cast<int>(fly), iz = static_cast<int>(flz);
   int dy = pitch, dz = slice;
   if (!INTERIOR) {  // void samples may lie anywhere: keep every access inside the box
@@ -175,7 +175,7 @@ __device__ __forceinline__ float staged_sample(const T *__restrict__ tile, CT rx
   const int i00 = __mul24(iz, slice) + __mul24(iy, pitch) + ix;
   float v;
   if (order == 0) {
-    v = load(tile + (i00 + (wz <= 0.5f ? 0 : dz) + (wy <= 0.5f ? 0 : dy) + (wx <= 0.5f ? 0 : 1)));
+    v = load(tile + (i00 + (dz_ <= CT(0.5) ? 0 : dz) + (dy_ <= CT(0.5) ? 0 : dy) + (dx_ <= CT(0.5) ? 0 : 1)));
   } else {
     const float x00 = lerp_pair(tile, i00, wx), x01 = lerp_pair(tile, i00 + dy, wx);
     const float x10 = lerp_pair(tile, i00 + dz, wx), x11 = lerp_pair(tile, i00 + dz + dy, wx);

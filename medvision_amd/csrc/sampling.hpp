@@ -11,19 +11,31 @@ namespace mv {
 // Border-replicating tap on one axis (reference: csrc/cuda/interpolation_helpers_3d.h:12-48):
 // outside the closed interval [-1, size] the sample is void; negatives snap to 0; a base index
 // at or beyond size-1 collapses both taps onto size-1.
-template <typename A>
-__device__ __forceinline__ bool clamped_tap(double v, int size, int &lo, int &hi, A &frac) {
+__device__ __forceinline__ bool clamped_tap64(double v, int size, int &lo, int &hi, double &frac) {
   if (v < -1.0 || v > static_cast<double>(size)) return false;
   v = v <= 0.0 ? 0.0 : v;
   const int base = static_cast<int>(v);
   if (base >= size - 1) {
     lo = hi = size - 1;
-    frac = A(0);
+    frac = 0.0;
   } else {
     lo = base;
     hi = base + 1;
-    frac = static_cast<A>(v - static_cast<double>(base));
+    frac = v - static_cast<double>(base);
   }
+  return true;
+}
+
+// order 1: fraction rounded once to the arithmetic type A.  order 0: the fraction becomes 0 or 1;
+// the pick "low index when 1 - frac >= 0.5" (csrc/cuda/interpolation_helpers_3d.h:186-194) is
+// decided on the fp64 fraction so that coordinates a few ulp from a tie fall on the same side as
+// in an fp64 evaluation.
+template <typename A>
+__device__ __forceinline__ bool clamped_tap(double v, int size, int &lo, int &hi, A &frac,
+                                            int order = 1) {
+  double f;
+  if (!clamped_tap64(v, size, lo, hi, f)) return false;
+  frac = order == 0 ? ((1.0 - f >= 0.5) ? A(0) : A(1)) : static_cast<A>(f);
   return true;
 }
 
@@ -40,14 +52,9 @@ __device__ __forceinline__ bool clamped_corners(int D, int H, int W, double z, d
                                                 int order, Corners<A> &c) {
   int z0, z1, y0, y1, x0, x1;
   A lz, ly, lx;
-  if (!clamped_tap(z, D, z0, z1, lz) || !clamped_tap(y, H, y0, y1, ly) ||
-      !clamped_tap(x, W, x0, x1, lx))
+  if (!clamped_tap(z, D, z0, z1, lz, order) || !clamped_tap(y, H, y0, y1, ly, order) ||
+      !clamped_tap(x, W, x0, x1, lx, order))
     return false;
-  if (order == 0) {
-    lz = (A(1) - lz >= A(0.5)) ? A(0) : A(1);
-    ly = (A(1) - ly >= A(0.5)) ? A(0) : A(1);
-    lx = (A(1) - lx >= A(0.5)) ? A(0) : A(1);
-  }
   const A hz = A(1) - lz, hy = A(1) - ly, hx = A(1) - lx;
   const long r00 = (static_cast<long>(z0) * H + y0) * W, r01 = (static_cast<long>(z0) * H + y1) * W;
   const long r10 = (static_cast<long>(z1) * H + y0) * W, r11 = (static_cast<long>(z1) * H + y1) * W;
@@ -65,13 +72,11 @@ __device__ __forceinline__ typename Acc<T>::type sample_clamped(const T *plane, 
   using A = typename Acc<T>::type;
   int z0, z1, y0, y1, x0, x1;
   A lz, ly, lx;
-  if (!clamped_tap(z, D, z0, z1, lz) || !clamped_tap(y, H, y0, y1, ly) ||
-      !clamped_tap(x, W, x0, x1, lx))
+  if (!clamped_tap(z, D, z0, z1, lz, order) || !clamped_tap(y, H, y0, y1, ly, order) ||
+      !clamped_tap(x, W, x0, x1, lx, order))
     return A(0);
   if (order == 0) {
-    const int zi = (A(1) - lz >= A(0.5)) ? z0 : z1;
-    const int yi = (A(1) - ly >= A(0.5)) ? y0 : y1;
-    const int xi = (A(1) - lx >= A(0.5)) ? x0 : x1;
+    const int zi = lz == A(0) ? z0 : z1, yi = ly == A(0) ? y0 : y1, xi = lx == A(0) ? x0 : x1;
     return load(plane + (static_cast<long>(zi) * H + yi) * W + xi);
   }
   const A hz = A(1) - lz, hy = A(1) - ly, hx = A(1) - lx;

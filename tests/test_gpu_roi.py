@@ -197,6 +197,44 @@ def test_config5_detection_head_reduced(ops, oracle, dtype):
     assert_close(x.grad, gwant, BWD_TOL[dtype], "backward")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("sr,order", [(2, 1), (-1, 1), (3, 1), (1, 0)])
+def test_pooled_kernel_paths(ops, oracle, dtype, sr, order):
+    """Plain boxes with small outputs run through the separable LDS kernels; this covers their
+    special cases: boxes larger than the LDS budget, adaptive grids whose tap tables overflow,
+    boxes (partly) outside the volume, degenerate and single-voxel boxes, several channel chunks."""
+    g = wl.gen(21)
+    feat = torch.randn(2, 40, 20, 40, 44, generator=g).to(dtype)
+    rois = torch.tensor([
+        [0, 0.0, 0.0, 0.0, 44.0, 40.0, 20.0],        # whole volume: 44*40*20 voxels per channel
+        [1, -30.0, -30.0, -30.0, 80.0, 90.0, 60.0],   # far larger than the volume
+        [1, 50.0, 45.0, 25.0, 60.0, 55.0, 30.0],      # completely outside: all samples void
+        [0, -5.1, -3.2, -2.3, 6.05, 4.1, 3.2],        # partly outside (no sample on an exact .5 tie)
+        [0, 10.2, 11.7, 5.1, 10.3, 11.8, 5.2],        # degenerate (extent clamped to 1)
+        [1, 43.0, 39.0, 19.0, 44.0, 40.0, 20.0],      # last voxel, taps clamp at the border
+        [1, 3.3, 2.2, 1.1, 17.9, 21.4, 9.6],
+    ])
+    x = feat.to(DEV).requires_grad_(True)
+    out = ops.RoIAlign((5, 6, 7), 1.0, sr)(x, rois.to(DEV), order=order)
+    eff = 1 if order == 0 else sr
+    want = oracle.roi_align_forward(feat, rois, (5, 6, 7), 1.0, eff, True, order)
+    assert_close(out, want, FWD_TOL[dtype], "pooled forward")
+    gy = torch.randn(out.shape, generator=g).to(dtype)
+    out.backward(gy.to(DEV))
+    gwant = oracle.roi_align_backward(gy, rois, feat.shape, 1.0, eff, True, order)
+    assert_close(x.grad, gwant, BWD_TOL[dtype], "pooled backward")
+    # 2-D twin
+    f2 = torch.randn(2, 5, 30, 34, generator=g).to(dtype)
+    r2 = torch.tensor([[0, 0.0, 0.0, 34.0, 30.0], [1, -4.0, 3.0, 9.5, 40.0], [1, 7.7, 8.8, 7.9, 8.9]])
+    x2 = f2.to(DEV).requires_grad_(True)
+    o2 = ops.RoIAlign((6, 7), 1.0, sr)(x2, r2.to(DEV), order=order)
+    assert_close(o2, oracle.roi_align_forward(f2, r2, (6, 7), 1.0, eff, True, order), FWD_TOL[dtype], "2-d")
+    gy2 = torch.randn(o2.shape, generator=g).to(dtype)
+    o2.backward(gy2.to(DEV))
+    assert_close(x2.grad, oracle.roi_align_backward(gy2, r2, f2.shape, 1.0, eff, True, order),
+                 BWD_TOL[dtype], "2-d backward")
+
+
 def test_config1_rois_on_gpu(ops, oracle):
     """BASELINE config 1 inputs (fp32 [2,16,32,64,64], 128 rois, 7^3, sr=2) through RoIAlign3D."""
     g = wl.gen(0)
