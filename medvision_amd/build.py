@@ -21,6 +21,7 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
 ]
+FILE_FLAGS = {}   # per-file additions, keyed by source file name
 
 
 def _run(cmd):
@@ -38,7 +39,8 @@ def build(verbose=False, jobs=None):
     objs = [os.path.join(obj_dir, os.path.basename(s)[:-4] + ".o") for s in sources]
     jobs = jobs or min(8, len(sources))
     with concurrent.futures.ThreadPoolExecutor(jobs) as pool:
-        outs = list(pool.map(lambda so: _run([HIPCC, *FLAGS, "-c", so[0], "-o", so[1]]),
+        outs = list(pool.map(lambda so: _run([HIPCC, *FLAGS, *FILE_FLAGS.get(os.path.basename(so[0]), []),
+                                              "-c", so[0], "-o", so[1]]),
                              zip(sources, objs)))
     link = _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs])
     if verbose:

@@ -42,6 +42,32 @@ __host__ __device__ inline int roi_columns(int ndim, int rotated) {
   return ndim == 2 ? (rotated ? 6 : 5) : (rotated ? 10 : 7);
 }
 
+// sin and cos of a moderate angle (|x| up to ~1e5 rad) in fp64: two-constant Cody-Waite reduction
+// to [-pi/4, pi/4] followed by the classic minimax polynomials (errors below 1 ulp).  Much less
+// code and latency than the general library routine, which matters for the tiny set-up kernels.
+__device__ inline void sincos_moderate(double x, double &s, double &c) {
+  const double k = rint(x * 0.63661977236758134308);            // x * 2/pi
+  double r = fma(-k, 1.57079632679489655800e+00, x);             // pi/2 high part
+  r = fma(-k, 6.12323399573676603587e-17, r);                    // pi/2 low part
+  const double z = r * r;
+  double ps = fma(z, 1.58969099521155010221e-10, -2.50507602534068634195e-08);
+  ps = fma(z, ps, 2.75573137070700676789e-06);
+  ps = fma(z, ps, -1.98412698298579493134e-04);
+  ps = fma(z, ps, 8.33333333332248946124e-03);
+  ps = fma(z, ps, -1.66666666666666324348e-01);
+  const double sr = fma(z * r, ps, r);
+  double pc = fma(z, -1.13596475577881948265e-11, 2.08757232129817482790e-09);
+  pc = fma(z, pc, -2.75573143513906633035e-07);
+  pc = fma(z, pc, 2.48015872894767294178e-05);
+  pc = fma(z, pc, -1.38888888888741095749e-03);
+  pc = fma(z, pc, 4.16666666666666019037e-02);
+  const double cr = fma(z * z, pc, fma(z, -0.5, 1.0));
+  const int q = static_cast<int>(k) & 3;
+  const double ss = (q & 1) ? cr : sr, cc = (q & 1) ? sr : cr;
+  s = (q & 2) ? -ss : ss;
+  c = ((q + 1) & 2) ? -cc : cc;
+}
+
 // Angles of a rotated roi (up to three); lanes 0..2 of a workgroup call this in parallel and
 // publish sin / cos through LDS before one lane assembles the geometry.
 template <typename RT>
@@ -49,7 +75,7 @@ __device__ inline void roi_trig(const RT *roi, const RoiProblem &p, int which, d
   s = 0.0; c = 1.0;
   if (!p.rotated) return;
   const int first = 1 + 2 * p.ndim, count = p.ndim == 3 ? 3 : 1;
-  if (which < count) sincos(static_cast<double>(roi[first + which]), &s, &c);
+  if (which < count) sincos_moderate(static_cast<double>(roi[first + which]), s, c);
 }
 
 // sn / cs: sines and cosines of (angle_x, angle_y, angle_z) in 3-D, (theta, -, -) in 2-D.
@@ -65,7 +91,9 @@ __device__ inline void build_geom(RoiGeom &g, const RT *roi, const RoiProblem &p
   const int b = static_cast<int>(roi[0]);
   g.batch = (b >= 0 && b < p.N) ? b : -1;
   const double s = p.scale;
-  for (int a = 0; a < nd; a++) {
+#pragma unroll
+  for (int a = 0; a < 3; a++) {
+    if (a >= nd) continue;
     double ext;
     if (p.rotated) {
       ext = static_cast<double>(roi[1 + nd + a]) * s;

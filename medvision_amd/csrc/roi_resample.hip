@@ -28,25 +28,33 @@ namespace mv {
 
 constexpr int kXcds = 8;
 
-struct TilePlan {          // 128 bytes
+struct TilePlan {          // 208 bytes
   double org[3];           // box-relative source position (x,y,z) of the tile's first output voxel
   double inc[9];           // d(source a)/d(output j) at inc[a * 3 + j], j = (x, y, z)
   int lo[3];               // first staged source voxel (x, y, z)
   int n[3];                // staged extent
   int batch;               // feature-map index of the roi
   int mode;                // 0 = all zero, 1 = staged (clipped box), 2 = gather, 3 = staged interior
+  int t0[3];               // first output voxel of the tile (x, y, z)
+  int roi;                 // roi index
+  int rp;                  // box rows copied per pass of the workgroup: `span` whole z-slices
+  int span;                // z-slices per pass
+  int passes;              // ceil(n[2] / span), or 0: the box does not go through registers
+  int spare;
+  float orgf[3], incf[9];  // org / inc rounded to fp32 (coordinate type of the 16-bit kernels)
 };
-static_assert(sizeof(TilePlan) == 128, "plan record size");
+static_assert(sizeof(TilePlan) == 208, "plan record size");
 
 struct PlanShape {
   int tiles_x, tiles_y, tiles_z;  // spatial tiles per roi
   int tx, ty, tz;                 // tile extent in output voxels
-  int vec;                        // elements per aligned 8-byte group (0: rows are not aligned)
+  int vec;                        // elements per aligned 16-byte group (0: rows are not aligned)
   int cap;                        // LDS capacity in elements
+  int threads, max_items;         // workgroup size, 16-byte groups one lane holds in registers
 };
 
 __device__ inline void plan_tile(const RoiGeom &g, const RoiProblem &p, const PlanShape &ps,
-                                 unsigned tile, TilePlan *dst) {
+                                 unsigned roi, unsigned tile, TilePlan *dst) {
   const int is3d = p.ndim == 3;
   const int t0[3] = {static_cast<int>(tile % ps.tiles_x) * ps.tx,
                      static_cast<int>((tile / ps.tiles_x) % ps.tiles_y) * ps.ty,
@@ -61,8 +69,9 @@ __device__ inline void plan_tile(const RoiGeom &g, const RoiProblem &p, const Pl
   }
   TilePlan plan;
   plan.batch = g.batch;
+  plan.roi = static_cast<int>(roi);
+  for (int j = 0; j < 3; j++) plan.t0[j] = t0[j];
   bool empty = false, clipped = false;
-  double vol = 1.0;
   for (int a = 0; a < 3; a++) {
     double mid = g.centre[a], reach = 0.0, pos = g.centre[a];
     for (int j = 0; j < 3; j++) {
@@ -83,266 +92,419 @@ __device__ inline void plan_tile(const RoiGeom &g, const RoiProblem &p, const Pl
     clipped |= rmin < 0.0 || rmax > S - 1;
     int l = static_cast<int>(fmin(floor(fmax(rmin, 0.0)), static_cast<double>(S - 1)));
     int h = static_cast<int>(fmin(floor(fmax(rmax, 0.0)) + 1.0, static_cast<double>(S - 1)));
-    if (a == 0 && ps.vec > 0) {  // whole 8-byte groups
+    if (a == 0 && ps.vec > 0) {  // whole 16-byte groups
       l = l / ps.vec * ps.vec;
       h = min((h / ps.vec + 1) * ps.vec, S) - 1;
     }
     plan.lo[a] = l;
     plan.n[a] = h - l + 1;
     plan.org[a] = pos - static_cast<double>(l);
-    vol *= (a == 0) ? static_cast<double>((plan.n[0] + 4) / 4 * 4) : static_cast<double>(plan.n[a]);
   }
+  // LDS row pitch: the row's 16-byte groups, or (unaligned rows) the row plus one finite pad
+  const int groups = ps.vec > 0 ? plan.n[0] / ps.vec : 0;
+  const int pitch = ps.vec > 0 ? plan.n[0] : plan.n[0] + 1;
+  const long rows = static_cast<long>(plan.n[1]) * plan.n[2];
+  // register staging: a pass copies `span` whole z-slices, one 16-byte group per lane
+  plan.rp = 0; plan.span = 0; plan.passes = 0; plan.spare = 0;
+  if (ps.vec > 0) {
+    const int per_slice = plan.n[1] * groups;
+    const int span = min(ps.threads / per_slice, plan.n[2]);
+    if (span >= 1 && (plan.n[2] + span - 1) / span <= ps.max_items) {
+      plan.span = span;
+      plan.rp = span * plan.n[1];
+      plan.passes = (plan.n[2] + span - 1) / span;
+    }
+  }
+  for (int a = 0; a < 3; a++) plan.orgf[a] = static_cast<float>(plan.org[a]);
+  for (int i = 0; i < 9; i++) plan.incf[i] = static_cast<float>(plan.inc[i]);
+  const bool fits = rows * pitch <= ps.cap;
   const bool grid_one = g.grid[0] == 1 && g.grid[1] == 1 && (!is3d || g.grid[2] == 1);
   if (g.batch < 0 || empty || !grid_one) plan.mode = 0;   // (grid != 1 cannot happen: ratio is 1)
-  else if (vol > ps.cap) plan.mode = 2;
+  else if (!fits) plan.mode = 2;
   else plan.mode = clipped ? 1 : 3;
   *dst = plan;
 }
 
-constexpr int kPlanThreads = 256;
-
-// One workgroup per roi: lanes 0..2 evaluate the trigonometry in parallel, lane 0 assembles the
-// geometry, then every lane plans a share of the roi's tiles.
-template <typename RT>
-__global__ __launch_bounds__(kPlanThreads) void roi_plan_kernel(const RT *__restrict__ rois,
-                                                                 TilePlan *__restrict__ plans,
-                                                                 const RoiProblem p,
-                                                                 const PlanShape ps) {
-  __shared__ RoiGeom g;
-  __shared__ double trig[6];
-  const unsigned n = blockIdx.x;
-  build_geom_block(g, trig, rois + static_cast<long>(n) * roi_columns(p.ndim, p.rotated), p);
-  const unsigned per_roi = static_cast<unsigned>(ps.tiles_x) * ps.tiles_y * ps.tiles_z;
-  for (unsigned tile = threadIdx.x; tile < per_roi; tile += kPlanThreads)
-    plan_tile(g, p, ps, tile, plans + static_cast<long>(n) * per_roi + tile);
-}
-
-
-// Two x-neighbouring elements from LDS using naturally aligned accesses only (unaligned LDS reads
-// stall the LDS pipeline).  16-bit types: read the two aligned dwords that contain the pair and
-// shift the pair out; rows start at even element offsets.
-// x-lerp of the pair (tile[idx], tile[idx + 1]) with weight w: a + w * (b - a), written as two
-// FMAs whose 16-bit operands the compiler folds into mixed-precision FMA instructions.
-__device__ __forceinline__ float lerp_pair(const float *tile, int idx, float w) {
-  const float a = tile[idx], b = tile[idx + 1];
-  return fmaf(w, b, fmaf(-w, a, a));
-}
-template <typename H>
-__device__ __forceinline__ unsigned read_pair16(const H *tile, int idx) {
-  const unsigned *w = reinterpret_cast<const unsigned *>(tile) + (idx >> 1);
-  return __builtin_amdgcn_alignbit(w[1], w[0], static_cast<unsigned>(idx & 1) * 16u);
-}
-__device__ __forceinline__ float lerp_pair(const __half *tile, int idx, float w) {
-  const unsigned bits = read_pair16(tile, idx);
-  const float a = __half2float(__ushort_as_half(static_cast<unsigned short>(bits & 0xffffu)));
-  const float b = __half2float(__ushort_as_half(static_cast<unsigned short>(bits >> 16)));
-  return fmaf(w, b, fmaf(-w, a, a));
-}
-__device__ __forceinline__ float lerp_pair(const __hip_bfloat16 *tile, int idx, float w) {
-  const unsigned bits = read_pair16(tile, idx);
-  const float a = __uint_as_float(bits << 16), b = __uint_as_float(bits & 0xffff0000u);
-  return fmaf(w, b, fmaf(-w, a, a));
-}
+constexpr unsigned kChunk = 32;     // consecutive items dealt to one XCD
+constexpr unsigned kPlanSlots = 16; // items per workgroup: their plan records are kept in LDS
+constexpr unsigned kDone = 0xffffffffu;
 
 __device__ __forceinline__ float clamp_ct(float v, float lo, float hi) { return __builtin_amdgcn_fmed3f(v, lo, hi); }
 __device__ __forceinline__ double clamp_ct(double v, double lo, double hi) { return fmin(fmax(v, lo), hi); }
+__device__ __forceinline__ float frac_of(float v) { return __builtin_amdgcn_fractf(v); }
+__device__ __forceinline__ double frac_of(double v) { return __builtin_amdgcn_fract(v); }
+__device__ __forceinline__ float mix(float w, float a, float b) { return fmaf(w, b, fmaf(-w, a, a)); }  // exact at w = 0, 1
+__device__ __forceinline__ int div_small(int i, float inv) { return static_cast<int>((static_cast<float>(i) + 0.5f) * inv); }
 
-template <typename CT> struct BoxLimits { CT vmin[3], vmax[3], cmin[3], cmax[3]; int n1[3]; };
+// Box-relative limits (wave-uniform): a sample is void outside [vmin, vmax]; coordinates clamp to
+// [0, cmax]; the low tap index is at most top = max(n - 2, 0) so that the high tap stays inside
+// the box (a coordinate on the last voxel gets weight 1 on the high tap).
+template <typename CT> struct BoxLimits { CT vmin[3], vmax[3], cmax[3], top[3]; };
 
-// One voxel from the staged box; (rx, ry, rz) are box-relative coordinates.
-template <typename T, typename CT, bool INTERIOR>
+// Element index of the low corner and the three fractions.  fp32 coordinates: floor / fraction /
+// index all in fp32 (indices stay far below 2^24, so the two FMAs are exact).
+__device__ __forceinline__ int corner_index(float lx, float ly, float lz, int pitch, int slice,
+                                            float pitch_f, float slice_f) {
+  return static_cast<int>(fmaf(lz, slice_f, fmaf(ly, pitch_f, lx)));
+}
+__device__ __forceinline__ int corner_index(double lx, double ly, double lz, int pitch, int slice,
+                                            float, float) {
+  return __mul24(static_cast<int>(lz), slice) + __mul24(static_cast<int>(ly), pitch) + static_cast<int>(lx);
+}
+
+// Wide variant for samples taken straight from the feature map.
+template <typename CT>
+__device__ __forceinline__ long corner_index_wide(CT lx, CT ly, CT lz, int pitch, long slice) {
+  return static_cast<long>(lz) * slice + static_cast<long>(static_cast<int>(ly)) * pitch + static_cast<int>(lx);
+}
+
+// One voxel from the staged box; (rx, ry, rz) are box-relative coordinates, dy / dz the element
+// distance to the upper y / z neighbour (0 when the box is one row / slice thick).
+// WIDE: `tile` is the feature map itself (box = whole map), indices need 64 bits.
+template <typename T, typename CT, bool INTERIOR, int ORDER, bool WIDE = false>
 __device__ __forceinline__ float staged_sample(const T *__restrict__ tile, CT rx, CT ry, CT rz,
-                                               const BoxLimits<CT> &b, int pitch, int slice,
-                                               int order) {
+                                               const BoxLimits<CT> &b, int pitch, long slice,
+                                               float pitch_f, float slice_f, int dy, long dz) {
   bool ok = true;
-  if (!INTERIOR) {
+  CT lx, ly, lz;
+  if (INTERIOR) {  // all taps of all samples lie inside the box
+    lx = floor(rx); ly = floor(ry); lz = floor(rz);
+  } else {
     ok = rx >= b.vmin[0] && rx <= b.vmax[0] && ry >= b.vmin[1] && ry <= b.vmax[1] &&
          rz >= b.vmin[2] && rz <= b.vmax[2];
-    rx = clamp_ct(rx, b.cmin[0], b.cmax[0]);
-    ry = clamp_ct(ry, b.cmin[1], b.cmax[1]);
-    rz = clamp_ct(rz, b.cmin[2], b.cmax[2]);
+    rx = clamp_ct(rx, CT(0), b.cmax[0]);
+    ry = clamp_ct(ry, CT(0), b.cmax[1]);
+    rz = clamp_ct(rz, CT(0), b.cmax[2]);
+    lx = fmin(floor(rx), b.top[0]); ly = fmin(floor(ry), b.top[1]); lz = fmin(floor(rz), b.top[2]);
   }
-  const CT flx = floor(rx), fly = floor(ry), flz = floor(rz);
-  const CT dx_ = rx - flx, dy_ = ry - fly, dz_ = rz - flz;
-  const float wx = static_cast<float>(dx_), wy = static_cast<float>(dy_), wz = static_cast<float>(dz_);
-  int ix = static_cast<int>(flx), iy = static_cast<int>(fly), iz = static_cast<int>(flz);
-  int dy = pitch, dz = slice;
-  if (!INTERIOR) {  // void samples may lie anywhere: keep every access inside the box
-    ix = min(max(ix, 0), b.n1[0]); iy = min(max(iy, 0), b.n1[1]); iz = min(max(iz, 0), b.n1[2]);
-    dy = iy < b.n1[1] ? pitch : 0;
-    dz = iz < b.n1[2] ? slice : 0;
-  }
-  const int i00 = __mul24(iz, slice) + __mul24(iy, pitch) + ix;
+  const CT fx = rx - lx, fy = ry - ly, fz = rz - lz;
+  const T *t = tile + (WIDE ? corner_index_wide(lx, ly, lz, pitch, slice)
+                            : corner_index(lx, ly, lz, pitch, static_cast<int>(slice), pitch_f, slice_f));
   float v;
-  if (order == 0) {
-    v = load(tile + (i00 + (dz_ <= CT(0.5) ? 0 : dz) + (dy_ <= CT(0.5) ? 0 : dy) + (dx_ <= CT(0.5) ? 0 : 1)));
+  if (ORDER == 0) {
+    v = load(t + ((fz <= CT(0.5) ? 0 : dz) + (fy <= CT(0.5) ? 0 : dy) + (fx <= CT(0.5) ? 0 : 1)));
   } else {
-    const float x00 = lerp_pair(tile, i00, wx), x01 = lerp_pair(tile, i00 + dy, wx);
-    const float x10 = lerp_pair(tile, i00 + dz, wx), x11 = lerp_pair(tile, i00 + dz + dy, wx);
-    const float y0 = x00 + wy * (x01 - x00), y1 = x10 + wy * (x11 - x10);
-    v = y0 + wz * (y1 - y0);
+    const float wx = static_cast<float>(fx), wy = static_cast<float>(fy), wz = static_cast<float>(fz);
+    const float x00 = mix(wx, load(t), load(t + 1)), x01 = mix(wx, load(t + dy), load(t + dy + 1));
+    const float x10 = mix(wx, load(t + dz), load(t + dz + 1));
+    const float x11 = mix(wx, load(t + dz + dy), load(t + dz + dy + 1));
+    v = mix(wz, mix(wy, x00, x01), mix(wy, x10, x11));
   }
   return ok ? v : 0.f;
 }
 
-// Gather path: one column of the tile straight from global memory (sampling grid 1).
-template <typename T>
-__device__ __noinline__ void gather_column(const T *__restrict__ src, T *__restrict__ drow,
-                                           long zstride, int count, double rx, double ry, double rz,
-                                           double sx, double sy, double sz, int D, int H, int W,
-                                           int order) {
-  for (int k = 0; k < count; k++)
-    drow[k * zstride] = store_cast<T>(sample_clamped<T>(src, D, H, W, rz + k * sz, ry + k * sy,
-                                                        rx + k * sx, order));
+// The lane's column of ZPL voxels, box-relative start b0..b2 and per-slice step s0..s2.
+template <typename T, typename CT, bool INTERIOR, int ORDER, int ZPL, bool WIDE = false>
+__device__ __forceinline__ void staged_column(const T *__restrict__ tile, float (&o)[ZPL], CT b0, CT b1,
+                                              CT b2, CT s0, CT s1, CT s2, const BoxLimits<CT> &lim,
+                                              int pitch, long slice, int dy, long dz) {
+  const float pitch_f = static_cast<float>(pitch), slice_f = static_cast<float>(slice);
+#pragma unroll
+  for (int k = 0; k < ZPL; k++) {
+    const CT kk = static_cast<CT>(k);
+    o[k] = staged_sample<T, CT, INTERIOR, ORDER, WIDE>(tile, b0 + kk * s0, b1 + kk * s1, b2 + kk * s2,
+                                                       lim, pitch, slice, pitch_f, slice_f, dy, dz);
+    // keep the scheduler from interleaving all voxels of the column (registers are scarce while
+    // the next box is in flight)
+    if (k % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+  }
 }
 
-template <typename T, int TX, int TY, int TZ, int THREADS, int LDS_BYTES>
-__global__ __launch_bounds__(THREADS) void roi_resample_kernel(
-    const T *__restrict__ feat, const TilePlan *__restrict__ plans, T *__restrict__ out,
-    const int C, const int D, const int H, const int W, const int od, const int oh, const int ow,
-    const int tiles_x, const int tiles_y, const int tiles_z, const unsigned total, const int vec,
-    const int order) {
+// A plan record held by a wave: lane l keeps dword l (the record has 52); fields are pulled into
+// scalar registers with v_readlane.  The records live in LDS, written by the workgroup itself.
+#define MV_PLAN_DW(field) (static_cast<int>(offsetof(TilePlan, field) / 4))
+struct PlanLanes {
+  unsigned v;
+  __device__ __forceinline__ int i32(int dw) const { return static_cast<int>(__builtin_amdgcn_readlane(v, dw)); }
+  __device__ __forceinline__ float f32(int dw) const { return __uint_as_float(__builtin_amdgcn_readlane(v, dw)); }
+  __device__ __forceinline__ double f64(int dw) const {
+    return __hiloint2double(static_cast<int>(__builtin_amdgcn_readlane(v, dw + 1)),
+                            static_cast<int>(__builtin_amdgcn_readlane(v, dw)));
+  }
+  __device__ __forceinline__ int lo(int a) const { return i32(MV_PLAN_DW(lo) + a); }
+  __device__ __forceinline__ int n(int a) const { return i32(MV_PLAN_DW(n) + a); }
+  __device__ __forceinline__ int t0(int a) const { return i32(MV_PLAN_DW(t0) + a); }
+  __device__ __forceinline__ int batch() const { return i32(MV_PLAN_DW(batch)); }
+  __device__ __forceinline__ int mode() const { return i32(MV_PLAN_DW(mode)); }
+  __device__ __forceinline__ int roi() const { return i32(MV_PLAN_DW(roi)); }
+  __device__ __forceinline__ int rp() const { return i32(MV_PLAN_DW(rp)); }
+  __device__ __forceinline__ int span() const { return i32(MV_PLAN_DW(span)); }
+  __device__ __forceinline__ int passes() const { return i32(MV_PLAN_DW(passes)); }
+};
+template <typename CT> __device__ __forceinline__ CT plan_org(const PlanLanes &p, int a);
+template <> __device__ __forceinline__ float plan_org<float>(const PlanLanes &p, int a) { return p.f32(MV_PLAN_DW(orgf) + a); }
+template <> __device__ __forceinline__ double plan_org<double>(const PlanLanes &p, int a) { return p.f64(MV_PLAN_DW(org) + 2 * a); }
+template <typename CT> __device__ __forceinline__ CT plan_inc(const PlanLanes &p, int i);
+template <> __device__ __forceinline__ float plan_inc<float>(const PlanLanes &p, int i) { return p.f32(MV_PLAN_DW(incf) + i); }
+template <> __device__ __forceinline__ double plan_inc<double>(const PlanLanes &p, int i) { return p.f64(MV_PLAN_DW(inc) + 2 * i); }
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+struct BoxShape { int mode, bx, by, bz, rp, span, passes; };  // wave-uniform part of a plan used for staging
+constexpr unsigned kOutOfRange = 0x80000000u;  // beyond every buffer: the load returns zeros
+
+// Persistent workgroups: each takes every `slots`-th item (tile, channel) of its XCD's contiguous
+// range.  Per item:   write the box (loaded into registers during the previous item) to LDS |
+// barrier | store the previous item's outputs, issue the global loads of the next item's box |
+// interpolate this item from LDS into registers | barrier.  Global latency is thereby covered by
+// the interpolation of the previous item, and stores by that of the next.
+// Box rows are copied as 16-byte groups with range-checked buffer loads: lane = (slice, row,
+// group) within a pass of `span` z-slices, one register quad per pass, passes `span` slices apart.
+template <typename T, int TX, int TY, int TZ, int THREADS, int LDS_BYTES, int KMAX>
+__global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
+    const T *__restrict__ feat, const float *__restrict__ rois, T *__restrict__ out, const RoiProblem p, const PlanShape ps, const unsigned total, const unsigned work) {
   using CT = typename std::conditional<(sizeof(T) == 2), float, double>::type;
   constexpr int kCap = LDS_BYTES / sizeof(T);
   constexpr int RZ = THREADS / (TX * TY);  // lane layers along z
   static_assert(RZ >= 1 && RZ * TX * TY == THREADS && TZ % RZ == 0, "tile shape");
   constexpr int ZPL = TZ / RZ;             // consecutive output slices per lane
+  constexpr int V = 16 / sizeof(T);        // elements per 16-byte group
+  constexpr int ES = sizeof(T);
   __shared__ __attribute__((aligned(16))) T tile[kCap];
+  __shared__ TilePlan lplans[kPlanSlots];
+  const int C = p.C, D = p.D, H = p.H, W = p.W, od = p.od, oh = p.oh, ow = p.ow;
+  const int vec = ps.vec, order = p.order;
 
-  // XCD-aware numbering: workgroup ids go round-robin over the XCDs; give each XCD a contiguous
-  // range of tiles.
-  unsigned id = blockIdx.x;
+  // Work distribution: items (channel * tiles + tile) are dealt to the XCDs in chunks of kChunk
+  // consecutive items (workgroup ids go round-robin over the XCDs, each with an L2 of its own, so
+  // tiles processed at the same time share their halos there).  In round i the workgroups of an
+  // XCD take the next `slots` positions of its queue, each workgroup a different one; the
+  // assignment is rotated from round to round so that a workgroup does not get the same tile
+  // position (border: cheap, centre: expensive) in every roi.
+  const unsigned parts = gridDim.x >= kXcds ? kXcds : 1;
+  const unsigned xcd = blockIdx.x % parts, slot = blockIdx.x / parts, slots = gridDim.x / parts;
+  auto item_of = [&](unsigned round) -> unsigned {
+    const unsigned k = round * slots + (slot + round * 27u) % slots;
+    const unsigned item = ((k / kChunk) * parts + xcd) * kChunk + k % kChunk;
+    return item < work ? item : kDone;   // only the last round of a queue is incomplete
+  };
+  const int tid = threadIdx.x;
+  if (item_of(0) == kDone) return;
+
+  // ---- plans of this workgroup's items (at most kPlanSlots): one lane per item, into LDS ------
+  const unsigned per_roi = static_cast<unsigned>(ps.tiles_x) * ps.tiles_y * ps.tiles_z;
   {
-    const unsigned per = total / kXcds;
-    if (id < per * kXcds) id = (id % kXcds) * per + id / kXcds;
-  }
-  const TilePlan &plan = plans[id];  // wave-uniform address: scalar loads
-  const int c = blockIdx.y;
-  const unsigned per_roi = static_cast<unsigned>(tiles_x) * tiles_y * tiles_z;
-  const unsigned n = id / per_roi, tile_id = id % per_roi;
-  const int tx0 = (tile_id % tiles_x) * TX;
-  const int ty0 = ((tile_id / tiles_x) % tiles_y) * TY;
-  const int tz0 = (tile_id / (tiles_x * tiles_y)) * TZ;
-  const int lx = threadIdx.x % TX, ly = (threadIdx.x / TX) % TY, lz = threadIdx.x / (TX * TY);
-  const int ox = tx0 + lx, oy = ty0 + ly, zb = tz0 + lz * ZPL;
-  const int count = (ox < ow && oy < oh) ? min(ZPL, od - zb) : 0;  // may be <= 0
-  const long zstride = static_cast<long>(oh) * ow;
-  T *drow = out + (static_cast<long>(n) * C + c) * od * zstride + (static_cast<long>(zb) * oh + oy) * ow + ox;
-  const int mode = plan.mode;
-
-  if (mode == 0) {
-    for (int k = 0; k < count; k++) drow[k * zstride] = store_cast<T>(0.f);
-    return;
-  }
-  const T *src = feat + (static_cast<long>(plan.batch) * C + c) * static_cast<long>(D) * H * W;
-  // box-relative position of this lane's first voxel and the per-slice increment
-  const double bxr = plan.org[0] + lx * plan.inc[0] + ly * plan.inc[1] + (lz * ZPL) * plan.inc[2];
-  const double byr = plan.org[1] + lx * plan.inc[3] + ly * plan.inc[4] + (lz * ZPL) * plan.inc[5];
-  const double bzr = plan.org[2] + lx * plan.inc[6] + ly * plan.inc[7] + (lz * ZPL) * plan.inc[8];
-  if (mode == 2) {
-    if (count > 0)
-      gather_column<T>(src, drow, zstride, count, bxr + plan.lo[0], byr + plan.lo[1], bzr + plan.lo[2],
-                       plan.inc[2], plan.inc[5], plan.inc[8], D, H, W, order);
-    return;
-  }
-
-  // ---- stage the box ---------------------------------------------------------------------
-  const int bx = plan.n[0], by = plan.n[1], bz = plan.n[2];
-  const int pitch = (bx + 4) / 4 * 4;  // >= bx + 1 (a finite pad ends every row), even
-  const int slice = by * pitch;
-  const int rows = by * bz;
-  {
-    const T *corner = src + (static_cast<long>(plan.lo[2]) * H + plan.lo[1]) * W + plan.lo[0];
-    const float inv_by = 1.0f / static_cast<float>(by);
-    if (vec > 0) {
-      // 8 bytes per lane and item; item i = (row, group).  Eight independent loads are issued
-      // before the first LDS store so that the copy is not serialised on memory latency.
-      constexpr int V = 8 / sizeof(T);
-      constexpr int kBatch = 8;
-      const int groups = bx / V + 1;  // + the pad group (zeros)
-      const int items = rows * groups;
-      const float inv_groups = 1.0f / static_cast<float>(groups);
-      for (int first = threadIdx.x; first < items; first += THREADS * kBatch) {
-        uint2 val[kBatch];
-        int dst_off[kBatch];
+    if (tid < static_cast<int>(kPlanSlots)) {
+      const unsigned r = tid, item = item_of(r);
+      if (item != kDone) {
+        const unsigned idx = C > 1 ? item % total : item, n = idx / per_roi;
+        const float *roi = rois + static_cast<long>(n) * roi_columns(p.ndim, p.rotated);
+        double sn[3], cs[3];
 #pragma unroll
-        for (int u = 0; u < kBatch; u++) {
-          const int i = first + u * THREADS;
-          val[u] = make_uint2(0u, 0u);
-          dst_off[u] = -1;
-          if (i < items) {
-            const int r = static_cast<int>((static_cast<float>(i) + 0.5f) * inv_groups), gi = i - r * groups;
-            const int zz = static_cast<int>((static_cast<float>(r) + 0.5f) * inv_by), yy = r - zz * by;
-            dst_off[u] = r * pitch + gi * V;
-            if (gi * V < bx)
-              val[u] = *reinterpret_cast<const uint2 *>(corner + (static_cast<long>(zz) * H + yy) * W + gi * V);
-          }
-        }
-#pragma unroll
-        for (int u = 0; u < kBatch; u++)
-          if (dst_off[u] >= 0) *reinterpret_cast<uint2 *>(tile + dst_off[u]) = val[u];
-      }
-    } else {
-      int lpr = 1;
-      while (lpr < pitch && lpr < kWave) lpr *= 2;
-      const int lane_e = threadIdx.x & (lpr - 1), lane_r = threadIdx.x / lpr;
-      for (int r = lane_r; r < rows; r += THREADS / lpr) {
-        const int zz = static_cast<int>((static_cast<float>(r) + 0.5f) * inv_by), yy = r - zz * by;
-        const T *row = corner + (static_cast<long>(zz) * H + yy) * W;
-        for (int e = lane_e; e < pitch; e += lpr) tile[r * pitch + e] = e < bx ? row[e] : store_cast<T>(0.f);
+        for (int a = 0; a < 3; a++) roi_trig(roi, p, a, sn[a], cs[a]);
+        RoiGeom g;
+        build_geom(g, roi, p, sn, cs);
+        plan_tile(g, p, ps, n, idx - n * per_roi, &lplans[r]);
       }
     }
   }
   __syncthreads();
-  if (count <= 0) return;
-  const CT b0 = static_cast<CT>(bxr), b1 = static_cast<CT>(byr), b2 = static_cast<CT>(bzr);
-  const CT s0 = static_cast<CT>(plan.inc[2]), s1 = static_cast<CT>(plan.inc[5]), s2 = static_cast<CT>(plan.inc[8]);
-  const int zslice = bz > 1 ? slice : 0;  // a single staged slice has no upper z neighbour
-  BoxLimits<CT> lim;
-  const int size[3] = {W, H, D};
-  for (int a = 0; a < 3; a++) {
-    lim.vmin[a] = static_cast<CT>(-1 - plan.lo[a]); lim.vmax[a] = static_cast<CT>(size[a] - plan.lo[a]);
-    lim.cmin[a] = static_cast<CT>(-plan.lo[a]); lim.cmax[a] = static_cast<CT>(size[a] - 1 - plan.lo[a]);
-    lim.n1[a] = plan.n[a] - 1;
-  }
-  if (mode == 3) {
+  auto fetch_plan = [&](unsigned r) -> PlanLanes {
+    const unsigned lane = tid & (kWave - 1);
+    PlanLanes pl;
+    pl.v = reinterpret_cast<const unsigned *>(&lplans[r])[lane < sizeof(TilePlan) / 4 ? lane : 0];
+    return pl;
+  };
+  unsigned round = 0;
+  unsigned w = item_of(0), wn = item_of(1);
+  unsigned c = C > 1 ? w / total : 0;
+
+  const int lx = tid % TX, ly = (tid / TX) % TY, lz = tid / (TX * TY);
+  const long zstride = static_cast<long>(oh) * ow;
+  const long plane = static_cast<long>(D) * H * W;
+
+  u32x4 val[KMAX];   // the next item's box: 16-byte group (zz0 + u * span, yy, gi) in val[u]
+  int st_zz = 0;     // zz0 of this lane (beyond every box for idle lanes)
+  int st_dst = 0;    // LDS element offset of the lane's first group
+  float o[ZPL];      // the previous item's outputs
+  T *pend_row = out;
+  int pend_count = 0;
+
+  // Issue the loads of one item's box into val[]: the buffer ends with the box's last row, so
+  // passes that run beyond the last z-slice read zeros without a test.
+  auto issue = [&](const PlanLanes &pl, unsigned ch) -> BoxShape {
+    BoxShape sh;
+    sh.mode = pl.mode(); sh.bx = pl.n(0); sh.by = pl.n(1); sh.bz = pl.n(2);
+    sh.rp = pl.rp(); sh.span = pl.span(); sh.passes = pl.passes();
+    const int passes = sh.passes;
+    if (vec == 0 || passes == 0 || (sh.mode != 1 && sh.mode != 3)) return sh;
+    const int bx = sh.bx, by = sh.by, bz = sh.bz;
+    const int groups = bx / V;
+    const int lr = div_small(tid, 1.0f / static_cast<float>(groups)), gi = tid - lr * groups;
+    const int zz = div_small(lr, 1.0f / static_cast<float>(by)), yy = lr - zz * by;
+    const long first = (static_cast<long>(pl.lo(2)) * H + pl.lo(1)) * W + pl.lo(0);
+    const T *corner = feat + (static_cast<long>(pl.batch()) * C + ch) * plane + first;
+    const int extent = (((bz - 1) * H + by - 1) * W + bx) * ES;
+    const __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(corner), 0, extent, 0x00020000);
+    const bool on = lr < sh.rp;
+    const unsigned voff = on ? static_cast<unsigned>(((zz * H + yy) * W + gi * V) * ES) : kOutOfRange;
+    const int stride = sh.span * H * W * ES;
+    st_zz = on ? zz : (1 << 28);
+    st_dst = lr * bx + gi * V;
 #pragma unroll
-    for (int k = 0; k < ZPL; k++) {
-      if (k < count) {
-        const CT kk = static_cast<CT>(k);
-        drow[k * zstride] = store_cast<T>(staged_sample<T, CT, true>(
-            tile, b0 + kk * s0, b1 + kk * s1, b2 + kk * s2, lim, pitch, zslice, order));
+    for (int u = 0; u < KMAX; u++)
+      if (u < passes) val[u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, u * stride, 0);  // wave-uniform test
+    return sh;
+  };
+  BoxShape cur = issue(fetch_plan(0), c);
+  while (true) {
+    const PlanLanes plan = fetch_plan(round);
+    const int mode = cur.mode;
+    const bool staged = mode == 1 || mode == 3;
+    const int bx = cur.bx, by = cur.by, bz = cur.bz;
+    const int pitch = vec > 0 ? bx : bx + 1;  // unaligned rows end with a finite pad
+    const int slice = by * pitch;
+    const T *src = feat + (static_cast<long>(plan.batch()) * C + c) * plane;
+
+    // ---- A: the box into LDS ---------------------------------------------------------------
+    // All loads issued for this item have to be back; waiting here on every path (vmcnt(0), other
+    // counters untouched) keeps the compiler from waiting again after the stores of phase B.
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    if (staged) {
+      const int rows = by * bz;
+      const T *corner = src + (static_cast<long>(plan.lo(2)) * H + plan.lo(1)) * W + plan.lo(0);
+      const float inv_by = 1.0f / static_cast<float>(by);
+      if (vec > 0) {
+        const int passes = cur.passes, groups = bx / V;
+        if (passes > 0) {
+          const int hop = cur.rp * pitch, span = cur.span;
+#pragma unroll
+          for (int u = 0; u < KMAX; u++)
+            if (u < passes && st_zz < bz - u * span) *reinterpret_cast<u32x4 *>(tile + st_dst + u * hop) = val[u];
+        } else {  // boxes with very long rows or very many slices: straight from global memory
+          const float inv_groups = 1.0f / static_cast<float>(groups);
+          for (int i = tid; i < rows * groups; i += THREADS) {
+            const int r = div_small(i, inv_groups), gi = i - r * groups;
+            const int zz = div_small(r, inv_by), yy = r - zz * by;
+            *reinterpret_cast<u32x4 *>(tile + r * pitch + gi * V) =
+                *reinterpret_cast<const u32x4 *>(corner + (static_cast<long>(zz) * H + yy) * W + gi * V);
+          }
+        }
+      } else {
+        int lpr = 1;
+        while (lpr < pitch && lpr < kWave) lpr *= 2;
+        const int lane_e = tid & (lpr - 1), lane_r = tid / lpr;
+        for (int r = lane_r; r < rows; r += THREADS / lpr) {
+          const int zz = div_small(r, inv_by), yy = r - zz * by;
+          const T *row = corner + (static_cast<long>(zz) * H + yy) * W;
+          for (int e = lane_e; e < pitch; e += lpr) tile[r * pitch + e] = e < bx ? row[e] : store_cast<T>(0.f);
+        }
       }
     }
-  } else {
-#pragma unroll 2
-    for (int k = 0; k < count; k++) {
-      const CT kk = static_cast<CT>(k);
-      drow[k * zstride] = store_cast<T>(staged_sample<T, CT, false>(
-          tile, b0 + kk * s0, b1 + kk * s1, b2 + kk * s2, lim, pitch, zslice, order));
+    __syncthreads();
+
+    // ---- B: previous outputs out, next box in flight ------------------------------------------
+#pragma unroll
+    for (int k = 0; k < ZPL; k++)
+      if (k < pend_count) pend_row[k * zstride] = store_cast<T>(o[k]);
+    const bool more = wn != kDone;
+    unsigned cn = 0;
+    BoxShape nxt = cur;
+    if (more) {
+      if (C > 1) cn = wn / total;
+      nxt = issue(fetch_plan(round + 1), cn);
     }
+
+    // ---- C: this item -------------------------------------------------------------------------
+    const int ox = plan.t0(0) + lx, oy = plan.t0(1) + ly, zb = plan.t0(2) + lz * ZPL;
+    const int count = (ox < ow && oy < oh) ? min(ZPL, od - zb) : 0;  // may be <= 0
+    T *drow = out + (static_cast<long>(plan.roi()) * C + c) * od * zstride +
+              (static_cast<long>(zb) * oh + oy) * ow + ox;
+    pend_row = drow;
+    pend_count = count;
+    if (mode == 0) {
+#pragma unroll
+      for (int k = 0; k < ZPL; k++) o[k] = 0.f;
+    } else if (count > 0) {
+      // position of this lane's first voxel and the per-slice increment, relative to the box (to
+      // the feature map for mode 2), in the coordinate type (the box margin covers the rounding
+      // of fp32 arithmetic)
+      const CT fx = static_cast<CT>(lx), fy = static_cast<CT>(ly), fz = static_cast<CT>(lz * ZPL);
+      CT b[3], st[3];
+#pragma unroll
+      for (int a = 0; a < 3; a++) {
+        b[a] = plan_org<CT>(plan, a) + fx * plan_inc<CT>(plan, a * 3) + fy * plan_inc<CT>(plan, a * 3 + 1) +
+               fz * plan_inc<CT>(plan, a * 3 + 2);
+        st[a] = plan_inc<CT>(plan, a * 3 + 2);
+      }
+      BoxLimits<CT> lim;
+      if (mode == 3) {
+        const int dy = by > 1 ? pitch : 0, dz = bz > 1 ? slice : 0;
+        if (order == 0) staged_column<T, CT, true, 0, ZPL>(tile, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, pitch, slice, dy, dz);
+        else staged_column<T, CT, true, 1, ZPL>(tile, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, pitch, slice, dy, dz);
+      } else {
+        const int size[3] = {W, H, D};
+        const int lo[3] = {mode == 2 ? 0 : plan.lo(0), mode == 2 ? 0 : plan.lo(1), mode == 2 ? 0 : plan.lo(2)};
+        const int n[3] = {mode == 2 ? W : bx, mode == 2 ? H : by, mode == 2 ? D : bz};
+        for (int a = 0; a < 3; a++) {
+          lim.vmin[a] = static_cast<CT>(-1 - lo[a]); lim.vmax[a] = static_cast<CT>(size[a] - lo[a]);
+          lim.cmax[a] = static_cast<CT>(size[a] - 1 - lo[a]);
+          lim.top[a] = static_cast<CT>(max(n[a] - 2, 0));
+        }
+        if (mode == 2) {  // the box does not fit in LDS: taps straight from the feature map
+          for (int a = 0; a < 3; a++) b[a] += static_cast<CT>(plan.lo(a));
+          const long hw = static_cast<long>(H) * W;
+          const int dy = H > 1 ? W : 0;
+          const long dz = D > 1 ? hw : 0;
+          if (order == 0) staged_column<T, CT, false, 0, ZPL, true>(src, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, W, hw, dy, dz);
+          else staged_column<T, CT, false, 1, ZPL, true>(src, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, W, hw, dy, dz);
+        } else {
+          const int dy = by > 1 ? pitch : 0, dz = bz > 1 ? slice : 0;
+          if (order == 0) staged_column<T, CT, false, 0, ZPL>(tile, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, pitch, slice, dy, dz);
+          else staged_column<T, CT, false, 1, ZPL>(tile, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, pitch, slice, dy, dz);
+        }
+      }
+    }
+    if (!more) break;
+    __syncthreads();  // every lane is done with the box
+    w = wn; c = cn; cur = nxt;
+    round++;
+    wn = item_of(round + 1);
   }
+#pragma unroll
+  for (int k = 0; k < ZPL; k++)
+    if (k < pend_count) pend_row[k * zstride] = store_cast<T>(o[k]);
 }
 
-template <typename T, int TX, int TY, int TZ, int THREADS, int LDS_BYTES>
+// Compute units of the current device (workgroups resident at once = units * LDS share).
+static unsigned compute_units() {
+  static int cus[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 256;
+  if (dev < 0 || dev >= 64) return 256;
+  if (cus[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cus[dev] = n;
+  }
+  return static_cast<unsigned>(cus[dev]);
+}
+
+template <typename T, int TX, int TY, int TZ, int THREADS, int LDS_BYTES, int KMAX>
 static int launch_resample(const T *feat, const float *rois, T *out, const RoiProblem &p,
                            void *workspace, size_t *need, hipStream_t s) {
   const long tx = (p.ow + TX - 1) / TX, ty = (p.oh + TY - 1) / TY, tz = (p.od + TZ - 1) / TZ;
-  const long total = tx * ty * tz * static_cast<long>(p.R);
-  if (total >= (1L << 31) || p.C > 65535) return -1;
-  if (need) { *need = static_cast<size_t>(total) * sizeof(TilePlan); return MV_OK; }
-  constexpr int V = 8 / sizeof(T);
+  const long per_roi = tx * ty * tz, total = per_roi * static_cast<long>(p.R), work = total * p.C;
+  if (work >= (1L << 31) || static_cast<long>(p.D) * p.H * p.W * sizeof(T) >= (1L << 31)) return -1;
+  if (need) { *need = 0; return MV_OK; }
+  constexpr int V = 16 / sizeof(T);
   PlanShape ps;
   ps.tiles_x = static_cast<int>(tx); ps.tiles_y = static_cast<int>(ty); ps.tiles_z = static_cast<int>(tz);
   ps.tx = TX; ps.ty = TY; ps.tz = TZ;
-  ps.vec = ((p.W % V == 0) && (reinterpret_cast<uintptr_t>(feat) % 8 == 0)) ? V : 0;
+  ps.vec = ((p.W % V == 0) && (reinterpret_cast<uintptr_t>(feat) % 16 == 0)) ? V : 0;
   ps.cap = LDS_BYTES / sizeof(T);
-  TilePlan *plans = static_cast<TilePlan *>(workspace);
-  hipLaunchKernelGGL((roi_plan_kernel<float>), dim3(p.R), dim3(kPlanThreads), 0, s, rois, plans, p, ps);
-  hipLaunchKernelGGL((roi_resample_kernel<T, TX, TY, TZ, THREADS, LDS_BYTES>),
-                     dim3(static_cast<unsigned>(total), p.C), dim3(THREADS), 0, s, feat, plans, out, p.C,
-                     p.D, p.H, p.W, p.od, p.oh, p.ow, ps.tiles_x, ps.tiles_y, ps.tiles_z,
-                     static_cast<unsigned>(total), ps.vec, p.order);
+  ps.threads = THREADS; ps.max_items = KMAX;
+  unsigned blocks = compute_units() * (160u * 1024u / (LDS_BYTES + sizeof(TilePlan) * kPlanSlots + 64u));
+  // As many workgroups as are resident at once, more when that would give one more than
+  // kPlanSlots items (the later ones start as the first finish).
+  if (work < blocks) blocks = static_cast<unsigned>(work);
+  // (a queue holds at most work / 8 + kChunk items and gets blocks / 8 workgroups)
+  const long by_slots = ((work + kPlanSlots - 1) / kPlanSlots + 2 * kXcds + kXcds - 1) / kXcds * kXcds;
+  if (blocks >= kXcds) blocks = blocks / kXcds * kXcds;  // the same number of workgroups on every XCD
+  if (by_slots > blocks && work > kPlanSlots) blocks = static_cast<unsigned>(by_slots);
+  hipLaunchKernelGGL((roi_resample_kernel<T, TX, TY, TZ, THREADS, LDS_BYTES, KMAX>), dim3(blocks),
+                     dim3(THREADS), 0, s, feat, rois, out, p, ps, static_cast<unsigned>(total),
+                     static_cast<unsigned>(work));
   return check_launch("roi_resample_kernel");
 }
 
@@ -352,18 +514,17 @@ int roi_forward_tiled(const void *input, const void *rois, void *output, int dty
                       const RoiProblem &p, void *workspace, size_t *need, hipStream_t s) {
   const long vox = static_cast<long>(p.od) * p.oh * p.ow;
   if (p.sampling_ratio != 1 || vox < 4096 || p.ow < 16 || p.R == 0) return -1;
-  if (!need && !workspace) return -1;
   const float *r = static_cast<const float *>(rois);
   switch (dtype) {
     case MV_F16:
-      return launch_resample<__half, 16, 16, 16, 512, 64 * 1024>(
+      return launch_resample<__half, 16, 16, 16, 512, 76 * 1024, 8>(
           static_cast<const __half *>(input), r, static_cast<__half *>(output), p, workspace, need, s);
     case MV_BF16:
-      return launch_resample<__hip_bfloat16, 16, 16, 16, 512, 64 * 1024>(
+      return launch_resample<__hip_bfloat16, 16, 16, 16, 512, 76 * 1024, 8>(
           static_cast<const __hip_bfloat16 *>(input), r, static_cast<__hip_bfloat16 *>(output), p,
           workspace, need, s);
     case MV_F32:
-      return launch_resample<float, 16, 16, 8, 512, 64 * 1024>(
+      return launch_resample<float, 16, 16, 8, 512, 76 * 1024, 6>(
           static_cast<const float *>(input), r, static_cast<float *>(output), p, workspace, need, s);
     default:
       return -1;
