@@ -208,6 +208,15 @@ int dcn_mfma_forward(const void *x, const void *off, const void *mask, const voi
                      const void *bias, void *y, const DcnDims &s, int dtype, void *workspace,
                      hipStream_t stream);
 
+// matrix-core backward for 16-bit tensors (dcn3d_mfma_backward.hip)
+bool dcn_mfma_backward_supported(const DcnDims &s, int dtype);
+size_t dcn_mfma_backward_workspace_bytes(const DcnDims &s);
+int dcn_mfma_backward(const void *x, const void *off, const void *mask, const void *wt,
+                      const void *gy, void *goff, void *gmask, const DcnDims &s, int dtype,
+                      void *workspace, float **gx32, float **gw32, float **gb32,
+                      hipStream_t stream);
+int dcn_planar_add(const float *gxt, void *gx, const DcnDims &s, int dtype, hipStream_t stream);
+
 static inline int blocks_for(long n, int per_block, int cap) {
   return static_cast<int>(std::min<long>((n + per_block - 1) / per_block, cap));
 }
@@ -236,6 +245,7 @@ size_t mv_dcn3d_backward_workspace_bytes(const mv_dcn3d_shape *shape, int dtype)
   DcnDims s;
   if (make_dcn_dims(s, shape)) return 0;
   if (dtype != MV_F16 && dtype != MV_BF16) return 0;
+  if (dcn_mfma_backward_supported(s, dtype)) return dcn_mfma_backward_workspace_bytes(s);
   // fp32 accumulators for grad_input, grad_weight, grad_bias
   const size_t n = static_cast<size_t>(s.B) * s.Cin * s.P + static_cast<size_t>(s.Cout) * s.cpg * s.K + s.Cout;
   return n * sizeof(float);
@@ -282,6 +292,28 @@ int mv_dcn3d_backward(const void *input, const void *offset, const void *mask, c
   hipStream_t hs = static_cast<hipStream_t>(stream);
   const long n_gx = static_cast<long>(s.B) * s.Cin * s.P, n_gw = static_cast<long>(s.Cout) * s.cpg * s.K;
   float *ws = static_cast<float *>(workspace);
+  if (dcn_mfma_backward_supported(s, dtype)) {
+    float *gx32, *gw32, *gb32;
+    st = dcn_mfma_backward(input, offset, mask, weight, grad_output, grad_offset, grad_mask, s, dtype,
+                           workspace, &gx32, &gw32, &gb32, hs);
+    if (st) return st;
+    st = dcn_planar_add(gx32, grad_input, s, dtype, hs);
+    if (st) return st;
+    MV_DISPATCH(dtype, {
+      if (sizeof(T) == 2) {
+        using G = float;
+        if (grad_bias)
+          hipLaunchKernelGGL((dcn_backward_bias_kernel<T, G>), dim3(s.Cout, s.B), dim3(256), 0, hs,
+                             static_cast<const T *>(grad_output), gb32, s);
+        hipLaunchKernelGGL((dcn_add_from_f32_kernel<T>), dim3(blocks_for(n_gw, 1024, 65536)), dim3(256),
+                           0, hs, static_cast<T *>(grad_weight), gw32, n_gw);
+        if (grad_bias)
+          hipLaunchKernelGGL((dcn_add_from_f32_kernel<T>), dim3(1), dim3(256), 0, hs,
+                             static_cast<T *>(grad_bias), gb32, static_cast<long>(s.Cout));
+      }
+    });
+    return check_launch("dcn3d backward");
+  }
   if (narrow) {
     const long n = n_gx + n_gw + s.Cout;
     hipLaunchKernelGGL(dcn_fill_zero_kernel, dim3(blocks_for(n, 1024, 65536)), dim3(256), 0, hs, ws, n);

@@ -20,52 +20,13 @@
 //     [lane][8] (workspace) so that a fragment is one coalesced 16-byte load per lane (L2 hits).
 // The sampling gather, not the matrix core, bounds this kernel: per (tap, position) 8 corners x
 // Cin channels are fetched, 8 x more bytes than the fragment holds.
-#include "dcn_common.hpp"
+#include "dcn_mfma.hpp"
 
 namespace mv {
 
-typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef float float16_t __attribute__((ext_vector_type(16)));
-
-template <typename T> struct Mfma;
-template <> struct Mfma<__half> {
-  using frag = half8_t;
-  static __device__ __forceinline__ float16_t run(frag a, frag b, float16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ float lo(unsigned w) {
-    return __half2float(__ushort_as_half(static_cast<unsigned short>(w & 0xffffu)));
-  }
-  static __device__ __forceinline__ float hi(unsigned w) {
-    return __half2float(__ushort_as_half(static_cast<unsigned short>(w >> 16)));
-  }
-  static __device__ __forceinline__ unsigned pack(float a, float b) {
-    return static_cast<unsigned>(__half_as_ushort(__float2half_rn(a))) |
-           (static_cast<unsigned>(__half_as_ushort(__float2half_rn(b))) << 16);
-  }
-};
-template <> struct Mfma<__hip_bfloat16> {
-  using frag = bf16x8_t;
-  static __device__ __forceinline__ float16_t run(frag a, frag b, float16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ float lo(unsigned w) { return __uint_as_float(w << 16); }
-  static __device__ __forceinline__ float hi(unsigned w) { return __uint_as_float(w & 0xffff0000u); }
-  static __device__ __forceinline__ unsigned pack(float a, float b) {
-    // round to nearest even on the upper 16 bits
-    const unsigned ua = __float_as_uint(a), ub = __float_as_uint(b);
-    const unsigned ra = (ua + 0x7fffu + ((ua >> 16) & 1u)) >> 16;
-    const unsigned rb = (ub + 0x7fffu + ((ub >> 16) & 1u)) & 0xffff0000u;
-    return ra | rb;
-  }
-};
-
 // x [B, Cin, P] -> xt [B, P, Cin]; one workgroup moves 64 positions of all channels through LDS
 template <typename T>
-__global__ __launch_bounds__(256) void dcn_channels_last_kernel(const T *__restrict__ x,
-                                                                T *__restrict__ xt, int Cin,
-                                                                long P) {
+__global__ void dcn_channels_last_kernel(const T *__restrict__ x, T *__restrict__ xt, int Cin, long P) {
   extern __shared__ unsigned short stage[];  // [64][Cin + 2]
   const int b = blockIdx.y;
   const long p0 = static_cast<long>(blockIdx.x) * 64;
@@ -215,6 +176,16 @@ __global__ __launch_bounds__(256) void dcn_forward_mfma_kernel(
   }
 }
 
+// [B, C, P] -> [B, P, C] for 16-bit elements (dtype only selects the element size)
+int dcn_channels_last(const void *x, void *xt, int B, int C, long P, hipStream_t stream) {
+  const long pblocks = (P + 63) / 64;
+  MV_REQUIRE(pblocks < (1L << 31) && B <= 65535, "volume too large");
+  hipLaunchKernelGGL((dcn_channels_last_kernel<__half>), dim3(static_cast<unsigned>(pblocks), B), dim3(256),
+                     64 * (C + 2) * sizeof(unsigned short), stream, static_cast<const __half *>(x),
+                     static_cast<__half *>(xt), C, P);
+  return check_launch("dcn_channels_last_kernel");
+}
+
 static size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 
 bool dcn_mfma_supported(const DcnDims &s, int dtype) {
@@ -239,11 +210,8 @@ static int dcn_mfma_run(const void *x, const void *off, const void *mask, const 
   T *xt = static_cast<T *>(workspace);
   T *wf = reinterpret_cast<T *>(static_cast<char *>(workspace) +
                                 align256(static_cast<size_t>(s.B) * s.P * s.Cin * 2));
-  const long pblocks = (s.P + 63) / 64;
-  MV_REQUIRE(pblocks < (1L << 31), "volume too large");
-  hipLaunchKernelGGL((dcn_channels_last_kernel<T>), dim3(static_cast<unsigned>(pblocks), s.B), dim3(256),
-                     64 * (s.Cin + 2) * sizeof(unsigned short), stream, static_cast<const T *>(x), xt,
-                     s.Cin, s.P);
+  const int st = dcn_channels_last(x, xt, s.B, s.Cin, s.P, stream);
+  if (st) return st;
   const long frag_lanes = static_cast<long>(s.groups) * s.K * (s.cpg / 16) * (s.opg / 32) * 64;
   hipLaunchKernelGGL((dcn_weight_fragments_kernel<T>), dim3(static_cast<unsigned>((frag_lanes + 255) / 256)),
                      dim3(256), 0, stream, static_cast<const T *>(wt), wf, s);

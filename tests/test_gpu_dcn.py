@@ -86,6 +86,39 @@ def test_matrix_core_path_vs_oracle(ops, oracle, dtype, modulated, groups, dg, s
     assert_close(y, want, FWD_TOL[dtype], "mfma forward")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("modulated,groups,dg,stride,pad,dil,cin,cout,size", [
+    (True, 1, 1, 1, 1, 1, 32, 64, (12, 12, 16)),    # config-4 geometry, Q % 8 == 0
+    (True, 2, 2, 1, 1, 1, 64, 128, (7, 9, 11)),     # groups, deformable groups, ragged tiles, Q odd
+    (False, 1, 2, 2, 1, 2, 64, 32, (9, 10, 12)),    # DCNv1, stride 2, dilation 2, two chunks per group
+    (True, 1, 1, 1, 0, 1, 32, 96, (6, 7, 9))])      # no padding, three 32-row output blocks
+def test_matrix_core_backward_vs_oracle(ops, oracle, dtype, modulated, groups, dg, stride, pad, dil,
+                                        cin, cout, size):
+    """Shapes that take the MFMA backward (channels per group / per deformable group % 32 == 0,
+    outputs per group % 32 == 0): all five gradients against the fp64 oracle."""
+    from medvision_amd.ops.deform_conv_3d import deform_conv
+    from medvision_amd.ops.modulated_deform_conv_3d import modulated_deform_conv
+    g = wl.gen(80 + groups + dg + cout)
+    x, off, mask, w, b = wl.dcn_inputs(g, 2, cin, cout, size, 3, dg, groups, dtype, stride, pad, dil,
+                                       modulated)
+    xs, offs, ms, ws, bs = [None if t is None else t.to(DEV).requires_grad_(True)
+                            for t in (x, off, mask, w, b)]
+    if modulated:
+        y = modulated_deform_conv(xs, offs, ms, ws, bs, stride, pad, dil, groups, dg)
+    else:
+        y = deform_conv(xs, offs, ws, bs, stride, pad, dil, groups, dg, 64)
+    gy = torch.randn(y.shape, generator=g).to(dtype)
+    y.backward(gy.to(DEV))
+    gx, goff, gm, gw, gb = oracle.dcn3d_backward(x, off, mask, w, gy, True, stride, pad, dil, groups, dg)
+    tol = BWD_TOL[dtype]
+    assert_close(xs.grad, gx, tol, "grad input")
+    assert_close(offs.grad, goff, tol, "grad offset")
+    assert_close(ws.grad, gw, tol, "grad weight")
+    assert_close(bs.grad, gb, tol, "grad bias")
+    if modulated:
+        assert_close(ms.grad, gm, tol, "grad mask")
+
+
 def test_config4_full_size_properties(ops):
     """Full config-4 shape [2,32,48^3] -> Cout 64: zero offsets and unit mask reduce DCN to a plain
     convolution (checked against torch's conv3d), and the op is linear in the mask."""
