@@ -171,7 +171,8 @@ __global__ __launch_bounds__(kGwThreads) void dcn_backward_weight_kernel(
   (void)slabs;
 }
 
-// ---- backward 3: grad wrt bias: workgroup = (o, b) --------------------------------------------
+// ---- backward 3: grad wrt bias: workgroup = (o, b, slab of positions) ----------------------------
+constexpr int kBiasSlab = 8192;
 template <typename T, typename G>
 __global__ __launch_bounds__(256) void dcn_backward_bias_kernel(const T *__restrict__ gy,
                                                                 G *__restrict__ gb,
@@ -179,8 +180,9 @@ __global__ __launch_bounds__(256) void dcn_backward_bias_kernel(const T *__restr
   using A = typename Acc<T>::type;
   const int o = blockIdx.x, b = blockIdx.y;
   const T *src = gy + (static_cast<long>(b) * s.Cout + o) * s.Q;
+  const long q_end = min(static_cast<long>(blockIdx.z + 1) * kBiasSlab, s.Q);
   A v = A(0);
-  for (long q = threadIdx.x; q < s.Q; q += 256) v += load(src + q);
+  for (long q = static_cast<long>(blockIdx.z) * kBiasSlab + threadIdx.x; q < q_end; q += 256) v += load(src + q);
   __shared__ A part[4];
   for (int d = kWave / 2; d > 0; d >>= 1) v += __shfl_down(v, d, kWave);
   if (threadIdx.x % kWave == 0) part[threadIdx.x / kWave] = v;
@@ -303,7 +305,7 @@ int mv_dcn3d_backward(const void *input, const void *offset, const void *mask, c
       if (sizeof(T) == 2) {
         using G = float;
         if (grad_bias)
-          hipLaunchKernelGGL((dcn_backward_bias_kernel<T, G>), dim3(s.Cout, s.B), dim3(256), 0, hs,
+          hipLaunchKernelGGL((dcn_backward_bias_kernel<T, G>), dim3(s.Cout, s.B, static_cast<unsigned>((s.Q + kBiasSlab - 1) / kBiasSlab)), dim3(256), 0, hs,
                              static_cast<const T *>(grad_output), gb32, s);
         hipLaunchKernelGGL((dcn_add_from_f32_kernel<T>), dim3(blocks_for(n_gw, 1024, 65536)), dim3(256),
                            0, hs, static_cast<T *>(grad_weight), gw32, n_gw);
@@ -342,7 +344,7 @@ int mv_dcn3d_backward(const void *input, const void *offset, const void *mask, c
                        static_cast<const T *>(offset), static_cast<const T *>(mask),
                        static_cast<const T *>(grad_output), gw, s, slabs);
     if (grad_bias)
-      hipLaunchKernelGGL((dcn_backward_bias_kernel<T, G>), dim3(s.Cout, s.B), dim3(256), 0, hs,
+      hipLaunchKernelGGL((dcn_backward_bias_kernel<T, G>), dim3(s.Cout, s.B, static_cast<unsigned>((s.Q + kBiasSlab - 1) / kBiasSlab)), dim3(256), 0, hs,
                          static_cast<const T *>(grad_output), gb, s);
     if (sizeof(T) == 2) {
       hipLaunchKernelGGL((dcn_add_from_f32_kernel<T>), dim3(blocks_for(n_gx, 1024, 65536)), dim3(256),

@@ -24,6 +24,8 @@
 
 namespace mv {
 
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
 // x [B, Cin, P] -> xt [B, P, Cin]; one workgroup moves 64 positions of all channels through LDS
 template <typename T>
 __global__ void dcn_channels_last_kernel(const T *__restrict__ x, T *__restrict__ xt, int Cin, long P) {
@@ -65,7 +67,7 @@ __global__ __launch_bounds__(256) void dcn_weight_fragments_kernel(const T *__re
 }
 
 template <typename T, int MT>
-__global__ __launch_bounds__(256) void dcn_forward_mfma_kernel(
+__global__ __launch_bounds__(256, MT <= 2 ? 4 : 3) void dcn_forward_mfma_kernel(
     const T *__restrict__ xt, const T *__restrict__ off, const T *__restrict__ mask,
     const T *__restrict__ wf, const T *__restrict__ bias, T *__restrict__ y, const DcnDims s) {
   using M = Mfma<T>;
@@ -82,7 +84,8 @@ __global__ __launch_bounds__(256) void dcn_forward_mfma_kernel(
   const int b = blockIdx.z;
   const int ow = qc % s.Wo, oh = (qc / s.Wo) % s.Ho, od = qc / (static_cast<long>(s.Wo) * s.Ho);
   const int bd = od * s.sd - s.pd, bh = oh * s.sh - s.ph, bw = ow * s.sw - s.pw;
-  const T *xb = xt + static_cast<long>(b) * s.P * s.Cin;
+  const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T *>(xt + static_cast<long>(b) * s.P * s.Cin), 0, static_cast<int>(s.P * s.Cin * 2), 0x00020000);
 
   float16_t acc[MT];
 #pragma unroll
@@ -114,25 +117,23 @@ __global__ __launch_bounds__(256) void dcn_forward_mfma_kernel(
       const float fd = floorf(pd), fh = floorf(ph), fw = floorf(pw);
       const int d0 = static_cast<int>(fd), h0 = static_cast<int>(fh), w0 = static_cast<int>(fw);
       const float ld = pd - fd, lh = ph - fh, lw = pw - fw;
-      unsigned coff[8];  // element offset of the corner's channel vector in xt, ~0u = outside
+      unsigned coff[8];  // byte offset of the corner's channel vector in xt
       float cw[8];
 #pragma unroll
       for (int c = 0; c < 8; c++) {
         const int a = c >> 2, bb = (c >> 1) & 1, e = c & 1;
         const int zd = d0 + a, zh = h0 + bb, zw = w0 + e;
         const bool in = ok && zd >= 0 && zd < s.D && zh >= 0 && zh < s.H && zw >= 0 && zw < s.W;
-        coff[c] = in ? static_cast<unsigned>((zd * s.H + zh) * s.W + zw) * cin + h * 8 : ~0u;
+        // byte offset; beyond the buffer for a corner outside the volume: the load returns zeros
+        coff[c] = in ? (static_cast<unsigned>((zd * s.H + zh) * s.W + zw) * cin + h * 8) * 2u : 0x80000000u;
         cw[c] = m * (a ? ld : 1.f - ld) * (bb ? lh : 1.f - lh) * (e ? lw : 1.f - lw);
       }
       for (int cc = cc_lo; cc < cc_hi; cc++) {
         const unsigned c0 = g * s.cpg + cc * 16;
         // this lane's 8 channels of the slice: c0 + h*8 .. + 7
-        uint4 raw[8];
+        u32x4 raw[8];
 #pragma unroll
-        for (int c = 0; c < 8; c++) {
-          raw[c] = make_uint4(0u, 0u, 0u, 0u);
-          if (coff[c] != ~0u) raw[c] = *reinterpret_cast<const uint4 *>(xb + (coff[c] + c0));
-        }
+        for (int c = 0; c < 8; c++) raw[c] = __builtin_amdgcn_raw_buffer_load_b128(xr, coff[c], c0 * 2u, 0);
         const T *wfk = wfg + (static_cast<long>(k) * slices + cc) * blocks * 512;
         uint4 araw[MT];
 #pragma unroll
@@ -192,7 +193,7 @@ bool dcn_mfma_supported(const DcnDims &s, int dtype) {
   if (dtype != MV_F16 && dtype != MV_BF16) return false;
   if (s.cpg % 16 || s.opg % 32 || s.cpd % 16) return false;
   if (s.Cin > 4096 || s.B > 65535) return false;
-  if (static_cast<long>(s.P) * s.Cin >= (1L << 31)) return false;  // 32-bit element offsets
+  if (static_cast<long>(s.P) * s.Cin * 2 >= (1L << 31)) return false;  // 32-bit byte offsets
   return true;
 }
 
