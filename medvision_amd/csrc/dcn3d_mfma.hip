@@ -113,21 +113,14 @@ __global__ __launch_bounds__(256, MT <= 2 ? 4 : 3) void dcn_forward_mfma_kernel(
       o += 3 * s.Q;
       if (mk) mk += s.Q;
       if (++kk == s.kw) { kk = 0; if (++kj == s.kh) { kj = 0; ++ki; } }
-      const bool ok = pd > -1.f && ph > -1.f && pw > -1.f && pd < s.D && ph < s.H && pw < s.W;
-      const float fd = floorf(pd), fh = floorf(ph), fw = floorf(pw);
-      const int d0 = static_cast<int>(fd), h0 = static_cast<int>(fh), w0 = static_cast<int>(fw);
-      const float ld = pd - fd, lh = ph - fh, lw = pw - fw;
-      unsigned coff[8];  // byte offset of the corner's channel vector in xt
+      // byte offsets of the corners' channel vectors in xt (beyond the buffer when outside: such
+      // loads return zeros) and corner weights times the mask
+      CornerTaps t;
+      corner_taps(s, pd, ph, pw, true, cin * 2u, static_cast<unsigned>(h) * 16u, 0x80000000u, t);
       float cw[8];
 #pragma unroll
-      for (int c = 0; c < 8; c++) {
-        const int a = c >> 2, bb = (c >> 1) & 1, e = c & 1;
-        const int zd = d0 + a, zh = h0 + bb, zw = w0 + e;
-        const bool in = ok && zd >= 0 && zd < s.D && zh >= 0 && zh < s.H && zw >= 0 && zw < s.W;
-        // byte offset; beyond the buffer for a corner outside the volume: the load returns zeros
-        coff[c] = in ? (static_cast<unsigned>((zd * s.H + zh) * s.W + zw) * cin + h * 8) * 2u : 0x80000000u;
-        cw[c] = m * (a ? ld : 1.f - ld) * (bb ? lh : 1.f - lh) * (e ? lw : 1.f - lw);
-      }
+      for (int c = 0; c < 8; c++) cw[c] = m * t.w[c];
+      const unsigned *coff = t.at;
       for (int cc = cc_lo; cc < cc_hi; cc++) {
         const unsigned c0 = g * s.cpg + cc * 16;
         // this lane's 8 channels of the slice: c0 + h*8 .. + 7

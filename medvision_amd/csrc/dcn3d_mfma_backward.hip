@@ -104,11 +104,11 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
       if (mk) mk += s.Q;
       if (++kk == s.kw) { kk = 0; if (++kj == s.kh) { kj = 0; ++ki; } }
       CornerTaps t;
-      corner_taps(s, pd, ph, pw, live, t);
+      corner_taps(s, pd, ph, pw, live, 1u, 0u, ~0u, t);
       if (h == 0) {
         float4 *dst = reinterpret_cast<float4 *>(tp[n]);
-        dst[0] = make_float4(__uint_as_float(t.vox[0]), __uint_as_float(t.vox[1]), __uint_as_float(t.vox[2]), __uint_as_float(t.vox[3]));
-        dst[1] = make_float4(__uint_as_float(t.vox[4]), __uint_as_float(t.vox[5]), __uint_as_float(t.vox[6]), __uint_as_float(t.vox[7]));
+        dst[0] = make_float4(__uint_as_float(t.at[0]), __uint_as_float(t.at[1]), __uint_as_float(t.at[2]), __uint_as_float(t.at[3]));
+        dst[1] = make_float4(__uint_as_float(t.at[4]), __uint_as_float(t.at[5]), __uint_as_float(t.at[6]), __uint_as_float(t.at[7]));
         dst[2] = make_float4(t.w[0], t.w[1], t.w[2], t.w[3]);
         dst[3] = make_float4(t.w[4], t.w[5], t.w[6], t.w[7]);
         dst[4] = make_float4(m, t.ld, t.lh, t.lw);
@@ -229,10 +229,10 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
       const float pw = static_cast<float>(ow * s.sw - s.pw + kk * s.dw) + load(ob + 2 * s.Q + qc);
       const float m = mb_ ? load(mb_ + qc) : 1.f;
       CornerTaps t;
-      corner_taps(s, pd, ph, pw, live, t);
+      corner_taps(s, pd, ph, pw, live, 1u, 0u, ~0u, t);
       float4 *dst = reinterpret_cast<float4 *>(tp[lane]);
-      dst[0] = make_float4(__uint_as_float(t.vox[0]), __uint_as_float(t.vox[1]), __uint_as_float(t.vox[2]), __uint_as_float(t.vox[3]));
-      dst[1] = make_float4(__uint_as_float(t.vox[4]), __uint_as_float(t.vox[5]), __uint_as_float(t.vox[6]), __uint_as_float(t.vox[7]));
+      dst[0] = make_float4(__uint_as_float(t.at[0]), __uint_as_float(t.at[1]), __uint_as_float(t.at[2]), __uint_as_float(t.at[3]));
+      dst[1] = make_float4(__uint_as_float(t.at[4]), __uint_as_float(t.at[5]), __uint_as_float(t.at[6]), __uint_as_float(t.at[7]));
       dst[2] = make_float4(m * t.w[0], m * t.w[1], m * t.w[2], m * t.w[3]);
       dst[3] = make_float4(m * t.w[4], m * t.w[5], m * t.w[6], m * t.w[7]);
     }

@@ -44,27 +44,34 @@ template <> struct Mfma<__hip_bfloat16> {
 // x [B, C, P] -> xt [B, P, C] for 16-bit elements; defined in dcn3d_mfma.hip
 int dcn_channels_last(const void *x, void *xt, int B, int C, long P, hipStream_t stream);
 
-// The 8 trilinear corners of one (tap, position): voxel index (~0u outside the volume or when the
-// sample is void) and weight; fractions for the derivative.  Positions are exact in fp32 for
-// 16-bit offsets (integer grid position + offset).
+// The 8 trilinear corners of one (tap, position), z-major order: `at[c]` = voxel index * scale + add
+// for a corner inside the volume, `outside` otherwise (also when the sample itself is void, i.e.
+// not -1 < p < size on every axis, or the lane is not live); w[c] the trilinear weight; ld/lh/lw
+// the fractions.  Branch-free: a corner is inside iff its index is, which per axis reads
+//   low  index valid  <=>  0 <= p < size        high index valid  <=>  -1 < p < size - 1.
+// Positions are exact in fp32 for 16-bit offsets (integer grid position + offset).
 struct CornerTaps {
-  unsigned vox[8];
+  unsigned at[8];
   float w[8];
   float ld, lh, lw;
 };
 __device__ __forceinline__ void corner_taps(const DcnDims &s, float pd, float ph, float pw, bool live,
+                                            unsigned scale, unsigned add, unsigned outside,
                                             CornerTaps &t) {
-  const bool ok = live && pd > -1.f && ph > -1.f && pw > -1.f && pd < s.D && ph < s.H && pw < s.W;
   const float fd = floorf(pd), fh = floorf(ph), fw = floorf(pw);
-  const int d0 = static_cast<int>(fd), h0 = static_cast<int>(fh), w0 = static_cast<int>(fw);
   t.ld = pd - fd; t.lh = ph - fh; t.lw = pw - fw;
+  const bool vd[2] = {pd >= 0.f && pd < static_cast<float>(s.D), pd > -1.f && pd < static_cast<float>(s.D - 1)};
+  const bool vh[2] = {ph >= 0.f && ph < static_cast<float>(s.H), ph > -1.f && ph < static_cast<float>(s.H - 1)};
+  const bool vw[2] = {live && pw >= 0.f && pw < static_cast<float>(s.W), live && pw > -1.f && pw < static_cast<float>(s.W - 1)};
+  const int base = (static_cast<int>(fd) * s.H + static_cast<int>(fh)) * s.W + static_cast<int>(fw);
+  const unsigned first = static_cast<unsigned>(base) * scale + add;  // wraps harmlessly when base < 0
+  const unsigned sw = scale, sh = static_cast<unsigned>(s.W) * scale, sd = static_cast<unsigned>(s.H * s.W) * scale;
+  const float wd[2] = {1.f - t.ld, t.ld}, wh[2] = {1.f - t.lh, t.lh}, ww[2] = {1.f - t.lw, t.lw};
 #pragma unroll
   for (int c = 0; c < 8; c++) {
     const int a = c >> 2, bb = (c >> 1) & 1, e = c & 1;
-    const int zd = d0 + a, zh = h0 + bb, zw = w0 + e;
-    const bool in = ok && zd >= 0 && zd < s.D && zh >= 0 && zh < s.H && zw >= 0 && zw < s.W;
-    t.vox[c] = in ? static_cast<unsigned>((zd * s.H + zh) * s.W + zw) : ~0u;
-    t.w[c] = (a ? t.ld : 1.f - t.ld) * (bb ? t.lh : 1.f - t.lh) * (e ? t.lw : 1.f - t.lw);
+    t.at[c] = (vd[a] && vh[bb] && vw[e]) ? first + a * sd + bb * sh + e * sw : outside;
+    t.w[c] = wd[a] * wh[bb] * ww[e];
   }
 }
 
