@@ -76,7 +76,18 @@ def bench_dcn(args, dtype=torch.float16):
 
     ms, _ = _events_ms(step, max(3, args.steps // 10), max(1, args.warmup // 5))
     flops = 2 * 2 * 64 * 32 * 27 * 48 ** 3
-    return {"ms": ms, "tflops": flops / ms / 1e9, "flops": flops}
+
+    # training step (forward + all five gradients), reported beside the forward figure
+    ins = [t.clone().requires_grad_(True) for t in (x, off, mask, w, b)]
+    gy = torch.randn(2, 64, 48, 48, 48, generator=g).to(dtype).to(dev)
+
+    def train_step(i):
+        for t in ins:
+            t.grad = None
+        modulated_deform_conv(*ins, 1, 1, 1, 1, 1).backward(gy)
+
+    train_ms, _ = _events_ms(train_step, max(3, args.steps // 20), 3)
+    return {"ms": ms, "tflops": flops / ms / 1e9, "flops": flops, "train_ms": train_ms}
 
 
 def cpu_baseline(args):
@@ -188,7 +199,7 @@ def main():
                    "buffer_sets": args.copies},
         "roofline": {"bound": "hbm", "achieved": round(a16["gbps"], 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(a16["gbps"] / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "roi_plan_kernel + roi_resample_kernel", "algorithmic_bytes_per_launch": a16["alg_bytes"],
+                     "kernel": "roi_resample_kernel", "algorithmic_bytes_per_launch": a16["alg_bytes"],
                      "avg_launch_us": round(a16["ms"] * 1e3, 3)},
         "fp32": {"gvox_s": round(a32["gvox_s"], 3), "gbps": round(a32["gbps"], 1),
                  "ms_per_step": round(a32["ms"], 6),
@@ -199,6 +210,7 @@ def main():
         line["dcn"] = {"metric": "DCNv2-3D forward (fp16 [2,32,48^3], 3^3, Cout 64)",
                        "value": round(d["tflops"], 3), "unit": "TFLOP/s",
                        "ms_per_step": round(d["ms"], 6),
+                       "forward_backward_ms": round(d["train_ms"], 4),
                        "roofline": {"bound": "mfma", "achieved": round(d["tflops"], 3),
                                     "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                                     "frac": round(d["tflops"] / MFMA_F16_PEAK_TFLOPS, 5),
