@@ -83,10 +83,9 @@ int mv_roi_align_rotated_3d_backward(const void *grad_output, const void *rois, 
                                      int order, void *workspace, void *stream);
 size_t mv_roi_align_backward_workspace_bytes(int dtype, int batch, int channels, int depth,
                                              int height, int width);
-/* Optional workspace of the forward entry points (plain, rotated and affine): with it, outputs of
- * at least 4096 voxels per (roi, channel) at sampling_ratio 1 (Resize / RandomAffine / Crop use)
- * run through the LDS-staged resampling kernel; with NULL every call uses the general kernel.
- * Results do not depend on the choice beyond rounding.  ndim = 2 or 3 (out_d ignored for 2).   */
+/* Workspace of the forward entry points (plain, rotated and affine).  The current kernels keep
+ * their per-call state in LDS, so the query returns 0 and NULL may be passed; callers should
+ * still query and pass what is asked for.  ndim = 2 or 3 (out_d ignored for 2).               */
 size_t mv_roi_align_forward_workspace_bytes(int dtype, int ndim, int channels, int num_rois,
                                             int out_d, int out_h, int out_w, int sampling_ratio);
 

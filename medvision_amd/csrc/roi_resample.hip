@@ -1,25 +1,22 @@
 // Forward resampling for LARGE outputs per roi (Resize / RandomAffine / Crop: one roi produces a
 // whole volume) with a sampling grid of 1x1x1.  Used by the rotated, plain and affine entry
-// points whenever one (roi, channel) yields at least a few thousand voxels and the caller passes
-// a workspace.
+// points whenever one (roi, channel) yields at least a few thousand voxels.
 //
-// Two launches:
-//   plan kernel    one lane per output tile (TX x TY x TZ voxels of one roi): builds the roi's
-//                  affine sample map r = Rot * p + centre in fp64 (three sincos), the interval
-//                  each source axis covers for the tile (centre +- sum_j |Rot[a][j]| * halfspan_j)
-//                  and from it the axis-aligned box of source voxels to stage, clipped to the
-//                  volume.  Writes one 128-byte tile plan: box, mode and the affine map expressed
-//                  relative to the box origin (position of the tile's first voxel + the three
-//                  per-voxel increments).
-//   resample kernel one workgroup per (tile, channel).  If the box fits in LDS the workgroup
-//                  copies it with coalesced 8-byte row loads and every lane produces a column of
-//                  the tile from LDS: lanes run along x, so LDS reads of neighbouring lanes touch
-//                  neighbouring banks and output stores are coalesced.  Otherwise (strong
-//                  down-scaling, extreme rotations) lanes gather from global memory.
+// One launch of persistent workgroups.  An item is (output tile of TX x TY x TZ voxels, channel):
+//   planning   (prologue) one lane per item of the workgroup: the roi's affine sample map
+//              r = Rot * p + centre in fp64, the interval each source axis covers for the tile
+//              (centre +- sum_j |Rot[a][j]| * halfspan_j) and from it the axis-aligned box of
+//              source voxels to stage, clipped to the volume; the map is re-expressed relative to
+//              the box origin.  The 208-byte records stay in LDS.
+//   staging    the box is copied to LDS as 16-byte row groups; the loads of item i+1 are issued
+//              into registers before item i is interpolated.
+//   sampling   every lane produces a column of the tile from LDS: lanes run along x, so LDS reads
+//              of neighbouring lanes touch neighbouring banks and output stores are coalesced.
+//              Boxes larger than the LDS buffer (strong down-scaling) are sampled straight from
+//              global memory by the same code.
 // Coordinates: box-relative, one FMA per axis and voxel in the coordinate type CT (fp32 for 16-bit
 // tensors, fp64 for fp32 tensors), then floor / fraction in CT.  Tiles whose box is not clipped
-// skip the [-1,S] tests and the border clamps.  Workgroup ids are permuted so that the workgroups
-// resident on one XCD (own L2) process neighbouring tiles and share their halos in that L2.
+// skip the [-1,S] tests and the border clamps.
 #include "common.hpp"
 #include "roi_geometry.hpp"
 #include "sampling.hpp"
