@@ -212,7 +212,7 @@ int dcn_mfma_forward(const void *x, const void *off, const void *mask, const voi
 
 // matrix-core backward for 16-bit tensors (dcn3d_mfma_backward.hip)
 bool dcn_mfma_backward_supported(const DcnDims &s, int dtype);
-size_t dcn_mfma_backward_workspace_bytes(const DcnDims &s);
+size_t dcn_mfma_backward_workspace_bytes(const DcnDims &s, int dtype);
 int dcn_mfma_backward(const void *x, const void *off, const void *mask, const void *wt,
                       const void *gy, void *goff, void *gmask, const DcnDims &s, int dtype,
                       void *workspace, float **gx32, float **gw32, float **gb32,
@@ -246,8 +246,8 @@ size_t mv_dcn3d_forward_workspace_bytes(const mv_dcn3d_shape *shape, int dtype) 
 size_t mv_dcn3d_backward_workspace_bytes(const mv_dcn3d_shape *shape, int dtype) {
   DcnDims s;
   if (make_dcn_dims(s, shape)) return 0;
+  if (dcn_mfma_backward_supported(s, dtype)) return dcn_mfma_backward_workspace_bytes(s, dtype);
   if (dtype != MV_F16 && dtype != MV_BF16) return 0;
-  if (dcn_mfma_backward_supported(s, dtype)) return dcn_mfma_backward_workspace_bytes(s);
   // fp32 accumulators for grad_input, grad_weight, grad_bias
   const size_t n = static_cast<size_t>(s.B) * s.Cin * s.P + static_cast<size_t>(s.Cout) * s.cpg * s.K + s.Cout;
   return n * sizeof(float);
@@ -290,7 +290,8 @@ int mv_dcn3d_backward(const void *input, const void *offset, const void *mask, c
   MV_REQUIRE((mask == nullptr) == (grad_mask == nullptr) || grad_mask == nullptr,
              "grad_mask given without mask");
   const bool narrow = dtype == MV_F16 || dtype == MV_BF16;
-  MV_REQUIRE(!narrow || workspace, "16-bit backward needs an fp32 workspace");
+  MV_REQUIRE((!narrow && !dcn_mfma_backward_supported(s, dtype)) || workspace,
+             "this backward needs a workspace of mv_dcn3d_backward_workspace_bytes()");
   hipStream_t hs = static_cast<hipStream_t>(stream);
   const long n_gx = static_cast<long>(s.B) * s.Cin * s.P, n_gw = static_cast<long>(s.Cout) * s.cpg * s.K;
   float *ws = static_cast<float *>(workspace);
@@ -302,7 +303,7 @@ int mv_dcn3d_backward(const void *input, const void *offset, const void *mask, c
     st = dcn_planar_add(gx32, grad_input, s, dtype, hs);
     if (st) return st;
     MV_DISPATCH(dtype, {
-      if (sizeof(T) == 2) {
+      if (sizeof(T) <= 4) {
         using G = float;
         if (grad_bias)
           hipLaunchKernelGGL((dcn_backward_bias_kernel<T, G>), dim3(s.Cout, s.B, static_cast<unsigned>((s.Q + kBiasSlab - 1) / kBiasSlab)), dim3(256), 0, hs,

@@ -24,17 +24,17 @@
 
 namespace mv {
 
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-
 // x [B, Cin, P] -> xt [B, P, Cin]; one workgroup moves 64 positions of all channels through LDS
-template <typename T>
-__global__ void dcn_channels_last_kernel(const T *__restrict__ x, T *__restrict__ xt, int Cin, long P) {
-  extern __shared__ unsigned short stage[];  // [64][Cin + 2]
+// (U = unsigned short / unsigned int: only the element size matters)
+template <typename U>
+__global__ void dcn_channels_last_kernel(const U *__restrict__ x, U *__restrict__ xt, int Cin, long P) {
+  extern __shared__ unsigned char stage_raw[];
+  U *stage = reinterpret_cast<U *>(stage_raw);  // [64][Cin + 2]
   const int b = blockIdx.y;
   const long p0 = static_cast<long>(blockIdx.x) * 64;
   const int pitch = Cin + 2;
-  const unsigned short *src = reinterpret_cast<const unsigned short *>(x) + static_cast<long>(b) * Cin * P;
-  unsigned short *dst = reinterpret_cast<unsigned short *>(xt) + (static_cast<long>(b) * P + p0) * Cin;
+  const U *src = x + static_cast<long>(b) * Cin * P;
+  U *dst = xt + (static_cast<long>(b) * P + p0) * Cin;
   const int lp = threadIdx.x % 64;
   for (int c = threadIdx.x / 64; c < Cin; c += 4)
     if (p0 + lp < P) stage[lp * pitch + c] = src[static_cast<long>(c) * P + p0 + lp];
@@ -46,12 +46,13 @@ __global__ void dcn_channels_last_kernel(const T *__restrict__ x, T *__restrict_
   }
 }
 
-// weight [Cout, cpg, K] -> A fragments [group][tap][slice][row block][lane][8]
+// weight [Cout, cpg, K] -> A pieces [group][tap][slice][row block][lane][kPiece]
 template <typename T>
 __global__ __launch_bounds__(256) void dcn_weight_fragments_kernel(const T *__restrict__ wt,
                                                                    T *__restrict__ wf,
                                                                    const DcnDims s) {
-  const int slices = s.cpg / 16, blocks = s.opg / 32;
+  constexpr int PC = Mfma<T>::kPiece;
+  const int slices = s.cpg / (2 * PC), blocks = s.opg / 32;
   const long total = static_cast<long>(s.groups) * s.K * slices * blocks * 64;
   const long id = blockIdx.x * 256L + threadIdx.x;
   if (id >= total) return;
@@ -62,8 +63,8 @@ __global__ __launch_bounds__(256) void dcn_weight_fragments_kernel(const T *__re
   const int k = r % s.K;
   const int g = static_cast<int>(r / s.K);
   const int o = g * s.opg + mb * 32 + lane % 32;
-  const int cl = cc * 16 + (lane / 32) * 8;
-  for (int i = 0; i < 8; i++) wf[id * 8 + i] = wt[(static_cast<long>(o) * s.cpg + cl + i) * s.K + k];
+  const int cl = cc * 2 * PC + (lane / 32) * PC;
+  for (int i = 0; i < PC; i++) wf[id * PC + i] = wt[(static_cast<long>(o) * s.cpg + cl + i) * s.K + k];
 }
 
 template <typename T, int MT>
@@ -71,6 +72,8 @@ __global__ __launch_bounds__(256, MT <= 2 ? 4 : 3) void dcn_forward_mfma_kernel(
     const T *__restrict__ xt, const T *__restrict__ off, const T *__restrict__ mask,
     const T *__restrict__ wf, const T *__restrict__ bias, T *__restrict__ y, const DcnDims s) {
   using M = Mfma<T>;
+  using P = typename std::conditional<(sizeof(T) == 2), float, double>::type;  // position type
+  constexpr int PC = M::kPiece, SL = 2 * PC, ES = sizeof(T);
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int n = lane % 32, h = lane / 32;
   const long q0 = (static_cast<long>(blockIdx.x) * 4 + wave) * 32;
@@ -78,14 +81,14 @@ __global__ __launch_bounds__(256, MT <= 2 ? 4 : 3) void dcn_forward_mfma_kernel(
   const long q = q0 + n;
   const bool live = q < s.Q;
   const long qc = live ? q : s.Q - 1;
-  const int slices = s.cpg / 16, blocks = s.opg / 32;
+  const int slices = s.cpg / SL, blocks = s.opg / 32;
   const int chunks = (blocks + MT - 1) / MT;
   const int g = blockIdx.y / chunks, mb0 = (blockIdx.y % chunks) * MT;
   const int b = blockIdx.z;
   const int ow = qc % s.Wo, oh = (qc / s.Wo) % s.Ho, od = qc / (static_cast<long>(s.Wo) * s.Ho);
   const int bd = od * s.sd - s.pd, bh = oh * s.sh - s.ph, bw = ow * s.sw - s.pw;
   const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<T *>(xt + static_cast<long>(b) * s.P * s.Cin), 0, static_cast<int>(s.P * s.Cin * 2), 0x00020000);
+      const_cast<T *>(xt + static_cast<long>(b) * s.P * s.Cin), 0, static_cast<int>(s.P * s.Cin * ES), 0x00020000);
 
   float16_t acc[MT];
 #pragma unroll
@@ -93,22 +96,22 @@ __global__ __launch_bounds__(256, MT <= 2 ? 4 : 3) void dcn_forward_mfma_kernel(
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[m][r] = 0.f;
 
-  // deformable groups that intersect this convolution group's channels, and the 16-channel
-  // slices of each (cpd % 16 == 0, so a slice never straddles two deformable groups)
+  // deformable groups that intersect this convolution group's channels, and the channel slices
+  // of each (cpd % 16 == 0, so a slice never straddles two deformable groups)
   const int dg_first = g * s.cpg / s.cpd, dg_last = (g * s.cpg + s.cpg - 1) / s.cpd;
   const unsigned cin = s.Cin;
-  const T *wfg = wf + ((static_cast<long>(g) * s.K * slices) * blocks + mb0) * 512 + lane * 8;
+  const T *wfg = wf + ((static_cast<long>(g) * s.K * slices) * blocks + mb0) * (64 * PC) + lane * PC;
   for (int dgi = dg_first; dgi <= dg_last; dgi++) {
     const int c_lo = max(g * s.cpg, dgi * s.cpd), c_hi = min(g * s.cpg + s.cpg, (dgi + 1) * s.cpd);
-    const int cc_lo = (c_lo - g * s.cpg) / 16, cc_hi = (c_hi - g * s.cpg) / 16;
+    const int cc_lo = (c_lo - g * s.cpg) / SL, cc_hi = (c_hi - g * s.cpg) / SL;
     const long bg = static_cast<long>(b) * s.dg + dgi;
     const T *o = off + bg * 3 * s.K * s.Q + qc;
     const T *mk = mask ? mask + bg * s.K * s.Q + qc : nullptr;
     int ki = 0, kj = 0, kk = 0;
     for (int k = 0; k < s.K; k++) {
-      const float pd = static_cast<float>(bd + ki * s.dd) + load(o);
-      const float ph = static_cast<float>(bh + kj * s.dh) + load(o + s.Q);
-      const float pw = static_cast<float>(bw + kk * s.dw) + load(o + 2 * s.Q);
+      const P pd = static_cast<P>(bd + ki * s.dd) + static_cast<P>(load(o));
+      const P ph = static_cast<P>(bh + kj * s.dh) + static_cast<P>(load(o + s.Q));
+      const P pw = static_cast<P>(bw + kk * s.dw) + static_cast<P>(load(o + 2 * s.Q));
       const float m = mk ? load(mk) : 1.f;
       o += 3 * s.Q;
       if (mk) mk += s.Q;
@@ -116,43 +119,31 @@ __global__ __launch_bounds__(256, MT <= 2 ? 4 : 3) void dcn_forward_mfma_kernel(
       // byte offsets of the corners' channel vectors in xt (beyond the buffer when outside: such
       // loads return zeros) and corner weights times the mask
       CornerTaps t;
-      corner_taps(s, pd, ph, pw, true, cin * 2u, static_cast<unsigned>(h) * 16u, 0x80000000u, t);
+      corner_taps<P>(s, pd, ph, pw, true, cin * ES, static_cast<unsigned>(h) * 16u, 0x80000000u, t);
       float cw[8];
 #pragma unroll
       for (int c = 0; c < 8; c++) cw[c] = m * t.w[c];
       const unsigned *coff = t.at;
       for (int cc = cc_lo; cc < cc_hi; cc++) {
-        const unsigned c0 = g * s.cpg + cc * 16;
-        // this lane's 8 channels of the slice: c0 + h*8 .. + 7
+        const unsigned c0 = g * s.cpg + cc * SL;
+        // this lane's channels of the slice: c0 + h * PC .. + PC - 1, one 16-byte load per corner
         u32x4 raw[8];
 #pragma unroll
-        for (int c = 0; c < 8; c++) raw[c] = __builtin_amdgcn_raw_buffer_load_b128(xr, coff[c], c0 * 2u, 0);
-        const T *wfk = wfg + (static_cast<long>(k) * slices + cc) * blocks * 512;
-        uint4 araw[MT];
+        for (int c = 0; c < 8; c++) raw[c] = __builtin_amdgcn_raw_buffer_load_b128(xr, coff[c], c0 * ES, 0);
+        const T *wfk = wfg + (static_cast<long>(k) * slices + cc) * blocks * (64 * PC);
+        u32x4 araw[MT];
 #pragma unroll
         for (int mm = 0; mm < MT; mm++)
-          if (mb0 + mm < blocks) araw[mm] = *reinterpret_cast<const uint4 *>(wfk + mm * 512);
-        float v[8];
+          if (mb0 + mm < blocks) araw[mm] = *reinterpret_cast<const u32x4 *>(wfk + mm * (64 * PC));
+        float v[PC];
 #pragma unroll
-        for (int i = 0; i < 8; i++) v[i] = 0.f;
+        for (int i = 0; i < PC; i++) v[i] = 0.f;
 #pragma unroll
-        for (int c = 0; c < 8; c++) {
-          const float w = cw[c];
-          v[0] += w * M::lo(raw[c].x); v[1] += w * M::hi(raw[c].x);
-          v[2] += w * M::lo(raw[c].y); v[3] += w * M::hi(raw[c].y);
-          v[4] += w * M::lo(raw[c].z); v[5] += w * M::hi(raw[c].z);
-          v[6] += w * M::lo(raw[c].w); v[7] += w * M::hi(raw[c].w);
-        }
-        union { uint4 u; typename M::frag f; } bfrag;
-        bfrag.u = make_uint4(M::pack(v[0], v[1]), M::pack(v[2], v[3]), M::pack(v[4], v[5]), M::pack(v[6], v[7]));
+        for (int c = 0; c < 8; c++) M::fma_piece(v, cw[c], raw[c]);
+        const u32x4 bfrag = M::pack(v);
 #pragma unroll
-        for (int mm = 0; mm < MT; mm++) {
-          if (mb0 + mm < blocks) {
-            union { uint4 u; typename M::frag f; } afrag;
-            afrag.u = araw[mm];
-            acc[mm] = M::run(afrag.f, bfrag.f, acc[mm]);
-          }
-        }
+        for (int mm = 0; mm < MT; mm++)
+          if (mb0 + mm < blocks) acc[mm] = M::run(araw[mm], bfrag, acc[mm]);
       }
     }
   }
@@ -170,30 +161,36 @@ __global__ __launch_bounds__(256, MT <= 2 ? 4 : 3) void dcn_forward_mfma_kernel(
   }
 }
 
-// [B, C, P] -> [B, P, C] for 16-bit elements (dtype only selects the element size)
-int dcn_channels_last(const void *x, void *xt, int B, int C, long P, hipStream_t stream) {
+// [B, C, P] -> [B, P, C] for elements of 2 or 4 bytes
+int dcn_channels_last(const void *x, void *xt, int B, int C, long P, int elem_bytes, hipStream_t stream) {
   const long pblocks = (P + 63) / 64;
   MV_REQUIRE(pblocks < (1L << 31) && B <= 65535, "volume too large");
-  hipLaunchKernelGGL((dcn_channels_last_kernel<__half>), dim3(static_cast<unsigned>(pblocks), B), dim3(256),
-                     64 * (C + 2) * sizeof(unsigned short), stream, static_cast<const __half *>(x),
-                     static_cast<__half *>(xt), C, P);
+  const dim3 grid(static_cast<unsigned>(pblocks), B);
+  if (elem_bytes == 2)
+    hipLaunchKernelGGL((dcn_channels_last_kernel<unsigned short>), grid, dim3(256), 64 * (C + 2) * 2, stream,
+                       static_cast<const unsigned short *>(x), static_cast<unsigned short *>(xt), C, P);
+  else
+    hipLaunchKernelGGL((dcn_channels_last_kernel<unsigned int>), grid, dim3(256), 64 * (C + 2) * 4, stream,
+                       static_cast<const unsigned int *>(x), static_cast<unsigned int *>(xt), C, P);
   return check_launch("dcn_channels_last_kernel");
 }
 
 static size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+static int elem_size(int dtype) { return dtype == MV_F32 ? 4 : 2; }
 
 bool dcn_mfma_supported(const DcnDims &s, int dtype) {
-  if (dtype != MV_F16 && dtype != MV_BF16) return false;
+  if (dtype != MV_F16 && dtype != MV_BF16 && dtype != MV_F32) return false;
   if (s.cpg % 16 || s.opg % 32 || s.cpd % 16) return false;
   if (s.Cin > 4096 || s.B > 65535) return false;
-  if (static_cast<long>(s.P) * s.Cin * 2 >= (1L << 31)) return false;  // 32-bit byte offsets
+  if (static_cast<long>(s.P) * s.Cin * elem_size(dtype) >= (1L << 31)) return false;  // 32-bit byte offsets
+  if (static_cast<size_t>(64) * (s.Cin + 2) * elem_size(dtype) > 64 * 1024) return false;  // transpose staging
   return true;
 }
 
 size_t dcn_mfma_workspace_bytes(const DcnDims &s, int dtype) {
-  (void)dtype;
-  const size_t xt = static_cast<size_t>(s.B) * s.P * s.Cin * 2;
-  const size_t wf = static_cast<size_t>(s.Cout) * s.cpg * s.K * 2;
+  const size_t es = elem_size(dtype);
+  const size_t xt = static_cast<size_t>(s.B) * s.P * s.Cin * es;
+  const size_t wf = static_cast<size_t>(s.Cout) * s.cpg * s.K * es;
   return align256(xt) + align256(wf);
 }
 
@@ -201,12 +198,13 @@ template <typename T>
 static int dcn_mfma_run(const void *x, const void *off, const void *mask, const void *wt,
                         const void *bias, void *y, const DcnDims &s, void *workspace,
                         hipStream_t stream) {
+  constexpr int PC = Mfma<T>::kPiece;
   T *xt = static_cast<T *>(workspace);
   T *wf = reinterpret_cast<T *>(static_cast<char *>(workspace) +
-                                align256(static_cast<size_t>(s.B) * s.P * s.Cin * 2));
-  const int st = dcn_channels_last(x, xt, s.B, s.Cin, s.P, stream);
+                                align256(static_cast<size_t>(s.B) * s.P * s.Cin * sizeof(T)));
+  const int st = dcn_channels_last(x, xt, s.B, s.Cin, s.P, sizeof(T), stream);
   if (st) return st;
-  const long frag_lanes = static_cast<long>(s.groups) * s.K * (s.cpg / 16) * (s.opg / 32) * 64;
+  const long frag_lanes = static_cast<long>(s.groups) * s.K * (s.cpg / (2 * PC)) * (s.opg / 32) * 64;
   hipLaunchKernelGGL((dcn_weight_fragments_kernel<T>), dim3(static_cast<unsigned>((frag_lanes + 255) / 256)),
                      dim3(256), 0, stream, static_cast<const T *>(wt), wf, s);
   const int blocks = s.opg / 32;
@@ -230,6 +228,7 @@ int dcn_mfma_forward(const void *x, const void *off, const void *mask, const voi
                      const void *bias, void *y, const DcnDims &s, int dtype, void *workspace,
                      hipStream_t stream) {
   if (dtype == MV_F16) return dcn_mfma_run<__half>(x, off, mask, wt, bias, y, s, workspace, stream);
+  if (dtype == MV_F32) return dcn_mfma_run<float>(x, off, mask, wt, bias, y, s, workspace, stream);
   return dcn_mfma_run<__hip_bfloat16>(x, off, mask, wt, bias, y, s, workspace, stream);
 }
 

@@ -24,13 +24,14 @@ namespace mv {
 constexpr unsigned kOob = 0x80000000u;  // byte offset beyond every buffer: loads give 0, atomics are dropped
 constexpr int kRsrcFlags = 0x00020000;
 
-// weight [Cout, cpg, K] -> B fragments [group][tap][32-channel block][16-row step][lane][8]:
-// lane l, element i = Wt[g*opg + step*16 + (l/32)*8 + i, block*32 + l%32, k]
+// weight [Cout, cpg, K] -> B pieces [group][tap][32-channel block][row step][lane][kPiece]:
+// lane l, element i = Wt[g*opg + step*2*kPiece + (l/32)*kPiece + i, block*32 + l%32, k]
 template <typename T>
 __global__ __launch_bounds__(256) void dcn_weight_bfragments_kernel(const T *__restrict__ wt,
                                                                     T *__restrict__ wb,
                                                                     const DcnDims s) {
-  const int cblocks = s.cpg / 32, steps = s.opg / 16;
+  constexpr int PC = Mfma<T>::kPiece;
+  const int cblocks = s.cpg / 32, steps = s.opg / (2 * PC);
   const long total = static_cast<long>(s.groups) * s.K * cblocks * steps * 64;
   const long id = blockIdx.x * 256L + threadIdx.x;
   if (id >= total) return;
@@ -41,8 +42,15 @@ __global__ __launch_bounds__(256) void dcn_weight_bfragments_kernel(const T *__r
   const int k = r % s.K;
   const int g = static_cast<int>(r / s.K);
   const int cl = cb * 32 + lane % 32;
-  const int o = g * s.opg + st * 16 + (lane / 32) * 8;
-  for (int i = 0; i < 8; i++) wb[id * 8 + i] = wt[(static_cast<long>(o + i) * s.cpg + cl) * s.K + k];
+  const int o = g * s.opg + st * 2 * PC + (lane / 32) * PC;
+  for (int i = 0; i < PC; i++) wb[id * PC + i] = wt[(static_cast<long>(o + i) * s.cpg + cl) * s.K + k];
+}
+
+// One element of x (channels-last) through a range-checked buffer load, as fp32.
+template <typename T>
+__device__ __forceinline__ float load_element(__amdgpu_buffer_rsrc_t rsrc, unsigned byte_offset) {
+  if (sizeof(T) == 4) return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, byte_offset, 0, 0));
+  return Mfma<T>::lo(__builtin_amdgcn_raw_buffer_load_b16(rsrc, byte_offset, 0, 0));
 }
 
 // Sum over the 32 lanes of each half-wavefront; the result is valid in lanes 16..31 and 48..63.
@@ -67,6 +75,8 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
     const T *__restrict__ gyt, const T *__restrict__ wb, float *__restrict__ gxt,
     T *__restrict__ goff, T *__restrict__ gmask, const DcnDims s) {
   using M = Mfma<T>;
+  using P = typename std::conditional<(sizeof(T) == 2), float, double>::type;  // position type
+  constexpr int PC = M::kPiece, SL = 2 * PC, ES = sizeof(T);
   __shared__ __attribute__((aligned(16))) float taps[4][32][kTapWords];
   __shared__ float sums[4][4][32];
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -80,13 +90,13 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
   const int ow = qc % s.Wo, oh = (qc / s.Wo) % s.Ho, od = qc / (static_cast<long>(s.Wo) * s.Ho);
   const int bd = od * s.sd - s.pd, bh = oh * s.sh - s.ph, bw = ow * s.sw - s.pw;
   const long bg = static_cast<long>(b) * s.dg + dgi;
-  const int cblocks = s.cpg / 32, steps = s.opg / 16;
+  const int cblocks = s.cpg / 32, steps = s.opg / SL;
 
   const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<T *>(xt + static_cast<long>(b) * s.P * s.Cin), 0, static_cast<int>(s.P * s.Cin * 2), kRsrcFlags);
+      const_cast<T *>(xt + static_cast<long>(b) * s.P * s.Cin), 0, static_cast<int>(s.P * s.Cin * ES), kRsrcFlags);
   const __amdgpu_buffer_rsrc_t gr = __builtin_amdgcn_make_buffer_rsrc(
       gxt + static_cast<long>(b) * s.P * s.Cin, 0, static_cast<int>(s.P * s.Cin * 4), kRsrcFlags);
-  const T *gyrow = gyt + (static_cast<long>(b) * s.Q + qc) * s.Cout + h * 8;
+  const T *gyrow = gyt + (static_cast<long>(b) * s.Q + qc) * s.Cout + h * PC;
   const T *o = off + bg * 3 * s.K * s.Q + qc;
   const T *mk = mask ? mask + bg * s.K * s.Q + qc : nullptr;
   float(*tp)[kTapWords] = taps[wave];
@@ -96,15 +106,15 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
   for (int k = 0; k < s.K; k++) {
     // ---- taps of (k, q0 + n): both half-wavefronts compute them, the lower one publishes -------
     {
-      const float pd = static_cast<float>(bd + ki * s.dd) + load(o);
-      const float ph = static_cast<float>(bh + kj * s.dh) + load(o + s.Q);
-      const float pw = static_cast<float>(bw + kk * s.dw) + load(o + 2 * s.Q);
+      const P pd = static_cast<P>(bd + ki * s.dd) + static_cast<P>(load(o));
+      const P ph = static_cast<P>(bh + kj * s.dh) + static_cast<P>(load(o + s.Q));
+      const P pw = static_cast<P>(bw + kk * s.dw) + static_cast<P>(load(o + 2 * s.Q));
       const float m = mk ? load(mk) : 1.f;
       o += 3 * s.Q;
       if (mk) mk += s.Q;
       if (++kk == s.kw) { kk = 0; if (++kj == s.kh) { kj = 0; ++ki; } }
       CornerTaps t;
-      corner_taps(s, pd, ph, pw, live, 1u, 0u, ~0u, t);
+      corner_taps<P>(s, pd, ph, pw, live, 1u, 0u, ~0u, t);
       if (h == 0) {
         float4 *dst = reinterpret_cast<float4 *>(tp[n]);
         dst[0] = make_float4(__uint_as_float(t.at[0]), __uint_as_float(t.at[1]), __uint_as_float(t.at[2]), __uint_as_float(t.at[3]));
@@ -125,16 +135,15 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
       float16_t acc;
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[r] = 0.f;
-      const T *wfrag = wb + ((((static_cast<long>(g) * s.K + k) * cblocks + cb) * steps) * 64 + lane) * 8;
+      const T *wfrag = wb + ((((static_cast<long>(g) * s.K + k) * cblocks + cb) * steps) * 64 + lane) * PC;
       const T *arow = gyrow + g * s.opg;
       for (int st = 0; st < steps; st++) {
-        union { uint4 u; typename M::frag f; } a, bf;
-        a.u = live ? *reinterpret_cast<const uint4 *>(arow + st * 16) : make_uint4(0u, 0u, 0u, 0u);
-        bf.u = *reinterpret_cast<const uint4 *>(wfrag + static_cast<long>(st) * 512);
-        acc = M::run(a.f, bf.f, acc);
+        const u32x4 a = live ? *reinterpret_cast<const u32x4 *>(arow + st * SL) : u32x4{0u, 0u, 0u, 0u};
+        const u32x4 bf = *reinterpret_cast<const u32x4 *>(wfrag + static_cast<long>(st) * (64 * PC));
+        acc = M::run(a, bf, acc);
       }
-      const unsigned cbyte2 = static_cast<unsigned>(c0 + n) * 2u, cbyte4 = static_cast<unsigned>(c0 + n) * 4u;
-      const unsigned cin2 = static_cast<unsigned>(s.Cin) * 2u, cin4 = static_cast<unsigned>(s.Cin) * 4u;
+      const unsigned cbyte2 = static_cast<unsigned>(c0 + n) * ES, cbyte4 = static_cast<unsigned>(c0 + n) * 4u;
+      const unsigned cin2 = static_cast<unsigned>(s.Cin) * ES, cin4 = static_cast<unsigned>(s.Cin) * 4u;
       // ---- register r: position 8*(r/4) + 4*h + r%4, channel c0 + n ------------------------------
 #pragma unroll
       for (int r = 0; r < 16; r++) {
@@ -150,9 +159,7 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
 #pragma unroll
         for (int c = 0; c < 8; c++) {
           const bool in = vox[c] != ~0u;
-          const unsigned short raw =
-              __builtin_amdgcn_raw_buffer_load_b16(xr, in ? vox[c] * cin2 + cbyte2 : kOob, 0, 0);
-          v[c] = M::lo(raw);
+          v[c] = load_element<T>(xr, in ? vox[c] * cin2 + cbyte2 : kOob);
           __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(w[c] * gm, gr, in ? vox[c] * cin4 + cbyte4 : kOob, 0, 0);
         }
         float val = 0.f;
@@ -190,6 +197,8 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
     const T *__restrict__ xt, const T *__restrict__ off, const T *__restrict__ mask,
     const T *__restrict__ gy, float *__restrict__ gw, const DcnDims s) {
   using M = Mfma<T>;
+  using P = typename std::conditional<(sizeof(T) == 2), float, double>::type;  // position type
+  constexpr int PC = M::kPiece, SL = 2 * PC, ES = sizeof(T);
   __shared__ __attribute__((aligned(16))) float taps[4][64][16];  // vox[8], w[8] * mask
   __shared__ float part[3][MT][16][64];                           // accumulators of wavefronts 1..3
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -202,11 +211,11 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
   const long bg = static_cast<long>(b) * s.dg + dgi;
   const int ki = k / (s.kh * s.kw), kj = (k / s.kw) % s.kh, kk = k % s.kw;
   const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<T *>(xt + static_cast<long>(b) * s.P * s.Cin), 0, static_cast<int>(s.P * s.Cin * 2), kRsrcFlags);
-  const unsigned cbyte2 = static_cast<unsigned>(c0 + n) * 2u, cin2 = static_cast<unsigned>(s.Cin) * 2u;
+      const_cast<T *>(xt + static_cast<long>(b) * s.P * s.Cin), 0, static_cast<int>(s.P * s.Cin * ES), kRsrcFlags);
+  const unsigned cbyte2 = static_cast<unsigned>(c0 + n) * ES, cin2 = static_cast<unsigned>(s.Cin) * ES;
   const T *ob = off + (bg * 3 * s.K + 3 * k) * s.Q;
   const T *mb_ = mask ? mask + (bg * s.K + k) * s.Q : nullptr;
-  const bool aligned = s.Q % 8 == 0;
+  const bool aligned = s.Q % PC == 0;
   float(*tp)[16] = taps[wave];
   (void)cblocks_all;
 
@@ -224,12 +233,12 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
       const bool live = q < s.Q;
       const long qc = live ? q : s.Q - 1;
       const int ow = qc % s.Wo, oh = (qc / s.Wo) % s.Ho, od = qc / (static_cast<long>(s.Wo) * s.Ho);
-      const float pd = static_cast<float>(od * s.sd - s.pd + ki * s.dd) + load(ob + qc);
-      const float ph = static_cast<float>(oh * s.sh - s.ph + kj * s.dh) + load(ob + s.Q + qc);
-      const float pw = static_cast<float>(ow * s.sw - s.pw + kk * s.dw) + load(ob + 2 * s.Q + qc);
+      const P pd = static_cast<P>(od * s.sd - s.pd + ki * s.dd) + static_cast<P>(load(ob + qc));
+      const P ph = static_cast<P>(oh * s.sh - s.ph + kj * s.dh) + static_cast<P>(load(ob + s.Q + qc));
+      const P pw = static_cast<P>(ow * s.sw - s.pw + kk * s.dw) + static_cast<P>(load(ob + 2 * s.Q + qc));
       const float m = mb_ ? load(mb_ + qc) : 1.f;
       CornerTaps t;
-      corner_taps(s, pd, ph, pw, live, 1u, 0u, ~0u, t);
+      corner_taps<P>(s, pd, ph, pw, live, 1u, 0u, ~0u, t);
       float4 *dst = reinterpret_cast<float4 *>(tp[lane]);
       dst[0] = make_float4(__uint_as_float(t.at[0]), __uint_as_float(t.at[1]), __uint_as_float(t.at[2]), __uint_as_float(t.at[3]));
       dst[1] = make_float4(__uint_as_float(t.at[4]), __uint_as_float(t.at[5]), __uint_as_float(t.at[6]), __uint_as_float(t.at[7]));
@@ -240,41 +249,38 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll 1
-    for (int st = 0; st < 4; st++) {  // 16 positions per MFMA step
-      // B fragment: column n = channel c0 + n, rows = positions st*16 + h*8 + i
-      float col[8];
+    for (int st = 0; st < kWave / SL; st++) {  // SL positions per step
+      // B piece: column n = channel c0 + n, rows = positions st*SL + h*PC + i
+      float col[PC];
 #pragma unroll
-      for (int i = 0; i < 8; i++) {
-        const float4 *src = reinterpret_cast<const float4 *>(tp[st * 16 + h * 8 + i]);
+      for (int i = 0; i < PC; i++) {
+        const float4 *src = reinterpret_cast<const float4 *>(tp[st * SL + h * PC + i]);
         const float4 v0 = src[0], v1 = src[1], w0 = src[2], w1 = src[3];
         const unsigned vox[8] = {__float_as_uint(v0.x), __float_as_uint(v0.y), __float_as_uint(v0.z), __float_as_uint(v0.w),
                                  __float_as_uint(v1.x), __float_as_uint(v1.y), __float_as_uint(v1.z), __float_as_uint(v1.w)};
         const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
         float a = 0.f;
 #pragma unroll
-        for (int c = 0; c < 8; c++) {
-          const unsigned short raw = __builtin_amdgcn_raw_buffer_load_b16(
-              xr, vox[c] != ~0u ? vox[c] * cin2 + cbyte2 : kOob, 0, 0);
-          a += w[c] * M::lo(raw);
-        }
+        for (int c = 0; c < 8; c++)
+          a += w[c] * load_element<T>(xr, vox[c] != ~0u ? vox[c] * cin2 + cbyte2 : kOob);
         col[i] = a;
       }
-      union { uint4 u; typename M::frag f; } bf;
-      bf.u = make_uint4(M::pack(col[0], col[1]), M::pack(col[2], col[3]), M::pack(col[4], col[5]), M::pack(col[6], col[7]));
-      // A fragments: row n = output channel, columns = the same 8 positions
-      const long qa = qg + st * 16 + h * 8;
+      const u32x4 bf = M::pack(col);
+      // A pieces: row n = output channel, columns = the same PC positions
+      const long qa = qg + st * SL + h * PC;
 #pragma unroll
       for (int m = 0; m < MT; m++) {
         const T *grow = gy + (static_cast<long>(b) * s.Cout + g * s.opg + m * 32 + n) * s.Q + qa;
-        union { uint4 u; typename M::frag f; unsigned short e[8]; } a;
-        if (aligned && qa + 8 <= s.Q) {
-          a.u = *reinterpret_cast<const uint4 *>(grow);
+        union { u32x4 u; T e[PC]; } a;
+        if (aligned && qa + PC <= s.Q) {
+          a.u = *reinterpret_cast<const u32x4 *>(grow);
         } else {
+          a.u = u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
-          for (int i = 0; i < 8; i++)
-            a.e[i] = qa + i < s.Q ? reinterpret_cast<const unsigned short *>(grow)[i] : static_cast<unsigned short>(0);
+          for (int i = 0; i < PC; i++)
+            if (qa + i < s.Q) a.e[i] = grow[i];
         }
-        acc[m] = M::run(a.f, bf.f, acc[m]);
+        acc[m] = M::run(a.u, bf, acc[m]);
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -334,8 +340,9 @@ __global__ void dcn_zero_f32_kernel(float *p, long n) {
 static size_t align256b(size_t v) { return (v + 255) / 256 * 256; }
 
 bool dcn_mfma_backward_supported(const DcnDims &s, int dtype) {
-  if (dtype != MV_F16 && dtype != MV_BF16) return false;
+  if (dtype != MV_F16 && dtype != MV_BF16 && dtype != MV_F32) return false;
   if (s.cpg % 32 || s.opg % 32 || s.cpd % 32 || s.opg > 128) return false;
+  if (static_cast<size_t>(64) * (max(s.Cin, s.Cout) + 2) * 4 > 64 * 1024) return false;  // transpose staging
   if (s.B > 65535 || s.dg > 65535) return false;
   if (static_cast<long>(s.P) * s.Cin * 4 >= (1L << 31)) return false;  // 32-bit byte offsets
   if (static_cast<long>(s.Cin / 32) * s.K >= (1L << 31) || (s.Q + kGwChunk - 1) / kGwChunk > 65535) return false;
@@ -346,12 +353,13 @@ bool dcn_mfma_backward_supported(const DcnDims &s, int dtype) {
 struct BackwardLayout {
   size_t xt, gyt, wb, gxt, gw, gb, total;
 };
-static BackwardLayout backward_layout(const DcnDims &s) {
+static BackwardLayout backward_layout(const DcnDims &s, int dtype) {
   BackwardLayout l;
+  const size_t es = dtype == MV_F32 ? 4 : 2;
   size_t at = 0;
-  l.xt = at; at += align256b(static_cast<size_t>(s.B) * s.P * s.Cin * 2);
-  l.gyt = at; at += align256b(static_cast<size_t>(s.B) * s.Q * s.Cout * 2);
-  l.wb = at; at += align256b(static_cast<size_t>(s.Cout) * s.cpg * s.K * 2);
+  l.xt = at; at += align256b(static_cast<size_t>(s.B) * s.P * s.Cin * es);
+  l.gyt = at; at += align256b(static_cast<size_t>(s.B) * s.Q * s.Cout * es);
+  l.wb = at; at += align256b(static_cast<size_t>(s.Cout) * s.cpg * s.K * es);
   l.gxt = at; at += align256b(static_cast<size_t>(s.B) * s.P * s.Cin * 4);
   l.gw = at; at += align256b(static_cast<size_t>(s.Cout) * s.cpg * s.K * 4);
   l.gb = at; at += align256b(static_cast<size_t>(s.Cout) * 4);
@@ -359,22 +367,22 @@ static BackwardLayout backward_layout(const DcnDims &s) {
   return l;
 }
 
-size_t dcn_mfma_backward_workspace_bytes(const DcnDims &s) { return backward_layout(s).total; }
+size_t dcn_mfma_backward_workspace_bytes(const DcnDims &s, int dtype) { return backward_layout(s, dtype).total; }
 
 template <typename T>
 static int backward_run(const void *x, const void *off, const void *mask, const void *wt,
                         const void *gy, void *goff, void *gmask, const DcnDims &s, void *workspace,
-                        float **gx32, float **gw32, float **gb32, hipStream_t stream) {
-  const BackwardLayout l = backward_layout(s);
+                        float **gx32, float **gw32, float **gb32, int dtype, hipStream_t stream) {
+  const BackwardLayout l = backward_layout(s, dtype);
   char *ws = static_cast<char *>(workspace);
   T *xt = reinterpret_cast<T *>(ws + l.xt), *gyt = reinterpret_cast<T *>(ws + l.gyt), *wb = reinterpret_cast<T *>(ws + l.wb);
   float *gxt = reinterpret_cast<float *>(ws + l.gxt);
   *gx32 = gxt; *gw32 = reinterpret_cast<float *>(ws + l.gw); *gb32 = reinterpret_cast<float *>(ws + l.gb);
-  int st = dcn_channels_last(x, xt, s.B, s.Cin, s.P, stream);
+  int st = dcn_channels_last(x, xt, s.B, s.Cin, s.P, sizeof(T), stream);
   if (st) return st;
-  st = dcn_channels_last(gy, gyt, s.B, s.Cout, s.Q, stream);
+  st = dcn_channels_last(gy, gyt, s.B, s.Cout, s.Q, sizeof(T), stream);
   if (st) return st;
-  const long frag_lanes = static_cast<long>(s.groups) * s.K * (s.cpg / 32) * (s.opg / 16) * 64;
+  const long frag_lanes = static_cast<long>(s.groups) * s.K * (s.cpg / 32) * (s.opg / (2 * Mfma<T>::kPiece)) * 64;
   hipLaunchKernelGGL((dcn_weight_bfragments_kernel<T>), dim3(static_cast<unsigned>((frag_lanes + 255) / 256)),
                      dim3(256), 0, stream, static_cast<const T *>(wt), wb, s);
   const long nz = static_cast<long>((l.total - l.gxt) / 4);
@@ -408,8 +416,10 @@ int dcn_mfma_backward(const void *x, const void *off, const void *mask, const vo
                       void *workspace, float **gx32, float **gw32, float **gb32,
                       hipStream_t stream) {
   if (dtype == MV_F16)
-    return backward_run<__half>(x, off, mask, wt, gy, goff, gmask, s, workspace, gx32, gw32, gb32, stream);
-  return backward_run<__hip_bfloat16>(x, off, mask, wt, gy, goff, gmask, s, workspace, gx32, gw32, gb32, stream);
+    return backward_run<__half>(x, off, mask, wt, gy, goff, gmask, s, workspace, gx32, gw32, gb32, dtype, stream);
+  if (dtype == MV_F32)
+    return backward_run<float>(x, off, mask, wt, gy, goff, gmask, s, workspace, gx32, gw32, gb32, dtype, stream);
+  return backward_run<__hip_bfloat16>(x, off, mask, wt, gy, goff, gmask, s, workspace, gx32, gw32, gb32, dtype, stream);
 }
 
 int dcn_planar_add(const float *gxt, void *gx, const DcnDims &s, int dtype, hipStream_t stream) {
@@ -419,6 +429,9 @@ int dcn_planar_add(const float *gxt, void *gx, const DcnDims &s, int dtype, hipS
   if (dtype == MV_F16)
     hipLaunchKernelGGL((dcn_planar_add_kernel<__half>), dim3(static_cast<unsigned>(pblocks), s.B), dim3(256), lds,
                        stream, gxt, static_cast<__half *>(gx), s.Cin, s.P);
+  else if (dtype == MV_F32)
+    hipLaunchKernelGGL((dcn_planar_add_kernel<float>), dim3(static_cast<unsigned>(pblocks), s.B), dim3(256), lds,
+                       stream, gxt, static_cast<float *>(gx), s.Cin, s.P);
   else
     hipLaunchKernelGGL((dcn_planar_add_kernel<__hip_bfloat16>), dim3(static_cast<unsigned>(pblocks), s.B), dim3(256),
                        lds, stream, gxt, static_cast<__hip_bfloat16 *>(gx), s.Cin, s.P);

@@ -7,12 +7,19 @@ namespace mv {
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
+// Element-type traits of the matrix-core kernels.  Every operand piece is 16 bytes per lane
+// (`kPiece` elements): for the 16-bit types one piece is the lane's share of a K = 16 fragment of
+// v_mfma_f32_32x32x16 (lane l: row / column l % 32, K indices (l / 32) * 8 .. + 7); for fp32 one
+// piece feeds four v_mfma_f32_32x32x2_f32 (K = 2: lane l holds K index l / 32), element t of the
+// piece in instruction t.  A "slice" is the 2 * kPiece channels (or rows) one such step covers:
+// lane half h = l / 32 owns elements h * kPiece .. + kPiece - 1 of the slice.
 template <typename T> struct Mfma;
 template <> struct Mfma<__half> {
-  using frag = half8_t;
-  static __device__ __forceinline__ float16_t run(frag a, frag b, float16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  static constexpr int kPiece = 8;
+  static __device__ __forceinline__ float16_t run(u32x4 a, u32x4 b, float16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
   }
   static __device__ __forceinline__ float lo(unsigned w) {
     return __half2float(__ushort_as_half(static_cast<unsigned short>(w & 0xffffu)));
@@ -20,49 +27,83 @@ template <> struct Mfma<__half> {
   static __device__ __forceinline__ float hi(unsigned w) {
     return __half2float(__ushort_as_half(static_cast<unsigned short>(w >> 16)));
   }
-  static __device__ __forceinline__ unsigned pack(float a, float b) {
+  static __device__ __forceinline__ unsigned pack2(float a, float b) {
     return static_cast<unsigned>(__half_as_ushort(__float2half_rn(a))) |
            (static_cast<unsigned>(__half_as_ushort(__float2half_rn(b))) << 16);
   }
+  // v[0..7] += w * piece
+  static __device__ __forceinline__ void fma_piece(float (&v)[8], float w, u32x4 r) {
+    v[0] += w * lo(r.x); v[1] += w * hi(r.x); v[2] += w * lo(r.y); v[3] += w * hi(r.y);
+    v[4] += w * lo(r.z); v[5] += w * hi(r.z); v[6] += w * lo(r.w); v[7] += w * hi(r.w);
+  }
+  static __device__ __forceinline__ u32x4 pack(const float (&v)[8]) {
+    return u32x4{pack2(v[0], v[1]), pack2(v[2], v[3]), pack2(v[4], v[5]), pack2(v[6], v[7])};
+  }
 };
 template <> struct Mfma<__hip_bfloat16> {
-  using frag = bf16x8_t;
-  static __device__ __forceinline__ float16_t run(frag a, frag b, float16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  static constexpr int kPiece = 8;
+  static __device__ __forceinline__ float16_t run(u32x4 a, u32x4 b, float16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
   }
   static __device__ __forceinline__ float lo(unsigned w) { return __uint_as_float(w << 16); }
   static __device__ __forceinline__ float hi(unsigned w) { return __uint_as_float(w & 0xffff0000u); }
-  static __device__ __forceinline__ unsigned pack(float a, float b) {
+  static __device__ __forceinline__ unsigned pack2(float a, float b) {
     // round to nearest even on the upper 16 bits
     const unsigned ua = __float_as_uint(a), ub = __float_as_uint(b);
     const unsigned ra = (ua + 0x7fffu + ((ua >> 16) & 1u)) >> 16;
     const unsigned rb = (ub + 0x7fffu + ((ub >> 16) & 1u)) & 0xffff0000u;
     return ra | rb;
   }
+  static __device__ __forceinline__ void fma_piece(float (&v)[8], float w, u32x4 r) {
+    v[0] += w * lo(r.x); v[1] += w * hi(r.x); v[2] += w * lo(r.y); v[3] += w * hi(r.y);
+    v[4] += w * lo(r.z); v[5] += w * hi(r.z); v[6] += w * lo(r.w); v[7] += w * hi(r.w);
+  }
+  static __device__ __forceinline__ u32x4 pack(const float (&v)[8]) {
+    return u32x4{pack2(v[0], v[1]), pack2(v[2], v[3]), pack2(v[4], v[5]), pack2(v[6], v[7])};
+  }
+};
+template <> struct Mfma<float> {
+  static constexpr int kPiece = 4;
+  static __device__ __forceinline__ float16_t run(u32x4 a, u32x4 b, float16_t c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float lo(unsigned w) { return __uint_as_float(w); }
+  static __device__ __forceinline__ void fma_piece(float (&v)[4], float w, u32x4 r) {
+    v[0] += w * __uint_as_float(r.x); v[1] += w * __uint_as_float(r.y);
+    v[2] += w * __uint_as_float(r.z); v[3] += w * __uint_as_float(r.w);
+  }
+  static __device__ __forceinline__ u32x4 pack(const float (&v)[4]) {
+    return u32x4{__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])};
+  }
 };
 
-// x [B, C, P] -> xt [B, P, C] for 16-bit elements; defined in dcn3d_mfma.hip
-int dcn_channels_last(const void *x, void *xt, int B, int C, long P, hipStream_t stream);
+// x [B, C, P] -> xt [B, P, C], elements of `elem_bytes` (2 or 4); defined in dcn3d_mfma.hip
+int dcn_channels_last(const void *x, void *xt, int B, int C, long P, int elem_bytes, hipStream_t stream);
 
 // The 8 trilinear corners of one (tap, position), z-major order: `at[c]` = voxel index * scale + add
 // for a corner inside the volume, `outside` otherwise (also when the sample itself is void, i.e.
 // not -1 < p < size on every axis, or the lane is not live); w[c] the trilinear weight; ld/lh/lw
 // the fractions.  Branch-free: a corner is inside iff its index is, which per axis reads
 //   low  index valid  <=>  0 <= p < size        high index valid  <=>  -1 < p < size - 1.
-// Positions are exact in fp32 for 16-bit offsets (integer grid position + offset).
+// Positions are exact in fp32 for 16-bit offsets (integer grid position + offset); fp32 tensors
+// pass them in fp64 (floor and fraction taken there, the fraction rounded once to fp32).
 struct CornerTaps {
   unsigned at[8];
   float w[8];
   float ld, lh, lw;
 };
-__device__ __forceinline__ void corner_taps(const DcnDims &s, float pd, float ph, float pw, bool live,
+template <typename P>
+__device__ __forceinline__ void corner_taps(const DcnDims &s, P pd, P ph, P pw, bool live,
                                             unsigned scale, unsigned add, unsigned outside,
                                             CornerTaps &t) {
-  const float fd = floorf(pd), fh = floorf(ph), fw = floorf(pw);
-  t.ld = pd - fd; t.lh = ph - fh; t.lw = pw - fw;
-  const bool vd[2] = {pd >= 0.f && pd < static_cast<float>(s.D), pd > -1.f && pd < static_cast<float>(s.D - 1)};
-  const bool vh[2] = {ph >= 0.f && ph < static_cast<float>(s.H), ph > -1.f && ph < static_cast<float>(s.H - 1)};
-  const bool vw[2] = {live && pw >= 0.f && pw < static_cast<float>(s.W), live && pw > -1.f && pw < static_cast<float>(s.W - 1)};
+  const P fd = floor(pd), fh = floor(ph), fw = floor(pw);
+  t.ld = static_cast<float>(pd - fd); t.lh = static_cast<float>(ph - fh); t.lw = static_cast<float>(pw - fw);
+  const bool vd[2] = {pd >= P(0) && pd < static_cast<P>(s.D), pd > P(-1) && pd < static_cast<P>(s.D - 1)};
+  const bool vh[2] = {ph >= P(0) && ph < static_cast<P>(s.H), ph > P(-1) && ph < static_cast<P>(s.H - 1)};
+  const bool vw[2] = {live && pw >= P(0) && pw < static_cast<P>(s.W), live && pw > P(-1) && pw < static_cast<P>(s.W - 1)};
   const int base = (static_cast<int>(fd) * s.H + static_cast<int>(fh)) * s.W + static_cast<int>(fw);
   const unsigned first = static_cast<unsigned>(base) * scale + add;  // wraps harmlessly when base < 0
   const unsigned sw = scale, sh = static_cast<unsigned>(s.W) * scale, sd = static_cast<unsigned>(s.H * s.W) * scale;

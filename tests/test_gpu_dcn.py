@@ -66,7 +66,7 @@ def test_config4_reduced_vs_oracle(ops, oracle, dtype):
     assert_close(y, want, FWD_TOL[dtype], "config 4 forward")
 
 
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("modulated,groups,dg,stride,pad,dil,cin,cout", [
     (True, 2, 2, 1, 1, 1, 64, 128), (False, 1, 2, 2, 1, 2, 32, 32), (True, 1, 1, 1, 0, 1, 16, 160)])
 def test_matrix_core_path_vs_oracle(ops, oracle, dtype, modulated, groups, dg, stride, pad, dil, cin, cout):
@@ -86,7 +86,7 @@ def test_matrix_core_path_vs_oracle(ops, oracle, dtype, modulated, groups, dg, s
     assert_close(y, want, FWD_TOL[dtype], "mfma forward")
 
 
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("modulated,groups,dg,stride,pad,dil,cin,cout,size", [
     (True, 1, 1, 1, 1, 1, 32, 64, (12, 12, 16)),    # config-4 geometry, Q % 8 == 0
     (True, 2, 2, 1, 1, 1, 64, 128, (7, 9, 11)),     # groups, deformable groups, ragged tiles, Q odd
