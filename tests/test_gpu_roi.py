@@ -181,6 +181,48 @@ def test_config3_resize_and_crops(ops, oracle):
     assert set(got.unique().tolist()) <= {0.0, 1.0}
 
 
+@pytest.mark.parametrize("dtype,channels,rois_n,size,out,order", [
+    (torch.float16, 3, 5, (20, 40, 48), (24, 40, 40), 1),    # ragged tiles, several channels and rois
+    (torch.bfloat16, 2, 3, (16, 24, 40), (16, 24, 32), 1),
+    (torch.float32, 3, 4, (20, 40, 44), (24, 40, 40), 1),    # rows of 44 fp32: 16-byte groups
+    (torch.float16, 2, 3, (20, 40, 46), (24, 40, 40), 1),    # rows of 46 fp16: unaligned, element-wise staging
+    (torch.float32, 2, 3, (18, 30, 37), (16, 32, 32), 0),    # unaligned fp32, nearest
+    (torch.float16, 64, 2, (24, 24, 24), (64, 64, 64), 1),   # more items than resident workgroups x 16
+])
+def test_tiled_resampler_shapes(ops, oracle, dtype, channels, rois_n, size, out, order):
+    """The persistent tiled kernel (outputs >= 4096 voxels per roi and channel, sampling_ratio 1) on
+    rotated, scaled, partly outside rois: several channels and rois, output sizes that are not
+    multiples of the tile, feature rows that are / are not multiples of 16 bytes, both orders."""
+    g = wl.gen(31 + channels + rois_n)
+    D, H, W = size
+    feat = torch.randn(2, channels, D, H, W, generator=g).to(dtype)
+    rows = []
+    for r in range(rois_n):
+        c = (torch.rand(3, generator=g) * 0.6 + 0.2) * torch.tensor([W, H, D], dtype=torch.float32)
+        ext = (torch.rand(3, generator=g) * 0.9 + 0.5) * torch.tensor([W, H, D], dtype=torch.float32)
+        ang = (torch.rand(3, generator=g) * 2 - 1) * math.radians(40)
+        rows.append([r % 2, *c.tolist(), *ext.tolist(), *ang.tolist()])
+    rois = torch.tensor(rows, dtype=torch.float32)
+    got = ops.affine_3d(feat.to(DEV), rois.to(DEV), out, 1.0, 1, True, order)
+    want = oracle.roi_align_forward(feat, rois, out, 1.0, 1, True, order, True)
+    if order == 1:
+        assert_close(got, want, FWD_TOL[dtype], "tiled forward")
+    else:
+        mism = (got.cpu().double() != want).float().mean()
+        assert float(mism) < 1e-4, f"nearest mismatches: {float(mism):.2e}"
+
+
+def test_tiled_resampler_2d(ops, oracle):
+    """2-D images through the same kernel (depth-1 volumes)."""
+    g = wl.gen(37)
+    img = torch.randn(2, 3, 96, 120, generator=g).half()
+    rois = torch.tensor([[0, 60.3, 47.1, 130.0, 90.0, 0.4], [1, 50.0, 40.0, 70.0, 110.0, -0.7],
+                         [0, 10.0, 90.0, 60.0, 60.0, 1.3]], dtype=torch.float32)
+    got = ops.affine_2d(img.to(DEV), rois.to(DEV), (80, 96), 1.0, 1, True, 1)
+    want = oracle.roi_align_forward(img, rois, (80, 96), 1.0, 1, True, 1, True)
+    assert_close(got, want, FWD_TOL[torch.float16], "tiled 2-D forward")
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 def test_config5_detection_head_reduced(ops, oracle, dtype):
     """BASELINE config 5 shape family (log-uniform extents, scale 0.25, 7^3, sr=2), reduced."""
