@@ -161,6 +161,146 @@ __global__ __launch_bounds__(256, MT <= 2 ? 4 : 3) void dcn_forward_mfma_kernel(
   }
 }
 
+// ---- 16 x 16 tiling ----------------------------------------------------------------------------
+// The gather is bound by the number of cache-line look-ups: with the 32 x 32 tiling above a lane
+// pair fetches 32 of the 64 (fp16: Cin = 32) bytes of a voxel per instruction, i.e. every voxel is
+// looked up once per 16-channel slice.  With v_mfma_f32_16x16x32 (fp32: 16x16x4) the B operand
+// gives lane l column l % 16 and K piece l / 16: four lanes fetch the four 16-byte pieces of ONE
+// voxel, a load instruction covers 16 positions x 4 * kPiece channels and a voxel is looked up
+// once per 32 (fp32: 16) channels.  The weight pieces of a tap come from LDS (filled by the
+// workgroup one tap ahead) instead of from the vector memory path.
+// weight [Cout, cpg, K] -> A pieces [group][tap][slice][16-row block][lane][kPiece]
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_weight_fragments16_kernel(const T *__restrict__ wt,
+                                                                     T *__restrict__ wf,
+                                                                     const DcnDims s) {
+  constexpr int PC = Mfma<T>::kPiece;
+  const int slices = s.cpg / (4 * PC), blocks = s.opg / 16;
+  const long total = static_cast<long>(s.groups) * s.K * slices * blocks * 64;
+  const long id = blockIdx.x * 256L + threadIdx.x;
+  if (id >= total) return;
+  const int lane = id % 64;
+  long r = id / 64;
+  const int mb = r % blocks; r /= blocks;
+  const int cc = r % slices; r /= slices;
+  const int k = r % s.K;
+  const int g = static_cast<int>(r / s.K);
+  const int o = g * s.opg + mb * 16 + lane % 16;
+  const int cl = cc * 4 * PC + (lane / 16) * PC;
+  for (int i = 0; i < PC; i++) wf[id * PC + i] = wt[(static_cast<long>(o) * s.cpg + cl + i) * s.K + k];
+}
+
+constexpr int kWeightLds = 16 * 1024;  // one tap's weight pieces of a group, per buffer
+
+template <typename T, int MB>
+__global__ __launch_bounds__(256, 4) void dcn_forward_mfma16_kernel(
+    const T *__restrict__ xt, const T *__restrict__ off, const T *__restrict__ mask,
+    const T *__restrict__ wf, const T *__restrict__ bias, T *__restrict__ y, const DcnDims s) {
+  using M = Mfma<T>;
+  using P = typename std::conditional<(sizeof(T) == 2), float, double>::type;  // position type
+  constexpr int PC = M::kPiece, SL = 4 * PC, ES = sizeof(T), NB = 2;
+  __shared__ __attribute__((aligned(16))) unsigned char wlds[2][kWeightLds];
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int j = lane % 16, kc = lane / 16;
+  const long q0 = (static_cast<long>(blockIdx.x) * 4 + wave) * (NB * 16);
+  const int slices = s.cpg / SL, blocks = s.opg / 16;
+  const int chunks = (blocks + MB - 1) / MB;
+  const int g = blockIdx.y / chunks, mb0 = (blockIdx.y % chunks) * MB;
+  const int b = blockIdx.z;
+  const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T *>(xt + static_cast<long>(b) * s.P * s.Cin), 0, static_cast<int>(s.P * s.Cin * ES), 0x00020000);
+
+  long qc[NB];
+  bool live[NB];
+  int bd[NB], bh[NB], bw[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; nb++) {
+    const long q = q0 + nb * 16 + j;
+    live[nb] = q < s.Q;
+    qc[nb] = live[nb] ? q : s.Q - 1;
+    const int ow = qc[nb] % s.Wo, oh = (qc[nb] / s.Wo) % s.Ho, od = qc[nb] / (static_cast<long>(s.Wo) * s.Ho);
+    bd[nb] = od * s.sd - s.pd; bh[nb] = oh * s.sh - s.ph; bw[nb] = ow * s.sw - s.pw;
+  }
+  float4_t acc[NB][MB];
+#pragma unroll
+  for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+    for (int m = 0; m < MB; m++) acc[nb][m] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  // weight pieces of one tap: [slice][block of this chunk][lane] 16 bytes, copied by the workgroup
+  const int tap_pieces = slices * MB * 64;                       // 16-byte pieces per tap
+  const T *wfg = wf + static_cast<long>(g) * s.K * slices * blocks * (64 * PC);
+  auto fill = [&](int k, int buf) {
+    for (int i = threadIdx.x; i < tap_pieces; i += 256) {
+      const int ln = i % 64, m = (i / 64) % MB, cc = i / (64 * MB);
+      u32x4 v = u32x4{0u, 0u, 0u, 0u};
+      if (mb0 + m < blocks)
+        v = *reinterpret_cast<const u32x4 *>(wfg + (((static_cast<long>(k) * slices + cc) * blocks + mb0 + m) * 64 + ln) * PC);
+      reinterpret_cast<u32x4 *>(wlds[buf])[i] = v;
+    }
+  };
+  fill(0, 0);
+  __syncthreads();
+
+  const int dg_first = g * s.cpg / s.cpd, dg_last = (g * s.cpg + s.cpg - 1) / s.cpd;
+  const unsigned cin = s.Cin;
+  int ki = 0, kj = 0, kk = 0;
+  for (int k = 0; k < s.K; k++) {
+    if (k + 1 < s.K) fill(k + 1, (k + 1) & 1);
+    const u32x4 *wl = reinterpret_cast<const u32x4 *>(wlds[k & 1]);
+    for (int dgi = dg_first; dgi <= dg_last; dgi++) {
+      const int c_lo = max(g * s.cpg, dgi * s.cpd), c_hi = min(g * s.cpg + s.cpg, (dgi + 1) * s.cpd);
+      const int cc_lo = (c_lo - g * s.cpg) / SL, cc_hi = (c_hi - g * s.cpg) / SL;
+      const long bg = static_cast<long>(b) * s.dg + dgi;
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++) {
+        const T *o = off + (bg * 3 * s.K + 3 * k) * s.Q + qc[nb];
+        const P pd = static_cast<P>(bd[nb] + ki * s.dd) + static_cast<P>(load(o));
+        const P ph = static_cast<P>(bh[nb] + kj * s.dh) + static_cast<P>(load(o + s.Q));
+        const P pw = static_cast<P>(bw[nb] + kk * s.dw) + static_cast<P>(load(o + 2 * s.Q));
+        const float m = mask ? load(mask + (bg * s.K + k) * s.Q + qc[nb]) : 1.f;
+        CornerTaps t;
+        corner_taps<P>(s, pd, ph, pw, true, cin * ES, static_cast<unsigned>(kc) * 16u, 0x80000000u, t);
+        float cw[8];
+#pragma unroll
+        for (int c = 0; c < 8; c++) cw[c] = m * t.w[c];
+        for (int cc = cc_lo; cc < cc_hi; cc++) {
+          const unsigned c0 = g * s.cpg + cc * SL;
+          u32x4 raw[8];
+#pragma unroll
+          for (int c = 0; c < 8; c++) raw[c] = __builtin_amdgcn_raw_buffer_load_b128(xr, t.at[c], c0 * ES, 0);
+          float v[PC];
+#pragma unroll
+          for (int i = 0; i < PC; i++) v[i] = 0.f;
+#pragma unroll
+          for (int c = 0; c < 8; c++) M::fma_piece(v, cw[c], raw[c]);
+          const u32x4 bpiece = M::pack(v);
+#pragma unroll
+          for (int mm = 0; mm < MB; mm++)
+            acc[nb][mm] = M::run16(wl[(cc * MB + mm) * 64 + lane], bpiece, acc[nb][mm]);
+        }
+      }
+    }
+    if (++kk == s.kw) { kk = 0; if (++kj == s.kh) { kj = 0; ++ki; } }
+    __syncthreads();  // the other buffer is complete, this one may be refilled
+  }
+#pragma unroll
+  for (int nb = 0; nb < NB; nb++) {
+    if (!live[nb] || q0 >= s.Q) continue;
+#pragma unroll
+    for (int m = 0; m < MB; m++) {
+      if (mb0 + m >= blocks) continue;
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        // 16x16 accumulator layout: register r of lane l holds row 4 * (l / 16) + r, column l % 16
+        const int o = g * s.opg + (mb0 + m) * 16 + kc * 4 + r;
+        const float val = acc[nb][m][r] + (bias ? load(bias + o) : 0.f);
+        y[(static_cast<long>(b) * s.Cout + o) * s.Q + q0 + nb * 16 + j] = store_cast<T>(val);
+      }
+    }
+  }
+}
+
 // [B, C, P] -> [B, P, C] for elements of 2 or 4 bytes
 int dcn_channels_last(const void *x, void *xt, int B, int C, long P, int elem_bytes, hipStream_t stream) {
   const long pblocks = (P + 63) / 64;
@@ -204,6 +344,30 @@ static int dcn_mfma_run(const void *x, const void *off, const void *mask, const 
                                 align256(static_cast<size_t>(s.B) * s.P * s.Cin * sizeof(T)));
   const int st = dcn_channels_last(x, xt, s.B, s.Cin, s.P, sizeof(T), stream);
   if (st) return st;
+  // 16 x 16 tiling: whole 4-piece slices per (deformable) group and a tap's weight pieces fit LDS
+  {
+    const int blocks16 = s.opg / 16;
+    const int mb = blocks16 >= 4 ? 4 : (blocks16 >= 2 ? 2 : 1);
+    const long tap_bytes = static_cast<long>(s.cpg / (4 * PC)) * mb * 64 * 16;
+    if (s.cpg % (4 * PC) == 0 && s.cpd % (4 * PC) == 0 && tap_bytes <= kWeightLds) {
+      const long lanes = static_cast<long>(s.groups) * s.K * (s.cpg / (4 * PC)) * blocks16 * 64;
+      hipLaunchKernelGGL((dcn_weight_fragments16_kernel<T>), dim3(static_cast<unsigned>((lanes + 255) / 256)),
+                         dim3(256), 0, stream, static_cast<const T *>(wt), wf, s);
+      const int chunks = (blocks16 + mb - 1) / mb;
+      const long qblocks = (s.Q + 127) / 128;
+      MV_REQUIRE(qblocks < (1L << 31) && static_cast<long>(s.groups) * chunks <= 65535, "grid too large");
+      const dim3 grid(static_cast<unsigned>(qblocks), s.groups * chunks, s.B), block(256);
+#define MV_LAUNCH_MFMA16(MBV)                                                                    \
+  hipLaunchKernelGGL((dcn_forward_mfma16_kernel<T, MBV>), grid, block, 0, stream, xt,            \
+                     static_cast<const T *>(off), static_cast<const T *>(mask), wf,              \
+                     static_cast<const T *>(bias), static_cast<T *>(y), s)
+      if (mb == 4) MV_LAUNCH_MFMA16(4);
+      else if (mb == 2) MV_LAUNCH_MFMA16(2);
+      else MV_LAUNCH_MFMA16(1);
+#undef MV_LAUNCH_MFMA16
+      return check_launch("dcn_forward_mfma16_kernel");
+    }
+  }
   const long frag_lanes = static_cast<long>(s.groups) * s.K * (s.cpg / (2 * PC)) * (s.opg / 32) * 64;
   hipLaunchKernelGGL((dcn_weight_fragments_kernel<T>), dim3(static_cast<unsigned>((frag_lanes + 255) / 256)),
                      dim3(256), 0, stream, static_cast<const T *>(wt), wf, s);

@@ -7,6 +7,7 @@ namespace mv {
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 // Element-type traits of the matrix-core kernels.  Every operand piece is 16 bytes per lane
@@ -15,11 +16,17 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 // piece feeds four v_mfma_f32_32x32x2_f32 (K = 2: lane l holds K index l / 32), element t of the
 // piece in instruction t.  A "slice" is the 2 * kPiece channels (or rows) one such step covers:
 // lane half h = l / 32 owns elements h * kPiece .. + kPiece - 1 of the slice.
+// `run16` is the 16 x 16 counterpart (v_mfma_f32_16x16x32 / four v_mfma_f32_16x16x4_f32): lane l holds
+// row / column l % 16 and the piece l / 16 of a slice of 4 * kPiece; accumulator register r of lane l
+// is row 4 * (l / 16) + r, column l % 16.
 template <typename T> struct Mfma;
 template <> struct Mfma<__half> {
   static constexpr int kPiece = 8;
   static __device__ __forceinline__ float16_t run(u32x4 a, u32x4 b, float16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float4_t run16(u32x4 a, u32x4 b, float4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
   }
   static __device__ __forceinline__ float lo(unsigned w) {
     return __half2float(__ushort_as_half(static_cast<unsigned short>(w & 0xffffu)));
@@ -45,6 +52,9 @@ template <> struct Mfma<__hip_bfloat16> {
   static __device__ __forceinline__ float16_t run(u32x4 a, u32x4 b, float16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
   }
+  static __device__ __forceinline__ float4_t run16(u32x4 a, u32x4 b, float4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  }
   static __device__ __forceinline__ float lo(unsigned w) { return __uint_as_float(w << 16); }
   static __device__ __forceinline__ float hi(unsigned w) { return __uint_as_float(w & 0xffff0000u); }
   static __device__ __forceinline__ unsigned pack2(float a, float b) {
@@ -69,6 +79,12 @@ template <> struct Mfma<float> {
     c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), c, 0, 0, 0);
     c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), c, 0, 0, 0);
     return __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float4_t run16(u32x4 a, u32x4 b, float4_t c) {
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a.x), __uint_as_float(b.x), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a.y), __uint_as_float(b.y), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a.z), __uint_as_float(b.z), c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a.w), __uint_as_float(b.w), c, 0, 0, 0);
   }
   static __device__ __forceinline__ float lo(unsigned w) { return __uint_as_float(w); }
   static __device__ __forceinline__ void fma_piece(float (&v)[4], float w, u32x4 r) {
