@@ -201,7 +201,9 @@ __global__ __launch_bounds__(256, 4) void dcn_forward_mfma16_kernel(
   constexpr int PC = M::kPiece, SL = 4 * PC, ES = sizeof(T), NB = 2;
   __shared__ __attribute__((aligned(16))) unsigned char wlds[2][kWeightLds];
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const int j = lane % 16, kc = lane / 16;
+  const int j = lane % 16, kc = lane / 16;   // matrix layout: position (column) and piece of this lane
+  const int lj = lane / 4, lk = lane % 4;    // load layout
+  const int from = (4 * j + kc) * 4;         // ds_bpermute byte address of the lane holding this lane's piece
   const long q0 = (static_cast<long>(blockIdx.x) * 4 + wave) * (NB * 16);
   const int slices = s.cpg / SL, blocks = s.opg / 16;
   const int chunks = (blocks + MB - 1) / MB;
@@ -210,14 +212,12 @@ __global__ __launch_bounds__(256, 4) void dcn_forward_mfma16_kernel(
   const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<T *>(xt + static_cast<long>(b) * s.P * s.Cin), 0, static_cast<int>(s.P * s.Cin * ES), 0x00020000);
 
-  long qc[NB];
-  bool live[NB];
+  long qc[NB];   // position this lane gathers for (load layout), clamped
   int bd[NB], bh[NB], bw[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) {
-    const long q = q0 + nb * 16 + j;
-    live[nb] = q < s.Q;
-    qc[nb] = live[nb] ? q : s.Q - 1;
+    const long q = q0 + nb * 16 + lj;
+    qc[nb] = q < s.Q ? q : s.Q - 1;
     const int ow = qc[nb] % s.Wo, oh = (qc[nb] / s.Wo) % s.Ho, od = qc[nb] / (static_cast<long>(s.Wo) * s.Ho);
     bd[nb] = od * s.sd - s.pd; bh[nb] = oh * s.sh - s.ph; bw[nb] = ow * s.sw - s.pw;
   }
@@ -260,7 +260,7 @@ __global__ __launch_bounds__(256, 4) void dcn_forward_mfma16_kernel(
         const P pw = static_cast<P>(bw[nb] + kk * s.dw) + static_cast<P>(load(o + 2 * s.Q));
         const float m = mask ? load(mask + (bg * s.K + k) * s.Q + qc[nb]) : 1.f;
         CornerTaps t;
-        corner_taps<P>(s, pd, ph, pw, true, cin * ES, static_cast<unsigned>(kc) * 16u, 0x80000000u, t);
+        corner_taps<P>(s, pd, ph, pw, true, cin * ES, static_cast<unsigned>(lk) * 16u, 0x80000000u, t);
         float cw[8];
 #pragma unroll
         for (int c = 0; c < 8; c++) cw[c] = m * t.w[c];
@@ -274,7 +274,12 @@ __global__ __launch_bounds__(256, 4) void dcn_forward_mfma16_kernel(
           for (int i = 0; i < PC; i++) v[i] = 0.f;
 #pragma unroll
           for (int c = 0; c < 8; c++) M::fma_piece(v, cw[c], raw[c]);
-          const u32x4 bpiece = M::pack(v);
+          const u32x4 mine = M::pack(v);   // piece lk of position lj; wanted: piece kc of position j
+          const u32x4 bpiece = u32x4{
+              static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(from, static_cast<int>(mine.x))),
+              static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(from, static_cast<int>(mine.y))),
+              static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(from, static_cast<int>(mine.z))),
+              static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(from, static_cast<int>(mine.w)))};
 #pragma unroll
           for (int mm = 0; mm < MB; mm++)
             acc[nb][mm] = M::run16(wl[(cc * MB + mm) * 64 + lane], bpiece, acc[nb][mm]);
@@ -286,7 +291,7 @@ __global__ __launch_bounds__(256, 4) void dcn_forward_mfma16_kernel(
   }
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) {
-    if (!live[nb] || q0 >= s.Q) continue;
+    if (q0 + nb * 16 + j >= s.Q) continue;
 #pragma unroll
     for (int m = 0; m < MB; m++) {
       if (mb0 + m >= blocks) continue;
