@@ -43,6 +43,35 @@ struct PoolShared {
   int chunk;       // channels per LDS pass
 };
 
+// The tap entries of one output cell (grid <= kTapRegs samples) in registers; unused entries have
+// weight 0 and index 0.
+constexpr int kTapRegs = 2;
+struct TapRegs {
+  int lo[kTapRegs], hi[kTapRegs];
+  float wlo[kTapRegs], whi[kTapRegs];
+  __device__ __forceinline__ void load(const AxisTaps &t, int cell) {
+#pragma unroll
+    for (int s = 0; s < kTapRegs; s++) {
+      const bool on = s < t.grid;
+      const int e = on ? cell * t.grid + s : 0;
+      lo[s] = on ? t.lo[e] : 0; hi[s] = on ? t.hi[e] : 0;
+      wlo[s] = on ? t.wlo[e] : 0.f; whi[s] = on ? t.whi[e] : 0.f;
+    }
+  }
+  // sum over the entries of w * row[index * stride]
+  template <typename E>
+  __device__ __forceinline__ float apply(const E *row, int stride) const {
+    float acc = 0.f;
+#pragma unroll
+    for (int s = 0; s < kTapRegs; s++)
+      acc += wlo[s] * load_any(row + lo[s] * stride) + whi[s] * load_any(row + hi[s] * stride);
+    return acc;
+  }
+  static __device__ __forceinline__ float load_any(const float *p) { return *p; }
+  static __device__ __forceinline__ float load_any(const __half *p) { return mv::load(p); }
+  static __device__ __forceinline__ float load_any(const __hip_bfloat16 *p) { return mv::load(p); }
+};
+
 // Builds geometry and tap tables for roi `roi`; all threads must call it (contains barriers).
 template <typename RT>
 __device__ inline void pool_setup(PoolShared &sh, const RT *roi, const RoiProblem &p, size_t elem_bytes) {
@@ -172,44 +201,102 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
     float *t2 = t1 + cs * nz * ny * p.ow;                                           // [cs][nz][oh][ow]
     const T *corner = src + static_cast<long>(cb - c_begin) * plane +
                       (static_cast<long>(tz.box_lo) * p.H + ty.box_lo) * p.W + tx.box_lo;
-    for (int i = threadIdx.x; i < cs * vol; i += kPoolThreads) {
-      const int c = fdiv(i, inv_vol), r0 = i - c * vol, z = fdiv(r0, inv_nxy), r1 = r0 - z * nx * ny;
-      const int y = fdiv(r1, inv_nx), x = r1 - y * nx;
-      box[i] = corner[c * plane + (static_cast<long>(z) * p.H + y) * p.W + x];
+    // copy the sub-box: eight independent loads in flight per lane before the first LDS store
+    for (int i0 = threadIdx.x; i0 < cs * vol; i0 += kPoolThreads * 8) {
+      T val[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const int i = i0 + u * kPoolThreads;
+        if (i < cs * vol) {
+          const int c = fdiv(i, inv_vol), r0 = i - c * vol, z = fdiv(r0, inv_nxy), r1 = r0 - z * nx * ny;
+          const int y = fdiv(r1, inv_nx), x = r1 - y * nx;
+          val[u] = corner[c * plane + (static_cast<long>(z) * p.H + y) * p.W + x];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const int i = i0 + u * kPoolThreads;
+        if (i < cs * vol) box[i] = val[u];
+      }
     }
     __syncthreads();
-    for (int i = threadIdx.x; i < cs * nz * ny * p.ow; i += kPoolThreads) {  // contract x
-      const int row = fdiv(i, inv_ow), pw = i - row * p.ow;                 // row = (c, z, y)
-      const T *r = box + row * nx;
-      float acc = 0.f;
-      for (int s = 0; s < gx; s++) {
-        const int e = pw * gx + s;
-        acc += tx.wlo[e] * load(r + tx.lo[e]) + tx.whi[e] * load(r + tx.hi[e]);
+    // Each pass gives a thread a FIXED output coordinate on the contracted axis, so its (at most
+    // kTapRegs) tap entries stay in registers while it walks over the rows; per element that leaves
+    // 2 * grid LDS reads, 2 * grid FMAs and one store.
+    if (gx <= kTapRegs && gy <= kTapRegs && gz <= kTapRegs) {
+      {  // contract x: thread = (row chunk, pw); rows are (c, z, y)
+        int lanes = 1;
+        while (lanes < p.ow) lanes *= 2;
+        const int pw = threadIdx.x % lanes, r0 = threadIdx.x / lanes, step = kPoolThreads / lanes;
+        const int rows = cs * nz * ny;
+        if (pw < p.ow) {
+          TapRegs t;
+          t.load(tx, pw);
+          for (int r = r0; r < rows; r += step) t1[r * p.ow + pw] = t.apply(box + r * nx, 1);
+        }
       }
-      t1[i] = acc;
-    }
-    __syncthreads();
-    for (int i = threadIdx.x; i < cs * nz * p.oh * p.ow; i += kPoolThreads) {  // contract y
-      const int cz = fdiv(i, inv_ohw), hw = i - cz * ohw, ph = fdiv(hw, inv_ow), pw = hw - ph * p.ow;  // cz = (c, z)
-      const float *r = t1 + cz * ny * p.ow + pw;
-      float acc = 0.f;
-      for (int s = 0; s < gy; s++) {
-        const int e = ph * gy + s;
-        acc += ty.wlo[e] * r[ty.lo[e] * p.ow] + ty.whi[e] * r[ty.hi[e] * p.ow];
+      __syncthreads();
+      {  // contract y: thread = (row chunk, ph, pw); rows are (c, z)
+        int lanes = 1;
+        while (lanes < ohw) lanes *= 2;
+        const int cell = threadIdx.x % lanes, r0 = threadIdx.x / lanes, step = kPoolThreads / lanes;
+        const int rows = cs * nz;
+        if (cell < ohw) {
+          const int ph = fdiv(cell, inv_ow), pw = cell - ph * p.ow;
+          TapRegs t;
+          t.load(ty, ph);
+          for (int r = r0; r < rows; r += step) t2[r * ohw + cell] = t.apply(t1 + r * ny * p.ow + pw, p.ow);
+        }
       }
-      t2[i] = acc;
-    }
-    __syncthreads();
-    T *o = dst + static_cast<long>(cb - c_begin) * cells;
-    for (int i = threadIdx.x; i < cs * cells; i += kPoolThreads) {  // contract z, store
-      const int c = fdiv(i, inv_cells), r0 = i - c * cells, pd = fdiv(r0, inv_ohw), hw = r0 - pd * ohw;
-      const float *r = t2 + c * nz * ohw + hw;
-      float acc = 0.f;
-      for (int s = 0; s < gz; s++) {
-        const int e = pd * gz + s;
-        acc += tz.wlo[e] * r[tz.lo[e] * ohw] + tz.whi[e] * r[tz.hi[e] * ohw];
+      __syncthreads();
+      {  // contract z, store: a wavefront takes (pd, half of the channels) items, its lanes run over
+         // (ph, pw): the taps of pd stay in registers over the channels and the stores are coalesced
+        T *o = dst + static_cast<long>(cb - c_begin) * cells;
+        const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+        const int half = (cs + 1) / 2;
+        for (int item = wave; item < 2 * p.od; item += kPoolThreads / kWave) {
+          const int pd = item >> 1, c_lo = (item & 1) * half, c_hi = min(cs, c_lo + half);
+          TapRegs t;
+          t.load(tz, pd);
+          for (int c = c_lo; c < c_hi; c++)
+            for (int hw = lane; hw < ohw; hw += kWave)
+              o[c * cells + pd * ohw + hw] = store_cast<T>(t.apply(t2 + c * nz * ohw + hw, ohw));
+        }
       }
-      o[i] = store_cast<T>(acc);
+    } else {
+      for (int i = threadIdx.x; i < cs * nz * ny * p.ow; i += kPoolThreads) {  // contract x
+        const int row = fdiv(i, inv_ow), pw = i - row * p.ow;                 // row = (c, z, y)
+        const T *r = box + row * nx;
+        float acc = 0.f;
+        for (int s = 0; s < gx; s++) {
+          const int e = pw * gx + s;
+          acc += tx.wlo[e] * load(r + tx.lo[e]) + tx.whi[e] * load(r + tx.hi[e]);
+        }
+        t1[i] = acc;
+      }
+      __syncthreads();
+      for (int i = threadIdx.x; i < cs * nz * p.oh * p.ow; i += kPoolThreads) {  // contract y
+        const int cz = fdiv(i, inv_ohw), hw = i - cz * ohw, ph = fdiv(hw, inv_ow), pw = hw - ph * p.ow;  // cz = (c, z)
+        const float *r = t1 + cz * ny * p.ow + pw;
+        float acc = 0.f;
+        for (int s = 0; s < gy; s++) {
+          const int e = ph * gy + s;
+          acc += ty.wlo[e] * r[ty.lo[e] * p.ow] + ty.whi[e] * r[ty.hi[e] * p.ow];
+        }
+        t2[i] = acc;
+      }
+      __syncthreads();
+      T *o = dst + static_cast<long>(cb - c_begin) * cells;
+      for (int i = threadIdx.x; i < cs * cells; i += kPoolThreads) {  // contract z, store
+        const int c = fdiv(i, inv_cells), r0 = i - c * cells, pd = fdiv(r0, inv_ohw), hw = r0 - pd * ohw;
+        const float *r = t2 + c * nz * ohw + hw;
+        float acc = 0.f;
+        for (int s = 0; s < gz; s++) {
+          const int e = pd * gz + s;
+          acc += tz.wlo[e] * r[tz.lo[e] * ohw] + tz.whi[e] * r[tz.hi[e] * ohw];
+        }
+        o[i] = store_cast<T>(acc);
+      }
     }
     __syncthreads();
   }
