@@ -92,8 +92,9 @@ size_t mv_roi_align_forward_workspace_bytes(int dtype, int ndim, int channels, i
 /* ---- affine resampling engine (forward only) ----------------------------------------------
  * replaces affine_2d  csrc/affine_2d.h (vision.cpp:74), affine_3d  csrc/affine_3d.h:40 (vision.cpp:75)
  * Same arguments and results as the rotated forward for order 0 / 1 (the reference kernel text
- * is identical, csrc/cuda_aug/affine_3d_cuda_kernel.cuh:14-120).  order 3 is rejected with
- * MV_INVALID_ARGUMENT.                                                                        */
+ * is identical, csrc/cuda_aug/affine_3d_cuda_kernel.cuh:14-120).  order 3 = clamped Catmull-Rom
+ * over 4 x 4 (x 4) voxels (csrc/cuda_aug/interpolation_helpers_3d.h:571-792); the RoIAlign entry
+ * points above reject it, as the reference's do.                                              */
 int mv_affine_2d(const void *input, const void *rois, void *output, int dtype, int batch,
                  int channels, int height, int width, int num_rois, int out_h, int out_w,
                  float spatial_scale, int sampling_ratio, int aligned, int order, void *workspace, void *stream);
@@ -134,7 +135,8 @@ int mv_dcn3d_backward(const void *input, const void *offset, const void *mask, c
 /* ---- displacement-field warp (elastic engine) -----------------------------------------------
  * replaces deform_2d / deform_3d  csrc/deform_2d.h, csrc/deform_3d.h:27 (vision.cpp:71-72) for the
  * way the reference calls them (ops/cuda_fun_tools.py:94-167: 1x1x1 kernel, identity weight,
- * zero bias): out[b,c,q] = S(img[b,c], q + off[b,:,q]) on the open interval (-1, size), else 0.
+ * zero bias): out[b,c,q] = S(img[b,c], q + off[b,:,q]) on the open interval (-1, size), else 0;
+ * order 0, 1 or 3 as for the affine engine.
  * img/out [B,C,(D,)H,W], offset [B, 2|3, (D,)H,W] (3-D: 0 = depth, 1 = height, 2 = width).       */
 int mv_deform_warp_2d(const void *img, const void *offset, void *output, int dtype, int batch,
                       int channels, int height, int width, int order, void *stream);

@@ -320,8 +320,8 @@ def _deform(fn_name, ndim, input, weight, bias, offset, kernel, stride, pad, dil
             or not torch.equal(weight, eye) or bool((bias != 0).any())):
         raise RuntimeError("deform_%dd supports the displacement-field warp only: 1x1 kernel, "
                            "stride 1, no padding, identity weight, zero bias" % ndim)
-    if order not in (0, 1):
-        raise RuntimeError(f"order {order} is not implemented")
+    if order not in (0, 1, 3):
+        raise RuntimeError(f"order {order} is not supported (0 nearest, 1 linear, 3 cubic)")
     _require_contiguous(input, "input")
     offset = offset.to(device=input.device, dtype=input.dtype).contiguous()
     if tuple(offset.shape) != (input.size(0), ndim, *input.shape[2:]):
@@ -359,8 +359,8 @@ def deform_warp(img, offset, order=1):
     offset = offset.to(device=img.device, dtype=img.dtype).contiguous()
     if tuple(offset.shape) != (img.size(0), ndim, *img.shape[2:]):
         raise RuntimeError("offset must have shape [B, %d, *spatial]" % ndim)
-    if order not in (0, 1):
-        raise RuntimeError(f"order {order} is not implemented")
+    if order not in (0, 1, 3):
+        raise RuntimeError(f"order {order} is not supported (0 nearest, 1 linear, 3 cubic)")
     out = torch.empty_like(img)
     fn = "mv_deform_warp_2d" if ndim == 2 else "mv_deform_warp_3d"
     with torch.cuda.device(img.device):

@@ -47,7 +47,8 @@ __global__ __launch_bounds__(kRoiThreads) void roi_forward_kernel(const T *__res
               ry = g.rot[3] * x + g.rot[4] * y + g.rot[5] * z + g.centre[1];
               rz = p.ndim == 3 ? g.rot[6] * x + g.rot[7] * y + g.rot[8] * z + g.centre[2] : 0.0;
             }
-            acc += sample_clamped<T>(src, p.D, p.H, p.W, rz, ry, rx, p.order);
+            acc += p.order == 3 ? sample_cubic<T>(src, p.ndim, p.D, p.H, p.W, rz, ry, rx)
+                                : sample_clamped<T>(src, p.D, p.H, p.W, rz, ry, rx, p.order);
           }
         }
       }
@@ -126,12 +127,15 @@ int roi_pool_backward(const void *grad_output, const void *rois, void *acc, int 
 
 static int make_problem(RoiProblem &p, int ndim, int rotated, int batch, int channels, int depth,
                         int height, int width, int num_rois, int out_d, int out_h, int out_w,
-                        float spatial_scale, int sampling_ratio, int aligned, int order) {
+                        float spatial_scale, int sampling_ratio, int aligned, int order,
+                        bool cubic_ok = false) {
   MV_REQUIRE(batch > 0 && channels > 0 && depth > 0 && height > 0 && width > 0,
              "feature dims must be positive (got %d,%d,%d,%d,%d)", batch, channels, depth, height, width);
   MV_REQUIRE(num_rois >= 0, "num_rois must be >= 0");
   MV_REQUIRE(out_d > 0 && out_h > 0 && out_w > 0, "output size must be positive");
-  MV_REQUIRE(order == 0 || order == 1, "only support order = 0 (nearest) or 1 (linear), got %d", order);
+  MV_REQUIRE(order == 0 || order == 1 || (cubic_ok && order == 3),
+             cubic_ok ? "order %d is not supported (0 nearest, 1 linear, 3 cubic)"
+                      : "only support order = 0 (nearest) or 1 (linear), got %d", order);
   const long per_roi = static_cast<long>(channels) * out_d * out_h * out_w;
   MV_REQUIRE(per_roi < (1L << 31), "channels*out_d*out_h*out_w must be < 2^31");
   const long chunks = (per_roi + kRoiChunk - 1) / kRoiChunk;
@@ -149,15 +153,16 @@ static int make_problem(RoiProblem &p, int ndim, int rotated, int batch, int cha
 int roi_forward(const void *input, const void *rois, void *output, int dtype, int ndim,
                 int rotated, int batch, int channels, int depth, int height, int width,
                 int num_rois, int out_d, int out_h, int out_w, float spatial_scale,
-                int sampling_ratio, int aligned, int order, void *workspace, void *stream) {
+                int sampling_ratio, int aligned, int order, void *workspace, void *stream,
+                bool cubic_ok = false) {
   RoiProblem p;
   int st = make_problem(p, ndim, rotated, batch, channels, depth, height, width, num_rois, out_d,
-                        out_h, out_w, spatial_scale, sampling_ratio, aligned, order);
+                        out_h, out_w, spatial_scale, sampling_ratio, aligned, order, cubic_ok);
   if (st) return st;
   if (num_rois == 0) return MV_OK;
   MV_REQUIRE(input && rois && output, "null pointer argument");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  {
+  if (order != 3) {
     const int tiled = roi_forward_tiled(input, rois, output, dtype, p, workspace, nullptr, s);
     if (tiled >= 0) return tiled;
     const int pooled = roi_pool_forward(input, rois, output, dtype, p, s);
@@ -320,21 +325,18 @@ size_t mv_roi_align_backward_workspace_bytes(int dtype, int batch, int channels,
 int mv_affine_2d(const void *input, const void *rois, void *output, int dtype, int batch,
                  int channels, int height, int width, int num_rois, int out_h, int out_w,
                  float spatial_scale, int sampling_ratio, int aligned, int order, void *workspace, void *stream) {
-  if (order == 3)
-    return mv::fail(MV_INVALID_ARGUMENT, "affine_2d: order 3 (cubic) is not implemented");
   return roi_forward(input, rois, output, dtype, 2, 1, batch, channels, 1, height, width, num_rois,
-                     1, out_h, out_w, spatial_scale, sampling_ratio, aligned, order, workspace, stream);
+                     1, out_h, out_w, spatial_scale, sampling_ratio, aligned, order, workspace,
+                     stream, true);
 }
 
 int mv_affine_3d(const void *input, const void *rois, void *output, int dtype, int batch,
                  int channels, int depth, int height, int width, int num_rois, int out_d,
                  int out_h, int out_w, float spatial_scale, int sampling_ratio, int aligned,
                  int order, void *workspace, void *stream) {
-  if (order == 3)
-    return mv::fail(MV_INVALID_ARGUMENT, "affine_3d: order 3 (cubic) is not implemented");
   return roi_forward(input, rois, output, dtype, 3, 1, batch, channels, depth, height, width,
                      num_rois, out_d, out_h, out_w, spatial_scale, sampling_ratio, aligned, order,
-                     workspace, stream);
+                     workspace, stream, true);
 }
 
 }  // extern "C"

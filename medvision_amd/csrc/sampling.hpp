@@ -90,4 +90,52 @@ __device__ __forceinline__ typename Acc<T>::type sample_clamped(const T *plane, 
          lz * (hy * (hx * v5 + lx * v6) + ly * (hx * v7 + lx * v8));
 }
 
+// Order 3: separable Catmull-Rom (cubic Hermite with central-difference tangents) over the 4 x 4
+// (x 4) neighbourhood base-1 .. base+2 with every index clamped into the image
+// (csrc/cuda_aug/interpolation_helpers_3d.h:571-792, 2-D twin interpolation_helpers_2d.h:335-423;
+// the reference spells the 64 weights out as polynomials, which factor into these per-axis
+// weights).  Same void region as the other orders (outside the closed interval [-1, size]) and
+// negatives snap to 0, but the base index is NOT folded back at the upper border: between size-1
+// and size the fraction keeps growing while the taps beyond the border repeat the last voxel.
+template <typename A>
+__device__ __forceinline__ bool cubic_tap(double v, int size, int idx[4], A w[4]) {
+  if (v < -1.0 || v > static_cast<double>(size)) return false;
+  v = v <= 0.0 ? 0.0 : v;
+  const int base = static_cast<int>(v);
+  const A u = static_cast<A>(v - static_cast<double>(base));
+  const A u2 = u * u, u3 = u2 * u;
+  w[0] = A(-0.5) * u3 + u2 - A(0.5) * u;
+  w[1] = A(1.5) * u3 - A(2.5) * u2 + A(1);
+  w[2] = A(-1.5) * u3 + A(2) * u2 + A(0.5) * u;
+  w[3] = A(0.5) * u3 - A(0.5) * u2;
+#pragma unroll
+  for (int k = 0; k < 4; k++) idx[k] = min(max(base - 1 + k, 0), size - 1);
+  return true;
+}
+
+// ndim == 2: the plane is [H][W] and z is ignored (one z tap of weight 1).
+template <typename T>
+__device__ __forceinline__ typename Acc<T>::type sample_cubic(const T *plane, int ndim, int D,
+                                                              int H, int W, double z, double y,
+                                                              double x) {
+  using A = typename Acc<T>::type;
+  int zi[4] = {0, 0, 0, 0}, yi[4], xi[4];
+  A wz[4] = {A(1), A(0), A(0), A(0)}, wy[4], wx[4];
+  if (ndim == 3 && !cubic_tap(z, D, zi, wz)) return A(0);
+  if (!cubic_tap(y, H, yi, wy) || !cubic_tap(x, W, xi, wx)) return A(0);
+  const int nz = ndim == 3 ? 4 : 1;
+  A acc = A(0);
+  for (int a = 0; a < nz; a++) {
+    A slab = A(0);
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+      const T *row = plane + (static_cast<long>(zi[a]) * H + yi[b]) * W;
+      slab += wy[b] * (wx[0] * load(row + xi[0]) + wx[1] * load(row + xi[1]) +
+                       wx[2] * load(row + xi[2]) + wx[3] * load(row + xi[3]));
+    }
+    acc += wz[a] * slab;
+  }
+  return acc;
+}
+
 }  // namespace mv

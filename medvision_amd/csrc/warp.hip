@@ -1,5 +1,5 @@
 // Displacement-field warp: out[b,c,q] = S(img[b,c], q + off[b,:,q]) for -1 < p < size, else 0,
-// with S the border-replicating sampler (order 0 / 1).  This is what the reference obtains from
+// with S the border-replicating sampler (order 0 / 1) or the clamped Catmull-Rom one (order 3).  This is what the reference obtains from
 // its augmentation DCN with a 1x1x1 kernel and an identity weight (ops/cuda_fun_tools.py:94-167,
 // csrc/cuda_aug/deform_3d_cuda_kernel.cuh:58-85) -- here without the column matrix, the C x C
 // GEMM and the permute copy.  One thread owns one voxel position and reuses its taps for all
@@ -25,6 +25,14 @@ __global__ __launch_bounds__(256) void deform_warp_kernel(const T *__restrict__ 
   const double ph = h + static_cast<double>(load(o + (ndim - 2) * P));
   const double pw = w + static_cast<double>(load(o + (ndim - 1) * P));
   const bool ok = ph > -1.0 && pw > -1.0 && ph < H && pw < W && (ndim == 2 || (pd > -1.0 && pd < D));
+  if (order == 3) {
+    for (int c = 0; c < C; c++) {
+      const long base = (static_cast<long>(b) * C + c) * P;
+      out[base + q] =
+          store_cast<T>(ok ? sample_cubic<T>(img + base, ndim, D, H, W, pd, ph, pw) : A(0));
+    }
+    return;
+  }
   Corners<A> cw;
   const bool live = ok && clamped_corners<A>(D, H, W, pd, ph, pw, order, cw);
   for (int c = 0; c < C; c++) {
@@ -44,7 +52,8 @@ static int deform_warp(const void *img, const void *offset, void *output, int dt
                        void *stream) {
   MV_REQUIRE(batch > 0 && channels > 0 && depth > 0 && height > 0 && width > 0,
              "tensor dims must be positive");
-  MV_REQUIRE(order == 0 || order == 1, "order %d is not implemented", order);
+  MV_REQUIRE(order == 0 || order == 1 || order == 3,
+             "order %d is not supported (0 nearest, 1 linear, 3 cubic)", order);
   MV_REQUIRE(img && offset && output, "null pointer argument");
   const long P = static_cast<long>(depth) * height * width;
   MV_REQUIRE(P < (1L << 31) && batch <= 65535, "volume too large");

@@ -3,7 +3,7 @@
 Interface of the reference's ``medvision/ops/cuda_fun_tools.py``: ``affine_2d`` / ``affine_3d``
 (:6-92) resample with rotated rois (Resize, RandomAffine, Crop); ``apply_offset_2d`` /
 ``apply_offset_3d`` (:94-167) warp an image by a dense displacement field
-(RandomElasticDeformation).  Order 3 (cubic) is not implemented.
+(RandomElasticDeformation).  Orders: 0 nearest, 1 linear, 3 cubic (Catmull-Rom).
 """
 import torch
 
@@ -16,8 +16,6 @@ def _affine(ndim, features, rois, out_size, spatial_scale, sampling_ratio, align
     assert features.dtype in [torch.float32, torch.float16, torch.bfloat16, torch.float64], \
         f'input must be a floating tensor but got {features.dtype}'
     assert order in [0, 1, 3], f'order {order} is not supported!'
-    if order == 3:
-        raise NotImplementedError("order 3 (cubic) resampling is not implemented")
     if order == 0:
         sampling_ratio = 1  # never average nearest-neighbour samples (reference :72-74)
     output = features.new_zeros(rois.size(0), features.size(1), *out)

@@ -43,6 +43,10 @@ def lib():
         _lib.orc_sample_clamped.argtypes = [_dp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                             ctypes.c_double, ctypes.c_double, ctypes.c_double,
                                             ctypes.c_int]
+        _lib.orc_sample_cubic.restype = ctypes.c_double
+        _lib.orc_sample_cubic.argtypes = [_dp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                          ctypes.c_int, ctypes.c_double, ctypes.c_double,
+                                          ctypes.c_double]
     return _lib
 
 
@@ -63,6 +67,15 @@ def sample_clamped(volume, z, y, x, order=1):
     v = _f64(volume)
     D, H, W = v.shape
     return lib().orc_sample_clamped(_ptr(v), D, H, W, float(z), float(y), float(x), int(order))
+
+
+def sample_cubic(volume, z, y, x):
+    """One order-3 sample on a [D,H,W] volume or, for a 2-D tensor, an [H,W] image
+    (cuda_aug/interpolation_helpers_3d.h:571-792, interpolation_helpers_2d.h:335-423)."""
+    v = _f64(volume)
+    ndim = v.dim()
+    D, H, W = v.shape if ndim == 3 else (1,) + tuple(v.shape)
+    return lib().orc_sample_cubic(_ptr(v), ndim, D, H, W, float(z), float(y), float(x))
 
 
 def _roi_common(features_shape, rois, rotated):

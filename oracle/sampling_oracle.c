@@ -22,6 +22,10 @@
  *   dcn3d_forward             F.conv3d at zero offsets, grid_sample(zeros, align_corners=True)
  *   dcn3d_backward            torch autograd through the grid_sample formulation
  *   deform3d_warp             grid_sample(border) on the open interval (-1, S)
+ *   sample_cubic              textbook cubic Hermite spline with central-difference tangents on an
+ *                             edge-padded copy (numpy), exact reproduction of quadratics in the
+ *                             interior, node interpolation, partition of unity, brute-force
+ *                             table around -1, 0, S-1, S
  */
 #include <math.h>
 #include <stdlib.h>
@@ -97,6 +101,55 @@ static double sample_clamped(const double *plane, int D, int H, int W, double z,
   double v = 0.0;
   for (int n = 0; n < 8; n++) v += w[n] * plane[idx[n]];
   return v;
+}
+
+/* Order 3, one axis: cuda_aug/interpolation_helpers_3d.h:578-621 (2-D: interpolation_helpers_2d.h
+ * :341-370).  Same void test and snap of negatives as above; base = (int)v WITHOUT the fold at the
+ * upper border; the four indices base-1 .. base+2 are walked back into [0, size-1] one by one
+ * (the while loops), i.e. clamped.  The 64 weights the reference spells out as polynomials
+ * (:700-763) are the products of these per-axis Catmull-Rom weights: e.g. w000 starts with
+ * -0.125 u^3 v^3 w^3 = (-0.5)^3, w111 ends with +1.  The reference rounds the fraction to float
+ * (:589-591) even for double tensors; here it stays fp64 (difference <= 6e-8 relative). */
+static int cubic_tap(double v, int size, int idx[4], double w[4]) {
+  if (v < -1.0 || v > (double)size) return 0;
+  if (v <= 0) v = 0;
+  int base = (int)v;
+  double u = v - base, u2 = u * u, u3 = u2 * u;
+  w[0] = -0.5 * u3 + u2 - 0.5 * u;
+  w[1] = 1.5 * u3 - 2.5 * u2 + 1.0;
+  w[2] = -1.5 * u3 + 2.0 * u2 + 0.5 * u;
+  w[3] = 0.5 * u3 - 0.5 * u2;
+  for (int k = 0; k < 4; k++) {
+    int i = base - 1 + k;
+    idx[k] = i < 0 ? 0 : (i > size - 1 ? size - 1 : i);
+  }
+  return 1;
+}
+
+/* ndim 2: plane [H][W], z ignored (hermite_2d_interpolate); ndim 3: hermite_3d_interpolate. */
+static double sample_cubic(const double *plane, int ndim, int D, int H, int W, double z, double y,
+                           double x) {
+  int zi[4] = {0, 0, 0, 0}, yi[4], xi[4];
+  double wz[4] = {1, 0, 0, 0}, wy[4], wx[4];
+  if (ndim == 3 && !cubic_tap(z, D, zi, wz)) return 0.0;
+  if (!cubic_tap(y, H, yi, wy) || !cubic_tap(x, W, xi, wx)) return 0.0;
+  double v = 0.0;
+  for (int a = 0; a < (ndim == 3 ? 4 : 1); a++)
+    for (int b = 0; b < 4; b++)
+      for (int c = 0; c < 4; c++)
+        v += wz[a] * wy[b] * wx[c] * plane[((long)zi[a] * H + yi[b]) * W + xi[c]];
+  return v;
+}
+
+static double sample_any(const double *plane, int ndim, int D, int H, int W, double z, double y,
+                         double x, int order) {
+  return order == 3 ? sample_cubic(plane, ndim, D, H, W, z, y, x)
+                    : sample_clamped(plane, D, H, W, z, y, x, order);
+}
+
+double orc_sample_cubic(const double *plane, int ndim, int D, int H, int W, double z, double y,
+                        double x) {
+  return sample_cubic(plane, ndim, D, H, W, z, y, x);
 }
 
 /* exported for the unit tests of S */
@@ -205,7 +258,8 @@ static int roi_cols(int ndim, int rotated) {
   return ndim == 2 ? (rotated ? 6 : 5) : (rotated ? 10 : 7);
 }
 
-/* Forward of all four RoI flavours.
+/* Forward of all four RoI flavours (order 0 / 1) and of the affine engine (also order 3:
+ * cuda_aug/affine_3d_cuda_kernel.cuh:104-112, whose geometry is the rotated one).
  * feat [N,C,D,H,W] (D = 1 for 2-D), rois [R, 5|7|6|10], out [R,C,od,oh,ow].
  * roi_align_{2,3}d_forward_cuda_kernel, roi_align_rotated_{2,3}d_forward_cuda_kernel. */
 void orc_roi_align_forward(const double *feat, const double *rois, double *out, int ndim,
@@ -236,7 +290,7 @@ void orc_roi_align_forward(const double *feat, const double *rois, double *out, 
                   double x = local_coord(&g, 0, pw, ix);
                   double r[3];
                   to_global(&g, ndim, x, y, z, r);
-                  acc += sample_clamped(src, D, H, W, r[2], r[1], r[0], order);
+                  acc += sample_any(src, ndim, D, H, W, r[2], r[1], r[0], order);
                 }
               }
             }
@@ -486,7 +540,7 @@ void orc_dcn3d_backward(const double *x, const double *off, const double *mask, 
  * Displacement-field warp: the 1x1x1, identity-weight use of the augmentation DCN
  * (ops/cuda_fun_tools.py:134-167 -> cuda_aug/deform_3d_cuda_kernel.cuh:58-85):
  *   out[b,c,q] = S(img[b,c], q + off[b,{0:d,1:h,2:w},q])  if  -1 < p < size on all axes, else 0
- * with S the clamped sampler above (order 0 or 1).  2-D images are depth-1 volumes with a
+ * with S the clamped sampler above (order 0 or 1) or the cubic one (order 3, :80-81).  2-D images are depth-1 volumes with a
  * 2-channel offset (0:h, 1:w), cuda_aug/deform_2d_cuda_kernel.cuh.
  * ---------------------------------------------------------------------------------------- */
 void orc_deform_warp(const double *img, const double *off, double *out, int ndim, int B, int C,
@@ -503,6 +557,6 @@ void orc_deform_warp(const double *img, const double *off, double *out, int ndim
       int ok = ph > -1 && pw > -1 && ph < H && pw < W && (ndim == 2 || (pd > -1 && pd < D));
       for (int c = 0; c < C; c++)
         out[((long)b * C + c) * P + q] =
-            ok ? sample_clamped(img + ((long)b * C + c) * P, D, H, W, pd, ph, pw, order) : 0.0;
+            ok ? sample_any(img + ((long)b * C + c) * P, ndim, D, H, W, pd, ph, pw, order) : 0.0;
     }
 }

@@ -61,7 +61,9 @@ def test_host_shim_rejects_cpu_tensors_and_bad_rois():
         roi_align_3d(feat, torch.zeros(1, 7), [2, 2, 2], 1.0, 2, 1)
     with pytest.raises(NotImplementedError):
         ops.ModulatedDeformConv3dPack(2, 3, 3, padding=1)(feat)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(AssertionError, match="order 2 is not supported"):
+        ops.affine_3d(feat, torch.zeros(1, 10), (2, 2, 2), 1.0, 1, True, 2)
+    with pytest.raises(RuntimeError, match="affine is not implemented on CPU"):
         ops.affine_3d(feat, torch.zeros(1, 10), (2, 2, 2), 1.0, 1, True, 3)
     m = ops.DeformConv3dPack(2, 4, 3, padding=1, bias=False)
     assert set(m.state_dict()) == {"weight", "bias", "conv_offset.weight", "conv_offset.bias"}

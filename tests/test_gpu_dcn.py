@@ -187,7 +187,7 @@ def test_dcn_errors(ops):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
-@pytest.mark.parametrize("order", [0, 1])
+@pytest.mark.parametrize("order", [0, 1, 3])
 def test_warp_vs_oracle(ops, oracle, dtype, order):
     g = wl.gen(8)
     img = torch.randn(2, 3, 10, 12, 14, generator=g).to(dtype)

@@ -110,6 +110,14 @@ def test_edge_cases_and_errors(ops):
         ops.RoIAlign((2, 2, 2), 1.0, 2)(feat.cpu(), torch.zeros(1, 7))
     with pytest.raises(AssertionError):
         ops.RoIAlign((2, 2, 2), 1.0, 2)(feat, torch.zeros(1, 7, device=DEV), order=3)
+    # order 3 exists for the affine engine only; the RoIAlign bindings reject it like the reference
+    from medvision_amd import _C
+    with pytest.raises(RuntimeError, match="only support order = 0"):
+        _C.roi_align_rotated_3d_forward(feat, torch.zeros(1, 10, device=DEV),
+                                        torch.zeros(1, 3, 2, 2, 2, device=DEV), 2, 2, 2, 1.0, 2, True, 3)
+    with pytest.raises(RuntimeError, match="order 2 is not supported"):
+        _C.affine_3d(feat, torch.zeros(1, 10, device=DEV), torch.zeros(1, 3, 2, 2, 2, device=DEV),
+                     2, 2, 2, 1.0, 2, True, 2)
     # non-contiguous features are accepted (made contiguous), result unchanged
     r = torch.tensor([[1, 1., 1., 1., 6., 5., 4.]], device=DEV)
     a = ops.RoIAlign((2, 2, 2), 1.0, 2)(feat, r)
@@ -221,6 +229,37 @@ def test_tiled_resampler_2d(ops, oracle):
     got = ops.affine_2d(img.to(DEV), rois.to(DEV), (80, 96), 1.0, 1, True, 1)
     want = oracle.roi_align_forward(img, rois, (80, 96), 1.0, 1, True, 1, True)
     assert_close(got, want, FWD_TOL[torch.float16], "tiled 2-D forward")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("ndim,sr", [(3, 1), (3, 2), (2, 1), (2, 0)])
+def test_cubic_affine_vs_oracle(ops, oracle, dtype, ndim, sr):
+    """Order 3 of the affine engine (Catmull-Rom over 4^ndim clamped taps): rotated rois that
+    reach beyond every border, so the clamped taps, the overshoot between S-1 and S and the void
+    beyond [-1, S] are all sampled."""
+    feat, rois = _random_case(ndim, True, 90 + ndim + sr)
+    feat = feat.to(dtype)
+    out = (5, 6, 7)[3 - ndim:]
+    fn = ops.affine_3d if ndim == 3 else ops.affine_2d
+    got = fn(feat.to(DEV), rois.to(DEV), out, 0.5, sr, True, 3)
+    want = oracle.roi_align_forward(feat, rois, out, 0.5, sr, True, 3, True)
+    assert float(want.abs().max()) > 0.5
+    assert_close(got, want, FWD_TOL[dtype], "cubic affine")
+    # identity roi at order 3 returns the volume itself (weights 0,1,0,0 at integer coordinates)
+    size = feat.shape[2:]
+    ident = torch.tensor([[0, *[s / 2 for s in size[::-1]], *size[::-1], *([0.0] * (2 * ndim - 3))]])
+    same = fn(feat.to(DEV), ident.to(DEV), tuple(size), 1.0, 1, True, 3)
+    assert torch.equal(same[0].cpu(), feat[0])
+
+
+def test_cubic_resize_larger_volume(ops, oracle):
+    """Resize of a 40x48x56 volume to 64x80x96 at order 3, as CudaResize(order=3) issues it."""
+    g = wl.gen(97)
+    vol = torch.randn(2, 2, 40, 48, 56, generator=g).half()
+    rois = torch.tensor([[b, 28, 24, 20, 56, 48, 40, 0, 0, 0] for b in range(2)], dtype=torch.float32)
+    got = ops.affine_3d(vol.to(DEV), rois.to(DEV), (64, 80, 96), 1.0, 1, True, 3)
+    want = oracle.roi_align_forward(vol, rois, (64, 80, 96), 1.0, 1, True, 3, True)
+    assert_close(got, want, FWD_TOL[torch.float16], "cubic resize")
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])

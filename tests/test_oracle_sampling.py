@@ -60,3 +60,73 @@ def test_nearest_table(oracle):
     for (z, iz), (y, iy), (x, ix) in itertools.product(axis.items(), repeat=3):
         want = 0.0 if None in (iz, iy, ix) else float(vol[iz, iy, ix])
         assert oracle.sample_clamped(vol, z, y, x, order=0) == want, (z, y, x)
+
+
+# ---- order 3 -----------------------------------------------------------------------------------
+def _hermite_axis(arr, v, axis):
+    """Textbook cubic Hermite spline through the samples of `arr` along `axis`, tangents = central
+    differences, evaluated at coordinate v >= 0 of an array whose borders were edge-padded by 3."""
+    import numpy as np
+    base = int(np.floor(v))
+    u = v - base
+    take = lambda i: np.take(arr, base + 3 + i, axis=axis)
+    p0, p1, p2, p3 = take(-1), take(0), take(1), take(2)
+    m1, m2 = (p2 - p0) / 2, (p3 - p1) / 2
+    h00, h10 = 2 * u ** 3 - 3 * u ** 2 + 1, u ** 3 - 2 * u ** 2 + u
+    h01, h11 = -2 * u ** 3 + 3 * u ** 2, u ** 3 - u ** 2
+    return h00 * p1 + h10 * m1 + h01 * p2 + h11 * m2
+
+
+def test_cubic_matches_hermite_spline_on_edge_padded_copy(oracle):
+    import numpy as np
+    g = torch.Generator().manual_seed(2)
+    vol = torch.randn(5, 6, 7, generator=g, dtype=torch.float64)
+    padded = np.pad(vol.numpy(), 3, mode="edge")
+    # coordinates over the whole live range [0, S] (above S-1 the spline runs on repeated voxels)
+    pts = torch.rand(300, 3, generator=g, dtype=torch.float64) * torch.tensor([5., 6., 7.])
+    for z, y, x in pts.tolist():
+        want = _hermite_axis(_hermite_axis(_hermite_axis(padded, x, 2), y, 1), z, 0)
+        assert abs(oracle.sample_cubic(vol, z, y, x) - float(want)) < 1e-12
+    # 2-D images: same spline without the z axis
+    img = vol[0]
+    for _, y, x in pts[:100].tolist():
+        want = _hermite_axis(_hermite_axis(padded[3], x, 1), y, 0)
+        assert abs(oracle.sample_cubic(img, 0.0, y, x) - float(want)) < 1e-12
+
+
+def test_cubic_reproduces_quadratics_and_voxels(oracle):
+    z, y, x = torch.meshgrid(torch.arange(6.), torch.arange(7.), torch.arange(8.), indexing="ij")
+    f = lambda z, y, x: (1 + 0.5 * z - 0.25 * z * z) * (2 - y + 0.125 * y * y) * (x * x - 3 * x + 0.5)
+    vol = f(z, y, x).double()
+    g = torch.Generator().manual_seed(3)
+    # away from the border (all four taps are real voxels) the spline is exact for quadratics
+    pts = 1 + torch.rand(200, 3, generator=g, dtype=torch.float64) * torch.tensor([3., 4., 5.])
+    for pz, py, px in pts.tolist():
+        assert abs(oracle.sample_cubic(vol, pz, py, px) - f(pz, py, px)) < 1e-9
+    rnd = torch.randn(3, 4, 5, generator=g, dtype=torch.float64)
+    for iz, iy, ix in itertools.product(range(3), range(4), range(5)):
+        assert oracle.sample_cubic(rnd, iz, iy, ix) == float(rnd[iz, iy, ix])
+    # weights sum to one: a constant volume stays constant everywhere inside [-1, S]
+    const = torch.full((3, 4, 5), 7.0, dtype=torch.float64)
+    for pz, py, px in [(-1, -1, -1), (0.3, 3.7, 4.9), (3, 4, 5), (2.5, 0.1, 4.01)]:
+        assert abs(oracle.sample_cubic(const, pz, py, px) - 7.0) < 1e-12
+
+
+def test_cubic_edge_table(oracle):
+    # answers worked out by hand from "taps base-1..base+2 clamped into the image"
+    vol = torch.tensor([10., 20., 40., 80.], dtype=torch.float64).reshape(1, 1, 4)
+    cases = {
+        -1.0000001: 0.0, -1.0: 10.0, -0.5: 10.0, 0.0: 10.0,
+        0.5: 13.75,        # taps 10,10,20,40 with weights (-1, 9, 9, -1)/16
+        1.5: 28.125,       # taps 10,20,40,80: (-10 + 180 + 360 - 80) / 16
+        3.0: 80.0,
+        3.5: 82.5,         # taps 40,80,80,80: overshoots past the last voxel (no fold at S-1)
+        4.0: 80.0,         # exactly S: base = S, fraction 0, all taps clamp to the last voxel
+        4.0000001: 0.0,
+    }
+    for x, want in cases.items():
+        assert abs(oracle.sample_cubic(vol, 0.0, 0.0, x) - want) < 1e-9, x
+    assert abs(oracle.sample_cubic(vol.reshape(1, 4, 1), 0.0, 3.5, 0.0) - 82.5) < 1e-9
+    assert abs(oracle.sample_cubic(vol.reshape(4, 1, 1), 3.5, 0.0, 0.0) - 82.5) < 1e-9
+    assert oracle.sample_cubic(vol.reshape(4, 1, 1), 4.0000001, 0.0, 0.0) == 0.0
+    assert abs(oracle.sample_cubic(vol.reshape(4, 1)[:, :], 0.0, 3.5, 0.0) - 82.5) < 1e-9  # 2-D
