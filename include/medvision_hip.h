@@ -132,6 +132,33 @@ int mv_dcn3d_backward(const void *input, const void *offset, const void *mask, c
                       void *grad_mask, void *grad_weight, void *grad_bias,
                       const mv_dcn3d_shape *shape, int dtype, void *workspace, void *stream);
 
+/* ---- deformable convolution 2-D -----------------------------------------------------------
+ * replaces deform_conv_2d_forward / _backward                 csrc/deform_conv_2d.h:41,76
+ *          modulated_deform_conv_2d_forward / _backward       csrc/modulated_deform_conv_2d.h:23,47
+ * (vision.cpp:50-51,56-59).  Same conventions as the 3-D entry points with images instead of
+ * volumes: input [B,Cin,H,W], offset [B, dg*2*K, Ho,Wo] (channel 2k+0 = height, 2k+1 = width
+ * displacement of tap k = i*kw + j), mask [B, dg*K, Ho,Wo], weight [Cout, Cin/groups, kh,kw].
+ * The same kernels run (an image is a depth-1 volume).                                        */
+typedef struct {
+  int batch, in_channels, height, width;
+  int out_channels, kernel_h, kernel_w;
+  int stride_h, stride_w;
+  int pad_h, pad_w;
+  int dil_h, dil_w;
+  int groups, deformable_groups;
+} mv_dcn2d_shape;
+
+int mv_dcn2d_output_dims(const mv_dcn2d_shape *shape, int *out_h, int *out_w);
+size_t mv_dcn2d_forward_workspace_bytes(const mv_dcn2d_shape *shape, int dtype);
+size_t mv_dcn2d_backward_workspace_bytes(const mv_dcn2d_shape *shape, int dtype);
+int mv_dcn2d_forward(const void *input, const void *offset, const void *mask, const void *weight,
+                     const void *bias, void *output, const mv_dcn2d_shape *shape, int dtype,
+                     void *workspace, void *stream);
+int mv_dcn2d_backward(const void *input, const void *offset, const void *mask, const void *weight,
+                      const void *grad_output, void *grad_input, void *grad_offset,
+                      void *grad_mask, void *grad_weight, void *grad_bias,
+                      const mv_dcn2d_shape *shape, int dtype, void *workspace, void *stream);
+
 /* ---- displacement-field warp (elastic engine) -----------------------------------------------
  * replaces deform_2d / deform_3d  csrc/deform_2d.h, csrc/deform_3d.h:27 (vision.cpp:71-72) for the
  * way the reference calls them (ops/cuda_fun_tools.py:94-167: 1x1x1 kernel, identity weight,

@@ -153,63 +153,81 @@ def affine_3d(input, rois, output, out_d, out_h, out_w, spatial_scale, sampling_
                  spatial_scale, sampling_ratio, (int(bool(aligned)), int(order)))
 
 
-# ---- deformable convolution 3-D -----------------------------------------------------------
+# ---- deformable convolution (3-D volumes, 2-D images) ----------------------------------------
 def _dcn_shape(input, weight, kernel, stride, pad, dil, group, deformable_group):
+    """Checked shape record; the rank of ``input`` (5 or 4) selects volumes or images."""
     _require_contiguous(input, "input")
     _require_contiguous(weight, "weight")
-    B, C, D, H, W = input.shape
-    Cout, ck, kd_, kh_, kw_ = weight.shape
-    kd, kh, kw = kernel
-    if (kd_, kh_, kw_) != (kd, kh, kw):
-        raise RuntimeError("Input shape and kernel shape wont match: (%d x %d x %d vs %d x %d x %d)."
-                           % (kh, kw, kd, kh_, kw_, kd_))
+    nd = len(kernel)
+    if input.dim() != nd + 2 or weight.dim() != nd + 2:
+        raise RuntimeError(f"expected {nd + 2}-d input and weight tensors")
+    B, C = input.shape[:2]
+    Cout, ck = weight.shape[:2]
+    if tuple(weight.shape[2:]) != tuple(kernel):
+        if nd == 3:
+            raise RuntimeError("Input shape and kernel shape wont match: (%d x %d x %d vs %d x %d x %d)."
+                               % (kernel[1], kernel[2], kernel[0], weight.shape[3], weight.shape[4],
+                                  weight.shape[2]))
+        raise RuntimeError("Input shape and kernel shape wont match: (%d x %d vs %d x %d)."
+                           % (*kernel, *weight.shape[2:]))
     if C != ck * group:
         raise RuntimeError("Input shape and kernel channels wont match: (%d vs %d)." % (C, ck * group))
     if C % group or Cout % group:
         raise RuntimeError("channels(%d) and channels_out(%d) must divide group(%d)" % (C, Cout, group))
     if C % deformable_group:
         raise RuntimeError("channels(%d) must divide deformable_group(%d)" % (C, deformable_group))
-    return _lib.DcnShape(B, C, D, H, W, Cout, kd, kh, kw, *stride, *pad, *dil, group,
-                         deformable_group)
+    cls = _lib.DcnShape if nd == 3 else _lib.Dcn2dShape
+    return cls(B, C, *input.shape[2:], Cout, *kernel, *stride, *pad, *dil, group, deformable_group)
+
+
+def _dcn_family(shape):
+    return "mv_dcn3d" if isinstance(shape, _lib.DcnShape) else "mv_dcn2d"
 
 
 def _dcn_out_dims(lib, shape):
-    od, oh, ow = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
-    _lib.check(lib.mv_dcn3d_output_dims(ctypes.byref(shape), ctypes.byref(od), ctypes.byref(oh),
-                                        ctypes.byref(ow)))
-    return od.value, oh.value, ow.value
+    nd = 3 if isinstance(shape, _lib.DcnShape) else 2
+    dims = [ctypes.c_int() for _ in range(nd)]
+    _lib.check(getattr(lib, _dcn_family(shape) + "_output_dims")(
+        ctypes.byref(shape), *[ctypes.byref(d) for d in dims]))
+    return tuple(d.value for d in dims)
+
+
+def _dcn_taps(shape):
+    return (shape.kernel_d if isinstance(shape, _lib.DcnShape) else 1) * shape.kernel_h * shape.kernel_w
 
 
 def _dcn_check_aux(shape, dims, offset, mask, K):
-    B, dg = shape.batch, shape.deformable_groups
-    if tuple(offset.shape) != (B, dg * 3 * K, *dims):
-        raise RuntimeError(f"offset has shape {tuple(offset.shape)}, expected {(B, dg * 3 * K, *dims)}")
+    B, dg, nd = shape.batch, shape.deformable_groups, len(dims)
+    if tuple(offset.shape) != (B, dg * nd * K, *dims):
+        raise RuntimeError(f"offset has shape {tuple(offset.shape)}, expected {(B, dg * nd * K, *dims)}")
     if mask is not None and tuple(mask.shape) != (B, dg * K, *dims):
         raise RuntimeError(f"mask has shape {tuple(mask.shape)}, expected {(B, dg * K, *dims)}")
 
 
 def _dcn_forward(input, offset, mask, weight, bias, output, shape):
     lib = _lib.load()
+    fam = _dcn_family(shape)
     dims = _dcn_out_dims(lib, shape)
-    K = shape.kernel_d * shape.kernel_h * shape.kernel_w
+    K = _dcn_taps(shape)
     offset = offset.to(input.dtype).contiguous()
     mask = mask.to(input.dtype).contiguous() if mask is not None else None
     _dcn_check_aux(shape, dims, offset, mask, K)
     if weight.dtype != input.dtype or (bias is not None and bias.dtype != input.dtype):
         raise RuntimeError("input, weight and bias must share one dtype")
     code = _lib.dtype_code(input)
-    nbytes = lib.mv_dcn3d_forward_workspace_bytes(ctypes.byref(shape), code)
+    nbytes = getattr(lib, fam + "_forward_workspace_bytes")(ctypes.byref(shape), code)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=input.device) if nbytes else None
     with torch.cuda.device(input.device):
-        _lib.check(lib.mv_dcn3d_forward(
+        _lib.check(getattr(lib, fam + "_forward")(
             _lib.ptr(input), _lib.ptr(offset), _lib.ptr(mask), _lib.ptr(weight), _lib.ptr(bias),
             _lib.ptr(output), ctypes.byref(shape), code, _lib.ptr(ws), _lib.stream_of(input)))
 
 
 def _dcn_backward(input, offset, mask, weight, grad_output, gi, goff, gmask, gw, gb, shape):
     lib = _lib.load()
+    fam = _dcn_family(shape)
     dims = _dcn_out_dims(lib, shape)
-    K = shape.kernel_d * shape.kernel_h * shape.kernel_w
+    K = _dcn_taps(shape)
     offset = offset.to(input.dtype).contiguous()
     mask = mask.to(input.dtype).contiguous() if mask is not None else None
     _dcn_check_aux(shape, dims, offset, mask, K)
@@ -220,50 +238,105 @@ def _dcn_backward(input, offset, mask, weight, grad_output, gi, goff, gmask, gw,
     for t, n in ((gi, "grad_input"), (goff, "grad_offset"), (gw, "grad_weight")):
         _require_contiguous(t, n)
     code = _lib.dtype_code(input)
-    nbytes = lib.mv_dcn3d_backward_workspace_bytes(ctypes.byref(shape), code)
+    nbytes = getattr(lib, fam + "_backward_workspace_bytes")(ctypes.byref(shape), code)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=input.device) if nbytes else None
     with torch.cuda.device(input.device):
-        _lib.check(lib.mv_dcn3d_backward(
+        _lib.check(getattr(lib, fam + "_backward")(
             _lib.ptr(input), _lib.ptr(offset), _lib.ptr(mask), _lib.ptr(weight),
             _lib.ptr(grad_output), _lib.ptr(gi), _lib.ptr(goff), _lib.ptr(gmask), _lib.ptr(gw),
             _lib.ptr(gb), ctypes.byref(shape), code, _lib.ptr(ws), _lib.stream_of(input)))
+
+
+def _im2col_step_check(batch, im2col_step):
+    step = min(batch, im2col_step)
+    if batch % step != 0:
+        raise RuntimeError("batch(%d) must divide im2col_step(%d)" % (batch, step))
+
+
+def _dcn_v1_forward(input, weight, bias, offset, kernel, stride, pad, dil, group, deformable_group,
+                    im2col_step):
+    if not input.is_cuda:
+        raise RuntimeError("Not implemented on the CPU")
+    _im2col_step_check(input.size(0), im2col_step)
+    shape = _dcn_shape(input, weight, kernel, stride, pad, dil, group, deformable_group)
+    dims = _dcn_out_dims(_lib.load(), shape)
+    output = torch.empty((input.size(0), weight.size(0), *dims), dtype=input.dtype, device=input.device)
+    _dcn_forward(input, offset, None, weight, bias.contiguous(), output, shape)
+    return output
+
+
+def _dcn_v1_backward(input, weight, bias, offset, grad_output, kernel, stride, pad, dil, group,
+                     deformable_group, im2col_step):
+    if not input.is_cuda:
+        raise RuntimeError("Not implemented on the CPU")
+    _im2col_step_check(input.size(0), im2col_step)
+    shape = _dcn_shape(input, weight, kernel, stride, pad, dil, group, deformable_group)
+    gi, goff = torch.zeros_like(input), torch.zeros_like(offset, dtype=input.dtype)
+    gw, gb = torch.zeros_like(weight), torch.zeros_like(bias)
+    _dcn_backward(input, offset, None, weight, grad_output, gi, goff, None, gw, gb, shape)
+    return [gi, goff, gw, gb]
+
+
+def _dcn_v2_forward(input, weight, bias, offset, mask, output, kernel, stride, pad, dil, group,
+                    deformable_group, with_bias):
+    if not input.is_cuda:
+        raise RuntimeError("Not implemented on the CPU")
+    shape = _dcn_shape(input, weight, kernel, stride, pad, dil, group, deformable_group)
+    dims = _dcn_out_dims(_lib.load(), shape)
+    want = (input.size(0), weight.size(0), *dims)
+    if output.numel() != torch.Size(want).numel() or not output.is_contiguous():
+        raise RuntimeError(f"output must be a contiguous tensor of shape {want}")
+    if output.dtype != input.dtype:
+        raise RuntimeError("output dtype must match input dtype")
+    _dcn_forward(input, offset, mask, weight, bias.contiguous() if with_bias else None, output, shape)
+
+
+def _dcn_v2_backward(input, weight, offset, mask, grad_input, grad_weight, grad_bias, grad_offset,
+                     grad_mask, grad_output, kernel, stride, pad, dil, group, deformable_group,
+                     with_bias):
+    if not input.is_cuda:
+        raise RuntimeError("Not implemented on the CPU")
+    shape = _dcn_shape(input, weight, kernel, stride, pad, dil, group, deformable_group)
+    for t in (grad_input, grad_weight, grad_offset, grad_mask):
+        if t.dtype != input.dtype:
+            raise RuntimeError("gradient buffers must have the dtype of input")
+    _require_contiguous(grad_mask, "grad_mask")
+    _dcn_backward(input, offset, mask, weight, grad_output, grad_input, grad_offset, grad_mask,
+                  grad_weight, grad_bias if with_bias else None, shape)
 
 
 # csrc/deform_conv_3d.h:48-129 (host: csrc/cuda/deform_conv_3d_cuda.cu:110-376)
 def deform_conv_3d_forward(input, weight, bias, offset, kernel_d, kernel_h, kernel_w, stride_d,
                            stride_h, stride_w, pad_d, pad_h, pad_w, dilation_d, dilation_h,
                            dilation_w, group, deformable_group, im2col_step):
-    if not input.is_cuda:
-        raise RuntimeError("Not implemented on the CPU")
-    batch = input.size(0)
-    step = min(batch, im2col_step)
-    if batch % step != 0:
-        raise RuntimeError("batch(%d) must divide im2col_step(%d)" % (batch, step))
-    shape = _dcn_shape(input, weight, (kernel_d, kernel_h, kernel_w), (stride_d, stride_h, stride_w),
-                       (pad_d, pad_h, pad_w), (dilation_d, dilation_h, dilation_w), group,
-                       deformable_group)
-    dims = _dcn_out_dims(_lib.load(), shape)
-    output = torch.empty((batch, weight.size(0), *dims), dtype=input.dtype, device=input.device)
-    _dcn_forward(input, offset, None, weight, bias.contiguous(), output, shape)
-    return output
+    return _dcn_v1_forward(input, weight, bias, offset, (kernel_d, kernel_h, kernel_w),
+                           (stride_d, stride_h, stride_w), (pad_d, pad_h, pad_w),
+                           (dilation_d, dilation_h, dilation_w), group, deformable_group, im2col_step)
 
 
 def deform_conv_3d_backward(input, weight, bias, offset, grad_output, kernel_d, kernel_h, kernel_w,
                             stride_d, stride_h, stride_w, pad_d, pad_h, pad_w, dilation_d,
                             dilation_h, dilation_w, group, deformable_group, im2col_step):
-    if not input.is_cuda:
-        raise RuntimeError("Not implemented on the CPU")
-    batch = input.size(0)
-    step = min(batch, im2col_step)
-    if batch % step != 0:
-        raise RuntimeError("batch(%d) must divide im2col_step(%d)" % (batch, step))
-    shape = _dcn_shape(input, weight, (kernel_d, kernel_h, kernel_w), (stride_d, stride_h, stride_w),
-                       (pad_d, pad_h, pad_w), (dilation_d, dilation_h, dilation_w), group,
-                       deformable_group)
-    gi, goff = torch.zeros_like(input), torch.zeros_like(offset, dtype=input.dtype)
-    gw, gb = torch.zeros_like(weight), torch.zeros_like(bias)
-    _dcn_backward(input, offset, None, weight, grad_output, gi, goff, None, gw, gb, shape)
-    return [gi, goff, gw, gb]
+    return _dcn_v1_backward(input, weight, bias, offset, grad_output, (kernel_d, kernel_h, kernel_w),
+                            (stride_d, stride_h, stride_w), (pad_d, pad_h, pad_w),
+                            (dilation_d, dilation_h, dilation_w), group, deformable_group, im2col_step)
+
+
+# csrc/deform_conv_2d.h:41-109 (host: csrc/cuda/deform_conv_2d_cuda.cu:110-330)
+def deform_conv_2d_forward(input, weight, bias, offset, kernel_h, kernel_w, stride_h, stride_w,
+                           pad_h, pad_w, dilation_h, dilation_w, group, deformable_group,
+                           im2col_step):
+    return _dcn_v1_forward(input, weight, bias, offset, (kernel_h, kernel_w), (stride_h, stride_w),
+                           (pad_h, pad_w), (dilation_h, dilation_w), group, deformable_group,
+                           im2col_step)
+
+
+def deform_conv_2d_backward(input, weight, bias, offset, grad_output, kernel_h, kernel_w, stride_h,
+                            stride_w, pad_h, pad_w, dilation_h, dilation_w, group, deformable_group,
+                            im2col_step):
+    return _dcn_v1_backward(input, weight, bias, offset, grad_output, (kernel_h, kernel_w),
+                            (stride_h, stride_w), (pad_h, pad_w), (dilation_h, dilation_w), group,
+                            deformable_group, im2col_step)
 
 
 # csrc/modulated_deform_conv_3d.h:61-117 (host: csrc/cuda/modulated_deform_conv_3d_cuda.cu:137-396)
@@ -272,18 +345,9 @@ def modulated_deform_conv_3d_forward(input, weight, bias, ones, offset, mask, ou
                                      pad_d, pad_h, pad_w, dilation_d, dilation_h, dilation_w,
                                      group, deformable_group, with_bias):
     """``ones`` and ``columns`` are scratch handles of the reference and are ignored."""
-    if not input.is_cuda:
-        raise RuntimeError("Not implemented on the CPU")
-    shape = _dcn_shape(input, weight, (kernel_d, kernel_h, kernel_w), (stride_d, stride_h, stride_w),
-                       (pad_d, pad_h, pad_w), (dilation_d, dilation_h, dilation_w), group,
-                       deformable_group)
-    dims = _dcn_out_dims(_lib.load(), shape)
-    want = (input.size(0), weight.size(0), *dims)
-    if output.numel() != torch.Size(want).numel() or not output.is_contiguous():
-        raise RuntimeError(f"output must be a contiguous tensor of shape {want}")
-    if output.dtype != input.dtype:
-        raise RuntimeError("output dtype must match input dtype")
-    _dcn_forward(input, offset, mask, weight, bias.contiguous() if with_bias else None, output, shape)
+    _dcn_v2_forward(input, weight, bias, offset, mask, output, (kernel_d, kernel_h, kernel_w),
+                    (stride_d, stride_h, stride_w), (pad_d, pad_h, pad_w),
+                    (dilation_d, dilation_h, dilation_w), group, deformable_group, with_bias)
 
 
 def modulated_deform_conv_3d_backward(input, weight, bias, ones, offset, mask, columns, grad_input,
@@ -295,17 +359,29 @@ def modulated_deform_conv_3d_backward(input, weight, bias, ones, offset, mask, c
     col2im over a truncated index range and writes the mask gradient with a 2-D channel index
     (csrc/cuda/modulated_deform_conv_3d_cuda.cu:64, ..._kernel.cuh:410-411); those two defects
     are not reproduced."""
-    if not input.is_cuda:
-        raise RuntimeError("Not implemented on the CPU")
-    shape = _dcn_shape(input, weight, (kernel_d, kernel_h, kernel_w), (stride_d, stride_h, stride_w),
-                       (pad_d, pad_h, pad_w), (dilation_d, dilation_h, dilation_w), group,
-                       deformable_group)
-    for t in (grad_input, grad_weight, grad_offset, grad_mask):
-        if t.dtype != input.dtype:
-            raise RuntimeError("gradient buffers must have the dtype of input")
-    _require_contiguous(grad_mask, "grad_mask")
-    _dcn_backward(input, offset, mask, weight, grad_output, grad_input, grad_offset, grad_mask,
-                  grad_weight, grad_bias if with_bias else None, shape)
+    _dcn_v2_backward(input, weight, offset, mask, grad_input, grad_weight, grad_bias, grad_offset,
+                     grad_mask, grad_output, (kernel_d, kernel_h, kernel_w),
+                     (stride_d, stride_h, stride_w), (pad_d, pad_h, pad_w),
+                     (dilation_d, dilation_h, dilation_w), group, deformable_group, with_bias)
+
+
+# csrc/modulated_deform_conv_2d.h:23-70 (host: csrc/cuda/modulated_deform_conv_2d_cuda.cu)
+def modulated_deform_conv_2d_forward(input, weight, bias, ones, offset, mask, output, columns,
+                                     kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w,
+                                     dilation_h, dilation_w, group, deformable_group, with_bias):
+    """``ones`` and ``columns`` are scratch handles of the reference and are ignored."""
+    _dcn_v2_forward(input, weight, bias, offset, mask, output, (kernel_h, kernel_w),
+                    (stride_h, stride_w), (pad_h, pad_w), (dilation_h, dilation_w), group,
+                    deformable_group, with_bias)
+
+
+def modulated_deform_conv_2d_backward(input, weight, bias, ones, offset, mask, columns, grad_input,
+                                      grad_weight, grad_bias, grad_offset, grad_mask, grad_output,
+                                      kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w,
+                                      dilation_h, dilation_w, group, deformable_group, with_bias):
+    _dcn_v2_backward(input, weight, offset, mask, grad_input, grad_weight, grad_bias, grad_offset,
+                     grad_mask, grad_output, (kernel_h, kernel_w), (stride_h, stride_w),
+                     (pad_h, pad_w), (dilation_h, dilation_w), group, deformable_group, with_bias)
 
 
 # csrc/deform_2d.h, csrc/deform_3d.h:27-65 as used by ops/cuda_fun_tools.py:94-167

@@ -25,7 +25,15 @@ class DcnShape(ctypes.Structure):
         "dil_h", "dil_w", "groups", "deformable_groups")]
 
 
+class Dcn2dShape(ctypes.Structure):
+    """Mirror of ``mv_dcn2d_shape``."""
+    _fields_ = [(n, _i) for n in (
+        "batch", "in_channels", "height", "width", "out_channels", "kernel_h", "kernel_w",
+        "stride_h", "stride_w", "pad_h", "pad_w", "dil_h", "dil_w", "groups", "deformable_groups")]
+
+
 _SHAPE_P = ctypes.POINTER(DcnShape)
+_SHAPE2_P = ctypes.POINTER(Dcn2dShape)
 
 # name -> (restype, argtypes); must list every symbol of include/medvision_hip.h
 SIGNATURES = {
@@ -48,6 +56,11 @@ SIGNATURES = {
     "mv_dcn3d_backward_workspace_bytes": (_sz, [_SHAPE_P, _i]),
     "mv_dcn3d_forward": (_i, [_p] * 6 + [_SHAPE_P, _i, _p, _p]),
     "mv_dcn3d_backward": (_i, [_p] * 10 + [_SHAPE_P, _i, _p, _p]),
+    "mv_dcn2d_output_dims": (_i, [_SHAPE2_P, ctypes.POINTER(_i), ctypes.POINTER(_i)]),
+    "mv_dcn2d_forward_workspace_bytes": (_sz, [_SHAPE2_P, _i]),
+    "mv_dcn2d_backward_workspace_bytes": (_sz, [_SHAPE2_P, _i]),
+    "mv_dcn2d_forward": (_i, [_p] * 6 + [_SHAPE2_P, _i, _p, _p]),
+    "mv_dcn2d_backward": (_i, [_p] * 10 + [_SHAPE2_P, _i, _p, _p]),
     "mv_deform_warp_2d": (_i, [_p, _p, _p, _i] + [_i] * 4 + [_i, _p]),
     "mv_deform_warp_3d": (_i, [_p, _p, _p, _i] + [_i] * 5 + [_i, _p]),
 }

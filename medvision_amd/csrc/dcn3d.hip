@@ -32,7 +32,7 @@ __global__ __launch_bounds__(kDcnThreads) void dcn_forward_kernel(
   const int c_begin = grp * s.cpg, c_end = c_begin + s.cpg;
   for (int dgi = c_begin / s.cpd; dgi <= (c_end - 1) / s.cpd; dgi++) {
     const int c_lo = max(c_begin, dgi * s.cpd), c_hi = min(c_end, (dgi + 1) * s.cpd);
-    const T *off_bg = off + (static_cast<long>(b) * s.dg + dgi) * 3 * s.K * s.Q;
+    const T *off_bg = off + (static_cast<long>(b) * s.dg + dgi) * s.nd * s.K * s.Q;
     const T *mask_bg = mask ? mask + (static_cast<long>(b) * s.dg + dgi) * s.K * s.Q : nullptr;
     for (int k = 0; k < s.K; k++) {
       double pd, ph, pw;
@@ -75,7 +75,7 @@ __global__ __launch_bounds__(kDcnThreads) void dcn_backward_data_kernel(
   const int ow = q % s.Wo, oh = (q / s.Wo) % s.Ho, od = q / (static_cast<long>(s.Wo) * s.Ho);
   const long bg = static_cast<long>(b) * s.dg + dgi;
   double pd, ph, pw;
-  dcn_position(s, off + bg * 3 * s.K * s.Q, k, od, oh, ow, q, pd, ph, pw);
+  dcn_position(s, off + bg * s.nd * s.K * s.Q, k, od, oh, ow, q, pd, ph, pw);
   ZTaps<A> t;
   zero_pad_taps(s, pd, ph, pw, t);
   A go_d = A(0), go_h = A(0), go_w = A(0), gm = A(0);
@@ -110,8 +110,9 @@ __global__ __launch_bounds__(kDcnThreads) void dcn_backward_data_kernel(
       go_d += dd * gcol * m; go_h += dh * gcol * m; go_w += dw * gcol * m;
     }
   }
-  T *o = goff + (bg * 3 * s.K + 3 * k) * s.Q + q;
-  o[0] = store_cast<T>(go_d); o[s.Q] = store_cast<T>(go_h); o[2 * s.Q] = store_cast<T>(go_w);
+  T *o = goff + (bg * s.nd * s.K + s.nd * k) * s.Q + q;
+  if (s.nd == 3) o[0] = store_cast<T>(go_d);
+  o[(s.nd - 2) * s.Q] = store_cast<T>(go_h); o[(s.nd - 1) * s.Q] = store_cast<T>(go_w);
   if (gmask) gmask[(bg * s.K + k) * s.Q + q] = store_cast<T>(gm);
 }
 
@@ -142,7 +143,7 @@ __global__ __launch_bounds__(kGwThreads) void dcn_backward_weight_kernel(
   for (long q = static_cast<long>(slab) * kGwPositions + threadIdx.x; q < q_end; q += kGwThreads) {
     const int ow = q % s.Wo, oh = (q / s.Wo) % s.Ho, od = q / (static_cast<long>(s.Wo) * s.Ho);
     double pd, ph, pw;
-    dcn_position(s, off + bg * 3 * s.K * s.Q, k, od, oh, ow, q, pd, ph, pw);
+    dcn_position(s, off + bg * s.nd * s.K * s.Q, k, od, oh, ow, q, pd, ph, pw);
     ZTaps<A> t;
     zero_pad_taps(s, pd, ph, pw, t);
     if (!t.ok) continue;
@@ -237,15 +238,11 @@ int mv_dcn3d_output_dims(const mv_dcn3d_shape *shape, int *out_d, int *out_h, in
   return MV_OK;
 }
 
-size_t mv_dcn3d_forward_workspace_bytes(const mv_dcn3d_shape *shape, int dtype) {
-  DcnDims s;
-  if (make_dcn_dims(s, shape)) return 0;
+static size_t forward_workspace(const DcnDims &s, int dtype) {
   return dcn_mfma_supported(s, dtype) ? dcn_mfma_workspace_bytes(s, dtype) : 0;
 }
 
-size_t mv_dcn3d_backward_workspace_bytes(const mv_dcn3d_shape *shape, int dtype) {
-  DcnDims s;
-  if (make_dcn_dims(s, shape)) return 0;
+static size_t backward_workspace(const DcnDims &s, int dtype) {
   if (dcn_mfma_backward_supported(s, dtype)) return dcn_mfma_backward_workspace_bytes(s, dtype);
   if (dtype != MV_F16 && dtype != MV_BF16) return 0;
   // fp32 accumulators for grad_input, grad_weight, grad_bias
@@ -253,12 +250,9 @@ size_t mv_dcn3d_backward_workspace_bytes(const mv_dcn3d_shape *shape, int dtype)
   return n * sizeof(float);
 }
 
-int mv_dcn3d_forward(const void *input, const void *offset, const void *mask, const void *weight,
-                     const void *bias, void *output, const mv_dcn3d_shape *shape, int dtype,
-                     void *workspace, void *stream) {
-  DcnDims s;
-  int st = make_dcn_dims(s, shape);
-  if (st) return st;
+static int dcn_forward_any(const void *input, const void *offset, const void *mask,
+                           const void *weight, const void *bias, void *output, const DcnDims &s,
+                           int dtype, void *workspace, void *stream) {
   MV_REQUIRE(input && offset && weight && output, "null pointer argument");
   hipStream_t hs = static_cast<hipStream_t>(stream);
   if (dcn_mfma_supported(s, dtype)) {
@@ -278,13 +272,11 @@ int mv_dcn3d_forward(const void *input, const void *offset, const void *mask, co
   return check_launch("dcn_forward_kernel");
 }
 
-int mv_dcn3d_backward(const void *input, const void *offset, const void *mask, const void *weight,
-                      const void *grad_output, void *grad_input, void *grad_offset,
-                      void *grad_mask, void *grad_weight, void *grad_bias,
-                      const mv_dcn3d_shape *shape, int dtype, void *workspace, void *stream) {
-  DcnDims s;
-  int st = make_dcn_dims(s, shape);
-  if (st) return st;
+static int dcn_backward_any(const void *input, const void *offset, const void *mask,
+                            const void *weight, const void *grad_output, void *grad_input,
+                            void *grad_offset, void *grad_mask, void *grad_weight, void *grad_bias,
+                            const DcnDims &s, int dtype, void *workspace, void *stream) {
+  int st = MV_OK;
   MV_REQUIRE(input && offset && weight && grad_output && grad_input && grad_offset && grad_weight,
              "null pointer argument");
   MV_REQUIRE((mask == nullptr) == (grad_mask == nullptr) || grad_mask == nullptr,
@@ -358,6 +350,82 @@ int mv_dcn3d_backward(const void *input, const void *offset, const void *mask, c
     }
   });
   return check_launch("dcn3d backward");
+}
+
+// An image layer as a depth-1 volume with a 1 x kh x kw kernel and two offset components per tap.
+static int make_dcn_dims_2d(DcnDims &d, const mv_dcn2d_shape *s) {
+  MV_REQUIRE(s != nullptr, "shape is null");
+  const mv_dcn3d_shape v = {s->batch, s->in_channels, 1, s->height, s->width, s->out_channels,
+                            1, s->kernel_h, s->kernel_w, 1, s->stride_h, s->stride_w,
+                            0, s->pad_h, s->pad_w, 1, s->dil_h, s->dil_w,
+                            s->groups, s->deformable_groups};
+  return make_dcn_dims(d, &v, 2);
+}
+
+size_t mv_dcn3d_forward_workspace_bytes(const mv_dcn3d_shape *shape, int dtype) {
+  DcnDims s;
+  return make_dcn_dims(s, shape) ? 0 : forward_workspace(s, dtype);
+}
+
+size_t mv_dcn3d_backward_workspace_bytes(const mv_dcn3d_shape *shape, int dtype) {
+  DcnDims s;
+  return make_dcn_dims(s, shape) ? 0 : backward_workspace(s, dtype);
+}
+
+int mv_dcn3d_forward(const void *input, const void *offset, const void *mask, const void *weight,
+                     const void *bias, void *output, const mv_dcn3d_shape *shape, int dtype,
+                     void *workspace, void *stream) {
+  DcnDims s;
+  const int st = make_dcn_dims(s, shape);
+  return st ? st : dcn_forward_any(input, offset, mask, weight, bias, output, s, dtype, workspace, stream);
+}
+
+int mv_dcn3d_backward(const void *input, const void *offset, const void *mask, const void *weight,
+                      const void *grad_output, void *grad_input, void *grad_offset,
+                      void *grad_mask, void *grad_weight, void *grad_bias,
+                      const mv_dcn3d_shape *shape, int dtype, void *workspace, void *stream) {
+  DcnDims s;
+  const int st = make_dcn_dims(s, shape);
+  return st ? st
+            : dcn_backward_any(input, offset, mask, weight, grad_output, grad_input, grad_offset,
+                               grad_mask, grad_weight, grad_bias, s, dtype, workspace, stream);
+}
+
+int mv_dcn2d_output_dims(const mv_dcn2d_shape *shape, int *out_h, int *out_w) {
+  DcnDims s;
+  const int st = make_dcn_dims_2d(s, shape);
+  if (st) return st;
+  *out_h = s.Ho; *out_w = s.Wo;
+  return MV_OK;
+}
+
+size_t mv_dcn2d_forward_workspace_bytes(const mv_dcn2d_shape *shape, int dtype) {
+  DcnDims s;
+  return make_dcn_dims_2d(s, shape) ? 0 : forward_workspace(s, dtype);
+}
+
+size_t mv_dcn2d_backward_workspace_bytes(const mv_dcn2d_shape *shape, int dtype) {
+  DcnDims s;
+  return make_dcn_dims_2d(s, shape) ? 0 : backward_workspace(s, dtype);
+}
+
+int mv_dcn2d_forward(const void *input, const void *offset, const void *mask, const void *weight,
+                     const void *bias, void *output, const mv_dcn2d_shape *shape, int dtype,
+                     void *workspace, void *stream) {
+  DcnDims s;
+  const int st = make_dcn_dims_2d(s, shape);
+  return st ? st : dcn_forward_any(input, offset, mask, weight, bias, output, s, dtype, workspace, stream);
+}
+
+int mv_dcn2d_backward(const void *input, const void *offset, const void *mask, const void *weight,
+                      const void *grad_output, void *grad_input, void *grad_offset,
+                      void *grad_mask, void *grad_weight, void *grad_bias,
+                      const mv_dcn2d_shape *shape, int dtype, void *workspace, void *stream) {
+  DcnDims s;
+  const int st = make_dcn_dims_2d(s, shape);
+  return st ? st
+            : dcn_backward_any(input, offset, mask, weight, grad_output, grad_input, grad_offset,
+                               grad_mask, grad_weight, grad_bias, s, dtype, workspace, stream);
 }
 
 }  // extern "C"

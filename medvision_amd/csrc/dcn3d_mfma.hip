@@ -105,15 +105,15 @@ __global__ __launch_bounds__(256, MT <= 2 ? 4 : 3) void dcn_forward_mfma_kernel(
     const int c_lo = max(g * s.cpg, dgi * s.cpd), c_hi = min(g * s.cpg + s.cpg, (dgi + 1) * s.cpd);
     const int cc_lo = (c_lo - g * s.cpg) / SL, cc_hi = (c_hi - g * s.cpg) / SL;
     const long bg = static_cast<long>(b) * s.dg + dgi;
-    const T *o = off + bg * 3 * s.K * s.Q + qc;
+    const T *o = off + bg * s.nd * s.K * s.Q + qc;
     const T *mk = mask ? mask + bg * s.K * s.Q + qc : nullptr;
     int ki = 0, kj = 0, kk = 0;
     for (int k = 0; k < s.K; k++) {
-      const P pd = static_cast<P>(bd + ki * s.dd) + static_cast<P>(load(o));
-      const P ph = static_cast<P>(bh + kj * s.dh) + static_cast<P>(load(o + s.Q));
-      const P pw = static_cast<P>(bw + kk * s.dw) + static_cast<P>(load(o + 2 * s.Q));
+      P pd, ph, pw;
+      dcn_offsets(s, o, pd, ph, pw);
+      pd += static_cast<P>(bd + ki * s.dd); ph += static_cast<P>(bh + kj * s.dh); pw += static_cast<P>(bw + kk * s.dw);
       const float m = mk ? load(mk) : 1.f;
-      o += 3 * s.Q;
+      o += s.nd * s.Q;
       if (mk) mk += s.Q;
       if (++kk == s.kw) { kk = 0; if (++kj == s.kh) { kj = 0; ++ki; } }
       // byte offsets of the corners' channel vectors in xt (beyond the buffer when outside: such
@@ -254,10 +254,9 @@ __global__ __launch_bounds__(256, 4) void dcn_forward_mfma16_kernel(
       const long bg = static_cast<long>(b) * s.dg + dgi;
 #pragma unroll
       for (int nb = 0; nb < NB; nb++) {
-        const T *o = off + (bg * 3 * s.K + 3 * k) * s.Q + qc[nb];
-        const P pd = static_cast<P>(bd[nb] + ki * s.dd) + static_cast<P>(load(o));
-        const P ph = static_cast<P>(bh[nb] + kj * s.dh) + static_cast<P>(load(o + s.Q));
-        const P pw = static_cast<P>(bw[nb] + kk * s.dw) + static_cast<P>(load(o + 2 * s.Q));
+        P pd, ph, pw;
+        dcn_offsets(s, off + (bg * s.nd * s.K + s.nd * k) * s.Q + qc[nb], pd, ph, pw);
+        pd += static_cast<P>(bd[nb] + ki * s.dd); ph += static_cast<P>(bh[nb] + kj * s.dh); pw += static_cast<P>(bw[nb] + kk * s.dw);
         const float m = mask ? load(mask + (bg * s.K + k) * s.Q + qc[nb]) : 1.f;
         CornerTaps t;
         corner_taps<P>(s, pd, ph, pw, true, cin * ES, static_cast<unsigned>(lk) * 16u, 0x80000000u, t);

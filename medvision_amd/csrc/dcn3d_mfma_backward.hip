@@ -97,7 +97,7 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
   const __amdgpu_buffer_rsrc_t gr = __builtin_amdgcn_make_buffer_rsrc(
       gxt + static_cast<long>(b) * s.P * s.Cin, 0, static_cast<int>(s.P * s.Cin * 4), kRsrcFlags);
   const T *gyrow = gyt + (static_cast<long>(b) * s.Q + qc) * s.Cout + h * PC;
-  const T *o = off + bg * 3 * s.K * s.Q + qc;
+  const T *o = off + bg * s.nd * s.K * s.Q + qc;
   const T *mk = mask ? mask + bg * s.K * s.Q + qc : nullptr;
   float(*tp)[kTapWords] = taps[wave];
   float(*sm)[32] = sums[wave];
@@ -106,11 +106,11 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
   for (int k = 0; k < s.K; k++) {
     // ---- taps of (k, q0 + n): both half-wavefronts compute them, the lower one publishes -------
     {
-      const P pd = static_cast<P>(bd + ki * s.dd) + static_cast<P>(load(o));
-      const P ph = static_cast<P>(bh + kj * s.dh) + static_cast<P>(load(o + s.Q));
-      const P pw = static_cast<P>(bw + kk * s.dw) + static_cast<P>(load(o + 2 * s.Q));
+      P pd, ph, pw;
+      dcn_offsets(s, o, pd, ph, pw);
+      pd += static_cast<P>(bd + ki * s.dd); ph += static_cast<P>(bh + kj * s.dh); pw += static_cast<P>(bw + kk * s.dw);
       const float m = mk ? load(mk) : 1.f;
-      o += 3 * s.Q;
+      o += s.nd * s.Q;
       if (mk) mk += s.Q;
       if (++kk == s.kw) { kk = 0; if (++kj == s.kh) { kj = 0; ++ki; } }
       CornerTaps t;
@@ -180,8 +180,9 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     if (h == 0 && live) {
-      T *go = goff + (bg * 3 * s.K + 3 * k) * s.Q + q;
-      go[0] = store_cast<T>(sm[0][n]); go[s.Q] = store_cast<T>(sm[1][n]); go[2 * s.Q] = store_cast<T>(sm[2][n]);
+      T *go = goff + (bg * s.nd * s.K + s.nd * k) * s.Q + q;
+      if (s.nd == 3) go[0] = store_cast<T>(sm[0][n]);
+      go[(s.nd - 2) * s.Q] = store_cast<T>(sm[1][n]); go[(s.nd - 1) * s.Q] = store_cast<T>(sm[2][n]);
       if (gmask) gmask[(bg * s.K + k) * s.Q + q] = store_cast<T>(sm[3][n]);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -213,7 +214,7 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
   const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<T *>(xt + static_cast<long>(b) * s.P * s.Cin), 0, static_cast<int>(s.P * s.Cin * ES), kRsrcFlags);
   const unsigned cbyte2 = static_cast<unsigned>(c0 + n) * ES, cin2 = static_cast<unsigned>(s.Cin) * ES;
-  const T *ob = off + (bg * 3 * s.K + 3 * k) * s.Q;
+  const T *ob = off + (bg * s.nd * s.K + s.nd * k) * s.Q;
   const T *mb_ = mask ? mask + (bg * s.K + k) * s.Q : nullptr;
   const bool aligned = s.Q % PC == 0;
   float(*tp)[16] = taps[wave];
@@ -233,9 +234,10 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
       const bool live = q < s.Q;
       const long qc = live ? q : s.Q - 1;
       const int ow = qc % s.Wo, oh = (qc / s.Wo) % s.Ho, od = qc / (static_cast<long>(s.Wo) * s.Ho);
-      const P pd = static_cast<P>(od * s.sd - s.pd + ki * s.dd) + static_cast<P>(load(ob + qc));
-      const P ph = static_cast<P>(oh * s.sh - s.ph + kj * s.dh) + static_cast<P>(load(ob + s.Q + qc));
-      const P pw = static_cast<P>(ow * s.sw - s.pw + kk * s.dw) + static_cast<P>(load(ob + 2 * s.Q + qc));
+      P pd, ph, pw;
+      dcn_offsets(s, ob + qc, pd, ph, pw);
+      pd += static_cast<P>(od * s.sd - s.pd + ki * s.dd); ph += static_cast<P>(oh * s.sh - s.ph + kj * s.dh);
+      pw += static_cast<P>(ow * s.sw - s.pw + kk * s.dw);
       const float m = mb_ ? load(mb_ + qc) : 1.f;
       CornerTaps t;
       corner_taps<P>(s, pd, ph, pw, live, 1u, 0u, ~0u, t);

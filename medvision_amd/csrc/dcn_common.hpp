@@ -1,8 +1,10 @@
-// Shapes and the zero-padded sampler of the 3-D deformable convolution kernels.
+// Shapes and the zero-padded sampler of the deformable convolution kernels (3-D, and 2-D as a
+// depth-1 volume whose offsets carry two components per tap instead of three).
 //
 // For output position q = (od,oh,ow), kernel tap k = (i*kh + j)*kw + kk and input channel c in
 // deformable group dgi = c / (Cin/dg):
 //   p = q*stride - pad + (i,j,kk)*dil + offset[b, dgi*3K + 3k + {0:d, 1:h, 2:w}, q]
+//       (images, nd = 2: offset[b, dgi*2K + 2k + {0:h, 1:w}, q] and p_d = 0)
 //   col[c*K + k, q] = mask[b, dgi*K + k, q] * Z(x[b,c], p)        (mask == 1 for DCNv1)
 //   y[b,o,q] = sum_{c in group(o), k} Wt[o, c_local, k] * col[c*K + k, q] + bias[o]
 // Z is trilinear interpolation with ZERO padding, evaluated only when -1 < p < size on all axes
@@ -16,12 +18,13 @@ struct DcnDims {
   int B, Cin, D, H, W, Cout;
   int kd, kh, kw, sd, sh, sw, pd, ph, pw, dd, dh, dw;
   int groups, dg;
+  int nd;             // offset components per tap: 3 (d,h,w) for volumes, 2 (h,w) for images
   int Do, Ho, Wo, K;
   int cpg, opg, cpd;  // in-channels / out-channels per group, in-channels per deformable group
   long Q, P;          // output / input positions per (sample, channel)
 };
 
-inline int make_dcn_dims(DcnDims &d, const mv_dcn3d_shape *s) {
+inline int make_dcn_dims(DcnDims &d, const mv_dcn3d_shape *s, int nd = 3) {
   MV_REQUIRE(s != nullptr, "shape is null");
   MV_REQUIRE(s->batch > 0 && s->in_channels > 0 && s->depth > 0 && s->height > 0 && s->width > 0 &&
                  s->out_channels > 0, "tensor dims must be positive");
@@ -42,6 +45,7 @@ inline int make_dcn_dims(DcnDims &d, const mv_dcn3d_shape *s) {
   d.pd = s->pad_d; d.ph = s->pad_h; d.pw = s->pad_w;
   d.dd = s->dil_d; d.dh = s->dil_h; d.dw = s->dil_w;
   d.groups = s->groups; d.dg = s->deformable_groups;
+  d.nd = nd;
   d.Do = (d.D + 2 * d.pd - (d.dd * (d.kd - 1) + 1)) / d.sd + 1;
   d.Ho = (d.H + 2 * d.ph - (d.dh * (d.kh - 1) + 1)) / d.sh + 1;
   d.Wo = (d.W + 2 * d.pw - (d.dw * (d.kw - 1) + 1)) / d.sw + 1;
@@ -83,16 +87,26 @@ __device__ __forceinline__ void zero_pad_taps(const DcnDims &s, double pd, doubl
   }
 }
 
+// Offset components of one (tap, position); `o` points at the tap's first component.
+template <typename P, typename T>
+__device__ __forceinline__ void dcn_offsets(const DcnDims &s, const T *__restrict__ o, P &fd, P &fh,
+                                            P &fw) {
+  fd = s.nd == 3 ? static_cast<P>(load(o)) : P(0);
+  fh = static_cast<P>(load(o + (s.nd - 2) * s.Q));
+  fw = static_cast<P>(load(o + (s.nd - 1) * s.Q));
+}
+
 // Sample position of tap k at output position (od,oh,ow) for (b, dgi).
 template <typename T>
 __device__ __forceinline__ void dcn_position(const DcnDims &s, const T *__restrict__ off_bg,
                                              int k, int od, int oh, int ow, long q, double &pd,
                                              double &ph, double &pw) {
   const int i = k / (s.kh * s.kw), j = (k / s.kw) % s.kh, kk = k % s.kw;
-  const T *o = off_bg + static_cast<long>(3 * k) * s.Q + q;
-  pd = static_cast<double>(od * s.sd - s.pd + i * s.dd) + static_cast<double>(load(o));
-  ph = static_cast<double>(oh * s.sh - s.ph + j * s.dh) + static_cast<double>(load(o + s.Q));
-  pw = static_cast<double>(ow * s.sw - s.pw + kk * s.dw) + static_cast<double>(load(o + 2 * s.Q));
+  double fd, fh, fw;
+  dcn_offsets(s, off_bg + static_cast<long>(s.nd * k) * s.Q + q, fd, fh, fw);
+  pd = static_cast<double>(od * s.sd - s.pd + i * s.dd) + fd;
+  ph = static_cast<double>(oh * s.sh - s.ph + j * s.dh) + fh;
+  pw = static_cast<double>(ow * s.sw - s.pw + kk * s.dw) + fw;
 }
 
 template <typename T, typename A>

@@ -143,25 +143,37 @@ def _triple(v):
 
 
 def _dcn_params(x, weight, stride, padding, dilation, groups, deformable_groups):
-    B, Cin, D, H, W = x.shape
-    Cout, _, kd, kh, kw = weight.shape
-    s, p, d = _triple(stride), _triple(padding), _triple(dilation)
-    arr = (ctypes.c_int * 20)(B, Cin, D, H, W, Cout, kd, kh, kw, *s, *p, *d, groups,
-                              deformable_groups)
+    """Shape record of the C oracle.  4-D ``x`` = image layer: a depth-1 volume with a 1 x kh x kw
+    kernel and two offset components per tap (returns the 2-D output size)."""
+    if x.dim() == 4:
+        B, Cin, H, W = x.shape
+        Cout, _, kh, kw = weight.shape
+        pair = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
+        (sh, sw), (ph, pw), (dh, dw) = pair(stride), pair(padding), pair(dilation)
+        arr = (ctypes.c_int * 21)(B, Cin, 1, H, W, Cout, 1, kh, kw, 1, sh, sw, 0, ph, pw, 1, dh, dw,
+                                  groups, deformable_groups, 2)
+    else:
+        B, Cin, D, H, W = x.shape
+        Cout, _, kd, kh, kw = weight.shape
+        s, p, d = _triple(stride), _triple(padding), _triple(dilation)
+        arr = (ctypes.c_int * 21)(B, Cin, D, H, W, Cout, kd, kh, kw, *s, *p, *d, groups,
+                                  deformable_groups, 3)
     dims = (ctypes.c_int * 3)()
     lib().orc_dcn3d_out_dims(arr, dims)
-    return arr, tuple(dims)
+    return arr, (tuple(dims)[1:] if x.dim() == 4 else tuple(dims))
 
 
 def dcn3d_forward(x, offset, mask, weight, bias=None, stride=1, padding=0, dilation=1, groups=1,
                   deformable_groups=1):
     """DCN 3-D forward; ``mask=None`` gives v1 (cuda/deform_conv_3d_cuda_kernel.cuh:178-254),
-    otherwise v2 (cuda/modulated_deform_conv_3d_cuda_kernel.cuh:178-257)."""
+    otherwise v2 (cuda/modulated_deform_conv_3d_cuda_kernel.cuh:178-257).  4-D tensors give the
+    2-D layers (cuda/deform_conv_2d_cuda_kernel.cuh, cuda/modulated_deform_conv_2d_cuda_kernel.cuh
+    :118-190: offset channels 2k = h, 2k+1 = w)."""
     xs, offs, ws = _f64(x), _f64(offset), _f64(weight)
     ms = _f64(mask) if mask is not None else None
     bs = _f64(bias) if bias is not None else None
-    arr, (Do, Ho, Wo) = _dcn_params(xs, ws, stride, padding, dilation, groups, deformable_groups)
-    y = torch.zeros((xs.shape[0], ws.shape[0], Do, Ho, Wo), dtype=torch.float64)
+    arr, out = _dcn_params(xs, ws, stride, padding, dilation, groups, deformable_groups)
+    y = torch.zeros((xs.shape[0], ws.shape[0], *out), dtype=torch.float64)
     lib().orc_dcn3d_forward(_ptr(xs), _ptr(offs), _ptr(ms), _ptr(ws), _ptr(bs), _ptr(y), arr)
     return y
 
@@ -178,6 +190,10 @@ def dcn3d_backward(x, offset, mask, weight, grad_output, with_bias=True, stride=
     lib().orc_dcn3d_backward(_ptr(xs), _ptr(offs), _ptr(ms), _ptr(ws), _ptr(gy), _ptr(gx),
                              _ptr(goff), _ptr(gm), _ptr(gw), _ptr(gb), arr)
     return gx, goff, gm, gw, gb
+
+
+dcn2d_forward = dcn3d_forward     # the rank of ``x`` selects the layer family
+dcn2d_backward = dcn3d_backward
 
 
 def deform_warp(img, offset, order=1):

@@ -397,8 +397,13 @@ static double zsample_grad(const double *plane, const ztap *t, int axis) {
 
 typedef struct {
   int B, Cin, D, H, W, Cout, kd, kh, kw, sd, sh, sw, pd, ph, pw, dd, dh, dw, groups, dg;
+  int nd; /* offset components per tap: 3 = (d,h,w) volumes; 2 = (h,w) images, which are depth-1
+           * volumes with kd = 1, pad_d = 0 and p_d = 0 (cuda/modulated_deform_conv_2d_cuda_kernel.cuh
+           * :143-176: offset channel 2k = h, 2k+1 = w of tap k = i*kw + j; bilinear with zero
+           * padding :9-40, evaluated when -1 < p < size :167) */
   int Do, Ho, Wo, K;
 } dcn_shape;
+#define DCN_INTS 21
 
 static void dcn_out_dims(dcn_shape *s) {
   s->Do = (s->D + 2 * s->pd - (s->dd * (s->kd - 1) + 1)) / s->sd + 1;
@@ -410,26 +415,27 @@ static void dcn_out_dims(dcn_shape *s) {
 static void dcn_taps(const dcn_shape *s, const double *off, int b, int dgi, int k, int od, int oh,
                      int ow, ztap *t) {
   const long Q = (long)s->Do * s->Ho * s->Wo, q = ((long)od * s->Ho + oh) * s->Wo + ow;
-  const double *o = off + ((long)b * s->dg + dgi) * 3 * s->K * Q;
+  const int nd = s->nd;
+  const double *o = off + ((long)b * s->dg + dgi) * nd * s->K * Q;
   int i = k / (s->kh * s->kw), j = (k / s->kw) % s->kh, kk = k % s->kw;
-  double pd = od * s->sd - s->pd + i * s->dd + o[(3L * k + 0) * Q + q];
-  double ph = oh * s->sh - s->ph + j * s->dh + o[(3L * k + 1) * Q + q];
-  double pw = ow * s->sw - s->pw + kk * s->dw + o[(3L * k + 2) * Q + q];
+  double pd = od * s->sd - s->pd + i * s->dd + (nd == 3 ? o[((long)nd * k + 0) * Q + q] : 0.0);
+  double ph = oh * s->sh - s->ph + j * s->dh + o[((long)nd * k + nd - 2) * Q + q];
+  double pw = ow * s->sw - s->pw + kk * s->dw + o[((long)nd * k + nd - 1) * Q + q];
   zero_pad_taps(s->D, s->H, s->W, pd, ph, pw, t);
 }
 
 void orc_dcn3d_out_dims(const int *p, int *dims) {
   dcn_shape s;
-  memcpy(&s, p, 20 * sizeof(int));
+  memcpy(&s, p, DCN_INTS * sizeof(int));
   dcn_out_dims(&s);
   dims[0] = s.Do; dims[1] = s.Ho; dims[2] = s.Wo;
 }
 
-/* p: the 20 ints of dcn_shape in declaration order.  mask, bias may be NULL. */
+/* p: the 21 ints of dcn_shape in declaration order.  mask, bias may be NULL. */
 void orc_dcn3d_forward(const double *x, const double *off, const double *mask, const double *wt,
                        const double *bias, double *y, const int *p) {
   dcn_shape s;
-  memcpy(&s, p, 20 * sizeof(int));
+  memcpy(&s, p, DCN_INTS * sizeof(int));
   dcn_out_dims(&s);
   const long Q = (long)s.Do * s.Ho * s.Wo, P = (long)s.D * s.H * s.W;
   const int cpg = s.Cin / s.groups, opg = s.Cout / s.groups, cpd = s.Cin / s.dg;
@@ -471,7 +477,7 @@ void orc_dcn3d_backward(const double *x, const double *off, const double *mask, 
                         const double *gy, double *gx, double *goff, double *gmask, double *gw,
                         double *gbias, const int *p) {
   dcn_shape s;
-  memcpy(&s, p, 20 * sizeof(int));
+  memcpy(&s, p, DCN_INTS * sizeof(int));
   dcn_out_dims(&s);
   const long Q = (long)s.Do * s.Ho * s.Wo, P = (long)s.D * s.H * s.W;
   const int cpg = s.Cin / s.groups, opg = s.Cout / s.groups, cpd = s.Cin / s.dg;
@@ -522,8 +528,8 @@ void orc_dcn3d_backward(const double *x, const double *off, const double *mask, 
             for (int a = 0; a < 3; a++) go[a] += zsample_grad(plane, &t, a) * gcol * m;
             gm += gcol * zsample(plane, &t);
           }
-          double *o = goff + ((long)b * s.dg + dgi) * 3 * s.K * Q;
-          for (int a = 0; a < 3; a++) o[(3L * k + a) * Q + q] += go[a];
+          double *o = goff + ((long)b * s.dg + dgi) * s.nd * s.K * Q;
+          for (int a = 3 - s.nd; a < 3; a++) o[((long)s.nd * k + a - (3 - s.nd)) * Q + q] += go[a];
           if (gmask) gmask[(((long)b * s.dg + dgi) * s.K + k) * Q + q] += gm;
         }
     }

@@ -186,6 +186,58 @@ def test_dcn_errors(ops):
         _C.deform_conv_3d_forward(x, w, b, off[:, :80].contiguous(), *args, 64)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("modulated,groups,dg,stride,pad,dil,cin,cout,size", [
+    (True, 1, 1, 1, 1, 1, 4, 6, (9, 11)),           # general kernels
+    (False, 2, 2, 2, 1, 2, 4, 6, (10, 13)),
+    (True, 1, 1, 1, 1, 1, 64, 64, (20, 24)),        # matrix-core forward and backward (16-bit, fp32)
+    (False, 2, 1, 1, 0, 1, 64, 64, (13, 17)),
+    (True, 1, 2, 2, 2, 2, 32, 96, (17, 19))])
+def test_2d_layers_vs_oracle(ops, oracle, dtype, modulated, groups, dg, stride, pad, dil, cin, cout, size):
+    """The 2-D layers (offset channels 2k = rows, 2k+1 = columns) forward and all gradients."""
+    from medvision_amd.ops.deform_conv_2d import deform_conv
+    from medvision_amd.ops.modulated_deform_conv_2d import modulated_deform_conv
+    g = wl.gen(120 + groups + dg + cout)
+    x, off, mask, w, b = wl.dcn_inputs(g, 2, cin, cout, size, 3, dg, groups, dtype, stride, pad, dil,
+                                       modulated)
+    xs, offs, ms, ws, bs = [None if t is None else t.to(DEV).requires_grad_(True)
+                            for t in (x, off, mask, w, b)]
+    if modulated:
+        y = modulated_deform_conv(xs, offs, ms, ws, bs, stride, pad, dil, groups, dg)
+    else:
+        y = deform_conv(xs, offs, ws, bs, stride, pad, dil, groups, dg, 64)
+    want = oracle.dcn2d_forward(x, off, mask, w, b, stride, pad, dil, groups, dg)
+    assert y.dtype == dtype and y.shape == want.shape
+    assert_close(y, want, FWD_TOL[dtype], "2-D forward")
+    gy = torch.randn(y.shape, generator=g).to(dtype)
+    y.backward(gy.to(DEV))
+    gx, goff, gm, gw, gb = oracle.dcn2d_backward(x, off, mask, w, gy, True, stride, pad, dil, groups, dg)
+    tol = BWD_TOL[dtype]
+    assert_close(xs.grad, gx, tol, "grad input")
+    assert_close(offs.grad, goff, tol, "grad offset")
+    assert_close(ws.grad, gw, tol, "grad weight")
+    assert_close(bs.grad, gb, tol, "grad bias")
+    if modulated:
+        assert_close(ms.grad, gm, tol, "grad mask")
+
+
+def test_2d_packs(ops):
+    """Pack modules: zero-initialised offset branch == plain convolution; state-dict keys."""
+    torch.manual_seed(0)
+    x = torch.randn(2, 8, 12, 14, device=DEV)
+    m1 = ops.DeformConv2dPack(8, 16, 3, padding=1).to(DEV)
+    assert set(m1.state_dict()) == {"weight", "bias", "conv_offset.weight", "conv_offset.bias"}
+    assert_close(m1(x), F.conv2d(x, m1.weight, m1.bias, padding=1), 1e-5, "v1 pack")
+    m2 = ops.ModulatedDeformConv2dPack(8, 16, 3, padding=1, stride=2).to(DEV)
+    assert set(m2.state_dict()) == {"weight", "bias", "conv_offset_mask.weight", "conv_offset_mask.bias"}
+    assert_close(m2(x), 0.5 * F.conv2d(x, m2.weight, None, stride=2, padding=1) + m2.bias.view(1, -1, 1, 1),
+                 1e-5, "v2 pack")
+    m2(x).sum().backward()
+    assert m2.conv_offset_mask.weight.grad is not None and m2.weight.grad is not None
+    with pytest.raises(RuntimeError, match="offset has shape"):
+        ops.DeformConv2d(8, 16, 3, 1, 1).to(DEV)(x, torch.zeros(2, 18, 12, 13, device=DEV))
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("order", [0, 1, 3])
 def test_warp_vs_oracle(ops, oracle, dtype, order):

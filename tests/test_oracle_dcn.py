@@ -4,6 +4,8 @@
 * integer offsets          ->  convolution of a shifted input
 * general                  ->  grid_sample(zeros, align_corners=True) + einsum (torch_ref.dcn3d)
 * gradients                ->  torch autograd through that formulation (all five inputs)
+* 2-D layers               ->  F.conv2d at zero offsets, a hand-shifted image for the channel order
+                              (2k = rows, 2k+1 = columns), 2-D grid_sample + autograd in general
 * warp                     ->  grid_sample(border) on the open interval, identity at zero offset
 """
 import pytest
@@ -81,6 +83,60 @@ def test_general_and_gradients_vs_autograd(oracle, v2, groups, dg):
         assert torch.allclose(gm, grads[4], atol=1e-10)
     else:
         assert gm is None
+
+
+@pytest.mark.parametrize("groups,stride,pad,dil", [(1, 1, 1, 1), (2, 2, 1, 1), (1, (1, 2), (2, 0), (2, 1))])
+def test_2d_zero_offset_is_conv2d(oracle, groups, stride, pad, dil):
+    g = _g(20)
+    x = torch.randn(2, 4, 9, 10, generator=g, dtype=torch.float64)
+    w = torch.randn(6, 4 // groups, 3, 2, generator=g, dtype=torch.float64)
+    b = torch.randn(6, generator=g, dtype=torch.float64)
+    want = F.conv2d(x, w, b, stride, pad, dil, groups)
+    off = torch.zeros(2, 2 * 6, *want.shape[2:], dtype=torch.float64)
+    got = oracle.dcn2d_forward(x, off, None, w, b, stride, pad, dil, groups, 1)
+    assert got.shape == want.shape and torch.allclose(got, want, atol=1e-11)
+
+
+def test_2d_offset_channel_order(oracle):
+    """Channel 2k moves tap k along the rows (h), 2k+1 along the columns (w)."""
+    g = _g(21)
+    x = torch.randn(1, 1, 6, 7, generator=g, dtype=torch.float64)
+    w = torch.ones(1, 1, 1, 1, dtype=torch.float64)
+    off = torch.zeros(1, 2, 6, 7, dtype=torch.float64)
+    off[:, 0] = 2.0   # rows
+    off[:, 1] = -1.0  # columns
+    got = oracle.dcn2d_forward(x, off, None, w, None)
+    want = torch.zeros_like(x)
+    want[0, 0, :4, 1:] = x[0, 0, 2:, :6]
+    assert torch.allclose(got, want)
+
+
+@pytest.mark.parametrize("v2,groups,dg", [(True, 1, 1), (True, 2, 2), (False, 1, 2), (False, 2, 1)])
+def test_2d_general_and_gradients_vs_autograd(oracle, v2, groups, dg):
+    g = _g(22 + groups + 2 * dg)
+    B, Cin, Cout, H, W = 2, 4, 6, 7, 8
+    k, stride, pad, dil = (3, 2), (2, 1), (1, 0), (1, 2)
+    K = 6
+    x = torch.randn(B, Cin, H, W, generator=g, dtype=torch.float64, requires_grad=True)
+    w = torch.randn(Cout, Cin // groups, *k, generator=g, dtype=torch.float64, requires_grad=True)
+    b = torch.randn(Cout, generator=g, dtype=torch.float64, requires_grad=True)
+    Ho, Wo = [(S + 2 * p_ - (d_ * (k_ - 1) + 1)) // s_ + 1
+              for S, p_, d_, k_, s_ in zip((H, W), pad, dil, k, stride)]
+    off = torch.randn(B, dg * 2 * K, Ho, Wo, generator=g, dtype=torch.float64) * 2.0
+    frac = off - off.floor()
+    off = (off.floor() + frac.clamp(0.05, 0.95)).requires_grad_(True)
+    m = torch.rand(B, dg * K, Ho, Wo, generator=g, dtype=torch.float64).requires_grad_(True) if v2 else None
+    want = torch_ref.dcn2d(x, off, m, w, b, stride, pad, dil, groups, dg)
+    got = oracle.dcn2d_forward(x, off, m, w, b, stride, pad, dil, groups, dg)
+    assert torch.allclose(got, want.detach(), atol=1e-11)
+    gy = torch.randn(want.shape, generator=g, dtype=torch.float64)
+    ins = [x, off, w, b] + ([m] if v2 else [])
+    grads = torch.autograd.grad(want, ins, gy)
+    gx, goff, gm, gw, gb = oracle.dcn2d_backward(x, off, m, w, gy, True, stride, pad, dil, groups, dg)
+    for got_, want_ in zip((gx, goff, gw, gb), grads[:4]):
+        assert torch.allclose(got_, want_, atol=1e-10)
+    if v2:
+        assert torch.allclose(gm, grads[4], atol=1e-10)
 
 
 def test_warp(oracle):

@@ -155,3 +155,43 @@ def dcn3d(x, offset, mask, weight, bias=None, stride=1, padding=0, dilation=1, g
     if bias is not None:
         y = y + bias.view(1, -1, 1, 1, 1)
     return y
+
+
+def dcn2d(x, offset, mask, weight, bias=None, stride=1, padding=0, dilation=1, groups=1,
+          deformable_groups=1):
+    """Differentiable fp64 DCN 2-D (v1 if mask is None): bilinear, zero-padded sampling with torch's
+    2-D grid_sample; offset channel 2k = row, 2k+1 = column displacement of tap k = i*kw + j."""
+    t2 = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v,) * 2
+    s, p, d = t2(stride), t2(padding), t2(dilation)
+    B, Cin, H, W = x.shape
+    Cout, cpg, kh, kw = weight.shape
+    K = kh * kw
+    Ho, Wo = [(S + 2 * pp - (dd * (k - 1) + 1)) // ss + 1
+              for S, pp, dd, k, ss in zip((H, W), p, d, (kh, kw), s)]
+    qh = (torch.arange(Ho, dtype=x.dtype) * s[0] - p[0])[:, None]
+    qw = (torch.arange(Wo, dtype=x.dtype) * s[1] - p[1])[None, :]
+    cpd = Cin // deformable_groups
+    col = []
+    for b in range(B):
+        per_dg = []
+        for g in range(deformable_groups):
+            xs = x[b:b + 1, g * cpd:(g + 1) * cpd]
+            taps = []
+            for k in range(K):
+                i, j = k // kw, k % kw
+                ph = qh + i * d[0] + offset[b, (g * K + k) * 2]
+                pw = qw + j * d[1] + offset[b, (g * K + k) * 2 + 1]
+                grid = torch.stack([2 * pw / max(W - 1, 1) - 1, 2 * ph / max(H - 1, 1) - 1], -1)
+                v = F.grid_sample(xs, grid[None], mode="bilinear", padding_mode="zeros",
+                                  align_corners=True)[0]
+                if mask is not None:
+                    v = v * mask[b, g * K + k][None]
+                taps.append(v)
+            per_dg.append(torch.stack(taps, 1))
+        col.append(torch.cat(per_dg, 0))
+    col = torch.stack(col).reshape(B, groups, Cin // groups, K, Ho, Wo)
+    wg = weight.reshape(groups, Cout // groups, cpg, K)
+    y = torch.einsum("bgckhw,gock->bgohw", col, wg).reshape(B, Cout, Ho, Wo)
+    if bias is not None:
+        y = y + bias.view(1, -1, 1, 1)
+    return y

@@ -43,14 +43,15 @@ def ct_like(g, shape, dtype=torch.float16):
 
 def dcn_inputs(g, B, Cin, Cout, size, k=3, dg=1, groups=1, dtype=torch.float32, stride=1, pad=1,
                dil=1, modulated=True, offset_std=2.0):
-    D, H, W = size
-    x = torch.randn(B, Cin, D, H, W, generator=g)
-    K = k ** 3
+    """Inputs of a deformable convolution; ``size`` with two entries gives the 2-D layer."""
+    nd = len(size)
+    x = torch.randn(B, Cin, *size, generator=g)
+    K = k ** nd
     bound = 1.0 / math.sqrt(Cin // groups * K)
-    w = (torch.rand(Cout, Cin // groups, k, k, k, generator=g) * 2 - 1) * bound
+    w = (torch.rand(Cout, Cin // groups, *([k] * nd), generator=g) * 2 - 1) * bound
     bias = (torch.rand(Cout, generator=g) * 2 - 1) * bound
-    od, oh, ow = [(s + 2 * pad - (dil * (k - 1) + 1)) // stride + 1 for s in size]
-    off = torch.randn(B, dg * 3 * K, od, oh, ow, generator=g) * offset_std
-    mask = torch.sigmoid(torch.randn(B, dg * K, od, oh, ow, generator=g)) if modulated else None
+    out = [(s + 2 * pad - (dil * (k - 1) + 1)) // stride + 1 for s in size]
+    off = torch.randn(B, dg * nd * K, *out, generator=g) * offset_std
+    mask = torch.sigmoid(torch.randn(B, dg * K, *out, generator=g)) if modulated else None
     cast = lambda t: None if t is None else t.to(dtype)
     return cast(x), cast(off), cast(mask), cast(w), cast(bias)
