@@ -24,25 +24,25 @@
 
 namespace mv {
 
-// x [B, Cin, P] -> xt [B, P, Cin]; one workgroup moves 64 positions of all channels through LDS
-// (U = unsigned short / unsigned int: only the element size matters)
+// x [B, Cin, P] -> xt [B, P, Cin]; one workgroup moves 64 positions of up to kLayoutChunk
+// channels through LDS (U = unsigned short / unsigned int: only the element size matters)
+constexpr int kLayoutChunk = 128;
 template <typename U>
 __global__ void dcn_channels_last_kernel(const U *__restrict__ x, U *__restrict__ xt, int Cin, long P) {
-  extern __shared__ unsigned char stage_raw[];
-  U *stage = reinterpret_cast<U *>(stage_raw);  // [64][Cin + 2]
+  __shared__ U stage[64][kLayoutChunk + 2];
   const int b = blockIdx.y;
   const long p0 = static_cast<long>(blockIdx.x) * 64;
-  const int pitch = Cin + 2;
-  const U *src = x + static_cast<long>(b) * Cin * P;
-  U *dst = xt + (static_cast<long>(b) * P + p0) * Cin;
+  const int c0 = blockIdx.z * kLayoutChunk, cn = min(kLayoutChunk, Cin - c0);
+  const U *src = x + (static_cast<long>(b) * Cin + c0) * P;
+  U *dst = xt + (static_cast<long>(b) * P + p0) * Cin + c0;
   const int lp = threadIdx.x % 64;
-  for (int c = threadIdx.x / 64; c < Cin; c += 4)
-    if (p0 + lp < P) stage[lp * pitch + c] = src[static_cast<long>(c) * P + p0 + lp];
+  for (int c = threadIdx.x / 64; c < cn; c += 4)
+    if (p0 + lp < P) stage[lp][c] = src[static_cast<long>(c) * P + p0 + lp];
   __syncthreads();
-  const long count = min(static_cast<long>(64), P - p0) * Cin;
-  for (long i = threadIdx.x; i < count; i += 256) {
-    const int pp = static_cast<int>(i / Cin), c = static_cast<int>(i % Cin);
-    dst[i] = stage[pp * pitch + c];
+  const int count = static_cast<int>(min(static_cast<long>(64), P - p0)) * cn;
+  for (int i = threadIdx.x; i < count; i += 256) {
+    const int pp = i / cn, c = i % cn;
+    dst[static_cast<long>(pp) * Cin + c] = stage[pp][c];
   }
 }
 
@@ -309,12 +309,12 @@ __global__ __launch_bounds__(256, 4) void dcn_forward_mfma16_kernel(
 int dcn_channels_last(const void *x, void *xt, int B, int C, long P, int elem_bytes, hipStream_t stream) {
   const long pblocks = (P + 63) / 64;
   MV_REQUIRE(pblocks < (1L << 31) && B <= 65535, "volume too large");
-  const dim3 grid(static_cast<unsigned>(pblocks), B);
+  const dim3 grid(static_cast<unsigned>(pblocks), B, (C + kLayoutChunk - 1) / kLayoutChunk);
   if (elem_bytes == 2)
-    hipLaunchKernelGGL((dcn_channels_last_kernel<unsigned short>), grid, dim3(256), 64 * (C + 2) * 2, stream,
+    hipLaunchKernelGGL((dcn_channels_last_kernel<unsigned short>), grid, dim3(256), 0, stream,
                        static_cast<const unsigned short *>(x), static_cast<unsigned short *>(xt), C, P);
   else
-    hipLaunchKernelGGL((dcn_channels_last_kernel<unsigned int>), grid, dim3(256), 64 * (C + 2) * 4, stream,
+    hipLaunchKernelGGL((dcn_channels_last_kernel<unsigned int>), grid, dim3(256), 0, stream,
                        static_cast<const unsigned int *>(x), static_cast<unsigned int *>(xt), C, P);
   return check_launch("dcn_channels_last_kernel");
 }
@@ -327,7 +327,6 @@ bool dcn_mfma_supported(const DcnDims &s, int dtype) {
   if (s.cpg % 16 || s.opg % 32 || s.cpd % 16) return false;
   if (s.Cin > 4096 || s.B > 65535) return false;
   if (static_cast<long>(s.P) * s.Cin * elem_size(dtype) >= (1L << 31)) return false;  // 32-bit byte offsets
-  if (static_cast<size_t>(64) * (s.Cin + 2) * elem_size(dtype) > 64 * 1024) return false;  // transpose staging
   return true;
 }
 

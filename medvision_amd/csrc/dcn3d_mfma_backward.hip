@@ -196,7 +196,7 @@ constexpr int kGwChunk = 2048;  // positions per workgroup
 template <typename T, int MT>
 __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
     const T *__restrict__ xt, const T *__restrict__ off, const T *__restrict__ mask,
-    const T *__restrict__ gy, float *__restrict__ gw, const DcnDims s) {
+    const T *__restrict__ gy, float *__restrict__ gw, const DcnDims s, const int mb0) {
   using M = Mfma<T>;
   using P = typename std::conditional<(sizeof(T) == 2), float, double>::type;  // position type
   constexpr int PC = M::kPiece, SL = 2 * PC, ES = sizeof(T);
@@ -272,7 +272,7 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
       const long qa = qg + st * SL + h * PC;
 #pragma unroll
       for (int m = 0; m < MT; m++) {
-        const T *grow = gy + (static_cast<long>(b) * s.Cout + g * s.opg + m * 32 + n) * s.Q + qa;
+        const T *grow = gy + (static_cast<long>(b) * s.Cout + g * s.opg + (mb0 + m) * 32 + n) * s.Q + qa;
         union { u32x4 u; T e[PC]; } a;
         if (aligned && qa + PC <= s.Q) {
           a.u = *reinterpret_cast<const u32x4 *>(grow);
@@ -303,33 +303,35 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
       for (int r = 0; r < 16; r++) {
         const float v = acc[m][r] + part[0][m][r][lane] + part[1][m][r][lane] + part[2][m][r][lane];
         // accumulator layout: register r of lane l = row 8*(r/4) + 4*(l/32) + r%4, column l%32
-        const int o = g * s.opg + m * 32 + 8 * (r / 4) + 4 * h + (r % 4);
+        const int o = g * s.opg + (mb0 + m) * 32 + 8 * (r / 4) + 4 * h + (r % 4);
         const int cl = c0 - g * s.cpg + n;
         atomicAdd(gw + (static_cast<long>(o) * s.cpg + cl) * s.K + k, v);
       }
   }
 }
 
-// gxt [B, P, C] fp32 -> gx [B, C, P] T, added to what gx holds; 64 positions per workgroup
+// gxt [B, P, C] fp32 -> gx [B, C, P] T, added to what gx holds; 64 positions x up to kAddChunk
+// channels per workgroup
+constexpr int kAddChunk = 128;
 template <typename T>
 __global__ __launch_bounds__(256) void dcn_planar_add_kernel(const float *__restrict__ gxt,
                                                              T *__restrict__ gx, int C, long P) {
-  extern __shared__ float stagef[];  // [64][C + 1]
+  __shared__ float stagef[64][kAddChunk + 1];
   const int b = blockIdx.y;
   const long p0 = static_cast<long>(blockIdx.x) * 64;
-  const int pitch = C + 1;
-  const long count = min(static_cast<long>(64), P - p0) * C;
-  const float *src = gxt + (static_cast<long>(b) * P + p0) * C;
-  for (long i = threadIdx.x; i < count; i += 256) {
-    const int pp = static_cast<int>(i / C), c = static_cast<int>(i % C);
-    stagef[pp * pitch + c] = src[i];
+  const int c0 = blockIdx.z * kAddChunk, cn = min(kAddChunk, C - c0);
+  const int count = static_cast<int>(min(static_cast<long>(64), P - p0)) * cn;
+  const float *src = gxt + (static_cast<long>(b) * P + p0) * C + c0;
+  for (int i = threadIdx.x; i < count; i += 256) {
+    const int pp = i / cn, c = i % cn;
+    stagef[pp][c] = src[static_cast<long>(pp) * C + c];
   }
   __syncthreads();
   const int lp = threadIdx.x % 64;
   if (p0 + lp < P)
-    for (int c = threadIdx.x / 64; c < C; c += 4) {
-      T *d = gx + (static_cast<long>(b) * C + c) * P + p0 + lp;
-      *d = store_cast<T>(load(d) + stagef[lp * pitch + c]);
+    for (int c = threadIdx.x / 64; c < cn; c += 4) {
+      T *d = gx + (static_cast<long>(b) * C + c0 + c) * P + p0 + lp;
+      *d = store_cast<T>(load(d) + stagef[lp][c]);
     }
 }
 
@@ -343,8 +345,7 @@ static size_t align256b(size_t v) { return (v + 255) / 256 * 256; }
 
 bool dcn_mfma_backward_supported(const DcnDims &s, int dtype) {
   if (dtype != MV_F16 && dtype != MV_BF16 && dtype != MV_F32) return false;
-  if (s.cpg % 32 || s.opg % 32 || s.cpd % 32 || s.opg > 128) return false;
-  if (static_cast<size_t>(64) * (max(s.Cin, s.Cout) + 2) * 4 > 64 * 1024) return false;  // transpose staging
+  if (s.cpg % 32 || s.opg % 32 || s.cpd % 32) return false;
   if (s.B > 65535 || s.dg > 65535) return false;
   if (static_cast<long>(s.P) * s.Cin * 4 >= (1L << 31)) return false;  // 32-bit byte offsets
   if (static_cast<long>(s.Cin / 32) * s.K >= (1L << 31) || (s.Q + kGwChunk - 1) / kGwChunk > 65535) return false;
@@ -400,13 +401,15 @@ static int backward_run(const void *x, const void *off, const void *mask, const 
 #define MV_LAUNCH_GW(MTV)                                                                          \
   hipLaunchKernelGGL((dcn_backward_weight_mfma_kernel<T, MTV>), wgrid, dim3(256), 0, stream, xt,   \
                      static_cast<const T *>(off), static_cast<const T *>(mask),                    \
-                     static_cast<const T *>(gy), *gw32, s)
-  switch (s.opg / 32) {
-    case 1: MV_LAUNCH_GW(1); break;
-    case 2: MV_LAUNCH_GW(2); break;
-    case 3: MV_LAUNCH_GW(3); break;
-    default: MV_LAUNCH_GW(4); break;
-  }
+                     static_cast<const T *>(gy), *gw32, s, mb0)
+  // up to four 32-row blocks of output channels per pass over the positions
+  for (int mb0 = 0; mb0 < s.opg / 32; mb0 += 4)
+    switch (min(s.opg / 32 - mb0, 4)) {
+      case 1: MV_LAUNCH_GW(1); break;
+      case 2: MV_LAUNCH_GW(2); break;
+      case 3: MV_LAUNCH_GW(3); break;
+      default: MV_LAUNCH_GW(4); break;
+    }
 #undef MV_LAUNCH_GW
   return check_launch("dcn3d mfma backward");
 }
@@ -427,16 +430,16 @@ int dcn_mfma_backward(const void *x, const void *off, const void *mask, const vo
 int dcn_planar_add(const float *gxt, void *gx, const DcnDims &s, int dtype, hipStream_t stream) {
   const long pblocks = (s.P + 63) / 64;
   MV_REQUIRE(pblocks < (1L << 31), "volume too large");
-  const size_t lds = 64 * (s.Cin + 1) * sizeof(float);
+  const dim3 grid(static_cast<unsigned>(pblocks), s.B, (s.Cin + kAddChunk - 1) / kAddChunk);
   if (dtype == MV_F16)
-    hipLaunchKernelGGL((dcn_planar_add_kernel<__half>), dim3(static_cast<unsigned>(pblocks), s.B), dim3(256), lds,
-                       stream, gxt, static_cast<__half *>(gx), s.Cin, s.P);
+    hipLaunchKernelGGL((dcn_planar_add_kernel<__half>), grid, dim3(256), 0, stream, gxt,
+                       static_cast<__half *>(gx), s.Cin, s.P);
   else if (dtype == MV_F32)
-    hipLaunchKernelGGL((dcn_planar_add_kernel<float>), dim3(static_cast<unsigned>(pblocks), s.B), dim3(256), lds,
-                       stream, gxt, static_cast<float *>(gx), s.Cin, s.P);
+    hipLaunchKernelGGL((dcn_planar_add_kernel<float>), grid, dim3(256), 0, stream, gxt,
+                       static_cast<float *>(gx), s.Cin, s.P);
   else
-    hipLaunchKernelGGL((dcn_planar_add_kernel<__hip_bfloat16>), dim3(static_cast<unsigned>(pblocks), s.B), dim3(256),
-                       lds, stream, gxt, static_cast<__hip_bfloat16 *>(gx), s.Cin, s.P);
+    hipLaunchKernelGGL((dcn_planar_add_kernel<__hip_bfloat16>), grid, dim3(256), 0, stream, gxt,
+                       static_cast<__hip_bfloat16 *>(gx), s.Cin, s.P);
   return check_launch("dcn_planar_add_kernel");
 }
 

@@ -91,7 +91,8 @@ def test_matrix_core_path_vs_oracle(ops, oracle, dtype, modulated, groups, dg, s
     (True, 1, 1, 1, 1, 1, 32, 64, (12, 12, 16)),    # config-4 geometry, Q % 8 == 0
     (True, 2, 2, 1, 1, 1, 64, 128, (7, 9, 11)),     # groups, deformable groups, ragged tiles, Q odd
     (False, 1, 2, 2, 1, 2, 64, 32, (9, 10, 12)),    # DCNv1, stride 2, dilation 2, two chunks per group
-    (True, 1, 1, 1, 0, 1, 32, 96, (6, 7, 9))])      # no padding, three 32-row output blocks
+    (True, 1, 1, 1, 0, 1, 32, 96, (6, 7, 9)),       # no padding, three 32-row output blocks
+    (False, 1, 1, 1, 1, 1, 160, 192, (5, 6, 7))])   # more than 128 channels in and out
 def test_matrix_core_backward_vs_oracle(ops, oracle, dtype, modulated, groups, dg, stride, pad, dil,
                                         cin, cout, size):
     """Shapes that take the MFMA backward (channels per group / per deformable group % 32 == 0,
@@ -192,7 +193,8 @@ def test_dcn_errors(ops):
     (False, 2, 2, 2, 1, 2, 4, 6, (10, 13)),
     (True, 1, 1, 1, 1, 1, 64, 64, (20, 24)),        # matrix-core forward and backward (16-bit, fp32)
     (False, 2, 1, 1, 0, 1, 64, 64, (13, 17)),
-    (True, 1, 2, 2, 2, 2, 32, 96, (17, 19))])
+    (True, 1, 2, 2, 2, 2, 32, 96, (17, 19)),
+    (True, 1, 1, 1, 1, 1, 256, 256, (10, 12))])     # FPN-sized layer: two channel chunks, two output passes
 def test_2d_layers_vs_oracle(ops, oracle, dtype, modulated, groups, dg, stride, pad, dil, cin, cout, size):
     """The 2-D layers (offset channels 2k = rows, 2k+1 = columns) forward and all gradients."""
     from medvision_amd.ops.deform_conv_2d import deform_conv
