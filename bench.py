@@ -90,6 +90,63 @@ def bench_dcn(args, dtype=torch.float16):
     return {"ms": ms, "tflops": flops / ms / 1e9, "flops": flops, "train_ms": train_ms}
 
 
+def bench_next_rows(args):
+    """Short timings of the operators either side of the headline path: order-3 resampling, the
+    elastic pipeline (control-grid upsampling + displacement warp), a 2-D DCNv2 layer of FPN size
+    and the augmentation stages that build the rois.  20 steps each, HIP events."""
+    import numpy as np
+    import medvision_amd.ops as ops
+    import medvision_amd.aug_cuda as aug
+    from medvision_amd.ops.modulated_deform_conv_2d import modulated_deform_conv
+    import workloads as wl
+    dev, n = "cuda:0", 20
+    g = wl.gen(7)
+    res = {}
+    vol = torch.randn(4, 1, 128, 128, 128, generator=g).half().to(dev)
+    rois = wl.affine_rois(g, 4, (128, 128, 128)).to(dev)
+    ms, _ = _events_ms(lambda i: ops.affine_3d(vol, rois, (128, 128, 128), 1.0, 1, True, 3), n, 3)
+    res["affine_3d_order3_config2"] = {"ms": round(ms, 4), "gvox_s": round(4 * 128 ** 3 / ms / 1e6, 2)}
+    grid = torch.randn(2, 3, 8, 8, 8, generator=g).to(dev)
+    groi = torch.tensor([[b, 4, 4, 4, 5, 5, 5, 0, 0, 0] for b in range(2)], dtype=torch.float32, device=dev)
+    ms, _ = _events_ms(lambda i: ops.affine_3d(grid, groi, (128, 128, 128), 1, 1, True, 3), n, 3)
+    res["elastic_grid_upsample_8to128_order3"] = {"ms": round(ms, 4)}
+    field = ops.affine_3d(grid, groi, (128, 128, 128), 1, 1, True, 3).half()
+    img = vol[:2]
+    ms, _ = _events_ms(lambda i: ops.apply_offset_3d(img, field, 1), n, 3)
+    res["apply_offset_3d_2x128^3_fp16"] = {"ms": round(ms, 4), "gvox_s": round(2 * 128 ** 3 / ms / 1e6, 2)}
+    B, C, H, W = 8, 256, 100, 152
+    x = torch.randn(B, C, H, W, generator=g).half().to(dev)
+    w = (torch.randn(C, C, 3, 3, generator=g) * 0.02).half().to(dev)
+    bias = torch.zeros(C, dtype=torch.float16, device=dev)
+    off = (torch.randn(B, 18, H, W, generator=g) * 2).half().to(dev)
+    msk = torch.sigmoid(torch.randn(B, 9, H, W, generator=g)).half().to(dev)
+    ms, _ = _events_ms(lambda i: modulated_deform_conv(x, off, msk, w, bias, 1, 1, 1, 1, 1), n, 3)
+    flops = 2 * B * C * C * 9 * H * W
+    xs, ws, offs, ms_ = [t.clone().requires_grad_(True) for t in (x, w, off, msk)]
+
+    def train(i):
+        y = modulated_deform_conv(xs, offs, ms_, ws, bias, 1, 1, 1, 1, 1)
+        y.backward(y)
+
+    tms, _ = _events_ms(train, 5, 2)
+    res["dcnv2_2d_fp16_[8,256,100,152]_3x3"] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 2),
+                                                "forward_backward_ms": round(tms, 3)}
+    # augmentation stages on one fp16 CT-sized sample [1, 128, 256, 256] with a label map
+    np.random.seed(0)
+    sample = {"img": torch.randn(1, 128, 256, 256, generator=g).half().to(dev),
+              "gt_seg": torch.randint(0, 3, (1, 128, 256, 256), generator=g, dtype=torch.int32).to(dev),
+              "img_dim": 3, "img_spacing": (1.0, 1.0, 1.0), "img_fields": ["img"], "seg_fields": ["gt_seg"],
+              "det_fields": []}
+    stages = {"CudaResize(0.75)": aug.CudaResize(factor=(0.75, 0.75, 0.75)),
+              "CudaRandomAffine": aug.CudaRandomAffine(1.0, 0.2, 0.1, 30),
+              "CudaCropRandomWithAffine(96^3)": aug.CudaCropRandomWithAffine((96, 96, 96), 0.2, 0.1, 30),
+              "CudaRandomElasticDeformation": aug.CudaRandomElasticDeformation(1.0, 8, 0.8)}
+    for name, stage in stages.items():
+        ms, wall = _events_ms(lambda i: stage(dict(sample)), 10, 2)
+        res["aug:" + name] = {"ms_gpu": round(ms, 3), "ms_wall": round(wall, 3)}
+    return res
+
+
 def cpu_baseline(args):
     """fp64 oracle (C, OpenMP) on the benchmark's config-2 inputs (all 4 samples), repeated until
     about 12 s of wall time have been spent; the median pass is reported."""
@@ -169,6 +226,7 @@ def main():
     ap.add_argument("--copies", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-dcn", action="store_true", help="skip the DCN leg")
+    ap.add_argument("--no-next", action="store_true", help="skip the timings of the neighbouring operators")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="wall time spent on the CPU oracle")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a device copy of 4*128^3 fp16 elements (counter calibration)")
@@ -215,6 +273,8 @@ def main():
                                     "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                                     "frac": round(d["tflops"] / MFMA_F16_PEAK_TFLOPS, 5),
                                     "traffic": None, "flops_per_launch": d["flops"]}}
+    if not args.no_next:
+        line["next_rows"] = bench_next_rows(args)
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(args)
         line["cpu_reference_paths"] = cpu_reference_paths(args)

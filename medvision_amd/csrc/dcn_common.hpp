@@ -91,9 +91,12 @@ __device__ __forceinline__ void zero_pad_taps(const DcnDims &s, double pd, doubl
 template <typename P, typename T>
 __device__ __forceinline__ void dcn_offsets(const DcnDims &s, const T *__restrict__ o, P &fd, P &fh,
                                             P &fw) {
-  fd = s.nd == 3 ? static_cast<P>(load(o)) : P(0);
-  fh = static_cast<P>(load(o + (s.nd - 2) * s.Q));
-  fw = static_cast<P>(load(o + (s.nd - 1) * s.Q));
+  // three unconditional loads (for images the first one re-reads the row component and is dropped)
+  const long step = (s.nd - 2) * s.Q;
+  const P first = static_cast<P>(load(o));
+  fd = s.nd == 3 ? first : P(0);
+  fh = static_cast<P>(load(o + step));
+  fw = static_cast<P>(load(o + step + s.Q));
 }
 
 // Sample position of tap k at output position (od,oh,ow) for (b, dgi).
