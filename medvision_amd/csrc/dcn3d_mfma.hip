@@ -190,15 +190,20 @@ __global__ __launch_bounds__(256) void dcn_weight_fragments16_kernel(const T *__
   for (int i = 0; i < PC; i++) wf[id * PC + i] = wt[(static_cast<long>(o) * s.cpg + cl + i) * s.K + k];
 }
 
-constexpr int kWeightLds = 16 * 1024;  // one tap's weight pieces of a group, per buffer
+// blocks of 16 positions per wavefront: one keeps the kernel at 96 registers = 5 wavefronts per
+// SIMD, which hides more of the gather latency than the reuse of two blocks would save
+#ifndef MV_DCN_NB
+#define MV_DCN_NB 1
+#endif
+constexpr int kWeightLds = 12 * 1024;  // one tap's weight pieces of a group, per buffer
 
-template <typename T, int MB>
-__global__ __launch_bounds__(256, 4) void dcn_forward_mfma16_kernel(
+template <typename T, int MB, int NB>
+__global__ __launch_bounds__(256, NB == 1 ? 5 : 4) void dcn_forward_mfma16_kernel(
     const T *__restrict__ xt, const T *__restrict__ off, const T *__restrict__ mask,
     const T *__restrict__ wf, const T *__restrict__ bias, T *__restrict__ y, const DcnDims s) {
   using M = Mfma<T>;
   using P = typename std::conditional<(sizeof(T) == 2), float, double>::type;  // position type
-  constexpr int PC = M::kPiece, SL = 4 * PC, ES = sizeof(T), NB = 2;
+  constexpr int PC = M::kPiece, SL = 4 * PC, ES = sizeof(T);
   __shared__ __attribute__((aligned(16))) unsigned char wlds[2][kWeightLds];
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int j = lane % 16, kc = lane / 16;   // matrix layout: position (column) and piece of this lane
@@ -230,9 +235,13 @@ __global__ __launch_bounds__(256, 4) void dcn_forward_mfma16_kernel(
   // weight pieces of one tap: [slice][block of this chunk][lane] 16 bytes, copied by the workgroup
   const int tap_pieces = slices * MB * 64;                       // 16-byte pieces per tap
   const T *wfg = wf + static_cast<long>(g) * s.K * slices * blocks * (64 * PC);
-  auto fill = [&](int k, int buf) {
-    for (int i = threadIdx.x; i < tap_pieces; i += 256) {
-      const int ln = i % 64, m = (i / 64) % MB, cc = i / (64 * MB);
+  // as many taps per refill as fit: one workgroup barrier per group of taps
+  const int group = max(1, min(s.K, kWeightLds / 16 / tap_pieces));
+  auto fill = [&](int k0, int buf) {
+    const int count = min(group, s.K - k0) * tap_pieces;
+    for (int i = threadIdx.x; i < count; i += 256) {
+      const int k = k0 + i / tap_pieces, rem = i % tap_pieces;
+      const int ln = rem % 64, m = (rem / 64) % MB, cc = rem / (64 * MB);
       u32x4 v = u32x4{0u, 0u, 0u, 0u};
       if (mb0 + m < blocks)
         v = *reinterpret_cast<const u32x4 *>(wfg + (((static_cast<long>(k) * slices + cc) * blocks + mb0 + m) * 64 + ln) * PC);
@@ -245,9 +254,9 @@ __global__ __launch_bounds__(256, 4) void dcn_forward_mfma16_kernel(
   const int dg_first = g * s.cpg / s.cpd, dg_last = (g * s.cpg + s.cpg - 1) / s.cpd;
   const unsigned cin = s.Cin;
   int ki = 0, kj = 0, kk = 0;
-  for (int k = 0; k < s.K; k++) {
-    if (k + 1 < s.K) fill(k + 1, (k + 1) & 1);
-    const u32x4 *wl = reinterpret_cast<const u32x4 *>(wlds[k & 1]);
+  for (int k = 0, in_group = 0, buf = 0; k < s.K; k++) {
+    if (in_group == 0 && k + group < s.K) fill(k + group, buf ^ 1);
+    const u32x4 *wl = reinterpret_cast<const u32x4 *>(wlds[buf]) + in_group * tap_pieces;
     for (int dgi = dg_first; dgi <= dg_last; dgi++) {
       const int c_lo = max(g * s.cpg, dgi * s.cpd), c_hi = min(g * s.cpg + s.cpg, (dgi + 1) * s.cpd);
       const int cc_lo = (c_lo - g * s.cpg) / SL, cc_hi = (c_hi - g * s.cpg) / SL;
@@ -286,7 +295,11 @@ __global__ __launch_bounds__(256, 4) void dcn_forward_mfma16_kernel(
       }
     }
     if (++kk == s.kw) { kk = 0; if (++kj == s.kh) { kj = 0; ++ki; } }
-    __syncthreads();  // the other buffer is complete, this one may be refilled
+    if (++in_group == group) {
+      in_group = 0;
+      buf ^= 1;
+      __syncthreads();  // the other buffer is complete, this one may be refilled
+    }
   }
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) {
@@ -357,11 +370,12 @@ static int dcn_mfma_run(const void *x, const void *off, const void *mask, const 
       hipLaunchKernelGGL((dcn_weight_fragments16_kernel<T>), dim3(static_cast<unsigned>((lanes + 255) / 256)),
                          dim3(256), 0, stream, static_cast<const T *>(wt), wf, s);
       const int chunks = (blocks16 + mb - 1) / mb;
-      const long qblocks = (s.Q + 127) / 128;
+      constexpr int kNb = MV_DCN_NB;
+      const long qblocks = (s.Q + 64 * kNb - 1) / (64 * kNb);
       MV_REQUIRE(qblocks < (1L << 31) && static_cast<long>(s.groups) * chunks <= 65535, "grid too large");
       const dim3 grid(static_cast<unsigned>(qblocks), s.groups * chunks, s.B), block(256);
 #define MV_LAUNCH_MFMA16(MBV)                                                                    \
-  hipLaunchKernelGGL((dcn_forward_mfma16_kernel<T, MBV>), grid, block, 0, stream, xt,            \
+  hipLaunchKernelGGL((dcn_forward_mfma16_kernel<T, MBV, kNb>), grid, block, 0, stream, xt,       \
                      static_cast<const T *>(off), static_cast<const T *>(mask), wf,              \
                      static_cast<const T *>(bias), static_cast<T *>(y), s)
       if (mb == 4) MV_LAUNCH_MFMA16(4);
