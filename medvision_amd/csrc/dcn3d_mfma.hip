@@ -195,16 +195,18 @@ __global__ __launch_bounds__(256) void dcn_weight_fragments16_kernel(const T *__
 #ifndef MV_DCN_NB
 #define MV_DCN_NB 1
 #endif
-constexpr int kWeightLds = 12 * 1024;  // one tap's weight pieces of a group, per buffer
+// bytes per weight buffer (two per workgroup): 12 KB lets five workgroups share a CU's LDS, 16 KB
+// (four workgroups) serves layers whose tap does not fit the smaller one
+constexpr int kWeightLdsSmall = 12 * 1024, kWeightLds = 16 * 1024;
 
-template <typename T, int MB, int NB>
+template <typename T, int MB, int NB, int WBYTES>
 __global__ __launch_bounds__(256, NB == 1 ? 5 : 4) void dcn_forward_mfma16_kernel(
     const T *__restrict__ xt, const T *__restrict__ off, const T *__restrict__ mask,
     const T *__restrict__ wf, const T *__restrict__ bias, T *__restrict__ y, const DcnDims s) {
   using M = Mfma<T>;
   using P = typename std::conditional<(sizeof(T) == 2), float, double>::type;  // position type
   constexpr int PC = M::kPiece, SL = 4 * PC, ES = sizeof(T);
-  __shared__ __attribute__((aligned(16))) unsigned char wlds[2][kWeightLds];
+  __shared__ __attribute__((aligned(16))) unsigned char wlds[2][WBYTES];
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int j = lane % 16, kc = lane / 16;   // matrix layout: position (column) and piece of this lane
   const int lj = lane / 4, lk = lane % 4;    // load layout
@@ -236,7 +238,7 @@ __global__ __launch_bounds__(256, NB == 1 ? 5 : 4) void dcn_forward_mfma16_kerne
   const int tap_pieces = slices * MB * 64;                       // 16-byte pieces per tap
   const T *wfg = wf + static_cast<long>(g) * s.K * slices * blocks * (64 * PC);
   // as many taps per refill as fit: one workgroup barrier per group of taps
-  const int group = max(1, min(s.K, kWeightLds / 16 / tap_pieces));
+  const int group = max(1, min(s.K, WBYTES / 16 / tap_pieces));
   auto fill = [&](int k0, int buf) {
     const int count = min(group, s.K - k0) * tap_pieces;
     for (int i = threadIdx.x; i < count; i += 256) {
@@ -374,13 +376,19 @@ static int dcn_mfma_run(const void *x, const void *off, const void *mask, const 
       const long qblocks = (s.Q + 64 * kNb - 1) / (64 * kNb);
       MV_REQUIRE(qblocks < (1L << 31) && static_cast<long>(s.groups) * chunks <= 65535, "grid too large");
       const dim3 grid(static_cast<unsigned>(qblocks), s.groups * chunks, s.B), block(256);
-#define MV_LAUNCH_MFMA16(MBV)                                                                    \
-  hipLaunchKernelGGL((dcn_forward_mfma16_kernel<T, MBV, kNb>), grid, block, 0, stream, xt,       \
+#define MV_LAUNCH_MFMA16(MBV, WB)                                                                \
+  hipLaunchKernelGGL((dcn_forward_mfma16_kernel<T, MBV, kNb, WB>), grid, block, 0, stream, xt,   \
                      static_cast<const T *>(off), static_cast<const T *>(mask), wf,              \
                      static_cast<const T *>(bias), static_cast<T *>(y), s)
-      if (mb == 4) MV_LAUNCH_MFMA16(4);
-      else if (mb == 2) MV_LAUNCH_MFMA16(2);
-      else MV_LAUNCH_MFMA16(1);
+      if (tap_bytes <= kWeightLdsSmall) {
+        if (mb == 4) MV_LAUNCH_MFMA16(4, kWeightLdsSmall);
+        else if (mb == 2) MV_LAUNCH_MFMA16(2, kWeightLdsSmall);
+        else MV_LAUNCH_MFMA16(1, kWeightLdsSmall);
+      } else {
+        if (mb == 4) MV_LAUNCH_MFMA16(4, kWeightLds);
+        else if (mb == 2) MV_LAUNCH_MFMA16(2, kWeightLds);
+        else MV_LAUNCH_MFMA16(1, kWeightLds);
+      }
 #undef MV_LAUNCH_MFMA16
       return check_launch("dcn_forward_mfma16_kernel");
     }
