@@ -50,81 +50,158 @@ struct PlanShape {
   int threads, max_items;         // workgroup size, 16-byte groups one lane holds in registers
 };
 
-__device__ inline void plan_tile(const RoiGeom &g, const RoiProblem &p, const PlanShape &ps,
-                                 unsigned roi, unsigned tile, TilePlan *dst) {
-  const int is3d = p.ndim == 3;
-  const int t0[3] = {static_cast<int>(tile % ps.tiles_x) * ps.tx,
-                     static_cast<int>((tile / ps.tiles_x) % ps.tiles_y) * ps.ty,
-                     static_cast<int>(tile / (ps.tiles_x * ps.tiles_y)) * ps.tz};
-  const int out[3] = {p.ow, p.oh, p.od}, size[3] = {p.W, p.H, p.D}, ext[3] = {ps.tx, ps.ty, ps.tz};
-  double first[3], half[3];  // local coordinate of the tile's first voxel, half span per axis
-  for (int j = 0; j < 3; j++) {
-    const int cells = min(ext[j], out[j] - t0[j]);
-    const bool live = j < p.ndim;
-    first[j] = live ? local_coord(g, j, t0[j], 0) : 0.0;
-    half[j] = live ? 0.5 * (cells - 1) * g.bin[j] : 0.0;
+constexpr unsigned kDone = 0xffffffffu;  // "no item"
+
+// Lane-parallel planning: four lanes per item, lane `a` = 0..2 owns source axis / roi angle `a`
+// (lane 3 idles), so the three sin / cos pairs, the per-axis divisions and the three box
+// intervals of an item are evaluated side by side; values of the other axes come in through
+// wave shuffles.  Every lane of the wavefront must call this (`item` may be kDone: nothing is
+// written).  Same formulas as build_geom / local_coord in roi_geometry.hpp.
+__device__ __forceinline__ double lane_get(double v, int src_lane) {
+  const int lo = __builtin_amdgcn_ds_bpermute(src_lane * 4, __double2loint(v));
+  const int hi = __builtin_amdgcn_ds_bpermute(src_lane * 4, __double2hiint(v));
+  return __hiloint2double(hi, lo);
+}
+__device__ __forceinline__ int lane_get(int v, int src_lane) {
+  return __builtin_amdgcn_ds_bpermute(src_lane * 4, v);
+}
+
+__device__ inline void plan_item_lanes(const float *__restrict__ rois, const RoiProblem &p,
+                                       const PlanShape &ps, unsigned item, unsigned total,
+                                       unsigned per_roi, TilePlan *dst) {
+  const int lane = threadIdx.x & (kWave - 1), a = lane & 3, base = lane & ~3;
+  const bool write = item != kDone && a < 3;
+  const unsigned it = item != kDone ? item : 0u;
+  const unsigned idx = p.C > 1 ? it % total : it, n = idx / per_roi, tile = idx - n * per_roi;
+  const int nd = p.ndim, is3d = nd == 3, ax = a < 3 ? a : 0;
+  const float *roi = rois + static_cast<long>(n) * roi_columns(nd, p.rotated);
+
+  // ---- angle `ax`, axis `ax` of the roi -------------------------------------------------------
+  double sn, cs;
+  roi_trig(roi, p, ax, sn, cs);
+  const int cells_all[3] = {p.ow, p.oh, p.od}, size_all[3] = {p.W, p.H, p.D}, ext_all[3] = {ps.tx, ps.ty, ps.tz};
+  const int out_cells = ax == 0 ? cells_all[0] : (ax == 1 ? cells_all[1] : cells_all[2]);
+  const int S = ax == 0 ? size_all[0] : (ax == 1 ? size_all[1] : size_all[2]);
+  const int tile_ext = ax == 0 ? ext_all[0] : (ax == 1 ? ext_all[1] : ext_all[2]);
+  const bool live_axis = ax < nd;
+  double centre = 0.0, start = 0.0, bin = 0.0, sub = 0.0;
+  int grid = 1;
+  if (live_axis) {
+    const double sc = p.scale;
+    double ext;
+    if (p.rotated) {
+      ext = static_cast<double>(roi[1 + nd + ax]) * sc;
+      if (!p.aligned) ext = fmax(ext, 1.0);
+      centre = static_cast<double>(roi[1 + ax]) * sc - (p.aligned ? 0.5 : 0.0);
+      start = -ext / 2.0;
+    } else {
+      const double lo = static_cast<double>(roi[1 + ax]) * sc, hi = static_cast<double>(roi[1 + nd + ax]) * sc;
+      ext = fmax(hi - lo, 1.0);
+      start = lo;
+    }
+    bin = ext / static_cast<double>(out_cells);
+    grid = p.sampling_ratio > 0 ? p.sampling_ratio : static_cast<int>(ceil(ext / static_cast<double>(out_cells)));
+    sub = bin / static_cast<double>(grid > 0 ? grid : 1);
   }
-  TilePlan plan;
-  plan.batch = g.batch;
-  plan.roi = static_cast<int>(roi);
-  for (int j = 0; j < 3; j++) plan.t0[j] = t0[j];
-  bool empty = false, clipped = false;
-  for (int a = 0; a < 3; a++) {
-    double mid = g.centre[a], reach = 0.0, pos = g.centre[a];
-    for (int j = 0; j < 3; j++) {
-      const double r = g.rot[a * 3 + j];
-      mid += r * (first[j] + half[j]);
-      reach += fabs(r * half[j]);
-      pos += r * first[j];
-      plan.inc[a * 3 + j] = (j < p.ndim) ? r * g.bin[j] : 0.0;
+  const int b = static_cast<int>(roi[0]);
+  const int batch = (b >= 0 && b < p.N) ? b : -1;
+
+  // ---- row `ax` of the rotation ----------------------------------------------------------------
+  double row[3] = {ax == 0 ? 1.0 : 0.0, ax == 1 ? 1.0 : 0.0, ax == 2 ? 1.0 : 0.0};
+  if (p.rotated) {
+    const double sg = lane_get(sn, base), cg = lane_get(cs, base);
+    const double sb = lane_get(sn, base + 1), cb = lane_get(cs, base + 1);
+    const double sa = lane_get(sn, base + 2), ca = lane_get(cs, base + 2);
+    if (is3d) {
+      if (ax == 0) { row[0] = ca * cb; row[1] = ca * sb * sg - sa * cg; row[2] = ca * sb * cg + sa * sg; }
+      else if (ax == 1) { row[0] = sa * cb; row[1] = sa * sb * sg + ca * cg; row[2] = sa * sb * cg - ca * sg; }
+      else { row[0] = -sb; row[1] = cb * sg; row[2] = cb * cg; }
+    } else {   // one angle, held by lane 0 of the group
+      if (ax == 0) { row[0] = cg; row[1] = -sg; }
+      else if (ax == 1) { row[0] = sg; row[1] = cg; }
     }
-    if (!is3d && a == 2) {
-      plan.lo[a] = 0; plan.n[a] = 1; plan.org[a] = 0.0;
-      continue;
-    }
+  }
+
+  // ---- the tile along axis `ax` -----------------------------------------------------------------
+  const unsigned qx = tile / static_cast<unsigned>(ps.tiles_x), qy = qx / static_cast<unsigned>(ps.tiles_y);
+  const int tpos = ax == 0 ? static_cast<int>(tile - qx * ps.tiles_x)
+                           : (ax == 1 ? static_cast<int>(qx - qy * ps.tiles_y) : static_cast<int>(qy));
+  const int t0 = tpos * tile_ext;
+  const int cells = min(tile_ext, out_cells - t0);
+  const double first = live_axis ? start + t0 * bin + static_cast<double>(.5f) * sub : 0.0;
+  const double half = live_axis ? 0.5 * (cells - 1) * bin : 0.0;
+  double mid = centre, reach = 0.0, pos = centre, inc[3];
+  int grids = 1;
+#pragma unroll
+  for (int j = 0; j < 3; j++) {
+    const double fj = lane_get(first, base + j), hj = lane_get(half, base + j), bj = lane_get(bin, base + j);
+    const int gj = lane_get(grid, base + j);
+    mid += row[j] * (fj + hj);
+    reach += fabs(row[j] * hj);
+    pos += row[j] * fj;
+    inc[j] = j < nd ? row[j] * bj : 0.0;
+    if (j < nd && gj != 1) grids = 0;
+  }
+  int lo = 0, cnt = 1, empty = 0, clipped = 0;
+  double org = 0.0;
+  if (is3d || ax < 2) {
     // widen by more than the rounding of the per-voxel coordinate arithmetic
     const double eps = 4e-5, rmin = mid - reach - eps, rmax = mid + reach + eps;
-    const int S = size[a];
-    empty |= rmax < -1.0 || rmin > S;
-    clipped |= rmin < 0.0 || rmax > S - 1;
+    empty = rmax < -1.0 || rmin > S;
+    clipped = rmin < 0.0 || rmax > S - 1;
     int l = static_cast<int>(fmin(floor(fmax(rmin, 0.0)), static_cast<double>(S - 1)));
     int h = static_cast<int>(fmin(floor(fmax(rmax, 0.0)) + 1.0, static_cast<double>(S - 1)));
-    if (a == 0 && ps.vec > 0) {  // whole 16-byte groups
-      l = l / ps.vec * ps.vec;
-      h = min((h / ps.vec + 1) * ps.vec, S) - 1;
+    if (ax == 0 && ps.vec > 0) {  // whole 16-byte groups (vec is 4 or 8)
+      const int sh = ps.vec == 8 ? 3 : 2;
+      l = (l >> sh) << sh;
+      h = min(((h >> sh) + 1) << sh, S) - 1;
     }
-    plan.lo[a] = l;
-    plan.n[a] = h - l + 1;
-    plan.org[a] = pos - static_cast<double>(l);
+    lo = l;
+    cnt = h - l + 1;
+    org = pos - static_cast<double>(l);
   }
+  const int n0 = lane_get(cnt, base), n1 = lane_get(cnt, base + 1), n2 = lane_get(cnt, base + 2);
+  const int any_empty = lane_get(empty, base) | lane_get(empty, base + 1) | lane_get(empty, base + 2);
+  const int any_clip = lane_get(clipped, base) | lane_get(clipped, base + 1) | lane_get(clipped, base + 2);
+  if (!write) return;
+  dst->org[a] = org;
+  dst->orgf[a] = static_cast<float>(org);
+#pragma unroll
+  for (int j = 0; j < 3; j++) {
+    dst->inc[a * 3 + j] = inc[j];
+    dst->incf[a * 3 + j] = static_cast<float>(inc[j]);
+  }
+  dst->lo[a] = lo;
+  dst->n[a] = cnt;
+  dst->t0[a] = t0;
+  if (a != 0) return;
   // LDS row pitch: the row's 16-byte groups, or (unaligned rows) the row plus one finite pad
-  const int groups = ps.vec > 0 ? plan.n[0] / ps.vec : 0;
-  const int pitch = ps.vec > 0 ? plan.n[0] : plan.n[0] + 1;
-  const long rows = static_cast<long>(plan.n[1]) * plan.n[2];
+  const int groups = ps.vec > 0 ? n0 / ps.vec : 0;
+  const int pitch = ps.vec > 0 ? n0 : n0 + 1;
+  const long rows = static_cast<long>(n1) * n2;
   // register staging: a pass copies `span` whole z-slices, one 16-byte group per lane
-  plan.rp = 0; plan.span = 0; plan.passes = 0; plan.spare = 0;
+  int rp = 0, span = 0, passes = 0;
   if (ps.vec > 0) {
-    const int per_slice = plan.n[1] * groups;
-    const int span = min(ps.threads / per_slice, plan.n[2]);
-    if (span >= 1 && (plan.n[2] + span - 1) / span <= ps.max_items) {
-      plan.span = span;
-      plan.rp = span * plan.n[1];
-      plan.passes = (plan.n[2] + span - 1) / span;
+    const int per_slice = n1 * groups;   // small integers: the float quotients below are exact
+    const int sp = min(static_cast<int>(static_cast<float>(ps.threads) / static_cast<float>(per_slice)), n2);
+    if (sp >= 1) {
+      const int ps_ = static_cast<int>(static_cast<float>(n2 + sp - 1) / static_cast<float>(sp));
+      if (ps_ <= ps.max_items) { span = sp; rp = sp * n1; passes = ps_; }
     }
   }
-  for (int a = 0; a < 3; a++) plan.orgf[a] = static_cast<float>(plan.org[a]);
-  for (int i = 0; i < 9; i++) plan.incf[i] = static_cast<float>(plan.inc[i]);
+  dst->batch = batch;
+  dst->roi = static_cast<int>(n);
+  dst->rp = rp; dst->span = span; dst->passes = passes; dst->spare = 0;
   const bool fits = rows * pitch <= ps.cap;
-  const bool grid_one = g.grid[0] == 1 && g.grid[1] == 1 && (!is3d || g.grid[2] == 1);
-  if (g.batch < 0 || empty || !grid_one) plan.mode = 0;   // (grid != 1 cannot happen: ratio is 1)
-  else if (!fits) plan.mode = 2;
-  else plan.mode = clipped ? 1 : 3;
-  *dst = plan;
+  int mode;
+  if (batch < 0 || any_empty || !grids) mode = 0;   // (grid != 1 cannot happen: ratio is 1)
+  else if (!fits) mode = 2;
+  else mode = any_clip ? 1 : 3;
+  dst->mode = mode;
 }
 
 constexpr unsigned kChunk = 32;     // consecutive items dealt to one XCD
 constexpr unsigned kPlanSlots = 16; // items per workgroup: their plan records are kept in LDS
-constexpr unsigned kDone = 0xffffffffu;
 
 __device__ __forceinline__ float clamp_ct(float v, float lo, float hi) { return __builtin_amdgcn_fmed3f(v, lo, hi); }
 __device__ __forceinline__ double clamp_ct(double v, double lo, double hi) { return fmin(fmax(v, lo), hi); }
@@ -277,22 +354,12 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
   const int tid = threadIdx.x;
   if (item_of(0) == kDone) return;
 
-  // ---- plans of this workgroup's items (at most kPlanSlots): one lane per item, into LDS ------
+  // ---- plans of this workgroup's items (at most kPlanSlots): four lanes per item, into LDS -----
   const unsigned per_roi = static_cast<unsigned>(ps.tiles_x) * ps.tiles_y * ps.tiles_z;
-  {
-    if (tid < static_cast<int>(kPlanSlots)) {
-      const unsigned r = tid, item = item_of(r);
-      if (item != kDone) {
-        const unsigned idx = C > 1 ? item % total : item, n = idx / per_roi;
-        const float *roi = rois + static_cast<long>(n) * roi_columns(p.ndim, p.rotated);
-        double sn[3], cs[3];
-#pragma unroll
-        for (int a = 0; a < 3; a++) roi_trig(roi, p, a, sn[a], cs[a]);
-        RoiGeom g;
-        build_geom(g, roi, p, sn, cs);
-        plan_tile(g, p, ps, n, idx - n * per_roi, &lplans[r]);
-      }
-    }
+  if (tid < kWave) {
+    static_assert(kPlanSlots * 4 == kWave, "four lanes per plan slot");
+    const unsigned r = tid >> 2;
+    plan_item_lanes(rois, p, ps, item_of(r), total, per_roi, &lplans[r]);
   }
   __syncthreads();
   auto fetch_plan = [&](unsigned r) -> PlanLanes {
