@@ -203,6 +203,11 @@ __device__ inline void plan_item_lanes(const float *__restrict__ rois, const Roi
 constexpr unsigned kChunk = 32;     // consecutive items dealt to one XCD
 constexpr unsigned kPlanSlots = 16; // items per workgroup: their plan records are kept in LDS
 
+// a wave-uniform value moved to a scalar register
+__device__ __forceinline__ float uniform(float v) { return __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(v))); }
+__device__ __forceinline__ double uniform(double v) {
+  return __hiloint2double(__builtin_amdgcn_readfirstlane(__double2hiint(v)), __builtin_amdgcn_readfirstlane(__double2loint(v)));
+}
 __device__ __forceinline__ float clamp_ct(float v, float lo, float hi) { return __builtin_amdgcn_fmed3f(v, lo, hi); }
 __device__ __forceinline__ double clamp_ct(double v, double lo, double hi) { return fmin(fmax(v, lo), hi); }
 __device__ __forceinline__ float frac_of(float v) { return __builtin_amdgcn_fractf(v); }
@@ -210,10 +215,10 @@ __device__ __forceinline__ double frac_of(double v) { return __builtin_amdgcn_fr
 __device__ __forceinline__ float mix(float w, float a, float b) { return fmaf(w, b, fmaf(-w, a, a)); }  // exact at w = 0, 1
 __device__ __forceinline__ int div_small(int i, float inv) { return static_cast<int>((static_cast<float>(i) + 0.5f) * inv); }
 
-// Box-relative limits (wave-uniform): a sample is void outside [vmin, vmax]; coordinates clamp to
-// [0, cmax]; the low tap index is at most top = max(n - 2, 0) so that the high tap stays inside
+// Box-relative limits (wave-uniform): coordinates clamp to [0, cmax] (a sample the clamp moves by
+// more than 1 lies outside [-1, size] of the volume and is void); the low tap index is at most top = max(n - 2, 0) so that the high tap stays inside
 // the box (a coordinate on the last voxel gets weight 1 on the high tap).
-template <typename CT> struct BoxLimits { CT vmin[3], vmax[3], cmax[3], top[3]; };
+template <typename CT> struct BoxLimits { CT cmax[3], top[3]; };
 
 // Element index of the low corner and the three fractions.  fp32 coordinates: floor / fraction /
 // index all in fp32 (indices stay far below 2^24, so the two FMAs are exact).
@@ -244,11 +249,14 @@ __device__ __forceinline__ float staged_sample(const T *__restrict__ tile, CT rx
   if (INTERIOR) {  // all taps of all samples lie inside the box
     lx = floor(rx); ly = floor(ry); lz = floor(rz);
   } else {
-    ok = rx >= b.vmin[0] && rx <= b.vmax[0] && ry >= b.vmin[1] && ry <= b.vmax[1] &&
-         rz >= b.vmin[2] && rz <= b.vmax[2];
+    // void outside [vmin, vmax] = [-1, size] of the volume: wherever the clamp to [0, cmax] can
+    // act it acts at the volume border (vmin = -1, vmax = cmax + 1), so "inside" is "moved by at
+    // most 1 by the clamp" (the differences are exact: one operand is 0 or within a factor of 2)
+    const CT ux = rx, uy = ry, uz = rz;
     rx = clamp_ct(rx, CT(0), b.cmax[0]);
     ry = clamp_ct(ry, CT(0), b.cmax[1]);
     rz = clamp_ct(rz, CT(0), b.cmax[2]);
+    ok = fmax(fmax(fabs(ux - rx), fabs(uy - ry)), fabs(uz - rz)) <= CT(1);
     lx = fmin(floor(rx), b.top[0]); ly = fmin(floor(ry), b.top[1]); lz = fmin(floor(rz), b.top[2]);
   }
   const CT fx = rx - lx, fy = ry - ly, fz = rz - lz;
@@ -268,14 +276,16 @@ __device__ __forceinline__ float staged_sample(const T *__restrict__ tile, CT rx
 }
 
 // The lane's column of ZPL voxels, box-relative start b0..b2 and per-slice step s0..s2.
-template <typename T, typename CT, bool INTERIOR, int ORDER, int ZPL, bool WIDE = false>
+// `before(k)` runs ahead of voxel k while o[k] still holds the previous item's value.
+template <typename T, typename CT, bool INTERIOR, int ORDER, int ZPL, bool WIDE = false, typename Hook>
 __device__ __forceinline__ void staged_column(const T *__restrict__ tile, float (&o)[ZPL], CT b0, CT b1,
                                               CT b2, CT s0, CT s1, CT s2, const BoxLimits<CT> &lim,
-                                              int pitch, long slice, int dy, long dz) {
-  const float pitch_f = static_cast<float>(pitch), slice_f = static_cast<float>(slice);
+                                              int pitch, long slice, int dy, long dz, Hook before) {
+  const float pitch_f = uniform(static_cast<float>(pitch)), slice_f = uniform(static_cast<float>(slice));
 #pragma unroll
   for (int k = 0; k < ZPL; k++) {
     const CT kk = static_cast<CT>(k);
+    before(k);
     o[k] = staged_sample<T, CT, INTERIOR, ORDER, WIDE>(tile, b0 + kk * s0, b1 + kk * s1, b2 + kk * s2,
                                                        lim, pitch, slice, pitch_f, slice_f, dy, dz);
     // keep the scheduler from interleaving all voxels of the column (registers are scarce while
@@ -313,6 +323,23 @@ template <> __device__ __forceinline__ float plan_inc<float>(const PlanLanes &p,
 template <> __device__ __forceinline__ double plan_inc<double>(const PlanLanes &p, int i) { return p.f64(MV_PLAN_DW(inc) + 2 * i); }
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// One element through a buffer descriptor: offsets beyond the buffer drop the store, so lanes
+// without an output need no branch.
+template <typename T>
+__device__ __forceinline__ void store_element(__amdgpu_buffer_rsrc_t rsrc, unsigned voff, int soff, float v) {
+  const T t = store_cast<T>(v);
+  if constexpr (sizeof(T) == 2) {
+    unsigned short bits;
+    __builtin_memcpy(&bits, &t, 2);
+    __builtin_amdgcn_raw_buffer_store_b16(bits, rsrc, voff, soff, 0);
+  } else {
+    unsigned bits;
+    __builtin_memcpy(&bits, &t, 4);
+    __builtin_amdgcn_raw_buffer_store_b32(bits, rsrc, voff, soff, 0);
+  }
+}
+
 struct BoxShape { int mode, bx, by, bz, rp, span, passes; };  // wave-uniform part of a plan used for staging
 constexpr unsigned kOutOfRange = 0x80000000u;  // beyond every buffer: the load returns zeros
 
@@ -380,16 +407,26 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
   int st_zz = 0;     // zz0 of this lane (beyond every box for idle lanes)
   int st_dst = 0;    // LDS element offset of the lane's first group
   float o[ZPL];      // the previous item's outputs
-  T *pend_row = out;
+  // outputs waiting to be stored: descriptor of the (roi, channel) volume, the lane's byte offset
+  // in it, the number of voxels of the lane's column that exist
+  __amdgpu_buffer_rsrc_t pend_rsrc = __builtin_amdgcn_make_buffer_rsrc(out, 0, 0, 0x00020000);
+  unsigned pend_voff = kOutOfRange;
   int pend_count = 0;
+  const int zbytes = static_cast<int>(zstride) * ES;
+  const int out_bytes = od * zbytes;   // bytes of one output volume (< 2^31, checked by the host)
 
-  // Issue the loads of one item's box into val[]: the buffer ends with the box's last row, so
-  // passes that run beyond the last z-slice read zeros without a test.
-  auto issue = [&](const PlanLanes &pl, unsigned ch) -> BoxShape {
+  // The loads of one item's box into val[]: the buffer ends with the box's last row, so passes
+  // that run beyond the last z-slice read zeros without a test.  `prepare` sets the addresses up,
+  // `load_pass(u)` issues pass u (u < ld_passes, wave-uniform).
+  __amdgpu_buffer_rsrc_t ld_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(feat), 0, 0, 0x00020000);
+  unsigned ld_voff = kOutOfRange;
+  int ld_stride = 0, ld_passes = 0;
+  auto prepare = [&](const PlanLanes &pl, unsigned ch) -> BoxShape {
     BoxShape sh;
     sh.mode = pl.mode(); sh.bx = pl.n(0); sh.by = pl.n(1); sh.bz = pl.n(2);
     sh.rp = pl.rp(); sh.span = pl.span(); sh.passes = pl.passes();
     const int passes = sh.passes;
+    ld_passes = 0;
     if (vec == 0 || passes == 0 || (sh.mode != 1 && sh.mode != 3)) return sh;
     const int bx = sh.bx, by = sh.by, bz = sh.bz;
     const int groups = bx / V;
@@ -398,19 +435,21 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
     const long first = (static_cast<long>(pl.lo(2)) * H + pl.lo(1)) * W + pl.lo(0);
     const T *corner = feat + (static_cast<long>(pl.batch()) * C + ch) * plane + first;
     const int extent = (((bz - 1) * H + by - 1) * W + bx) * ES;
-    const __amdgpu_buffer_rsrc_t rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(corner), 0, extent, 0x00020000);
+    ld_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(corner), 0, extent, 0x00020000);
     const bool on = lr < sh.rp;
-    const unsigned voff = on ? static_cast<unsigned>(((zz * H + yy) * W + gi * V) * ES) : kOutOfRange;
-    const int stride = sh.span * H * W * ES;
+    ld_voff = on ? static_cast<unsigned>(((zz * H + yy) * W + gi * V) * ES) : kOutOfRange;
+    ld_stride = sh.span * H * W * ES;
+    ld_passes = passes;
     st_zz = on ? zz : (1 << 28);
     st_dst = lr * bx + gi * V;
-#pragma unroll
-    for (int u = 0; u < KMAX; u++)
-      if (u < passes) val[u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, u * stride, 0);  // wave-uniform test
     return sh;
   };
-  BoxShape cur = issue(fetch_plan(0), c);
+  auto load_pass = [&](int u) {
+    if (u < ld_passes) val[u] = __builtin_amdgcn_raw_buffer_load_b128(ld_rsrc, ld_voff, u * ld_stride, 0);
+  };
+  BoxShape cur = prepare(fetch_plan(0), c);
+#pragma unroll
+  for (int u = 0; u < KMAX; u++) load_pass(u);
   while (true) {
     const PlanLanes plan = fetch_plan(round);
     const int mode = cur.mode;
@@ -457,29 +496,33 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
     }
     __syncthreads();
 
-    // ---- B: previous outputs out, next box in flight ------------------------------------------
-#pragma unroll
-    for (int k = 0; k < ZPL; k++)
-      if (k < pend_count) pend_row[k * zstride] = store_cast<T>(o[k]);
+    // ---- B + C: this item; ahead of voxel k the previous item's voxel k is stored and a share of
+    // the next box's loads is issued, so that neither piles up in the memory pipeline -------------
     const bool more = wn != kDone;
     unsigned cn = 0;
     BoxShape nxt = cur;
+    ld_passes = 0;
     if (more) {
       if (C > 1) cn = wn / total;
-      nxt = issue(fetch_plan(round + 1), cn);
+      nxt = prepare(fetch_plan(round + 1), cn);
     }
-
-    // ---- C: this item -------------------------------------------------------------------------
+    auto before = [&](int k) {
+      store_element<T>(pend_rsrc, k < pend_count ? pend_voff : kOutOfRange, k * zbytes, o[k]);
+#pragma unroll
+      for (int u = 0; u < KMAX; u++)
+        if (u >= k * KMAX / ZPL && u < (k + 1) * KMAX / ZPL)   // compile-time share of the loads
+          val[u] = __builtin_amdgcn_raw_buffer_load_b128(ld_rsrc, u < ld_passes ? ld_voff : kOutOfRange,
+                                                         u * ld_stride, 0);
+    };
     const int ox = plan.t0(0) + lx, oy = plan.t0(1) + ly, zb = plan.t0(2) + lz * ZPL;
     const int count = (ox < ow && oy < oh) ? min(ZPL, od - zb) : 0;  // may be <= 0
-    T *drow = out + (static_cast<long>(plan.roi()) * C + c) * od * zstride +
-              (static_cast<long>(zb) * oh + oy) * ow + ox;
-    pend_row = drow;
-    pend_count = count;
     if (mode == 0) {
 #pragma unroll
-      for (int k = 0; k < ZPL; k++) o[k] = 0.f;
-    } else if (count > 0) {
+      for (int k = 0; k < ZPL; k++) {
+        before(k);
+        o[k] = 0.f;
+      }
+    } else {
       // position of this lane's first voxel and the per-slice increment, relative to the box (to
       // the feature map for mode 2), in the coordinate type (the box margin covers the rounding
       // of fp32 arithmetic)
@@ -490,35 +533,42 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
         b[a] = plan_org<CT>(plan, a) + fx * plan_inc<CT>(plan, a * 3) + fy * plan_inc<CT>(plan, a * 3 + 1) +
                fz * plan_inc<CT>(plan, a * 3 + 2);
         st[a] = plan_inc<CT>(plan, a * 3 + 2);
+        // lanes beyond the output keep step with the others (their part of the stores and loads
+        // is issued from the same code) and sample along the ray from the box origin (reads that
+        // leave the box return garbage or zero and are never stored)
+        if (count <= 0) b[a] = CT(0);
       }
       BoxLimits<CT> lim;
       if (mode == 3) {
         const int dy = by > 1 ? pitch : 0, dz = bz > 1 ? slice : 0;
-        if (order == 0) staged_column<T, CT, true, 0, ZPL>(tile, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, pitch, slice, dy, dz);
-        else staged_column<T, CT, true, 1, ZPL>(tile, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, pitch, slice, dy, dz);
+        if (order == 0) staged_column<T, CT, true, 0, ZPL>(tile, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, pitch, slice, dy, dz, before);
+        else staged_column<T, CT, true, 1, ZPL>(tile, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, pitch, slice, dy, dz, before);
       } else {
         const int size[3] = {W, H, D};
         const int lo[3] = {mode == 2 ? 0 : plan.lo(0), mode == 2 ? 0 : plan.lo(1), mode == 2 ? 0 : plan.lo(2)};
         const int n[3] = {mode == 2 ? W : bx, mode == 2 ? H : by, mode == 2 ? D : bz};
         for (int a = 0; a < 3; a++) {
-          lim.vmin[a] = static_cast<CT>(-1 - lo[a]); lim.vmax[a] = static_cast<CT>(size[a] - lo[a]);
-          lim.cmax[a] = static_cast<CT>(size[a] - 1 - lo[a]);
-          lim.top[a] = static_cast<CT>(max(n[a] - 2, 0));
+          lim.cmax[a] = uniform(static_cast<CT>(size[a] - 1 - lo[a]));
+          lim.top[a] = uniform(static_cast<CT>(max(n[a] - 2, 0)));
         }
         if (mode == 2) {  // the box does not fit in LDS: taps straight from the feature map
-          for (int a = 0; a < 3; a++) b[a] += static_cast<CT>(plan.lo(a));
+          for (int a = 0; a < 3; a++) b[a] += count > 0 ? static_cast<CT>(plan.lo(a)) : CT(0);
           const long hw = static_cast<long>(H) * W;
           const int dy = H > 1 ? W : 0;
           const long dz = D > 1 ? hw : 0;
-          if (order == 0) staged_column<T, CT, false, 0, ZPL, true>(src, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, W, hw, dy, dz);
-          else staged_column<T, CT, false, 1, ZPL, true>(src, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, W, hw, dy, dz);
+          if (order == 0) staged_column<T, CT, false, 0, ZPL, true>(src, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, W, hw, dy, dz, before);
+          else staged_column<T, CT, false, 1, ZPL, true>(src, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, W, hw, dy, dz, before);
         } else {
           const int dy = by > 1 ? pitch : 0, dz = bz > 1 ? slice : 0;
-          if (order == 0) staged_column<T, CT, false, 0, ZPL>(tile, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, pitch, slice, dy, dz);
-          else staged_column<T, CT, false, 1, ZPL>(tile, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, pitch, slice, dy, dz);
+          if (order == 0) staged_column<T, CT, false, 0, ZPL>(tile, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, pitch, slice, dy, dz, before);
+          else staged_column<T, CT, false, 1, ZPL>(tile, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, pitch, slice, dy, dz, before);
         }
       }
     }
+    pend_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        out + (static_cast<long>(plan.roi()) * C + c) * od * zstride, 0, out_bytes, 0x00020000);
+    pend_voff = static_cast<unsigned>(((zb * oh + oy) * ow + ox) * ES);
+    pend_count = count;
     if (!more) break;
     __syncthreads();  // every lane is done with the box
     w = wn; c = cn; cur = nxt;
@@ -527,7 +577,7 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
   }
 #pragma unroll
   for (int k = 0; k < ZPL; k++)
-    if (k < pend_count) pend_row[k * zstride] = store_cast<T>(o[k]);
+    store_element<T>(pend_rsrc, k < pend_count ? pend_voff : kOutOfRange, k * zbytes, o[k]);
 }
 
 // Compute units of the current device (workgroups resident at once = units * LDS share).
@@ -578,6 +628,7 @@ int roi_forward_tiled(const void *input, const void *rois, void *output, int dty
                       const RoiProblem &p, void *workspace, size_t *need, hipStream_t s) {
   const long vox = static_cast<long>(p.od) * p.oh * p.ow;
   if (p.sampling_ratio != 1 || vox < 4096 || p.ow < 16 || p.R == 0) return -1;
+  if (vox * 4 >= (1L << 31)) return -1;   // 32-bit byte offsets inside one output volume
   const float *r = static_cast<const float *>(rois);
   switch (dtype) {
     case MV_F16:
