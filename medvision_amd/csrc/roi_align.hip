@@ -162,10 +162,10 @@ int roi_forward(const void *input, const void *rois, void *output, int dtype, in
   if (num_rois == 0) return MV_OK;
   MV_REQUIRE(input && rois && output, "null pointer argument");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (order != 3) {
+  {
     const int tiled = roi_forward_tiled(input, rois, output, dtype, p, workspace, nullptr, s);
     if (tiled >= 0) return tiled;
-    const int pooled = roi_pool_forward(input, rois, output, dtype, p, s);
+    const int pooled = order != 3 ? roi_pool_forward(input, rois, output, dtype, p, s) : -1;
     if (pooled >= 0) return pooled;
   }
   const dim3 grid(p.chunks * num_rois), block(kRoiThreads);

@@ -48,6 +48,7 @@ struct PlanShape {
   int vec;                        // elements per aligned 16-byte group (0: rows are not aligned)
   int cap;                        // LDS capacity in elements
   int threads, max_items;         // workgroup size, 16-byte groups one lane holds in registers
+  int halo_lo, halo_hi;           // voxels needed below / above the cell of a sample: 0 / 1, order 3: 1 / 2
 };
 
 constexpr unsigned kDone = 0xffffffffu;  // "no item"
@@ -148,9 +149,9 @@ __device__ inline void plan_item_lanes(const float *__restrict__ rois, const Roi
     // widen by more than the rounding of the per-voxel coordinate arithmetic
     const double eps = 4e-5, rmin = mid - reach - eps, rmax = mid + reach + eps;
     empty = rmax < -1.0 || rmin > S;
-    clipped = rmin < 0.0 || rmax > S - 1;
-    int l = static_cast<int>(fmin(floor(fmax(rmin, 0.0)), static_cast<double>(S - 1)));
-    int h = static_cast<int>(fmin(floor(fmax(rmax, 0.0)) + 1.0, static_cast<double>(S - 1)));
+    clipped = rmin < static_cast<double>(ps.halo_lo) || rmax > S - ps.halo_hi;
+    int l = static_cast<int>(fmin(fmax(floor(fmax(rmin, 0.0)) - ps.halo_lo, 0.0), static_cast<double>(S - 1)));
+    int h = static_cast<int>(fmin(floor(fmax(rmax, 0.0)) + ps.halo_hi, static_cast<double>(S - 1)));
     if (ax == 0 && ps.vec > 0) {  // whole 16-byte groups (vec is 4 or 8)
       const int sh = ps.vec == 8 ? 3 : 2;
       l = (l >> sh) << sh;
@@ -218,7 +219,7 @@ __device__ __forceinline__ int div_small(int i, float inv) { return static_cast<
 // Box-relative limits (wave-uniform): coordinates clamp to [0, cmax] (a sample the clamp moves by
 // more than 1 lies outside [-1, size] of the volume and is void); the low tap index is at most top = max(n - 2, 0) so that the high tap stays inside
 // the box (a coordinate on the last voxel gets weight 1 on the high tap).
-template <typename CT> struct BoxLimits { CT cmax[3], top[3]; };
+template <typename CT> struct BoxLimits { CT cmax[3], top[3]; int one; };
 
 // Element index of the low corner and the three fractions.  fp32 coordinates: floor / fraction /
 // index all in fp32 (indices stay far below 2^24, so the two FMAs are exact).
@@ -273,6 +274,80 @@ __device__ __forceinline__ float staged_sample(const T *__restrict__ tile, CT rx
     v = mix(wz, mix(wy, x00, x01), mix(wy, x10, x11));
   }
   return ok ? v : 0.f;
+}
+
+// Order 3 from the staged box: clamped Catmull-Rom over 4 x 4 x 4 voxels (see cubic_tap in
+// sampling.hpp).  INTERIOR: all 64 taps of all samples are voxels of the box, no test, no clamp.
+// Otherwise a sample below -1 or above `size` (box-relative: b.cmax) is void, negatives snap to 0,
+// and the tap indices base-1 .. base+2 are clamped into the box, whose clipped sides are the
+// volume's own borders.  dy / dz are 0 for boxes one row / slice thick (images: every z tap reads
+// slice 0 and the z weights sum to 1).
+__device__ __forceinline__ void catmull_rom(float u, float (&w)[4]) {
+  const float u2 = u * u, u3 = u2 * u;
+  w[0] = -0.5f * u3 + u2 - 0.5f * u;
+  w[1] = 1.5f * u3 - 2.5f * u2 + 1.f;
+  w[2] = -1.5f * u3 + 2.f * u2 + 0.5f * u;
+  w[3] = 0.5f * u3 - 0.5f * u2;
+}
+
+template <typename T, typename CT, bool INTERIOR, bool WIDE>
+__device__ __forceinline__ float staged_cubic(const T *__restrict__ tile, CT rx, CT ry, CT rz,
+                                              const BoxLimits<CT> &b, int pitch, long slice, int dy, long dz) {
+  // void samples: an all-zero bit mask applied to the result (kept as data so that the 64 taps
+  // stay one straight-line block)
+  unsigned keep = 0xffffffffu;
+  if (!INTERIOR) {
+    const bool ok = rx >= CT(-1) && rx <= b.cmax[0] && ry >= CT(-1) && ry <= b.cmax[1] && rz >= CT(-1) && rz <= b.cmax[2];
+    keep = ok ? 0xffffffffu : 0u;
+    rx = fmax(rx, CT(0)); ry = fmax(ry, CT(0)); rz = fmax(rz, CT(0));
+  }
+  const CT lx = floor(rx), ly = floor(ry), lz = floor(rz);
+  float wx[4], wy[4], wz[4];
+  catmull_rom(static_cast<float>(rx - lx), wx);
+  catmull_rom(static_cast<float>(ry - ly), wy);
+  catmull_rom(static_cast<float>(rz - lz), wz);
+  float acc = 0.f;
+  if (INTERIOR) {
+    // `one` is 1, but only at run time: the four taps of a row must stay four 2-byte reads (merged
+    // into one 8-byte read at 2-byte alignment they take the slow unaligned LDS path)
+    const int one = b.one;
+    const int ix = static_cast<int>(lx) - 1, iy = static_cast<int>(ly) - 1, iz = static_cast<int>(lz) - 1;
+    const T *row = tile + (static_cast<long>(iz) * dz + static_cast<long>(iy) * dy + ix);
+#pragma unroll
+    for (int a = 0; a < 4; a++) {
+      float plane = 0.f;
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        plane += wy[c] * (wx[0] * load(row) + wx[1] * load(row + one) + wx[2] * load(row + 2 * one) +
+                          wx[3] * load(row + 3 * one));
+        row += dy;
+      }
+      row += dz - 4 * static_cast<long>(dy);
+      acc += wz[a] * plane;
+    }
+  } else {
+    // element offsets fit 32 bits: LDS boxes trivially, feature maps by the host's size check
+    const int bx = static_cast<int>(lx), by = static_cast<int>(ly), bz = static_cast<int>(lz);
+    const int tx = static_cast<int>(b.top[0]), ty = static_cast<int>(b.top[1]), tz = static_cast<int>(b.top[2]);
+    const int sy = WIDE ? pitch : dy, sz = static_cast<int>(WIDE ? slice : dz);
+    int ox[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) ox[k] = min(max(bx - 1 + k, 0), tx);
+#pragma unroll
+    for (int a = 0; a < 4; a++) {
+      const int za = min(max(bz - 1 + a, 0), tz) * sz;
+      float plane = 0.f;
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const T *row = tile + (za + min(max(by - 1 + c, 0), ty) * sy);
+        plane += wy[c] * (wx[0] * load(row + ox[0]) + wx[1] * load(row + ox[1]) + wx[2] * load(row + ox[2]) +
+                          wx[3] * load(row + ox[3]));
+      }
+      acc += wz[a] * plane;
+    }
+  }
+  (void)pitch; (void)slice;
+  return __uint_as_float(__float_as_uint(acc) & keep);
 }
 
 // The lane's column of ZPL voxels, box-relative start b0..b2 and per-slice step s0..s2.
@@ -581,6 +656,139 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
 }
 
 // Compute units of the current device (workgroups resident at once = units * LDS share).
+
+// Order-3 twin of the kernel above, kept simple because 64 taps per voxel dominate everything
+// else: same items, same work distribution and plans (boxes carry a halo of 1 / 2 voxels), but
+// the box is copied to LDS in place (no register prefetch) and every lane walks its column of
+// voxels in a rolled loop, storing as it goes.
+template <typename T, int TX, int TY, int TZ, int THREADS, int LDS_BYTES>
+__global__ __launch_bounds__(THREADS, 4) void roi_resample_cubic_kernel(
+    const T *__restrict__ feat, const float *__restrict__ rois, T *__restrict__ out, const RoiProblem p,
+    const PlanShape ps, const unsigned total, const unsigned work) {
+  using CT = typename std::conditional<(sizeof(T) == 2), float, double>::type;
+  constexpr int kCap = LDS_BYTES / sizeof(T);
+  constexpr int RZ = THREADS / (TX * TY), ZPL = TZ / RZ, V = 16 / sizeof(T);
+  __shared__ __attribute__((aligned(16))) T tile[kCap];
+  __shared__ TilePlan lplans[kPlanSlots];
+  const int C = p.C, D = p.D, H = p.H, W = p.W, od = p.od, oh = p.oh, ow = p.ow;
+  const int vec = ps.vec;
+  const unsigned parts = gridDim.x >= kXcds ? kXcds : 1;
+  const unsigned xcd = blockIdx.x % parts, slot = blockIdx.x / parts, slots = gridDim.x / parts;
+  auto item_of = [&](unsigned round) -> unsigned {
+    const unsigned k = round * slots + (slot + round * 27u) % slots;
+    const unsigned item = ((k / kChunk) * parts + xcd) * kChunk + k % kChunk;
+    return item < work ? item : kDone;
+  };
+  const int tid = threadIdx.x;
+  if (item_of(0) == kDone) return;
+  const unsigned per_roi = static_cast<unsigned>(ps.tiles_x) * ps.tiles_y * ps.tiles_z;
+  if (tid < kWave) plan_item_lanes(rois, p, ps, item_of(tid >> 2), total, per_roi, &lplans[tid >> 2]);
+  __syncthreads();
+  const int lx = tid % TX, ly = (tid / TX) % TY, lz = tid / (TX * TY);
+  const long zstride = static_cast<long>(oh) * ow, plane = static_cast<long>(D) * H * W;
+  for (unsigned round = 0;; round++) {
+    const unsigned w = item_of(round);
+    if (w == kDone) break;
+    const unsigned c = C > 1 ? w / total : 0;
+    PlanLanes plan;
+    {
+      const unsigned lane = tid & (kWave - 1);
+      plan.v = reinterpret_cast<const unsigned *>(&lplans[round])[lane < sizeof(TilePlan) / 4 ? lane : 0];
+    }
+    const int mode = plan.mode();
+    const int bx = plan.n(0), by = plan.n(1), bz = plan.n(2);
+    const int pitch = vec > 0 ? bx : bx + 1, slice = by * pitch;
+    const T *src = feat + (static_cast<long>(plan.batch()) * C + c) * plane;
+    if (mode == 1 || mode == 3) {   // the box into LDS
+      const int rows = by * bz;
+      const T *corner = src + (static_cast<long>(plan.lo(2)) * H + plan.lo(1)) * W + plan.lo(0);
+      const float inv_by = 1.0f / static_cast<float>(by);
+      if (vec > 0) {
+        const int groups = bx / V;
+        const float inv_groups = 1.0f / static_cast<float>(groups);
+        // eight independent 16-byte loads in flight per lane before the first LDS store
+        for (int i0 = tid; i0 < rows * groups; i0 += THREADS * 8) {
+          u32x4 v[8];
+#pragma unroll
+          for (int u = 0; u < 8; u++) {
+            const int i = i0 + u * THREADS;
+            if (i < rows * groups) {
+              const int r = div_small(i, inv_groups), gi = i - r * groups;
+              const int zz = div_small(r, inv_by), yy = r - zz * by;
+              v[u] = *reinterpret_cast<const u32x4 *>(corner + (static_cast<long>(zz) * H + yy) * W + gi * V);
+            }
+          }
+#pragma unroll
+          for (int u = 0; u < 8; u++) {
+            const int i = i0 + u * THREADS;
+            if (i < rows * groups) {
+              const int r = div_small(i, inv_groups), gi = i - r * groups;
+              *reinterpret_cast<u32x4 *>(tile + r * pitch + gi * V) = v[u];
+            }
+          }
+        }
+      } else {
+        for (int i = tid; i < rows * pitch; i += THREADS) {
+          const int r = i / pitch, e = i - r * pitch;
+          const int zz = div_small(r, inv_by), yy = r - zz * by;
+          tile[i] = e < bx ? corner[(static_cast<long>(zz) * H + yy) * W + e] : store_cast<T>(0.f);
+        }
+      }
+    }
+    __syncthreads();
+    const int ox = plan.t0(0) + lx, oy = plan.t0(1) + ly, zb = plan.t0(2) + lz * ZPL;
+    const int count = (ox < ow && oy < oh) ? min(ZPL, od - zb) : 0;
+    T *drow = out + (static_cast<long>(plan.roi()) * C + c) * od * zstride + (static_cast<long>(zb) * oh + oy) * ow + ox;
+    if (count > 0) {
+      const CT fx = static_cast<CT>(lx), fy = static_cast<CT>(ly), fz = static_cast<CT>(lz * ZPL);
+      CT b[3], st[3];
+#pragma unroll
+      for (int a = 0; a < 3; a++) {
+        b[a] = plan_org<CT>(plan, a) + fx * plan_inc<CT>(plan, a * 3) + fy * plan_inc<CT>(plan, a * 3 + 1) +
+               fz * plan_inc<CT>(plan, a * 3 + 2);
+        st[a] = plan_inc<CT>(plan, a * 3 + 2);
+      }
+      BoxLimits<CT> lim;
+      lim.one = ps.halo_lo;
+      const int size[3] = {W, H, D};
+      const int n[3] = {mode == 2 ? W : bx, mode == 2 ? H : by, mode == 2 ? D : bz};
+      for (int a = 0; a < 3; a++) {  // the volume's far end (inclusive) and the last index of the box
+        lim.cmax[a] = static_cast<CT>(size[a] - (mode == 2 ? 0 : plan.lo(a)));
+        lim.top[a] = static_cast<CT>(max(n[a] - 1, 0));
+      }
+      if (mode == 0) {
+        for (int k = 0; k < count; k++) drow[k * zstride] = store_cast<T>(0.f);
+      } else if (mode == 3) {
+        const int dy = by > 1 ? pitch : 0, dz = bz > 1 ? slice : 0;
+#pragma unroll 1
+        for (int k = 0; k < count; k++) {
+          const CT kk = static_cast<CT>(k);
+          drow[k * zstride] = store_cast<T>(staged_cubic<T, CT, true, false>(
+              tile, b[0] + kk * st[0], b[1] + kk * st[1], b[2] + kk * st[2], lim, pitch, slice, dy, dz));
+        }
+      } else if (mode == 2) {  // the box does not fit in LDS: taps straight from the feature map
+        for (int a = 0; a < 3; a++) b[a] += static_cast<CT>(plan.lo(a));
+        const long hw = static_cast<long>(H) * W;
+#pragma unroll 1
+        for (int k = 0; k < count; k++) {
+          const CT kk = static_cast<CT>(k);
+          drow[k * zstride] = store_cast<T>(staged_cubic<T, CT, false, true>(
+              src, b[0] + kk * st[0], b[1] + kk * st[1], b[2] + kk * st[2], lim, W, hw, W, hw));
+        }
+      } else {
+        const int dy = by > 1 ? pitch : 0, dz = bz > 1 ? slice : 0;
+#pragma unroll 1
+        for (int k = 0; k < count; k++) {
+          const CT kk = static_cast<CT>(k);
+          drow[k * zstride] = store_cast<T>(staged_cubic<T, CT, false, false>(
+              tile, b[0] + kk * st[0], b[1] + kk * st[1], b[2] + kk * st[2], lim, pitch, slice, dy, dz));
+        }
+      }
+    }
+    __syncthreads();  // every lane is done with the box
+  }
+}
+
 static unsigned compute_units() {
   static int cus[64] = {0};
   int dev = 0;
@@ -594,7 +802,7 @@ static unsigned compute_units() {
   return static_cast<unsigned>(cus[dev]);
 }
 
-template <typename T, int TX, int TY, int TZ, int THREADS, int LDS_BYTES, int KMAX>
+template <typename T, int TX, int TY, int TZ, int THREADS, int LDS_BYTES, int KMAX, bool CUBIC = false>
 static int launch_resample(const T *feat, const float *rois, T *out, const RoiProblem &p,
                            void *workspace, size_t *need, hipStream_t s) {
   const long tx = (p.ow + TX - 1) / TX, ty = (p.oh + TY - 1) / TY, tz = (p.od + TZ - 1) / TZ;
@@ -608,6 +816,7 @@ static int launch_resample(const T *feat, const float *rois, T *out, const RoiPr
   ps.vec = ((p.W % V == 0) && (reinterpret_cast<uintptr_t>(feat) % 16 == 0)) ? V : 0;
   ps.cap = LDS_BYTES / sizeof(T);
   ps.threads = THREADS; ps.max_items = KMAX;
+  ps.halo_lo = CUBIC ? 1 : 0; ps.halo_hi = CUBIC ? 2 : 1;
   unsigned blocks = compute_units() * (160u * 1024u / (LDS_BYTES + sizeof(TilePlan) * kPlanSlots + 64u));
   // As many workgroups as are resident at once, more when that would give one more than
   // kPlanSlots items (the later ones start as the first finish).
@@ -616,9 +825,14 @@ static int launch_resample(const T *feat, const float *rois, T *out, const RoiPr
   const long by_slots = ((work + kPlanSlots - 1) / kPlanSlots + 2 * kXcds + kXcds - 1) / kXcds * kXcds;
   if (blocks >= kXcds) blocks = blocks / kXcds * kXcds;  // the same number of workgroups on every XCD
   if (by_slots > blocks && work > kPlanSlots) blocks = static_cast<unsigned>(by_slots);
-  hipLaunchKernelGGL((roi_resample_kernel<T, TX, TY, TZ, THREADS, LDS_BYTES, KMAX>), dim3(blocks),
-                     dim3(THREADS), 0, s, feat, rois, out, p, ps, static_cast<unsigned>(total),
-                     static_cast<unsigned>(work));
+  if (CUBIC)
+    hipLaunchKernelGGL((roi_resample_cubic_kernel<T, TX, TY, TZ, THREADS, LDS_BYTES>), dim3(blocks),
+                       dim3(THREADS), 0, s, feat, rois, out, p, ps, static_cast<unsigned>(total),
+                       static_cast<unsigned>(work));
+  else
+    hipLaunchKernelGGL((roi_resample_kernel<T, TX, TY, TZ, THREADS, LDS_BYTES, KMAX>), dim3(blocks),
+                       dim3(THREADS), 0, s, feat, rois, out, p, ps, static_cast<unsigned>(total),
+                       static_cast<unsigned>(work));
   return check_launch("roi_resample_kernel");
 }
 
@@ -630,6 +844,22 @@ int roi_forward_tiled(const void *input, const void *rois, void *output, int dty
   if (p.sampling_ratio != 1 || vox < 4096 || p.ow < 16 || p.R == 0) return -1;
   if (vox * 4 >= (1L << 31)) return -1;   // 32-bit byte offsets inside one output volume
   const float *r = static_cast<const float *>(rois);
+  if (p.order == 3) {
+    switch (dtype) {
+      case MV_F16:
+        return launch_resample<__half, 16, 16, 8, 512, 76 * 1024, 8, true>(
+            static_cast<const __half *>(input), r, static_cast<__half *>(output), p, workspace, need, s);
+      case MV_BF16:
+        return launch_resample<__hip_bfloat16, 16, 16, 8, 512, 76 * 1024, 8, true>(
+            static_cast<const __hip_bfloat16 *>(input), r, static_cast<__hip_bfloat16 *>(output), p,
+            workspace, need, s);
+      case MV_F32:
+        return launch_resample<float, 16, 16, 8, 512, 76 * 1024, 6, true>(
+            static_cast<const float *>(input), r, static_cast<float *>(output), p, workspace, need, s);
+      default:
+        return -1;
+    }
+  }
   switch (dtype) {
     case MV_F16:
       return launch_resample<__half, 16, 16, 16, 512, 76 * 1024, 8>(

@@ -196,6 +196,9 @@ def test_config3_resize_and_crops(ops, oracle):
     (torch.float16, 2, 3, (20, 40, 46), (24, 40, 40), 1),    # rows of 46 fp16: unaligned, element-wise staging
     (torch.float32, 2, 3, (18, 30, 37), (16, 32, 32), 0),    # unaligned fp32, nearest
     (torch.float16, 64, 2, (24, 24, 24), (64, 64, 64), 1),   # more items than resident workgroups x 16
+    (torch.float16, 2, 3, (20, 40, 48), (24, 40, 40), 3),    # order 3: halo boxes, clamped and interior tiles
+    (torch.float32, 1, 3, (18, 30, 37), (16, 32, 32), 3),    # order 3, fp32, rows that are not 16-byte multiples
+    (torch.bfloat16, 2, 2, (6, 7, 8), (48, 56, 64), 3),      # order 3 up-sampling of a tiny volume (every tile clamped)
 ])
 def test_tiled_resampler_shapes(ops, oracle, dtype, channels, rois_n, size, out, order):
     """The persistent tiled kernel (outputs >= 4096 voxels per roi and channel, sampling_ratio 1) on
@@ -213,7 +216,7 @@ def test_tiled_resampler_shapes(ops, oracle, dtype, channels, rois_n, size, out,
     rois = torch.tensor(rows, dtype=torch.float32)
     got = ops.affine_3d(feat.to(DEV), rois.to(DEV), out, 1.0, 1, True, order)
     want = oracle.roi_align_forward(feat, rois, out, 1.0, 1, True, order, True)
-    if order == 1:
+    if order != 0:
         assert_close(got, want, FWD_TOL[dtype], "tiled forward")
     else:
         mism = (got.cpu().double() != want).float().mean()
@@ -226,9 +229,10 @@ def test_tiled_resampler_2d(ops, oracle):
     img = torch.randn(2, 3, 96, 120, generator=g).half()
     rois = torch.tensor([[0, 60.3, 47.1, 130.0, 90.0, 0.4], [1, 50.0, 40.0, 70.0, 110.0, -0.7],
                          [0, 10.0, 90.0, 60.0, 60.0, 1.3]], dtype=torch.float32)
-    got = ops.affine_2d(img.to(DEV), rois.to(DEV), (80, 96), 1.0, 1, True, 1)
-    want = oracle.roi_align_forward(img, rois, (80, 96), 1.0, 1, True, 1, True)
-    assert_close(got, want, FWD_TOL[torch.float16], "tiled 2-D forward")
+    for order in (1, 3):
+        got = ops.affine_2d(img.to(DEV), rois.to(DEV), (80, 96), 1.0, 1, True, order)
+        want = oracle.roi_align_forward(img, rois, (80, 96), 1.0, 1, True, order, True)
+        assert_close(got, want, FWD_TOL[torch.float16], f"tiled 2-D forward, order {order}")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
