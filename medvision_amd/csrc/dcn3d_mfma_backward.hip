@@ -312,7 +312,7 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
 
 // gxt [B, P, C] fp32 -> gx [B, C, P] T, added to what gx holds; 64 positions x up to kAddChunk
 // channels per workgroup
-constexpr int kAddChunk = 128;
+constexpr int kAddChunk = 64;
 template <typename T>
 __global__ __launch_bounds__(256) void dcn_planar_add_kernel(const float *__restrict__ gxt,
                                                              T *__restrict__ gx, int C, long P) {
