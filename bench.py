@@ -90,6 +90,61 @@ def bench_dcn(args, dtype=torch.float16):
     return {"ms": ms, "tflops": flops / ms / 1e9, "flops": flops, "train_ms": train_ms}
 
 
+def bench_other_configs(args):
+    """The remaining measurement configurations of the path on the GPU (HIP events, a few steps
+    each): config 1 rois through the HIP RoIAlign3D, config 2 backward, config 3 (CT resize + 16
+    rotated crops), config 5 (detection head: 4000 rois x 256 channels x 7^3) forward / backward.
+    GB/s are algorithmic bytes (inputs read once + outputs written once) over the measured time."""
+    import medvision_amd.ops as ops
+    from medvision_amd import _C
+    import workloads as wl
+    dev = "cuda:0"
+    res = {}
+    g = wl.gen(0)
+    feat = torch.randn(2, 16, 32, 64, 64, generator=g).to(dev)
+    rois = wl.roi3d_detection(g, 128, 2, (64, 64, 32), (4.0, 24.0)).to(dev)
+    out = torch.empty(128, 16, 7, 7, 7, device=dev)
+    ms, _ = _events_ms(lambda i: _C.roi_align_3d_forward(feat, rois, out, 7, 7, 7, 1.0, 2, 1), 20, 3)
+    res["config1_roialign3d_fp32"] = {"ms": round(ms, 4), "outputs_per_s": round(out.numel() / ms * 1e3, 1)}
+    g = wl.gen(1)
+    for dt, name in ((torch.float32, "fp32"), (torch.float16, "fp16")):
+        vol = torch.randn(4, 1, 128, 128, 128, generator=g).to(dt).to(dev)
+        r = wl.affine_rois(g, 4, (128, 128, 128)).to(dev)
+        gy = torch.randn(4, 1, 128, 128, 128, generator=g).to(dt).to(dev)
+        gi = torch.zeros_like(vol)
+        ms, _ = _events_ms(lambda i: _C.roi_align_rotated_3d_backward(gy, r, gi, 128, 128, 128, 1.0, 1, True, 1), 10, 2)
+        res["config2_backward_" + name] = {"ms": round(ms, 4)}
+    g = wl.gen(2)
+    vol = wl.ct_like(g, (2, 1, 256, 512, 512)).to(dev)
+    full = torch.tensor([[b, 256, 256, 128, 512, 512, 256, 0, 0, 0] for b in range(2)], dtype=torch.float32).to(dev)
+    ms, _ = _events_ms(lambda i: ops.affine_3d(vol, full, (160, 256, 256), 1.0, 1, True, 1), 10, 2)
+    nbytes = (vol.numel() + 2 * 160 * 256 * 256) * 2
+    res["config3_resize_fp16"] = {"ms": round(ms, 4), "gbps": round(nbytes / ms / 1e6, 1)}
+    small = ops.affine_3d(vol, full, (160, 256, 256), 1.0, 1, True, 1)
+    crops = []
+    for b in range(2):
+        for _ in range(8):
+            c = torch.rand(3, generator=g) * torch.tensor([256 - 96., 256 - 96., 160 - 96.]) + 48
+            crops.append([b, *c.tolist(), 96, 96, 96, 0, 0, (float(torch.rand(1, generator=g)) * 2 - 1) * math.radians(15)])
+    crops = torch.tensor(crops).to(dev)
+    ms, _ = _events_ms(lambda i: ops.affine_3d(small, crops, (96, 96, 96), 1.0, 1, True, 1), 10, 2)
+    res["config3_16_crops_96^3_fp16"] = {"ms": round(ms, 4), "gbps": round(2 * 16 * 96 ** 3 * 2 / ms / 1e6, 1)}
+    del vol, small
+    g = wl.gen(4)
+    feat = torch.randn(2, 256, 24, 96, 96, generator=g).half().to(dev)
+    rois = wl.roi3d_detection(g, 4000, 2, (384, 384, 96), (2.0, 48.0), log_uniform=True).to(dev)
+    out = torch.empty(4000, 256, 7, 7, 7, dtype=torch.float16, device=dev)
+    ms, _ = _events_ms(lambda i: _C.roi_align_3d_forward(feat, rois, out, 7, 7, 7, 0.25, 2, 1), 5, 1)
+    nbytes = (feat.numel() + out.numel()) * 2
+    res["config5_forward_fp16"] = {"ms": round(ms, 4), "goutputs_s": round(out.numel() / ms / 1e6, 2),
+                                   "gbps": round(nbytes / ms / 1e6, 1)}
+    gy = torch.randn_like(out)
+    gi = torch.zeros_like(feat)
+    ms, _ = _events_ms(lambda i: _C.roi_align_3d_backward(gy, rois, gi, 7, 7, 7, 0.25, 2, 1), 3, 1)
+    res["config5_backward_fp16"] = {"ms": round(ms, 4), "gbps": round(nbytes / ms / 1e6, 1)}
+    return res
+
+
 def bench_next_rows(args):
     """Short timings of the operators either side of the headline path: order-3 resampling, the
     elastic pipeline (control-grid upsampling + displacement warp), a 2-D DCNv2 layer of FPN size
@@ -227,6 +282,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-dcn", action="store_true", help="skip the DCN leg")
     ap.add_argument("--no-next", action="store_true", help="skip the timings of the neighbouring operators")
+    ap.add_argument("--no-configs", action="store_true", help="skip configs 1, 2-backward, 3 and 5")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="wall time spent on the CPU oracle")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a device copy of 4*128^3 fp16 elements (counter calibration)")
@@ -273,6 +329,8 @@ def main():
                                     "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                                     "frac": round(d["tflops"] / MFMA_F16_PEAK_TFLOPS, 5),
                                     "traffic": None, "flops_per_launch": d["flops"]}}
+    if not args.no_configs:
+        line["other_configs"] = bench_other_configs(args)
     if not args.no_next:
         line["next_rows"] = bench_next_rows(args)
     if not args.no_cpu:
