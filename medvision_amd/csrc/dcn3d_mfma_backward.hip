@@ -427,20 +427,25 @@ int dcn_mfma_backward(const void *x, const void *off, const void *mask, const vo
   return backward_run<__hip_bfloat16>(x, off, mask, wt, gy, goff, gmask, s, workspace, gx32, gw32, gb32, dtype, stream);
 }
 
-int dcn_planar_add(const float *gxt, void *gx, const DcnDims &s, int dtype, hipStream_t stream) {
-  const long pblocks = (s.P + 63) / 64;
-  MV_REQUIRE(pblocks < (1L << 31), "volume too large");
-  const dim3 grid(static_cast<unsigned>(pblocks), s.B, (s.Cin + kAddChunk - 1) / kAddChunk);
+// dst [B, C, P] (element type of `dtype`) += src [B, P, C] fp32
+int planar_add_f32(const float *src, void *dst, int B, int C, long P, int dtype, hipStream_t stream) {
+  const long pblocks = (P + 63) / 64;
+  MV_REQUIRE(pblocks < (1L << 31) && B <= 65535 && (C + kAddChunk - 1) / kAddChunk <= 65535, "volume too large");
+  const dim3 grid(static_cast<unsigned>(pblocks), B, (C + kAddChunk - 1) / kAddChunk);
   if (dtype == MV_F16)
-    hipLaunchKernelGGL((dcn_planar_add_kernel<__half>), grid, dim3(256), 0, stream, gxt,
-                       static_cast<__half *>(gx), s.Cin, s.P);
+    hipLaunchKernelGGL((dcn_planar_add_kernel<__half>), grid, dim3(256), 0, stream, src,
+                       static_cast<__half *>(dst), C, P);
   else if (dtype == MV_F32)
-    hipLaunchKernelGGL((dcn_planar_add_kernel<float>), grid, dim3(256), 0, stream, gxt,
-                       static_cast<float *>(gx), s.Cin, s.P);
+    hipLaunchKernelGGL((dcn_planar_add_kernel<float>), grid, dim3(256), 0, stream, src,
+                       static_cast<float *>(dst), C, P);
   else
-    hipLaunchKernelGGL((dcn_planar_add_kernel<__hip_bfloat16>), grid, dim3(256), 0, stream, gxt,
-                       static_cast<__hip_bfloat16 *>(gx), s.Cin, s.P);
+    hipLaunchKernelGGL((dcn_planar_add_kernel<__hip_bfloat16>), grid, dim3(256), 0, stream, src,
+                       static_cast<__hip_bfloat16 *>(dst), C, P);
   return check_launch("dcn_planar_add_kernel");
+}
+
+int dcn_planar_add(const float *gxt, void *gx, const DcnDims &s, int dtype, hipStream_t stream) {
+  return planar_add_f32(gxt, gx, s.B, s.Cin, s.P, dtype, stream);
 }
 
 }  // namespace mv

@@ -123,7 +123,10 @@ int roi_forward_tiled(const void *input, const void *rois, void *output, int dty
 int roi_pool_forward(const void *input, const void *rois, void *output, int dtype,
                      const RoiProblem &p, hipStream_t s);
 int roi_pool_backward(const void *grad_output, const void *rois, void *acc, int dtype,
-                      const RoiProblem &p, hipStream_t s);
+                      const RoiProblem &p, hipStream_t s, bool channels_last);
+bool roi_pool_applies(int dtype, const RoiProblem &p);
+// dcn3d_mfma_backward.hip: dst [B, C, P] += src [B, P, C] fp32
+int planar_add_f32(const float *src, void *dst, int B, int C, long P, int dtype, hipStream_t stream);
 
 static int make_problem(RoiProblem &p, int ndim, int rotated, int batch, int channels, int depth,
                         int height, int width, int num_rois, int out_d, int out_h, int out_w,
@@ -203,8 +206,13 @@ int roi_backward(const void *grad_output, const void *rois, void *grad_input, in
     hipLaunchKernelGGL(fill_zero_kernel, dim3(fill_blocks), dim3(256), 0, s,
                        static_cast<float *>(workspace), total);
   }
-  const int pooled = roi_pool_backward(grad_output, rois, narrow ? workspace : grad_input, dtype, p, s);
+  // 16-bit pooled path: the fp32 workspace is used channels-last and folded in by a transposing add
+  const bool channels_last = narrow && roi_pool_applies(dtype, p);
+  const int pooled = roi_pool_backward(grad_output, rois, narrow ? workspace : grad_input, dtype, p, s, channels_last);
   if (pooled > 0) return pooled;
+  if (pooled == 0 && channels_last)
+    return planar_add_f32(static_cast<const float *>(workspace), grad_input, batch, channels,
+                          static_cast<long>(depth) * height * width, dtype, s);
   MV_DISPATCH(dtype, {
     using RT = typename std::conditional<std::is_same<T, double>::value, double, float>::type;
     using G = typename std::conditional<(sizeof(T) == 2), float, T>::type;

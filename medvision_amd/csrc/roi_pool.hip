@@ -303,7 +303,10 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
 }
 
 // G = element type of the accumulation buffer (T for fp32, float for 16-bit T).
-template <typename T, typename G, typename RT>
+// CL: the accumulation buffer is channels-last [N, D*H*W, C] (the fp32 workspace of the 16-bit
+// path): the lanes of a wavefront then add neighbouring channels of a voxel, contiguous bytes,
+// instead of one element in each of many rows (a scattered atomic moves a whole memory sector).
+template <typename T, typename G, typename RT, bool CL>
 __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
     const T *__restrict__ gout, const RT *__restrict__ rois, G *__restrict__ gin, const RoiProblem p,
     const int channels_per_block) {
@@ -318,6 +321,7 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
   const long plane = static_cast<long>(p.D) * p.H * p.W;
   const T *src = gout + (static_cast<long>(n) * p.C + c_begin) * cells;
   G *dst = gin + (static_cast<long>(sh.g.batch) * p.C + c_begin) * plane;
+  G *dst_cl = gin + static_cast<long>(sh.g.batch) * plane * p.C + c_begin;   // CL: voxel v, channel c at v * C + c
   if (sh.staged == 0) {  // per-output scatter
     const int total = (c_end - c_begin) * cells;
     const int gz = p.ndim == 3 ? sh.g.grid[2] : 1, gy = sh.g.grid[1], gx = sh.g.grid[0];
@@ -333,7 +337,8 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
             if (!clamped_corners<float>(p.D, p.H, p.W, z, y, local_coord(sh.g, 0, pw, ix), p.order, cw)) continue;
 #pragma unroll
             for (int k = 0; k < 8; k++)
-              if (cw.w[k] != 0.f) atomic_add(dst + c * plane + cw.idx[k], static_cast<G>(top * cw.w[k]));
+              if (cw.w[k] != 0.f)
+                atomic_add(CL ? dst_cl + cw.idx[k] * p.C + c : dst + c * plane + cw.idx[k], static_cast<G>(top * cw.w[k]));
           }
         }
       }
@@ -348,6 +353,108 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
   const float inv_vol = 1.f / vol, inv_nxy = 1.f / (nx * ny), inv_nx = 1.f / nx, inv_ow = 1.f / p.ow,
               inv_ohw = 1.f / ohw, inv_nzohw = 1.f / (nz * ohw), inv_nyow = 1.f / (ny * p.ow),
               inv_gx = 1.f / gx, inv_gy = 1.f / gy, inv_gz = 1.f / gz;
+  // Dense form for the usual small boxes (<= 8 cells per axis, box of <= 32 voxels per axis): per
+  // axis the tap table becomes a small matrix Wd[source index][cell] (sum of the weights of the
+  // cell's samples that touch the source index), and each transposed contraction is "load the
+  // cell values of a line into registers, emit one dot product per source index": no per-entry
+  // branches, the matrix rows are LDS broadcasts.
+  constexpr int kDenseSrc = 32, kDenseCells = 8;
+  __shared__ __attribute__((aligned(16))) float wd[3][kDenseSrc][kDenseCells];
+  const bool dense = nx <= kDenseSrc && ny <= kDenseSrc && nz <= kDenseSrc && p.ow <= kDenseCells &&
+                     p.oh <= kDenseCells && p.od <= kDenseCells;
+  if (dense) {
+    const int ncell[3] = {p.ow, p.oh, p.od}, nsrc[3] = {nx, ny, nz};
+    for (int i = threadIdx.x; i < 3 * kDenseSrc * kDenseCells; i += kPoolThreads) {
+      const int a = i / (kDenseSrc * kDenseCells), src_i = (i / kDenseCells) % kDenseSrc, cell = i % kDenseCells;
+      const AxisTaps &t = sh.ax[a];
+      float w = 0.f;
+      if (src_i < nsrc[a] && cell < ncell[a])
+        for (int e = cell * t.grid; e < (cell + 1) * t.grid; e++) {
+          if (t.lo[e] == src_i) w += t.wlo[e];
+          if (t.hi[e] == src_i) w += t.whi[e];
+        }
+      wd[a][src_i][cell] = w;
+    }
+    __syncthreads();
+    const float inv_ow = 1.f / p.ow;
+    for (int cb = c_begin; cb < c_end; cb += sh.chunk) {
+      const int cs = min(sh.chunk, c_end - cb);
+      float *t2 = reinterpret_cast<float *>(lds);      // [cs][nz][oh][ow]
+      float *t1 = t2 + cs * nz * ohw;                  // [cs][nz][ny][ow]; CL: [nz][ny][cs][ow]
+      float *gbox = t1 + cs * nz * ny * p.ow;          // [cs][nz][ny][nx] (planar accumulation only)
+      const T *go = src + static_cast<long>(cb - c_begin) * cells;
+      const float inv_cs = 1.f / cs;
+      // z: thread = (c, ph, pw); its grad_output values stay in registers
+      for (int i = threadIdx.x; i < cs * ohw; i += kPoolThreads) {
+        const int c = fdiv(i, inv_ohw), hw = i - c * ohw;
+        float g[kDenseCells];
+#pragma unroll
+        for (int k = 0; k < kDenseCells; k++) g[k] = k < p.od ? load(go + c * cells + k * ohw + hw) : 0.f;
+        for (int z = 0; z < nz; z++) {
+          float acc = 0.f;
+#pragma unroll
+          for (int k = 0; k < kDenseCells; k++) acc += wd[2][z][k] * g[k];
+          t2[(c * nz + z) * ohw + hw] = acc;
+        }
+      }
+      __syncthreads();
+      // y: thread = (c, z, pw)
+      for (int i = threadIdx.x; i < cs * nz * p.ow; i += kPoolThreads) {
+        const int cz = fdiv(i, inv_ow), pw = i - cz * p.ow;
+        const int c = fdiv(cz, 1.f / nz), z = cz - c * nz;
+        float g[kDenseCells];
+#pragma unroll
+        for (int k = 0; k < kDenseCells; k++) g[k] = k < p.oh ? t2[cz * ohw + k * p.ow + pw] : 0.f;
+        for (int y = 0; y < ny; y++) {
+          float acc = 0.f;
+#pragma unroll
+          for (int k = 0; k < kDenseCells; k++) acc += wd[1][y][k] * g[k];
+          t1[(CL ? ((z * ny + y) * cs + c) : (cz * ny + y)) * p.ow + pw] = acc;
+        }
+      }
+      __syncthreads();
+      // x: thread = one (c, z, y) line
+      const long first = (static_cast<long>(tz.box_lo) * p.H + ty.box_lo) * p.W + tx.box_lo;
+      if (CL) {   // channel fastest across the lanes: a wavefront adds runs of cs contiguous floats
+        for (int i = threadIdx.x; i < cs * nz * ny; i += kPoolThreads) {
+          const int zy = fdiv(i, inv_cs), c = i - zy * cs, z = fdiv(zy, 1.f / ny), y = zy - z * ny;
+          float g[kDenseCells];
+#pragma unroll
+          for (int k = 0; k < kDenseCells; k++) g[k] = k < p.ow ? t1[i * p.ow + k] : 0.f;
+          G *row = dst_cl + (first + (static_cast<long>(z) * p.H + y) * p.W) * p.C + (cb - c_begin) + c;
+          for (int x = 0; x < nx; x++) {
+            float acc = 0.f;
+#pragma unroll
+            for (int k = 0; k < kDenseCells; k++) acc += wd[0][x][k] * g[k];
+            if (acc != 0.f) atomic_add(row + static_cast<long>(x) * p.C, static_cast<G>(acc));
+          }
+        }
+      } else {    // through LDS, so that the lanes of a wavefront add runs of nx contiguous elements
+        for (int i = threadIdx.x; i < cs * nz * ny; i += kPoolThreads) {
+          float g[kDenseCells];
+#pragma unroll
+          for (int k = 0; k < kDenseCells; k++) g[k] = k < p.ow ? t1[i * p.ow + k] : 0.f;
+          for (int x = 0; x < nx; x++) {
+            float acc = 0.f;
+#pragma unroll
+            for (int k = 0; k < kDenseCells; k++) acc += wd[0][x][k] * g[k];
+            gbox[i * nx + x] = acc;
+          }
+        }
+        __syncthreads();
+        G *corner = dst + static_cast<long>(cb - c_begin) * plane + first;
+        for (int i = threadIdx.x; i < cs * vol; i += kPoolThreads) {
+          const float v = gbox[i];
+          if (v == 0.f) continue;
+          const int c = fdiv(i, inv_vol), r0 = i - c * vol, z = fdiv(r0, inv_nxy), r1 = r0 - z * nx * ny;
+          const int y = fdiv(r1, inv_nx), x = r1 - y * nx;
+          atomic_add(corner + c * plane + (static_cast<long>(z) * p.H + y) * p.W + x, static_cast<G>(v));
+        }
+      }
+      __syncthreads();
+    }
+    return;
+  }
   for (int cb = c_begin; cb < c_end; cb += sh.chunk) {
     const int cs = min(sh.chunk, c_end - cb);
     float *gbox = reinterpret_cast<float *>(lds);    // [cs][nz][ny][nx]
@@ -393,14 +500,15 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
       gbox[i] = acc;
     }
     __syncthreads();
-    G *corner = dst + static_cast<long>(cb - c_begin) * plane +
-                (static_cast<long>(tz.box_lo) * p.H + ty.box_lo) * p.W + tx.box_lo;
+    const long first = (static_cast<long>(tz.box_lo) * p.H + ty.box_lo) * p.W + tx.box_lo;
+    G *corner = dst + static_cast<long>(cb - c_begin) * plane + first;
     for (int i = threadIdx.x; i < cs * vol; i += kPoolThreads) {
       const float v = gbox[i];
       if (v == 0.f) continue;
       const int c = fdiv(i, inv_vol), r0 = i - c * vol, z = fdiv(r0, inv_nxy), r1 = r0 - z * nx * ny;
       const int y = fdiv(r1, inv_nx), x = r1 - y * nx;
-      atomic_add(corner + c * plane + (static_cast<long>(z) * p.H + y) * p.W + x, static_cast<G>(v));
+      const long voxel = (static_cast<long>(z) * p.H + y) * p.W + x;
+      atomic_add(CL ? dst_cl + (first + voxel) * p.C + (cb - c_begin) + c : corner + c * plane + voxel, static_cast<G>(v));
     }
     __syncthreads();
   }
@@ -440,9 +548,12 @@ int roi_pool_forward(const void *input, const void *rois, void *output, int dtyp
   return check_launch("roi_pool_forward_kernel");
 }
 
-// `acc` is the accumulation buffer: grad_input itself for fp32, the fp32 workspace for 16-bit.
+bool roi_pool_applies(int dtype, const RoiProblem &p) { return pool_applies(dtype, p) && (p.C + 31) / 32 <= 65535; }
+
+// `acc` is the accumulation buffer: grad_input itself for fp32, the fp32 workspace for 16-bit
+// (channels-last [N, D*H*W, C] when `channels_last` is set; 16-bit types only).
 int roi_pool_backward(const void *grad_output, const void *rois, void *acc, int dtype,
-                      const RoiProblem &p, hipStream_t s) {
+                      const RoiProblem &p, hipStream_t s, bool channels_last) {
   if (!pool_applies(dtype, p)) return -1;
   const int cpb = 32;
   const long cblocks = (p.C + cpb - 1) / cpb;
@@ -451,17 +562,25 @@ int roi_pool_backward(const void *grad_output, const void *rois, void *acc, int 
   const float *r = static_cast<const float *>(rois);
   switch (dtype) {
     case MV_F32:
-      hipLaunchKernelGGL((roi_pool_backward_kernel<float, float, float>), grid, block, 0, s,
+      if (channels_last) return fail(MV_INVALID_ARGUMENT, "channels-last accumulation is for 16-bit tensors");
+      hipLaunchKernelGGL((roi_pool_backward_kernel<float, float, float, false>), grid, block, 0, s,
                          static_cast<const float *>(grad_output), r, static_cast<float *>(acc), p, cpb);
       break;
     case MV_F16:
-      hipLaunchKernelGGL((roi_pool_backward_kernel<__half, float, float>), grid, block, 0, s,
-                         static_cast<const __half *>(grad_output), r, static_cast<float *>(acc), p, cpb);
+      if (channels_last)
+        hipLaunchKernelGGL((roi_pool_backward_kernel<__half, float, float, true>), grid, block, 0, s,
+                           static_cast<const __half *>(grad_output), r, static_cast<float *>(acc), p, cpb);
+      else
+        hipLaunchKernelGGL((roi_pool_backward_kernel<__half, float, float, false>), grid, block, 0, s,
+                           static_cast<const __half *>(grad_output), r, static_cast<float *>(acc), p, cpb);
       break;
     default:
-      hipLaunchKernelGGL((roi_pool_backward_kernel<__hip_bfloat16, float, float>), grid, block, 0, s,
-                         static_cast<const __hip_bfloat16 *>(grad_output), r, static_cast<float *>(acc),
-                         p, cpb);
+      if (channels_last)
+        hipLaunchKernelGGL((roi_pool_backward_kernel<__hip_bfloat16, float, float, true>), grid, block, 0, s,
+                           static_cast<const __hip_bfloat16 *>(grad_output), r, static_cast<float *>(acc), p, cpb);
+      else
+        hipLaunchKernelGGL((roi_pool_backward_kernel<__hip_bfloat16, float, float, false>), grid, block, 0, s,
+                           static_cast<const __hip_bfloat16 *>(grad_output), r, static_cast<float *>(acc), p, cpb);
   }
   return check_launch("roi_pool_backward_kernel");
 }
