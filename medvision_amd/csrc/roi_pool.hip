@@ -152,6 +152,45 @@ __device__ inline void pool_setup(PoolShared &sh, const RT *roi, const RoiProble
   __syncthreads();
 }
 
+// Dense form of the tap tables for the usual small boxes (<= kDenseCells cells per axis, box of
+// <= kDenseSrc voxels per axis): per axis a matrix Wd[source index][cell] = sum of the weights of
+// the cell's samples that touch the source index.  A contraction then is "walk the line, multiply
+// each value into all cells" (forward) or "load the cells of a line, one dot product per source
+// index" (backward): no per-entry branches, the matrix rows are LDS broadcasts.
+constexpr int kDenseSrc = 32, kDenseCells = 8;
+typedef float DenseTaps[3][kDenseSrc][kDenseCells];
+
+__device__ __forceinline__ bool dense_applies(const PoolShared &sh, const RoiProblem &p) {
+  for (int a = 0; a < 3; a++)
+    if (sh.ax[a].box_hi - sh.ax[a].box_lo + 1 > kDenseSrc) return false;
+  return p.ow <= kDenseCells && p.oh <= kDenseCells && p.od <= kDenseCells;
+}
+
+// all threads of the workgroup; followed by a barrier
+__device__ inline void dense_build(const PoolShared &sh, const RoiProblem &p, DenseTaps &wd) {
+  const int ncell[3] = {p.ow, p.oh, p.od};
+  for (int i = threadIdx.x; i < 3 * kDenseSrc * kDenseCells; i += kPoolThreads) {
+    const int a = i / (kDenseSrc * kDenseCells), src_i = (i / kDenseCells) % kDenseSrc, cell = i % kDenseCells;
+    const AxisTaps &t = sh.ax[a];
+    float w = 0.f;
+    if (src_i <= t.box_hi - t.box_lo && cell < ncell[a])
+      for (int e = cell * t.grid; e < (cell + 1) * t.grid; e++) {
+        if (t.lo[e] == src_i) w += t.wlo[e];
+        if (t.hi[e] == src_i) w += t.whi[e];
+      }
+    wd[a][src_i][cell] = w;
+  }
+  __syncthreads();
+}
+
+// acc[k] += Wd row[k] * v for the kDenseCells cells
+__device__ __forceinline__ void dense_axpy(float (&acc)[kDenseCells], const float *row, float v) {
+  const float4 w0 = *reinterpret_cast<const float4 *>(row), w1 = *reinterpret_cast<const float4 *>(row + 4);
+  acc[0] += w0.x * v; acc[1] += w0.y * v; acc[2] += w0.z * v; acc[3] += w0.w * v;
+  acc[4] += w1.x * v; acc[5] += w1.y * v; acc[6] += w1.z * v; acc[7] += w1.w * v;
+}
+static_assert(kDenseCells == 8, "dense_axpy is written for 8 cells");
+
 template <typename T, typename RT>
 __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
     const T *__restrict__ feat, const RT *__restrict__ rois, T *__restrict__ out, const RoiProblem p,
@@ -194,6 +233,9 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
   const int ohw = p.oh * p.ow;
   const float inv_vol = 1.f / vol, inv_nxy = 1.f / (nx * ny), inv_nx = 1.f / nx, inv_ow = 1.f / p.ow,
               inv_ohw = 1.f / ohw, inv_cells = 1.f / cells;
+  __shared__ __attribute__((aligned(16))) DenseTaps wd;
+  const bool dense = dense_applies(sh, p);
+  if (dense) dense_build(sh, p, wd);
   for (int cb = c_begin; cb < c_end; cb += sh.chunk) {
     const int cs = min(sh.chunk, c_end - cb);
     T *box = reinterpret_cast<T *>(lds);                                            // [cs][nz][ny][nx]
@@ -223,7 +265,40 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
     // Each pass gives a thread a FIXED output coordinate on the contracted axis, so its (at most
     // kTapRegs) tap entries stay in registers while it walks over the rows; per element that leaves
     // 2 * grid LDS reads, 2 * grid FMAs and one store.
-    if (gx <= kTapRegs && gy <= kTapRegs && gz <= kTapRegs) {
+    if (dense) {
+      // x: thread = one (c, z, y) row of the box, all its cells at once
+      for (int r = threadIdx.x; r < cs * nz * ny; r += kPoolThreads) {
+        float a[kDenseCells] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        const T *row = box + r * nx;
+        for (int x = 0; x < nx; x++) dense_axpy(a, wd[0][x], load(row + x));
+#pragma unroll
+        for (int k = 0; k < kDenseCells; k++)
+          if (k < p.ow) t1[r * p.ow + k] = a[k];
+      }
+      __syncthreads();
+      // y: thread = (c, z, pw)
+      for (int i = threadIdx.x; i < cs * nz * p.ow; i += kPoolThreads) {
+        const int cz = fdiv(i, inv_ow), pw = i - cz * p.ow;
+        float a[kDenseCells] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        const float *col = t1 + cz * ny * p.ow + pw;
+        for (int yy = 0; yy < ny; yy++) dense_axpy(a, wd[1][yy], col[yy * p.ow]);
+#pragma unroll
+        for (int k = 0; k < kDenseCells; k++)
+          if (k < p.oh) t2[cz * ohw + k * p.ow + pw] = a[k];
+      }
+      __syncthreads();
+      // z, store: thread = (c, ph, pw)
+      T *o = dst + static_cast<long>(cb - c_begin) * cells;
+      for (int i = threadIdx.x; i < cs * ohw; i += kPoolThreads) {
+        const int c = fdiv(i, inv_ohw), hw = i - c * ohw;
+        float a[kDenseCells] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        const float *col = t2 + c * nz * ohw + hw;
+        for (int zz = 0; zz < nz; zz++) dense_axpy(a, wd[2][zz], col[zz * ohw]);
+#pragma unroll
+        for (int k = 0; k < kDenseCells; k++)
+          if (k < p.od) o[c * cells + k * ohw + hw] = store_cast<T>(a[k]);
+      }
+    } else if (gx <= kTapRegs && gy <= kTapRegs && gz <= kTapRegs) {
       {  // contract x: thread = (row chunk, pw); rows are (c, z, y)
         int lanes = 1;
         while (lanes < p.ow) lanes *= 2;
@@ -353,29 +428,9 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
   const float inv_vol = 1.f / vol, inv_nxy = 1.f / (nx * ny), inv_nx = 1.f / nx, inv_ow = 1.f / p.ow,
               inv_ohw = 1.f / ohw, inv_nzohw = 1.f / (nz * ohw), inv_nyow = 1.f / (ny * p.ow),
               inv_gx = 1.f / gx, inv_gy = 1.f / gy, inv_gz = 1.f / gz;
-  // Dense form for the usual small boxes (<= 8 cells per axis, box of <= 32 voxels per axis): per
-  // axis the tap table becomes a small matrix Wd[source index][cell] (sum of the weights of the
-  // cell's samples that touch the source index), and each transposed contraction is "load the
-  // cell values of a line into registers, emit one dot product per source index": no per-entry
-  // branches, the matrix rows are LDS broadcasts.
-  constexpr int kDenseSrc = 32, kDenseCells = 8;
-  __shared__ __attribute__((aligned(16))) float wd[3][kDenseSrc][kDenseCells];
-  const bool dense = nx <= kDenseSrc && ny <= kDenseSrc && nz <= kDenseSrc && p.ow <= kDenseCells &&
-                     p.oh <= kDenseCells && p.od <= kDenseCells;
-  if (dense) {
-    const int ncell[3] = {p.ow, p.oh, p.od}, nsrc[3] = {nx, ny, nz};
-    for (int i = threadIdx.x; i < 3 * kDenseSrc * kDenseCells; i += kPoolThreads) {
-      const int a = i / (kDenseSrc * kDenseCells), src_i = (i / kDenseCells) % kDenseSrc, cell = i % kDenseCells;
-      const AxisTaps &t = sh.ax[a];
-      float w = 0.f;
-      if (src_i < nsrc[a] && cell < ncell[a])
-        for (int e = cell * t.grid; e < (cell + 1) * t.grid; e++) {
-          if (t.lo[e] == src_i) w += t.wlo[e];
-          if (t.hi[e] == src_i) w += t.whi[e];
-        }
-      wd[a][src_i][cell] = w;
-    }
-    __syncthreads();
+  __shared__ __attribute__((aligned(16))) DenseTaps wd;
+  if (dense_applies(sh, p)) {
+    dense_build(sh, p, wd);
     const float inv_ow = 1.f / p.ow;
     for (int cb = c_begin; cb < c_end; cb += sh.chunk) {
       const int cs = min(sh.chunk, c_end - cb);
@@ -523,10 +578,18 @@ static bool pool_applies(int dtype, const RoiProblem &p) {
 }
 
 // Returns -1 when the pooled kernels do not apply.
+// Channels per workgroup: 32, doubled while that still leaves a few thousand workgroups (the tap
+// tables are built once per workgroup, so with many rois fewer, longer workgroups are cheaper).
+static int pool_channels_per_block(const RoiProblem &p) {
+  int cpb = 32;
+  while (cpb < 256 && cpb < p.C && static_cast<long>(p.R) * ((p.C + 2 * cpb - 1) / (2 * cpb)) >= 6144) cpb *= 2;
+  return cpb;
+}
+
 int roi_pool_forward(const void *input, const void *rois, void *output, int dtype,
                      const RoiProblem &p, hipStream_t s) {
   if (!pool_applies(dtype, p)) return -1;
-  const int cpb = 32;
+  const int cpb = pool_channels_per_block(p);
   const long cblocks = (p.C + cpb - 1) / cpb;
   if (cblocks > 65535) return -1;
   const dim3 grid(p.R, static_cast<unsigned>(cblocks)), block(kPoolThreads);
@@ -555,7 +618,7 @@ bool roi_pool_applies(int dtype, const RoiProblem &p) { return pool_applies(dtyp
 int roi_pool_backward(const void *grad_output, const void *rois, void *acc, int dtype,
                       const RoiProblem &p, hipStream_t s, bool channels_last) {
   if (!pool_applies(dtype, p)) return -1;
-  const int cpb = 32;
+  const int cpb = pool_channels_per_block(p);
   const long cblocks = (p.C + cpb - 1) / cpb;
   if (cblocks > 65535) return -1;
   const dim3 grid(p.R, static_cast<unsigned>(cblocks)), block(kPoolThreads);
