@@ -304,7 +304,7 @@ def main():
         "value": round(a16["gvox_s"], 3), "unit": "Gvox/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(a16["ms"], 6), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f16 storage, f32 interpolation, f64 coordinates",
+        "vs_baseline": None, "dtype": "f16 storage; f32 interpolation and per-voxel coordinates; f64 roi geometry",
         "data": "synthetic",
         "config": {"workload": "BASELINE config 2: RoIAlignRotated3D as RandomAffine resampling, "
                                "volume fp16 [4,1,128,128,128] N(0,1), one full-volume roi per sample, "
