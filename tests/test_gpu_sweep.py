@@ -1,0 +1,201 @@
+"""Seeded random sweeps of the hot path against the fp64 oracle: shapes, roi geometry, sampling
+grids, orders, layer hyper-parameters and dtypes are drawn per case (odd sizes, rois partly or
+wholly outside, degenerate extents, 16-byte and ragged rows, channel counts on either side of the
+matrix-core kernels' limits).  Each sweep runs a few hundred tiny cases in a few seconds."""
+import math
+import random
+
+import pytest
+import torch
+
+from parity import BWD_TOL, FWD_TOL, rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.float16, torch.bfloat16, torch.float64]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import medvision_amd.ops as ops_
+    from medvision_amd import _lib
+    _lib.load()
+    return ops_
+
+
+def _nearest_ok(got, want, tol):
+    """Order 0: a coordinate within rounding of a .5 tie may pick the other neighbour (the
+    reference's own pick there is rounding noise too); all but 0.2 % of the voxels must agree."""
+    diff = (got.detach().cpu().double() - want.double()).abs()
+    den = max(1e-30, float(want.abs().max()))
+    return float((diff > tol * den).double().mean()) <= 2e-3
+
+
+def _roi_case(seed):
+    rnd = random.Random(seed)
+    g = torch.Generator().manual_seed(seed)
+    ndim = rnd.choice([2, 3])
+    rotated = rnd.random() < 0.6
+    big = rnd.random() < 0.25
+    size = [rnd.randint(1, 70 if big else 24) for _ in range(ndim)]
+    batch = rnd.randint(1, 3)
+    channels = rnd.choice([1, 2]) if big else rnd.choice([1, 1, 2, 3, 5, 33])
+    dtype = rnd.choice(DTYPES)
+    out = [rnd.randint(1, 40 if big else 12) for _ in range(ndim)]
+    n = rnd.randint(1, 5)
+    scale = rnd.choice([0.25, 0.5, 1.0, 1.0, 2.0])
+    sr = rnd.choice([-1, 0, 1, 1, 2, 3])
+    order = rnd.choice([0, 1, 1, 1])
+    aligned = rnd.random() < 0.6
+    feat = torch.randn(batch, channels, *size, generator=g).to(dtype)
+    ext = torch.tensor(size[::-1], dtype=torch.float32) / scale
+    cols = {(2, False): 5, (3, False): 7, (2, True): 6, (3, True): 10}[(ndim, rotated)]
+    rois = torch.zeros(n, cols)
+    rois[:, 0] = torch.randint(0, batch, (n,), generator=g)
+    if rotated:
+        rois[:, 1:1 + ndim] = (torch.rand(n, ndim, generator=g) * 1.6 - 0.3) * ext
+        rois[:, 1 + ndim:1 + 2 * ndim] = torch.rand(n, ndim, generator=g) * ext * rnd.choice([0.3, 1.0, 1.5, 2.5])
+        rois[:, 1 + 2 * ndim:] = (torch.rand(n, cols - 1 - 2 * ndim, generator=g) - 0.5) * rnd.choice([0.0, 0.5, 2.0, 6.3])
+    else:
+        lo = (torch.rand(n, ndim, generator=g) * 1.4 - 0.3) * ext
+        rois[:, 1:1 + ndim] = lo
+        rois[:, 1 + ndim:] = lo + torch.rand(n, ndim, generator=g) * ext * rnd.choice([0.2, 0.8, 1.6])
+    if rnd.random() < 0.2:   # a roi of zero extent
+        rois[0, 1 + ndim:1 + 2 * ndim] = 0.0 if rotated else rois[0, 1:1 + ndim]
+    return g, ndim, rotated, feat, rois, tuple(out), scale, sr, order, aligned, dtype
+
+
+def test_roi_sweep(ops, oracle):
+    for seed in range(7000, 7300):
+        g, ndim, rotated, feat, rois, out, scale, sr, order, aligned, dtype = _roi_case(seed)
+        mod = ops.RoIAlignRotated(out, scale, sr, aligned) if rotated else ops.RoIAlign(out, scale, sr)
+        fg = feat.to(DEV).requires_grad_(True)
+        got = mod(fg, rois.to(DEV), order=order)
+        eff = 1 if order == 0 else sr
+        want = oracle.roi_align_forward(feat, rois, out, scale, eff, aligned, order, rotated)
+        what = f"seed {seed}: {ndim}-D rotated={rotated} {tuple(feat.shape)} -> {out} sr={sr} order={order} {dtype}"
+        if order == 0:
+            assert _nearest_ok(got, want, FWD_TOL[dtype]), what
+            continue
+        assert rel_err(got, want) <= FWD_TOL[dtype], what
+        gy = torch.randn(got.shape, generator=g).to(dtype)
+        got.backward(gy.to(DEV))
+        gwant = oracle.roi_align_backward(gy, rois, feat.shape, scale, eff, aligned, order, rotated)
+        assert rel_err(fg.grad, gwant) <= BWD_TOL[dtype], what + " (backward)"
+
+
+def test_affine_and_warp_sweep(ops, oracle):
+    """Larger outputs, so that the LDS-tiled resampler (orders 0 / 1 and 3) takes most cases."""
+    for seed in range(8000, 8120):
+        rnd = random.Random(seed)
+        g = torch.Generator().manual_seed(seed)
+        ndim = rnd.choice([2, 3])
+        hi = 64 if ndim == 3 else 150
+        size = [rnd.randint(1, hi) for _ in range(ndim)]
+        if rnd.random() < 0.3:
+            size[-1] = rnd.choice([8, 16, 24, 32, 40, 64])   # rows of whole 16-byte groups
+        batch, channels = rnd.randint(1, 2), rnd.choice([1, 1, 1, 2, 3])
+        dtype = rnd.choice(DTYPES)
+        out = tuple(rnd.randint(1, hi) for _ in range(ndim))
+        order = rnd.choice([0, 1, 1, 3, 3])
+        sr = 1 if order == 0 else rnd.choice([1, 1, 1, 2, 0])
+        scale = rnd.choice([0.5, 1.0, 1.0, 2.0])
+        aligned = rnd.random() < 0.7
+        feat = torch.randn(batch, channels, *size, generator=g).to(dtype)
+        ext = torch.tensor(size[::-1], dtype=torch.float32) / scale
+        n = rnd.randint(1, 3)
+        cols = 6 if ndim == 2 else 10
+        rois = torch.zeros(n, cols)
+        rois[:, 0] = torch.randint(0, batch, (n,), generator=g)
+        spread = rnd.choice([0.05, 0.2, 1.0])   # never exactly centred: no systematic .5 ties at order 0
+        rois[:, 1:1 + ndim] = ext / 2 + (torch.rand(n, ndim, generator=g) - 0.5) * ext * spread
+        rois[:, 1 + ndim:1 + 2 * ndim] = ext * (0.3 + torch.rand(n, ndim, generator=g) * rnd.choice([0.7, 1.0, 1.5]))
+        rois[:, 1 + 2 * ndim:] = (torch.rand(n, cols - 1 - 2 * ndim, generator=g) - 0.5) * rnd.choice([0.0, 0.3, 1.0, 3.0])
+        what = f"seed {seed}: {ndim}-D {tuple(feat.shape)} -> {out} sr={sr} order={order} {dtype}"
+        fn = ops.affine_3d if ndim == 3 else ops.affine_2d
+        got = fn(feat.to(DEV), rois.to(DEV), out, scale, sr, aligned, order)
+        want = oracle.roi_align_forward(feat, rois, out, scale, sr, aligned, order, True)
+        if order == 0:
+            assert _nearest_ok(got, want, FWD_TOL[dtype]), what
+        else:
+            assert rel_err(got, want) <= FWD_TOL[dtype], what
+        worder = rnd.choice([0, 1, 3])
+        off = (torch.randn(batch, ndim, *size, generator=g) * rnd.choice([0.0, 0.7, 3.0])).to(dtype)
+        warp = ops.apply_offset_3d if ndim == 3 else ops.apply_offset_2d
+        gotw = warp(feat.to(DEV), off.to(DEV), worder)
+        wantw = oracle.deform_warp(feat, off, worder)
+        if worder == 0:
+            assert _nearest_ok(gotw, wantw, FWD_TOL[dtype]), what + f" (warp order {worder})"
+        else:
+            assert rel_err(gotw, wantw) <= FWD_TOL[dtype], what + f" (warp order {worder})"
+
+
+def test_dcn_sweep(ops, oracle):
+    from medvision_amd.ops.deform_conv_2d import deform_conv as dc2
+    from medvision_amd.ops.deform_conv_3d import deform_conv as dc3
+    from medvision_amd.ops.modulated_deform_conv_2d import modulated_deform_conv as mdc2
+    from medvision_amd.ops.modulated_deform_conv_3d import modulated_deform_conv as mdc3
+    ran = 0
+    for seed in range(9000, 9260):
+        rnd = random.Random(seed)
+        g = torch.Generator().manual_seed(seed)
+        nd = rnd.choice([2, 3])
+        modulated = rnd.random() < 0.5
+        groups, dg = rnd.choice([1, 1, 2, 4]), rnd.choice([1, 1, 2])
+        matrix = rnd.random() < 0.5   # channel counts the matrix-core kernels accept
+        if matrix:
+            cin, cout = rnd.choice([16, 32, 48]) * groups, rnd.choice([32, 64, 96]) * groups
+            if cin % dg or (cin // dg) % 16:
+                dg = 1
+        else:
+            cin, cout = groups * dg * rnd.randint(1, 3), groups * rnd.randint(1, 5)
+        batch = rnd.randint(1, 3)
+        size = [rnd.randint(2, 9 if matrix else 11) for _ in range(nd)]
+        dtype = rnd.choice(DTYPES)
+        if modulated:   # one stride / padding / dilation for all axes, as the reference's layer
+            k = [rnd.randint(1, 3)] * nd if rnd.random() < 0.5 else [rnd.randint(1, 3) for _ in range(nd)]
+            st, pa, di = [rnd.randint(1, 2)] * nd, [rnd.randint(0, 2)] * nd, [rnd.randint(1, 2)] * nd
+        else:
+            k = [rnd.randint(1, 3) for _ in range(nd)]
+            st = [rnd.randint(1, 2) for _ in range(nd)]
+            pa = [rnd.randint(0, 2) for _ in range(nd)]
+            di = [rnd.randint(1, 2) for _ in range(nd)]
+        out = [(s + 2 * p - (d * (kk - 1) + 1)) // t + 1 for s, p, d, kk, t in zip(size, pa, di, k, st)]
+        if min(out) < 1:
+            continue
+        ran += 1
+        taps = math.prod(k)
+        x = torch.randn(batch, cin, *size, generator=g)
+        w = (torch.rand(cout, cin // groups, *k, generator=g) * 2 - 1) / math.sqrt(cin // groups * taps)
+        b = torch.rand(cout, generator=g) * 2 - 1
+        off = torch.randn(batch, dg * nd * taps, *out, generator=g) * rnd.choice([0.0, 0.5, 2.0, 6.0])
+        if rnd.random() < 0.3:
+            off = off.round()   # lattice points: the offset gradient is one-sided there, not compared
+        mask = torch.sigmoid(torch.randn(batch, dg * taps, *out, generator=g)) if modulated else None
+        x, w, b, off = [t.to(dtype) for t in (x, w, b, off)]
+        mask = None if mask is None else mask.to(dtype)
+        what = (f"seed {seed}: {nd}-D v{2 if modulated else 1} groups={groups} dg={dg} {cin}->{cout} "
+                f"{size} k={k} stride={st} pad={pa} dil={di} {dtype}")
+        xs, offs, ws, bs = [t.to(DEV).requires_grad_(True) for t in (x, off, w, b)]
+        ms = None if mask is None else mask.to(DEV).requires_grad_(True)
+        if modulated:
+            y = (mdc3 if nd == 3 else mdc2)(xs, offs, ms, ws, bs, st[0], pa[0], di[0], groups, dg)
+        else:
+            y = (dc3 if nd == 3 else dc2)(xs, offs, ws, bs, tuple(st), tuple(pa), tuple(di), groups, dg, 64)
+        want = oracle.dcn3d_forward(x, off, mask, w, b, tuple(st), tuple(pa), tuple(di), groups, dg)
+        # bf16 matrix-core path: the blended columns are rounded to bf16 as well as the output
+        ftol = FWD_TOL[dtype] * (1.5 if dtype == torch.bfloat16 else 1.0)
+        assert rel_err(y, want) <= ftol, what
+        gy = torch.randn(y.shape, generator=g).to(dtype)
+        y.backward(gy.to(DEV))
+        gx, goff, gm, gw, gb = oracle.dcn3d_backward(x, off, mask, w, gy, True, tuple(st), tuple(pa), tuple(di), groups, dg)
+        tol = BWD_TOL[dtype]
+        assert rel_err(xs.grad, gx) <= tol, what + " (grad input)"
+        assert rel_err(ws.grad, gw) <= tol, what + " (grad weight)"
+        assert rel_err(bs.grad, gb) <= tol, what + " (grad bias)"
+        on_lattice = bool((off == off.round()).all()) and float(off.abs().max()) > 0
+        if not on_lattice:
+            assert rel_err(offs.grad, goff) <= tol, what + " (grad offset)"
+        if modulated:
+            assert rel_err(ms.grad, gm) <= tol, what + " (grad mask)"
+    assert ran > 200
