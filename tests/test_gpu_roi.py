@@ -341,3 +341,30 @@ def test_non_default_stream_and_determinism(ops):
         again = ops.affine_3d(vol, rois, (32, 32, 32), 1.0, 2, True, 1)
     s.synchronize()
     assert torch.equal(ref, again)
+
+
+def test_volume_beyond_2_31_elements(ops):
+    """A 1300^3 fp16 volume (2.2e9 elements): crops at its far corner come back exactly, and the
+    backward pass puts the gradient there (the reference's `int` index arithmetic overflows at this
+    size, roi_align_3d_cuda_kernel.cuh:28-50; offsets here are 64-bit)."""
+    S, n = 1300, 64
+    vol = torch.empty(1, 1, S, S, S, dtype=torch.float16, device=DEV)
+    ar = torch.arange(S, device=DEV, dtype=torch.float32)
+    for z in range(S):
+        vol[0, 0, z] = (((ar[:, None] * 7 + ar[None, :] * 3 + z * 11) % 251) - 125).half()
+    lo = S - n - 3
+    c = lo + n / 2
+    rois = torch.tensor([[0, c, c, c, n, n, n, 0, 0, 0]], dtype=torch.float32, device=DEV)
+    want = vol[0, 0, lo:lo + n, lo:lo + n, lo:lo + n]
+    assert torch.equal(ops.RoIAlignRotated((n, n, n), 1.0, 1, True)(vol, rois)[0, 0], want)
+    assert torch.equal(ops.affine_3d(vol, rois, (n, n, n), 1.0, 1, True, 1)[0, 0], want)
+    box = torch.tensor([[0, lo, lo, lo, lo + n, lo + n, lo + n]], dtype=torch.float32, device=DEV)
+    got = ops.RoIAlign((n, n, n), 1.0, 1)(vol, box)[0, 0].float()   # samples at cell centres: mean of 8
+    w = vol[0, 0, lo:lo + n + 1, lo:lo + n + 1, lo:lo + n + 1].float()
+    mean8 = sum(w[a:a + n, b:b + n, e:e + n] for a in (0, 1) for b in (0, 1) for e in (0, 1)) / 8
+    assert float((got - mean8).abs().max()) <= 0.13   # fp16 rounding of values up to 125
+    vol.requires_grad_(True)
+    out = ops.RoIAlignRotated((n, n, n), 1.0, 1, True)(vol, rois)
+    out.backward(torch.ones_like(out))
+    assert float(vol.grad[0, 0, lo:lo + n, lo:lo + n, lo:lo + n].float().sum()) == n ** 3
+    assert float(vol.grad[0, 0, lo, lo, lo]) == 1.0 and float(vol.grad[0, 0, 0, 0, 0]) == 0.0
