@@ -579,10 +579,13 @@ static bool pool_applies(int dtype, const RoiProblem &p) {
 
 // Returns -1 when the pooled kernels do not apply.
 // Channels per workgroup: 32, doubled while that still leaves a few thousand workgroups (the tap
-// tables are built once per workgroup, so with many rois fewer, longer workgroups are cheaper).
+// tables are built once per workgroup, so with many rois fewer, longer workgroups are cheaper) and
+// halved while there are too few workgroups to fill the compute units (few rois, few channels: a
+// workgroup walks its channels in LDS-sized chunks one after the other).
 static int pool_channels_per_block(const RoiProblem &p) {
   int cpb = 32;
   while (cpb < 256 && cpb < p.C && static_cast<long>(p.R) * ((p.C + 2 * cpb - 1) / (2 * cpb)) >= 6144) cpb *= 2;
+  while (cpb > 1 && static_cast<long>(p.R) * ((p.C + cpb - 1) / cpb) < 1024) cpb /= 2;
   return cpb;
 }
 
