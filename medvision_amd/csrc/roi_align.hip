@@ -125,6 +125,9 @@ int roi_pool_forward(const void *input, const void *rois, void *output, int dtyp
 int roi_pool_backward(const void *grad_output, const void *rois, void *acc, int dtype,
                       const RoiProblem &p, hipStream_t s, bool channels_last);
 bool roi_pool_applies(int dtype, const RoiProblem &p);
+// roi_gather_backward.hip: atomic-free backward for resampling-sized problems; -1 when not applicable
+int roi_backward_gather(const void *grad_output, const void *rois, void *grad_input, int dtype,
+                        const RoiProblem &p, hipStream_t s);
 // dcn3d_mfma_backward.hip: dst [B, C, P] += src [B, P, C] fp32
 int planar_add_f32(const float *src, void *dst, int B, int C, long P, int dtype, hipStream_t stream);
 
@@ -199,6 +202,8 @@ int roi_backward(const void *grad_output, const void *rois, void *grad_input, in
   const bool narrow = dtype == MV_F16 || dtype == MV_BF16;
   MV_REQUIRE(!narrow || workspace, "16-bit backward needs an fp32 workspace");
   hipStream_t s = static_cast<hipStream_t>(stream);
+  const int gathered = roi_backward_gather(grad_output, rois, grad_input, dtype, p, s);
+  if (gathered >= 0) return gathered;
   const dim3 grid(p.chunks * num_rois), block(kRoiThreads);
   const long total = static_cast<long>(batch) * channels * depth * height * width;
   const int fill_blocks = static_cast<int>(std::min<long>((total + 1023) / 1024, 65536));

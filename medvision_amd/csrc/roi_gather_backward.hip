@@ -1,0 +1,225 @@
+// Backward of RoIAlign / RoIAlignRotated for resampling-sized problems, as a gather.
+//
+// The adjoint of a resampling (one sample per output voxel, an output about as large as the input,
+// a roi or two per image: RandomAffine, Resize) is usually written as a scatter, eight atomic adds
+// per output voxel.  Here every INPUT voxel collects its own gradient instead: the output voxels
+// whose sample lies within one voxel of it form a small parallelepiped in output space, which is
+// enumerated row by row (the extent along the fastest output axis is solved for exactly, the other
+// two axes come from a bounding box), each candidate is evaluated with the very sampler of the
+// forward pass (`clamped_tap`: closed interval [-1, size], border replicate, nearest ties low) and
+// contributes grad_output * weight when the voxel is one of its taps.  No atomics, no fp32
+// workspace for 16-bit tensors, one rounding per voxel, and a result that does not depend on the
+// order in which workgroups run.
+#include "common.hpp"
+#include "roi_geometry.hpp"
+#include "sampling.hpp"
+
+namespace mv {
+
+constexpr int kGatherThreads = 256;
+constexpr int kGatherPerThread = 4;   // input voxels per thread
+
+struct GatherShared {
+  RoiGeom g;
+  double trig[6];
+  double reach[3];   // per local axis j: sum_a |rot[a][j]| + margin = how far (in local
+                     // coordinates) a sample may be from the voxel and still touch it
+  double inv_bin[3]; // 1 / bin (0 for a degenerate axis)
+  // fp32 copies for the row test (it only has to be conservative: `slack` covers its rounding)
+  float r1[3], r2[3];  // rot[a][1], rot[a][2]
+  float inv_m[3];      // 1 / rot[a][0] (0 when source axis a does not move along an output row)
+  float half[3];       // (1 + slack) * |inv_m|
+  float inv_bin0, off0;  // cell along the row = x * inv_bin0 - off0
+  float slack, slack_u;
+};
+
+// a wave-uniform value moved to scalar registers (LDS reads land in vector registers)
+__device__ __forceinline__ float scalar(float v) { return __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(v))); }
+__device__ __forceinline__ double scalar(double v) {
+  return __hiloint2double(__builtin_amdgcn_readfirstlane(__double2hiint(v)), __builtin_amdgcn_readfirstlane(__double2loint(v)));
+}
+
+// weight with which tap (lo, hi, frac) of one axis falls on index v
+template <typename A>
+__device__ __forceinline__ A axis_weight(int v, int lo, int hi, A frac) {
+  return (v == lo ? A(1) - frac : A(0)) + (v == hi ? frac : A(0));
+}
+
+template <typename T, typename RT>
+__global__ __launch_bounds__(kGatherThreads) void roi_backward_gather_kernel(
+    const T *__restrict__ gout, const RT *__restrict__ rois, T *__restrict__ gin, const RoiProblem p) {
+  using A = typename Acc<T>::type;
+  __shared__ GatherShared sh;
+  const int b = blockIdx.z, c = blockIdx.y;
+  const long plane = static_cast<long>(p.D) * p.H * p.W;
+  const long first = static_cast<long>(blockIdx.x) * (kGatherThreads * kGatherPerThread) + threadIdx.x;
+  const int cols = roi_columns(p.ndim, p.rotated);
+  const int nd = p.ndim;
+  const int cells[3] = {p.ow, p.oh, p.od};
+  const long ocells = static_cast<long>(p.od) * p.oh * p.ow;
+  constexpr double kSlack = 1e-6;   // the per-axis candidate ranges are widened by this much
+
+  T *dst = gin + (static_cast<long>(b) * p.C + c) * plane;
+  // per-voxel sums over the rois of the image (a thread's own slots; LDS because the voxel loop is
+  // not unrolled): the gradient is rounded to the tensor type once
+  __shared__ A sums[kGatherPerThread * kGatherThreads];
+  for (int k = 0; k < kGatherPerThread; k++) sums[k * kGatherThreads + threadIdx.x] = A(0);
+  const unsigned row = p.W, slice = static_cast<unsigned>(p.W) * p.H;   // plane < 2^31 (checked on the host)
+
+  for (int r = 0; r < p.R; r++) {
+    const RT *roi = rois + static_cast<long>(r) * cols;
+    if (static_cast<int>(roi[0]) != b) continue;   // uniform over the workgroup
+    __syncthreads();                                // the previous roi's geometry is no longer read
+    build_geom_block(sh.g, sh.trig, roi, p);
+    if (threadIdx.x < 3) {
+      const int j = threadIdx.x;
+      sh.reach[j] = fabs(sh.g.rot[j]) + fabs(sh.g.rot[3 + j]) + fabs(sh.g.rot[6 + j]) + kSlack;
+      sh.inv_bin[j] = sh.g.bin[j] > 1e-12 ? 1.0 / sh.g.bin[j] : 0.0;
+      const float slack = 1e-3f + 1e-6f * static_cast<float>(p.W + p.H + p.D);
+      sh.r1[j] = static_cast<float>(sh.g.rot[3 * j + 1]);
+      sh.r2[j] = static_cast<float>(sh.g.rot[3 * j + 2]);
+      sh.inv_m[j] = fabs(sh.g.rot[3 * j]) > 1e-6 ? static_cast<float>(1.0 / sh.g.rot[3 * j]) : 0.f;
+      sh.half[j] = (1.f + slack) * fabsf(sh.inv_m[j]);
+      if (j == 0) {
+        sh.inv_bin0 = static_cast<float>(sh.inv_bin[0]);
+        sh.off0 = static_cast<float>(sh.g.start[0] * sh.inv_bin[0] + 0.5);
+        sh.slack = slack;
+        sh.slack_u = 1e-3f + 1e-6f * static_cast<float>(p.ow) + slack * sh.inv_bin0;
+      }
+    }
+    __syncthreads();
+    // the roi's constants, in scalar registers for the loops below
+    RoiGeom g;
+#pragma unroll
+    for (int i = 0; i < 9; i++) g.rot[i] = scalar(sh.g.rot[i]);
+#pragma unroll
+    for (int i = 0; i < 3; i++) {
+      g.centre[i] = scalar(sh.g.centre[i]); g.start[i] = scalar(sh.g.start[i]);
+      g.bin[i] = scalar(sh.g.bin[i]); g.sub[i] = scalar(sh.g.sub[i]);
+    }
+    g.count = sh.g.count;
+    double reach[3], inv_bin[3];
+    float r1[3], r2[3], inv_m[3], half[3];
+#pragma unroll
+    for (int i = 0; i < 3; i++) {
+      reach[i] = scalar(sh.reach[i]); inv_bin[i] = scalar(sh.inv_bin[i]);
+      r1[i] = scalar(sh.r1[i]); r2[i] = scalar(sh.r2[i]); inv_m[i] = scalar(sh.inv_m[i]); half[i] = scalar(sh.half[i]);
+    }
+    const float inv_bin0 = scalar(sh.inv_bin0), off0 = scalar(sh.off0), slack = scalar(sh.slack), slack_u = scalar(sh.slack_u);
+    const T *go = gout + (static_cast<long>(r) * p.C + c) * ocells;
+    const A inv_count = A(1) / static_cast<A>(g.count);
+
+#pragma unroll 1
+    for (int k = 0; k < kGatherPerThread; k++) {
+      const long vi = first + static_cast<long>(k) * kGatherThreads;
+      if (vi >= plane) continue;
+      const unsigned vu = static_cast<unsigned>(vi), vzz = vu / slice, rem = vu - vzz * slice, vyy = rem / row;
+      const int v[3] = {static_cast<int>(rem - vyy * row), static_cast<int>(vyy), static_cast<int>(vzz)};
+      // the voxel in the roi's local frame: q = Rot^T (v - centre)
+      const double dx = v[0] - g.centre[0], dy = v[1] - g.centre[1], dz = nd == 3 ? v[2] - g.centre[2] : 0.0;
+      int lo[3], hi[3];
+      bool any = true;
+#pragma unroll
+      for (int j = 0; j < 3; j++) {
+        if (j >= nd) { lo[j] = 0; hi[j] = 0; continue; }
+        const double q = g.rot[j] * dx + g.rot[3 + j] * dy + g.rot[6 + j] * dz;
+        // cells u with |start + (u + .5) * bin - q| <= reach
+        const double a0 = q - reach[j] - g.start[j], a1 = q + reach[j] - g.start[j];
+        if (inv_bin[j] != 0.0) {
+          const double u0 = fmin(fmax(a0 * inv_bin[j] - 0.5 - kSlack, -1.0), static_cast<double>(cells[j]));
+          const double u1 = fmin(fmax(a1 * inv_bin[j] - 0.5 + kSlack, -1.0), static_cast<double>(cells[j]));
+          lo[j] = max(static_cast<int>(ceil(u0)), 0);
+          hi[j] = min(static_cast<int>(floor(u1)), cells[j] - 1);
+        } else {   // every cell samples the same coordinate
+          lo[j] = 0;
+          hi[j] = (a0 <= 0.0 && a1 >= 0.0) ? cells[j] - 1 : -1;
+        }
+        any = any && lo[j] <= hi[j];
+      }
+      if (!any) continue;
+      A sum = A(0);
+      const float cv[3] = {static_cast<float>(-dx), static_cast<float>(-dy), static_cast<float>(-dz)};
+      const float cells0 = static_cast<float>(cells[0]);
+      for (int uz = lo[2]; uz <= hi[2]; uz++) {
+        const double z = nd == 3 ? local_coord(g, 2, uz, 0) : 0.0;
+        const float zf = static_cast<float>(z);
+        const float bz[3] = {fmaf(r2[0], zf, cv[0]), fmaf(r2[1], zf, cv[1]), fmaf(r2[2], zf, cv[2])};
+        for (int uy = lo[1]; uy <= hi[1]; uy++) {
+          const double y = local_coord(g, 1, uy, 0);
+          const float yf = static_cast<float>(y);
+          // samples of this output row: r_a(x) - v_a = rot[a][0] * x + base_a; keep it within +-1
+          float xl = -3e38f, xh = 3e38f;
+#pragma unroll
+          for (int a = 0; a < 3; a++) {
+            if (a >= nd) continue;
+            const float base = fmaf(r1[a], yf, bz[a]);
+            if (inv_m[a] != 0.f) {
+              const float mid = -base * inv_m[a];
+              xl = fmaxf(xl, mid - half[a]);
+              xh = fminf(xh, mid + half[a]);
+            } else if (fabsf(base) > 1.f + 2.f * slack) {
+              xh = -3e38f;
+            }
+          }
+          if (xl > xh) continue;
+          int x0 = lo[0], x1 = hi[0];
+          if (inv_bin0 != 0.f) {
+            const float u0 = fminf(fmaxf(fmaf(xl, inv_bin0, -off0) - slack_u, -1.f), cells0);
+            const float u1 = fminf(fmaxf(fmaf(xh, inv_bin0, -off0) + slack_u, -1.f), cells0);
+            x0 = max(x0, static_cast<int>(ceilf(u0)));
+            x1 = min(x1, static_cast<int>(floorf(u1)));
+          }
+          if (x0 > x1) continue;
+          // sample positions of the row in fp64: rot[a][0] * x + row term
+          const double bx = g.rot[1] * y + g.rot[2] * z + g.centre[0];
+          const double by = g.rot[4] * y + g.rot[5] * z + g.centre[1];
+          const double bw = g.rot[7] * y + g.rot[8] * z + g.centre[2];
+          for (int ux = x0; ux <= x1; ux++) {
+            const double x = local_coord(g, 0, ux, 0);
+            const double rx = fma(g.rot[0], x, bx), ry = fma(g.rot[3], x, by);
+            const double rz = nd == 3 ? fma(g.rot[6], x, bw) : 0.0;
+            int z0, z1, y0, y1, c0, c1;
+            A lz, ly, lx;
+            if (!clamped_tap(rz, p.D, z0, z1, lz, p.order) || !clamped_tap(ry, p.H, y0, y1, ly, p.order) ||
+                !clamped_tap(rx, p.W, c0, c1, lx, p.order))
+              continue;
+            const A w = axis_weight(v[2], z0, z1, lz) * axis_weight(v[1], y0, y1, ly) * axis_weight(v[0], c0, c1, lx);
+            if (w != A(0))
+              sum += load(go + (static_cast<long>(uz) * p.oh + uy) * p.ow + ux) * inv_count * w;
+          }
+        }
+      }
+      if (sum != A(0)) sums[k * kGatherThreads + threadIdx.x] += sum;
+    }
+  }
+  // this thread owns its voxels: plain read-modify-write
+  for (int k = 0; k < kGatherPerThread; k++) {
+    const long vi = first + static_cast<long>(k) * kGatherThreads;
+    const A total = sums[k * kGatherThreads + threadIdx.x];
+    if (vi < plane && total != A(0)) dst[vi] = store_cast<T>(load(dst + vi) + total);
+  }
+}
+
+// Applies when the problem is a resampling: one sample per cell, outputs of at least 4096 voxels
+// that are not much smaller than the image, at most two rois per image on average (every input
+// voxel walks over all rois of its image).  Returns -1 otherwise.
+int roi_backward_gather(const void *grad_output, const void *rois, void *grad_input, int dtype,
+                        const RoiProblem &p, hipStream_t s) {
+  const long plane = static_cast<long>(p.D) * p.H * p.W;
+  const long ocells = static_cast<long>(p.od) * p.oh * p.ow;
+  if (p.sampling_ratio != 1 || (p.order != 0 && p.order != 1)) return -1;
+  if (ocells < 4096 || ocells * 8 < plane || p.R > 2 * p.N) return -1;
+  if (p.C > 65535 || p.N > 65535 || plane >= (1L << 31)) return -1;
+  const long blocks = (plane + kGatherThreads * kGatherPerThread - 1) / (kGatherThreads * kGatherPerThread);
+  if (blocks >= (1L << 31)) return -1;
+  const dim3 grid(static_cast<unsigned>(blocks), p.C, p.N), block(kGatherThreads);
+  MV_DISPATCH(dtype, {
+    using RT = typename std::conditional<std::is_same<T, double>::value, double, float>::type;
+    hipLaunchKernelGGL((roi_backward_gather_kernel<T, RT>), grid, block, 0, s,
+                       static_cast<const T *>(grad_output), static_cast<const RT *>(rois),
+                       static_cast<T *>(grad_input), p);
+  });
+  return check_launch("roi_backward_gather_kernel");
+}
+
+}  // namespace mv

@@ -199,3 +199,53 @@ def test_dcn_sweep(ops, oracle):
         if modulated:
             assert rel_err(ms.grad, gm) <= tol, what + " (grad mask)"
     assert ran > 200
+
+
+def test_resampling_backward_sweep(ops, oracle):
+    """Backward of resampling-sized problems (one sample per cell, outputs about as large as the
+    image, a roi or two per image): these take the atomic-free gather kernel.  Plain and rotated
+    rois that reach beyond every border, up- and down-sampling, zero extents, orders 0 and 1."""
+    for seed in range(9500, 9580):
+        rnd = random.Random(seed)
+        g = torch.Generator().manual_seed(seed)
+        ndim = rnd.choice([2, 3])
+        rotated = rnd.random() < 0.7
+        hi = 40 if ndim == 3 else 120
+        lo = 12 if ndim == 3 else 50
+        size = [rnd.randint(lo, hi) for _ in range(ndim)]
+        out = tuple(rnd.randint(max(lo, s // 2), hi) for s in size)   # >= 4096 cells, >= plane / 8
+        batch, channels = rnd.randint(1, 3), rnd.choice([1, 1, 2])
+        n = rnd.randint(1, 2 * batch)
+        dtype = rnd.choice(DTYPES)
+        order = rnd.choice([0, 1, 1, 1])
+        scale = rnd.choice([0.5, 1.0, 1.0, 2.0])
+        aligned = rnd.random() < 0.7
+        feat = torch.randn(batch, channels, *size, generator=g).to(dtype)
+        ext = torch.tensor(size[::-1], dtype=torch.float32) / scale
+        cols = {(2, False): 5, (3, False): 7, (2, True): 6, (3, True): 10}[(ndim, rotated)]
+        rois = torch.zeros(n, cols)
+        rois[:, 0] = torch.randint(0, batch, (n,), generator=g)
+        if rotated:
+            rois[:, 1:1 + ndim] = ext / 2 + (torch.rand(n, ndim, generator=g) - 0.5) * ext * rnd.choice([0.1, 0.5, 1.2])
+            rois[:, 1 + ndim:1 + 2 * ndim] = ext * (0.2 + torch.rand(n, ndim, generator=g) * rnd.choice([0.8, 1.3, 2.5]))
+            rois[:, 1 + 2 * ndim:] = (torch.rand(n, cols - 1 - 2 * ndim, generator=g) - 0.5) * rnd.choice([0.0, 0.4, 1.2, 6.3])
+        else:
+            start = (torch.rand(n, ndim, generator=g) * 0.8 - 0.3) * ext
+            rois[:, 1:1 + ndim] = start
+            rois[:, 1 + ndim:] = start + ext * (0.2 + torch.rand(n, ndim, generator=g) * rnd.choice([0.8, 1.5]))
+        if rnd.random() < 0.15:
+            rois[0, 1 + ndim:1 + 2 * ndim] = 0.0 if rotated else rois[0, 1:1 + ndim]   # zero extent
+        mod = ops.RoIAlignRotated(out, scale, 1, aligned) if rotated else ops.RoIAlign(out, scale, 1)
+        fg = feat.to(DEV).requires_grad_(True)
+        got = mod(fg, rois.to(DEV), order=order)
+        gy = torch.randn(got.shape, generator=g).to(dtype)
+        got.backward(gy.to(DEV))
+        want = oracle.roi_align_backward(gy, rois, feat.shape, scale, 1, aligned, order, rotated)
+        what = f"seed {seed}: {ndim}-D rotated={rotated} {tuple(feat.shape)} -> {out} rois={n} order={order} {dtype}"
+        if order == 0:   # a sample within rounding of a .5 tie may go to the other neighbour
+            diff = (fg.grad.cpu().double() - want.double()).abs()
+            assert float((diff > BWD_TOL[dtype] * float(want.abs().max())).double().mean()) <= 4e-3, what
+        else:
+            # no atomics, fp32 sums, one rounding per voxel: 16-bit results carry half an ulp
+            tol = BWD_TOL[dtype] if dtype in (torch.float32, torch.float64) else FWD_TOL[dtype]
+            assert rel_err(fg.grad, want) <= tol, what
