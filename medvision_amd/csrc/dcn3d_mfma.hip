@@ -195,12 +195,19 @@ __global__ __launch_bounds__(256) void dcn_weight_fragments16_kernel(const T *__
 #ifndef MV_DCN_NB
 #define MV_DCN_NB 1
 #endif
+#ifndef MV_DCN_WAVES_2D
+#define MV_DCN_WAVES_2D 6
+#endif
 // bytes per weight buffer (two per workgroup): 12 KB lets five workgroups share a CU's LDS, 16 KB
 // (four workgroups) serves layers whose tap does not fit the smaller one
 constexpr int kWeightLdsSmall = 12 * 1024, kWeightLds = 16 * 1024;
 
-template <typename T, int MB, int NB, int WBYTES>
-__global__ __launch_bounds__(256, NB == 1 ? 5 : 4) void dcn_forward_mfma16_kernel(
+// NC: corners per sample, 8 for volumes, 4 for images (a depth-1 volume: the upper z slice never
+// exists, so its loads, weights and blend steps are left out at compile time).
+// UNITS: a tap's weight pieces do not fit one LDS buffer and are walked in units of fewer channel
+// slices (layers with many channels per group); otherwise a refill brings whole taps.
+template <typename T, int MB, int NB, int WBYTES, int NC, bool UNITS>
+__global__ __launch_bounds__(256, NB == 1 ? (NC == 4 && WBYTES <= 12 * 1024 ? MV_DCN_WAVES_2D : 5) : 4) void dcn_forward_mfma16_kernel(
     const T *__restrict__ xt, const T *__restrict__ off, const T *__restrict__ mask,
     const T *__restrict__ wf, const T *__restrict__ bias, T *__restrict__ y, const DcnDims s) {
   using M = Mfma<T>;
@@ -234,18 +241,24 @@ __global__ __launch_bounds__(256, NB == 1 ? 5 : 4) void dcn_forward_mfma16_kerne
 #pragma unroll
     for (int m = 0; m < MB; m++) acc[nb][m] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-  // weight pieces of one tap: [slice][block of this chunk][lane] 16 bytes, copied by the workgroup
-  const int tap_pieces = slices * MB * 64;                       // 16-byte pieces per tap
+  // Weight pieces in LDS, double-buffered: a "unit" is one tap restricted to `sc` channel slices,
+  // [slice][block of this chunk][lane] 16 bytes.  Usually sc = all slices and a refill brings as
+  // many whole taps as fit (one workgroup barrier per refill); layers with many channels per group
+  // walk a tap in several units (nunits > 1), the tap's corner offsets and weights staying in
+  // registers in between.
+  const int sc = UNITS ? min(slices, WBYTES / 16 / (MB * 64)) : slices;
+  const int nunits = UNITS ? (slices + sc - 1) / sc : 1;         // units per tap
+  const int unit_pieces = sc * MB * 64;
+  const int total_units = s.K * nunits;
   const T *wfg = wf + static_cast<long>(g) * s.K * slices * blocks * (64 * PC);
-  // as many taps per refill as fit: one workgroup barrier per group of taps
-  const int group = max(1, min(s.K, WBYTES / 16 / tap_pieces));
-  auto fill = [&](int k0, int buf) {
-    const int count = min(group, s.K - k0) * tap_pieces;
+  const int group = nunits == 1 ? max(1, min(s.K, WBYTES / 16 / unit_pieces)) : 1;   // units per refill
+  auto fill = [&](int u0, int buf) {
+    const int count = min(group, total_units - u0) * unit_pieces;
     for (int i = threadIdx.x; i < count; i += 256) {
-      const int k = k0 + i / tap_pieces, rem = i % tap_pieces;
-      const int ln = rem % 64, m = (rem / 64) % MB, cc = rem / (64 * MB);
+      const int u = u0 + i / unit_pieces, rem = i % unit_pieces;
+      const int ln = rem % 64, m = (rem / 64) % MB, cc = (u % nunits) * sc + rem / (64 * MB), k = u / nunits;
       u32x4 v = u32x4{0u, 0u, 0u, 0u};
-      if (mb0 + m < blocks)
+      if (mb0 + m < blocks && cc < slices)
         v = *reinterpret_cast<const u32x4 *>(wfg + (((static_cast<long>(k) * slices + cc) * blocks + mb0 + m) * 64 + ln) * PC);
       reinterpret_cast<u32x4 *>(wlds[buf])[i] = v;
     }
@@ -254,36 +267,43 @@ __global__ __launch_bounds__(256, NB == 1 ? 5 : 4) void dcn_forward_mfma16_kerne
   __syncthreads();
 
   const int dg_first = g * s.cpg / s.cpd, dg_last = (g * s.cpg + s.cpg - 1) / s.cpd;
+  const bool one_dg = dg_first == dg_last;   // then a tap's corners are kept from unit to unit
   const unsigned cin = s.Cin;
   int ki = 0, kj = 0, kk = 0;
-  for (int k = 0, in_group = 0, buf = 0; k < s.K; k++) {
-    if (in_group == 0 && k + group < s.K) fill(k + group, buf ^ 1);
-    const u32x4 *wl = reinterpret_cast<const u32x4 *>(wlds[buf]) + in_group * tap_pieces;
+  float cw[NB][NC];
+  unsigned at[NB][NC];
+  for (int u = 0, k = 0, unit = 0, in_group = 0, buf = 0; u < total_units; u++) {
+    if (in_group == 0 && u + group < total_units) fill(u + group, buf ^ 1);
+    const u32x4 *wl = reinterpret_cast<const u32x4 *>(wlds[buf]) + in_group * unit_pieces;
+    const int s_lo = UNITS ? unit * sc : 0, s_hi = UNITS ? min(slices, s_lo + sc) : slices;   // slices of this unit
     for (int dgi = dg_first; dgi <= dg_last; dgi++) {
       const int c_lo = max(g * s.cpg, dgi * s.cpd), c_hi = min(g * s.cpg + s.cpg, (dgi + 1) * s.cpd);
-      const int cc_lo = (c_lo - g * s.cpg) / SL, cc_hi = (c_hi - g * s.cpg) / SL;
+      const int cc_lo = max((c_lo - g * s.cpg) / SL, s_lo), cc_hi = min((c_hi - g * s.cpg) / SL, s_hi);
+      if (cc_lo >= cc_hi) continue;
       const long bg = static_cast<long>(b) * s.dg + dgi;
 #pragma unroll
       for (int nb = 0; nb < NB; nb++) {
-        P pd, ph, pw;
-        dcn_offsets(s, off + (bg * s.nd * s.K + s.nd * k) * s.Q + qc[nb], pd, ph, pw);
-        pd += static_cast<P>(bd[nb] + ki * s.dd); ph += static_cast<P>(bh[nb] + kj * s.dh); pw += static_cast<P>(bw[nb] + kk * s.dw);
-        const float m = mask ? load(mask + (bg * s.K + k) * s.Q + qc[nb]) : 1.f;
-        CornerTaps t;
-        corner_taps<P>(s, pd, ph, pw, true, cin * ES, static_cast<unsigned>(lk) * 16u, 0x80000000u, t);
-        float cw[8];
+        if (!UNITS || unit == 0 || !one_dg) {
+          P pd, ph, pw;
+          dcn_offsets(s, off + (bg * s.nd * s.K + s.nd * k) * s.Q + qc[nb], pd, ph, pw);
+          pd += static_cast<P>(bd[nb] + ki * s.dd); ph += static_cast<P>(bh[nb] + kj * s.dh); pw += static_cast<P>(bw[nb] + kk * s.dw);
+          if (NC == 4) pd = P(0);   // images: the only slice
+          const float m = mask ? load(mask + (bg * s.K + k) * s.Q + qc[nb]) : 1.f;
+          CornerTaps t;
+          corner_taps<P>(s, pd, ph, pw, true, cin * ES, static_cast<unsigned>(lk) * 16u, 0x80000000u, t);
 #pragma unroll
-        for (int c = 0; c < 8; c++) cw[c] = m * t.w[c];
+          for (int c = 0; c < NC; c++) { cw[nb][c] = m * t.w[c]; at[nb][c] = t.at[c]; }
+        }
         for (int cc = cc_lo; cc < cc_hi; cc++) {
           const unsigned c0 = g * s.cpg + cc * SL;
-          u32x4 raw[8];
+          u32x4 raw[NC];
 #pragma unroll
-          for (int c = 0; c < 8; c++) raw[c] = __builtin_amdgcn_raw_buffer_load_b128(xr, t.at[c], c0 * ES, 0);
+          for (int c = 0; c < NC; c++) raw[c] = __builtin_amdgcn_raw_buffer_load_b128(xr, at[nb][c], c0 * ES, 0);
           float v[PC];
 #pragma unroll
           for (int i = 0; i < PC; i++) v[i] = 0.f;
 #pragma unroll
-          for (int c = 0; c < 8; c++) M::fma_piece(v, cw[c], raw[c]);
+          for (int c = 0; c < NC; c++) M::fma_piece(v, cw[nb][c], raw[c]);
           const u32x4 mine = M::pack(v);   // piece lk of position lj; wanted: piece kc of position j
           const u32x4 bpiece = u32x4{
               static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(from, static_cast<int>(mine.x))),
@@ -292,11 +312,15 @@ __global__ __launch_bounds__(256, NB == 1 ? 5 : 4) void dcn_forward_mfma16_kerne
               static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(from, static_cast<int>(mine.w)))};
 #pragma unroll
           for (int mm = 0; mm < MB; mm++)
-            acc[nb][mm] = M::run16(wl[(cc * MB + mm) * 64 + lane], bpiece, acc[nb][mm]);
+            acc[nb][mm] = M::run16(wl[((cc - s_lo) * MB + mm) * 64 + lane], bpiece, acc[nb][mm]);
         }
       }
     }
-    if (++kk == s.kw) { kk = 0; if (++kj == s.kh) { kj = 0; ++ki; } }
+    if (!UNITS || ++unit == nunits) {
+      unit = 0;
+      k++;
+      if (++kk == s.kw) { kk = 0; if (++kj == s.kh) { kj = 0; ++ki; } }
+    }
     if (++in_group == group) {
       in_group = 0;
       buf ^= 1;
@@ -365,9 +389,14 @@ static int dcn_mfma_run(const void *x, const void *off, const void *mask, const 
   // 16 x 16 tiling: whole 4-piece slices per (deformable) group and a tap's weight pieces fit LDS
   {
     const int blocks16 = s.opg / 16;
-    const int mb = blocks16 >= 4 ? 4 : (blocks16 >= 2 ? 2 : 1);
+    // output blocks of 16 per wavefront: up to 8 (128 output channels: every pass over the output
+    // channels repeats the gather, so wide layers want few passes)
+    const int mb = (blocks16 >= 8 && s.nd == 2) ? 8 : (blocks16 >= 4 ? 4 : (blocks16 >= 2 ? 2 : 1));
     const long tap_bytes = static_cast<long>(s.cpg / (4 * PC)) * mb * 64 * 16;
-    if (s.cpg % (4 * PC) == 0 && s.cpd % (4 * PC) == 0 && tap_bytes <= kWeightLds) {
+    // a tap that does not fit one weight buffer is walked in units of fewer channel slices; that
+    // keeps the tap's corners in registers, which needs one deformable group per convolution group
+    const bool fits = tap_bytes <= kWeightLds || s.cpd % s.cpg == 0;
+    if (s.cpg % (4 * PC) == 0 && s.cpd % (4 * PC) == 0 && fits) {
       const long lanes = static_cast<long>(s.groups) * s.K * (s.cpg / (4 * PC)) * blocks16 * 64;
       hipLaunchKernelGGL((dcn_weight_fragments16_kernel<T>), dim3(static_cast<unsigned>((lanes + 255) / 256)),
                          dim3(256), 0, stream, static_cast<const T *>(wt), wf, s);
@@ -376,11 +405,27 @@ static int dcn_mfma_run(const void *x, const void *off, const void *mask, const 
       const long qblocks = (s.Q + 64 * kNb - 1) / (64 * kNb);
       MV_REQUIRE(qblocks < (1L << 31) && static_cast<long>(s.groups) * chunks <= 65535, "grid too large");
       const dim3 grid(static_cast<unsigned>(qblocks), s.groups * chunks, s.B), block(256);
-#define MV_LAUNCH_MFMA16(MBV, WB)                                                                \
-  hipLaunchKernelGGL((dcn_forward_mfma16_kernel<T, MBV, kNb, WB>), grid, block, 0, stream, xt,   \
-                     static_cast<const T *>(off), static_cast<const T *>(mask), wf,              \
+#define MV_LAUNCH_MFMA16_K(MBV, WB, NCV, UV)                                                          \
+  hipLaunchKernelGGL((dcn_forward_mfma16_kernel<T, MBV, kNb, WB, NCV, UV>), grid, block, 0, stream, xt, \
+                     static_cast<const T *>(off), static_cast<const T *>(mask), wf,                  \
                      static_cast<const T *>(bias), static_cast<T *>(y), s)
-      if (tap_bytes <= kWeightLdsSmall) {
+      // whole taps per refill unless the tap is larger than the (large) buffer
+#define MV_LAUNCH_MFMA16_NC(MBV, WB, NCV)                                                             \
+  do {                                                                                                \
+    if (WB == kWeightLds && static_cast<long>(s.cpg / (4 * PC)) * MBV * 64 * 16 > kWeightLds)         \
+      MV_LAUNCH_MFMA16_K(MBV, kWeightLds, NCV, true);                                                 \
+    else                                                                                              \
+      MV_LAUNCH_MFMA16_K(MBV, WB, NCV, false);                                                        \
+  } while (0)
+#define MV_LAUNCH_MFMA16(MBV, WB)                                                                \
+  do {                                                                                            \
+    if (s.nd == 2 && s.D == 1 && s.kd == 1 && s.pd == 0)                                          \
+      MV_LAUNCH_MFMA16_NC(MBV, WB, 4);                                                            \
+    else                                                                                          \
+      MV_LAUNCH_MFMA16_NC(MBV, WB, 8);                                                            \
+  } while (0)
+      if (mb == 8) MV_LAUNCH_MFMA16(8, kWeightLds);
+      else if (tap_bytes <= kWeightLdsSmall) {
         if (mb == 4) MV_LAUNCH_MFMA16(4, kWeightLdsSmall);
         else if (mb == 2) MV_LAUNCH_MFMA16(2, kWeightLdsSmall);
         else MV_LAUNCH_MFMA16(1, kWeightLdsSmall);
@@ -390,6 +435,8 @@ static int dcn_mfma_run(const void *x, const void *off, const void *mask, const 
         else MV_LAUNCH_MFMA16(1, kWeightLds);
       }
 #undef MV_LAUNCH_MFMA16
+#undef MV_LAUNCH_MFMA16_NC
+#undef MV_LAUNCH_MFMA16_K
       return check_launch("dcn_forward_mfma16_kernel");
     }
   }
