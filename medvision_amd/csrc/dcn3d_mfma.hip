@@ -20,6 +20,8 @@
 //     [lane][8] (workspace) so that a fragment is one coalesced 16-byte load per lane (L2 hits).
 // The sampling gather, not the matrix core, bounds this kernel: per (tap, position) 8 corners x
 // Cin channels are fetched, 8 x more bytes than the fragment holds.
+#include <cstdint>
+
 #include "dcn_mfma.hpp"
 
 namespace mv {
@@ -43,6 +45,41 @@ __global__ void dcn_channels_last_kernel(const U *__restrict__ x, U *__restrict_
   for (int i = threadIdx.x; i < count; i += 256) {
     const int pp = i / cn, c = i % cn;
     dst[static_cast<long>(pp) * Cin + c] = stage[pp][c];
+  }
+}
+
+// The same move with 16-byte global accesses: rows of x are read as groups of 16 bytes (V
+// positions of one channel), kept in LDS as [channel][position], and every lane writes V channels
+// of one position.  Needs P and Cin to be multiples of V and 16-byte aligned tensors.
+constexpr int kLayoutPos = 128;
+template <typename U>
+__global__ __launch_bounds__(256) void dcn_channels_last_wide_kernel(const U *__restrict__ x, U *__restrict__ xt,
+                                                                     int Cin, long P) {
+  constexpr int V = 16 / sizeof(U), CH = 256 / sizeof(U);   // CH channels per workgroup: 128 (2 bytes), 64 (4 bytes)
+  constexpr int PITCH = kLayoutPos + V;
+  __shared__ __attribute__((aligned(16))) U stage[CH * PITCH];
+  const int b = blockIdx.y;
+  const long p0 = static_cast<long>(blockIdx.x) * kLayoutPos;
+  const int c0 = blockIdx.z * CH, cn = min(CH, Cin - c0);
+  const int np = static_cast<int>(min(static_cast<long>(kLayoutPos), P - p0));   // a multiple of V
+  const U *src = x + (static_cast<long>(b) * Cin + c0) * P + p0;
+  U *dst = xt + (static_cast<long>(b) * P + p0) * Cin + c0;
+  constexpr int PG = kLayoutPos / V;
+  for (int i = threadIdx.x; i < cn * PG; i += 256) {
+    const int c = i / PG, pg = i % PG;
+    if (pg * V < np)
+      *reinterpret_cast<u32x4 *>(stage + c * PITCH + pg * V) = *reinterpret_cast<const u32x4 *>(src + static_cast<long>(c) * P + pg * V);
+  }
+  __syncthreads();
+  const int cg_n = cn / V;
+  for (int i = threadIdx.x; i < np * cg_n; i += 256) {
+    const int pp = i / cg_n, cg = i % cg_n;
+    U out[V];
+#pragma unroll
+    for (int e = 0; e < V; e++) out[e] = stage[(cg * V + e) * PITCH + pp];
+    u32x4 packed;
+    __builtin_memcpy(&packed, out, 16);
+    *reinterpret_cast<u32x4 *>(dst + static_cast<long>(pp) * Cin + cg * V) = packed;
   }
 }
 
@@ -346,6 +383,21 @@ __global__ __launch_bounds__(256, NB == 1 ? (NC == 4 && WBYTES <= 12 * 1024 ? MV
 
 // [B, C, P] -> [B, P, C] for elements of 2 or 4 bytes
 int dcn_channels_last(const void *x, void *xt, int B, int C, long P, int elem_bytes, hipStream_t stream) {
+  const int vec = 16 / elem_bytes;
+  const bool aligned = reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(xt) % 16 == 0;
+  if (aligned && P % vec == 0 && C % vec == 0) {
+    const long wblocks = (P + kLayoutPos - 1) / kLayoutPos;
+    const int ch = 256 / elem_bytes;
+    MV_REQUIRE(wblocks < (1L << 31) && B <= 65535 && (C + ch - 1) / ch <= 65535, "volume too large");
+    const dim3 wgrid(static_cast<unsigned>(wblocks), B, (C + ch - 1) / ch);
+    if (elem_bytes == 2)
+      hipLaunchKernelGGL((dcn_channels_last_wide_kernel<unsigned short>), wgrid, dim3(256), 0, stream,
+                         static_cast<const unsigned short *>(x), static_cast<unsigned short *>(xt), C, P);
+    else
+      hipLaunchKernelGGL((dcn_channels_last_wide_kernel<unsigned int>), wgrid, dim3(256), 0, stream,
+                         static_cast<const unsigned int *>(x), static_cast<unsigned int *>(xt), C, P);
+    return check_launch("dcn_channels_last_wide_kernel");
+  }
   const long pblocks = (P + 63) / 64;
   MV_REQUIRE(pblocks < (1L << 31) && B <= 65535, "volume too large");
   const dim3 grid(static_cast<unsigned>(pblocks), B, (C + kLayoutChunk - 1) / kLayoutChunk);
