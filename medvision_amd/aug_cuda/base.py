@@ -19,6 +19,19 @@ import numpy as np
 import torch
 
 
+def _peak_mib():
+    """Peak of allocated GPU memory in MiB, as ``torch.cuda.max_memory_allocated`` reports it; read
+    from the allocator's counters directly (the public call flattens the whole statistics tree
+    first, tens of microseconds per stage)."""
+    if not torch.cuda.is_available():
+        return 0.0
+    try:
+        stats = torch._C._cuda_memoryStats(torch.cuda.current_device())
+        return stats["allocated_bytes"]["all"]["peak"] / 2 ** 20
+    except Exception:   # private interface: fall back to the public one
+        return torch.cuda.max_memory_allocated() / 2 ** 20
+
+
 class CudaAugBase:
     batched = False     # True: tensors carry a leading batch axis
 
@@ -100,6 +113,7 @@ class CudaAugBase:
 
     # ---- driver ------------------------------------------------------------------------------
     def _apply_all(self, result):
+        self._device_rois = None   # images and segmentations share one upload of the stage's rois
         self.apply_to_img(result)
         self.apply_to_cls(result)
         self.apply_to_seg(result)
@@ -116,7 +130,7 @@ class CudaAugBase:
             self._apply_all(result)
         for key in ('history', 'time', 'memory'):
             result.setdefault(key, [])
-        peak = torch.cuda.max_memory_allocated() / 2 ** 20 if torch.cuda.is_available() else 0.0
+        peak = _peak_mib()
         result['history'].append(self.name)
         result['memory'].append(f"{self.name}-{peak:.02f}MB")
         started = datetime.fromtimestamp(tic).strftime('%H:%M:%S.%f')

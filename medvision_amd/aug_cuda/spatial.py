@@ -39,7 +39,9 @@ class _Resampler:
         lead = 2 if self.batched else 1
         assert tensor.ndim == self.dim + lead, 'image should be [batch,] channel, **dim'
         fn = affine_2d if self.dim == 2 else affine_3d
-        rois = torch.from_numpy(self._rois()).to(tensor.device)
+        rois = getattr(self, '_device_rois', None)
+        if rois is None or rois.device != tensor.device:
+            rois = self._device_rois = torch.from_numpy(self._rois()).to(tensor.device)
         batch = tensor if self.batched else tensor.unsqueeze(0)
         out = fn(batch, rois, tuple(int(v) for v in self._out_size()), 1.0, sampling_ratio, True, order)
         return out if self.batched else out.squeeze(0)
