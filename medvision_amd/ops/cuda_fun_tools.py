@@ -18,7 +18,8 @@ def _affine(ndim, features, rois, out_size, spatial_scale, sampling_ratio, align
     assert order in [0, 1, 3], f'order {order} is not supported!'
     if order == 0:
         sampling_ratio = 1  # never average nearest-neighbour samples (reference :72-74)
-    output = features.new_zeros(rois.size(0), features.size(1), *out)
+    # every output element is written by the kernel (zeros where a sample is void): no zero fill
+    output = features.new_empty(rois.size(0), features.size(1), *out)
     fn = _C.affine_2d if ndim == 2 else _C.affine_3d
     fn(features, rois, output, *out, spatial_scale, sampling_ratio, aligned, order)
     return output

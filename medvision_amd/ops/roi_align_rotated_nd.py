@@ -29,7 +29,8 @@ def _forward(ndim, ctx, features, rois, output_size, spatial_scale, sampling_rat
     ctx.aligned, ctx.order = aligned, order
     ctx.save_for_backward(rois)
     ctx.feature_size = features.size()
-    output = features.new_zeros(rois.size(0), features.size(1), *out)
+    # every output element is written by the kernel (zeros where a sample is void): no zero fill
+    output = features.new_empty(rois.size(0), features.size(1), *out)
     _kernels(ndim)[0](features, rois, output, *out, spatial_scale, sampling_ratio, aligned, order)
     return output
 

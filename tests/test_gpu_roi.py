@@ -368,3 +368,38 @@ def test_volume_beyond_2_31_elements(ops):
     out.backward(torch.ones_like(out))
     assert float(vol.grad[0, 0, lo:lo + n, lo:lo + n, lo:lo + n].float().sum()) == n ** 3
     assert float(vol.grad[0, 0, lo, lo, lo]) == 1.0 and float(vol.grad[0, 0, 0, 0, 0]) == 0.0
+
+
+@pytest.mark.parametrize("order", [0, 1, 3])
+@pytest.mark.parametrize("out", [(6, 7, 8), (24, 40, 48)])   # general / pooled kernels, tiled kernels
+def test_every_output_element_is_written(ops, oracle, order, out):
+    """The operators allocate their outputs uninitialised: every element has to be stored by the
+    kernels, zeros included (rois wholly outside the volume, rois of an image that does not exist,
+    void samples at the borders).  The buffers handed to the shim here are full of NaN."""
+    from medvision_amd import _C
+    g = wl.gen(31 + order)
+    feat = torch.randn(2, 3, 10, 12, 16, generator=g).half()
+    rot = torch.tensor([[0, 8.0, 6.0, 5.0, 20.0, 14.0, 12.0, 0.3, -0.2, 0.5],        # reaches beyond every border
+                        [1, 200.0, 6.0, 5.0, 10.0, 10.0, 10.0, 0.0, 0.0, 0.4],      # wholly outside
+                        [1, -50.0, -60.0, -70.0, 8.0, 8.0, 8.0, 0.1, 0.0, 0.0],     # wholly outside
+                        [5, 8.0, 6.0, 5.0, 8.0, 8.0, 8.0, 0.0, 0.0, 0.0]])          # no such image
+    output = torch.full((4, 3, *out), float("nan"), dtype=torch.float16, device=DEV)
+    _C.affine_3d(feat.to(DEV), rot.to(DEV), output, *out, 1.0, 1, True, order)
+    assert not bool(torch.isnan(output).any())
+    assert float(output[1:].abs().max()) == 0.0
+    assert_close(output[:1], oracle.roi_align_forward(feat, rot[:1], out, 1.0, 1, True, order, True),
+                 FWD_TOL[torch.float16], "affine")
+    if order == 3:
+        return
+    output.fill_(float("nan"))
+    sr = 1 if order == 0 else 2   # the operator classes never average nearest-neighbour samples
+    _C.roi_align_rotated_3d_forward(feat.to(DEV), rot.to(DEV), output, *out, 1.0, sr, True, order)
+    assert not bool(torch.isnan(output).any()) and float(output[1:].abs().max()) == 0.0
+    # (extents that put no sample on a .5 tie: at order 0 rounding would decide those)
+    box = torch.tensor([[0, -3.1, 2.2, 1.3, 12.4, 15.1, 9.2], [1, 300.0, 2.0, 1.0, 312.0, 9.0, 8.0],
+                        [7, 1.0, 2.0, 1.0, 9.0, 9.0, 8.0]])
+    output = torch.full((3, 3, *out), float("nan"), dtype=torch.float16, device=DEV)
+    _C.roi_align_3d_forward(feat.to(DEV), box.to(DEV), output, *out, 1.0, sr, order)
+    assert not bool(torch.isnan(output).any()) and float(output[1:].abs().max()) == 0.0
+    assert_close(output[:1], oracle.roi_align_forward(feat, box[:1], out, 1.0, sr, True, order, False),
+                 FWD_TOL[torch.float16], "plain boxes")
