@@ -74,7 +74,7 @@ def bench_dcn(args, dtype=torch.float16):
         with torch.no_grad():
             modulated_deform_conv(x, off, mask, w, b, 1, 1, 1, 1, 1)
 
-    ms, _ = _events_ms(step, max(3, args.steps // 10), max(1, args.warmup // 5))
+    ms, _ = _events_ms(step, max(3, args.steps), max(1, args.warmup))
     flops = 2 * 2 * 64 * 32 * 27 * 48 ** 3
 
     # training step (forward + all five gradients), reported beside the forward figure
@@ -86,7 +86,7 @@ def bench_dcn(args, dtype=torch.float16):
             t.grad = None
         modulated_deform_conv(*ins, 1, 1, 1, 1, 1).backward(gy)
 
-    train_ms, _ = _events_ms(train_step, max(3, args.steps // 20), 3)
+    train_ms, _ = _events_ms(train_step, max(3, args.steps // 4), 3)
     return {"ms": ms, "tflops": flops / ms / 1e9, "flops": flops, "train_ms": train_ms}
 
 
