@@ -74,7 +74,7 @@ def bench_dcn(args, dtype=torch.float16):
         with torch.no_grad():
             modulated_deform_conv(x, off, mask, w, b, 1, 1, 1, 1, 1)
 
-    ms, _ = _events_ms(step, max(3, args.steps), max(1, args.warmup))
+    ms, _ = _events_ms(step, max(3, min(args.steps, 400)), max(1, min(args.warmup, 40)))
     flops = 2 * 2 * 64 * 32 * 27 * 48 ** 3
 
     # training step (forward + all five gradients), reported beside the forward figure
@@ -86,7 +86,7 @@ def bench_dcn(args, dtype=torch.float16):
             t.grad = None
         modulated_deform_conv(*ins, 1, 1, 1, 1, 1).backward(gy)
 
-    train_ms, _ = _events_ms(train_step, max(3, args.steps // 4), 3)
+    train_ms, _ = _events_ms(train_step, max(3, min(args.steps // 4, 50)), 3)
     return {"ms": ms, "tflops": flops / ms / 1e9, "flops": flops, "train_ms": train_ms}
 
 
@@ -276,8 +276,8 @@ def copy_calibration(args):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--copies", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-dcn", action="store_true", help="skip the DCN leg")
