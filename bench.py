@@ -91,7 +91,7 @@ def bench_dcn(args, dtype=torch.float16):
 
 
 def bench_other_configs(args):
-    """The remaining measurement configurations of the path on the GPU (HIP events, a few steps
+    """The remaining measurement configurations of the path on the GPU (HIP events, 10 to 200 steps
     each): config 1 rois through the HIP RoIAlign3D, config 2 backward, config 3 (CT resize + 16
     rotated crops), config 5 (detection head: 4000 rois x 256 channels x 7^3) forward / backward.
     GB/s are algorithmic bytes (inputs read once + outputs written once) over the measured time."""
@@ -104,7 +104,7 @@ def bench_other_configs(args):
     feat = torch.randn(2, 16, 32, 64, 64, generator=g).to(dev)
     rois = wl.roi3d_detection(g, 128, 2, (64, 64, 32), (4.0, 24.0)).to(dev)
     out = torch.empty(128, 16, 7, 7, 7, device=dev)
-    ms, _ = _events_ms(lambda i: _C.roi_align_3d_forward(feat, rois, out, 7, 7, 7, 1.0, 2, 1), 20, 3)
+    ms, _ = _events_ms(lambda i: _C.roi_align_3d_forward(feat, rois, out, 7, 7, 7, 1.0, 2, 1), 200, 20)
     res["config1_roialign3d_fp32"] = {"ms": round(ms, 4), "outputs_per_s": round(out.numel() / ms * 1e3, 1)}
     g = wl.gen(1)
     for dt, name in ((torch.float32, "fp32"), (torch.float16, "fp16")):
@@ -112,12 +112,12 @@ def bench_other_configs(args):
         r = wl.affine_rois(g, 4, (128, 128, 128)).to(dev)
         gy = torch.randn(4, 1, 128, 128, 128, generator=g).to(dt).to(dev)
         gi = torch.zeros_like(vol)
-        ms, _ = _events_ms(lambda i: _C.roi_align_rotated_3d_backward(gy, r, gi, 128, 128, 128, 1.0, 1, True, 1), 10, 2)
+        ms, _ = _events_ms(lambda i: _C.roi_align_rotated_3d_backward(gy, r, gi, 128, 128, 128, 1.0, 1, True, 1), 50, 5)
         res["config2_backward_" + name] = {"ms": round(ms, 4)}
     g = wl.gen(2)
     vol = wl.ct_like(g, (2, 1, 256, 512, 512)).to(dev)
     full = torch.tensor([[b, 256, 256, 128, 512, 512, 256, 0, 0, 0] for b in range(2)], dtype=torch.float32).to(dev)
-    ms, _ = _events_ms(lambda i: ops.affine_3d(vol, full, (160, 256, 256), 1.0, 1, True, 1), 10, 2)
+    ms, _ = _events_ms(lambda i: ops.affine_3d(vol, full, (160, 256, 256), 1.0, 1, True, 1), 100, 10)
     nbytes = (vol.numel() + 2 * 160 * 256 * 256) * 2
     res["config3_resize_fp16"] = {"ms": round(ms, 4), "gbps": round(nbytes / ms / 1e6, 1)}
     small = ops.affine_3d(vol, full, (160, 256, 256), 1.0, 1, True, 1)
@@ -127,20 +127,20 @@ def bench_other_configs(args):
             c = torch.rand(3, generator=g) * torch.tensor([256 - 96., 256 - 96., 160 - 96.]) + 48
             crops.append([b, *c.tolist(), 96, 96, 96, 0, 0, (float(torch.rand(1, generator=g)) * 2 - 1) * math.radians(15)])
     crops = torch.tensor(crops).to(dev)
-    ms, _ = _events_ms(lambda i: ops.affine_3d(small, crops, (96, 96, 96), 1.0, 1, True, 1), 10, 2)
+    ms, _ = _events_ms(lambda i: ops.affine_3d(small, crops, (96, 96, 96), 1.0, 1, True, 1), 100, 10)
     res["config3_16_crops_96^3_fp16"] = {"ms": round(ms, 4), "gbps": round(2 * 16 * 96 ** 3 * 2 / ms / 1e6, 1)}
     del vol, small
     g = wl.gen(4)
     feat = torch.randn(2, 256, 24, 96, 96, generator=g).half().to(dev)
     rois = wl.roi3d_detection(g, 4000, 2, (384, 384, 96), (2.0, 48.0), log_uniform=True).to(dev)
     out = torch.empty(4000, 256, 7, 7, 7, dtype=torch.float16, device=dev)
-    ms, _ = _events_ms(lambda i: _C.roi_align_3d_forward(feat, rois, out, 7, 7, 7, 0.25, 2, 1), 5, 1)
+    ms, _ = _events_ms(lambda i: _C.roi_align_3d_forward(feat, rois, out, 7, 7, 7, 0.25, 2, 1), 20, 3)
     nbytes = (feat.numel() + out.numel()) * 2
     res["config5_forward_fp16"] = {"ms": round(ms, 4), "goutputs_s": round(out.numel() / ms / 1e6, 2),
                                    "gbps": round(nbytes / ms / 1e6, 1)}
     gy = torch.randn_like(out)
     gi = torch.zeros_like(feat)
-    ms, _ = _events_ms(lambda i: _C.roi_align_3d_backward(gy, rois, gi, 7, 7, 7, 0.25, 2, 1), 3, 1)
+    ms, _ = _events_ms(lambda i: _C.roi_align_3d_backward(gy, rois, gi, 7, 7, 7, 0.25, 2, 1), 10, 2)
     res["config5_backward_fp16"] = {"ms": round(ms, 4), "gbps": round(nbytes / ms / 1e6, 1)}
     return res
 
