@@ -148,26 +148,26 @@ def bench_other_configs(args):
 def bench_next_rows(args):
     """Short timings of the operators either side of the headline path: order-3 resampling, the
     elastic pipeline (control-grid upsampling + displacement warp), a 2-D DCNv2 layer of FPN size
-    and the augmentation stages that build the rois.  20 steps each, HIP events."""
+    and the augmentation stages that build the rois.  100 steps each (stages 50), HIP events."""
     import numpy as np
     import medvision_amd.ops as ops
     import medvision_amd.aug_cuda as aug
     from medvision_amd.ops.modulated_deform_conv_2d import modulated_deform_conv
     import workloads as wl
-    dev, n = "cuda:0", 20
+    dev, n = "cuda:0", 100
     g = wl.gen(7)
     res = {}
     vol = torch.randn(4, 1, 128, 128, 128, generator=g).half().to(dev)
     rois = wl.affine_rois(g, 4, (128, 128, 128)).to(dev)
-    ms, _ = _events_ms(lambda i: ops.affine_3d(vol, rois, (128, 128, 128), 1.0, 1, True, 3), n, 3)
+    ms, _ = _events_ms(lambda i: ops.affine_3d(vol, rois, (128, 128, 128), 1.0, 1, True, 3), n, 10)
     res["affine_3d_order3_config2"] = {"ms": round(ms, 4), "gvox_s": round(4 * 128 ** 3 / ms / 1e6, 2)}
     grid = torch.randn(2, 3, 8, 8, 8, generator=g).to(dev)
     groi = torch.tensor([[b, 4, 4, 4, 5, 5, 5, 0, 0, 0] for b in range(2)], dtype=torch.float32, device=dev)
-    ms, _ = _events_ms(lambda i: ops.affine_3d(grid, groi, (128, 128, 128), 1, 1, True, 3), n, 3)
+    ms, _ = _events_ms(lambda i: ops.affine_3d(grid, groi, (128, 128, 128), 1, 1, True, 3), n, 10)
     res["elastic_grid_upsample_8to128_order3"] = {"ms": round(ms, 4)}
     field = ops.affine_3d(grid, groi, (128, 128, 128), 1, 1, True, 3).half()
     img = vol[:2]
-    ms, _ = _events_ms(lambda i: ops.apply_offset_3d(img, field, 1), n, 3)
+    ms, _ = _events_ms(lambda i: ops.apply_offset_3d(img, field, 1), n, 10)
     res["apply_offset_3d_2x128^3_fp16"] = {"ms": round(ms, 4), "gvox_s": round(2 * 128 ** 3 / ms / 1e6, 2)}
     B, C, H, W = 8, 256, 100, 152
     x = torch.randn(B, C, H, W, generator=g).half().to(dev)
@@ -175,7 +175,7 @@ def bench_next_rows(args):
     bias = torch.zeros(C, dtype=torch.float16, device=dev)
     off = (torch.randn(B, 18, H, W, generator=g) * 2).half().to(dev)
     msk = torch.sigmoid(torch.randn(B, 9, H, W, generator=g)).half().to(dev)
-    ms, _ = _events_ms(lambda i: modulated_deform_conv(x, off, msk, w, bias, 1, 1, 1, 1, 1), n, 3)
+    ms, _ = _events_ms(lambda i: modulated_deform_conv(x, off, msk, w, bias, 1, 1, 1, 1, 1), n, 10)
     flops = 2 * B * C * C * 9 * H * W
     xs, ws, offs, ms_ = [t.clone().requires_grad_(True) for t in (x, w, off, msk)]
 
@@ -183,7 +183,7 @@ def bench_next_rows(args):
         y = modulated_deform_conv(xs, offs, ms_, ws, bias, 1, 1, 1, 1, 1)
         y.backward(y)
 
-    tms, _ = _events_ms(train, 5, 2)
+    tms, _ = _events_ms(train, 20, 3)
     res["dcnv2_2d_fp16_[8,256,100,152]_3x3"] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 2),
                                                 "forward_backward_ms": round(tms, 3)}
     # augmentation stages on one fp16 CT-sized sample [1, 128, 256, 256] with a label map
@@ -197,7 +197,7 @@ def bench_next_rows(args):
               "CudaCropRandomWithAffine(96^3)": aug.CudaCropRandomWithAffine((96, 96, 96), 0.2, 0.1, 30),
               "CudaRandomElasticDeformation": aug.CudaRandomElasticDeformation(1.0, 8, 0.8)}
     for name, stage in stages.items():
-        ms, wall = _events_ms(lambda i: stage(dict(sample)), 10, 2)
+        ms, wall = _events_ms(lambda i: stage(dict(sample)), 50, 10)
         res["aug:" + name] = {"ms_gpu": round(ms, 3), "ms_wall": round(wall, 3)}
     return res
 
