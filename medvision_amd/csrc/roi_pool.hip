@@ -397,7 +397,13 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
   const T *src = gout + (static_cast<long>(n) * p.C + c_begin) * cells;
   G *dst = gin + (static_cast<long>(sh.g.batch) * p.C + c_begin) * plane;
   G *dst_cl = gin + static_cast<long>(sh.g.batch) * plane * p.C + c_begin;   // CL: voxel v, channel c at v * C + c
-  if (sh.staged == 0) {  // per-output scatter
+  // The transposed contractions below look entries up by source index through `first`, which
+  // holds kPoolEntries + 4 indices: a box wider than that on any axis (few cells spread over many
+  // voxels) takes the per-output scatter, like a box that does not fit LDS.
+  bool wide = false;
+  if (sh.staged == 1)
+    for (int a = 0; a < 3; a++) wide = wide || sh.ax[a].box_hi - sh.ax[a].box_lo + 1 > kPoolEntries + 2;
+  if (sh.staged == 0 || wide) {  // per-output scatter
     const int total = (c_end - c_begin) * cells;
     const int gz = p.ndim == 3 ? sh.g.grid[2] : 1, gy = sh.g.grid[1], gx = sh.g.grid[0];
     for (int i = threadIdx.x; i < total; i += kPoolThreads) {

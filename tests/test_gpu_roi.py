@@ -403,3 +403,25 @@ def test_every_output_element_is_written(ops, oracle, order, out):
     assert not bool(torch.isnan(output).any()) and float(output[1:].abs().max()) == 0.0
     assert_close(output[:1], oracle.roi_align_forward(feat, box[:1], out, 1.0, sr, True, order, False),
                  FWD_TOL[torch.float16], "plain boxes")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_pooled_boxes_wider_than_the_tap_tables(ops, oracle, dtype):
+    """Few cells spread over many voxels: boxes of 70-100 voxels on one axis with 7 cells of 2
+    samples.  The separable backward kernel indexes its tap ranges by source voxel and has to hand
+    such boxes to the per-output scatter."""
+    g = wl.gen(77)
+    img = torch.randn(2, 6, 110, 120, generator=g).to(dtype)
+    rois2 = torch.tensor([[0, 3.0, 5.0, 98.0, 60.0], [1, 10.5, 2.0, 105.0, 101.0], [0, 40.0, 40.0, 47.0, 46.0],
+                          [1, -20.0, 30.0, 70.0, 90.0]])
+    vol = torch.randn(1, 5, 9, 10, 96, generator=g).to(dtype)
+    rois3 = torch.tensor([[0, 2.0, 1.0, 1.0, 88.0, 7.5, 7.0], [0, 10.0, 2.0, 0.5, 93.0, 8.0, 8.5]])
+    for feat, rois, out in ((img, rois2, (7, 7)), (vol, rois3, (7, 7, 7))):
+        mod = ops.RoIAlign(out, 1.0, 2)
+        x = feat.to(DEV).requires_grad_(True)
+        y = mod(x, rois.to(DEV))
+        assert_close(y, oracle.roi_align_forward(feat, rois, out, 1.0, 2, True, 1, False), FWD_TOL[dtype], "forward")
+        gy = torch.randn(y.shape, generator=g).to(dtype)
+        y.backward(gy.to(DEV))
+        want = oracle.roi_align_backward(gy, rois, feat.shape, 1.0, 2, True, 1, False)
+        assert_close(x.grad, want, BWD_TOL[dtype], "backward")
