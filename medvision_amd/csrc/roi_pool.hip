@@ -152,25 +152,27 @@ __device__ inline void pool_setup(PoolShared &sh, const RT *roi, const RoiProble
   __syncthreads();
 }
 
-// Dense form of the tap tables for the usual small boxes (<= kDenseCells cells per axis, box of
+// Dense form of the tap tables for the usual small boxes (<= CELLS cells per axis, box of
 // <= kDenseSrc voxels per axis): per axis a matrix Wd[source index][cell] = sum of the weights of
 // the cell's samples that touch the source index.  A contraction then is "walk the line, multiply
 // each value into all cells" (forward) or "load the cells of a line, one dot product per source
 // index" (backward): no per-entry branches, the matrix rows are LDS broadcasts.
-constexpr int kDenseSrc = 32, kDenseCells = 8;
-typedef float DenseTaps[3][kDenseSrc][kDenseCells];
+// The kernels are instantiated for CELLS = 8 (7^3 detection heads) and 16 (14 x 14 mask heads).
+constexpr int kDenseSrc = 32;
 
+template <int CELLS>
 __device__ __forceinline__ bool dense_applies(const PoolShared &sh, const RoiProblem &p) {
   for (int a = 0; a < 3; a++)
     if (sh.ax[a].box_hi - sh.ax[a].box_lo + 1 > kDenseSrc) return false;
-  return p.ow <= kDenseCells && p.oh <= kDenseCells && p.od <= kDenseCells;
+  return p.ow <= CELLS && p.oh <= CELLS && p.od <= CELLS;
 }
 
 // all threads of the workgroup; followed by a barrier
-__device__ inline void dense_build(const PoolShared &sh, const RoiProblem &p, DenseTaps &wd) {
+template <int CELLS>
+__device__ inline void dense_build(const PoolShared &sh, const RoiProblem &p, float (&wd)[3][kDenseSrc][CELLS]) {
   const int ncell[3] = {p.ow, p.oh, p.od};
-  for (int i = threadIdx.x; i < 3 * kDenseSrc * kDenseCells; i += kPoolThreads) {
-    const int a = i / (kDenseSrc * kDenseCells), src_i = (i / kDenseCells) % kDenseSrc, cell = i % kDenseCells;
+  for (int i = threadIdx.x; i < 3 * kDenseSrc * CELLS; i += kPoolThreads) {
+    const int a = i / (kDenseSrc * CELLS), src_i = (i / CELLS) % kDenseSrc, cell = i % CELLS;
     const AxisTaps &t = sh.ax[a];
     float w = 0.f;
     if (src_i <= t.box_hi - t.box_lo && cell < ncell[a])
@@ -183,15 +185,18 @@ __device__ inline void dense_build(const PoolShared &sh, const RoiProblem &p, De
   __syncthreads();
 }
 
-// acc[k] += Wd row[k] * v for the kDenseCells cells
-__device__ __forceinline__ void dense_axpy(float (&acc)[kDenseCells], const float *row, float v) {
-  const float4 w0 = *reinterpret_cast<const float4 *>(row), w1 = *reinterpret_cast<const float4 *>(row + 4);
-  acc[0] += w0.x * v; acc[1] += w0.y * v; acc[2] += w0.z * v; acc[3] += w0.w * v;
-  acc[4] += w1.x * v; acc[5] += w1.y * v; acc[6] += w1.z * v; acc[7] += w1.w * v;
+// acc[k] += Wd row[k] * v for the CELLS cells
+template <int CELLS>
+__device__ __forceinline__ void dense_axpy(float (&acc)[CELLS], const float *row, float v) {
+  static_assert(CELLS % 4 == 0, "rows are read as 16-byte groups");
+#pragma unroll
+  for (int q = 0; q < CELLS / 4; q++) {
+    const float4 w = *reinterpret_cast<const float4 *>(row + 4 * q);
+    acc[4 * q] += w.x * v; acc[4 * q + 1] += w.y * v; acc[4 * q + 2] += w.z * v; acc[4 * q + 3] += w.w * v;
+  }
 }
-static_assert(kDenseCells == 8, "dense_axpy is written for 8 cells");
 
-template <typename T, typename RT>
+template <typename T, typename RT, int CELLS>
 __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
     const T *__restrict__ feat, const RT *__restrict__ rois, T *__restrict__ out, const RoiProblem p,
     const int channels_per_block) {
@@ -233,9 +238,11 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
   const int ohw = p.oh * p.ow;
   const float inv_vol = 1.f / vol, inv_nxy = 1.f / (nx * ny), inv_nx = 1.f / nx, inv_ow = 1.f / p.ow,
               inv_ohw = 1.f / ohw, inv_cells = 1.f / cells;
-  __shared__ __attribute__((aligned(16))) DenseTaps wd;
-  const bool dense = dense_applies(sh, p);
-  if (dense) dense_build(sh, p, wd);
+  __shared__ __attribute__((aligned(16))) float wd[3][kDenseSrc][CELLS];
+  // (with 9..16 cells per axis a row of the matrix is mostly zeros: the tap-register form below is
+  // faster for the forward pass; the backward pass still gains from the dense form)
+  const bool dense = CELLS == 8 && dense_applies<CELLS>(sh, p);
+  if (dense) dense_build<CELLS>(sh, p, wd);
   for (int cb = c_begin; cb < c_end; cb += sh.chunk) {
     const int cs = min(sh.chunk, c_end - cb);
     T *box = reinterpret_cast<T *>(lds);                                            // [cs][nz][ny][nx]
@@ -268,22 +275,22 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
     if (dense) {
       // x: thread = one (c, z, y) row of the box, all its cells at once
       for (int r = threadIdx.x; r < cs * nz * ny; r += kPoolThreads) {
-        float a[kDenseCells] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        float a[CELLS] = {};
         const T *row = box + r * nx;
         for (int x = 0; x < nx; x++) dense_axpy(a, wd[0][x], load(row + x));
 #pragma unroll
-        for (int k = 0; k < kDenseCells; k++)
+        for (int k = 0; k < CELLS; k++)
           if (k < p.ow) t1[r * p.ow + k] = a[k];
       }
       __syncthreads();
       // y: thread = (c, z, pw)
       for (int i = threadIdx.x; i < cs * nz * p.ow; i += kPoolThreads) {
         const int cz = fdiv(i, inv_ow), pw = i - cz * p.ow;
-        float a[kDenseCells] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        float a[CELLS] = {};
         const float *col = t1 + cz * ny * p.ow + pw;
         for (int yy = 0; yy < ny; yy++) dense_axpy(a, wd[1][yy], col[yy * p.ow]);
 #pragma unroll
-        for (int k = 0; k < kDenseCells; k++)
+        for (int k = 0; k < CELLS; k++)
           if (k < p.oh) t2[cz * ohw + k * p.ow + pw] = a[k];
       }
       __syncthreads();
@@ -291,11 +298,11 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
       T *o = dst + static_cast<long>(cb - c_begin) * cells;
       for (int i = threadIdx.x; i < cs * ohw; i += kPoolThreads) {
         const int c = fdiv(i, inv_ohw), hw = i - c * ohw;
-        float a[kDenseCells] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        float a[CELLS] = {};
         const float *col = t2 + c * nz * ohw + hw;
         for (int zz = 0; zz < nz; zz++) dense_axpy(a, wd[2][zz], col[zz * ohw]);
 #pragma unroll
-        for (int k = 0; k < kDenseCells; k++)
+        for (int k = 0; k < CELLS; k++)
           if (k < p.od) o[c * cells + k * ohw + hw] = store_cast<T>(a[k]);
       }
     } else if (gx <= kTapRegs && gy <= kTapRegs && gz <= kTapRegs) {
@@ -381,7 +388,7 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
 // CL: the accumulation buffer is channels-last [N, D*H*W, C] (the fp32 workspace of the 16-bit
 // path): the lanes of a wavefront then add neighbouring channels of a voxel, contiguous bytes,
 // instead of one element in each of many rows (a scattered atomic moves a whole memory sector).
-template <typename T, typename G, typename RT, bool CL>
+template <typename T, typename G, typename RT, bool CL, int CELLS>
 __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
     const T *__restrict__ gout, const RT *__restrict__ rois, G *__restrict__ gin, const RoiProblem p,
     const int channels_per_block) {
@@ -434,9 +441,9 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
   const float inv_vol = 1.f / vol, inv_nxy = 1.f / (nx * ny), inv_nx = 1.f / nx, inv_ow = 1.f / p.ow,
               inv_ohw = 1.f / ohw, inv_nzohw = 1.f / (nz * ohw), inv_nyow = 1.f / (ny * p.ow),
               inv_gx = 1.f / gx, inv_gy = 1.f / gy, inv_gz = 1.f / gz;
-  __shared__ __attribute__((aligned(16))) DenseTaps wd;
-  if (dense_applies(sh, p)) {
-    dense_build(sh, p, wd);
+  __shared__ __attribute__((aligned(16))) float wd[3][kDenseSrc][CELLS];
+  if (dense_applies<CELLS>(sh, p)) {
+    dense_build<CELLS>(sh, p, wd);
     const float inv_ow = 1.f / p.ow;
     for (int cb = c_begin; cb < c_end; cb += sh.chunk) {
       const int cs = min(sh.chunk, c_end - cb);
@@ -448,13 +455,13 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
       // z: thread = (c, ph, pw); its grad_output values stay in registers
       for (int i = threadIdx.x; i < cs * ohw; i += kPoolThreads) {
         const int c = fdiv(i, inv_ohw), hw = i - c * ohw;
-        float g[kDenseCells];
+        float g[CELLS];
 #pragma unroll
-        for (int k = 0; k < kDenseCells; k++) g[k] = k < p.od ? load(go + c * cells + k * ohw + hw) : 0.f;
+        for (int k = 0; k < CELLS; k++) g[k] = k < p.od ? load(go + c * cells + k * ohw + hw) : 0.f;
         for (int z = 0; z < nz; z++) {
           float acc = 0.f;
 #pragma unroll
-          for (int k = 0; k < kDenseCells; k++) acc += wd[2][z][k] * g[k];
+          for (int k = 0; k < CELLS; k++) acc += wd[2][z][k] * g[k];
           t2[(c * nz + z) * ohw + hw] = acc;
         }
       }
@@ -463,13 +470,13 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
       for (int i = threadIdx.x; i < cs * nz * p.ow; i += kPoolThreads) {
         const int cz = fdiv(i, inv_ow), pw = i - cz * p.ow;
         const int c = fdiv(cz, 1.f / nz), z = cz - c * nz;
-        float g[kDenseCells];
+        float g[CELLS];
 #pragma unroll
-        for (int k = 0; k < kDenseCells; k++) g[k] = k < p.oh ? t2[cz * ohw + k * p.ow + pw] : 0.f;
+        for (int k = 0; k < CELLS; k++) g[k] = k < p.oh ? t2[cz * ohw + k * p.ow + pw] : 0.f;
         for (int y = 0; y < ny; y++) {
           float acc = 0.f;
 #pragma unroll
-          for (int k = 0; k < kDenseCells; k++) acc += wd[1][y][k] * g[k];
+          for (int k = 0; k < CELLS; k++) acc += wd[1][y][k] * g[k];
           t1[(CL ? ((z * ny + y) * cs + c) : (cz * ny + y)) * p.ow + pw] = acc;
         }
       }
@@ -479,26 +486,26 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
       if (CL) {   // channel fastest across the lanes: a wavefront adds runs of cs contiguous floats
         for (int i = threadIdx.x; i < cs * nz * ny; i += kPoolThreads) {
           const int zy = fdiv(i, inv_cs), c = i - zy * cs, z = fdiv(zy, 1.f / ny), y = zy - z * ny;
-          float g[kDenseCells];
+          float g[CELLS];
 #pragma unroll
-          for (int k = 0; k < kDenseCells; k++) g[k] = k < p.ow ? t1[i * p.ow + k] : 0.f;
+          for (int k = 0; k < CELLS; k++) g[k] = k < p.ow ? t1[i * p.ow + k] : 0.f;
           G *row = dst_cl + (first + (static_cast<long>(z) * p.H + y) * p.W) * p.C + (cb - c_begin) + c;
           for (int x = 0; x < nx; x++) {
             float acc = 0.f;
 #pragma unroll
-            for (int k = 0; k < kDenseCells; k++) acc += wd[0][x][k] * g[k];
+            for (int k = 0; k < CELLS; k++) acc += wd[0][x][k] * g[k];
             if (acc != 0.f) atomic_add(row + static_cast<long>(x) * p.C, static_cast<G>(acc));
           }
         }
       } else {    // through LDS, so that the lanes of a wavefront add runs of nx contiguous elements
         for (int i = threadIdx.x; i < cs * nz * ny; i += kPoolThreads) {
-          float g[kDenseCells];
+          float g[CELLS];
 #pragma unroll
-          for (int k = 0; k < kDenseCells; k++) g[k] = k < p.ow ? t1[i * p.ow + k] : 0.f;
+          for (int k = 0; k < CELLS; k++) g[k] = k < p.ow ? t1[i * p.ow + k] : 0.f;
           for (int x = 0; x < nx; x++) {
             float acc = 0.f;
 #pragma unroll
-            for (int k = 0; k < kDenseCells; k++) acc += wd[0][x][k] * g[k];
+            for (int k = 0; k < CELLS; k++) acc += wd[0][x][k] * g[k];
             gbox[i * nx + x] = acc;
           }
         }
@@ -595,27 +602,44 @@ static int pool_channels_per_block(const RoiProblem &p) {
   return cpb;
 }
 
+template <typename T, int CELLS>
+static void launch_pool_forward(const void *input, const float *r, void *output, const RoiProblem &p, int cpb,
+                                dim3 grid, hipStream_t s) {
+  hipLaunchKernelGGL((roi_pool_forward_kernel<T, float, CELLS>), grid, dim3(kPoolThreads), 0, s,
+                     static_cast<const T *>(input), r, static_cast<T *>(output), p, cpb);
+}
+
+template <typename T, bool CL, int CELLS>
+static void launch_pool_backward(const void *grad_output, const float *r, void *acc, const RoiProblem &p, int cpb,
+                                 dim3 grid, hipStream_t s) {
+  hipLaunchKernelGGL((roi_pool_backward_kernel<T, float, float, CL, CELLS>), grid, dim3(kPoolThreads), 0, s,
+                     static_cast<const T *>(grad_output), r, static_cast<float *>(acc), p, cpb);
+}
+
+// dense-matrix width of the kernel instance: 8 cells per axis when the output allows it
+static bool pool_small_cells(const RoiProblem &p) { return p.od <= 8 && p.oh <= 8 && p.ow <= 8; }
+
 int roi_pool_forward(const void *input, const void *rois, void *output, int dtype,
                      const RoiProblem &p, hipStream_t s) {
   if (!pool_applies(dtype, p)) return -1;
   const int cpb = pool_channels_per_block(p);
   const long cblocks = (p.C + cpb - 1) / cpb;
   if (cblocks > 65535) return -1;
-  const dim3 grid(p.R, static_cast<unsigned>(cblocks)), block(kPoolThreads);
+  const dim3 grid(p.R, static_cast<unsigned>(cblocks));
   const float *r = static_cast<const float *>(rois);
+  const bool small = pool_small_cells(p);
   switch (dtype) {
     case MV_F32:
-      hipLaunchKernelGGL((roi_pool_forward_kernel<float, float>), grid, block, 0, s,
-                         static_cast<const float *>(input), r, static_cast<float *>(output), p, cpb);
+      small ? launch_pool_forward<float, 8>(input, r, output, p, cpb, grid, s)
+            : launch_pool_forward<float, 16>(input, r, output, p, cpb, grid, s);
       break;
     case MV_F16:
-      hipLaunchKernelGGL((roi_pool_forward_kernel<__half, float>), grid, block, 0, s,
-                         static_cast<const __half *>(input), r, static_cast<__half *>(output), p, cpb);
+      small ? launch_pool_forward<__half, 8>(input, r, output, p, cpb, grid, s)
+            : launch_pool_forward<__half, 16>(input, r, output, p, cpb, grid, s);
       break;
     default:
-      hipLaunchKernelGGL((roi_pool_forward_kernel<__hip_bfloat16, float>), grid, block, 0, s,
-                         static_cast<const __hip_bfloat16 *>(input), r,
-                         static_cast<__hip_bfloat16 *>(output), p, cpb);
+      small ? launch_pool_forward<__hip_bfloat16, 8>(input, r, output, p, cpb, grid, s)
+            : launch_pool_forward<__hip_bfloat16, 16>(input, r, output, p, cpb, grid, s);
   }
   return check_launch("roi_pool_forward_kernel");
 }
@@ -630,30 +654,26 @@ int roi_pool_backward(const void *grad_output, const void *rois, void *acc, int 
   const int cpb = pool_channels_per_block(p);
   const long cblocks = (p.C + cpb - 1) / cpb;
   if (cblocks > 65535) return -1;
-  const dim3 grid(p.R, static_cast<unsigned>(cblocks)), block(kPoolThreads);
+  const dim3 grid(p.R, static_cast<unsigned>(cblocks));
   const float *r = static_cast<const float *>(rois);
+  const bool small = pool_small_cells(p);
+#define MV_POOL_BACKWARD(TYPE, CLV)                                                          \
+  (small ? launch_pool_backward<TYPE, CLV, 8>(grad_output, r, acc, p, cpb, grid, s)          \
+         : launch_pool_backward<TYPE, CLV, 16>(grad_output, r, acc, p, cpb, grid, s))
   switch (dtype) {
     case MV_F32:
       if (channels_last) return fail(MV_INVALID_ARGUMENT, "channels-last accumulation is for 16-bit tensors");
-      hipLaunchKernelGGL((roi_pool_backward_kernel<float, float, float, false>), grid, block, 0, s,
-                         static_cast<const float *>(grad_output), r, static_cast<float *>(acc), p, cpb);
+      MV_POOL_BACKWARD(float, false);
       break;
     case MV_F16:
-      if (channels_last)
-        hipLaunchKernelGGL((roi_pool_backward_kernel<__half, float, float, true>), grid, block, 0, s,
-                           static_cast<const __half *>(grad_output), r, static_cast<float *>(acc), p, cpb);
-      else
-        hipLaunchKernelGGL((roi_pool_backward_kernel<__half, float, float, false>), grid, block, 0, s,
-                           static_cast<const __half *>(grad_output), r, static_cast<float *>(acc), p, cpb);
+      if (channels_last) MV_POOL_BACKWARD(__half, true);
+      else MV_POOL_BACKWARD(__half, false);
       break;
     default:
-      if (channels_last)
-        hipLaunchKernelGGL((roi_pool_backward_kernel<__hip_bfloat16, float, float, true>), grid, block, 0, s,
-                           static_cast<const __hip_bfloat16 *>(grad_output), r, static_cast<float *>(acc), p, cpb);
-      else
-        hipLaunchKernelGGL((roi_pool_backward_kernel<__hip_bfloat16, float, float, false>), grid, block, 0, s,
-                           static_cast<const __hip_bfloat16 *>(grad_output), r, static_cast<float *>(acc), p, cpb);
+      if (channels_last) MV_POOL_BACKWARD(__hip_bfloat16, true);
+      else MV_POOL_BACKWARD(__hip_bfloat16, false);
   }
+#undef MV_POOL_BACKWARD
   return check_launch("roi_pool_backward_kernel");
 }
 

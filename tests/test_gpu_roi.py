@@ -425,3 +425,23 @@ def test_pooled_boxes_wider_than_the_tap_tables(ops, oracle, dtype):
         y.backward(gy.to(DEV))
         want = oracle.roi_align_backward(gy, rois, feat.shape, 1.0, 2, True, 1, False)
         assert_close(x.grad, want, BWD_TOL[dtype], "backward")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_pooled_heads_with_9_to_16_cells(ops, oracle, dtype):
+    """14 x 14 mask heads and a 10 x 12 x 14 volume head: the pooled kernels' 16-cell instance
+    (dense per-axis matrices in the backward pass, tap registers in the forward pass)."""
+    g = wl.gen(78)
+    img = torch.randn(2, 9, 40, 52, generator=g).to(dtype)
+    rois2 = wl.roi3d_detection(g, 12, 2, (52, 40, 1), (5.0, 28.0))[:, [0, 1, 2, 4, 5]]
+    vol = torch.randn(2, 5, 14, 20, 24, generator=g).to(dtype)
+    rois3 = wl.roi3d_detection(g, 8, 2, (24, 20, 14), (4.0, 14.0))
+    for feat, rois, out, sr in ((img, rois2, (14, 14), 2), (vol, rois3, (10, 12, 14), 2), (img, rois2, (14, 9), 0)):
+        mod = ops.RoIAlign(out, 1.0, sr)
+        x = feat.to(DEV).requires_grad_(True)
+        y = mod(x, rois.to(DEV))
+        assert_close(y, oracle.roi_align_forward(feat, rois, out, 1.0, sr, True, 1, False), FWD_TOL[dtype], "forward")
+        gy = torch.randn(y.shape, generator=g).to(dtype)
+        y.backward(gy.to(DEV))
+        want = oracle.roi_align_backward(gy, rois, feat.shape, 1.0, sr, True, 1, False)
+        assert_close(x.grad, want, BWD_TOL[dtype], "backward")
