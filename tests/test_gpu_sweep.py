@@ -249,3 +249,36 @@ def test_resampling_backward_sweep(ops, oracle):
             # no atomics, fp32 sums, one rounding per voxel: 16-bit results carry half an ulp
             tol = BWD_TOL[dtype] if dtype in (torch.float32, torch.float64) else FWD_TOL[dtype]
             assert rel_err(fg.grad, want) <= tol, what
+
+
+def test_pooled_sweep(ops, oracle):
+    """Plain boxes with at most 16 cells per axis (the pooled kernels): boxes from a fraction of a
+    voxel to more than a hundred voxels wide, elongated volumes, fixed and adaptive sampling grids."""
+    for seed in range(9600, 9750):
+        rnd = random.Random(seed)
+        g = torch.Generator().manual_seed(seed)
+        ndim = rnd.choice([2, 3])
+        size = [rnd.randint(1, 130) for _ in range(2)] if ndim == 2 else \
+            [rnd.randint(1, 20), rnd.randint(1, 40), rnd.randint(1, 110)]
+        batch, channels = rnd.randint(1, 2), rnd.choice([1, 2, 3, 7, 40])
+        dtype = rnd.choice([torch.float32, torch.float16, torch.bfloat16])
+        out = tuple(rnd.randint(1, 16) for _ in range(ndim))
+        n = rnd.randint(1, 6)
+        scale = rnd.choice([0.25, 0.5, 1.0, 1.0])
+        sr = rnd.choice([-1, 0, 1, 2, 2, 3, 4])
+        feat = torch.randn(batch, channels, *size, generator=g).to(dtype)
+        ext = torch.tensor(size[::-1], dtype=torch.float32) / scale
+        rois = torch.zeros(n, 1 + 2 * ndim)
+        rois[:, 0] = torch.randint(0, batch, (n,), generator=g)
+        lo = (torch.rand(n, ndim, generator=g) * 1.3 - 0.2) * ext
+        rois[:, 1:1 + ndim] = lo
+        rois[:, 1 + ndim:] = lo + torch.rand(n, ndim, generator=g) * ext * rnd.choice([0.1, 0.5, 1.0, 1.5])
+        what = f"seed {seed}: {ndim}-D {tuple(feat.shape)} -> {out} rois={n} scale={scale} sr={sr} {dtype}"
+        fg = feat.to(DEV).requires_grad_(True)
+        got = ops.RoIAlign(out, scale, sr)(fg, rois.to(DEV))
+        want = oracle.roi_align_forward(feat, rois, out, scale, sr, True, 1, False)
+        assert rel_err(got, want) <= FWD_TOL[dtype], what
+        gy = torch.randn(got.shape, generator=g).to(dtype)
+        got.backward(gy.to(DEV))
+        gwant = oracle.roi_align_backward(gy, rois, feat.shape, scale, sr, True, 1, False)
+        assert rel_err(fg.grad, gwant) <= BWD_TOL[dtype], what + " (backward)"
