@@ -304,13 +304,14 @@ def main():
         "value": round(a16["gvox_s"], 3), "unit": "Gvox/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(a16["ms"], 6), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f16 storage; f32 interpolation and per-voxel coordinates; f64 roi geometry",
+        "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": "BASELINE config 2: RoIAlignRotated3D as RandomAffine resampling, "
                                "volume fp16 [4,1,128,128,128] N(0,1), one full-volume roi per sample, "
                                "angles U(+-30deg), scale U(0.8,1.2), shift +-10 vox, out 128^3, "
                                "sampling_ratio 1, aligned, order 1",
-                   "buffer_sets": args.copies},
+                   "buffer_sets": args.copies, "storage": "f16",
+                   "arithmetic": "f32 interpolation and per-voxel coordinates, f64 roi geometry"},
         "roofline": {"bound": "hbm", "achieved": round(a16["gbps"], 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(a16["gbps"] / HBM_PEAK_GBPS, 4), "traffic": None,
                      "kernel": "roi_resample_kernel", "algorithmic_bytes_per_launch": a16["alg_bytes"],
