@@ -1,7 +1,7 @@
 #!/usr/bin/env python
 """Benchmark of the trilinear-sampling hot path on one MI355X.
 
-A "step" is one RoIAlignRotated3D forward over one batch of BASELINE config 2 (fp16 volume
+A "step" is one RoIAlignRotated3D forward over one batch of benchmark configuration 2 (fp16 volume
 [4,1,128^3] -> 128^3, one rotated full-volume roi per sample, sampling_ratio 1), inputs resident in
 HBM.  ``value`` is output Gvox/s.  Inputs/outputs rotate over ``--copies`` buffer sets (default 16,
 ~540 MB) so that consecutive steps are not served from the 256 MB Infinity Cache.  The same JSON

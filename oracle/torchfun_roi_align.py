@@ -1,4 +1,4 @@
-"""TEST / BASELINE INFRASTRUCTURE ONLY: restatement of the reference's pure-torch RoIAlign.
+"""TEST AND CPU-BASELINE INFRASTRUCTURE ONLY: restatement of the reference's pure-torch RoIAlign.
 
 Follows ``medvision/ops/pytorch_ops/roi_align.py:22-105`` (class ``RoIAlign``): fp32 only, one
 sample per output cell (``sampling_ratio`` is ignored), boxes DIVIDED by ``spatial_scale``, a Python

@@ -55,7 +55,7 @@ def test_functions_vs_oracle(ops, oracle, dtype, modulated, groups, dg, stride, 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 def test_config4_reduced_vs_oracle(ops, oracle, dtype):
-    """BASELINE config 4 channel / kernel geometry (Cin 32, Cout 64, 3^3, pad 1, dg 1,
+    """Benchmark configuration 4 channel / kernel geometry (Cin 32, Cout 64, 3^3, pad 1, dg 1,
     offsets N(0,2), sigmoid mask) on a 12x12x16 volume so the CPU oracle finishes in seconds."""
     from medvision_amd.ops.modulated_deform_conv_3d import modulated_deform_conv
     g = wl.gen(3)

@@ -127,7 +127,7 @@ def test_edge_cases_and_errors(ops):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 def test_config2_affine_resampling_full_size(ops, oracle, dtype):
-    """BASELINE config 2: [4,1,128^3] -> 128^3, one rotated full-volume roi per sample, sr=1."""
+    """Benchmark configuration 2: [4,1,128^3] -> 128^3, one rotated full-volume roi per sample, sr=1."""
     g = wl.gen(1)
     vol = torch.randn(4, 1, 128, 128, 128, generator=g).to(dtype)
     rois = wl.affine_rois(g, 4, (128, 128, 128))
@@ -166,7 +166,7 @@ def test_config2_backward_adjoint_full_size(ops, oracle):
 
 
 def test_config3_resize_and_crops(ops, oracle):
-    """BASELINE config 3 at reduced size: CT-like fp16 volume, resize then rotated 3-D crops."""
+    """Benchmark configuration 3 at reduced size: CT-like fp16 volume, resize then rotated 3-D crops."""
     g = wl.gen(2)
     vol = wl.ct_like(g, (2, 1, 64, 128, 128))
     full = torch.tensor([[b, 64, 64, 32, 128, 128, 64, 0, 0, 0] for b in range(2)], dtype=torch.float32)
@@ -268,7 +268,7 @@ def test_cubic_resize_larger_volume(ops, oracle):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 def test_config5_detection_head_reduced(ops, oracle, dtype):
-    """BASELINE config 5 shape family (log-uniform extents, scale 0.25, 7^3, sr=2), reduced."""
+    """Benchmark configuration 5 shape family (log-uniform extents, scale 0.25, 7^3, sr=2), reduced."""
     g = wl.gen(4)
     feat = torch.randn(2, 16, 12, 48, 48, generator=g).to(dtype)
     rois = wl.roi3d_detection(g, 200, 2, (192, 192, 48), (2.0, 48.0), log_uniform=True)
@@ -321,7 +321,7 @@ def test_pooled_kernel_paths(ops, oracle, dtype, sr, order):
 
 
 def test_config1_rois_on_gpu(ops, oracle):
-    """BASELINE config 1 inputs (fp32 [2,16,32,64,64], 128 rois, 7^3, sr=2) through RoIAlign3D."""
+    """Benchmark configuration 1 inputs (fp32 [2,16,32,64,64], 128 rois, 7^3, sr=2) through RoIAlign3D."""
     g = wl.gen(0)
     feat = torch.randn(2, 16, 32, 64, 64, generator=g)
     rois = wl.roi3d_detection(g, 128, 2, (64, 64, 32), (4.0, 24.0))
