@@ -445,3 +445,62 @@ def test_pooled_heads_with_9_to_16_cells(ops, oracle, dtype):
         y.backward(gy.to(DEV))
         want = oracle.roi_align_backward(gy, rois, feat.shape, 1.0, sr, True, 1, False)
         assert_close(x.grad, want, BWD_TOL[dtype], "backward")
+
+
+def test_config3_full_size_properties(ops):
+    """Benchmark configuration 3 at its full size (fp16 [2,1,256,512,512] -> 160x256x256, then 16
+    crops of 96^3): properties that need no oracle run.  A constant volume stays constant under
+    resize and rotated crops (weights sum to one wherever no sample is void); crops with zero
+    angles on whole-voxel centres are slices of the resized volume; resizing is linear."""
+    g = wl.gen(2)
+    vol = wl.ct_like(g, (2, 1, 256, 512, 512)).to(DEV)
+    full = torch.tensor([[b, 256, 256, 128, 512, 512, 256, 0, 0, 0] for b in range(2)], dtype=torch.float32, device=DEV)
+    small = ops.affine_3d(vol, full, (160, 256, 256), 1.0, 1, True, 1)
+    const = torch.full_like(vol, 3.25)
+    assert torch.equal(ops.affine_3d(const, full, (160, 256, 256), 1.0, 1, True, 1), torch.full_like(small, 3.25))
+    twice = ops.affine_3d(vol * 2, full, (160, 256, 256), 1.0, 1, True, 1)   # exact: powers of two
+    assert torch.equal(twice, small * 2)
+    lo = torch.tensor([[30, 40, 20], [100, 17, 60]])
+    crops = torch.tensor([[b, lo[b, 0] + 48, lo[b, 1] + 48, lo[b, 2] + 48, 96, 96, 96, 0, 0, 0] for b in range(2)],
+                         dtype=torch.float32, device=DEV)
+    got = ops.affine_3d(small, crops, (96, 96, 96), 1.0, 1, True, 1)
+    for b in range(2):
+        x, y, z = lo[b].tolist()
+        assert torch.equal(got[b, 0], small[b, 0, z:z + 96, y:y + 96, x:x + 96])
+    rot = crops.clone()
+    rot[:, 9] = torch.tensor([0.2, -0.25])
+    csmall = torch.full_like(small, -7.5)
+    assert torch.equal(ops.affine_3d(csmall, rot, (96, 96, 96), 1.0, 1, True, 1),
+                       torch.full((2, 1, 96, 96, 96), -7.5, dtype=torch.float16, device=DEV))
+
+
+def test_config5_full_size_properties(ops):
+    """Benchmark configuration 5 at its full size (fp16 [2,256,24,96,96], 4000 rois, 7^3, sr 2,
+    scale 0.25): a constant feature map pools to the constant (all boxes lie inside the volume),
+    pooling is linear, and the backward pass conserves the gradient mass per image and channel."""
+    g = wl.gen(4)
+    rois = wl.roi3d_detection(g, 4000, 2, (384, 384, 96), (2.0, 48.0), log_uniform=True)
+    feat = torch.randn(2, 256, 24, 96, 96, generator=g).half().to(DEV)
+    mod = ops.RoIAlign((7, 7, 7), 0.25, 2)
+    r = rois.to(DEV)
+    # boxes narrower than one voxel are widened to one and may then reach beyond the volume, where
+    # samples are void: 16 of the 4000; the properties below hold for the others
+    lo, hi = rois[:, 1:4] * 0.25, rois[:, 4:7] * 0.25
+    inside = ((lo + (hi - lo).clamp(min=1.0)) <= torch.tensor([96.0, 96.0, 24.0])).all(dim=1)
+    assert int(inside.sum()) >= 3950
+    const = mod(torch.full_like(feat, 1.5), r)
+    assert float((const[inside.to(DEV)].float() - 1.5).abs().max()) <= 1.5 * 2 ** -10   # one fp16 rounding of the sum
+    x = feat.clone().requires_grad_(True)
+    y = mod(x, r)
+    assert_close(mod(feat * 2, r), y.detach() * 2, 1e-6, "linearity")
+    gy = torch.randn(y.shape, generator=g).half()
+    gy[~inside] = 0
+    gy = gy.to(DEV)
+    y.backward(gy)
+    # every sample lies inside the volume: each output's gradient is spread with weights summing to 1
+    for b in range(2):
+        pick = (rois[:, 0] == b).to(DEV)
+        want = gy[pick].double().sum(dim=(0, 2, 3, 4))
+        got = x.grad[b].double().sum(dim=(1, 2, 3))
+        scale = float(gy[pick].double().abs().sum(dim=(0, 2, 3, 4)).max())
+        assert float((got - want).abs().max()) <= 2e-3 * scale   # fp16 rounding of 1.8 M accumulated cells
