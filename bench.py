@@ -339,7 +339,10 @@ def main():
         line["cpu_reference_paths"] = cpu_reference_paths(args)
     traffic = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(traffic):   # HBM bytes per launch measured with rocprofv3 --pmc (see profiles/)
-        line["roofline"]["traffic"] = json.load(open(traffic)).get("roi_resample_fp16_config2")
+        measured = json.load(open(traffic))
+        line["roofline"]["traffic"] = measured.get("roi_resample_fp16_config2")
+        if "dcn" in line:
+            line["dcn"]["roofline"]["traffic"] = measured.get("dcn_forward_mfma16_fp16_config4")
     print(json.dumps(line))
 
 
