@@ -82,4 +82,12 @@ __device__ __forceinline__ void atomic_add(double *p, double v) { unsafeAtomicAd
 
 constexpr int kWave = 64;
 
+// Workgroup ids are dealt round-robin to the 8 XCDs, each with an L2 of its own.  This renumbering
+// hands every XCD one contiguous eighth of a grid's x range (the ids beyond the last multiple of 8
+// keep their place), so that workgroups sharing an L2 work on neighbouring data.
+__device__ __forceinline__ unsigned xcd_contiguous(unsigned id, unsigned count) {
+  const unsigned per_xcd = count / 8;
+  return id < per_xcd * 8 ? (id % 8) * per_xcd + id / 8 : id;
+}
+
 }  // namespace mv

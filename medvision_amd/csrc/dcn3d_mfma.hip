@@ -113,7 +113,7 @@ __global__ __launch_bounds__(256, MT <= 2 ? 4 : 3) void dcn_forward_mfma_kernel(
   constexpr int PC = M::kPiece, SL = 2 * PC, ES = sizeof(T);
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int n = lane % 32, h = lane / 32;
-  const long q0 = (static_cast<long>(blockIdx.x) * 4 + wave) * 32;
+  const long q0 = (static_cast<long>(xcd_contiguous(blockIdx.x, gridDim.x)) * 4 + wave) * 32;
   if (q0 >= s.Q) return;  // whole wave idle (no barriers in this kernel)
   const long q = q0 + n;
   const bool live = q < s.Q;
@@ -255,7 +255,9 @@ __global__ __launch_bounds__(256, NB == 1 ? (NC == 4 && WBYTES <= 12 * 1024 ? MV
   const int j = lane % 16, kc = lane / 16;   // matrix layout: position (column) and piece of this lane
   const int lj = lane / 4, lk = lane % 4;    // load layout
   const int from = (4 * j + kc) * 4;         // ds_bpermute byte address of the lane holding this lane's piece
-  const long q0 = (static_cast<long>(blockIdx.x) * 4 + wave) * (NB * 16);
+  // every XCD takes one contiguous eighth of the positions: its L2 then holds an eighth of the
+  // input (plus the reach of the offsets) instead of every XCD streaming the whole volume
+  const long q0 = (static_cast<long>(xcd_contiguous(blockIdx.x, gridDim.x)) * 4 + wave) * (NB * 16);
   const int slices = s.cpg / SL, blocks = s.opg / 16;
   const int chunks = (blocks + MB - 1) / MB;
   const int g = blockIdx.y / chunks, mb0 = (blockIdx.y % chunks) * MB;

@@ -81,7 +81,8 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
   __shared__ float sums[4][4][32];
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int n = lane % 32, h = lane / 32;
-  const long q0 = (static_cast<long>(blockIdx.x) * 4 + wave) * 32;
+  // one contiguous eighth of the positions per XCD (see xcd_contiguous)
+  const long q0 = (static_cast<long>(xcd_contiguous(blockIdx.x, gridDim.x)) * 4 + wave) * 32;
   if (q0 >= s.Q) return;  // whole wavefront idle (no workgroup barriers in this kernel)
   const long q = q0 + n;
   const bool live = q < s.Q;
