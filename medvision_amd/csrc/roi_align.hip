@@ -66,7 +66,10 @@ __global__ __launch_bounds__(kRoiThreads) void roi_backward_kernel(const T *__re
   using A = typename Acc<T>::type;
   __shared__ RoiGeom g;
   __shared__ double trig[6];
-  const unsigned n = blockIdx.x / p.chunks, chunk = blockIdx.x % p.chunks;
+  // a contiguous eighth of the chunks per XCD: the atomics of neighbouring chunks then meet in
+  // fewer places at a time (11 % faster on large outputs; the forward kernel lost by it)
+  const unsigned wg = xcd_contiguous(blockIdx.x, gridDim.x);
+  const unsigned n = wg / p.chunks, chunk = wg % p.chunks;
   build_geom_block(g, trig, rois + static_cast<long>(n) * roi_columns(p.ndim, p.rotated), p);
   if (g.batch < 0) return;
   const unsigned begin = chunk * kRoiChunk;
