@@ -2,7 +2,8 @@
 // cores and channels-last buffers.
 //
 //   gcol[c, k, q] = sum_o Wt[o, c, k] * gy[o, q]                    (GEMM, MFMA)
-//   gx[corner_n(k, q), c] += w_n * mask * gcol                       (scatter, fp32 atomics)
+//   gx[corner_n(k, q), c] += w_n * mask * gcol                       (scatter: fp32 atomics, and for
+//                                                                     unit-stride 3^3 layers LDS tiles)
 //   goff_a[k, q] = mask * sum_c gcol * dZ/dp_a ,  gmask[k, q] = sum_c gcol * Z
 //   gw[o, c, k]  = sum_{b, q} gy[o, q] * col[c, k, q]                (GEMM over positions, MFMA)
 //
@@ -13,6 +14,9 @@
 // x (for the offset / mask gradients) and the fp32 atomic adds into the channels-last gradient
 // buffer are 64- and 128-byte contiguous.  The four per-position sums over channels are reduced
 // across the half-wavefront with DPP adds.
+// Scatter kernel (layers whose taps fit its tile): the corners that land near their position are
+// summed per brick of positions in a 64-bit fixed-point LDS tile and reach the gradient buffer as
+// one atomic per (voxel, channel) of the tile; the data kernel then adds only the other corners.
 // Weight kernel: a workgroup owns (tap, 32-channel block, range of positions); lanes rebuild the
 // column values of their channel for 16 positions at a time (same coalesced corner reads), which
 // is exactly the MFMA B fragment; A is gy read in its own layout.  Accumulators stay in registers
@@ -67,13 +71,105 @@ __device__ __forceinline__ float half_wave_sum(float v) {
   return v;
 }
 
-constexpr int kTapWords = 20;  // vox[8], w[8], mask, ld, lh, lw
+// ---- bricks and tiles of the LDS scatter (dcn_backward_scatter_kernel below) ----------------------
+// A brick is kSbD x kSbH x kSbW output positions; its tile the kStD x kStH x kStW input voxels
+// centred on the reach of the brick's undeformed taps.  A corner is "local" when its voxel lies in
+// the tile of its position's brick: local corners are summed in LDS by the scatter kernel, all
+// others are added to the gradient buffer by the data kernel, 128 bytes per request.
+constexpr int kSbD = 4, kSbH = 8, kSbW = 8;
+constexpr int kStD = 10, kStH = 14, kStW = 14;
+constexpr int kStVox = kStD * kStH * kStW;
+struct TileOrigin { int d, h, w; };
+__device__ __forceinline__ TileOrigin tile_origin(const DcnDims &s, int bz, int by, int bx) {
+  TileOrigin t;
+  t.d = bz * kSbD * s.sd - s.pd - (kStD - ((kSbD - 1) * s.sd + (s.kd - 1) * s.dd + 1)) / 2;
+  t.h = by * kSbH * s.sh - s.ph - (kStH - ((kSbH - 1) * s.sh + (s.kh - 1) * s.dh + 1)) / 2;
+  t.w = bx * kSbW * s.sw - s.pw - (kStW - ((kSbW - 1) * s.sw + (s.kw - 1) * s.dw + 1)) / 2;
+  return t;
+}
+// bit c: corner c (z-major) of the sample whose first corner is voxel (id, ih, iw) lies in the tile;
+// `first` its cell index there
+__device__ __forceinline__ unsigned tile_bits(const TileOrigin &t, int id, int ih, int iw, int &first) {
+  const int zd = id - t.d, zh = ih - t.h, zw = iw - t.w;
+  const bool fd[2] = {zd >= 0 && zd < kStD, zd >= -1 && zd < kStD - 1};
+  const bool fh[2] = {zh >= 0 && zh < kStH, zh >= -1 && zh < kStH - 1};
+  const bool fw[2] = {zw >= 0 && zw < kStW, zw >= -1 && zw < kStW - 1};
+  unsigned bits = 0;
+#pragma unroll
+  for (int c = 0; c < 8; c++) bits |= (fd[c >> 2] && fh[(c >> 1) & 1] && fw[c & 1]) ? 1u << c : 0u;
+  first = (zd * kStH + zh) * kStW + zw;
+  return bits;
+}
 
+// The LDS sums are 64-bit fixed point (LDS float atomics retire one lane at a time, integer ones
+// a wavefront in a few clocks).  Every term is w * mask * gcol with 0 <= w <= 1, so
+//   |term| <= max|mask| * max|grad_output| * max_{c,k} sum_o |Wt[o,c,k]|  =: bound < 2^ex,
+// and a voxel takes at most one corner of each (position, tap) of the brick.  Terms are scaled by
+// 2^(50 - ex) and rounded to integers (adding 1.5 * 2^52 in fp64 leaves round(x) in the low
+// mantissa bits for |x| < 2^51): a term loses less than 2^-49 of the bound, and the up to
+// 2^13 terms of a voxel stay below 2^63.  words[0..2] hold the bit patterns of the three maxima
+// (of |.|, so they order like unsigned integers; a NaN or infinity anywhere gives a non-finite
+// bound, and then no corner is treated as local).
+constexpr double kRoundMagic = 6755399441055744.0;  // 1.5 * 2^52
+struct ScatterScale { bool valid; double up, down; };
+__device__ __forceinline__ ScatterScale scatter_scale(const unsigned *__restrict__ words, bool has_mask) {
+  const float bound = 1.001f * __uint_as_float(words[0]) * __uint_as_float(words[1]) *
+                      (has_mask ? __uint_as_float(words[2]) : 1.f);
+  ScatterScale r;
+  r.valid = bound < __builtin_inff() && bound == bound;
+  int ex = 0;
+  frexpf(fmaxf(bound, 1e-30f), &ex);  // bound < 2^ex
+  r.up = ldexp(1.0, 50 - ex);
+  r.down = ldexp(1.0, ex - 50);
+  return r;
+}
+__device__ __forceinline__ unsigned long long fixed_term(float t, double up) {
+  return static_cast<unsigned long long>(__double_as_longlong(fma(static_cast<double>(t), up, kRoundMagic))) -
+         static_cast<unsigned long long>(__double_as_longlong(kRoundMagic));
+}
+
+// max |p[i]| as a bit pattern, folded into *out (which starts at 0) with one atomic per workgroup
+__device__ __forceinline__ void fold_max(unsigned bits, unsigned *out) {
+  __shared__ unsigned part[4];
+  for (int sh = 32; sh > 0; sh >>= 1) bits = max(bits, static_cast<unsigned>(__shfl_xor(static_cast<int>(bits), sh)));
+  if (threadIdx.x % kWave == 0) part[threadIdx.x / kWave] = bits;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const unsigned m = max(max(part[0], part[1]), max(part[2], part[3]));
+    if (m) atomicMax(out, m);
+  }
+}
 template <typename T>
+__global__ __launch_bounds__(256) void dcn_absmax_kernel(const T *__restrict__ p, long n, unsigned *out) {
+  float m = 0.f;
+  bool bad = false;
+  for (long i = blockIdx.x * 256L + threadIdx.x; i < n; i += gridDim.x * 256L) {
+    const float v = fabsf(static_cast<float>(load(p + i)));
+    bad = bad || !(v == v);
+    m = fmaxf(m, v);
+  }
+  fold_max(bad ? 0x7fc00000u : __float_as_uint(m), out);
+}
+// max over (group, c, k) of sum_o |Wt[o, c, k]|
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_weight_colsum_kernel(const T *__restrict__ wt, const DcnDims s, unsigned *out) {
+  const long cols = static_cast<long>(s.cpg) * s.K, id = blockIdx.x * 256L + threadIdx.x;
+  float sum = 0.f;
+  if (id < cols * s.groups) {
+    const long g = id / cols, ck = id - g * cols;
+    for (int o = 0; o < s.opg; o++) sum += fabsf(static_cast<float>(load(wt + (g * s.opg + o) * cols + ck)));
+  }
+  fold_max(sum == sum ? __float_as_uint(sum) : 0x7fc00000u, out);
+}
+
+constexpr int kTapWords = 24;  // vox[8], w[8], mask, ld, lh, lw, local bits, padding
+
+// SPLIT: corners that are local to their brick's tile are left to the scatter kernel.
+template <typename T, bool SPLIT>
 __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
     const T *__restrict__ xt, const T *__restrict__ off, const T *__restrict__ mask,
     const T *__restrict__ gyt, const T *__restrict__ wb, float *__restrict__ gxt,
-    T *__restrict__ goff, T *__restrict__ gmask, const DcnDims s) {
+    T *__restrict__ goff, T *__restrict__ gmask, const DcnDims s, const unsigned *__restrict__ bounds) {
   using M = Mfma<T>;
   using P = typename std::conditional<(sizeof(T) == 2), float, double>::type;  // position type
   constexpr int PC = M::kPiece, SL = 2 * PC, ES = sizeof(T);
@@ -102,6 +198,8 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
   const T *mk = mask ? mask + bg * s.K * s.Q + qc : nullptr;
   float(*tp)[kTapWords] = taps[wave];
   float(*sm)[32] = sums[wave];
+  const TileOrigin origin = tile_origin(s, od / kSbD, oh / kSbH, ow / kSbW);
+  const bool split = SPLIT && scatter_scale(bounds, mask != nullptr).valid;
 
   int ki = 0, kj = 0, kk = 0;
   for (int k = 0; k < s.K; k++) {
@@ -116,8 +214,12 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
       if (++kk == s.kw) { kk = 0; if (++kj == s.kh) { kj = 0; ++ki; } }
       CornerTaps t;
       corner_taps<P>(s, pd, ph, pw, live, 1u, 0u, ~0u, t);
+      int first;
+      const unsigned local = split ? tile_bits(origin, static_cast<int>(floor(pd)), static_cast<int>(floor(ph)),
+                                               static_cast<int>(floor(pw)), first) : 0u;
       if (h == 0) {
         float4 *dst = reinterpret_cast<float4 *>(tp[n]);
+        if (SPLIT) dst[5] = make_float4(__uint_as_float(local), 0.f, 0.f, 0.f);
         dst[0] = make_float4(__uint_as_float(t.at[0]), __uint_as_float(t.at[1]), __uint_as_float(t.at[2]), __uint_as_float(t.at[3]));
         dst[1] = make_float4(__uint_as_float(t.at[4]), __uint_as_float(t.at[5]), __uint_as_float(t.at[6]), __uint_as_float(t.at[7]));
         dst[2] = make_float4(t.w[0], t.w[1], t.w[2], t.w[3]);
@@ -155,13 +257,15 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
                                  __float_as_uint(v1.x), __float_as_uint(v1.y), __float_as_uint(v1.z), __float_as_uint(v1.w)};
         const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
         const float m = e.x, ld = e.y, lh = e.z, lw = e.w;
+        const unsigned local = SPLIT ? __float_as_uint(src[5].x) : 0u;
         const float gm = acc[r] * m;
         float v[8];
 #pragma unroll
         for (int c = 0; c < 8; c++) {
           const bool in = vox[c] != ~0u;
           v[c] = load_element<T>(xr, in ? vox[c] * cin2 + cbyte2 : kOob);
-          __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(w[c] * gm, gr, in ? vox[c] * cin4 + cbyte4 : kOob, 0, 0);
+          const bool mine = in && !(SPLIT && ((local >> c) & 1u));
+          __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(w[c] * gm, gr, mine ? vox[c] * cin4 + cbyte4 : kOob, 0, 0);
         }
         float val = 0.f;
 #pragma unroll
@@ -188,6 +292,209 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
+  }
+}
+
+// ---- gradient of the input, local corners: summed in LDS, then added to the buffer ----------------
+// A workgroup owns a brick of positions and eight channels; its sixteen wavefronts are kScatterSplit
+// groups of eight, every group covers the 256 positions of the brick and takes a contiguous share
+// of the taps.  gcol comes from the 16 x 16 MFMA with the channels as rows: lane l holds position
+// l % 16 of a 16-position block and the channels l / 16 and l / 16 + 4, so one LDS add instruction
+// covers 16 positions x 4 adjacent channels; a voxel's 8 sums are 9 qwords apart from the next
+// voxel's to spread the banks.  After the taps the tile's non-zero sums are converted and added
+// to the gradient buffer: one global atomic per (voxel, channel) of the tile instead of one per
+// (position, tap, corner, channel).
+constexpr int kScatterSplit = 2, kScatterWaves = 8 * kScatterSplit, kScatterStride = 9;
+constexpr int kScatterKeep = 4;  // slices of grad_output a wavefront keeps in registers over the taps
+
+// weight [Cout, cpg, K] -> A pieces [group][tap][8-channel block][row step][lane][kPiece]: lane l
+// is MFMA row l % 16 = channel (row / 4) + 4 * (row % 2) of the block (rows 4j + 2, 4j + 3 repeat
+// rows 4j, 4j + 1 and are not used), element i the output channel g*opg + step*4*kPiece +
+// (l/16)*kPiece + i
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_weight_afragments8_kernel(const T *__restrict__ wt,
+                                                                     T *__restrict__ wa,
+                                                                     const DcnDims s) {
+  constexpr int PC = Mfma<T>::kPiece;
+  const int cblocks = s.cpg / 8, steps = s.opg / (4 * PC);
+  const long total = static_cast<long>(s.groups) * s.K * cblocks * steps * 64;
+  const long id = blockIdx.x * 256L + threadIdx.x;
+  if (id >= total) return;
+  const int lane = id % 64;
+  long r = id / 64;
+  const int st = r % steps; r /= steps;
+  const int cb = r % cblocks; r /= cblocks;
+  const int k = r % s.K;
+  const int g = static_cast<int>(r / s.K);
+  const int row = lane % 16, cl = cb * 8 + row / 4 + 4 * (row % 2);
+  const int o = g * s.opg + st * 4 * PC + (lane / 16) * PC;
+  for (int i = 0; i < PC; i++) wa[id * PC + i] = wt[(static_cast<long>(o + i) * s.cpg + cl) * s.K + k];
+}
+
+template <typename T>
+__global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter_kernel(
+    const T *__restrict__ off, const T *__restrict__ mask, const T *__restrict__ gyt,
+    const T *__restrict__ wa, float *__restrict__ gxt, const DcnDims s, const int nbh, const int nbw,
+    const unsigned *__restrict__ bounds) {
+  using M = Mfma<T>;
+  using P = typename std::conditional<(sizeof(T) == 2), float, double>::type;
+  constexpr int PC = M::kPiece, SL = 4 * PC;
+  __shared__ unsigned long long tile[kStVox * kScatterStride];
+  __shared__ __attribute__((aligned(16))) float recs[kScatterWaves][32][8];
+  const ScatterScale scale = scatter_scale(bounds, mask != nullptr);
+  if (!scale.valid) return;  // every corner went through the data kernel
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int n = lane % 32, p16 = lane % 16, j = lane / 16;
+  const int pg = wave % 8, tg = wave / 8;
+  const unsigned brick = xcd_contiguous(blockIdx.x, gridDim.x);
+  const int bx = brick % nbw, by = (brick / nbw) % nbh, bz = brick / (nbw * nbh);
+  const int c0 = blockIdx.y * 8, b = blockIdx.z;
+  const int dgi = c0 / s.cpd, g = c0 / s.cpg, cb = (c0 - g * s.cpg) / 8;
+  const long bg = static_cast<long>(b) * s.dg + dgi;
+  const int cblocks = s.cpg / 8, steps = s.opg / SL;
+  const TileOrigin origin = tile_origin(s, bz, by, bx);
+
+  for (int i = threadIdx.x; i < kStVox * kScatterStride; i += kScatterWaves * 64) tile[i] = 0ull;
+  __syncthreads();
+
+  // position of brick index i: depth slice i / 64, row (i / 8) % 8, column i % 8
+  auto position = [&](int i, bool &live) {
+    const int od = bz * kSbD + i / (kSbH * kSbW), oh = by * kSbH + (i / kSbW) % kSbH, ow = bx * kSbW + i % kSbW;
+    live = od < s.Do && oh < s.Ho && ow < s.Wo;
+    return (static_cast<long>(min(od, s.Do - 1)) * s.Ho + min(oh, s.Ho - 1)) * s.Wo + min(ow, s.Wo - 1);
+  };
+  // the lane's own position for the taps (both halves of the wavefront compute them)
+  bool live;
+  const long q = position(pg * 32 + n, live);
+  const int ow = q % s.Wo, oh = (q / s.Wo) % s.Ho, od = q / (static_cast<long>(s.Wo) * s.Ho);
+  const int bd = od * s.sd - s.pd, bh = oh * s.sh - s.ph, bw = ow * s.sw - s.pw;
+  // grad_output of the lane's column in the two 16-position blocks (MFMA B operand)
+  bool blive[2];
+  const T *grow[2];
+  u32x4 keep[2][kScatterKeep];
+#pragma unroll
+  for (int blk = 0; blk < 2; blk++) {
+    const long qb = position(pg * 32 + blk * 16 + p16, blive[blk]);
+    grow[blk] = gyt + (static_cast<long>(b) * s.Q + qb) * s.Cout + g * s.opg + j * PC;
+#pragma unroll
+    for (int st = 0; st < kScatterKeep; st++)
+      keep[blk][st] = (blive[blk] && st < steps) ? *reinterpret_cast<const u32x4 *>(grow[blk] + st * SL)
+                                                : u32x4{0u, 0u, 0u, 0u};
+  }
+  const int per = (s.K + kScatterSplit - 1) / kScatterSplit, k0 = min(tg * per, s.K), k1 = min(s.K, k0 + per);
+  const T *o = off + (bg * s.nd * s.K + static_cast<long>(s.nd) * k0) * s.Q + q;
+  const T *mk = mask ? mask + (bg * s.K + k0) * s.Q + q : nullptr;
+  float(*rec)[8] = recs[wave];
+
+  int ki = k0 / (s.kh * s.kw), kj = (k0 / s.kw) % s.kh, kk = k0 % s.kw;
+  P fd = P(0), fh = P(0), fw = P(0);
+  float fm = 1.f;
+  if (k0 < k1) {
+    dcn_offsets(s, o, fd, fh, fw);
+    if (mk) fm = load(mk);
+  }
+  // weight pieces of the current tap, loaded one tap ahead
+  const long tap_stride = static_cast<long>(cblocks) * steps * 64 * PC;
+  const T *afrag = wa + (((static_cast<long>(g) * s.K + k0) * cblocks + cb) * steps * 64 + lane) * PC;
+  u32x4 wcur[kScatterKeep];
+#pragma unroll
+  for (int st = 0; st < kScatterKeep; st++)
+    wcur[st] = (k0 < k1 && st < steps) ? *reinterpret_cast<const u32x4 *>(afrag + static_cast<long>(st) * (64 * PC))
+                                       : u32x4{0u, 0u, 0u, 0u};
+  for (int k = k0; k < k1; k++) {
+    u32x4 wnext[kScatterKeep];
+#pragma unroll
+    for (int st = 0; st < kScatterKeep; st++)
+      wnext[st] = (k + 1 < k1 && st < steps)
+                      ? *reinterpret_cast<const u32x4 *>(afrag + tap_stride + static_cast<long>(st) * (64 * PC))
+                      : u32x4{0u, 0u, 0u, 0u};
+    {
+      const P pd = fd + static_cast<P>(bd + ki * s.dd), ph = fh + static_cast<P>(bh + kj * s.dh),
+              pw = fw + static_cast<P>(bw + kk * s.dw);
+      const float m = fm;
+      o += s.nd * s.Q;
+      if (mk) mk += s.Q;
+      if (++kk == s.kw) { kk = 0; if (++kj == s.kh) { kj = 0; ++ki; } }
+      if (k + 1 < k1) {  // the next tap's offsets are in flight during this tap's adds
+        dcn_offsets(s, o, fd, fh, fw);
+        if (mk) fm = load(mk);
+      }
+      CornerTaps t;
+      corner_taps<P>(s, pd, ph, pw, live, 1u, 0u, ~0u, t);
+      int first;
+      unsigned bits = tile_bits(origin, static_cast<int>(floor(pd)), static_cast<int>(floor(ph)),
+                                static_cast<int>(floor(pw)), first);
+      unsigned inside = 0;
+#pragma unroll
+      for (int c = 0; c < 8; c++) inside |= t.at[c] != ~0u ? 1u << c : 0u;
+      bits &= inside;
+      if (lane < 32) {
+        float4 *dst = reinterpret_cast<float4 *>(rec[n]);
+        dst[0] = make_float4(__int_as_float(first), __uint_as_float(bits), m, t.ld);
+        dst[1] = make_float4(t.lh, t.lw, 0.f, 0.f);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    float4_t acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+    for (int st = 0; st < kScatterKeep; st++)
+      if (st < steps) {
+        acc[0] = M::run16(wcur[st], keep[0][st], acc[0]);
+        acc[1] = M::run16(wcur[st], keep[1][st], acc[1]);
+      }
+    for (int st = kScatterKeep; st < steps; st++) {
+      const u32x4 a = *reinterpret_cast<const u32x4 *>(afrag + static_cast<long>(st) * (64 * PC));
+#pragma unroll
+      for (int blk = 0; blk < 2; blk++) {
+        const u32x4 bv = blive[blk] ? *reinterpret_cast<const u32x4 *>(grow[blk] + st * SL) : u32x4{0u, 0u, 0u, 0u};
+        acc[blk] = M::run16(a, bv, acc[blk]);
+      }
+    }
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++) {
+      const float4 *src = reinterpret_cast<const float4 *>(rec[blk * 16 + p16]);
+      const float4 ra = src[0], rb = src[1];
+      const int first = __float_as_int(ra.x);
+      const unsigned bits = __float_as_uint(ra.y);
+      const float gv[2] = {acc[blk][0] * ra.z, acc[blk][1] * ra.z};  // the lane's two channels
+      const float wd[2] = {1.f - ra.w, ra.w}, wh[2] = {1.f - rb.x, rb.x}, ww[2] = {1.f - rb.y, rb.y};
+#pragma unroll
+      for (int c = 0; c < 8; c++) {
+        const int ca = c >> 2, cb2 = (c >> 1) & 1, ce = c & 1;
+        if ((bits >> c) & 1u) {
+          const float wc = wd[ca] * wh[cb2] * ww[ce];
+          unsigned long long *dst = tile + (first + ca * (kStH * kStW) + cb2 * kStW + ce) * kScatterStride + j;
+#pragma unroll
+          for (int r = 0; r < 2; r++)
+            __hip_atomic_fetch_add(dst + 4 * r, fixed_term(wc * gv[r], scale.up), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    afrag += tap_stride;
+#pragma unroll
+    for (int st = 0; st < kScatterKeep; st++) wcur[st] = wnext[st];
+  }
+  __syncthreads();
+  // ---- the tile's voxels inside the volume go to the gradient buffer, 8 channels per voxel --------
+  const __amdgpu_buffer_rsrc_t gr = __builtin_amdgcn_make_buffer_rsrc(
+      gxt + static_cast<long>(b) * s.P * s.Cin, 0, static_cast<int>(s.P * s.Cin * 4), kRsrcFlags);
+  const unsigned cin4 = static_cast<unsigned>(s.Cin) * 4u;
+  const int ch = threadIdx.x % 8;
+  for (int cell = threadIdx.x / 8; cell < kStVox; cell += kScatterWaves * 8) {
+    const int zw = cell % kStW + origin.w, zh = (cell / kStW) % kStH + origin.h, zd = cell / (kStW * kStH) + origin.d;
+    const unsigned long long sum = tile[cell * kScatterStride + ch];
+    if (zd >= 0 && zd < s.D && zh >= 0 && zh < s.H && zw >= 0 && zw < s.W && sum != 0ull) {
+      const double v = static_cast<double>(static_cast<long long>(sum)) * scale.down;
+      __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(
+          static_cast<float>(v), gr,
+          static_cast<unsigned>((zd * s.H + zh) * s.W + zw) * cin4 + static_cast<unsigned>(c0 + ch) * 4u, 0, 0);
+    }
   }
 }
 
@@ -342,6 +649,14 @@ __global__ void dcn_zero_f32_kernel(float *p, long n) {
     p[i] = 0.f;
 }
 
+// The LDS scatter pays when its tile holds the reach of a brick's undeformed taps with a voxel to
+// spare on either side (offsets beyond the tile still work, through the data kernel's atomics).
+static bool scatter_tile_applies(const DcnDims &s) {
+  const int ed = (kSbD - 1) * s.sd + (s.kd - 1) * s.dd + 1, eh = (kSbH - 1) * s.sh + (s.kh - 1) * s.dh + 1,
+            ew = (kSbW - 1) * s.sw + (s.kw - 1) * s.dw + 1;
+  return s.nd == 3 && ed + 2 <= kStD && eh + 2 <= kStH && ew + 2 <= kStW;
+}
+
 static size_t align256b(size_t v) { return (v + 255) / 256 * 256; }
 
 bool dcn_mfma_backward_supported(const DcnDims &s, int dtype) {
@@ -353,9 +668,10 @@ bool dcn_mfma_backward_supported(const DcnDims &s, int dtype) {
   return true;
 }
 
-// workspace: xt | gyt | weight fragments | gxt (fp32) | gw (fp32) | gb (fp32)
+// workspace: xt | gyt | weight fragments (32- and 8-channel blocks) | gxt (fp32) | gw (fp32) | gb (fp32) |
+// the three maxima of the scatter scale; everything from gxt on starts at zero
 struct BackwardLayout {
-  size_t xt, gyt, wb, gxt, gw, gb, total;
+  size_t xt, gyt, wb, wa, gxt, gw, gb, bounds, total;
 };
 static BackwardLayout backward_layout(const DcnDims &s, int dtype) {
   BackwardLayout l;
@@ -364,9 +680,11 @@ static BackwardLayout backward_layout(const DcnDims &s, int dtype) {
   l.xt = at; at += align256b(static_cast<size_t>(s.B) * s.P * s.Cin * es);
   l.gyt = at; at += align256b(static_cast<size_t>(s.B) * s.Q * s.Cout * es);
   l.wb = at; at += align256b(static_cast<size_t>(s.Cout) * s.cpg * s.K * es);
+  l.wa = at; at += align256b(2 * static_cast<size_t>(s.Cout) * s.cpg * s.K * es);  // 16 MFMA rows per 8 channels
   l.gxt = at; at += align256b(static_cast<size_t>(s.B) * s.P * s.Cin * 4);
   l.gw = at; at += align256b(static_cast<size_t>(s.Cout) * s.cpg * s.K * 4);
   l.gb = at; at += align256b(static_cast<size_t>(s.Cout) * 4);
+  l.bounds = at; at += 256;
   l.total = at;
   return l;
 }
@@ -394,9 +712,35 @@ static int backward_run(const void *x, const void *off, const void *mask, const 
                      0, stream, gxt, nz);
   const long qblocks = (s.Q + 127) / 128;
   MV_REQUIRE(qblocks < (1L << 31), "grid too large");
-  hipLaunchKernelGGL((dcn_backward_data_mfma_kernel<T>), dim3(static_cast<unsigned>(qblocks), s.dg, s.B),
-                     dim3(256), 0, stream, xt, static_cast<const T *>(off), static_cast<const T *>(mask), gyt,
-                     wb, gxt, static_cast<T *>(goff), static_cast<T *>(gmask), s);
+  if (scatter_tile_applies(s)) {
+    unsigned *bounds = reinterpret_cast<unsigned *>(ws + l.bounds);
+    const long ngy = static_cast<long>(s.B) * s.Cout * s.Q, nmask = static_cast<long>(s.B) * s.dg * s.K * s.Q;
+    const long ncols = static_cast<long>(s.groups) * s.cpg * s.K;
+    hipLaunchKernelGGL((dcn_absmax_kernel<T>), dim3(static_cast<unsigned>(min((ngy + 4095) / 4096, 1024L))), dim3(256),
+                       0, stream, static_cast<const T *>(gy), ngy, bounds);
+    hipLaunchKernelGGL((dcn_weight_colsum_kernel<T>), dim3(static_cast<unsigned>((ncols + 255) / 256)), dim3(256), 0,
+                       stream, static_cast<const T *>(wt), s, bounds + 1);
+    if (mask)
+      hipLaunchKernelGGL((dcn_absmax_kernel<T>), dim3(static_cast<unsigned>(min((nmask + 4095) / 4096, 1024L))),
+                         dim3(256), 0, stream, static_cast<const T *>(mask), nmask, bounds + 2);
+    hipLaunchKernelGGL((dcn_backward_data_mfma_kernel<T, true>), dim3(static_cast<unsigned>(qblocks), s.dg, s.B),
+                       dim3(256), 0, stream, xt, static_cast<const T *>(off), static_cast<const T *>(mask), gyt,
+                       wb, gxt, static_cast<T *>(goff), static_cast<T *>(gmask), s, bounds);
+    T *wa = reinterpret_cast<T *>(ws + l.wa);
+    const long lanes8 = static_cast<long>(s.groups) * s.K * (s.cpg / 8) * (s.opg / (4 * Mfma<T>::kPiece)) * 64;
+    hipLaunchKernelGGL((dcn_weight_afragments8_kernel<T>), dim3(static_cast<unsigned>((lanes8 + 255) / 256)),
+                       dim3(256), 0, stream, static_cast<const T *>(wt), wa, s);
+    const long nbd = (s.Do + kSbD - 1) / kSbD, nbh = (s.Ho + kSbH - 1) / kSbH, nbw = (s.Wo + kSbW - 1) / kSbW;
+    MV_REQUIRE(nbd * nbh * nbw < (1L << 31) && s.Cin / 8 <= 65535, "grid too large");
+    hipLaunchKernelGGL((dcn_backward_scatter_kernel<T>), dim3(static_cast<unsigned>(nbd * nbh * nbw), s.Cin / 8, s.B),
+                       dim3(kScatterWaves * 64), 0, stream, static_cast<const T *>(off),
+                       static_cast<const T *>(mask), gyt, wa, gxt, s, static_cast<int>(nbh), static_cast<int>(nbw),
+                       bounds);
+  } else {
+    hipLaunchKernelGGL((dcn_backward_data_mfma_kernel<T, false>), dim3(static_cast<unsigned>(qblocks), s.dg, s.B),
+                       dim3(256), 0, stream, xt, static_cast<const T *>(off), static_cast<const T *>(mask), gyt,
+                       wb, gxt, static_cast<T *>(goff), static_cast<T *>(gmask), s, nullptr);
+  }
   const dim3 wgrid(static_cast<unsigned>(static_cast<long>(s.Cin / 32) * s.K),
                    static_cast<unsigned>((s.Q + kGwChunk - 1) / kGwChunk), s.B);
 #define MV_LAUNCH_GW(MTV)                                                                          \

@@ -120,6 +120,53 @@ def test_matrix_core_backward_vs_oracle(ops, oracle, dtype, modulated, groups, d
         assert_close(ms.grad, gm, tol, "grad mask")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("size,offset_std,gy_scale", [
+    ((12, 16, 16), 0.0, 1.0),       # every corner inside its brick's LDS tile
+    ((12, 16, 16), 0.7, 1.0),       # offsets within the tile's margin
+    ((12, 16, 16), 8.0, 1.0),       # most corners leave the tile: global atomics of the data kernel
+    ((3, 5, 7), 2.0, 1.0),          # volume smaller than a brick
+    ((9, 17, 10), 2.0, 3.0e4),      # ragged bricks; large and small gradients: the fixed-point scale
+    ((9, 17, 10), 2.0, 1.0e-4)])    # of the LDS sums follows max |grad_output|
+def test_input_gradient_through_lds_tiles(ops, oracle, dtype, size, offset_std, gy_scale):
+    """Unit-stride 3^3 layers sum the input gradient of corners near their position in 64-bit
+    fixed-point LDS tiles (the rest goes through global atomics): all gradients against the oracle
+    for offsets from zero to far beyond the tile and for gradients of very different magnitude."""
+    from medvision_amd.ops.modulated_deform_conv_3d import modulated_deform_conv
+    if dtype == torch.float16 and gy_scale > 1e3:
+        gy_scale = 200.0    # keep fp16 gradients finite
+    g = wl.gen(400 + int(offset_std * 10) + size[0])
+    x, off, mask, w, b = wl.dcn_inputs(g, 2, 32, 64, size, 3, 1, 1, dtype, 1, 1, 1, True, offset_std)
+    xs, offs, ms, ws, bs = [t.to(DEV).requires_grad_(True) for t in (x, off, mask, w, b)]
+    y = modulated_deform_conv(xs, offs, ms, ws, bs, 1, 1, 1, 1, 1)
+    gy = (torch.randn(y.shape, generator=g) * gy_scale).to(dtype)
+    y.backward(gy.to(DEV))
+    gx, goff, gm, gw, gb = oracle.dcn3d_backward(x, off, mask, w, gy, True, 1, 1, 1, 1, 1)
+    tol = BWD_TOL[dtype]
+    assert_close(xs.grad, gx, tol, "grad input")
+    assert_close(offs.grad, goff, tol, "grad offset")
+    assert_close(ms.grad, gm, tol, "grad mask")
+    assert_close(ws.grad, gw, tol, "grad weight")
+
+
+def test_input_gradient_with_non_finite_values(ops, oracle):
+    """An infinity in grad_output makes the bound of the fixed-point sums non-finite: every corner
+    then goes through the fp32 atomics, and NaN / infinity reach exactly the voxels the oracle's do."""
+    from medvision_amd.ops.modulated_deform_conv_3d import modulated_deform_conv
+    g = wl.gen(431)
+    x, off, mask, w, b = wl.dcn_inputs(g, 1, 32, 32, (6, 8, 8), 3, 1, 1, torch.float32, 1, 1, 1, True, 1.0)
+    xs, offs, ms, ws, bs = [t.to(DEV).requires_grad_(True) for t in (x, off, mask, w, b)]
+    y = modulated_deform_conv(xs, offs, ms, ws, bs, 1, 1, 1, 1, 1)
+    gy = torch.randn(y.shape, generator=g)
+    gy[0, 3, 2, 4, 5] = float("inf")
+    y.backward(gy.to(DEV))
+    gx = oracle.dcn3d_backward(x, off, mask, w, gy, True, 1, 1, 1, 1, 1)[0]
+    got = xs.grad.cpu()
+    assert torch.equal(torch.isfinite(got), torch.isfinite(gx))
+    fin = torch.isfinite(gx)
+    assert_close(got[fin], gx[fin], BWD_TOL[torch.float32], "finite part of grad input")
+
+
 def test_config4_full_size_properties(ops):
     """Full config-4 shape [2,32,48^3] -> Cout 64: zero offsets and unit mask reduce DCN to a plain
     convolution (checked against torch's conv3d), and the op is linear in the mask."""
