@@ -123,9 +123,11 @@ __device__ __forceinline__ ScatterScale scatter_scale(const unsigned *__restrict
   r.down = ldexp(1.0, ex - 50);
   return r;
 }
-__device__ __forceinline__ unsigned long long fixed_term(float t, double up) {
-  return static_cast<unsigned long long>(__double_as_longlong(fma(static_cast<double>(t), up, kRoundMagic))) -
-         static_cast<unsigned long long>(__double_as_longlong(kRoundMagic));
+// round(w * scaled) as a 64-bit integer; the low word of the magic number's bit pattern is zero
+__device__ __forceinline__ unsigned long long fixed_term(float w, double scaled) {
+  const double x = fma(static_cast<double>(w), scaled, kRoundMagic);
+  const unsigned lo = static_cast<unsigned>(__double2loint(x)), hi = static_cast<unsigned>(__double2hiint(x)) - 0x43380000u;
+  return (static_cast<unsigned long long>(hi) << 32) | lo;
 }
 
 // max |p[i]| as a bit pattern, folded into *out (which starts at 0) with one atomic per workgroup
@@ -162,7 +164,7 @@ __global__ __launch_bounds__(256) void dcn_weight_colsum_kernel(const T *__restr
   fold_max(sum == sum ? __float_as_uint(sum) : 0x7fc00000u, out);
 }
 
-constexpr int kTapWords = 24;  // vox[8], w[8], mask, ld, lh, lw, local bits, padding
+constexpr int kTapWords = 28;  // byte offsets of the corners in x [8] and in the gradient buffer [8], w[8], mask, ld, lh, lw
 
 // SPLIT: corners that are local to their brick's tile are left to the scatter kernel.
 template <typename T, bool SPLIT>
@@ -175,8 +177,12 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
   constexpr int PC = M::kPiece, SL = 2 * PC, ES = sizeof(T);
   __shared__ __attribute__((aligned(16))) float taps[4][32][kTapWords];
   __shared__ float sums[4][4][32];
+  // x at the 8 corners of the two positions of an accumulator register, 32 channels each, in two
+  // alternating buffers per wavefront: fetched 16 bytes per lane, read back one channel per lane
+  __shared__ __attribute__((aligned(16))) T stage[4][2][16][32];
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int n = lane % 32, h = lane / 32;
+  constexpr int LPC = 2 * ES, FETCHES = ES / 2;  // lanes per corner (16 bytes each), fetches per register
   // one contiguous eighth of the positions per XCD (see xcd_contiguous)
   const long q0 = (static_cast<long>(xcd_contiguous(blockIdx.x, gridDim.x)) * 4 + wave) * 32;
   if (q0 >= s.Q) return;  // whole wavefront idle (no workgroup barriers in this kernel)
@@ -193,6 +199,7 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
       const_cast<T *>(xt + static_cast<long>(b) * s.P * s.Cin), 0, static_cast<int>(s.P * s.Cin * ES), kRsrcFlags);
   const __amdgpu_buffer_rsrc_t gr = __builtin_amdgcn_make_buffer_rsrc(
       gxt + static_cast<long>(b) * s.P * s.Cin, 0, static_cast<int>(s.P * s.Cin * 4), kRsrcFlags);
+  const unsigned cin2 = static_cast<unsigned>(s.Cin) * ES;
   const T *gyrow = gyt + (static_cast<long>(b) * s.Q + qc) * s.Cout + h * PC;
   const T *o = off + bg * s.nd * s.K * s.Q + qc;
   const T *mk = mask ? mask + bg * s.K * s.Q + qc : nullptr;
@@ -212,19 +219,25 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
       o += s.nd * s.Q;
       if (mk) mk += s.Q;
       if (++kk == s.kw) { kk = 0; if (++kj == s.kh) { kj = 0; ++ki; } }
+      // corner offsets in bytes (x: element size ES, gradient buffer: 4); kOob for a corner outside
+      // the volume and, in the gradient buffer, for one the scatter kernel sums
       CornerTaps t;
-      corner_taps<P>(s, pd, ph, pw, live, 1u, 0u, ~0u, t);
+      corner_taps<P>(s, pd, ph, pw, live, cin2, 0u, kOob, t);
       int first;
       const unsigned local = split ? tile_bits(origin, static_cast<int>(floor(pd)), static_cast<int>(floor(ph)),
                                                static_cast<int>(floor(pw)), first) : 0u;
+      unsigned ag[8];
+#pragma unroll
+      for (int c = 0; c < 8; c++) ag[c] = (t.at[c] == kOob || ((local >> c) & 1u)) ? kOob : t.at[c] * (4u / ES);
       if (h == 0) {
         float4 *dst = reinterpret_cast<float4 *>(tp[n]);
-        if (SPLIT) dst[5] = make_float4(__uint_as_float(local), 0.f, 0.f, 0.f);
         dst[0] = make_float4(__uint_as_float(t.at[0]), __uint_as_float(t.at[1]), __uint_as_float(t.at[2]), __uint_as_float(t.at[3]));
         dst[1] = make_float4(__uint_as_float(t.at[4]), __uint_as_float(t.at[5]), __uint_as_float(t.at[6]), __uint_as_float(t.at[7]));
         dst[2] = make_float4(t.w[0], t.w[1], t.w[2], t.w[3]);
         dst[3] = make_float4(t.w[4], t.w[5], t.w[6], t.w[7]);
         dst[4] = make_float4(m, t.ld, t.lh, t.lw);
+        dst[5] = make_float4(__uint_as_float(ag[0]), __uint_as_float(ag[1]), __uint_as_float(ag[2]), __uint_as_float(ag[3]));
+        dst[6] = make_float4(__uint_as_float(ag[4]), __uint_as_float(ag[5]), __uint_as_float(ag[6]), __uint_as_float(ag[7]));
         sm[0][n] = 0.f; sm[1][n] = 0.f; sm[2][n] = 0.f; sm[3][n] = 0.f;
       }
     }
@@ -245,35 +258,57 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
         const u32x4 bf = *reinterpret_cast<const u32x4 *>(wfrag + static_cast<long>(st) * (64 * PC));
         acc = M::run(a, bf, acc);
       }
-      const unsigned cbyte2 = static_cast<unsigned>(c0 + n) * ES, cbyte4 = static_cast<unsigned>(c0 + n) * 4u;
-      const unsigned cin2 = static_cast<unsigned>(s.Cin) * ES, cin4 = static_cast<unsigned>(s.Cin) * 4u;
+      const unsigned cbyte4 = static_cast<unsigned>(c0 + n) * 4u;
       // ---- register r: position 8*(r/4) + 4*h + r%4, channel c0 + n ------------------------------
+      // fetch f of register r: lane l holds 16 bytes of corner (f * 64 + l) / LPC of the register's
+      // two positions (corners 0..7 of the lower half-wavefront's position, then the upper one's).
+      // kOob plus a channel offset stays beyond the buffers: such loads give 0, such adds are dropped
+      auto fetch = [&](int r, u32x4 (&dst)[FETCHES]) {
+#pragma unroll
+        for (int f = 0; f < FETCHES; f++) {
+          const int corner = (f * 64 + lane) / LPC, pp = 8 * (r / 4) + 4 * (corner / 8) + (r % 4);
+          const unsigned at = __float_as_uint(tp[pp][corner % 8]);
+          dst[f] = __builtin_amdgcn_raw_buffer_load_b128(xr, at + static_cast<unsigned>(c0) * ES + (lane % LPC) * 16u, 0, 0);
+        }
+      };
+      u32x4 cur[FETCHES];
+      fetch(0, cur);
 #pragma unroll
       for (int r = 0; r < 16; r++) {
         const int p = 8 * (r / 4) + 4 * h + (r % 4);
+        T(*sg)[32] = stage[wave][r & 1];
+#pragma unroll
+        for (int f = 0; f < FETCHES; f++)
+          *reinterpret_cast<u32x4 *>(&sg[(f * 64 + lane) / LPC][(lane % LPC) * (16 / ES)]) = cur[f];
+        if (r + 1 < 16) fetch(r + 1, cur);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         const float4 *src = reinterpret_cast<const float4 *>(tp[p]);
-        const float4 v0 = src[0], v1 = src[1], w0 = src[2], w1 = src[3], e = src[4];
-        const unsigned vox[8] = {__float_as_uint(v0.x), __float_as_uint(v0.y), __float_as_uint(v0.z), __float_as_uint(v0.w),
-                                 __float_as_uint(v1.x), __float_as_uint(v1.y), __float_as_uint(v1.z), __float_as_uint(v1.w)};
+        const float4 w0 = src[2], w1 = src[3], e = src[4], g0 = src[5], g1 = src[6];
+        const unsigned ag[8] = {__float_as_uint(g0.x), __float_as_uint(g0.y), __float_as_uint(g0.z), __float_as_uint(g0.w),
+                                __float_as_uint(g1.x), __float_as_uint(g1.y), __float_as_uint(g1.z), __float_as_uint(g1.w)};
         const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
         const float m = e.x, ld = e.y, lh = e.z, lw = e.w;
-        const unsigned local = SPLIT ? __float_as_uint(src[5].x) : 0u;
         const float gm = acc[r] * m;
         float v[8];
 #pragma unroll
         for (int c = 0; c < 8; c++) {
-          const bool in = vox[c] != ~0u;
-          v[c] = load_element<T>(xr, in ? vox[c] * cin2 + cbyte2 : kOob);
-          const bool mine = in && !(SPLIT && ((local >> c) & 1u));
-          __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(w[c] * gm, gr, mine ? vox[c] * cin4 + cbyte4 : kOob, 0, 0);
+          v[c] = load(&sg[h * 8 + c][n]);
+          // with the scatter kernel at work most instructions would find no lane with an add left
+          if (!SPLIT || ag[c] != kOob)
+            __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(w[c] * gm, gr, ag[c] + cbyte4, 0, 0);
         }
-        float val = 0.f;
-#pragma unroll
-        for (int c = 0; c < 8; c++) val += w[c] * v[c];
-        const float hd = 1.f - ld, hh = 1.f - lh, hw = 1.f - lw;
-        const float dd = hh * (hw * (v[4] - v[0]) + lw * (v[5] - v[1])) + lh * (hw * (v[6] - v[2]) + lw * (v[7] - v[3]));
-        const float dh = hd * (hw * (v[2] - v[0]) + lw * (v[3] - v[1])) + ld * (hw * (v[6] - v[4]) + lw * (v[7] - v[5]));
-        const float dw = hd * (hh * (v[1] - v[0]) + lh * (v[3] - v[2])) + ld * (hh * (v[5] - v[4]) + lh * (v[7] - v[6]));
+        // value and the three partial derivatives of the trilinear form, sharing the differences
+        const float x0 = v[1] - v[0], x1 = v[3] - v[2], x2 = v[5] - v[4], x3 = v[7] - v[6];
+        const float a0 = fmaf(lw, x0, v[0]), a1 = fmaf(lw, x1, v[2]), a2 = fmaf(lw, x2, v[4]), a3 = fmaf(lw, x3, v[6]);
+        const float b0 = fmaf(lh, x1 - x0, x0), b1 = fmaf(lh, x3 - x2, x2);
+        const float dw = fmaf(ld, b1 - b0, b0);
+        const float y0 = a1 - a0, y1 = a3 - a2;
+        const float c0v = fmaf(lh, y0, a0), c1v = fmaf(lh, y1, a2);
+        const float dh = fmaf(ld, y1 - y0, y0);
+        const float dd = c1v - c0v;
+        const float val = fmaf(ld, dd, c0v);
         const float s0 = half_wave_sum(dd * gm), s1 = half_wave_sum(dh * gm), s2 = half_wave_sum(dw * gm);
         const float s3 = half_wave_sum(acc[r] * val);
         if (n == 16) {  // one lane per half-wavefront; the chunks of a deformable group accumulate
@@ -459,7 +494,9 @@ __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter_kerne
       const float4 ra = src[0], rb = src[1];
       const int first = __float_as_int(ra.x);
       const unsigned bits = __float_as_uint(ra.y);
-      const float gv[2] = {acc[blk][0] * ra.z, acc[blk][1] * ra.z};  // the lane's two channels
+      // the lane's two channels, times the mask and the fixed-point scale
+      const double gv[2] = {static_cast<double>(acc[blk][0] * ra.z) * scale.up,
+                            static_cast<double>(acc[blk][1] * ra.z) * scale.up};
       const float wd[2] = {1.f - ra.w, ra.w}, wh[2] = {1.f - rb.x, rb.x}, ww[2] = {1.f - rb.y, rb.y};
 #pragma unroll
       for (int c = 0; c < 8; c++) {
@@ -469,7 +506,7 @@ __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter_kerne
           unsigned long long *dst = tile + (first + ca * (kStH * kStW) + cb2 * kStW + ce) * kScatterStride + j;
 #pragma unroll
           for (int r = 0; r < 2; r++)
-            __hip_atomic_fetch_add(dst + 4 * r, fixed_term(wc * gv[r], scale.up), __ATOMIC_RELAXED,
+            __hip_atomic_fetch_add(dst + 4 * r, fixed_term(wc, gv[r]), __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_WORKGROUP);
         }
       }
@@ -508,7 +545,7 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
   using M = Mfma<T>;
   using P = typename std::conditional<(sizeof(T) == 2), float, double>::type;  // position type
   constexpr int PC = M::kPiece, SL = 2 * PC, ES = sizeof(T);
-  __shared__ __attribute__((aligned(16))) float taps[4][64][16];  // vox[8], w[8] * mask
+  __shared__ __attribute__((aligned(16))) float taps[4][64][16];  // byte offsets in x [8], w[8] * mask
   __shared__ float part[3][MT][16][64];                           // accumulators of wavefronts 1..3
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int n = lane % 32, h = lane / 32;
@@ -548,7 +585,7 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
       pw += static_cast<P>(ow * s.sw - s.pw + kk * s.dw);
       const float m = mb_ ? load(mb_ + qc) : 1.f;
       CornerTaps t;
-      corner_taps<P>(s, pd, ph, pw, live, 1u, 0u, ~0u, t);
+      corner_taps<P>(s, pd, ph, pw, live, cin2, 0u, kOob, t);  // byte offsets in x; kOob outside the volume
       float4 *dst = reinterpret_cast<float4 *>(tp[lane]);
       dst[0] = make_float4(__uint_as_float(t.at[0]), __uint_as_float(t.at[1]), __uint_as_float(t.at[2]), __uint_as_float(t.at[3]));
       dst[1] = make_float4(__uint_as_float(t.at[4]), __uint_as_float(t.at[5]), __uint_as_float(t.at[6]), __uint_as_float(t.at[7]));
@@ -566,13 +603,12 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
       for (int i = 0; i < PC; i++) {
         const float4 *src = reinterpret_cast<const float4 *>(tp[st * SL + h * PC + i]);
         const float4 v0 = src[0], v1 = src[1], w0 = src[2], w1 = src[3];
-        const unsigned vox[8] = {__float_as_uint(v0.x), __float_as_uint(v0.y), __float_as_uint(v0.z), __float_as_uint(v0.w),
-                                 __float_as_uint(v1.x), __float_as_uint(v1.y), __float_as_uint(v1.z), __float_as_uint(v1.w)};
+        const unsigned ax[8] = {__float_as_uint(v0.x), __float_as_uint(v0.y), __float_as_uint(v0.z), __float_as_uint(v0.w),
+                                __float_as_uint(v1.x), __float_as_uint(v1.y), __float_as_uint(v1.z), __float_as_uint(v1.w)};
         const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
         float a = 0.f;
 #pragma unroll
-        for (int c = 0; c < 8; c++)
-          a += w[c] * load_element<T>(xr, vox[c] != ~0u ? vox[c] * cin2 + cbyte2 : kOob);
+        for (int c = 0; c < 8; c++) a += w[c] * load_element<T>(xr, ax[c] + cbyte2);  // kOob + channel: reads 0
         col[i] = a;
       }
       const u32x4 bf = M::pack(col);
