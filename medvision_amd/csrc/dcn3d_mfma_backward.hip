@@ -143,25 +143,43 @@ __device__ __forceinline__ void fold_max(unsigned bits, unsigned *out) {
 }
 template <typename T>
 __global__ __launch_bounds__(256) void dcn_absmax_kernel(const T *__restrict__ p, long n, unsigned *out) {
+  constexpr int V = 16 / sizeof(T);  // elements per 16-byte load
   float m = 0.f;
   bool bad = false;
-  for (long i = blockIdx.x * 256L + threadIdx.x; i < n; i += gridDim.x * 256L) {
-    const float v = fabsf(static_cast<float>(load(p + i)));
+  auto take = [&](T e) {
+    const float v = fabsf(static_cast<float>(load(&e)));
     bad = bad || !(v == v);
     m = fmaxf(m, v);
+  };
+  const long head = min(n, static_cast<long>((16 - reinterpret_cast<size_t>(p) % 16) % 16 / sizeof(T)));
+  const long groups = (n - head) / V, tid = blockIdx.x * 256L + threadIdx.x;
+  for (long i = tid; i < groups; i += gridDim.x * 256L) {
+    union { u32x4 u; T e[V]; } piece;
+    piece.u = *reinterpret_cast<const u32x4 *>(p + head + i * V);
+#pragma unroll
+    for (int j = 0; j < V; j++) take(piece.e[j]);
   }
+  if (tid < head) take(p[tid]);
+  const long tail = head + groups * V;
+  if (tid < n - tail) take(p[tail + tid]);
   fold_max(bad ? 0x7fc00000u : __float_as_uint(m), out);
 }
-// max over (group, c, k) of sum_o |Wt[o, c, k]|
+// max over (group, c, k) of sum_o |Wt[o, c, k]|: a workgroup takes 64 columns, its four wavefronts
+// a quarter of the rows each
 template <typename T>
 __global__ __launch_bounds__(256) void dcn_weight_colsum_kernel(const T *__restrict__ wt, const DcnDims s, unsigned *out) {
-  const long cols = static_cast<long>(s.cpg) * s.K, id = blockIdx.x * 256L + threadIdx.x;
+  __shared__ float part[4][64];
+  const long cols = static_cast<long>(s.cpg) * s.K, id = blockIdx.x * 64L + threadIdx.x % 64;
+  const int wave = threadIdx.x / 64;
   float sum = 0.f;
   if (id < cols * s.groups) {
     const long g = id / cols, ck = id - g * cols;
-    for (int o = 0; o < s.opg; o++) sum += fabsf(static_cast<float>(load(wt + (g * s.opg + o) * cols + ck)));
+    for (int o = wave; o < s.opg; o += 4) sum += fabsf(static_cast<float>(load(wt + (g * s.opg + o) * cols + ck)));
   }
-  fold_max(sum == sum ? __float_as_uint(sum) : 0x7fc00000u, out);
+  part[wave][threadIdx.x % 64] = sum;
+  __syncthreads();
+  if (wave == 0) sum = part[0][threadIdx.x] + part[1][threadIdx.x] + part[2][threadIdx.x] + part[3][threadIdx.x];
+  fold_max(wave == 0 ? (sum == sum ? __float_as_uint(sum) : 0x7fc00000u) : 0u, out);
 }
 
 constexpr int kTapWords = 28;  // byte offsets of the corners in x [8] and in the gradient buffer [8], w[8], mask, ld, lh, lw
@@ -752,12 +770,12 @@ static int backward_run(const void *x, const void *off, const void *mask, const 
     unsigned *bounds = reinterpret_cast<unsigned *>(ws + l.bounds);
     const long ngy = static_cast<long>(s.B) * s.Cout * s.Q, nmask = static_cast<long>(s.B) * s.dg * s.K * s.Q;
     const long ncols = static_cast<long>(s.groups) * s.cpg * s.K;
-    hipLaunchKernelGGL((dcn_absmax_kernel<T>), dim3(static_cast<unsigned>(min((ngy + 4095) / 4096, 1024L))), dim3(256),
+    hipLaunchKernelGGL((dcn_absmax_kernel<T>), dim3(static_cast<unsigned>(min((ngy + 8191) / 8192, 256L))), dim3(256),
                        0, stream, static_cast<const T *>(gy), ngy, bounds);
-    hipLaunchKernelGGL((dcn_weight_colsum_kernel<T>), dim3(static_cast<unsigned>((ncols + 255) / 256)), dim3(256), 0,
+    hipLaunchKernelGGL((dcn_weight_colsum_kernel<T>), dim3(static_cast<unsigned>((ncols + 63) / 64)), dim3(256), 0,
                        stream, static_cast<const T *>(wt), s, bounds + 1);
     if (mask)
-      hipLaunchKernelGGL((dcn_absmax_kernel<T>), dim3(static_cast<unsigned>(min((nmask + 4095) / 4096, 1024L))),
+      hipLaunchKernelGGL((dcn_absmax_kernel<T>), dim3(static_cast<unsigned>(min((nmask + 8191) / 8192, 256L))),
                          dim3(256), 0, stream, static_cast<const T *>(mask), nmask, bounds + 2);
     hipLaunchKernelGGL((dcn_backward_data_mfma_kernel<T, true>), dim3(static_cast<unsigned>(qblocks), s.dg, s.B),
                        dim3(256), 0, stream, xt, static_cast<const T *>(off), static_cast<const T *>(mask), gyt,
