@@ -72,55 +72,61 @@ __device__ __forceinline__ float half_wave_sum(float v) {
 }
 
 // ---- bricks and tiles of the LDS scatter (dcn_backward_scatter_kernel below) ----------------------
-// A brick is kSbD x kSbH x kSbW output positions; its tile the kStD x kStH x kStW input voxels
-// centred on the reach of the brick's undeformed taps.  A corner is "local" when its voxel lies in
+// A brick is BD x BH x BW output positions; its tile the TD x TH x TW input voxels centred on the
+// reach of the brick's undeformed taps.  A corner is "local" when its voxel lies in
 // the tile of its position's brick: local corners are summed in LDS by the scatter kernel, all
 // others are added to the gradient buffer by the data kernel, 128 bytes per request.
-constexpr int kSbD = 4, kSbH = 8, kSbW = 8;
-constexpr int kStD = 10, kStH = 14, kStW = 14;
-constexpr int kStVox = kStD * kStH * kStW;
+// Volumes use 4 x 8 x 8 bricks with 10 x 14 x 14 tiles.  (Images: 16 x 16 bricks with 44 x 44 tiles
+// were measured on 256-channel FPN layers and gained nothing there: four of the eight corner slots
+// are empty and every 8-channel workgroup repeats the tap geometry; they keep the atomics.)
+struct VolumeBricks { static constexpr int BD = 4, BH = 8, BW = 8, TD = 10, TH = 14, TW = 14; };
+constexpr int kBrickPositions = 256, kTileVoxMax = 1960;
 struct TileOrigin { int d, h, w; };
+template <typename S>
 __device__ __forceinline__ TileOrigin tile_origin(const DcnDims &s, int bz, int by, int bx) {
   TileOrigin t;
-  t.d = bz * kSbD * s.sd - s.pd - (kStD - ((kSbD - 1) * s.sd + (s.kd - 1) * s.dd + 1)) / 2;
-  t.h = by * kSbH * s.sh - s.ph - (kStH - ((kSbH - 1) * s.sh + (s.kh - 1) * s.dh + 1)) / 2;
-  t.w = bx * kSbW * s.sw - s.pw - (kStW - ((kSbW - 1) * s.sw + (s.kw - 1) * s.dw + 1)) / 2;
+  t.d = bz * S::BD * s.sd - s.pd - (S::TD - ((S::BD - 1) * s.sd + (s.kd - 1) * s.dd + 1)) / 2;
+  t.h = by * S::BH * s.sh - s.ph - (S::TH - ((S::BH - 1) * s.sh + (s.kh - 1) * s.dh + 1)) / 2;
+  t.w = bx * S::BW * s.sw - s.pw - (S::TW - ((S::BW - 1) * s.sw + (s.kw - 1) * s.dw + 1)) / 2;
   return t;
 }
 // bit c: corner c (z-major) of the sample whose first corner is voxel (id, ih, iw) lies in the tile;
 // `first` its cell index there
+template <typename S>
 __device__ __forceinline__ unsigned tile_bits(const TileOrigin &t, int id, int ih, int iw, int &first) {
   const int zd = id - t.d, zh = ih - t.h, zw = iw - t.w;
-  const bool fd[2] = {zd >= 0 && zd < kStD, zd >= -1 && zd < kStD - 1};
-  const bool fh[2] = {zh >= 0 && zh < kStH, zh >= -1 && zh < kStH - 1};
-  const bool fw[2] = {zw >= 0 && zw < kStW, zw >= -1 && zw < kStW - 1};
+  const bool fd[2] = {zd >= 0 && zd < S::TD, zd >= -1 && zd < S::TD - 1};
+  const bool fh[2] = {zh >= 0 && zh < S::TH, zh >= -1 && zh < S::TH - 1};
+  const bool fw[2] = {zw >= 0 && zw < S::TW, zw >= -1 && zw < S::TW - 1};
   unsigned bits = 0;
 #pragma unroll
   for (int c = 0; c < 8; c++) bits |= (fd[c >> 2] && fh[(c >> 1) & 1] && fw[c & 1]) ? 1u << c : 0u;
-  first = (zd * kStH + zh) * kStW + zw;
+  first = (zd * S::TH + zh) * S::TW + zw;
   return bits;
 }
 
 // The LDS sums are 64-bit fixed point (LDS float atomics retire one lane at a time, integer ones
 // a wavefront in a few clocks).  Every term is w * mask * gcol with 0 <= w <= 1, so
 //   |term| <= max|mask| * max|grad_output| * max_{c,k} sum_o |Wt[o,c,k]|  =: bound < 2^ex,
-// and a voxel takes at most one corner of each (position, tap) of the brick.  Terms are scaled by
-// 2^(50 - ex) and rounded to integers (adding 1.5 * 2^52 in fp64 leaves round(x) in the low
-// mantissa bits for |x| < 2^51): a term loses less than 2^-49 of the bound, and the up to
-// 2^13 terms of a voxel stay below 2^63.  words[0..2] hold the bit patterns of the three maxima
-// (of |.|, so they order like unsigned integers; a NaN or infinity anywhere gives a non-finite
-// bound, and then no corner is treated as local).
+// and a voxel takes at most one corner of each (position, tap) of the brick: 256 * taps terms.
+// Terms are scaled by 2^(shift - ex), shift = min(50, 62 - ceil(log2(terms))), and rounded to
+// integers (adding 1.5 * 2^52 in fp64 leaves round(x) in the low mantissa bits for |x| < 2^51):
+// a term loses less than 2^-shift of the bound (2^-49 for up to 4096 terms), and the sum of a
+// voxel stays below 2^63.  words[0..2] hold the bit patterns of the three maxima (of |.|, so they
+// order like unsigned integers; a NaN or infinity anywhere gives a non-finite bound, and then no
+// corner is treated as local).
 constexpr double kRoundMagic = 6755399441055744.0;  // 1.5 * 2^52
 struct ScatterScale { bool valid; double up, down; };
-__device__ __forceinline__ ScatterScale scatter_scale(const unsigned *__restrict__ words, bool has_mask) {
+__device__ __forceinline__ ScatterScale scatter_scale(const unsigned *__restrict__ words, int taps, bool has_mask) {
   const float bound = 1.001f * __uint_as_float(words[0]) * __uint_as_float(words[1]) *
                       (has_mask ? __uint_as_float(words[2]) : 1.f);
   ScatterScale r;
   r.valid = bound < __builtin_inff() && bound == bound;
   int ex = 0;
   frexpf(fmaxf(bound, 1e-30f), &ex);  // bound < 2^ex
-  r.up = ldexp(1.0, 50 - ex);
-  r.down = ldexp(1.0, ex - 50);
+  const int terms = kBrickPositions * taps, shift = min(50, 62 - (32 - __clz(terms - 1)));
+  r.up = ldexp(1.0, shift - ex);
+  r.down = ldexp(1.0, ex - shift);
   return r;
 }
 // round(w * scaled) as a 64-bit integer; the low word of the magic number's bit pattern is zero
@@ -184,8 +190,8 @@ __global__ __launch_bounds__(256) void dcn_weight_colsum_kernel(const T *__restr
 
 constexpr int kTapWords = 28;  // byte offsets of the corners in x [8] and in the gradient buffer [8], w[8], mask, ld, lh, lw
 
-// SPLIT: corners that are local to their brick's tile are left to the scatter kernel.
-template <typename T, bool SPLIT>
+// SPLIT: corners that are local to their brick's tile (shape S) are left to the scatter kernel.
+template <typename T, bool SPLIT, typename S>
 __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
     const T *__restrict__ xt, const T *__restrict__ off, const T *__restrict__ mask,
     const T *__restrict__ gyt, const T *__restrict__ wb, float *__restrict__ gxt,
@@ -223,8 +229,8 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
   const T *mk = mask ? mask + bg * s.K * s.Q + qc : nullptr;
   float(*tp)[kTapWords] = taps[wave];
   float(*sm)[32] = sums[wave];
-  const TileOrigin origin = tile_origin(s, od / kSbD, oh / kSbH, ow / kSbW);
-  const bool split = SPLIT && scatter_scale(bounds, mask != nullptr).valid;
+  const TileOrigin origin = tile_origin<S>(s, od / S::BD, oh / S::BH, ow / S::BW);
+  const bool split = SPLIT && scatter_scale(bounds, s.K, mask != nullptr).valid;
 
   int ki = 0, kj = 0, kk = 0;
   for (int k = 0; k < s.K; k++) {
@@ -242,7 +248,7 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
       CornerTaps t;
       corner_taps<P>(s, pd, ph, pw, live, cin2, 0u, kOob, t);
       int first;
-      const unsigned local = split ? tile_bits(origin, static_cast<int>(floor(pd)), static_cast<int>(floor(ph)),
+      const unsigned local = split ? tile_bits<S>(origin, static_cast<int>(floor(pd)), static_cast<int>(floor(ph)),
                                                static_cast<int>(floor(pw)), first) : 0u;
       unsigned ag[8];
 #pragma unroll
@@ -384,7 +390,7 @@ __global__ __launch_bounds__(256) void dcn_weight_afragments8_kernel(const T *__
   for (int i = 0; i < PC; i++) wa[id * PC + i] = wt[(static_cast<long>(o + i) * s.cpg + cl) * s.K + k];
 }
 
-template <typename T>
+template <typename T, typename S>
 __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter_kernel(
     const T *__restrict__ off, const T *__restrict__ mask, const T *__restrict__ gyt,
     const T *__restrict__ wa, float *__restrict__ gxt, const DcnDims s, const int nbh, const int nbw,
@@ -392,9 +398,11 @@ __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter_kerne
   using M = Mfma<T>;
   using P = typename std::conditional<(sizeof(T) == 2), float, double>::type;
   constexpr int PC = M::kPiece, SL = 4 * PC;
-  __shared__ unsigned long long tile[kStVox * kScatterStride];
+  constexpr int VOX = S::TD * S::TH * S::TW;
+  static_assert(VOX <= kTileVoxMax && S::BD * S::BH * S::BW == kBrickPositions, "brick and tile sizes");
+  __shared__ unsigned long long tile[VOX * kScatterStride];
   __shared__ __attribute__((aligned(16))) float recs[kScatterWaves][32][8];
-  const ScatterScale scale = scatter_scale(bounds, mask != nullptr);
+  const ScatterScale scale = scatter_scale(bounds, s.K, mask != nullptr);
   if (!scale.valid) return;  // every corner went through the data kernel
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int n = lane % 32, p16 = lane % 16, j = lane / 16;
@@ -405,14 +413,14 @@ __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter_kerne
   const int dgi = c0 / s.cpd, g = c0 / s.cpg, cb = (c0 - g * s.cpg) / 8;
   const long bg = static_cast<long>(b) * s.dg + dgi;
   const int cblocks = s.cpg / 8, steps = s.opg / SL;
-  const TileOrigin origin = tile_origin(s, bz, by, bx);
+  const TileOrigin origin = tile_origin<S>(s, bz, by, bx);
 
-  for (int i = threadIdx.x; i < kStVox * kScatterStride; i += kScatterWaves * 64) tile[i] = 0ull;
+  for (int i = threadIdx.x; i < VOX * kScatterStride; i += kScatterWaves * 64) tile[i] = 0ull;
   __syncthreads();
 
-  // position of brick index i: depth slice i / 64, row (i / 8) % 8, column i % 8
+  // position of brick index i, columns fastest
   auto position = [&](int i, bool &live) {
-    const int od = bz * kSbD + i / (kSbH * kSbW), oh = by * kSbH + (i / kSbW) % kSbH, ow = bx * kSbW + i % kSbW;
+    const int od = bz * S::BD + i / (S::BH * S::BW), oh = by * S::BH + (i / S::BW) % S::BH, ow = bx * S::BW + i % S::BW;
     live = od < s.Do && oh < s.Ho && ow < s.Wo;
     return (static_cast<long>(min(od, s.Do - 1)) * s.Ho + min(oh, s.Ho - 1)) * s.Wo + min(ow, s.Wo - 1);
   };
@@ -475,7 +483,7 @@ __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter_kerne
       CornerTaps t;
       corner_taps<P>(s, pd, ph, pw, live, 1u, 0u, ~0u, t);
       int first;
-      unsigned bits = tile_bits(origin, static_cast<int>(floor(pd)), static_cast<int>(floor(ph)),
+      unsigned bits = tile_bits<S>(origin, static_cast<int>(floor(pd)), static_cast<int>(floor(ph)),
                                 static_cast<int>(floor(pw)), first);
       unsigned inside = 0;
 #pragma unroll
@@ -521,7 +529,7 @@ __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter_kerne
         const int ca = c >> 2, cb2 = (c >> 1) & 1, ce = c & 1;
         if ((bits >> c) & 1u) {
           const float wc = wd[ca] * wh[cb2] * ww[ce];
-          unsigned long long *dst = tile + (first + ca * (kStH * kStW) + cb2 * kStW + ce) * kScatterStride + j;
+          unsigned long long *dst = tile + (first + ca * (S::TH * S::TW) + cb2 * S::TW + ce) * kScatterStride + j;
 #pragma unroll
           for (int r = 0; r < 2; r++)
             __hip_atomic_fetch_add(dst + 4 * r, fixed_term(wc, gv[r]), __ATOMIC_RELAXED,
@@ -541,8 +549,8 @@ __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter_kerne
       gxt + static_cast<long>(b) * s.P * s.Cin, 0, static_cast<int>(s.P * s.Cin * 4), kRsrcFlags);
   const unsigned cin4 = static_cast<unsigned>(s.Cin) * 4u;
   const int ch = threadIdx.x % 8;
-  for (int cell = threadIdx.x / 8; cell < kStVox; cell += kScatterWaves * 8) {
-    const int zw = cell % kStW + origin.w, zh = (cell / kStW) % kStH + origin.h, zd = cell / (kStW * kStH) + origin.d;
+  for (int cell = threadIdx.x / 8; cell < VOX; cell += kScatterWaves * 8) {
+    const int zw = cell % S::TW + origin.w, zh = (cell / S::TW) % S::TH + origin.h, zd = cell / (S::TW * S::TH) + origin.d;
     const unsigned long long sum = tile[cell * kScatterStride + ch];
     if (zd >= 0 && zd < s.D && zh >= 0 && zh < s.H && zw >= 0 && zw < s.W && sum != 0ull) {
       const double v = static_cast<double>(static_cast<long long>(sum)) * scale.down;
@@ -705,10 +713,12 @@ __global__ void dcn_zero_f32_kernel(float *p, long n) {
 
 // The LDS scatter pays when its tile holds the reach of a brick's undeformed taps with a voxel to
 // spare on either side (offsets beyond the tile still work, through the data kernel's atomics).
+template <typename S>
 static bool scatter_tile_applies(const DcnDims &s) {
-  const int ed = (kSbD - 1) * s.sd + (s.kd - 1) * s.dd + 1, eh = (kSbH - 1) * s.sh + (s.kh - 1) * s.dh + 1,
-            ew = (kSbW - 1) * s.sw + (s.kw - 1) * s.dw + 1;
-  return s.nd == 3 && ed + 2 <= kStD && eh + 2 <= kStH && ew + 2 <= kStW;
+  const int ed = (S::BD - 1) * s.sd + (s.kd - 1) * s.dd + 1, eh = (S::BH - 1) * s.sh + (s.kh - 1) * s.dh + 1,
+            ew = (S::BW - 1) * s.sw + (s.kw - 1) * s.dw + 1;
+  return ed + 2 <= S::TD && eh + 2 <= S::TH && ew + 2 <= S::TW &&
+         static_cast<long>(kBrickPositions) * s.K < (1L << 20);
 }
 
 static size_t align256b(size_t v) { return (v + 255) / 256 * 256; }
@@ -766,7 +776,7 @@ static int backward_run(const void *x, const void *off, const void *mask, const 
                      0, stream, gxt, nz);
   const long qblocks = (s.Q + 127) / 128;
   MV_REQUIRE(qblocks < (1L << 31), "grid too large");
-  if (scatter_tile_applies(s)) {
+  if (s.nd == 3 && scatter_tile_applies<VolumeBricks>(s)) {
     unsigned *bounds = reinterpret_cast<unsigned *>(ws + l.bounds);
     const long ngy = static_cast<long>(s.B) * s.Cout * s.Q, nmask = static_cast<long>(s.B) * s.dg * s.K * s.Q;
     const long ncols = static_cast<long>(s.groups) * s.cpg * s.K;
@@ -777,23 +787,30 @@ static int backward_run(const void *x, const void *off, const void *mask, const 
     if (mask)
       hipLaunchKernelGGL((dcn_absmax_kernel<T>), dim3(static_cast<unsigned>(min((nmask + 8191) / 8192, 256L))),
                          dim3(256), 0, stream, static_cast<const T *>(mask), nmask, bounds + 2);
-    hipLaunchKernelGGL((dcn_backward_data_mfma_kernel<T, true>), dim3(static_cast<unsigned>(qblocks), s.dg, s.B),
-                       dim3(256), 0, stream, xt, static_cast<const T *>(off), static_cast<const T *>(mask), gyt,
-                       wb, gxt, static_cast<T *>(goff), static_cast<T *>(gmask), s, bounds);
     T *wa = reinterpret_cast<T *>(ws + l.wa);
     const long lanes8 = static_cast<long>(s.groups) * s.K * (s.cpg / 8) * (s.opg / (4 * Mfma<T>::kPiece)) * 64;
     hipLaunchKernelGGL((dcn_weight_afragments8_kernel<T>), dim3(static_cast<unsigned>((lanes8 + 255) / 256)),
                        dim3(256), 0, stream, static_cast<const T *>(wt), wa, s);
-    const long nbd = (s.Do + kSbD - 1) / kSbD, nbh = (s.Ho + kSbH - 1) / kSbH, nbw = (s.Wo + kSbW - 1) / kSbW;
-    MV_REQUIRE(nbd * nbh * nbw < (1L << 31) && s.Cin / 8 <= 65535, "grid too large");
-    hipLaunchKernelGGL((dcn_backward_scatter_kernel<T>), dim3(static_cast<unsigned>(nbd * nbh * nbw), s.Cin / 8, s.B),
-                       dim3(kScatterWaves * 64), 0, stream, static_cast<const T *>(off),
-                       static_cast<const T *>(mask), gyt, wa, gxt, s, static_cast<int>(nbh), static_cast<int>(nbw),
-                       bounds);
+    MV_REQUIRE(s.Cin / 8 <= 65535, "grid too large");
+#define MV_LAUNCH_SPLIT(S)                                                                                        \
+  {                                                                                                               \
+    hipLaunchKernelGGL((dcn_backward_data_mfma_kernel<T, true, S>), dim3(static_cast<unsigned>(qblocks), s.dg, s.B), \
+                       dim3(256), 0, stream, xt, static_cast<const T *>(off), static_cast<const T *>(mask), gyt,  \
+                       wb, gxt, static_cast<T *>(goff), static_cast<T *>(gmask), s, bounds);                      \
+    const long nbd = (s.Do + S::BD - 1) / S::BD, nbh = (s.Ho + S::BH - 1) / S::BH, nbw = (s.Wo + S::BW - 1) / S::BW; \
+    MV_REQUIRE(nbd * nbh * nbw < (1L << 31), "grid too large");                                                   \
+    hipLaunchKernelGGL((dcn_backward_scatter_kernel<T, S>),                                                       \
+                       dim3(static_cast<unsigned>(nbd * nbh * nbw), s.Cin / 8, s.B), dim3(kScatterWaves * 64), 0, \
+                       stream, static_cast<const T *>(off), static_cast<const T *>(mask), gyt, wa, gxt, s,        \
+                       static_cast<int>(nbh), static_cast<int>(nbw), bounds);                                     \
+  }
+    MV_LAUNCH_SPLIT(VolumeBricks)
+#undef MV_LAUNCH_SPLIT
   } else {
-    hipLaunchKernelGGL((dcn_backward_data_mfma_kernel<T, false>), dim3(static_cast<unsigned>(qblocks), s.dg, s.B),
-                       dim3(256), 0, stream, xt, static_cast<const T *>(off), static_cast<const T *>(mask), gyt,
-                       wb, gxt, static_cast<T *>(goff), static_cast<T *>(gmask), s, nullptr);
+    hipLaunchKernelGGL((dcn_backward_data_mfma_kernel<T, false, VolumeBricks>),
+                       dim3(static_cast<unsigned>(qblocks), s.dg, s.B), dim3(256), 0, stream, xt,
+                       static_cast<const T *>(off), static_cast<const T *>(mask), gyt, wb, gxt,
+                       static_cast<T *>(goff), static_cast<T *>(gmask), s, nullptr);
   }
   const dim3 wgrid(static_cast<unsigned>(static_cast<long>(s.Cin / 32) * s.K),
                    static_cast<unsigned>((s.Q + kGwChunk - 1) / kGwChunk), s.B);
