@@ -219,6 +219,7 @@ int dcn_mfma_backward(const void *x, const void *off, const void *mask, const vo
                       void *workspace, float **gx32, float **gw32, float **gb32,
                       hipStream_t stream);
 int dcn_planar_add(const float *gxt, void *gx, const DcnDims &s, int dtype, hipStream_t stream);
+int dcn_weight_add(const float *acc, void *gw, const DcnDims &s, int dtype, hipStream_t stream);
 
 static inline int blocks_for(long n, int per_block, int cap) {
   return static_cast<int>(std::min<long>((n + per_block - 1) / per_block, cap));
@@ -300,13 +301,13 @@ static int dcn_backward_any(const void *input, const void *offset, const void *m
         if (grad_bias)
           hipLaunchKernelGGL((dcn_backward_bias_kernel<T, G>), dim3(s.Cout, s.B, static_cast<unsigned>((s.Q + kBiasSlab - 1) / kBiasSlab)), dim3(256), 0, hs,
                              static_cast<const T *>(grad_output), gb32, s);
-        hipLaunchKernelGGL((dcn_add_from_f32_kernel<T>), dim3(blocks_for(n_gw, 1024, 65536)), dim3(256),
-                           0, hs, static_cast<T *>(grad_weight), gw32, n_gw);
         if (grad_bias)
           hipLaunchKernelGGL((dcn_add_from_f32_kernel<T>), dim3(1), dim3(256), 0, hs,
                              static_cast<T *>(grad_bias), gb32, static_cast<long>(s.Cout));
       }
     });
+    st = dcn_weight_add(gw32, grad_weight, s, dtype, hs);
+    if (st) return st;
     return check_launch("dcn3d backward");
   }
   if (narrow) {

@@ -23,6 +23,8 @@
 // over the whole range and are added to the fp32 gradient once per workgroup.
 #include "dcn_mfma.hpp"
 
+#include <cstdlib>
+
 namespace mv {
 
 constexpr unsigned kOob = 0x80000000u;  // byte offset beyond every buffer: loads give 0, atomics are dropped
@@ -195,7 +197,8 @@ template <typename T, bool SPLIT, typename S>
 __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
     const T *__restrict__ xt, const T *__restrict__ off, const T *__restrict__ mask,
     const T *__restrict__ gyt, const T *__restrict__ wb, float *__restrict__ gxt,
-    T *__restrict__ goff, T *__restrict__ gmask, const DcnDims s, const unsigned *__restrict__ bounds) {
+    T *__restrict__ goff, T *__restrict__ gmask, const DcnDims s, const unsigned *__restrict__ bounds,
+    T *__restrict__ col, const long qp) {
   using M = Mfma<T>;
   using P = typename std::conditional<(sizeof(T) == 2), float, double>::type;  // position type
   constexpr int PC = M::kPiece, SL = 2 * PC, ES = sizeof(T);
@@ -283,6 +286,8 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
         acc = M::run(a, bf, acc);
       }
       const unsigned cbyte4 = static_cast<unsigned>(c0 + n) * 4u;
+      float colv[4];
+      T *colrow = col ? col + ((static_cast<long>(b) * s.K + k) * (s.Cin / 32) + c0 / 32) * qp * 32 : nullptr;
       // ---- register r: position 8*(r/4) + 4*h + r%4, channel c0 + n ------------------------------
       // fetch f of register r: lane l holds 16 bytes of corner (f * 64 + l) / LPC of the register's
       // two positions (corners 0..7 of the lower half-wavefront's position, then the upper one's).
@@ -337,6 +342,18 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
         const float s3 = half_wave_sum(acc[r] * val);
         if (n == 16) {  // one lane per half-wavefront; the chunks of a deformable group accumulate
           sm[0][p] += s0; sm[1][p] += s1; sm[2][p] += s2; sm[3][p] += s3;
+        }
+        // ---- the column values mask * Z(x) for the weight kernel: registers 4g .. 4g + 3 are four
+        // consecutive positions, pieces are [position / kPiece][channel][kPiece] ----------------------
+        colv[r % 4] = m * val;
+        if (col && r % 4 == 3) {
+          const long first = q0 + 8 * (r / 4) + 4 * h;  // position of colv[0]
+          T *dst = colrow + ((first / PC) * 32 + n) * PC + first % PC;
+          if constexpr (ES == 2) {
+            *reinterpret_cast<uint2 *>(dst) = make_uint2(M::pack2(colv[0], colv[1]), M::pack2(colv[2], colv[3]));
+          } else {
+            *reinterpret_cast<float4 *>(dst) = make_float4(colv[0], colv[1], colv[2], colv[3]);
+          }
         }
       }
     }
@@ -564,10 +581,14 @@ __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter_kerne
 // ---- grad wrt weight ---------------------------------------------------------------------------
 constexpr int kGwChunk = 2048;  // positions per workgroup
 
-template <typename T, int MT>
+// COL: the column values come from the buffer the data kernel wrote (pieces [position / kPiece]
+// [channel][kPiece] per (sample, tap, 32-channel block), `qp` positions each) instead of being
+// gathered again.
+template <typename T, int MT, bool COL>
 __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
     const T *__restrict__ xt, const T *__restrict__ off, const T *__restrict__ mask,
-    const T *__restrict__ gy, float *__restrict__ gw, const DcnDims s, const int mb0) {
+    const T *__restrict__ gy, float *__restrict__ gw, const DcnDims s, const int mb0,
+    const T *__restrict__ col, const long qp) {
   using M = Mfma<T>;
   using P = typename std::conditional<(sizeof(T) == 2), float, double>::type;  // position type
   constexpr int PC = M::kPiece, SL = 2 * PC, ES = sizeof(T);
@@ -598,9 +619,10 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
     for (int r = 0; r < 16; r++) acc[m][r] = 0.f;
 
   const long qend = min(qbase + kGwChunk, s.Q);
+  const T *colrow = COL ? col + ((static_cast<long>(b) * s.K + k) * cblocks_all + cbi) * qp * 32 : nullptr;
   for (long qg = qbase + wave * 64; qg < qend; qg += 256) {
     // ---- taps of the 64 positions qg + lane ------------------------------------------------------
-    {
+    if (!COL) {
       const long q = qg + lane;
       const bool live = q < s.Q;
       const long qc = live ? q : s.Q - 1;
@@ -621,10 +643,28 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll 1
+    // gathering: one step at a time (registers); from the column buffer: all loads of the 64
+    // positions in flight together
+    constexpr int kStepUnroll = COL ? kWave / SL : 1;
+#pragma unroll kStepUnroll
     for (int st = 0; st < kWave / SL; st++) {  // SL positions per step
       // B piece: column n = channel c0 + n, rows = positions st*SL + h*PC + i
-      float col[PC];
+      u32x4 bf;
+      const long qa = qg + st * SL + h * PC;
+      if (COL) {
+        union { u32x4 u; T e[PC]; } piece;
+        piece.u = u32x4{0u, 0u, 0u, 0u};
+        if (qa < s.Q) {
+          piece.u = *reinterpret_cast<const u32x4 *>(colrow + ((qa / PC) * 32 + n) * PC);
+          if (qa + PC > s.Q) {
+#pragma unroll
+            for (int i = 0; i < PC; i++)
+              if (qa + i >= s.Q) piece.e[i] = store_cast<T>(0.f);
+          }
+        }
+        bf = piece.u;
+      } else {
+      float colv[PC];
 #pragma unroll
       for (int i = 0; i < PC; i++) {
         const float4 *src = reinterpret_cast<const float4 *>(tp[st * SL + h * PC + i]);
@@ -635,11 +675,11 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
         float a = 0.f;
 #pragma unroll
         for (int c = 0; c < 8; c++) a += w[c] * load_element<T>(xr, ax[c] + cbyte2);  // kOob + channel: reads 0
-        col[i] = a;
+        colv[i] = a;
       }
-      const u32x4 bf = M::pack(col);
+      bf = M::pack(colv);
+      }
       // A pieces: row n = output channel, columns = the same PC positions
-      const long qa = qg + st * SL + h * PC;
 #pragma unroll
       for (int m = 0; m < MT; m++) {
         const T *grow = gy + (static_cast<long>(b) * s.Cout + g * s.opg + (mb0 + m) * 32 + n) * s.Q + qa;
@@ -675,7 +715,8 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
         // accumulator layout: register r of lane l = row 8*(r/4) + 4*(l/32) + r%4, column l%32
         const int o = g * s.opg + (mb0 + m) * 32 + 8 * (r / 4) + 4 * h + (r % 4);
         const int cl = c0 - g * s.cpg + n;
-        atomicAdd(gw + (static_cast<long>(o) * s.cpg + cl) * s.K + k, v);
+        // tap-major accumulator [K][Cout][cpg]: the 32 lanes of a row add to 128 contiguous bytes
+        atomicAdd(gw + (static_cast<long>(k) * s.Cout + o) * s.cpg + cl, v);
       }
   }
 }
@@ -735,8 +776,16 @@ bool dcn_mfma_backward_supported(const DcnDims &s, int dtype) {
 // workspace: xt | gyt | weight fragments (32- and 8-channel blocks) | gxt (fp32) | gw (fp32) | gb (fp32) |
 // the three maxima of the scatter scale; everything from gxt on starts at zero
 struct BackwardLayout {
-  size_t xt, gyt, wb, wa, gxt, gw, gb, bounds, total;
+  size_t xt, gyt, wb, wa, col, gxt, gw, gb, bounds, total;
+  long qp;  // positions per row of the column buffer; 0: no buffer (the weight kernel gathers again)
 };
+// The column buffer holds mask * Z(x) for every (sample, tap, channel, position): it saves the
+// weight kernel the second gather of x.  Layers whose columns exceed the budget (1 GiB, or the value
+// of MV_DCN_COLUMN_BYTES) do without.
+static size_t column_budget() {
+  const char *e = getenv("MV_DCN_COLUMN_BYTES");
+  return e ? static_cast<size_t>(strtoull(e, nullptr, 10)) : (static_cast<size_t>(1) << 30);
+}
 static BackwardLayout backward_layout(const DcnDims &s, int dtype) {
   BackwardLayout l;
   const size_t es = dtype == MV_F32 ? 4 : 2;
@@ -745,6 +794,10 @@ static BackwardLayout backward_layout(const DcnDims &s, int dtype) {
   l.gyt = at; at += align256b(static_cast<size_t>(s.B) * s.Q * s.Cout * es);
   l.wb = at; at += align256b(static_cast<size_t>(s.Cout) * s.cpg * s.K * es);
   l.wa = at; at += align256b(2 * static_cast<size_t>(s.Cout) * s.cpg * s.K * es);  // 16 MFMA rows per 8 channels
+  const long qp = (s.Q + 63) / 64 * 64;
+  const size_t col_bytes = static_cast<size_t>(s.B) * s.K * s.Cin * qp * es;
+  l.qp = col_bytes <= column_budget() ? qp : 0;
+  l.col = at; at += l.qp ? align256b(col_bytes) : 0;
   l.gxt = at; at += align256b(static_cast<size_t>(s.B) * s.P * s.Cin * 4);
   l.gw = at; at += align256b(static_cast<size_t>(s.Cout) * s.cpg * s.K * 4);
   l.gb = at; at += align256b(static_cast<size_t>(s.Cout) * 4);
@@ -763,6 +816,7 @@ static int backward_run(const void *x, const void *off, const void *mask, const 
   char *ws = static_cast<char *>(workspace);
   T *xt = reinterpret_cast<T *>(ws + l.xt), *gyt = reinterpret_cast<T *>(ws + l.gyt), *wb = reinterpret_cast<T *>(ws + l.wb);
   float *gxt = reinterpret_cast<float *>(ws + l.gxt);
+  T *col = l.qp ? reinterpret_cast<T *>(ws + l.col) : nullptr;
   *gx32 = gxt; *gw32 = reinterpret_cast<float *>(ws + l.gw); *gb32 = reinterpret_cast<float *>(ws + l.gb);
   int st = dcn_channels_last(x, xt, s.B, s.Cin, s.P, sizeof(T), stream);
   if (st) return st;
@@ -796,7 +850,7 @@ static int backward_run(const void *x, const void *off, const void *mask, const 
   {                                                                                                               \
     hipLaunchKernelGGL((dcn_backward_data_mfma_kernel<T, true, S>), dim3(static_cast<unsigned>(qblocks), s.dg, s.B), \
                        dim3(256), 0, stream, xt, static_cast<const T *>(off), static_cast<const T *>(mask), gyt,  \
-                       wb, gxt, static_cast<T *>(goff), static_cast<T *>(gmask), s, bounds);                      \
+                       wb, gxt, static_cast<T *>(goff), static_cast<T *>(gmask), s, bounds, col, l.qp);           \
     const long nbd = (s.Do + S::BD - 1) / S::BD, nbh = (s.Ho + S::BH - 1) / S::BH, nbw = (s.Wo + S::BW - 1) / S::BW; \
     MV_REQUIRE(nbd * nbh * nbw < (1L << 31), "grid too large");                                                   \
     hipLaunchKernelGGL((dcn_backward_scatter_kernel<T, S>),                                                       \
@@ -810,14 +864,19 @@ static int backward_run(const void *x, const void *off, const void *mask, const 
     hipLaunchKernelGGL((dcn_backward_data_mfma_kernel<T, false, VolumeBricks>),
                        dim3(static_cast<unsigned>(qblocks), s.dg, s.B), dim3(256), 0, stream, xt,
                        static_cast<const T *>(off), static_cast<const T *>(mask), gyt, wb, gxt,
-                       static_cast<T *>(goff), static_cast<T *>(gmask), s, nullptr);
+                       static_cast<T *>(goff), static_cast<T *>(gmask), s, nullptr, col, l.qp);
   }
   const dim3 wgrid(static_cast<unsigned>(static_cast<long>(s.Cin / 32) * s.K),
                    static_cast<unsigned>((s.Q + kGwChunk - 1) / kGwChunk), s.B);
-#define MV_LAUNCH_GW(MTV)                                                                          \
-  hipLaunchKernelGGL((dcn_backward_weight_mfma_kernel<T, MTV>), wgrid, dim3(256), 0, stream, xt,   \
-                     static_cast<const T *>(off), static_cast<const T *>(mask),                    \
-                     static_cast<const T *>(gy), *gw32, s, mb0)
+#define MV_LAUNCH_GW(MTV)                                                                              \
+  if (col)                                                                                             \
+    hipLaunchKernelGGL((dcn_backward_weight_mfma_kernel<T, MTV, true>), wgrid, dim3(256), 0, stream, xt, \
+                       static_cast<const T *>(off), static_cast<const T *>(mask),                      \
+                       static_cast<const T *>(gy), *gw32, s, mb0, col, l.qp);                          \
+  else                                                                                                 \
+    hipLaunchKernelGGL((dcn_backward_weight_mfma_kernel<T, MTV, false>), wgrid, dim3(256), 0, stream, xt, \
+                       static_cast<const T *>(off), static_cast<const T *>(mask),                      \
+                       static_cast<const T *>(gy), *gw32, s, mb0, col, l.qp)
   // up to four 32-row blocks of output channels per pass over the positions
   for (int mb0 = 0; mb0 < s.opg / 32; mb0 += 4)
     switch (min(s.opg / 32 - mb0, 4)) {
@@ -831,7 +890,8 @@ static int backward_run(const void *x, const void *off, const void *mask, const 
 }
 
 // Runs the data and weight kernels; grad_offset / grad_mask are written, the fp32 gradients of
-// input (channels-last), weight and bias accumulators are returned for the caller to fold in.
+// input (channels-last; dcn_planar_add), weight (tap-major; dcn_weight_add) and bias accumulators
+// are returned for the caller to fold in.
 int dcn_mfma_backward(const void *x, const void *off, const void *mask, const void *wt,
                       const void *gy, void *goff, void *gmask, const DcnDims &s, int dtype,
                       void *workspace, float **gx32, float **gw32, float **gb32,
@@ -858,6 +918,29 @@ int planar_add_f32(const float *src, void *dst, int B, int C, long P, int dtype,
     hipLaunchKernelGGL((dcn_planar_add_kernel<__hip_bfloat16>), grid, dim3(256), 0, stream, src,
                        static_cast<__hip_bfloat16 *>(dst), C, P);
   return check_launch("dcn_planar_add_kernel");
+}
+
+// grad_weight [Cout][cpg][K] += the tap-major fp32 accumulator [K][Cout][cpg] of the weight kernel
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_weight_add_kernel(const float *__restrict__ acc, T *__restrict__ gw,
+                                                             const DcnDims s) {
+  const long n = static_cast<long>(s.Cout) * s.cpg * s.K;
+  for (long i = blockIdx.x * 256L + threadIdx.x; i < n; i += gridDim.x * 256L) {
+    const long k = i % s.K, oc = i / s.K;
+    gw[i] = store_cast<T>(load(gw + i) + acc[k * s.Cout * s.cpg + oc]);
+  }
+}
+int dcn_weight_add(const float *acc, void *gw, const DcnDims &s, int dtype, hipStream_t stream) {
+  const long n = static_cast<long>(s.Cout) * s.cpg * s.K;
+  const dim3 grid(static_cast<unsigned>(min((n + 255) / 256, 4096L)));
+  if (dtype == MV_F16)
+    hipLaunchKernelGGL((dcn_weight_add_kernel<__half>), grid, dim3(256), 0, stream, acc, static_cast<__half *>(gw), s);
+  else if (dtype == MV_F32)
+    hipLaunchKernelGGL((dcn_weight_add_kernel<float>), grid, dim3(256), 0, stream, acc, static_cast<float *>(gw), s);
+  else
+    hipLaunchKernelGGL((dcn_weight_add_kernel<__hip_bfloat16>), grid, dim3(256), 0, stream, acc,
+                       static_cast<__hip_bfloat16 *>(gw), s);
+  return check_launch("dcn_weight_add_kernel");
 }
 
 int dcn_planar_add(const float *gxt, void *gx, const DcnDims &s, int dtype, hipStream_t stream) {

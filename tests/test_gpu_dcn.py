@@ -166,6 +166,24 @@ def test_input_gradient_through_lds_tiles_5x5x5(ops, oracle):
     assert_close(ws.grad, gw, tol, "grad weight")
 
 
+def test_weight_gradient_without_column_buffer(ops, oracle, monkeypatch):
+    """Layers whose column values would not fit the buffer's budget gather x a second time in the
+    weight kernel: forced here through MV_DCN_COLUMN_BYTES."""
+    from medvision_amd.ops.modulated_deform_conv_3d import modulated_deform_conv
+    monkeypatch.setenv("MV_DCN_COLUMN_BYTES", "0")
+    g = wl.gen(450)
+    x, off, mask, w, b = wl.dcn_inputs(g, 2, 32, 64, (7, 9, 11), 3, 1, 1, torch.float16, 1, 1, 1, True, 2.0)
+    xs, offs, ms, ws, bs = [t.to(DEV).requires_grad_(True) for t in (x, off, mask, w, b)]
+    y = modulated_deform_conv(xs, offs, ms, ws, bs, 1, 1, 1, 1, 1)
+    gy = torch.randn(y.shape, generator=g).half()
+    y.backward(gy.to(DEV))
+    gx, goff, gm, gw, gb = oracle.dcn3d_backward(x, off, mask, w, gy, True, 1, 1, 1, 1, 1)
+    tol = BWD_TOL[torch.float16]
+    assert_close(ws.grad, gw, tol, "grad weight")
+    assert_close(xs.grad, gx, tol, "grad input")
+    assert_close(offs.grad, goff, tol, "grad offset")
+
+
 def test_input_gradient_with_non_finite_values(ops, oracle):
     """An infinity in grad_output makes the bound of the fixed-point sums non-finite: every corner
     then goes through the fp32 atomics, and NaN / infinity reach exactly the voxels the oracle's do."""
