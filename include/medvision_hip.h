@@ -123,6 +123,9 @@ typedef struct {
 
 int mv_dcn3d_output_dims(const mv_dcn3d_shape *shape, int *out_d, int *out_h, int *out_w);
 size_t mv_dcn3d_forward_workspace_bytes(const mv_dcn3d_shape *shape, int dtype);
+/* The backward workspace of 16-bit / fp32 layers on the matrix-core path includes a buffer of column
+ * values (batch x taps x in_channels x positions elements) while that stays below 1 GiB or the number
+ * of bytes in the environment variable MV_DCN_COLUMN_BYTES (read by the query and by the call). */
 size_t mv_dcn3d_backward_workspace_bytes(const mv_dcn3d_shape *shape, int dtype);
 int mv_dcn3d_forward(const void *input, const void *offset, const void *mask, const void *weight,
                      const void *bias, void *output, const mv_dcn3d_shape *shape, int dtype,
