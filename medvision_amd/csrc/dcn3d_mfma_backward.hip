@@ -581,14 +581,10 @@ __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter_kerne
 // ---- grad wrt weight ---------------------------------------------------------------------------
 constexpr int kGwChunk = 2048;  // positions per workgroup
 
-// COL: the column values come from the buffer the data kernel wrote (pieces [position / kPiece]
-// [channel][kPiece] per (sample, tap, 32-channel block), `qp` positions each) instead of being
-// gathered again.
-template <typename T, int MT, bool COL>
+template <typename T, int MT>
 __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
     const T *__restrict__ xt, const T *__restrict__ off, const T *__restrict__ mask,
-    const T *__restrict__ gy, float *__restrict__ gw, const DcnDims s, const int mb0,
-    const T *__restrict__ col, const long qp) {
+    const T *__restrict__ gy, float *__restrict__ gw, const DcnDims s, const int mb0) {
   using M = Mfma<T>;
   using P = typename std::conditional<(sizeof(T) == 2), float, double>::type;  // position type
   constexpr int PC = M::kPiece, SL = 2 * PC, ES = sizeof(T);
@@ -619,10 +615,9 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
     for (int r = 0; r < 16; r++) acc[m][r] = 0.f;
 
   const long qend = min(qbase + kGwChunk, s.Q);
-  const T *colrow = COL ? col + ((static_cast<long>(b) * s.K + k) * cblocks_all + cbi) * qp * 32 : nullptr;
   for (long qg = qbase + wave * 64; qg < qend; qg += 256) {
     // ---- taps of the 64 positions qg + lane ------------------------------------------------------
-    if (!COL) {
+    {
       const long q = qg + lane;
       const bool live = q < s.Q;
       const long qc = live ? q : s.Q - 1;
@@ -643,27 +638,9 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    // gathering: one step at a time (registers); from the column buffer: all loads of the 64
-    // positions in flight together
-    constexpr int kStepUnroll = COL ? kWave / SL : 1;
-#pragma unroll kStepUnroll
+#pragma unroll 1
     for (int st = 0; st < kWave / SL; st++) {  // SL positions per step
       // B piece: column n = channel c0 + n, rows = positions st*SL + h*PC + i
-      u32x4 bf;
-      const long qa = qg + st * SL + h * PC;
-      if (COL) {
-        union { u32x4 u; T e[PC]; } piece;
-        piece.u = u32x4{0u, 0u, 0u, 0u};
-        if (qa < s.Q) {
-          piece.u = *reinterpret_cast<const u32x4 *>(colrow + ((qa / PC) * 32 + n) * PC);
-          if (qa + PC > s.Q) {
-#pragma unroll
-            for (int i = 0; i < PC; i++)
-              if (qa + i >= s.Q) piece.e[i] = store_cast<T>(0.f);
-          }
-        }
-        bf = piece.u;
-      } else {
       float colv[PC];
 #pragma unroll
       for (int i = 0; i < PC; i++) {
@@ -677,9 +654,9 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
         for (int c = 0; c < 8; c++) a += w[c] * load_element<T>(xr, ax[c] + cbyte2);  // kOob + channel: reads 0
         colv[i] = a;
       }
-      bf = M::pack(colv);
-      }
+      const u32x4 bf = M::pack(colv);
       // A pieces: row n = output channel, columns = the same PC positions
+      const long qa = qg + st * SL + h * PC;
 #pragma unroll
       for (int m = 0; m < MT; m++) {
         const T *grow = gy + (static_cast<long>(b) * s.Cout + g * s.opg + (mb0 + m) * 32 + n) * s.Q + qa;
@@ -718,6 +695,103 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_mfma_kernel(
         // tap-major accumulator [K][Cout][cpg]: the 32 lanes of a row add to 128 contiguous bytes
         atomicAdd(gw + (static_cast<long>(k) * s.Cout + o) * s.cpg + cl, v);
       }
+  }
+}
+
+// The same contraction with the column values read from the buffer the data kernel wrote (pieces
+// [position / kPiece][channel][kPiece] per (sample, tap, 32-channel block), `qp` positions each): no
+// gather, and a workgroup takes TPW taps at once so that a piece of grad_output (16 useful bytes of
+// a 64-byte request per lane) serves TPW products.
+template <typename T, int MT, int TPW>
+__global__ __launch_bounds__(256) void dcn_backward_weight_columns_kernel(
+    const T *__restrict__ col, const T *__restrict__ gy, float *__restrict__ gw, const DcnDims s,
+    const int mb0, const long qp) {
+  using M = Mfma<T>;
+  constexpr int PC = M::kPiece, SL = 2 * PC;
+  __shared__ float part[3][16][64];  // an accumulator of wavefronts 1..3
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int n = lane % 32, h = lane / 32;
+  const int tgroups = (s.K + TPW - 1) / TPW, cblocks_all = s.Cin / 32;
+  const int k0 = (blockIdx.x % tgroups) * TPW, cbi = blockIdx.x / tgroups;
+  const int c0 = cbi * 32, g = c0 / s.cpg, b = blockIdx.z;
+  const long qbase = static_cast<long>(blockIdx.y) * kGwChunk, qend = min(qbase + kGwChunk, s.Q);
+  const bool aligned = s.Q % PC == 0;
+  const T *colrow[TPW];  // taps beyond the last one repeat it; their products are not used
+#pragma unroll
+  for (int t = 0; t < TPW; t++)
+    colrow[t] = col + ((static_cast<long>(b) * s.K + min(k0 + t, s.K - 1)) * cblocks_all + cbi) * qp * 32;
+
+  float16_t acc[TPW][MT];
+#pragma unroll
+  for (int t = 0; t < TPW; t++)
+#pragma unroll
+    for (int m = 0; m < MT; m++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[t][m][r] = 0.f;
+
+  for (long qg = qbase + wave * 64; qg < qend; qg += 256) {
+#pragma unroll
+    for (int st = 0; st < kWave / SL; st++) {  // SL positions per step
+      const long qa = qg + st * SL + h * PC;
+      // A pieces: row n = output channel, columns = PC positions
+      u32x4 a[MT];
+#pragma unroll
+      for (int m = 0; m < MT; m++) {
+        const T *grow = gy + (static_cast<long>(b) * s.Cout + g * s.opg + (mb0 + m) * 32 + n) * s.Q + qa;
+        union { u32x4 u; T e[PC]; } piece;
+        if (aligned && qa + PC <= s.Q) {
+          piece.u = *reinterpret_cast<const u32x4 *>(grow);
+        } else {
+          piece.u = u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+          for (int i = 0; i < PC; i++)
+            if (qa + i < s.Q) piece.e[i] = grow[i];
+        }
+        a[m] = piece.u;
+      }
+      // B pieces: column n = channel c0 + n, rows = the same PC positions.  Positions beyond Q
+      // contribute nothing because their A elements are zero, but the buffer must not be read
+      // where nothing was written.
+#pragma unroll
+      for (int t = 0; t < TPW; t++) {
+        union { u32x4 u; T e[PC]; } piece;
+        piece.u = u32x4{0u, 0u, 0u, 0u};
+        if (qa < s.Q) {
+          piece.u = *reinterpret_cast<const u32x4 *>(colrow[t] + ((qa / PC) * 32 + n) * PC);
+          if (qa + PC > s.Q) {
+#pragma unroll
+            for (int i = 0; i < PC; i++)
+              if (qa + i >= s.Q) piece.e[i] = store_cast<T>(0.f);
+          }
+        }
+#pragma unroll
+        for (int m = 0; m < MT; m++) acc[t][m] = M::run(a[m], piece.u, acc[t][m]);
+      }
+    }
+  }
+  // ---- reduce the four wavefronts, then one atomic per (o, c, tap) -------------------------------
+#pragma unroll
+  for (int t = 0; t < TPW; t++) {
+    if (k0 + t >= s.K) break;  // the same for every thread
+#pragma unroll
+    for (int m = 0; m < MT; m++) {
+      __syncthreads();
+      if (wave > 0) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) part[wave - 1][r][lane] = acc[t][m][r];
+      }
+      __syncthreads();
+      if (wave == 0) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const float v = acc[t][m][r] + part[0][r][lane] + part[1][r][lane] + part[2][r][lane];
+          // accumulator layout: register r of lane l = row 8*(r/4) + 4*(l/32) + r%4, column l%32
+          const int o = g * s.opg + (mb0 + m) * 32 + 8 * (r / 4) + 4 * h + (r % 4);
+          const int cl = c0 - g * s.cpg + n;
+          atomicAdd(gw + (static_cast<long>(k0 + t) * s.Cout + o) * s.cpg + cl, v);
+        }
+      }
+    }
   }
 }
 
@@ -868,22 +942,24 @@ static int backward_run(const void *x, const void *off, const void *mask, const 
   }
   const dim3 wgrid(static_cast<unsigned>(static_cast<long>(s.Cin / 32) * s.K),
                    static_cast<unsigned>((s.Q + kGwChunk - 1) / kGwChunk), s.B);
-#define MV_LAUNCH_GW(MTV)                                                                              \
-  if (col)                                                                                             \
-    hipLaunchKernelGGL((dcn_backward_weight_mfma_kernel<T, MTV, true>), wgrid, dim3(256), 0, stream, xt, \
+#define MV_LAUNCH_GW(MTV, TPW)                                                                         \
+  if (col) {                                                                                           \
+    const dim3 cgrid(static_cast<unsigned>(static_cast<long>(s.Cin / 32) * ((s.K + TPW - 1) / TPW)), wgrid.y, s.B); \
+    hipLaunchKernelGGL((dcn_backward_weight_columns_kernel<T, MTV, TPW>), cgrid, dim3(256), 0, stream, \
+                       col, static_cast<const T *>(gy), *gw32, s, mb0, l.qp);                          \
+  } else                                                                                               \
+    hipLaunchKernelGGL((dcn_backward_weight_mfma_kernel<T, MTV>), wgrid, dim3(256), 0, stream, xt,     \
                        static_cast<const T *>(off), static_cast<const T *>(mask),                      \
-                       static_cast<const T *>(gy), *gw32, s, mb0, col, l.qp);                          \
-  else                                                                                                 \
-    hipLaunchKernelGGL((dcn_backward_weight_mfma_kernel<T, MTV, false>), wgrid, dim3(256), 0, stream, xt, \
-                       static_cast<const T *>(off), static_cast<const T *>(mask),                      \
-                       static_cast<const T *>(gy), *gw32, s, mb0, col, l.qp)
-  // up to four 32-row blocks of output channels per pass over the positions
-  for (int mb0 = 0; mb0 < s.opg / 32; mb0 += 4)
-    switch (min(s.opg / 32 - mb0, 4)) {
-      case 1: MV_LAUNCH_GW(1); break;
-      case 2: MV_LAUNCH_GW(2); break;
-      case 3: MV_LAUNCH_GW(3); break;
-      default: MV_LAUNCH_GW(4); break;
+                       static_cast<const T *>(gy), *gw32, s, mb0)
+  // up to four 32-row blocks of output channels per pass over the positions when gathering; with
+  // the column buffer two blocks and three taps per workgroup (the accumulators fill the registers)
+  const int mstep = col ? 2 : 4;
+  for (int mb0 = 0; mb0 < s.opg / 32; mb0 += mstep)
+    switch (min(s.opg / 32 - mb0, mstep)) {
+      case 1: MV_LAUNCH_GW(1, 3); break;
+      case 2: MV_LAUNCH_GW(2, 3); break;
+      case 3: MV_LAUNCH_GW(3, 1); break;
+      default: MV_LAUNCH_GW(4, 1); break;
     }
 #undef MV_LAUNCH_GW
   return check_launch("dcn3d mfma backward");
