@@ -1,26 +1,27 @@
-// Backward of the 3-D deformable convolution for fp16 / bf16 tensors, built around the matrix
-// cores and channels-last buffers.
+// Backward of the 3-D deformable convolution for fp16 / bf16 / fp32 tensors, built around the
+// matrix cores and channels-last buffers.
 //
 //   gcol[c, k, q] = sum_o Wt[o, c, k] * gy[o, q]                    (GEMM, MFMA)
-//   gx[corner_n(k, q), c] += w_n * mask * gcol                       (scatter: fp32 atomics, and for
-//                                                                     unit-stride 3^3 layers LDS tiles)
+//   gx[corner_n(k, q), c] += w_n * mask * gcol                       (scatter: LDS tiles + fp32 atomics)
 //   goff_a[k, q] = mask * sum_c gcol * dZ/dp_a ,  gmask[k, q] = sum_c gcol * Z
 //   gw[o, c, k]  = sum_{b, q} gy[o, q] * col[c, k, q]                (GEMM over positions, MFMA)
 //
 // Data kernel: a wavefront owns 32 output positions.  Per tap it forms the 32 x 32 block
 // gcol[position, channel] with MFMA 32x32x16 (A = gy channels-last, B = weight fragments); the
-// accumulator layout gives every lane ONE channel and 16 positions, so for each position the 32
-// lanes of a half-wavefront touch 32 consecutive channels of a channels-last voxel: the reads of
-// x (for the offset / mask gradients) and the fp32 atomic adds into the channels-last gradient
-// buffer are 64- and 128-byte contiguous.  The four per-position sums over channels are reduced
-// across the half-wavefront with DPP adds.
-// Scatter kernel (layers whose taps fit its tile): the corners that land near their position are
-// summed per brick of positions in a 64-bit fixed-point LDS tile and reach the gradient buffer as
-// one atomic per (voxel, channel) of the tile; the data kernel then adds only the other corners.
-// Weight kernel: a workgroup owns (tap, 32-channel block, range of positions); lanes rebuild the
-// column values of their channel for 16 positions at a time (same coalesced corner reads), which
-// is exactly the MFMA B fragment; A is gy read in its own layout.  Accumulators stay in registers
-// over the whole range and are added to the fp32 gradient once per workgroup.
+// accumulator layout gives every lane ONE channel and 16 positions.  x at the corners is fetched 16
+// bytes per lane into an LDS stage and read back one channel per lane; the fp32 atomic adds into
+// the channels-last gradient buffer are 128-byte contiguous per position.  The four per-position
+// sums over channels are reduced across the half-wavefront with DPP adds.  The column values
+// mask * Z(x) are stored for the weight kernel.
+// Scatter kernel (unit-stride layers whose taps fit its tile): the corners that land near their
+// position are summed per brick of positions in a 64-bit fixed-point LDS tile and reach the
+// gradient buffer as one atomic per (voxel, channel) of the tile; the data kernel then adds only the
+// other corners.
+// Weight kernels: a workgroup owns (taps, 32-channel block, range of positions); the MFMA B
+// fragment is the column values of a channel for 16 positions at a time — read from the column
+// buffer, or (layers beyond its budget) rebuilt by the lanes with a second gather of x; A is gy read
+// in its own layout.  Accumulators stay in registers over the whole range and are added to a
+// tap-major fp32 gradient once per workgroup.
 #include "dcn_mfma.hpp"
 
 #include <cstdlib>
