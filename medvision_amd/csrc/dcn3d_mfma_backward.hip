@@ -79,11 +79,12 @@ __device__ __forceinline__ float half_wave_sum(float v) {
 // reach of the brick's undeformed taps.  A corner is "local" when its voxel lies in
 // the tile of its position's brick: local corners are summed in LDS by the scatter kernel, all
 // others are added to the gradient buffer by the data kernel, 128 bytes per request.
-// Volumes use 4 x 8 x 8 bricks with 10 x 14 x 14 tiles.  (Images: 16 x 16 bricks with 44 x 44 tiles
-// were measured on 256-channel FPN layers and gained nothing there: four of the eight corner slots
-// are empty and every 8-channel workgroup repeats the tap geometry; they keep the atomics.)
+// Volumes use 4 x 8 x 8 bricks with 10 x 14 x 14 tiles, images 32 x 32 bricks with 44 x 44 tiles (a
+// workgroup's fixed costs — clearing and flushing the tile — need more than nine taps of 256
+// positions to pay: 16 x 16 bricks gained nothing on 256-channel FPN layers).
 struct VolumeBricks { static constexpr int BD = 4, BH = 8, BW = 8, TD = 10, TH = 14, TW = 14; };
-constexpr int kBrickPositions = 256, kTileVoxMax = 1960;
+struct ImageBricks { static constexpr int BD = 1, BH = 32, BW = 32, TD = 1, TH = 44, TW = 44; };
+constexpr int kTileVoxMax = 1960;
 struct TileOrigin { int d, h, w; };
 template <typename S>
 __device__ __forceinline__ TileOrigin tile_origin(const DcnDims &s, int bz, int by, int bx) {
@@ -111,7 +112,7 @@ __device__ __forceinline__ unsigned tile_bits(const TileOrigin &t, int id, int i
 // The LDS sums are 64-bit fixed point (LDS float atomics retire one lane at a time, integer ones
 // a wavefront in a few clocks).  Every term is w * mask * gcol with 0 <= w <= 1, so
 //   |term| <= max|mask| * max|grad_output| * max_{c,k} sum_o |Wt[o,c,k]|  =: bound < 2^ex,
-// and a voxel takes at most one corner of each (position, tap) of the brick: 256 * taps terms.
+// and a voxel takes at most one corner of each (position, tap) of the brick: positions * taps terms.
 // Terms are scaled by 2^(shift - ex), shift = min(50, 62 - ceil(log2(terms))), and rounded to
 // integers (adding 1.5 * 2^52 in fp64 leaves round(x) in the low mantissa bits for |x| < 2^51):
 // a term loses less than 2^-shift of the bound (2^-49 for up to 4096 terms), and the sum of a
@@ -120,14 +121,14 @@ __device__ __forceinline__ unsigned tile_bits(const TileOrigin &t, int id, int i
 // corner is treated as local).
 constexpr double kRoundMagic = 6755399441055744.0;  // 1.5 * 2^52
 struct ScatterScale { bool valid; double up, down; };
-__device__ __forceinline__ ScatterScale scatter_scale(const unsigned *__restrict__ words, int taps, bool has_mask) {
+__device__ __forceinline__ ScatterScale scatter_scale(const unsigned *__restrict__ words, int terms, bool has_mask) {
   const float bound = 1.001f * __uint_as_float(words[0]) * __uint_as_float(words[1]) *
                       (has_mask ? __uint_as_float(words[2]) : 1.f);
   ScatterScale r;
   r.valid = bound < __builtin_inff() && bound == bound;
   int ex = 0;
   frexpf(fmaxf(bound, 1e-30f), &ex);  // bound < 2^ex
-  const int terms = kBrickPositions * taps, shift = min(50, 62 - (32 - __clz(terms - 1)));
+  const int shift = min(50, 62 - (32 - __clz(terms - 1)));
   r.up = ldexp(1.0, shift - ex);
   r.down = ldexp(1.0, ex - shift);
   return r;
@@ -234,7 +235,7 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
   float(*tp)[kTapWords] = taps[wave];
   float(*sm)[32] = sums[wave];
   const TileOrigin origin = tile_origin<S>(s, od / S::BD, oh / S::BH, ow / S::BW);
-  const bool split = SPLIT && scatter_scale(bounds, s.K, mask != nullptr).valid;
+  const bool split = SPLIT && scatter_scale(bounds, S::BD * S::BH * S::BW * s.K, mask != nullptr).valid;
 
   int ki = 0, kj = 0, kk = 0;
   for (int k = 0; k < s.K; k++) {
@@ -374,15 +375,15 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
 
 // ---- gradient of the input, local corners: summed in LDS, then added to the buffer ----------------
 // A workgroup owns a brick of positions and eight channels; its sixteen wavefronts are kScatterSplit
-// groups of eight, every group covers the 256 positions of the brick and takes a contiguous share
-// of the taps.  gcol comes from the 16 x 16 MFMA with the channels as rows: lane l holds position
+// groups of eight, every group covers the positions of the brick (32 per wavefront at a time) and
+// takes a contiguous share of the taps.  gcol comes from the 16 x 16 MFMA with the channels as rows: lane l holds position
 // l % 16 of a 16-position block and the channels l / 16 and l / 16 + 4, so one LDS add instruction
 // covers 16 positions x 4 adjacent channels; a voxel's 8 sums are 9 qwords apart from the next
 // voxel's to spread the banks.  After the taps the tile's non-zero sums are converted and added
 // to the gradient buffer: one global atomic per (voxel, channel) of the tile instead of one per
 // (position, tap, corner, channel).
 constexpr int kScatterSplit = 2, kScatterWaves = 8 * kScatterSplit, kScatterStride = 9;
-constexpr int kScatterKeep = 4;  // slices of grad_output a wavefront keeps in registers over the taps
+constexpr int kScatterKeep = 4;  // slices of grad_output a wavefront keeps in registers over the taps (all of them)
 
 // weight [Cout, cpg, K] -> A pieces [group][tap][8-channel block][row step][lane][kPiece]: lane l
 // is MFMA row l % 16 = channel (row / 4) + 4 * (row % 2) of the block (rows 4j + 2, 4j + 3 repeat
@@ -417,14 +418,15 @@ __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter_kerne
   using P = typename std::conditional<(sizeof(T) == 2), float, double>::type;
   constexpr int PC = M::kPiece, SL = 4 * PC;
   constexpr int VOX = S::TD * S::TH * S::TW;
-  static_assert(VOX <= kTileVoxMax && S::BD * S::BH * S::BW == kBrickPositions, "brick and tile sizes");
+  constexpr int GROUPS = S::BD * S::BH * S::BW / 32;  // 32-position groups of the brick
+  static_assert(VOX <= kTileVoxMax && GROUPS % 8 == 0, "brick and tile sizes");
   __shared__ unsigned long long tile[VOX * kScatterStride];
   __shared__ __attribute__((aligned(16))) float recs[kScatterWaves][32][8];
-  const ScatterScale scale = scatter_scale(bounds, s.K, mask != nullptr);
+  const ScatterScale scale = scatter_scale(bounds, S::BD * S::BH * S::BW * s.K, mask != nullptr);
   if (!scale.valid) return;  // every corner went through the data kernel
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int n = lane % 32, p16 = lane % 16, j = lane / 16;
-  const int pg = wave % 8, tg = wave / 8;
+  const int tg = wave / 8;
   const unsigned brick = xcd_contiguous(blockIdx.x, gridDim.x);
   const int bx = brick % nbw, by = (brick / nbw) % nbh, bz = brick / (nbw * nbh);
   const int c0 = blockIdx.y * 8, b = blockIdx.z;
@@ -442,6 +444,7 @@ __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter_kerne
     live = od < s.Do && oh < s.Ho && ow < s.Wo;
     return (static_cast<long>(min(od, s.Do - 1)) * s.Ho + min(oh, s.Ho - 1)) * s.Wo + min(ow, s.Wo - 1);
   };
+  for (int pg = wave % 8; pg < GROUPS; pg += 8) {
   // the lane's own position for the taps (both halves of the wavefront compute them)
   bool live;
   const long q = position(pg * 32 + n, live);
@@ -524,14 +527,6 @@ __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter_kerne
         acc[0] = M::run16(wcur[st], keep[0][st], acc[0]);
         acc[1] = M::run16(wcur[st], keep[1][st], acc[1]);
       }
-    for (int st = kScatterKeep; st < steps; st++) {
-      const u32x4 a = *reinterpret_cast<const u32x4 *>(afrag + static_cast<long>(st) * (64 * PC));
-#pragma unroll
-      for (int blk = 0; blk < 2; blk++) {
-        const u32x4 bv = blive[blk] ? *reinterpret_cast<const u32x4 *>(grow[blk] + st * SL) : u32x4{0u, 0u, 0u, 0u};
-        acc[blk] = M::run16(a, bv, acc[blk]);
-      }
-    }
 #pragma unroll
     for (int blk = 0; blk < 2; blk++) {
       const float4 *src = reinterpret_cast<const float4 *>(rec[blk * 16 + p16]);
@@ -545,7 +540,7 @@ __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter_kerne
 #pragma unroll
       for (int c = 0; c < 8; c++) {
         const int ca = c >> 2, cb2 = (c >> 1) & 1, ce = c & 1;
-        if ((bits >> c) & 1u) {
+        if ((S::TD > 1 || ca == 0) && ((bits >> c) & 1u)) {  // images have no second slice
           const float wc = wd[ca] * wh[cb2] * ww[ce];
           unsigned long long *dst = tile + (first + ca * (S::TH * S::TW) + cb2 * S::TW + ce) * kScatterStride + j;
 #pragma unroll
@@ -560,6 +555,7 @@ __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter_kerne
     afrag += tap_stride;
 #pragma unroll
     for (int st = 0; st < kScatterKeep; st++) wcur[st] = wnext[st];
+  }
   }
   __syncthreads();
   // ---- the tile's voxels inside the volume go to the gradient buffer, 8 channels per voxel --------
@@ -830,11 +826,15 @@ __global__ void dcn_zero_f32_kernel(float *p, long n) {
 // The LDS scatter pays when its tile holds the reach of a brick's undeformed taps with a voxel to
 // spare on either side (offsets beyond the tile still work, through the data kernel's atomics).
 template <typename S>
-static bool scatter_tile_applies(const DcnDims &s) {
+static bool scatter_tile_applies(const DcnDims &s, int dtype) {
+  // the scatter kernel keeps grad_output of its positions in registers: up to kScatterKeep slices
+  // of 4 * kPiece output channels per group (128 for 16-bit tensors, 64 for fp32); wider layers
+  // would repeat too much per 8-channel workgroup and keep the atomics
+  if (s.opg > kScatterKeep * (dtype == MV_F32 ? 16 : 32)) return false;
   const int ed = (S::BD - 1) * s.sd + (s.kd - 1) * s.dd + 1, eh = (S::BH - 1) * s.sh + (s.kh - 1) * s.dh + 1,
             ew = (S::BW - 1) * s.sw + (s.kw - 1) * s.dw + 1;
-  return ed + 2 <= S::TD && eh + 2 <= S::TH && ew + 2 <= S::TW &&
-         static_cast<long>(kBrickPositions) * s.K < (1L << 20);
+  return (S::TD == 1 || ed + 2 <= S::TD) && eh + 2 <= S::TH && ew + 2 <= S::TW &&
+         static_cast<long>(S::BD * S::BH * S::BW) * s.K < (1L << 20);
 }
 
 static size_t align256b(size_t v) { return (v + 255) / 256 * 256; }
@@ -905,7 +905,8 @@ static int backward_run(const void *x, const void *off, const void *mask, const 
                      0, stream, gxt, nz);
   const long qblocks = (s.Q + 127) / 128;
   MV_REQUIRE(qblocks < (1L << 31), "grid too large");
-  if (s.nd == 3 && scatter_tile_applies<VolumeBricks>(s)) {
+  const bool image = s.nd == 2;
+  if (image ? scatter_tile_applies<ImageBricks>(s, dtype) : scatter_tile_applies<VolumeBricks>(s, dtype)) {
     unsigned *bounds = reinterpret_cast<unsigned *>(ws + l.bounds);
     const long ngy = static_cast<long>(s.B) * s.Cout * s.Q, nmask = static_cast<long>(s.B) * s.dg * s.K * s.Q;
     const long ncols = static_cast<long>(s.groups) * s.cpg * s.K;
@@ -933,7 +934,7 @@ static int backward_run(const void *x, const void *off, const void *mask, const 
                        stream, static_cast<const T *>(off), static_cast<const T *>(mask), gyt, wa, gxt, s,        \
                        static_cast<int>(nbh), static_cast<int>(nbw), bounds);                                     \
   }
-    MV_LAUNCH_SPLIT(VolumeBricks)
+    if (image) MV_LAUNCH_SPLIT(ImageBricks) else MV_LAUNCH_SPLIT(VolumeBricks)
 #undef MV_LAUNCH_SPLIT
   } else {
     hipLaunchKernelGGL((dcn_backward_data_mfma_kernel<T, false, VolumeBricks>),
