@@ -376,10 +376,10 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
 // ---- gradient of the input, local corners: summed in LDS, then added to the buffer ----------------
 // A workgroup owns a brick of positions and eight channels; its sixteen wavefronts are kScatterSplit
 // groups of eight, every group covers the positions of the brick (32 per wavefront at a time) and
-// takes a contiguous share of the taps.  gcol comes from the 16 x 16 MFMA with the channels as rows: lane l holds position
-// l % 16 of a 16-position block and the channels l / 16 and l / 16 + 4, so one LDS add instruction
-// covers 16 positions x 4 adjacent channels; a voxel's 8 sums are 9 qwords apart from the next
-// voxel's to spread the banks.  After the taps the tile's non-zero sums are converted and added
+// takes a contiguous share of the taps.  gcol comes from the 16 x 16 MFMA with the channels as
+// rows: lane l holds position l % 16 of a 16-position block and the channels l / 16 and l / 16 + 4,
+// so one LDS add instruction covers 16 positions x 4 adjacent channels; a voxel's 8 sums are 9
+// qwords apart from the next voxel's to spread the banks.  After the taps the tile's non-zero sums are converted and added
 // to the gradient buffer: one global atomic per (voxel, channel) of the tile instead of one per
 // (position, tap, corner, channel).
 constexpr int kScatterSplit = 2, kScatterWaves = 8 * kScatterSplit, kScatterStride = 9;
