@@ -131,19 +131,35 @@ def test_affine_and_warp_sweep(ops, oracle):
 
 
 def test_dcn_sweep(ops, oracle):
+    assert _dcn_sweep(oracle, range(9000, 9260), tiles=False) > 200
+
+
+def test_dcn_sweep_of_the_lds_scatter_path(ops, oracle):
+    """Unit-stride layers with 32 or 64 channels per group and up to 160 output channels per group,
+    volumes larger and smaller than a brick of positions, 1 to 125 taps: the layers whose input
+    gradient goes through the LDS tiles (and their neighbours that just miss the conditions)."""
+    assert _dcn_sweep(oracle, range(9500, 9580), tiles=True) > 60
+
+
+def _dcn_sweep(oracle, seeds, tiles):
     from medvision_amd.ops.deform_conv_2d import deform_conv as dc2
     from medvision_amd.ops.deform_conv_3d import deform_conv as dc3
     from medvision_amd.ops.modulated_deform_conv_2d import modulated_deform_conv as mdc2
     from medvision_amd.ops.modulated_deform_conv_3d import modulated_deform_conv as mdc3
     ran = 0
-    for seed in range(9000, 9260):
+    for seed in seeds:
         rnd = random.Random(seed)
         g = torch.Generator().manual_seed(seed)
         nd = rnd.choice([2, 3])
         modulated = rnd.random() < 0.5
         groups, dg = rnd.choice([1, 1, 2, 4]), rnd.choice([1, 1, 2])
         matrix = rnd.random() < 0.5   # channel counts the matrix-core kernels accept
-        if matrix:
+        if tiles:
+            groups = rnd.choice([1, 1, 2])
+            cin, cout = rnd.choice([32, 32, 64]) * groups, rnd.choice([32, 64, 96, 128, 160]) * groups
+            if cin % dg or (cin // dg) % 32:
+                dg = 1
+        elif matrix:
             cin, cout = rnd.choice([16, 32, 48]) * groups, rnd.choice([32, 64, 96]) * groups
             if cin % dg or (cin // dg) % 16:
                 dg = 1
@@ -152,7 +168,14 @@ def test_dcn_sweep(ops, oracle):
         batch = rnd.randint(1, 3)
         size = [rnd.randint(2, 9 if matrix else 11) for _ in range(nd)]
         dtype = rnd.choice(DTYPES)
-        if modulated:   # one stride / padding / dilation for all axes, as the reference's layer
+        if tiles:
+            batch = rnd.randint(1, 2)
+            size = [rnd.randint(3, 13) for _ in range(nd)] if nd == 3 else [rnd.randint(5, 40) for _ in range(nd)]
+            dtype = rnd.choice([torch.float32, torch.float16, torch.bfloat16])
+            kk = rnd.choice([1, 2, 3, 3, 3, 5]) if nd == 3 else rnd.choice([1, 3, 3, 5])
+            k = [kk] * nd if rnd.random() < 0.7 else [rnd.randint(1, 3) for _ in range(nd)]
+            st, pa, di = [1] * nd, [rnd.randint(0, 2)] * nd, [rnd.choice([1, 1, 2])] * nd
+        elif modulated:   # one stride / padding / dilation for all axes, as the reference's layer
             k = [rnd.randint(1, 3)] * nd if rnd.random() < 0.5 else [rnd.randint(1, 3) for _ in range(nd)]
             st, pa, di = [rnd.randint(1, 2)] * nd, [rnd.randint(0, 2)] * nd, [rnd.randint(1, 2)] * nd
         else:
@@ -198,7 +221,7 @@ def test_dcn_sweep(ops, oracle):
             assert rel_err(offs.grad, goff) <= tol, what + " (grad offset)"
         if modulated:
             assert rel_err(ms.grad, gm) <= tol, what + " (grad mask)"
-    assert ran > 200
+    return ran
 
 
 def test_resampling_backward_sweep(ops, oracle):
