@@ -125,7 +125,7 @@ int mv_dcn3d_output_dims(const mv_dcn3d_shape *shape, int *out_d, int *out_h, in
 size_t mv_dcn3d_forward_workspace_bytes(const mv_dcn3d_shape *shape, int dtype);
 /* The backward workspace of 16-bit / fp32 layers on the matrix-core path includes a buffer of column
  * values (batch x taps x in_channels x positions elements) while that stays below 1 GiB or the number
- * of bytes in the environment variable MV_DCN_COLUMN_BYTES (read by the query and by the call). */
+ * of bytes set with mv_dcn_set_column_budget() / the environment variable MV_DCN_COLUMN_BYTES. */
 size_t mv_dcn3d_backward_workspace_bytes(const mv_dcn3d_shape *shape, int dtype);
 int mv_dcn3d_forward(const void *input, const void *offset, const void *mask, const void *weight,
                      const void *bias, void *output, const mv_dcn3d_shape *shape, int dtype,
@@ -134,6 +134,13 @@ int mv_dcn3d_backward(const void *input, const void *offset, const void *mask, c
                       const void *grad_output, void *grad_input, void *grad_offset,
                       void *grad_mask, void *grad_weight, void *grad_bias,
                       const mv_dcn3d_shape *shape, int dtype, void *workspace, void *stream);
+
+/* Budget of the backward pass's column buffer in bytes (default 1 GiB, or MV_DCN_COLUMN_BYTES in the
+ * environment when the library is first asked).  Changing it changes what
+ * mv_dcn{2,3}d_backward_workspace_bytes() returns: query again.  No counterpart in the reference
+ * (its column buffer is a tensor argument, csrc/modulated_deform_conv_3d.h:89).               */
+void mv_dcn_set_column_budget(size_t bytes);
+size_t mv_dcn_column_budget(void);
 
 /* ---- deformable convolution 2-D -----------------------------------------------------------
  * replaces deform_conv_2d_forward / _backward                 csrc/deform_conv_2d.h:41,76

@@ -25,6 +25,44 @@ def _require_cuda(t, what):
         raise RuntimeError(f"{what} is not implemented on CPU")
 
 
+def _same_device(ref, **tensors):
+    """Every tensor whose address goes to a kernel must live on the device the kernel runs on (a
+    host or foreign pointer would fault on the GPU instead of raising)."""
+    for name, t in tensors.items():
+        if t is not None and t.device != ref.device:
+            raise RuntimeError(f"{name} is on {t.device}, expected {ref.device} like the input tensor")
+
+
+class _on_device:
+    """``torch.cuda.device`` only when the tensor's device is not already current."""
+    __slots__ = ("guard",)
+
+    def __init__(self, t):
+        idx = t.device.index
+        self.guard = None if idx is None or idx == torch.cuda.current_device() else torch.cuda.device(idx)
+
+    def __enter__(self):
+        if self.guard is not None:
+            self.guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            self.guard.__exit__(*exc)
+        return False
+
+
+_ws_bytes_cache = {}
+
+
+def _cached_bytes(fn, *key):
+    """Workspace sizes depend on the shape key alone: ask the library once per key."""
+    k = (fn, key)
+    n = _ws_bytes_cache.get(k)
+    if n is None:
+        n = _ws_bytes_cache[k] = getattr(_lib.load(), fn)(*key)
+    return n
+
+
 def _prep_rois(rois, features, cols):
     if rois.dim() != 2 or rois.size(1) != cols:
         raise RuntimeError(f"wrong roi size! size_rois should be {cols}")
@@ -41,6 +79,7 @@ def _roi_forward(fn_name, what, ndim, cols, input, rois, output, out_sizes, spat
                  sampling_ratio, extra):
     _require_cuda(input, what)
     lib = _lib.load()
+    _same_device(input, output=output)
     _require_contiguous(output, "output")
     if output.dtype != input.dtype:
         raise RuntimeError("output dtype must match input dtype")
@@ -54,10 +93,10 @@ def _roi_forward(fn_name, what, ndim, cols, input, rois, output, out_sizes, spat
         raise RuntimeError(f"output has shape {tuple(output.shape)}, expected {want_shape}")
     code = _lib.dtype_code(feats)
     out3 = out_sizes if ndim == 3 else (1, *out_sizes)
-    ws_bytes = lib.mv_roi_align_forward_workspace_bytes(code, ndim, dims[1], r.size(0), *out3,
-                                                        int(sampling_ratio))
+    ws_bytes = _cached_bytes("mv_roi_align_forward_workspace_bytes", code, ndim, dims[1], r.size(0),
+                             *out3, int(sampling_ratio))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=feats.device) if ws_bytes else None
-    with torch.cuda.device(feats.device):
+    with _on_device(feats):
         _lib.check(getattr(lib, fn_name)(
             _lib.ptr(feats), _lib.ptr(r), _lib.ptr(output), code, *dims,
             r.size(0), *out_sizes, float(spatial_scale), int(sampling_ratio), *extra,
@@ -68,6 +107,7 @@ def _roi_backward(fn_name, what, ndim, cols, top_grad, rois, bottom_grad, out_si
                   spatial_scale, sampling_ratio, extra):
     _require_cuda(top_grad, what)
     lib = _lib.load()
+    _same_device(top_grad, bottom_grad=bottom_grad)
     _require_contiguous(bottom_grad, "bottom_grad")
     if bottom_grad.dtype != top_grad.dtype:
         raise RuntimeError("bottom_grad dtype must match top_grad dtype")
@@ -81,9 +121,9 @@ def _roi_backward(fn_name, what, ndim, cols, top_grad, rois, bottom_grad, out_si
         raise RuntimeError(f"top_grad has shape {tuple(g.shape)}, expected {want_shape}")
     code = _lib.dtype_code(g)
     d5 = dims if ndim == 3 else [dims[0], dims[1], 1, dims[2], dims[3]]
-    ws_bytes = lib.mv_roi_align_backward_workspace_bytes(code, *d5)
+    ws_bytes = _cached_bytes("mv_roi_align_backward_workspace_bytes", code, *d5)
     ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=g.device) if ws_bytes else None
-    with torch.cuda.device(g.device):
+    with _on_device(g):
         _lib.check(getattr(lib, fn_name)(
             _lib.ptr(g), _lib.ptr(r), _lib.ptr(bottom_grad), code, *dims, r.size(0), *out_sizes,
             float(spatial_scale), int(sampling_ratio), *extra, _lib.ptr(ws), _lib.stream_of(g)))
@@ -204,8 +244,17 @@ def _dcn_check_aux(shape, dims, offset, mask, K):
         raise RuntimeError(f"mask has shape {tuple(mask.shape)}, expected {(B, dg * K, *dims)}")
 
 
+def _dcn_bytes(fn, shape, code):
+    k = (fn, code, bytes(shape))
+    n = _ws_bytes_cache.get(k)
+    if n is None:
+        n = _ws_bytes_cache[k] = getattr(_lib.load(), fn)(ctypes.byref(shape), code)
+    return n
+
+
 def _dcn_forward(input, offset, mask, weight, bias, output, shape):
     lib = _lib.load()
+    _same_device(input, offset=offset, mask=mask, weight=weight, bias=bias, output=output)
     fam = _dcn_family(shape)
     dims = _dcn_out_dims(lib, shape)
     K = _dcn_taps(shape)
@@ -215,9 +264,9 @@ def _dcn_forward(input, offset, mask, weight, bias, output, shape):
     if weight.dtype != input.dtype or (bias is not None and bias.dtype != input.dtype):
         raise RuntimeError("input, weight and bias must share one dtype")
     code = _lib.dtype_code(input)
-    nbytes = getattr(lib, fam + "_forward_workspace_bytes")(ctypes.byref(shape), code)
+    nbytes = _dcn_bytes(fam + "_forward_workspace_bytes", shape, code)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=input.device) if nbytes else None
-    with torch.cuda.device(input.device):
+    with _on_device(input):
         _lib.check(getattr(lib, fam + "_forward")(
             _lib.ptr(input), _lib.ptr(offset), _lib.ptr(mask), _lib.ptr(weight), _lib.ptr(bias),
             _lib.ptr(output), ctypes.byref(shape), code, _lib.ptr(ws), _lib.stream_of(input)))
@@ -225,6 +274,8 @@ def _dcn_forward(input, offset, mask, weight, bias, output, shape):
 
 def _dcn_backward(input, offset, mask, weight, grad_output, gi, goff, gmask, gw, gb, shape):
     lib = _lib.load()
+    _same_device(input, offset=offset, mask=mask, weight=weight, grad_output=grad_output,
+                 grad_input=gi, grad_offset=goff, grad_mask=gmask, grad_weight=gw, grad_bias=gb)
     fam = _dcn_family(shape)
     dims = _dcn_out_dims(lib, shape)
     K = _dcn_taps(shape)
@@ -238,13 +289,23 @@ def _dcn_backward(input, offset, mask, weight, grad_output, gi, goff, gmask, gw,
     for t, n in ((gi, "grad_input"), (goff, "grad_offset"), (gw, "grad_weight")):
         _require_contiguous(t, n)
     code = _lib.dtype_code(input)
-    nbytes = getattr(lib, fam + "_backward_workspace_bytes")(ctypes.byref(shape), code)
+    nbytes = _dcn_bytes(fam + "_backward_workspace_bytes", shape, code)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=input.device) if nbytes else None
-    with torch.cuda.device(input.device):
+    with _on_device(input):
         _lib.check(getattr(lib, fam + "_backward")(
             _lib.ptr(input), _lib.ptr(offset), _lib.ptr(mask), _lib.ptr(weight),
             _lib.ptr(grad_output), _lib.ptr(gi), _lib.ptr(goff), _lib.ptr(gmask), _lib.ptr(gw),
             _lib.ptr(gb), ctypes.byref(shape), code, _lib.ptr(ws), _lib.stream_of(input)))
+
+
+def set_dcn_column_budget(nbytes):
+    """Budget (bytes) of the column buffer the DCN backward keeps for its weight kernel; layers
+    beyond it gather the input a second time.  Returns the previous budget."""
+    lib = _lib.load()
+    old = lib.mv_dcn_column_budget()
+    lib.mv_dcn_set_column_budget(int(nbytes))
+    _ws_bytes_cache.clear()   # workspace sizes depend on it
+    return old
 
 
 def _im2col_step_check(batch, im2col_step):
@@ -385,15 +446,35 @@ def modulated_deform_conv_2d_backward(input, weight, bias, ones, offset, mask, c
 
 
 # csrc/deform_2d.h, csrc/deform_3d.h:27-65 as used by ops/cuda_fun_tools.py:94-167
+_identity_verdicts = {}   # (weight address, version, bias address, version) -> bool
+
+
+def _is_identity_warp(weight, bias, C, ndim):
+    """True when ``weight`` is the C x C identity over a 1x1(x1) kernel and ``bias`` is zero.
+    Reading the verdict back blocks the host, so it is taken once per (tensor, version) and
+    remembered: a caller that reuses its weight, as the reference's own caller could, pays no
+    synchronisation per call."""
+    if tuple(weight.shape) != (C, C, *([1] * ndim)) or tuple(bias.shape) != (C,):
+        return False
+    key = (weight.data_ptr(), weight._version, bias.data_ptr(), bias._version, C, weight.dtype)
+    ok = _identity_verdicts.get(key)
+    if ok is None:
+        if len(_identity_verdicts) > 64:
+            _identity_verdicts.clear()
+        eye = torch.eye(C, dtype=weight.dtype, device=weight.device)
+        ok = bool(((weight.reshape(C, C) == eye).all() & (bias == 0).all()).item())
+        _identity_verdicts[key] = ok
+    return ok
+
+
 def _deform(fn_name, ndim, input, weight, bias, offset, kernel, stride, pad, dil, group,
             deformable_group, order):
     if not input.is_cuda:
         raise RuntimeError("Not implemented on the CPU")
-    C = input.size(1)
-    eye = torch.eye(C, dtype=weight.dtype, device=weight.device).reshape(C, C, *([1] * ndim))
+    _same_device(input, weight=weight, bias=bias)
     if (any(k != 1 for k in kernel) or any(s != 1 for s in stride) or any(p != 0 for p in pad)
-            or group != 1 or deformable_group != 1 or tuple(weight.shape) != tuple(eye.shape)
-            or not torch.equal(weight, eye) or bool((bias != 0).any())):
+            or group != 1 or deformable_group != 1
+            or not _is_identity_warp(weight, bias, input.size(1), ndim)):
         raise RuntimeError("deform_%dd supports the displacement-field warp only: 1x1 kernel, "
                            "stride 1, no padding, identity weight, zero bias" % ndim)
     if order not in (0, 1, 3):
@@ -403,7 +484,7 @@ def _deform(fn_name, ndim, input, weight, bias, offset, kernel, stride, pad, dil
     if tuple(offset.shape) != (input.size(0), ndim, *input.shape[2:]):
         raise RuntimeError("offset must have shape [B, %d, *spatial]" % ndim)
     out = torch.empty_like(input)
-    with torch.cuda.device(input.device):
+    with _on_device(input):
         _lib.check(getattr(_lib.load(), fn_name)(
             _lib.ptr(input), _lib.ptr(offset), _lib.ptr(out), _lib.dtype_code(input),
             *input.shape, int(order), _lib.stream_of(input)))
@@ -439,7 +520,7 @@ def deform_warp(img, offset, order=1):
         raise RuntimeError(f"order {order} is not supported (0 nearest, 1 linear, 3 cubic)")
     out = torch.empty_like(img)
     fn = "mv_deform_warp_2d" if ndim == 2 else "mv_deform_warp_3d"
-    with torch.cuda.device(img.device):
+    with _on_device(img):
         _lib.check(getattr(_lib.load(), fn)(
             _lib.ptr(img), _lib.ptr(offset), _lib.ptr(out), _lib.dtype_code(img), *img.shape,
             int(order), _lib.stream_of(img)))

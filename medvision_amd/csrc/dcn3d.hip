@@ -5,6 +5,8 @@
 // Nothing here materialises the reference's column matrix: the trilinear gather feeds the weight
 // contraction directly, and the 8 corner offsets / weights of a (tap, position) pair are computed
 // once and reused for all channels of the deformable group.
+#include <atomic>
+
 #include "dcn_common.hpp"
 
 namespace mv {
@@ -218,6 +220,8 @@ int dcn_mfma_backward(const void *x, const void *off, const void *mask, const vo
                       const void *gy, void *goff, void *gmask, const DcnDims &s, int dtype,
                       void *workspace, float **gx32, float **gw32, float **gb32,
                       hipStream_t stream);
+void dcn_set_column_budget(size_t bytes);
+size_t dcn_column_budget();
 int dcn_planar_add(const float *gxt, void *gx, const DcnDims &s, int dtype, hipStream_t stream);
 int dcn_weight_add(const float *acc, void *gw, const DcnDims &s, int dtype, hipStream_t stream);
 
@@ -362,6 +366,9 @@ static int make_dcn_dims_2d(DcnDims &d, const mv_dcn2d_shape *s) {
                             s->groups, s->deformable_groups};
   return make_dcn_dims(d, &v, 2);
 }
+
+void mv_dcn_set_column_budget(size_t bytes) { dcn_set_column_budget(bytes); }
+size_t mv_dcn_column_budget(void) { return dcn_column_budget(); }
 
 size_t mv_dcn3d_forward_workspace_bytes(const mv_dcn3d_shape *shape, int dtype) {
   DcnDims s;

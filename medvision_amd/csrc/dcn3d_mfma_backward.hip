@@ -24,6 +24,7 @@
 // tap-major fp32 gradient once per workgroup.
 #include "dcn_mfma.hpp"
 
+#include <atomic>
 #include <cstdlib>
 
 namespace mv {
@@ -855,12 +856,19 @@ struct BackwardLayout {
   long qp;  // positions per row of the column buffer; 0: no buffer (the weight kernel gathers again)
 };
 // The column buffer holds mask * Z(x) for every (sample, tap, channel, position): it saves the
-// weight kernel the second gather of x.  Layers whose columns exceed the budget (1 GiB, or the value
-// of MV_DCN_COLUMN_BYTES) do without.
-static size_t column_budget() {
-  const char *e = getenv("MV_DCN_COLUMN_BYTES");
-  return e ? static_cast<size_t>(strtoull(e, nullptr, 10)) : (static_cast<size_t>(1) << 30);
+// weight kernel the second gather of x.  Layers whose columns exceed the budget do without.  The
+// budget is 1 GiB unless the environment variable MV_DCN_COLUMN_BYTES (read once, when the library
+// is first asked) or mv_dcn_set_column_budget() says otherwise.
+static std::atomic<size_t> &column_budget_cell() {
+  static std::atomic<size_t> cell{[] {
+    const char *e = getenv("MV_DCN_COLUMN_BYTES");
+    return e ? static_cast<size_t>(strtoull(e, nullptr, 10)) : (static_cast<size_t>(1) << 30);
+  }()};
+  return cell;
 }
+static size_t column_budget() { return column_budget_cell().load(std::memory_order_relaxed); }
+void dcn_set_column_budget(size_t bytes) { column_budget_cell().store(bytes, std::memory_order_relaxed); }
+size_t dcn_column_budget() { return column_budget(); }
 static BackwardLayout backward_layout(const DcnDims &s, int dtype) {
   BackwardLayout l;
   const size_t es = dtype == MV_F32 ? 4 : 2;

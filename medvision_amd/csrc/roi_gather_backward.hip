@@ -74,7 +74,7 @@ __global__ __launch_bounds__(kGatherThreads) void roi_backward_gather_kernel(
     if (threadIdx.x < 3) {
       const int j = threadIdx.x;
       sh.reach[j] = fabs(sh.g.rot[j]) + fabs(sh.g.rot[3 + j]) + fabs(sh.g.rot[6 + j]) + kSlack;
-      sh.inv_bin[j] = sh.g.bin[j] > 1e-12 ? 1.0 / sh.g.bin[j] : 0.0;
+      sh.inv_bin[j] = fabs(sh.g.bin[j]) > 1e-12 ? 1.0 / sh.g.bin[j] : 0.0;   // negative for a mirrored roi
       const float slack = 1e-3f + 1e-6f * static_cast<float>(p.W + p.H + p.D);
       sh.r1[j] = static_cast<float>(sh.g.rot[3 * j + 1]);
       sh.r2[j] = static_cast<float>(sh.g.rot[3 * j + 2]);
@@ -84,7 +84,7 @@ __global__ __launch_bounds__(kGatherThreads) void roi_backward_gather_kernel(
         sh.inv_bin0 = static_cast<float>(sh.inv_bin[0]);
         sh.off0 = static_cast<float>(sh.g.start[0] * sh.inv_bin[0] + 0.5);
         sh.slack = slack;
-        sh.slack_u = 1e-3f + 1e-6f * static_cast<float>(p.ow) + slack * sh.inv_bin0;
+        sh.slack_u = 1e-3f + 1e-6f * static_cast<float>(p.ow) + slack * fabsf(sh.inv_bin0);
       }
     }
     __syncthreads();
@@ -126,8 +126,10 @@ __global__ __launch_bounds__(kGatherThreads) void roi_backward_gather_kernel(
         // cells u with |start + (u + .5) * bin - q| <= reach
         const double a0 = q - reach[j] - g.start[j], a1 = q + reach[j] - g.start[j];
         if (inv_bin[j] != 0.0) {
-          const double u0 = fmin(fmax(a0 * inv_bin[j] - 0.5 - kSlack, -1.0), static_cast<double>(cells[j]));
-          const double u1 = fmin(fmax(a1 * inv_bin[j] - 0.5 + kSlack, -1.0), static_cast<double>(cells[j]));
+          // (a negative bin, i.e. a mirrored roi, swaps the two ends)
+          const double e0 = a0 * inv_bin[j] - 0.5, e1 = a1 * inv_bin[j] - 0.5;
+          const double u0 = fmin(fmax(fmin(e0, e1) - kSlack, -1.0), static_cast<double>(cells[j]));
+          const double u1 = fmin(fmax(fmax(e0, e1) + kSlack, -1.0), static_cast<double>(cells[j]));
           lo[j] = max(static_cast<int>(ceil(u0)), 0);
           hi[j] = min(static_cast<int>(floor(u1)), cells[j] - 1);
         } else {   // every cell samples the same coordinate
@@ -164,8 +166,9 @@ __global__ __launch_bounds__(kGatherThreads) void roi_backward_gather_kernel(
           if (xl > xh) continue;
           int x0 = lo[0], x1 = hi[0];
           if (inv_bin0 != 0.f) {
-            const float u0 = fminf(fmaxf(fmaf(xl, inv_bin0, -off0) - slack_u, -1.f), cells0);
-            const float u1 = fminf(fmaxf(fmaf(xh, inv_bin0, -off0) + slack_u, -1.f), cells0);
+            const float e0 = fmaf(xl, inv_bin0, -off0), e1 = fmaf(xh, inv_bin0, -off0);
+            const float u0 = fminf(fmaxf(fminf(e0, e1) - slack_u, -1.f), cells0);
+            const float u1 = fminf(fmaxf(fmaxf(e0, e1) + slack_u, -1.f), cells0);
             x0 = max(x0, static_cast<int>(ceilf(u0)));
             x1 = min(x1, static_cast<int>(floorf(u1)));
           }

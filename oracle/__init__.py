@@ -118,6 +118,24 @@ def roi_align_forward(features, rois, output_size, spatial_scale=1.0, sampling_r
     return out[:, :, 0] if ndim == 2 else out
 
 
+def roi_decision_margin(features_shape, rois, output_size, spatial_scale=1.0, sampling_ratio=0,
+                        aligned=True, rotated=False):
+    """[R, (od,) oh, ow]: distance (voxels) of each output cell's samples from a decision of the
+    nearest-neighbour sampler (a 0.5 tie between two voxels, or the -1 / S edge of the void).
+    A test may accept a differing order-0 output only where this is within the coordinate
+    rounding of the kernel under test."""
+    ndim, N, C, D, H, W = _roi_common(tuple(features_shape), rois, rotated)
+    od, oh, ow = _out_dims(ndim, output_size)
+    r = _f64(rois)
+    R = r.shape[0]
+    out = torch.zeros((R, od, oh, ow), dtype=torch.float64)
+    if R:
+        lib().orc_roi_decision_margin(_ptr(r), _ptr(out), ndim, int(bool(rotated)), D, H, W, R,
+                                      od, oh, ow, ctypes.c_double(_f32(spatial_scale)),
+                                      int(sampling_ratio), int(bool(aligned)))
+    return out[:, 0] if ndim == 2 else out
+
+
 def roi_align_backward(grad_output, rois, features_shape, spatial_scale=1.0, sampling_ratio=0,
                        aligned=True, order=1, rotated=False):
     """Adjoint of :func:`roi_align_forward`; returns grad wrt features (fp64, zero-initialised)."""

@@ -299,6 +299,62 @@ void orc_roi_align_forward(const double *feat, const double *rois, double *out, 
     }
 }
 
+/* How far the samples of each output cell are from a DECISION of the order-0 (nearest) sampler:
+ * a coordinate at exactly -1 or S (value or void, interpolation_helpers_3d.h:136) or a fraction of
+ * exactly 0.5 (low or high neighbour, :186-194).  out [R,od,oh,ow] receives the smallest such
+ * distance over the cell's samples and axes, in voxels; a sample that is void by more than the
+ * distance on one axis does not count on the others.  Tests use it to tell a legitimate
+ * difference (arithmetic of different precision picks the other side of a tie) from a wrong
+ * voxel.  Same geometry code as the forward above. */
+static double axis_margin(double v, int size) {
+  double m = fmin(fabs(v + 1.0), fabs(v - (double)size));
+  if (v < -1.0 || v > (double)size) return -m;          /* outside: negative distance */
+  if (v <= 0) v = 0;
+  int base = (int)v;
+  if (base < size - 1) m = fmin(m, fabs((v - base) - 0.5));
+  return m;
+}
+
+void orc_roi_decision_margin(const double *rois, double *out, int ndim, int rotated, int D, int H,
+                             int W, int R, int od, int oh, int ow, double scale, int sr,
+                             int aligned) {
+  const int cols = roi_cols(ndim, rotated);
+  const int cells[3] = {ow, oh, od};
+  const int size[3] = {W, H, D};
+  const long oplane = (long)od * oh * ow;
+#pragma omp parallel for schedule(dynamic)
+  for (int n = 0; n < R; n++) {
+    roi_geom g;
+    if (rotated) geom_rotated(&g, rois + (long)n * cols, ndim, scale, sr, aligned, cells);
+    else geom_plain(&g, rois + (long)n * cols, ndim, scale, sr, cells);
+    const int gz = ndim == 3 ? g.grid[2] : 1;
+    for (int pd = 0; pd < od; pd++)
+      for (int ph = 0; ph < oh; ph++)
+        for (int pw = 0; pw < ow; pw++) {
+          double best = 1e300;
+          for (int iz = 0; iz < gz; iz++) {
+            double z = ndim == 3 ? local_coord(&g, 2, pd, iz) : 0.0;
+            for (int iy = 0; iy < g.grid[1]; iy++) {
+              double y = local_coord(&g, 1, ph, iy);
+              for (int ix = 0; ix < g.grid[0]; ix++) {
+                double x = local_coord(&g, 0, pw, ix);
+                double r[3];
+                to_global(&g, ndim, x, y, z, r);
+                double inside = 1e300, outside = 0.0;
+                for (int a = 0; a < ndim; a++) {
+                  double m = axis_margin(r[a], size[a]);
+                  if (m < 0) outside = fmax(outside, -m);
+                  else inside = fmin(inside, m);
+                }
+                best = fmin(best, outside > 0 ? outside : inside);
+              }
+            }
+          }
+          out[(long)n * oplane + ((long)pd * oh + ph) * ow + pw] = best;
+        }
+  }
+}
+
 /* Backward (adjoint) of the above: grad_in [N,C,D,H,W] is ACCUMULATED into, as the reference
  * kernels do with atomicAdd on a caller-zeroed buffer.
  * roi_align_3d_backward_cuda_kernel (cuda/roi_align_3d_cuda_kernel.cuh:90-202) and twins. */

@@ -81,3 +81,14 @@ def test_product_does_not_import_the_oracle():
         for f in files:
             if f.endswith((".py", ".hip", ".hpp", ".h")):
                 assert "oracle" not in open(os.path.join(dirpath, f)).read().lower(), f
+
+
+def test_foreign_device_tensors_are_refused():
+    """Every tensor handed to a kernel must sit on the input's device; the check runs on the host."""
+    from medvision_amd import _C
+    here, there = torch.zeros(2), torch.zeros(2, device="meta")
+    _C._same_device(here, weight=here, bias=None)
+    with pytest.raises(RuntimeError, match="weight is on meta"):
+        _C._same_device(here, weight=there)
+    with pytest.raises(RuntimeError, match="grad_input is on meta"):
+        _C._same_device(here, output=here, grad_input=there)

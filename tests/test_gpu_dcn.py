@@ -166,11 +166,19 @@ def test_input_gradient_through_lds_tiles_5x5x5(ops, oracle):
     assert_close(ws.grad, gw, tol, "grad weight")
 
 
-def test_weight_gradient_without_column_buffer(ops, oracle, monkeypatch):
+def test_weight_gradient_without_column_buffer(ops, oracle):
     """Layers whose column values would not fit the buffer's budget gather x a second time in the
-    weight kernel: forced here through MV_DCN_COLUMN_BYTES."""
+    weight kernel: forced here by a budget of zero bytes."""
+    from medvision_amd import _C
     from medvision_amd.ops.modulated_deform_conv_3d import modulated_deform_conv
-    monkeypatch.setenv("MV_DCN_COLUMN_BYTES", "0")
+    old = _C.set_dcn_column_budget(0)
+    try:
+        _weight_gradient_without_column_buffer(oracle, modulated_deform_conv)
+    finally:
+        _C.set_dcn_column_budget(old)
+
+
+def _weight_gradient_without_column_buffer(oracle, modulated_deform_conv):
     g = wl.gen(450)
     x, off, mask, w, b = wl.dcn_inputs(g, 2, 32, 64, (7, 9, 11), 3, 1, 1, torch.float16, 1, 1, 1, True, 2.0)
     xs, offs, ms, ws, bs = [t.to(DEV).requires_grad_(True) for t in (x, off, mask, w, b)]
@@ -215,6 +223,58 @@ def test_config4_full_size_properties(ops):
     y1 = modulated_deform_conv(xs, offs, ms, ws, None, 1, 1, 1, 1, 1)
     y2 = modulated_deform_conv(xs, offs, ms * 0.5, ws, None, 1, 1, 1, 1, 1)
     assert_close(y2.float() * 2, y1.float(), 4e-3, "mask linearity")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_config4_full_size_backward_properties(ops, dtype):
+    """The backward pass at the full config-4 size [2,32,48^3] -> 64 channels, where the CPU oracle
+    would take minutes.  (1) Zero offsets and a unit mask make the layer a plain convolution: the
+    gradients of input, weight and bias must equal torch's conv3d autograd in fp32.  (2) At the
+    configuration's own offsets (sigma = 2 voxels) and mask the output is linear in the input, in
+    the weight and in the mask, so <gy, y - bias> = <gx, x> = <gw, w> = <gmask, mask>; the offset
+    gradient is checked through a central difference along a random direction (the trilinear form
+    is piecewise linear in the offsets)."""
+    from medvision_amd.ops.modulated_deform_conv_3d import modulated_deform_conv
+    g = wl.gen(6)
+    x, off, mask, w, b = wl.dcn_inputs(g, 2, 32, 64, (48, 48, 48), 3, 1, 1, dtype)
+    gy = torch.randn(2, 64, 48, 48, 48, generator=g).to(dtype)
+    tol = {torch.float32: 1e-4, torch.float16: 4e-3, torch.bfloat16: 1.6e-2}[dtype]
+
+    # (1) plain convolution
+    xs, ws, bs = [t.to(DEV).requires_grad_(True) for t in (x, w, b)]
+    offs = torch.zeros_like(off, device=DEV)
+    ms = torch.ones_like(mask, device=DEV)
+    y = modulated_deform_conv(xs, offs, ms, ws, bs, 1, 1, 1, 1, 1)
+    y.backward(gy.to(DEV))
+    xr, wr, br = [t.to(DEV).float().requires_grad_(True) for t in (x, w, b)]
+    F.conv3d(xr, wr, br, 1, 1).backward(gy.to(DEV).float())
+    assert_close(xs.grad, xr.grad, tol, "grad input == conv3d")
+    assert_close(ws.grad, wr.grad, tol, "grad weight == conv3d")
+    assert_close(bs.grad, br.grad, tol, "grad bias == conv3d")
+    del xr, wr, br, y
+
+    # (2) adjoint identities at the real offsets
+    xs, offs, ms, ws = [t.to(DEV).requires_grad_(True) for t in (x, off, mask, w)]
+    y = modulated_deform_conv(xs, offs, ms, ws, None, 1, 1, 1, 1, 1)
+    gyd = gy.to(DEV)
+    y.backward(gyd)
+    dot = lambda a, c: float((a.double() * c.double()).sum())
+    lhs = dot(gyd, y)
+    scale = float(gyd.double().norm() * y.double().norm())
+    for name, grad, val in (("input", xs.grad, xs), ("weight", ws.grad, ws), ("mask", ms.grad, ms)):
+        assert abs(dot(grad, val) - lhs) <= tol * scale, (name, dot(grad, val), lhs, scale)
+    assert torch.isfinite(offs.grad).all()
+    if dtype == torch.float32:   # a directional derivative needs the resolution of fp32 outputs
+        # direction along the gradient's signs: the derivative is a sum of positive terms
+        d = torch.randn(off.shape, generator=g).abs().to(DEV) * offs.grad.sign()
+        eps = 1e-3
+        with torch.no_grad():
+            yp = modulated_deform_conv(xs, offs + eps * d, ms, ws, None, 1, 1, 1, 1, 1)
+            ym = modulated_deform_conv(xs, offs - eps * d, ms, ws, None, 1, 1, 1, 1, 1)
+        fd = dot(gyd, yp - ym) / (2 * eps)
+        an = dot(offs.grad, d)
+        # samples that cross a voxel boundary within +-eps (under 1 % of them) see a kink
+        assert an > 0 and abs(fd - an) <= 3e-2 * an, (fd, an)
 
 
 def test_modules_state_dict_and_autocast_training(ops):
@@ -267,6 +327,11 @@ def test_dcn_errors(ops):
         _C.deform_conv_3d_forward(x.cpu(), w.cpu(), b.cpu(), off.cpu(), *args, 64)
     with pytest.raises(RuntimeError, match="offset has shape"):
         _C.deform_conv_3d_forward(x, w, b, off[:, :80].contiguous(), *args, 64)
+    # a tensor left on the host must raise on the host, not fault on the GPU
+    with pytest.raises(RuntimeError, match="weight is on cpu"):
+        _C.deform_conv_3d_forward(x, w.cpu(), b, off, *args, 64)
+    with pytest.raises(RuntimeError, match="bias is on cpu"):
+        _C.deform_conv_3d_forward(x, w, b.cpu(), off, *args, 64)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16, torch.bfloat16])

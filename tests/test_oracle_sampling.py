@@ -130,3 +130,23 @@ def test_cubic_edge_table(oracle):
     assert abs(oracle.sample_cubic(vol.reshape(4, 1, 1), 3.5, 0.0, 0.0) - 82.5) < 1e-9
     assert oracle.sample_cubic(vol.reshape(4, 1, 1), 4.0000001, 0.0, 0.0) == 0.0
     assert abs(oracle.sample_cubic(vol.reshape(4, 1)[:, :], 0.0, 3.5, 0.0) - 82.5) < 1e-9  # 2-D
+
+
+def test_decision_margin_hand_values(oracle):
+    """Distance of nearest-neighbour samples from a tie / the edge of the void, by hand: an
+    identity roi samples voxel centres (0.5 from every tie, the last voxel 1 from the edge S); a
+    quarter-voxel shift puts samples at -0.25 (clamped to 0: no tie), 0.75 and 1.75; a half-voxel
+    shift puts them exactly on ties; far outside the distance to the volume counts."""
+    shape = (1, 1, 3, 3, 3)
+    roi = lambda cx: torch.tensor([[0, cx, 1.5, 1.5, 3, 3, 3, 0, 0, 0.]])
+    m = oracle.roi_decision_margin(shape, roi(1.5), (3, 3, 3), 1.0, 1, True, True)
+    assert m.shape == (1, 3, 3, 3) and float(m[0, 0, 0, 0]) == 0.5 and float(m[0, 2, 2, 2]) == 1.0
+    m = oracle.roi_decision_margin(shape, roi(1.25), (3, 3, 3), 1.0, 1, True, True)
+    assert m[0, 0, 0].tolist() == [0.5, 0.25, 0.25]
+    m = oracle.roi_decision_margin(shape, roi(2.0), (3, 3, 3), 1.0, 1, True, True)
+    assert m[0, 0, 0].tolist() == [0.0, 0.0, 0.5]          # 0.5, 1.5 are ties; 2.5 clamps to 2
+    m = oracle.roi_decision_margin(shape, roi(7.0), (3, 3, 3), 1.0, 1, True, True)
+    assert m[0, 1, 1].tolist() == [2.5, 3.5, 4.5]          # samples at 5.5, 6.5, 7.5; S = 3
+    # plain boxes, 2-D, two samples per cell: the smaller of the two distances
+    m = oracle.roi_decision_margin((1, 1, 4, 4), torch.tensor([[0, 0.0, 0.0, 4.0, 4.0]]), (2, 2), 1.0, 2, True, False)
+    assert m.shape == (1, 2, 2) and float(m[0, 0, 0]) == 0.0   # samples at 0.5 and 1.5
