@@ -6,7 +6,7 @@ import math
 import pytest
 import torch
 
-from parity import BWD_TOL, FWD_TOL, assert_close, rel_err
+from parity import BWD_TOL, FWD_TOL, assert_close, assert_nearest, rel_err
 import workloads as wl
 
 pytestmark = pytest.mark.gpu
