@@ -142,6 +142,20 @@ int mv_dcn3d_backward(const void *input, const void *offset, const void *mask, c
 void mv_dcn_set_column_budget(size_t bytes);
 size_t mv_dcn_column_budget(void);
 
+/* mv_dcn3d_forward for callers that cannot allocate or provide device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): no counterpart in the reference.
+ * Same arguments and results as mv_dcn3d_forward without `workspace`: the layout buffers live in a
+ * fixed array of MV_DCN3D_STATIC_SCRATCH_BYTES in the library's device image (every GPU the
+ * library runs on holds it until the process ends).  Calls no hipMalloc / hipFree or allocating
+ * library routine; the first call on a device looks the array's address up.  Layers whose
+ * mv_dcn3d_forward_workspace_bytes() exceeds the array are rejected with MV_INVALID_ARGUMENT.
+ * All calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads)
+ * race; serialise them.                                                                        */
+#define MV_DCN3D_STATIC_SCRATCH_BYTES ((size_t)32 << 20)
+int mv_dcn3d_forward_static(const void *input, const void *offset, const void *mask,
+                            const void *weight, const void *bias, void *output,
+                            const mv_dcn3d_shape *shape, int dtype, void *stream);
+
 /* ---- deformable convolution 2-D -----------------------------------------------------------
  * replaces deform_conv_2d_forward / _backward                 csrc/deform_conv_2d.h:41,76
  *          modulated_deform_conv_2d_forward / _backward       csrc/modulated_deform_conv_2d.h:23,47

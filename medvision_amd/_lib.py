@@ -58,6 +58,7 @@ SIGNATURES = {
     "mv_dcn3d_backward": (_i, [_p] * 10 + [_SHAPE_P, _i, _p, _p]),
     "mv_dcn_set_column_budget": (None, [_sz]),
     "mv_dcn_column_budget": (_sz, []),
+    "mv_dcn3d_forward_static": (_i, [_p] * 6 + [_SHAPE_P, _i, _p]),
     "mv_dcn2d_output_dims": (_i, [_SHAPE2_P, ctypes.POINTER(_i), ctypes.POINTER(_i)]),
     "mv_dcn2d_forward_workspace_bytes": (_sz, [_SHAPE2_P, _i]),
     "mv_dcn2d_backward_workspace_bytes": (_sz, [_SHAPE2_P, _i]),

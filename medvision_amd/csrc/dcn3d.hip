@@ -399,6 +399,48 @@ int mv_dcn3d_backward(const void *input, const void *offset, const void *mask, c
                                grad_mask, grad_weight, grad_bias, s, dtype, workspace, stream);
 }
 
+// ---- forward without any allocation --------------------------------------------------------
+// Callers that cannot allocate (code under graph capture, serving loops, harnesses that forbid
+// hipMalloc) get the forward pass with the workspace taken from a fixed array in device memory.
+// Each GPU the library runs on holds its own copy of the array at its own address; the address is
+// looked up once per device, on the first call there, and only that pointer is handed to kernels.
+constexpr size_t kStaticScratchBytes = MV_DCN3D_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kScratchDevices = 64;
+static std::atomic<void *> scratch_address[kScratchDevices];
+
+static int static_scratch(void **ptr) {
+  int dev = -1;
+  MV_HIP_CHECK(hipGetDevice(&dev));
+  MV_REQUIRE(dev >= 0 && dev < kScratchDevices, "device index beyond the table of scratch addresses");
+  void *p = scratch_address[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {   // first call on this device (two threads racing resolve the same address)
+    MV_HIP_CHECK(hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(scratch)));
+    MV_REQUIRE(p != nullptr, "the static scratch array has no address on this device");
+    scratch_address[dev].store(p, std::memory_order_release);
+  }
+  *ptr = p;
+  return MV_OK;
+}
+
+int mv_dcn3d_forward_static(const void *input, const void *offset, const void *mask,
+                            const void *weight, const void *bias, void *output,
+                            const mv_dcn3d_shape *shape, int dtype, void *stream) {
+  DcnDims s;
+  const int st = make_dcn_dims(s, shape);
+  if (st) return st;
+  const size_t need = forward_workspace(s, dtype);
+  MV_REQUIRE(need <= kStaticScratchBytes,
+             "mv_dcn3d_forward_static: this layer needs a workspace of %zu bytes, the static scratch holds "
+             "%zu; use mv_dcn3d_forward with a caller-provided workspace", need, kStaticScratchBytes);
+  void *ws = nullptr;
+  if (need > 0) {
+    const int sc = static_scratch(&ws);
+    if (sc) return sc;
+  }
+  return dcn_forward_any(input, offset, mask, weight, bias, output, s, dtype, ws, stream);
+}
+
 int mv_dcn2d_output_dims(const mv_dcn2d_shape *shape, int *out_h, int *out_w) {
   DcnDims s;
   const int st = make_dcn_dims_2d(s, shape);
