@@ -25,22 +25,62 @@ namespace mv {
 
 constexpr int kXcds = 8;
 
-struct TilePlan {          // 208 bytes
-  double org[3];           // box-relative source position (x,y,z) of the tile's first output voxel
-  double inc[9];           // d(source a)/d(output j) at inc[a * 3 + j], j = (x, y, z)
-  int lo[3];               // first staged source voxel (x, y, z)
-  int n[3];                // staged extent
-  int batch;               // feature-map index of the roi
-  int mode;                // 0 = all zero, 1 = staged (clipped box), 2 = gather, 3 = staged interior
-  int t0[3];               // first output voxel of the tile (x, y, z)
-  int roi;                 // roi index
-  int rp;                  // box rows copied per pass of the workgroup: `span` whole z-slices
-  int span;                // z-slices per pass
-  int passes;              // ceil(n[2] / span), or 0: the box does not go through registers
-  int spare;
-  float orgf[3], incf[9];  // org / inc rounded to fp32 (coordinate type of the 16-bit kernels)
+// What the workgroup's first wavefront works out per item and every wavefront then reads from LDS.
+// Values a wavefront needs in scalar registers sit in the first 64 dwords (lane l fetches dword l,
+// fields are pulled out with v_readlane); values only the vector unit uses are read as broadcasts.
+struct TilePlan {            // 320 bytes
+  // per source axis a, at [4 * a .. 4 * a + 3]: the box-relative source position of the tile's
+  // first output voxel, then d(source a)/d(output j) for j = (x, y, z)
+  double map[12];            // dword 0
+  float mapf[12];            // dword 24: the same rounded to fp32 (coordinate type of the 16-bit kernels)
+  int mode;                  // dword 36: 0 = all zero, 1 = staged (clipped box), 2 = gather, 3 = staged interior, 4 = no item
+  int passes;                // copy passes through registers (ceil(n[2] / span)), 0: the box is copied in place
+  unsigned src_lo, src_hi;   // byte offset of the box's first voxel in the feature tensor
+  int extent;                // bytes from there to the end of the box's last row
+  int stride;                // bytes between the passes of a lane (span slices)
+  unsigned out_lo, out_hi;   // byte offset of the item's (roi, channel) volume in the output tensor
+  int zcount;                // output slices from the tile's first one to the end of the volume
+  int pad0[3];
+  // dword 48: a lane splits its index into (slice, row, 16-byte group) with two multiplications
+  float inv_groups, inv_rows;
+  int groups, by;
+  // dword 52
+  int rp;                    // box rows per pass (span whole slices)
+  int pad1;
+  int bz, span;
+  // dword 56: LDS geometry in bytes (dy / dz: 0 when the box is one row / slice thick)
+  int pitch_b, slice_b, dy_b, dz_b;
+  // dword 60: the tile in the output volume
+  int tile_off;              // byte offset of the tile's first voxel
+  int xlim, ylim;            // columns / rows from the tile's first voxel to the end of the volume
+  int hop_b;                 // LDS bytes per pass
+  // dword 64
+  int lo[3];                 // first staged source voxel (x, y, z)
+  int n[3];                  // staged extent
+  int t0[3];                 // first output voxel of the tile (x, y, z)
+  int roi;                   // roi index
+  int batch;                 // feature-map index of the roi
+  unsigned vol_lo, vol_hi;   // byte offset of the item's (image, channel) volume in the feature tensor
+  int pad2[3];
+  // dword 80: box-relative limits of a clipped box as fp32: coordinates clamp to [0, cmax], the
+  // low tap index is at most top = max(n - 2, 0)
+  float cmaxf[4], topf[4];
 };
-static_assert(sizeof(TilePlan) == 208, "plan record size");
+static_assert(sizeof(TilePlan) == 352 && offsetof(TilePlan, inv_groups) == 192 && offsetof(TilePlan, lo) == 256, "plan record layout");
+
+// Division of n < 2^31 by a divisor fixed at launch: one 64-bit product and a shift.
+struct FastDiv {
+  unsigned mul, shift;
+  __host__ void set(unsigned d) {
+    unsigned s = 0;
+    while ((2u << s) <= d && s < 30) s++;          // s = floor(log2 d)
+    if ((d & (d - 1)) == 0) { mul = 0x80000000u; shift = 31 + s; }
+    else { mul = static_cast<unsigned>(((1ull << (32 + s)) + d - 1) / d); shift = 32 + s; }
+  }
+  __device__ __forceinline__ unsigned div(unsigned n) const {
+    return static_cast<unsigned>((static_cast<unsigned long long>(n) * mul) >> shift);
+  }
+};
 
 struct PlanShape {
   int tiles_x, tiles_y, tiles_z;  // spatial tiles per roi
@@ -48,6 +88,8 @@ struct PlanShape {
   int vec;                        // elements per aligned 16-byte group (0: rows are not aligned)
   int cap;                        // LDS capacity in elements
   int threads, max_items;         // workgroup size, 16-byte groups one lane holds in registers
+  int es;                         // bytes per element
+  FastDiv by_per_roi, by_tiles_x, by_tiles_y, by_total, by_slots;
   int halo_lo, halo_hi;           // voxels needed below / above the cell of a sample: 0 / 1, order 3: 1 / 2
 };
 
@@ -73,7 +115,8 @@ __device__ inline void plan_item_lanes(const float *__restrict__ rois, const Roi
   const int lane = threadIdx.x & (kWave - 1), a = lane & 3, base = lane & ~3;
   const bool write = item != kDone && a < 3;
   const unsigned it = item != kDone ? item : 0u;
-  const unsigned idx = p.C > 1 ? it % total : it, n = idx / per_roi, tile = idx - n * per_roi;
+  const unsigned chan = p.C > 1 ? ps.by_total.div(it) : 0u;
+  const unsigned idx = it - chan * total, n = ps.by_per_roi.div(idx), tile = idx - n * per_roi;
   const int nd = p.ndim, is3d = nd == 3, ax = a < 3 ? a : 0;
   const float *roi = rois + static_cast<long>(n) * roi_columns(nd, p.rotated);
 
@@ -124,7 +167,7 @@ __device__ inline void plan_item_lanes(const float *__restrict__ rois, const Roi
   }
 
   // ---- the tile along axis `ax` -----------------------------------------------------------------
-  const unsigned qx = tile / static_cast<unsigned>(ps.tiles_x), qy = qx / static_cast<unsigned>(ps.tiles_y);
+  const unsigned qx = ps.by_tiles_x.div(tile), qy = ps.by_tiles_y.div(qx);
   const int tpos = ax == 0 ? static_cast<int>(tile - qx * ps.tiles_x)
                            : (ax == 1 ? static_cast<int>(qx - qy * ps.tiles_y) : static_cast<int>(qy));
   const int t0 = tpos * tile_ext;
@@ -162,43 +205,75 @@ __device__ inline void plan_item_lanes(const float *__restrict__ rois, const Roi
     org = pos - static_cast<double>(l);
   }
   const int n0 = lane_get(cnt, base), n1 = lane_get(cnt, base + 1), n2 = lane_get(cnt, base + 2);
+  const int l0 = lane_get(lo, base), l1 = lane_get(lo, base + 1), l2 = lane_get(lo, base + 2);
+  const int ty0 = lane_get(t0, base + 1), tz0 = lane_get(t0, base + 2);
   const int any_empty = lane_get(empty, base) | lane_get(empty, base + 1) | lane_get(empty, base + 2);
   const int any_clip = lane_get(clipped, base) | lane_get(clipped, base + 1) | lane_get(clipped, base + 2);
+  // LDS row pitch: the row's 16-byte groups, or (unaligned rows) the row plus one finite pad
+  const int groups = ps.vec > 0 ? n0 / ps.vec : 0;
+  const int pitch = ps.vec > 0 ? n0 : n0 + 1;
+  const int es = ps.es;
+  const long hw = static_cast<long>(p.H) * p.W;
+  const long vol = (static_cast<long>(batch < 0 ? 0 : batch) * p.C + chan) * (hw * p.D) * es;
+  int span = 0;
+  if (a == 0) {
+    if (item == kDone) {
+      dst->mode = 4;
+    } else {
+      const long rows = static_cast<long>(n1) * n2;
+      // register staging: a pass copies `span` whole z-slices, one 16-byte group per lane
+      int passes = 0;
+      if (ps.vec > 0) {
+        const int per_slice = n1 * groups;   // small integers: the float quotients below are exact
+        const int sp = min(static_cast<int>(static_cast<float>(ps.threads) / static_cast<float>(per_slice)), n2);
+        if (sp >= 1) {
+          const int ps_ = static_cast<int>(static_cast<float>(n2 + sp - 1) / static_cast<float>(sp));
+          if (ps_ <= ps.max_items) { span = sp; passes = ps_; }
+        }
+      }
+      const bool fits = rows * pitch <= ps.cap;
+      int mode;
+      if (batch < 0 || any_empty || !grids) mode = 0;   // (grid != 1 cannot happen: ratio is 1)
+      else if (!fits) mode = 2;
+      else mode = any_clip ? 1 : 3;
+      const int rp = span * n1;
+      const long src = vol + ((static_cast<long>(l2) * p.H + l1) * p.W + l0) * es;
+      dst->mode = mode;
+      dst->passes = passes;
+      dst->src_lo = static_cast<unsigned>(src); dst->src_hi = static_cast<unsigned>(src >> 32);
+      dst->extent = static_cast<int>((((n2 - 1) * hw + static_cast<long>(n1 - 1) * p.W + n0) * es));
+      dst->stride = static_cast<int>(span * hw * es);
+      dst->inv_groups = 1.0f / static_cast<float>(max(groups, 1));
+      dst->inv_rows = 1.0f / static_cast<float>(n1);
+      dst->groups = groups; dst->by = n1;
+      dst->rp = rp; dst->bz = n2; dst->span = span;
+      dst->hop_b = rp * pitch * es;
+    }
+  }
   if (!write) return;
-  dst->org[a] = org;
-  dst->orgf[a] = static_cast<float>(org);
+  dst->map[a * 4] = org;
+  dst->mapf[a * 4] = static_cast<float>(org);
 #pragma unroll
   for (int j = 0; j < 3; j++) {
-    dst->inc[a * 3 + j] = inc[j];
-    dst->incf[a * 3 + j] = static_cast<float>(inc[j]);
+    dst->map[a * 4 + 1 + j] = inc[j];
+    dst->mapf[a * 4 + 1 + j] = static_cast<float>(inc[j]);
   }
   dst->lo[a] = lo;
   dst->n[a] = cnt;
   dst->t0[a] = t0;
+  dst->cmaxf[a] = static_cast<float>(S - 1 - lo);
+  dst->topf[a] = static_cast<float>(max(cnt - 2, 0));
   if (a != 0) return;
-  // LDS row pitch: the row's 16-byte groups, or (unaligned rows) the row plus one finite pad
-  const int groups = ps.vec > 0 ? n0 / ps.vec : 0;
-  const int pitch = ps.vec > 0 ? n0 : n0 + 1;
-  const long rows = static_cast<long>(n1) * n2;
-  // register staging: a pass copies `span` whole z-slices, one 16-byte group per lane
-  int rp = 0, span = 0, passes = 0;
-  if (ps.vec > 0) {
-    const int per_slice = n1 * groups;   // small integers: the float quotients below are exact
-    const int sp = min(static_cast<int>(static_cast<float>(ps.threads) / static_cast<float>(per_slice)), n2);
-    if (sp >= 1) {
-      const int ps_ = static_cast<int>(static_cast<float>(n2 + sp - 1) / static_cast<float>(sp));
-      if (ps_ <= ps.max_items) { span = sp; rp = sp * n1; passes = ps_; }
-    }
-  }
-  dst->batch = batch;
+  const long outv = (static_cast<long>(n) * p.C + chan) * (static_cast<long>(p.od) * p.oh * p.ow) * es;
+  dst->out_lo = static_cast<unsigned>(outv); dst->out_hi = static_cast<unsigned>(outv >> 32);
+  dst->zcount = p.od - tz0;
+  dst->pitch_b = pitch * es; dst->slice_b = n1 * pitch * es;
+  dst->dy_b = n1 > 1 ? pitch * es : 0; dst->dz_b = n2 > 1 ? n1 * pitch * es : 0;
+  dst->tile_off = ((tz0 * p.oh + ty0) * p.ow + t0) * es;
+  dst->xlim = p.ow - t0; dst->ylim = p.oh - ty0;
   dst->roi = static_cast<int>(n);
-  dst->rp = rp; dst->span = span; dst->passes = passes; dst->spare = 0;
-  const bool fits = rows * pitch <= ps.cap;
-  int mode;
-  if (batch < 0 || any_empty || !grids) mode = 0;   // (grid != 1 cannot happen: ratio is 1)
-  else if (!fits) mode = 2;
-  else mode = any_clip ? 1 : 3;
-  dst->mode = mode;
+  dst->batch = batch;
+  dst->vol_lo = static_cast<unsigned>(vol); dst->vol_hi = static_cast<unsigned>(vol >> 32);
 }
 
 constexpr unsigned kChunk = 32;     // consecutive items dealt to one XCD
@@ -369,35 +444,27 @@ __device__ __forceinline__ void staged_column(const T *__restrict__ tile, float 
   }
 }
 
-// A plan record held by a wave: lane l keeps dword l (the record has 52); fields are pulled into
-// scalar registers with v_readlane.  The records live in LDS, written by the workgroup itself.
+// The scalar part of a plan record held by a wavefront: lane l keeps dword l of the first 64; fields
+// are pulled into scalar registers with v_readlane.  The records live in LDS, written by the
+// workgroup itself.
 #define MV_PLAN_DW(field) (static_cast<int>(offsetof(TilePlan, field) / 4))
 struct PlanLanes {
   unsigned v;
   __device__ __forceinline__ int i32(int dw) const { return static_cast<int>(__builtin_amdgcn_readlane(v, dw)); }
-  __device__ __forceinline__ float f32(int dw) const { return __uint_as_float(__builtin_amdgcn_readlane(v, dw)); }
-  __device__ __forceinline__ double f64(int dw) const {
-    return __hiloint2double(static_cast<int>(__builtin_amdgcn_readlane(v, dw + 1)),
-                            static_cast<int>(__builtin_amdgcn_readlane(v, dw)));
+  __device__ __forceinline__ unsigned long u64(int dw) const {
+    return (static_cast<unsigned long>(__builtin_amdgcn_readlane(v, dw + 1)) << 32) | __builtin_amdgcn_readlane(v, dw);
   }
-  __device__ __forceinline__ int lo(int a) const { return i32(MV_PLAN_DW(lo) + a); }
-  __device__ __forceinline__ int n(int a) const { return i32(MV_PLAN_DW(n) + a); }
-  __device__ __forceinline__ int t0(int a) const { return i32(MV_PLAN_DW(t0) + a); }
-  __device__ __forceinline__ int batch() const { return i32(MV_PLAN_DW(batch)); }
-  __device__ __forceinline__ int mode() const { return i32(MV_PLAN_DW(mode)); }
-  __device__ __forceinline__ int roi() const { return i32(MV_PLAN_DW(roi)); }
-  __device__ __forceinline__ int rp() const { return i32(MV_PLAN_DW(rp)); }
-  __device__ __forceinline__ int span() const { return i32(MV_PLAN_DW(span)); }
-  __device__ __forceinline__ int passes() const { return i32(MV_PLAN_DW(passes)); }
 };
-template <typename CT> __device__ __forceinline__ CT plan_org(const PlanLanes &p, int a);
-template <> __device__ __forceinline__ float plan_org<float>(const PlanLanes &p, int a) { return p.f32(MV_PLAN_DW(orgf) + a); }
-template <> __device__ __forceinline__ double plan_org<double>(const PlanLanes &p, int a) { return p.f64(MV_PLAN_DW(org) + 2 * a); }
-template <typename CT> __device__ __forceinline__ CT plan_inc(const PlanLanes &p, int i);
-template <> __device__ __forceinline__ float plan_inc<float>(const PlanLanes &p, int i) { return p.f32(MV_PLAN_DW(incf) + i); }
-template <> __device__ __forceinline__ double plan_inc<double>(const PlanLanes &p, int i) { return p.f64(MV_PLAN_DW(inc) + 2 * i); }
+// A field of a record read straight from LDS into a scalar register (paths that are not hot).
+__device__ __forceinline__ int plan_scalar(const int *field) { return __builtin_amdgcn_readfirstlane(*field); }
+
+// the coordinate map of a record in the coordinate type CT
+template <typename CT> __device__ __forceinline__ const CT *plan_map(const TilePlan *r);
+template <> __device__ __forceinline__ const float *plan_map<float>(const TilePlan *r) { return r->mapf; }
+template <> __device__ __forceinline__ const double *plan_map<double>(const TilePlan *r) { return r->map; }
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 // One element through a buffer descriptor: offsets beyond the buffer drop the store, so lanes
 // without an output need no branch.
@@ -415,8 +482,175 @@ __device__ __forceinline__ void store_element(__amdgpu_buffer_rsrc_t rsrc, unsig
   }
 }
 
-struct BoxShape { int mode, bx, by, bz, rp, span, passes; };  // wave-uniform part of a plan used for staging
 constexpr unsigned kOutOfRange = 0x80000000u;  // beyond every buffer: the load returns zeros
+
+// floor as an integer in one instruction
+__device__ __forceinline__ int floor_int(float v) {
+  int i;
+  asm("v_cvt_flr_i32_f32 %0, %1" : "=v"(i) : "v"(v));
+  return i;
+}
+
+// The eight taps of one voxel of an INTERIOR tile (all taps of all samples lie inside the staged
+// box, coordinates are non-negative) with fp32 coordinates: floor as integer conversion, fraction
+// by v_fract, the byte offset of the low corner from two 24-bit multiply-adds.  `issue` sends the
+// LDS reads, `finish` blends; a column keeps the reads of the next voxel in flight while it
+// blends the current one.  g = (pitch, slice, dy, dz) in bytes.
+// fn(integral_constant<int, k>) for k = K .. N - 1
+template <int K, int N, typename F> __device__ __forceinline__ void column_steps(F fn) {
+  if constexpr (K < N) {
+    fn(std::integral_constant<int, K>{});
+    column_steps<K + 1, N>(fn);
+  }
+}
+
+template <typename T> struct Taps {
+  T v[8];
+  float wx, wy, wz;
+};
+// (On this hardware a wavefront's v_add_f32 / v_sub_f32 / v_mul_f32 / v_add_u32 take half the time
+// of three-operand and conversion instructions, so sums of products are written as separate
+// multiplications and additions where that does not cost accuracy: contraction is switched off.)
+template <typename T, int ORDER>
+__device__ __forceinline__ void interior_issue(Taps<T> &q, const T *__restrict__ tile, float rx, float ry,
+                                               float rz, const i32x4 g, float pitch_f, float slice_f) {
+#pragma clang fp contract(off)
+  const float lx = floorf(rx), ly = floorf(ry), lz = floorf(rz);
+  q.wx = rx - lx; q.wy = ry - ly; q.wz = rz - lz;
+  constexpr unsigned E = sizeof(T);
+  // byte offset of the low corner, exact in fp32 (far below 2^24)
+  const float row = ly * pitch_f, sl = lz * slice_f, xb = E == 2 ? lx + lx : lx * static_cast<float>(E);
+  const unsigned at = static_cast<unsigned>((xb + row) + sl);
+  const char *t = reinterpret_cast<const char *>(tile) + at;
+  const unsigned dy = g.z, dz = g.w;
+  if (ORDER == 0) {
+    const unsigned off = (q.wz <= 0.5f ? 0u : dz) + (q.wy <= 0.5f ? 0u : dy) + (q.wx <= 0.5f ? 0u : E);
+    q.v[0] = *reinterpret_cast<const T *>(t + off);
+  } else {
+    q.v[0] = *reinterpret_cast<const T *>(t);
+    q.v[1] = *reinterpret_cast<const T *>(t + E);
+    q.v[2] = *reinterpret_cast<const T *>(t + dy);
+    q.v[3] = *reinterpret_cast<const T *>(t + dy + E);
+    q.v[4] = *reinterpret_cast<const T *>(t + dz);
+    q.v[5] = *reinterpret_cast<const T *>(t + dz + E);
+    q.v[6] = *reinterpret_cast<const T *>(t + dz + dy);
+    q.v[7] = *reinterpret_cast<const T *>(t + dz + dy + E);
+  }
+}
+template <typename T, int ORDER, bool EXACT_ENDS>
+__device__ __forceinline__ float interior_finish(const Taps<T> &q) {
+  if (ORDER == 0) return load(&q.v[0]);
+  // the last tap read comes first: one wait covers all eight
+  const float x11 = mix(q.wx, load(&q.v[6]), load(&q.v[7])), x10 = mix(q.wx, load(&q.v[4]), load(&q.v[5]));
+  const float x01 = mix(q.wx, load(&q.v[2]), load(&q.v[3])), x00 = mix(q.wx, load(&q.v[0]), load(&q.v[1]));
+  if (EXACT_ENDS) return mix(q.wz, mix(q.wy, x00, x01), mix(q.wy, x10, x11));
+  // fractions below 1: a + w * (b - a), the difference on the fast path
+  const float y0 = fmaf(q.wy, x01 - x00, x00), y1 = fmaf(q.wy, x11 - x10, x10);
+  return fmaf(q.wz, y1 - y0, y0);
+}
+
+// Coordinate of slice k of a column from that of slice 0 with additions and multiplications by
+// 2 and 4 only (at most three roundings for k < 8): r(k) = r(k - 1) + s for odd k, r(k - 2) + 2 s
+// for k = 2 mod 4, r(k - 4) + 4 s for multiples of 4.
+struct ColumnCoord {
+  float last[3], anchor[3];
+  __device__ __forceinline__ void start(float b0, float b1, float b2) {
+    last[0] = anchor[0] = b0; last[1] = anchor[1] = b1; last[2] = anchor[2] = b2;
+  }
+  template <int K> __device__ __forceinline__ void step(float s0, float s1, float s2) {
+    const float s[3] = {s0, s1, s2};
+#pragma unroll
+    for (int a = 0; a < 3; a++) {
+      if (K % 2 == 1) last[a] = last[a] + s[a];
+      else if (K % 4 == 2) last[a] = fmaf(2.0f, s[a], anchor[a]);
+      else { last[a] = fmaf(4.0f, s[a], anchor[a]); anchor[a] = last[a]; }
+    }
+  }
+};
+
+// The lane's column of ZPL voxels of an interior tile, fp32 coordinates.  `before(k)` runs ahead
+// of voxel k while o[k] still holds the previous item's value.
+template <typename T, int ORDER, int ZPL, typename Hook>
+__device__ __forceinline__ void interior_column(const T *__restrict__ tile, float (&o)[ZPL], float b0, float b1,
+                                                float b2, float s0, float s1, float s2, const i32x4 g, Hook before) {
+  const float pitch_f = static_cast<float>(g.x), slice_f = static_cast<float>(g.y);
+  Taps<T> cur, nxt;
+  ColumnCoord r;
+  r.start(b0, b1, b2);
+  interior_issue<T, ORDER>(cur, tile, b0, b1, b2, g, pitch_f, slice_f);
+  column_steps<0, ZPL>([&](auto kc) {
+    constexpr int k = decltype(kc)::value;
+    before(k);
+    if constexpr (k + 1 < ZPL) {
+      r.template step<k + 1>(s0, s1, s2);
+      interior_issue<T, ORDER>(nxt, tile, r.last[0], r.last[1], r.last[2], g, pitch_f, slice_f);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    o[k] = interior_finish<T, ORDER, false>(cur);
+    cur = nxt;
+    __builtin_amdgcn_sched_barrier(0);
+  });
+}
+
+// The same for a CLIPPED box (some side of it is the volume's border), fp32 coordinates: the
+// coordinate is clamped to [0, cmax]; a sample the clamp moves by more than 1 lies outside [-1, size]
+// of the volume and is void (the differences are exact: one operand is 0 or within a factor of
+// 2); the low tap index is at most `top`, so that the high tap stays inside the box (a
+// coordinate on the last voxel gets weight 1 on the high tap).
+template <typename T, int ORDER>
+__device__ __forceinline__ bool clipped_issue(Taps<T> &q, const T *__restrict__ tile, float rx, float ry,
+                                              float rz, const i32x4 g, const float (&cmax)[3], const float (&top)[3],
+                                              float pitch_f, float slice_f) {
+#pragma clang fp contract(off)
+  const float cx = clamp_ct(rx, 0.f, cmax[0]), cy = clamp_ct(ry, 0.f, cmax[1]), cz = clamp_ct(rz, 0.f, cmax[2]);
+  const bool ok = fmaxf(fmaxf(fabsf(rx - cx), fabsf(ry - cy)), fabsf(rz - cz)) <= 1.f;
+  const float lx = fminf(floorf(cx), top[0]), ly = fminf(floorf(cy), top[1]), lz = fminf(floorf(cz), top[2]);
+  q.wx = cx - lx; q.wy = cy - ly; q.wz = cz - lz;
+  constexpr unsigned E = sizeof(T);
+  // byte offset of the low corner, exact in fp32 (far below 2^24)
+  const float row = ly * pitch_f, sl = lz * slice_f, xb = E == 2 ? lx + lx : lx * static_cast<float>(E);
+  const unsigned at = static_cast<unsigned>((xb + row) + sl);
+  const char *t = reinterpret_cast<const char *>(tile) + at;
+  const unsigned dy = g.z, dz = g.w;
+  if (ORDER == 0) {
+    const unsigned off = (q.wz <= 0.5f ? 0u : dz) + (q.wy <= 0.5f ? 0u : dy) + (q.wx <= 0.5f ? 0u : E);
+    q.v[0] = *reinterpret_cast<const T *>(t + off);
+  } else {
+    q.v[0] = *reinterpret_cast<const T *>(t);
+    q.v[1] = *reinterpret_cast<const T *>(t + E);
+    q.v[2] = *reinterpret_cast<const T *>(t + dy);
+    q.v[3] = *reinterpret_cast<const T *>(t + dy + E);
+    q.v[4] = *reinterpret_cast<const T *>(t + dz);
+    q.v[5] = *reinterpret_cast<const T *>(t + dz + E);
+    q.v[6] = *reinterpret_cast<const T *>(t + dz + dy);
+    q.v[7] = *reinterpret_cast<const T *>(t + dz + dy + E);
+  }
+  return ok;
+}
+template <typename T, int ORDER, int ZPL, typename Hook>
+__device__ __forceinline__ void clipped_column(const T *__restrict__ tile, float (&o)[ZPL], float b0, float b1,
+                                               float b2, float s0, float s1, float s2, const i32x4 g,
+                                               const float (&cmax)[3], const float (&top)[3], Hook before) {
+  const float pitch_f = static_cast<float>(g.x), slice_f = static_cast<float>(g.y);
+  Taps<T> cur, nxt;
+  ColumnCoord r;
+  r.start(b0, b1, b2);
+  bool ok = clipped_issue<T, ORDER>(cur, tile, b0, b1, b2, g, cmax, top, pitch_f, slice_f), ok_next = false;
+  column_steps<0, ZPL>([&](auto kc) {
+    constexpr int k = decltype(kc)::value;
+    before(k);
+    if constexpr (k + 1 < ZPL) {
+      r.template step<k + 1>(s0, s1, s2);
+      ok_next = clipped_issue<T, ORDER>(nxt, tile, r.last[0], r.last[1], r.last[2], g, cmax, top, pitch_f, slice_f);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    const float v = interior_finish<T, ORDER, true>(cur);
+    o[k] = ok ? v : 0.f;
+    cur = nxt;
+    ok = ok_next;
+    __builtin_amdgcn_sched_barrier(0);
+  });
+}
 
 // Persistent workgroups: each takes every `slots`-th item (tile, channel) of its XCD's contiguous
 // range.  Per item:   write the box (loaded into registers during the previous item) to LDS |
@@ -425,20 +659,23 @@ constexpr unsigned kOutOfRange = 0x80000000u;  // beyond every buffer: the load 
 // the interpolation of the previous item, and stores by that of the next.
 // Box rows are copied as 16-byte groups with range-checked buffer loads: lane = (slice, row,
 // group) within a pass of `span` z-slices, one register quad per pass, passes `span` slices apart.
-template <typename T, int TX, int TY, int TZ, int THREADS, int LDS_BYTES, int KMAX>
+// Everything that is the same for all lanes of an item (addresses, extents, LDS geometry) is in
+// the item's record, so a wavefront spends a handful of v_readlane and broadcast reads per item;
+// conditions that hold for a whole wavefront (a pass that exists, an output slice that exists)
+// select between the real buffer extent and an empty one on the scalar unit.
+template <typename T, int TX, int TY, int TZ, int THREADS, int LDS_BYTES, int KMAX, int ORDER>
 __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
     const T *__restrict__ feat, const float *__restrict__ rois, T *__restrict__ out, const RoiProblem p, const PlanShape ps, const unsigned total, const unsigned work) {
   using CT = typename std::conditional<(sizeof(T) == 2), float, double>::type;
   constexpr int kCap = LDS_BYTES / sizeof(T);
   constexpr int RZ = THREADS / (TX * TY);  // lane layers along z
   static_assert(RZ >= 1 && RZ * TX * TY == THREADS && TZ % RZ == 0, "tile shape");
+  static_assert((TX * TY) % kWave == 0, "a wavefront's lanes share their z layer");
   constexpr int ZPL = TZ / RZ;             // consecutive output slices per lane
-  constexpr int V = 16 / sizeof(T);        // elements per 16-byte group
   constexpr int ES = sizeof(T);
   __shared__ __attribute__((aligned(16))) T tile[kCap];
-  __shared__ TilePlan lplans[kPlanSlots];
-  const int C = p.C, D = p.D, H = p.H, W = p.W, od = p.od, oh = p.oh, ow = p.ow;
-  const int vec = ps.vec, order = p.order;
+  __shared__ __attribute__((aligned(16))) TilePlan lplans[kPlanSlots];
+  const int H = p.H, W = p.W, oh = p.oh, ow = p.ow;
 
   // Work distribution: items (channel * tiles + tile) are dealt to the XCDs in chunks of kChunk
   // consecutive items (workgroup ids go round-robin over the XCDs, each with an L2 of its own, so
@@ -446,126 +683,152 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
   // XCD take the next `slots` positions of its queue, each workgroup a different one; the
   // assignment is rotated from round to round so that a workgroup does not get the same tile
   // position (border: cheap, centre: expensive) in every roi.
-  const unsigned parts = gridDim.x >= kXcds ? kXcds : 1;
-  const unsigned xcd = blockIdx.x % parts, slot = blockIdx.x / parts, slots = gridDim.x / parts;
-  auto item_of = [&](unsigned round) -> unsigned {
-    const unsigned k = round * slots + (slot + round * 27u) % slots;
-    const unsigned item = ((k / kChunk) * parts + xcd) * kChunk + k % kChunk;
-    return item < work ? item : kDone;   // only the last round of a queue is incomplete
-  };
   const int tid = threadIdx.x;
-  if (item_of(0) == kDone) return;
-
-  // ---- plans of this workgroup's items (at most kPlanSlots): four lanes per item, into LDS -----
   const unsigned per_roi = static_cast<unsigned>(ps.tiles_x) * ps.tiles_y * ps.tiles_z;
-  if (tid < kWave) {
-    static_assert(kPlanSlots * 4 == kWave, "four lanes per plan slot");
-    const unsigned r = tid >> 2;
-    plan_item_lanes(rois, p, ps, item_of(r), total, per_roi, &lplans[r]);
-  }
-  __syncthreads();
   auto fetch_plan = [&](unsigned r) -> PlanLanes {
-    const unsigned lane = tid & (kWave - 1);
     PlanLanes pl;
-    pl.v = reinterpret_cast<const unsigned *>(&lplans[r])[lane < sizeof(TilePlan) / 4 ? lane : 0];
+    pl.v = reinterpret_cast<const unsigned *>(&lplans[r])[tid & (kWave - 1)];
     return pl;
   };
   unsigned round = 0;
-  unsigned w = item_of(0), wn = item_of(1);
-  unsigned c = C > 1 ? w / total : 0;
+  int mode = 4;
 
+  // what a lane keeps for the whole kernel: its place in the tile and in the copy passes
   const int lx = tid % TX, ly = (tid / TX) % TY, lz = tid / (TX * TY);
-  const long zstride = static_cast<long>(oh) * ow;
-  const long plane = static_cast<long>(D) * H * W;
+  const CT fx = static_cast<CT>(lx), fy = static_cast<CT>(ly), fz = static_cast<CT>(lz * ZPL);
+  const float tid_h = static_cast<float>(tid) + 0.5f;
+  const int zbytes = oh * ow * ES;
+  const int out_bytes = p.od * zbytes;   // bytes of one output volume (< 2^31, checked by the host)
+  const unsigned lane_out = static_cast<unsigned>(((lz * ZPL * oh + ly) * ow + lx) * ES);
+  const int w_bytes = W * ES;
+  const unsigned hw_bytes = static_cast<unsigned>(H) * W * ES;   // < 2^31, checked by the host
+  char *const tile_lane = reinterpret_cast<char *>(tile) + tid * 16;   // lane `tid` holds group `tid` of every pass
 
   u32x4 val[KMAX];   // the next item's box: 16-byte group (zz0 + u * span, yy, gi) in val[u]
   int st_zz = 0;     // zz0 of this lane (beyond every box for idle lanes)
-  int st_dst = 0;    // LDS element offset of the lane's first group
   float o[ZPL];      // the previous item's outputs
-  // outputs waiting to be stored: descriptor of the (roi, channel) volume, the lane's byte offset
-  // in it, the number of voxels of the lane's column that exist
-  __amdgpu_buffer_rsrc_t pend_rsrc = __builtin_amdgcn_make_buffer_rsrc(out, 0, 0, 0x00020000);
+  // outputs waiting to be stored: the (roi, channel) volume, the lane's byte offset in it (out of
+  // range for lanes beyond the output's rows / columns)
+  const char *pend_base = reinterpret_cast<const char *>(out);
   unsigned pend_voff = kOutOfRange;
-  int pend_count = 0;
-  const int zbytes = static_cast<int>(zstride) * ES;
-  const int out_bytes = od * zbytes;   // bytes of one output volume (< 2^31, checked by the host)
+  int pend_bytes = 0;   // 0 until there is something to store
 
-  // The loads of one item's box into val[]: the buffer ends with the box's last row, so passes
-  // that run beyond the last z-slice read zeros without a test.  `prepare` sets the addresses up,
-  // `load_pass(u)` issues pass u (u < ld_passes, wave-uniform).
-  __amdgpu_buffer_rsrc_t ld_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(feat), 0, 0, 0x00020000);
+  // The loads of one item's box into val[]: the buffer ends with the box's last row.  `prepare`
+  // sets the addresses up and returns the item's mode (4: there is no such item).
+  const char *ld_base = reinterpret_cast<const char *>(feat);
+  int ld_extent = 0;
   unsigned ld_voff = kOutOfRange;
   int ld_stride = 0, ld_passes = 0;
-  auto prepare = [&](const PlanLanes &pl, unsigned ch) -> BoxShape {
-    BoxShape sh;
-    sh.mode = pl.mode(); sh.bx = pl.n(0); sh.by = pl.n(1); sh.bz = pl.n(2);
-    sh.rp = pl.rp(); sh.span = pl.span(); sh.passes = pl.passes();
-    const int passes = sh.passes;
+  // `pl`: the record's scalar part, `sp` = (1 / groups, 1 / rows as float bits, groups, rows), `rp`:
+  // read by the caller well ahead (one batch of LDS reads per item).
+  auto prepare = [&](bool exists, const PlanLanes &pl, const i32x4 sp, int rp) -> int {
     ld_passes = 0;
-    if (vec == 0 || passes == 0 || (sh.mode != 1 && sh.mode != 3)) return sh;
-    const int bx = sh.bx, by = sh.by, bz = sh.bz;
-    const int groups = bx / V;
-    const int lr = div_small(tid, 1.0f / static_cast<float>(groups)), gi = tid - lr * groups;
-    const int zz = div_small(lr, 1.0f / static_cast<float>(by)), yy = lr - zz * by;
-    const long first = (static_cast<long>(pl.lo(2)) * H + pl.lo(1)) * W + pl.lo(0);
-    const T *corner = feat + (static_cast<long>(pl.batch()) * C + ch) * plane + first;
-    const int extent = (((bz - 1) * H + by - 1) * W + bx) * ES;
-    ld_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(corner), 0, extent, 0x00020000);
-    const bool on = lr < sh.rp;
-    ld_voff = on ? static_cast<unsigned>(((zz * H + yy) * W + gi * V) * ES) : kOutOfRange;
-    ld_stride = sh.span * H * W * ES;
+    ld_extent = 0;    // an empty buffer: every load returns zeros
+    if (!exists) return 4;
+    const int m = pl.i32(MV_PLAN_DW(mode));
+    const int passes = pl.i32(MV_PLAN_DW(passes));
+    if (m == 4 || (m & 1) == 0 || passes == 0) return m;   // staged modes are 1 and 3
+    const float inv_groups = __int_as_float(sp.x), inv_rows = __int_as_float(sp.y);
+    const int groups = sp.z, by = sp.w;
+    const int lr = static_cast<int>(tid_h * inv_groups), gi = tid - __mul24(lr, groups);
+    const int zz = static_cast<int>((static_cast<float>(lr) + 0.5f) * inv_rows), yy = lr - __mul24(zz, by);
+    ld_base = reinterpret_cast<const char *>(feat) + pl.u64(MV_PLAN_DW(src_lo));
+    ld_extent = pl.i32(MV_PLAN_DW(extent));
+    ld_stride = pl.i32(MV_PLAN_DW(stride));
     ld_passes = passes;
+    const bool on = lr < rp;
+    ld_voff = on ? static_cast<unsigned>(zz) * hw_bytes + static_cast<unsigned>(__mul24(yy, w_bytes) + gi * 16) : kOutOfRange;
     st_zz = on ? zz : (1 << 28);
-    st_dst = lr * bx + gi * V;
-    return sh;
+    return m;
   };
+  // Pass u.  The scalar offset takes part in the range check, so a pass beyond the box's last
+  // slice (u >= ld_passes) reads zeros without touching memory.
   auto load_pass = [&](int u) {
-    if (u < ld_passes) val[u] = __builtin_amdgcn_raw_buffer_load_b128(ld_rsrc, ld_voff, u * ld_stride, 0);
+    const __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(ld_base), 0, ld_extent, 0x00020000);
+    val[u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ld_voff, u * ld_stride, 0);
   };
-  BoxShape cur = prepare(fetch_plan(0), c);
+  // The first wavefront plans this workgroup's items (at most kPlanSlots), four lanes per item.
+  if (tid < kWave) {
+    static_assert(kPlanSlots * 4 == kWave, "four lanes per plan slot");
+    const unsigned parts = gridDim.x >= kXcds ? kXcds : 1;
+    const unsigned xcd = parts > 1 ? blockIdx.x % kXcds : 0, slot = parts > 1 ? blockIdx.x / kXcds : blockIdx.x;
+    const unsigned slots = gridDim.x / parts;
+    const unsigned r = tid >> 2;
+    const unsigned sr = slot + r * 27u;
+    const unsigned k = r * slots + (sr - ps.by_slots.div(sr) * slots);
+    const unsigned item = ((k / kChunk) * parts + xcd) * kChunk + k % kChunk;
+    plan_item_lanes(rois, p, ps, item < work ? item : kDone, total, per_roi, &lplans[r]);
+  }
+  __syncthreads();
+  mode = prepare(true, fetch_plan(0), *reinterpret_cast<const i32x4 *>(&lplans[0].inv_groups), lplans[0].rp);
+  if (mode == 4) return;
 #pragma unroll
-  for (int u = 0; u < KMAX; u++) load_pass(u);
+  for (int u = 0; u < KMAX; u++)
+    if (u < ld_passes) load_pass(u);
   while (true) {
+    // everything this item needs from its record and the next one's, requested in one batch ahead
+    // of the wait for the box (the records are read-only from here on)
+    const TilePlan *rec = &lplans[round];
+    const bool has_next = round + 1 < kPlanSlots;
+    const TilePlan *nrec = &lplans[has_next ? round + 1 : round];
     const PlanLanes plan = fetch_plan(round);
-    const int mode = cur.mode;
-    const bool staged = mode == 1 || mode == 3;
-    const int bx = cur.bx, by = cur.by, bz = cur.bz;
-    const int pitch = vec > 0 ? bx : bx + 1;  // unaligned rows end with a finite pad
-    const int slice = by * pitch;
-    const T *src = feat + (static_cast<long>(plan.batch()) * C + c) * plane;
+    PlanLanes nplan;
+    nplan.v = reinterpret_cast<const unsigned *>(nrec)[tid & (kWave - 1)];
+    const i32x4 nsp = *reinterpret_cast<const i32x4 *>(&nrec->inv_groups);
+    const int nrp = nrec->rp;
+    const i32x4 cpy = *reinterpret_cast<const i32x4 *>(&rec->rp);          // rp, -, bz, span
+    const i32x4 g = *reinterpret_cast<const i32x4 *>(&rec->pitch_b);       // pitch, slice, dy, dz in bytes
+    const i32x4 t = *reinterpret_cast<const i32x4 *>(&rec->tile_off);      // tile_off, xlim, ylim, hop_b
+    CT m[12];
+#pragma unroll
+    for (int i = 0; i < 12; i++) m[i] = plan_map<CT>(rec)[i];
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    const f32x4 lim4 = *reinterpret_cast<const f32x4 *>(rec->cmaxf), top4 = *reinterpret_cast<const f32x4 *>(rec->topf);
+    const bool staged = (mode & 1) != 0;
 
     // ---- A: the box into LDS ---------------------------------------------------------------
     // All loads issued for this item have to be back; waiting here on every path (vmcnt(0), other
     // counters untouched) keeps the compiler from waiting again after the stores of phase B.
     __builtin_amdgcn_s_waitcnt(0x0F70);
     if (staged) {
-      const int rows = by * bz;
-      const T *corner = src + (static_cast<long>(plan.lo(2)) * H + plan.lo(1)) * W + plan.lo(0);
-      const float inv_by = 1.0f / static_cast<float>(by);
-      if (vec > 0) {
-        const int passes = cur.passes, groups = bx / V;
-        if (passes > 0) {
-          const int hop = cur.rp * pitch, span = cur.span;
+      if (ld_passes > 0) {   // still this item's: the next `prepare` comes after the barrier
+        const int bz = cpy.z, span = cpy.w, hop_b = t.w;
+        int zc = st_zz;
+        char *dst = tile_lane;
 #pragma unroll
-          for (int u = 0; u < KMAX; u++)
-            if (u < passes && st_zz < bz - u * span) *reinterpret_cast<u32x4 *>(tile + st_dst + u * hop) = val[u];
-        } else {  // boxes with very long rows or very many slices: straight from global memory
-          const float inv_groups = 1.0f / static_cast<float>(groups);
-          for (int i = tid; i < rows * groups; i += THREADS) {
-            const int r = div_small(i, inv_groups), gi = i - r * groups;
-            const int zz = div_small(r, inv_by), yy = r - zz * by;
-            *reinterpret_cast<u32x4 *>(tile + r * pitch + gi * V) =
-                *reinterpret_cast<const u32x4 *>(corner + (static_cast<long>(zz) * H + yy) * W + gi * V);
+        for (int u = 0; u < KMAX; u++) {
+          if (u < ld_passes) {   // a scalar branch
+            if (zc < bz) *reinterpret_cast<u32x4 *>(dst) = val[u];
+            zc += span;
+            dst += hop_b;
           }
         }
       } else {
-        int lpr = 1;
-        while (lpr < pitch && lpr < kWave) lpr *= 2;
-        const int lane_e = tid & (lpr - 1), lane_r = tid / lpr;
-        for (int r = lane_r; r < rows; r += THREADS / lpr) {
-          const int zz = div_small(r, inv_by), yy = r - zz * by;
-          const T *row = corner + (static_cast<long>(zz) * H + yy) * W;
-          for (int e = lane_e; e < pitch; e += lpr) tile[r * pitch + e] = e < bx ? row[e] : store_cast<T>(0.f);
+        // boxes with very long rows, very many slices or unaligned rows: straight from global memory
+        const int bx = plan_scalar(&rec->n[0]), by = plan_scalar(&rec->n[1]), bz = plan_scalar(&rec->n[2]);
+        const int vec = ps.vec, pitch = vec > 0 ? bx : bx + 1, rows = by * bz;
+        const T *corner = reinterpret_cast<const T *>(
+            reinterpret_cast<const char *>(feat) + plan.u64(MV_PLAN_DW(src_lo)));
+        const float inv_by = rec->inv_rows;
+        if (vec > 0) {
+          const int groups = bx / vec;
+          const float inv_groups = rec->inv_groups;
+          for (int i = tid; i < rows * groups; i += THREADS) {
+            const int r = div_small(i, inv_groups), gi = i - r * groups;
+            const int zz = div_small(r, inv_by), yy = r - zz * by;
+            *reinterpret_cast<u32x4 *>(tile + r * pitch + gi * vec) =
+                *reinterpret_cast<const u32x4 *>(corner + (static_cast<long>(zz) * H + yy) * W + gi * vec);
+          }
+        } else {
+          int lpr = 1;
+          while (lpr < pitch && lpr < kWave) lpr *= 2;
+          const int lane_e = tid & (lpr - 1), lane_r = tid / lpr;
+          for (int r = lane_r; r < rows; r += THREADS / lpr) {
+            const int zz = div_small(r, inv_by), yy = r - zz * by;
+            const T *row = corner + (static_cast<long>(zz) * H + yy) * W;
+            for (int e = lane_e; e < pitch; e += lpr) tile[r * pitch + e] = e < bx ? row[e] : store_cast<T>(0.f);
+          }
         }
       }
     }
@@ -573,24 +836,16 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
 
     // ---- B + C: this item; ahead of voxel k the previous item's voxel k is stored and a share of
     // the next box's loads is issued, so that neither piles up in the memory pipeline -------------
-    const bool more = wn != kDone;
-    unsigned cn = 0;
-    BoxShape nxt = cur;
-    ld_passes = 0;
-    if (more) {
-      if (C > 1) cn = wn / total;
-      nxt = prepare(fetch_plan(round + 1), cn);
-    }
+    const int next_mode = prepare(has_next, nplan, nsp, nrp);
     auto before = [&](int k) {
-      store_element<T>(pend_rsrc, k < pend_count ? pend_voff : kOutOfRange, k * zbytes, o[k]);
+      // (slices beyond the volume's last one are beyond the buffer: scalar offsets are range-checked)
+      const __amdgpu_buffer_rsrc_t rsrc =
+          __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(pend_base), 0, pend_bytes, 0x00020000);
+      store_element<T>(rsrc, pend_voff, k * zbytes, o[k]);
 #pragma unroll
       for (int u = 0; u < KMAX; u++)
-        if (u >= k * KMAX / ZPL && u < (k + 1) * KMAX / ZPL)   // compile-time share of the loads
-          val[u] = __builtin_amdgcn_raw_buffer_load_b128(ld_rsrc, u < ld_passes ? ld_voff : kOutOfRange,
-                                                         u * ld_stride, 0);
+        if (u >= k * KMAX / ZPL && u < (k + 1) * KMAX / ZPL) load_pass(u);   // compile-time share of the loads
     };
-    const int ox = plan.t0(0) + lx, oy = plan.t0(1) + ly, zb = plan.t0(2) + lz * ZPL;
-    const int count = (ox < ow && oy < oh) ? min(ZPL, od - zb) : 0;  // may be <= 0
     if (mode == 0) {
 #pragma unroll
       for (int k = 0; k < ZPL; k++) {
@@ -600,59 +855,69 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
     } else {
       // position of this lane's first voxel and the per-slice increment, relative to the box (to
       // the feature map for mode 2), in the coordinate type (the box margin covers the rounding
-      // of fp32 arithmetic)
-      const CT fx = static_cast<CT>(lx), fy = static_cast<CT>(ly), fz = static_cast<CT>(lz * ZPL);
+      // of fp32 arithmetic); the record's values come as broadcast reads.  Lanes beyond the
+      // output run the same code: their reads stay inside the box or miss the LDS (zeros), and
+      // their stores are dropped.
       CT b[3], st[3];
 #pragma unroll
       for (int a = 0; a < 3; a++) {
-        b[a] = plan_org<CT>(plan, a) + fx * plan_inc<CT>(plan, a * 3) + fy * plan_inc<CT>(plan, a * 3 + 1) +
-               fz * plan_inc<CT>(plan, a * 3 + 2);
-        st[a] = plan_inc<CT>(plan, a * 3 + 2);
-        // lanes beyond the output keep step with the others (their part of the stores and loads
-        // is issued from the same code) and sample along the ray from the box origin (reads that
-        // leave the box return garbage or zero and are never stored)
-        if (count <= 0) b[a] = CT(0);
+        b[a] = m[4 * a] + fx * m[4 * a + 1] + fy * m[4 * a + 2] + fz * m[4 * a + 3];
+        st[a] = m[4 * a + 3];
       }
-      BoxLimits<CT> lim;
-      if (mode == 3) {
-        const int dy = by > 1 ? pitch : 0, dz = bz > 1 ? slice : 0;
-        if (order == 0) staged_column<T, CT, true, 0, ZPL>(tile, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, pitch, slice, dy, dz, before);
-        else staged_column<T, CT, true, 1, ZPL>(tile, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, pitch, slice, dy, dz, before);
-      } else {
-        const int size[3] = {W, H, D};
-        const int lo[3] = {mode == 2 ? 0 : plan.lo(0), mode == 2 ? 0 : plan.lo(1), mode == 2 ? 0 : plan.lo(2)};
-        const int n[3] = {mode == 2 ? W : bx, mode == 2 ? H : by, mode == 2 ? D : bz};
-        for (int a = 0; a < 3; a++) {
-          lim.cmax[a] = uniform(static_cast<CT>(size[a] - 1 - lo[a]));
-          lim.top[a] = uniform(static_cast<CT>(max(n[a] - 2, 0)));
+      if (mode == 3 && sizeof(CT) == 4) {
+        if constexpr (sizeof(CT) == 4)
+          interior_column<T, ORDER, ZPL>(tile, o, b[0], b[1], b[2], st[0], st[1], st[2], g, before);
+      } else if (mode == 1 && sizeof(CT) == 4) {
+        if constexpr (sizeof(CT) == 4) {
+          const float cmax[3] = {lim4.x, lim4.y, lim4.z}, top[3] = {top4.x, top4.y, top4.z};
+          clipped_column<T, ORDER, ZPL>(tile, o, b[0], b[1], b[2], st[0], st[1], st[2], g, cmax, top, before);
         }
-        if (mode == 2) {  // the box does not fit in LDS: taps straight from the feature map
-          for (int a = 0; a < 3; a++) b[a] += count > 0 ? static_cast<CT>(plan.lo(a)) : CT(0);
-          const long hw = static_cast<long>(H) * W;
-          const int dy = H > 1 ? W : 0;
-          const long dz = D > 1 ? hw : 0;
-          if (order == 0) staged_column<T, CT, false, 0, ZPL, true>(src, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, W, hw, dy, dz, before);
-          else staged_column<T, CT, false, 1, ZPL, true>(src, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, W, hw, dy, dz, before);
+      } else {
+        const int pitch = g.x / ES, slice = g.y / ES, dy = g.z / ES, dz = g.w / ES;
+        BoxLimits<CT> lim;
+        if (mode == 3) {
+          staged_column<T, CT, true, ORDER, ZPL>(tile, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, pitch, slice, dy, dz, before);
         } else {
-          const int dy = by > 1 ? pitch : 0, dz = bz > 1 ? slice : 0;
-          if (order == 0) staged_column<T, CT, false, 0, ZPL>(tile, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, pitch, slice, dy, dz, before);
-          else staged_column<T, CT, false, 1, ZPL>(tile, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, pitch, slice, dy, dz, before);
+          const int size[3] = {W, H, p.D};
+#pragma unroll
+          for (int a = 0; a < 3; a++) {
+            const int lo = mode == 2 ? 0 : plan_scalar(&rec->lo[a]);
+            const int n = mode == 2 ? size[a] : plan_scalar(&rec->n[a]);
+            lim.cmax[a] = uniform(static_cast<CT>(size[a] - 1 - lo));
+            lim.top[a] = uniform(static_cast<CT>(max(n - 2, 0)));
+          }
+          if (mode == 2) {  // the box does not fit in LDS: taps straight from the feature map
+            for (int a = 0; a < 3; a++) b[a] += static_cast<CT>(plan_scalar(&rec->lo[a]));
+            const T *src = reinterpret_cast<const T *>(
+                reinterpret_cast<const char *>(feat) +
+                ((static_cast<unsigned long>(static_cast<unsigned>(plan_scalar(reinterpret_cast<const int *>(&rec->vol_hi)))) << 32) |
+                 static_cast<unsigned>(plan_scalar(reinterpret_cast<const int *>(&rec->vol_lo)))));
+            const long hw = static_cast<long>(H) * W;
+            const int dyw = H > 1 ? W : 0;
+            const long dzw = p.D > 1 ? hw : 0;
+            staged_column<T, CT, false, ORDER, ZPL, true>(src, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, W, hw, dyw, dzw, before);
+          } else {
+            staged_column<T, CT, false, ORDER, ZPL>(tile, o, b[0], b[1], b[2], st[0], st[1], st[2], lim, pitch, slice, dy, dz, before);
+          }
         }
       }
     }
-    pend_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        out + (static_cast<long>(plan.roi()) * C + c) * od * zstride, 0, out_bytes, 0x00020000);
-    pend_voff = static_cast<unsigned>(((zb * oh + oy) * ow + ox) * ES);
-    pend_count = count;
-    if (!more) break;
+    {
+      pend_base = reinterpret_cast<const char *>(out) + plan.u64(MV_PLAN_DW(out_lo));
+      pend_voff = (lx < t.y && ly < t.z) ? lane_out + static_cast<unsigned>(t.x) : kOutOfRange;
+      pend_bytes = out_bytes;
+    }
+    if (next_mode == 4) break;
     __syncthreads();  // every lane is done with the box
-    w = wn; c = cn; cur = nxt;
+    mode = next_mode;
     round++;
-    wn = item_of(round + 1);
   }
 #pragma unroll
-  for (int k = 0; k < ZPL; k++)
-    store_element<T>(pend_rsrc, k < pend_count ? pend_voff : kOutOfRange, k * zbytes, o[k]);
+  for (int k = 0; k < ZPL; k++) {
+    const __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(pend_base), 0, pend_bytes, 0x00020000);
+    store_element<T>(rsrc, pend_voff, k * zbytes, o[k]);
+  }
 }
 
 // Compute units of the current device (workgroups resident at once = units * LDS share).
@@ -690,18 +955,15 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_cubic_kernel(
     const unsigned w = item_of(round);
     if (w == kDone) break;
     const unsigned c = C > 1 ? w / total : 0;
-    PlanLanes plan;
-    {
-      const unsigned lane = tid & (kWave - 1);
-      plan.v = reinterpret_cast<const unsigned *>(&lplans[round])[lane < sizeof(TilePlan) / 4 ? lane : 0];
-    }
-    const int mode = plan.mode();
-    const int bx = plan.n(0), by = plan.n(1), bz = plan.n(2);
+    const TilePlan *rec = &lplans[round];
+    const int mode = plan_scalar(&rec->mode);
+    const int bx = plan_scalar(&rec->n[0]), by = plan_scalar(&rec->n[1]), bz = plan_scalar(&rec->n[2]);
+    const int lo[3] = {plan_scalar(&rec->lo[0]), plan_scalar(&rec->lo[1]), plan_scalar(&rec->lo[2])};
     const int pitch = vec > 0 ? bx : bx + 1, slice = by * pitch;
-    const T *src = feat + (static_cast<long>(plan.batch()) * C + c) * plane;
+    const T *src = feat + (static_cast<long>(plan_scalar(&rec->batch)) * C + c) * plane;
     if (mode == 1 || mode == 3) {   // the box into LDS
       const int rows = by * bz;
-      const T *corner = src + (static_cast<long>(plan.lo(2)) * H + plan.lo(1)) * W + plan.lo(0);
+      const T *corner = src + (static_cast<long>(lo[2]) * H + lo[1]) * W + lo[0];
       const float inv_by = 1.0f / static_cast<float>(by);
       if (vec > 0) {
         const int groups = bx / V;
@@ -736,24 +998,24 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_cubic_kernel(
       }
     }
     __syncthreads();
-    const int ox = plan.t0(0) + lx, oy = plan.t0(1) + ly, zb = plan.t0(2) + lz * ZPL;
+    const int ox = plan_scalar(&rec->t0[0]) + lx, oy = plan_scalar(&rec->t0[1]) + ly, zb = plan_scalar(&rec->t0[2]) + lz * ZPL;
     const int count = (ox < ow && oy < oh) ? min(ZPL, od - zb) : 0;
-    T *drow = out + (static_cast<long>(plan.roi()) * C + c) * od * zstride + (static_cast<long>(zb) * oh + oy) * ow + ox;
+    T *drow = out + (static_cast<long>(plan_scalar(&rec->roi)) * C + c) * od * zstride + (static_cast<long>(zb) * oh + oy) * ow + ox;
     if (count > 0) {
       const CT fx = static_cast<CT>(lx), fy = static_cast<CT>(ly), fz = static_cast<CT>(lz * ZPL);
       CT b[3], st[3];
 #pragma unroll
       for (int a = 0; a < 3; a++) {
-        b[a] = plan_org<CT>(plan, a) + fx * plan_inc<CT>(plan, a * 3) + fy * plan_inc<CT>(plan, a * 3 + 1) +
-               fz * plan_inc<CT>(plan, a * 3 + 2);
-        st[a] = plan_inc<CT>(plan, a * 3 + 2);
+        const CT *m = plan_map<CT>(rec) + 4 * a;
+        b[a] = m[0] + fx * m[1] + fy * m[2] + fz * m[3];
+        st[a] = m[3];
       }
       BoxLimits<CT> lim;
       lim.one = ps.halo_lo;
       const int size[3] = {W, H, D};
       const int n[3] = {mode == 2 ? W : bx, mode == 2 ? H : by, mode == 2 ? D : bz};
       for (int a = 0; a < 3; a++) {  // the volume's far end (inclusive) and the last index of the box
-        lim.cmax[a] = static_cast<CT>(size[a] - (mode == 2 ? 0 : plan.lo(a)));
+        lim.cmax[a] = static_cast<CT>(size[a] - (mode == 2 ? 0 : lo[a]));
         lim.top[a] = static_cast<CT>(max(n[a] - 1, 0));
       }
       if (mode == 0) {
@@ -767,7 +1029,7 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_cubic_kernel(
               tile, b[0] + kk * st[0], b[1] + kk * st[1], b[2] + kk * st[2], lim, pitch, slice, dy, dz));
         }
       } else if (mode == 2) {  // the box does not fit in LDS: taps straight from the feature map
-        for (int a = 0; a < 3; a++) b[a] += static_cast<CT>(plan.lo(a));
+        for (int a = 0; a < 3; a++) b[a] += static_cast<CT>(lo[a]);
         const long hw = static_cast<long>(H) * W;
 #pragma unroll 1
         for (int k = 0; k < count; k++) {
@@ -817,6 +1079,11 @@ static int launch_resample(const T *feat, const float *rois, T *out, const RoiPr
   ps.cap = LDS_BYTES / sizeof(T);
   ps.threads = THREADS; ps.max_items = KMAX;
   ps.halo_lo = CUBIC ? 1 : 0; ps.halo_hi = CUBIC ? 2 : 1;
+  ps.es = static_cast<int>(sizeof(T));
+  ps.by_per_roi.set(static_cast<unsigned>(per_roi));
+  ps.by_tiles_x.set(static_cast<unsigned>(tx));
+  ps.by_tiles_y.set(static_cast<unsigned>(ty));
+  ps.by_total.set(static_cast<unsigned>(total));
   unsigned blocks = compute_units() * (160u * 1024u / (LDS_BYTES + sizeof(TilePlan) * kPlanSlots + 64u));
   // As many workgroups as are resident at once, more when that would give one more than
   // kPlanSlots items (the later ones start as the first finish).
@@ -825,12 +1092,17 @@ static int launch_resample(const T *feat, const float *rois, T *out, const RoiPr
   const long by_slots = ((work + kPlanSlots - 1) / kPlanSlots + 2 * kXcds + kXcds - 1) / kXcds * kXcds;
   if (blocks >= kXcds) blocks = blocks / kXcds * kXcds;  // the same number of workgroups on every XCD
   if (by_slots > blocks && work > kPlanSlots) blocks = static_cast<unsigned>(by_slots);
-  if (CUBIC)
+  ps.by_slots.set(blocks >= kXcds ? blocks / kXcds : blocks);
+  if constexpr (CUBIC)
     hipLaunchKernelGGL((roi_resample_cubic_kernel<T, TX, TY, TZ, THREADS, LDS_BYTES>), dim3(blocks),
                        dim3(THREADS), 0, s, feat, rois, out, p, ps, static_cast<unsigned>(total),
                        static_cast<unsigned>(work));
+  else if (p.order == 0)
+    hipLaunchKernelGGL((roi_resample_kernel<T, TX, TY, TZ, THREADS, LDS_BYTES, KMAX, 0>), dim3(blocks),
+                       dim3(THREADS), 0, s, feat, rois, out, p, ps, static_cast<unsigned>(total),
+                       static_cast<unsigned>(work));
   else
-    hipLaunchKernelGGL((roi_resample_kernel<T, TX, TY, TZ, THREADS, LDS_BYTES, KMAX>), dim3(blocks),
+    hipLaunchKernelGGL((roi_resample_kernel<T, TX, TY, TZ, THREADS, LDS_BYTES, KMAX, 1>), dim3(blocks),
                        dim3(THREADS), 0, s, feat, rois, out, p, ps, static_cast<unsigned>(total),
                        static_cast<unsigned>(work));
   return check_launch("roi_resample_kernel");
@@ -847,14 +1119,14 @@ int roi_forward_tiled(const void *input, const void *rois, void *output, int dty
   if (p.order == 3) {
     switch (dtype) {
       case MV_F16:
-        return launch_resample<__half, 16, 16, 8, 512, 76 * 1024, 8, true>(
+        return launch_resample<__half, 16, 16, 8, 512, 74 * 1024, 8, true>(
             static_cast<const __half *>(input), r, static_cast<__half *>(output), p, workspace, need, s);
       case MV_BF16:
-        return launch_resample<__hip_bfloat16, 16, 16, 8, 512, 76 * 1024, 8, true>(
+        return launch_resample<__hip_bfloat16, 16, 16, 8, 512, 74 * 1024, 8, true>(
             static_cast<const __hip_bfloat16 *>(input), r, static_cast<__hip_bfloat16 *>(output), p,
             workspace, need, s);
       case MV_F32:
-        return launch_resample<float, 16, 16, 8, 512, 76 * 1024, 6, true>(
+        return launch_resample<float, 16, 16, 8, 512, 74 * 1024, 6, true>(
             static_cast<const float *>(input), r, static_cast<float *>(output), p, workspace, need, s);
       default:
         return -1;
@@ -862,14 +1134,14 @@ int roi_forward_tiled(const void *input, const void *rois, void *output, int dty
   }
   switch (dtype) {
     case MV_F16:
-      return launch_resample<__half, 16, 16, 16, 512, 76 * 1024, 8>(
+      return launch_resample<__half, 16, 16, 16, 512, 74 * 1024, 8>(
           static_cast<const __half *>(input), r, static_cast<__half *>(output), p, workspace, need, s);
     case MV_BF16:
-      return launch_resample<__hip_bfloat16, 16, 16, 16, 512, 76 * 1024, 8>(
+      return launch_resample<__hip_bfloat16, 16, 16, 16, 512, 74 * 1024, 8>(
           static_cast<const __hip_bfloat16 *>(input), r, static_cast<__hip_bfloat16 *>(output), p,
           workspace, need, s);
     case MV_F32:
-      return launch_resample<float, 16, 16, 8, 512, 76 * 1024, 6>(
+      return launch_resample<float, 16, 16, 8, 512, 74 * 1024, 6>(
           static_cast<const float *>(input), r, static_cast<float *>(output), p, workspace, need, s);
     default:
       return -1;
