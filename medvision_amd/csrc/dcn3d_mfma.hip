@@ -21,6 +21,7 @@
 // The sampling gather, not the matrix core, bounds this kernel: per (tap, position) 8 corners x
 // Cin channels are fetched, 8 x more bytes than the fragment holds.
 #include <cstdint>
+#include <cstdlib>
 
 #include "dcn_mfma.hpp"
 
@@ -383,6 +384,201 @@ __global__ __launch_bounds__(256, NB == 1 ? (NC == 4 && WBYTES <= 12 * 1024 ? MV
   }
 }
 
+// ---- taps worked out once per position ------------------------------------------------------------
+// In the kernel above the four lanes that share a position each repeat the tap's geometry (offsets,
+// floor / fraction, 8 corner offsets, 8 weights: about as many vector instructions as the blend of
+// 32 channels).  Here a workgroup of four wavefronts owns 64 positions and alternates two phases
+// per group of TG = 4 taps:
+//   G  wavefront w takes tap w of the group with ONE position per lane (the offset planes are read
+//      as 128 contiguous bytes), and leaves the 8 corner offsets and 8 mask-scaled weights as a
+//      64-byte record in LDS; all lanes also bring the group's weight pieces into LDS;
+//   B  wavefront w takes positions 16 w .. 16 w + 15 in the load layout (position l / 4, piece
+//      l % 4), reads each tap's record as four broadcast 16-byte LDS reads, gathers, blends and
+//      feeds the matrix core as above.
+// The geometry then costs a quarter of what it did per (tap, 16 positions), and the offsets of
+// the next group are requested a whole B phase ahead.  One convolution group must lie inside one
+// deformable group, and a tap's weight pieces (SLICES x MB x 1 KB) are kept to 8 KB.
+template <typename T, int MB, int SLICES, int NC>
+__global__ __launch_bounds__(256, 5) void dcn_forward_shared_taps_kernel(
+    const T *__restrict__ xt, const T *__restrict__ off, const T *__restrict__ mask,
+    const T *__restrict__ wf, const T *__restrict__ bias, T *__restrict__ y, const DcnDims s) {
+  using M = Mfma<T>;
+  constexpr int PC = M::kPiece, SL = 4 * PC, ES = sizeof(T), TG = 4;
+  static_assert(sizeof(T) == 2, "16-bit tensors");
+  constexpr int REC = 2 * NC;                     // dwords per record: NC corner offsets, NC weights
+  constexpr int WT = SLICES * MB * 64;            // 16-byte weight pieces per tap
+  constexpr int WREG = (TG * WT + 255) / 256;     // pieces a thread moves per group
+  constexpr unsigned kOutside = 0x80000000u;      // beyond the buffer: such loads return zeros
+  __shared__ __attribute__((aligned(16))) unsigned rec[TG][64][REC];
+  __shared__ __attribute__((aligned(16))) u32x4 wl[TG * WT];
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int j = lane % 16, kc = lane / 16;   // matrix layout: position (column) and piece of this lane
+  const int lj = lane / 4, lk = lane % 4;    // load layout
+  const int from = (4 * j + kc) * 4;         // ds_bpermute byte address of the lane holding this lane's piece
+  const long q0 = static_cast<long>(xcd_contiguous(blockIdx.x, gridDim.x)) * 64;
+  const int blocks = s.opg / 16;
+  const int chunks = (blocks + MB - 1) / MB;
+  const int g = blockIdx.y / chunks, mb0 = (blockIdx.y % chunks) * MB;
+  const int b = blockIdx.z;
+  const int dgi = g * s.cpg / s.cpd;
+  const long bg = static_cast<long>(b) * s.dg + dgi;
+  const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T *>(xt + static_cast<long>(b) * s.P * s.Cin), 0, static_cast<int>(s.P * s.Cin * ES), 0x00020000);
+
+  // phase G: this lane's position, its grid origin, and the planes it reads (scalar offsets per
+  // tap and component; sizes below 2^31 bytes are checked by the host)
+  const long qg = q0 + lane;
+  const bool live = qg < s.Q;
+  const long qgc = live ? qg : s.Q - 1;
+  float base_d, base_h, base_w;
+  {
+    const int ow = qgc % s.Wo, oh = (qgc / s.Wo) % s.Ho, od = qgc / (static_cast<long>(s.Wo) * s.Ho);
+    base_d = static_cast<float>(od * s.sd - s.pd); base_h = static_cast<float>(oh * s.sh - s.ph);
+    base_w = live ? static_cast<float>(ow * s.sw - s.pw) : -1e30f;   // a dead lane's samples are void
+  }
+  const int plane_bytes = static_cast<int>(s.Q) * ES;
+  const __amdgpu_buffer_rsrc_t offr = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T *>(off + bg * s.nd * s.K * s.Q), 0, s.nd * s.K * plane_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t maskr = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T *>(mask ? mask + bg * s.K * s.Q : off), 0, mask ? s.K * plane_bytes : 0, 0x00020000);
+  const unsigned q_bytes = static_cast<unsigned>(qgc) * ES;
+  auto as_float = [](unsigned short bits) { T t; __builtin_memcpy(&t, &bits, 2); return load(&t); };
+  // (d), h, w offsets and the mask value of tap k, requested one group ahead (a tap beyond the
+  // last one reads zeros: scalar offsets take part in the range check)
+  unsigned short rd = 0, rh = 0, rw = 0, rm = 0;
+  auto request = [&](int k) {
+    const int first = s.nd * k * plane_bytes;
+    if (s.nd == 3) rd = __builtin_amdgcn_raw_buffer_load_b16(offr, q_bytes, first, 0);
+    rh = __builtin_amdgcn_raw_buffer_load_b16(offr, q_bytes, first + (s.nd - 2) * plane_bytes, 0);
+    rw = __builtin_amdgcn_raw_buffer_load_b16(offr, q_bytes, first + (s.nd - 1) * plane_bytes, 0);
+    rm = __builtin_amdgcn_raw_buffer_load_b16(maskr, q_bytes, k * plane_bytes, 0);
+  };
+  // element strides of the channels-last input in bytes, and the corner offsets relative to the first
+  const unsigned cb = s.Cin * ES, wb = static_cast<unsigned>(s.W) * cb, hwb = static_cast<unsigned>(s.H) * wb;
+  // the group's weight pieces: piece `id` of the group = (tap id / WT, slice, block, lane)
+  const int tap_bytes = SLICES * blocks * 64 * 16;   // bytes of one tap's pieces in wf
+  const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T *>(wf + static_cast<long>(g) * s.K * SLICES * blocks * (64 * PC)), 0, s.K * tap_bytes, 0x00020000);
+  unsigned wsrc[WREG];
+#pragma unroll
+  for (int i = 0; i < WREG; i++) {
+    const int id = i * 256 + tid, t = id / WT, rem = id % WT;
+    const int ln = rem % 64, m = (rem / 64) % MB, cc = rem / (64 * MB);
+    wsrc[i] = (id < TG * WT && mb0 + m < blocks) ? static_cast<unsigned>(t * tap_bytes + ((cc * blocks + mb0 + m) * 64 + ln) * 16)
+                                                 : kOutside;
+  }
+
+  float4_t acc[MB];
+#pragma unroll
+  for (int m = 0; m < MB; m++) acc[m] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  // tap of this wavefront in the current group as (i, j, k) kernel indices: advanced by TG per group
+  const int khw = s.kh * s.kw;
+  int ki = wave / khw, kj = (wave % khw) / s.kw, kk = wave % s.kw;
+  request(wave);
+  for (int k0 = 0; k0 < s.K; k0 += TG) {
+    const int taps = min(TG, s.K - k0);
+    // ---- G: the group's weight pieces (requested first, stored last) and this wavefront's tap ----
+    u32x4 wreg[WREG];
+#pragma unroll
+    for (int i = 0; i < WREG; i++) wreg[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, wsrc[i], k0 * tap_bytes, 0);
+    const int k = k0 + wave;
+    if (k < s.K) {
+      const float m = mask ? as_float(rm) : 1.f;
+      float pd = base_d + static_cast<float>(ki * s.dd) + as_float(rd);
+      const float ph = base_h + static_cast<float>(kj * s.dh) + as_float(rh);
+      const float pw = base_w + static_cast<float>(kk * s.dw) + as_float(rw);
+      if (NC == 4) pd = 0.f;   // images: the only slice
+      // A corner is inside iff its index is: with f = floor(p) the low one iff 0 <= f < size, the
+      // high one iff 0 <= f + 1 < size (a sample at -1 exactly keeps a high corner of weight 0).
+      const float fd = floorf(pd), fh = floorf(ph), fw = floorf(pw);
+      const float ld = pd - fd, lh = ph - fh, lw = pw - fw;
+      // (huge positions saturate in the conversion and fail the unsigned comparisons)
+      const int id = static_cast<int>(fd), ih = static_cast<int>(fh), iw = static_cast<int>(fw);
+      const bool vd0 = static_cast<unsigned>(id) < static_cast<unsigned>(s.D), vd1 = static_cast<unsigned>(id + 1) < static_cast<unsigned>(s.D);
+      const bool vh0 = static_cast<unsigned>(ih) < static_cast<unsigned>(s.H), vh1 = static_cast<unsigned>(ih + 1) < static_cast<unsigned>(s.H);
+      const bool vw0 = static_cast<unsigned>(iw) < static_cast<unsigned>(s.W), vw1 = static_cast<unsigned>(iw + 1) < static_cast<unsigned>(s.W);
+      const unsigned first = static_cast<unsigned>(id) * hwb + static_cast<unsigned>(ih) * wb + static_cast<unsigned>(iw) * cb;
+      const float md1 = m * ld, md0 = m - md1;   // mask times the depth weights
+      const float wh1 = lh, wh0 = 1.f - lh, ww1 = lw, ww0 = 1.f - lw;
+      const float hw00 = wh0 * ww0, hw01 = wh0 * ww1, hw10 = wh1 * ww0, hw11 = wh1 * ww1;
+      unsigned at[8];
+      float w[8];
+      at[0] = (vd0 && vh0 && vw0) ? first : kOutside;                 w[0] = md0 * hw00;
+      at[1] = (vd0 && vh0 && vw1) ? first + cb : kOutside;            w[1] = md0 * hw01;
+      at[2] = (vd0 && vh1 && vw0) ? first + wb : kOutside;            w[2] = md0 * hw10;
+      at[3] = (vd0 && vh1 && vw1) ? first + wb + cb : kOutside;       w[3] = md0 * hw11;
+      at[4] = (vd1 && vh0 && vw0) ? first + hwb : kOutside;           w[4] = md1 * hw00;
+      at[5] = (vd1 && vh0 && vw1) ? first + hwb + cb : kOutside;      w[5] = md1 * hw01;
+      at[6] = (vd1 && vh1 && vw0) ? first + hwb + wb : kOutside;      w[6] = md1 * hw10;
+      at[7] = (vd1 && vh1 && vw1) ? first + hwb + wb + cb : kOutside; w[7] = md1 * hw11;
+      unsigned *r = rec[wave][lane];
+#pragma unroll
+      for (int c = 0; c < NC; c += 4) {
+        *reinterpret_cast<u32x4 *>(r + c) = u32x4{at[c], at[c + 1], at[c + 2], at[c + 3]};
+        *reinterpret_cast<u32x4 *>(r + NC + c) = u32x4{__float_as_uint(w[c]), __float_as_uint(w[c + 1]),
+                                                      __float_as_uint(w[c + 2]), __float_as_uint(w[c + 3])};
+      }
+    }
+    request(k + TG);
+    kk += TG;
+    while (kk >= s.kw) { kk -= s.kw; kj++; }
+    while (kj >= s.kh) { kj -= s.kh; ki++; }
+#pragma unroll
+    for (int i = 0; i < WREG; i++)
+      if (i * 256 + tid < TG * WT) wl[i * 256 + tid] = wreg[i];
+    __syncthreads();
+    // ---- B: positions 16 * wave .. + 15, every tap of the group -----------------------------------
+    for (int t = 0; t < taps; t++) {
+      const unsigned *r = rec[t][16 * wave + lj];
+      unsigned at[NC];
+      float cw[NC];
+#pragma unroll
+      for (int c = 0; c < NC; c += 4) {
+        const u32x4 a = *reinterpret_cast<const u32x4 *>(r + c), w4 = *reinterpret_cast<const u32x4 *>(r + NC + c);
+        at[c] = a.x + lk * 16u; at[c + 1] = a.y + lk * 16u; at[c + 2] = a.z + lk * 16u; at[c + 3] = a.w + lk * 16u;
+        cw[c] = __uint_as_float(w4.x); cw[c + 1] = __uint_as_float(w4.y);
+        cw[c + 2] = __uint_as_float(w4.z); cw[c + 3] = __uint_as_float(w4.w);
+      }
+#pragma unroll
+      for (int cc = 0; cc < SLICES; cc++) {
+        const unsigned c0 = g * s.cpg + cc * SL;
+        u32x4 raw[NC];
+#pragma unroll
+        for (int c = 0; c < NC; c++) raw[c] = __builtin_amdgcn_raw_buffer_load_b128(xr, at[c], c0 * ES, 0);
+        float v[PC];
+#pragma unroll
+        for (int i = 0; i < PC; i++) v[i] = 0.f;
+#pragma unroll
+        for (int c = 0; c < NC; c++) M::fma_piece(v, cw[c], raw[c]);
+        const u32x4 mine = M::pack(v);   // piece lk of position lj; wanted: piece kc of position j
+        const u32x4 bpiece = u32x4{
+            static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(from, static_cast<int>(mine.x))),
+            static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(from, static_cast<int>(mine.y))),
+            static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(from, static_cast<int>(mine.z))),
+            static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(from, static_cast<int>(mine.w)))};
+#pragma unroll
+        for (int mm = 0; mm < MB; mm++) acc[mm] = M::run16(wl[t * WT + (cc * MB + mm) * 64 + lane], bpiece, acc[mm]);
+      }
+    }
+    __syncthreads();   // records and weight pieces may be overwritten
+  }
+  const long qo = q0 + 16 * wave + j;
+  if (qo >= s.Q) return;
+#pragma unroll
+  for (int m = 0; m < MB; m++) {
+    if (mb0 + m >= blocks) continue;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      // 16x16 accumulator layout: register r of lane l holds row 4 * (l / 16) + r, column l % 16
+      const int o = g * s.opg + (mb0 + m) * 16 + kc * 4 + r;
+      const float val = acc[m][r] + (bias ? load(bias + o) : 0.f);
+      y[(static_cast<long>(b) * s.Cout + o) * s.Q + qo] = store_cast<T>(val);
+    }
+  }
+}
+
 // [B, C, P] -> [B, P, C] for elements of 2 or 4 bytes
 int dcn_channels_last(const void *x, void *xt, int B, int C, long P, int elem_bytes, hipStream_t stream) {
   const int vec = 16 / elem_bytes;
@@ -413,6 +609,11 @@ int dcn_channels_last(const void *x, void *xt, int B, int C, long P, int elem_by
 }
 
 static size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+// MV_DCN_SHARED_TAPS=0 keeps every layer on the kernels that work the taps out per lane
+static bool dcn_shared_taps_enabled() {
+  static const bool on = [] { const char *e = getenv("MV_DCN_SHARED_TAPS"); return !(e && e[0] == '0'); }();
+  return on;
+}
 static int elem_size(int dtype) { return dtype == MV_F32 ? 4 : 2; }
 
 bool dcn_mfma_supported(const DcnDims &s, int dtype) {
@@ -455,6 +656,28 @@ static int dcn_mfma_run(const void *x, const void *off, const void *mask, const 
       hipLaunchKernelGGL((dcn_weight_fragments16_kernel<T>), dim3(static_cast<unsigned>((lanes + 255) / 256)),
                          dim3(256), 0, stream, static_cast<const T *>(wt), wf, s);
       const int chunks = (blocks16 + mb - 1) / mb;
+      if constexpr (sizeof(T) == 2) {
+        // volumes with 32 or 64 channels per group inside one deformable group: taps shared through LDS
+        const int slices = s.cpg / (4 * PC);
+        const bool volume = !(s.nd == 2 && s.D == 1 && s.kd == 1 && s.pd == 0);
+        const bool small = static_cast<long>(s.nd) * s.K * s.Q * 2 < (1L << 31) &&
+                           static_cast<long>(s.K) * slices * blocks16 * 1024 < (1L << 31);
+        if (dcn_shared_taps_enabled() && (slices == 1 || slices == 2) && s.cpd % s.cpg == 0 && blocks16 >= 4 && volume && small) {
+          const int chunks4 = (blocks16 + 3) / 4;
+          const long qb = (s.Q + 63) / 64;
+          MV_REQUIRE(qb < (1L << 31) && static_cast<long>(s.groups) * chunks4 <= 65535, "grid too large");
+          const dim3 grid(static_cast<unsigned>(qb), s.groups * chunks4, s.B), block(256);
+          if (slices == 1)
+            hipLaunchKernelGGL((dcn_forward_shared_taps_kernel<T, 4, 1, 8>), grid, block, 0, stream, xt,
+                               static_cast<const T *>(off), static_cast<const T *>(mask), wf,
+                               static_cast<const T *>(bias), static_cast<T *>(y), s);
+          else
+            hipLaunchKernelGGL((dcn_forward_shared_taps_kernel<T, 4, 2, 8>), grid, block, 0, stream, xt,
+                               static_cast<const T *>(off), static_cast<const T *>(mask), wf,
+                               static_cast<const T *>(bias), static_cast<T *>(y), s);
+          return check_launch("dcn_forward_shared_taps_kernel");
+        }
+      }
       constexpr int kNb = MV_DCN_NB;
       const long qblocks = (s.Q + 64 * kNb - 1) / (64 * kNb);
       MV_REQUIRE(qblocks < (1L << 31) && static_cast<long>(s.groups) * chunks <= 65535, "grid too large");

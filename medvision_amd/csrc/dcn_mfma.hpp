@@ -34,9 +34,11 @@ template <> struct Mfma<__half> {
   static __device__ __forceinline__ float hi(unsigned w) {
     return __half2float(__ushort_as_half(static_cast<unsigned short>(w >> 16)));
   }
+  // two values rounded to nearest even and packed, in one instruction
   static __device__ __forceinline__ unsigned pack2(float a, float b) {
-    return static_cast<unsigned>(__half_as_ushort(__float2half_rn(a))) |
-           (static_cast<unsigned>(__half_as_ushort(__float2half_rn(b))) << 16);
+    unsigned r;
+    asm("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
   }
   // v[0..7] += w * piece
   static __device__ __forceinline__ void fma_piece(float (&v)[8], float w, u32x4 r) {
@@ -57,12 +59,11 @@ template <> struct Mfma<__hip_bfloat16> {
   }
   static __device__ __forceinline__ float lo(unsigned w) { return __uint_as_float(w << 16); }
   static __device__ __forceinline__ float hi(unsigned w) { return __uint_as_float(w & 0xffff0000u); }
+  // two values rounded to nearest even and packed, in one instruction
   static __device__ __forceinline__ unsigned pack2(float a, float b) {
-    // round to nearest even on the upper 16 bits
-    const unsigned ua = __float_as_uint(a), ub = __float_as_uint(b);
-    const unsigned ra = (ua + 0x7fffu + ((ua >> 16) & 1u)) >> 16;
-    const unsigned rb = (ub + 0x7fffu + ((ub >> 16) & 1u)) & 0xffff0000u;
-    return ra | rb;
+    unsigned r;
+    asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
   }
   static __device__ __forceinline__ void fma_piece(float (&v)[8], float w, u32x4 r) {
     v[0] += w * lo(r.x); v[1] += w * hi(r.x); v[2] += w * lo(r.y); v[3] += w * hi(r.y);
