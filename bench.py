@@ -23,6 +23,11 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense fp16/bf16
+# Measured on this part (microbenchmark, 4 wavefronts per SIMD): a three-operand vector instruction
+# of one wavefront (v_fma_f32, v_fma_mix_f32, conversions) takes 2.03 ns of its SIMD; the vector L1
+# returns 64 bytes per clock and compute unit at the ~1.97 GHz these kernels run at.
+VALU_NS_PER_WAVE_INSTR = 2.03
+SIMDS, CUS, L1_BYTES_PER_CLK, SHADER_GHZ = 1024, 256, 64, 1.97
 
 
 def _events_ms(fn, steps, warmup):
@@ -56,11 +61,13 @@ def bench_affine(args, dtype=torch.float16):
         _C.roi_align_rotated_3d_forward(vols[j], rois[j], outs[j], S, S, S, 1.0, 1, True, 1)
 
     ms, wall_ms = _events_ms(step, args.steps, args.warmup)
+    # practical ceiling of a launch of this size: a plain device copy of the same bytes
+    copy_ms, _ = _events_ms(lambda i: outs[i % args.copies].copy_(vols[(i + 1) % args.copies]), args.steps, args.warmup)
     vox = B * S ** 3
     esz = torch.finfo(dtype).bits // 8
     alg_bytes = 2 * vox * esz            # read every input voxel once + write every output voxel
     return {"ms": ms, "wall_ms": wall_ms, "gvox_s": vox / ms / 1e6, "gbps": alg_bytes / ms / 1e6,
-            "alg_bytes": alg_bytes, "vox": vox}
+            "alg_bytes": alg_bytes, "vox": vox, "copy_ms": copy_ms}
 
 
 def bench_dcn(args, dtype=torch.float16):
@@ -74,8 +81,13 @@ def bench_dcn(args, dtype=torch.float16):
         with torch.no_grad():
             modulated_deform_conv(x, off, mask, w, b, 1, 1, 1, 1, 1)
 
-    ms, _ = _events_ms(step, max(3, min(args.steps, 400)), max(1, min(args.warmup, 40)))
+    ms, wall_ms = _events_ms(step, max(3, min(args.steps, 400)), max(1, min(args.warmup, 40)))
     flops = 2 * 2 * 64 * 32 * 27 * 48 ** 3
+    # floors of the fused gather + blend: per (tap, position) 8 corners x 32 channels are blended in
+    # fp32 (one fma per wavefront instruction and 64 lanes), and 8 x 64 bytes pass through the L1
+    taps_pos = 2 * 48 ** 3 * 27
+    blend_floor_us = taps_pos * 8 * 32 / 64 / SIMDS * VALU_NS_PER_WAVE_INSTR / 1e3
+    gather_floor_us = taps_pos * 8 * 64 / (CUS * L1_BYTES_PER_CLK * SHADER_GHZ * 1e9) * 1e6
 
     # training step (forward + all five gradients), reported beside the forward figure
     ins = [t.clone().requires_grad_(True) for t in (x, off, mask, w, b)]
@@ -87,7 +99,8 @@ def bench_dcn(args, dtype=torch.float16):
         modulated_deform_conv(*ins, 1, 1, 1, 1, 1).backward(gy)
 
     train_ms, _ = _events_ms(train_step, max(3, min(args.steps // 4, 50)), 3)
-    return {"ms": ms, "tflops": flops / ms / 1e9, "flops": flops, "train_ms": train_ms}
+    return {"ms": ms, "wall_ms": wall_ms, "tflops": flops / ms / 1e9, "flops": flops, "train_ms": train_ms,
+            "blend_floor_us": blend_floor_us, "gather_floor_us": gather_floor_us}
 
 
 def bench_other_configs(args):
@@ -221,43 +234,76 @@ def cpu_baseline(args):
         oracle.roi_align_forward(vol, rois, (S, S, S), 1.0, 1, True, 1, True)
         times.append(time.perf_counter() - t0)
     t = sorted(times)[len(times) // 2]
+    # one thread, one of the four samples (a quarter of the work), one pass
+    oracle.set_threads(1)
+    t0 = time.perf_counter()
+    oracle.roi_align_forward(vol[:1], rois[:1], (S, S, S), 1.0, 1, True, 1, True)
+    t1 = time.perf_counter() - t0
+    oracle.set_threads(cores)
     return {"value": round(B * S ** 3 / t / 1e9, 4), "unit": "Gvox/s", "cores": cores, "kind": "port",
+            "one_thread": {"value": round(S ** 3 / t1 / 1e9, 4), "unit": "Gvox/s",
+                           "sample": f"one sample of config 2, one pass ({t1 * 1e3:.0f} ms)"},
+            "cpu_count": os.cpu_count(),
             "sample": f"config 2 (fp16 [4,1,128^3] -> 128^3) through the fp64 C oracle, OpenMP x{cores}, "
                       f"median of {len(times)} passes after 1 warm-up ({t * 1e3:.0f} ms per pass)"}
 
 
 def cpu_reference_paths(args):
     """The reference's own CPU paths, restated (baseline only, no parity claim): the torch-function
-    RoIAlign on config 1 and the aug_cpu affine steps (scipy.ndimage) on one 128^3 volume."""
+    RoIAlign on config 1 (aligned as the configuration says, and with the class's default), the
+    aug_cpu affine steps (scipy.ndimage) and its elastic step on one 128^3 volume, each with all
+    threads and with one."""
     import numpy as np
     import workloads as wl
     from oracle.torchfun_roi_align import torchfun_roi_align
-    res = {"threads": torch.get_num_threads()}
+    res = {"cpu_count": os.cpu_count(), "torch_threads": torch.get_num_threads()}
     g = wl.gen(0)
     feat = torch.randn(2, 16, 32, 64, 64, generator=g)
     rois = wl.roi3d_detection(g, 128, 2, (64, 64, 32), (4.0, 24.0))
     torchfun_roi_align(feat, rois[:8], (7, 7, 7), 1.0)
-    ts = []
-    for _ in range(3):
-        t0 = time.perf_counter()
-        out = torchfun_roi_align(feat, rois, (7, 7, 7), 1.0)
-        ts.append(time.perf_counter() - t0)
-    t = sorted(ts)[1]
-    res["torchfun_roialign_config1"] = {"ms": round(t * 1e3, 2), "outputs_per_s": round(out.numel() / t, 1)}
+
+    def timed(fn, reps=3):
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            out = fn()
+            ts.append(time.perf_counter() - t0)
+        return sorted(ts)[len(ts) // 2], out
+
+    all_threads = torch.get_num_threads()
+    for aligned in (True, False):
+        entry = {}
+        for threads in (all_threads, 1):
+            torch.set_num_threads(threads)
+            t, out = timed(lambda: torchfun_roi_align(feat, rois, (7, 7, 7), 1.0, aligned=aligned))
+            entry["threads_%d" % threads] = {"ms": round(t * 1e3, 2), "outputs_per_s": round(out.numel() / t, 1)}
+        torch.set_num_threads(all_threads)
+        res["torchfun_roialign_config1_aligned_%s" % aligned] = entry
     try:
         from scipy import ndimage as ndi
-        vol = np.random.default_rng(0).standard_normal((1, 128, 128, 128)).astype(np.float32)
+        rng = np.random.default_rng(0)
+        vol = rng.standard_normal((1, 128, 128, 128)).astype(np.float32)
         steps = {
             "rotate_order1": lambda: ndi.rotate(vol, 20.0, axes=(3, 2), reshape=False, order=1),
             "shift_order1": lambda: ndi.shift(vol, (0, 5.5, -3.2, 7.1), order=1),
             "zoom_order1": lambda: ndi.zoom(vol, (1, 1.1, 1.1, 1.1), order=1),
             "resize_zoom_order2": lambda: ndi.zoom(vol, (1, 0.625, 0.5, 0.5), order=2),
         }
-        for name, fn in steps.items():
-            t0 = time.perf_counter()
-            o = fn()
-            dt = time.perf_counter() - t0
-            res["scipy_" + name] = {"ms": round(dt * 1e3, 1), "gvox_s": round(o.size / dt / 1e9, 5)}
+        # Elastic step (aug_cpu/aug_spatial.py:604-638 goes through SimpleITK, which is not installed:
+        # the same two stages with scipy): a coarse 8^3 field of three components is upsampled to the
+        # volume with cubic splines, then the volume is sampled at identity + field, order 1.
+        coarse = (rng.random((3, 8, 8, 8)).astype(np.float32) * 2 - 1) * 6.0
+        ident = np.meshgrid(*[np.arange(128, dtype=np.float32)] * 3, indexing="ij")
+
+        def elastic():
+            field = [ndi.zoom(c, 16.0, order=3) for c in coarse]
+            coords = [ident[a] + field[a] for a in range(3)]
+            return ndi.map_coordinates(vol[0], coords, order=1, mode="nearest")
+
+        steps["elastic_zoom3_plus_map_coordinates1"] = elastic
+        for name, fn in steps.items():   # scipy.ndimage runs on one thread
+            dt, o = timed(fn, 1)
+            res["scipy_" + name] = {"ms": round(dt * 1e3, 1), "gvox_s": round(o.size / dt / 1e9, 5), "threads": 1}
     except Exception as e:  # scipy missing on the box
         res["scipy"] = f"unavailable: {e}"
     return res
@@ -303,7 +349,8 @@ def main():
         "metric": "RoIAlignRotated3D output throughput (fp16 [4,1,128^3] -> 128^3, sr=1)",
         "value": round(a16["gvox_s"], 3), "unit": "Gvox/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(a16["ms"], 6), "higher_is_better": True, "scaling": "weak",
+        "ms_per_step": round(a16["ms"], 6), "wall_ms_per_step": round(a16["wall_ms"], 6),
+        "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": "BASELINE config 2: RoIAlignRotated3D as RandomAffine resampling, "
@@ -315,7 +362,9 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(a16["gbps"], 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(a16["gbps"] / HBM_PEAK_GBPS, 4), "traffic": None,
                      "kernel": "roi_resample_kernel", "algorithmic_bytes_per_launch": a16["alg_bytes"],
-                     "avg_launch_us": round(a16["ms"] * 1e3, 3)},
+                     "avg_launch_us": round(a16["ms"] * 1e3, 3),
+                     "copy_ceiling_us": round(a16["copy_ms"] * 1e3, 3),
+                     "frac_of_copy_ceiling": round(a16["copy_ms"] / a16["ms"], 4)},
         "fp32": {"gvox_s": round(a32["gvox_s"], 3), "gbps": round(a32["gbps"], 1),
                  "ms_per_step": round(a32["ms"], 6),
                  "frac": round(a32["gbps"] / HBM_PEAK_GBPS, 4)},
@@ -324,12 +373,15 @@ def main():
         d = bench_dcn(args)
         line["dcn"] = {"metric": "DCNv2-3D forward (fp16 [2,32,48^3], 3^3, Cout 64)",
                        "value": round(d["tflops"], 3), "unit": "TFLOP/s",
-                       "ms_per_step": round(d["ms"], 6),
+                       "ms_per_step": round(d["ms"], 6), "wall_ms_per_step": round(d["wall_ms"], 6),
                        "forward_backward_ms": round(d["train_ms"], 4),
                        "roofline": {"bound": "mfma", "achieved": round(d["tflops"], 3),
                                     "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                                     "frac": round(d["tflops"] / MFMA_F16_PEAK_TFLOPS, 5),
-                                    "traffic": None, "flops_per_launch": d["flops"]}}
+                                    "traffic": None, "flops_per_launch": d["flops"],
+                                    "vector_blend_floor_us": round(d["blend_floor_us"], 1),
+                                    "l1_gather_floor_us": round(d["gather_floor_us"], 1),
+                                    "frac_of_gather_floor": round(d["gather_floor_us"] / (d["ms"] * 1e3), 4)}}
     if not args.no_configs:
         line["other_configs"] = bench_other_configs(args)
     if not args.no_next:
@@ -342,7 +394,7 @@ def main():
         measured = json.load(open(traffic))
         line["roofline"]["traffic"] = measured.get("roi_resample_fp16_config2")
         if "dcn" in line:
-            line["dcn"]["roofline"]["traffic"] = measured.get("dcn_forward_mfma16_fp16_config4")
+            line["dcn"]["roofline"]["traffic"] = measured.get("dcn_forward_fp16_config4")
     print(json.dumps(line))
 
 
