@@ -17,6 +17,7 @@
 #include "common.hpp"
 #include "roi_geometry.hpp"
 #include "sampling.hpp"
+#include "dcn_mfma.hpp"
 
 namespace mv {
 
@@ -39,8 +40,6 @@ struct AxisTaps {
 struct PoolShared {
   RoiGeom g;
   AxisTaps ax[3];  // x, y, z
-  int staged;      // 1: LDS path, 0: per-output gather, -1: every output is zero
-  int chunk;       // channels per LDS pass
 };
 
 // The tap entries of one output cell (grid <= kTapRegs samples) in registers; unused entries have
@@ -72,84 +71,134 @@ struct TapRegs {
   static __device__ __forceinline__ float load_any(const __hip_bfloat16 *p) { return mv::load(p); }
 };
 
+struct PoolPlan {
+  int staged;      // 1: LDS path, 0: per-output gather, -1: every output is zero
+  int chunk;       // channels per LDS pass
+};
+
+static_assert(kPoolEntries == kWave, "one wavefront builds the tap table of one axis, one entry per lane");
+__device__ __forceinline__ int wave_min(int v) {
+#pragma unroll
+  for (int m = 1; m < kWave; m *= 2) v = min(v, __shfl_xor(v, m));
+  return v;
+}
+
+constexpr int kDenseSrc = 32;   // source voxels per axis of the dense weight matrices (see below)
+
 // Builds geometry and tap tables for roi `roi`; all threads must call it (contains barriers).
-template <typename RT>
-__device__ inline void pool_setup(PoolShared &sh, const RT *roi, const RoiProblem &p, size_t elem_bytes) {
-  if (threadIdx.x == 0) {
-    const double sn[3] = {0, 0, 0}, cs[3] = {1, 1, 1};
-    build_geom(sh.g, roi, p, sn, cs);
-    const int cells[3] = {p.ow, p.oh, p.od};
-    for (int a = 0; a < 3; a++) {
-      sh.ax[a].grid = a < p.ndim ? sh.g.grid[a] : 1;
-      sh.ax[a].entries = cells[a] * max(sh.ax[a].grid, 0);
-      sh.ax[a].box_lo = 1 << 30;
-      sh.ax[a].box_hi = -1;
-    }
-    sh.staged = 1;
-    if (sh.g.batch < 0) sh.staged = -1;
-    for (int a = 0; a < 3; a++) {
-      if (sh.ax[a].entries > kPoolEntries) sh.staged = min(sh.staged, 0);
-      if (sh.ax[a].entries <= 0) sh.staged = -1;  // empty sampling grid: outputs are zero
-    }
-  }
-  __syncthreads();
-  if (sh.staged <= 0) return;
+// Wavefront a (0..2) works out axis a on its own: the axis geometry (the same expressions as
+// build_geom), one tap entry per lane, the box bounds by a reduction inside the wavefront and, when
+// `wd` is given and the axis fits, the dense weight matrix wd[a][source index][cell] = sum of the
+// weights of the cell's samples that touch the source index (samples in their order; a wavefront's
+// LDS operations execute in order).  The fourth wavefront writes the whole geometry for the plain
+// gather / scatter paths.  One barrier (two with `with_first`, the entry ranges per source index).
+template <typename RT, int CELLS>
+__device__ inline PoolPlan pool_setup(PoolShared &sh, const RT *roi, const RoiProblem &p, size_t elem_bytes,
+                                      bool with_first, float (*wd)[kDenseSrc][CELLS]) {
+  const int nd = p.ndim;
+  const int cells[3] = {p.ow, p.oh, p.od};
   const int size[3] = {p.W, p.H, p.D};
-  for (int e = threadIdx.x; e < 3 * kPoolEntries; e += kPoolThreads) {
-    const int a = e / kPoolEntries, i = e % kPoolEntries;
+  const int b = static_cast<int>(roi[0]);
+  // extents and sampling grids of all axes (every lane the same): they decide the path
+  double start[3], ext[3];
+  int grid[3], entries[3];
+  PoolPlan plan{1, 0};
+  if (b < 0 || b >= p.N) plan.staged = -1;
+#pragma unroll
+  for (int a = 0; a < 3; a++) {
+    start[a] = 0.0; ext[a] = 0.0; grid[a] = 1;
+    if (a < nd) {
+      const double lo = static_cast<double>(roi[1 + a]) * p.scale;
+      const double hi = static_cast<double>(roi[1 + nd + a]) * p.scale;
+      ext[a] = fmax(hi - lo, 1.0);
+      start[a] = lo;
+      grid[a] = p.sampling_ratio > 0 ? p.sampling_ratio
+                                     : static_cast<int>(ceil(ext[a] / static_cast<double>(cells[a])));
+    }
+    entries[a] = cells[a] * max(grid[a], 0);
+    if (entries[a] > kPoolEntries) plan.staged = min(plan.staged, 0);
+  }
+#pragma unroll
+  for (int a = 0; a < 3; a++)
+    if (entries[a] <= 0) plan.staged = -1;  // empty sampling grid: outputs are zero
+  const int a = threadIdx.x / kWave, i = threadIdx.x % kWave;
+  if (a == 3 || plan.staged <= 0) {
+    if (a == 3 || plan.staged == 0) {   // (plan.staged == 0: every wavefront the same values)
+      const double sn[3] = {0, 0, 0}, cs[3] = {1, 1, 1};
+      RoiGeom g;
+      build_geom(g, roi, p, sn, cs);
+      if (i == 0) sh.g = g;
+    }
+  } else {
     AxisTaps &t = sh.ax[a];
-    if (i >= t.entries) continue;
-    const int cell = i / t.grid, sub = i % t.grid;
-    const double v = a < p.ndim ? local_coord(sh.g, a, cell, sub) : 0.0;
-    int lo, hi;
-    float frac;
-    const bool ok = clamped_tap<float>(v, size[a], lo, hi, frac, p.order);
-    const float inv = 1.f / static_cast<float>(t.grid);
-    // void samples keep weight 0; park them at the matching end so that `lo` stays monotonic
-    t.lo[i] = ok ? lo : (v > 0.0 ? -2 : -1);
-    t.hi[i] = t.lo[i] < 0 ? t.lo[i] : hi;
-    t.wlo[i] = ok ? (1.f - frac) * inv : 0.f;
-    t.whi[i] = ok ? frac * inv : 0.f;
-    if (ok) {
-      atomicMin(&t.box_lo, lo);
-      atomicMax(&t.box_hi, hi);
+    const int gr = a == 0 ? grid[0] : (a == 1 ? grid[1] : grid[2]);
+    const int en = a == 0 ? entries[0] : (a == 1 ? entries[1] : entries[2]);
+    const int sz = a == 0 ? size[0] : (a == 1 ? size[1] : size[2]);
+    const int nc = a == 0 ? cells[0] : (a == 1 ? cells[1] : cells[2]);
+    const double st = a == 0 ? start[0] : (a == 1 ? start[1] : start[2]);
+    const double ex = a == 0 ? ext[0] : (a == 1 ? ext[1] : ext[2]);
+    const double bin = a < nd ? ex / static_cast<double>(nc) : 0.0;
+    const double sub_step = bin / static_cast<double>(gr > 0 ? gr : 1);
+    const bool on = i < en;
+    const int cell = on ? i / gr : 0, sub = on ? i % gr : 0;
+    // (local_coord's expression)
+    const double v = a < nd ? st + cell * bin + static_cast<double>(static_cast<float>(sub) + .5f) * sub_step : 0.0;
+    int lo = 0, hi = 0;
+    float frac = 0.f;
+    const bool ok = clamped_tap<float>(v, sz, lo, hi, frac, p.order) && on;
+    const float inv = 1.f / static_cast<float>(gr);
+    const int box_lo = wave_min(ok ? lo : (1 << 30)), box_hi = -wave_min(ok ? -hi : 1);
+    const int top = box_hi - box_lo;
+    const float wlo = ok ? (1.f - frac) * inv : 0.f, whi = ok ? frac * inv : 0.f;
+    // void samples keep weight 0; they are parked at the matching end so that `lo` stays monotonic
+    const int rlo = ok ? lo - box_lo : (v > 0.0 ? top : 0), rhi = ok ? hi - box_lo : (v > 0.0 ? top : 0);
+    if (on) {
+      t.lo[i] = rlo; t.hi[i] = rhi;
+      t.wlo[i] = wlo; t.whi[i] = whi;
+    }
+    if (i == 0) {
+      t.box_lo = box_lo; t.box_hi = box_hi;
+      t.entries = en; t.grid = gr;
+    }
+    if (wd != nullptr && box_hi >= 0 && top < kDenseSrc && nc <= CELLS) {
+      float *m = &wd[a][0][0];
+      for (int k = i; k < kDenseSrc * CELLS / 4; k += kWave) reinterpret_cast<float4 *>(m)[k] = float4{0.f, 0.f, 0.f, 0.f};
+      for (int sidx = 0; sidx < gr; sidx++) {
+        __builtin_amdgcn_wave_barrier();   // (keeps the samples' read-modify-write rounds apart)
+        if (ok && sub == sidx) {
+          m[rlo * CELLS + cell] += wlo;
+          m[rhi * CELLS + cell] += whi;
+        }
+      }
     }
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    long vol = 1;
-    for (int a = 0; a < 3; a++) {
-      if (sh.ax[a].box_hi < 0) { sh.staged = -1; break; }  // no valid sample on this axis
-      vol *= sh.ax[a].box_hi - sh.ax[a].box_lo + 1;
-    }
-    if (sh.staged == 1) {
-      const long nz = sh.ax[2].box_hi - sh.ax[2].box_lo + 1, ny = sh.ax[1].box_hi - sh.ax[1].box_lo + 1;
-      const long per_channel = vol * static_cast<long>(elem_bytes) + (nz * ny * p.ow + nz * p.oh * p.ow) * 4 + 16;
-      const long chunk = kPoolLdsBytes / per_channel;
-      if (chunk < 1) sh.staged = 0;
-      sh.chunk = static_cast<int>(min(chunk, 64L));
-    }
+  if (plan.staged <= 0) return plan;
+  long vol = 1;
+#pragma unroll
+  for (int k = 0; k < 3; k++) {
+    if (sh.ax[k].box_hi < 0) plan.staged = -1;  // no valid sample on this axis
+    vol *= sh.ax[k].box_hi - sh.ax[k].box_lo + 1;
   }
-  __syncthreads();
-  if (sh.staged != 1) return;
-  for (int e = threadIdx.x; e < 3 * kPoolEntries; e += kPoolThreads) {  // make indices box-relative
-    const int a = e / kPoolEntries, i = e % kPoolEntries;
-    AxisTaps &t = sh.ax[a];
-    if (i >= t.entries) continue;
-    const int top = t.box_hi - t.box_lo;
-    t.lo[i] = t.lo[i] == -1 ? 0 : (t.lo[i] == -2 ? top : t.lo[i] - t.box_lo);
-    t.hi[i] = t.hi[i] == -1 ? 0 : (t.hi[i] == -2 ? top : t.hi[i] - t.box_lo);
+  if (plan.staged != 1) return plan;
+  {
+    const long nz = sh.ax[2].box_hi - sh.ax[2].box_lo + 1, ny = sh.ax[1].box_hi - sh.ax[1].box_lo + 1;
+    const long per_channel = vol * static_cast<long>(elem_bytes) + (nz * ny * p.ow + nz * p.oh * p.ow) * 4 + 16;
+    const long chunk = kPoolLdsBytes / per_channel;
+    if (chunk < 1) plan.staged = 0;
+    plan.chunk = static_cast<int>(min(chunk, 64L));
   }
-  __syncthreads();
+  if (plan.staged != 1 || !with_first) return plan;
   for (int e = threadIdx.x; e < 3 * (kPoolEntries + 4); e += kPoolThreads) {  // entry ranges per source index
-    const int a = e / (kPoolEntries + 4), i = e % (kPoolEntries + 4);
-    AxisTaps &t = sh.ax[a];
-    if (i > t.box_hi - t.box_lo + 1) continue;
+    const int k = e / (kPoolEntries + 4), j = e % (kPoolEntries + 4);
+    AxisTaps &t = sh.ax[k];
+    if (j > t.box_hi - t.box_lo + 1) continue;
     int f = 0;
-    while (f < t.entries && t.lo[f] < i) f++;
-    t.first[i] = f;
+    while (f < t.entries && t.lo[f] < j) f++;
+    t.first[j] = f;
   }
   __syncthreads();
+  return plan;
 }
 
 // Dense form of the tap tables for the usual small boxes (<= CELLS cells per axis, box of
@@ -158,8 +207,6 @@ __device__ inline void pool_setup(PoolShared &sh, const RT *roi, const RoiProble
 // each value into all cells" (forward) or "load the cells of a line, one dot product per source
 // index" (backward): no per-entry branches, the matrix rows are LDS broadcasts.
 // The kernels are instantiated for CELLS = 8 (7^3 detection heads) and 16 (14 x 14 mask heads).
-constexpr int kDenseSrc = 32;
-
 template <int CELLS>
 __device__ __forceinline__ bool dense_applies(const PoolShared &sh, const RoiProblem &p) {
   for (int a = 0; a < 3; a++)
@@ -196,6 +243,248 @@ __device__ __forceinline__ void dense_axpy(float (&acc)[CELLS], const float *row
   }
 }
 
+// Forward pass of one (roi, channel block) on the matrix cores, fp16 tensors, <= 8 cells per axis,
+// box rows times padded box columns <= kMfmaYx.  The contraction over (y, x) is one GEMM per group
+// of four box slices,
+//     T[(channel, slice)][(ph, pw)] = sum_(y, x) box[(channel, slice)][(y, x)] * (Wy[y][ph] Wx[x][pw]),
+// with the box chunk and the weight products in LDS as 16-byte K pieces; K = y * NXP + x with the
+// box row padded to NXP = a multiple of four columns (zero weights on the pad), so that a box row is
+// staged as 8-byte pieces: one 2-byte-aligned buffer load and one LDS store per four voxels.  The
+// per-lane offset (channel within the pass, slice, y, x piece) stays fixed while the channel moves
+// through the scalar offset: no index arithmetic per element, and slices or channels outside the box
+// or the block read zeros through the range check.
+// Rows are ordered (channel, slice % 4), so the 16 x 16 accumulator hands every lane the four slices
+// of ONE channel at one (ph, pw): for two slice groups that is exactly the 8-element K piece of a
+// second matrix product with rows (ph, pw), K = (channel, slice) and a block-diagonal right-hand side
+//     out[(ph, pw)][(channel', pd)] = sum_(channel, z) T[(ph, pw)][(channel, z)] * (channel == channel') Wz[z][pd],
+// whose pieces every lane forms from the z matrix by itself (as an fp16 pair high + low, so the z
+// weights keep 22 bits).  The contraction over z thereby runs on the matrix cores too, without moving
+// T (it is rounded to fp16 once); a lane ends up with four neighbouring cells of one (channel, pd).
+constexpr int kMfmaYx = 224;
+template <typename T>
+__device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__restrict__ dst, const RoiProblem &p,
+                                         const PoolShared &sh, const float (&wd)[3][kDenseSrc][8],
+                                         unsigned char *lds, int c_count, long range_bytes) {
+  using M = Mfma<T>;
+  typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+  constexpr int ES = static_cast<int>(sizeof(T));
+  auto uni = [](int v) { return __builtin_amdgcn_readfirstlane(v); };   // values read from LDS are the same in every lane
+  const int nx = uni(sh.ax[0].box_hi - sh.ax[0].box_lo + 1), ny = uni(sh.ax[1].box_hi - sh.ax[1].box_lo + 1),
+            nz = uni(sh.ax[2].box_hi - sh.ax[2].box_lo + 1);
+  const int x_lo = uni(sh.ax[0].box_lo), y_lo = uni(sh.ax[1].box_lo), z_lo = uni(sh.ax[2].box_lo);
+  const int NXP = (nx + 3) & ~3, pieces = ny * NXP / 4;              // 8-byte pieces of one box slice
+  const int KP = (ny * NXP + 31) / 32 * 32, WS = KP + 8;             // weight rows: KP products + a pad against bank conflicts
+  int KC = min(KP, 96);                                              // box rows: one K chunk
+  while (64 * WS * ES + 16 * 4 * (KC + 8) * ES > kPoolLdsBytes) KC -= 32;
+  const int RS = KC + 8;
+  const int ohw = p.oh * p.ow, cells = p.od * ohw;
+  const long plane = static_cast<long>(p.D) * p.H * p.W;
+  const int hw = p.H * p.W;
+  T *w = reinterpret_cast<T *>(lds);            // [64 cells (ph, pw)][WS]
+  T *box = w + 64 * WS;                         // [CH channels][4 * ZS slices][RS]
+  // groups of four slices staged at once (the whole box for the usual small ones; one group when the
+  // box needs several K chunks, whose products accumulate in the same registers)
+  const int zgroups = (nz + 3) / 4;
+  const int fit = (kPoolLdsBytes - 64 * WS * ES) / (16 * 4 * RS * ES);
+  const int ZS = KP > KC ? 1 : max(1, min(min(zgroups, fit), 2));
+  const int ZS4 = ZS * 4;
+  const bool one_stage = zgroups <= ZS && KP <= KC;   // the usual case: the whole box in one stage
+  // channels per stage: up to four blocks of 16 when the whole box fits (fewer, longer stages: every
+  // stage costs two barriers and one round trip to memory)
+  const int CH = 16 * (one_stage ? max(1, min(min(4, fit / ZS), (c_count + 15) / 16)) : 1);
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const float inv_ow = 1.f / p.ow, inv_nxp = 1.f / NXP;
+  {  // weight products: thread = (cell, quarter of the K range), pairs of neighbouring K
+    const int n = tid / 4, q = tid % 4, ph = fdiv(n, inv_ow), pw = n - ph * p.ow;
+    const bool nv = n < ohw;
+    const int kq = KP / 4;
+    int k = q * kq, y = fdiv(k, inv_nxp), x = k - y * NXP;
+    T *wr = w + n * WS + k;
+    for (int i = 0; i < kq; i += 2) {
+      float v[2];
+#pragma unroll
+      for (int e = 0; e < 2; e++) {
+        v[e] = (nv && y < ny && x < nx) ? wd[1][y < ny ? y : 0][ph & 7] * wd[0][x < nx ? x : 0][pw] : 0.f;
+        x++;
+        if (x == NXP) { x = 0; y++; }
+      }
+      *reinterpret_cast<unsigned *>(wr + i) = M::pack2(v[0], v[1]);
+    }
+  }
+  // the box rows start out as zeros: the staging never writes K positions beyond the last piece
+  for (int i = tid; i < CH * ZS4 * RS / 2; i += kPoolThreads) reinterpret_cast<unsigned *>(box)[i] = 0u;
+  const int col = lane % 16, quad = lane / 16;
+  // staging: an item is (channel of the pass, slice, piece); a thread keeps its item while the passes
+  // walk over the channels
+  const int QV = min(KC / 4, pieces), ipc = ZS4 * QV, cpp = min(CH, kPoolThreads / ipc), passes = (CH + cpp - 1) / cpp;
+  const float inv_ipc = 1.f / ipc, inv_qv = 1.f / QV;
+  const int c_sub = fdiv(tid, inv_ipc), rem = tid - c_sub * ipc, zslot = fdiv(rem, inv_qv), ql = rem - zslot * QV;
+  const bool item = c_sub < cpp;
+  const unsigned long long sp = reinterpret_cast<unsigned long long>(src_any);
+  const T *src = reinterpret_cast<const T *>(static_cast<unsigned long long>(uni(static_cast<int>(sp))) & 0xffffffffull |
+                                             static_cast<unsigned long long>(uni(static_cast<int>(sp >> 32))) << 32);
+  const __amdgpu_buffer_rsrc_t fr = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T *>(src), 0, static_cast<int>(range_bytes), 0x00020000);
+  const unsigned corner = static_cast<unsigned>(((static_cast<long>(z_lo) * p.H + y_lo) * p.W + x_lo) * ES);
+  const int plane_bytes = static_cast<int>(plane) * ES;
+  constexpr unsigned kNowhere = 0x80000000u;
+  unsigned voff, keep_lo, keep_hi;   // the item's byte offset; masks that clear the columns beyond the box row
+  auto item_offset = [&](int zg, int kc) {
+    const int z = zg * 4 + zslot, q = kc / 4 + ql, y = fdiv(q * 4, inv_nxp), x0 = q * 4 - y * NXP;
+    const bool ok = item && z < nz && q < pieces;
+    voff = ok ? corner + static_cast<unsigned>(c_sub * plane_bytes + (z * hw + y * p.W + x0) * ES) : kNowhere;
+    const int left = nx - x0;   // >= 1 for a piece of the row
+    keep_lo = left >= 2 ? 0xffffffffu : 0x0000ffffu;
+    keep_hi = left >= 4 ? 0xffffffffu : (left == 3 ? 0x0000ffffu : 0u);
+  };
+  item_offset(0, 0);
+  T *box_item = box + (c_sub * ZS4 + zslot) * RS + ql * 4;
+  const int pass_elems = cpp * ZS4 * RS;
+  // right-hand side of the z product for the stage that starts with slice group zg: column n = 16 h + col
+  // is (channel' = n / 8, pd = n % 8); this lane's K group is channel `quad`, slices 4 zg .. 4 zg + 7
+  auto z_pieces = [&](int zg, u32x4 (&zhi)[2], u32x4 (&zlo)[2]) {
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      const int n = 16 * h + col, pd = n % 8;
+      const bool mine = n / 8 == quad;
+      float zw[8], zr[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        const int z = zg * 4 + i;
+        zw[i] = (mine && i < ZS4 && z < nz) ? wd[2][z < kDenseSrc ? z : 0][pd] : 0.f;
+      }
+      zhi[h] = M::pack(zw);
+      zr[0] = zw[0] - M::lo(zhi[h].x); zr[1] = zw[1] - M::hi(zhi[h].x);
+      zr[2] = zw[2] - M::lo(zhi[h].y); zr[3] = zw[3] - M::hi(zhi[h].y);
+      zr[4] = zw[4] - M::lo(zhi[h].z); zr[5] = zw[5] - M::hi(zhi[h].z);
+      zr[6] = zw[6] - M::lo(zhi[h].w); zr[7] = zw[7] - M::hi(zhi[h].w);
+      zlo[h] = M::pack(zr);
+    }
+  };
+  u32x4 zhi0[2], zlo0[2];
+  z_pieces(0, zhi0, zlo0);
+  // box rows of channels cb .. cb + CH - 1 for the stage (zg, kc): up to eight passes of loads in
+  // flight together; between two barriers
+  auto stage = [&](int cb) {
+    for (int ps0 = 0; ps0 < passes; ps0 += 8) {
+      u32x2 val[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        val[u] = u32x2{0u, 0u};
+        if (ps0 + u < passes)
+          val[u] = __builtin_amdgcn_raw_buffer_load_b64(fr, voff, (cb + (ps0 + u) * cpp) * plane_bytes, 0);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        if (ps0 + u < passes && item && (ps0 + u) * cpp + c_sub < CH) {
+          uint2 v2;
+          v2.x = val[u].x & keep_lo;
+          v2.y = val[u].y & keep_hi;
+          *reinterpret_cast<uint2 *>(box_item + (ps0 + u) * pass_elems) = v2;
+        }
+      }
+    }
+  };
+  // this wavefront: channels 4 * wave .. + 3 of the 16-channel block sb, rows (channel, slice % 4) of
+  // every staged slice group, K chunk kc
+  auto first_product = [&](int sb, int kc, float4_t (&acc)[2][4]) {
+    for (int k0 = 0; k0 < KC && kc + k0 < KP; k0 += 32) {
+      u32x4 b[4];
+#pragma unroll
+      for (int nt = 0; nt < 4; nt++)
+        b[nt] = *reinterpret_cast<const u32x4 *>(w + (nt * 16 + col) * WS + kc + k0 + quad * 8);
+#pragma unroll
+      for (int zs = 0; zs < 2; zs++) {
+        if (zs < ZS) {
+          const int c_local = sb * 16 + wave * 4 + col / 4, zrow = zs * 4 + col % 4;
+          const u32x4 a = *reinterpret_cast<const u32x4 *>(box + (c_local * ZS4 + zrow) * RS + k0 + quad * 8);
+#pragma unroll
+          for (int nt = 0; nt < 4; nt++) acc[zs][nt] = M::run16(a, b[nt], acc[zs][nt]);
+        }
+      }
+    }
+  };
+  // contraction over the (up to eight) slices of a stage
+  auto second_product = [&](const float4_t (&acc)[2][4], const u32x4 (&zhi)[2], const u32x4 (&zlo)[2], float4_t (&oacc)[4][2]) {
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) {
+      const u32x4 ta = u32x4{M::pack2(acc[0][nt][0], acc[0][nt][1]), M::pack2(acc[0][nt][2], acc[0][nt][3]),
+                             M::pack2(acc[1][nt][0], acc[1][nt][1]), M::pack2(acc[1][nt][2], acc[1][nt][3])};
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        oacc[nt][h] = M::run16(ta, zlo[h], oacc[nt][h]);
+        oacc[nt][h] = M::run16(ta, zhi[h], oacc[nt][h]);
+      }
+    }
+  };
+  // register r of oacc[nt][h]: cell nt * 16 + 4 * quad + r of (channel c16 + 4 * wave + 2 h + col / 8, pd col % 8)
+  auto store_cells = [&](int c16, const float4_t (&oacc)[4][2]) {
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      const int c = c16 + wave * 4 + 2 * h + col / 8, pd = col % 8;
+      if (c < c_count && pd < p.od) {
+        T *o = dst + static_cast<long>(c) * cells + pd * ohw;
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++) {
+          const int n = nt * 16 + 4 * quad;
+          if (n + 3 < ohw) {   // four neighbouring cells as one 8-byte store (2-byte aligned)
+            struct __attribute__((packed, aligned(2))) Cells4 { unsigned lo, hi; };
+            Cells4 v4;
+            v4.lo = M::pack2(oacc[nt][h][0], oacc[nt][h][1]);
+            v4.hi = M::pack2(oacc[nt][h][2], oacc[nt][h][3]);
+            *reinterpret_cast<Cells4 *>(o + n) = v4;
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+              if (n + r < ohw) o[n + r] = store_cast<T>(oacc[nt][h][r]);
+          }
+        }
+      }
+    }
+  };
+  auto clear = [](float4_t (&acc)[2][4], float4_t *oacc) {
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      acc[i / 4][i % 4] = float4_t{0.f, 0.f, 0.f, 0.f};
+      if (oacc) oacc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+  };
+  if (one_stage) {
+    for (int cb = 0; cb < c_count; cb += CH) {
+      __syncthreads();   // the weights are complete / the previous stage has been consumed
+      stage(cb);
+      __syncthreads();
+      for (int sb = 0; sb < CH / 16 && cb + sb * 16 < c_count; sb++) {
+        float4_t acc[2][4], oacc[4][2];
+        clear(acc, &oacc[0][0]);
+        first_product(sb, 0, acc);
+        second_product(acc, zhi0, zlo0, oacc);
+        store_cells(cb + sb * 16, oacc);
+      }
+    }
+    return;
+  }
+  for (int cb = 0; cb < c_count; cb += 16) {
+    float4_t oacc[4][2];   // [cell tile][half of the (channel', pd) columns]: cells 4 * quad .. + 3 of the tile
+    float4_t acc[2][4];    // [slice group of the stage][cell tile]
+    clear(acc, &oacc[0][0]);
+    for (int zg = 0; zg < zgroups; zg += ZS) {
+      clear(acc, nullptr);
+      for (int kc = 0; kc < KP; kc += KC) {
+        item_offset(zg, kc);
+        __syncthreads();
+        stage(cb);
+        __syncthreads();
+        first_product(0, kc, acc);
+      }
+      u32x4 zhi[2] = {zhi0[0], zhi0[1]}, zlo[2] = {zlo0[0], zlo0[1]};
+      if (zg > 0) z_pieces(zg, zhi, zlo);
+      second_product(acc, zhi, zlo, oacc);
+    }
+    store_cells(cb, oacc);
+  }
+}
+
 template <typename T, typename RT, int CELLS>
 __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
     const T *__restrict__ feat, const RT *__restrict__ rois, T *__restrict__ out, const RoiProblem p,
@@ -204,17 +493,19 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
   __shared__ __attribute__((aligned(16))) unsigned char lds[kPoolLdsBytes];
   const unsigned n = blockIdx.x;
   const int c_begin = blockIdx.y * channels_per_block, c_end = min(c_begin + channels_per_block, p.C);
-  pool_setup(sh, rois + static_cast<long>(n) * roi_columns(p.ndim, 0), p, sizeof(T));
+  __shared__ __attribute__((aligned(16))) float wd[3][kDenseSrc][CELLS];
+  const PoolPlan plan = pool_setup<RT, CELLS>(sh, rois + static_cast<long>(n) * roi_columns(p.ndim, 0), p, sizeof(T), false,
+                                              CELLS == 8 ? wd : nullptr);
   const int cells = p.od * p.oh * p.ow;
   const long plane = static_cast<long>(p.D) * p.H * p.W;
   T *dst = out + (static_cast<long>(n) * p.C + c_begin) * cells;
   const int total = (c_end - c_begin) * cells;
-  if (sh.staged < 0) {
+  if (plan.staged < 0) {
     for (int i = threadIdx.x; i < total; i += kPoolThreads) dst[i] = store_cast<T>(0.f);
     return;
   }
   const T *src = feat + (static_cast<long>(sh.g.batch) * p.C + c_begin) * plane;
-  if (sh.staged == 0) {  // per-output gather
+  if (plan.staged == 0) {  // per-output gather
     const int gz = p.ndim == 3 ? sh.g.grid[2] : 1, gy = sh.g.grid[1], gx = sh.g.grid[0];
     for (int i = threadIdx.x; i < total; i += kPoolThreads) {
       const int pw = i % p.ow, ph = (i / p.ow) % p.oh, pd = (i / (p.ow * p.oh)) % p.od, c = i / cells;
@@ -238,13 +529,28 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
   const int ohw = p.oh * p.ow;
   const float inv_vol = 1.f / vol, inv_nxy = 1.f / (nx * ny), inv_nx = 1.f / nx, inv_ow = 1.f / p.ow,
               inv_ohw = 1.f / ohw, inv_cells = 1.f / cells;
-  __shared__ __attribute__((aligned(16))) float wd[3][kDenseSrc][CELLS];
   // (with 9..16 cells per axis a row of the matrix is mostly zeros: the tap-register form below is
   // faster for the forward pass; the backward pass still gains from the dense form)
-  const bool dense = CELLS == 8 && dense_applies<CELLS>(sh, p);
-  if (dense) dense_build<CELLS>(sh, p, wd);
-  for (int cb = c_begin; cb < c_end; cb += sh.chunk) {
-    const int cs = min(sh.chunk, c_end - cb);
+  const bool dense = CELLS == 8 && dense_applies<CELLS>(sh, p);   // (the set-up has built the matrices)
+  // (fp16 only: weight products rounded to bf16's 8 bits would cost the output half its tolerance)
+  if constexpr (CELLS == 8 && std::is_same<T, __half>::value) {
+    // The staging addresses a block's channels with 32-bit byte offsets and reads box rows as 8-byte
+    // pieces that may reach up to three voxels past the row: the buffer range ends with the tensor
+    // (or 64 channels after the block), and a box whose last piece would cross that end takes the
+    // plain path below.
+    const int nxp = (nx + 3) & ~3;
+    const long es = sizeof(T), near = (c_end - c_begin + 64) * plane * es;
+    const long left = (static_cast<long>(p.N - sh.g.batch) * p.C - c_begin) * plane * es;
+    const long last = ((c_end - c_begin - 1) * plane + (static_cast<long>(tz.box_hi) * p.H + ty.box_hi) * p.W + tx.box_lo + nxp) * es;
+    const int kp = (ny * nxp + 31) / 32 * 32;
+    const bool room = 64 * (kp + 8) * es + 16 * 4 * (32 + 8) * es <= kPoolLdsBytes;   // weights + the smallest box chunk
+    if (dense && ny * nxp <= kMfmaYx && room && near < (1L << 31) && last <= left) {
+      pool_forward_mfma<T>(src, dst, p, sh, wd, lds, c_end - c_begin, min(near, left));
+      return;
+    }
+  }
+  for (int cb = c_begin; cb < c_end; cb += plan.chunk) {
+    const int cs = min(plan.chunk, c_end - cb);
     T *box = reinterpret_cast<T *>(lds);                                            // [cs][nz][ny][nx]
     float *t1 = reinterpret_cast<float *>(lds + ((static_cast<size_t>(cs) * vol * sizeof(T) + 15) / 16) * 16);  // [cs][nz][ny][ow]
     float *t2 = t1 + cs * nz * ny * p.ow;                                           // [cs][nz][oh][ow]
@@ -397,8 +703,8 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
   const unsigned n = blockIdx.x;
   const int c_begin = blockIdx.y * channels_per_block, c_end = min(c_begin + channels_per_block, p.C);
   // intermediates are fp32 here, so size the chunk with 4-byte box elements
-  pool_setup(sh, rois + static_cast<long>(n) * roi_columns(p.ndim, 0), p, sizeof(float));
-  if (sh.staged < 0) return;
+  const PoolPlan plan = pool_setup<RT, CELLS>(sh, rois + static_cast<long>(n) * roi_columns(p.ndim, 0), p, sizeof(float), true, nullptr);
+  if (plan.staged < 0) return;
   const int cells = p.od * p.oh * p.ow;
   const long plane = static_cast<long>(p.D) * p.H * p.W;
   const T *src = gout + (static_cast<long>(n) * p.C + c_begin) * cells;
@@ -408,9 +714,9 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
   // holds kPoolEntries + 4 indices: a box wider than that on any axis (few cells spread over many
   // voxels) takes the per-output scatter, like a box that does not fit LDS.
   bool wide = false;
-  if (sh.staged == 1)
+  if (plan.staged == 1)
     for (int a = 0; a < 3; a++) wide = wide || sh.ax[a].box_hi - sh.ax[a].box_lo + 1 > kPoolEntries + 2;
-  if (sh.staged == 0 || wide) {  // per-output scatter
+  if (plan.staged == 0 || wide) {  // per-output scatter
     const int total = (c_end - c_begin) * cells;
     const int gz = p.ndim == 3 ? sh.g.grid[2] : 1, gy = sh.g.grid[1], gx = sh.g.grid[0];
     for (int i = threadIdx.x; i < total; i += kPoolThreads) {
@@ -445,8 +751,8 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
   if (dense_applies<CELLS>(sh, p)) {
     dense_build<CELLS>(sh, p, wd);
     const float inv_ow = 1.f / p.ow;
-    for (int cb = c_begin; cb < c_end; cb += sh.chunk) {
-      const int cs = min(sh.chunk, c_end - cb);
+    for (int cb = c_begin; cb < c_end; cb += plan.chunk) {
+      const int cs = min(plan.chunk, c_end - cb);
       float *t2 = reinterpret_cast<float *>(lds);      // [cs][nz][oh][ow]
       float *t1 = t2 + cs * nz * ohw;                  // [cs][nz][ny][ow]; CL: [nz][ny][cs][ow]
       float *gbox = t1 + cs * nz * ny * p.ow;          // [cs][nz][ny][nx] (planar accumulation only)
@@ -523,8 +829,8 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
     }
     return;
   }
-  for (int cb = c_begin; cb < c_end; cb += sh.chunk) {
-    const int cs = min(sh.chunk, c_end - cb);
+  for (int cb = c_begin; cb < c_end; cb += plan.chunk) {
+    const int cs = min(plan.chunk, c_end - cb);
     float *gbox = reinterpret_cast<float *>(lds);    // [cs][nz][ny][nx]
     float *t1 = gbox + cs * vol;                     // [cs][nz][ny][ow]
     float *t2 = t1 + cs * nz * ny * p.ow;            // [cs][nz][oh][ow]

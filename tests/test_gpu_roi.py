@@ -499,7 +499,14 @@ def test_config5_full_size_properties(ops):
     assert float((const[inside.to(DEV)].float() - 1.5).abs().max()) <= 1.5 * 2 ** -10   # one fp16 rounding of the sum
     x = feat.clone().requires_grad_(True)
     y = mod(x, r)
-    assert_close(mod(feat * 2, r), y.detach() * 2, 1e-6, "linearity")
+    # doubling the features doubles every intermediate exactly, except where an fp16 intermediate of
+    # the matrix-core path is subnormal (fixed spacing 2^-24): that may move a result by one rounding
+    # step, in a tiny share of the outputs
+    twice, dbl = mod(feat * 2, r).float(), y.detach().float() * 2
+    dev = (twice - dbl).abs()
+    assert bool((dev <= 2.0 ** -10 * dbl.abs() + 2.0 ** -23).all())
+    assert float((dev > 0).float().mean()) <= 1e-4
+    del twice, dbl, dev
     gy = torch.randn(y.shape, generator=g).half()
     gy[~inside] = 0
     gy = gy.to(DEV)
