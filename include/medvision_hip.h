@@ -26,7 +26,8 @@
 extern "C" {
 #endif
 
-typedef enum { MV_F32 = 0, MV_F16 = 1, MV_BF16 = 2, MV_F64 = 3 } mv_dtype;
+typedef enum { MV_F32 = 0, MV_F16 = 1, MV_BF16 = 2, MV_F64 = 3,
+               MV_I32 = 4 /* label maps: mv_deform_warp_2d / _3d with order 0 only */ } mv_dtype;
 typedef enum { MV_OK = 0, MV_INVALID_ARGUMENT = 1, MV_HIP_ERROR = 2 } mv_status;
 
 const char *mv_last_error(void);
@@ -188,7 +189,10 @@ int mv_dcn2d_backward(const void *input, const void *offset, const void *mask, c
  * way the reference calls them (ops/cuda_fun_tools.py:94-167: 1x1x1 kernel, identity weight,
  * zero bias): out[b,c,q] = S(img[b,c], q + off[b,:,q]) on the open interval (-1, size), else 0;
  * order 0, 1 or 3 as for the affine engine.
- * img/out [B,C,(D,)H,W], offset [B, 2|3, (D,)H,W] (3-D: 0 = depth, 1 = height, 2 = width).       */
+ * img/out [B,C,(D,)H,W], offset [B, 2|3, (D,)H,W] (3-D: 0 = depth, 1 = height, 2 = width).
+ * dtype MV_I32 (order 0 only): img/out are int32 label maps and offset is float32 -- the voxel the
+ * reference picks after converting the labels to float (aug_cuda/aug_spatial.py:664-668), without
+ * the two conversion passes.                                                                      */
 int mv_deform_warp_2d(const void *img, const void *offset, void *output, int dtype, int batch,
                       int channels, int height, int width, int order, void *stream);
 int mv_deform_warp_3d(const void *img, const void *offset, void *output, int dtype, int batch,

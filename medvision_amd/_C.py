@@ -513,7 +513,10 @@ def deform_warp(img, offset, order=1):
     if not img.is_cuda:
         raise RuntimeError("Not implemented on the CPU")
     img = img.contiguous()
-    offset = offset.to(device=img.device, dtype=img.dtype).contiguous()
+    labels = img.dtype == torch.int32   # label maps: order 0 picks voxels, so they are warped as they are
+    if labels and order != 0:
+        raise RuntimeError("int32 label maps are warped at order 0 only")
+    offset = offset.to(device=img.device, dtype=torch.float32 if labels else img.dtype).contiguous()
     if tuple(offset.shape) != (img.size(0), ndim, *img.shape[2:]):
         raise RuntimeError("offset must have shape [B, %d, *spatial]" % ndim)
     if order not in (0, 1, 3):
@@ -522,6 +525,6 @@ def deform_warp(img, offset, order=1):
     fn = "mv_deform_warp_2d" if ndim == 2 else "mv_deform_warp_3d"
     with _on_device(img):
         _lib.check(getattr(_lib.load(), fn)(
-            _lib.ptr(img), _lib.ptr(offset), _lib.ptr(out), _lib.dtype_code(img), *img.shape,
-            int(order), _lib.stream_of(img)))
+            _lib.ptr(img), _lib.ptr(offset), _lib.ptr(out), _lib.MV_I32 if labels else _lib.dtype_code(img),
+            *img.shape, int(order), _lib.stream_of(img)))
     return out

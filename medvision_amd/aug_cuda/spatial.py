@@ -369,9 +369,13 @@ class CudaRandomElasticDeformation(CudaAugBase):
 
     def elastic_transform(self, image, order=1):
         field = self.dense_field(image.device)
+        fn = apply_offset_2d if self.dim == 2 else apply_offset_3d
+        if order == 0 and image.dtype == torch.int32:
+            # the reference converts labels to float, warps and converts back
+            # (aug_cuda/aug_spatial.py:664-668); the warp takes int32 maps as they are
+            return fn(image.unsqueeze(0), field.unsqueeze(0), order=0).squeeze(0)
         if order == 0:
             image = image.to(self.img_type)
-        fn = apply_offset_2d if self.dim == 2 else apply_offset_3d
         out = fn(image.unsqueeze(0), field.unsqueeze(0).to(image.dtype), order=order).squeeze(0)
         return out.int() if order == 0 else out
 

@@ -922,10 +922,20 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
 
 // Compute units of the current device (workgroups resident at once = units * LDS share).
 
+// One output index of an axis-aligned order-3 tile: the four clamped box indices and weights of its taps
+struct AxisTaps3 {
+  int idx[4];
+  float w[4];
+};
+
 // Order-3 twin of the kernel above, kept simple because 64 taps per voxel dominate everything
 // else: same items, same work distribution and plans (boxes carry a halo of 1 / 2 voxels), but
 // the box is copied to LDS in place (no register prefetch) and every lane walks its column of
 // voxels in a rolled loop, storing as it goes.
+// A roi without rotation (resizes, the control-grid upsampling of the elastic deformation) has
+// separable taps: the tile then contracts x, y and z one after the other through two fp32
+// intermediates in the unused part of the LDS tile (4 + 4 + 4 taps per voxel and less instead of 64),
+// with the same per-axis weights, indices and void rule as the general form.
 template <typename T, int TX, int TY, int TZ, int THREADS, int LDS_BYTES>
 __global__ __launch_bounds__(THREADS, 4) void roi_resample_cubic_kernel(
     const T *__restrict__ feat, const float *__restrict__ rois, T *__restrict__ out, const RoiProblem p,
@@ -997,11 +1007,68 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_cubic_kernel(
         }
       }
     }
+    // separable form: axis-aligned map, box in LDS, room for the intermediates behind it
+    const int first_f = static_cast<int>((static_cast<size_t>(by) * bz * pitch * sizeof(T) + 15) / 16 * 4);
+    float *t1 = reinterpret_cast<float *>(tile) + first_f;   // [bz][by][TX]
+    float *t2 = t1 + bz * by * TX;                           // [bz][TY][TX]
+    AxisTaps3 *tab = reinterpret_cast<AxisTaps3 *>(t2 + bz * TY * TX);   // [3][16]
+    bool sep = false;
+    if (mode == 1 || mode == 3) {
+      const CT *m = plan_map<CT>(rec);
+      sep = m[2] == CT(0) && m[3] == CT(0) && m[5] == CT(0) && m[7] == CT(0) && m[9] == CT(0) && m[10] == CT(0) &&
+            (static_cast<long>(first_f) + bz * by * TX + bz * TY * TX) * 4 + 3 * 16 * static_cast<long>(sizeof(AxisTaps3)) <= LDS_BYTES;
+      if (sep && tid < TX + TY + TZ) {
+        const int a = tid < TX ? 0 : (tid < TX + TY ? 1 : 2), o = tid - (a == 0 ? 0 : (a == 1 ? TX : TX + TY));
+        CT r;
+        if (a == 0) r = m[0] + static_cast<CT>(o) * m[1];
+        else if (a == 1) r = m[4] + static_cast<CT>(o) * m[6];
+        else r = (m[8] + static_cast<CT>(o / ZPL * ZPL) * m[11]) + static_cast<CT>(o % ZPL) * m[11];
+        const int size_a = a == 0 ? W : (a == 1 ? H : D), n_a = a == 0 ? bx : (a == 1 ? by : bz);
+        const CT cmax = static_cast<CT>(size_a - (a == 0 ? lo[0] : (a == 1 ? lo[1] : lo[2])));
+        const int top = max(n_a - 1, 0);
+        const bool ok = r >= CT(-1) && r <= cmax;
+        r = fmax(r, CT(0));
+        const CT l = floor(r);
+        AxisTaps3 e;
+        catmull_rom(static_cast<float>(r - l), e.w);
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+          e.idx[k] = min(max(static_cast<int>(l) - 1 + k, 0), top);
+          if (!ok) e.w[k] = 0.f;
+        }
+        tab[a * 16 + o] = e;
+      }
+    }
     __syncthreads();
     const int ox = plan_scalar(&rec->t0[0]) + lx, oy = plan_scalar(&rec->t0[1]) + ly, zb = plan_scalar(&rec->t0[2]) + lz * ZPL;
     const int count = (ox < ow && oy < oh) ? min(ZPL, od - zb) : 0;
     T *drow = out + (static_cast<long>(plan_scalar(&rec->roi)) * C + c) * od * zstride + (static_cast<long>(zb) * oh + oy) * ow + ox;
-    if (count > 0) {
+    if (sep) {
+      {
+        const AxisTaps3 e = tab[lx];   // (tid % TX == lx)
+        for (int i = tid; i < bz * by * TX; i += THREADS) {
+          const T *row = tile + (i / TX) * pitch;
+          t1[i] = e.w[0] * load(row + e.idx[0]) + e.w[1] * load(row + e.idx[1]) + e.w[2] * load(row + e.idx[2]) +
+                  e.w[3] * load(row + e.idx[3]);
+        }
+      }
+      __syncthreads();
+      {
+        const AxisTaps3 e = tab[16 + ly];   // ((tid / TX) % TY == ly)
+        for (int i = tid; i < bz * TY * TX; i += THREADS) {
+          const float *col = t1 + (i / (TY * TX)) * by * TX + lx;
+          t2[i] = e.w[0] * col[e.idx[0] * TX] + e.w[1] * col[e.idx[1] * TX] + e.w[2] * col[e.idx[2] * TX] +
+                  e.w[3] * col[e.idx[3] * TX];
+        }
+      }
+      __syncthreads();
+      for (int k = 0; k < count; k++) {
+        const AxisTaps3 e = tab[32 + lz * ZPL + k];
+        const float *col = t2 + ly * TX + lx;
+        drow[k * zstride] = store_cast<T>(e.w[0] * col[e.idx[0] * TY * TX] + e.w[1] * col[e.idx[1] * TY * TX] +
+                                          e.w[2] * col[e.idx[2] * TY * TX] + e.w[3] * col[e.idx[3] * TY * TX]);
+      }
+    } else if (count > 0) {
       const CT fx = static_cast<CT>(lx), fy = static_cast<CT>(ly), fz = static_cast<CT>(lz * ZPL);
       CT b[3], st[3];
 #pragma unroll
@@ -1117,6 +1184,26 @@ int roi_forward_tiled(const void *input, const void *rois, void *output, int dty
   if (vox * 4 >= (1L << 31)) return -1;   // 32-bit byte offsets inside one output volume
   const float *r = static_cast<const float *>(rois);
   if (p.order == 3) {
+    // A source of a few hundred voxels per channel (the control grid of the elastic deformation) needs
+    // no 74 KB tile: the instance with a small one keeps twice as many workgroups per compute unit busy.
+    const long rows = static_cast<long>(p.D) * p.H;
+    const long small_f32 = rows * (p.W + 1) * 4 + (rows * 16 + p.D * 256L) * 4 + 3 * 16 * 32;
+    if (small_f32 <= 20 * 1024) {
+      switch (dtype) {
+        case MV_F16:
+          return launch_resample<__half, 16, 16, 8, 512, 20 * 1024, 8, true>(
+              static_cast<const __half *>(input), r, static_cast<__half *>(output), p, workspace, need, s);
+        case MV_BF16:
+          return launch_resample<__hip_bfloat16, 16, 16, 8, 512, 20 * 1024, 8, true>(
+              static_cast<const __hip_bfloat16 *>(input), r, static_cast<__hip_bfloat16 *>(output), p,
+              workspace, need, s);
+        case MV_F32:
+          return launch_resample<float, 16, 16, 8, 512, 20 * 1024, 6, true>(
+              static_cast<const float *>(input), r, static_cast<float *>(output), p, workspace, need, s);
+        default:
+          return -1;
+      }
+    }
     switch (dtype) {
       case MV_F16:
         return launch_resample<__half, 16, 16, 8, 512, 74 * 1024, 8, true>(

@@ -47,6 +47,33 @@ __global__ __launch_bounds__(256) void deform_warp_kernel(const T *__restrict__ 
   }
 }
 
+// Order 0 on int32 label maps with fp32 offsets: the voxel the float path picks (low index when
+// 1 - frac >= 0.5, csrc/cuda/interpolation_helpers_3d.h:186-194), copied as an integer.
+__global__ __launch_bounds__(256) void deform_warp_labels_kernel(const int *__restrict__ img,
+                                                                 const float *__restrict__ off,
+                                                                 int *__restrict__ out, int ndim, int C,
+                                                                 int D, int H, int W) {
+  const long P = static_cast<long>(D) * H * W;
+  const long q = blockIdx.x * 256L + threadIdx.x;
+  const int b = blockIdx.y;
+  if (q >= P) return;
+  const int w = q % W, h = (q / W) % H, d = q / (static_cast<long>(W) * H);
+  const float *o = off + static_cast<long>(b) * ndim * P + q;
+  const double pd = ndim == 3 ? d + static_cast<double>(o[0]) : 0.0;
+  const double ph = h + static_cast<double>(o[(ndim - 2) * P]);
+  const double pw = w + static_cast<double>(o[(ndim - 1) * P]);
+  bool ok = ph > -1.0 && pw > -1.0 && ph < H && pw < W && (ndim == 2 || (pd > -1.0 && pd < D));
+  int z0 = 0, z1 = 0, y0 = 0, y1 = 0, x0 = 0, x1 = 0;
+  float lz = 0.f, ly = 0.f, lx = 0.f;
+  ok = ok && clamped_tap<float>(pd, D, z0, z1, lz, 0) && clamped_tap<float>(ph, H, y0, y1, ly, 0) &&
+       clamped_tap<float>(pw, W, x0, x1, lx, 0);
+  const long at = (static_cast<long>(lz == 0.f ? z0 : z1) * H + (ly == 0.f ? y0 : y1)) * W + (lx == 0.f ? x0 : x1);
+  for (int c = 0; c < C; c++) {
+    const long base = (static_cast<long>(b) * C + c) * P;
+    out[base + q] = ok ? img[base + at] : 0;
+  }
+}
+
 // Order 3 for volumes: 64 taps per sample make the plain kernel above a stream of scattered 2-byte
 // global loads.  Here a workgroup owns a tile of TX x TY x TZ positions (a thread: one column along
 // z), finds the box of source voxels its samples touch (minimum and maximum of floor(p) over the
@@ -193,6 +220,14 @@ static int deform_warp(const void *img, const void *offset, void *output, int dt
   MV_REQUIRE(img && offset && output, "null pointer argument");
   const long P = static_cast<long>(depth) * height * width;
   MV_REQUIRE(P < (1L << 31) && batch <= 65535, "volume too large");
+  if (dtype == MV_I32) {
+    MV_REQUIRE(order == 0, "int32 label maps are warped at order 0 only (got %d)", order);
+    hipLaunchKernelGGL(deform_warp_labels_kernel, dim3(static_cast<unsigned>((P + 255) / 256), batch), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const int *>(img),
+                       static_cast<const float *>(offset), static_cast<int *>(output), ndim, channels, depth,
+                       height, width);
+    return check_launch("deform_warp_labels_kernel");
+  }
   if (order == 3 && ndim == 3 && P >= 4096 && dtype != MV_F64) {
     const int th = (height + 15) / 16;
     const long tzb = static_cast<long>((depth + 7) / 8) * batch;

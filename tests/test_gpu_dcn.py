@@ -387,6 +387,25 @@ def test_2d_packs(ops):
         ops.DeformConv2d(8, 16, 3, 1, 1).to(DEV)(x, torch.zeros(2, 18, 12, 13, device=DEV))
 
 
+def test_warp_int32_labels(ops, oracle):
+    """int32 label maps at order 0: the voxel the float path picks (the reference converts the labels
+    to float, warps and converts back, aug_cuda/aug_spatial.py:664-668), void positions are 0."""
+    g = wl.gen(18)
+    for shape in [(2, 2, 10, 12, 14), (2, 3, 20, 24)]:
+        nd = len(shape) - 2
+        seg = torch.randint(-5, 2 ** 20, shape, generator=g, dtype=torch.int32)
+        off = torch.randn(shape[0], nd, *shape[2:], generator=g) * 3
+        warp = ops.apply_offset_3d if nd == 3 else ops.apply_offset_2d
+        got = warp(seg.to(DEV), off.to(DEV), 0)
+        assert got.dtype == torch.int32
+        want = oracle.deform_warp(seg.double(), off, 0)
+        assert torch.equal(got.cpu().double(), want.double())
+        assert float((want == 0).double().mean()) > 0.01     # positions outside the image
+    with pytest.raises(RuntimeError, match="order 0 only"):
+        ops.apply_offset_3d(torch.zeros(1, 1, 4, 4, 4, dtype=torch.int32, device=DEV),
+                            torch.zeros(1, 3, 4, 4, 4, device=DEV), 1)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("order", [0, 1, 3])
 def test_warp_vs_oracle(ops, oracle, dtype, order):

@@ -270,6 +270,41 @@ def test_cubic_resize_larger_volume(ops, oracle):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("ndim", [3, 2])
+def test_cubic_unrotated_windows(ops, oracle, dtype, ndim):
+    """Order 3 without rotation (the separable form of the tiled kernel): windows that reach beyond
+    the volume on either side (clamped taps, the overshoot up to S and the void beyond), an
+    up-sampling of a tiny control grid as the elastic deformation issues it, and a down-sampling
+    whose boxes leave no room for the intermediates (general form)."""
+    g = wl.gen(61 + ndim)
+    size = (20, 24, 28)[3 - ndim:]
+    vol = torch.randn(2, 3, *size, generator=g).to(dtype)
+    xyz = list(size[::-1])
+    zeros = [0.0] * (2 * ndim - 3)
+    rois = torch.tensor([[0, *[0.3 * s for s in xyz], *[1.2 * s for s in xyz], *zeros],
+                         [1, *[0.8 * s for s in xyz], *[0.9 * s for s in xyz], *zeros],
+                         [1, *[0.5 * s for s in xyz], *[0.25 * s for s in xyz], *zeros]], dtype=torch.float32)
+    out = (32, 40, 48)[3 - ndim:]
+    fn = ops.affine_3d if ndim == 3 else ops.affine_2d
+    got = fn(vol.to(DEV), rois.to(DEV), out, 1.0, 1, True, 3)
+    want = oracle.roi_align_forward(vol, rois, out, 1.0, 1, True, 3, True)
+    assert float((want == 0).float().mean()) > 0.05            # the void is sampled
+    assert_close(got, want, FWD_TOL[dtype], "cubic windows")
+    grid = torch.randn(1, 3, *([8] * ndim), generator=g).to(dtype)
+    groi = torch.tensor([[0, *([4.0] * ndim), *([5.0] * ndim), *zeros]], dtype=torch.float32)
+    big = (64, 64, 80)[3 - ndim:]
+    got = fn(grid.to(DEV), groi.to(DEV), big, 1.0, 1, True, 3)
+    want = oracle.roi_align_forward(grid, groi, big, 1.0, 1, True, 3, True)
+    assert_close(got, want, FWD_TOL[dtype], "control-grid upsampling")
+    if ndim == 3:
+        wide = torch.randn(1, 1, 40, 72, 80, generator=g).to(dtype)
+        wroi = torch.tensor([[0, 40.0, 36.0, 20.0, 80.0, 72.0, 40.0, 0, 0, 0]], dtype=torch.float32)
+        got = fn(wide.to(DEV), wroi.to(DEV), (16, 24, 32), 1.0, 1, True, 3)
+        want = oracle.roi_align_forward(wide, wroi, (16, 24, 32), 1.0, 1, True, 3, True)
+        assert_close(got, want, FWD_TOL[dtype], "cubic down-sampling")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 def test_config5_detection_head_reduced(ops, oracle, dtype):
     """Benchmark configuration 5 shape family (log-uniform extents, scale 0.25, 7^3, sr=2), reduced."""
     g = wl.gen(4)
