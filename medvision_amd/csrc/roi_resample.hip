@@ -1011,12 +1011,14 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_cubic_kernel(
     const int first_f = static_cast<int>((static_cast<size_t>(by) * bz * pitch * sizeof(T) + 15) / 16 * 4);
     float *t1 = reinterpret_cast<float *>(tile) + first_f;   // [bz][by][TX]
     float *t2 = t1 + bz * by * TX;                           // [bz][TY][TX]
-    AxisTaps3 *tab = reinterpret_cast<AxisTaps3 *>(t2 + bz * TY * TX);   // [3][16]
+    constexpr int TS = TZ > 16 ? TZ : 16;                               // table entries per axis
+    static_assert(TX <= TS && TY <= TS, "table entries per axis");
+    AxisTaps3 *tab = reinterpret_cast<AxisTaps3 *>(t2 + bz * TY * TX);   // [3][TS]
     bool sep = false;
     if (mode == 1 || mode == 3) {
       const CT *m = plan_map<CT>(rec);
       sep = m[2] == CT(0) && m[3] == CT(0) && m[5] == CT(0) && m[7] == CT(0) && m[9] == CT(0) && m[10] == CT(0) &&
-            (static_cast<long>(first_f) + bz * by * TX + bz * TY * TX) * 4 + 3 * 16 * static_cast<long>(sizeof(AxisTaps3)) <= LDS_BYTES;
+            (static_cast<long>(first_f) + bz * by * TX + bz * TY * TX) * 4 + 3 * TS * static_cast<long>(sizeof(AxisTaps3)) <= LDS_BYTES;
       if (sep && tid < TX + TY + TZ) {
         const int a = tid < TX ? 0 : (tid < TX + TY ? 1 : 2), o = tid - (a == 0 ? 0 : (a == 1 ? TX : TX + TY));
         CT r;
@@ -1036,7 +1038,7 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_cubic_kernel(
           e.idx[k] = min(max(static_cast<int>(l) - 1 + k, 0), top);
           if (!ok) e.w[k] = 0.f;
         }
-        tab[a * 16 + o] = e;
+        tab[a * TS + o] = e;
       }
     }
     __syncthreads();
@@ -1054,7 +1056,7 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_cubic_kernel(
       }
       __syncthreads();
       {
-        const AxisTaps3 e = tab[16 + ly];   // ((tid / TX) % TY == ly)
+        const AxisTaps3 e = tab[TS + ly];   // ((tid / TX) % TY == ly)
         for (int i = tid; i < bz * TY * TX; i += THREADS) {
           const float *col = t1 + (i / (TY * TX)) * by * TX + lx;
           t2[i] = e.w[0] * col[e.idx[0] * TX] + e.w[1] * col[e.idx[1] * TX] + e.w[2] * col[e.idx[2] * TX] +
@@ -1063,7 +1065,7 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_cubic_kernel(
       }
       __syncthreads();
       for (int k = 0; k < count; k++) {
-        const AxisTaps3 e = tab[32 + lz * ZPL + k];
+        const AxisTaps3 e = tab[2 * TS + lz * ZPL + k];
         const float *col = t2 + ly * TX + lx;
         drow[k * zstride] = store_cast<T>(e.w[0] * col[e.idx[0] * TY * TX] + e.w[1] * col[e.idx[1] * TY * TX] +
                                           e.w[2] * col[e.idx[2] * TY * TX] + e.w[3] * col[e.idx[3] * TY * TX]);
@@ -1187,18 +1189,18 @@ int roi_forward_tiled(const void *input, const void *rois, void *output, int dty
     // A source of a few hundred voxels per channel (the control grid of the elastic deformation) needs
     // no 74 KB tile: the instance with a small one keeps twice as many workgroups per compute unit busy.
     const long rows = static_cast<long>(p.D) * p.H;
-    const long small_f32 = rows * (p.W + 1) * 4 + (rows * 16 + p.D * 256L) * 4 + 3 * 16 * 32;
+    const long small_f32 = rows * (p.W + 1) * 4 + (rows * 16 + p.D * 256L) * 4 + 3 * 32 * 32;
     if (small_f32 <= 20 * 1024) {
       switch (dtype) {
         case MV_F16:
-          return launch_resample<__half, 16, 16, 8, 512, 20 * 1024, 8, true>(
+          return launch_resample<__half, 16, 16, 32, 512, 20 * 1024, 8, true>(
               static_cast<const __half *>(input), r, static_cast<__half *>(output), p, workspace, need, s);
         case MV_BF16:
-          return launch_resample<__hip_bfloat16, 16, 16, 8, 512, 20 * 1024, 8, true>(
+          return launch_resample<__hip_bfloat16, 16, 16, 32, 512, 20 * 1024, 8, true>(
               static_cast<const __hip_bfloat16 *>(input), r, static_cast<__hip_bfloat16 *>(output), p,
               workspace, need, s);
         case MV_F32:
-          return launch_resample<float, 16, 16, 8, 512, 20 * 1024, 6, true>(
+          return launch_resample<float, 16, 16, 32, 512, 20 * 1024, 6, true>(
               static_cast<const float *>(input), r, static_cast<float *>(output), p, workspace, need, s);
         default:
           return -1;
