@@ -91,10 +91,10 @@ constexpr int kDenseSrc = 32;   // source voxels per axis of the dense weight ma
 // `wd` is given and the axis fits, the dense weight matrix wd[a][source index][cell] = sum of the
 // weights of the cell's samples that touch the source index (samples in their order; a wavefront's
 // LDS operations execute in order).  The fourth wavefront writes the whole geometry for the plain
-// gather / scatter paths.  One barrier (two with `with_first`, the entry ranges per source index).
+// gather / scatter paths.  One barrier.
 template <typename RT, int CELLS>
 __device__ inline PoolPlan pool_setup(PoolShared &sh, const RT *roi, const RoiProblem &p, size_t elem_bytes,
-                                      bool with_first, float (*wd)[kDenseSrc][CELLS]) {
+                                      float (*wd)[kDenseSrc][CELLS]) {
   const int nd = p.ndim;
   const int cells[3] = {p.ow, p.oh, p.od};
   const int size[3] = {p.W, p.H, p.D};
@@ -188,8 +188,12 @@ __device__ inline PoolPlan pool_setup(PoolShared &sh, const RT *roi, const RoiPr
     if (chunk < 1) plan.staged = 0;
     plan.chunk = static_cast<int>(min(chunk, 64L));
   }
-  if (plan.staged != 1 || !with_first) return plan;
-  for (int e = threadIdx.x; e < 3 * (kPoolEntries + 4); e += kPoolThreads) {  // entry ranges per source index
+  return plan;
+}
+
+// The entry ranges per source index (`first`) of a staged roi; all threads, ends with a barrier.
+__device__ inline void pool_first(PoolShared &sh) {
+  for (int e = threadIdx.x; e < 3 * (kPoolEntries + 4); e += kPoolThreads) {
     const int k = e / (kPoolEntries + 4), j = e % (kPoolEntries + 4);
     AxisTaps &t = sh.ax[k];
     if (j > t.box_hi - t.box_lo + 1) continue;
@@ -198,7 +202,6 @@ __device__ inline PoolPlan pool_setup(PoolShared &sh, const RT *roi, const RoiPr
     t.first[j] = f;
   }
   __syncthreads();
-  return plan;
 }
 
 // Dense form of the tap tables for the usual small boxes (<= CELLS cells per axis, box of
@@ -494,7 +497,7 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
   const unsigned n = blockIdx.x;
   const int c_begin = blockIdx.y * channels_per_block, c_end = min(c_begin + channels_per_block, p.C);
   __shared__ __attribute__((aligned(16))) float wd[3][kDenseSrc][CELLS];
-  const PoolPlan plan = pool_setup<RT, CELLS>(sh, rois + static_cast<long>(n) * roi_columns(p.ndim, 0), p, sizeof(T), false,
+  const PoolPlan plan = pool_setup<RT, CELLS>(sh, rois + static_cast<long>(n) * roi_columns(p.ndim, 0), p, sizeof(T),
                                               CELLS == 8 ? wd : nullptr);
   const int cells = p.od * p.oh * p.ow;
   const long plane = static_cast<long>(p.D) * p.H * p.W;
@@ -690,6 +693,124 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
   }
 }
 
+// Backward pass of one (roi, channel block) on the matrix cores: fp16 gradients, <= 8 cells per
+// axis, channels-last fp32 accumulation buffer.  Per 16 channels and box slice z,
+//     dBox[(y, x)][channel] = sum_(ph, pw) (Wy[y][ph] Wx[x][pw]) * U_z[(ph, pw)][channel],
+//     U_z[(ph, pw)][channel] = sum_pd Wz[z][pd] * gout[channel][pd][(ph, pw)],
+// with the weight products in LDS (rows (y, x) as in the forward pass: box rows padded to a multiple of
+// four columns) and U_z formed by every lane in registers straight from its 16-byte loads of the
+// gradient, already in the layout of the right-hand operand (column = channel, K = cell).  The
+// accumulator then holds, per lane, four neighbouring voxels of one box row for one channel: lanes
+// 0..15 are 16 neighbouring channels of the channels-last buffer, so an atomic instruction adds runs
+// of 64 contiguous bytes.  Wavefronts work on different channel blocks and share nothing but the
+// weights: no barrier after the set-up.
+constexpr int kPoolBwdRow = 72;   // fp16 elements per row of the transposed weights: 64 cells + pad
+template <typename T>
+__device__ inline void pool_backward_mfma(const T *__restrict__ src_any, float *__restrict__ dst_any, const RoiProblem &p,
+                                          const PoolShared &sh, const float (&wd)[3][kDenseSrc][8],
+                                          unsigned char *lds, int c_count) {
+  using M = Mfma<T>;
+  auto uni = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
+  const int nx = uni(sh.ax[0].box_hi - sh.ax[0].box_lo + 1), ny = uni(sh.ax[1].box_hi - sh.ax[1].box_lo + 1),
+            nz = uni(sh.ax[2].box_hi - sh.ax[2].box_lo + 1);
+  const int x_lo = uni(sh.ax[0].box_lo), y_lo = uni(sh.ax[1].box_lo), z_lo = uni(sh.ax[2].box_lo);
+  const int NXP = (nx + 3) & ~3, QX = NXP / 4, KT = (ny * NXP + 15) / 16;
+  const int ohw = p.oh * p.ow, cells = p.od * ohw;
+  const int KS = ohw > 32 ? 2 : 1;                    // K steps of 32 cells
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int col = lane % 16, quad = lane / 16;
+  T *wt = reinterpret_cast<T *>(lds);                 // [KT * 16 rows (y, x)][kPoolBwdRow]
+  {  // weight products: thread = (row of the pass, quarter of the cells)
+    const float inv_ow = 1.f / p.ow, inv_nxp = 1.f / NXP;
+    const int q = tid % 4;
+    float wxy[2][16];   // not kept: the cells' (ph, pw) are the same for every row
+    int phs[16], pws[16];
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+      const int n = q * 16 + j;
+      phs[j] = fdiv(n, inv_ow);
+      pws[j] = n - phs[j] * p.ow;
+      if (n >= ohw) { phs[j] = -1; pws[j] = 0; }
+    }
+    (void)wxy;
+    for (int k = tid / 4; k < KT * 16; k += kPoolThreads / 4) {
+      const int y = fdiv(k, inv_nxp), x = k - y * NXP;
+      const bool kv = y < ny && x < nx;
+      const float *wy = wd[1][kv ? y : 0], *wx = wd[0][kv ? x : 0];
+      unsigned packed[8];
+#pragma unroll
+      for (int j = 0; j < 16; j += 2) {
+        const float a = (kv && phs[j] >= 0) ? wy[phs[j]] * wx[pws[j]] : 0.f;
+        const float b = (kv && phs[j + 1] >= 0) ? wy[phs[j + 1]] * wx[pws[j + 1]] : 0.f;
+        packed[j / 2] = M::pack2(a, b);
+      }
+      u32x4 *row = reinterpret_cast<u32x4 *>(wt + k * kPoolBwdRow + q * 16);
+      row[0] = u32x4{packed[0], packed[1], packed[2], packed[3]};
+      row[1] = u32x4{packed[4], packed[5], packed[6], packed[7]};
+    }
+  }
+  __syncthreads();
+  auto uni_ptr = [&](const void *ptr) {
+    const unsigned long long v = reinterpret_cast<unsigned long long>(ptr);
+    return static_cast<unsigned long long>(static_cast<unsigned>(uni(static_cast<int>(v)))) |
+           static_cast<unsigned long long>(static_cast<unsigned>(uni(static_cast<int>(v >> 32)))) << 32;
+  };
+  const T *src = reinterpret_cast<const T *>(uni_ptr(src_any));
+  float *dst = reinterpret_cast<float *>(uni_ptr(dst_any));
+  // this roi's gradient rows of the block; reads beyond the block's channels return zeros
+  const __amdgpu_buffer_rsrc_t gr = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T *>(src), 0, c_count * cells * 2 + 16, 0x00020000);
+  const int blocks = (c_count + 15) / 16;
+  for (int blk = wave; blk < blocks; blk += kPoolThreads / kWave) {
+    const int c = blk * 16 + col;
+    const bool cv = c < c_count;
+    // the lane's gradient pieces: cells quad * 8 .. + 7 (+ 32) of every pd of its channel
+    u32x4 g[8][2];
+    const unsigned g0 = cv ? static_cast<unsigned>(c * cells + quad * 8) * 2u : 0x80000000u;
+#pragma unroll
+    for (int pd = 0; pd < 8; pd++)
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++) {
+        g[pd][ks] = u32x4{0u, 0u, 0u, 0u};
+        if (pd < p.od && ks * 32 + quad * 8 < ohw)
+          g[pd][ks] = __builtin_amdgcn_raw_buffer_load_b128(gr, g0, (pd * ohw + ks * 32) * 2, 0);
+      }
+    for (int z = 0; z < nz; z++) {
+      float wz[8];
+      {
+        const float4 lo4 = *reinterpret_cast<const float4 *>(&wd[2][z][0]), hi4 = *reinterpret_cast<const float4 *>(&wd[2][z][4]);
+        wz[0] = lo4.x; wz[1] = lo4.y; wz[2] = lo4.z; wz[3] = lo4.w; wz[4] = hi4.x; wz[5] = hi4.y; wz[6] = hi4.z; wz[7] = hi4.w;
+      }
+      u32x4 bop[2];
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++) {
+        float u[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (ks < KS) {
+#pragma unroll
+          for (int pd = 0; pd < 8; pd++)
+            if (pd < p.od) M::fma_piece(u, wz[pd], g[pd][ks]);
+        }
+        bop[ks] = M::pack(u);
+      }
+      const unsigned slice = static_cast<unsigned>((z_lo + z) * p.H + y_lo) * p.W + x_lo;   // voxel index of the slice's box corner
+      for (int kt = 0; kt < KT; kt++) {
+        float4_t acc = float4_t{0.f, 0.f, 0.f, 0.f};
+        const T *arow = wt + (kt * 16 + col) * kPoolBwdRow + quad * 8;
+        acc = M::run16(*reinterpret_cast<const u32x4 *>(arow), bop[0], acc);
+        if (KS == 2) acc = M::run16(*reinterpret_cast<const u32x4 *>(arow + 32), bop[1], acc);
+        // rows 4 * quad .. + 3 of the tile = piece m of the padded box rows: four neighbouring x
+        const int m = kt * 4 + quad, y = m / QX, x0 = (m - y * QX) * 4;
+        if (cv && y < ny) {
+          float *at = dst + (static_cast<size_t>(slice + static_cast<unsigned>(y * p.W + x0)) * p.C + c);
+#pragma unroll
+          for (int r = 0; r < 4; r++)
+            if (x0 + r < nx && acc[r] != 0.f) atomic_add(at + static_cast<size_t>(r) * p.C, acc[r]);
+        }
+      }
+    }
+  }
+}
+
 // G = element type of the accumulation buffer (T for fp32, float for 16-bit T).
 // CL: the accumulation buffer is channels-last [N, D*H*W, C] (the fp32 workspace of the 16-bit
 // path): the lanes of a wavefront then add neighbouring channels of a voxel, contiguous bytes,
@@ -703,7 +824,8 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
   const unsigned n = blockIdx.x;
   const int c_begin = blockIdx.y * channels_per_block, c_end = min(c_begin + channels_per_block, p.C);
   // intermediates are fp32 here, so size the chunk with 4-byte box elements
-  const PoolPlan plan = pool_setup<RT, CELLS>(sh, rois + static_cast<long>(n) * roi_columns(p.ndim, 0), p, sizeof(float), true, nullptr);
+  __shared__ __attribute__((aligned(16))) float wd[3][kDenseSrc][CELLS];
+  const PoolPlan plan = pool_setup<RT, CELLS>(sh, rois + static_cast<long>(n) * roi_columns(p.ndim, 0), p, sizeof(float), wd);
   if (plan.staged < 0) return;
   const int cells = p.od * p.oh * p.ow;
   const long plane = static_cast<long>(p.D) * p.H * p.W;
@@ -747,9 +869,20 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
   const float inv_vol = 1.f / vol, inv_nxy = 1.f / (nx * ny), inv_nx = 1.f / nx, inv_ow = 1.f / p.ow,
               inv_ohw = 1.f / ohw, inv_nzohw = 1.f / (nz * ohw), inv_nyow = 1.f / (ny * p.ow),
               inv_gx = 1.f / gx, inv_gy = 1.f / gy, inv_gz = 1.f / gz;
-  __shared__ __attribute__((aligned(16))) float wd[3][kDenseSrc][CELLS];
-  if (dense_applies<CELLS>(sh, p)) {
-    dense_build<CELLS>(sh, p, wd);
+  if (dense_applies<CELLS>(sh, p)) {   // (the set-up has built the matrices)
+    if constexpr (CL && CELLS == 8 && std::is_same<T, __half>::value && std::is_same<G, float>::value) {
+      // matrix-core form: 32-bit offsets into the image's accumulation buffer and into this roi's
+      // gradient; its 16-byte loads may reach 14 bytes past a row of cells, so the roi whose rows end
+      // the tensor stays with the form below
+      const int nxp = (nx + 3) & ~3, kt = (ny * nxp + 15) / 16;
+      const bool fits = ny * nxp <= kMfmaYx && kt * 16 * kPoolBwdRow * 2 <= kPoolLdsBytes;
+      const bool small = plane * p.C * 4 < (1L << 32) && static_cast<long>(c_end - c_begin) * cells * 2 + 64 < (1L << 31);
+      const bool last = n + 1 == static_cast<unsigned>(p.R) && c_end == p.C;
+      if (fits && small && !last) {
+        pool_backward_mfma(src, dst_cl, p, sh, wd, lds, c_end - c_begin);
+        return;
+      }
+    }
     const float inv_ow = 1.f / p.ow;
     for (int cb = c_begin; cb < c_end; cb += plan.chunk) {
       const int cs = min(plan.chunk, c_end - cb);
@@ -829,6 +962,7 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
     }
     return;
   }
+  pool_first(sh);
   for (int cb = c_begin; cb < c_end; cb += plan.chunk) {
     const int cs = min(plan.chunk, c_end - cb);
     float *gbox = reinterpret_cast<float *>(lds);    // [cs][nz][ny][nx]
