@@ -250,19 +250,22 @@ __device__ __forceinline__ void dense_axpy(float (&acc)[CELLS], const float *row
 // box rows times padded box columns <= kMfmaYx.  The contraction over (y, x) is one GEMM per group
 // of four box slices,
 //     T[(channel, slice)][(ph, pw)] = sum_(y, x) box[(channel, slice)][(y, x)] * (Wy[y][ph] Wx[x][pw]),
-// with the box chunk and the weight products in LDS as 16-byte K pieces; K = y * NXP + x with the
-// box row padded to NXP = a multiple of four columns (zero weights on the pad), so that a box row is
-// staged as 8-byte pieces: one 2-byte-aligned buffer load and one LDS store per four voxels.  The
-// per-lane offset (channel within the pass, slice, y, x piece) stays fixed while the channel moves
-// through the scalar offset: no index arithmetic per element, and slices or channels outside the box
-// or the block read zeros through the range check.
-// Rows are ordered (channel, slice % 4), so the 16 x 16 accumulator hands every lane the four slices
-// of ONE channel at one (ph, pw): for two slice groups that is exactly the 8-element K piece of a
-// second matrix product with rows (ph, pw), K = (channel, slice) and a block-diagonal right-hand side
+// K = y * NXP + x with the box row padded to NXP = a multiple of four columns (zero weights on the
+// pad).  The weight products sit in LDS as 16-byte K pieces; the box does not: a lane's 8-element K
+// piece of the left operand is two 4-voxel pieces of a box row, which it reads straight from the
+// feature map with two 2-byte-aligned 8-byte buffer loads (per-lane offset = (channel, slice) of its
+// row plus the pieces of the K step, the tile's channels in the scalar offset; slices or channels
+// outside the box or the block read zeros through the range check, columns beyond the box row are
+// masked).  Rows are ordered (channel, slice % 4), so the 16 x 16 accumulator hands every lane the
+// four slices of ONE channel at one (ph, pw): for two slice groups that is exactly the 8-element K
+// piece of a second matrix product with rows (ph, pw), K = (channel, slice) and a block-diagonal
+// right-hand side
 //     out[(ph, pw)][(channel', pd)] = sum_(channel, z) T[(ph, pw)][(channel, z)] * (channel == channel') Wz[z][pd],
 // whose pieces every lane forms from the z matrix by itself (as an fp16 pair high + low, so the z
 // weights keep 22 bits).  The contraction over z thereby runs on the matrix cores too, without moving
 // T (it is rounded to fp16 once); a lane ends up with four neighbouring cells of one (channel, pd).
+// A wavefront owns tiles of four channels and shares nothing but the weights with the others: no
+// barrier after the set-up.
 constexpr int kMfmaYx = 224;
 template <typename T>
 __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__restrict__ dst, const RoiProblem &p,
@@ -275,28 +278,15 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
   const int nx = uni(sh.ax[0].box_hi - sh.ax[0].box_lo + 1), ny = uni(sh.ax[1].box_hi - sh.ax[1].box_lo + 1),
             nz = uni(sh.ax[2].box_hi - sh.ax[2].box_lo + 1);
   const int x_lo = uni(sh.ax[0].box_lo), y_lo = uni(sh.ax[1].box_lo), z_lo = uni(sh.ax[2].box_lo);
-  const int NXP = (nx + 3) & ~3, pieces = ny * NXP / 4;              // 8-byte pieces of one box slice
+  const int NXP = (nx + 3) & ~3, QX = NXP / 4, pieces = ny * QX;     // 8-byte pieces of one box slice
   const int KP = (ny * NXP + 31) / 32 * 32, WS = KP + 8;             // weight rows: KP products + a pad against bank conflicts
-  int KC = min(KP, 96);                                              // box rows: one K chunk
-  while (64 * WS * ES + 16 * 4 * (KC + 8) * ES > kPoolLdsBytes) KC -= 32;
-  const int RS = KC + 8;
   const int ohw = p.oh * p.ow, cells = p.od * ohw;
   const long plane = static_cast<long>(p.D) * p.H * p.W;
   const int hw = p.H * p.W;
   T *w = reinterpret_cast<T *>(lds);            // [64 cells (ph, pw)][WS]
-  T *box = w + 64 * WS;                         // [CH channels][4 * ZS slices][RS]
-  // groups of four slices staged at once (the whole box for the usual small ones; one group when the
-  // box needs several K chunks, whose products accumulate in the same registers)
   const int zgroups = (nz + 3) / 4;
-  const int fit = (kPoolLdsBytes - 64 * WS * ES) / (16 * 4 * RS * ES);
-  const int ZS = KP > KC ? 1 : max(1, min(min(zgroups, fit), 2));
-  const int ZS4 = ZS * 4;
-  const bool one_stage = zgroups <= ZS && KP <= KC;   // the usual case: the whole box in one stage
-  // channels per stage: up to four blocks of 16 when the whole box fits (fewer, longer stages: every
-  // stage costs two barriers and one round trip to memory)
-  const int CH = 16 * (one_stage ? max(1, min(min(4, fit / ZS), (c_count + 15) / 16)) : 1);
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
-  const float inv_ow = 1.f / p.ow, inv_nxp = 1.f / NXP;
+  const float inv_ow = 1.f / p.ow, inv_nxp = 1.f / NXP, inv_qx = 1.f / QX;
   {  // weight products: thread = (cell, quarter of the K range), pairs of neighbouring K
     const int n = tid / 4, q = tid % 4, ph = fdiv(n, inv_ow), pw = n - ph * p.ow;
     const bool nv = n < ohw;
@@ -314,35 +304,29 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
       *reinterpret_cast<unsigned *>(wr + i) = M::pack2(v[0], v[1]);
     }
   }
-  // the box rows start out as zeros: the staging never writes K positions beyond the last piece
-  for (int i = tid; i < CH * ZS4 * RS / 2; i += kPoolThreads) reinterpret_cast<unsigned *>(box)[i] = 0u;
+  __syncthreads();
   const int col = lane % 16, quad = lane / 16;
-  // staging: an item is (channel of the pass, slice, piece); a thread keeps its item while the passes
-  // walk over the channels
-  const int QV = min(KC / 4, pieces), ipc = ZS4 * QV, cpp = min(CH, kPoolThreads / ipc), passes = (CH + cpp - 1) / cpp;
-  const float inv_ipc = 1.f / ipc, inv_qv = 1.f / QV;
-  const int c_sub = fdiv(tid, inv_ipc), rem = tid - c_sub * ipc, zslot = fdiv(rem, inv_qv), ql = rem - zslot * QV;
-  const bool item = c_sub < cpp;
   const unsigned long long sp = reinterpret_cast<unsigned long long>(src_any);
-  const T *src = reinterpret_cast<const T *>(static_cast<unsigned long long>(uni(static_cast<int>(sp))) & 0xffffffffull |
-                                             static_cast<unsigned long long>(uni(static_cast<int>(sp >> 32))) << 32);
+  const T *src = reinterpret_cast<const T *>(static_cast<unsigned long long>(static_cast<unsigned>(uni(static_cast<int>(sp)))) |
+                                             static_cast<unsigned long long>(static_cast<unsigned>(uni(static_cast<int>(sp >> 32)))) << 32);
   const __amdgpu_buffer_rsrc_t fr = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<T *>(src), 0, static_cast<int>(range_bytes), 0x00020000);
-  const unsigned corner = static_cast<unsigned>(((static_cast<long>(z_lo) * p.H + y_lo) * p.W + x_lo) * ES);
   const int plane_bytes = static_cast<int>(plane) * ES;
   constexpr unsigned kNowhere = 0x80000000u;
-  unsigned voff, keep_lo, keep_hi;   // the item's byte offset; masks that clear the columns beyond the box row
-  auto item_offset = [&](int zg, int kc) {
-    const int z = zg * 4 + zslot, q = kc / 4 + ql, y = fdiv(q * 4, inv_nxp), x0 = q * 4 - y * NXP;
-    const bool ok = item && z < nz && q < pieces;
-    voff = ok ? corner + static_cast<unsigned>(c_sub * plane_bytes + (z * hw + y * p.W + x0) * ES) : kNowhere;
-    const int left = nx - x0;   // >= 1 for a piece of the row
-    keep_lo = left >= 2 ? 0xffffffffu : 0x0000ffffu;
-    keep_hi = left >= 4 ? 0xffffffffu : (left == 3 ? 0x0000ffffu : 0u);
+  // this lane's row of the left operand: channel col / 4 of the tile, slice col % 4 of the group
+  const unsigned row_off = static_cast<unsigned>(((static_cast<long>(z_lo + col % 4) * p.H + y_lo) * p.W + x_lo) * ES) +
+                           static_cast<unsigned>(col / 4) * static_cast<unsigned>(plane_bytes);
+  // the two pieces of the lane's K positions in step ks: byte offset inside the slice and the masks
+  // that clear the columns beyond the box row
+  struct Piece { unsigned off, keep_lo, keep_hi; };
+  auto piece = [&](int m) {
+    const int y = fdiv(m, inv_qx), x0 = (m - y * QX) * 4, left = nx - x0;
+    Piece e;
+    e.off = m < pieces ? static_cast<unsigned>((y * p.W + x0) * ES) : kNowhere;
+    e.keep_lo = left >= 2 ? 0xffffffffu : 0x0000ffffu;
+    e.keep_hi = left >= 4 ? 0xffffffffu : (left == 3 ? 0x0000ffffu : 0u);
+    return e;
   };
-  item_offset(0, 0);
-  T *box_item = box + (c_sub * ZS4 + zslot) * RS + ql * 4;
-  const int pass_elems = cpp * ZS4 * RS;
   // right-hand side of the z product for the stage that starts with slice group zg: column n = 16 h + col
   // is (channel' = n / 8, pd = n % 8); this lane's K group is channel `quad`, slices 4 zg .. 4 zg + 7
   auto z_pieces = [&](int zg, u32x4 (&zhi)[2], u32x4 (&zlo)[2]) {
@@ -354,7 +338,7 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
 #pragma unroll
       for (int i = 0; i < 8; i++) {
         const int z = zg * 4 + i;
-        zw[i] = (mine && i < ZS4 && z < nz) ? wd[2][z < kDenseSrc ? z : 0][pd] : 0.f;
+        zw[i] = (mine && z < nz) ? wd[2][z < kDenseSrc ? z : 0][pd] : 0.f;
       }
       zhi[h] = M::pack(zw);
       zr[0] = zw[0] - M::lo(zhi[h].x); zr[1] = zw[1] - M::hi(zhi[h].x);
@@ -366,125 +350,108 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
   };
   u32x4 zhi0[2], zlo0[2];
   z_pieces(0, zhi0, zlo0);
-  // box rows of channels cb .. cb + CH - 1 for the stage (zg, kc): up to eight passes of loads in
-  // flight together; between two barriers
-  auto stage = [&](int cb) {
-    for (int ps0 = 0; ps0 < passes; ps0 += 8) {
-      u32x2 val[8];
+  // The steps (tile, slice-group pair, K step of 32) of this wavefront form one sequence; the loads
+  // of a step are issued one step ahead, so they are in flight during the previous step's products
+  // and stores.
+  const int tiles = (c_count + 3) / 4;
+  struct Step { int tile, zg, k0; };
+  struct Loaded { u32x2 va[2], vb[2]; Piece pa, pb; };
+  auto next_of = [&](Step st) {
+    st.k0 += 32;
+    if (st.k0 >= KP) {
+      st.k0 = 0; st.zg += 2;
+      if (st.zg >= zgroups) { st.zg = 0; st.tile += kPoolThreads / kWave; }
+    }
+    return st;
+  };
+  auto issue = [&](const Step &st, Loaded &ld) {
+    // rows whose slice lies outside the box read zeros
+    const unsigned row0 = st.zg * 4 + col % 4 < nz ? row_off : kNowhere;
+    const unsigned row1 = st.zg * 4 + 4 + col % 4 < nz ? row_off : kNowhere;
+    const int soff = st.tile * 4 * plane_bytes + st.zg * 4 * hw * ES;
+    ld.pa = piece(st.k0 / 4 + quad * 2);
+    ld.pb = piece(st.k0 / 4 + quad * 2 + 1);
 #pragma unroll
-      for (int u = 0; u < 8; u++) {
-        val[u] = u32x2{0u, 0u};
-        if (ps0 + u < passes)
-          val[u] = __builtin_amdgcn_raw_buffer_load_b64(fr, voff, (cb + (ps0 + u) * cpp) * plane_bytes, 0);
-      }
-#pragma unroll
-      for (int u = 0; u < 8; u++) {
-        if (ps0 + u < passes && item && (ps0 + u) * cpp + c_sub < CH) {
-          uint2 v2;
-          v2.x = val[u].x & keep_lo;
-          v2.y = val[u].y & keep_hi;
-          *reinterpret_cast<uint2 *>(box_item + (ps0 + u) * pass_elems) = v2;
-        }
-      }
+    for (int zs = 0; zs < 2; zs++) {
+      const unsigned row = zs == 0 ? row0 : row1;
+      // (an offset with the top bit set is beyond the range, whatever the other term adds)
+      ld.va[zs] = __builtin_amdgcn_raw_buffer_load_b64(fr, (row + ld.pa.off) | ((row | ld.pa.off) & kNowhere), soff + zs * 4 * hw * ES, 0);
+      ld.vb[zs] = __builtin_amdgcn_raw_buffer_load_b64(fr, (row + ld.pb.off) | ((row | ld.pb.off) & kNowhere), soff + zs * 4 * hw * ES, 0);
     }
   };
-  // this wavefront: channels 4 * wave .. + 3 of the 16-channel block sb, rows (channel, slice % 4) of
-  // every staged slice group, K chunk kc
-  auto first_product = [&](int sb, int kc, float4_t (&acc)[2][4]) {
-    for (int k0 = 0; k0 < KC && kc + k0 < KP; k0 += 32) {
+  Step cur{wave, 0, 0};
+  Loaded ld;
+  if (cur.tile < tiles) issue(cur, ld);
+  float4_t oacc[4][2];   // [cell tile][half of the (channel', pd) columns]: cells 4 * quad .. + 3 of the tile
+  float4_t acc[2][4];    // [slice group][cell tile]
+  while (cur.tile < tiles) {
+    const Step nxt = next_of(cur);
+    Loaded ahead;
+    if (nxt.tile < tiles) issue(nxt, ahead);
+    if (cur.k0 == 0) {
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        acc[i / 4][i % 4] = float4_t{0.f, 0.f, 0.f, 0.f};
+        if (cur.zg == 0) oacc[i / 2][i % 2] = float4_t{0.f, 0.f, 0.f, 0.f};
+      }
+    }
+    {
       u32x4 b[4];
 #pragma unroll
       for (int nt = 0; nt < 4; nt++)
-        b[nt] = *reinterpret_cast<const u32x4 *>(w + (nt * 16 + col) * WS + kc + k0 + quad * 8);
+        b[nt] = *reinterpret_cast<const u32x4 *>(w + (nt * 16 + col) * WS + cur.k0 + quad * 8);
 #pragma unroll
       for (int zs = 0; zs < 2; zs++) {
-        if (zs < ZS) {
-          const int c_local = sb * 16 + wave * 4 + col / 4, zrow = zs * 4 + col % 4;
-          const u32x4 a = *reinterpret_cast<const u32x4 *>(box + (c_local * ZS4 + zrow) * RS + k0 + quad * 8);
+        if (cur.zg + zs < zgroups) {
+          const u32x4 a = u32x4{ld.va[zs].x & ld.pa.keep_lo, ld.va[zs].y & ld.pa.keep_hi,
+                                ld.vb[zs].x & ld.pb.keep_lo, ld.vb[zs].y & ld.pb.keep_hi};
 #pragma unroll
           for (int nt = 0; nt < 4; nt++) acc[zs][nt] = M::run16(a, b[nt], acc[zs][nt]);
         }
       }
     }
-  };
-  // contraction over the (up to eight) slices of a stage
-  auto second_product = [&](const float4_t (&acc)[2][4], const u32x4 (&zhi)[2], const u32x4 (&zlo)[2], float4_t (&oacc)[4][2]) {
+    if (cur.k0 + 32 >= KP) {
+      // contraction over the (up to eight) slices of the two groups
+      u32x4 zhi[2] = {zhi0[0], zhi0[1]}, zlo[2] = {zlo0[0], zlo0[1]};
+      if (cur.zg > 0) z_pieces(cur.zg, zhi, zlo);
 #pragma unroll
-    for (int nt = 0; nt < 4; nt++) {
-      const u32x4 ta = u32x4{M::pack2(acc[0][nt][0], acc[0][nt][1]), M::pack2(acc[0][nt][2], acc[0][nt][3]),
-                             M::pack2(acc[1][nt][0], acc[1][nt][1]), M::pack2(acc[1][nt][2], acc[1][nt][3])};
+      for (int nt = 0; nt < 4; nt++) {
+        const u32x4 ta = u32x4{M::pack2(acc[0][nt][0], acc[0][nt][1]), M::pack2(acc[0][nt][2], acc[0][nt][3]),
+                               M::pack2(acc[1][nt][0], acc[1][nt][1]), M::pack2(acc[1][nt][2], acc[1][nt][3])};
 #pragma unroll
-      for (int h = 0; h < 2; h++) {
-        oacc[nt][h] = M::run16(ta, zlo[h], oacc[nt][h]);
-        oacc[nt][h] = M::run16(ta, zhi[h], oacc[nt][h]);
+        for (int h = 0; h < 2; h++) {
+          oacc[nt][h] = M::run16(ta, zlo[h], oacc[nt][h]);
+          oacc[nt][h] = M::run16(ta, zhi[h], oacc[nt][h]);
+        }
       }
-    }
-  };
-  // register r of oacc[nt][h]: cell nt * 16 + 4 * quad + r of (channel c16 + 4 * wave + 2 h + col / 8, pd col % 8)
-  auto store_cells = [&](int c16, const float4_t (&oacc)[4][2]) {
+      if (cur.zg + 2 >= zgroups) {
+        // register r of oacc[nt][h]: cell nt * 16 + 4 * quad + r of (channel 4 tile + 2 h + col / 8, pd col % 8)
 #pragma unroll
-    for (int h = 0; h < 2; h++) {
-      const int c = c16 + wave * 4 + 2 * h + col / 8, pd = col % 8;
-      if (c < c_count && pd < p.od) {
-        T *o = dst + static_cast<long>(c) * cells + pd * ohw;
+        for (int h = 0; h < 2; h++) {
+          const int c = cur.tile * 4 + 2 * h + col / 8, pd = col % 8;
+          if (c < c_count && pd < p.od) {
+            T *o = dst + static_cast<long>(c) * cells + pd * ohw;
 #pragma unroll
-        for (int nt = 0; nt < 4; nt++) {
-          const int n = nt * 16 + 4 * quad;
-          if (n + 3 < ohw) {   // four neighbouring cells as one 8-byte store (2-byte aligned)
-            struct __attribute__((packed, aligned(2))) Cells4 { unsigned lo, hi; };
-            Cells4 v4;
-            v4.lo = M::pack2(oacc[nt][h][0], oacc[nt][h][1]);
-            v4.hi = M::pack2(oacc[nt][h][2], oacc[nt][h][3]);
-            *reinterpret_cast<Cells4 *>(o + n) = v4;
-          } else {
+            for (int nt = 0; nt < 4; nt++) {
+              const int n = nt * 16 + 4 * quad;
+              if (n + 3 < ohw) {   // four neighbouring cells as one 8-byte store (2-byte aligned)
+                struct __attribute__((packed, aligned(2))) Cells4 { unsigned lo, hi; };
+                Cells4 v4;
+                v4.lo = M::pack2(oacc[nt][h][0], oacc[nt][h][1]);
+                v4.hi = M::pack2(oacc[nt][h][2], oacc[nt][h][3]);
+                *reinterpret_cast<Cells4 *>(o + n) = v4;
+              } else {
 #pragma unroll
-            for (int r = 0; r < 4; r++)
-              if (n + r < ohw) o[n + r] = store_cast<T>(oacc[nt][h][r]);
+                for (int r = 0; r < 4; r++)
+                  if (n + r < ohw) o[n + r] = store_cast<T>(oacc[nt][h][r]);
+              }
+            }
           }
         }
       }
     }
-  };
-  auto clear = [](float4_t (&acc)[2][4], float4_t *oacc) {
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-      acc[i / 4][i % 4] = float4_t{0.f, 0.f, 0.f, 0.f};
-      if (oacc) oacc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
-    }
-  };
-  if (one_stage) {
-    for (int cb = 0; cb < c_count; cb += CH) {
-      __syncthreads();   // the weights are complete / the previous stage has been consumed
-      stage(cb);
-      __syncthreads();
-      for (int sb = 0; sb < CH / 16 && cb + sb * 16 < c_count; sb++) {
-        float4_t acc[2][4], oacc[4][2];
-        clear(acc, &oacc[0][0]);
-        first_product(sb, 0, acc);
-        second_product(acc, zhi0, zlo0, oacc);
-        store_cells(cb + sb * 16, oacc);
-      }
-    }
-    return;
-  }
-  for (int cb = 0; cb < c_count; cb += 16) {
-    float4_t oacc[4][2];   // [cell tile][half of the (channel', pd) columns]: cells 4 * quad .. + 3 of the tile
-    float4_t acc[2][4];    // [slice group of the stage][cell tile]
-    clear(acc, &oacc[0][0]);
-    for (int zg = 0; zg < zgroups; zg += ZS) {
-      clear(acc, nullptr);
-      for (int kc = 0; kc < KP; kc += KC) {
-        item_offset(zg, kc);
-        __syncthreads();
-        stage(cb);
-        __syncthreads();
-        first_product(0, kc, acc);
-      }
-      u32x4 zhi[2] = {zhi0[0], zhi0[1]}, zlo[2] = {zlo0[0], zlo0[1]};
-      if (zg > 0) z_pieces(zg, zhi, zlo);
-      second_product(acc, zhi, zlo, oacc);
-    }
-    store_cells(cb, oacc);
+    cur = nxt;
+    ld = ahead;
   }
 }
 
@@ -546,7 +513,7 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
     const long left = (static_cast<long>(p.N - sh.g.batch) * p.C - c_begin) * plane * es;
     const long last = ((c_end - c_begin - 1) * plane + (static_cast<long>(tz.box_hi) * p.H + ty.box_hi) * p.W + tx.box_lo + nxp) * es;
     const int kp = (ny * nxp + 31) / 32 * 32;
-    const bool room = 64 * (kp + 8) * es + 16 * 4 * (32 + 8) * es <= kPoolLdsBytes;   // weights + the smallest box chunk
+    const bool room = 64 * (kp + 8) * es <= kPoolLdsBytes;   // the weight products
     if (dense && ny * nxp <= kMfmaYx && room && near < (1L << 31) && last <= left) {
       pool_forward_mfma<T>(src, dst, p, sh, wd, lds, c_end - c_begin, min(near, left));
       return;
