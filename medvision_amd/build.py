@@ -21,7 +21,12 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
 ]
-FILE_FLAGS = {}   # per-file additions, keyed by source file name
+# per-file additions, keyed by source file name
+FILE_FLAGS = {
+    # matrix-core accumulators in ordinary vector registers: the kernel packs and stores them right
+    # away, and copies between the two register classes would outnumber its arithmetic
+    "roi_pool.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+}
 
 
 def _run(cmd):
