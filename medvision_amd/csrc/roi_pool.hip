@@ -399,7 +399,7 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
       u32x4 b[4];
 #pragma unroll
       for (int nt = 0; nt < 4; nt++)
-        b[nt] = *reinterpret_cast<const u32x4 *>(w + (nt * 16 + col) * WS + cur.k0 + quad * 8);
+        b[nt] = *reinterpret_cast<const u32x4 *>(w + ((nt / 2) * 32 + (col / 4) * 8 + (nt % 2) * 4 + col % 4) * WS + cur.k0 + quad * 8);
 #pragma unroll
       for (int zs = 0; zs < 2; zs++) {
         if (cur.zg + zs < zgroups) {
@@ -425,25 +425,29 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
         }
       }
       if (cur.zg + 2 >= zgroups) {
-        // register r of oacc[nt][h]: cell nt * 16 + 4 * quad + r of (channel 4 tile + 2 h + col / 8, pd col % 8)
+        // register r of oacc[nt][h]: cell (nt / 2) * 32 + 8 * quad + (nt % 2) * 4 + r (the order in which
+        // the weight rows were read) of (channel 4 tile + 2 h + col / 8, pd col % 8): a lane holds
+        // two runs of eight neighbouring cells
 #pragma unroll
         for (int h = 0; h < 2; h++) {
           const int c = cur.tile * 4 + 2 * h + col / 8, pd = col % 8;
           if (c < c_count && pd < p.od) {
             T *o = dst + static_cast<long>(c) * cells + pd * ohw;
 #pragma unroll
-            for (int nt = 0; nt < 4; nt++) {
-              const int n = nt * 16 + 4 * quad;
-              if (n + 3 < ohw) {   // four neighbouring cells as one 8-byte store (2-byte aligned)
-                struct __attribute__((packed, aligned(2))) Cells4 { unsigned lo, hi; };
-                Cells4 v4;
-                v4.lo = M::pack2(oacc[nt][h][0], oacc[nt][h][1]);
-                v4.hi = M::pack2(oacc[nt][h][2], oacc[nt][h][3]);
-                *reinterpret_cast<Cells4 *>(o + n) = v4;
+            for (int half = 0; half < 2; half++) {
+              const int n = half * 32 + 8 * quad;
+              if (n + 7 < ohw) {   // eight neighbouring cells as one 16-byte store (2-byte aligned)
+                struct __attribute__((packed, aligned(2))) Cells8 { unsigned v[4]; };
+                Cells8 v8;
+                v8.v[0] = M::pack2(oacc[2 * half][h][0], oacc[2 * half][h][1]);
+                v8.v[1] = M::pack2(oacc[2 * half][h][2], oacc[2 * half][h][3]);
+                v8.v[2] = M::pack2(oacc[2 * half + 1][h][0], oacc[2 * half + 1][h][1]);
+                v8.v[3] = M::pack2(oacc[2 * half + 1][h][2], oacc[2 * half + 1][h][3]);
+                *reinterpret_cast<Cells8 *>(o + n) = v8;
               } else {
 #pragma unroll
-                for (int r = 0; r < 4; r++)
-                  if (n + r < ohw) o[n + r] = store_cast<T>(oacc[nt][h][r]);
+                for (int r = 0; r < 8; r++)
+                  if (n + r < ohw) o[n + r] = store_cast<T>(oacc[2 * half + r / 4][h][r % 4]);
               }
             }
           }

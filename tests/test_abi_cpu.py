@@ -92,3 +92,43 @@ def test_foreign_device_tensors_are_refused():
         _C._same_device(here, weight=there)
     with pytest.raises(RuntimeError, match="grad_input is on meta"):
         _C._same_device(here, output=here, grad_input=there)
+
+
+def test_host_shim_cost_per_call(monkeypatch):
+    """Host time of one call through the Python shim with the library stubbed out (argument checks,
+    roi cast, workspace query cache, pointer and stream marshalling): the part of a launch that the
+    shim adds on top of the C entry point.  Printed for the record; the bound is loose because the
+    machine running the CPU suite is shared."""
+    import ctypes
+    import time
+    import torch
+    from medvision_amd import _C, _lib
+
+    class Stub:
+        def __getattr__(self, name):
+            return lambda *a: 0
+
+    class NoGuard:
+        def __init__(self, t): pass
+        def __enter__(self): pass
+        def __exit__(self, *e): return False
+
+    monkeypatch.setattr(_lib, "load", lambda: Stub())
+    monkeypatch.setattr(_lib, "stream_of", lambda t: ctypes.c_void_p(0))
+    monkeypatch.setattr(_C, "_require_cuda", lambda t, what: None)
+    monkeypatch.setattr(_C, "_on_device", NoGuard)
+    monkeypatch.setattr(_C, "_ws_bytes_cache", {})
+    vol = torch.zeros(1, 1, 16, 16, 16, dtype=torch.float16)
+    roi = torch.tensor([[0, 8, 8, 8, 16, 16, 16, 0, 0, 0]], dtype=torch.float32)
+    out = torch.empty(1, 1, 16, 16, 16, dtype=torch.float16)
+    call = lambda: _C.roi_align_rotated_3d_forward(vol, roi, out, 16, 16, 16, 1.0, 1, True, 1)
+    for _ in range(200):
+        call()
+    best = 1e9
+    for _ in range(5):
+        t = time.perf_counter()
+        for _ in range(2000):
+            call()
+        best = min(best, (time.perf_counter() - t) / 2000 * 1e6)
+    print(f"roi_align_rotated_3d_forward shim: {best:.1f} us per call")
+    assert best < 50.0
