@@ -89,6 +89,16 @@ size_t mv_roi_align_backward_workspace_bytes(int dtype, int batch, int channels,
  * still query and pass what is asked for.  ndim = 2 or 3 (out_d ignored for 2).               */
 size_t mv_roi_align_forward_workspace_bytes(int dtype, int ndim, int channels, int num_rois,
                                             int out_d, int out_h, int out_w, int sampling_ratio);
+/* The same query with the input's shape: at least the value above, and for fp16 detection heads
+ * (plain rois, outputs of up to 8 cells per axis, about as many pooled outputs as input voxels or
+ * more, width a multiple of four) the size of a re-ordered copy of the features that
+ * mv_roi_align_2d_forward / _3d_forward then read instead of the input (a few voxels of a box row no
+ * longer cost a whole memory sector each).  A non-NULL `workspace` passed to those two entry points
+ * must hold this many bytes; NULL selects the kernels that need none.  depth ignored for ndim 2.
+ * No counterpart in the reference.                                                              */
+size_t mv_roi_align_forward_workspace_bytes_for_input(int dtype, int ndim, int batch, int channels, int depth,
+                                                      int height, int width, int num_rois, int out_d,
+                                                      int out_h, int out_w, int sampling_ratio);
 
 /* ---- affine resampling engine (forward only) ----------------------------------------------
  * replaces affine_2d  csrc/affine_2d.h (vision.cpp:74), affine_3d  csrc/affine_3d.h:40 (vision.cpp:75)

@@ -123,8 +123,9 @@ int roi_forward_tiled(const void *input, const void *rois, void *output, int dty
                       const RoiProblem &p, void *workspace, size_t *need, hipStream_t s);
 
 // roi_pool.hip: separable LDS kernels for plain boxes with small outputs; -1 when not applicable
+size_t roi_pool_forward_workspace(int dtype, const RoiProblem &p);
 int roi_pool_forward(const void *input, const void *rois, void *output, int dtype,
-                     const RoiProblem &p, hipStream_t s);
+                     const RoiProblem &p, void *workspace, hipStream_t s);
 int roi_pool_backward(const void *grad_output, const void *rois, void *acc, int dtype,
                       const RoiProblem &p, hipStream_t s, bool channels_last);
 bool roi_pool_applies(int dtype, const RoiProblem &p);
@@ -174,7 +175,7 @@ int roi_forward(const void *input, const void *rois, void *output, int dtype, in
   {
     const int tiled = roi_forward_tiled(input, rois, output, dtype, p, workspace, nullptr, s);
     if (tiled >= 0) return tiled;
-    const int pooled = order != 3 ? roi_pool_forward(input, rois, output, dtype, p, s) : -1;
+    const int pooled = order != 3 ? roi_pool_forward(input, rois, output, dtype, p, workspace, s) : -1;
     if (pooled >= 0) return pooled;
   }
   const dim3 grid(p.chunks * num_rois), block(kRoiThreads);
@@ -330,6 +331,19 @@ size_t mv_roi_align_forward_workspace_bytes(int dtype, int ndim, int channels, i
   size_t need = 0;
   if (mv::roi_forward_tiled(nullptr, nullptr, nullptr, dtype, p, nullptr, &need, nullptr) != MV_OK) return 0;
   return need;
+}
+
+size_t mv_roi_align_forward_workspace_bytes_for_input(int dtype, int ndim, int batch, int channels, int depth,
+                                                      int height, int width, int num_rois, int out_d,
+                                                      int out_h, int out_w, int sampling_ratio) {
+  const size_t basic = mv_roi_align_forward_workspace_bytes(dtype, ndim, channels, num_rois, out_d, out_h, out_w,
+                                                            sampling_ratio);
+  mv::RoiProblem p = {};
+  p.ndim = ndim; p.N = batch; p.C = channels; p.D = ndim == 2 ? 1 : depth; p.H = height; p.W = width; p.R = num_rois;
+  p.od = ndim == 2 ? 1 : out_d; p.oh = out_h; p.ow = out_w; p.sampling_ratio = sampling_ratio; p.order = 1;
+  if (batch <= 0 || channels <= 0 || p.D <= 0 || height <= 0 || width <= 0 || num_rois <= 0) return basic;
+  const size_t pooled = mv::roi_pool_forward_workspace(dtype, p);
+  return pooled > basic ? pooled : basic;
 }
 
 size_t mv_roi_align_backward_workspace_bytes(int dtype, int batch, int channels, int depth,

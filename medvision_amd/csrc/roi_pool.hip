@@ -270,7 +270,7 @@ constexpr int kMfmaYx = 224;
 template <typename T>
 __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__restrict__ dst, const RoiProblem &p,
                                          const PoolShared &sh, const float (&wd)[3][kDenseSrc][8],
-                                         unsigned char *lds, int c_count, long range_bytes) {
+                                         unsigned char *lds, int c_count, long range_bytes, bool blocked, int Wb) {
   using M = Mfma<T>;
   typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
   constexpr int ES = static_cast<int>(sizeof(T));
@@ -278,14 +278,19 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
   const int nx = uni(sh.ax[0].box_hi - sh.ax[0].box_lo + 1), ny = uni(sh.ax[1].box_hi - sh.ax[1].box_lo + 1),
             nz = uni(sh.ax[2].box_hi - sh.ax[2].box_lo + 1);
   const int x_lo = uni(sh.ax[0].box_lo), y_lo = uni(sh.ax[1].box_lo), z_lo = uni(sh.ax[2].box_lo);
-  const int NXP = (nx + 3) & ~3, QX = NXP / 4, pieces = ny * QX;     // 8-byte pieces of one box slice
+  // 8-byte pieces of one box row: four voxels from the row's first column on, or (blocked copy of the
+  // features) the aligned units of four columns that the row touches, the box starting x_shift
+  // columns into the first
+  const int xb_lo = x_lo >> 2, x_shift = blocked ? x_lo - 4 * xb_lo : 0;
+  const int QX = blocked ? ((x_lo + nx - 1) >> 2) - xb_lo + 1 : (nx + 3) / 4, NXP = 4 * QX, pieces = ny * QX;
   const int KP = (ny * NXP + 31) / 32 * 32, WS = KP + 8;             // weight rows: KP products + a pad against bank conflicts
   const int ohw = p.oh * p.ow, cells = p.od * ohw;
   const long plane = static_cast<long>(p.D) * p.H * p.W;
   const int hw = p.H * p.W;
   T *w = reinterpret_cast<T *>(lds);            // [64 cells (ph, pw)][WS]
   const int zgroups = (nz + 3) / 4;
-  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);   // (a scalar for the compiler too)
   const float inv_ow = 1.f / p.ow, inv_nxp = 1.f / NXP, inv_qx = 1.f / QX;
   {  // weight products: thread = (cell, quarter of the K range), pairs of neighbouring K
     const int n = tid / 4, q = tid % 4, ph = fdiv(n, inv_ow), pw = n - ph * p.ow;
@@ -297,7 +302,8 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
       float v[2];
 #pragma unroll
       for (int e = 0; e < 2; e++) {
-        v[e] = (nv && y < ny && x < nx) ? wd[1][y < ny ? y : 0][ph & 7] * wd[0][x < nx ? x : 0][pw] : 0.f;
+        const int xr = x - x_shift;   // column of the box
+        v[e] = (nv && y < ny && xr >= 0 && xr < nx) ? wd[1][y < ny ? y : 0][ph & 7] * wd[0][(xr >= 0 && xr < nx) ? xr : 0][pw] : 0.f;
         x++;
         if (x == NXP) { x = 0; y++; }
       }
@@ -314,14 +320,26 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
   const int plane_bytes = static_cast<int>(plane) * ES;
   constexpr unsigned kNowhere = 0x80000000u;
   // this lane's row of the left operand: channel col / 4 of the tile, slice col % 4 of the group
-  const unsigned row_off = static_cast<unsigned>(((static_cast<long>(z_lo + col % 4) * p.H + y_lo) * p.W + x_lo) * ES) +
-                           static_cast<unsigned>(col / 4) * static_cast<unsigned>(plane_bytes);
+  // (blocked copy: [slice][row][unit of four columns][channel][4], a unit of one channel is 8 bytes)
+  const unsigned unit_row = static_cast<unsigned>(Wb) * p.C * 8u;   // bytes of one row of units
+  const unsigned row_off =
+      blocked ? static_cast<unsigned>((static_cast<long>(z_lo + col % 4) * p.H + y_lo) * unit_row) +
+                    static_cast<unsigned>(xb_lo) * p.C * 8u + static_cast<unsigned>(col / 4) * 8u
+              : static_cast<unsigned>(((static_cast<long>(z_lo + col % 4) * p.H + y_lo) * p.W + x_lo) * ES) +
+                    static_cast<unsigned>(col / 4) * static_cast<unsigned>(plane_bytes);
+  const int tile_bytes = blocked ? 4 * 8 : 4 * plane_bytes;                       // from one tile of four channels to the next
+  const int group_bytes = blocked ? 4 * p.H * static_cast<int>(unit_row) : 4 * hw * ES;   // from one group of four slices to the next
   // the two pieces of the lane's K positions in step ks: byte offset inside the slice and the masks
   // that clear the columns beyond the box row
   struct Piece { unsigned off, keep_lo, keep_hi; };
   auto piece = [&](int m) {
     const int y = fdiv(m, inv_qx), x0 = (m - y * QX) * 4, left = nx - x0;
     Piece e;
+    if (blocked) {   // whole units; the columns outside the box meet zero weights
+      e.off = m < pieces ? static_cast<unsigned>(y) * unit_row + static_cast<unsigned>(m - y * QX) * p.C * 8u : kNowhere;
+      e.keep_lo = e.keep_hi = 0xffffffffu;
+      return e;
+    }
     e.off = m < pieces ? static_cast<unsigned>((y * p.W + x0) * ES) : kNowhere;
     e.keep_lo = left >= 2 ? 0xffffffffu : 0x0000ffffu;
     e.keep_hi = left >= 4 ? 0xffffffffu : (left == 3 ? 0x0000ffffu : 0u);
@@ -360,7 +378,7 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
     st.k0 += 32;
     if (st.k0 >= KP) {
       st.k0 = 0; st.zg += 2;
-      if (st.zg >= zgroups) { st.zg = 0; st.tile += kPoolThreads / kWave; }
+      if (st.zg >= zgroups) { st.zg = 0; st.tile += st.tile % 2 == 0 ? 1 : 2 * (kPoolThreads / kWave) - 1; }
     }
     return st;
   };
@@ -368,18 +386,25 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
     // rows whose slice lies outside the box read zeros
     const unsigned row0 = st.zg * 4 + col % 4 < nz ? row_off : kNowhere;
     const unsigned row1 = st.zg * 4 + 4 + col % 4 < nz ? row_off : kNowhere;
-    const int soff = st.tile * 4 * plane_bytes + st.zg * 4 * hw * ES;
+    const int soff = st.tile * tile_bytes + st.zg * group_bytes;
     ld.pa = piece(st.k0 / 4 + quad * 2);
     ld.pb = piece(st.k0 / 4 + quad * 2 + 1);
 #pragma unroll
     for (int zs = 0; zs < 2; zs++) {
       const unsigned row = zs == 0 ? row0 : row1;
       // (an offset with the top bit set is beyond the range, whatever the other term adds)
-      ld.va[zs] = __builtin_amdgcn_raw_buffer_load_b64(fr, (row + ld.pa.off) | ((row | ld.pa.off) & kNowhere), soff + zs * 4 * hw * ES, 0);
-      ld.vb[zs] = __builtin_amdgcn_raw_buffer_load_b64(fr, (row + ld.pb.off) | ((row | ld.pb.off) & kNowhere), soff + zs * 4 * hw * ES, 0);
+      const unsigned at_a = (row + ld.pa.off) | ((row | ld.pa.off) & kNowhere);
+      if (QX % 2 == 0 && !blocked) {   // both pieces lie in one box row: one 16-byte load
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(fr, at_a, soff + zs * group_bytes, 0);
+        ld.va[zs] = u32x2{v.x, v.y};
+        ld.vb[zs] = u32x2{v.z, v.w};
+      } else {
+        ld.va[zs] = __builtin_amdgcn_raw_buffer_load_b64(fr, at_a, soff + zs * group_bytes, 0);
+        ld.vb[zs] = __builtin_amdgcn_raw_buffer_load_b64(fr, (row + ld.pb.off) | ((row | ld.pb.off) & kNowhere), soff + zs * group_bytes, 0);
+      }
     }
   };
-  Step cur{wave, 0, 0};
+  Step cur{2 * wave, 0, 0};   // tiles 2 w, 2 w + 1, then 2 (w + 4), ...: neighbours in memory back to back
   Loaded ld;
   if (cur.tile < tiles) issue(cur, ld);
   float4_t oacc[4][2];   // [cell tile][half of the (channel', pd) columns]: cells 4 * quad .. + 3 of the tile
@@ -462,7 +487,7 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
 template <typename T, typename RT, int CELLS>
 __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
     const T *__restrict__ feat, const RT *__restrict__ rois, T *__restrict__ out, const RoiProblem p,
-    const int channels_per_block) {
+    const int channels_per_block, const T *__restrict__ blocked, const int Wb) {
   __shared__ PoolShared sh;
   __shared__ __attribute__((aligned(16))) unsigned char lds[kPoolLdsBytes];
   const unsigned n = blockIdx.x;
@@ -518,8 +543,17 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
     const long last = ((c_end - c_begin - 1) * plane + (static_cast<long>(tz.box_hi) * p.H + ty.box_hi) * p.W + tx.box_lo + nxp) * es;
     const int kp = (ny * nxp + 31) / 32 * 32;
     const bool room = 64 * (kp + 8) * es <= kPoolLdsBytes;   // the weight products
+    if (blocked != nullptr && dense) {   // from the blocked copy (the host has checked its size)
+      const int units = ((tx.box_hi >> 2) - (tx.box_lo >> 2) + 1) * 4;
+      const long image = static_cast<long>(p.D) * p.H * Wb * p.C * 4;   // elements of one image of the copy
+      if (ny * units <= kMfmaYx && 64 * ((ny * units + 31) / 32 * 32 + 8) * es <= kPoolLdsBytes) {
+        pool_forward_mfma<T>(blocked + sh.g.batch * image + c_begin * 4, dst, p, sh, wd, lds, c_end - c_begin,
+                             (image - c_begin * 4) * es, true, Wb);
+        return;
+      }
+    }
     if (dense && ny * nxp <= kMfmaYx && room && near < (1L << 31) && last <= left) {
-      pool_forward_mfma<T>(src, dst, p, sh, wd, lds, c_end - c_begin, min(near, left));
+      pool_forward_mfma<T>(src, dst, p, sh, wd, lds, c_end - c_begin, min(near, left), false, 0);
       return;
     }
   }
@@ -688,7 +722,8 @@ __device__ inline void pool_backward_mfma(const T *__restrict__ src_any, float *
   const int NXP = (nx + 3) & ~3, QX = NXP / 4, KT = (ny * NXP + 15) / 16;
   const int ohw = p.oh * p.ow, cells = p.od * ohw;
   const int KS = ohw > 32 ? 2 : 1;                    // K steps of 32 cells
-  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);   // (a scalar for the compiler too)
   const int col = lane % 16, quad = lane / 16;
   T *wt = reinterpret_cast<T *>(lds);                 // [KT * 16 rows (y, x)][kPoolBwdRow]
   {  // weight products: thread = (row of the pass, quarter of the cells)
@@ -993,6 +1028,46 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
   }
 }
 
+// Blocked copy of fp16 / bf16 features for the pooled forward pass: [N][C][D*H][W] ->
+// [N][D*H][W / 4][C][4].  A unit of four columns of one channel is 8 bytes, and the units of all
+// channels of one place are neighbours: the rows of a roi's box, a few voxels long, then share their
+// 64-byte sectors with the other channels of the same workgroup instead of with voxels nobody asked
+// for.  A workgroup moves 64 channels x 16 units of one row through LDS (reads along the row,
+// writes along the channels).
+__global__ __launch_bounds__(256) void pool_block_features_kernel(const uint2 *__restrict__ src, uint2 *__restrict__ dst,
+                                                                   int C, long rows, int Wb) {
+  __shared__ uint2 tile[16][65];
+  const long row = blockIdx.x;            // n * D * H + (z * H + y)
+  const long nimg = row / rows, r = row - nimg * rows;
+  const int xb0 = blockIdx.y * 16, c0 = blockIdx.z * 64;
+  const int t = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int cl = t / 16 + 16 * i, xq = t % 16;
+    uint2 v = make_uint2(0u, 0u);
+    if (c0 + cl < C && xb0 + xq < Wb) v = src[((nimg * C + c0 + cl) * rows + r) * Wb + xb0 + xq];
+    tile[xq][cl] = v;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int cl = t % 64, xq = t / 64 + 4 * i;
+    if (c0 + cl < C && xb0 + xq < Wb) dst[(row * Wb + xb0 + xq) * C + c0 + cl] = tile[xq][cl];
+  }
+}
+
+// The blocked copy pays when the rois read more than the copy costs: about as many pooled outputs as
+// input voxels.  fp16 only (the matrix-core forward pass), rows of a multiple of four voxels.
+static size_t pool_blocked_bytes(int dtype, const RoiProblem &p) {
+  if (dtype != MV_F16 || p.rotated || p.order == 3 || p.W % 4 != 0) return 0;
+  if (p.od > 8 || p.oh > 8 || p.ow > 8) return 0;
+  const long voxels = static_cast<long>(p.N) * p.D * p.H * p.W, cells = static_cast<long>(p.od) * p.oh * p.ow;
+  if (static_cast<long>(p.R) * cells < voxels) return 0;
+  const long image = static_cast<long>(p.D) * p.H * p.W * p.C * 2;
+  if (image >= (1L << 31)) return 0;   // 32-bit byte offsets inside one image
+  return static_cast<size_t>(voxels) * p.C * 2;
+}
+
 static bool pool_applies(int dtype, const RoiProblem &p) {
   if (p.rotated || dtype == MV_F64) return false;
   const long cells = static_cast<long>(p.od) * p.oh * p.ow;
@@ -1015,9 +1090,10 @@ static int pool_channels_per_block(const RoiProblem &p) {
 
 template <typename T, int CELLS>
 static void launch_pool_forward(const void *input, const float *r, void *output, const RoiProblem &p, int cpb,
-                                dim3 grid, hipStream_t s) {
+                                dim3 grid, hipStream_t s, const void *blocked = nullptr) {
   hipLaunchKernelGGL((roi_pool_forward_kernel<T, float, CELLS>), grid, dim3(kPoolThreads), 0, s,
-                     static_cast<const T *>(input), r, static_cast<T *>(output), p, cpb);
+                     static_cast<const T *>(input), r, static_cast<T *>(output), p, cpb,
+                     static_cast<const T *>(blocked), p.W / 4);
 }
 
 template <typename T, bool CL, int CELLS>
@@ -1030,9 +1106,25 @@ static void launch_pool_backward(const void *grad_output, const float *r, void *
 // dense-matrix width of the kernel instance: 8 cells per axis when the output allows it
 static bool pool_small_cells(const RoiProblem &p) { return p.od <= 8 && p.oh <= 8 && p.ow <= 8; }
 
+size_t roi_pool_forward_workspace(int dtype, const RoiProblem &p) {
+  return pool_applies(dtype, p) ? pool_blocked_bytes(dtype, p) : 0;
+}
+
 int roi_pool_forward(const void *input, const void *rois, void *output, int dtype,
-                     const RoiProblem &p, hipStream_t s) {
+                     const RoiProblem &p, void *workspace, hipStream_t s) {
   if (!pool_applies(dtype, p)) return -1;
+  const void *blocked = nullptr;
+  if (workspace != nullptr && pool_blocked_bytes(dtype, p) > 0 && reinterpret_cast<uintptr_t>(input) % 8 == 0 &&
+      reinterpret_cast<uintptr_t>(workspace) % 8 == 0) {
+    const long rows = static_cast<long>(p.D) * p.H;
+    const int Wb = p.W / 4;
+    const dim3 grid(static_cast<unsigned>(p.N * rows), (Wb + 15) / 16, (p.C + 63) / 64);
+    if (p.N * rows < (1L << 31) && grid.y <= 65535 && grid.z <= 65535) {
+      hipLaunchKernelGGL(pool_block_features_kernel, grid, dim3(256), 0, s, static_cast<const uint2 *>(input),
+                         static_cast<uint2 *>(workspace), p.C, rows, Wb);
+      blocked = workspace;
+    }
+  }
   const int cpb = pool_channels_per_block(p);
   const long cblocks = (p.C + cpb - 1) / cpb;
   if (cblocks > 65535) return -1;
@@ -1045,7 +1137,7 @@ int roi_pool_forward(const void *input, const void *rois, void *output, int dtyp
             : launch_pool_forward<float, 16>(input, r, output, p, cpb, grid, s);
       break;
     case MV_F16:
-      small ? launch_pool_forward<__half, 8>(input, r, output, p, cpb, grid, s)
+      small ? launch_pool_forward<__half, 8>(input, r, output, p, cpb, grid, s, blocked)
             : launch_pool_forward<__half, 16>(input, r, output, p, cpb, grid, s);
       break;
     default:
