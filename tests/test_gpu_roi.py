@@ -320,6 +320,39 @@ def test_config5_detection_head_reduced(ops, oracle, dtype):
     assert_close(x.grad, gwant, BWD_TOL[dtype], "backward")
 
 
+@pytest.mark.parametrize("ndim", [3, 2])
+def test_pooled_forward_from_blocked_copy(ops, oracle, ndim):
+    """fp16 detection heads with about as many pooled outputs as input voxels read a re-ordered copy
+    of the features (units of four columns, channels innermost): boxes starting at every column
+    phase, sticking out of the volume on every side, of one voxel, larger than the matrix-core form
+    takes (plain form from the same launch); channel counts that are no multiple of the tile or of the
+    copy's chunk; a width whose units do not fill the copy's last chunk."""
+    from medvision_amd import _lib
+    g = wl.gen(77 + ndim)
+    size = (10, 24, 40)[3 - ndim:]
+    channels = 70
+    feat = torch.randn(2, channels, *size, generator=g).half()
+    xyz = torch.tensor(size[::-1], dtype=torch.float32)
+    n = 900 if ndim == 3 else 120
+    lo = (torch.rand(n, ndim, generator=g) * 1.3 - 0.15) * xyz
+    ext = torch.exp(torch.rand(n, ndim, generator=g) * math.log(30.0)) * 0.6      # 0.6 .. 18 voxels
+    ext[:8] = xyz * 1.2                                                            # whole-volume boxes
+    rois = torch.cat([torch.randint(0, 2, (n, 1), generator=g).float(), lo, lo + ext], 1)
+    out = (7, 7, 7)[3 - ndim:]
+    out3 = out if ndim == 3 else (1, *out)
+    in3 = size if ndim == 3 else (1, *size)
+    need = _lib.load().mv_roi_align_forward_workspace_bytes_for_input(_lib.MV_F16, ndim, 2, channels, *in3, n, *out3, 2)
+    assert need == feat.numel() * 2     # the copy is in use
+    got = ops.RoIAlign(out, 1.0, 2)(feat.to(DEV), rois.to(DEV))
+    want = oracle.roi_align_forward(feat, rois, out, 1.0, 2)
+    assert_close(got, want, FWD_TOL[torch.float16], "pooled forward from the blocked copy")
+    # few rois: no copy, same kernels from the input itself
+    few = rois[:15]
+    assert _lib.load().mv_roi_align_forward_workspace_bytes_for_input(_lib.MV_F16, ndim, 2, channels, *in3, 15, *out3, 2) == 0
+    got = ops.RoIAlign(out, 1.0, 2)(feat.to(DEV), few.to(DEV))
+    assert_close(got, want[:15], FWD_TOL[torch.float16], "pooled forward from the input")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("sr,order", [(2, 1), (-1, 1), (3, 1), (1, 0)])
 def test_pooled_kernel_paths(ops, oracle, dtype, sr, order):
