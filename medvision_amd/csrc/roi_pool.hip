@@ -77,12 +77,6 @@ struct PoolPlan {
 };
 
 static_assert(kPoolEntries == kWave, "one wavefront builds the tap table of one axis, one entry per lane");
-__device__ __forceinline__ int wave_min(int v) {
-#pragma unroll
-  for (int m = 1; m < kWave; m *= 2) v = min(v, __shfl_xor(v, m));
-  return v;
-}
-
 constexpr int kDenseSrc = 32;   // source voxels per axis of the dense weight matrices (see below)
 
 // Builds geometry and tap tables for roi `roi`; all threads must call it (contains barriers).
@@ -147,7 +141,11 @@ __device__ inline PoolPlan pool_setup(PoolShared &sh, const RT *roi, const RoiPr
     float frac = 0.f;
     const bool ok = clamped_tap<float>(v, sz, lo, hi, frac, p.order) && on;
     const float inv = 1.f / static_cast<float>(gr);
-    const int box_lo = wave_min(ok ? lo : (1 << 30)), box_hi = -wave_min(ok ? -hi : 1);
+    // the coordinates grow with the lane (plain boxes have positive extents): the box runs from the low
+    // tap of the first valid sample to the high tap of the last one
+    const unsigned long long valid = __ballot(ok);
+    const int box_lo = valid ? __builtin_amdgcn_readlane(lo, __builtin_ctzll(valid)) : (1 << 30);
+    const int box_hi = valid ? __builtin_amdgcn_readlane(hi, 63 - __builtin_clzll(valid)) : -1;
     const int top = box_hi - box_lo;
     const float wlo = ok ? (1.f - frac) * inv : 0.f, whi = ok ? frac * inv : 0.f;
     // void samples keep weight 0; they are parked at the matching end so that `lo` stays monotonic
