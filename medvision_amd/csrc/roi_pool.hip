@@ -14,6 +14,12 @@
 // (config 5: ~64 instead of 21 952).
 // rois whose sub-box or tables exceed the LDS budget are handled in the same workgroup by a plain
 // per-output gather / scatter.
+// fp16 heads with up to 8 cells per axis (7 x 7 x 7 detection heads) take matrix-core forms of the
+// same contractions instead (pool_forward_mfma, pool_backward_mfma): the (y, x) contraction as a
+// GEMM against the products Wy[y][ph] Wx[x][pw] held in LDS, operands read straight from global
+// memory, no barrier after the set-up; the forward pass optionally from a blocked copy of the
+// features (pool_block_features_kernel) in which the few voxels of a box row share their memory
+// sectors with the other channels.
 #include "common.hpp"
 #include "roi_geometry.hpp"
 #include "sampling.hpp"
