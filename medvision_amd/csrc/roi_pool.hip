@@ -491,10 +491,10 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
 template <typename T, typename RT, int CELLS>
 __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
     const T *__restrict__ feat, const RT *__restrict__ rois, T *__restrict__ out, const RoiProblem p,
-    const int channels_per_block, const T *__restrict__ blocked, const int Wb) {
+    const int channels_per_block, const T *__restrict__ blocked, const int Wb, const unsigned *__restrict__ order) {
   __shared__ PoolShared sh;
   __shared__ __attribute__((aligned(16))) unsigned char lds[kPoolLdsBytes];
-  const unsigned n = blockIdx.x;
+  const unsigned n = order ? order[blockIdx.x] : blockIdx.x;   // (largest rois first, see pool_order_rois_kernel)
   const int c_begin = blockIdx.y * channels_per_block, c_end = min(c_begin + channels_per_block, p.C);
   __shared__ __attribute__((aligned(16))) float wd[3][kDenseSrc][CELLS];
   const PoolPlan plan = pool_setup<RT, CELLS>(sh, rois + static_cast<long>(n) * roi_columns(p.ndim, 0), p, sizeof(T),
@@ -1060,6 +1060,34 @@ __global__ __launch_bounds__(256) void pool_block_features_kernel(const uint2 *_
   }
 }
 
+// Launch order of the rois for the forward pass: descending estimated cost (box volume), so that the
+// few rois that take ten times longer than the rest start first instead of finishing alone after
+// the others.  One workgroup, a counting sort over 64 logarithmic buckets; the order inside a bucket
+// is whatever the atomics give (it changes the schedule, not the results).
+constexpr int kOrderBuckets = 64, kOrderMaxRois = 1 << 17;
+__global__ __launch_bounds__(1024) void pool_order_rois_kernel(const float *__restrict__ rois, unsigned *__restrict__ order,
+                                                               int R, int ndim, float scale) {
+  __shared__ unsigned count[kOrderBuckets], start[kOrderBuckets];
+  const int cols = 1 + 2 * ndim;
+  auto bucket = [&](int i) {
+    const float *r = rois + static_cast<long>(i) * cols;
+    float vol = 1.f;
+    for (int a = 0; a < ndim; a++) vol *= fmaxf((r[1 + ndim + a] - r[1 + a]) * scale, 1.f) + 2.f;
+    const int b = static_cast<int>(4.f * log2f(fminf(fmaxf(vol, 1.f), 6.0e4f)));   // 0 .. 63
+    return kOrderBuckets - 1 - min(b, kOrderBuckets - 1);                          // large boxes first
+  };
+  if (threadIdx.x < kOrderBuckets) count[threadIdx.x] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < R; i += 1024) atomicAdd(&count[bucket(i)], 1u);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned sum = 0;
+    for (int b = 0; b < kOrderBuckets; b++) { start[b] = sum; sum += count[b]; }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < R; i += 1024) order[atomicAdd(&start[bucket(i)], 1u)] = static_cast<unsigned>(i);
+}
+
 // The blocked copy pays when the rois read more than the copy costs: about as many pooled outputs as
 // input voxels.  fp16 only (the matrix-core forward pass), rows of a multiple of four voxels.
 static size_t pool_blocked_bytes(int dtype, const RoiProblem &p) {
@@ -1069,7 +1097,7 @@ static size_t pool_blocked_bytes(int dtype, const RoiProblem &p) {
   if (static_cast<long>(p.R) * cells < voxels) return 0;
   const long image = static_cast<long>(p.D) * p.H * p.W * p.C * 2;
   if (image >= (1L << 31)) return 0;   // 32-bit byte offsets inside one image
-  return static_cast<size_t>(voxels) * p.C * 2;
+  return static_cast<size_t>(voxels) * p.C * 2 + (p.R <= kOrderMaxRois ? static_cast<size_t>(p.R) * 4 : 0);
 }
 
 static bool pool_applies(int dtype, const RoiProblem &p) {
@@ -1094,10 +1122,10 @@ static int pool_channels_per_block(const RoiProblem &p) {
 
 template <typename T, int CELLS>
 static void launch_pool_forward(const void *input, const float *r, void *output, const RoiProblem &p, int cpb,
-                                dim3 grid, hipStream_t s, const void *blocked = nullptr) {
+                                dim3 grid, hipStream_t s, const void *blocked = nullptr, const unsigned *order = nullptr) {
   hipLaunchKernelGGL((roi_pool_forward_kernel<T, float, CELLS>), grid, dim3(kPoolThreads), 0, s,
                      static_cast<const T *>(input), r, static_cast<T *>(output), p, cpb,
-                     static_cast<const T *>(blocked), p.W / 4);
+                     static_cast<const T *>(blocked), p.W / 4, order);
 }
 
 template <typename T, bool CL, int CELLS>
@@ -1118,6 +1146,7 @@ int roi_pool_forward(const void *input, const void *rois, void *output, int dtyp
                      const RoiProblem &p, void *workspace, hipStream_t s) {
   if (!pool_applies(dtype, p)) return -1;
   const void *blocked = nullptr;
+  const unsigned *order = nullptr;
   if (workspace != nullptr && pool_blocked_bytes(dtype, p) > 0 && reinterpret_cast<uintptr_t>(input) % 8 == 0 &&
       reinterpret_cast<uintptr_t>(workspace) % 8 == 0) {
     const long rows = static_cast<long>(p.D) * p.H;
@@ -1127,6 +1156,12 @@ int roi_pool_forward(const void *input, const void *rois, void *output, int dtyp
       hipLaunchKernelGGL(pool_block_features_kernel, grid, dim3(256), 0, s, static_cast<const uint2 *>(input),
                          static_cast<uint2 *>(workspace), p.C, rows, Wb);
       blocked = workspace;
+      if (p.R <= kOrderMaxRois) {   // (behind the copy; its size is a multiple of 8 bytes)
+        unsigned *ord = reinterpret_cast<unsigned *>(static_cast<char *>(workspace) + static_cast<size_t>(p.N) * rows * p.W * p.C * 2);
+        hipLaunchKernelGGL(pool_order_rois_kernel, dim3(1), dim3(1024), 0, s, static_cast<const float *>(rois), ord,
+                           p.R, p.ndim, static_cast<float>(p.scale));
+        order = ord;
+      }
     }
   }
   const int cpb = pool_channels_per_block(p);
@@ -1141,7 +1176,7 @@ int roi_pool_forward(const void *input, const void *rois, void *output, int dtyp
             : launch_pool_forward<float, 16>(input, r, output, p, cpb, grid, s);
       break;
     case MV_F16:
-      small ? launch_pool_forward<__half, 8>(input, r, output, p, cpb, grid, s, blocked)
+      small ? launch_pool_forward<__half, 8>(input, r, output, p, cpb, grid, s, blocked, order)
             : launch_pool_forward<__half, 16>(input, r, output, p, cpb, grid, s);
       break;
     default:
