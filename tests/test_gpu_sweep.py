@@ -97,6 +97,35 @@ def test_roi_sweep(ops, oracle):
         assert rel_err(fg.grad, gwant) <= BWD_TOL[dtype], what + " (backward)"
 
 
+def test_pooled_many_rois_sweep(ops, oracle):
+    """fp16 heads with many rois on small maps: the matrix-core pooled forward from the input and from
+    the blocked copy of the features (widths that are and are not multiples of four, channel counts
+    around the tile and chunk sizes, 2-D and 3-D, boxes inside, across and outside the volume)."""
+    for seed in range(80):
+        rnd = random.Random(seed)
+        g = torch.Generator().manual_seed(seed)
+        ndim = rnd.choice([2, 3])
+        size = [rnd.randint(1, 20) for _ in range(ndim - 1)] + [4 * rnd.randint(1, 9) if rnd.random() < 0.8 else rnd.randint(1, 30)]
+        channels, batch = rnd.choice([1, 3, 4, 8, 17, 64, 130]), rnd.randint(1, 3)
+        feat = torch.randn(batch, channels, *size, generator=g).half()
+        out = [rnd.randint(1, 8) for _ in range(ndim)]
+        cells, voxels = 1, batch
+        for o in out:
+            cells *= o
+        for n in size:
+            voxels *= n
+        count = max(1, min(3000, int(voxels / cells * rnd.choice([0.5, 1.0, 1.5, 3.0])) + 1))
+        scale, sr = rnd.choice([0.5, 1.0, 1.0, 2.0]), rnd.choice([0, 1, 2, 2, 3])
+        ext = torch.tensor(size[::-1], dtype=torch.float32) / scale
+        lo = (torch.rand(count, ndim, generator=g) * 1.4 - 0.3) * ext
+        hi = lo + torch.rand(count, ndim, generator=g) * ext * rnd.choice([0.1, 0.3, 0.8, 1.6])
+        rois = torch.cat([torch.randint(0, batch, (count, 1), generator=g).float(), lo, hi], 1)
+        got = ops.RoIAlign(tuple(out), scale, sr)(feat.to(DEV), rois.to(DEV))
+        want = oracle.roi_align_forward(feat, rois, tuple(out), scale, sr)
+        what = f"seed {seed}: {ndim}-D {tuple(feat.shape)} -> {out} x {count} rois, scale {scale}, sr {sr}"
+        assert rel_err(got, want) <= FWD_TOL[torch.float16], what
+
+
 def test_affine_and_warp_sweep(ops, oracle):
     """Larger outputs, so that the LDS-tiled resampler (orders 0 / 1 and 3) takes most cases."""
     for seed in range(8000, 8120):
