@@ -91,9 +91,11 @@ struct PlanShape {
   int es;                         // bytes per element
   FastDiv by_per_roi, by_tiles_x, by_tiles_y, by_total, by_slots;
   int halo_lo, halo_hi;           // voxels needed below / above the cell of a sample: 0 / 1, order 3: 1 / 2
+  unsigned warm_groups;           // 16-byte groups of the input to pull into the caches during planning (0: none)
 };
 
 constexpr unsigned kDone = 0xffffffffu;  // "no item"
+constexpr unsigned kWarmStride = 4;      // words between the loads of the cache warm-up
 
 // Lane-parallel planning: four lanes per item, lane `a` = 0..2 owns source axis / roi angle `a`
 // (lane 3 idles), so the three sin / cos pairs, the per-axis divisions and the three box
@@ -748,6 +750,19 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
         __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(ld_base), 0, ld_extent, 0x00020000);
     val[u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ld_voff, u * ld_stride, 0);
   };
+  // While the first wavefront plans, the others pull this workgroup's share of a small input through
+  // the caches: the workgroups' first boxes, requested all at once when the plans are ready, then
+  // come from the caches instead of from memory in one burst.
+  if (tid >= kWave && ps.warm_groups > 0) {
+    const unsigned per = (ps.warm_groups + gridDim.x - 1) / gridDim.x, first = blockIdx.x * per;
+    const unsigned *words = reinterpret_cast<const unsigned *>(feat);
+    unsigned seen = 0;
+    // (one word per 16-byte group: four neighbouring lanes share a 64-byte sector, which costs four
+    // times the instructions of one lane per sector and was measured 1.1 us faster)
+    for (unsigned i = tid - kWave; i < per; i += THREADS - kWave)
+      if (first + i < ps.warm_groups) seen |= words[static_cast<size_t>(first + i) * kWarmStride];
+    asm volatile("" ::"v"(seen));
+  }
   // The first wavefront plans this workgroup's items (at most kPlanSlots), four lanes per item.
   if (tid < kWave) {
     static_assert(kPlanSlots * 4 == kWave, "four lanes per plan slot");
@@ -1148,6 +1163,11 @@ static int launch_resample(const T *feat, const float *rois, T *out, const RoiPr
   ps.cap = LDS_BYTES / sizeof(T);
   ps.threads = THREADS; ps.max_items = KMAX;
   ps.halo_lo = CUBIC ? 1 : 0; ps.halo_hi = CUBIC ? 2 : 1;
+  {
+    // inputs that fit the L2s and are read about once (resampling: no more rois than images)
+    const long in_bytes = static_cast<long>(p.N) * p.C * p.D * p.H * p.W * static_cast<long>(sizeof(T));
+    ps.warm_groups = (!CUBIC && ps.vec > 0 && p.R <= p.N && in_bytes <= (24L << 20)) ? static_cast<unsigned>(in_bytes / (4 * kWarmStride)) : 0u;
+  }
   ps.es = static_cast<int>(sizeof(T));
   ps.by_per_roi.set(static_cast<unsigned>(per_roi));
   ps.by_tiles_x.set(static_cast<unsigned>(tx));
