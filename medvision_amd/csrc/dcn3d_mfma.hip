@@ -54,14 +54,13 @@ __global__ void dcn_channels_last_kernel(const U *__restrict__ x, U *__restrict_
 // of one position.  Needs P and Cin to be multiples of V and 16-byte aligned tensors.
 constexpr int kLayoutPos = 128;
 template <typename U>
-__global__ __launch_bounds__(256) void dcn_channels_last_wide_kernel(const U *__restrict__ x, U *__restrict__ xt,
-                                                                     int Cin, long P) {
+__device__ __forceinline__ void channels_last_wide_block(const U *__restrict__ x, U *__restrict__ xt, int Cin, long P,
+                                                         unsigned bx, int b, int bz) {
   constexpr int V = 16 / sizeof(U), CH = 256 / sizeof(U);   // CH channels per workgroup: 128 (2 bytes), 64 (4 bytes)
   constexpr int PITCH = kLayoutPos + V;
   __shared__ __attribute__((aligned(16))) U stage[CH * PITCH];
-  const int b = blockIdx.y;
-  const long p0 = static_cast<long>(blockIdx.x) * kLayoutPos;
-  const int c0 = blockIdx.z * CH, cn = min(CH, Cin - c0);
+  const long p0 = static_cast<long>(bx) * kLayoutPos;
+  const int c0 = bz * CH, cn = min(CH, Cin - c0);
   const int np = static_cast<int>(min(static_cast<long>(kLayoutPos), P - p0));   // a multiple of V
   const U *src = x + (static_cast<long>(b) * Cin + c0) * P + p0;
   U *dst = xt + (static_cast<long>(b) * P + p0) * Cin + c0;
@@ -82,6 +81,11 @@ __global__ __launch_bounds__(256) void dcn_channels_last_wide_kernel(const U *__
     __builtin_memcpy(&packed, out, 16);
     *reinterpret_cast<u32x4 *>(dst + static_cast<long>(pp) * Cin + cg * V) = packed;
   }
+}
+template <typename U>
+__global__ __launch_bounds__(256) void dcn_channels_last_wide_kernel(const U *__restrict__ x, U *__restrict__ xt,
+                                                                     int Cin, long P) {
+  channels_last_wide_block<U>(x, xt, Cin, P, blockIdx.x, blockIdx.y, blockIdx.z);
 }
 
 // weight [Cout, cpg, K] -> A pieces [group][tap][slice][row block][lane][kPiece]
@@ -209,13 +213,12 @@ __global__ __launch_bounds__(256, MT <= 2 ? 4 : 3) void dcn_forward_mfma_kernel(
 // workgroup one tap ahead) instead of from the vector memory path.
 // weight [Cout, cpg, K] -> A pieces [group][tap][slice][16-row block][lane][kPiece]
 template <typename T>
-__global__ __launch_bounds__(256) void dcn_weight_fragments16_kernel(const T *__restrict__ wt,
-                                                                     T *__restrict__ wf,
-                                                                     const DcnDims s) {
-  constexpr int PC = Mfma<T>::kPiece;
+__device__ __forceinline__ void weight_fragments16_block(const T *__restrict__ wt, T *__restrict__ wf, const DcnDims &s,
+                                                         unsigned block) {
+  constexpr int PC = 16 / static_cast<int>(sizeof(T));   // = Mfma<T>::kPiece
   const int slices = s.cpg / (4 * PC), blocks = s.opg / 16;
   const long total = static_cast<long>(s.groups) * s.K * slices * blocks * 64;
-  const long id = blockIdx.x * 256L + threadIdx.x;
+  const long id = block * 256L + threadIdx.x;
   if (id >= total) return;
   const int lane = id % 64;
   long r = id / 64;
@@ -226,6 +229,26 @@ __global__ __launch_bounds__(256) void dcn_weight_fragments16_kernel(const T *__
   const int o = g * s.opg + mb * 16 + lane % 16;
   const int cl = cc * 4 * PC + (lane / 16) * PC;
   for (int i = 0; i < PC; i++) wf[id * PC + i] = wt[(static_cast<long>(o) * s.cpg + cl + i) * s.K + k];
+}
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_weight_fragments16_kernel(const T *__restrict__ wt,
+                                                                     T *__restrict__ wf,
+                                                                     const DcnDims s) {
+  weight_fragments16_block<T>(wt, wf, s, blockIdx.x);
+}
+// Both layout moves of a forward call in one launch (the weights are a few thousand pieces: a
+// launch of their own costs more than the move): the first `nt` workgroups transpose x, the others
+// order the weight pieces.  U = the element as an integer of its size.
+template <typename U>
+__global__ __launch_bounds__(256) void dcn_forward_layout_kernel(const U *__restrict__ x, U *__restrict__ xt,
+                                                                 const U *__restrict__ wt, U *__restrict__ wf,
+                                                                 const DcnDims s, unsigned wblocks, unsigned nt) {
+  if (blockIdx.x < nt) {
+    const unsigned bx = blockIdx.x % wblocks, r = blockIdx.x / wblocks;
+    channels_last_wide_block<U>(x, xt, s.Cin, s.P, bx, static_cast<int>(r % s.B), static_cast<int>(r / s.B));
+  } else {
+    weight_fragments16_block<U>(wt, wf, s, blockIdx.x - nt);
+  }
 }
 
 // blocks of 16 positions per wavefront: one keeps the kernel at 96 registers = 5 wavefronts per
@@ -639,9 +662,33 @@ static int dcn_mfma_run(const void *x, const void *off, const void *mask, const 
   T *xt = static_cast<T *>(workspace);
   T *wf = reinterpret_cast<T *>(static_cast<char *>(workspace) +
                                 align256(static_cast<size_t>(s.B) * s.P * s.Cin * sizeof(T)));
-  const int st = dcn_channels_last(x, xt, s.B, s.Cin, s.P, sizeof(T), stream);
-  if (st) return st;
   // 16 x 16 tiling: whole 4-piece slices per (deformable) group and a tap's weight pieces fit LDS
+  bool fused = false;   // x and the weights laid out by one launch
+  {
+    using U = typename std::conditional<(sizeof(T) == 2), unsigned short, unsigned int>::type;
+    const int blocks16 = s.opg / 16;
+    const int mb = (blocks16 >= 8 && s.nd == 2) ? 8 : (blocks16 >= 4 ? 4 : (blocks16 >= 2 ? 2 : 1));
+    const long tap_bytes = static_cast<long>(s.cpg / (4 * PC)) * mb * 64 * 16;
+    const bool tiling16 = s.cpg % (4 * PC) == 0 && s.cpd % (4 * PC) == 0 && (tap_bytes <= kWeightLds || s.cpd % s.cpg == 0);
+    constexpr int V = 16 / static_cast<int>(sizeof(T)), CH = 256 / static_cast<int>(sizeof(T));
+    const bool aligned = reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(xt) % 16 == 0;
+    const long wblocks = (s.P + kLayoutPos - 1) / kLayoutPos;
+    const long nt = wblocks * s.B * ((s.Cin + CH - 1) / CH);
+    const long lanes = static_cast<long>(s.groups) * s.K * (s.cpg / (4 * PC)) * blocks16 * 64;
+    const long nw = (lanes + 255) / 256;
+    if (tiling16 && aligned && s.P % V == 0 && s.Cin % V == 0 && nt + nw < (1L << 31)) {
+      hipLaunchKernelGGL((dcn_forward_layout_kernel<U>), dim3(static_cast<unsigned>(nt + nw)), dim3(256), 0, stream,
+                         reinterpret_cast<const U *>(x), reinterpret_cast<U *>(xt), reinterpret_cast<const U *>(wt),
+                         reinterpret_cast<U *>(wf), s, static_cast<unsigned>(wblocks), static_cast<unsigned>(nt));
+      const int st = check_launch("dcn_forward_layout_kernel");
+      if (st) return st;
+      fused = true;
+    }
+  }
+  if (!fused) {
+    const int st = dcn_channels_last(x, xt, s.B, s.Cin, s.P, sizeof(T), stream);
+    if (st) return st;
+  }
   {
     const int blocks16 = s.opg / 16;
     // output blocks of 16 per wavefront: up to 8 (128 output channels: every pass over the output
@@ -653,8 +700,9 @@ static int dcn_mfma_run(const void *x, const void *off, const void *mask, const 
     const bool fits = tap_bytes <= kWeightLds || s.cpd % s.cpg == 0;
     if (s.cpg % (4 * PC) == 0 && s.cpd % (4 * PC) == 0 && fits) {
       const long lanes = static_cast<long>(s.groups) * s.K * (s.cpg / (4 * PC)) * blocks16 * 64;
-      hipLaunchKernelGGL((dcn_weight_fragments16_kernel<T>), dim3(static_cast<unsigned>((lanes + 255) / 256)),
-                         dim3(256), 0, stream, static_cast<const T *>(wt), wf, s);
+      if (!fused)
+        hipLaunchKernelGGL((dcn_weight_fragments16_kernel<T>), dim3(static_cast<unsigned>((lanes + 255) / 256)),
+                           dim3(256), 0, stream, static_cast<const T *>(wt), wf, s);
       const int chunks = (blocks16 + mb - 1) / mb;
       if constexpr (sizeof(T) == 2) {
         // volumes with 32 or 64 channels per group inside one deformable group: taps shared through LDS
