@@ -818,6 +818,43 @@ __global__ __launch_bounds__(256) void dcn_planar_add_kernel(const float *__rest
     }
 }
 
+// The same move with 16-byte accesses on both sides (whole tiles of 64 positions x 64 channels, P a
+// multiple of 64, 16-byte aligned tensors): a lane reads four channels of one position, then adds
+// V = 16 / sizeof(T) neighbouring positions of one channel to the gradient in one read-modify-write.
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_planar_add_wide_kernel(const float *__restrict__ gxt,
+                                                                  T *__restrict__ gx, int C, long P) {
+  constexpr int V = 16 / static_cast<int>(sizeof(T));
+  __shared__ __attribute__((aligned(16))) float stagef[64][kAddChunk + 4];
+  const int b = blockIdx.y;
+  const long p0 = static_cast<long>(blockIdx.x) * 64;
+  const int c0 = blockIdx.z * kAddChunk, cn = min(kAddChunk, C - c0);   // cn: a multiple of 4
+  const float *src = gxt + (static_cast<long>(b) * P + p0) * C + c0;
+  float4 in[4];
+#pragma unroll
+  for (int u = 0; u < 4; u++) {
+    const int i = threadIdx.x + u * 256, pp = i / 16, cq = i % 16;
+    in[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (cq * 4 < cn) in[u] = *reinterpret_cast<const float4 *>(src + static_cast<long>(pp) * C + cq * 4);
+  }
+#pragma unroll
+  for (int u = 0; u < 4; u++) {
+    const int i = threadIdx.x + u * 256, pp = i / 16, cq = i % 16;
+    *reinterpret_cast<float4 *>(&stagef[pp][cq * 4]) = in[u];
+  }
+  __syncthreads();
+  constexpr int PG = 64 / V;   // position groups per channel
+  for (int i = threadIdx.x; i < cn * PG; i += 256) {
+    const int c = i / PG, pg = i % PG;
+    T *d = gx + (static_cast<long>(b) * C + c0 + c) * P + p0 + pg * V;
+    union { u32x4 u; T e[V]; } piece;
+    piece.u = *reinterpret_cast<const u32x4 *>(d);
+#pragma unroll
+    for (int e = 0; e < V; e++) piece.e[e] = store_cast<T>(load(&piece.e[e]) + stagef[pg * V + e][c]);
+    *reinterpret_cast<u32x4 *>(d) = piece.u;
+  }
+}
+
 __global__ void dcn_zero_f32_kernel(float *p, long n) {
   for (long i = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; i < n;
        i += static_cast<long>(gridDim.x) * blockDim.x)
@@ -994,6 +1031,19 @@ int planar_add_f32(const float *src, void *dst, int B, int C, long P, int dtype,
   const long pblocks = (P + 63) / 64;
   MV_REQUIRE(pblocks < (1L << 31) && B <= 65535 && (C + kAddChunk - 1) / kAddChunk <= 65535, "volume too large");
   const dim3 grid(static_cast<unsigned>(pblocks), B, (C + kAddChunk - 1) / kAddChunk);
+  if (P % 64 == 0 && C % 4 == 0 && reinterpret_cast<uintptr_t>(src) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(dst) % 16 == 0) {
+    if (dtype == MV_F16)
+      hipLaunchKernelGGL((dcn_planar_add_wide_kernel<__half>), grid, dim3(256), 0, stream, src,
+                         static_cast<__half *>(dst), C, P);
+    else if (dtype == MV_F32)
+      hipLaunchKernelGGL((dcn_planar_add_wide_kernel<float>), grid, dim3(256), 0, stream, src,
+                         static_cast<float *>(dst), C, P);
+    else
+      hipLaunchKernelGGL((dcn_planar_add_wide_kernel<__hip_bfloat16>), grid, dim3(256), 0, stream, src,
+                         static_cast<__hip_bfloat16 *>(dst), C, P);
+    return check_launch("dcn_planar_add_wide_kernel");
+  }
   if (dtype == MV_F16)
     hipLaunchKernelGGL((dcn_planar_add_kernel<__half>), grid, dim3(256), 0, stream, src,
                        static_cast<__half *>(dst), C, P);
