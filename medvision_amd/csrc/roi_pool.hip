@@ -1,5 +1,7 @@
 // RoIAlign for plain (axis-aligned) boxes with SMALL outputs per roi (detection heads: thousands of
-// rois, 7x7x7 cells, hundreds of channels), forward and backward.
+// rois, 7x7x7 cells, hundreds of channels), forward and backward.  Same results as the reference's
+// one-thread-per-output kernels (csrc/cuda/roi_align_3d_cuda_kernel.cuh:11-86 forward, :90-202
+// backward with eight atomicAdd per sample, :189-196; 2-D twin roi_align_2d_cuda_kernel.cuh).
 //
 // For an axis-aligned box the sample coordinates are separable: x depends only on (pw, ix), y on
 // (ph, iy), z on (pd, iz).  Each axis therefore has a short tap table (cells * grid entries of

@@ -1,22 +1,26 @@
 // Forward resampling for LARGE outputs per roi (Resize / RandomAffine / Crop: one roi produces a
 // whole volume) with a sampling grid of 1x1x1.  Used by the rotated, plain and affine entry
-// points whenever one (roi, channel) yields at least a few thousand voxels.
+// points whenever one (roi, channel) yields at least a few thousand voxels.  Same results as the
+// reference's one-thread-per-output kernels (csrc/cuda/roi_align_rotated_3d_cuda_kernel.cuh:15-120,
+// csrc/cuda_aug/affine_3d_cuda_kernel.cuh:14-120 and their 2-D twins).
 //
 // One launch of persistent workgroups.  An item is (output tile of TX x TY x TZ voxels, channel):
-//   planning   (prologue) one lane per item of the workgroup: the roi's affine sample map
-//              r = Rot * p + centre in fp64, the interval each source axis covers for the tile
-//              (centre +- sum_j |Rot[a][j]| * halfspan_j) and from it the axis-aligned box of
-//              source voxels to stage, clipped to the volume; the map is re-expressed relative to
-//              the box origin.  The 208-byte records stay in LDS.
+//   planning   (prologue) the first wavefront, four lanes per item of the workgroup: the roi's
+//              affine sample map r = Rot * p + centre in fp64, the interval each source axis covers
+//              for the tile (centre +- sum_j |Rot[a][j]| * halfspan_j) and from it the axis-aligned
+//              box of source voxels to stage, clipped to the volume; the map is re-expressed
+//              relative to the box origin.  The records (TilePlan, every wave-uniform value an item
+//              needs) stay in LDS.  Meanwhile the other wavefronts pull a small input through the
+//              caches.
 //   staging    the box is copied to LDS as 16-byte row groups; the loads of item i+1 are issued
-//              into registers before item i is interpolated.
+//              into registers while item i is interpolated.
 //   sampling   every lane produces a column of the tile from LDS: lanes run along x, so LDS reads
 //              of neighbouring lanes touch neighbouring banks and output stores are coalesced.
 //              Boxes larger than the LDS buffer (strong down-scaling) are sampled straight from
 //              global memory by the same code.
-// Coordinates: box-relative, one FMA per axis and voxel in the coordinate type CT (fp32 for 16-bit
-// tensors, fp64 for fp32 tensors), then floor / fraction in CT.  Tiles whose box is not clipped
-// skip the [-1,S] tests and the border clamps.
+// Coordinates: box-relative in the coordinate type CT (fp32 for 16-bit tensors, fp64 for fp32
+// tensors), then floor / fraction in CT.  Tiles whose box is not clipped skip the [-1,S] tests and
+// the border clamps.
 #include "common.hpp"
 #include "roi_geometry.hpp"
 #include "sampling.hpp"
@@ -28,7 +32,7 @@ constexpr int kXcds = 8;
 // What the workgroup's first wavefront works out per item and every wavefront then reads from LDS.
 // Values a wavefront needs in scalar registers sit in the first 64 dwords (lane l fetches dword l,
 // fields are pulled out with v_readlane); values only the vector unit uses are read as broadcasts.
-struct TilePlan {            // 320 bytes
+struct TilePlan {            // 352 bytes
   // per source axis a, at [4 * a .. 4 * a + 3]: the box-relative source position of the tile's
   // first output voxel, then d(source a)/d(output j) for j = (x, y, z)
   double map[12];            // dword 0
