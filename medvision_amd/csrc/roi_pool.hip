@@ -1034,43 +1034,15 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
   }
 }
 
-// Blocked copy of fp16 / bf16 features for the pooled forward pass: [N][C][D*H][W] ->
-// [N][D*H][W / 4][C][4].  A unit of four columns of one channel is 8 bytes, and the units of all
-// channels of one place are neighbours: the rows of a roi's box, a few voxels long, then share their
-// 64-byte sectors with the other channels of the same workgroup instead of with voxels nobody asked
-// for.  A workgroup moves 64 channels x 16 units of one row through LDS (reads along the row,
-// writes along the channels).
-__global__ __launch_bounds__(256) void pool_block_features_kernel(const uint2 *__restrict__ src, uint2 *__restrict__ dst,
-                                                                   int C, long rows, int Wb) {
-  __shared__ uint2 tile[16][65];
-  const long row = blockIdx.x;            // n * D * H + (z * H + y)
-  const long nimg = row / rows, r = row - nimg * rows;
-  const int xb0 = blockIdx.y * 16, c0 = blockIdx.z * 64;
-  const int t = threadIdx.x;
-#pragma unroll
-  for (int i = 0; i < 4; i++) {
-    const int cl = t / 16 + 16 * i, xq = t % 16;
-    uint2 v = make_uint2(0u, 0u);
-    if (c0 + cl < C && xb0 + xq < Wb) v = src[((nimg * C + c0 + cl) * rows + r) * Wb + xb0 + xq];
-    tile[xq][cl] = v;
-  }
-  __syncthreads();
-#pragma unroll
-  for (int i = 0; i < 4; i++) {
-    const int cl = t % 64, xq = t / 64 + 4 * i;
-    if (c0 + cl < C && xb0 + xq < Wb) dst[(row * Wb + xb0 + xq) * C + c0 + cl] = tile[xq][cl];
-  }
-}
-
 // Launch order of the rois for the forward pass: descending estimated cost (box volume), so that the
 // few rois that take ten times longer than the rest start first instead of finishing alone after
 // the others.  One workgroup, a counting sort over 64 logarithmic buckets; the order inside a bucket
 // is whatever the atomics give (it changes the schedule, not the results).
 constexpr int kOrderBuckets = 64, kOrderMaxRois = 1 << 17;
-__global__ __launch_bounds__(1024) void pool_order_rois_kernel(const float *__restrict__ rois, unsigned *__restrict__ order,
-                                                               int R, int ndim, float scale) {
+__device__ inline void pool_order_rois(const float *__restrict__ rois, unsigned *__restrict__ order, int R, int ndim,
+                                       float scale) {
   __shared__ unsigned count[kOrderBuckets], start[kOrderBuckets];
-  const int cols = 1 + 2 * ndim;
+  const int cols = 1 + 2 * ndim, step = blockDim.x;
   auto bucket = [&](int i) {
     const float *r = rois + static_cast<long>(i) * cols;
     float vol = 1.f;
@@ -1080,14 +1052,53 @@ __global__ __launch_bounds__(1024) void pool_order_rois_kernel(const float *__re
   };
   if (threadIdx.x < kOrderBuckets) count[threadIdx.x] = 0;
   __syncthreads();
-  for (int i = threadIdx.x; i < R; i += 1024) atomicAdd(&count[bucket(i)], 1u);
+  for (int i = threadIdx.x; i < R; i += step) atomicAdd(&count[bucket(i)], 1u);
   __syncthreads();
   if (threadIdx.x == 0) {
     unsigned sum = 0;
     for (int b = 0; b < kOrderBuckets; b++) { start[b] = sum; sum += count[b]; }
   }
   __syncthreads();
-  for (int i = threadIdx.x; i < R; i += 1024) order[atomicAdd(&start[bucket(i)], 1u)] = static_cast<unsigned>(i);
+  for (int i = threadIdx.x; i < R; i += step) order[atomicAdd(&start[bucket(i)], 1u)] = static_cast<unsigned>(i);
+}
+
+// Blocked copy of fp16 / bf16 features for the pooled forward pass: [N][C][D*H][W] ->
+// [N][D*H][W / 4][C][4].  A unit of four columns of one channel is 8 bytes, and the units of all
+// channels of one place are neighbours: the rows of a roi's box, a few voxels long, then share their
+// 64-byte sectors with the other channels of the same workgroup instead of with voxels nobody asked
+// for.  A workgroup moves 64 channels x up to 32 units of one row through LDS (reads along the row,
+// writes along the channels).  The first workgroup of the launch orders the rois instead (when `order`
+// is given): the two jobs do not depend on each other.
+constexpr int kBlockUnits = 32;
+__global__ __launch_bounds__(256) void pool_block_features_kernel(const uint2 *__restrict__ src, uint2 *__restrict__ dst,
+                                                                   int C, long rows, int Wb,
+                                                                   const float *__restrict__ rois, unsigned *__restrict__ order,
+                                                                   int R, int ndim, float scale) {
+  if (order != nullptr && blockIdx.x == 0) {   // (first, so that it is over long before the copy)
+    pool_order_rois(rois, order, R, ndim, scale);
+    return;
+  }
+  __shared__ uint2 tile[kBlockUnits * 65];
+  const int ux = min(Wb, kBlockUnits), xchunks = (Wb + ux - 1) / ux, cchunks = (C + 63) / 64;
+  unsigned id = blockIdx.x - (order != nullptr ? 1u : 0u);
+  const int cz = id % cchunks; id /= cchunks;
+  const int xc = id % xchunks;
+  const long row = id / xchunks;            // n * D * H + (z * H + y)
+  const long nimg = row / rows, r = row - nimg * rows;
+  const int xb0 = xc * ux, c0 = cz * 64;
+  const int t = threadIdx.x;
+  const float inv_ux = 1.f / ux;
+  for (int i = t; i < 64 * ux; i += 256) {
+    const int cl = fdiv(i, inv_ux), xq = i - cl * ux;
+    uint2 v = make_uint2(0u, 0u);
+    if (c0 + cl < C && xb0 + xq < Wb) v = src[((nimg * C + c0 + cl) * rows + r) * Wb + xb0 + xq];
+    tile[xq * 65 + cl] = v;
+  }
+  __syncthreads();
+  for (int i = t; i < 64 * ux; i += 256) {
+    const int xq = i / 64, cl = i % 64;
+    if (c0 + cl < C && xb0 + xq < Wb) dst[(row * Wb + xb0 + xq) * C + c0 + cl] = tile[xq * 65 + cl];
+  }
 }
 
 // The blocked copy pays when the rois read more than the copy costs: about as many pooled outputs as
@@ -1152,18 +1163,18 @@ int roi_pool_forward(const void *input, const void *rois, void *output, int dtyp
   if (workspace != nullptr && pool_blocked_bytes(dtype, p) > 0 && reinterpret_cast<uintptr_t>(input) % 8 == 0 &&
       reinterpret_cast<uintptr_t>(workspace) % 8 == 0) {
     const long rows = static_cast<long>(p.D) * p.H;
-    const int Wb = p.W / 4;
-    const dim3 grid(static_cast<unsigned>(p.N * rows), (Wb + 15) / 16, (p.C + 63) / 64);
-    if (p.N * rows < (1L << 31) && grid.y <= 65535 && grid.z <= 65535) {
-      hipLaunchKernelGGL(pool_block_features_kernel, grid, dim3(256), 0, s, static_cast<const uint2 *>(input),
-                         static_cast<uint2 *>(workspace), p.C, rows, Wb);
+    const int Wb = p.W / 4, ux = std::min(Wb, kBlockUnits);
+    const long copy_blocks = p.N * rows * ((Wb + ux - 1) / ux) * ((p.C + 63) / 64);
+    if (copy_blocks + 1 < (1L << 31)) {
+      unsigned *ord = nullptr;   // (behind the copy; its size is a multiple of 8 bytes)
+      if (p.R <= kOrderMaxRois)
+        ord = reinterpret_cast<unsigned *>(static_cast<char *>(workspace) + static_cast<size_t>(p.N) * rows * p.W * p.C * 2);
+      hipLaunchKernelGGL(pool_block_features_kernel, dim3(static_cast<unsigned>(copy_blocks + (ord ? 1 : 0))), dim3(256), 0, s,
+                         static_cast<const uint2 *>(input), static_cast<uint2 *>(workspace), p.C, rows, Wb,
+                         static_cast<const float *>(rois), ord, p.R, p.ndim,
+                         static_cast<float>(p.scale));
       blocked = workspace;
-      if (p.R <= kOrderMaxRois) {   // (behind the copy; its size is a multiple of 8 bytes)
-        unsigned *ord = reinterpret_cast<unsigned *>(static_cast<char *>(workspace) + static_cast<size_t>(p.N) * rows * p.W * p.C * 2);
-        hipLaunchKernelGGL(pool_order_rois_kernel, dim3(1), dim3(1024), 0, s, static_cast<const float *>(rois), ord,
-                           p.R, p.ndim, static_cast<float>(p.scale));
-        order = ord;
-      }
+      order = ord;
     }
   }
   const int cpb = pool_channels_per_block(p);
