@@ -325,14 +325,17 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
       const_cast<T *>(src), 0, static_cast<int>(range_bytes), 0x00020000);
   const int plane_bytes = static_cast<int>(plane) * ES;
   constexpr unsigned kNowhere = 0x80000000u;
-  // this lane's row of the left operand: channel col / 4 of the tile, slice col % 4 of the group
+  // The row of the left operand this lane LOADS: channel col % 4 of the tile, slice col / 4 of the
+  // group, so that four neighbouring lanes read the four channels of one place (32 contiguous bytes
+  // of the blocked copy: one request instead of four).  The accumulator rows come out as (slice,
+  // channel) and are transposed across the four lane groups before the second product.
   // (blocked copy: [slice][row][unit of four columns][channel][4], a unit of one channel is 8 bytes)
   const unsigned unit_row = static_cast<unsigned>(Wb) * p.C * 8u;   // bytes of one row of units
   const unsigned row_off =
-      blocked ? static_cast<unsigned>((static_cast<long>(z_lo + col % 4) * p.H + y_lo) * unit_row) +
-                    static_cast<unsigned>(xb_lo) * p.C * 8u + static_cast<unsigned>(col / 4) * 8u
-              : static_cast<unsigned>(((static_cast<long>(z_lo + col % 4) * p.H + y_lo) * p.W + x_lo) * ES) +
-                    static_cast<unsigned>(col / 4) * static_cast<unsigned>(plane_bytes);
+      blocked ? static_cast<unsigned>((static_cast<long>(z_lo + col / 4) * p.H + y_lo) * unit_row) +
+                    static_cast<unsigned>(xb_lo) * p.C * 8u + static_cast<unsigned>(col % 4) * 8u
+              : static_cast<unsigned>(((static_cast<long>(z_lo + col / 4) * p.H + y_lo) * p.W + x_lo) * ES) +
+                    static_cast<unsigned>(col % 4) * static_cast<unsigned>(plane_bytes);
   const int tile_bytes = blocked ? 4 * 8 : 4 * plane_bytes;                       // from one tile of four channels to the next
   const int group_bytes = blocked ? 4 * p.H * static_cast<int>(unit_row) : 4 * hw * ES;   // from one group of four slices to the next
   // the two pieces of the lane's K positions in step ks: byte offset inside the slice and the masks
@@ -390,8 +393,8 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
   };
   auto issue = [&](const Step &st, Loaded &ld) {
     // rows whose slice lies outside the box read zeros
-    const unsigned row0 = st.zg * 4 + col % 4 < nz ? row_off : kNowhere;
-    const unsigned row1 = st.zg * 4 + 4 + col % 4 < nz ? row_off : kNowhere;
+    const unsigned row0 = st.zg * 4 + col / 4 < nz ? row_off : kNowhere;
+    const unsigned row1 = st.zg * 4 + 4 + col / 4 < nz ? row_off : kNowhere;
     const int soff = st.tile * tile_bytes + st.zg * group_bytes;
     ld.pa = piece(st.k0 / 4 + quad * 2);
     ld.pb = piece(st.k0 / 4 + quad * 2 + 1);
@@ -442,6 +445,18 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
       }
     }
     if (cur.k0 + 32 >= KP) {
+      // rows (slice, channel) -> (channel, slice): register r of lane group q becomes register q of
+      // lane group r (v_permlane32_swap exchanges the upper half of one register with the lower half
+      // of another, v_permlane16_swap the odd 16-lane rows of one with the even rows of another)
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        float4_t &v = acc[i / 4][i % 4];
+        const auto s02 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[0]), __float_as_uint(v[2]), false, false);
+        const auto s13 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[1]), __float_as_uint(v[3]), false, false);
+        const auto n01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
+        const auto n23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
+        v = float4_t{__uint_as_float(n01[0]), __uint_as_float(n01[1]), __uint_as_float(n23[0]), __uint_as_float(n23[1])};
+      }
       // contraction over the (up to eight) slices of the two groups
       u32x4 zhi[2] = {zhi0[0], zhi0[1]}, zlo[2] = {zlo0[0], zlo0[1]};
       if (cur.zg > 0) z_pieces(cur.zg, zhi, zlo);
