@@ -355,34 +355,32 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
     return e;
   };
   // right-hand side of the z product for the stage that starts with slice group zg: column n = 16 h + col
-  // is (channel' = n / 8, pd = n % 8); this lane's K group is channel `quad`, slices 4 zg .. 4 zg + 7
-  auto z_pieces = [&](int zg, u32x4 (&zhi)[2], u32x4 (&zlo)[2]) {
+  // is (channel' = n / 8, pd = n % 8); this lane's K group is channel `quad`, slices 4 zg .. 4 zg + 7, so
+  // its pieces are zero except in the half h = quad / 2 (and there only for col / 8 == quad % 2)
+  auto z_pieces = [&](int zg, u32x4 &zhi, u32x4 &zlo) {
+    const int pd = col % 8;
+    const bool mine = col / 8 == quad % 2;
+    float zw[8], zr[8];
 #pragma unroll
-    for (int h = 0; h < 2; h++) {
-      const int n = 16 * h + col, pd = n % 8;
-      const bool mine = n / 8 == quad;
-      float zw[8], zr[8];
-#pragma unroll
-      for (int i = 0; i < 8; i++) {
-        const int z = zg * 4 + i;
-        zw[i] = (mine && z < nz) ? wd[2][z < kDenseSrc ? z : 0][pd] : 0.f;
-      }
-      zhi[h] = M::pack(zw);
-      zr[0] = zw[0] - M::lo(zhi[h].x); zr[1] = zw[1] - M::hi(zhi[h].x);
-      zr[2] = zw[2] - M::lo(zhi[h].y); zr[3] = zw[3] - M::hi(zhi[h].y);
-      zr[4] = zw[4] - M::lo(zhi[h].z); zr[5] = zw[5] - M::hi(zhi[h].z);
-      zr[6] = zw[6] - M::lo(zhi[h].w); zr[7] = zw[7] - M::hi(zhi[h].w);
-      zlo[h] = M::pack(zr);
+    for (int i = 0; i < 8; i++) {
+      const int z = zg * 4 + i;
+      zw[i] = (mine && z < nz) ? wd[2][z < kDenseSrc ? z : 0][pd] : 0.f;
     }
+    zhi = M::pack(zw);
+    zr[0] = zw[0] - M::lo(zhi.x); zr[1] = zw[1] - M::hi(zhi.x);
+    zr[2] = zw[2] - M::lo(zhi.y); zr[3] = zw[3] - M::hi(zhi.y);
+    zr[4] = zw[4] - M::lo(zhi.z); zr[5] = zw[5] - M::hi(zhi.z);
+    zr[6] = zw[6] - M::lo(zhi.w); zr[7] = zw[7] - M::hi(zhi.w);
+    zlo = M::pack(zr);
   };
-  u32x4 zhi0[2], zlo0[2];
+  u32x4 zhi0, zlo0;
   z_pieces(0, zhi0, zlo0);
   // The steps (tile, slice-group pair, K step of 32) of this wavefront form one sequence; the loads
   // of a step are issued one step ahead, so they are in flight during the previous step's products
   // and stores.
   const int tiles = (c_count + 3) / 4;
   struct Step { int tile, zg, k0; };
-  struct Loaded { u32x2 va[2], vb[2]; Piece pa, pb; };
+  struct Loaded { u32x2 va[2], vb[2]; };
   auto next_of = [&](Step st) {
     st.k0 += 32;
     if (st.k0 >= KP) {
@@ -393,35 +391,33 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
   };
   auto issue = [&](const Step &st, Loaded &ld) {
     // rows whose slice lies outside the box read zeros
-    const unsigned row0 = st.zg * 4 + col / 4 < nz ? row_off : kNowhere;
-    const unsigned row1 = st.zg * 4 + 4 + col / 4 < nz ? row_off : kNowhere;
-    const int soff = st.tile * tile_bytes + st.zg * group_bytes;
-    ld.pa = piece(st.k0 / 4 + quad * 2);
-    ld.pb = piece(st.k0 / 4 + quad * 2 + 1);
+    // (a step beyond the last tile loads nothing: the number of loads per step stays fixed, so the
+    // wait before a step's products can leave the loads of the next step in flight)
+    const bool any = st.tile < tiles;
+    const unsigned row0 = any && st.zg * 4 + col / 4 < nz ? row_off : kNowhere;
+    const unsigned row1 = any && st.zg * 4 + 4 + col / 4 < nz ? row_off : kNowhere;
+    const int soff = any ? st.tile * tile_bytes + st.zg * group_bytes : 0;
+    const Piece pa = piece(st.k0 / 4 + quad * 2), pb = piece(st.k0 / 4 + quad * 2 + 1);
 #pragma unroll
     for (int zs = 0; zs < 2; zs++) {
       const unsigned row = zs == 0 ? row0 : row1;
       // (an offset with the top bit set is beyond the range, whatever the other term adds)
-      const unsigned at_a = (row + ld.pa.off) | ((row | ld.pa.off) & kNowhere);
+      const unsigned at_a = (row + pa.off) | ((row | pa.off) & kNowhere);
       if (QX % 2 == 0 && !blocked) {   // both pieces lie in one box row: one 16-byte load
         const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(fr, at_a, soff + zs * group_bytes, 0);
         ld.va[zs] = u32x2{v.x, v.y};
         ld.vb[zs] = u32x2{v.z, v.w};
       } else {
         ld.va[zs] = __builtin_amdgcn_raw_buffer_load_b64(fr, at_a, soff + zs * group_bytes, 0);
-        ld.vb[zs] = __builtin_amdgcn_raw_buffer_load_b64(fr, (row + ld.pb.off) | ((row | ld.pb.off) & kNowhere), soff + zs * group_bytes, 0);
+        ld.vb[zs] = __builtin_amdgcn_raw_buffer_load_b64(fr, (row + pb.off) | ((row | pb.off) & kNowhere), soff + zs * group_bytes, 0);
       }
     }
   };
-  Step cur{2 * wave, 0, 0};   // tiles 2 w, 2 w + 1, then 2 (w + 4), ...: neighbours in memory back to back
-  Loaded ld;
-  if (cur.tile < tiles) issue(cur, ld);
   float4_t oacc[4][2];   // [cell tile][half of the (channel', pd) columns]: cells 4 * quad .. + 3 of the tile
   float4_t acc[2][4];    // [slice group][cell tile]
-  while (cur.tile < tiles) {
-    const Step nxt = next_of(cur);
-    Loaded ahead;
-    if (nxt.tile < tiles) issue(nxt, ahead);
+  u32x4 kept[2][2];      // [half of the columns][run of eight cells]: a finished tile, packed
+  int kept_tile = -1;
+  auto products = [&](const Step &cur, const Loaded &ld) {
     if (cur.k0 == 0) {
 #pragma unroll
       for (int i = 0; i < 8; i++) {
@@ -430,6 +426,7 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
       }
     }
     {
+      const Piece pa = piece(cur.k0 / 4 + quad * 2), pb = piece(cur.k0 / 4 + quad * 2 + 1);   // (for the masks)
       u32x4 b[4];
 #pragma unroll
       for (int nt = 0; nt < 4; nt++)
@@ -437,8 +434,8 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
 #pragma unroll
       for (int zs = 0; zs < 2; zs++) {
         if (cur.zg + zs < zgroups) {
-          const u32x4 a = u32x4{ld.va[zs].x & ld.pa.keep_lo, ld.va[zs].y & ld.pa.keep_hi,
-                                ld.vb[zs].x & ld.pb.keep_lo, ld.vb[zs].y & ld.pb.keep_hi};
+          const u32x4 a = u32x4{ld.va[zs].x & pa.keep_lo, ld.va[zs].y & pa.keep_hi,
+                                ld.vb[zs].x & pb.keep_lo, ld.vb[zs].y & pb.keep_hi};
 #pragma unroll
           for (int nt = 0; nt < 4; nt++) acc[zs][nt] = M::run16(a, b[nt], acc[zs][nt]);
         }
@@ -458,51 +455,96 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
         v = float4_t{__uint_as_float(n01[0]), __uint_as_float(n01[1]), __uint_as_float(n23[0]), __uint_as_float(n23[1])};
       }
       // contraction over the (up to eight) slices of the two groups
-      u32x4 zhi[2] = {zhi0[0], zhi0[1]}, zlo[2] = {zlo0[0], zlo0[1]};
+      u32x4 zhi = zhi0, zlo = zlo0;
       if (cur.zg > 0) z_pieces(cur.zg, zhi, zlo);
+      const u32x4 none = u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
-      for (int nt = 0; nt < 4; nt++) {
-        const u32x4 ta = u32x4{M::pack2(acc[0][nt][0], acc[0][nt][1]), M::pack2(acc[0][nt][2], acc[0][nt][3]),
-                               M::pack2(acc[1][nt][0], acc[1][nt][1]), M::pack2(acc[1][nt][2], acc[1][nt][3])};
+      for (int h = 0; h < 2; h++) {
+        const u32x4 zh = quad / 2 == h ? zhi : none, zl = quad / 2 == h ? zlo : none;
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
-          oacc[nt][h] = M::run16(ta, zlo[h], oacc[nt][h]);
-          oacc[nt][h] = M::run16(ta, zhi[h], oacc[nt][h]);
+        for (int nt = 0; nt < 4; nt++) {
+          const u32x4 ta = u32x4{M::pack2(acc[0][nt][0], acc[0][nt][1]), M::pack2(acc[0][nt][2], acc[0][nt][3]),
+                                 M::pack2(acc[1][nt][0], acc[1][nt][1]), M::pack2(acc[1][nt][2], acc[1][nt][3])};
+          oacc[nt][h] = M::run16(ta, zl, oacc[nt][h]);
+          oacc[nt][h] = M::run16(ta, zh, oacc[nt][h]);
         }
       }
       if (cur.zg + 2 >= zgroups) {
         // register r of oacc[nt][h]: cell (nt / 2) * 32 + 8 * quad + (nt % 2) * 4 + r (the order in which
         // the weight rows were read) of (channel 4 tile + 2 h + col / 8, pd col % 8): a lane holds
-        // two runs of eight neighbouring cells
+        // two runs of eight neighbouring cells.  They are kept packed and stored during the next step.
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
-          const int c = cur.tile * 4 + 2 * h + col / 8, pd = col % 8;
-          if (c < c_count && pd < p.od) {
-            T *o = dst + static_cast<long>(c) * cells + pd * ohw;
+        for (int h = 0; h < 2; h++)
 #pragma unroll
-            for (int half = 0; half < 2; half++) {
-              const int n = half * 32 + 8 * quad;
-              if (n + 7 < ohw) {   // eight neighbouring cells as one 16-byte store (2-byte aligned)
-                struct __attribute__((packed, aligned(2))) Cells8 { unsigned v[4]; };
-                Cells8 v8;
-                v8.v[0] = M::pack2(oacc[2 * half][h][0], oacc[2 * half][h][1]);
-                v8.v[1] = M::pack2(oacc[2 * half][h][2], oacc[2 * half][h][3]);
-                v8.v[2] = M::pack2(oacc[2 * half + 1][h][0], oacc[2 * half + 1][h][1]);
-                v8.v[3] = M::pack2(oacc[2 * half + 1][h][2], oacc[2 * half + 1][h][3]);
-                *reinterpret_cast<Cells8 *>(o + n) = v8;
-              } else {
+          for (int half = 0; half < 2; half++)
+            kept[h][half] = u32x4{M::pack2(oacc[2 * half][h][0], oacc[2 * half][h][1]),
+                                  M::pack2(oacc[2 * half][h][2], oacc[2 * half][h][3]),
+                                  M::pack2(oacc[2 * half + 1][h][0], oacc[2 * half + 1][h][1]),
+                                  M::pack2(oacc[2 * half + 1][h][2], oacc[2 * half + 1][h][3])};
+        kept_tile = cur.tile;
+      }
+    }
+  };
+  // The stores of a finished tile wait in `kept` until the loads of the following step have arrived:
+  // a wait for loads also waits for every store issued before it, and a store takes as long as a load.
+  auto store_kept = [&]() {
+    if (kept_tile < 0) return;
 #pragma unroll
-                for (int r = 0; r < 8; r++)
-                  if (n + r < ohw) o[n + r] = store_cast<T>(oacc[2 * half + r / 4][h][r % 4]);
-              }
-            }
+    for (int h = 0; h < 2; h++) {
+      const int c = kept_tile * 4 + 2 * h + col / 8, pd = col % 8;
+      if (c < c_count && pd < p.od) {
+        T *o = dst + static_cast<long>(c) * cells + pd * ohw;
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+          const int n = half * 32 + 8 * quad;
+          const u32x4 v = kept[h][half];
+          struct __attribute__((packed, aligned(2))) Cells8 { unsigned v[4]; };
+          struct __attribute__((packed, aligned(2))) Cells4 { unsigned v[2]; };
+          struct __attribute__((packed, aligned(2))) Cells2 { unsigned v; };
+          const int left = ohw - n;   // cells of this run that exist
+          if (left >= 8) {            // eight neighbouring cells as one 16-byte store (2-byte aligned)
+            *reinterpret_cast<Cells8 *>(o + n) = Cells8{{v.x, v.y, v.z, v.w}};
+          } else if (left > 0) {      // 4 + 2 + 1 cells
+            const bool l4 = left & 4, l2 = left & 2;
+            if (l4) *reinterpret_cast<Cells4 *>(o + n) = Cells4{{v.x, v.y}};
+            if (l2) *reinterpret_cast<Cells2 *>(o + n + (left & 4)) = Cells2{l4 ? v.z : v.x};
+            if (left & 1)
+              reinterpret_cast<unsigned short *>(o)[n + (left & 6)] =
+                  static_cast<unsigned short>(l4 ? (l2 ? v.w : v.z) : (l2 ? v.y : v.x));
           }
         }
       }
     }
-    cur = nxt;
-    ld = ahead;
+    kept_tile = -1;
+  };
+  // a use of the loaded registers that the compiler cannot move: the wait for them lands here
+  auto arrived = [&](Loaded &ld) {
+    asm volatile("" : "+v"(ld.va[0]), "+v"(ld.va[1]), "+v"(ld.vb[0]), "+v"(ld.vb[1]) : : "memory");
+  };
+  // kAhead sets of load registers used in turn: while a step's products run, the loads of the next
+  // kAhead - 1 steps are in flight (a wavefront spends most of a tile waiting for memory otherwise).
+  constexpr int kAhead = 3;
+  Step q[kAhead];
+  Loaded ld[kAhead];
+  q[0] = Step{2 * wave, 0, 0};   // tiles 2 w, 2 w + 1, then 2 (w + 4), ...: neighbours in memory back to back
+#pragma unroll
+  for (int u = 0; u < kAhead; u++) {
+    if (u > 0) q[u] = next_of(q[u - 1]);
+    issue(q[u], ld[u]);
   }
+  while (q[0].tile < tiles) {   // (q[0] is the oldest step here)
+#pragma unroll
+    for (int u = 0; u < kAhead; u++) {
+      arrived(ld[u]);
+      if (q[u].tile < tiles) {
+        store_kept();
+        products(q[u], ld[u]);
+      }
+      q[u] = next_of(q[(u + kAhead - 1) % kAhead]);
+      issue(q[u], ld[u]);
+    }
+  }
+  store_kept();
 }
 
 template <typename T, typename RT, int CELLS>
