@@ -297,26 +297,7 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
   const int zgroups = (nz + 3) / 4;
   const int tid = threadIdx.x, lane = tid % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);   // (a scalar for the compiler too)
-  const float inv_ow = 1.f / p.ow, inv_nxp = 1.f / NXP, inv_qx = 1.f / QX;
-  {  // weight products: thread = (cell, quarter of the K range), pairs of neighbouring K
-    const int n = tid / 4, q = tid % 4, ph = fdiv(n, inv_ow), pw = n - ph * p.ow;
-    const bool nv = n < ohw;
-    const int kq = KP / 4;
-    int k = q * kq, y = fdiv(k, inv_nxp), x = k - y * NXP;
-    T *wr = w + n * WS + k;
-    for (int i = 0; i < kq; i += 2) {
-      float v[2];
-#pragma unroll
-      for (int e = 0; e < 2; e++) {
-        const int xr = x - x_shift;   // column of the box
-        v[e] = (nv && y < ny && xr >= 0 && xr < nx) ? wd[1][y < ny ? y : 0][ph & 7] * wd[0][(xr >= 0 && xr < nx) ? xr : 0][pw] : 0.f;
-        x++;
-        if (x == NXP) { x = 0; y++; }
-      }
-      *reinterpret_cast<unsigned *>(wr + i) = M::pack2(v[0], v[1]);
-    }
-  }
-  __syncthreads();
+  const float inv_ow = 1.f / p.ow, inv_qx = 1.f / QX;
   const int col = lane % 16, quad = lane / 16;
   const unsigned long long sp = reinterpret_cast<unsigned long long>(src_any);
   const T *src = reinterpret_cast<const T *>(static_cast<unsigned long long>(static_cast<unsigned>(uni(static_cast<int>(sp)))) |
@@ -413,6 +394,40 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
       }
     }
   };
+  // kAhead sets of load registers used in turn: while a step's products run, the loads of the next
+  // kAhead - 1 steps are in flight (a wavefront spends most of a tile waiting for memory otherwise).
+  constexpr int kAhead = 3;
+  Step q[kAhead];
+  Loaded ld[kAhead];
+  q[0] = Step{2 * wave, 0, 0};   // tiles 2 w, 2 w + 1, then 2 (w + 4), ...: neighbours in memory back to back
+#pragma unroll
+  for (int u = 0; u < kAhead; u++) {
+    if (u > 0) q[u] = next_of(q[u - 1]);
+    issue(q[u], ld[u]);
+  }
+  // (the first loads are under way while the weight products are formed)
+  {  // weight products: thread = (cell, every fourth piece of four neighbouring K); the iterations
+     // are independent, so their LDS reads overlap
+    const int n = tid / 4, q = tid % 4, ph = fdiv(n, inv_ow), pw = n - ph * p.ow;
+    const bool nv = n < ohw;
+    uint2 *wr = reinterpret_cast<uint2 *>(w + n * WS);
+    for (int m0 = q; m0 < KP / 4; m0 += 8) {   // (KP / 4 is a multiple of eight)
+#pragma unroll
+      for (int u = 0; u < 2; u++) {
+        const int m = m0 + 4 * u;
+        const int y = fdiv(m, inv_qx), x0 = (m - y * QX) * 4 - x_shift;   // first column of the piece in the box
+        const float wy = (nv && y < ny) ? wd[1][y < ny ? y : 0][ph & 7] : 0.f;
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const bool in = x0 + j >= 0 && x0 + j < nx;
+          v[j] = in ? wy * wd[0][in ? x0 + j : 0][pw] : 0.f;
+        }
+        wr[m] = uint2{M::pack2(v[0], v[1]), M::pack2(v[2], v[3])};
+      }
+    }
+  }
+  __syncthreads();
   float4_t oacc[4][2];   // [cell tile][half of the (channel', pd) columns]: cells 4 * quad .. + 3 of the tile
   float4_t acc[2][4];    // [slice group][cell tile]
   u32x4 kept[2][2];      // [half of the columns][run of eight cells]: a finished tile, packed
@@ -420,10 +435,11 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
   auto products = [&](const Step &cur, const Loaded &ld) {
     if (cur.k0 == 0) {
 #pragma unroll
-      for (int i = 0; i < 8; i++) {
-        acc[i / 4][i % 4] = float4_t{0.f, 0.f, 0.f, 0.f};
-        if (cur.zg == 0) oacc[i / 2][i % 2] = float4_t{0.f, 0.f, 0.f, 0.f};
-      }
+      for (int i = 0; i < 8; i++) acc[i / 4][i % 4] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+    if (cur.k0 == 0 && cur.zg == 0) {
+#pragma unroll
+      for (int i = 0; i < 8; i++) oacc[i / 2][i % 2] = float4_t{0.f, 0.f, 0.f, 0.f};
     }
     {
       const Piece pa = piece(cur.k0 / 4 + quad * 2), pb = piece(cur.k0 / 4 + quad * 2 + 1);   // (for the masks)
@@ -521,17 +537,6 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
   auto arrived = [&](Loaded &ld) {
     asm volatile("" : "+v"(ld.va[0]), "+v"(ld.va[1]), "+v"(ld.vb[0]), "+v"(ld.vb[1]) : : "memory");
   };
-  // kAhead sets of load registers used in turn: while a step's products run, the loads of the next
-  // kAhead - 1 steps are in flight (a wavefront spends most of a tile waiting for memory otherwise).
-  constexpr int kAhead = 3;
-  Step q[kAhead];
-  Loaded ld[kAhead];
-  q[0] = Step{2 * wave, 0, 0};   // tiles 2 w, 2 w + 1, then 2 (w + 4), ...: neighbours in memory back to back
-#pragma unroll
-  for (int u = 0; u < kAhead; u++) {
-    if (u > 0) q[u] = next_of(q[u - 1]);
-    issue(q[u], ld[u]);
-  }
   while (q[0].tile < tiles) {   // (q[0] is the oldest step here)
 #pragma unroll
     for (int u = 0; u < kAhead; u++) {
