@@ -558,7 +558,7 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
     const int channels_per_block, const T *__restrict__ blocked, const int Wb, const unsigned *__restrict__ order) {
   __shared__ PoolShared sh;
   __shared__ __attribute__((aligned(16))) unsigned char lds[kPoolLdsBytes];
-  const unsigned n = order ? order[blockIdx.x] : blockIdx.x;   // (largest rois first, see pool_order_rois_kernel)
+  const unsigned n = order ? order[blockIdx.x] : blockIdx.x;   // (largest rois first, see pool_order_rois)
   const int c_begin = blockIdx.y * channels_per_block, c_end = min(c_begin + channels_per_block, p.C);
   __shared__ __attribute__((aligned(16))) float wd[3][kDenseSrc][CELLS];
   const PoolPlan plan = pool_setup<RT, CELLS>(sh, rois + static_cast<long>(n) * roi_columns(p.ndim, 0), p, sizeof(T),
