@@ -589,15 +589,24 @@ __global__ __launch_bounds__(256, 5) void dcn_forward_shared_taps_kernel(
   }
   const long qo = q0 + 16 * wave + j;
   if (qo >= s.Q) return;
+  // 16x16 accumulator layout: register r of lane l holds row 4 * (l / 16) + r, column l % 16.
+  // All bias values first (the lane's four channels of a block are 8 contiguous bytes; no bias: an
+  // empty range), then the stores: a load between two stores would wait for the first.
+  typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+  const __amdgpu_buffer_rsrc_t br = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T *>(bias), 0, bias ? s.Cout * ES : 0, 0x00020000);
+  u32x2 braw[MB];
+#pragma unroll
+  for (int m = 0; m < MB; m++)
+    braw[m] = __builtin_amdgcn_raw_buffer_load_b64(br, (g * s.opg + (mb0 + m) * 16 + kc * 4) * ES, 0, 0);
 #pragma unroll
   for (int m = 0; m < MB; m++) {
     if (mb0 + m >= blocks) continue;
+    const float bv[4] = {M::lo(braw[m].x), M::hi(braw[m].x), M::lo(braw[m].y), M::hi(braw[m].y)};
 #pragma unroll
     for (int r = 0; r < 4; r++) {
-      // 16x16 accumulator layout: register r of lane l holds row 4 * (l / 16) + r, column l % 16
       const int o = g * s.opg + (mb0 + m) * 16 + kc * 4 + r;
-      const float val = acc[m][r] + (bias ? load(bias + o) : 0.f);
-      y[(static_cast<long>(b) * s.Cout + o) * s.Q + qo] = store_cast<T>(val);
+      y[(static_cast<long>(b) * s.Cout + o) * s.Q + qo] = store_cast<T>(acc[m][r] + bv[r]);
     }
   }
 }
