@@ -335,27 +335,29 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
     e.keep_hi = left >= 4 ? 0xffffffffu : (left == 3 ? 0x0000ffffu : 0u);
     return e;
   };
-  // right-hand side of the z product for the stage that starts with slice group zg: column n = 16 h + col
-  // is (channel' = n / 8, pd = n % 8); this lane's K group is channel `quad`, slices 4 zg .. 4 zg + 7, so
-  // its pieces are zero except in the half h = quad / 2 (and there only for col / 8 == quad % 2)
-  auto z_pieces = [&](int zg, u32x4 &zhi, u32x4 &zlo) {
-    const int pd = col % 8;
-    const bool mine = col / 8 == quad % 2;
-    float zw[8], zr[8];
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-      const int z = zg * 4 + i;
-      zw[i] = (mine && z < nz) ? wd[2][z < kDenseSrc ? z : 0][pd] : 0.f;
-    }
-    zhi = M::pack(zw);
-    zr[0] = zw[0] - M::lo(zhi.x); zr[1] = zw[1] - M::hi(zhi.x);
-    zr[2] = zw[2] - M::lo(zhi.y); zr[3] = zw[3] - M::hi(zhi.y);
-    zr[4] = zw[4] - M::lo(zhi.z); zr[5] = zw[5] - M::hi(zhi.z);
-    zr[6] = zw[6] - M::lo(zhi.w); zr[7] = zw[7] - M::hi(zhi.w);
-    zlo = M::pack(zr);
+  // Right-hand side of the z product for the stage that starts with slice group zg.  The accumulator
+  // of the first product hands lane group `quad` the rows (slice quad, channels 0..3) of each of the
+  // two slice groups: packed, that is the K piece {(slice 4 zg + quad, channel i), i = 0..3;
+  // (slice 4 zg + 4 + quad, channel i)} of the second product.  Column n = 16 h + col of its
+  // right-hand side is (channel' = n / 8, pd = n % 8), block-diagonal in the channel: of the lane's
+  // eight elements only i = channel' and i = channel' + 4 are non-zero, Wz[slice][pd] each.  As fp16
+  // pairs: dword h, half col / 8 for the first slice group, dword 2 + h for the second; the two
+  // weights are kept as a high and a low fp16 part.
+  struct ZPair { unsigned a_hi, b_hi, a_lo, b_lo; };
+  auto z_pair = [&](int zg) {
+    const int pd = col % 8, za_i = zg * 4 + quad, zb_i = za_i + 4;
+    const bool up = col / 8 != 0;
+    const float za = za_i < nz ? wd[2][za_i < kDenseSrc ? za_i : 0][pd] : 0.f;
+    const float zb = zb_i < nz ? wd[2][zb_i < kDenseSrc ? zb_i : 0][pd] : 0.f;
+    ZPair z;
+    z.a_hi = M::pack2(up ? 0.f : za, up ? za : 0.f);
+    z.b_hi = M::pack2(up ? 0.f : zb, up ? zb : 0.f);
+    const float ra = za - (up ? M::hi(z.a_hi) : M::lo(z.a_hi)), rb = zb - (up ? M::hi(z.b_hi) : M::lo(z.b_hi));
+    z.a_lo = M::pack2(up ? 0.f : ra, up ? ra : 0.f);
+    z.b_lo = M::pack2(up ? 0.f : rb, up ? rb : 0.f);
+    return z;
   };
-  u32x4 zhi0, zlo0;
-  z_pieces(0, zhi0, zlo0);
+  const ZPair z0 = z_pair(0);
   // The steps (tile, slice-group pair, K step of 32) of this wavefront form one sequence; the loads
   // of a step are issued one step ahead, so they are in flight during the previous step's products
   // and stores.
@@ -458,31 +460,19 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
       }
     }
     if (cur.k0 + 32 >= KP) {
-      // rows (slice, channel) -> (channel, slice): register r of lane group q becomes register q of
-      // lane group r (v_permlane32_swap exchanges the upper half of one register with the lower half
-      // of another, v_permlane16_swap the odd 16-lane rows of one with the even rows of another)
-#pragma unroll
-      for (int i = 0; i < 8; i++) {
-        float4_t &v = acc[i / 4][i % 4];
-        const auto s02 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[0]), __float_as_uint(v[2]), false, false);
-        const auto s13 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[1]), __float_as_uint(v[3]), false, false);
-        const auto n01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
-        const auto n23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
-        v = float4_t{__uint_as_float(n01[0]), __uint_as_float(n01[1]), __uint_as_float(n23[0]), __uint_as_float(n23[1])};
-      }
       // contraction over the (up to eight) slices of the two groups
-      u32x4 zhi = zhi0, zlo = zlo0;
-      if (cur.zg > 0) z_pieces(cur.zg, zhi, zlo);
-      const u32x4 none = u32x4{0u, 0u, 0u, 0u};
+      ZPair z = z0;
+      if (cur.zg > 0) z = z_pair(cur.zg);
+      const u32x4 zh[2] = {u32x4{z.a_hi, 0u, z.b_hi, 0u}, u32x4{0u, z.a_hi, 0u, z.b_hi}};
+      const u32x4 zl[2] = {u32x4{z.a_lo, 0u, z.b_lo, 0u}, u32x4{0u, z.a_lo, 0u, z.b_lo}};
 #pragma unroll
-      for (int h = 0; h < 2; h++) {
-        const u32x4 zh = quad / 2 == h ? zhi : none, zl = quad / 2 == h ? zlo : none;
+      for (int nt = 0; nt < 4; nt++) {
+        const u32x4 ta = u32x4{M::pack2(acc[0][nt][0], acc[0][nt][1]), M::pack2(acc[0][nt][2], acc[0][nt][3]),
+                               M::pack2(acc[1][nt][0], acc[1][nt][1]), M::pack2(acc[1][nt][2], acc[1][nt][3])};
 #pragma unroll
-        for (int nt = 0; nt < 4; nt++) {
-          const u32x4 ta = u32x4{M::pack2(acc[0][nt][0], acc[0][nt][1]), M::pack2(acc[0][nt][2], acc[0][nt][3]),
-                                 M::pack2(acc[1][nt][0], acc[1][nt][1]), M::pack2(acc[1][nt][2], acc[1][nt][3])};
-          oacc[nt][h] = M::run16(ta, zl, oacc[nt][h]);
-          oacc[nt][h] = M::run16(ta, zh, oacc[nt][h]);
+        for (int h = 0; h < 2; h++) {
+          oacc[nt][h] = M::run16(ta, zl[h], oacc[nt][h]);
+          oacc[nt][h] = M::run16(ta, zh[h], oacc[nt][h]);
         }
       }
       if (cur.zg + 2 >= zgroups) {
