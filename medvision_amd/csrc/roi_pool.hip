@@ -372,6 +372,7 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
     }
     return st;
   };
+  const Piece pa0 = piece(quad * 2), pb0 = piece(quad * 2 + 1);   // the pieces of the first K step
   auto issue = [&](const Step &st, Loaded &ld) {
     // rows whose slice lies outside the box read zeros
     // (a step beyond the last tile loads nothing: the number of loads per step stays fixed, so the
@@ -380,7 +381,8 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
     const unsigned row0 = any && st.zg * 4 + col / 4 < nz ? row_off : kNowhere;
     const unsigned row1 = any && st.zg * 4 + 4 + col / 4 < nz ? row_off : kNowhere;
     const int soff = any ? st.tile * tile_bytes + st.zg * group_bytes : 0;
-    const Piece pa = piece(st.k0 / 4 + quad * 2), pb = piece(st.k0 / 4 + quad * 2 + 1);
+    Piece pa = pa0, pb = pb0;   // (most boxes have one K step)
+    if (st.k0 != 0) { pa = piece(st.k0 / 4 + quad * 2); pb = piece(st.k0 / 4 + quad * 2 + 1); }
 #pragma unroll
     for (int zs = 0; zs < 2; zs++) {
       const unsigned row = zs == 0 ? row0 : row1;
@@ -444,7 +446,8 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
       for (int i = 0; i < 8; i++) oacc[i / 2][i % 2] = float4_t{0.f, 0.f, 0.f, 0.f};
     }
     {
-      const Piece pa = piece(cur.k0 / 4 + quad * 2), pb = piece(cur.k0 / 4 + quad * 2 + 1);   // (for the masks)
+      Piece pa = pa0, pb = pb0;   // (for the masks)
+      if (cur.k0 != 0) { pa = piece(cur.k0 / 4 + quad * 2); pb = piece(cur.k0 / 4 + quad * 2 + 1); }
       u32x4 b[4];
 #pragma unroll
       for (int nt = 0; nt < 4; nt++)
