@@ -496,13 +496,14 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
   };
   // The stores of a finished tile wait in `kept` until the loads of the following step have arrived:
   // a wait for loads also waits for every store issued before it, and a store takes as long as a load.
+  T *const lane_dst = dst + (col / 8) * cells + (col % 8) * ohw;   // the lane's (channel, pd) in tile 0
   auto store_kept = [&]() {
     if (kept_tile < 0) return;
 #pragma unroll
     for (int h = 0; h < 2; h++) {
       const int c = kept_tile * 4 + 2 * h + col / 8, pd = col % 8;
       if (c < c_count && pd < p.od) {
-        T *o = dst + static_cast<long>(c) * cells + pd * ohw;
+        T *o = lane_dst + (kept_tile * 4 + 2 * h) * cells;   // (the same step for every lane)
 #pragma unroll
         for (int half = 0; half < 2; half++) {
           const int n = half * 32 + 8 * quad;
