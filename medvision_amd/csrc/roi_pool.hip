@@ -255,21 +255,22 @@ __device__ __forceinline__ void dense_axpy(float (&acc)[CELLS], const float *row
 // Forward pass of one (roi, channel block) on the matrix cores, fp16 tensors, <= 8 cells per axis,
 // box rows times padded box columns <= kMfmaYx.  The contraction over (y, x) is one GEMM per group
 // of four box slices,
-//     T[(channel, slice)][(ph, pw)] = sum_(y, x) box[(channel, slice)][(y, x)] * (Wy[y][ph] Wx[x][pw]),
+//     T[(slice, channel)][(ph, pw)] = sum_(y, x) box[(slice, channel)][(y, x)] * (Wy[y][ph] Wx[x][pw]),
 // K = y * NXP + x with the box row padded to NXP = a multiple of four columns (zero weights on the
 // pad).  The weight products sit in LDS as 16-byte K pieces; the box does not: a lane's 8-element K
 // piece of the left operand is two 4-voxel pieces of a box row, which it reads straight from the
-// feature map with two 2-byte-aligned 8-byte buffer loads (per-lane offset = (channel, slice) of its
+// feature map with two 2-byte-aligned 8-byte buffer loads (per-lane offset = (slice, channel) of its
 // row plus the pieces of the K step, the tile's channels in the scalar offset; slices or channels
 // outside the box or the block read zeros through the range check, columns beyond the box row are
-// masked).  Rows are ordered (channel, slice % 4), so the 16 x 16 accumulator hands every lane the
-// four slices of ONE channel at one (ph, pw): for two slice groups that is exactly the 8-element K
-// piece of a second matrix product with rows (ph, pw), K = (channel, slice) and a block-diagonal
-// right-hand side
-//     out[(ph, pw)][(channel', pd)] = sum_(channel, z) T[(ph, pw)][(channel, z)] * (channel == channel') Wz[z][pd],
-// whose pieces every lane forms from the z matrix by itself (as an fp16 pair high + low, so the z
-// weights keep 22 bits).  The contraction over z thereby runs on the matrix cores too, without moving
-// T (it is rounded to fp16 once); a lane ends up with four neighbouring cells of one (channel, pd).
+// masked).  Rows are ordered (slice % 4, channel), so the 16 x 16 accumulator hands every lane one
+// slice of the tile's four channels at one (ph, pw): for two slice groups that is exactly the
+// 8-element K piece of a second matrix product with rows (ph, pw), K = (slice, channel) and a
+// block-diagonal right-hand side
+//     out[(ph, pw)][(channel', pd)] = sum_(z, channel) T[(ph, pw)][(z, channel)] * (channel == channel') Wz[z][pd],
+// whose pieces (two non-zero elements) every lane forms from the z matrix by itself (as an fp16 pair
+// high + low, so the z weights keep 22 bits).  The contraction over z thereby runs on the matrix
+// cores too, without moving T (it is rounded to fp16 once); a lane ends up with four neighbouring
+// cells of one (channel, pd).
 // A wavefront owns tiles of four channels and shares nothing but the weights with the others: no
 // barrier after the set-up.
 constexpr int kMfmaYx = 224;
@@ -309,7 +310,7 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
   // The row of the left operand this lane LOADS: channel col % 4 of the tile, slice col / 4 of the
   // group, so that four neighbouring lanes read the four channels of one place (32 contiguous bytes
   // of the blocked copy: one request instead of four).  The accumulator rows come out as (slice,
-  // channel) and are transposed across the four lane groups before the second product.
+  // channel), the order of the second product's K index.
   // (blocked copy: [slice][row][unit of four columns][channel][4], a unit of one channel is 8 bytes)
   const unsigned unit_row = static_cast<unsigned>(Wb) * p.C * 8u;   // bytes of one row of units
   const unsigned row_off =
