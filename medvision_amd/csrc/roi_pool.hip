@@ -1180,7 +1180,11 @@ __global__ __launch_bounds__(256) void pool_block_features_kernel(const uint2 *_
   for (int i = t; i < 64 * ux; i += 256) {
     const int cl = fdiv(i, inv_ux), xq = i - cl * ux;
     uint2 v = make_uint2(0u, 0u);
-    if (c0 + cl < C && xb0 + xq < Wb) v = src[((nimg * C + c0 + cl) * rows + r) * Wb + xb0 + xq];
+    if (c0 + cl < C && xb0 + xq < Wb) {   // (read once: nontemporal, the cache is for the copy)
+      const unsigned long long raw = __builtin_nontemporal_load(
+          reinterpret_cast<const unsigned long long *>(src + ((nimg * C + c0 + cl) * rows + r) * Wb + xb0 + xq));
+      v = make_uint2(static_cast<unsigned>(raw), static_cast<unsigned>(raw >> 32));
+    }
     tile[xq * 65 + cl] = v;
   }
   __syncthreads();
