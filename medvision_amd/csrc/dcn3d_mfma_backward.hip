@@ -835,7 +835,11 @@ __global__ __launch_bounds__(256) void dcn_planar_add_wide_kernel(const float *_
   for (int u = 0; u < 4; u++) {
     const int i = threadIdx.x + u * 256, pp = i / 16, cq = i % 16;
     in[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (cq * 4 < cn) in[u] = *reinterpret_cast<const float4 *>(src + static_cast<long>(pp) * C + cq * 4);
+    if (cq * 4 < cn) {   // (the accumulation buffer is read once and the result not read here again: nontemporal)
+      typedef float f32x4 __attribute__((ext_vector_type(4)));
+      const f32x4 t = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(src + static_cast<long>(pp) * C + cq * 4));
+      in[u] = make_float4(t.x, t.y, t.z, t.w);
+    }
   }
 #pragma unroll
   for (int u = 0; u < 4; u++) {
@@ -851,7 +855,7 @@ __global__ __launch_bounds__(256) void dcn_planar_add_wide_kernel(const float *_
     piece.u = *reinterpret_cast<const u32x4 *>(d);
 #pragma unroll
     for (int e = 0; e < V; e++) piece.e[e] = store_cast<T>(load(&piece.e[e]) + stagef[pg * V + e][c]);
-    *reinterpret_cast<u32x4 *>(d) = piece.u;
+    __builtin_nontemporal_store(piece.u, reinterpret_cast<u32x4 *>(d));
   }
 }
 
