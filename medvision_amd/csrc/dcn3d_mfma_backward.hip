@@ -353,7 +353,9 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
           const long first = q0 + 8 * (r / 4) + 4 * h;  // position of colv[0]
           T *dst = colrow + ((first / PC) * 32 + n) * PC + first % PC;
           if constexpr (ES == 2) {
-            *reinterpret_cast<uint2 *>(dst) = make_uint2(M::pack2(colv[0], colv[1]), M::pack2(colv[2], colv[3]));
+            // (nontemporal: the buffer is larger than the caches and read once, by the weight kernel)
+            __builtin_nontemporal_store((static_cast<unsigned long long>(M::pack2(colv[2], colv[3])) << 32) | M::pack2(colv[0], colv[1]),
+                                        reinterpret_cast<unsigned long long *>(dst));
           } else {
             *reinterpret_cast<float4 *>(dst) = make_float4(colv[0], colv[1], colv[2], colv[3]);
           }
@@ -755,7 +757,7 @@ __global__ __launch_bounds__(256) void dcn_backward_weight_columns_kernel(
         union { u32x4 u; T e[PC]; } piece;
         piece.u = u32x4{0u, 0u, 0u, 0u};
         if (qa < s.Q) {
-          piece.u = *reinterpret_cast<const u32x4 *>(colrow[t] + ((qa / PC) * 32 + n) * PC);
+          piece.u = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(colrow[t] + ((qa / PC) * 32 + n) * PC));   // (read once)
           if (qa + PC > s.Q) {
 #pragma unroll
             for (int i = 0; i < PC; i++)
