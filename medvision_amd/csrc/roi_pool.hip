@@ -507,12 +507,27 @@ __device__ inline void pool_forward_mfma(const T *__restrict__ src_any, T *__res
             // 32 of them, as oh * ow >= 32; behind the last row: the spare room): the runs of the
             // second half are written first, and the first halves of all rows overwrite what spilt.
             if (pd < p.od) {
-              unsigned short *row = reinterpret_cast<unsigned short *>(stage) + (2 * h + col / 8) * cells + pd * ohw + 8 * quad;
+              // A run of eight cells starts at a 2-byte-aligned place.  Where that is a multiple of
+              // 4 bytes the lane writes dwords 0..2 and the two halves of dword 3, elsewhere cell 0,
+              // the three dwords of cells 1..6 and cell 7: three 4-byte and two 2-byte writes either way
+              // (2-byte LDS writes take several times as long as 4-byte ones).
+              const int first = (2 * h + col / 8) * cells + pd * ohw + 8 * quad;   // in cells
+              const bool odd = first & 1;
+              unsigned short *row = reinterpret_cast<unsigned short *>(stage) + first;
 #pragma unroll
-              for (int half = 1; half >= 0; half--)
-#pragma unroll
-                for (int j = 0; j < 8; j++)
-                  row[half * 32 + j] = static_cast<unsigned short>(j % 2 ? run[half][j / 2] >> 16 : run[half][j / 2]);
+              for (int half = 1; half >= 0; half--) {
+                const u32x4 v = run[half];
+                unsigned short *at = row + half * 32;
+                unsigned *mid = reinterpret_cast<unsigned *>(at + (odd ? 1 : 0));
+                mid[0] = odd ? __builtin_amdgcn_alignbit(v.y, v.x, 16) : v.x;
+                mid[1] = odd ? __builtin_amdgcn_alignbit(v.z, v.y, 16) : v.y;
+                mid[2] = odd ? __builtin_amdgcn_alignbit(v.w, v.z, 16) : v.z;
+                at[odd ? 0 : 6] = static_cast<unsigned short>(odd ? v.x : v.w);
+                at[7] = static_cast<unsigned short>(v.w >> 16);
+                // (the order matters across lanes, which the compiler does not see: it may not move
+                // or merge writes of the two halves past each other)
+                asm volatile("" ::: "memory");
+              }
             }
           } else {
             const int c = cur.tile * 4 + 2 * h + col / 8;
