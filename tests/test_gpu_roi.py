@@ -353,6 +353,33 @@ def test_pooled_forward_from_blocked_copy(ops, oracle, ndim):
     assert_close(got, want[:15], FWD_TOL[torch.float16], "pooled forward from the input")
 
 
+@pytest.mark.parametrize("out", [(8, 8, 8), (3, 6, 6), (2, 5, 7), (7, 4, 8), (5, 5, 5), (6, 6), (4, 8), (5, 5)])
+@pytest.mark.parametrize("channels", [8, 12, 10])
+def test_pooled_forward_output_layouts(ops, oracle, out, channels):
+    """The matrix-core pooled forward writes a finished tile of four channels through LDS when a row
+    of cells (oh * ow) has at least 32 of them and the channel block is a whole number of tiles:
+    rows of exactly 32 and 64 cells, rows whose last run of eight is cut, rows too short for that
+    form, a channel count that is no multiple of four, outputs of odd rois (whose address is no
+    multiple of 8 bytes when channels * cells is odd), images and volumes."""
+    ndim = len(out)
+    g = wl.gen(400 + 10 * ndim + channels + sum(out))
+    size = (6, 12, 16)[3 - ndim:]
+    feat = torch.randn(2, channels, *size, generator=g).half()
+    xyz = torch.tensor(size[::-1], dtype=torch.float32)
+    cells = 1
+    for o in out:
+        cells *= o
+    n = max(40, 3 * feat[:, 0].numel() // cells)        # enough rois for the re-ordered copy of the features
+    lo = (torch.rand(n, ndim, generator=g) * 1.2 - 0.1) * xyz
+    ext = torch.exp(torch.rand(n, ndim, generator=g) * math.log(12.0)) * 0.8
+    rois = torch.cat([torch.randint(0, 2, (n, 1), generator=g).float(), lo, lo + ext], 1)
+    got = ops.RoIAlign(out, 1.0, 2)(feat.to(DEV), rois.to(DEV))
+    want = oracle.roi_align_forward(feat, rois, out, 1.0, 2)
+    assert_close(got, want, FWD_TOL[torch.float16], f"pooled forward {out} x {channels} channels")
+    got = ops.RoIAlign(out, 1.0, 2)(feat.to(DEV), rois[:7].to(DEV))      # few rois: from the input itself
+    assert_close(got, want[:7], FWD_TOL[torch.float16], f"pooled forward {out} x {channels} channels, few rois")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("sr,order", [(2, 1), (-1, 1), (3, 1), (1, 0)])
 def test_pooled_kernel_paths(ops, oracle, dtype, sr, order):
