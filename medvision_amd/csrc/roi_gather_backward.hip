@@ -45,10 +45,33 @@ __device__ __forceinline__ A axis_weight(int v, int lo, int hi, A frac) {
   return (v == lo ? A(1) - frac : A(0)) + (v == hi ? frac : A(0));
 }
 
+// `clamped_tap` (sampling.hpp) in the coordinate type C
+template <typename C, typename A>
+__device__ __forceinline__ bool clamped_tap_in(C v, int size, int &lo, int &hi, A &frac, int order) {
+  if (v < C(-1) || v > static_cast<C>(size)) return false;
+  v = v <= C(0) ? C(0) : v;
+  const int base = static_cast<int>(v);
+  C f = C(0);
+  if (base >= size - 1) {
+    lo = hi = size - 1;
+  } else {
+    lo = base;
+    hi = base + 1;
+    f = v - static_cast<C>(base);
+  }
+  frac = order == 0 ? ((C(1) - f >= C(0.5)) ? A(0) : A(1)) : static_cast<A>(f);
+  return true;
+}
+
 template <typename T, typename RT>
 __global__ __launch_bounds__(kGatherThreads) void roi_backward_gather_kernel(
     const T *__restrict__ gout, const RT *__restrict__ rois, T *__restrict__ gin, const RoiProblem p) {
   using A = typename Acc<T>::type;
+  // Coordinates of the candidates: fp32 unless the tensors are fp64 (a sample that falls on the other
+  // side of a voxel boundary than in fp64 does so with a weight of ~1e-5; the coordinate's own
+  // rounding, ~1e-5 of a voxel at 128, stays below the gradient's tolerance of 1e-4).  The candidate
+  // RANGES are always conservative.
+  using C = typename std::conditional<(sizeof(T) <= 4), float, double>::type;
   __shared__ GatherShared sh;
   const int b = blockIdx.z, c = blockIdx.y;
   const long plane = static_cast<long>(p.D) * p.H * p.W;
@@ -107,6 +130,8 @@ __global__ __launch_bounds__(kGatherThreads) void roi_backward_gather_kernel(
     }
     const float inv_bin0 = scalar(sh.inv_bin0), off0 = scalar(sh.off0), slack = scalar(sh.slack), slack_u = scalar(sh.slack_u);
     const T *go = gout + (static_cast<long>(r) * p.C + c) * ocells;
+    const C m0 = static_cast<C>(g.rot[0]), m3 = static_cast<C>(g.rot[3]), m6 = static_cast<C>(g.rot[6]);
+    const C xbin = static_cast<C>(g.bin[0]), xoff = static_cast<C>(g.start[0] + 0.5 * g.sub[0]);
     const A inv_count = A(1) / static_cast<A>(g.count);
 
 #pragma unroll 1
@@ -173,18 +198,18 @@ __global__ __launch_bounds__(kGatherThreads) void roi_backward_gather_kernel(
             x1 = min(x1, static_cast<int>(floorf(u1)));
           }
           if (x0 > x1) continue;
-          // sample positions of the row in fp64: rot[a][0] * x + row term
-          const double bx = g.rot[1] * y + g.rot[2] * z + g.centre[0];
-          const double by = g.rot[4] * y + g.rot[5] * z + g.centre[1];
-          const double bw = g.rot[7] * y + g.rot[8] * z + g.centre[2];
+          // sample positions of the row: rot[a][0] * x + row term
+          const C bx = static_cast<C>(g.rot[1] * y + g.rot[2] * z + g.centre[0]);
+          const C by = static_cast<C>(g.rot[4] * y + g.rot[5] * z + g.centre[1]);
+          const C bw = static_cast<C>(g.rot[7] * y + g.rot[8] * z + g.centre[2]);
           for (int ux = x0; ux <= x1; ux++) {
-            const double x = local_coord(g, 0, ux, 0);
-            const double rx = fma(g.rot[0], x, bx), ry = fma(g.rot[3], x, by);
-            const double rz = nd == 3 ? fma(g.rot[6], x, bw) : 0.0;
+            const C x = static_cast<C>(ux) * xbin + xoff;   // local_coord(g, 0, ux, 0)
+            const C rx = fma(m0, x, bx), ry = fma(m3, x, by);
+            const C rz = nd == 3 ? fma(m6, x, bw) : C(0);
             int z0, z1, y0, y1, c0, c1;
             A lz, ly, lx;
-            if (!clamped_tap(rz, p.D, z0, z1, lz, p.order) || !clamped_tap(ry, p.H, y0, y1, ly, p.order) ||
-                !clamped_tap(rx, p.W, c0, c1, lx, p.order))
+            if (!clamped_tap_in<C, A>(rz, p.D, z0, z1, lz, p.order) || !clamped_tap_in<C, A>(ry, p.H, y0, y1, ly, p.order) ||
+                !clamped_tap_in<C, A>(rx, p.W, c0, c1, lx, p.order))
               continue;
             const A w = axis_weight(v[2], z0, z1, lz) * axis_weight(v[1], y0, y1, ly) * axis_weight(v[0], c0, c1, lx);
             if (w != A(0))
