@@ -131,7 +131,12 @@ __global__ __launch_bounds__(kGatherThreads) void roi_backward_gather_kernel(
     const float inv_bin0 = scalar(sh.inv_bin0), off0 = scalar(sh.off0), slack = scalar(sh.slack), slack_u = scalar(sh.slack_u);
     const T *go = gout + (static_cast<long>(r) * p.C + c) * ocells;
     const C m0 = static_cast<C>(g.rot[0]), m3 = static_cast<C>(g.rot[3]), m6 = static_cast<C>(g.rot[6]);
+    const C m1 = static_cast<C>(g.rot[1]), m4 = static_cast<C>(g.rot[4]), m7 = static_cast<C>(g.rot[7]);
+    const C m2 = static_cast<C>(g.rot[2]), m5 = static_cast<C>(g.rot[5]), m8 = static_cast<C>(g.rot[8]);
+    const C c0x = static_cast<C>(g.centre[0]), c0y = static_cast<C>(g.centre[1]), c0z = static_cast<C>(g.centre[2]);
     const C xbin = static_cast<C>(g.bin[0]), xoff = static_cast<C>(g.start[0] + 0.5 * g.sub[0]);
+    const C ybin = static_cast<C>(g.bin[1]), yoff = static_cast<C>(g.start[1] + 0.5 * g.sub[1]);
+    const C zbin = static_cast<C>(g.bin[2]), zoff = static_cast<C>(g.start[2] + 0.5 * g.sub[2]);
     const A inv_count = A(1) / static_cast<A>(g.count);
 
 #pragma unroll 1
@@ -141,25 +146,30 @@ __global__ __launch_bounds__(kGatherThreads) void roi_backward_gather_kernel(
       const unsigned vu = static_cast<unsigned>(vi), vzz = vu / slice, rem = vu - vzz * slice, vyy = rem / row;
       const int v[3] = {static_cast<int>(rem - vyy * row), static_cast<int>(vyy), static_cast<int>(vzz)};
       // the voxel in the roi's local frame: q = Rot^T (v - centre)
-      const double dx = v[0] - g.centre[0], dy = v[1] - g.centre[1], dz = nd == 3 ? v[2] - g.centre[2] : 0.0;
+      // (in the coordinate type; in fp32 the ranges are widened by what its rounding can move them)
+      const C dx = static_cast<C>(v[0] - g.centre[0]), dy = static_cast<C>(v[1] - g.centre[1]),
+              dz = nd == 3 ? static_cast<C>(v[2] - g.centre[2]) : C(0);
+      const C wide = sizeof(C) == 4 ? static_cast<C>(slack) : static_cast<C>(kSlack);
       int lo[3], hi[3];
       bool any = true;
 #pragma unroll
       for (int j = 0; j < 3; j++) {
         if (j >= nd) { lo[j] = 0; hi[j] = 0; continue; }
-        const double q = g.rot[j] * dx + g.rot[3 + j] * dy + g.rot[6 + j] * dz;
+        const C q = static_cast<C>(g.rot[j]) * dx + static_cast<C>(g.rot[3 + j]) * dy + static_cast<C>(g.rot[6 + j]) * dz;
         // cells u with |start + (u + .5) * bin - q| <= reach
-        const double a0 = q - reach[j] - g.start[j], a1 = q + reach[j] - g.start[j];
+        const C rj = static_cast<C>(reach[j]) + wide, sj = static_cast<C>(g.start[j]), ib = static_cast<C>(inv_bin[j]);
+        const C a0 = q - rj - sj, a1 = q + rj - sj;
         if (inv_bin[j] != 0.0) {
           // (a negative bin, i.e. a mirrored roi, swaps the two ends)
-          const double e0 = a0 * inv_bin[j] - 0.5, e1 = a1 * inv_bin[j] - 0.5;
-          const double u0 = fmin(fmax(fmin(e0, e1) - kSlack, -1.0), static_cast<double>(cells[j]));
-          const double u1 = fmin(fmax(fmax(e0, e1) + kSlack, -1.0), static_cast<double>(cells[j]));
+          const C e0 = a0 * ib - C(0.5), e1 = a1 * ib - C(0.5);
+          const C extra = wide * (C(1) + fabs(ib));
+          const C u0 = fmin(fmax(fmin(e0, e1) - extra, C(-1)), static_cast<C>(cells[j]));
+          const C u1 = fmin(fmax(fmax(e0, e1) + extra, C(-1)), static_cast<C>(cells[j]));
           lo[j] = max(static_cast<int>(ceil(u0)), 0);
           hi[j] = min(static_cast<int>(floor(u1)), cells[j] - 1);
         } else {   // every cell samples the same coordinate
           lo[j] = 0;
-          hi[j] = (a0 <= 0.0 && a1 >= 0.0) ? cells[j] - 1 : -1;
+          hi[j] = (a0 <= C(0) && a1 >= C(0)) ? cells[j] - 1 : -1;
         }
         any = any && lo[j] <= hi[j];
       }
@@ -168,12 +178,14 @@ __global__ __launch_bounds__(kGatherThreads) void roi_backward_gather_kernel(
       const float cv[3] = {static_cast<float>(-dx), static_cast<float>(-dy), static_cast<float>(-dz)};
       const float cells0 = static_cast<float>(cells[0]);
       for (int uz = lo[2]; uz <= hi[2]; uz++) {
-        const double z = nd == 3 ? local_coord(g, 2, uz, 0) : 0.0;
-        const float zf = static_cast<float>(z);
+        const C zc = nd == 3 ? static_cast<C>(uz) * zbin + zoff : C(0);   // local_coord(g, 2, uz, 0)
+        const float zf = static_cast<float>(zc);
         const float bz[3] = {fmaf(r2[0], zf, cv[0]), fmaf(r2[1], zf, cv[1]), fmaf(r2[2], zf, cv[2])};
+        // the slice's share of the sample positions
+        const C zx = fma(m2, zc, c0x), zy = fma(m5, zc, c0y), zw = fma(m8, zc, c0z);
         for (int uy = lo[1]; uy <= hi[1]; uy++) {
-          const double y = local_coord(g, 1, uy, 0);
-          const float yf = static_cast<float>(y);
+          const C yc = static_cast<C>(uy) * ybin + yoff;   // local_coord(g, 1, uy, 0)
+          const float yf = static_cast<float>(yc);
           // samples of this output row: r_a(x) - v_a = rot[a][0] * x + base_a; keep it within +-1
           float xl = -3e38f, xh = 3e38f;
 #pragma unroll
@@ -199,9 +211,7 @@ __global__ __launch_bounds__(kGatherThreads) void roi_backward_gather_kernel(
           }
           if (x0 > x1) continue;
           // sample positions of the row: rot[a][0] * x + row term
-          const C bx = static_cast<C>(g.rot[1] * y + g.rot[2] * z + g.centre[0]);
-          const C by = static_cast<C>(g.rot[4] * y + g.rot[5] * z + g.centre[1]);
-          const C bw = static_cast<C>(g.rot[7] * y + g.rot[8] * z + g.centre[2]);
+          const C bx = fma(m1, yc, zx), by = fma(m4, yc, zy), bw = fma(m7, yc, zw);
           for (int ux = x0; ux <= x1; ux++) {
             const C x = static_cast<C>(ux) * xbin + xoff;   // local_coord(g, 0, ux, 0)
             const C rx = fma(m0, x, bx), ry = fma(m3, x, by);
