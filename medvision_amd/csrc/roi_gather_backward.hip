@@ -64,7 +64,7 @@ __device__ __forceinline__ bool clamped_tap_in(C v, int size, int &lo, int &hi, 
 }
 
 template <typename T, typename RT>
-__global__ __launch_bounds__(kGatherThreads) void roi_backward_gather_kernel(
+__global__ __launch_bounds__(kGatherThreads) __attribute__((amdgpu_waves_per_eu(5))) void roi_backward_gather_kernel(
     const T *__restrict__ gout, const RT *__restrict__ rois, T *__restrict__ gin, const RoiProblem p) {
   using A = typename Acc<T>::type;
   // Coordinates of the candidates: fp32 unless the tensors are fp64 (a sample that falls on the other
