@@ -540,12 +540,16 @@ __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter_kerne
       const double gv[2] = {static_cast<double>(acc[blk][0] * ra.z) * scale.up,
                             static_cast<double>(acc[blk][1] * ra.z) * scale.up};
       const float wd[2] = {1.f - ra.w, ra.w}, wh[2] = {1.f - rb.x, rb.x}, ww[2] = {1.f - rb.y, rb.y};
+      // the lane's qword of the first corner, as a 32-bit byte offset worked out once: the corners
+      // differ by constants that go into the instructions' offset fields
+      char *const cell0 = reinterpret_cast<char *>(tile) + (static_cast<unsigned>(first) * kScatterStride + j) * 8u;
 #pragma unroll
       for (int c = 0; c < 8; c++) {
         const int ca = c >> 2, cb2 = (c >> 1) & 1, ce = c & 1;
         if ((S::TD > 1 || ca == 0) && ((bits >> c) & 1u)) {  // images have no second slice
           const float wc = wd[ca] * wh[cb2] * ww[ce];
-          unsigned long long *dst = tile + (first + ca * (S::TH * S::TW) + cb2 * S::TW + ce) * kScatterStride + j;
+          unsigned long long *dst = reinterpret_cast<unsigned long long *>(
+              cell0 + (ca * (S::TH * S::TW) + cb2 * S::TW + ce) * (kScatterStride * 8));
 #pragma unroll
           for (int r = 0; r < 2; r++)
             __hip_atomic_fetch_add(dst + 4 * r, fixed_term(wc, gv[r]), __ATOMIC_RELAXED,
