@@ -115,7 +115,7 @@ struct GatherDims { int nd, D, H, W, od, oh, ow, order; };
 // that is on no face of the volume no candidate comes near such an edge, and fp32 positions (off by
 // ~1e-5 of a voxel, weights by as much) decide nothing differently from fp64.  The voxels on the
 // faces, and order 0, which jumps wherever a fraction passes 0.5, are worked out in fp64 with the
-// oracle's own expressions.
+// expressions of the fp64 reference.
 template <typename T, typename C>
 __device__ __forceinline__ typename Acc<T>::type gather_voxel(const GatherGeo &q, const GatherDims &d, const T *go,
                                                               const int (&v)[3]) {
