@@ -208,6 +208,18 @@ int mv_deform_warp_2d(const void *img, const void *offset, void *output, int dty
 int mv_deform_warp_3d(const void *img, const void *offset, void *output, int dtype, int batch,
                       int channels, int depth, int height, int width, int order, void *stream);
 
+/* ---- augmentation DCN in general ----------------------------------------------------------------
+ * replaces deform_2d / deform_3d  csrc/deform_2d.h, csrc/deform_3d.h:27 (vision.cpp:71-72; host
+ * csrc/cuda_aug/deform_3d_cuda.cu:43-152, kernel csrc/cuda_aug/deform_3d_cuda_kernel.cuh:8-89) for
+ * any kernel, stride, padding, dilation, groups and weight: the DCNv1 forward whose column value is
+ * the border-replicating sampler of the affine engine, S(x[b,c], p) when -1 < p < size on every
+ * axis and 0 otherwise (order 0, 1 or 3), instead of the zero-padded trilinear form.
+ * Tensors as for mv_dcn3d_forward / mv_dcn2d_forward without mask; bias may be NULL.            */
+int mv_deform_conv_3d(const void *input, const void *offset, const void *weight, const void *bias,
+                      void *output, const mv_dcn3d_shape *shape, int dtype, int order, void *stream);
+int mv_deform_conv_2d(const void *input, const void *offset, const void *weight, const void *bias,
+                      void *output, const mv_dcn2d_shape *shape, int dtype, int order, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -473,26 +473,43 @@ def _is_identity_warp(weight, bias, C, ndim):
 
 
 def _deform(fn_name, ndim, input, weight, bias, offset, kernel, stride, pad, dil, group,
-            deformable_group, order):
+            deformable_group, im2col_step, order):
+    """csrc/deform_3d.h:27 -> csrc/cuda_aug/deform_3d_cuda.cu:43-152.  The way the reference calls
+    it (1x1x1 kernel, identity weight, zero bias: ops/cuda_fun_tools.py:134-167) is a displacement-
+    field warp and runs as one; anything else is the DCNv1 forward with the clamped samplers."""
     if not input.is_cuda:
         raise RuntimeError("Not implemented on the CPU")
     _same_device(input, weight=weight, bias=bias)
-    if (any(k != 1 for k in kernel) or any(s != 1 for s in stride) or any(p != 0 for p in pad)
-            or group != 1 or deformable_group != 1
-            or not _is_identity_warp(weight, bias, input.size(1), ndim)):
-        raise RuntimeError("deform_%dd supports the displacement-field warp only: 1x1 kernel, "
-                           "stride 1, no padding, identity weight, zero bias" % ndim)
     if order not in (0, 1, 3):
         raise RuntimeError(f"order {order} is not supported (0 nearest, 1 linear, 3 cubic)")
     _require_contiguous(input, "input")
     offset = offset.to(device=input.device, dtype=input.dtype).contiguous()
-    if tuple(offset.shape) != (input.size(0), ndim, *input.shape[2:]):
-        raise RuntimeError("offset must have shape [B, %d, *spatial]" % ndim)
-    out = torch.empty_like(input)
+    if (all(k == 1 for k in kernel) and all(s == 1 for s in stride) and all(p == 0 for p in pad)
+            and group == 1 and deformable_group == 1
+            and _is_identity_warp(weight, bias, input.size(1), ndim)):
+        if tuple(offset.shape) != (input.size(0), ndim, *input.shape[2:]):
+            raise RuntimeError("offset must have shape [B, %d, *spatial]" % ndim)
+        out = torch.empty_like(input)
+        with _on_device(input):
+            _lib.check(getattr(_lib.load(), fn_name)(
+                _lib.ptr(input), _lib.ptr(offset), _lib.ptr(out), _lib.dtype_code(input),
+                *input.shape, int(order), _lib.stream_of(input)))
+        return out
+    _im2col_step_check(input.size(0), im2col_step)
+    shape = _dcn_shape(input, weight, kernel, stride, pad, dil, group, deformable_group)
+    lib = _lib.load()
+    dims = _dcn_out_dims(lib, shape)
+    _dcn_check_aux(shape, dims, offset, None, _dcn_taps(shape))
+    bias = bias.contiguous()
+    if weight.dtype != input.dtype or bias.dtype != input.dtype:
+        raise RuntimeError("input, weight and bias must share one dtype")
+    if tuple(bias.shape) != (weight.size(0),):
+        raise RuntimeError("bias must have one entry per output channel")
+    out = torch.empty((input.size(0), weight.size(0), *dims), dtype=input.dtype, device=input.device)
     with _on_device(input):
-        _lib.check(getattr(_lib.load(), fn_name)(
-            _lib.ptr(input), _lib.ptr(offset), _lib.ptr(out), _lib.dtype_code(input),
-            *input.shape, int(order), _lib.stream_of(input)))
+        _lib.check(getattr(lib, "mv_deform_conv_%dd" % ndim)(
+            _lib.ptr(input), _lib.ptr(offset), _lib.ptr(weight), _lib.ptr(bias), _lib.ptr(out),
+            ctypes.byref(shape), _lib.dtype_code(input), int(order), _lib.stream_of(input)))
     return out
 
 
@@ -500,7 +517,7 @@ def deform_2d(input, weight, bias, offset, kernel_h, kernel_w, stride_h, stride_
               dilation_h, dilation_w, group, deformable_group, im2col_step, order):
     return _deform("mv_deform_warp_2d", 2, input, weight, bias, offset, (kernel_h, kernel_w),
                    (stride_h, stride_w), (pad_h, pad_w), (dilation_h, dilation_w), group,
-                   deformable_group, order)
+                   deformable_group, im2col_step, order)
 
 
 def deform_3d(input, weight, bias, offset, kernel_d, kernel_h, kernel_w, stride_d, stride_h,
@@ -509,7 +526,7 @@ def deform_3d(input, weight, bias, offset, kernel_d, kernel_h, kernel_w, stride_
     return _deform("mv_deform_warp_3d", 3, input, weight, bias, offset,
                    (kernel_d, kernel_h, kernel_w), (stride_d, stride_h, stride_w),
                    (pad_d, pad_h, pad_w), (dilation_d, dilation_h, dilation_w), group,
-                   deformable_group, order)
+                   deformable_group, im2col_step, order)
 
 
 def deform_warp(img, offset, order=1):

@@ -68,6 +68,8 @@ SIGNATURES = {
     "mv_dcn2d_backward": (_i, [_p] * 10 + [_SHAPE2_P, _i, _p, _p]),
     "mv_deform_warp_2d": (_i, [_p, _p, _p, _i] + [_i] * 4 + [_i, _p]),
     "mv_deform_warp_3d": (_i, [_p, _p, _p, _i] + [_i] * 5 + [_i, _p]),
+    "mv_deform_conv_3d": (_i, [_p] * 6 + [_i, _i, _p]),
+    "mv_deform_conv_2d": (_i, [_p] * 6 + [_i, _i, _p]),
 }
 
 _lib = None

@@ -8,6 +8,7 @@
 #include <atomic>
 
 #include "dcn_common.hpp"
+#include "sampling.hpp"
 
 namespace mv {
 
@@ -45,6 +46,62 @@ __global__ __launch_bounds__(kDcnThreads) void dcn_forward_kernel(
       const A m = mask_bg ? load(mask_bg + static_cast<long>(k) * s.Q + q) : A(1);
       for (int c = c_lo; c < c_hi; c++) {
         const A col = zsample<T, A>(x + (static_cast<long>(b) * s.Cin + c) * s.P, t) * m;
+        const T *wrow = wt + (static_cast<long>(o_begin) * s.cpg + (c - c_begin)) * s.K + k;
+#pragma unroll
+        for (int i = 0; i < kOutTile; i++)
+          if (i < o_count) acc[i] += load(wrow + static_cast<long>(i) * s.cpg * s.K) * col;
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kOutTile; i++)
+    if (i < o_count) {
+      const int o = o_begin + i;
+      y[(static_cast<long>(b) * s.Cout + o) * s.Q + q] =
+          store_cast<T>(acc[i] + (bias ? load(bias + o) : A(0)));
+    }
+}
+
+// ---- augmentation DCN: the v1 forward with the border-replicating samplers ---------------------
+// Column value = S(x[b,c], p) when -1 < p < size on every axis, else 0, with S nearest, linear
+// or cubic by `order` (reference: csrc/cuda_aug/deform_3d_cuda_kernel.cuh:8-89, contraction with
+// the weight and bias csrc/cuda_aug/deform_3d_cuda.cu:43-152).  Same thread layout as above.
+template <typename T>
+__global__ __launch_bounds__(kDcnThreads) void deform_conv_clamped_kernel(
+    const T *__restrict__ x, const T *__restrict__ off, const T *__restrict__ wt,
+    const T *__restrict__ bias, T *__restrict__ y, const DcnDims s, const int order) {
+  using A = typename Acc<T>::type;
+  const long q = blockIdx.x * static_cast<long>(kDcnThreads) + threadIdx.x;
+  const int tiles_per_group = (s.opg + kOutTile - 1) / kOutTile;
+  const int grp = blockIdx.y / tiles_per_group, tile = blockIdx.y % tiles_per_group;
+  const int b = blockIdx.z;
+  if (q >= s.Q) return;
+  const int ow = q % s.Wo, oh = (q / s.Wo) % s.Ho, od = q / (static_cast<long>(s.Wo) * s.Ho);
+  const int o_begin = grp * s.opg + tile * kOutTile;
+  const int o_count = min(kOutTile, grp * s.opg + s.opg - o_begin);
+  A acc[kOutTile];
+#pragma unroll
+  for (int i = 0; i < kOutTile; i++) acc[i] = A(0);
+  const int c_begin = grp * s.cpg, c_end = c_begin + s.cpg;
+  for (int dgi = c_begin / s.cpd; dgi <= (c_end - 1) / s.cpd; dgi++) {
+    const int c_lo = max(c_begin, dgi * s.cpd), c_hi = min(c_end, (dgi + 1) * s.cpd);
+    const T *off_bg = off + (static_cast<long>(b) * s.dg + dgi) * s.nd * s.K * s.Q;
+    for (int k = 0; k < s.K; k++) {
+      double pd, ph, pw;
+      dcn_position(s, off_bg, k, od, oh, ow, q, pd, ph, pw);
+      if (!(ph > -1.0 && pw > -1.0 && ph < s.H && pw < s.W && (s.nd == 2 || (pd > -1.0 && pd < s.D))))
+        continue;
+      Corners<A> cw;
+      if (order != 3 && !clamped_corners<A>(s.D, s.H, s.W, pd, ph, pw, order, cw)) continue;
+      for (int c = c_lo; c < c_hi; c++) {
+        const T *plane = x + (static_cast<long>(b) * s.Cin + c) * s.P;
+        A col = A(0);
+        if (order == 3) {
+          col = sample_cubic<T>(plane, s.nd, s.D, s.H, s.W, pd, ph, pw);
+        } else {
+#pragma unroll
+          for (int n = 0; n < 8; n++) col += cw.w[n] * load(plane + cw.idx[n]);
+        }
         const T *wrow = wt + (static_cast<long>(o_begin) * s.cpg + (c - c_begin)) * s.K + k;
 #pragma unroll
         for (int i = 0; i < kOutTile; i++)
@@ -277,6 +334,25 @@ static int dcn_forward_any(const void *input, const void *offset, const void *ma
   return check_launch("dcn_forward_kernel");
 }
 
+static int deform_conv_any(const void *input, const void *offset, const void *weight,
+                           const void *bias, void *output, const DcnDims &s, int dtype, int order,
+                           void *stream) {
+  MV_REQUIRE(input && offset && weight && output, "null pointer argument");
+  MV_REQUIRE(order == 0 || order == 1 || order == 3,
+             "order %d is not supported (0 nearest, 1 linear, 3 cubic)", order);
+  const long qb = (s.Q + kDcnThreads - 1) / kDcnThreads;
+  const long yb = static_cast<long>(s.groups) * ((s.opg + kOutTile - 1) / kOutTile);
+  MV_REQUIRE(qb < (1L << 31) && yb <= 65535 && s.B <= 65535, "grid too large");
+  const dim3 grid(static_cast<unsigned>(qb), static_cast<unsigned>(yb), s.B), block(kDcnThreads);
+  MV_DISPATCH(dtype, {
+    hipLaunchKernelGGL((deform_conv_clamped_kernel<T>), grid, block, 0,
+                       static_cast<hipStream_t>(stream), static_cast<const T *>(input),
+                       static_cast<const T *>(offset), static_cast<const T *>(weight),
+                       static_cast<const T *>(bias), static_cast<T *>(output), s, order);
+  });
+  return check_launch("deform_conv_clamped_kernel");
+}
+
 static int dcn_backward_any(const void *input, const void *offset, const void *mask,
                             const void *weight, const void *grad_output, void *grad_input,
                             void *grad_offset, void *grad_mask, void *grad_weight, void *grad_bias,
@@ -476,6 +552,20 @@ int mv_dcn2d_backward(const void *input, const void *offset, const void *mask, c
   return st ? st
             : dcn_backward_any(input, offset, mask, weight, grad_output, grad_input, grad_offset,
                                grad_mask, grad_weight, grad_bias, s, dtype, workspace, stream);
+}
+
+int mv_deform_conv_3d(const void *input, const void *offset, const void *weight, const void *bias,
+                      void *output, const mv_dcn3d_shape *shape, int dtype, int order, void *stream) {
+  DcnDims s;
+  const int st = make_dcn_dims(s, shape);
+  return st ? st : deform_conv_any(input, offset, weight, bias, output, s, dtype, order, stream);
+}
+
+int mv_deform_conv_2d(const void *input, const void *offset, const void *weight, const void *bias,
+                      void *output, const mv_dcn2d_shape *shape, int dtype, int order, void *stream) {
+  DcnDims s;
+  const int st = make_dcn_dims_2d(s, shape);
+  return st ? st : deform_conv_any(input, offset, weight, bias, output, s, dtype, order, stream);
 }
 
 }  // extern "C"

@@ -226,6 +226,19 @@ def deform_warp(img, offset, order=1):
     return out
 
 
+def deform_conv(x, offset, weight, bias=None, stride=1, padding=0, dilation=1, groups=1,
+                deformable_groups=1, order=1):
+    """The augmentation DCN in general: v1 forward with the clamped samplers, any kernel and weight
+    (cuda_aug/deform_3d_cuda.cu:43-152, cuda_aug/deform_3d_cuda_kernel.cuh:8-89; 4-D tensors: the
+    2-D twin, cuda_aug/deform_2d_cuda_kernel.cuh)."""
+    xs, offs, ws = _f64(x), _f64(offset), _f64(weight)
+    bs = _f64(bias) if bias is not None else None
+    arr, out = _dcn_params(xs, ws, stride, padding, dilation, groups, deformable_groups)
+    y = torch.zeros((xs.shape[0], ws.shape[0], *out), dtype=torch.float64)
+    lib().orc_deform_conv(_ptr(xs), _ptr(offs), _ptr(ws), _ptr(bs), _ptr(y), arr, int(order))
+    return y
+
+
 def set_threads(n):
     """Number of OpenMP threads the oracle uses (for the CPU baseline timing)."""
     omp = ctypes.CDLL("libgomp.so.1")

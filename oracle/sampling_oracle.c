@@ -22,6 +22,8 @@
  *   dcn3d_forward             F.conv3d at zero offsets, grid_sample(zeros, align_corners=True)
  *   dcn3d_backward            torch autograd through the grid_sample formulation
  *   deform3d_warp             grid_sample(border) on the open interval (-1, S)
+ *   deform_conv               F.conv3d / F.conv2d at zero offsets (orders 0, 1, 3), a 1x1x1 conv
+ *                             of the warp above, grid_sample(border) per tap x open-interval mask
  *   sample_cubic              textbook cubic Hermite spline with central-difference tangents on an
  *                             edge-padded copy (numpy), exact reproduction of quadratics in the
  *                             interior, node interpolation, partition of unity, brute-force
@@ -620,5 +622,47 @@ void orc_deform_warp(const double *img, const double *off, double *out, int ndim
       for (int c = 0; c < C; c++)
         out[((long)b * C + c) * P + q] =
             ok ? sample_any(img + ((long)b * C + c) * P, ndim, D, H, W, pd, ph, pw, order) : 0.0;
+    }
+}
+
+/* ------------------------------------------------------------------------------------------
+ * General augmentation DCN: the v1 forward with the CLAMPED samplers, for any kernel, stride,
+ * padding, dilation, groups and weight (cuda_aug/deform_3d_cuda_kernel.cuh:8-89: column value
+ * = S(x[b,c], p) when -1 < p < size on every axis, else 0, S = nearest / linear / Hermite by
+ * `order`, offset channel nd*k + axis of tap k as in the DCN; cuda_aug/deform_3d_cuda.cu:43-152:
+ * y = bias + W . columns per group; images: cuda_aug/deform_2d_cuda_kernel.cuh, offset channels
+ * 2k = h, 2k+1 = w).  p: the 21 ints of dcn_shape.  bias may be NULL.
+ * ---------------------------------------------------------------------------------------- */
+void orc_deform_conv(const double *x, const double *off, const double *wt, const double *bias,
+                     double *y, const int *p, int order) {
+  dcn_shape s;
+  memcpy(&s, p, DCN_INTS * sizeof(int));
+  dcn_out_dims(&s);
+  const long Q = (long)s.Do * s.Ho * s.Wo, P = (long)s.D * s.H * s.W;
+  const int cpg = s.Cin / s.groups, opg = s.Cout / s.groups, cpd = s.Cin / s.dg, nd = s.nd;
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int b = 0; b < s.B; b++)
+    for (long q = 0; q < Q; q++) {
+      int ow = q % s.Wo, oh = (q / s.Wo) % s.Ho, od = q / ((long)s.Wo * s.Ho);
+      double *acc = (double *)calloc(s.Cout, sizeof(double));
+      for (int dgi = 0; dgi < s.dg; dgi++)
+        for (int k = 0; k < s.K; k++) {
+          const double *o = off + ((long)b * s.dg + dgi) * nd * s.K * Q;
+          int i = k / (s.kh * s.kw), j = (k / s.kw) % s.kh, kk = k % s.kw;
+          double pd = od * s.sd - s.pd + i * s.dd + (nd == 3 ? o[((long)nd * k + 0) * Q + q] : 0.0);
+          double ph = oh * s.sh - s.ph + j * s.dh + o[((long)nd * k + nd - 2) * Q + q];
+          double pw = ow * s.sw - s.pw + kk * s.dw + o[((long)nd * k + nd - 1) * Q + q];
+          int ok = ph > -1 && pw > -1 && ph < s.H && pw < s.W && (nd == 2 || (pd > -1 && pd < s.D));
+          if (!ok) continue;
+          for (int c = dgi * cpd; c < (dgi + 1) * cpd; c++) {
+            double col = sample_any(x + ((long)b * s.Cin + c) * P, nd, s.D, s.H, s.W, pd, ph, pw, order);
+            int grp = c / cpg, cl = c % cpg;
+            for (int o2 = grp * opg; o2 < (grp + 1) * opg; o2++)
+              acc[o2] += wt[((long)o2 * cpg + cl) * s.K + k] * col;
+          }
+        }
+      for (int o2 = 0; o2 < s.Cout; o2++)
+        y[((long)b * s.Cout + o2) * Q + q] = acc[o2] + (bias ? bias[o2] : 0.0);
+      free(acc);
     }
 }

@@ -424,3 +424,45 @@ def test_warp_vs_oracle(ops, oracle, dtype, order):
     same = _C.deform_3d(img.to(DEV), eye, torch.zeros(3, device=DEV, dtype=dtype), off.to(DEV),
                         1, 1, 1, 1, 1, 1, 0, 0, 0, 1, 1, 1, 1, 1, 64, order)
     assert torch.equal(same, ops.apply_offset_3d(img.to(DEV), off.to(DEV), order))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("order", [0, 1, 3])
+def test_general_deform_vs_oracle(ops, oracle, dtype, order):
+    """`_C.deform_3d` / `_C.deform_2d` with a real kernel and weight: the DCNv1 forward with the
+    clamped samplers (csrc/cuda_aug/deform_3d_cuda.cu:43-152)."""
+    from medvision_amd import _C
+    g = wl.gen(300 + order)
+    cases = [  # Cin, Cout, size, kernel, stride, pad, dil, groups, dg
+        (4, 6, (6, 7, 8), (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1), 1, 1),
+        (4, 70, (5, 9, 8), (2, 3, 1), (1, 2, 1), (0, 2, 1), (2, 1, 1), 2, 2),
+        (6, 3, (7, 6, 9), (1, 1, 1), (1, 1, 1), (0, 0, 0), (1, 1, 1), 1, 3),
+        (4, 4, (12, 11), (3, 2), (2, 1), (1, 0), (1, 2), 2, 1),
+        (3, 5, (9, 10), (1, 1), (1, 1), (0, 0), (1, 1), 1, 1),
+    ]
+    for Cin, Cout, size, k, stride, pad, dil, groups, dg in cases:
+        nd = len(size)
+        x = torch.randn(2, Cin, *size, generator=g).to(dtype)
+        w = (torch.randn(Cout, Cin // groups, *k, generator=g) * 0.3).to(dtype)
+        b = torch.randn(Cout, generator=g).to(dtype)
+        out = [(s + 2 * p - (d * (kk - 1) + 1)) // st + 1 for s, p, d, kk, st in zip(size, pad, dil, k, stride)]
+        K = 1
+        for kk in k:
+            K *= kk
+        off = (torch.randn(2, dg * nd * K, *out, generator=g) * 2.5).to(dtype)
+        fn = _C.deform_3d if nd == 3 else _C.deform_2d
+        got = fn(x.to(DEV), w.to(DEV), b.to(DEV), off.to(DEV), *k, *stride, *pad, *dil, groups, dg, 64, order)
+        want = oracle.deform_conv(x, off, w, b, stride, pad, dil, groups, dg, order)
+        assert tuple(got.shape) == tuple(want.shape)
+        assert_close(got, want, FWD_TOL[dtype], f"deform_{nd}d {size} k={k} order={order}")
+        assert float((want == b.double().view(1, -1, *([1] * nd))).double().mean()) < 0.9
+    x = torch.zeros(2, 4, 4, 4, 4, device=DEV)
+    with pytest.raises(RuntimeError, match="kernel shape wont match"):
+        _C.deform_3d(x, torch.zeros(4, 4, 3, 3, 3, device=DEV), torch.zeros(4, device=DEV),
+                     torch.zeros(2, 3, 4, 4, 4, device=DEV), 1, 1, 1, 1, 1, 1, 0, 0, 0, 1, 1, 1, 1, 1, 64, 1)
+    with pytest.raises(RuntimeError, match="kernel channels wont match"):
+        _C.deform_3d(x, torch.zeros(4, 3, 1, 1, 1, device=DEV), torch.zeros(4, device=DEV),
+                     torch.zeros(2, 3, 4, 4, 4, device=DEV), 1, 1, 1, 1, 1, 1, 0, 0, 0, 1, 1, 1, 1, 1, 64, 1)
+    with pytest.raises(RuntimeError, match="order 2 is not supported"):
+        _C.deform_3d(x, torch.zeros(4, 4, 1, 1, 1, device=DEV), torch.zeros(4, device=DEV),
+                     torch.zeros(2, 3, 4, 4, 4, device=DEV), 1, 1, 1, 1, 1, 1, 0, 0, 0, 1, 1, 1, 1, 1, 64, 2)

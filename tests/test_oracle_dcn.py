@@ -7,6 +7,9 @@
 * 2-D layers               ->  F.conv2d at zero offsets, a hand-shifted image for the channel order
                               (2k = rows, 2k+1 = columns), 2-D grid_sample + autograd in general
 * warp                     ->  grid_sample(border) on the open interval, identity at zero offset
+* augmentation DCN         ->  F.conv3d / F.conv2d at zero offsets for orders 0, 1 and 3; a pointwise
+                              convolution of the (pinned) warp; grid_sample(border) per tap on the
+                              open interval for kernels, strides, paddings, dilations and groups
 """
 import pytest
 import torch
@@ -165,3 +168,72 @@ def test_warp(oracle):
             if -1 < sh < 6 and -1 < sw < 8:
                 want[0, 0, h, w_] = im2[0, 0, min(max(sh, 0), 5), min(max(sw, 0), 7)]
     assert torch.allclose(got, want)
+
+
+@pytest.mark.parametrize("order", [0, 1, 3])
+def test_deform_conv_zero_offset_is_conv(oracle, order):
+    g = _g(20 + order)
+    x = torch.randn(2, 4, 6, 7, 8, generator=g, dtype=torch.float64)
+    w = torch.randn(6, 2, 3, 2, 3, generator=g, dtype=torch.float64)
+    b = torch.randn(6, generator=g, dtype=torch.float64)
+    stride, pad, dil = (1, 2, 1), (2, 1, 3), (1, 1, 2)
+    want = F.conv3d(x, w, b, stride, pad, dil, 2)
+    off = torch.zeros(2, 2 * 3 * 18, *want.shape[2:], dtype=torch.float64)
+    got = oracle.deform_conv(x, off, w, b, stride, pad, dil, 2, 2, order)
+    assert got.shape == want.shape and torch.allclose(got, want, atol=1e-11)
+    x2 = torch.randn(2, 4, 9, 8, generator=g, dtype=torch.float64)
+    w2 = torch.randn(2, 4, 3, 2, generator=g, dtype=torch.float64)
+    want = F.conv2d(x2, w2, None, (2, 1), (1, 2), (2, 1))
+    off = torch.zeros(2, 2 * 6, *want.shape[2:], dtype=torch.float64)
+    got = oracle.deform_conv(x2, off, w2, None, (2, 1), (1, 2), (2, 1), 1, 1, order)
+    assert got.shape == want.shape and torch.allclose(got, want, atol=1e-11)
+
+
+@pytest.mark.parametrize("order", [0, 1, 3])
+def test_deform_conv_pointwise_is_conv_of_warp(oracle, order):
+    g = _g(30 + order)
+    x = torch.randn(2, 4, 5, 6, 7, generator=g, dtype=torch.float64)
+    w = torch.randn(6, 2, 1, 1, 1, generator=g, dtype=torch.float64)
+    b = torch.randn(6, generator=g, dtype=torch.float64)
+    off = torch.randn(2, 2 * 3, 5, 6, 7, generator=g, dtype=torch.float64) * 2   # two offset groups
+    warped = torch.cat([oracle.deform_warp(x[:, :2], off[:, :3], order),
+                        oracle.deform_warp(x[:, 2:], off[:, 3:], order)], 1)
+    want = F.conv3d(warped, w, b, groups=2)
+    got = oracle.deform_conv(x, off, w, b, 1, 0, 1, 2, 2, order)
+    assert torch.allclose(got, want, atol=1e-11)
+    x2, off2 = x[:, :, 0].contiguous(), off[:, [1, 2, 4, 5], 0].contiguous()
+    warped = torch.cat([oracle.deform_warp(x2[:, :2], off2[:, :2], order),
+                        oracle.deform_warp(x2[:, 2:], off2[:, 2:], order)], 1)
+    want = F.conv2d(warped, w[:, :, 0], b, groups=2)
+    got = oracle.deform_conv(x2, off2, w[:, :, 0].contiguous(), b, 1, 0, 1, 2, 2, order)
+    assert torch.allclose(got, want, atol=1e-11)
+
+
+@pytest.mark.parametrize("groups,dg", [(1, 1), (2, 2), (2, 1)])
+def test_deform_conv_linear_vs_grid_sample(oracle, groups, dg):
+    g = _g(40 + groups + 2 * dg)
+    B, Cin, Cout, D, H, W = 2, 4, 4, 4, 5, 6
+    k, stride, pad, dil = (2, 3, 2), (1, 2, 1), (1, 1, 0), (1, 1, 2)
+    K = 12
+    x = torch.randn(B, Cin, D, H, W, generator=g, dtype=torch.float64)
+    w = torch.randn(Cout, Cin // groups, *k, generator=g, dtype=torch.float64)
+    b = torch.randn(Cout, generator=g, dtype=torch.float64)
+    Do, Ho, Wo = [(S + 2 * p_ - (d_ * (k_ - 1) + 1)) // s_ + 1
+                  for S, p_, d_, k_, s_ in zip((D, H, W), pad, dil, k, stride)]
+    off = torch.randn(B, dg * 3 * K, Do, Ho, Wo, generator=g, dtype=torch.float64) * 2.0
+    want = torch_ref.dcn3d(x, off, None, w, b, stride, pad, dil, groups, dg,
+                           sampler=torch_ref.sample_border_open)
+    got = oracle.deform_conv(x, off, w, b, stride, pad, dil, groups, dg, 1)
+    assert torch.allclose(got, want, atol=1e-11)
+    # image layer = the depth-1 volume with offset channels (2k, 2k+1) = (rows, columns)
+    x2 = torch.randn(B, Cin, 7, 6, generator=g, dtype=torch.float64)
+    w2 = torch.randn(Cout, Cin // groups, 3, 2, generator=g, dtype=torch.float64)
+    Ho, Wo = (7 + 2 - 3) // 2 + 1, (6 + 0 - 3) // 1 + 1
+    off2 = torch.randn(B, dg * 2 * 6, Ho, Wo, generator=g, dtype=torch.float64) * 2.0
+    off3 = torch.zeros(B, dg * 6, 3, 1, Ho, Wo, dtype=torch.float64)
+    off3[:, :, 1:, 0] = off2.reshape(B, dg * 6, 2, Ho, Wo)
+    want = torch_ref.dcn3d(x2[:, :, None], off3.reshape(B, dg * 18, 1, Ho, Wo), None, w2[:, :, None],
+                           b, (1, 2, 1), (0, 1, 0), (1, 1, 2), groups, dg,
+                           sampler=torch_ref.sample_border_open)[:, :, 0]
+    got = oracle.deform_conv(x2, off2, w2, b, (2, 1), (1, 0), (1, 2), groups, dg, 1)
+    assert torch.allclose(got, want, atol=1e-11)

@@ -118,8 +118,15 @@ def roi_align(features, rois, output_size, spatial_scale=1.0, sampling_ratio=0, 
     return out[:, :, 0] if ndim == 2 else out
 
 
+def sample_border_open(plane, z, y, x):
+    """Clamped trilinear sampler on the OPEN interval (-1, S): what the augmentation DCN evaluates."""
+    _, D, H, W = plane.shape
+    inside = (z > -1) & (z < D) & (y > -1) & (y < H) & (x > -1) & (x < W)
+    return sample_border(plane, z, y, x) * inside.to(plane.dtype)
+
+
 def dcn3d(x, offset, mask, weight, bias=None, stride=1, padding=0, dilation=1, groups=1,
-          deformable_groups=1):
+          deformable_groups=1, sampler=sample_zeros):
     """Differentiable fp64 DCN 3-D (v1 if mask is None) from grid_sample + einsum."""
     t3 = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v,) * 3
     s, p, d = t3(stride), t3(padding), t3(dilation)
@@ -141,8 +148,8 @@ def dcn3d(x, offset, mask, weight, bias=None, stride=1, padding=0, dilation=1, g
             for k in range(K):
                 i, j, kk = k // (kh * kw), (k // kw) % kh, k % kw
                 o = offset[b, g * 3 * K + 3 * k: g * 3 * K + 3 * k + 3]
-                v = sample_zeros(xs, qd + i * d[0] + o[0], qh + j * d[1] + o[1],
-                                 qw + kk * d[2] + o[2])
+                v = sampler(xs, qd + i * d[0] + o[0], qh + j * d[1] + o[1],
+                            qw + kk * d[2] + o[2])
                 if mask is not None:
                     v = v * mask[b, g * K + k][None]
                 taps.append(v)
