@@ -1201,10 +1201,74 @@ static int launch_resample(const T *feat, const float *rois, T *out, const RoiPr
   return check_launch("roi_resample_kernel");
 }
 
-// The tiled path pays when one (roi, channel) yields many voxels and the sampling grid is 1.
-// With `need` set only the workspace size is computed.  Returns -1 when the path does not apply.
+int roi_forward_tiled(const void *input, const void *rois, void *output, int dtype,
+                      const RoiProblem &p, void *workspace, size_t *need, hipStream_t s);
+
+// Mean over the g^ndim samples of a bin: `fine` holds one sample per element, [planes][od*g][oh*g][ow*g]
+// ([planes][oh*g][ow*g] for images, gz = 1).
+template <typename T>
+__global__ __launch_bounds__(256) void roi_bin_mean_kernel(const T *__restrict__ fine, T *__restrict__ out,
+                                                           long cells, int od, int oh, int ow, int g,
+                                                           int gz) {
+  const long i = blockIdx.x * 256L + threadIdx.x;
+  if (i >= cells) return;
+  const int x = i % ow, y = (i / ow) % oh, z = (i / (static_cast<long>(ow) * oh)) % od;
+  const long plane = i / (static_cast<long>(ow) * oh * od);
+  const long fw = static_cast<long>(ow) * g, fh = static_cast<long>(oh) * g, fd = static_cast<long>(od) * gz;
+  const T *src = fine + ((plane * fd + static_cast<long>(z) * gz) * fh + static_cast<long>(y) * g) * fw +
+                 static_cast<long>(x) * g;
+  float sum = 0.f;
+  for (int a = 0; a < gz; a++)
+    for (int b = 0; b < g; b++)
+      for (int c = 0; c < g; c++) sum += static_cast<float>(load(src + (a * fh + b) * fw + c));
+  out[i] = store_cast<T>(sum / static_cast<float>(gz * g * g));
+}
+
+// A fixed sampling grid of 2..4 per axis on a large output: the bins' samples are exactly the voxels
+// of the same roi resampled at grid 1 onto an output g times finer (start + (cell * g + sub + 0.5) *
+// bin / g), so the tiled kernel writes that finer volume into the workspace and a second pass takes
+// the means.  16-bit samples are rounded before the mean is; fp16's two roundings stay within its
+// tolerance, bf16's would not, so bf16 keeps the general kernel.
+static int roi_forward_tiled_grid(const void *input, const void *rois, void *output, int dtype,
+                                  const RoiProblem &p, void *workspace, size_t *need, hipStream_t s) {
+  const int g = p.sampling_ratio, gz = p.ndim == 3 ? g : 1;
+  if (dtype != MV_F16 && dtype != MV_F32) return -1;
+  if (!need && p.order != 1 && p.order != 3) return -1;
+  // Outputs that the grid-1 rule sends here, except those of <= 16 cells per axis (the pooled kernels
+  // take plain boxes of that size).  Only values that the workspace query also knows may decide.
+  if (static_cast<long>(p.od) * p.oh * p.ow < 4096 || p.ow < 16) return -1;
+  if (p.od <= 16 && p.oh <= 16 && p.ow <= 16) return -1;
+  RoiProblem f = p;
+  f.sampling_ratio = 1;
+  f.od = p.od * gz; f.oh = p.oh * g; f.ow = p.ow * g;
+  const long cells = static_cast<long>(p.R) * p.C * p.od * p.oh * p.ow;
+  const long fine = cells * gz * g * g;
+  if (fine >= (1L << 31) || (cells + 255) / 256 >= (1L << 31)) return -1;
+  size_t inner = 0;
+  if (roi_forward_tiled(nullptr, nullptr, nullptr, dtype, f, nullptr, &inner, nullptr) != MV_OK) return -1;
+  inner = (inner + 255) & ~static_cast<size_t>(255);
+  if (need) { *need = inner + static_cast<size_t>(fine) * dtype_size(dtype); return MV_OK; }
+  if (workspace == nullptr) return -1;
+  void *samples = static_cast<char *>(workspace) + inner;
+  const int st = roi_forward_tiled(input, rois, samples, dtype, f, workspace, nullptr, s);
+  if (st != MV_OK) return st;   // -1: the finer problem does not fit the tiled kernel after all
+  const dim3 grid(static_cast<unsigned>((cells + 255) / 256)), block(256);
+  if (dtype == MV_F16)
+    hipLaunchKernelGGL((roi_bin_mean_kernel<__half>), grid, block, 0, s, static_cast<const __half *>(samples),
+                       static_cast<__half *>(output), cells, p.od, p.oh, p.ow, g, gz);
+  else
+    hipLaunchKernelGGL((roi_bin_mean_kernel<float>), grid, block, 0, s, static_cast<const float *>(samples),
+                       static_cast<float *>(output), cells, p.od, p.oh, p.ow, g, gz);
+  return check_launch("roi_bin_mean_kernel");
+}
+
+// The tiled path pays when one (roi, channel) yields many voxels and the sampling grid is 1 (or a
+// fixed 2..4, in two passes).  With `need` set only the workspace size is computed.  Returns -1
+// when the path does not apply.
 int roi_forward_tiled(const void *input, const void *rois, void *output, int dtype,
                       const RoiProblem &p, void *workspace, size_t *need, hipStream_t s) {
+  if (p.sampling_ratio >= 2 && p.sampling_ratio <= 4)
+    return roi_forward_tiled_grid(input, rois, output, dtype, p, workspace, need, s);
   const long vox = static_cast<long>(p.od) * p.oh * p.ow;
   if (p.sampling_ratio != 1 || vox < 4096 || p.ow < 16 || p.R == 0) return -1;
   if (vox * 4 >= (1L << 31)) return -1;   // 32-bit byte offsets inside one output volume

@@ -259,6 +259,38 @@ def test_cubic_affine_vs_oracle(ops, oracle, dtype, ndim, sr):
     assert torch.equal(same[0].cpu(), feat[0])
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("sr", [2, 3, 4])
+def test_large_outputs_with_a_sampling_grid(ops, oracle, dtype, sr):
+    """sampling_ratio 2..4 on outputs of resampling size: the tiled kernel writes the samples of the
+    sr times finer grid and a second pass takes the bin means (fp16 / fp32; bf16 stays on the general
+    kernel).  Rotated and plain rois in 3-D and 2-D, order 1, and order 3 through the affine engine."""
+    g = wl.gen(700 + sr)
+    feat = torch.randn(2, 2, 24, 40, 48, generator=g).to(dtype)
+    out = (20, 24, 32) if sr < 4 else (10, 24, 32)
+    rois = wl.affine_rois(g, 2, (48, 40, 24))
+    got = ops.RoIAlignRotated(out, 1.0, sr)(feat.to(DEV), rois.to(DEV))
+    want = oracle.roi_align_forward(feat, rois, out, 1.0, sr, True, 1, True)
+    assert float((want == 0).double().mean()) > 0.01       # bins with samples in the void
+    assert_close(got, want, FWD_TOL[dtype], "rotated 3-D")
+    boxes = torch.tensor([[0, 2.3, 1.2, 0.5, 40.1, 33.3, 20.7], [1, -3.0, 5.0, 2.0, 30.0, 45.0, 30.0]])
+    got = ops.RoIAlign(out, 0.5, sr)(feat.to(DEV), (boxes * torch.tensor([1.] + [2.] * 6)).to(DEV))
+    want = oracle.roi_align_forward(feat, boxes * torch.tensor([1.] + [2.] * 6), out, 0.5, sr, True, 1, False)
+    assert_close(got, want, FWD_TOL[dtype], "plain 3-D")
+    img = torch.randn(2, 3, 70, 90, generator=g).to(dtype)
+    r2 = torch.tensor([[0, 45.0, 35.0, 80.0, 60.0, 0.4], [1, 40.0, 30.0, 100.0, 50.0, -1.2]])
+    got = ops.RoIAlignRotated((64, 80), 1.0, sr)(img.to(DEV), r2.to(DEV))
+    want = oracle.roi_align_forward(img, r2, (64, 80), 1.0, sr, True, 1, True)
+    assert_close(got, want, FWD_TOL[dtype], "rotated 2-D")
+    if dtype != torch.bfloat16:
+        got = ops.affine_3d(feat.to(DEV), rois.to(DEV), out, 1.0, sr, True, 3)
+        want = oracle.roi_align_forward(feat, rois, out, 1.0, sr, True, 3, True)
+        assert_close(got, want, FWD_TOL[dtype], "order 3")
+        got = ops.affine_2d(img.to(DEV), r2.to(DEV), (64, 80), 1.0, sr, False, 3)
+        want = oracle.roi_align_forward(img, r2, (64, 80), 1.0, sr, False, 3, True)
+        assert_close(got, want, FWD_TOL[dtype], "order 3, images")
+
+
 def test_cubic_resize_larger_volume(ops, oracle):
     """Resize of a 40x48x56 volume to 64x80x96 at order 3, as CudaResize(order=3) issues it."""
     g = wl.gen(97)
