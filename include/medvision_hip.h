@@ -84,9 +84,12 @@ int mv_roi_align_rotated_3d_backward(const void *grad_output, const void *rois, 
                                      int order, void *workspace, void *stream);
 size_t mv_roi_align_backward_workspace_bytes(int dtype, int batch, int channels, int depth,
                                              int height, int width);
-/* Workspace of the forward entry points (plain, rotated and affine).  The current kernels keep
- * their per-call state in LDS, so the query returns 0 and NULL may be passed; callers should
- * still query and pass what is asked for.  ndim = 2 or 3 (out_d ignored for 2).               */
+/* Workspace of the forward entry points (plain, rotated and affine).  0 for a sampling grid of 1
+ * (the kernels keep their per-call state in LDS); for fp16 / fp32 outputs of resampling size with a
+ * fixed sampling_ratio of 2..4 the bytes of the bins' samples (sampling_ratio^ndim per output
+ * element), which a second pass averages.  A non-NULL `workspace` must hold what this query
+ * returns for the call's arguments; NULL selects the kernels that need none.  ndim = 2 or 3
+ * (out_d ignored for 2).                                                                       */
 size_t mv_roi_align_forward_workspace_bytes(int dtype, int ndim, int channels, int num_rois,
                                             int out_d, int out_h, int out_w, int sampling_ratio);
 /* The same query with the input's shape: at least the value above, and for fp16 detection heads
