@@ -1,24 +1,30 @@
-// Matrix-core (MFMA) forward of the 3-D deformable convolution for fp16 / bf16 tensors.
+// Matrix-core (MFMA) forward of the 3-D deformable convolution for fp16 / bf16 / fp32 tensors.
 //
 //   y[b, o, q] = sum_{k, c} Wt[o, c, k] * col[c, k, q] + bias[o],
 //   col[c, k, q] = mask[k, q] * Z(x[b, c], p(k, q))           (zero-padded trilinear sample)
 //
 // is a GEMM whose B operand (the column matrix, Cin*K x positions) is never written to memory:
-// every wavefront owns 32 output positions and builds the 16 x 32 B fragment of one (tap, 16
-// channel) slice directly in registers, then issues v_mfma_f32_32x32x16_{f16,bf16} against the
-// weight fragments of up to MT 32-row blocks of output channels, accumulating in fp32.
+// wavefronts build the fragment of one (tap, channel slice) directly in registers from the gathered
+// corners and multiply it with weight fragments, accumulating in fp32.  Three kernels share that plan:
+//   * dcn_forward_shared_taps_kernel: 16-bit tensors with 32 or 64 channels per group (the usual
+//     layers).  A workgroup owns 64 positions; per group of four taps one wavefront per tap works
+//     the tap geometry out with one position per lane and leaves a 64-byte record per (tap,
+//     position) in LDS; then each wavefront gathers and blends 16 positions in the load layout
+//     (position l / 4, 16-byte piece l % 4: the four pieces of a voxel in one cache look-up), moves
+//     the piece to the matrix layout with ds_bpermute and issues v_mfma_f32_16x16x32_{f16,bf16}.
+//   * dcn_forward_mfma16_kernel: the same 16 x 16 x 32 tiling with the geometry worked out by the
+//     lanes that load (other channel counts that are multiples of 32, fp32 through 16x16x4).
+//   * dcn_forward_mfma_kernel: 32 positions per wavefront and v_mfma_f32_32x32x16, for channel
+//     counts that are multiples of 16 but not of 32.
 //
 // Data layout chosen for the gather, not for the GEMM:
-//   * x is first transposed to channels-last [B, D*H*W, Cin] (workspace).  The MFMA B fragment
-//     gives lane l the 8 consecutive K rows (l / 32) * 8 .. + 7 of column l % 32, so with
-//     channels-last storage ONE 16-byte load per trilinear corner brings exactly the 8 channels a
-//     lane needs: 8 loads + 64 mixed-precision FMAs per lane produce its part of the fragment;
-//   * the 8 corner offsets / weights (x mask) of a (tap, position) are computed once per lane and
-//     reused for every channel slice of the deformable group (positions are exact in fp32 for
-//     16-bit offsets);
-//   * weights are re-laid out once per call into A-fragment order [group][tap][slice][row block]
-//     [lane][8] (workspace) so that a fragment is one coalesced 16-byte load per lane (L2 hits).
-// The sampling gather, not the matrix core, bounds this kernel: per (tap, position) 8 corners x
+//   * x is first transposed to channels-last [B, D*H*W, Cin] (workspace), so that ONE 16-byte load
+//     per trilinear corner brings the 8 consecutive channels a lane contributes to a fragment;
+//   * the 8 corner offsets / weights (x mask) of a (tap, position) are computed once and reused for
+//     every channel slice of the deformable group (positions are exact in fp32 for 16-bit offsets);
+//   * weights are re-laid out once per call into fragment order (workspace) so that a fragment is
+//     one coalesced 16-byte load per lane, or one LDS read where a workgroup shares them.
+// The sampling gather, not the matrix core, bounds these kernels: per (tap, position) 8 corners x
 // Cin channels are fetched, 8 x more bytes than the fragment holds.
 #include <cstdint>
 #include <cstdlib>
