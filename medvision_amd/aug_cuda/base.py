@@ -21,15 +21,12 @@ import torch
 
 def _peak_mib():
     """Peak of allocated GPU memory in MiB, as ``torch.cuda.max_memory_allocated`` reports it; read
-    from the allocator's counters directly (the public call flattens the whole statistics tree
-    first, tens of microseconds per stage)."""
+    from the nested statistics (that call flattens the whole tree first, tens of microseconds per
+    stage)."""
     if not torch.cuda.is_available():
         return 0.0
-    try:
-        stats = torch._C._cuda_memoryStats(torch.cuda.current_device())
-        return stats["allocated_bytes"]["all"]["peak"] / 2 ** 20
-    except Exception:   # private interface: fall back to the public one
-        return torch.cuda.max_memory_allocated() / 2 ** 20
+    stats = torch.cuda.memory_stats_as_nested_dict()     # {} before the first GPU call
+    return stats.get("allocated_bytes", {}).get("all", {}).get("peak", 0) / 2 ** 20
 
 
 class CudaAugBase:
