@@ -122,6 +122,12 @@ __global__ void add_from_f32_kernel(T *dst, const float *src, long n) {
 int roi_forward_tiled(const void *input, const void *rois, void *output, int dtype,
                       const RoiProblem &p, void *workspace, size_t *need, hipStream_t s);
 
+// roi_resample.hip: backward of the same problems through LDS tiles of the source boxes; `acc` is the
+// fp32 buffer the gradient is added to; -1 when it does not apply
+bool roi_backward_tiled_applies(int dtype, const RoiProblem &p);
+int roi_backward_tiled(const void *grad_output, const void *rois, float *acc, int dtype,
+                       const RoiProblem &p, hipStream_t s);
+
 // roi_pool.hip: separable LDS kernels for plain boxes with small outputs; -1 when not applicable
 size_t roi_pool_forward_workspace(int dtype, const RoiProblem &p);
 int roi_pool_forward(const void *input, const void *rois, void *output, int dtype,
@@ -206,11 +212,25 @@ int roi_backward(const void *grad_output, const void *rois, void *grad_input, in
   const bool narrow = dtype == MV_F16 || dtype == MV_BF16;
   MV_REQUIRE(!narrow || workspace, "16-bit backward needs an fp32 workspace");
   hipStream_t s = static_cast<hipStream_t>(stream);
+  const long total = static_cast<long>(batch) * channels * depth * height * width;
+  const int fill_blocks = static_cast<int>(std::min<long>((total + 1023) / 1024, 65536));
+  if (roi_backward_tiled_applies(dtype, p)) {
+    // 16-bit tensors: sums in the fp32 workspace; fp32: sums in grad_input
+    float *ws = static_cast<float *>(workspace);
+    if (narrow) hipLaunchKernelGGL(fill_zero_kernel, dim3(fill_blocks), dim3(256), 0, s, ws, total);
+    st = roi_backward_tiled(grad_output, rois, narrow ? ws : static_cast<float *>(grad_input), dtype, p, s);
+    if (st) return st;
+    if (!narrow) return MV_OK;
+    MV_DISPATCH(dtype, {
+      if constexpr (sizeof(T) == 2)
+        hipLaunchKernelGGL((add_from_f32_kernel<T>), dim3(fill_blocks), dim3(256), 0, s,
+                           static_cast<T *>(grad_input), static_cast<const float *>(workspace), total);
+    });
+    return check_launch("add_from_f32_kernel");
+  }
   const int gathered = roi_backward_gather(grad_output, rois, grad_input, dtype, p, s);
   if (gathered >= 0) return gathered;
   const dim3 grid(p.chunks * num_rois), block(kRoiThreads);
-  const long total = static_cast<long>(batch) * channels * depth * height * width;
-  const int fill_blocks = static_cast<int>(std::min<long>((total + 1023) / 1024, 65536));
   if (narrow) {
     hipLaunchKernelGGL(fill_zero_kernel, dim3(fill_blocks), dim3(256), 0, s,
                        static_cast<float *>(workspace), total);

@@ -21,6 +21,8 @@
 // Coordinates: box-relative in the coordinate type CT (fp32 for 16-bit tensors, fp64 for fp32
 // tensors), then floor / fraction in CT.  Tiles whose box is not clipped skip the [-1,S] tests and
 // the border clamps.
+#include <algorithm>
+
 #include "common.hpp"
 #include "roi_geometry.hpp"
 #include "sampling.hpp"
@@ -1323,6 +1325,200 @@ int roi_forward_tiled(const void *input, const void *rois, void *output, int dty
     default:
       return -1;
   }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Backward of the same problems (grid 1, orders 0 and 1).  The forward's plan is used in reverse: an
+// item is (output tile, channel), its source box becomes an LDS tile of 32-bit FIXED-POINT sums, every
+// output voxel of the tile adds weight * grad_output to the <= 8 voxels its sample touches, and the
+// tile's non-zero sums go to the fp32 gradient buffer as one atomic per voxel, contiguous along x
+// (one request per 64-byte sector instead of eight scattered ones per output voxel).  Integer sums
+// because an LDS fp32 atomic retires one lane at a time.  Scale: |term| <= max|grad_output| < 2^e
+// is mapped to 2^t quanta, t = 30 - ceil(log2(terms a voxel can get from one tile)) >= 19 (a tile has
+// 2^11 voxels; bins of about a voxel give t = 23), so no sum leaves 31 bits and a term is rounded by
+// at most 2^-(t+1) of that bound.  Sample coordinates and the tap decisions are fp64, as in the general
+// kernel.  Boxes beyond the LDS tile, and every term when grad_output holds a NaN or an infinity,
+// go to the buffer as single fp32 atomics.
+constexpr int kScatterThreads = 512;
+constexpr int kScatterLds = 74 * 1024;
+constexpr int kScatterCells = 2048;   // output voxels per item
+constexpr int kTermBits = 19;
+
+template <typename T, int TX, int TY, int TZ>
+__global__ __launch_bounds__(kScatterThreads, 4) void roi_backward_tiles_kernel(
+    const T *__restrict__ gout, const float *__restrict__ rois, float *__restrict__ acc, const RoiProblem p,
+    const PlanShape ps, const unsigned total, const unsigned work) {
+  static_assert(TX * TY * TZ == kScatterCells && kScatterCells <= (1 << (30 - kTermBits)), "tile shape");
+  constexpr int kPerThread = kScatterCells / kScatterThreads, kWaves = kScatterThreads / kWave;
+  __shared__ TilePlan plans[kPlanSlots];
+  __shared__ __attribute__((aligned(16))) int tile[kScatterLds / 4];
+  __shared__ unsigned bound_part[2][kWaves];
+  const unsigned per_roi = static_cast<unsigned>(ps.tiles_x) * ps.tiles_y * ps.tiles_z;
+  if (threadIdx.x < kWave) {
+    const unsigned item = blockIdx.x + (threadIdx.x >> 2) * gridDim.x;
+    plan_item_lanes(rois, p, ps, item < work ? item : kDone, total, per_roi, &plans[threadIdx.x >> 2]);
+  }
+  // the tile starts at zero; the flush of an item leaves it at zero for the next one
+  for (int i = threadIdx.x * 4; i < kScatterLds / 4; i += kScatterThreads * 4)
+    *reinterpret_cast<int4 *>(tile + i) = int4{0, 0, 0, 0};
+  __syncthreads();
+  const long plane = static_cast<long>(p.D) * p.H * p.W, ovol = static_cast<long>(p.od) * p.oh * p.ow;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  for (unsigned slot = 0; slot < kPlanSlots; slot++) {
+    const unsigned item = blockIdx.x + slot * gridDim.x;
+    if (item >= work) break;
+    const TilePlan &r = plans[slot];
+    const int mode = r.mode;
+    if (mode == 0 || mode == 4) continue;
+    const int n0 = r.n[0], n1 = r.n[1], n2 = r.n[2], l0 = r.lo[0], l1 = r.lo[1], l2 = r.lo[2];
+    const unsigned chan = p.C > 1 ? ps.by_total.div(item) : 0u;
+    float *const vol = acc + (static_cast<long>(r.batch) * p.C + chan) * plane;
+    const T *const gsrc = gout + (static_cast<long>(r.roi) * p.C + chan) * ovol;
+    // The item's grad_output, and the largest magnitude in it as the bit pattern of a float (patterns
+    // of non-negative floats order like unsigned integers, NaNs above infinity).
+    float gv[kPerThread];
+    unsigned bits = 0;
+#pragma unroll
+    for (int k = 0; k < kPerThread; k++) {
+      const int c = threadIdx.x + k * kScatterThreads;
+      const int ox = r.t0[0] + c % TX, oy = r.t0[1] + (c / TX) % TY, oz = r.t0[2] + c / (TX * TY);
+      const bool in = ox < p.ow && oy < p.oh && oz < p.od;
+      gv[k] = in ? static_cast<float>(load(gsrc + (static_cast<long>(oz) * p.oh + oy) * p.ow + ox)) : 0.f;
+      bits = max(bits, __float_as_uint(fabsf(gv[k])));
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) bits = max(bits, static_cast<unsigned>(__shfl_xor(static_cast<int>(bits), d)));
+    if (lane == 0) bound_part[slot & 1][wave] = bits;
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < kWaves; w++) bits = max(bits, bound_part[slot & 1][w]);
+    bits = __builtin_amdgcn_readfirstlane(bits);
+    if (bits == 0) continue;                                  // nothing to add
+    const bool in_lds = bits < 0x7f800000u && mode != 2;      // finite terms, box within the tile
+    // Quanta per unit: a voxel gets at most one term from each output voxel whose sample lies within
+    // one voxel of it on every axis, i.e. inside a ball of radius sqrt(3); along output axis j (bin
+    // b_j = length of column j of the map) that leaves floor(2 sqrt(3) / b_j) + 1 indices.
+    int terms = 1;
+#pragma unroll
+    for (int j = 0; j < 3; j++) {
+      const float bj = sqrtf(r.mapf[1 + j] * r.mapf[1 + j] + r.mapf[5 + j] * r.mapf[5 + j] + r.mapf[9 + j] * r.mapf[9 + j]);
+      const int ext = j == 0 ? TX : (j == 1 ? TY : TZ);
+      terms *= static_cast<int>(fminf(3.4642f / bj * 1.00001f + 1.f, static_cast<float>(ext)));
+    }
+    const int term_bits = 30 - (32 - __clz(terms - 1));   // 30 - ceil(log2 terms) >= kTermBits
+    const int ex = min(max(127 + 126 + term_bits - static_cast<int>(bits >> 23), 1), 253);   // 2^(ex - 127) = 2^term_bits / 2^e
+    const float to_quanta = __uint_as_float(static_cast<unsigned>(ex) << 23);
+    const float from_quanta = __uint_as_float(static_cast<unsigned>(254 - ex) << 23);
+#pragma unroll
+    for (int k = 0; k < kPerThread; k++) {
+      const int c = threadIdx.x + k * kScatterThreads;
+      const int x = c % TX, y = (c / TX) % TY, z = c / (TX * TY);
+      const float g = gv[k];
+      if (g == 0.f) continue;
+      const double vx = r.map[0] + l0 + r.map[1] * x + r.map[2] * y + r.map[3] * z;
+      const double vy = r.map[4] + l1 + r.map[5] * x + r.map[6] * y + r.map[7] * z;
+      const double vz = r.map[8] + l2 + r.map[9] * x + r.map[10] * y + r.map[11] * z;
+      int xi[2], yi[2], zi[2];
+      float fx, fy, fz;
+      if (!clamped_tap<float>(vx, p.W, xi[0], xi[1], fx, p.order) || !clamped_tap<float>(vy, p.H, yi[0], yi[1], fy, p.order) ||
+          !clamped_tap<float>(vz, p.D, zi[0], zi[1], fz, p.order))
+        continue;
+      const float wx[2] = {1.f - fx, fx}, wy[2] = {1.f - fy, fy}, wz[2] = {1.f - fz, fz};
+#pragma unroll
+      for (int n = 0; n < 8; n++) {
+        const int a = n >> 2, b = (n >> 1) & 1, e = n & 1;
+        const float w = wz[a] * wy[b] * wx[e];
+        if (w == 0.f) continue;
+        const float term = g * w;
+        const unsigned bx = static_cast<unsigned>(xi[e] - l0), by = static_cast<unsigned>(yi[b] - l1),
+                       bz = static_cast<unsigned>(zi[a] - l2);
+        if (in_lds && bx < static_cast<unsigned>(n0) && by < static_cast<unsigned>(n1) && bz < static_cast<unsigned>(n2))
+          __hip_atomic_fetch_add(tile + (bz * n1 + by) * n0 + bx, __float2int_rn(term * to_quanta),
+                                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        else
+          atomic_add(vol + (static_cast<long>(zi[a]) * p.H + yi[b]) * p.W + xi[e], term);
+      }
+    }
+    if (in_lds) {
+      __syncthreads();
+      // a wavefront takes `per` rows of the box at a time (two or more when a row is short)
+      const int rows = n1 * n2, per = n0 <= kWave / 2 ? kWave / n0 : 1;
+      const int sub = per > 1 ? lane / n0 : 0, bx0 = per > 1 ? lane - sub * n0 : lane;
+      for (int row0 = wave * per; row0 < rows; row0 += (kScatterThreads / kWave) * per) {
+        const int row = row0 + sub;
+        if (sub >= per || row >= rows) continue;
+        const int bz = row / n1, by = row - bz * n1;
+        float *const dst = vol + (static_cast<long>(bz + l2) * p.H + (by + l1)) * p.W + l0;
+        for (int bx = bx0; bx < n0; bx += kWave) {
+          const int q = tile[row * n0 + bx];
+          if (q != 0) {
+            tile[row * n0 + bx] = 0;
+            atomic_add(dst + bx, static_cast<float>(q) * from_quanta);
+          }
+        }
+      }
+      __syncthreads();
+    }
+  }
+}
+
+struct ScatterTiling { int TX, TY, TZ; long tx, ty, tz, per_roi, total, work; };
+static ScatterTiling scatter_tiling(const RoiProblem &p) {
+  ScatterTiling t;
+  const bool flat = p.ndim == 2;
+  t.TX = flat ? 32 : 16; t.TY = flat ? 64 : 16; t.TZ = flat ? 1 : 8;
+  t.tx = (p.ow + t.TX - 1) / t.TX; t.ty = (p.oh + t.TY - 1) / t.TY; t.tz = (p.od + t.TZ - 1) / t.TZ;
+  t.per_roi = t.tx * t.ty * t.tz; t.total = t.per_roi * static_cast<long>(p.R); t.work = t.total * p.C;
+  return t;
+}
+
+bool roi_backward_tiled_applies(int dtype, const RoiProblem &p) {
+  const long vox = static_cast<long>(p.od) * p.oh * p.ow;
+  if (p.sampling_ratio != 1 || (p.order != 0 && p.order != 1) || vox < 4096 || p.ow < 16 || p.R == 0) return false;
+  if (dtype != MV_F16 && dtype != MV_BF16 && dtype != MV_F32) return false;
+  return scatter_tiling(p).work < (1L << 31) && static_cast<long>(p.D) * p.H * p.W * 4 < (1L << 31);
+}
+
+// `acc`: fp32 gradient buffer [N, C, D, H, W] that the terms are added to.  Returns -1 when the path
+// does not apply.
+int roi_backward_tiled(const void *grad_output, const void *rois, float *acc, int dtype,
+                       const RoiProblem &p, hipStream_t s) {
+  if (!roi_backward_tiled_applies(dtype, p)) return -1;
+  const ScatterTiling t = scatter_tiling(p);
+  const bool flat = p.ndim == 2;
+  const int TX = t.TX, TY = t.TY, TZ = t.TZ;
+  const long tx = t.tx, ty = t.ty, tz = t.tz, per_roi = t.per_roi, total = t.total, work = t.work;
+  PlanShape ps;
+  ps.tiles_x = static_cast<int>(tx); ps.tiles_y = static_cast<int>(ty); ps.tiles_z = static_cast<int>(tz);
+  ps.tx = TX; ps.ty = TY; ps.tz = TZ;
+  ps.vec = 0;
+  ps.cap = kScatterLds / 4;
+  ps.threads = kScatterThreads; ps.max_items = 0;
+  ps.halo_lo = 0; ps.halo_hi = 1;
+  ps.warm_groups = 0;
+  ps.es = 4;
+  ps.by_per_roi.set(static_cast<unsigned>(per_roi));
+  ps.by_tiles_x.set(static_cast<unsigned>(tx));
+  ps.by_tiles_y.set(static_cast<unsigned>(ty));
+  ps.by_total.set(static_cast<unsigned>(total));
+  ps.by_slots.set(1);
+  long blocks = std::min<long>(work, 2L * compute_units());
+  blocks = std::max(blocks, (work + kPlanSlots - 1) / kPlanSlots);
+  MV_DISPATCH(dtype, {
+    if constexpr (sizeof(T) <= 4) {
+      if (flat)
+        hipLaunchKernelGGL((roi_backward_tiles_kernel<T, 32, 64, 1>), dim3(static_cast<unsigned>(blocks)),
+                           dim3(kScatterThreads), 0, s, static_cast<const T *>(grad_output),
+                           static_cast<const float *>(rois), acc, p, ps, static_cast<unsigned>(total),
+                           static_cast<unsigned>(work));
+      else
+        hipLaunchKernelGGL((roi_backward_tiles_kernel<T, 16, 16, 8>), dim3(static_cast<unsigned>(blocks)),
+                           dim3(kScatterThreads), 0, s, static_cast<const T *>(grad_output),
+                           static_cast<const float *>(rois), acc, p, ps, static_cast<unsigned>(total),
+                           static_cast<unsigned>(work));
+    }
+  });
+  return check_launch("roi_backward_tiles_kernel");
 }
 
 }  // namespace mv
