@@ -1340,15 +1340,22 @@ int roi_forward_tiled(const void *input, const void *rois, void *output, int dty
 // kernel.  Boxes beyond the LDS tile, and every term when grad_output holds a NaN or an infinity,
 // go to the buffer as single fp32 atomics.
 constexpr int kScatterThreads = 512;
-constexpr int kScatterLds = 74 * 1024;
-constexpr int kScatterCells = 2048;   // output voxels per item
+#ifndef MV_SCATTER_SHAPE
+#define MV_SCATTER_SHAPE 16, 16, 8
+#define MV_SCATTER_SHAPE_2D 32, 64, 1
+#define MV_SCATTER_LDS (74 * 1024)
+#define MV_SCATTER_WGS 2
+#endif
+constexpr int kScatterLds = MV_SCATTER_LDS;
+constexpr int kScatterWgs = MV_SCATTER_WGS;     // workgroups per compute unit
 constexpr int kTermBits = 19;
 
 template <typename T, int TX, int TY, int TZ>
-__global__ __launch_bounds__(kScatterThreads, 4) void roi_backward_tiles_kernel(
+__global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward_tiles_kernel(
     const T *__restrict__ gout, const float *__restrict__ rois, float *__restrict__ acc, const RoiProblem p,
     const PlanShape ps, const unsigned total, const unsigned work) {
-  static_assert(TX * TY * TZ == kScatterCells && kScatterCells <= (1 << (30 - kTermBits)), "tile shape");
+  constexpr int kScatterCells = TX * TY * TZ;   // output voxels per item
+  static_assert(kScatterCells % kScatterThreads == 0 && kScatterCells <= (1 << (30 - kTermBits)), "tile shape");
   constexpr int kPerThread = kScatterCells / kScatterThreads, kWaves = kScatterThreads / kWave;
   __shared__ TilePlan plans[kPlanSlots];
   __shared__ __attribute__((aligned(16))) int tile[kScatterLds / 4];
@@ -1368,12 +1375,20 @@ __global__ __launch_bounds__(kScatterThreads, 4) void roi_backward_tiles_kernel(
     const unsigned item = blockIdx.x + slot * gridDim.x;
     if (item >= work) break;
     const TilePlan &r = plans[slot];
-    const int mode = r.mode;
+    const int mode = plan_scalar(&r.mode);
     if (mode == 0 || mode == 4) continue;
-    const int n0 = r.n[0], n1 = r.n[1], n2 = r.n[2], l0 = r.lo[0], l1 = r.lo[1], l2 = r.lo[2];
+    // the record's values in scalar registers: the LDS atomics below keep the compiler from holding
+    // anything it reads from LDS across them
+    const int n0 = plan_scalar(&r.n[0]), n1 = plan_scalar(&r.n[1]), n2 = plan_scalar(&r.n[2]);
+    const int l0 = plan_scalar(&r.lo[0]), l1 = plan_scalar(&r.lo[1]), l2 = plan_scalar(&r.lo[2]);
+    const int t0x = plan_scalar(&r.t0[0]), t0y = plan_scalar(&r.t0[1]), t0z = plan_scalar(&r.t0[2]);
+    double map[12];
+#pragma unroll
+    for (int i = 0; i < 12; i++) map[i] = uniform(r.map[i]);
+    map[0] += l0; map[4] += l1; map[8] += l2;   // to volume coordinates
     const unsigned chan = p.C > 1 ? ps.by_total.div(item) : 0u;
-    float *const vol = acc + (static_cast<long>(r.batch) * p.C + chan) * plane;
-    const T *const gsrc = gout + (static_cast<long>(r.roi) * p.C + chan) * ovol;
+    float *const vol = acc + (static_cast<long>(plan_scalar(&r.batch)) * p.C + chan) * plane;
+    const T *const gsrc = gout + (static_cast<long>(plan_scalar(&r.roi)) * p.C + chan) * ovol;
     // The item's grad_output, and the largest magnitude in it as the bit pattern of a float (patterns
     // of non-negative floats order like unsigned integers, NaNs above infinity).
     float gv[kPerThread];
@@ -1381,7 +1396,7 @@ __global__ __launch_bounds__(kScatterThreads, 4) void roi_backward_tiles_kernel(
 #pragma unroll
     for (int k = 0; k < kPerThread; k++) {
       const int c = threadIdx.x + k * kScatterThreads;
-      const int ox = r.t0[0] + c % TX, oy = r.t0[1] + (c / TX) % TY, oz = r.t0[2] + c / (TX * TY);
+      const int ox = t0x + c % TX, oy = t0y + (c / TX) % TY, oz = t0z + c / (TX * TY);
       const bool in = ox < p.ow && oy < p.oh && oz < p.od;
       gv[k] = in ? static_cast<float>(load(gsrc + (static_cast<long>(oz) * p.oh + oy) * p.ow + ox)) : 0.f;
       bits = max(bits, __float_as_uint(fabsf(gv[k])));
@@ -1401,7 +1416,8 @@ __global__ __launch_bounds__(kScatterThreads, 4) void roi_backward_tiles_kernel(
     int terms = 1;
 #pragma unroll
     for (int j = 0; j < 3; j++) {
-      const float bj = sqrtf(r.mapf[1 + j] * r.mapf[1 + j] + r.mapf[5 + j] * r.mapf[5 + j] + r.mapf[9 + j] * r.mapf[9 + j]);
+      const float c0 = static_cast<float>(map[1 + j]), c1 = static_cast<float>(map[5 + j]), c2 = static_cast<float>(map[9 + j]);
+      const float bj = sqrtf(c0 * c0 + c1 * c1 + c2 * c2);
       const int ext = j == 0 ? TX : (j == 1 ? TY : TZ);
       terms *= static_cast<int>(fminf(3.4642f / bj * 1.00001f + 1.f, static_cast<float>(ext)));
     }
@@ -1409,52 +1425,96 @@ __global__ __launch_bounds__(kScatterThreads, 4) void roi_backward_tiles_kernel(
     const int ex = min(max(127 + 126 + term_bits - static_cast<int>(bits >> 23), 1), 253);   // 2^(ex - 127) = 2^term_bits / 2^e
     const float to_quanta = __uint_as_float(static_cast<unsigned>(ex) << 23);
     const float from_quanta = __uint_as_float(static_cast<unsigned>(254 - ex) << 23);
+    // One copy of the loop per (interior, order): a box that is not clipped holds samples in
+    // [0, size - 1) only, so the low tap is the floor and neither the void test nor the clamps are needed.
+    auto scatter_cells = [&](auto interior_tag, auto order_tag) {
+    constexpr bool kInterior = decltype(interior_tag)::value;
+    constexpr int kOrder = decltype(order_tag)::value;
 #pragma unroll
     for (int k = 0; k < kPerThread; k++) {
       const int c = threadIdx.x + k * kScatterThreads;
       const int x = c % TX, y = (c / TX) % TY, z = c / (TX * TY);
       const float g = gv[k];
       if (g == 0.f) continue;
-      const double vx = r.map[0] + l0 + r.map[1] * x + r.map[2] * y + r.map[3] * z;
-      const double vy = r.map[4] + l1 + r.map[5] * x + r.map[6] * y + r.map[7] * z;
-      const double vz = r.map[8] + l2 + r.map[9] * x + r.map[10] * y + r.map[11] * z;
+      const double vx = map[0] + map[1] * x + map[2] * y + map[3] * z;
+      const double vy = map[4] + map[5] * x + map[6] * y + map[7] * z;
+      const double vz = map[8] + map[9] * x + map[10] * y + map[11] * z;
       int xi[2], yi[2], zi[2];
       float fx, fy, fz;
-      if (!clamped_tap<float>(vx, p.W, xi[0], xi[1], fx, p.order) || !clamped_tap<float>(vy, p.H, yi[0], yi[1], fy, p.order) ||
-          !clamped_tap<float>(vz, p.D, zi[0], zi[1], fz, p.order))
+      if constexpr (kInterior) {
+        const double flx = floor(vx), fly = floor(vy), flz = floor(vz);
+        xi[0] = static_cast<int>(flx); yi[0] = static_cast<int>(fly); zi[0] = static_cast<int>(flz);
+        xi[1] = xi[0] + 1; yi[1] = yi[0] + 1; zi[1] = zi[0] + 1;
+        const double dx = vx - flx, dy = vy - fly, dz = vz - flz;
+        if constexpr (kOrder == 0) {
+          fx = (1.0 - dx >= 0.5) ? 0.f : 1.f; fy = (1.0 - dy >= 0.5) ? 0.f : 1.f; fz = (1.0 - dz >= 0.5) ? 0.f : 1.f;
+        } else {
+          fx = static_cast<float>(dx); fy = static_cast<float>(dy); fz = static_cast<float>(dz);
+        }
+      } else if (!clamped_tap<float>(vx, p.W, xi[0], xi[1], fx, kOrder) || !clamped_tap<float>(vy, p.H, yi[0], yi[1], fy, kOrder) ||
+                 !clamped_tap<float>(vz, p.D, zi[0], zi[1], fz, kOrder)) {
         continue;
-      const float wx[2] = {1.f - fx, fx}, wy[2] = {1.f - fy, fy}, wz[2] = {1.f - fz, fz};
-#pragma unroll
-      for (int n = 0; n < 8; n++) {
-        const int a = n >> 2, b = (n >> 1) & 1, e = n & 1;
-        const float w = wz[a] * wy[b] * wx[e];
-        if (w == 0.f) continue;
-        const float term = g * w;
-        const unsigned bx = static_cast<unsigned>(xi[e] - l0), by = static_cast<unsigned>(yi[b] - l1),
-                       bz = static_cast<unsigned>(zi[a] - l2);
-        if (in_lds && bx < static_cast<unsigned>(n0) && by < static_cast<unsigned>(n1) && bz < static_cast<unsigned>(n2))
-          __hip_atomic_fetch_add(tile + (bz * n1 + by) * n0 + bx, __float2int_rn(term * to_quanta),
-                                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        else
-          atomic_add(vol + (static_cast<long>(zi[a]) * p.H + yi[b]) * p.W + xi[e], term);
       }
+      const float wx[2] = {1.f - fx, fx}, wy[2] = {1.f - fy, fy}, wz[2] = {1.f - fz, fz};
+      const float wzy[4] = {wz[0] * wy[0], wz[0] * wy[1], wz[1] * wy[0], wz[1] * wy[1]};
+      const unsigned bx[2] = {static_cast<unsigned>(xi[0] - l0), static_cast<unsigned>(xi[1] - l0)};
+      const unsigned by[2] = {static_cast<unsigned>(yi[0] - l1), static_cast<unsigned>(yi[1] - l1)};
+      const unsigned bz[2] = {static_cast<unsigned>(zi[0] - l2), static_cast<unsigned>(zi[1] - l2)};
+      // the box holds every voxel a sample of the tile touches; a cell that disagrees takes the slow way
+      const bool inside = in_lds && max(bx[0], bx[1]) < static_cast<unsigned>(n0) &&
+                          max(by[0], by[1]) < static_cast<unsigned>(n1) && max(bz[0], bz[1]) < static_cast<unsigned>(n2);
+      if (inside) {
+        const float gq = g * to_quanta;   // a power of two: the products below are the terms in quanta
+        const int rows[4] = {__mul24(__mul24(bz[0], n1) + by[0], n0), __mul24(__mul24(bz[0], n1) + by[1], n0),
+                             __mul24(__mul24(bz[1], n1) + by[0], n0), __mul24(__mul24(bz[1], n1) + by[1], n0)};
+#pragma unroll
+        for (int n = 0; n < 8; n++)
+          __hip_atomic_fetch_add(tile + rows[n >> 1] + static_cast<int>(bx[n & 1]),
+                                 __float2int_rn(gq * (wzy[n >> 1] * wx[n & 1])), __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_WORKGROUP);
+      } else {
+#pragma unroll 1
+        for (int n = 0; n < 8; n++) {
+          const float w = wzy[n >> 1] * wx[n & 1];
+          if (w != 0.f)
+            atomic_add(vol + (static_cast<long>(zi[n >> 2]) * p.H + yi[(n >> 1) & 1]) * p.W + xi[n & 1], g * w);
+        }
+      }
+    }
+    };
+    using Yes = std::true_type;
+    using No = std::false_type;
+    if (mode == 3 && p.ndim == 3) {
+      if (p.order == 0) scatter_cells(Yes{}, std::integral_constant<int, 0>{});
+      else scatter_cells(Yes{}, std::integral_constant<int, 1>{});
+    } else {
+      if (p.order == 0) scatter_cells(No{}, std::integral_constant<int, 0>{});
+      else scatter_cells(No{}, std::integral_constant<int, 1>{});
     }
     if (in_lds) {
       __syncthreads();
-      // a wavefront takes `per` rows of the box at a time (two or more when a row is short)
-      const int rows = n1 * n2, per = n0 <= kWave / 2 ? kWave / n0 : 1;
-      const int sub = per > 1 ? lane / n0 : 0, bx0 = per > 1 ? lane - sub * n0 : lane;
-      for (int row0 = wave * per; row0 < rows; row0 += (kScatterThreads / kWave) * per) {
-        const int row = row0 + sub;
-        if (sub >= per || row >= rows) continue;
-        const int bz = row / n1, by = row - bz * n1;
-        float *const dst = vol + (static_cast<long>(bz + l2) * p.H + (by + l1)) * p.W + l0;
-        for (int bx = bx0; bx < n0; bx += kWave) {
-          const int q = tile[row * n0 + bx];
-          if (q != 0) {
-            tile[row * n0 + bx] = 0;
-            atomic_add(dst + bx, static_cast<float>(q) * from_quanta);
-          }
+      // Lanes run along the box's cells in memory order (consecutive lanes = consecutive voxels of a
+      // row = one request per 64-byte sector); several independent reads per lane are in flight
+      // before the first is looked at.
+      constexpr int kAtOnce = 8;
+      const int box = n0 * n1 * n2;
+      const float inv_row = 1.f / static_cast<float>(n0), inv_rows = 1.f / static_cast<float>(n1);
+      for (int base = threadIdx.x; base < box; base += kScatterThreads * kAtOnce) {
+        int q[kAtOnce];
+#pragma unroll
+        for (int u = 0; u < kAtOnce; u++) {
+          const int i = base + u * kScatterThreads;
+          q[u] = i < box ? tile[i] : 0;
+        }
+#pragma unroll
+        for (int u = 0; u < kAtOnce; u++) {
+          if (q[u] == 0) continue;
+          const int i = base + u * kScatterThreads;
+          tile[i] = 0;
+          const int row = div_small(i, inv_row), bx = i - row * n0;
+          const int bz = div_small(row, inv_rows), by = row - bz * n1;
+          atomic_add(vol + (static_cast<long>(bz + l2) * p.H + (by + l1)) * p.W + (l0 + bx),
+                     static_cast<float>(q[u]) * from_quanta);
         }
       }
       __syncthreads();
@@ -1466,7 +1526,8 @@ struct ScatterTiling { int TX, TY, TZ; long tx, ty, tz, per_roi, total, work; };
 static ScatterTiling scatter_tiling(const RoiProblem &p) {
   ScatterTiling t;
   const bool flat = p.ndim == 2;
-  t.TX = flat ? 32 : 16; t.TY = flat ? 64 : 16; t.TZ = flat ? 1 : 8;
+  const int vol[3] = {MV_SCATTER_SHAPE}, img[3] = {MV_SCATTER_SHAPE_2D};
+  t.TX = flat ? img[0] : vol[0]; t.TY = flat ? img[1] : vol[1]; t.TZ = flat ? img[2] : vol[2];
   t.tx = (p.ow + t.TX - 1) / t.TX; t.ty = (p.oh + t.TY - 1) / t.TY; t.tz = (p.od + t.TZ - 1) / t.TZ;
   t.per_roi = t.tx * t.ty * t.tz; t.total = t.per_roi * static_cast<long>(p.R); t.work = t.total * p.C;
   return t;
@@ -1502,17 +1563,17 @@ int roi_backward_tiled(const void *grad_output, const void *rois, float *acc, in
   ps.by_tiles_y.set(static_cast<unsigned>(ty));
   ps.by_total.set(static_cast<unsigned>(total));
   ps.by_slots.set(1);
-  long blocks = std::min<long>(work, 2L * compute_units());
+  long blocks = std::min<long>(work, static_cast<long>(kScatterWgs) * compute_units());
   blocks = std::max(blocks, (work + kPlanSlots - 1) / kPlanSlots);
   MV_DISPATCH(dtype, {
     if constexpr (sizeof(T) <= 4) {
       if (flat)
-        hipLaunchKernelGGL((roi_backward_tiles_kernel<T, 32, 64, 1>), dim3(static_cast<unsigned>(blocks)),
+        hipLaunchKernelGGL((roi_backward_tiles_kernel<T, MV_SCATTER_SHAPE_2D>), dim3(static_cast<unsigned>(blocks)),
                            dim3(kScatterThreads), 0, s, static_cast<const T *>(grad_output),
                            static_cast<const float *>(rois), acc, p, ps, static_cast<unsigned>(total),
                            static_cast<unsigned>(work));
       else
-        hipLaunchKernelGGL((roi_backward_tiles_kernel<T, 16, 16, 8>), dim3(static_cast<unsigned>(blocks)),
+        hipLaunchKernelGGL((roi_backward_tiles_kernel<T, MV_SCATTER_SHAPE>), dim3(static_cast<unsigned>(blocks)),
                            dim3(kScatterThreads), 0, s, static_cast<const T *>(grad_output),
                            static_cast<const float *>(rois), acc, p, ps, static_cast<unsigned>(total),
                            static_cast<unsigned>(work));
