@@ -6,7 +6,7 @@ import math
 import pytest
 import torch
 
-from parity import BWD_TOL, FWD_TOL, assert_close, assert_nearest, rel_err
+from parity import BWD_TOL, FWD_TOL, NEAREST_EPS, assert_close, assert_nearest, rel_err
 import workloads as wl
 
 pytestmark = pytest.mark.gpu
@@ -165,6 +165,63 @@ def test_config2_backward_adjoint_full_size(ops, oracle):
     assert abs(lhs - rhs) <= 1e-5 * max(abs(lhs), 1.0)
     gwant = oracle.roi_align_backward(gy, rois, vol.shape, 1.0, 1, True, 1, True)
     assert_close(x.grad, gwant, BWD_TOL[torch.float32], "config 2 backward")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("order", [1, 0])
+def test_backward_through_source_box_tiles(ops, oracle, dtype, order):
+    """Backward of resampling-sized outputs (grid 1): output tiles add into an LDS tile of their source
+    box.  Several channels, rois that overlap on one image, rotated and plain rois, images, and a
+    strong reduction whose boxes exceed the LDS tile (every term then goes out as a single atomic)."""
+    g = wl.gen(800 + order)
+
+    def check(feat_shape, rois, out, rotated, what):
+        gy = torch.randn(rois.shape[0], feat_shape[1], *out, generator=g).to(dtype)
+        if order == 0:
+            # plain boxes with rational bins put samples exactly on 0.5 ties, where the rounding of the
+            # coordinate arithmetic decides: as in the forward tests those cells prove nothing
+            margin = oracle.roi_decision_margin(feat_shape, rois, out, 1.0, 1, True, rotated)
+            gy = gy * (margin > NEAREST_EPS[torch.float32])[:, None].to(dtype)
+        x = torch.zeros(feat_shape, dtype=dtype, device=DEV, requires_grad=True)
+        mod = (ops.RoIAlignRotated if rotated else ops.RoIAlign)(out, 1.0, 1)
+        mod(x, rois.to(DEV), order=order).backward(gy.to(DEV))
+        want = oracle.roi_align_backward(gy, rois, feat_shape, 1.0, 1, True, order, rotated)
+        assert float(want.abs().max()) > 0
+        assert_close(x.grad, want, BWD_TOL[dtype], what)
+
+    rois = torch.cat([wl.affine_rois(g, 2, (48, 40, 24)), wl.affine_rois(g, 2, (48, 40, 24))[:1]])
+    check((2, 3, 24, 40, 48), rois, (20, 24, 40), True, "rotated volumes")
+    boxes = torch.tensor([[0, 2.3, 1.2, 0.5, 40.1, 33.3, 20.7], [1, -3.0, 5.0, 2.0, 30.0, 45.0, 30.0],
+                          [1, 10.0, 3.0, 4.0, 52.0, 30.0, 18.0]])
+    check((2, 2, 24, 40, 48), boxes, (18, 24, 32), False, "plain volumes")
+    r2 = torch.tensor([[0, 45.0, 35.0, 80.0, 60.0, 0.4], [1, 40.0, 30.0, 100.0, 50.0, -1.2], [0, 30.0, 40.0, 50.0, 70.0, 2.0]])
+    check((2, 3, 70, 90), r2, (72, 80), True, "rotated images")
+    big = torch.tensor([[0, 64.0, 48.0, 24.0, 150.0, 110.0, 60.0, 0.2, -0.3, 0.5]])
+    check((1, 2, 48, 96, 128), big, (16, 20, 24), True, "boxes beyond the tile")
+
+
+def test_backward_tiles_with_zero_and_infinite_gradients(ops, oracle):
+    """A grad_output of zeros leaves the gradient untouched; an infinity reaches the voxels the oracle
+    sends it to (the tile that holds it adds its terms one by one, the others stay in fixed point)."""
+    g = wl.gen(820)
+    rois = wl.affine_rois(g, 2, (48, 40, 24))
+    shape, out = (2, 1, 24, 40, 48), (20, 24, 40)
+    for dtype in (torch.float32, torch.float16):
+        x = torch.zeros(shape, dtype=dtype, device=DEV, requires_grad=True)
+        y = ops.RoIAlignRotated(out, 1.0, 1)(x, rois.to(DEV))
+        y.backward(torch.zeros_like(y))
+        assert float(x.grad.abs().max()) == 0.0
+        gy = torch.randn(2, 1, *out, generator=g).to(dtype)
+        gy[1, 0, 9, 11, 17] = float("inf")
+        x = torch.zeros(shape, dtype=dtype, device=DEV, requires_grad=True)
+        ops.RoIAlignRotated(out, 1.0, 1)(x, rois.to(DEV)).backward(gy.to(DEV))
+        want = oracle.roi_align_backward(gy, rois, shape, 1.0, 1, True, 1, True)
+        got = x.grad.cpu().double()
+        assert torch.equal(torch.isfinite(got), torch.isfinite(want)) and int((~torch.isfinite(want)).sum()) == 8
+        assert torch.equal(got[~torch.isfinite(want)], want[~torch.isfinite(want)])
+        fin = torch.isfinite(want)
+        assert_close(torch.where(fin, got, torch.zeros_like(got)), torch.where(fin, want, torch.zeros_like(want)),
+                     BWD_TOL[dtype], "finite part")
 
 
 def test_config3_resize_and_crops(ops, oracle):
