@@ -242,7 +242,29 @@ __global__ __launch_bounds__(256) void dcn_backward_bias_kernel(const T *__restr
   const T *src = gy + (static_cast<long>(b) * s.Cout + o) * s.Q;
   const long q_end = min(static_cast<long>(blockIdx.z + 1) * kBiasSlab, s.Q);
   A v = A(0);
-  for (long q = static_cast<long>(blockIdx.z) * kBiasSlab + threadIdx.x; q < q_end; q += 256) v += load(src + q);
+  long q0 = static_cast<long>(blockIdx.z) * kBiasSlab;
+  if constexpr (sizeof(T) <= 4) {
+    // 16-byte pieces, four independent loads per lane and step (one load in flight per wavefront
+    // leaves the memory system idle most of the time)
+    constexpr int V = 16 / sizeof(T);
+    if (reinterpret_cast<uintptr_t>(src + q0) % 16 == 0) {
+      const long groups = (q_end - q0) / V;
+      const uint4 *pieces = reinterpret_cast<const uint4 *>(src + q0);
+      for (long i = threadIdx.x; i < groups; i += 1024) {
+        uint4 raw[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) raw[u] = i + u * 256 < groups ? pieces[i + u * 256] : uint4{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+          const T *e = reinterpret_cast<const T *>(&raw[u]);
+#pragma unroll
+          for (int j = 0; j < V; j++) v += load(e + j);
+        }
+      }
+      q0 += groups * V;
+    }
+  }
+  for (long q = q0 + threadIdx.x; q < q_end; q += 256) v += load(src + q);
   __shared__ A part[4];
   for (int d = kWave / 2; d > 0; d >>= 1) v += __shfl_down(v, d, kWave);
   if (threadIdx.x % kWave == 0) part[threadIdx.x / kWave] = v;

@@ -164,11 +164,16 @@ __global__ __launch_bounds__(256) void dcn_absmax_kernel(const T *__restrict__ p
   };
   const long head = min(n, static_cast<long>((16 - reinterpret_cast<size_t>(p) % 16) % 16 / sizeof(T)));
   const long groups = (n - head) / V, tid = blockIdx.x * 256L + threadIdx.x;
-  for (long i = tid; i < groups; i += gridDim.x * 256L) {
-    union { u32x4 u; T e[V]; } piece;
-    piece.u = *reinterpret_cast<const u32x4 *>(p + head + i * V);
+  // four independent loads per lane and step
+  for (long i = blockIdx.x * 1024L + threadIdx.x; i < groups; i += gridDim.x * 1024L) {
+    union { u32x4 u; T e[V]; } piece[4];
 #pragma unroll
-    for (int j = 0; j < V; j++) take(piece.e[j]);
+    for (int u = 0; u < 4; u++)
+      piece[u].u = i + u * 256 < groups ? *reinterpret_cast<const u32x4 *>(p + head + (i + u * 256) * V) : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+#pragma unroll
+      for (int j = 0; j < V; j++) take(piece[u].e[j]);
   }
   if (tid < head) take(p[tid]);
   const long tail = head + groups * V;
