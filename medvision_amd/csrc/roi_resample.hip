@@ -1371,6 +1371,7 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
   __syncthreads();
   const long plane = static_cast<long>(p.D) * p.H * p.W, ovol = static_cast<long>(p.od) * p.oh * p.ow;
   const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  int turn = 0;
   for (unsigned slot = 0; slot < kPlanSlots; slot++) {
     const unsigned item = blockIdx.x + slot * gridDim.x;
     if (item >= work) break;
@@ -1403,10 +1404,13 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
     }
 #pragma unroll
     for (int d = 32; d >= 1; d >>= 1) bits = max(bits, static_cast<unsigned>(__shfl_xor(static_cast<int>(bits), d)));
-    if (lane == 0) bound_part[slot & 1][wave] = bits;
+    // two buffers taken in turn: between two uses of one lies the barrier of the use in between
+    // (items that were skipped above pass no barrier and take no turn)
+    if (lane == 0) bound_part[turn][wave] = bits;
     __syncthreads();
 #pragma unroll
-    for (int w = 0; w < kWaves; w++) bits = max(bits, bound_part[slot & 1][w]);
+    for (int w = 0; w < kWaves; w++) bits = max(bits, bound_part[turn][w]);
+    turn ^= 1;
     bits = __builtin_amdgcn_readfirstlane(bits);
     if (bits == 0) continue;                                  // nothing to add
     const bool in_lds = bits < 0x7f800000u && mode != 2;      // finite terms, box within the tile
