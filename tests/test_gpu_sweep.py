@@ -127,7 +127,8 @@ def test_pooled_many_rois_sweep(ops, oracle):
 
 
 def test_rotated_backward_sweep(ops, oracle):
-    """Backward of resampling-sized rotated rois (the gather over input voxels): volumes and images,
+    """Backward of resampling-sized rotated rois (tiles of the source boxes; fp64 tensors and narrow
+    outputs: the gather over input voxels): volumes and images,
     orders 0 and 1, several rois per image, mirrored rois, rotations up to 180 degrees.  Among the
     seeds are cases in which a sample lies within 1e-5 of the edge of [-1, size], where it turns
     void, or of a nearest-neighbour tie: decided in fp32, each of them misses the tolerance."""
@@ -159,6 +160,55 @@ def test_rotated_backward_sweep(ops, oracle):
         want = oracle.roi_align_backward(gy, rois, vol.shape, 1.0, 1, True, order, True)
         what = f"seed {seed}: {ndim}-D {tuple(vol.shape)} -> {out}, {n} rois, order {order}, {dtype}"
         assert rel_err(x.grad, want) <= BWD_TOL[dtype], what
+
+
+def test_resampling_backward_mixed_sweep(ops, oracle):
+    """Backward of resampling-sized outputs through tiles of the source boxes: plain and rotated rois,
+    1 - 3 channels, up to four rois that share images, spatial scales, reductions whose boxes exceed
+    the tile, enlargements with many terms per voxel, bf16.  Order 0: cells whose sample sits within
+    1e-9 voxel of a tie or of the void's edge carry no gradient (the rounding of the coordinate
+    arithmetic decides them)."""
+    for seed in range(5000, 5060):
+        rnd = random.Random(seed)
+        g = torch.Generator().manual_seed(seed)
+        ndim = rnd.choice([3, 3, 2])
+        dtype = rnd.choice([torch.float32, torch.float16, torch.bfloat16])
+        rotated = rnd.random() < 0.6
+        hi = 56 if ndim == 3 else 160
+        size = [rnd.randint(5, hi) for _ in range(ndim)]           # D, H, W
+        batch, channels = rnd.randint(1, 2), rnd.choice([1, 1, 2, 3])
+        out = [max(16 if i == ndim - 1 else 4, int(s * rnd.choice([0.4, 0.7, 1.0, 1.0, 1.5]))) for i, s in enumerate(size)]
+        while math.prod(out) < 4096:
+            out = [o + 4 for o in out]
+        xyz = torch.tensor(size[::-1], dtype=torch.float32)
+        n = rnd.randint(1, 4)
+        idx = torch.tensor([rnd.randint(0, batch - 1) for _ in range(n)], dtype=torch.float32)[:, None]
+        ctr = xyz / 2 + (torch.rand(n, ndim, generator=g) * 2 - 1) * xyz * rnd.choice([0.05, 0.2, 0.6])
+        ext = xyz * (0.3 + torch.rand(n, ndim, generator=g) * rnd.choice([0.5, 1.2, 3.0]))
+        if rotated:
+            if rnd.random() < 0.1:
+                ext[0, 0] = -ext[0, 0]
+            ang = (torch.rand(n, 3 if ndim == 3 else 1, generator=g) * 2 - 1) * math.radians(rnd.choice([0, 5, 30, 90, 180]))
+            rois = torch.cat([idx, ctr, ext, ang], 1)
+        else:
+            rois = torch.cat([idx, ctr - ext / 2, ctr + ext / 2], 1)
+        order = rnd.choice([1, 1, 0])
+        scale = rnd.choice([1.0, 1.0, 0.5])
+        rois[:, 1:1 + 2 * ndim] /= scale
+        shape = (batch, channels, *size)
+        gy = torch.randn(n, channels, *out, generator=g).to(dtype)
+        if order == 0:
+            margin = oracle.roi_decision_margin(shape, rois, tuple(out), scale, 1, True, rotated)
+            gy = gy * (margin > NEAREST_EPS[torch.float32])[:, None].to(dtype)
+        x = torch.zeros(shape, dtype=dtype, device=DEV, requires_grad=True)
+        mod = (ops.RoIAlignRotated if rotated else ops.RoIAlign)(tuple(out), scale, 1)
+        mod(x, rois.to(DEV), order=order).backward(gy.to(DEV))
+        want = oracle.roi_align_backward(gy, rois, shape, scale, 1, True, order, rotated)
+        what = f"seed {seed}: {ndim}-D {shape} -> {out}, {n} rois, rotated {rotated}, order {order}, scale {scale}, {dtype}"
+        if float(want.abs().max()) > 0:
+            assert rel_err(x.grad, want) <= BWD_TOL[dtype], what
+        else:
+            assert float(x.grad.abs().max()) == 0, what
 
 
 def test_affine_and_warp_sweep(ops, oracle):
