@@ -96,7 +96,7 @@ constexpr int kDenseSrc = 32;   // source voxels per axis of the dense weight ma
 // gather / scatter paths.  One barrier.
 template <typename RT, int CELLS>
 __device__ inline PoolPlan pool_setup(PoolShared &sh, const RT *roi, const RoiProblem &p, size_t elem_bytes,
-                                      float (*wd)[kDenseSrc][CELLS]) {
+                                      float (*wd)[kDenseSrc][CELLS], bool slabs = false) {
   const int nd = p.ndim;
   const int cells[3] = {p.ow, p.oh, p.od};
   const int size[3] = {p.W, p.H, p.D};
@@ -191,7 +191,7 @@ __device__ inline PoolPlan pool_setup(PoolShared &sh, const RT *roi, const RoiPr
     const long nz = sh.ax[2].box_hi - sh.ax[2].box_lo + 1, ny = sh.ax[1].box_hi - sh.ax[1].box_lo + 1;
     const long per_channel = vol * static_cast<long>(elem_bytes) + (nz * ny * p.ow + nz * p.oh * p.ow) * 4 + 16;
     const long chunk = kPoolLdsBytes / per_channel;
-    if (chunk < 1) plan.staged = 0;
+    if (chunk < 1 && !slabs) plan.staged = 0;   // (a caller that works in slabs of box planes sizes them itself)
     plan.chunk = static_cast<int>(min(chunk, 64L));
   }
   return plan;
@@ -941,7 +941,7 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
   const int c_begin = blockIdx.y * channels_per_block, c_end = min(c_begin + channels_per_block, p.C);
   // intermediates are fp32 here, so size the chunk with 4-byte box elements
   __shared__ __attribute__((aligned(16))) float wd[3][kDenseSrc][CELLS];
-  const PoolPlan plan = pool_setup<RT, CELLS>(sh, rois + static_cast<long>(n) * roi_columns(p.ndim, 0), p, sizeof(float), wd);
+  PoolPlan plan = pool_setup<RT, CELLS>(sh, rois + static_cast<long>(n) * roi_columns(p.ndim, 0), p, sizeof(float), wd, true);
   if (plan.staged < 0) return;
   const int cells = p.od * p.oh * p.ow;
   const long plane = static_cast<long>(p.D) * p.H * p.W;
@@ -954,6 +954,23 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
   bool wide = false;
   if (plan.staged == 1)
     for (int a = 0; a < 3; a++) wide = wide || sh.ax[a].box_hi - sh.ax[a].box_lo + 1 > kPoolEntries + 2;
+  const bool dense = plan.staged == 1 && dense_applies<CELLS>(sh, p);
+  // Channels per pass and box planes per pass.  A box too large for a pass of enough channels (an atomic
+  // request should carry a sector's worth of them, a planar row of gradients a few) is worked through
+  // in slabs of planes: the transposed contractions of different planes do not depend on each other.
+  int zs = 0;
+  if (plan.staged == 1 && !wide) {
+    const long bx = sh.ax[0].box_hi - sh.ax[0].box_lo + 1, by = sh.ax[1].box_hi - sh.ax[1].box_lo + 1;
+    zs = sh.ax[2].box_hi - sh.ax[2].box_lo + 1;
+    const bool box = !(CL && dense);                       // the slab of the box itself is staged
+    const long per_plane = (box ? by * bx * 4 : 0L) + (by * p.ow + static_cast<long>(p.oh) * p.ow) * 4;
+    const int want = min(CL ? 16 : 4, c_end - c_begin);
+    if (plan.chunk < want) {
+      zs = static_cast<int>(min(max((kPoolLdsBytes / want - 16) / per_plane, 1L), static_cast<long>(zs)));
+      plan.chunk = static_cast<int>(min(kPoolLdsBytes / (zs * per_plane + 16), 64L));
+      if (plan.chunk < 1) plan.staged = 0;
+    }
+  }
   if (plan.staged == 0 || wide) {  // per-output scatter
     const int total = (c_end - c_begin) * cells;
     const int gz = p.ndim == 3 ? sh.g.grid[2] : 1, gy = sh.g.grid[1], gx = sh.g.grid[0];
@@ -979,13 +996,12 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
   }
   const AxisTaps &tx = sh.ax[0], &ty = sh.ax[1], &tz = sh.ax[2];
   const int nx = tx.box_hi - tx.box_lo + 1, ny = ty.box_hi - ty.box_lo + 1, nz = tz.box_hi - tz.box_lo + 1;
-  const int vol = nx * ny * nz;
   const int ohw = p.oh * p.ow;
   const int gx = tx.grid, gy = ty.grid, gz = tz.grid;
-  const float inv_vol = 1.f / vol, inv_nxy = 1.f / (nx * ny), inv_nx = 1.f / nx, inv_ow = 1.f / p.ow,
-              inv_ohw = 1.f / ohw, inv_nzohw = 1.f / (nz * ohw), inv_nyow = 1.f / (ny * p.ow),
+  const float inv_nxy = 1.f / (nx * ny), inv_nx = 1.f / nx, inv_ow = 1.f / p.ow,
+              inv_ohw = 1.f / ohw, inv_nyow = 1.f / (ny * p.ow),
               inv_gx = 1.f / gx, inv_gy = 1.f / gy, inv_gz = 1.f / gz;
-  if (dense_applies<CELLS>(sh, p)) {   // (the set-up has built the matrices)
+  if (dense) {   // (the set-up has built the matrices)
     if constexpr (CL && CELLS == 8 && std::is_same<T, __half>::value && std::is_same<G, float>::value) {
       // matrix-core form: 32-bit offsets into the image's accumulation buffer and into this roi's
       // gradient; its 16-byte loads may reach 14 bytes past a row of cells, so the roi whose rows end
@@ -1002,9 +1018,13 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
     const float inv_ow = 1.f / p.ow;
     for (int cb = c_begin; cb < c_end; cb += plan.chunk) {
       const int cs = min(plan.chunk, c_end - cb);
-      float *t2 = reinterpret_cast<float *>(lds);      // [cs][nz][oh][ow]
-      float *t1 = t2 + cs * nz * ohw;                  // [cs][nz][ny][ow]; CL: [nz][ny][cs][ow]
-      float *gbox = t1 + cs * nz * ny * p.ow;          // [cs][nz][ny][nx] (planar accumulation only)
+      for (int z0 = 0; z0 < nz; z0 += zs) {   // slabs of box planes
+      const int nzs = min(zs, nz - z0);
+      const int vol_s = nx * ny * nzs;
+      const float inv_vol_s = 1.f / vol_s;
+      float *t2 = reinterpret_cast<float *>(lds);      // [cs][nzs][oh][ow]
+      float *t1 = t2 + cs * nzs * ohw;                  // [cs][nzs][ny][ow]; CL: [nzs][ny][cs][ow]
+      float *gbox = t1 + cs * nzs * ny * p.ow;          // [cs][nzs][ny][nx] (planar accumulation only)
       const T *go = src + static_cast<long>(cb - c_begin) * cells;
       const float inv_cs = 1.f / cs;
       // z: thread = (c, ph, pw); its grad_output values stay in registers
@@ -1013,18 +1033,18 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
         float g[CELLS];
 #pragma unroll
         for (int k = 0; k < CELLS; k++) g[k] = k < p.od ? load(go + c * cells + k * ohw + hw) : 0.f;
-        for (int z = 0; z < nz; z++) {
+        for (int z = 0; z < nzs; z++) {
           float acc = 0.f;
 #pragma unroll
-          for (int k = 0; k < CELLS; k++) acc += wd[2][z][k] * g[k];
-          t2[(c * nz + z) * ohw + hw] = acc;
+          for (int k = 0; k < CELLS; k++) acc += wd[2][z0 + z][k] * g[k];
+          t2[(c * nzs + z) * ohw + hw] = acc;
         }
       }
       __syncthreads();
       // y: thread = (c, z, pw)
-      for (int i = threadIdx.x; i < cs * nz * p.ow; i += kPoolThreads) {
+      for (int i = threadIdx.x; i < cs * nzs * p.ow; i += kPoolThreads) {
         const int cz = fdiv(i, inv_ow), pw = i - cz * p.ow;
-        const int c = fdiv(cz, 1.f / nz), z = cz - c * nz;
+        const int c = fdiv(cz, 1.f / nzs), z = cz - c * nzs;
         float g[CELLS];
 #pragma unroll
         for (int k = 0; k < CELLS; k++) g[k] = k < p.oh ? t2[cz * ohw + k * p.ow + pw] : 0.f;
@@ -1037,9 +1057,9 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
       }
       __syncthreads();
       // x: thread = one (c, z, y) line
-      const long first = (static_cast<long>(tz.box_lo) * p.H + ty.box_lo) * p.W + tx.box_lo;
+      const long first = (static_cast<long>(tz.box_lo + z0) * p.H + ty.box_lo) * p.W + tx.box_lo;
       if (CL) {   // channel fastest across the lanes: a wavefront adds runs of cs contiguous floats
-        for (int i = threadIdx.x; i < cs * nz * ny; i += kPoolThreads) {
+        for (int i = threadIdx.x; i < cs * nzs * ny; i += kPoolThreads) {
           const int zy = fdiv(i, inv_cs), c = i - zy * cs, z = fdiv(zy, 1.f / ny), y = zy - z * ny;
           float g[CELLS];
 #pragma unroll
@@ -1053,7 +1073,7 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
           }
         }
       } else {    // through LDS, so that the lanes of a wavefront add runs of nx contiguous elements
-        for (int i = threadIdx.x; i < cs * nz * ny; i += kPoolThreads) {
+        for (int i = threadIdx.x; i < cs * nzs * ny; i += kPoolThreads) {
           float g[CELLS];
 #pragma unroll
           for (int k = 0; k < CELLS; k++) g[k] = k < p.ow ? t1[i * p.ow + k] : 0.f;
@@ -1066,41 +1086,47 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
         }
         __syncthreads();
         G *corner = dst + static_cast<long>(cb - c_begin) * plane + first;
-        for (int i = threadIdx.x; i < cs * vol; i += kPoolThreads) {
+        for (int i = threadIdx.x; i < cs * vol_s; i += kPoolThreads) {
           const float v = gbox[i];
           if (v == 0.f) continue;
-          const int c = fdiv(i, inv_vol), r0 = i - c * vol, z = fdiv(r0, inv_nxy), r1 = r0 - z * nx * ny;
+          const int c = fdiv(i, inv_vol_s), r0 = i - c * vol_s, z = fdiv(r0, inv_nxy), r1 = r0 - z * nx * ny;
           const int y = fdiv(r1, inv_nx), x = r1 - y * nx;
           atomic_add(corner + c * plane + (static_cast<long>(z) * p.H + y) * p.W + x, static_cast<G>(v));
         }
       }
       __syncthreads();
     }
+    }
     return;
   }
   pool_first(sh);
   for (int cb = c_begin; cb < c_end; cb += plan.chunk) {
     const int cs = min(plan.chunk, c_end - cb);
+    for (int z0 = 0; z0 < nz; z0 += zs) {   // slabs of box planes
+    const int nzs = min(zs, nz - z0);
+    const int vol_s = nx * ny * nzs;
+    const float inv_vol_s = 1.f / vol_s, inv_nzsohw = 1.f / (nzs * ohw);
     float *gbox = reinterpret_cast<float *>(lds);    // [cs][nz][ny][nx]
-    float *t1 = gbox + cs * vol;                     // [cs][nz][ny][ow]
-    float *t2 = t1 + cs * nz * ny * p.ow;            // [cs][nz][oh][ow]
+    float *t1 = gbox + cs * vol_s;                     // [cs][nzs][ny][ow]
+    float *t2 = t1 + cs * nzs * ny * p.ow;            // [cs][nzs][oh][ow]
     const T *go = src + static_cast<long>(cb - c_begin) * cells;
     // Transposed contractions as gathers.  Entries are sorted by coordinate, so the entries whose
     // low tap is source index i form the range [first[i], first[i+1]) and those whose high tap is
     // i are the low-tap entries of i - 1 (a clamped edge entry has lo == hi and zero high weight).
-    for (int i = threadIdx.x; i < cs * nz * ohw; i += kPoolThreads) {  // transpose of "contract z"
-      const int c = fdiv(i, inv_nzohw), r0 = i - c * nz * ohw, z = fdiv(r0, inv_ohw), hw = r0 - z * ohw;
+    for (int i = threadIdx.x; i < cs * nzs * ohw; i += kPoolThreads) {  // transpose of "contract z"
+      const int c = fdiv(i, inv_nzsohw), r0 = i - c * nzs * ohw, z = fdiv(r0, inv_ohw), hw = r0 - z * ohw;
       const T *r = go + c * cells + hw;
-      const int mid = tz.first[z], e0 = z > 0 ? tz.first[z - 1] : mid, e1 = tz.first[z + 1];
+      const int zq = z0 + z;   // plane of the box
+      const int mid = tz.first[zq], e0 = zq > 0 ? tz.first[zq - 1] : mid, e1 = tz.first[zq + 1];
       float acc = 0.f;
       for (int e = e0; e < e1; e++) {
-        const float w = e < mid ? (tz.hi[e] == z ? tz.whi[e] : 0.f) : tz.wlo[e];
+        const float w = e < mid ? (tz.hi[e] == zq ? tz.whi[e] : 0.f) : tz.wlo[e];
         acc += w * load(r + fdiv(e, inv_gz) * ohw);
       }
       t2[i] = acc;
     }
     __syncthreads();
-    for (int i = threadIdx.x; i < cs * nz * ny * p.ow; i += kPoolThreads) {  // transpose of "contract y"
+    for (int i = threadIdx.x; i < cs * nzs * ny * p.ow; i += kPoolThreads) {  // transpose of "contract y"
       const int cz = fdiv(i, inv_nyow), r0 = i - cz * ny * p.ow, y = fdiv(r0, inv_ow), pw = r0 - y * p.ow;
       const float *r = t2 + cz * ohw + pw;
       const int mid = ty.first[y], e0 = y > 0 ? ty.first[y - 1] : mid, e1 = ty.first[y + 1];
@@ -1112,7 +1138,7 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
       t1[i] = acc;
     }
     __syncthreads();
-    for (int i = threadIdx.x; i < cs * vol; i += kPoolThreads) {  // transpose of "contract x"
+    for (int i = threadIdx.x; i < cs * vol_s; i += kPoolThreads) {  // transpose of "contract x"
       const int row = fdiv(i, inv_nx), x = i - row * nx;
       const float *r = t1 + row * p.ow;
       const int mid = tx.first[x], e0 = x > 0 ? tx.first[x - 1] : mid, e1 = tx.first[x + 1];
@@ -1124,17 +1150,18 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
       gbox[i] = acc;
     }
     __syncthreads();
-    const long first = (static_cast<long>(tz.box_lo) * p.H + ty.box_lo) * p.W + tx.box_lo;
+    const long first = (static_cast<long>(tz.box_lo + z0) * p.H + ty.box_lo) * p.W + tx.box_lo;
     G *corner = dst + static_cast<long>(cb - c_begin) * plane + first;
-    for (int i = threadIdx.x; i < cs * vol; i += kPoolThreads) {
+    for (int i = threadIdx.x; i < cs * vol_s; i += kPoolThreads) {
       const float v = gbox[i];
       if (v == 0.f) continue;
-      const int c = fdiv(i, inv_vol), r0 = i - c * vol, z = fdiv(r0, inv_nxy), r1 = r0 - z * nx * ny;
+      const int c = fdiv(i, inv_vol_s), r0 = i - c * vol_s, z = fdiv(r0, inv_nxy), r1 = r0 - z * nx * ny;
       const int y = fdiv(r1, inv_nx), x = r1 - y * nx;
       const long voxel = (static_cast<long>(z) * p.H + y) * p.W + x;
       atomic_add(CL ? dst_cl + (first + voxel) * p.C + (cb - c_begin) + c : corner + c * plane + voxel, static_cast<G>(v));
     }
     __syncthreads();
+    }
   }
 }
 

@@ -224,6 +224,39 @@ def test_backward_tiles_with_zero_and_infinite_gradients(ops, oracle):
                      BWD_TOL[dtype], "finite part")
 
 
+@pytest.mark.parametrize("shape,out,sr,extent,dtype", [
+    ((2, 20, 30, 40, 48), (7, 7, 7), 2, (18, 30), torch.float16),     # dense matrices, channels-last sums
+    ((2, 20, 30, 40, 48), (7, 7, 7), 2, (18, 30), torch.float32),     # dense matrices, planar sums
+    ((2, 20, 30, 40, 48), (7, 7, 7), 2, (18, 30), torch.bfloat16),
+    ((1, 8, 40, 44, 60), (6, 5, 7), 3, (28, 44), torch.float16),      # boxes beyond the dense matrices: tap tables
+    ((1, 8, 40, 44, 60), (6, 5, 7), 3, (28, 44), torch.float32),
+    ((2, 6, 24, 36, 40), (12, 10, 14), 1, (20, 34), torch.float16),   # more than 8 cells per axis
+    ((2, 70, 90, 120), (14, 14), 2, (40, 64), torch.float32),         # images
+])
+def test_pooled_kernels_with_large_boxes(ops, oracle, shape, out, sr, extent, dtype):
+    """Boxes of 18 - 64 voxels per axis with many channels: the pooled backward works through such a
+    box in slabs of planes, so that a pass still takes enough channels for whole-sector atomics (it
+    used to fall back to one atomic per corner of every sample: 240 ms instead of 19 ms for 1000 rois
+    of 24^3 voxels x 256 channels)."""
+    g = wl.gen(77)
+    nd = len(shape) - 2
+    size = torch.tensor(shape[2:][::-1], dtype=torch.float32)
+    n = 6
+    e = torch.minimum(extent[0] + torch.rand(n, nd, generator=g) * (extent[1] - extent[0]), size + 4)
+    lo = torch.rand(n, nd, generator=g) * (size - e + 6) - 3
+    rois = torch.cat([torch.randint(0, shape[0], (n, 1), generator=g).float(), lo, lo + e], 1)
+    for order in (1, 0):
+        feat = torch.randn(shape, generator=g).to(dtype)
+        x = feat.to(DEV).requires_grad_(True)
+        y = ops.RoIAlign(out, 1.0, sr)(x, rois.to(DEV), order=order)
+        eff = 1 if order == 0 else sr
+        assert_close(y, oracle.roi_align_forward(feat, rois, out, 1.0, eff, True, order, False), FWD_TOL[dtype], "forward")
+        gy = torch.randn(y.shape, generator=g).to(dtype)
+        y.backward(gy.to(DEV))
+        assert_close(x.grad, oracle.roi_align_backward(gy, rois, shape, 1.0, eff, True, order, False), BWD_TOL[dtype],
+                     "backward")
+
+
 def test_config3_resize_and_crops(ops, oracle):
     """Benchmark configuration 3 at reduced size: CT-like fp16 volume, resize then rotated 3-D crops."""
     g = wl.gen(2)
