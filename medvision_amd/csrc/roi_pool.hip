@@ -31,6 +31,7 @@ namespace mv {
 
 constexpr int kPoolThreads = 256;
 constexpr int kPoolEntries = 64;               // tap-table entries per axis (cells * grid)
+constexpr int kPoolFirst = 256;                // widest box (voxels per axis) of the transposed contractions
 constexpr int kPoolLdsBytes = 40 * 1024;       // staged data + intermediates of one channel chunk
 
 // i / d for 0 <= i < 2^21 and 0 < d < 2^12, with inv = 1.0f / d (exact: the product is at least
@@ -40,7 +41,7 @@ __device__ __forceinline__ int fdiv(int i, float inv) { return static_cast<int>(
 struct AxisTaps {
   int lo[kPoolEntries], hi[kPoolEntries];      // box-relative tap indices
   float wlo[kPoolEntries], whi[kPoolEntries];  // weights (0 for void samples), include 1 / grid
-  int first[kPoolEntries + 4];                 // first[i] = first entry whose low tap is >= i (box-relative)
+  int first[kPoolFirst + 4];                   // first[i] = first entry whose low tap is >= i (box-relative)
   int box_lo, box_hi;                          // inclusive source range covered by valid taps
   int entries, grid;
 };
@@ -199,8 +200,8 @@ __device__ inline PoolPlan pool_setup(PoolShared &sh, const RT *roi, const RoiPr
 
 // The entry ranges per source index (`first`) of a staged roi; all threads, ends with a barrier.
 __device__ inline void pool_first(PoolShared &sh) {
-  for (int e = threadIdx.x; e < 3 * (kPoolEntries + 4); e += kPoolThreads) {
-    const int k = e / (kPoolEntries + 4), j = e % (kPoolEntries + 4);
+  for (int e = threadIdx.x; e < 3 * (kPoolFirst + 4); e += kPoolThreads) {
+    const int k = e / (kPoolFirst + 4), j = e % (kPoolFirst + 4);
     AxisTaps &t = sh.ax[k];
     if (j > t.box_hi - t.box_lo + 1) continue;
     int f = 0;
@@ -949,11 +950,11 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
   G *dst = gin + (static_cast<long>(sh.g.batch) * p.C + c_begin) * plane;
   G *dst_cl = gin + static_cast<long>(sh.g.batch) * plane * p.C + c_begin;   // CL: voxel v, channel c at v * C + c
   // The transposed contractions below look entries up by source index through `first`, which
-  // holds kPoolEntries + 4 indices: a box wider than that on any axis (few cells spread over many
+  // holds kPoolFirst + 4 indices: a box wider than that on any axis (few cells spread over many
   // voxels) takes the per-output scatter, like a box that does not fit LDS.
   bool wide = false;
   if (plan.staged == 1)
-    for (int a = 0; a < 3; a++) wide = wide || sh.ax[a].box_hi - sh.ax[a].box_lo + 1 > kPoolEntries + 2;
+    for (int a = 0; a < 3; a++) wide = wide || sh.ax[a].box_hi - sh.ax[a].box_lo + 1 > kPoolFirst + 2;
   const bool dense = plan.staged == 1 && dense_applies<CELLS>(sh, p);
   // Channels per pass and box planes per pass.  A box too large for a pass of enough channels (an atomic
   // request should carry a sector's worth of them, a planar row of gradients a few) is worked through
@@ -962,7 +963,7 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
   if (plan.staged == 1 && !wide) {
     const long bx = sh.ax[0].box_hi - sh.ax[0].box_lo + 1, by = sh.ax[1].box_hi - sh.ax[1].box_lo + 1;
     zs = sh.ax[2].box_hi - sh.ax[2].box_lo + 1;
-    const bool box = !(CL && dense);                       // the slab of the box itself is staged
+    const bool box = !CL;                                  // planar sums: the slab of the box itself is staged
     const long per_plane = (box ? by * bx * 4 : 0L) + (by * p.ow + static_cast<long>(p.oh) * p.ow) * 4;
     const int want = min(CL ? 16 : 4, c_end - c_begin);
     if (plan.chunk < want) {
@@ -1106,8 +1107,8 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
     const int nzs = min(zs, nz - z0);
     const int vol_s = nx * ny * nzs;
     const float inv_vol_s = 1.f / vol_s, inv_nzsohw = 1.f / (nzs * ohw);
-    float *gbox = reinterpret_cast<float *>(lds);    // [cs][nz][ny][nx]
-    float *t1 = gbox + cs * vol_s;                     // [cs][nzs][ny][ow]
+    float *gbox = reinterpret_cast<float *>(lds);    // [cs][nzs][ny][nx] (planar accumulation only)
+    float *t1 = gbox + (CL ? 0 : cs * vol_s);          // [cs][nzs][ny][ow]
     float *t2 = t1 + cs * nzs * ny * p.ow;            // [cs][nzs][oh][ow]
     const T *go = src + static_cast<long>(cb - c_begin) * cells;
     // Transposed contractions as gathers.  Entries are sorted by coordinate, so the entries whose
@@ -1138,27 +1139,47 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
       t1[i] = acc;
     }
     __syncthreads();
-    for (int i = threadIdx.x; i < cs * vol_s; i += kPoolThreads) {  // transpose of "contract x"
-      const int row = fdiv(i, inv_nx), x = i - row * nx;
-      const float *r = t1 + row * p.ow;
-      const int mid = tx.first[x], e0 = x > 0 ? tx.first[x - 1] : mid, e1 = tx.first[x + 1];
-      float acc = 0.f;
-      for (int e = e0; e < e1; e++) {
-        const float w = e < mid ? (tx.hi[e] == x ? tx.whi[e] : 0.f) : tx.wlo[e];
-        acc += w * r[fdiv(e, inv_gx)];
-      }
-      gbox[i] = acc;
-    }
-    __syncthreads();
     const long first = (static_cast<long>(tz.box_lo + z0) * p.H + ty.box_lo) * p.W + tx.box_lo;
-    G *corner = dst + static_cast<long>(cb - c_begin) * plane + first;
-    for (int i = threadIdx.x; i < cs * vol_s; i += kPoolThreads) {
-      const float v = gbox[i];
-      if (v == 0.f) continue;
-      const int c = fdiv(i, inv_vol_s), r0 = i - c * vol_s, z = fdiv(r0, inv_nxy), r1 = r0 - z * nx * ny;
-      const int y = fdiv(r1, inv_nx), x = r1 - y * nx;
-      const long voxel = (static_cast<long>(z) * p.H + y) * p.W + x;
-      atomic_add(CL ? dst_cl + (first + voxel) * p.C + (cb - c_begin) + c : corner + c * plane + voxel, static_cast<G>(v));
+    if (CL) {
+      // transpose of "contract x" straight into the buffer: a thread takes one (z, y) row of one channel,
+      // channels fastest across the lanes, so that a wavefront's atomics are runs of cs contiguous floats
+      const float inv_cs = 1.f / cs;
+      for (int i = threadIdx.x; i < cs * nzs * ny; i += kPoolThreads) {
+        const int zy = fdiv(i, inv_cs), c = i - zy * cs;
+        const int z = fdiv(zy, 1.f / ny), y = zy - z * ny;
+        const float *r = t1 + (c * nzs * ny + zy) * p.ow;
+        G *row = dst_cl + (first + (static_cast<long>(z) * p.H + y) * p.W) * p.C + (cb - c_begin) + c;
+        for (int x = 0; x < nx; x++) {
+          const int mid = tx.first[x], e0 = x > 0 ? tx.first[x - 1] : mid, e1 = tx.first[x + 1];
+          float acc = 0.f;
+          for (int e = e0; e < e1; e++) {
+            const float w = e < mid ? (tx.hi[e] == x ? tx.whi[e] : 0.f) : tx.wlo[e];
+            acc += w * r[fdiv(e, inv_gx)];
+          }
+          if (acc != 0.f) atomic_add(row + static_cast<long>(x) * p.C, static_cast<G>(acc));
+        }
+      }
+    } else {
+      for (int i = threadIdx.x; i < cs * vol_s; i += kPoolThreads) {  // transpose of "contract x"
+        const int row = fdiv(i, inv_nx), x = i - row * nx;
+        const float *r = t1 + row * p.ow;
+        const int mid = tx.first[x], e0 = x > 0 ? tx.first[x - 1] : mid, e1 = tx.first[x + 1];
+        float acc = 0.f;
+        for (int e = e0; e < e1; e++) {
+          const float w = e < mid ? (tx.hi[e] == x ? tx.whi[e] : 0.f) : tx.wlo[e];
+          acc += w * r[fdiv(e, inv_gx)];
+        }
+        gbox[i] = acc;
+      }
+      __syncthreads();
+      G *corner = dst + static_cast<long>(cb - c_begin) * plane + first;
+      for (int i = threadIdx.x; i < cs * vol_s; i += kPoolThreads) {
+        const float v = gbox[i];
+        if (v == 0.f) continue;
+        const int c = fdiv(i, inv_vol_s), r0 = i - c * vol_s, z = fdiv(r0, inv_nxy), r1 = r0 - z * nx * ny;
+        const int y = fdiv(r1, inv_nx), x = r1 - y * nx;
+        atomic_add(corner + c * plane + (static_cast<long>(z) * p.H + y) * p.W + x, static_cast<G>(v));
+      }
     }
     __syncthreads();
     }

@@ -628,15 +628,18 @@ def test_every_output_element_is_written(ops, oracle, order, out):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 def test_pooled_boxes_wider_than_the_tap_tables(ops, oracle, dtype):
     """Few cells spread over many voxels: boxes of 70-100 voxels on one axis with 7 cells of 2
-    samples.  The separable backward kernel indexes its tap ranges by source voxel and has to hand
-    such boxes to the per-output scatter."""
+    samples, and of more than 258.  The separable backward kernel indexes its tap ranges by source
+    voxel through a table of 260 entries and has to hand wider boxes to the per-output scatter (with
+    68 entries and no such hand-over it once ran off the table and never finished)."""
     g = wl.gen(77)
     img = torch.randn(2, 6, 110, 120, generator=g).to(dtype)
     rois2 = torch.tensor([[0, 3.0, 5.0, 98.0, 60.0], [1, 10.5, 2.0, 105.0, 101.0], [0, 40.0, 40.0, 47.0, 46.0],
                           [1, -20.0, 30.0, 70.0, 90.0]])
     vol = torch.randn(1, 5, 9, 10, 96, generator=g).to(dtype)
     rois3 = torch.tensor([[0, 2.0, 1.0, 1.0, 88.0, 7.5, 7.0], [0, 10.0, 2.0, 0.5, 93.0, 8.0, 8.5]])
-    for feat, rois, out in ((img, rois2, (7, 7)), (vol, rois3, (7, 7, 7))):
+    wide = torch.randn(1, 3, 12, 300, generator=g).to(dtype)
+    rois4 = torch.tensor([[0, 4.0, 1.0, 292.5, 10.0], [0, 20.0, 2.0, 278.0, 11.0], [0, -5.0, 0.0, 310.0, 12.0]])
+    for feat, rois, out in ((img, rois2, (7, 7)), (vol, rois3, (7, 7, 7)), (wide, rois4, (7, 7))):
         mod = ops.RoIAlign(out, 1.0, 2)
         x = feat.to(DEV).requires_grad_(True)
         y = mod(x, rois.to(DEV))
