@@ -30,7 +30,7 @@
 namespace mv {
 
 constexpr int kPoolThreads = 256;
-constexpr int kPoolEntries = 64;               // tap-table entries per axis (cells * grid)
+constexpr int kPoolEntries = 128;              // tap-table entries per axis (cells * grid)
 constexpr int kPoolFirst = 256;                // widest box (voxels per axis) of the transposed contractions
 constexpr int kPoolLdsBytes = 40 * 1024;       // staged data + intermediates of one channel chunk
 
@@ -39,9 +39,9 @@ constexpr int kPoolLdsBytes = 40 * 1024;       // staged data + intermediates of
 __device__ __forceinline__ int fdiv(int i, float inv) { return static_cast<int>((static_cast<float>(i) + 0.5f) * inv); }
 
 struct AxisTaps {
-  int lo[kPoolEntries], hi[kPoolEntries];      // box-relative tap indices
+  short lo[kPoolEntries], hi[kPoolEntries];    // box-relative tap indices (16 bits: the tables decide how many workgroups share a compute unit's LDS)
   float wlo[kPoolEntries], whi[kPoolEntries];  // weights (0 for void samples), include 1 / grid
-  int first[kPoolFirst + 4];                   // first[i] = first entry whose low tap is >= i (box-relative)
+  short first[kPoolFirst + 4];                 // first[i] = first entry whose low tap is >= i (box-relative)
   int box_lo, box_hi;                          // inclusive source range covered by valid taps
   int entries, grid;
 };
@@ -85,7 +85,7 @@ struct PoolPlan {
   int chunk;       // channels per LDS pass
 };
 
-static_assert(kPoolEntries == kWave, "one wavefront builds the tap table of one axis, one entry per lane");
+static_assert(kPoolEntries % kWave == 0, "one wavefront builds the tap table of one axis, kPoolEntries / kWave entries per lane");
 constexpr int kDenseSrc = 32;   // source voxels per axis of the dense weight matrices (see below)
 
 // Builds geometry and tap tables for roi `roi`; all threads must call it (contains barriers).
@@ -142,32 +142,53 @@ __device__ inline PoolPlan pool_setup(PoolShared &sh, const RT *roi, const RoiPr
     const double ex = a == 0 ? ext[0] : (a == 1 ? ext[1] : ext[2]);
     const double bin = a < nd ? ex / static_cast<double>(nc) : 0.0;
     const double sub_step = bin / static_cast<double>(gr > 0 ? gr : 1);
-    const bool on = i < en;
-    const int cell = on ? i / gr : 0, sub = on ? i % gr : 0;
-    // (local_coord's expression)
-    const double v = a < nd ? st + cell * bin + static_cast<double>(static_cast<float>(sub) + .5f) * sub_step : 0.0;
-    int lo = 0, hi = 0;
-    float frac = 0.f;
-    const bool ok = clamped_tap<float>(v, sz, lo, hi, frac, p.order) && on;
+    // entries e = i, i + 64, ...: the coordinates grow with the entry (plain boxes have positive
+    // extents), so the box runs from the low tap of the first valid sample to the high tap of the last
+    constexpr int kPer = kPoolEntries / kWave;
     const float inv = 1.f / static_cast<float>(gr);
-    // the coordinates grow with the lane (plain boxes have positive extents): the box runs from the low
-    // tap of the first valid sample to the high tap of the last one
-    const unsigned long long valid = __ballot(ok);
-    const int box_lo = valid ? __builtin_amdgcn_readlane(lo, __builtin_ctzll(valid)) : (1 << 30);
-    const int box_hi = valid ? __builtin_amdgcn_readlane(hi, 63 - __builtin_clzll(valid)) : -1;
-    const int top = box_hi - box_lo;
-    const float wlo = ok ? (1.f - frac) * inv : 0.f, whi = ok ? frac * inv : 0.f;
-    // void samples keep weight 0; they are parked at the matching end so that `lo` stays monotonic
-    const int rlo = ok ? lo - box_lo : (v > 0.0 ? top : 0), rhi = ok ? hi - box_lo : (v > 0.0 ? top : 0);
-    if (on) {
-      t.lo[i] = rlo; t.hi[i] = rhi;
-      t.wlo[i] = wlo; t.whi[i] = whi;
+    int lo_[kPer], hi_[kPer], cell_[kPer], sub_[kPer];
+    float frac_[kPer];
+    bool ok_[kPer], up_[kPer];
+    int box_lo = 1 << 30, box_hi = -1;
+#pragma unroll
+    for (int h = 0; h < kPer; h++) {
+      const int e = i + h * kWave;
+      const bool on = e < en;
+      cell_[h] = on ? e / gr : 0; sub_[h] = on ? e % gr : 0;
+      // (local_coord's expression)
+      const double v = a < nd ? st + cell_[h] * bin + static_cast<double>(static_cast<float>(sub_[h]) + .5f) * sub_step : 0.0;
+      lo_[h] = 0; hi_[h] = 0; frac_[h] = 0.f;
+      ok_[h] = clamped_tap<float>(v, sz, lo_[h], hi_[h], frac_[h], p.order) && on;
+      up_[h] = v > 0.0;
+      const unsigned long long valid = __ballot(ok_[h]);
+      if (valid) {
+        if (box_hi < 0) box_lo = __builtin_amdgcn_readlane(lo_[h], __builtin_ctzll(valid));
+        box_hi = __builtin_amdgcn_readlane(hi_[h], 63 - __builtin_clzll(valid));
+      }
     }
+    const int top = box_hi - box_lo;
+    const bool on = i < en;   // (first entry of the lane: what the dense matrices below are built from)
+    const bool ok = ok_[0];
+    const int cell = cell_[0], sub = sub_[0];
+    const float wlo = ok ? (1.f - frac_[0]) * inv : 0.f, whi = ok ? frac_[0] * inv : 0.f;
+    const int rlo = ok ? lo_[0] - box_lo : (up_[0] ? top : 0), rhi = ok ? hi_[0] - box_lo : (up_[0] ? top : 0);
+#pragma unroll
+    for (int h = 0; h < kPer; h++) {
+      const int e = i + h * kWave;
+      if (e < en) {
+        // void samples keep weight 0; they are parked at the matching end so that `lo` stays monotonic
+        t.lo[e] = ok_[h] ? lo_[h] - box_lo : (up_[h] ? top : 0);
+        t.hi[e] = ok_[h] ? hi_[h] - box_lo : (up_[h] ? top : 0);
+        t.wlo[e] = ok_[h] ? (1.f - frac_[h]) * inv : 0.f;
+        t.whi[e] = ok_[h] ? frac_[h] * inv : 0.f;
+      }
+    }
+    (void)on;
     if (i == 0) {
       t.box_lo = box_lo; t.box_hi = box_hi;
       t.entries = en; t.grid = gr;
     }
-    if (wd != nullptr && box_hi >= 0 && top < kDenseSrc && nc <= CELLS) {
+    if (wd != nullptr && box_hi >= 0 && top < kDenseSrc && nc <= CELLS && en <= kWave) {
       float *m = &wd[a][0][0];
       for (int k = i; k < kDenseSrc * CELLS / 4; k += kWave) reinterpret_cast<float4 *>(m)[k] = float4{0.f, 0.f, 0.f, 0.f};
       for (int sidx = 0; sidx < gr; sidx++) {
@@ -220,7 +241,7 @@ __device__ inline void pool_first(PoolShared &sh) {
 template <int CELLS>
 __device__ __forceinline__ bool dense_applies(const PoolShared &sh, const RoiProblem &p) {
   for (int a = 0; a < 3; a++)
-    if (sh.ax[a].box_hi - sh.ax[a].box_lo + 1 > kDenseSrc) return false;
+    if (sh.ax[a].box_hi - sh.ax[a].box_lo + 1 > kDenseSrc || sh.ax[a].entries > kWave) return false;
   return p.ow <= CELLS && p.oh <= CELLS && p.od <= CELLS;
 }
 
