@@ -650,6 +650,27 @@ def test_pooled_boxes_wider_than_the_tap_tables(ops, oracle, dtype):
         assert_close(x.grad, want, BWD_TOL[dtype], "backward")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_pooled_kernels_with_adaptive_grids_on_large_boxes(ops, oracle, dtype):
+    """sampling_ratio 0 (the reference's default): ceil(box / cells) samples per bin, so boxes of 64 -
+    126 voxels need 65 - 128 tap entries per axis (two per lane of the wavefront that builds a table);
+    beyond that the per-sample kernels take over."""
+    g = wl.gen(79)
+    img = torch.randn(2, 5, 140, 150, generator=g).to(dtype)
+    rois2 = torch.tensor([[0, 3.0, 5.0, 98.0, 80.0], [1, 10.5, 2.0, 135.0, 121.0], [0, 40.0, 40.0, 47.0, 46.0],
+                          [1, -20.0, 30.0, 70.0, 150.0], [0, 1.0, 1.0, 149.0, 139.0]])
+    vol = torch.randn(1, 3, 9, 10, 120, generator=g).to(dtype)
+    rois3 = torch.tensor([[0, 2.0, 1.0, 1.0, 88.0, 7.5, 7.0], [0, 10.0, 2.0, 0.5, 118.0, 8.0, 8.5]])
+    for feat, rois, out in ((img, rois2, (7, 7)), (img, rois2, (14, 14)), (vol, rois3, (7, 7, 7))):
+        x = feat.to(DEV).requires_grad_(True)
+        y = ops.RoIAlign(out, 1.0, 0)(x, rois.to(DEV))
+        assert_close(y, oracle.roi_align_forward(feat, rois, out, 1.0, 0, True, 1, False), FWD_TOL[dtype], "forward")
+        gy = torch.randn(y.shape, generator=g).to(dtype)
+        y.backward(gy.to(DEV))
+        want = oracle.roi_align_backward(gy, rois, feat.shape, 1.0, 0, True, 1, False)
+        assert_close(x.grad, want, BWD_TOL[dtype], "backward")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 def test_pooled_heads_with_9_to_16_cells(ops, oracle, dtype):
     """14 x 14 mask heads and a 10 x 12 x 14 volume head: the pooled kernels' 16-cell instance
