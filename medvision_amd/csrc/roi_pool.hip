@@ -625,8 +625,8 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
   const unsigned n = order ? order[blockIdx.x] : blockIdx.x;   // (largest rois first, see pool_order_rois)
   const int c_begin = blockIdx.y * channels_per_block, c_end = min(c_begin + channels_per_block, p.C);
   __shared__ __attribute__((aligned(16))) float wd[3][kDenseSrc][CELLS];
-  const PoolPlan plan = pool_setup<RT, CELLS>(sh, rois + static_cast<long>(n) * roi_columns(p.ndim, 0), p, sizeof(T),
-                                              CELLS == 8 ? wd : nullptr);
+  PoolPlan plan = pool_setup<RT, CELLS>(sh, rois + static_cast<long>(n) * roi_columns(p.ndim, 0), p, sizeof(T),
+                                        CELLS == 8 ? wd : nullptr, true);
   const int cells = p.od * p.oh * p.ow;
   const long plane = static_cast<long>(p.D) * p.H * p.W;
   T *dst = out + (static_cast<long>(n) * p.C + c_begin) * cells;
@@ -636,6 +636,83 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
     return;
   }
   const T *src = feat + (static_cast<long>(sh.g.batch) * p.C + c_begin) * plane;
+  if (plan.staged == 1 && plan.chunk < 1) {
+    // A box too large for LDS with all its planes is worked through in slabs of planes: x and y are
+    // contracted per slab, and the z contraction adds each slab's share to sums kept per output.
+    const AxisTaps &tx = sh.ax[0], &ty = sh.ax[1], &tz = sh.ax[2];
+    const int nx = tx.box_hi - tx.box_lo + 1, ny = ty.box_hi - ty.box_lo + 1, nz = tz.box_hi - tz.box_lo + 1;
+    const int gx = tx.grid, gy = ty.grid, gz = tz.grid, ohw = p.oh * p.ow;
+    const long box_plane = (static_cast<long>(ny) * nx * sizeof(T) + 15) / 16 * 16;
+    const long per_plane = box_plane + (static_cast<long>(ny) * p.ow + ohw) * 4;
+    int cs = 0, zs = 0;
+    // (measured on 24^3 - 32^3 boxes: the per-output gather below costs about as much as the slabs with
+    // 27 samples per output, a third with 8, twice with 64)
+    for (int c = gx * gy * gz > 27 ? 8 : 0; c >= 1 && cs == 0; c >>= 1) {
+      const int cn = min(c, c_end - c_begin);
+      const long planes = (kPoolLdsBytes - 32 - cn * static_cast<long>(cells) * 4) / (cn * per_plane);
+      if (planes >= 1) { cs = cn; zs = static_cast<int>(min(planes, static_cast<long>(nz))); }
+    }
+    if (cs == 0) {
+      plan.staged = 0;   // not even one plane: per-output gather below
+    } else {
+      float *sums = reinterpret_cast<float *>(lds);                                   // [cs][cells]
+      T *box = reinterpret_cast<T *>(sums + cs * cells);                              // [cs][zs][ny][nx]
+      float *t1 = reinterpret_cast<float *>(lds + ((static_cast<size_t>(cs) * cells * 4 + static_cast<size_t>(cs) * zs * box_plane + 15) / 16) * 16);  // [cs][zs][ny][ow]
+      float *t2 = t1 + cs * zs * ny * p.ow;                                           // [cs][zs][oh][ow]
+      for (int cb = c_begin; cb < c_end; cb += cs) {
+        const int cn = min(cs, c_end - cb);
+        for (int i = threadIdx.x; i < cn * cells; i += kPoolThreads) sums[i] = 0.f;
+        for (int z0 = 0; z0 < nz; z0 += zs) {
+          const int nzs = min(zs, nz - z0), rows = nzs * ny, vol_s = rows * nx;
+          __syncthreads();   // the slab before has been read
+          const T *corner = src + static_cast<long>(cb - c_begin) * plane +
+                            (static_cast<long>(tz.box_lo + z0) * p.H + ty.box_lo) * p.W + tx.box_lo;
+          for (int i = threadIdx.x; i < cn * vol_s; i += kPoolThreads) {
+            const int c = i / vol_s, r0 = i - c * vol_s, row = r0 / nx, x = r0 - row * nx, z = row / ny, y = row - z * ny;
+            box[i] = corner[c * plane + (static_cast<long>(z) * p.H + y) * p.W + x];
+          }
+          __syncthreads();
+          for (int i = threadIdx.x; i < cn * rows * p.ow; i += kPoolThreads) {        // contract x
+            const int row = i / p.ow, pw = i - row * p.ow;                             // row = (c, z, y)
+            const T *r = box + row * nx;
+            float acc = 0.f;
+            for (int k = 0; k < gx; k++) {
+              const int e = pw * gx + k;
+              acc += tx.wlo[e] * load(r + tx.lo[e]) + tx.whi[e] * load(r + tx.hi[e]);
+            }
+            t1[i] = acc;
+          }
+          __syncthreads();
+          for (int i = threadIdx.x; i < cn * nzs * ohw; i += kPoolThreads) {          // contract y
+            const int cz = i / ohw, hw = i - cz * ohw, ph = hw / p.ow, pw = hw - ph * p.ow;   // cz = (c, z)
+            const float *r = t1 + cz * ny * p.ow + pw;
+            float acc = 0.f;
+            for (int k = 0; k < gy; k++) {
+              const int e = ph * gy + k;
+              acc += ty.wlo[e] * r[ty.lo[e] * p.ow] + ty.whi[e] * r[ty.hi[e] * p.ow];
+            }
+            t2[i] = acc;
+          }
+          __syncthreads();
+          for (int i = threadIdx.x; i < cn * cells; i += kPoolThreads) {              // the slab's share of z
+            const int c = i / cells, r0 = i - c * cells, pd = r0 / ohw, hw = r0 - pd * ohw;
+            const float *r = t2 + c * nzs * ohw + hw;
+            float acc = 0.f;
+            for (int k = 0; k < gz; k++) {
+              const int e = pd * gz + k;
+              const unsigned zl = static_cast<unsigned>(tz.lo[e] - z0), zh = static_cast<unsigned>(tz.hi[e] - z0);
+              if (zl < static_cast<unsigned>(nzs)) acc += tz.wlo[e] * r[zl * ohw];
+              if (zh < static_cast<unsigned>(nzs)) acc += tz.whi[e] * r[zh * ohw];
+            }
+            sums[i] += acc;   // (element i belongs to this thread in every slab)
+          }
+        }
+        T *o = dst + static_cast<long>(cb - c_begin) * cells;
+        for (int i = threadIdx.x; i < cn * cells; i += kPoolThreads) o[i] = store_cast<T>(sums[i]);
+      }
+      return;
+    }
+  }
   if (plan.staged == 0) {  // per-output gather
     const int gz = p.ndim == 3 ? sh.g.grid[2] : 1, gy = sh.g.grid[1], gx = sh.g.grid[0];
     for (int i = threadIdx.x; i < total; i += kPoolThreads) {

@@ -661,7 +661,12 @@ def test_pooled_kernels_with_adaptive_grids_on_large_boxes(ops, oracle, dtype):
                           [1, -20.0, 30.0, 70.0, 150.0], [0, 1.0, 1.0, 149.0, 139.0]])
     vol = torch.randn(1, 3, 9, 10, 120, generator=g).to(dtype)
     rois3 = torch.tensor([[0, 2.0, 1.0, 1.0, 88.0, 7.5, 7.0], [0, 10.0, 2.0, 0.5, 118.0, 8.0, 8.5]])
-    for feat, rois, out in ((img, rois2, (7, 7)), (img, rois2, (14, 14)), (vol, rois3, (7, 7, 7))):
+    # boxes of 26 - 36 voxels on every axis: too large for LDS with all their planes, four or five samples
+    # per bin and axis (the forward pass then goes through slabs of planes as well)
+    cube = torch.randn(2, 10, 30, 34, 40, generator=g).to(dtype)
+    rois5 = torch.tensor([[0, 2.0, 1.0, 1.0, 30.0, 29.5, 27.0], [1, 5.0, 2.0, 0.5, 39.0, 33.0, 29.5],
+                          [1, -4.0, -3.0, -2.0, 32.0, 31.0, 28.0]])
+    for feat, rois, out in ((img, rois2, (7, 7)), (img, rois2, (14, 14)), (vol, rois3, (7, 7, 7)), (cube, rois5, (7, 7, 7))):
         x = feat.to(DEV).requires_grad_(True)
         y = ops.RoIAlign(out, 1.0, 0)(x, rois.to(DEV))
         assert_close(y, oracle.roi_align_forward(feat, rois, out, 1.0, 0, True, 1, False), FWD_TOL[dtype], "forward")
