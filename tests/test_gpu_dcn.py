@@ -466,3 +466,33 @@ def test_general_deform_vs_oracle(ops, oracle, dtype, order):
     with pytest.raises(RuntimeError, match="order 2 is not supported"):
         _C.deform_3d(x, torch.zeros(4, 4, 1, 1, 1, device=DEV), torch.zeros(4, device=DEV),
                      torch.zeros(2, 3, 4, 4, 4, device=DEV), 1, 1, 1, 1, 1, 1, 0, 0, 0, 1, 1, 1, 1, 1, 64, 2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("cin,cout,dg,modulated", [(24, 40, 2, True), (16, 16, 1, True), (48, 24, 1, False)])
+def test_channel_counts_padded_for_the_matrix_cores(ops, oracle, dtype, cin, cout, dg, modulated):
+    """Layers of one weight group whose channel counts are no multiples of 32 run the matrix-core
+    kernels on zero-padded copies (the shim pads and slices): all outputs and gradients as without."""
+    from medvision_amd.ops.deform_conv_3d import deform_conv
+    from medvision_amd.ops.modulated_deform_conv_3d import modulated_deform_conv
+    from medvision_amd import _C, _lib
+    g = wl.gen(500 + cin + cout)
+    x, off, mask, w, b = wl.dcn_inputs(g, 2, cin, cout, (5, 8, 9), 3, dg, 1, dtype, 1, 1, 1, modulated)
+    shape = _lib.DcnShape(2, cin, 5, 8, 9, cout, 3, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, dg)
+    assert _C._dcn_pad_plan(x.to(DEV), w.to(DEV), shape) is not None
+    xs, offs, ms, ws, bs = [None if t is None else t.to(DEV).requires_grad_(True) for t in (x, off, mask, w, b)]
+    if modulated:
+        y = modulated_deform_conv(xs, offs, ms, ws, bs, 1, 1, 1, 1, dg)
+    else:
+        y = deform_conv(xs, offs, ws, bs, 1, 1, 1, 1, dg, 64)
+    assert_close(y, oracle.dcn3d_forward(x, off, mask, w, b, 1, 1, 1, 1, dg), FWD_TOL[dtype], "forward")
+    gy = torch.randn(y.shape, generator=g).to(dtype)
+    y.backward(gy.to(DEV))
+    gx, goff, gm, gw, gb = oracle.dcn3d_backward(x, off, mask, w, gy, True, 1, 1, 1, 1, dg)
+    tol = BWD_TOL[dtype]
+    assert_close(xs.grad, gx, tol, "grad input")
+    assert_close(offs.grad, goff, tol, "grad offset")
+    assert_close(ws.grad, gw, tol, "grad weight")
+    assert_close(bs.grad, gb, tol, "grad bias")
+    if modulated:
+        assert_close(ms.grad, gm, tol, "grad mask")
