@@ -1273,6 +1273,10 @@ int roi_forward_tiled(const void *input, const void *rois, void *output, int dty
     return roi_forward_tiled_grid(input, rois, output, dtype, p, workspace, need, s);
   const long vox = static_cast<long>(p.od) * p.oh * p.ow;
   if (p.sampling_ratio != 1 || vox < 4096 || p.ow < 16 || p.R == 0) return -1;
+  // Images: a tile's z extent is 1, so a lane's column is a single pixel and the per-item work of the
+  // persistent kernel buys nothing; the one-thread-per-output kernel is about twice as fast for them
+  // (measured: [8,3,512,512] rotated 0.070 against 0.159 ms, order 3 0.109 against 0.185 ms).
+  if (p.ndim == 2) return -1;
   if (vox * 4 >= (1L << 31)) return -1;   // 32-bit byte offsets inside one output volume
   const float *r = static_cast<const float *>(rois);
   if (p.order == 3) {
