@@ -317,7 +317,8 @@ def test_tiled_resampler_shapes(ops, oracle, dtype, channels, rois_n, size, out,
 
 
 def test_tiled_resampler_2d(ops, oracle):
-    """2-D images through the same kernel (depth-1 volumes)."""
+    """2-D images of resampling size (they take the one-thread-per-output kernel: a tile of depth 1
+    gives a lane a single pixel per item)."""
     g = wl.gen(37)
     img = torch.randn(2, 3, 96, 120, generator=g).half()
     rois = torch.tensor([[0, 60.3, 47.1, 130.0, 90.0, 0.4], [1, 50.0, 40.0, 70.0, 110.0, -0.7],
