@@ -6,7 +6,8 @@ A "step" is one RoIAlignRotated3D forward over one batch of benchmark configurat
 HBM.  ``value`` is output Gvox/s.  Inputs/outputs rotate over ``--copies`` buffer sets (default 16,
 ~540 MB) so that consecutive steps are not served from the 256 MB Infinity Cache.  The same JSON
 line carries the roofline of that kernel, the DCNv2-3D forward figure of config 4 (``dcn``) and the
-CPU baseline (the fp64 oracle timed on the host cores, bounded sample).
+CPU baseline (the reference's torch-function RoIAlign on the same shape, timed on the host cores on a
+bounded sample; the fp64 oracle beside it).
 """
 import argparse
 import json
@@ -28,9 +29,25 @@ MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense fp16/bf16
 # returns 64 bytes per clock and compute unit at the ~1.97 GHz these kernels run at.
 VALU_NS_PER_WAVE_INSTR = 2.03
 SIMDS, CUS, L1_BYTES_PER_CLK, SHADER_GHZ = 1024, 256, 64, 1.97
+DCN_L1_MISS_REQUESTS = 3.16e7   # config 4 forward, 64-byte requests from the L1s to the L2s per launch
+L2_GATHER_TBPS = 15.0           # measured line rate of the L2s for scattered 16-byte gathers
 
 
-def _events_ms(fn, steps, warmup):
+PREHEAT_S = 0.3   # untimed launches of the same step before every timed leg, whatever --steps / --warmup say
+_preheat_log = []
+
+
+def _events_ms(fn, steps, warmup, preheat_s=None):
+    # A short run reads the clocks of an idle GPU (20 steps of 25 us end long before the power
+    # management has settled): keep the GPU busy with the same launches for a fixed time first.
+    preheat_s = PREHEAT_S if preheat_s is None else preheat_s
+    t_heat, n = time.perf_counter(), 0
+    while preheat_s > 0 and time.perf_counter() - t_heat < preheat_s:
+        for i in range(50):
+            fn(n + i)
+        n += 50
+        torch.cuda.synchronize()
+    _preheat_log.append(round((time.perf_counter() - t_heat) * 1e3, 1))
     for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()
@@ -61,13 +78,14 @@ def bench_affine(args, dtype=torch.float16):
         _C.roi_align_rotated_3d_forward(vols[j], rois[j], outs[j], S, S, S, 1.0, 1, True, 1)
 
     ms, wall_ms = _events_ms(step, args.steps, args.warmup)
+    preheat_ms = _preheat_log[-1]
     # practical ceiling of a launch of this size: a plain device copy of the same bytes
     copy_ms, _ = _events_ms(lambda i: outs[i % args.copies].copy_(vols[(i + 1) % args.copies]), args.steps, args.warmup)
     vox = B * S ** 3
     esz = torch.finfo(dtype).bits // 8
     alg_bytes = 2 * vox * esz            # read every input voxel once + write every output voxel
     return {"ms": ms, "wall_ms": wall_ms, "gvox_s": vox / ms / 1e6, "gbps": alg_bytes / ms / 1e6,
-            "alg_bytes": alg_bytes, "vox": vox, "copy_ms": copy_ms}
+            "alg_bytes": alg_bytes, "vox": vox, "copy_ms": copy_ms, "preheat_ms": preheat_ms}
 
 
 def bench_dcn(args, dtype=torch.float16):
@@ -88,6 +106,11 @@ def bench_dcn(args, dtype=torch.float16):
     taps_pos = 2 * 48 ** 3 * 27
     blend_floor_us = taps_pos * 8 * 32 / 64 / SIMDS * VALU_NS_PER_WAVE_INSTR / 1e3
     gather_floor_us = taps_pos * 8 * 64 / (CUS * L1_BYTES_PER_CLK * SHADER_GHZ * 1e9) * 1e6
+    # second floor, the L2 side of the gather: the kernel's corner reads miss the vector L1 for
+    # DCN_L1_MISS_REQUESTS 64-byte requests per launch (TCP_TCC_READ_REQ_sum of the rocprofv3 counter
+    # profile of this layer), and a microbenchmark of 16-byte gathers at random places of an 8 MB buffer
+    # puts the L2s' line rate at L2_GATHER_TBPS over the chip
+    l2_floor_us = DCN_L1_MISS_REQUESTS * 64 / (L2_GATHER_TBPS * 1e12) * 1e6
 
     # training step (forward + all five gradients), reported beside the forward figure
     ins = [t.clone().requires_grad_(True) for t in (x, off, mask, w, b)]
@@ -100,7 +123,7 @@ def bench_dcn(args, dtype=torch.float16):
 
     train_ms, _ = _events_ms(train_step, max(3, min(args.steps // 4, 50)), 3)
     return {"ms": ms, "wall_ms": wall_ms, "tflops": flops / ms / 1e9, "flops": flops, "train_ms": train_ms,
-            "blend_floor_us": blend_floor_us, "gather_floor_us": gather_floor_us}
+            "blend_floor_us": blend_floor_us, "gather_floor_us": gather_floor_us, "l2_floor_us": l2_floor_us}
 
 
 def bench_other_configs(args):
@@ -126,7 +149,10 @@ def bench_other_configs(args):
         gy = torch.randn(4, 1, 128, 128, 128, generator=g).to(dt).to(dev)
         gi = torch.zeros_like(vol)
         ms, _ = _events_ms(lambda i: _C.roi_align_rotated_3d_backward(gy, r, gi, 128, 128, 128, 1.0, 1, True, 1), 50, 5)
-        res["config2_backward_" + name] = {"ms": round(ms, 4)}
+        # algorithmic bytes: grad_output read once, grad_input read and written once (it accumulates)
+        nbytes = 3 * vol.numel() * vol.element_size()
+        res["config2_backward_" + name] = {"ms": round(ms, 4), "gbps": round(nbytes / ms / 1e6, 1),
+                                           "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
     g = wl.gen(2)
     vol = wl.ct_like(g, (2, 1, 256, 512, 512)).to(dev)
     full = torch.tensor([[b, 256, 256, 128, 512, 512, 256, 0, 0, 0] for b in range(2)], dtype=torch.float32).to(dev)
@@ -216,36 +242,63 @@ def bench_next_rows(args):
 
 
 def cpu_baseline(args):
-    """fp64 oracle (C, OpenMP) on the benchmark's config-2 inputs (all 4 samples), repeated until
-    about 12 s of wall time have been spent; the median pass is reported."""
+    """The reference's own CPU path on the shape of config 2: its torch-function RoIAlign (affine_grid +
+    grid_sample per roi, fp32, medvision/ops/pytorch_ops/roi_align.py:22-105, restated in
+    oracle/torchfun_roi_align.py) on a [4,1,128^3] volume with one full-volume box per sample and a
+    128^3 output -- the class takes plain boxes only, so the rois carry no rotation; the work per output
+    voxel (one trilinear sample) is that of the GPU step.  Passes are repeated for about half of
+    --cpu-seconds with all torch threads, then a few passes with one thread; medians are reported.
+    The fp64 C oracle (the checker of the parity tests) is timed on the rotated rois of the GPU step
+    for the other half and reported under ``oracle_port``."""
     import oracle
     import workloads as wl
+    from oracle.torchfun_roi_align import torchfun_roi_align
+    g = wl.gen(1)
+    B, S = 4, 128
+    vol = torch.randn(B, 1, S, S, S, generator=g)
+    boxes = torch.tensor([[b, 0, 0, 0, S, S, S] for b in range(B)], dtype=torch.float32)
+    threads = torch.get_num_threads()
+
+    def passes(budget_s, fn, at_most=200):
+        fn()   # warm-up
+        times, t_start = [], time.perf_counter()
+        while time.perf_counter() - t_start < budget_s and len(times) < at_most:
+            t0 = time.perf_counter()
+            fn()
+            times.append(time.perf_counter() - t0)
+        return sorted(times)[len(times) // 2], len(times)
+
+    t_all, n_all = passes(args.cpu_seconds * 0.35, lambda: torchfun_roi_align(vol, boxes, (S, S, S), 1.0))
+    torch.set_num_threads(1)
+    t_one, n_one = passes(args.cpu_seconds * 0.15, lambda: torchfun_roi_align(vol[:1], boxes[:1], (S, S, S), 1.0), 5)
+    torch.set_num_threads(threads)
+
+    # the fp64 oracle on the benchmark's own (rotated) rois
     oracle.build()
     cores = min(os.cpu_count() or 1, 16)
     oracle.set_threads(cores)
-    g = wl.gen(1)
-    B, S = 4, 128
-    vol = torch.randn(B, 1, S, S, S, generator=g).half()
+    half = vol.half()
     rois = wl.affine_rois(g, B, (S, S, S))
-    oracle.roi_align_forward(vol, rois, (S, S, S), 1.0, 1, True, 1, True)   # warm-up
-    times, t_start = [], time.perf_counter()
-    while time.perf_counter() - t_start < args.cpu_seconds and len(times) < 200:
-        t0 = time.perf_counter()
-        oracle.roi_align_forward(vol, rois, (S, S, S), 1.0, 1, True, 1, True)
-        times.append(time.perf_counter() - t0)
-    t = sorted(times)[len(times) // 2]
-    # one thread, one of the four samples (a quarter of the work), one pass
+    t_orc, n_orc = passes(args.cpu_seconds * 0.4, lambda: oracle.roi_align_forward(half, rois, (S, S, S), 1.0, 1, True, 1, True))
     oracle.set_threads(1)
     t0 = time.perf_counter()
-    oracle.roi_align_forward(vol[:1], rois[:1], (S, S, S), 1.0, 1, True, 1, True)
-    t1 = time.perf_counter() - t0
+    oracle.roi_align_forward(half[:1], rois[:1], (S, S, S), 1.0, 1, True, 1, True)
+    t_orc1 = time.perf_counter() - t0
     oracle.set_threads(cores)
-    return {"value": round(B * S ** 3 / t / 1e9, 4), "unit": "Gvox/s", "cores": cores, "kind": "port",
-            "one_thread": {"value": round(S ** 3 / t1 / 1e9, 4), "unit": "Gvox/s",
-                           "sample": f"one sample of config 2, one pass ({t1 * 1e3:.0f} ms)"},
+    return {"value": round(B * S ** 3 / t_all / 1e9, 4), "unit": "Gvox/s", "cores": threads, "kind": "port",
+            "reference_path": "medvision/ops/pytorch_ops/roi_align.py:22-105 (torch-function RoIAlign: affine_grid + "
+                              "grid_sample per roi, fp32), restated line by line in oracle/torchfun_roi_align.py",
+            "sample": f"config 2 shape: fp32 [4,1,128^3] -> 128^3, one full-volume box per sample (the class has no "
+                      f"rotation), median of {n_all} passes after 1 warm-up ({t_all * 1e3:.0f} ms per pass), "
+                      f"{threads} torch threads",
+            "one_thread": {"value": round(S ** 3 / t_one / 1e9, 4), "unit": "Gvox/s", "cores": 1,
+                           "sample": f"one sample of the same, median of {n_one} passes ({t_one * 1e3:.0f} ms per pass)"},
             "cpu_count": os.cpu_count(),
-            "sample": f"config 2 (fp16 [4,1,128^3] -> 128^3) through the fp64 C oracle, OpenMP x{cores}, "
-                      f"median of {len(times)} passes after 1 warm-up ({t * 1e3:.0f} ms per pass)"}
+            "oracle_port": {"value": round(B * S ** 3 / t_orc / 1e9, 4), "unit": "Gvox/s", "cores": cores,
+                            "sample": f"config 2 with its rotated rois (fp16 [4,1,128^3] -> 128^3) through the fp64 C "
+                                      f"oracle, OpenMP x{cores}, median of {n_orc} passes ({t_orc * 1e3:.0f} ms per pass)",
+                            "one_thread": {"value": round(S ** 3 / t_orc1 / 1e9, 4), "unit": "Gvox/s",
+                                           "sample": f"one sample, one pass ({t_orc1 * 1e3:.0f} ms)"}}}
 
 
 def cpu_reference_paths(args):
@@ -362,7 +415,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(a16["gbps"], 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(a16["gbps"] / HBM_PEAK_GBPS, 4), "traffic": None,
                      "kernel": "roi_resample_kernel", "algorithmic_bytes_per_launch": a16["alg_bytes"],
-                     "avg_launch_us": round(a16["ms"] * 1e3, 3),
+                     "avg_launch_us": round(a16["ms"] * 1e3, 3), "preheat_ms": a16["preheat_ms"],
                      "copy_ceiling_us": round(a16["copy_ms"] * 1e3, 3),
                      "frac_of_copy_ceiling": round(a16["copy_ms"] / a16["ms"], 4)},
         "fp32": {"gvox_s": round(a32["gvox_s"], 3), "gbps": round(a32["gbps"], 1),
@@ -381,7 +434,9 @@ def main():
                                     "traffic": None, "flops_per_launch": d["flops"],
                                     "vector_blend_floor_us": round(d["blend_floor_us"], 1),
                                     "l1_gather_floor_us": round(d["gather_floor_us"], 1),
-                                    "frac_of_gather_floor": round(d["gather_floor_us"] / (d["ms"] * 1e3), 4)}}
+                                    "frac_of_gather_floor": round(d["gather_floor_us"] / (d["ms"] * 1e3), 4),
+                                    "l2_gather_floor_us": round(d["l2_floor_us"], 1),
+                                    "frac_of_l2_floor": round(d["l2_floor_us"] / (d["ms"] * 1e3), 4)}}
     if not args.no_configs:
         line["other_configs"] = bench_other_configs(args)
     if not args.no_next:

@@ -44,7 +44,8 @@ int mv_version(void);
 int mv_roi_align_2d_forward(const void *input, const void *rois, void *output, int dtype,
                             int batch, int channels, int height, int width, int num_rois,
                             int out_h, int out_w, float spatial_scale, int sampling_ratio,
-                            int order, void *workspace, void *stream);
+                            int order, void *workspace,
+                            size_t workspace_bytes, void *stream);
 int mv_roi_align_2d_backward(const void *grad_output, const void *rois, void *grad_input,
                              int dtype, int batch, int channels, int height, int width,
                              int num_rois, int out_h, int out_w, float spatial_scale,
@@ -52,7 +53,8 @@ int mv_roi_align_2d_backward(const void *grad_output, const void *rois, void *gr
 int mv_roi_align_3d_forward(const void *input, const void *rois, void *output, int dtype,
                             int batch, int channels, int depth, int height, int width,
                             int num_rois, int out_d, int out_h, int out_w, float spatial_scale,
-                            int sampling_ratio, int order, void *workspace, void *stream);
+                            int sampling_ratio, int order, void *workspace,
+                            size_t workspace_bytes, void *stream);
 int mv_roi_align_3d_backward(const void *grad_output, const void *rois, void *grad_input,
                              int dtype, int batch, int channels, int depth, int height, int width,
                              int num_rois, int out_d, int out_h, int out_w, float spatial_scale,
@@ -66,7 +68,8 @@ int mv_roi_align_3d_backward(const void *grad_output, const void *rois, void *gr
 int mv_roi_align_rotated_2d_forward(const void *input, const void *rois, void *output, int dtype,
                                     int batch, int channels, int height, int width, int num_rois,
                                     int out_h, int out_w, float spatial_scale, int sampling_ratio,
-                                    int aligned, int order, void *workspace, void *stream);
+                                    int aligned, int order, void *workspace,
+                                    size_t workspace_bytes, void *stream);
 int mv_roi_align_rotated_2d_backward(const void *grad_output, const void *rois, void *grad_input,
                                      int dtype, int batch, int channels, int height, int width,
                                      int num_rois, int out_h, int out_w, float spatial_scale,
@@ -76,7 +79,8 @@ int mv_roi_align_rotated_3d_forward(const void *input, const void *rois, void *o
                                     int batch, int channels, int depth, int height, int width,
                                     int num_rois, int out_d, int out_h, int out_w,
                                     float spatial_scale, int sampling_ratio, int aligned,
-                                    int order, void *workspace, void *stream);
+                                    int order, void *workspace,
+                                    size_t workspace_bytes, void *stream);
 int mv_roi_align_rotated_3d_backward(const void *grad_output, const void *rois, void *grad_input,
                                      int dtype, int batch, int channels, int depth, int height,
                                      int width, int num_rois, int out_d, int out_h, int out_w,
@@ -87,17 +91,18 @@ size_t mv_roi_align_backward_workspace_bytes(int dtype, int batch, int channels,
 /* Workspace of the forward entry points (plain, rotated and affine).  0 for a sampling grid of 1
  * (the kernels keep their per-call state in LDS); for fp16 / fp32 outputs of resampling size with a
  * fixed sampling_ratio of 2..4 the bytes of the bins' samples (sampling_ratio^ndim per output
- * element), which a second pass averages.  A non-NULL `workspace` must hold what this query
- * returns for the call's arguments; NULL selects the kernels that need none.  ndim = 2 or 3
- * (out_d ignored for 2).                                                                       */
+ * element), which a second pass averages.  The forward entry points take the workspace together
+ * with its size in bytes (`workspace_bytes`) and use a path only when the workspace holds what that
+ * path needs: NULL, or a workspace that is too small, selects the kernels that need none (same
+ * results, slower), never an access beyond `workspace_bytes`.  ndim = 2 or 3 (out_d ignored for 2). */
 size_t mv_roi_align_forward_workspace_bytes(int dtype, int ndim, int channels, int num_rois,
                                             int out_d, int out_h, int out_w, int sampling_ratio);
 /* The same query with the input's shape: at least the value above, and for fp16 detection heads
  * (plain rois, outputs of up to 8 cells per axis, about as many pooled outputs as input voxels or
  * more, width a multiple of four) the size of a re-ordered copy of the features that
  * mv_roi_align_2d_forward / _3d_forward then read instead of the input (a few voxels of a box row no
- * longer cost a whole memory sector each).  A non-NULL `workspace` passed to those two entry points
- * must hold this many bytes; NULL selects the kernels that need none.  depth ignored for ndim 2.
+ * longer cost a whole memory sector each).  Those two entry points make the copy only when
+ * `workspace_bytes` is at least this value.  depth ignored for ndim 2.
  * No counterpart in the reference.                                                              */
 size_t mv_roi_align_forward_workspace_bytes_for_input(int dtype, int ndim, int batch, int channels, int depth,
                                                       int height, int width, int num_rois, int out_d,
@@ -111,11 +116,13 @@ size_t mv_roi_align_forward_workspace_bytes_for_input(int dtype, int ndim, int b
  * points above reject it, as the reference's do.                                              */
 int mv_affine_2d(const void *input, const void *rois, void *output, int dtype, int batch,
                  int channels, int height, int width, int num_rois, int out_h, int out_w,
-                 float spatial_scale, int sampling_ratio, int aligned, int order, void *workspace, void *stream);
+                 float spatial_scale, int sampling_ratio, int aligned, int order, void *workspace,
+                 size_t workspace_bytes, void *stream);
 int mv_affine_3d(const void *input, const void *rois, void *output, int dtype, int batch,
                  int channels, int depth, int height, int width, int num_rois, int out_d,
                  int out_h, int out_w, float spatial_scale, int sampling_ratio, int aligned,
-                 int order, void *workspace, void *stream);
+                 int order, void *workspace,
+                 size_t workspace_bytes, void *stream);
 
 /* ---- deformable convolution 3-D -----------------------------------------------------------
  * replaces deform_conv_3d_forward / _backward                 csrc/deform_conv_3d.h:48,87
@@ -161,7 +168,9 @@ size_t mv_dcn_column_budget(void);
  * Same arguments and results as mv_dcn3d_forward without `workspace`: the layout buffers live in a
  * fixed array of MV_DCN3D_STATIC_SCRATCH_BYTES in the library's device image (every GPU the
  * library runs on holds it until the process ends).  Calls no hipMalloc / hipFree or allocating
- * library routine; the first call on a device looks the array's address up.  Layers whose
+ * library routine; the first call on a device looks the array's address up (hipGetSymbolAddress,
+ * which may load the code object): make that call once OUTSIDE any graph capture.  Every process that
+ * loads the library holds the array on each GPU it runs kernels on.  Layers whose
  * mv_dcn3d_forward_workspace_bytes() exceeds the array are rejected with MV_INVALID_ARGUMENT.
  * All calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads)
  * race; serialise them.                                                                        */

@@ -105,7 +105,7 @@ def _roi_forward(fn_name, what, ndim, cols, input, rois, output, out_sizes, spat
         _lib.check(getattr(lib, fn_name)(
             _lib.ptr(feats), _lib.ptr(r), _lib.ptr(output), code, *dims,
             r.size(0), *out_sizes, float(spatial_scale), int(sampling_ratio), *extra,
-            _lib.ptr(ws), _lib.stream_of(feats)))
+            _lib.ptr(ws), ws_bytes, _lib.stream_of(feats)))
 
 
 def _roi_backward(fn_name, what, ndim, cols, top_grad, rois, bottom_grad, out_sizes,
@@ -525,25 +525,15 @@ def modulated_deform_conv_2d_backward(input, weight, bias, ones, offset, mask, c
 
 
 # csrc/deform_2d.h, csrc/deform_3d.h:27-65 as used by ops/cuda_fun_tools.py:94-167
-_identity_verdicts = {}   # (weight address, version, bias address, version) -> bool
-
-
 def _is_identity_warp(weight, bias, C, ndim):
     """True when ``weight`` is the C x C identity over a 1x1(x1) kernel and ``bias`` is zero.
-    Reading the verdict back blocks the host, so it is taken once per (tensor, version) and
-    remembered: a caller that reuses its weight, as the reference's own caller could, pays no
-    synchronisation per call."""
+    Checked on every call (one read-back): a tensor's address and version do not identify its
+    contents (the allocator reuses addresses, writes through ``.data`` leave the version alone), so
+    a remembered verdict could send a real 1x1x1 convolution down the warp path."""
     if tuple(weight.shape) != (C, C, *([1] * ndim)) or tuple(bias.shape) != (C,):
         return False
-    key = (weight.data_ptr(), weight._version, bias.data_ptr(), bias._version, C, weight.dtype)
-    ok = _identity_verdicts.get(key)
-    if ok is None:
-        if len(_identity_verdicts) > 64:
-            _identity_verdicts.clear()
-        eye = torch.eye(C, dtype=weight.dtype, device=weight.device)
-        ok = bool(((weight.reshape(C, C) == eye).all() & (bias == 0).all()).item())
-        _identity_verdicts[key] = ok
-    return ok
+    eye = torch.eye(C, dtype=weight.dtype, device=weight.device)
+    return bool(((weight.reshape(C, C) == eye).all() & (bias == 0).all()).item())
 
 
 def _deform(fn_name, ndim, input, weight, bias, offset, kernel, stride, pad, dil, group,

@@ -40,19 +40,19 @@ _SHAPE2_P = ctypes.POINTER(Dcn2dShape)
 SIGNATURES = {
     "mv_last_error": (ctypes.c_char_p, []),
     "mv_version": (_i, []),
-    "mv_roi_align_2d_forward": (_i, [_p, _p, _p, _i] + [_i] * 7 + [_f, _i, _i, _p, _p]),
+    "mv_roi_align_2d_forward": (_i, [_p, _p, _p, _i] + [_i] * 7 + [_f, _i, _i, _p, _sz, _p]),
     "mv_roi_align_2d_backward": (_i, [_p, _p, _p, _i] + [_i] * 7 + [_f, _i, _i, _p, _p]),
-    "mv_roi_align_3d_forward": (_i, [_p, _p, _p, _i] + [_i] * 9 + [_f, _i, _i, _p, _p]),
+    "mv_roi_align_3d_forward": (_i, [_p, _p, _p, _i] + [_i] * 9 + [_f, _i, _i, _p, _sz, _p]),
     "mv_roi_align_3d_backward": (_i, [_p, _p, _p, _i] + [_i] * 9 + [_f, _i, _i, _p, _p]),
-    "mv_roi_align_rotated_2d_forward": (_i, [_p, _p, _p, _i] + [_i] * 7 + [_f, _i, _i, _i, _p, _p]),
+    "mv_roi_align_rotated_2d_forward": (_i, [_p, _p, _p, _i] + [_i] * 7 + [_f, _i, _i, _i, _p, _sz, _p]),
     "mv_roi_align_rotated_2d_backward": (_i, [_p, _p, _p, _i] + [_i] * 7 + [_f, _i, _i, _i, _p, _p]),
-    "mv_roi_align_rotated_3d_forward": (_i, [_p, _p, _p, _i] + [_i] * 9 + [_f, _i, _i, _i, _p, _p]),
+    "mv_roi_align_rotated_3d_forward": (_i, [_p, _p, _p, _i] + [_i] * 9 + [_f, _i, _i, _i, _p, _sz, _p]),
     "mv_roi_align_rotated_3d_backward": (_i, [_p, _p, _p, _i] + [_i] * 9 + [_f, _i, _i, _i, _p, _p]),
     "mv_roi_align_backward_workspace_bytes": (_sz, [_i] * 6),
     "mv_roi_align_forward_workspace_bytes": (_sz, [_i] * 8),
     "mv_roi_align_forward_workspace_bytes_for_input": (_sz, [_i] * 12),
-    "mv_affine_2d": (_i, [_p, _p, _p, _i] + [_i] * 7 + [_f, _i, _i, _i, _p, _p]),
-    "mv_affine_3d": (_i, [_p, _p, _p, _i] + [_i] * 9 + [_f, _i, _i, _i, _p, _p]),
+    "mv_affine_2d": (_i, [_p, _p, _p, _i] + [_i] * 7 + [_f, _i, _i, _i, _p, _sz, _p]),
+    "mv_affine_3d": (_i, [_p, _p, _p, _i] + [_i] * 9 + [_f, _i, _i, _i, _p, _sz, _p]),
     "mv_dcn3d_output_dims": (_i, [_SHAPE_P, ctypes.POINTER(_i), ctypes.POINTER(_i), ctypes.POINTER(_i)]),
     "mv_dcn3d_forward_workspace_bytes": (_sz, [_SHAPE_P, _i]),
     "mv_dcn3d_backward_workspace_bytes": (_sz, [_SHAPE_P, _i]),

@@ -120,7 +120,7 @@ __global__ void add_from_f32_kernel(T *dst, const float *src, long n) {
 
 // roi_resample.hip: tiled LDS-staged forward; returns -1 when it does not apply
 int roi_forward_tiled(const void *input, const void *rois, void *output, int dtype,
-                      const RoiProblem &p, void *workspace, size_t *need, hipStream_t s);
+                      const RoiProblem &p, void *workspace, size_t capacity, size_t *need, hipStream_t s);
 
 // roi_resample.hip: backward of the same problems through LDS tiles of the source boxes; `acc` is the
 // fp32 buffer the gradient is added to; -1 when it does not apply
@@ -131,7 +131,7 @@ int roi_backward_tiled(const void *grad_output, const void *rois, float *acc, in
 // roi_pool.hip: separable LDS kernels for plain boxes with small outputs; -1 when not applicable
 size_t roi_pool_forward_workspace(int dtype, const RoiProblem &p);
 int roi_pool_forward(const void *input, const void *rois, void *output, int dtype,
-                     const RoiProblem &p, void *workspace, hipStream_t s);
+                     const RoiProblem &p, void *workspace, size_t capacity, hipStream_t s);
 int roi_pool_backward(const void *grad_output, const void *rois, void *acc, int dtype,
                       const RoiProblem &p, hipStream_t s, bool channels_last);
 bool roi_pool_applies(int dtype, const RoiProblem &p);
@@ -169,8 +169,8 @@ static int make_problem(RoiProblem &p, int ndim, int rotated, int batch, int cha
 int roi_forward(const void *input, const void *rois, void *output, int dtype, int ndim,
                 int rotated, int batch, int channels, int depth, int height, int width,
                 int num_rois, int out_d, int out_h, int out_w, float spatial_scale,
-                int sampling_ratio, int aligned, int order, void *workspace, void *stream,
-                bool cubic_ok = false) {
+                int sampling_ratio, int aligned, int order, void *workspace, size_t workspace_bytes,
+                void *stream, bool cubic_ok = false) {
   RoiProblem p;
   int st = make_problem(p, ndim, rotated, batch, channels, depth, height, width, num_rois, out_d,
                         out_h, out_w, spatial_scale, sampling_ratio, aligned, order, cubic_ok);
@@ -179,9 +179,11 @@ int roi_forward(const void *input, const void *rois, void *output, int dtype, in
   MV_REQUIRE(input && rois && output, "null pointer argument");
   hipStream_t s = static_cast<hipStream_t>(stream);
   {
-    const int tiled = roi_forward_tiled(input, rois, output, dtype, p, workspace, nullptr, s);
+    // (a workspace too small for a path selects the kernels that need none)
+    const size_t capacity = workspace ? workspace_bytes : 0;
+    const int tiled = roi_forward_tiled(input, rois, output, dtype, p, workspace, capacity, nullptr, s);
     if (tiled >= 0) return tiled;
-    const int pooled = order != 3 ? roi_pool_forward(input, rois, output, dtype, p, workspace, s) : -1;
+    const int pooled = order != 3 ? roi_pool_forward(input, rois, output, dtype, p, workspace, capacity, s) : -1;
     if (pooled >= 0) return pooled;
   }
   const dim3 grid(p.chunks * num_rois), block(kRoiThreads);
@@ -274,9 +276,10 @@ extern "C" {
 int mv_roi_align_2d_forward(const void *input, const void *rois, void *output, int dtype,
                             int batch, int channels, int height, int width, int num_rois,
                             int out_h, int out_w, float spatial_scale, int sampling_ratio,
-                            int order, void *workspace, void *stream) {
+                            int order, void *workspace,
+                            size_t workspace_bytes, void *stream) {
   return roi_forward(input, rois, output, dtype, 2, 0, batch, channels, 1, height, width, num_rois,
-                     1, out_h, out_w, spatial_scale, sampling_ratio, 1, order, workspace, stream);
+                     1, out_h, out_w, spatial_scale, sampling_ratio, 1, order, workspace, workspace_bytes, stream);
 }
 
 int mv_roi_align_2d_backward(const void *grad_output, const void *rois, void *grad_input,
@@ -291,9 +294,10 @@ int mv_roi_align_2d_backward(const void *grad_output, const void *rois, void *gr
 int mv_roi_align_3d_forward(const void *input, const void *rois, void *output, int dtype,
                             int batch, int channels, int depth, int height, int width,
                             int num_rois, int out_d, int out_h, int out_w, float spatial_scale,
-                            int sampling_ratio, int order, void *workspace, void *stream) {
+                            int sampling_ratio, int order, void *workspace,
+                            size_t workspace_bytes, void *stream) {
   return roi_forward(input, rois, output, dtype, 3, 0, batch, channels, depth, height, width,
-                     num_rois, out_d, out_h, out_w, spatial_scale, sampling_ratio, 1, order, workspace, stream);
+                     num_rois, out_d, out_h, out_w, spatial_scale, sampling_ratio, 1, order, workspace, workspace_bytes, stream);
 }
 
 int mv_roi_align_3d_backward(const void *grad_output, const void *rois, void *grad_input,
@@ -308,9 +312,10 @@ int mv_roi_align_3d_backward(const void *grad_output, const void *rois, void *gr
 int mv_roi_align_rotated_2d_forward(const void *input, const void *rois, void *output, int dtype,
                                     int batch, int channels, int height, int width, int num_rois,
                                     int out_h, int out_w, float spatial_scale, int sampling_ratio,
-                                    int aligned, int order, void *workspace, void *stream) {
+                                    int aligned, int order, void *workspace,
+                                    size_t workspace_bytes, void *stream) {
   return roi_forward(input, rois, output, dtype, 2, 1, batch, channels, 1, height, width, num_rois,
-                     1, out_h, out_w, spatial_scale, sampling_ratio, aligned, order, workspace, stream);
+                     1, out_h, out_w, spatial_scale, sampling_ratio, aligned, order, workspace, workspace_bytes, stream);
 }
 
 int mv_roi_align_rotated_2d_backward(const void *grad_output, const void *rois, void *grad_input,
@@ -327,10 +332,11 @@ int mv_roi_align_rotated_3d_forward(const void *input, const void *rois, void *o
                                     int batch, int channels, int depth, int height, int width,
                                     int num_rois, int out_d, int out_h, int out_w,
                                     float spatial_scale, int sampling_ratio, int aligned,
-                                    int order, void *workspace, void *stream) {
+                                    int order, void *workspace,
+                                    size_t workspace_bytes, void *stream) {
   return roi_forward(input, rois, output, dtype, 3, 1, batch, channels, depth, height, width,
                      num_rois, out_d, out_h, out_w, spatial_scale, sampling_ratio, aligned, order,
-                     workspace, stream);
+                     workspace, workspace_bytes, stream);
 }
 
 int mv_roi_align_rotated_3d_backward(const void *grad_output, const void *rois, void *grad_input,
@@ -349,7 +355,7 @@ size_t mv_roi_align_forward_workspace_bytes(int dtype, int ndim, int channels, i
   p.ndim = ndim; p.C = channels; p.R = num_rois;
   p.od = ndim == 2 ? 1 : out_d; p.oh = out_h; p.ow = out_w; p.sampling_ratio = sampling_ratio;
   size_t need = 0;
-  if (mv::roi_forward_tiled(nullptr, nullptr, nullptr, dtype, p, nullptr, &need, nullptr) != MV_OK) return 0;
+  if (mv::roi_forward_tiled(nullptr, nullptr, nullptr, dtype, p, nullptr, 0, &need, nullptr) != MV_OK) return 0;
   return need;
 }
 
@@ -374,19 +380,20 @@ size_t mv_roi_align_backward_workspace_bytes(int dtype, int batch, int channels,
 
 int mv_affine_2d(const void *input, const void *rois, void *output, int dtype, int batch,
                  int channels, int height, int width, int num_rois, int out_h, int out_w,
-                 float spatial_scale, int sampling_ratio, int aligned, int order, void *workspace, void *stream) {
+                 float spatial_scale, int sampling_ratio, int aligned, int order, void *workspace,
+                 size_t workspace_bytes, void *stream) {
   return roi_forward(input, rois, output, dtype, 2, 1, batch, channels, 1, height, width, num_rois,
-                     1, out_h, out_w, spatial_scale, sampling_ratio, aligned, order, workspace,
-                     stream, true);
+                     1, out_h, out_w, spatial_scale, sampling_ratio, aligned, order, workspace, workspace_bytes, stream, true);
 }
 
 int mv_affine_3d(const void *input, const void *rois, void *output, int dtype, int batch,
                  int channels, int depth, int height, int width, int num_rois, int out_d,
                  int out_h, int out_w, float spatial_scale, int sampling_ratio, int aligned,
-                 int order, void *workspace, void *stream) {
+                 int order, void *workspace,
+                 size_t workspace_bytes, void *stream) {
   return roi_forward(input, rois, output, dtype, 3, 1, batch, channels, depth, height, width,
                      num_rois, out_d, out_h, out_w, spatial_scale, sampling_ratio, aligned, order,
-                     workspace, stream, true);
+                     workspace, workspace_bytes, stream, true);
 }
 
 }  // extern "C"

@@ -1411,11 +1411,12 @@ size_t roi_pool_forward_workspace(int dtype, const RoiProblem &p) {
 }
 
 int roi_pool_forward(const void *input, const void *rois, void *output, int dtype,
-                     const RoiProblem &p, void *workspace, hipStream_t s) {
+                     const RoiProblem &p, void *workspace, size_t capacity, hipStream_t s) {
   if (!pool_applies(dtype, p)) return -1;
   const void *blocked = nullptr;
   const unsigned *order = nullptr;
-  if (workspace != nullptr && pool_blocked_bytes(dtype, p) > 0 && reinterpret_cast<uintptr_t>(input) % 8 == 0 &&
+  if (workspace != nullptr && pool_blocked_bytes(dtype, p) > 0 && capacity >= pool_blocked_bytes(dtype, p) &&
+      reinterpret_cast<uintptr_t>(input) % 8 == 0 &&
       reinterpret_cast<uintptr_t>(workspace) % 8 == 0) {
     const long rows = static_cast<long>(p.D) * p.H;
     const int Wb = p.W / 4, ux = std::min(Wb, kBlockUnits);

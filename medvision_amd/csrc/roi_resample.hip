@@ -1204,7 +1204,7 @@ static int launch_resample(const T *feat, const float *rois, T *out, const RoiPr
 }
 
 int roi_forward_tiled(const void *input, const void *rois, void *output, int dtype,
-                      const RoiProblem &p, void *workspace, size_t *need, hipStream_t s);
+                      const RoiProblem &p, void *workspace, size_t capacity, size_t *need, hipStream_t s);
 
 // Mean over the g^ndim samples of a bin: `fine` holds one sample per element, [planes][od*g][oh*g][ow*g]
 // ([planes][oh*g][ow*g] for images, gz = 1).
@@ -1232,7 +1232,7 @@ __global__ __launch_bounds__(256) void roi_bin_mean_kernel(const T *__restrict__
 // the means.  16-bit samples are rounded before the mean is; fp16's two roundings stay within its
 // tolerance, bf16's would not, so bf16 keeps the general kernel.
 static int roi_forward_tiled_grid(const void *input, const void *rois, void *output, int dtype,
-                                  const RoiProblem &p, void *workspace, size_t *need, hipStream_t s) {
+                                  const RoiProblem &p, void *workspace, size_t capacity, size_t *need, hipStream_t s) {
   const int g = p.sampling_ratio, gz = p.ndim == 3 ? g : 1;
   if (dtype != MV_F16 && dtype != MV_F32) return -1;
   if (!need && p.order != 1 && p.order != 3) return -1;
@@ -1247,12 +1247,12 @@ static int roi_forward_tiled_grid(const void *input, const void *rois, void *out
   const long fine = cells * gz * g * g;
   if (fine >= (1L << 31) || (cells + 255) / 256 >= (1L << 31)) return -1;
   size_t inner = 0;
-  if (roi_forward_tiled(nullptr, nullptr, nullptr, dtype, f, nullptr, &inner, nullptr) != MV_OK) return -1;
+  if (roi_forward_tiled(nullptr, nullptr, nullptr, dtype, f, nullptr, 0, &inner, nullptr) != MV_OK) return -1;
   inner = (inner + 255) & ~static_cast<size_t>(255);
   if (need) { *need = inner + static_cast<size_t>(fine) * dtype_size(dtype); return MV_OK; }
-  if (workspace == nullptr) return -1;
+  if (workspace == nullptr || capacity < inner + static_cast<size_t>(fine) * dtype_size(dtype)) return -1;
   void *samples = static_cast<char *>(workspace) + inner;
-  const int st = roi_forward_tiled(input, rois, samples, dtype, f, workspace, nullptr, s);
+  const int st = roi_forward_tiled(input, rois, samples, dtype, f, workspace, inner, nullptr, s);
   if (st != MV_OK) return st;   // -1: the finer problem does not fit the tiled kernel after all
   const dim3 grid(static_cast<unsigned>((cells + 255) / 256)), block(256);
   if (dtype == MV_F16)
@@ -1268,9 +1268,9 @@ static int roi_forward_tiled_grid(const void *input, const void *rois, void *out
 // fixed 2..4, in two passes).  With `need` set only the workspace size is computed.  Returns -1
 // when the path does not apply.
 int roi_forward_tiled(const void *input, const void *rois, void *output, int dtype,
-                      const RoiProblem &p, void *workspace, size_t *need, hipStream_t s) {
+                      const RoiProblem &p, void *workspace, size_t capacity, size_t *need, hipStream_t s) {
   if (p.sampling_ratio >= 2 && p.sampling_ratio <= 4)
-    return roi_forward_tiled_grid(input, rois, output, dtype, p, workspace, need, s);
+    return roi_forward_tiled_grid(input, rois, output, dtype, p, workspace, capacity, need, s);
   const long vox = static_cast<long>(p.od) * p.oh * p.ow;
   if (p.sampling_ratio != 1 || vox < 4096 || p.ow < 16 || p.R == 0) return -1;
   // Images: a tile's z extent is 1, so a lane's column is a single pixel and the per-item work of the

@@ -210,19 +210,21 @@ def test_input_gradient_with_non_finite_values(ops, oracle):
     assert_close(got[fin], gx[fin], BWD_TOL[torch.float32], "finite part of grad input")
 
 
-def test_config4_full_size_properties(ops):
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_config4_full_size_properties(ops, dtype):
     """Full config-4 shape [2,32,48^3] -> Cout 64: zero offsets and unit mask reduce DCN to a plain
-    convolution (checked against torch's conv3d), and the op is linear in the mask."""
+    convolution (checked against torch's conv3d in fp64 on the stored values), and the op is linear
+    in the mask."""
     from medvision_amd.ops.modulated_deform_conv_3d import modulated_deform_conv
     g = wl.gen(5)
-    x, off, mask, w, b = wl.dcn_inputs(g, 2, 32, 64, (48, 48, 48), 3, 1, 1, torch.float16)
+    x, off, mask, w, b = wl.dcn_inputs(g, 2, 32, 64, (48, 48, 48), 3, 1, 1, dtype)
     xs, offs, ms, ws, bs = _to(DEV, x, off, mask, w, b)
     y0 = modulated_deform_conv(xs, torch.zeros_like(offs), torch.ones_like(ms), ws, bs, 1, 1, 1, 1, 1)
-    ref = F.conv3d(xs.float(), ws.float(), bs.float(), 1, 1)
-    assert_close(y0, ref, FWD_TOL[torch.float16], "zero-offset == conv3d")
+    ref = F.conv3d(xs.double(), ws.double(), bs.double(), 1, 1)
+    assert_close(y0, ref, FWD_TOL[dtype], "zero-offset == conv3d")
     y1 = modulated_deform_conv(xs, offs, ms, ws, None, 1, 1, 1, 1, 1)
     y2 = modulated_deform_conv(xs, offs, ms * 0.5, ws, None, 1, 1, 1, 1, 1)
-    assert_close(y2.float() * 2, y1.float(), 4e-3, "mask linearity")
+    assert_close(y2.float() * 2, y1.float(), 2 * FWD_TOL[dtype], "mask linearity")
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
@@ -456,6 +458,29 @@ def test_general_deform_vs_oracle(ops, oracle, dtype, order):
         assert tuple(got.shape) == tuple(want.shape)
         assert_close(got, want, FWD_TOL[dtype], f"deform_{nd}d {size} k={k} order={order}")
         assert float((want == b.double().view(1, -1, *([1] * nd))).double().mean()) < 0.9
+    if order == 1 and dtype in (torch.float32, torch.float16):
+        # an identity weight (the warp) and then a real 1x1x1 weight of the same shape and type: a
+        # verdict remembered by address or version would send the second one down the warp path
+        x = torch.randn(1, 4, 6, 7, 8, generator=g).to(dtype)
+        off = (torch.randn(1, 3, 6, 7, 8, generator=g) * 1.5).to(dtype)
+        zero = torch.zeros(4, dtype=dtype)
+        for rep in range(3):
+            eye = torch.eye(4).view(4, 4, 1, 1, 1).to(dtype).to(DEV)
+            got = _C.deform_3d(x.to(DEV), eye, zero.to(DEV), off.to(DEV), 1, 1, 1, 1, 1, 1, 0, 0, 0, 1, 1, 1, 1, 1, 64, 1)
+            assert_close(got, oracle.deform_conv(x, off, eye.cpu(), zero, (1, 1, 1), (0, 0, 0), (1, 1, 1), 1, 1, 1),
+                         FWD_TOL[dtype], "identity weight")
+            del eye
+            w = torch.randn(4, 4, 1, 1, 1, generator=g).to(dtype)
+            wd = w.to(DEV)
+            got = _C.deform_3d(x.to(DEV), wd, zero.to(DEV), off.to(DEV), 1, 1, 1, 1, 1, 1, 0, 0, 0, 1, 1, 1, 1, 1, 64, 1)
+            assert_close(got, oracle.deform_conv(x, off, w, zero, (1, 1, 1), (0, 0, 0), (1, 1, 1), 1, 1, 1),
+                         FWD_TOL[dtype], "random 1x1x1 weight after an identity one")
+            ident = torch.eye(4).view(4, 4, 1, 1, 1).to(dtype).to(DEV)
+            ident.data.mul_(2.0)     # (a write that leaves the tensor's version alone)
+            got = _C.deform_3d(x.to(DEV), ident, zero.to(DEV), off.to(DEV), 1, 1, 1, 1, 1, 1, 0, 0, 0, 1, 1, 1, 1, 1, 64, 1)
+            assert_close(got, oracle.deform_conv(x, off, ident.cpu(), zero, (1, 1, 1), (0, 0, 0), (1, 1, 1), 1, 1, 1),
+                         FWD_TOL[dtype], "identity weight edited through .data")
+            del wd, ident
     x = torch.zeros(2, 4, 4, 4, 4, device=DEV)
     with pytest.raises(RuntimeError, match="kernel shape wont match"):
         _C.deform_3d(x, torch.zeros(4, 4, 3, 3, 3, device=DEV), torch.zeros(4, device=DEV),

@@ -279,6 +279,10 @@ def test_config3_resize_and_crops(ops, oracle):
     seg = (vol > 0).to(torch.float16)
     got = ops.affine_3d(seg.to(DEV), crops.to(DEV), (24, 24, 24), 1.0, 1, True, 0)
     assert set(got.unique().tolist()) <= {0.0, 1.0}
+    want = oracle.roi_align_forward(seg, crops, (24, 24, 24), 1.0, 1, True, 0, True)
+    margin = oracle.roi_decision_margin(seg.shape, crops, (24, 24, 24), 1.0, 1, True, True)
+    frac = assert_nearest(got, want, margin, torch.float16, "nearest crops of the label map")
+    assert frac < 1e-3, f"nearest mismatches: {frac:.2e}"
 
 
 @pytest.mark.parametrize("dtype,channels,rois_n,size,out,order", [
@@ -474,6 +478,19 @@ def test_pooled_forward_from_blocked_copy(ops, oracle, ndim):
     assert _lib.load().mv_roi_align_forward_workspace_bytes_for_input(_lib.MV_F16, ndim, 2, channels, *in3, 15, *out3, 2) == 0
     got = ops.RoIAlign(out, 1.0, 2)(feat.to(DEV), few.to(DEV))
     assert_close(got, want[:15], FWD_TOL[torch.float16], "pooled forward from the input")
+    # straight through the C ABI with a workspace that is too small for the copy (a caller that sized
+    # its arena with the query that does not know the input): the entry point must not use it
+    import ctypes
+    lib = _lib.load()
+    x, r = feat.to(DEV), rois.to(DEV)
+    raw = torch.full((n, channels, *out), float("nan"), dtype=torch.float16, device=DEV)
+    small = torch.full((4096,), 7, dtype=torch.uint8, device=DEV)
+    fn = lib.mv_roi_align_3d_forward if ndim == 3 else lib.mv_roi_align_2d_forward
+    _lib.check(fn(_lib.ptr(x), _lib.ptr(r), _lib.ptr(raw), _lib.MV_F16, *x.shape, n, *out, 1.0, 2, 1,
+                  _lib.ptr(small), 4096, _lib.stream_of(x)))
+    torch.cuda.synchronize()
+    assert bool((small == 7).all()), "the undersized workspace was written"
+    assert_close(raw, want, FWD_TOL[torch.float16], "pooled forward, workspace too small for the copy")
 
 
 @pytest.mark.parametrize("out", [(8, 8, 8), (3, 6, 6), (2, 5, 7), (7, 4, 8), (5, 5, 5), (6, 6), (4, 8), (5, 5)])
