@@ -372,6 +372,49 @@ def copy_calibration(args):
                       "gbps": 4 * n / ms / 1e6}))
 
 
+def resample_timeline(args):
+    """In-kernel phase times of the tiled resampler on config 2 (fp16): runs the instrumented twin of the
+    library (time stamps of thread 0 of every workgroup, 100 MHz wall clock, see MV_TL in
+    csrc/roi_resample.hip) and prints, per marked point, the minimum / median / maximum over the
+    workgroups of the last launch in microseconds since the first workgroup entered the kernel."""
+    import ctypes
+    import numpy as np
+    from medvision_amd import _lib, build
+    import workloads as wl
+    _lib.LIB_PATH = build.TIMELINE_LIB_PATH
+    _lib.load()
+    from medvision_amd import _C
+    dev, B, S = "cuda:0", 4, 128
+    g = wl.gen(1)
+    vols = [torch.randn(B, 1, S, S, S, generator=g).half().to(dev) for _ in range(args.copies)]
+    rois = [wl.affine_rois(g, B, (S, S, S)).to(dev) for _ in range(args.copies)]
+    outs = [torch.empty(B, 1, S, S, S, dtype=torch.float16, device=dev) for _ in range(args.copies)]
+    ms, _ = _events_ms(lambda i: _C.roi_align_rotated_3d_forward(vols[i % args.copies], rois[i % args.copies],
+                                                                  outs[i % args.copies], S, S, S, 1.0, 1, True, 1),
+                       args.steps, args.warmup)
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    buf = np.zeros(4096 * 16, dtype=np.uint64)
+    rc = raw.mv_debug_resample_timeline(ctypes.c_void_p(buf.ctypes.data), ctypes.c_size_t(buf.nbytes))
+    if rc != 0:
+        sys.exit("mv_debug_resample_timeline failed: %d" % rc)
+    t = buf.reshape(4096, 16).astype(np.int64)
+    t = t[t[:, 0] > 0]
+    t0 = t[:, 0].min()
+    names = ["kernel entered", "first wavefront starts planning", "plans written", "past the barrier behind the plans",
+             "first box arrived in registers", "box of item 0 in LDS", "box of item 1 in LDS", "box of item 2 in LDS",
+             "box of item 3 in LDS", "last item interpolated", "stores drained"]
+    rows = []
+    for k, name in enumerate(names):
+        v = (t[:, k] - t0)[t[:, k] > 0] / 100.0
+        rows.append({"point": name, "min_us": round(float(v.min()), 2), "median_us": round(float(np.median(v)), 2),
+                     "max_us": round(float(v.max()), 2)})
+    # the two workgroups of a compute unit: blocks i and i + half the grid of an XCD share one (the older is served first)
+    done = (t[:, 10] - t0) / 100.0
+    print(json.dumps({"workgroups": int(len(t)), "instrumented_kernel_us": round(ms * 1e3, 2), "points": rows,
+                      "finish_us_by_launch_order": {"first_half_of_each_xcd": round(float(np.median(done[: len(done) // 2])), 2),
+                                                    "second_half_of_each_xcd": round(float(np.median(done[len(done) // 2:])), 2)}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -383,6 +426,8 @@ def main():
     ap.add_argument("--no-next", action="store_true", help="skip the timings of the neighbouring operators")
     ap.add_argument("--no-configs", action="store_true", help="skip configs 1, 2-backward, 3 and 5")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="wall time spent on the CPU oracle")
+    ap.add_argument("--timeline", action="store_true",
+                    help="only print the in-kernel phase times of the tiled resampler (instrumented library)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a device copy of 4*128^3 fp16 elements (counter calibration)")
     args = ap.parse_args()
@@ -391,6 +436,9 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
     from medvision_amd import _lib
+    if args.timeline:
+        resample_timeline(args)
+        return
     _lib.load()
     if args.copy_calibration:
         copy_calibration(args)

@@ -13,6 +13,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libmedvision_hip.so")
+# the same library with in-kernel time stamps in the tiled resampler (a measuring aid: `bench.py --timeline`)
+TIMELINE_LIB_PATH = os.path.join(LIB_DIR, "libmedvision_hip_timeline.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -48,6 +50,12 @@ def build(verbose=False, jobs=None):
                                               "-c", so[0], "-o", so[1]]),
                              zip(sources, objs)))
     link = _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs])
+    # instrumented twin: only roi_resample.hip differs
+    tl_src = os.path.join(CSRC, "roi_resample.hip")
+    tl_obj = os.path.join(obj_dir, "roi_resample_timeline.o")
+    outs.append(_run([HIPCC, *FLAGS, "-DMV_RESAMPLE_TIMELINE", "-c", tl_src, "-o", tl_obj]))
+    tl_objs = [tl_obj if os.path.basename(o) == "roi_resample.o" else o for o in objs]
+    link += _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", TIMELINE_LIB_PATH, *tl_objs])
     if verbose:
         for o in outs + [link]:
             if o.strip():

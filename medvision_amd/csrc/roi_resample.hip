@@ -29,6 +29,22 @@
 
 namespace mv {
 
+// In-kernel time stamps of the tiled forward kernel (instrumented build only, -DMV_RESAMPLE_TIMELINE:
+// a second library beside the product, read back by mv_debug_resample_timeline): thread 0 of every
+// workgroup notes the 100 MHz wall clock at the points MV_TL marks.  Slots: 0 kernel entered, 1 first
+// wavefront starts planning, 2 plans written, 3 past the barrier behind the plans, 4 first box has
+// arrived in registers, 5..8 box of item 0..3 is in LDS, 9 last item interpolated, 10 stores drained.
+#ifdef MV_RESAMPLE_TIMELINE
+constexpr int kTimelineSlots = 16, kTimelineGroups = 4096;
+__device__ unsigned long long mv_timeline[kTimelineGroups * kTimelineSlots];
+#define MV_TL(i)                                                                                          \
+  do {                                                                                                    \
+    if (threadIdx.x == 0 && blockIdx.x < kTimelineGroups) mv_timeline[blockIdx.x * kTimelineSlots + (i)] = wall_clock64(); \
+  } while (0)
+#else
+#define MV_TL(i) do { } while (0)
+#endif
+
 constexpr int kXcds = 8;
 
 // What the workgroup's first wavefront works out per item and every wavefront then reads from LDS.
@@ -700,6 +716,8 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
   // assignment is rotated from round to round so that a workgroup does not get the same tile
   // position (border: cheap, centre: expensive) in every roi.
   const int tid = threadIdx.x;
+  MV_TL(0);
+  [[maybe_unused]] int tl_item = 0;
   const unsigned per_roi = static_cast<unsigned>(ps.tiles_x) * ps.tiles_y * ps.tiles_z;
   auto fetch_plan = [&](unsigned r) -> PlanLanes {
     PlanLanes pl;
@@ -789,9 +807,12 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
     const unsigned sr = slot + r * 27u;
     const unsigned k = r * slots + (sr - ps.by_slots.div(sr) * slots);
     const unsigned item = ((k / kChunk) * parts + xcd) * kChunk + k % kChunk;
+    MV_TL(1);
     plan_item_lanes(rois, p, ps, item < work ? item : kDone, total, per_roi, &lplans[r]);
+    MV_TL(2);
   }
   __syncthreads();
+  MV_TL(3);
   mode = prepare(true, fetch_plan(0), *reinterpret_cast<const i32x4 *>(&lplans[0].inv_groups), lplans[0].rp, lplans[0].gap_b);
   if (mode == 4) return;
 #pragma unroll
@@ -822,6 +843,7 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
     // All loads issued for this item have to be back; waiting here on every path (vmcnt(0), other
     // counters untouched) keeps the compiler from waiting again after the stores of phase B.
     __builtin_amdgcn_s_waitcnt(0x0F70);
+    if (tl_item == 0) MV_TL(4);
     if (staged) {
       if (ld_passes > 0) {   // still this item's: the next `prepare` comes after the barrier
         const int bz = cpy.z, span = cpy.w, hop_b = t.w;
@@ -865,6 +887,8 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
     }
     __syncthreads();
 
+    if (tl_item < 4) MV_TL(5 + tl_item);
+    tl_item++;
     // ---- B + C: this item; ahead of voxel k the previous item's voxel k is stored and a share of
     // the next box's loads is issued, so that neither piles up in the memory pipeline -------------
     const int next_mode = prepare(has_next, nplan, nsp, nrp, ngap);
@@ -949,6 +973,11 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
         __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(pend_base), 0, pend_bytes, 0x00020000);
     store_element<T>(rsrc, pend_voff, k * zbytes, o[k]);
   }
+#ifdef MV_RESAMPLE_TIMELINE
+  MV_TL(9);
+  __builtin_amdgcn_s_waitcnt(0);
+  MV_TL(10);
+#endif
 }
 
 // Compute units of the current device (workgroups resident at once = units * LDS share).
@@ -1603,3 +1632,12 @@ int roi_backward_tiled(const void *grad_output, const void *rois, float *acc, in
 }
 
 }  // namespace mv
+
+#ifdef MV_RESAMPLE_TIMELINE
+// Copies the time stamps of the last tiled forward launches to `host` (kTimelineGroups x kTimelineSlots
+// 64-bit words, 100 MHz ticks); synchronises the device.
+extern "C" int mv_debug_resample_timeline(void *host, size_t bytes) {
+  const size_t all = sizeof(unsigned long long) * mv::kTimelineGroups * mv::kTimelineSlots;
+  return static_cast<int>(hipMemcpyFromSymbol(host, HIP_SYMBOL(mv::mv_timeline), bytes < all ? bytes : all));
+}
+#endif
