@@ -2,8 +2,10 @@
 ``affine_2d`` / ``affine_3d`` / ``apply_offset_*`` in the reference's ``medvision.aug_cuda`` and
 ``medvision.aug_cuda_batch``)."""
 from .base import BatchCudaAugBase, CudaAugBase
-from .spatial import (BatchCudaCropCenterWithAffine, BatchCudaCropRandomWithAffine,
-                      BatchCudaRandomAffine, BatchCudaRandomRotate, BatchCudaRandomScale,
+from .spatial import (BatchCudaCropCenterWithAffine, BatchCudaCropDetWithAffine,
+                      BatchCudaCropFirstDetWithAffine, BatchCudaCropForegroundWithAffine,
+                      BatchCudaCropRandomWithAffine,
+                      BatchCudaRandomAffine, BatchCudaRandomElasticDeformation, BatchCudaRandomRotate, BatchCudaRandomScale,
                       BatchCudaRandomShift, BatchCudaResize, CudaCropCenterWithAffine,
                       CudaCropFirstDetWithAffine, CudaCropRandomWithAffine, CudaRandomAffine,
                       CudaRandomElasticDeformation, CudaRandomRotate, CudaRandomScale,

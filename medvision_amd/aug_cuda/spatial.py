@@ -8,6 +8,7 @@ aug_spatial.py`` (:69-202, :356-597, :600-850).  Every image stage boils down to
 segmentations go through the same rois at order 0 as float and come back as int32.
 """
 import itertools
+import random
 import math
 import warnings
 
@@ -291,19 +292,28 @@ class CudaCropFirstDetWithAffine(CudaCropRandomWithAffine):
         self.border = border
         super().__init__(*args, **kwargs)
 
+    def _start_around(self, lo_zyx, hi_zyx):
+        """A window start (z, y, x) drawn so that [lo, hi) widened by ``border`` lies inside the window
+        where the patch and the volume allow it."""
+        start = []
+        for axis in range(self.dim):
+            room = self.image_shape[axis] - self.patch_size[axis]
+            first = min(max(hi_zyx[axis] + self.border - self.patch_size[axis], 0), room)
+            last = min(max(lo_zyx[axis] - self.border, 0), room)
+            start.append(np.random.randint(min(first, last), max(first, last) + 1))
+        return tuple(start)
+
+    def _start_around_box(self, box):
+        """``box`` = (x1, y1[, z1], x2, y2[, z2], ...) as the detection fields store it."""
+        box = box.cpu().numpy() if torch.is_tensor(box) else np.asarray(box)
+        return self._start_around([box[self.dim - axis - 1] for axis in range(self.dim)],
+                                  [box[2 * self.dim - axis - 1] for axis in range(self.dim)])
+
     def _crop_start(self, result, sample):
         assert 'gt_det' in result, "it only used for detection tasks"
         if len(result['gt_det']) == 0:
             return super()._crop_start(result, sample)
-        box = result['gt_det'][0].cpu().numpy()
-        start = []
-        for axis in range(self.dim):    # z, y, x; boxes are stored x, y, z
-            lo, hi = box[self.dim - axis - 1], box[2 * self.dim - axis - 1]
-            room = self.image_shape[axis] - self.patch_size[axis]
-            first = min(max(hi + self.border - self.patch_size[axis], 0), room)
-            last = min(max(lo - self.border, 0), room)
-            start.append(np.random.randint(min(first, last), max(first, last) + 1))
-        return tuple(start)
+        return self._start_around_box(result['gt_det'][0])
 
 
 class BatchCudaCropRandomWithAffine(CudaCropRandomWithAffine, BatchCudaAugBase):
@@ -314,16 +324,57 @@ class BatchCudaCropCenterWithAffine(CudaCropCenterWithAffine, BatchCudaAugBase):
     pass
 
 
+class BatchCudaCropFirstDetWithAffine(CudaCropFirstDetWithAffine, BatchCudaAugBase):
+    """aug_cuda_batch/aug_spatial.py:928-960: every sample's window is drawn around the first box."""
+
+    def __init__(self, border=12, **kwargs):
+        super().__init__(border, **kwargs)
+
+    def _crop_start(self, result, sample):
+        assert 'gt_det' in result, "it only used for detection tasks"
+        return self._start_around_box(result['gt_det'][0])
+
+
+class BatchCudaCropDetWithAffine(BatchCudaCropFirstDetWithAffine):
+    """aug_cuda_batch/aug_spatial.py:893-925: the boxes take turns, one per drawn window."""
+
+    def __init__(self, border=12, **kwargs):
+        super().__init__(border, **kwargs)
+        self.current_repeat_idx = 0
+
+    def _crop_start(self, result, sample):
+        assert 'gt_det' in result, "it only used for detection tasks"
+        pick = min(self.current_repeat_idx % self.repeats, len(result['gt_det']) - 1)
+        self.current_repeat_idx += 1
+        return self._start_around_box(result['gt_det'][pick])
+
+
+class BatchCudaCropForegroundWithAffine(BatchCudaCropFirstDetWithAffine):
+    """aug_cuda_batch/aug_spatial.py:852-890: the window is drawn around one connected component of the
+    sample's label map (``gt_seg``, else ``pseudo_mask``), anywhere when the map is empty."""
+
+    def _crop_start(self, result, sample):
+        from scipy import ndimage as ndi
+        assert 'gt_seg' in result or 'pseudo_mask' in result
+        mask = result['gt_seg' if 'gt_seg' in result else 'pseudo_mask'][sample, 0]
+        objs = ndi.find_objects(ndi.label(mask.cpu().numpy())[0])
+        if not objs:
+            return CudaCropRandomWithAffine._crop_start(self, result, sample)
+        obj = random.choice(objs)
+        return self._start_around([o.start for o in obj], [o.stop for o in obj])
+
+
 # ---- elastic deformation ---------------------------------------------------------------------------
 class CudaRandomElasticDeformation(CudaAugBase):
     """Random displacements on a coarse control grid (two locked border layers), upsampled to a
     dense field with the order-3 affine engine and applied with the displacement-field warp."""
 
-    def __init__(self, p, num_control_points=8, max_displacement=0.8):
+    def __init__(self, p, num_control_points=8, max_displacement=0.8, order=3):
         super().__init__()
         self.p = p
         self.num_control_points = num_control_points   # z, y, x
         self.max_displacement = max_displacement       # fraction of half a grid cell
+        self.INTER_ORDER = order                       # of the control grid's upsampling
         self.num_locked_borders = 2
         assert max_displacement <= 1.0
         self.tmp_params = None
@@ -341,12 +392,16 @@ class CudaRandomElasticDeformation(CudaAugBase):
         self._init_params(result)
         grid = self.to_tuple(self.num_control_points, self.dim)
         cell = np.array(self.image_shape) / (np.array(grid) - 1)
-        coarse = 2 * np.random.rand(*grid, self.dim).astype(np.float32) - 1
-        coarse *= self.max_displacement * cell / 2          # per component (z, y, x)
         inner = tuple(slice(self.num_locked_borders, n - self.num_locked_borders) for n in grid)
-        locked = np.zeros_like(coarse)
-        locked[inner] = coarse[inner]
-        self.params = locked
+        fields = []
+        for _ in range(self.batch):      # one draw per sample, in sample order
+            coarse = 2 * np.random.rand(*grid, self.dim).astype(np.float32) - 1
+            coarse *= self.max_displacement * cell / 2          # per component (z, y, x)
+            locked = np.zeros_like(coarse)
+            locked[inner] = coarse[inner]
+            fields.append(locked)
+        # per-sample stage: [*grid, dim]; batch stage: [batch, *grid, dim]
+        self.params = np.array(fields) if self.batched else fields[0]
         result[self.key_name] = self.params
 
     def _backward_params(self, result):
@@ -357,27 +412,35 @@ class CudaRandomElasticDeformation(CudaAugBase):
             self.params = -params
 
     def dense_field(self, device):
-        """[dim, *image_shape] displacements (z, y, x components), cached per draw."""
+        """[dim, *image_shape] displacements (z, y, x components) -- the batch stage: [batch, dim,
+        *image_shape] -- cached per draw."""
         if self.tmp_params is None:
-            grid = torch.from_numpy(self.params).permute(self.dim, *range(self.dim)) / 2
-            shape_xyz = list(grid.shape[1:])[::-1]
-            roi = geometry.window_rois(self.dim, [1.5] * self.dim, [s - 1.5 for s in shape_xyz])
+            coarse = torch.from_numpy(self.params if self.batched else self.params[None])
+            grid = coarse.permute(0, self.dim + 1, *range(1, self.dim + 1)) / 2
+            shape_xyz = list(grid.shape[2:])[::-1]
+            roi = geometry.window_rois(self.dim, [1.5] * self.dim, [s - 1.5 for s in shape_xyz],
+                                       index=np.arange(grid.shape[0]))
             fn = affine_2d if self.dim == 2 else affine_3d
-            self.tmp_params = fn(grid.to(device).unsqueeze(0).contiguous(), torch.from_numpy(roi).to(device),
-                                 tuple(self.image_shape), 1, 1, True, 3).squeeze(0)
+            dense = fn(grid.to(device).contiguous(), torch.from_numpy(roi).to(device),
+                       tuple(self.image_shape), 1, 1, True, self.INTER_ORDER)
+            self.tmp_params = dense if self.batched else dense.squeeze(0)
         return self.tmp_params
 
     def elastic_transform(self, image, order=1):
         field = self.dense_field(image.device)
         fn = apply_offset_2d if self.dim == 2 else apply_offset_3d
+        if not self.batched:
+            image, field = image.unsqueeze(0), field.unsqueeze(0)
         if order == 0 and image.dtype == torch.int32:
             # the reference converts labels to float, warps and converts back
             # (aug_cuda/aug_spatial.py:664-668); the warp takes int32 maps as they are
-            return fn(image.unsqueeze(0), field.unsqueeze(0), order=0).squeeze(0)
-        if order == 0:
-            image = image.to(self.img_type)
-        out = fn(image.unsqueeze(0), field.unsqueeze(0).to(image.dtype), order=order).squeeze(0)
-        return out.int() if order == 0 else out
+            out = fn(image, field, order=0)
+        else:
+            if order == 0:
+                image = image.to(self.img_type)
+            out = fn(image, field.to(image.dtype), order=order)
+            out = out.int() if order == 0 else out
+        return out if self.batched else out.squeeze(0)
 
     def apply_to_img(self, result):
         for key in result.get('img_fields', []):
@@ -389,6 +452,8 @@ class CudaRandomElasticDeformation(CudaAugBase):
 
     def apply_to_det(self, result):
         for key in result.get('det_fields', []):
+            if self.batched:   # as in the reference (aug_cuda_batch/aug_spatial.py:318-320)
+                raise NotImplementedError
             boxes = np.copy(result[key].cpu().numpy())
             field = self.dense_field(result[key].device).cpu().numpy()
             top = np.array(self.image_shape) - 1
@@ -402,3 +467,8 @@ class CudaRandomElasticDeformation(CudaAugBase):
                 box[:self.dim] = corners.min(0)
                 box[self.dim:2 * self.dim] = corners.max(0)
             result[key] = torch.from_numpy(boxes).to(result[key].device)
+
+
+class BatchCudaRandomElasticDeformation(CudaRandomElasticDeformation, BatchCudaAugBase):
+    """aug_cuda_batch/aug_spatial.py:204-320: one control grid per sample of the batch (drawn in sample
+    order), all upsampled by one call of the affine engine and applied by one warp."""

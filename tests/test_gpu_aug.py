@@ -193,3 +193,73 @@ def test_elastic(aug, oracle, dim):
     still = aug.CudaRandomElasticDeformation(1.0, 7, 0.0)
     res2, img2, _ = _sample(g, shape)
     assert torch.equal(still(res2)["img"].cpu(), img2)
+
+
+@pytest.mark.parametrize("dim", [2, 3])
+def test_batch_elastic_equals_per_sample(aug, oracle, dim):
+    """The batch stage draws one control grid per sample in sample order and warps the batch in one
+    call: sample b must equal the per-sample stage run on that grid, and the oracle."""
+    g = wl.gen(230 + dim)
+    shape = (36, 44) if dim == 2 else (20, 24, 28)
+    B = 3
+    img = torch.randn(B, 2, *shape, generator=g)
+    seg = torch.randint(0, 4, (B, 1, *shape), generator=g, dtype=torch.int32)
+    res = {"img": img.to(DEV), "gt_seg": seg.to(DEV), "img_dim": dim, "img_fields": ["img"], "seg_fields": ["gt_seg"],
+           "det_fields": []}
+    stage = aug.BatchCudaRandomElasticDeformation(1.0, num_control_points=7, max_displacement=0.9)
+    np.random.seed(31)
+    out = stage(res)
+    grids = out["BatchCudaRandomElasticDeformation_params"]
+    assert grids.shape == (B, *([7] * dim), dim)
+    np.random.seed(31)   # the same draws, one sample at a time
+    for b in range(B):
+        want_grid = 2 * np.random.rand(*([7] * dim), dim).astype(np.float32) - 1
+        inner = tuple(slice(2, 5) for _ in range(dim))
+        assert np.all(grids[b][inner] != 0) and np.count_nonzero(grids[b]) == 3 ** dim * dim
+        assert np.allclose(np.sign(grids[b][inner]), np.sign(want_grid[inner]))
+        coarse = torch.from_numpy(grids[b]).permute(dim, *range(dim))[None] / 2
+        roi = torch.tensor([[0, *([3.5] * dim), *([4.0] * dim), *([0.0] * (2 * dim - 3))]])
+        field = oracle.roi_align_forward(coarse, roi, shape, 1.0, 1, True, 3, True)
+        assert_close(stage.tmp_params[b], field[0], FWD_TOL[torch.float32], "dense field of sample %d" % b)
+        f32 = stage.tmp_params[b].cpu()[None]
+        assert_close(out["img"][b], oracle.deform_warp(img[b][None], f32, 1)[0], FWD_TOL[torch.float32], "warped image")
+        assert torch.equal(out["gt_seg"][b].cpu().double(), oracle.deform_warp(seg[b][None].float(), f32, 0)[0])
+    assert float((stage.tmp_params[0] - stage.tmp_params[1]).abs().max()) > 0.1   # samples differ
+    with pytest.raises(NotImplementedError):
+        stage.apply_to_det({"det_fields": ["gt_det"], "gt_det": torch.zeros(1, 6)})
+
+
+def test_batch_crops_around_boxes_and_foreground(aug):
+    """The windows of the detection / foreground crop stages contain the box or component they were
+    drawn around (plus the border where the patch has room); identity affine == slicing."""
+    g = wl.gen(240)
+    B, shape, patch = 3, (24, 28, 32), (12, 14, 16)
+    img = torch.randn(B, 1, *shape, generator=g)
+    seg = torch.zeros(B, 1, *shape, dtype=torch.int32)
+    blobs = [(3, 4, 5), (10, 12, 20), (18, 20, 6)]
+    for b, (z, y, x) in enumerate(blobs):
+        seg[b, 0, z:z + 3, y:y + 4, x:x + 5] = 1
+    det = torch.tensor([[6., 5., 4., 11., 9., 7., 1., 1.], [20., 12., 10., 25., 16., 13., 1., 1.]], dtype=torch.float64)
+    base = {"img_dim": 3, "img_fields": ["img"], "seg_fields": ["gt_seg"], "det_fields": []}
+    random.seed(5)
+    np.random.seed(5)
+    fg = aug.BatchCudaCropForegroundWithAffine(border=2, patch_size=patch, scale=0, shift=0, rotate=0)
+    out = fg({**base, "img": img.to(DEV), "gt_seg": seg.to(DEV)})
+    p = out["BatchCudaCropForegroundWithAffine_params"]
+    for b, (z, y, x) in enumerate(blobs):
+        sx, sy, sz = p["start"][b]
+        assert sz <= z and z + 3 <= sz + patch[0] and sy <= y and y + 4 <= sy + patch[1] and sx <= x and x + 5 <= sx + patch[2]
+        assert torch.equal(out["img"][b].cpu(), img[b, :, sz:sz + patch[0], sy:sy + patch[1], sx:sx + patch[2]])
+        assert int(out["gt_seg"][b].sum()) == 60
+    first = aug.BatchCudaCropFirstDetWithAffine(border=1, patch_size=patch, scale=0, shift=0, rotate=0)
+    out = first({**base, "seg_fields": [], "img": img.to(DEV), "gt_det": det.to(DEV)})
+    for b in range(B):
+        sx, sy, sz = out["BatchCudaCropFirstDetWithAffine_params"]["start"][b]
+        assert sx <= 6 and 11 <= sx + patch[2] and sy <= 5 and 9 <= sy + patch[1] and sz <= 4 and 7 <= sz + patch[0]
+    turns = aug.BatchCudaCropDetWithAffine(border=1, patch_size=patch, scale=0, shift=0, rotate=0, times=2)
+    turns._init_params({"img": img.to(DEV), "img_dim": 3})
+    picks = []
+    for _ in range(4):
+        sz, sy, sx = turns._crop_start({"gt_det": det.to(DEV)}, 0)
+        picks.append(0 if sx <= 6 and 11 <= sx + patch[2] else 1)
+    assert picks == [0, 1, 0, 1]
