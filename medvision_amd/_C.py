@@ -257,65 +257,8 @@ def _dcn_bytes(fn, shape, code):
     return n
 
 
-# Channel counts the matrix-core kernels take: multiples of 32 per deformable group and of 32 output
-# channels (csrc/dcn3d_mfma.hip, dcn3d_mfma_backward.hip).  Other layers of one weight group (16, 24,
-# 40, 48 ... channels) would run the general kernels, 50 - 100 times slower, so they are padded with
-# zero channels here: zero inputs and zero weight rows / columns add nothing to any output or gradient.
-_DCN_PAD = 32
-
-
-def _dcn_pad_plan(input, weight, shape):
-    cin, cout, dg = shape.in_channels, shape.out_channels, shape.deformable_groups
-    if shape.groups != 1 or input.dtype not in (torch.float16, torch.bfloat16, torch.float32):
-        return None
-    cpd = cin // dg
-    cpd_p = -(-cpd // _DCN_PAD) * _DCN_PAD
-    cout_p = -(-cout // _DCN_PAD) * _DCN_PAD
-    if (cpd_p == cpd and cout_p == cout) or cin * cout < 256:
-        return None
-    return cpd, cpd_p, cout_p
-
-
-def _pad_groups(t, dim, groups, per_new):
-    """``t`` with its ``groups`` blocks of channels along ``dim`` widened to ``per_new`` (zeros)."""
-    shape = list(t.shape)
-    per = shape[dim] // groups
-    if per == per_new:
-        return t
-    out = t.new_zeros(*shape[:dim], groups, per_new, *shape[dim + 1:])
-    out.narrow(dim + 1, 0, per).copy_(t.reshape(*shape[:dim], groups, per, *shape[dim + 1:]))
-    return out.reshape(*shape[:dim], groups * per_new, *shape[dim + 1:])
-
-
-def _unpad_groups(t, dim, groups, per):
-    shape = list(t.shape)
-    per_p = shape[dim] // groups
-    if per == per_p:
-        return t
-    v = t.reshape(*shape[:dim], groups, per_p, *shape[dim + 1:]).narrow(dim + 1, 0, per)
-    return v.reshape(*shape[:dim], groups * per, *shape[dim + 1:])
-
-
-def _dcn_padded_shape(shape, cin_p, cout_p):
-    padded = type(shape).from_buffer_copy(shape)
-    padded.in_channels, padded.out_channels = cin_p, cout_p
-    return padded
-
-
 def _dcn_forward(input, offset, mask, weight, bias, output, shape):
     lib = _lib.load()
-    plan = _dcn_pad_plan(input, weight, shape)
-    if plan is not None:
-        _same_device(input, offset=offset, mask=mask, weight=weight, bias=bias, output=output)
-        cpd, cpd_p, cout_p = plan
-        dg, cout = shape.deformable_groups, shape.out_channels
-        wide = torch.empty((output.size(0), cout_p, *output.shape[2:]), dtype=output.dtype, device=output.device)
-        _dcn_forward(_pad_groups(input, 1, dg, cpd_p), offset, mask,
-                     _pad_groups(_pad_groups(weight, 1, dg, cpd_p), 0, 1, cout_p),
-                     None if bias is None else _pad_groups(bias, 0, 1, cout_p), wide,
-                     _dcn_padded_shape(shape, dg * cpd_p, cout_p))
-        output.copy_(wide[:, :cout])
-        return
     _same_device(input, offset=offset, mask=mask, weight=weight, bias=bias, output=output)
     fam = _dcn_family(shape)
     dims = _dcn_out_dims(lib, shape)
@@ -336,23 +279,6 @@ def _dcn_forward(input, offset, mask, weight, bias, output, shape):
 
 def _dcn_backward(input, offset, mask, weight, grad_output, gi, goff, gmask, gw, gb, shape):
     lib = _lib.load()
-    plan = _dcn_pad_plan(input, weight, shape)
-    if plan is not None:
-        _same_device(input, offset=offset, mask=mask, weight=weight, grad_output=grad_output,
-                     grad_input=gi, grad_offset=goff, grad_mask=gmask, grad_weight=gw, grad_bias=gb)
-        cpd, cpd_p, cout_p = plan
-        dg, cout = shape.deformable_groups, shape.out_channels
-        x_p = _pad_groups(input, 1, dg, cpd_p)
-        w_p = _pad_groups(_pad_groups(weight, 1, dg, cpd_p), 0, 1, cout_p)
-        gi_p, gw_p = torch.zeros_like(x_p), torch.zeros_like(w_p)
-        gb_p = None if gb is None else gb.new_zeros(cout_p)
-        _dcn_backward(x_p, offset, mask, w_p, _pad_groups(grad_output.to(input.dtype), 1, 1, cout_p), gi_p, goff,
-                      gmask, gw_p, gb_p, _dcn_padded_shape(shape, dg * cpd_p, cout_p))
-        gi.add_(_unpad_groups(gi_p, 1, dg, cpd))          # (the buffers accumulate, as without padding)
-        gw.add_(_unpad_groups(gw_p[:cout], 1, dg, cpd))
-        if gb is not None:
-            gb.add_(gb_p[:cout])
-        return
     _same_device(input, offset=offset, mask=mask, weight=weight, grad_output=grad_output,
                  grad_input=gi, grad_offset=goff, grad_mask=gmask, grad_weight=gw, grad_bias=gb)
     fam = _dcn_family(shape)

@@ -8,6 +8,7 @@
 #include <atomic>
 
 #include "dcn_common.hpp"
+#include "dcn_pad.hpp"
 #include "sampling.hpp"
 
 namespace mv {
@@ -322,12 +323,47 @@ int mv_dcn3d_output_dims(const mv_dcn3d_shape *shape, int *out_d, int *out_h, in
   return MV_OK;
 }
 
+// Layers whose channel counts the matrix-core kernels do not take run as the next larger layer
+// that they do (dcn_pad.hip).  Workspace of such a call: padded copies first, then the workspace
+// of the padded layer.
+static size_t align256p(size_t v) { return (v + 255) / 256 * 256; }
+struct PadLayout {
+  size_t x, w, b, y, gy, inner, total;   // byte offsets (x, w, b / gy, y: padded copies; y only when Cout is padded)
+  bool x_padded, y_padded;
+};
+static PadLayout pad_layout(const DcnDims &s, const DcnPad &pad, int dtype, bool backward) {
+  const size_t es = dtype == MV_F32 ? 4 : 2;
+  const DcnDims &p = pad.p;
+  PadLayout l;
+  l.x_padded = p.Cin != s.Cin; l.y_padded = p.Cout != s.Cout;
+  size_t at = 0;
+  l.x = at; at += l.x_padded ? align256p(static_cast<size_t>(p.B) * p.Cin * p.P * es) : 0;
+  l.w = at; at += align256p(static_cast<size_t>(p.Cout) * p.cpg * p.K * es);
+  l.b = at; at += align256p(static_cast<size_t>(p.Cout) * es);
+  l.y = at; at += (!backward && l.y_padded) ? align256p(static_cast<size_t>(p.B) * p.Cout * p.Q * es) : 0;
+  l.gy = at; at += (backward && l.y_padded) ? align256p(static_cast<size_t>(p.B) * p.Cout * p.Q * es) : 0;
+  l.inner = at;
+  at += backward ? dcn_mfma_backward_workspace_bytes(p, dtype) : dcn_mfma_workspace_bytes(p, dtype);
+  l.total = at;
+  return l;
+}
+static bool forward_pads(const DcnDims &s, int dtype, DcnPad &pad) {
+  return !dcn_mfma_supported(s, dtype) && dcn_pad_plan(s, dtype, pad) && dcn_mfma_supported(pad.p, dtype);
+}
+static bool backward_pads(const DcnDims &s, int dtype, DcnPad &pad) {
+  return !dcn_mfma_backward_supported(s, dtype) && dcn_pad_plan(s, dtype, pad) && dcn_mfma_backward_supported(pad.p, dtype);
+}
+
 static size_t forward_workspace(const DcnDims &s, int dtype) {
-  return dcn_mfma_supported(s, dtype) ? dcn_mfma_workspace_bytes(s, dtype) : 0;
+  if (dcn_mfma_supported(s, dtype)) return dcn_mfma_workspace_bytes(s, dtype);
+  DcnPad pad;
+  return forward_pads(s, dtype, pad) ? pad_layout(s, pad, dtype, false).total : 0;
 }
 
 static size_t backward_workspace(const DcnDims &s, int dtype) {
   if (dcn_mfma_backward_supported(s, dtype)) return dcn_mfma_backward_workspace_bytes(s, dtype);
+  DcnPad pad;
+  if (backward_pads(s, dtype, pad)) return pad_layout(s, pad, dtype, true).total;
   if (dtype != MV_F16 && dtype != MV_BF16) return 0;
   // fp32 accumulators for grad_input, grad_weight, grad_bias
   const size_t n = static_cast<size_t>(s.B) * s.Cin * s.P + static_cast<size_t>(s.Cout) * s.cpg * s.K + s.Cout;
@@ -342,6 +378,30 @@ static int dcn_forward_any(const void *input, const void *offset, const void *ma
   if (dcn_mfma_supported(s, dtype)) {
     MV_REQUIRE(workspace, "this shape needs a workspace of mv_dcn3d_forward_workspace_bytes()");
     return dcn_mfma_forward(input, offset, mask, weight, bias, output, s, dtype, workspace, hs);
+  }
+  DcnPad pad;
+  if (forward_pads(s, dtype, pad)) {
+    MV_REQUIRE(workspace, "this shape needs a workspace of mv_dcn3d_forward_workspace_bytes()");
+    const PadLayout l = pad_layout(s, pad, dtype, false);
+    const int es = dtype == MV_F32 ? 4 : 2;
+    char *ws = static_cast<char *>(workspace);
+    const void *xp = input;
+    int st = MV_OK;
+    if (l.x_padded) {
+      st = dcn_pad_channels(input, ws + l.x, s.B, s.Cin, s.P, pad.unit, pad.unit_p, es, hs);
+      if (st) return st;
+      xp = ws + l.x;
+    }
+    st = dcn_pad_weight(weight, ws + l.w, s, pad, es, hs);
+    if (st) return st;
+    if (bias) {
+      st = dcn_pad_channels(bias, ws + l.b, 1, s.Cout, 1, s.opg, pad.p.opg, es, hs);
+      if (st) return st;
+    }
+    void *yp = l.y_padded ? static_cast<void *>(ws + l.y) : output;
+    st = dcn_mfma_forward(xp, offset, mask, ws + l.w, bias ? ws + l.b : nullptr, yp, pad.p, dtype, ws + l.inner, hs);
+    if (st || !l.y_padded) return st;
+    return dcn_unpad_channels(yp, output, s.B, s.Cout, s.Q, s.opg, pad.p.opg, es, hs);
   }
   const long qb = (s.Q + kDcnThreads - 1) / kDcnThreads;
   const long yb = static_cast<long>(s.groups) * ((s.opg + kOutTile - 1) / kOutTile);
@@ -385,9 +445,48 @@ static int dcn_backward_any(const void *input, const void *offset, const void *m
   MV_REQUIRE((mask == nullptr) == (grad_mask == nullptr) || grad_mask == nullptr,
              "grad_mask given without mask");
   const bool narrow = dtype == MV_F16 || dtype == MV_BF16;
-  MV_REQUIRE((!narrow && !dcn_mfma_backward_supported(s, dtype)) || workspace,
+  DcnPad pad;
+  const bool padded = backward_pads(s, dtype, pad);
+  MV_REQUIRE((!narrow && !dcn_mfma_backward_supported(s, dtype) && !padded) || workspace,
              "this backward needs a workspace of mv_dcn3d_backward_workspace_bytes()");
   hipStream_t hs = static_cast<hipStream_t>(stream);
+  if (padded) {
+    const PadLayout l = pad_layout(s, pad, dtype, true);
+    const int es = dtype == MV_F32 ? 4 : 2;
+    char *wsb = static_cast<char *>(workspace);
+    const void *xp = input, *gyp = grad_output;
+    if (l.x_padded) {
+      st = dcn_pad_channels(input, wsb + l.x, s.B, s.Cin, s.P, pad.unit, pad.unit_p, es, hs);
+      if (st) return st;
+      xp = wsb + l.x;
+    }
+    st = dcn_pad_weight(weight, wsb + l.w, s, pad, es, hs);
+    if (st) return st;
+    if (l.y_padded) {
+      st = dcn_pad_channels(grad_output, wsb + l.gy, s.B, s.Cout, s.Q, s.opg, pad.p.opg, es, hs);
+      if (st) return st;
+      gyp = wsb + l.gy;
+    }
+    float *gx32, *gw32, *gb32;
+    st = dcn_mfma_backward(xp, offset, mask, wsb + l.w, gyp, grad_offset, grad_mask, pad.p, dtype, wsb + l.inner,
+                           &gx32, &gw32, &gb32, hs);
+    if (st) return st;
+    st = dcn_planar_add_padded(gx32, grad_input, s, pad, dtype, hs);
+    if (st) return st;
+    MV_DISPATCH(dtype, {
+      if (sizeof(T) <= 4) {
+        if (grad_bias) {   // from the real output gradient, into the (zeroed) accumulator of the padded layer
+          hipLaunchKernelGGL((dcn_backward_bias_kernel<T, float>), dim3(s.Cout, s.B, static_cast<unsigned>((s.Q + kBiasSlab - 1) / kBiasSlab)), dim3(256), 0, hs,
+                             static_cast<const T *>(grad_output), gb32, s);
+          hipLaunchKernelGGL((dcn_add_from_f32_kernel<T>), dim3(1), dim3(256), 0, hs,
+                             static_cast<T *>(grad_bias), gb32, static_cast<long>(s.Cout));
+        }
+      }
+    });
+    st = dcn_weight_add_padded(gw32, grad_weight, nullptr, nullptr, s, pad, dtype, hs);
+    if (st) return st;
+    return check_launch("dcn3d backward (padded channels)");
+  }
   const long n_gx = static_cast<long>(s.B) * s.Cin * s.P, n_gw = static_cast<long>(s.Cout) * s.cpg * s.K;
   float *ws = static_cast<float *>(workspace);
   if (dcn_mfma_backward_supported(s, dtype)) {

@@ -496,15 +496,18 @@ def test_general_deform_vs_oracle(ops, oracle, dtype, order):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("cin,cout,dg,modulated", [(24, 40, 2, True), (16, 16, 1, True), (48, 24, 1, False)])
 def test_channel_counts_padded_for_the_matrix_cores(ops, oracle, dtype, cin, cout, dg, modulated):
-    """Layers of one weight group whose channel counts are no multiples of 32 run the matrix-core
-    kernels on zero-padded copies (the shim pads and slices): all outputs and gradients as without."""
+    """Layers whose channel counts are no multiples of 32 run the matrix-core kernels on zero-padded
+    copies made inside the library: all outputs and gradients as without."""
     from medvision_amd.ops.deform_conv_3d import deform_conv
     from medvision_amd.ops.modulated_deform_conv_3d import modulated_deform_conv
     from medvision_amd import _C, _lib
     g = wl.gen(500 + cin + cout)
     x, off, mask, w, b = wl.dcn_inputs(g, 2, cin, cout, (5, 8, 9), 3, dg, 1, dtype, 1, 1, 1, modulated)
+    import ctypes
     shape = _lib.DcnShape(2, cin, 5, 8, 9, cout, 3, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, dg)
-    assert _C._dcn_pad_plan(x.to(DEV), w.to(DEV), shape) is not None
+    code = _lib.DTYPES[dtype]
+    assert _lib.load().mv_dcn3d_forward_workspace_bytes(ctypes.byref(shape), code) > 0    # padded copies + layouts
+    assert _lib.load().mv_dcn3d_backward_workspace_bytes(ctypes.byref(shape), code) > 0
     xs, offs, ms, ws, bs = [None if t is None else t.to(DEV).requires_grad_(True) for t in (x, off, mask, w, b)]
     if modulated:
         y = modulated_deform_conv(xs, offs, ms, ws, bs, 1, 1, 1, 1, dg)
@@ -521,3 +524,100 @@ def test_channel_counts_padded_for_the_matrix_cores(ops, oracle, dtype, cin, cou
     assert_close(bs.grad, gb, tol, "grad bias")
     if modulated:
         assert_close(ms.grad, gm, tol, "grad mask")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("cin,cout,groups,dg,modulated", [
+    (24, 40, 1, 1, True), (40, 24, 2, 1, True), (48, 48, 2, 2, False), (48, 80, 2, 4, True), (24, 64, 1, 3, False)])
+def test_raw_abi_with_any_channel_count(oracle, dtype, cin, cout, groups, dg, modulated):
+    """mv_dcn3d_forward / mv_dcn3d_backward called straight through ctypes (no shim in between) with
+    channel counts that are no multiples of 32, several weight groups and deformable groups that
+    nest either way: results against the oracle, and on the matrix-core kernels (timed against a
+    bound the general kernels miss by an order of magnitude)."""
+    import ctypes
+    from medvision_amd import _lib
+    lib = _lib.load()
+    g = wl.gen(900 + cin + cout + groups + dg)
+    size = (12, 16, 24)
+    x, off, mask, w, b = wl.dcn_inputs(g, 2, cin, cout, size, 3, dg, groups, dtype, 1, 1, 1, modulated)
+    # An offset far below the rounding of the coordinate it is added to (4 - 6e-8) puts the sample ON a
+    # voxel in the kernels' fp32 positions and just below it in the oracle's fp64 ones: the derivative
+    # with respect to the offset jumps there, and either side is right.  Keep the draws off that case.
+    off[off.abs() < 1e-4] = 0
+    shape = _lib.DcnShape(2, cin, *size, cout, 3, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, groups, dg)
+    code = _lib.DTYPES[dtype]
+    xs, offs, ms, ws, bs = _to(DEV, x, off, mask, w, b)
+    y = torch.full((2, cout, *size), float("nan"), dtype=dtype, device=DEV)
+    nf = lib.mv_dcn3d_forward_workspace_bytes(ctypes.byref(shape), code)
+    assert nf > 0
+    wsf = torch.empty(nf, dtype=torch.uint8, device=DEV)
+    stream = _lib.stream_of(xs)
+
+    def forward():
+        _lib.check(lib.mv_dcn3d_forward(_lib.ptr(xs), _lib.ptr(offs), _lib.ptr(ms), _lib.ptr(ws), _lib.ptr(bs), _lib.ptr(y),
+                                        ctypes.byref(shape), code, _lib.ptr(wsf), stream))
+    forward()
+    assert_close(y, oracle.dcn3d_forward(x, off, mask, w, b, 1, 1, 1, groups, dg), FWD_TOL[dtype], "forward")
+    gy = torch.randn(y.shape, generator=g).to(dtype)
+    gys = gy.to(DEV)
+    gi, goff, gw, gb = torch.zeros_like(xs), torch.zeros_like(offs), torch.zeros_like(ws), torch.zeros_like(bs)
+    gm = torch.zeros_like(ms) if modulated else None
+    nb = lib.mv_dcn3d_backward_workspace_bytes(ctypes.byref(shape), code)
+    assert nb > 0
+    wsb = torch.empty(nb, dtype=torch.uint8, device=DEV)
+
+    def backward():
+        _lib.check(lib.mv_dcn3d_backward(_lib.ptr(xs), _lib.ptr(offs), _lib.ptr(ms), _lib.ptr(ws), _lib.ptr(gys), _lib.ptr(gi),
+                                         _lib.ptr(goff), _lib.ptr(gm), _lib.ptr(gw), _lib.ptr(gb), ctypes.byref(shape), code,
+                                         _lib.ptr(wsb), stream))
+    backward()
+    want = oracle.dcn3d_backward(x, off, mask, w, gy, True, 1, 1, 1, groups, dg)
+    tol = BWD_TOL[dtype]
+    assert_close(gi, want[0], tol, "grad input")
+    assert_close(goff, want[1], tol, "grad offset")
+    assert_close(gw, want[3], tol, "grad weight")
+    assert_close(gb, want[4], tol, "grad bias")
+    if modulated:
+        assert_close(gm, want[2], tol, "grad mask")
+    # the gradients accumulate: a second call doubles input / weight / bias gradients
+    backward()
+    assert_close(gi, 2 * want[0], tol, "grad input accumulates")
+    assert_close(gw, 2 * want[3], tol, "grad weight accumulates")
+    # timing: against the next larger layer that needs no padding (the layer the library runs inside);
+    # the general kernels are 10 - 50 times slower than that
+    unit = min(cin // groups, cin // dg)
+    cin_n, cout_n = cin // unit * (-(-unit // 32) * 32), groups * (-(-(cout // groups) // 32) * 32)
+    xn, offn, mn, wn, bn = _to(DEV, *wl.dcn_inputs(g, 2, cin_n, cout_n, size, 3, dg, groups, dtype, 1, 1, 1, modulated))
+    shape_n = _lib.DcnShape(2, cin_n, *size, cout_n, 3, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, groups, dg)
+    yn = torch.empty((2, cout_n, *size), dtype=dtype, device=DEV)
+    wsn = torch.empty(max(lib.mv_dcn3d_forward_workspace_bytes(ctypes.byref(shape_n), code),
+                          lib.mv_dcn3d_backward_workspace_bytes(ctypes.byref(shape_n), code)), dtype=torch.uint8, device=DEV)
+    gin, goffn, gwn, gbn = torch.zeros_like(xn), torch.zeros_like(offn), torch.zeros_like(wn), torch.zeros_like(bn)
+    gmn = torch.zeros_like(mn) if modulated else None
+
+    def forward_native():
+        _lib.check(lib.mv_dcn3d_forward(_lib.ptr(xn), _lib.ptr(offn), _lib.ptr(mn), _lib.ptr(wn), _lib.ptr(bn), _lib.ptr(yn),
+                                        ctypes.byref(shape_n), code, _lib.ptr(wsn), stream))
+
+    def backward_native():
+        _lib.check(lib.mv_dcn3d_backward(_lib.ptr(xn), _lib.ptr(offn), _lib.ptr(mn), _lib.ptr(wn), _lib.ptr(yn), _lib.ptr(gin),
+                                         _lib.ptr(goffn), _lib.ptr(gmn), _lib.ptr(gwn), _lib.ptr(gbn), ctypes.byref(shape_n),
+                                         code, _lib.ptr(wsn), stream))
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(10):
+            fn()
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) / 10
+
+    for fn, native in ((forward, forward_native), (backward, backward_native)):
+        ms_call, ms_native = timed(fn), timed(native)
+        print(f"\n{fn.__name__} {dtype} cin={cin} cout={cout} groups={groups} dg={dg}: {ms_call:.3f} ms, "
+              f"[{cin_n} -> {cout_n}] without padding {ms_native:.3f} ms")
+        assert ms_call < 2.5 * ms_native + 0.15, f"{fn.__name__} takes {ms_call:.3f} ms: not on the matrix-core kernels"
