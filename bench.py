@@ -181,6 +181,20 @@ def bench_other_configs(args):
     gi = torch.zeros_like(feat)
     ms, _ = _events_ms(lambda i: _C.roi_align_3d_backward(gy, rois, gi, 7, 7, 7, 0.25, 2, 1), 10, 2)
     res["config5_backward_fp16"] = {"ms": round(ms, 4), "gbps": round(nbytes / ms / 1e6, 1)}
+    del feat, out, gy, gi
+    # rotated detection head: 1000 rotated rois of 6 - 24 voxels x 64 channels x 7^3 cells, grid 2
+    g = wl.gen(9)
+    feat = torch.randn(2, 64, 48, 96, 96, generator=g).half().to(dev)
+    ctr = torch.rand(1000, 3, generator=g) * torch.tensor([96., 96., 48.])
+    ext = 6 + torch.rand(1000, 3, generator=g) * 18
+    ang = (torch.rand(1000, 3, generator=g) * 2 - 1) * math.radians(30)
+    rois = torch.cat([torch.randint(0, 2, (1000, 1), generator=g).float(), ctr, ext, ang], 1).to(dev)
+    out = torch.empty(1000, 64, 7, 7, 7, dtype=torch.float16, device=dev)
+    ms, _ = _events_ms(lambda i: _C.roi_align_rotated_3d_forward(feat, rois, out, 7, 7, 7, 1.0, 2, True, 1), 20, 3)
+    gy = torch.randn_like(out)
+    gi = torch.zeros_like(feat)
+    bms, _ = _events_ms(lambda i: _C.roi_align_rotated_3d_backward(gy, rois, gi, 7, 7, 7, 1.0, 2, True, 1), 10, 2)
+    res["rotated_head_1000x64x7^3_fp16"] = {"forward_ms": round(ms, 4), "backward_ms": round(bms, 4)}
     return res
 
 

@@ -136,6 +136,10 @@ int roi_pool_backward(const void *grad_output, const void *rois, void *acc, int 
                       const RoiProblem &p, hipStream_t s, bool channels_last);
 bool roi_pool_applies(int dtype, const RoiProblem &p);
 // roi_gather_backward.hip: atomic-free backward for resampling-sized problems; -1 when not applicable
+// roi_box.hip: backward of small outputs that the pooled kernels do not take (rotated boxes, large
+// grids), one workgroup per (roi, channel group) with LDS tiles of the source boxes; -1 when not applicable
+int roi_box_backward(const void *grad_output, const void *rois, float *acc, int dtype, const RoiProblem &p, hipStream_t s);
+
 int roi_backward_gather(const void *grad_output, const void *rois, void *grad_input, int dtype,
                         const RoiProblem &p, hipStream_t s);
 // dcn3d_mfma_backward.hip: dst [B, C, P] += src [B, P, C] fp32
@@ -244,12 +248,14 @@ int roi_backward(const void *grad_output, const void *rois, void *grad_input, in
   if (pooled == 0 && channels_last)
     return planar_add_f32(static_cast<const float *>(workspace), grad_input, batch, channels,
                           static_cast<long>(depth) * height * width, dtype, s);
+  const int boxed = pooled < 0 ? roi_box_backward(grad_output, rois, static_cast<float *>(narrow ? workspace : grad_input), dtype, p, s) : -1;
+  if (boxed > 0) return boxed;
   MV_DISPATCH(dtype, {
     using RT = typename std::conditional<std::is_same<T, double>::value, double, float>::type;
     using G = typename std::conditional<(sizeof(T) == 2), float, T>::type;
     G *acc = narrow ? static_cast<G *>(workspace) : static_cast<G *>(grad_input);
-    if (pooled == 0) {
-      // gradient already accumulated by the pooled kernel
+    if (pooled == 0 || boxed == 0) {
+      // gradient already accumulated by the pooled / box kernel
     } else if (rotated)
       hipLaunchKernelGGL((roi_backward_kernel<T, G, RT, true>), grid, block, 0, s,
                          static_cast<const T *>(grad_output), static_cast<const RT *>(rois), acc, p);

@@ -1,0 +1,373 @@
+// RoIAlign / RoIAlignRotated BACKWARD for small outputs per roi (detection heads: 7^3, 14^2 ... cells)
+// that the separable pooled kernels do not take: rotated boxes, sampling grids above 4, heads of more
+// than 1024 cells.  Same results as the reference's one-thread-per-output kernel with one atomicAdd per
+// sample corner (csrc/cuda/roi_align_rotated_3d_cuda_kernel.cuh:124-265 and the 2-D twin).
+//
+// A workgroup owns (one roi, a group of channels).  The roi's geometry (fp64) is worked out once; its
+// output cells are taken in blocks small enough for the axis-aligned box of source voxels that a
+// block's samples touch to fit an LDS tile of 32-bit FIXED-POINT sums (an LDS fp32 atomic retires one
+// lane at a time): every sample adds weight * grad_output / count to the <= 8 voxels it touches, and
+// the tile's non-zero sums then go to the fp32 gradient buffer as one atomic per voxel with lanes along
+// x (one request per 64-byte sector) instead of one scattered atomic per sample corner.  The tile
+// holds as many of the workgroup's channels side by side as fit, so a sample's taps are worked out
+// once for all of them.  Scale per (block, channel): max |grad_output| / count < 2^e is mapped to 2^t
+// quanta, t = 30 - ceil(log2(samples that can reach one voxel)); a term is rounded by at most
+// 2^-(t+1) of that bound.  Rois with t < 20 (fp32 tensors; 12 for 16-bit ones: boxes of about a voxel,
+// where thousands of samples meet), blocks of one cell whose box still does not fit, and channels whose
+// gradient holds a NaN or an infinity add per sample, as the general kernel does, inside the same launch.
+// Sample coordinates, tap decisions and the void rule are those of the general kernels (sampling.hpp,
+// fp64).
+//
+// (The forward pass of the same problems stays on the general kernel: copying a block's box to LDS was
+// measured slower -- rotated rois of 6 - 24 voxels read a voxel of the box less than once -- and so was
+// sharing a sample's taps between channels with the samples of a cell in neighbouring lanes.)
+#include "common.hpp"
+#include "roi_geometry.hpp"
+#include "sampling.hpp"
+
+namespace mv {
+
+constexpr int kBoxThreads = 256;
+constexpr int kBoxLds = 48 * 1024;   // three workgroups per compute unit
+
+// The roi's output cells are worked through in blocks of blk[0] x blk[1] x blk[2] cells, small enough for
+// the axis-aligned box of source voxels that a block's samples touch (n[0] x n[1] x n[2], the same for
+// every block of the roi) to fit the tile.
+struct BoxPlan {
+  int n[3], blk[3];
+  int mode;        // 0: no sample of the roi reads or writes anything, 1: boxes in LDS, 2: per-sample path
+  int term_bits;   // backward: binary digits of a term below the channel's bound
+  double reach[3]; // half the extent of a block's samples along each source axis (with a margin)
+};
+
+// One thread: the block shape and the box extent.
+__device__ inline void plan_box(BoxPlan &b, const RoiGeom &g, const RoiProblem &p, int cap_voxels, int min_term_bits) {
+  const int cells[3] = {p.ow, p.oh, p.od}, size[3] = {p.W, p.H, p.D};
+  bool empty = g.batch < 0 || g.grid[0] <= 0 || g.grid[1] <= 0 || (p.ndim == 3 && g.grid[2] <= 0);
+  // the whole roi: void when its samples' bounding box lies outside [-1, size] on some axis
+  for (int a = 0; a < p.ndim && !empty; a++) {
+    double c = g.centre[a], reach = 0.0;
+    for (int j = 0; j < p.ndim; j++) {
+      const double first = local_coord(g, j, 0, 0), last = local_coord(g, j, cells[j] - 1, g.grid[j] - 1);
+      c += g.rot[3 * a + j] * 0.5 * (first + last);
+      reach += fabs(g.rot[3 * a + j] * 0.5 * (last - first));
+    }
+    const double rmin = c - reach - 1e-6, rmax = c + reach + 1e-6;
+    if (rmax < -1.0 || rmin > static_cast<double>(size[a]) || !(rmin == rmin) || !(rmax == rmax)) empty = true;
+  }
+  for (int j = 0; j < 3; j++) { b.blk[j] = j < p.ndim ? cells[j] : 1; b.n[j] = 1; b.reach[j] = 0.0; }
+  bool fits = false;
+  for (int round = 0; round < 40 && !empty; round++) {
+    double half[3] = {0.0, 0.0, 0.0};
+    for (int j = 0; j < p.ndim; j++) half[j] = 0.5 * ((b.blk[j] - 1) * g.bin[j] + (g.grid[j] - 1) * g.sub[j]);
+    long voxels = 1;
+    for (int a = 0; a < p.ndim; a++) {
+      double reach = 1e-6;   // (wider than the rounding of the per-sample arithmetic, which evaluates the same affine map)
+      for (int j = 0; j < p.ndim; j++) reach += fabs(g.rot[3 * a + j] * half[j]);
+      b.reach[a] = reach;
+      // integers in [floor(c - reach), floor(c + reach) + 1]: at most floor(2 reach) + 3
+      b.n[a] = static_cast<int>(fmin(floor(2.0 * reach) + 3.0, static_cast<double>(size[a])));
+      voxels *= b.n[a];
+    }
+    if (voxels <= cap_voxels) { fits = true; break; }
+    int widest = -1;
+    for (int j = 0; j < p.ndim; j++)
+      if (b.blk[j] > 1 && (widest < 0 || half[j] > half[widest])) widest = j;
+    if (widest < 0) break;
+    b.blk[widest] = (b.blk[widest] + 1) / 2;
+  }
+  // samples that can reach one voxel: those within a ball of radius sqrt(3) on the lattice of spacing sub
+  long terms = 1;
+  for (int j = 0; j < p.ndim; j++) {
+    const double along = static_cast<double>(cells[j]) * g.grid[j];
+    terms *= static_cast<long>(fmin(3.4642 / fmax(g.sub[j], 1e-9) + 1.0, fmax(along, 1.0)));
+  }
+  int bits = 0;
+  while ((1L << bits) < terms && bits < 40) bits++;
+  b.term_bits = 30 - bits;
+  b.mode = empty ? 0 : ((fits && b.term_bits >= min_term_bits) ? 1 : 2);
+}
+
+// A block of cells: its first cell and cell counts per axis, and where its box starts in the volume.
+struct BoxBlock {
+  int c0[3], cnt[3], lo[3];
+  int cells;
+};
+__device__ __forceinline__ BoxBlock box_block(const RoiGeom &g, const RoiProblem &p, const BoxPlan &b, int block) {
+  const int cells[3] = {p.ow, p.oh, p.od}, size[3] = {p.W, p.H, p.D};
+  const int nbx = (cells[0] + b.blk[0] - 1) / b.blk[0], nby = (cells[1] + b.blk[1] - 1) / b.blk[1];
+  const int idx[3] = {block % nbx, (block / nbx) % nby, block / (nbx * nby)};
+  BoxBlock k;
+  double mid[3] = {0.0, 0.0, 0.0};
+  k.cells = 1;
+#pragma unroll
+  for (int j = 0; j < 3; j++) {
+    k.c0[j] = idx[j] * b.blk[j];
+    k.cnt[j] = min(b.blk[j], cells[j] - k.c0[j]);
+    k.cells *= k.cnt[j];
+    if (j < p.ndim) mid[j] = 0.5 * (local_coord(g, j, k.c0[j], 0) + local_coord(g, j, k.c0[j] + k.cnt[j] - 1, g.grid[j] - 1));
+  }
+#pragma unroll
+  for (int a = 0; a < 3; a++) {
+    k.lo[a] = 0;
+    if (a >= p.ndim) continue;
+    double c = g.centre[a];
+#pragma unroll
+    for (int j = 0; j < 3; j++)
+      if (j < p.ndim) c += g.rot[3 * a + j] * mid[j];
+    const int l = static_cast<int>(fmin(floor(fmax(c - b.reach[a], 0.0)), static_cast<double>(size[a] - 1)));
+    k.lo[a] = max(min(l, size[a] - b.n[a]), 0);   // (the box stays inside the volume: n <= size)
+  }
+  return k;
+}
+__device__ __forceinline__ int box_blocks(const RoiProblem &p, const BoxPlan &b) {
+  return ((p.ow + b.blk[0] - 1) / b.blk[0]) * ((p.oh + b.blk[1] - 1) / b.blk[1]) * ((p.od + b.blk[2] - 1) / b.blk[2]);
+}
+// cell `i` of a block as a cell of the roi
+__device__ __forceinline__ unsigned block_cell(const RoiProblem &p, const BoxBlock &k, unsigned i) {
+  const unsigned bx = i % k.cnt[0], t = i / k.cnt[0], by = t % k.cnt[1], bz = t / k.cnt[1];
+  return ((k.c0[2] + bz) * p.oh + (k.c0[1] + by)) * p.ow + (k.c0[0] + bx);
+}
+
+// The workgroup's geometry record as wave-uniform values: read once from LDS and moved to scalar
+// registers, so that the sample loops below keep no per-lane copy of its ~30 doubles.
+__device__ __forceinline__ double uniform_f64(double v) {
+  return __hiloint2double(__builtin_amdgcn_readfirstlane(__double2hiint(v)), __builtin_amdgcn_readfirstlane(__double2loint(v)));
+}
+__device__ __forceinline__ RoiGeom uniform_geom(const RoiGeom &shared) {
+  RoiGeom u;
+#pragma unroll
+  for (int i = 0; i < 9; i++) u.rot[i] = uniform_f64(shared.rot[i]);
+#pragma unroll
+  for (int a = 0; a < 3; a++) {
+    u.centre[a] = uniform_f64(shared.centre[a]); u.start[a] = uniform_f64(shared.start[a]);
+    u.bin[a] = uniform_f64(shared.bin[a]); u.sub[a] = uniform_f64(shared.sub[a]);
+    u.grid[a] = __builtin_amdgcn_readfirstlane(shared.grid[a]);
+  }
+  u.batch = __builtin_amdgcn_readfirstlane(shared.batch);
+  u.count = __builtin_amdgcn_readfirstlane(shared.count);
+  return u;
+}
+__device__ __forceinline__ BoxPlan uniform_plan(const BoxPlan &shared) {
+  BoxPlan u;
+#pragma unroll
+  for (int a = 0; a < 3; a++) {
+    u.n[a] = __builtin_amdgcn_readfirstlane(shared.n[a]);
+    u.blk[a] = __builtin_amdgcn_readfirstlane(shared.blk[a]);
+    u.reach[a] = uniform_f64(shared.reach[a]);
+  }
+  u.mode = __builtin_amdgcn_readfirstlane(shared.mode);
+  u.term_bits = __builtin_amdgcn_readfirstlane(shared.term_bits);
+  return u;
+}
+
+// The taps of sub-sample `sub` (z, y, x order) of output cell `cell`.  Returns false for a void sample.
+struct BoxTaps {
+  int xi[2], yi[2], zi[2];
+  float fx, fy, fz;
+  int cell;
+};
+template <bool ROT>
+__device__ __forceinline__ bool box_taps(const RoiGeom &g, const RoiProblem &p, unsigned cell, unsigned sub, BoxTaps &t) {
+  const unsigned pw = cell % p.ow, t1 = cell / p.ow, ph = t1 % p.oh, pd = t1 / p.oh;
+  const unsigned ix = sub % g.grid[0], t2 = sub / g.grid[0], iy = t2 % g.grid[1], iz = t2 / g.grid[1];
+  const double x = local_coord(g, 0, pw, ix), y = local_coord(g, 1, ph, iy);
+  const double z = p.ndim == 3 ? local_coord(g, 2, pd, iz) : 0.0;
+  double rx = x, ry = y, rz = z;
+  if (ROT) {
+    rx = g.rot[0] * x + g.rot[1] * y + g.rot[2] * z + g.centre[0];
+    ry = g.rot[3] * x + g.rot[4] * y + g.rot[5] * z + g.centre[1];
+    rz = p.ndim == 3 ? g.rot[6] * x + g.rot[7] * y + g.rot[8] * z + g.centre[2] : 0.0;
+  }
+  t.cell = static_cast<int>(cell);
+  return clamped_tap<float>(rz, p.D, t.zi[0], t.zi[1], t.fz, p.order) && clamped_tap<float>(ry, p.H, t.yi[0], t.yi[1], t.fy, p.order) &&
+         clamped_tap<float>(rx, p.W, t.xi[0], t.xi[1], t.fx, p.order);
+}
+
+// A sample's taps relative to the box: offset of the low corner, the steps to the high taps (0 where
+// they collapse onto the low ones at the volume's upper border), the eight weights.
+struct BoxSample {
+  int at;        // >= 0: inside the box; -1: void; -2: touches voxels beyond the box
+  int dx, dy, dz;
+  float w[8];    // z-major corner order
+};
+template <bool ROT>
+__device__ __forceinline__ BoxSample box_sample(const RoiGeom &g, const RoiProblem &p, const BoxPlan &b, const int (&lo)[3],
+                                                unsigned cell, unsigned sub, BoxTaps &t) {
+  BoxSample k;
+  k.at = -1; k.dx = k.dy = k.dz = 0;
+  if (!box_taps<ROT>(g, p, cell, sub, t)) return k;
+  const float wx[2] = {1.f - t.fx, t.fx}, wy[2] = {1.f - t.fy, t.fy}, wz[2] = {1.f - t.fz, t.fz};
+#pragma unroll
+  for (int m = 0; m < 8; m++) k.w[m] = wz[m >> 2] * wy[(m >> 1) & 1] * wx[m & 1];
+  const unsigned bx0 = t.xi[0] - lo[0], bx1 = t.xi[1] - lo[0], by0 = t.yi[0] - lo[1], by1 = t.yi[1] - lo[1];
+  const unsigned bz0 = t.zi[0] - lo[2], bz1 = t.zi[1] - lo[2];
+  const bool inside = b.mode == 1 && max(bx0, bx1) < static_cast<unsigned>(b.n[0]) && max(by0, by1) < static_cast<unsigned>(b.n[1]) &&
+                      max(bz0, bz1) < static_cast<unsigned>(b.n[2]);
+  if (!inside) { k.at = -2; return k; }
+  k.at = static_cast<int>((bz0 * b.n[1] + by0) * b.n[0] + bx0);
+  k.dx = t.xi[1] != t.xi[0] ? 1 : 0;
+  k.dy = t.yi[1] != t.yi[0] ? b.n[0] : 0;
+  k.dz = t.zi[1] != t.zi[0] ? b.n[0] * b.n[1] : 0;
+  return k;
+}
+
+constexpr int kBoxChannels = 16;   // channels a workgroup's tile holds at most (and a workgroup owns at most)
+
+// ---- backward ------------------------------------------------------------------------------------
+// `per_group` <= kBoxChannels channels per workgroup; the tile holds `cpt` = as many of them as fit
+// side by side, so a sample's taps are worked out once per cpt channels.
+template <typename T, bool ROT>
+__global__ __launch_bounds__(kBoxThreads, 3) void roi_box_backward_kernel(const T *__restrict__ gout,
+                                                                          const float *__restrict__ rois,
+                                                                          float *__restrict__ acc, const RoiProblem p,
+                                                                          const int per_group) {
+  __shared__ RoiGeom gs;
+  __shared__ double trig[6];
+  __shared__ BoxPlan plan;
+  __shared__ __attribute__((aligned(16))) int tile[kBoxLds / 4];
+  __shared__ unsigned bound[kBoxChannels];
+  const unsigned n = blockIdx.x;
+  build_geom_block(gs, trig, rois + static_cast<long>(n) * roi_columns(p.ndim, p.rotated), p);
+  // fixed-point sums only where a term keeps 20 binary digits below the channel's bound (fp32 tensors; 12
+  // for 16-bit ones): boxes of a voxel or less, where thousands of samples meet in one voxel, add per sample
+  if (threadIdx.x == 0) plan_box(plan, gs, p, kBoxLds / 4, sizeof(T) == 4 ? 20 : 12);
+  for (int i = threadIdx.x * 4; i < kBoxLds / 4; i += kBoxThreads * 4) *reinterpret_cast<int4 *>(tile + i) = int4{0, 0, 0, 0};
+  if (threadIdx.x < kBoxChannels) bound[threadIdx.x] = 0;
+  __syncthreads();
+  const BoxPlan b = uniform_plan(plan);
+  if (b.mode == 0) return;
+  const RoiGeom g = uniform_geom(gs);
+  const int cells = p.od * p.oh * p.ow;
+  const unsigned count = static_cast<unsigned>(g.count);
+  const long plane = static_cast<long>(p.D) * p.H * p.W;
+  const int c_first = blockIdx.y * per_group, c_end = min(c_first + per_group, p.C);
+  const float inv_count = 1.f / static_cast<float>(g.count);
+  const int count_shift = 31 - __clz(g.count);   // floor(log2 count): |g| / count < 2^(e - count_shift)
+  const int n0 = b.n[0], box = b.n[0] * b.n[1] * b.n[2];
+  const int cpt = b.mode == 1 ? min(per_group, (kBoxLds / 4) / box) : per_group;
+  const float inv_row = 1.f / static_cast<float>(n0), inv_rows = 1.f / static_cast<float>(b.n[1]), inv_box = 1.f / static_cast<float>(box);
+  const int blocks = box_blocks(p, b);
+  for (int block = 0; block < blocks; block++) {
+    const BoxBlock k = box_block(g, p, b, block);
+    for (int c0 = c_first; c0 < c_end; c0 += cpt) {
+      const int nc = min(cpt, c_end - c0);
+      const T *gsrc = gout + (static_cast<long>(n) * p.C + c0) * cells;
+      float *vol = acc + (static_cast<long>(g.batch) * p.C + c0) * plane;
+      // per channel the largest |grad_output| of the block as the bit pattern of a float (NaNs order above infinity)
+      for (int i = threadIdx.x; i < nc * k.cells; i += kBoxThreads) {
+        const int ch = i / k.cells;
+        atomicMax(&bound[ch], __float_as_uint(fabsf(static_cast<float>(load(gsrc + static_cast<long>(ch) * cells + block_cell(p, k, i - ch * k.cells))))));
+      }
+      __syncthreads();
+      // |term| <= max |g| / count < 2^(e - 126 - count_shift): quanta of 2^-term_bits of that power of two.
+      // A channel with a NaN or an infinity in its gradient takes the per-sample path.
+      auto channel_scale = [&](int ch, float &to_quanta) -> bool {
+        const unsigned bits = bound[ch];
+        const int ex = min(max(127 + 126 + count_shift + b.term_bits - static_cast<int>(bits >> 23), 1), 253);
+        to_quanta = __uint_as_float(static_cast<unsigned>(ex) << 23) * inv_count;
+        return bits < 0x7f800000u;
+      };
+      auto scatter = [&](unsigned cell, unsigned sub) {
+        BoxTaps t;
+        const BoxSample q = box_sample<ROT>(g, p, b, k.lo, cell, sub, t);
+        if (q.at == -1) return;
+        for (int ch = 0; ch < nc; ch++) {
+          const float gv = static_cast<float>(load(gsrc + static_cast<long>(ch) * cells + cell));
+          if (gv == 0.f) continue;
+          float to_quanta;
+          if (channel_scale(ch, to_quanta) && q.at >= 0) {
+            const float gq = gv * to_quanta;
+            int *cell0 = tile + ch * box + q.at;
+#pragma unroll
+            for (int m = 0; m < 8; m++) {
+              const int v = __float2int_rn(gq * q.w[m]);
+              if (v != 0)
+                __hip_atomic_fetch_add(cell0 + ((m >> 2) ? q.dz : 0) + (((m >> 1) & 1) ? q.dy : 0) + ((m & 1) ? q.dx : 0), v,
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+          } else {
+            const float top = gv * inv_count;
+            float *dst = vol + static_cast<long>(ch) * plane;
+#pragma unroll
+            for (int m = 0; m < 8; m++)
+              if (q.w[m] != 0.f)
+                atomic_add(dst + (static_cast<long>(t.zi[m >> 2]) * p.H + t.yi[(m >> 1) & 1]) * p.W + t.xi[m & 1], top * q.w[m]);
+          }
+        }
+      };
+      if (static_cast<long>(k.cells) * count < (1L << 31)) {
+        // sample s = cell * count + sub: neighbouring lanes take neighbouring samples
+        const unsigned total = static_cast<unsigned>(k.cells) * count;
+        for (unsigned s = threadIdx.x; s < total; s += kBoxThreads) scatter(block_cell(p, k, s / count), s % count);
+      } else {
+        for (unsigned i = threadIdx.x; i < static_cast<unsigned>(k.cells); i += kBoxThreads)
+          for (unsigned sub = 0; sub < count; sub++) scatter(block_cell(p, k, i), sub);
+      }
+      __syncthreads();
+      if (b.mode == 1) {
+        // lanes along the box's rows: neighbouring lanes add to neighbouring voxels of the buffer
+        for (int i = threadIdx.x; i < nc * box; i += kBoxThreads) {
+          const int q = tile[i];
+          if (q == 0) continue;
+          tile[i] = 0;
+          const int ch = static_cast<int>((static_cast<float>(i) + 0.5f) * inv_box), v = i - ch * box;
+          const int row = static_cast<int>((static_cast<float>(v) + 0.5f) * inv_row), bx = v - row * n0;
+          const int bz = static_cast<int>((static_cast<float>(row) + 0.5f) * inv_rows), by = row - bz * b.n[1];
+          const unsigned bits = bound[ch];
+          const int ex = min(max(127 + 126 + count_shift + b.term_bits - static_cast<int>(bits >> 23), 1), 253);
+          const float from_quanta = __uint_as_float(static_cast<unsigned>(254 - ex) << 23);
+          atomic_add(vol + static_cast<long>(ch) * plane + (static_cast<long>(bz + k.lo[2]) * p.H + (by + k.lo[1])) * p.W + (k.lo[0] + bx),
+                     static_cast<float>(q) * from_quanta);
+        }
+      }
+      __syncthreads();
+      if (threadIdx.x < kBoxChannels) bound[threadIdx.x] = 0;
+      __syncthreads();   // (the next pass takes its maxima behind this barrier)
+    }
+  }
+}
+
+// Small outputs per roi in 16- or 32-bit tensors, orders 0 / 1; what the tiled, gathering and pooled
+// backward kernels have not taken arrives here (rotated boxes, large grids, heads of more than 1024 cells).
+bool roi_box_applies(int dtype, const RoiProblem &p) {
+  if (dtype != MV_F16 && dtype != MV_BF16 && dtype != MV_F32) return false;
+  if (p.order != 0 && p.order != 1) return false;
+  const long cells = static_cast<long>(p.od) * p.oh * p.ow;
+  return cells <= 4096 && p.R <= 0x7fffffff && p.C >= 1;
+}
+
+// Channels per workgroup: the set-up (geometry, box, the samples' taps) is shared by them, so as many as
+// leave enough workgroups to fill the compute units three times over.
+static int box_channels_per_group(const RoiProblem &p) {
+  int per = kBoxChannels;
+  while (per > 1 && static_cast<long>(p.R) * ((p.C + per - 1) / per) < 3 * 768) per /= 2;
+  return per;
+}
+
+// `acc`: the fp32 buffer the gradient is added to (grad_input itself for fp32 tensors, the workspace for
+// 16-bit ones), laid out like grad_input.
+int roi_box_backward(const void *grad_output, const void *rois, float *acc, int dtype, const RoiProblem &p, hipStream_t s) {
+  if (!roi_box_applies(dtype, p)) return -1;
+  const int per = box_channels_per_group(p);
+  const long groups = (p.C + per - 1) / per;
+  if (groups > 65535) return -1;
+  const dim3 grid(p.R, static_cast<unsigned>(groups)), block(kBoxThreads);
+  const float *r = static_cast<const float *>(rois);
+#define MV_BOX_BACKWARD(TYPE)                                                                                              \
+  if (p.rotated)                                                                                                           \
+    hipLaunchKernelGGL((roi_box_backward_kernel<TYPE, true>), grid, block, 0, s, static_cast<const TYPE *>(grad_output), r, \
+                       acc, p, per);                                                                                       \
+  else                                                                                                                     \
+    hipLaunchKernelGGL((roi_box_backward_kernel<TYPE, false>), grid, block, 0, s, static_cast<const TYPE *>(grad_output), r, \
+                       acc, p, per)
+  switch (dtype) {
+    case MV_F32: MV_BOX_BACKWARD(float); break;
+    case MV_F16: MV_BOX_BACKWARD(__half); break;
+    default: MV_BOX_BACKWARD(__hip_bfloat16);
+  }
+#undef MV_BOX_BACKWARD
+  return check_launch("roi_box_backward_kernel");
+}
+
+}  // namespace mv

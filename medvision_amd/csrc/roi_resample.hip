@@ -251,7 +251,6 @@ __device__ inline void plan_item_lanes(const float *__restrict__ rois, const Roi
     if (item == kDone) {
       dst->mode = 4;
     } else {
-      const long rows = static_cast<long>(n1) * n2;
       // register staging: a pass copies `span` whole z-slices, one 16-byte group per lane
       int passes = 0;
       if (ps.vec > 0) {

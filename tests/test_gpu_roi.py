@@ -782,3 +782,50 @@ def test_config5_full_size_properties(ops):
         got = x.grad[b].double().sum(dim=(1, 2, 3))
         scale = float(gy[pick].double().abs().sum(dim=(0, 2, 3, 4)).max())
         assert float((got - want).abs().max()) <= 2e-3 * scale   # fp16 rounding of 1.8 M accumulated cells
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("ndim", [3, 2])
+def test_rotated_heads_backward_through_box_tiles(ops, oracle, dtype, ndim):
+    """Rotated rois with detection-head outputs (7^3 / 14^2 cells): the backward pass sums each block of
+    cells in an LDS tile of the source box.  Rois from a fraction of a voxel (thousands of samples in one
+    voxel: per-sample path) to half the volume (several blocks per roi), sticking out of the volume,
+    fixed and adaptive grids, more channels than a workgroup's tile holds, a NaN in one gradient."""
+    g = wl.gen(610 + ndim)
+    size = (20, 44, 52)[3 - ndim:]
+    out = (7, 7, 7) if ndim == 3 else (14, 14)
+    C = 21
+    feat = torch.randn(2, C, *size, generator=g).to(dtype)
+    xyz = torch.tensor(size[::-1], dtype=torch.float32)
+    n = 40
+    ctr = (torch.rand(n, ndim, generator=g) * 1.2 - 0.1) * xyz
+    ext = torch.exp(torch.rand(n, ndim, generator=g) * math.log(100.0)) * 0.3      # 0.3 .. 30 voxels
+    ext[:3] = xyz * 0.6
+    ang = (torch.rand(n, 3 if ndim == 3 else 1, generator=g) * 2 - 1) * math.radians(40)
+    rois = torch.cat([torch.randint(0, 2, (n, 1), generator=g).float(), ctr, ext, ang], 1)
+    for sr in (2, 0, 3):
+        x = feat.to(DEV).requires_grad_(True)
+        y = ops.RoIAlignRotated(out, 1.0, sr, True)(x, rois.to(DEV))
+        assert_close(y, oracle.roi_align_forward(feat, rois, out, 1.0, sr, True, 1, True), FWD_TOL[dtype], f"forward sr={sr}")
+        gy = torch.randn(y.shape, generator=g).to(dtype)
+        y.backward(gy.to(DEV))
+        want = oracle.roi_align_backward(gy, rois, feat.shape, 1.0, sr, True, 1, True)
+        assert_close(x.grad, want, BWD_TOL[dtype], f"backward sr={sr}")
+    # order 0 (a grid of one)
+    x = feat.to(DEV).requires_grad_(True)
+    y = ops.RoIAlignRotated(out, 1.0, 2, True)(x, rois.to(DEV), order=0)
+    gy = torch.randn(y.shape, generator=g).to(dtype)
+    y.backward(gy.to(DEV))
+    assert_close(x.grad, oracle.roi_align_backward(gy, rois, feat.shape, 1.0, 1, True, 0, True), BWD_TOL[dtype], "order 0")
+    # a NaN in one channel of one roi's gradient: that channel adds per sample, and the voxels its samples
+    # touch are NaN as in the oracle (roi 0 covers most of the volume: interior samples, no zero weights)
+    x = feat.to(DEV).requires_grad_(True)
+    y = ops.RoIAlignRotated(out, 1.0, 2, True)(x, rois.to(DEV))
+    gy = torch.randn(y.shape, generator=g).to(dtype)
+    gy[0, 3].view(-1)[gy[0, 3].numel() // 2] = float("nan")
+    y.backward(gy.to(DEV))
+    want = oracle.roi_align_backward(gy, rois, feat.shape, 1.0, 2, True, 1, True)
+    got = x.grad.cpu()
+    assert torch.isnan(want).any() and torch.equal(torch.isnan(got), torch.isnan(want))
+    ok = ~torch.isnan(want)
+    assert_close(got[ok], want[ok], BWD_TOL[dtype], "a NaN gradient")
