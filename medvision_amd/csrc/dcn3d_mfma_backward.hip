@@ -381,6 +381,284 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
   }
 }
 
+// ---- the data kernel with one POSITION per lane (layers that run the scatter kernel) --------------
+// The product is formed the other way round: A = weight fragments (rows = channels), B = gy (columns
+// = positions), so lane l holds position l % 32 and sixteen channels (16 * (l / 32) .. + 15 of the
+// 32-channel block, the fragment kernel orders the MFMA rows accordingly).  The taps stay in the
+// lane's registers, x at a corner arrives as the lane's own 16-byte loads (no LDS stage), and the
+// four sums over channels are serial adds with one exchange between the half-wavefronts per tap.
+// The column values pass through an LDS block laid out like the column buffer and leave as
+// 16-byte stores.  Corners the scatter kernel does not take are rare here; their channels go through
+// a [position][channel] LDS block so that an atomic instruction still adds 128 contiguous bytes:
+// the wavefront lists its far corners once per tap and walks the list two entries at a time.
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_weight_afragments32_kernel(const T *__restrict__ wt,
+                                                                      T *__restrict__ wa,
+                                                                      const DcnDims s) {
+  constexpr int PC = Mfma<T>::kPiece;
+  const int cblocks = s.cpg / 32, steps = s.opg / (2 * PC);
+  const long total = static_cast<long>(s.groups) * s.K * cblocks * steps * 64;
+  const long id = blockIdx.x * 256L + threadIdx.x;
+  if (id >= total) return;
+  const int lane = id % 64;
+  long r = id / 64;
+  const int st = r % steps; r /= steps;
+  const int cb = r % cblocks; r /= cblocks;
+  const int k = r % s.K;
+  const int g = static_cast<int>(r / s.K);
+  // accumulator register r of half h is MFMA row 8 * (r / 4) + 4 * h + r % 4: that row carries channel 16 * h + r
+  const int row = lane % 32, cl = cb * 32 + 16 * ((row / 4) % 2) + 4 * (row / 8) + row % 4;
+  const int o = g * s.opg + st * 2 * PC + (lane / 32) * PC;
+  for (int i = 0; i < PC; i++) wa[id * PC + i] = wt[(static_cast<long>(o + i) * s.cpg + cl) * s.K + k];
+}
+
+template <typename T, typename S>
+__global__ __launch_bounds__(256, 3) void dcn_backward_data_lanes_kernel(
+    const T *__restrict__ xt, const T *__restrict__ off, const T *__restrict__ mask,
+    const T *__restrict__ gyt, const T *__restrict__ wa, float *__restrict__ gxt,
+    T *__restrict__ goff, T *__restrict__ gmask, const DcnDims s, const unsigned *__restrict__ bounds,
+    T *__restrict__ col, const long qp) {
+  using M = Mfma<T>;
+  using P = typename std::conditional<(sizeof(T) == 2), float, double>::type;  // position type
+  constexpr int PC = M::kPiece, SL = 2 * PC, ES = sizeof(T);
+  constexpr int CH = 32 / ES, CHUNKS = 16 / CH;  // channels of a lane per pass: 32 bytes per corner
+  // LDS of a wavefront.  Gather stage: rows of 64 bytes (the two halves' 32 bytes of a corner) for 4
+  // corners x 32 positions, 80 bytes apart so that the 16-byte reads of 8 lanes cover all banks.
+  // The column block and the far corners' channels reuse the stage once x sits in registers; with
+  // two passes per block (fp32) the column block outlives a pass and lies behind the stage.
+  constexpr int kRow = 80, kStage = 4 * 32 * kRow;
+  constexpr int kColAt = CHUNKS > 1 ? kStage : 0, kFarAt = CHUNKS > 1 ? 0 : 4096;
+  constexpr int kListAt = kStage + (CHUNKS > 1 ? 32 * 32 * ES : 0), kTapsAt = kListAt + 256 * 8;
+  constexpr int kWaveBytes = kTapsAt + 32 * 32;
+  static_assert(32 * 32 * ES <= 4096 && 4096 + 32 * 33 * 4 <= kStage, "column block and far channels fit the stage");
+  __shared__ __attribute__((aligned(16))) unsigned char lds[4][kWaveBytes];
+  const int lane = threadIdx.x % kWave, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int n = lane % 32, h = lane / 32;
+  const long q0 = (static_cast<long>(xcd_contiguous(blockIdx.x, gridDim.x)) * 4 + wave) * 32;
+  if (q0 >= s.Q) return;  // whole wavefront idle (no workgroup barriers in this kernel)
+  const long q = q0 + n;
+  const bool live = q < s.Q;
+  const long qc = live ? q : s.Q - 1;
+  const int dgi = blockIdx.y, b = blockIdx.z;
+  const int ow = qc % s.Wo, oh = (qc / s.Wo) % s.Ho, od = qc / (static_cast<long>(s.Wo) * s.Ho);
+  const int bd = od * s.sd - s.pd, bh = oh * s.sh - s.ph, bw = ow * s.sw - s.pw;
+  const long bg = static_cast<long>(b) * s.dg + dgi;
+  const int cblocks = s.cpg / 32, steps = s.opg / SL;
+
+  const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T *>(xt + static_cast<long>(b) * s.P * s.Cin), 0, static_cast<int>(s.P * s.Cin * ES), kRsrcFlags);
+  const __amdgpu_buffer_rsrc_t gr = __builtin_amdgcn_make_buffer_rsrc(
+      gxt + static_cast<long>(b) * s.P * s.Cin, 0, static_cast<int>(s.P * s.Cin * 4), kRsrcFlags);
+  const unsigned cin2 = static_cast<unsigned>(s.Cin) * ES;
+  const T *gyrow = gyt + (static_cast<long>(b) * s.Q + qc) * s.Cout + h * PC;
+  const T *o = off + bg * s.nd * s.K * s.Q + qc;
+  const T *mk = mask ? mask + bg * s.K * s.Q + qc : nullptr;
+  unsigned char *const stg = lds[wave];
+  float *const fg = reinterpret_cast<float *>(stg + kFarAt);
+  T *const cs = reinterpret_cast<T *>(stg + kColAt);
+  uint2 *const fl = reinterpret_cast<uint2 *>(stg + kListAt);  // per far (position, corner): {offset in the gradient buffer | position, weight}
+  unsigned char *const tp = stg + kTapsAt;                     // the corners' byte offsets in x: [position][8]
+  const TileOrigin origin = tile_origin<S>(s, od / S::BD, oh / S::BH, ow / S::BW);
+  const bool split = scatter_scale(bounds, S::BD * S::BH * S::BW * s.K, mask != nullptr).valid;
+  // the gather fetches a voxel's 64 bytes with four adjacent lanes (one request instead of four):
+  // lane l fetches quarter l % 4 of the voxels of positions l / 4 and l / 4 + 16
+  const int gp = lane / 4, gq = lane % 4;
+  const unsigned gbyte = static_cast<unsigned>((gq / 2) * (16 * ES) + (gq % 2) * 16);
+  // grad_output of the lane's position does not change with the tap: kept when the deformable
+  // group lies in one weight group and the slices fit four registers each
+  const bool hoist = s.cpd <= s.cpg && steps <= 4;
+  u32x4 bkeep[4];
+#pragma unroll
+  for (int st = 0; st < 4; st++)
+    bkeep[st] = (hoist && live && st < steps)
+                    ? *reinterpret_cast<const u32x4 *>(gyrow + (dgi * s.cpd / s.cpg) * s.opg + st * SL)
+                    : u32x4{0u, 0u, 0u, 0u};
+
+  int ki = 0, kj = 0, kk = 0;
+  P fd, fh, fw;  // offsets and mask of the coming tap, loaded one tap ahead
+  dcn_offsets(s, o, fd, fh, fw);
+  float fm = mk ? load(mk) : 1.f;
+  for (int k = 0; k < s.K; k++) {
+    // ---- taps of (k, q0 + n), in the lane's registers ---------------------------------------------
+    const P pd = fd + static_cast<P>(bd + ki * s.dd), ph = fh + static_cast<P>(bh + kj * s.dh),
+            pw = fw + static_cast<P>(bw + kk * s.dw);
+    const float m = fm;
+    o += s.nd * s.Q;
+    if (mk) mk += s.Q;
+    if (++kk == s.kw) { kk = 0; if (++kj == s.kh) { kj = 0; ++ki; } }
+    if (k + 1 < s.K) {
+      dcn_offsets(s, o, fd, fh, fw);
+      if (mk) fm = load(mk);
+    }
+    CornerTaps t;  // byte offsets of the corners in x; kOob outside the volume
+    corner_taps<P>(s, pd, ph, pw, live, cin2, 0u, kOob, t);
+    int first;
+    const unsigned local = split ? tile_bits<S>(origin, static_cast<int>(floor(pd)), static_cast<int>(floor(ph)),
+                                             static_cast<int>(floor(pw)), first) : 0u;
+    unsigned farbits = 0;  // corners inside the volume that the scatter kernel does not sum
+#pragma unroll
+    for (int c = 0; c < 8; c++) farbits |= (t.at[c] != kOob && !((local >> c) & 1u)) ? 1u << c : 0u;
+    const float ld = t.ld, lh = t.lh, lw = t.lw;
+    if (h == 0) {
+      reinterpret_cast<u32x4 *>(tp + n * 32)[0] = u32x4{t.at[0], t.at[1], t.at[2], t.at[3]};
+      reinterpret_cast<u32x4 *>(tp + n * 32)[1] = u32x4{t.at[4], t.at[5], t.at[6], t.at[7]};
+    }
+    // the far corners of the wavefront's 32 positions, listed once per tap: a voxel's channels start
+    // at a multiple of 128 bytes, so the position fits below the offset.  Both half-wavefronts hold
+    // the same taps; the lower one writes.
+    int far_count = 0;
+    if (__ballot(farbits != 0) != 0) {
+      const float wd[2] = {1.f - ld, ld}, wh[2] = {1.f - lh, lh}, ww[2] = {1.f - lw, lw};
+#pragma unroll
+      for (int c = 0; c < 8; c++) {
+        const bool is_far = (farbits >> c) & 1u;
+        const unsigned owners = static_cast<unsigned>(__ballot(is_far));  // low 32 bits: the positions
+        if (is_far && h == 0)
+          fl[far_count + __builtin_amdgcn_mbcnt_lo(owners, 0u)] =
+              make_uint2(t.at[c] * (4u / ES) | static_cast<unsigned>(n),
+                         __float_as_uint(wd[c >> 2] * wh[(c >> 1) & 1] * ww[c & 1]));
+        far_count += __builtin_popcount(owners);
+      }
+    }
+    const bool any_far = far_count != 0;
+    float t0 = 0.f, t1 = 0.f, t2 = 0.f, t3 = 0.f;  // sums over the lane's channels of gcol * {dZ/dd, dZ/dh, dZ/dw, Z}
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    for (int cc = 0; cc < s.cpd / 32; cc++) {
+      const int c0 = dgi * s.cpd + cc * 32, g = c0 / s.cpg, cb = (c0 - g * s.cpg) / 32;
+      // x at the 8 corners, the lane's 32 bytes each: fetched a voxel per four lanes, passed through
+      // the stage four corners at a time
+      u32x4 xv[8][2];
+      auto gather = [&](int chunk) {
+        const unsigned cbyte = static_cast<unsigned>(c0) * ES + gbyte + static_cast<unsigned>(chunk * 32);
+        u32x4 raw[2][2][4];
+#pragma unroll
+        for (int r = 0; r < 2; r++)
+#pragma unroll
+          for (int p = 0; p < 2; p++) {
+            const u32x4 at4 = *reinterpret_cast<const u32x4 *>(tp + (gp + 16 * p) * 32 + r * 16);
+#pragma unroll
+            for (int c4 = 0; c4 < 4; c4++)
+              raw[r][p][c4] = __builtin_amdgcn_raw_buffer_load_b128(xr, at4[c4] + cbyte, 0, 0);  // kOob + small: reads 0
+          }
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+#pragma unroll
+          for (int p = 0; p < 2; p++)
+#pragma unroll
+            for (int c4 = 0; c4 < 4; c4++)
+              *reinterpret_cast<u32x4 *>(stg + (c4 * 32 + gp + 16 * p) * kRow + gq * 16) = raw[r][p][c4];
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+          for (int c4 = 0; c4 < 4; c4++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+              xv[4 * r + c4][j] = *reinterpret_cast<const u32x4 *>(stg + (c4 * 32 + n) * kRow + 32 * h + 16 * j);
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+      };
+      // ---- gcol[32 channels x 32 positions] = Wt_k^T[32 x opg] * gy^T[opg x 32] -------------------
+      float16_t acc;
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[r] = 0.f;
+      const T *wfrag = wa + ((((static_cast<long>(g) * s.K + k) * cblocks + cb) * steps) * 64 + lane) * PC;
+      const T *brow = gyrow + g * s.opg;
+#pragma unroll
+      for (int st = 0; st < 4; st++)
+        if (st < steps) {
+          const u32x4 af = *reinterpret_cast<const u32x4 *>(wfrag + static_cast<long>(st) * (64 * PC));
+          const u32x4 bf = hoist ? bkeep[st]
+                                 : (live ? *reinterpret_cast<const u32x4 *>(brow + st * SL) : u32x4{0u, 0u, 0u, 0u});
+          acc = M::run(af, bf, acc);
+        }
+      for (int st = 4; st < steps; st++) {
+        const u32x4 af = *reinterpret_cast<const u32x4 *>(wfrag + static_cast<long>(st) * (64 * PC));
+        const u32x4 bf = live ? *reinterpret_cast<const u32x4 *>(brow + st * SL) : u32x4{0u, 0u, 0u, 0u};
+        acc = M::run(af, bf, acc);
+      }
+#pragma unroll
+      for (int chunk = 0; chunk < CHUNKS; chunk++) {
+        gather(chunk);
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+          const int r = chunk * CH + i;  // channel c0 + 16 * h + r
+          float v[8];
+#pragma unroll
+          for (int c = 0; c < 8; c++) {
+            if constexpr (ES == 4) {
+              v[c] = __uint_as_float(xv[c][i / 4][i % 4]);
+            } else {
+              const unsigned word = xv[c][i / 8][(i % 8) / 2];
+              v[c] = (i % 2) ? M::hi(word) : M::lo(word);
+            }
+          }
+          // value and the three partial derivatives of the trilinear form, sharing the differences
+          const float x0 = v[1] - v[0], x1 = v[3] - v[2], x2 = v[5] - v[4], x3 = v[7] - v[6];
+          const float a0 = fmaf(lw, x0, v[0]), a1 = fmaf(lw, x1, v[2]), a2 = fmaf(lw, x2, v[4]), a3 = fmaf(lw, x3, v[6]);
+          const float b0 = fmaf(lh, x1 - x0, x0), b1 = fmaf(lh, x3 - x2, x2);
+          const float dw = fmaf(ld, b1 - b0, b0);
+          const float y0 = a1 - a0, y1 = a3 - a2;
+          const float c0v = fmaf(lh, y0, a0), c1v = fmaf(lh, y1, a2);
+          const float dh = fmaf(ld, y1 - y0, y0);
+          const float dd = c1v - c0v;
+          const float val = fmaf(ld, dd, c0v);
+          const float gc = acc[r];
+          t0 = fmaf(dd, gc, t0); t1 = fmaf(dh, gc, t1); t2 = fmaf(dw, gc, t2); t3 = fmaf(val, gc, t3);
+          // column value of (channel 16 * h + r, position n), pieces [position / kPiece][channel][kPiece]
+          cs[((n / PC) * 32 + 16 * h + r) * PC + n % PC] = store_cast<T>(m * val);
+          // one channel at a time, its sums formed here (left alone the compiler moves the sums
+          // behind the stores below and keeps every channel's differences alive until then)
+          asm volatile("" : "+v"(t0), "+v"(t1), "+v"(t2), "+v"(t3));
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      if (any_far) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) fg[n * 33 + 16 * h + r] = acc[r] * m;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      if (col) {
+        // the wavefront's block of the column buffer is contiguous: 32 positions x 32 channels
+        T *dst = col + ((static_cast<long>(b) * s.K + k) * (s.Cin / 32) + c0 / 32) * qp * 32 + q0 * 32 + lane * 16;
+#pragma unroll
+        for (int j = 0; j < ES; j++) {
+          const u32x4 piece = *reinterpret_cast<const u32x4 *>(cs + lane * 16 + j * (16 / ES));
+          // (nontemporal: the buffer is larger than the caches and read once, by the weight kernel)
+          __builtin_nontemporal_store(piece, reinterpret_cast<u32x4 *>(dst + j * (16 / ES)));
+        }
+      }
+      if (any_far) {
+        // the lower half adds the 32 channels of list entry i, the upper half those of entry i + 1
+        const unsigned cbyte4 = static_cast<unsigned>(c0 + n) * 4u;
+        for (int i = h; i < far_count; i += 2) {
+          const uint2 e = fl[i];
+          const float gmv = fg[(e.x & 31u) * 33 + n];
+          __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(__uint_as_float(e.y) * gmv, gr, (e.x & ~127u) + cbyte4, 0, 0);
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    // ---- the other half-wavefront's sixteen channels, then grad offset / grad mask -----------------
+    t0 += __shfl_xor(t0, 32); t1 += __shfl_xor(t1, 32); t2 += __shfl_xor(t2, 32); t3 += __shfl_xor(t3, 32);
+    if (h == 0 && live) {
+      T *go = goff + (bg * s.nd * s.K + s.nd * k) * s.Q + q;
+      if (s.nd == 3) go[0] = store_cast<T>(m * t0);
+      go[(s.nd - 2) * s.Q] = store_cast<T>(m * t1); go[(s.nd - 1) * s.Q] = store_cast<T>(m * t2);
+      if (gmask) gmask[(bg * s.K + k) * s.Q + q] = store_cast<T>(t3);
+    }
+  }
+}
+
 // ---- gradient of the input, local corners: summed in LDS, then added to the buffer ----------------
 // A workgroup owns a brick of positions and eight channels; its sixteen wavefronts are kScatterSplit
 // groups of eight, every group covers the positions of the brick (32 per wavefront at a time) and
@@ -584,6 +862,252 @@ __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter_kerne
           static_cast<float>(v), gr,
           static_cast<unsigned>((zd * s.H + zh) * s.W + zw) * cin4 + static_cast<unsigned>(c0 + ch) * 4u, 0, 0);
     }
+  }
+}
+
+// ---- the same sums in 32-bit cells, for 16-bit tensors ---------------------------------------------
+// A workgroup owns a brick and SIXTEEN channels (all 16 rows of the 16 x 16 MFMA): the taps, the
+// records and grad_output serve twice the channels, an LDS add moves 4 bytes instead of 8 and a term
+// costs one fma and one subtraction.  32 bits leave 30 - ceil(log2(positions * taps)) bits for a
+// term (17 for 3 x 3 x 3 taps), so the scale comes from the data: a first sweep over the brick's
+// taps forms gcol alone (matrix cores, no geometry) and takes max |gcol| of the workgroup; every
+// term is then below max |gcol| * max |mask| < 2^ex and is rounded to a multiple of 2^(ex - shift)
+// (adding 1.5 * 2^23 in fp32 leaves round(x) in the low mantissa bits for |x| < 2^22).  The error of
+// a voxel's sum stays below terms * 2^(ex - shift - 1), about 2^-15 of the values it sums for the
+// 3 x 3 x 3 layer — a sixteenth of the last bit of the 16-bit result.
+constexpr int kScatter32Stride = 17;    // dwords between voxels: 16 channels and one to spread the banks
+constexpr int kScatter32MinShift = 14;  // fewer bits per term: the 64-bit kernel takes the layer
+__host__ __device__ constexpr int scatter32_shift(int terms) {
+  int bits = 0;
+  while ((1L << bits) < terms) bits++;
+  return 30 - bits;
+}
+
+// weight [Cout, cpg, K] -> A pieces [group][tap][16-channel block][row step][lane][kPiece]: lane l is
+// MFMA row l % 16 = channel l % 16 of the block, element i the output channel
+// g*opg + step*4*kPiece + (l/16)*kPiece + i
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_weight_afragments16_kernel(const T *__restrict__ wt,
+                                                                      T *__restrict__ wa,
+                                                                      const DcnDims s) {
+  constexpr int PC = Mfma<T>::kPiece;
+  const int cblocks = s.cpg / 16, steps = s.opg / (4 * PC);
+  const long total = static_cast<long>(s.groups) * s.K * cblocks * steps * 64;
+  const long id = blockIdx.x * 256L + threadIdx.x;
+  if (id >= total) return;
+  const int lane = id % 64;
+  long r = id / 64;
+  const int st = r % steps; r /= steps;
+  const int cb = r % cblocks; r /= cblocks;
+  const int k = r % s.K;
+  const int g = static_cast<int>(r / s.K);
+  const int cl = cb * 16 + lane % 16;
+  const int o = g * s.opg + st * 4 * PC + (lane / 16) * PC;
+  for (int i = 0; i < PC; i++) wa[id * PC + i] = wt[(static_cast<long>(o + i) * s.cpg + cl) * s.K + k];
+}
+
+template <typename T, typename S>
+__global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter32_kernel(
+    const T *__restrict__ off, const T *__restrict__ mask, const T *__restrict__ gyt,
+    const T *__restrict__ wa, float *__restrict__ gxt, const DcnDims s, const int nbh, const int nbw,
+    const unsigned *__restrict__ bounds) {
+  using M = Mfma<T>;
+  using P = typename std::conditional<(sizeof(T) == 2), float, double>::type;
+  constexpr int PC = M::kPiece, SL = 4 * PC;
+  constexpr int VOX = S::TD * S::TH * S::TW;
+  constexpr int GROUPS = S::BD * S::BH * S::BW / 32;  // 32-position groups of the brick
+  static_assert(VOX <= kTileVoxMax && GROUPS % 8 == 0, "brick and tile sizes");
+  __shared__ int tile[VOX * kScatter32Stride];
+  __shared__ __attribute__((aligned(16))) float recs[kScatterWaves][32][8];
+  __shared__ unsigned wgmax;
+  // (the validity of the data kernel's split: no NaN or infinity anywhere, products finite)
+  if (!scatter_scale(bounds, S::BD * S::BH * S::BW * s.K, mask != nullptr).valid) return;
+  const float mask_max = mask ? __uint_as_float(bounds[2]) : 1.f;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int n = lane % 32, p16 = lane % 16, j = lane / 16;
+  const int tg = wave / 8;
+  const unsigned brick = xcd_contiguous(blockIdx.x, gridDim.x);
+  const int bx = brick % nbw, by = (brick / nbw) % nbh, bz = brick / (nbw * nbh);
+  const int c0 = blockIdx.y * 16, b = blockIdx.z;
+  const int dgi = c0 / s.cpd, g = c0 / s.cpg, cb = (c0 - g * s.cpg) / 16;
+  const long bg = static_cast<long>(b) * s.dg + dgi;
+  const int cblocks = s.cpg / 16, steps = s.opg / SL;
+  const TileOrigin origin = tile_origin<S>(s, bz, by, bx);
+  const int per = (s.K + kScatterSplit - 1) / kScatterSplit, k0 = min(tg * per, s.K), k1 = min(s.K, k0 + per);
+  const long tap_stride = static_cast<long>(cblocks) * steps * 64 * PC;
+  const T *afrag0 = wa + (((static_cast<long>(g) * s.K + k0) * cblocks + cb) * steps * 64 + lane) * PC;
+
+  for (int i = threadIdx.x; i < VOX * kScatter32Stride; i += kScatterWaves * 64) tile[i] = 0;
+  if (threadIdx.x == 0) wgmax = 0u;
+  __syncthreads();
+
+  // position of brick index i, columns fastest
+  auto position = [&](int i, bool &live) {
+    const int od = bz * S::BD + i / (S::BH * S::BW), oh = by * S::BH + (i / S::BW) % S::BH, ow = bx * S::BW + i % S::BW;
+    live = od < s.Do && oh < s.Ho && ow < s.Wo;
+    return (static_cast<long>(min(od, s.Do - 1)) * s.Ho + min(oh, s.Ho - 1)) * s.Wo + min(ow, s.Wo - 1);
+  };
+  // grad_output of the lane's column in the two 16-position blocks of a group (MFMA B operand)
+  auto load_keep = [&](int pg, u32x4 (&keep)[2][kScatterKeep]) {
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++) {
+      bool blive;
+      const long qb = position(pg * 32 + blk * 16 + p16, blive);
+      const T *grow = gyt + (static_cast<long>(b) * s.Q + qb) * s.Cout + g * s.opg + j * PC;
+#pragma unroll
+      for (int st = 0; st < kScatterKeep; st++)
+        keep[blk][st] = (blive && st < steps) ? *reinterpret_cast<const u32x4 *>(grow + st * SL) : u32x4{0u, 0u, 0u, 0u};
+    }
+  };
+  auto load_weights = [&](const T *afrag, bool on, u32x4 (&w)[kScatterKeep]) {
+#pragma unroll
+    for (int st = 0; st < kScatterKeep; st++)
+      w[st] = (on && st < steps) ? *reinterpret_cast<const u32x4 *>(afrag + static_cast<long>(st) * (64 * PC))
+                                 : u32x4{0u, 0u, 0u, 0u};
+  };
+
+  // ---- first sweep: max |gcol| over the brick's positions, the taps and the 16 channels -----------
+  {
+    float top = 0.f;
+    for (int pg = wave % 8; pg < GROUPS; pg += 8) {
+      u32x4 keep[2][kScatterKeep];
+      load_keep(pg, keep);
+      const T *afrag = afrag0;
+      for (int k = k0; k < k1; k++) {
+        u32x4 w[kScatterKeep];
+        load_weights(afrag, true, w);
+        afrag += tap_stride;
+        float4_t acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+        for (int st = 0; st < kScatterKeep; st++)
+          if (st < steps) {
+            acc[0] = M::run16(w[st], keep[0][st], acc[0]);
+            acc[1] = M::run16(w[st], keep[1][st], acc[1]);
+          }
+#pragma unroll
+        for (int i = 0; i < 4; i++) top = fmaxf(top, fmaxf(fabsf(acc[0][i]), fabsf(acc[1][i])));
+      }
+    }
+    for (int sh = 32; sh > 0; sh >>= 1) top = fmaxf(top, __shfl_xor(top, sh));
+    if (lane == 0 && top > 0.f) atomicMax(&wgmax, __float_as_uint(top));
+  }
+  __syncthreads();
+  const float bound = fmaxf(1.001f * __uint_as_float(wgmax), 1e-30f) * mask_max;
+  if (!(bound > 0.f)) return;  // nothing but zeros to add (the whole workgroup leaves together)
+  const int shift = scatter32_shift(S::BD * S::BH * S::BW * s.K);
+  int ex = 0;
+  frexpf(bound, &ex);  // bound < 2^ex
+  const float up = ldexpf(1.f, shift - ex), down = ldexpf(1.f, ex - shift);
+  constexpr float kMagic = 12582912.f;  // 1.5 * 2^23
+
+  for (int pg = wave % 8; pg < GROUPS; pg += 8) {
+  // the lane's own position for the taps (both halves of the wavefront compute them)
+  bool live;
+  const long q = position(pg * 32 + n, live);
+  const int ow = q % s.Wo, oh = (q / s.Wo) % s.Ho, od = q / (static_cast<long>(s.Wo) * s.Ho);
+  const int bd = od * s.sd - s.pd, bh = oh * s.sh - s.ph, bw = ow * s.sw - s.pw;
+  u32x4 keep[2][kScatterKeep];
+  load_keep(pg, keep);
+  const T *o = off + (bg * s.nd * s.K + static_cast<long>(s.nd) * k0) * s.Q + q;
+  const T *mk = mask ? mask + (bg * s.K + k0) * s.Q + q : nullptr;
+  float(*rec)[8] = recs[wave];
+
+  int ki = k0 / (s.kh * s.kw), kj = (k0 / s.kw) % s.kh, kk = k0 % s.kw;
+  P fd = P(0), fh = P(0), fw = P(0);
+  float fm = 1.f;
+  if (k0 < k1) {
+    dcn_offsets(s, o, fd, fh, fw);
+    if (mk) fm = load(mk);
+  }
+  // weight pieces of the current tap, loaded one tap ahead
+  const T *afrag = afrag0;
+  u32x4 wcur[kScatterKeep];
+  load_weights(afrag, k0 < k1, wcur);
+  for (int k = k0; k < k1; k++) {
+    u32x4 wnext[kScatterKeep];
+    load_weights(afrag + tap_stride, k + 1 < k1, wnext);
+    {
+      const P pd = fd + static_cast<P>(bd + ki * s.dd), ph = fh + static_cast<P>(bh + kj * s.dh),
+              pw = fw + static_cast<P>(bw + kk * s.dw);
+      const float m = fm;
+      o += s.nd * s.Q;
+      if (mk) mk += s.Q;
+      if (++kk == s.kw) { kk = 0; if (++kj == s.kh) { kj = 0; ++ki; } }
+      if (k + 1 < k1) {  // the next tap's offsets are in flight during this tap's adds
+        dcn_offsets(s, o, fd, fh, fw);
+        if (mk) fm = load(mk);
+      }
+      CornerTaps t;
+      corner_taps<P>(s, pd, ph, pw, live, 1u, 0u, ~0u, t);
+      int first;
+      unsigned bits = tile_bits<S>(origin, static_cast<int>(floor(pd)), static_cast<int>(floor(ph)),
+                                static_cast<int>(floor(pw)), first);
+      unsigned inside = 0;
+#pragma unroll
+      for (int c = 0; c < 8; c++) inside |= t.at[c] != ~0u ? 1u << c : 0u;
+      bits &= inside;
+      if (lane < 32) {
+        float4 *dst = reinterpret_cast<float4 *>(rec[n]);
+        dst[0] = make_float4(__int_as_float(first), __uint_as_float(bits), m * up, t.ld);
+        dst[1] = make_float4(t.lh, t.lw, 0.f, 0.f);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    float4_t acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+    for (int st = 0; st < kScatterKeep; st++)
+      if (st < steps) {
+        acc[0] = M::run16(wcur[st], keep[0][st], acc[0]);
+        acc[1] = M::run16(wcur[st], keep[1][st], acc[1]);
+      }
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++) {
+      const float4 *src = reinterpret_cast<const float4 *>(rec[blk * 16 + p16]);
+      const float4 ra = src[0], rb = src[1];
+      const int first = __float_as_int(ra.x);
+      const unsigned bits = __float_as_uint(ra.y);
+      // the lane's four channels 4j .. 4j + 3, times the mask and the fixed-point scale
+      const float gv[4] = {acc[blk][0] * ra.z, acc[blk][1] * ra.z, acc[blk][2] * ra.z, acc[blk][3] * ra.z};
+      const float wd[2] = {1.f - ra.w, ra.w}, wh[2] = {1.f - rb.x, rb.x}, ww[2] = {1.f - rb.y, rb.y};
+      // the lane's first dword of the first corner, as a 32-bit byte offset worked out once: the
+      // corners and channels differ by constants that go into the instructions' offset fields
+      char *const cell0 = reinterpret_cast<char *>(tile) + (static_cast<unsigned>(first) * kScatter32Stride + 4 * j) * 4u;
+#pragma unroll
+      for (int c = 0; c < 8; c++) {
+        const int ca = c >> 2, cb2 = (c >> 1) & 1, ce = c & 1;
+        if ((S::TD > 1 || ca == 0) && ((bits >> c) & 1u)) {  // images have no second slice
+          const float wc = wd[ca] * wh[cb2] * ww[ce];
+          int *dst = reinterpret_cast<int *>(cell0 + (ca * (S::TH * S::TW) + cb2 * S::TW + ce) * (kScatter32Stride * 4));
+#pragma unroll
+          for (int r = 0; r < 4; r++)
+            __hip_atomic_fetch_add(dst + r, __float_as_int(fmaf(wc, gv[r], kMagic)) - 0x4B400000, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    afrag += tap_stride;
+#pragma unroll
+    for (int st = 0; st < kScatterKeep; st++) wcur[st] = wnext[st];
+  }
+  }
+  __syncthreads();
+  // ---- the tile's voxels inside the volume go to the gradient buffer, 16 channels per voxel -------
+  const __amdgpu_buffer_rsrc_t gr = __builtin_amdgcn_make_buffer_rsrc(
+      gxt + static_cast<long>(b) * s.P * s.Cin, 0, static_cast<int>(s.P * s.Cin * 4), kRsrcFlags);
+  const unsigned cin4 = static_cast<unsigned>(s.Cin) * 4u;
+  const int ch = threadIdx.x % 16;
+  for (int cell = threadIdx.x / 16; cell < VOX; cell += kScatterWaves * 4) {
+    const int zw = cell % S::TW + origin.w, zh = (cell / S::TW) % S::TH + origin.h, zd = cell / (S::TW * S::TH) + origin.d;
+    const int sum = tile[cell * kScatter32Stride + ch];
+    if (zd >= 0 && zd < s.D && zh >= 0 && zh < s.H && zw >= 0 && zw < s.W && sum != 0)
+      __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(
+          static_cast<float>(sum) * down, gr,
+          static_cast<unsigned>((zd * s.H + zh) * s.W + zw) * cin4 + static_cast<unsigned>(c0 + ch) * 4u, 0, 0);
   }
 }
 
@@ -957,16 +1481,23 @@ static int backward_run(const void *x, const void *off, const void *mask, const 
   if (st) return st;
   st = dcn_channels_last(gy, gyt, s.B, s.Cout, s.Q, sizeof(T), stream);
   if (st) return st;
+  const bool image = s.nd == 2;
+  const bool tiles = image ? scatter_tile_applies<ImageBricks>(s, dtype) : scatter_tile_applies<VolumeBricks>(s, dtype);
+  // 32-channel weight fragments: B operands (columns = channels) for the data kernel with a channel
+  // per lane, A operands (rows = channels) for the one with a position per lane
   const long frag_lanes = static_cast<long>(s.groups) * s.K * (s.cpg / 32) * (s.opg / (2 * Mfma<T>::kPiece)) * 64;
-  hipLaunchKernelGGL((dcn_weight_bfragments_kernel<T>), dim3(static_cast<unsigned>((frag_lanes + 255) / 256)),
-                     dim3(256), 0, stream, static_cast<const T *>(wt), wb, s);
+  if (tiles)
+    hipLaunchKernelGGL((dcn_weight_afragments32_kernel<T>), dim3(static_cast<unsigned>((frag_lanes + 255) / 256)),
+                       dim3(256), 0, stream, static_cast<const T *>(wt), wb, s);
+  else
+    hipLaunchKernelGGL((dcn_weight_bfragments_kernel<T>), dim3(static_cast<unsigned>((frag_lanes + 255) / 256)),
+                       dim3(256), 0, stream, static_cast<const T *>(wt), wb, s);
   const long nz = static_cast<long>((l.total - l.gxt) / 4);
   hipLaunchKernelGGL(dcn_zero_f32_kernel, dim3(static_cast<unsigned>(min((nz + 1023) / 1024, 65536L))), dim3(256),
                      0, stream, gxt, nz);
   const long qblocks = (s.Q + 127) / 128;
   MV_REQUIRE(qblocks < (1L << 31), "grid too large");
-  const bool image = s.nd == 2;
-  if (image ? scatter_tile_applies<ImageBricks>(s, dtype) : scatter_tile_applies<VolumeBricks>(s, dtype)) {
+  if (tiles) {
     unsigned *bounds = reinterpret_cast<unsigned *>(ws + l.bounds);
     const long ngy = static_cast<long>(s.B) * s.Cout * s.Q, nmask = static_cast<long>(s.B) * s.dg * s.K * s.Q;
     const long ncols = static_cast<long>(s.groups) * s.cpg * s.K;
@@ -978,21 +1509,36 @@ static int backward_run(const void *x, const void *off, const void *mask, const 
       hipLaunchKernelGGL((dcn_absmax_kernel<T>), dim3(static_cast<unsigned>(min((nmask + 8191) / 8192, 256L))),
                          dim3(256), 0, stream, static_cast<const T *>(mask), nmask, bounds + 2);
     T *wa = reinterpret_cast<T *>(ws + l.wa);
-    const long lanes8 = static_cast<long>(s.groups) * s.K * (s.cpg / 8) * (s.opg / (4 * Mfma<T>::kPiece)) * 64;
-    hipLaunchKernelGGL((dcn_weight_afragments8_kernel<T>), dim3(static_cast<unsigned>((lanes8 + 255) / 256)),
-                       dim3(256), 0, stream, static_cast<const T *>(wt), wa, s);
+    // 16-bit tensors: 32-bit cells and 16 channels per workgroup, while a term keeps enough bits
+    const int terms = (image ? ImageBricks::BD * ImageBricks::BH * ImageBricks::BW
+                             : VolumeBricks::BD * VolumeBricks::BH * VolumeBricks::BW) * s.K;
+    const bool narrow = sizeof(T) == 2 && scatter32_shift(terms) >= kScatter32MinShift;
+    const int wch = narrow ? 16 : 8;
+    const long lanes = static_cast<long>(s.groups) * s.K * (s.cpg / wch) * (s.opg / (4 * Mfma<T>::kPiece)) * 64;
+    if (narrow)
+      hipLaunchKernelGGL((dcn_weight_afragments16_kernel<T>), dim3(static_cast<unsigned>((lanes + 255) / 256)),
+                         dim3(256), 0, stream, static_cast<const T *>(wt), wa, s);
+    else
+      hipLaunchKernelGGL((dcn_weight_afragments8_kernel<T>), dim3(static_cast<unsigned>((lanes + 255) / 256)),
+                         dim3(256), 0, stream, static_cast<const T *>(wt), wa, s);
     MV_REQUIRE(s.Cin / 8 <= 65535, "grid too large");
 #define MV_LAUNCH_SPLIT(S)                                                                                        \
   {                                                                                                               \
-    hipLaunchKernelGGL((dcn_backward_data_mfma_kernel<T, true, S>), dim3(static_cast<unsigned>(qblocks), s.dg, s.B), \
+    hipLaunchKernelGGL((dcn_backward_data_lanes_kernel<T, S>), dim3(static_cast<unsigned>(qblocks), s.dg, s.B),   \
                        dim3(256), 0, stream, xt, static_cast<const T *>(off), static_cast<const T *>(mask), gyt,  \
                        wb, gxt, static_cast<T *>(goff), static_cast<T *>(gmask), s, bounds, col, l.qp);           \
     const long nbd = (s.Do + S::BD - 1) / S::BD, nbh = (s.Ho + S::BH - 1) / S::BH, nbw = (s.Wo + S::BW - 1) / S::BW; \
     MV_REQUIRE(nbd * nbh * nbw < (1L << 31), "grid too large");                                                   \
-    hipLaunchKernelGGL((dcn_backward_scatter_kernel<T, S>),                                                       \
-                       dim3(static_cast<unsigned>(nbd * nbh * nbw), s.Cin / 8, s.B), dim3(kScatterWaves * 64), 0, \
-                       stream, static_cast<const T *>(off), static_cast<const T *>(mask), gyt, wa, gxt, s,        \
-                       static_cast<int>(nbh), static_cast<int>(nbw), bounds);                                     \
+    if (narrow)                                                                                                   \
+      hipLaunchKernelGGL((dcn_backward_scatter32_kernel<T, S>),                                                   \
+                         dim3(static_cast<unsigned>(nbd * nbh * nbw), s.Cin / 16, s.B), dim3(kScatterWaves * 64), 0, \
+                         stream, static_cast<const T *>(off), static_cast<const T *>(mask), gyt, wa, gxt, s,      \
+                         static_cast<int>(nbh), static_cast<int>(nbw), bounds);                                   \
+    else                                                                                                          \
+      hipLaunchKernelGGL((dcn_backward_scatter_kernel<T, S>),                                                     \
+                         dim3(static_cast<unsigned>(nbd * nbh * nbw), s.Cin / 8, s.B), dim3(kScatterWaves * 64), 0, \
+                         stream, static_cast<const T *>(off), static_cast<const T *>(mask), gyt, wa, gxt, s,      \
+                         static_cast<int>(nbh), static_cast<int>(nbw), bounds);                                   \
   }
     if (image) MV_LAUNCH_SPLIT(ImageBricks) else MV_LAUNCH_SPLIT(VolumeBricks)
 #undef MV_LAUNCH_SPLIT
