@@ -638,10 +638,14 @@ __global__ __launch_bounds__(256, 3) void dcn_backward_data_lanes_kernel(
       if (any_far) {
         // the lower half adds the 32 channels of list entry i, the upper half those of entry i + 1
         const unsigned cbyte4 = static_cast<unsigned>(c0 + n) * 4u;
-        for (int i = h; i < far_count; i += 2) {
-          const uint2 e = fl[i];
-          const float gmv = fg[(e.x & 31u) * 33 + n];
-          __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(__uint_as_float(e.y) * gmv, gr, (e.x & ~127u) + cbyte4, 0, 0);
+        // (four entries per turn, so that the LDS reads of one overlap those of the other)
+        for (int i = h; i < far_count; i += 4) {
+          const bool two = i + 2 < far_count;
+          const uint2 e0 = fl[i], e1 = fl[min(i + 2, 255)];
+          const float g0 = fg[(e0.x & 31u) * 33 + n], g1 = fg[(e1.x & 31u) * 33 + n];
+          __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(__uint_as_float(e0.y) * g0, gr, (e0.x & ~127u) + cbyte4, 0, 0);
+          __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(__uint_as_float(e1.y) * g1, gr,
+                                                          two ? (e1.x & ~127u) + cbyte4 : kOob, 0, 0);
         }
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -918,7 +922,7 @@ __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter32_ker
   constexpr int GROUPS = S::BD * S::BH * S::BW / 32;  // 32-position groups of the brick
   static_assert(VOX <= kTileVoxMax && GROUPS % 8 == 0, "brick and tile sizes");
   __shared__ int tile[VOX * kScatter32Stride];
-  __shared__ __attribute__((aligned(16))) float recs[kScatterWaves][32][8];
+  __shared__ __attribute__((aligned(8))) float recs[kScatterWaves][64][6];
   __shared__ unsigned wgmax;
   // (the validity of the data kernel's split: no NaN or infinity anywhere, products finite)
   if (!scatter_scale(bounds, S::BD * S::BH * S::BW * s.K, mask != nullptr).valid) return;
@@ -1001,44 +1005,50 @@ __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter32_ker
   constexpr float kMagic = 12582912.f;  // 1.5 * 2^23
 
   for (int pg = wave % 8; pg < GROUPS; pg += 8) {
-  // the lane's own position for the taps (both halves of the wavefront compute them)
+  // the taps are worked out two at a time: the lower half-wavefront takes tap k of the group's 32
+  // positions, the upper half tap k + 1
+  const int hh = lane / 32;
   bool live;
   const long q = position(pg * 32 + n, live);
   const int ow = q % s.Wo, oh = (q / s.Wo) % s.Ho, od = q / (static_cast<long>(s.Wo) * s.Ho);
   const int bd = od * s.sd - s.pd, bh = oh * s.sh - s.ph, bw = ow * s.sw - s.pw;
   u32x4 keep[2][kScatterKeep];
   load_keep(pg, keep);
-  const T *o = off + (bg * s.nd * s.K + static_cast<long>(s.nd) * k0) * s.Q + q;
-  const T *mk = mask ? mask + (bg * s.K + k0) * s.Q + q : nullptr;
-  float(*rec)[8] = recs[wave];
+  int kt = k0 + hh;  // the lane's own tap
+  const T *o = off + (bg * s.nd * s.K + static_cast<long>(s.nd) * kt) * s.Q + q;
+  const T *mk = mask ? mask + (bg * s.K + kt) * s.Q + q : nullptr;
+  float(*rec)[6] = recs[wave];
 
-  int ki = k0 / (s.kh * s.kw), kj = (k0 / s.kw) % s.kh, kk = k0 % s.kw;
+  int ki = kt / (s.kh * s.kw), kj = (kt / s.kw) % s.kh, kk = kt % s.kw;
   P fd = P(0), fh = P(0), fw = P(0);
   float fm = 1.f;
-  if (k0 < k1) {
+  if (kt < k1) {
     dcn_offsets(s, o, fd, fh, fw);
     if (mk) fm = load(mk);
   }
-  // weight pieces of the current tap, loaded one tap ahead
   const T *afrag = afrag0;
-  u32x4 wcur[kScatterKeep];
-  load_weights(afrag, k0 < k1, wcur);
-  for (int k = k0; k < k1; k++) {
-    u32x4 wnext[kScatterKeep];
-    load_weights(afrag + tap_stride, k + 1 < k1, wnext);
+  for (int k = k0; k < k1; k += 2) {
+    // weight pieces of the two taps (the taps' geometry below hides their latency)
+    u32x4 wpair[2][kScatterKeep];
+    load_weights(afrag, true, wpair[0]);
+    load_weights(afrag + tap_stride, k + 1 < k1, wpair[1]);
     {
       const P pd = fd + static_cast<P>(bd + ki * s.dd), ph = fh + static_cast<P>(bh + kj * s.dh),
               pw = fw + static_cast<P>(bw + kk * s.dw);
       const float m = fm;
-      o += s.nd * s.Q;
-      if (mk) mk += s.Q;
-      if (++kk == s.kw) { kk = 0; if (++kj == s.kh) { kj = 0; ++ki; } }
-      if (k + 1 < k1) {  // the next tap's offsets are in flight during this tap's adds
+      const bool tap_on = kt < k1;
+      kt += 2;
+      o += 2 * s.nd * s.Q;
+      if (mk) mk += 2 * s.Q;
+#pragma unroll
+      for (int u = 0; u < 2; u++)
+        if (++kk == s.kw) { kk = 0; if (++kj == s.kh) { kj = 0; ++ki; } }
+      if (kt < k1) {  // the next pair's offsets are in flight during this pair's adds
         dcn_offsets(s, o, fd, fh, fw);
         if (mk) fm = load(mk);
       }
       CornerTaps t;
-      corner_taps<P>(s, pd, ph, pw, live, 1u, 0u, ~0u, t);
+      corner_taps<P>(s, pd, ph, pw, live && tap_on, 1u, 0u, ~0u, t);
       int first;
       unsigned bits = tile_bits<S>(origin, static_cast<int>(floor(pd)), static_cast<int>(floor(ph)),
                                 static_cast<int>(floor(pw)), first);
@@ -1046,53 +1056,54 @@ __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter32_ker
 #pragma unroll
       for (int c = 0; c < 8; c++) inside |= t.at[c] != ~0u ? 1u << c : 0u;
       bits &= inside;
-      if (lane < 32) {
-        float4 *dst = reinterpret_cast<float4 *>(rec[n]);
-        dst[0] = make_float4(__int_as_float(first), __uint_as_float(bits), m * up, t.ld);
-        dst[1] = make_float4(t.lh, t.lw, 0.f, 0.f);
-      }
+      float2 *dst = reinterpret_cast<float2 *>(rec[lane]);
+      dst[0] = make_float2(__int_as_float(first), __uint_as_float(bits));
+      dst[1] = make_float2(m * up, t.ld);
+      dst[2] = make_float2(t.lh, t.lw);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-    float4_t acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-    for (int st = 0; st < kScatterKeep; st++)
-      if (st < steps) {
-        acc[0] = M::run16(wcur[st], keep[0][st], acc[0]);
-        acc[1] = M::run16(wcur[st], keep[1][st], acc[1]);
-      }
+    for (int u = 0; u < 2; u++) {
+      if (k + u >= k1) break;
+      float4_t acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-    for (int blk = 0; blk < 2; blk++) {
-      const float4 *src = reinterpret_cast<const float4 *>(rec[blk * 16 + p16]);
-      const float4 ra = src[0], rb = src[1];
-      const int first = __float_as_int(ra.x);
-      const unsigned bits = __float_as_uint(ra.y);
-      // the lane's four channels 4j .. 4j + 3, times the mask and the fixed-point scale
-      const float gv[4] = {acc[blk][0] * ra.z, acc[blk][1] * ra.z, acc[blk][2] * ra.z, acc[blk][3] * ra.z};
-      const float wd[2] = {1.f - ra.w, ra.w}, wh[2] = {1.f - rb.x, rb.x}, ww[2] = {1.f - rb.y, rb.y};
-      // the lane's first dword of the first corner, as a 32-bit byte offset worked out once: the
-      // corners and channels differ by constants that go into the instructions' offset fields
-      char *const cell0 = reinterpret_cast<char *>(tile) + (static_cast<unsigned>(first) * kScatter32Stride + 4 * j) * 4u;
+      for (int st = 0; st < kScatterKeep; st++)
+        if (st < steps) {
+          acc[0] = M::run16(wpair[u][st], keep[0][st], acc[0]);
+          acc[1] = M::run16(wpair[u][st], keep[1][st], acc[1]);
+        }
 #pragma unroll
-      for (int c = 0; c < 8; c++) {
-        const int ca = c >> 2, cb2 = (c >> 1) & 1, ce = c & 1;
-        if ((S::TD > 1 || ca == 0) && ((bits >> c) & 1u)) {  // images have no second slice
-          const float wc = wd[ca] * wh[cb2] * ww[ce];
-          int *dst = reinterpret_cast<int *>(cell0 + (ca * (S::TH * S::TW) + cb2 * S::TW + ce) * (kScatter32Stride * 4));
+      for (int blk = 0; blk < 2; blk++) {
+        const float2 *src = reinterpret_cast<const float2 *>(rec[u * 32 + blk * 16 + p16]);
+        const float2 ra = src[0], rb = src[1], rc = src[2];
+        const int first = __float_as_int(ra.x);
+        const unsigned bits = __float_as_uint(ra.y);
+        // the lane's four channels 4j .. 4j + 3, times the mask and the fixed-point scale
+        const float gv[4] = {acc[blk][0] * rb.x, acc[blk][1] * rb.x, acc[blk][2] * rb.x, acc[blk][3] * rb.x};
+        const float wd[2] = {1.f - rb.y, rb.y}, wh[2] = {1.f - rc.x, rc.x}, ww[2] = {1.f - rc.y, rc.y};
+        // the lane's first dword of the first corner, as a 32-bit byte offset worked out once: the
+        // corners and channels differ by constants that go into the instructions' offset fields
+        char *const cell0 = reinterpret_cast<char *>(tile) + (static_cast<unsigned>(first) * kScatter32Stride + 4 * j) * 4u;
 #pragma unroll
-          for (int r = 0; r < 4; r++)
-            __hip_atomic_fetch_add(dst + r, __float_as_int(fmaf(wc, gv[r], kMagic)) - 0x4B400000, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_WORKGROUP);
+        for (int c = 0; c < 8; c++) {
+          const int ca = c >> 2, cb2 = (c >> 1) & 1, ce = c & 1;
+          if ((S::TD > 1 || ca == 0) && ((bits >> c) & 1u)) {  // images have no second slice
+            const float wc = wd[ca] * wh[cb2] * ww[ce];
+            int *dst = reinterpret_cast<int *>(cell0 + (ca * (S::TH * S::TW) + cb2 * S::TW + ce) * (kScatter32Stride * 4));
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+              __hip_atomic_fetch_add(dst + r, __float_as_int(fmaf(wc, gv[r], kMagic)) - 0x4B400000, __ATOMIC_RELAXED,
+                                     __HIP_MEMORY_SCOPE_WORKGROUP);
+          }
         }
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
-    afrag += tap_stride;
-#pragma unroll
-    for (int st = 0; st < kScatterKeep; st++) wcur[st] = wnext[st];
+    afrag += 2 * tap_stride;
   }
   }
   __syncthreads();
