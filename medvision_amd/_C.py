@@ -93,13 +93,11 @@ def _roi_forward(fn_name, what, ndim, cols, input, rois, output, out_sizes, spat
         raise RuntimeError(f"output has shape {tuple(output.shape)}, expected {want_shape}")
     code = _lib.dtype_code(feats)
     out3 = out_sizes if ndim == 3 else (1, *out_sizes)
-    if "rotated" in fn_name:
-        ws_bytes = _cached_bytes("mv_roi_align_forward_workspace_bytes", code, ndim, dims[1], r.size(0),
-                                 *out3, int(sampling_ratio))
-    else:   # plain boxes: detection heads may get a re-ordered copy of the features
-        in3 = dims[2:] if ndim == 3 else [1, *dims[2:]]
-        ws_bytes = _cached_bytes("mv_roi_align_forward_workspace_bytes_for_input", code, ndim, dims[0], dims[1],
-                                 *in3, r.size(0), *out3, int(sampling_ratio))
+    # the tiled resampler's plans, a re-ordered copy of the features for detection heads with plain
+    # boxes, a channels-last copy for heads the separable kernels do not take
+    in3 = dims[2:] if ndim == 3 else [1, *dims[2:]]
+    ws_bytes = _cached_bytes("mv_roi_align_forward_workspace_bytes_for_input", code, ndim, dims[0], dims[1],
+                             *in3, r.size(0), *out3, int(sampling_ratio))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=feats.device) if ws_bytes else None
     with _on_device(feats):
         _lib.check(getattr(lib, fn_name)(

@@ -139,6 +139,10 @@ bool roi_pool_applies(int dtype, const RoiProblem &p);
 // roi_box.hip: backward of small outputs that the pooled kernels do not take (rotated boxes, large
 // grids), one workgroup per (roi, channel group) with LDS tiles of the source boxes; -1 when not applicable
 int roi_box_backward(const void *grad_output, const void *rois, float *acc, int dtype, const RoiProblem &p, hipStream_t s);
+// Many small outputs over wide feature maps, read from a channels-last copy in the workspace (roi_cl.hip).
+size_t roi_forward_cl_workspace(int dtype, const RoiProblem &p);
+int roi_forward_cl(const void *input, const void *rois, void *output, int dtype, const RoiProblem &p,
+                   void *workspace, size_t capacity, hipStream_t s);
 
 int roi_backward_gather(const void *grad_output, const void *rois, void *grad_input, int dtype,
                         const RoiProblem &p, hipStream_t s);
@@ -189,6 +193,8 @@ int roi_forward(const void *input, const void *rois, void *output, int dtype, in
     if (tiled >= 0) return tiled;
     const int pooled = order != 3 ? roi_pool_forward(input, rois, output, dtype, p, workspace, capacity, s) : -1;
     if (pooled >= 0) return pooled;
+    const int wide = order != 3 ? roi_forward_cl(input, rois, output, dtype, p, workspace, capacity, s) : -1;
+    if (wide >= 0) return wide;
   }
   const dim3 grid(p.chunks * num_rois), block(kRoiThreads);
   MV_DISPATCH(dtype, {
@@ -374,8 +380,9 @@ size_t mv_roi_align_forward_workspace_bytes_for_input(int dtype, int ndim, int b
   p.ndim = ndim; p.N = batch; p.C = channels; p.D = ndim == 2 ? 1 : depth; p.H = height; p.W = width; p.R = num_rois;
   p.od = ndim == 2 ? 1 : out_d; p.oh = out_h; p.ow = out_w; p.sampling_ratio = sampling_ratio; p.order = 1;
   if (batch <= 0 || channels <= 0 || p.D <= 0 || height <= 0 || width <= 0 || num_rois <= 0) return basic;
+  if (basic) return basic;   // (the tiled resampler takes the problem)
   const size_t pooled = mv::roi_pool_forward_workspace(dtype, p);
-  return pooled > basic ? pooled : basic;
+  return pooled ? pooled : mv::roi_forward_cl_workspace(dtype, p);
 }
 
 size_t mv_roi_align_backward_workspace_bytes(int dtype, int batch, int channels, int depth,

@@ -829,3 +829,66 @@ def test_rotated_heads_backward_through_box_tiles(ops, oracle, dtype, ndim):
     assert torch.isnan(want).any() and torch.equal(torch.isnan(got), torch.isnan(want))
     ok = ~torch.isnan(want)
     assert_close(got[ok], want[ok], BWD_TOL[dtype], "a NaN gradient")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("ndim,rotated,C,out", [(3, True, 24, (7, 7, 7)), (3, True, 72, (7, 7, 7)),
+                                                (2, True, 520, (14, 14)), (2, False, 32, (20, 20))])
+def test_heads_forward_from_channels_last_copy(ops, oracle, dtype, ndim, rotated, C, out):
+    """Detection heads that the separable pooled kernels do not take (rotated boxes, more than 16 cells per
+    axis) read a channels-last copy of the features, a lane per (cell, 16 bytes of channels): channel
+    counts that fill part of a wavefront, leave lanes idle (72 -> 9 lanes per cell) or need two passes
+    (520), fixed and adaptive grids, order 0, rois sticking out of the image, a NaN feature; and the
+    same call with a workspace too small for the copy (general kernel) gives the same numbers."""
+    import ctypes
+    from medvision_amd import _lib
+    g = wl.gen(640 + ndim + C)
+    size = (12, 20, 24)[3 - ndim:] if ndim == 3 else (40, 48)
+    feat = torch.randn(2, C, *size, generator=g).to(dtype)
+    xyz = torch.tensor(size[::-1], dtype=torch.float32)
+    n = 30
+    ctr = (torch.rand(n, ndim, generator=g) * 1.2 - 0.1) * xyz
+    ext = torch.exp(torch.rand(n, ndim, generator=g) * math.log(40.0)) * 0.5      # 0.5 .. 20 voxels
+    idx = torch.randint(0, 2, (n, 1), generator=g).float()
+    ctr[:3], ext[:3], idx[0] = xyz * 0.5, xyz * 0.6, 0.0      # three rois over the middle of the image, one of them in image 0
+    if rotated:
+        ang = (torch.rand(n, 3 if ndim == 3 else 1, generator=g) * 2 - 1) * math.radians(40)
+        rois = torch.cat([idx, ctr, ext, ang], 1)
+        op = lambda sr: ops.RoIAlignRotated(out, 1.0, sr, True)
+    else:
+        rois = torch.cat([idx, ctr - ext / 2, ctr + ext / 2], 1)
+        op = lambda sr: ops.RoIAlign(out, 1.0, sr)
+    lib = _lib.load()
+    in3, out3 = ([1, *size] if ndim == 2 else list(size)), ([1, *out] if ndim == 2 else list(out))
+    need = lib.mv_roi_align_forward_workspace_bytes_for_input(_lib.dtype_code(feat), ndim, 2, C, *in3, n, *out3, 2)
+    assert need == feat.numel() * feat.element_size(), "the channels-last path does not take this problem"
+    x, r = feat.to(DEV), rois.to(DEV)
+    for sr in (2, 0, 3):
+        assert_close(op(sr)(x, r), oracle.roi_align_forward(feat, rois, out, 1.0, sr, True, 1, rotated),
+                     FWD_TOL[dtype], f"forward sr={sr}")
+    # without room for the copy the general kernel runs: same sample positions and tap decisions (the
+    # same fp64 expressions), the same order of the sums -- order 0, which only picks voxels, must agree
+    # exactly
+    fn = {(3, True): lib.mv_roi_align_rotated_3d_forward, (2, True): lib.mv_roi_align_rotated_2d_forward,
+          (2, False): lib.mv_roi_align_2d_forward}[(ndim, rotated)]
+    # (through the C entry point: the module turns order 0 into a grid of one sample, too few for this path)
+    small, room = torch.empty(1024, dtype=torch.uint8, device=DEV), torch.empty(need, dtype=torch.uint8, device=DEV)
+
+    def raw(order, ws):
+        y = torch.empty(n, C, *out, dtype=dtype, device=DEV)
+        extra = (1, order) if rotated else (order,)
+        _lib.check(fn(_lib.ptr(x), _lib.ptr(r), _lib.ptr(y), _lib.dtype_code(feat), 2, C, *size, n, *out,
+                      ctypes.c_float(1.0), 2, *extra, _lib.ptr(ws), ctypes.c_size_t(ws.numel()), _lib.stream_of(x)))
+        torch.cuda.synchronize()
+        return y
+
+    assert torch.equal(raw(1, room), op(2)(x, r))
+    assert_close(raw(1, small), raw(1, room).cpu(), {torch.float32: 2e-6, torch.float16: 1.1e-3, torch.bfloat16: 8.5e-3}[dtype],
+                 "general kernel")
+    assert torch.equal(raw(0, small), raw(0, room)), "order 0 against the general kernel"
+    # a NaN feature reaches exactly the outputs it reaches in the oracle
+    bad = feat.clone()
+    bad[(0, 1) + tuple(v // 2 for v in size)] = float("nan")
+    got = op(2)(bad.to(DEV), r).cpu()
+    want = oracle.roi_align_forward(bad, rois, out, 1.0, 2, True, 1, rotated)
+    assert torch.isnan(want).any() and torch.equal(torch.isnan(got), torch.isnan(want))
