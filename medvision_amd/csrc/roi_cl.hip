@@ -9,6 +9,7 @@
 // workgroup owns a roi: a lane takes one output cell and 16 bytes of channels (8 16-bit or 4 fp32
 // ones), the lanes of a cell sit side by side, so a tap is one 16-byte load per lane from the run of
 // C contiguous channels of its voxel, and the taps of a sample serve all of the lane's channels.
+// The lanes of a cell split its samples' geometry between them.
 // Sample coordinates, tap decisions and the void rule are those of the general kernels
 // (sampling.hpp, fp64); sums in fp32 in the order of the general kernel's sample loop.
 #include "common.hpp"
@@ -52,55 +53,80 @@ __global__ __launch_bounds__(kClThreads) void roi_forward_cl_kernel(const T *__r
       const_cast<T *>(xt + static_cast<long>(max(g.batch, 0)) * plane * p.C), 0, static_cast<int>(plane * p.C * ES), 0x00020000);
   const unsigned cbytes = static_cast<unsigned>(p.C) * ES;
   const float count = static_cast<float>(g.count);
+  const unsigned sy = static_cast<unsigned>(p.W) * cbytes, sz = static_cast<unsigned>(p.H) * sy;
   for (int pass = 0; pass < cs.passes; pass++) {
     const int c0 = (pass * cs.lanes + part) * V;   // the lane's first channel
-    const bool active = slot < cs.slots && c0 < p.C;
+    const bool loads = slot < cs.slots && c0 < p.C;
     for (unsigned first = begin + wave * cs.slots; first < end; first += (kClThreads / kWave) * cs.slots) {
       const unsigned cell = first + slot;
-      if (!active || cell >= end) continue;
+      const bool cell_on = slot < cs.slots && cell < end;
       float acc[V];
 #pragma unroll
       for (int i = 0; i < V; i++) acc[i] = 0.f;
-      for (int sub = 0; sub < samples; sub++) {
-        BoxTaps t;
-        if (!box_taps<ROT>(g, p, cell, sub, t)) continue;
-        auto take = [&](u32x4 r, float (&v)[V]) {
-          if constexpr (ES == 4) {
-            v[0] = __uint_as_float(r.x); v[1] = __uint_as_float(r.y); v[2] = __uint_as_float(r.z); v[3] = __uint_as_float(r.w);
-          } else {
-            union { u32x4 u; T e[8]; } w;
-            w.u = r;
-#pragma unroll
-            for (int i = 0; i < 8; i++) v[i] = static_cast<float>(load(&w.e[i]));
+      // The lanes of a cell share its samples: lane j of the group works out the taps of samples j,
+      // j + lanes, ... (fp64 geometry, once per sample instead of once per lane) and hands them to
+      // the others through ds_bpermute; every lane then adds the sample for its own channels.
+      for (int s0 = 0; s0 < samples; s0 += cs.lanes) {
+        int rec_at = -1;           // byte offset of the low corner's channels; -1: void sample
+        unsigned rec_step = 0;     // bit 0 / 1 / 2: the high tap differs from the low one along x / y / z
+        float rec_fx = 0.f, rec_fy = 0.f, rec_fz = 0.f;
+        if (cell_on && s0 + part < samples) {
+          BoxTaps t;
+          if (box_taps<ROT>(g, p, cell, s0 + part, t)) {
+            int zi = t.zi[0], yi = t.yi[0], xi = t.xi[0];
+            if (p.order == 0) {   // the picked voxel becomes the low corner
+              zi = t.fz == 0.f ? t.zi[0] : t.zi[1]; yi = t.fy == 0.f ? t.yi[0] : t.yi[1]; xi = t.fx == 0.f ? t.xi[0] : t.xi[1];
+            }
+            rec_at = static_cast<int>(static_cast<unsigned>((zi * p.H + yi) * p.W + xi) * cbytes);
+            rec_step = (t.xi[1] != t.xi[0] ? 1u : 0u) | (t.yi[1] != t.yi[0] ? 2u : 0u) | (t.zi[1] != t.zi[0] ? 4u : 0u);
+            rec_fx = t.fx; rec_fy = t.fy; rec_fz = t.fz;
           }
-        };
-        auto at = [&](int zi, int yi, int xi) {
-          return static_cast<unsigned>((zi * p.H + yi) * p.W + xi) * cbytes + static_cast<unsigned>(c0) * ES;
-        };
-        if (p.order == 0) {
-          const int zi = t.fz == 0.f ? t.zi[0] : t.zi[1], yi = t.fy == 0.f ? t.yi[0] : t.yi[1], xi = t.fx == 0.f ? t.xi[0] : t.xi[1];
-          float v[V];
-          take(__builtin_amdgcn_raw_buffer_load_b128(xr, at(zi, yi, xi), 0, 0), v);
-#pragma unroll
-          for (int i = 0; i < V; i++) acc[i] += v[i];
-          continue;
         }
-        u32x4 raw[8];
+        const int turns = min(cs.lanes, samples - s0);
+        for (int j = 0; j < turns; j++) {
+          const int from = min(slot * cs.lanes + j, kWave - 1);
+          const int at0 = __shfl(rec_at, from);
+          const unsigned step = __shfl(rec_step, from);
+          const float lx = __shfl(rec_fx, from), ly = __shfl(rec_fy, from), lz = __shfl(rec_fz, from);
+          if (at0 < 0 || !loads) continue;
+          const unsigned at = static_cast<unsigned>(at0) + static_cast<unsigned>(c0) * ES;
+          auto take = [&](u32x4 r, float (&v)[V]) {
+            if constexpr (ES == 4) {
+              v[0] = __uint_as_float(r.x); v[1] = __uint_as_float(r.y); v[2] = __uint_as_float(r.z); v[3] = __uint_as_float(r.w);
+            } else {
+              union { u32x4 u; T e[8]; } w;
+              w.u = r;
 #pragma unroll
-        for (int k = 0; k < 8; k++)
-          raw[k] = __builtin_amdgcn_raw_buffer_load_b128(xr, at(t.zi[k >> 2], t.yi[(k >> 1) & 1], t.xi[k & 1]), 0, 0);
-        const float lx = t.fx, ly = t.fy, lz = t.fz, hx = 1.f - lx, hy = 1.f - ly, hz = 1.f - lz;
-        float v[8][V];
+              for (int i = 0; i < 8; i++) v[i] = static_cast<float>(load(&w.e[i]));
+            }
+          };
+          if (p.order == 0) {
+            float v[V];
+            take(__builtin_amdgcn_raw_buffer_load_b128(xr, at, 0, 0), v);
 #pragma unroll
-        for (int k = 0; k < 8; k++) take(raw[k], v[k]);
+            for (int i = 0; i < V; i++) acc[i] += v[i];
+            continue;
+          }
+          const unsigned dx = (step & 1u) ? cbytes : 0u, dy = (step & 2u) ? sy : 0u, dz = (step & 4u) ? sz : 0u;
+          u32x4 raw[8];
 #pragma unroll
-        for (int i = 0; i < V; i++)
-          acc[i] += hz * (hy * (hx * v[0][i] + lx * v[1][i]) + ly * (hx * v[2][i] + lx * v[3][i])) +
-                    lz * (hy * (hx * v[4][i] + lx * v[5][i]) + ly * (hx * v[6][i] + lx * v[7][i]));
+          for (int k = 0; k < 8; k++)
+            raw[k] = __builtin_amdgcn_raw_buffer_load_b128(xr, at + ((k & 4) ? dz : 0u) + ((k & 2) ? dy : 0u) + ((k & 1) ? dx : 0u), 0, 0);
+          const float hx = 1.f - lx, hy = 1.f - ly, hz = 1.f - lz;
+          float v[8][V];
+#pragma unroll
+          for (int k = 0; k < 8; k++) take(raw[k], v[k]);
+#pragma unroll
+          for (int i = 0; i < V; i++)
+            acc[i] += hz * (hy * (hx * v[0][i] + lx * v[1][i]) + ly * (hx * v[2][i] + lx * v[3][i])) +
+                      lz * (hy * (hx * v[4][i] + lx * v[5][i]) + ly * (hx * v[6][i] + lx * v[7][i]));
+        }
       }
-      T *dst = out + (static_cast<long>(n) * p.C + c0) * cells + cell;
+      if (cell_on && loads) {
+        T *dst = out + (static_cast<long>(n) * p.C + c0) * cells + cell;
 #pragma unroll
-      for (int i = 0; i < V; i++) dst[static_cast<long>(i) * cells] = store_cast<T>(acc[i] / count);
+        for (int i = 0; i < V; i++) dst[static_cast<long>(i) * cells] = store_cast<T>(acc[i] / count);
+      }
     }
   }
 }
