@@ -149,6 +149,32 @@ def test_input_gradient_through_lds_tiles(ops, oracle, dtype, size, offset_std, 
     assert_close(ws.grad, gw, tol, "grad weight")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("nd,cout,groups", [(3, 160, 1), (3, 512, 2), (2, 288, 1)])
+def test_gradients_of_wide_layers(ops, oracle, dtype, nd, cout, groups):
+    """More than 128 output channels per group (FPN layers): beyond what the scatter kernel keeps of
+    grad_output in registers, so every corner of the input gradient goes through the data kernel."""
+    g = wl.gen(470 + cout)
+    if nd == 3:
+        from medvision_amd.ops.modulated_deform_conv_3d import modulated_deform_conv
+        size = (5, 9, 12)
+    else:
+        from medvision_amd.ops.modulated_deform_conv_2d import modulated_deform_conv
+        size = (37, 40)
+    x, off, mask, w, b = wl.dcn_inputs(g, 2, 32 * groups, cout, size, 3, 1, groups, dtype, 1, 1, 1, True, 1.5)
+    xs, offs, ms, ws, bs = [t.to(DEV).requires_grad_(True) for t in (x, off, mask, w, b)]
+    y = modulated_deform_conv(xs, offs, ms, ws, bs, 1, 1, 1, groups, 1)
+    gy = torch.randn(y.shape, generator=g).to(dtype)
+    y.backward(gy.to(DEV))
+    # (4-D tensors give the 2-D layer)
+    gx, goff, gm, gw, gb = oracle.dcn3d_backward(x, off, mask, w, gy, True, 1, 1, 1, groups, 1)
+    tol = BWD_TOL[dtype]
+    assert_close(xs.grad, gx, tol, "grad input")
+    assert_close(offs.grad, goff, tol, "grad offset")
+    assert_close(ms.grad, gm, tol, "grad mask")
+    assert_close(ws.grad, gw, tol, "grad weight")
+
+
 def test_input_gradient_through_lds_tiles_5x5x5(ops, oracle):
     """125 taps: 32 000 terms per tile voxel, the fixed-point scale leaves room for them."""
     from medvision_amd.ops.modulated_deform_conv_3d import modulated_deform_conv
