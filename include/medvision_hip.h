@@ -97,11 +97,14 @@ size_t mv_roi_align_backward_workspace_bytes(int dtype, int batch, int channels,
  * results, slower), never an access beyond `workspace_bytes`.  ndim = 2 or 3 (out_d ignored for 2). */
 size_t mv_roi_align_forward_workspace_bytes(int dtype, int ndim, int channels, int num_rois,
                                             int out_d, int out_h, int out_w, int sampling_ratio);
-/* The same query with the input's shape: at least the value above, and for fp16 detection heads
- * (plain rois, outputs of up to 8 cells per axis, about as many pooled outputs as input voxels or
- * more, width a multiple of four) the size of a re-ordered copy of the features that
+/* The same query with the input's shape: the value above when it is not 0; otherwise, for fp16
+ * detection heads (plain rois, outputs of up to 8 cells per axis, about as many pooled outputs as
+ * input voxels or more, width a multiple of four) the size of a re-ordered copy of the features that
  * mv_roi_align_2d_forward / _3d_forward then read instead of the input (a few voxels of a box row no
- * longer cost a whole memory sector each).  Those two entry points make the copy only when
+ * longer cost a whole memory sector each); and for the heads those kernels do not take (rotated
+ * boxes, sampling grids above 4, more than 16 cells per axis; fp16 / bf16 / fp32 with channels in
+ * whole 16-byte pieces, at least as many samples as input voxels; plain and rotated entry points) the
+ * size of a channels-last copy of the features.  An entry point makes its copy only when
  * `workspace_bytes` is at least this value.  depth ignored for ndim 2.
  * No counterpart in the reference.                                                              */
 size_t mv_roi_align_forward_workspace_bytes_for_input(int dtype, int ndim, int batch, int channels, int depth,
