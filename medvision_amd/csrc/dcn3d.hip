@@ -298,12 +298,14 @@ bool dcn_mfma_backward_supported(const DcnDims &s, int dtype);
 size_t dcn_mfma_backward_workspace_bytes(const DcnDims &s, int dtype);
 int dcn_mfma_backward(const void *x, const void *off, const void *mask, const void *wt,
                       const void *gy, void *goff, void *gmask, const DcnDims &s, int dtype,
-                      void *workspace, float **gx32, float **gw32, float **gb32,
+                      void *workspace, bool want_bias, float **gx32, float **gw32, float **gb32,
                       hipStream_t stream);
 void dcn_set_column_budget(size_t bytes);
 size_t dcn_column_budget();
 int dcn_planar_add(const float *gxt, void *gx, const DcnDims &s, int dtype, hipStream_t stream);
 int dcn_weight_add(const float *acc, void *gw, const DcnDims &s, int dtype, hipStream_t stream);
+int dcn_backward_fold(const float *gxt, const float *gw32, const float *gb32, void *grad_input, void *grad_weight,
+                      void *grad_bias, const DcnDims &s, int dtype, hipStream_t stream);
 
 static inline int blocks_for(long n, int per_block, int cap) {
   return static_cast<int>(std::min<long>((n + per_block - 1) / per_block, cap));
@@ -469,7 +471,7 @@ static int dcn_backward_any(const void *input, const void *offset, const void *m
     }
     float *gx32, *gw32, *gb32;
     st = dcn_mfma_backward(xp, offset, mask, wsb + l.w, gyp, grad_offset, grad_mask, pad.p, dtype, wsb + l.inner,
-                           &gx32, &gw32, &gb32, hs);
+                           false, &gx32, &gw32, &gb32, hs);
     if (st) return st;
     st = dcn_planar_add_padded(gx32, grad_input, s, pad, dtype, hs);
     if (st) return st;
@@ -492,17 +494,15 @@ static int dcn_backward_any(const void *input, const void *offset, const void *m
   if (dcn_mfma_backward_supported(s, dtype)) {
     float *gx32, *gw32, *gb32;
     st = dcn_mfma_backward(input, offset, mask, weight, grad_output, grad_offset, grad_mask, s, dtype,
-                           workspace, &gx32, &gw32, &gb32, hs);
+                           workspace, grad_bias != nullptr, &gx32, &gw32, &gb32, hs);
     if (st) return st;
+    st = dcn_backward_fold(gx32, gw32, gb32, grad_input, grad_weight, grad_bias, s, dtype, hs);
+    if (st >= 0) return st;   // (one launch for the three folds; -1: not with these tensors)
     st = dcn_planar_add(gx32, grad_input, s, dtype, hs);
     if (st) return st;
     MV_DISPATCH(dtype, {
       if (sizeof(T) <= 4) {
-        using G = float;
-        if (grad_bias)
-          hipLaunchKernelGGL((dcn_backward_bias_kernel<T, G>), dim3(s.Cout, s.B, static_cast<unsigned>((s.Q + kBiasSlab - 1) / kBiasSlab)), dim3(256), 0, hs,
-                             static_cast<const T *>(grad_output), gb32, s);
-        if (grad_bias)
+        if (grad_bias)   // (the sums of grad_output are in the accumulator already)
           hipLaunchKernelGGL((dcn_add_from_f32_kernel<T>), dim3(1), dim3(256), 0, hs,
                              static_cast<T *>(grad_bias), gb32, static_cast<long>(s.Cout));
       }

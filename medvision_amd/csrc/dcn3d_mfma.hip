@@ -55,39 +55,6 @@ __global__ void dcn_channels_last_kernel(const U *__restrict__ x, U *__restrict_
   }
 }
 
-// The same move with 16-byte global accesses: rows of x are read as groups of 16 bytes (V
-// positions of one channel), kept in LDS as [channel][position], and every lane writes V channels
-// of one position.  Needs P and Cin to be multiples of V and 16-byte aligned tensors.
-constexpr int kLayoutPos = 128;
-template <typename U>
-__device__ __forceinline__ void channels_last_wide_block(const U *__restrict__ x, U *__restrict__ xt, int Cin, long P,
-                                                         unsigned bx, int b, int bz) {
-  constexpr int V = 16 / sizeof(U), CH = 256 / sizeof(U);   // CH channels per workgroup: 128 (2 bytes), 64 (4 bytes)
-  constexpr int PITCH = kLayoutPos + V;
-  __shared__ __attribute__((aligned(16))) U stage[CH * PITCH];
-  const long p0 = static_cast<long>(bx) * kLayoutPos;
-  const int c0 = bz * CH, cn = min(CH, Cin - c0);
-  const int np = static_cast<int>(min(static_cast<long>(kLayoutPos), P - p0));   // a multiple of V
-  const U *src = x + (static_cast<long>(b) * Cin + c0) * P + p0;
-  U *dst = xt + (static_cast<long>(b) * P + p0) * Cin + c0;
-  constexpr int PG = kLayoutPos / V;
-  for (int i = threadIdx.x; i < cn * PG; i += 256) {
-    const int c = i / PG, pg = i % PG;
-    if (pg * V < np)
-      *reinterpret_cast<u32x4 *>(stage + c * PITCH + pg * V) = *reinterpret_cast<const u32x4 *>(src + static_cast<long>(c) * P + pg * V);
-  }
-  __syncthreads();
-  const int cg_n = cn / V;
-  for (int i = threadIdx.x; i < np * cg_n; i += 256) {
-    const int pp = i / cg_n, cg = i % cg_n;
-    U out[V];
-#pragma unroll
-    for (int e = 0; e < V; e++) out[e] = stage[(cg * V + e) * PITCH + pp];
-    u32x4 packed;
-    __builtin_memcpy(&packed, out, 16);
-    *reinterpret_cast<u32x4 *>(dst + static_cast<long>(pp) * Cin + cg * V) = packed;
-  }
-}
 template <typename U>
 __global__ __launch_bounds__(256) void dcn_channels_last_wide_kernel(const U *__restrict__ x, U *__restrict__ xt,
                                                                      int Cin, long P) {

@@ -35,13 +35,11 @@ constexpr int kRsrcFlags = 0x00020000;
 // weight [Cout, cpg, K] -> B pieces [group][tap][32-channel block][row step][lane][kPiece]:
 // lane l, element i = Wt[g*opg + step*2*kPiece + (l/32)*kPiece + i, block*32 + l%32, k]
 template <typename T>
-__global__ __launch_bounds__(256) void dcn_weight_bfragments_kernel(const T *__restrict__ wt,
-                                                                    T *__restrict__ wb,
-                                                                    const DcnDims s) {
+__device__ __forceinline__ void dcn_weight_bfragments_block(const T *__restrict__ wt, T *__restrict__ wb, const DcnDims s, const unsigned bid) {
   constexpr int PC = Mfma<T>::kPiece;
   const int cblocks = s.cpg / 32, steps = s.opg / (2 * PC);
   const long total = static_cast<long>(s.groups) * s.K * cblocks * steps * 64;
-  const long id = blockIdx.x * 256L + threadIdx.x;
+  const long id = bid * 256L + threadIdx.x;
   if (id >= total) return;
   const int lane = id % 64;
   long r = id / 64;
@@ -53,6 +51,10 @@ __global__ __launch_bounds__(256) void dcn_weight_bfragments_kernel(const T *__r
   const int o = g * s.opg + st * 2 * PC + (lane / 32) * PC;
   for (int i = 0; i < PC; i++) wb[id * PC + i] = wt[(static_cast<long>(o + i) * s.cpg + cl) * s.K + k];
 }
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_weight_bfragments_kernel(const T *__restrict__ wt,
+                                                                    T *__restrict__ wb,
+                                                                    const DcnDims s) { dcn_weight_bfragments_block<T>(wt, wb, s, blockIdx.x); }
 
 // One element of x (channels-last) through a range-checked buffer load, as fp32.
 template <typename T>
@@ -149,11 +151,16 @@ __device__ __forceinline__ void fold_max(unsigned bits, unsigned *out) {
   __syncthreads();
   if (threadIdx.x == 0) {
     const unsigned m = max(max(part[0], part[1]), max(part[2], part[3]));
-    if (m) atomicMax(out, m);
+    // (atomics on one address retire one after the other: a workgroup that cannot raise the value it
+    // reads — possibly an older one, which is never above the current one — leaves it alone)
+    if (m > __hip_atomic_load(out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(out, m);
   }
 }
+// (block `bid` of `nblocks`: the kernels below call these bodies with their own block index or with a
+// share of a launch that does several small jobs at once)
 template <typename T>
-__global__ __launch_bounds__(256) void dcn_absmax_kernel(const T *__restrict__ p, long n, unsigned *out) {
+__device__ __forceinline__ void dcn_absmax_block(const T *__restrict__ p, long n, unsigned *out, const unsigned bid,
+                                                 const unsigned nblocks) {
   constexpr int V = 16 / sizeof(T);  // elements per 16-byte load
   float m = 0.f;
   bool bad = false;
@@ -163,9 +170,9 @@ __global__ __launch_bounds__(256) void dcn_absmax_kernel(const T *__restrict__ p
     m = fmaxf(m, v);
   };
   const long head = min(n, static_cast<long>((16 - reinterpret_cast<size_t>(p) % 16) % 16 / sizeof(T)));
-  const long groups = (n - head) / V, tid = blockIdx.x * 256L + threadIdx.x;
+  const long groups = (n - head) / V, tid = bid * 256L + threadIdx.x;
   // four independent loads per lane and step
-  for (long i = blockIdx.x * 1024L + threadIdx.x; i < groups; i += gridDim.x * 1024L) {
+  for (long i = bid * 1024L + threadIdx.x; i < groups; i += nblocks * 1024L) {
     union { u32x4 u; T e[V]; } piece[4];
 #pragma unroll
     for (int u = 0; u < 4; u++)
@@ -180,12 +187,16 @@ __global__ __launch_bounds__(256) void dcn_absmax_kernel(const T *__restrict__ p
   if (tid < n - tail) take(p[tail + tid]);
   fold_max(bad ? 0x7fc00000u : __float_as_uint(m), out);
 }
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_absmax_kernel(const T *__restrict__ p, long n, unsigned *out) {
+  dcn_absmax_block<T>(p, n, out, blockIdx.x, gridDim.x);
+}
 // max over (group, c, k) of sum_o |Wt[o, c, k]|: a workgroup takes 64 columns, its four wavefronts
 // a quarter of the rows each
 template <typename T>
-__global__ __launch_bounds__(256) void dcn_weight_colsum_kernel(const T *__restrict__ wt, const DcnDims s, unsigned *out) {
+__device__ __forceinline__ void dcn_weight_colsum_block(const T *__restrict__ wt, const DcnDims s, unsigned *out, const unsigned bid) {
   __shared__ float part[4][64];
-  const long cols = static_cast<long>(s.cpg) * s.K, id = blockIdx.x * 64L + threadIdx.x % 64;
+  const long cols = static_cast<long>(s.cpg) * s.K, id = bid * 64L + threadIdx.x % 64;
   const int wave = threadIdx.x / 64;
   float sum = 0.f;
   if (id < cols * s.groups) {
@@ -196,6 +207,10 @@ __global__ __launch_bounds__(256) void dcn_weight_colsum_kernel(const T *__restr
   __syncthreads();
   if (wave == 0) sum = part[0][threadIdx.x] + part[1][threadIdx.x] + part[2][threadIdx.x] + part[3][threadIdx.x];
   fold_max(wave == 0 ? (sum == sum ? __float_as_uint(sum) : 0x7fc00000u) : 0u, out);
+}
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_weight_colsum_kernel(const T *__restrict__ wt, const DcnDims s, unsigned *out) {
+  dcn_weight_colsum_block<T>(wt, s, out, blockIdx.x);
 }
 
 constexpr int kTapWords = 28;  // byte offsets of the corners in x [8] and in the gradient buffer [8], w[8], mask, ld, lh, lw
@@ -392,13 +407,11 @@ __global__ __launch_bounds__(256) void dcn_backward_data_mfma_kernel(
 // a [position][channel] LDS block so that an atomic instruction still adds 128 contiguous bytes:
 // the wavefront lists its far corners once per tap and walks the list two entries at a time.
 template <typename T>
-__global__ __launch_bounds__(256) void dcn_weight_afragments32_kernel(const T *__restrict__ wt,
-                                                                      T *__restrict__ wa,
-                                                                      const DcnDims s) {
+__device__ __forceinline__ void dcn_weight_afragments32_block(const T *__restrict__ wt, T *__restrict__ wa, const DcnDims s, const unsigned bid) {
   constexpr int PC = Mfma<T>::kPiece;
   const int cblocks = s.cpg / 32, steps = s.opg / (2 * PC);
   const long total = static_cast<long>(s.groups) * s.K * cblocks * steps * 64;
-  const long id = blockIdx.x * 256L + threadIdx.x;
+  const long id = bid * 256L + threadIdx.x;
   if (id >= total) return;
   const int lane = id % 64;
   long r = id / 64;
@@ -411,9 +424,13 @@ __global__ __launch_bounds__(256) void dcn_weight_afragments32_kernel(const T *_
   const int o = g * s.opg + st * 2 * PC + (lane / 32) * PC;
   for (int i = 0; i < PC; i++) wa[id * PC + i] = wt[(static_cast<long>(o + i) * s.cpg + cl) * s.K + k];
 }
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_weight_afragments32_kernel(const T *__restrict__ wt,
+                                                                      T *__restrict__ wa,
+                                                                      const DcnDims s) { dcn_weight_afragments32_block<T>(wt, wa, s, blockIdx.x); }
 
 template <typename T, typename S>
-__global__ __launch_bounds__(256, 3) void dcn_backward_data_lanes_kernel(
+__global__ __launch_bounds__(256, sizeof(T) == 2 ? 3 : 2) void dcn_backward_data_lanes_kernel(
     const T *__restrict__ xt, const T *__restrict__ off, const T *__restrict__ mask,
     const T *__restrict__ gyt, const T *__restrict__ wa, float *__restrict__ gxt,
     T *__restrict__ goff, T *__restrict__ gmask, const DcnDims s, const unsigned *__restrict__ bounds,
@@ -680,13 +697,11 @@ constexpr int kScatterKeep = 4;  // slices of grad_output a wavefront keeps in r
 // rows 4j, 4j + 1 and are not used), element i the output channel g*opg + step*4*kPiece +
 // (l/16)*kPiece + i
 template <typename T>
-__global__ __launch_bounds__(256) void dcn_weight_afragments8_kernel(const T *__restrict__ wt,
-                                                                     T *__restrict__ wa,
-                                                                     const DcnDims s) {
+__device__ __forceinline__ void dcn_weight_afragments8_block(const T *__restrict__ wt, T *__restrict__ wa, const DcnDims s, const unsigned bid) {
   constexpr int PC = Mfma<T>::kPiece;
   const int cblocks = s.cpg / 8, steps = s.opg / (4 * PC);
   const long total = static_cast<long>(s.groups) * s.K * cblocks * steps * 64;
-  const long id = blockIdx.x * 256L + threadIdx.x;
+  const long id = bid * 256L + threadIdx.x;
   if (id >= total) return;
   const int lane = id % 64;
   long r = id / 64;
@@ -698,6 +713,10 @@ __global__ __launch_bounds__(256) void dcn_weight_afragments8_kernel(const T *__
   const int o = g * s.opg + st * 4 * PC + (lane / 16) * PC;
   for (int i = 0; i < PC; i++) wa[id * PC + i] = wt[(static_cast<long>(o + i) * s.cpg + cl) * s.K + k];
 }
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_weight_afragments8_kernel(const T *__restrict__ wt,
+                                                                     T *__restrict__ wa,
+                                                                     const DcnDims s) { dcn_weight_afragments8_block<T>(wt, wa, s, blockIdx.x); }
 
 template <typename T, typename S>
 __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter_kernel(
@@ -891,13 +910,11 @@ __host__ __device__ constexpr int scatter32_shift(int terms) {
 // MFMA row l % 16 = channel l % 16 of the block, element i the output channel
 // g*opg + step*4*kPiece + (l/16)*kPiece + i
 template <typename T>
-__global__ __launch_bounds__(256) void dcn_weight_afragments16_kernel(const T *__restrict__ wt,
-                                                                      T *__restrict__ wa,
-                                                                      const DcnDims s) {
+__device__ __forceinline__ void dcn_weight_afragments16_block(const T *__restrict__ wt, T *__restrict__ wa, const DcnDims s, const unsigned bid) {
   constexpr int PC = Mfma<T>::kPiece;
   const int cblocks = s.cpg / 16, steps = s.opg / (4 * PC);
   const long total = static_cast<long>(s.groups) * s.K * cblocks * steps * 64;
-  const long id = blockIdx.x * 256L + threadIdx.x;
+  const long id = bid * 256L + threadIdx.x;
   if (id >= total) return;
   const int lane = id % 64;
   long r = id / 64;
@@ -909,6 +926,10 @@ __global__ __launch_bounds__(256) void dcn_weight_afragments16_kernel(const T *_
   const int o = g * s.opg + st * 4 * PC + (lane / 16) * PC;
   for (int i = 0; i < PC; i++) wa[id * PC + i] = wt[(static_cast<long>(o + i) * s.cpg + cl) * s.K + k];
 }
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_weight_afragments16_kernel(const T *__restrict__ wt,
+                                                                      T *__restrict__ wa,
+                                                                      const DcnDims s) { dcn_weight_afragments16_block<T>(wt, wa, s, blockIdx.x); }
 
 template <typename T, typename S>
 __global__ __launch_bounds__(kScatterWaves * 64) void dcn_backward_scatter32_kernel(
@@ -1368,13 +1389,12 @@ __global__ __launch_bounds__(256) void dcn_planar_add_kernel(const float *__rest
 // multiple of 64, 16-byte aligned tensors): a lane reads four channels of one position, then adds
 // V = 16 / sizeof(T) neighbouring positions of one channel to the gradient in one read-modify-write.
 template <typename T>
-__global__ __launch_bounds__(256) void dcn_planar_add_wide_kernel(const float *__restrict__ gxt,
-                                                                  T *__restrict__ gx, int C, long P) {
+__device__ __forceinline__ void dcn_planar_add_wide_block(const float *__restrict__ gxt, T *__restrict__ gx, int C, long P,
+                                                          const unsigned bx, const int b, const int bz) {
   constexpr int V = 16 / static_cast<int>(sizeof(T));
   __shared__ __attribute__((aligned(16))) float stagef[64][kAddChunk + 4];
-  const int b = blockIdx.y;
-  const long p0 = static_cast<long>(blockIdx.x) * 64;
-  const int c0 = blockIdx.z * kAddChunk, cn = min(kAddChunk, C - c0);   // cn: a multiple of 4
+  const long p0 = static_cast<long>(bx) * 64;
+  const int c0 = bz * kAddChunk, cn = min(kAddChunk, C - c0);   // cn: a multiple of 4
   const float *src = gxt + (static_cast<long>(b) * P + p0) * C + c0;
   float4 in[4];
 #pragma unroll
@@ -1404,11 +1424,120 @@ __global__ __launch_bounds__(256) void dcn_planar_add_wide_kernel(const float *_
     __builtin_nontemporal_store(piece.u, reinterpret_cast<u32x4 *>(d));
   }
 }
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_planar_add_wide_kernel(const float *__restrict__ gxt,
+                                                                  T *__restrict__ gx, int C, long P) {
+  dcn_planar_add_wide_block<T>(gxt, gx, C, P, blockIdx.x, blockIdx.y, blockIdx.z);
+}
 
-__global__ void dcn_zero_f32_kernel(float *p, long n) {
-  for (long i = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; i < n;
-       i += static_cast<long>(gridDim.x) * blockDim.x)
-    p[i] = 0.f;
+__device__ __forceinline__ void dcn_zero_f32_block(float *p, long n, const unsigned bid, const unsigned nblocks) {
+  for (long i = bid * 256L + threadIdx.x; i < n; i += nblocks * 256L) p[i] = 0.f;
+}
+__global__ __launch_bounds__(256) void dcn_zero_f32_kernel(float *p, long n) { dcn_zero_f32_block(p, n, blockIdx.x, gridDim.x); }
+
+// One pass over a slab of grad_output[b, o, .]: its sum into the fp32 bias accumulator and (`out`
+// given) its largest magnitude as a bit pattern into *out.  Workgroup = (o, b, slab of `slab_len`
+// positions); about 512 workgroups in all — enough loads in flight for the memory system, and few enough
+// for the atomics on the one word of the maximum, which retire one after the other (~10 ns each).
+static long gy_slab_len(const DcnDims &s) {
+  const long rows = static_cast<long>(s.Cout) * s.B;
+  const long slabs = std::max(1L, std::min((s.Q + 2047) / 2048, (512 + rows - 1) / rows));
+  return ((s.Q + slabs - 1) / slabs + 1023) / 1024 * 1024;
+}
+template <typename T>
+__device__ __forceinline__ void dcn_gy_sum_max_block(const T *__restrict__ gy, float *__restrict__ gb32, unsigned *out,
+                                                     const DcnDims s, const long slab_len, const unsigned bid) {
+  constexpr int V = 16 / static_cast<int>(sizeof(T));
+  __shared__ float sums[4];
+  const unsigned slabs = static_cast<unsigned>((s.Q + slab_len - 1) / slab_len);
+  const unsigned slab = bid % slabs, r = bid / slabs;
+  const int b = static_cast<int>(r % s.B), o = static_cast<int>(r / s.B);
+  const T *src = gy + (static_cast<long>(b) * s.Cout + o) * s.Q;
+  long q0 = static_cast<long>(slab) * slab_len;
+  const long q_end = min(q0 + slab_len, s.Q);
+  float v = 0.f, m = 0.f;
+  bool bad = false;
+  auto take = [&](T e) {
+    const float x = static_cast<float>(load(&e));
+    v += x;
+    bad = bad || !(x == x);
+    m = fmaxf(m, fabsf(x));
+  };
+  if (reinterpret_cast<uintptr_t>(src + q0) % 16 == 0) {
+    // 16-byte pieces, four independent loads per lane and step
+    const long groups = (q_end - q0) / V;
+    const u32x4 *pieces = reinterpret_cast<const u32x4 *>(src + q0);
+    for (long i = threadIdx.x; i < groups; i += 1024) {
+      union { u32x4 u; T e[V]; } raw[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) raw[u].u = i + u * 256 < groups ? pieces[i + u * 256] : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int u = 0; u < 4; u++)
+#pragma unroll
+        for (int e = 0; e < V; e++) take(raw[u].e[e]);
+    }
+    q0 += groups * V;
+  }
+  for (long q = q0 + threadIdx.x; q < q_end; q += 256) take(src[q]);
+  for (int sh = 32; sh > 0; sh >>= 1) v += __shfl_xor(v, sh);
+  if (threadIdx.x % kWave == 0) sums[threadIdx.x / kWave] = v;
+  if (out) fold_max(bad ? 0x7fc00000u : __float_as_uint(m), out);   // (contains the barrier)
+  else __syncthreads();
+  if (threadIdx.x == 0) atomicAdd(gb32 + o, (sums[0] + sums[1]) + (sums[2] + sums[3]));
+}
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_gy_sum_kernel(const T *__restrict__ gy, float *__restrict__ gb32, const DcnDims s,
+                                                         const long slab_len) {
+  dcn_gy_sum_max_block<T>(gy, gb32, nullptr, s, slab_len, blockIdx.x);
+}
+
+// The small jobs in front of the data kernel of a layer with tiles, in two launches instead of eight
+// (a dependent launch costs ~2.7 us before its first instruction, and kernels of a few microseconds do
+// not fill the machine): first the two layout passes, the weight fragments and the zero fill of the
+// accumulators and of the maxima's words; then the maxima, which need those words at zero.
+struct PrepareJobs {
+  unsigned x_end, gy_end, f32_end, fsc_end, zero_end;   // block ranges of the first launch
+  unsigned wbx, wbq;                                    // 128-position blocks of the input / the output
+  int wide16;                                           // scatter fragments: 16-channel blocks (else 8)
+};
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_backward_prepare_kernel(const T *__restrict__ x, T *__restrict__ xt,
+                                                                   const T *__restrict__ gy, T *__restrict__ gyt,
+                                                                   const T *__restrict__ wt, T *__restrict__ wb,
+                                                                   T *__restrict__ wa, float *__restrict__ zero,
+                                                                   const long nz, const DcnDims s, const PrepareJobs j) {
+  using U = typename std::conditional<(sizeof(T) == 2), unsigned short, unsigned int>::type;
+  const unsigned id = blockIdx.x;
+  if (id < j.x_end) {
+    channels_last_wide_block<U>(reinterpret_cast<const U *>(x), reinterpret_cast<U *>(xt), s.Cin, s.P, id % j.wbx,
+                                static_cast<int>((id / j.wbx) % s.B), static_cast<int>(id / (j.wbx * s.B)));
+  } else if (id < j.gy_end) {
+    const unsigned r = id - j.x_end;
+    channels_last_wide_block<U>(reinterpret_cast<const U *>(gy), reinterpret_cast<U *>(gyt), s.Cout, s.Q, r % j.wbq,
+                                static_cast<int>((r / j.wbq) % s.B), static_cast<int>(r / (j.wbq * s.B)));
+  } else if (id < j.f32_end) {
+    dcn_weight_afragments32_block<T>(wt, wb, s, id - j.gy_end);
+  } else if (id < j.fsc_end) {
+    if (j.wide16) dcn_weight_afragments16_block<T>(wt, wa, s, id - j.f32_end);
+    else dcn_weight_afragments8_block<T>(wt, wa, s, id - j.f32_end);
+  } else {
+    dcn_zero_f32_block(zero, nz, id - j.fsc_end, j.zero_end - j.fsc_end);
+  }
+}
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_backward_maxima_kernel(const T *__restrict__ gy, const long ngy,
+                                                                  const T *__restrict__ mask, const long nmask,
+                                                                  const T *__restrict__ wt, const DcnDims s,
+                                                                  unsigned *__restrict__ bounds, float *__restrict__ gb32,
+                                                                  const long slab_len, const unsigned gy_blocks,
+                                                                  const unsigned mask_blocks) {
+  const unsigned id = blockIdx.x;
+  if (id < gy_blocks) {
+    // with a bias gradient to form the pass over grad_output also sums it, a workgroup per (o, b, slab)
+    if (gb32) dcn_gy_sum_max_block<T>(gy, gb32, bounds, s, slab_len, id);
+    else dcn_absmax_block<T>(gy, ngy, bounds, id, gy_blocks);
+  } else if (id < gy_blocks + mask_blocks) dcn_absmax_block<T>(mask, nmask, bounds + 2, id - gy_blocks, mask_blocks);
+  else dcn_weight_colsum_block<T>(wt, s, bounds + 1, id - gy_blocks - mask_blocks);
 }
 
 // The LDS scatter pays when its tile holds the reach of a brick's undeformed taps with a voxel to
@@ -1481,57 +1610,93 @@ size_t dcn_mfma_backward_workspace_bytes(const DcnDims &s, int dtype) { return b
 template <typename T>
 static int backward_run(const void *x, const void *off, const void *mask, const void *wt,
                         const void *gy, void *goff, void *gmask, const DcnDims &s, void *workspace,
-                        float **gx32, float **gw32, float **gb32, int dtype, hipStream_t stream) {
+                        float **gx32, float **gw32, float **gb32, int dtype, bool want_bias, hipStream_t stream) {
   const BackwardLayout l = backward_layout(s, dtype);
   char *ws = static_cast<char *>(workspace);
   T *xt = reinterpret_cast<T *>(ws + l.xt), *gyt = reinterpret_cast<T *>(ws + l.gyt), *wb = reinterpret_cast<T *>(ws + l.wb);
   float *gxt = reinterpret_cast<float *>(ws + l.gxt);
   T *col = l.qp ? reinterpret_cast<T *>(ws + l.col) : nullptr;
   *gx32 = gxt; *gw32 = reinterpret_cast<float *>(ws + l.gw); *gb32 = reinterpret_cast<float *>(ws + l.gb);
-  int st = dcn_channels_last(x, xt, s.B, s.Cin, s.P, sizeof(T), stream);
-  if (st) return st;
-  st = dcn_channels_last(gy, gyt, s.B, s.Cout, s.Q, sizeof(T), stream);
-  if (st) return st;
   const bool image = s.nd == 2;
   const bool tiles = image ? scatter_tile_applies<ImageBricks>(s, dtype) : scatter_tile_applies<VolumeBricks>(s, dtype);
+  // 16-bit tensors: 32-bit cells and 16 channels per workgroup, while a term keeps enough bits
+  const int terms = (image ? ImageBricks::BD * ImageBricks::BH * ImageBricks::BW
+                           : VolumeBricks::BD * VolumeBricks::BH * VolumeBricks::BW) * s.K;
+  const bool narrow = sizeof(T) == 2 && scatter32_shift(terms) >= kScatter32MinShift;
+  const int wch = narrow ? 16 : 8;
+  T *wa = reinterpret_cast<T *>(ws + l.wa);
+  unsigned *bounds = reinterpret_cast<unsigned *>(ws + l.bounds);
   // 32-channel weight fragments: B operands (columns = channels) for the data kernel with a channel
   // per lane, A operands (rows = channels) for the one with a position per lane
   const long frag_lanes = static_cast<long>(s.groups) * s.K * (s.cpg / 32) * (s.opg / (2 * Mfma<T>::kPiece)) * 64;
-  if (tiles)
-    hipLaunchKernelGGL((dcn_weight_afragments32_kernel<T>), dim3(static_cast<unsigned>((frag_lanes + 255) / 256)),
-                       dim3(256), 0, stream, static_cast<const T *>(wt), wb, s);
-  else
-    hipLaunchKernelGGL((dcn_weight_bfragments_kernel<T>), dim3(static_cast<unsigned>((frag_lanes + 255) / 256)),
-                       dim3(256), 0, stream, static_cast<const T *>(wt), wb, s);
+  const long scatter_lanes = static_cast<long>(s.groups) * s.K * (s.cpg / wch) * (s.opg / (4 * Mfma<T>::kPiece)) * 64;
   const long nz = static_cast<long>((l.total - l.gxt) / 4);
-  hipLaunchKernelGGL(dcn_zero_f32_kernel, dim3(static_cast<unsigned>(min((nz + 1023) / 1024, 65536L))), dim3(256),
-                     0, stream, gxt, nz);
+  const long ngy = static_cast<long>(s.B) * s.Cout * s.Q, nmask = static_cast<long>(s.B) * s.dg * s.K * s.Q;
+  const long ncols = static_cast<long>(s.groups) * s.cpg * s.K;
+  constexpr int V = 16 / static_cast<int>(sizeof(T)), CH = 256 / static_cast<int>(sizeof(T));
+  auto aligned16 = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  const long wbx = (s.P + kLayoutPos - 1) / kLayoutPos, wbq = (s.Q + kLayoutPos - 1) / kLayoutPos;
+  const long nx = wbx * s.B * ((s.Cin + CH - 1) / CH), ngyb = wbq * s.B * ((s.Cout + CH - 1) / CH);
+  const long nf32 = (frag_lanes + 255) / 256, nfsc = (scatter_lanes + 255) / 256, nzb = min((nz + 1023) / 1024, 4096L);
+  int st = MV_OK;
+  bool bias_summed = false;
+  if (tiles && aligned16(x) && aligned16(xt) && aligned16(gy) && aligned16(gyt) && s.P % V == 0 && s.Q % V == 0 &&
+      s.Cin % V == 0 && s.Cout % V == 0 && nx + ngyb + nf32 + nfsc + nzb < (1L << 31)) {
+    PrepareJobs j;
+    j.x_end = static_cast<unsigned>(nx); j.gy_end = j.x_end + static_cast<unsigned>(ngyb);
+    j.f32_end = j.gy_end + static_cast<unsigned>(nf32); j.fsc_end = j.f32_end + static_cast<unsigned>(nfsc);
+    j.zero_end = j.fsc_end + static_cast<unsigned>(nzb);
+    j.wbx = static_cast<unsigned>(wbx); j.wbq = static_cast<unsigned>(wbq); j.wide16 = narrow;
+    hipLaunchKernelGGL((dcn_backward_prepare_kernel<T>), dim3(j.zero_end), dim3(256), 0, stream, static_cast<const T *>(x), xt,
+                       static_cast<const T *>(gy), gyt, static_cast<const T *>(wt), wb, wa, gxt, nz, s, j);
+    const long slab_len = gy_slab_len(s);
+    const long sum_blocks = static_cast<long>(s.Cout) * s.B * ((s.Q + slab_len - 1) / slab_len);
+    const bool sums = want_bias && sum_blocks < (1L << 30);
+    const unsigned gy_blocks = sums ? static_cast<unsigned>(sum_blocks) : static_cast<unsigned>(min((ngy + 8191) / 8192, 256L));
+    const unsigned mask_blocks = mask ? static_cast<unsigned>(min((nmask + 8191) / 8192, 256L)) : 0u;
+    hipLaunchKernelGGL((dcn_backward_maxima_kernel<T>), dim3(gy_blocks + mask_blocks + static_cast<unsigned>((ncols + 63) / 64)),
+                       dim3(256), 0, stream, static_cast<const T *>(gy), ngy, static_cast<const T *>(mask), nmask,
+                       static_cast<const T *>(wt), s, bounds, sums ? *gb32 : nullptr, slab_len, gy_blocks, mask_blocks);
+    bias_summed = sums;
+  } else {
+    st = dcn_channels_last(x, xt, s.B, s.Cin, s.P, sizeof(T), stream);
+    if (st) return st;
+    st = dcn_channels_last(gy, gyt, s.B, s.Cout, s.Q, sizeof(T), stream);
+    if (st) return st;
+    if (tiles)
+      hipLaunchKernelGGL((dcn_weight_afragments32_kernel<T>), dim3(static_cast<unsigned>(nf32)), dim3(256), 0, stream,
+                         static_cast<const T *>(wt), wb, s);
+    else
+      hipLaunchKernelGGL((dcn_weight_bfragments_kernel<T>), dim3(static_cast<unsigned>(nf32)), dim3(256), 0, stream,
+                         static_cast<const T *>(wt), wb, s);
+    hipLaunchKernelGGL(dcn_zero_f32_kernel, dim3(static_cast<unsigned>(min((nz + 1023) / 1024, 65536L))), dim3(256),
+                       0, stream, gxt, nz);
+    if (tiles) {
+      hipLaunchKernelGGL((dcn_absmax_kernel<T>), dim3(static_cast<unsigned>(min((ngy + 8191) / 8192, 256L))), dim3(256),
+                         0, stream, static_cast<const T *>(gy), ngy, bounds);
+      hipLaunchKernelGGL((dcn_weight_colsum_kernel<T>), dim3(static_cast<unsigned>((ncols + 63) / 64)), dim3(256), 0,
+                         stream, static_cast<const T *>(wt), s, bounds + 1);
+      if (mask)
+        hipLaunchKernelGGL((dcn_absmax_kernel<T>), dim3(static_cast<unsigned>(min((nmask + 8191) / 8192, 256L))),
+                           dim3(256), 0, stream, static_cast<const T *>(mask), nmask, bounds + 2);
+      if (narrow)
+        hipLaunchKernelGGL((dcn_weight_afragments16_kernel<T>), dim3(static_cast<unsigned>(nfsc)), dim3(256), 0, stream,
+                           static_cast<const T *>(wt), wa, s);
+      else
+        hipLaunchKernelGGL((dcn_weight_afragments8_kernel<T>), dim3(static_cast<unsigned>(nfsc)), dim3(256), 0, stream,
+                           static_cast<const T *>(wt), wa, s);
+    }
+  }
+  if (want_bias && !bias_summed) {
+    const long slab_len = gy_slab_len(s);
+    const long sum_blocks = static_cast<long>(s.Cout) * s.B * ((s.Q + slab_len - 1) / slab_len);
+    MV_REQUIRE(sum_blocks < (1L << 31), "grid too large");
+    hipLaunchKernelGGL((dcn_gy_sum_kernel<T>), dim3(static_cast<unsigned>(sum_blocks)), dim3(256), 0, stream,
+                       static_cast<const T *>(gy), *gb32, s, slab_len);
+  }
   const long qblocks = (s.Q + 127) / 128;
   MV_REQUIRE(qblocks < (1L << 31), "grid too large");
   if (tiles) {
-    unsigned *bounds = reinterpret_cast<unsigned *>(ws + l.bounds);
-    const long ngy = static_cast<long>(s.B) * s.Cout * s.Q, nmask = static_cast<long>(s.B) * s.dg * s.K * s.Q;
-    const long ncols = static_cast<long>(s.groups) * s.cpg * s.K;
-    hipLaunchKernelGGL((dcn_absmax_kernel<T>), dim3(static_cast<unsigned>(min((ngy + 8191) / 8192, 256L))), dim3(256),
-                       0, stream, static_cast<const T *>(gy), ngy, bounds);
-    hipLaunchKernelGGL((dcn_weight_colsum_kernel<T>), dim3(static_cast<unsigned>((ncols + 63) / 64)), dim3(256), 0,
-                       stream, static_cast<const T *>(wt), s, bounds + 1);
-    if (mask)
-      hipLaunchKernelGGL((dcn_absmax_kernel<T>), dim3(static_cast<unsigned>(min((nmask + 8191) / 8192, 256L))),
-                         dim3(256), 0, stream, static_cast<const T *>(mask), nmask, bounds + 2);
-    T *wa = reinterpret_cast<T *>(ws + l.wa);
-    // 16-bit tensors: 32-bit cells and 16 channels per workgroup, while a term keeps enough bits
-    const int terms = (image ? ImageBricks::BD * ImageBricks::BH * ImageBricks::BW
-                             : VolumeBricks::BD * VolumeBricks::BH * VolumeBricks::BW) * s.K;
-    const bool narrow = sizeof(T) == 2 && scatter32_shift(terms) >= kScatter32MinShift;
-    const int wch = narrow ? 16 : 8;
-    const long lanes = static_cast<long>(s.groups) * s.K * (s.cpg / wch) * (s.opg / (4 * Mfma<T>::kPiece)) * 64;
-    if (narrow)
-      hipLaunchKernelGGL((dcn_weight_afragments16_kernel<T>), dim3(static_cast<unsigned>((lanes + 255) / 256)),
-                         dim3(256), 0, stream, static_cast<const T *>(wt), wa, s);
-    else
-      hipLaunchKernelGGL((dcn_weight_afragments8_kernel<T>), dim3(static_cast<unsigned>((lanes + 255) / 256)),
-                         dim3(256), 0, stream, static_cast<const T *>(wt), wa, s);
     MV_REQUIRE(s.Cin / 8 <= 65535, "grid too large");
 #define MV_LAUNCH_SPLIT(S)                                                                                        \
   {                                                                                                               \
@@ -1585,17 +1750,18 @@ static int backward_run(const void *x, const void *off, const void *mask, const 
 }
 
 // Runs the data and weight kernels; grad_offset / grad_mask are written, the fp32 gradients of
-// input (channels-last; dcn_planar_add), weight (tap-major; dcn_weight_add) and bias accumulators
-// are returned for the caller to fold in.
+// input (channels-last; dcn_planar_add) and weight (tap-major; dcn_weight_add) and the bias
+// accumulator (zero; with `want_bias` the sums of grad_output over samples and positions) are returned
+// for the caller to fold in.
 int dcn_mfma_backward(const void *x, const void *off, const void *mask, const void *wt,
                       const void *gy, void *goff, void *gmask, const DcnDims &s, int dtype,
-                      void *workspace, float **gx32, float **gw32, float **gb32,
+                      void *workspace, bool want_bias, float **gx32, float **gw32, float **gb32,
                       hipStream_t stream) {
   if (dtype == MV_F16)
-    return backward_run<__half>(x, off, mask, wt, gy, goff, gmask, s, workspace, gx32, gw32, gb32, dtype, stream);
+    return backward_run<__half>(x, off, mask, wt, gy, goff, gmask, s, workspace, gx32, gw32, gb32, dtype, want_bias, stream);
   if (dtype == MV_F32)
-    return backward_run<float>(x, off, mask, wt, gy, goff, gmask, s, workspace, gx32, gw32, gb32, dtype, stream);
-  return backward_run<__hip_bfloat16>(x, off, mask, wt, gy, goff, gmask, s, workspace, gx32, gw32, gb32, dtype, stream);
+    return backward_run<float>(x, off, mask, wt, gy, goff, gmask, s, workspace, gx32, gw32, gb32, dtype, want_bias, stream);
+  return backward_run<__hip_bfloat16>(x, off, mask, wt, gy, goff, gmask, s, workspace, gx32, gw32, gb32, dtype, want_bias, stream);
 }
 
 // dst [B, C, P] (element type of `dtype`) += src [B, P, C] fp32
@@ -1630,13 +1796,60 @@ int planar_add_f32(const float *src, void *dst, int B, int C, long P, int dtype,
 
 // grad_weight [Cout][cpg][K] += the tap-major fp32 accumulator [K][Cout][cpg] of the weight kernel
 template <typename T>
-__global__ __launch_bounds__(256) void dcn_weight_add_kernel(const float *__restrict__ acc, T *__restrict__ gw,
-                                                             const DcnDims s) {
+__device__ __forceinline__ void dcn_weight_add_block(const float *__restrict__ acc, T *__restrict__ gw, const DcnDims s,
+                                                     const unsigned bid, const unsigned nblocks) {
   const long n = static_cast<long>(s.Cout) * s.cpg * s.K;
-  for (long i = blockIdx.x * 256L + threadIdx.x; i < n; i += gridDim.x * 256L) {
+  for (long i = bid * 256L + threadIdx.x; i < n; i += nblocks * 256L) {
     const long k = i % s.K, oc = i / s.K;
     gw[i] = store_cast<T>(load(gw + i) + acc[k * s.Cout * s.cpg + oc]);
   }
+}
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_weight_add_kernel(const float *__restrict__ acc, T *__restrict__ gw,
+                                                             const DcnDims s) {
+  dcn_weight_add_block<T>(acc, gw, s, blockIdx.x, gridDim.x);
+}
+
+// The folds behind the backward kernels in one launch: channels-last fp32 grad input -> grad_input,
+// tap-major fp32 grad weight -> grad_weight, the fp32 bias sums -> grad_bias.
+template <typename T>
+__global__ __launch_bounds__(256) void dcn_backward_fold_kernel(const float *__restrict__ gxt, T *__restrict__ gx,
+                                                                const float *__restrict__ gw32, T *__restrict__ gw,
+                                                                const float *__restrict__ gb32, T *__restrict__ gb,
+                                                                const DcnDims s, const unsigned pblocks,
+                                                                const unsigned add_end, const unsigned weight_end) {
+  const unsigned id = blockIdx.x;
+  if (id < add_end)
+    dcn_planar_add_wide_block<T>(gxt, gx, s.Cin, s.P, id % pblocks, static_cast<int>((id / pblocks) % s.B),
+                                 static_cast<int>(id / (pblocks * s.B)));
+  else if (id < weight_end)
+    dcn_weight_add_block<T>(gw32, gw, s, id - add_end, weight_end - add_end);
+  else
+    for (int o = threadIdx.x; o < s.Cout; o += 256) gb[o] = store_cast<T>(static_cast<float>(load(gb + o)) + gb32[o]);
+}
+
+// All three folds of a layer on the matrix-core path.  Returns -1 when the tensors do not allow the
+// 16-byte accesses of the one-launch form (the caller then folds one by one).
+int dcn_backward_fold(const float *gxt, const float *gw32, const float *gb32, void *grad_input, void *grad_weight,
+                      void *grad_bias, const DcnDims &s, int dtype, hipStream_t stream) {
+  if (dtype != MV_F16 && dtype != MV_BF16 && dtype != MV_F32) return -1;
+  auto aligned16 = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  if (s.P % 64 || s.Cin % 4 || !aligned16(gxt) || !aligned16(grad_input)) return -1;
+  const long pblocks = s.P / 64, add_blocks = pblocks * s.B * ((s.Cin + kAddChunk - 1) / kAddChunk);
+  const long n = static_cast<long>(s.Cout) * s.cpg * s.K, weight_blocks = min((n + 255) / 256, 1024L);
+  const long bias_blocks = grad_bias ? 1 : 0;
+  if (add_blocks + weight_blocks + bias_blocks >= (1L << 31)) return -1;
+  const unsigned add_end = static_cast<unsigned>(add_blocks), weight_end = add_end + static_cast<unsigned>(weight_blocks);
+#define MV_FOLD(T)                                                                                                  \
+  hipLaunchKernelGGL((dcn_backward_fold_kernel<T>), dim3(weight_end + static_cast<unsigned>(bias_blocks)), dim3(256), 0, \
+                     stream, gxt, static_cast<T *>(grad_input), gw32, static_cast<T *>(grad_weight),               \
+                     gb32, static_cast<T *>(grad_bias), s,                                                         \
+                     static_cast<unsigned>(pblocks), add_end, weight_end)
+  if (dtype == MV_F16) MV_FOLD(__half);
+  else if (dtype == MV_BF16) MV_FOLD(__hip_bfloat16);
+  else MV_FOLD(float);
+#undef MV_FOLD
+  return check_launch("dcn_backward_fold_kernel");
 }
 int dcn_weight_add(const float *acc, void *gw, const DcnDims &s, int dtype, hipStream_t stream) {
   const long n = static_cast<long>(s.Cout) * s.cpg * s.K;
