@@ -195,6 +195,18 @@ def bench_other_configs(args):
     gi = torch.zeros_like(feat)
     bms, _ = _events_ms(lambda i: _C.roi_align_rotated_3d_backward(gy, rois, gi, 7, 7, 7, 1.0, 2, True, 1), 10, 2)
     res["rotated_head_1000x64x7^3_fp16"] = {"forward_ms": round(ms, 4), "backward_ms": round(bms, 4)}
+    del feat, out, gy, gi
+    # RandomAffine on images: fp16 [8,3,512,512], one full-image rotated roi per sample (the tiled kernel with
+    # the image rows as slices)
+    g = wl.gen(10)
+    img = torch.randn(8, 3, 512, 512, generator=g).half().to(dev)
+    ang = (torch.rand(8, 1, generator=g) * 2 - 1) * math.radians(30)
+    sc = 0.8 + torch.rand(8, 1, generator=g) * 0.4
+    sh = (torch.rand(8, 2, generator=g) * 2 - 1) * 10
+    rois = torch.cat([torch.arange(8, dtype=torch.float32)[:, None], 256 + sh, 512 / sc.expand(8, 2), ang], 1).to(dev)
+    ms, _ = _events_ms(lambda i: ops.affine_2d(img, rois, (512, 512), 1.0, 1, True, 1), 100, 10)
+    res["affine_2d_8x3x512^2_fp16"] = {"ms": round(ms, 4), "gpix_s": round(img.numel() / ms / 1e6, 2),
+                                       "gbps": round(2 * img.numel() * 2 / ms / 1e6, 1)}
     return res
 
 

@@ -320,17 +320,46 @@ def test_tiled_resampler_shapes(ops, oracle, dtype, channels, rois_n, size, out,
         assert frac < 1e-4, f"nearest mismatches: {frac:.2e}"
 
 
-def test_tiled_resampler_2d(ops, oracle):
-    """2-D images of resampling size (they take the one-thread-per-output kernel: a tile of depth 1
-    gives a lane a single pixel per item)."""
-    g = wl.gen(37)
-    img = torch.randn(2, 3, 96, 120, generator=g).half()
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width", [120, 123])
+def test_tiled_resampler_2d(ops, oracle, dtype, width):
+    """Images of resampling size run the tiled kernel as volumes whose slices are the image rows (the
+    rois are rewritten on the device: one cell on the middle axis that samples row 0, the rotation about
+    that axis): rotated rois beyond every border, both `aligned` settings, a spatial scale that is no
+    power of two, orders 0 and 1, rows of whole 16-byte groups and ragged ones, plain boxes, several
+    channels; order 3 stays on the one-thread-per-output kernel."""
+    g = wl.gen(37 + width)
+    img = torch.randn(2, 3, 96, width, generator=g).to(dtype)
     rois = torch.tensor([[0, 60.3, 47.1, 130.0, 90.0, 0.4], [1, 50.0, 40.0, 70.0, 110.0, -0.7],
-                         [0, 10.0, 90.0, 60.0, 60.0, 1.3]], dtype=torch.float32)
+                         [0, 10.0, 90.0, 60.0, 60.0, 1.3], [1, 61.3, 48.2, 121.0, 97.0, 0.0]], dtype=torch.float32)
+    x, r = img.to(DEV), rois.to(DEV)
+    out = (80, 96)
+    for aligned in (True, False):
+        for scale in (1.0, 0.3):
+            rs = rois.clone()
+            rs[:, 1:5] /= scale
+            got = ops.RoIAlignRotated(out, scale, 1, aligned)(x, rs.to(DEV))
+            want = oracle.roi_align_forward(img, rs, out, scale, 1, aligned, 1, True)
+            assert float(want.abs().max()) > 0.5
+            assert_close(got, want, FWD_TOL[dtype], f"image tiles, aligned {aligned}, scale {scale}")
     for order in (1, 3):
-        got = ops.affine_2d(img.to(DEV), rois.to(DEV), (80, 96), 1.0, 1, True, order)
-        want = oracle.roi_align_forward(img, rois, (80, 96), 1.0, 1, True, order, True)
-        assert_close(got, want, FWD_TOL[torch.float16], f"tiled 2-D forward, order {order}")
+        got = ops.affine_2d(x, r, out, 1.0, 1, True, order)
+        want = oracle.roi_align_forward(img, rois, out, 1.0, 1, True, order, True)
+        assert_close(got, want, FWD_TOL[dtype], f"affine_2d, order {order}")
+    got = ops.affine_2d(x, r, out, 1.0, 1, True, 0)
+    want = oracle.roi_align_forward(img, rois, out, 1.0, 1, True, 0, True)
+    margin = oracle.roi_decision_margin(img.shape, rois, out, 1.0, 1, True, True)
+    frac = assert_nearest(got, want, margin, dtype, "image tiles, nearest")
+    assert frac < 2e-4, f"nearest mismatches: {frac:.2e}"
+    # an identity roi copies the image (rows as slices: the output's rows are the volume's slices)
+    ident = torch.tensor([[b, width / 2, 48, width, 96, 0] for b in range(2)], dtype=torch.float32)
+    same = ops.affine_2d(x, ident.to(DEV), (96, width), 1.0, 1, True, 1)
+    assert torch.equal(same.cpu(), img)
+    # plain boxes with one sample per cell
+    boxes = torch.tensor([[0, 3.2, 1.7, 100.4, 80.9], [1, -10.0, 20.0, 60.0, 120.0]], dtype=torch.float32)
+    got = ops.RoIAlign(out, 1.0, 1)(x, boxes.to(DEV))
+    want = oracle.roi_align_forward(img, boxes, out, 1.0, 1, True, 1, False)
+    assert_close(got, want, FWD_TOL[dtype], "plain boxes")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
