@@ -88,8 +88,9 @@ int mv_roi_align_rotated_3d_backward(const void *grad_output, const void *rois, 
                                      int order, void *workspace, void *stream);
 size_t mv_roi_align_backward_workspace_bytes(int dtype, int batch, int channels, int depth,
                                              int height, int width);
-/* Workspace of the forward entry points (plain, rotated and affine).  0 for a sampling grid of 1
- * (the kernels keep their per-call state in LDS); for fp16 / fp32 outputs of resampling size with a
+/* Workspace of the forward entry points (plain, rotated and affine).  0 for a sampling grid of 1 on
+ * volumes (the kernels keep their per-call state in LDS), 40 bytes per roi for images of resampling
+ * size (orders 0 / 1: their rois are rewritten for the tiled kernel); for fp16 / fp32 outputs of resampling size with a
  * fixed sampling_ratio of 2..4 the bytes of the bins' samples (sampling_ratio^ndim per output
  * element), which a second pass averages.  The forward entry points take the workspace together
  * with its size in bytes (`workspace_bytes`) and use a path only when the workspace holds what that
