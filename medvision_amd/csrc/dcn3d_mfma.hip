@@ -412,7 +412,18 @@ __global__ __launch_bounds__(256, 5) void dcn_forward_shared_taps_kernel(
   const int j = lane % 16, kc = lane / 16;   // matrix layout: position (column) and piece of this lane
   const int lj = lane / 4, lk = lane % 4;    // load layout
   const int from = (4 * j + kc) * 4;         // ds_bpermute byte address of the lane holding this lane's piece
-  const long q0 = static_cast<long>(xcd_contiguous(blockIdx.x, gridDim.x)) * 64;
+  // The workgroup's 64 positions are a brick of 8 x 4 x 2 output voxels (8 x 8 of a single slice):
+  // their corners overlap far more than those of 64 positions along a row, which is what the vector
+  // L1 sees.  Local index l of the brick is voxel (l / 32, (l / 8) % 4, l % 8); positions of a
+  // brick that reach past the volume are dead.
+  const int bdz = s.Do > 1 ? 2 : 1, bhy = 8 / bdz;
+  const int nbw = (s.Wo + 7) / 8, nbh = (s.Ho + bhy - 1) / bhy;
+  const int wg = xcd_contiguous(blockIdx.x, gridDim.x);
+  const int w0 = (wg % nbw) * 8, h0 = ((wg / nbw) % nbh) * bhy, d0 = (wg / (nbw * nbh)) * bdz;
+  auto position = [&](int l) -> long {   // linear output position of local index l, -1 when dead
+    const int ow = w0 + l % 8, oh = h0 + (l / 8) % bhy, od = d0 + l / (8 * bhy);
+    return (ow < s.Wo && oh < s.Ho && od < s.Do) ? (static_cast<long>(od) * s.Ho + oh) * s.Wo + ow : -1;
+  };
   const int blocks = s.opg / 16;
   const int chunks = (blocks + MB - 1) / MB;
   const int g = blockIdx.y / chunks, mb0 = (blockIdx.y % chunks) * MB;
@@ -424,8 +435,8 @@ __global__ __launch_bounds__(256, 5) void dcn_forward_shared_taps_kernel(
 
   // phase G: this lane's position, its grid origin, and the planes it reads (scalar offsets per
   // tap and component; sizes below 2^31 bytes are checked by the host)
-  const long qg = q0 + lane;
-  const bool live = qg < s.Q;
+  const long qg = position(lane);
+  const bool live = qg >= 0;
   const long qgc = live ? qg : s.Q - 1;
   float base_d, base_h, base_w;
   {
@@ -560,8 +571,8 @@ __global__ __launch_bounds__(256, 5) void dcn_forward_shared_taps_kernel(
     }
     __syncthreads();   // records and weight pieces may be overwritten
   }
-  const long qo = q0 + 16 * wave + j;
-  if (qo >= s.Q) return;
+  const long qo = position(16 * wave + j);
+  if (qo < 0) return;
   // 16x16 accumulator layout: register r of lane l holds row 4 * (l / 16) + r, column l % 16.
   // All bias values first (the lane's four channels of a block are 8 contiguous bytes; no bias: an
   // empty range), then the stores: a load between two stores would wait for the first.
@@ -694,7 +705,9 @@ static int dcn_mfma_run(const void *x, const void *off, const void *mask, const 
                            static_cast<long>(s.K) * slices * blocks16 * 1024 < (1L << 31);
         if (dcn_shared_taps_enabled() && (slices == 1 || slices == 2) && s.cpd % s.cpg == 0 && blocks16 >= 4 && volume && small) {
           const int chunks4 = (blocks16 + 3) / 4;
-          const long qb = (s.Q + 63) / 64;
+          // bricks of 8 x 4 x 2 output voxels (8 x 8 of a single slice), one per workgroup
+          const int bdz = s.Do > 1 ? 2 : 1, bhy = 8 / bdz;
+          const long qb = static_cast<long>((s.Wo + 7) / 8) * ((s.Ho + bhy - 1) / bhy) * ((s.Do + bdz - 1) / bdz);
           MV_REQUIRE(qb < (1L << 31) && static_cast<long>(s.groups) * chunks4 <= 65535, "grid too large");
           const dim3 grid(static_cast<unsigned>(qb), s.groups * chunks4, s.B), block(256);
           if (slices == 1)
