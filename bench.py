@@ -153,6 +153,14 @@ def bench_other_configs(args):
         nbytes = 3 * vol.numel() * vol.element_size()
         res["config2_backward_" + name] = {"ms": round(ms, 4), "gbps": round(nbytes / ms / 1e6, 1),
                                            "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    # config 2 with a sampling grid of 2 per axis (8 samples per output voxel, means taken inside the
+    # tiled kernel)
+    g = wl.gen(1)
+    r = wl.affine_rois(g, 4, (128, 128, 128)).to(dev)
+    for dt, name in ((torch.float16, "fp16"), (torch.bfloat16, "bf16")):
+        vol = torch.randn(4, 1, 128, 128, 128, generator=g).to(dt).to(dev)
+        ms, _ = _events_ms(lambda i: ops.affine_3d(vol, r, (128, 128, 128), 1.0, 2, True, 1), 50, 5)
+        res["config2_sampling_ratio_2_" + name] = {"ms": round(ms, 4), "gsamples_s": round(8 * vol.numel() / ms / 1e6, 1)}
     g = wl.gen(2)
     vol = wl.ct_like(g, (2, 1, 256, 512, 512)).to(dev)
     full = torch.tensor([[b, 256, 256, 128, 512, 512, 256, 0, 0, 0] for b in range(2)], dtype=torch.float32).to(dev)

@@ -694,7 +694,10 @@ __device__ __forceinline__ void clipped_column(const T *__restrict__ tile, float
 // the item's record, so a wavefront spends a handful of v_readlane and broadcast reads per item;
 // conditions that hold for a whole wavefront (a pass that exists, an output slice that exists)
 // select between the real buffer extent and an empty one on the scalar unit.
-template <typename T, int TX, int TY, int TZ, int THREADS, int LDS_BYTES, int KMAX, int ORDER>
+// G > 1: the problem handed in is the one on the G times finer grid of the bins' samples (cell * G + sub
+// of a fixed sampling grid of G per axis), and every G x G x G block of its voxels leaves as one mean:
+// G slices summed in the lane, the x and y neighbours through lane exchanges, one store per block.
+template <typename T, int TX, int TY, int TZ, int THREADS, int LDS_BYTES, int KMAX, int ORDER, int G = 1>
 __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
     const T *__restrict__ feat, const float *__restrict__ rois, T *__restrict__ out, const RoiProblem p, const PlanShape ps, const unsigned total, const unsigned work) {
   using CT = typename std::conditional<(sizeof(T) == 2), float, double>::type;
@@ -704,6 +707,9 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
   static_assert((TX * TY) % kWave == 0, "a wavefront's lanes share their z layer");
   constexpr int ZPL = TZ / RZ;             // consecutive output slices per lane
   constexpr int ES = sizeof(T);
+  constexpr int ZO = ZPL / G;              // slices a lane stores
+  static_assert(G == 1 || (ZPL % G == 0 && TX % G == 0 && (kWave / TX) % G == 0 && kWave % TX == 0 && TY % (kWave / TX) == 0),
+                "blocks of G x G x G voxels lie inside a wavefront's lanes and a lane's column");
   __shared__ __attribute__((aligned(16))) T tile[kCap];
   __shared__ __attribute__((aligned(16))) TilePlan lplans[kPlanSlots];
   const int H = p.H, W = p.W, oh = p.oh, ow = p.ow;
@@ -730,9 +736,11 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
   const int lx = tid % TX, ly = (tid / TX) % TY, lz = tid / (TX * TY);
   const CT fx = static_cast<CT>(lx), fy = static_cast<CT>(ly), fz = static_cast<CT>(lz * ZPL);
   const float tid_h = static_cast<float>(tid) + 0.5f;
-  const int zbytes = oh * ow * ES;
-  const int out_bytes = p.od * zbytes;   // bytes of one output volume (< 2^31, checked by the host)
-  const unsigned lane_out = static_cast<unsigned>(((lz * ZPL * oh + ly) * ow + lx) * ES);
+  const int oh_o = oh / G, ow_o = ow / G;   // the volume that is written
+  const int zbytes = oh_o * ow_o * ES;
+  const int out_bytes = (p.od / G) * zbytes;   // bytes of one output volume (< 2^31, checked by the host)
+  const unsigned lane_out = static_cast<unsigned>(((lz * ZO * oh_o + ly / G) * ow_o + lx / G) * ES);
+  const bool lane_stores = lx % G == 0 && ly % G == 0;
   const int w_bytes = W * ES;
   const unsigned hw_bytes = static_cast<unsigned>(H) * W * ES;   // < 2^31, checked by the host
   // lane `tid` holds group `tid` of every pass: its place in LDS, slices `gap` bytes apart
@@ -741,6 +749,11 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
   u32x4 val[KMAX];   // the next item's box: 16-byte group (zz0 + u * span, yy, gi) in val[u]
   int st_zz = 0;     // zz0 of this lane (beyond every box for idle lanes)
   float o[ZPL];      // the previous item's outputs
+  [[maybe_unused]] float held[ZO];   // G > 1: the previous item's means (o then belongs to the current item)
+  auto pending = [&](int k) -> float {
+    if constexpr (G == 1) return o[k];
+    else return held[k];
+  };
   // outputs waiting to be stored: the (roi, channel) volume, the lane's byte offset in it (out of
   // range for lanes beyond the output's rows / columns)
   const char *pend_base = reinterpret_cast<const char *>(out);
@@ -895,7 +908,7 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
       // (slices beyond the volume's last one are beyond the buffer: scalar offsets are range-checked)
       const __amdgpu_buffer_rsrc_t rsrc =
           __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(pend_base), 0, pend_bytes, 0x00020000);
-      store_element<T>(rsrc, pend_voff, k * zbytes, o[k]);
+      if (k < ZO) store_element<T>(rsrc, pend_voff, k * zbytes, pending(k));
 #pragma unroll
       for (int u = 0; u < KMAX; u++)
         if (u >= k * KMAX / ZPL && u < (k + 1) * KMAX / ZPL) load_pass(u);   // compile-time share of the loads
@@ -956,9 +969,28 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
         }
       }
     }
-    {
+    if constexpr (G == 1) {
       pend_base = reinterpret_cast<const char *>(out) + plan.u64(MV_PLAN_DW(out_lo));
       pend_voff = (lx < t.y && ly < t.z) ? lane_out + static_cast<unsigned>(t.x) : kOutOfRange;
+      pend_bytes = out_bytes;
+    } else {
+      // means of the blocks: slices in the lane, then the lanes G - 1 to the right and G - 1 rows on
+#pragma unroll
+      for (int kk = 0; kk < ZO; kk++) {
+        float sum = o[kk * G];
+#pragma unroll
+        for (int j = 1; j < G; j++) sum += o[kk * G + j];
+        sum += __shfl_down(sum, 1);
+        if (G == 4) sum += __shfl_down(sum, 2);
+        sum += __shfl_down(sum, TX);
+        if (G == 4) sum += __shfl_down(sum, 2 * TX);
+        held[kk] = sum * (1.f / static_cast<float>(G * G * G));
+      }
+      // the (roi, channel) volume and the tile's first block in it (tile origins are multiples of G)
+      const int bx = plan_scalar(&rec->t0[0]) / G, by0 = plan_scalar(&rec->t0[1]) / G, bz0 = plan_scalar(&rec->t0[2]) / G;
+      pend_base = reinterpret_cast<const char *>(out) + plan.u64(MV_PLAN_DW(out_lo)) / (G * G * G);
+      pend_voff = (lane_stores && lx < t.y && ly < t.z)
+                      ? lane_out + static_cast<unsigned>(((bz0 * oh_o + by0) * ow_o + bx) * ES) : kOutOfRange;
       pend_bytes = out_bytes;
     }
     if (next_mode == 4) break;
@@ -967,10 +999,10 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
     round++;
   }
 #pragma unroll
-  for (int k = 0; k < ZPL; k++) {
+  for (int k = 0; k < ZO; k++) {
     const __amdgpu_buffer_rsrc_t rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(pend_base), 0, pend_bytes, 0x00020000);
-    store_element<T>(rsrc, pend_voff, k * zbytes, o[k]);
+    store_element<T>(rsrc, pend_voff, k * zbytes, pending(k));
   }
 #ifdef MV_RESAMPLE_TIMELINE
   MV_TL(9);
@@ -1192,7 +1224,9 @@ static unsigned compute_units() {
   return static_cast<unsigned>(cus[dev]);
 }
 
-template <typename T, int TX, int TY, int TZ, int THREADS, int LDS_BYTES, int KMAX, bool CUBIC = false>
+// G > 1: `p` is the problem on the finer grid of a fixed sampling grid of G per axis (order 1), `out` the
+// volume of the bins' means.
+template <typename T, int TX, int TY, int TZ, int THREADS, int LDS_BYTES, int KMAX, bool CUBIC = false, int G = 1>
 static int launch_resample(const T *feat, const float *rois, T *out, const RoiProblem &p,
                            void *workspace, size_t *need, hipStream_t s) {
   const long tx = (p.ow + TX - 1) / TX, ty = (p.oh + TY - 1) / TY, tz = (p.od + TZ - 1) / TZ;
@@ -1231,6 +1265,10 @@ static int launch_resample(const T *feat, const float *rois, T *out, const RoiPr
     hipLaunchKernelGGL((roi_resample_cubic_kernel<T, TX, TY, TZ, THREADS, LDS_BYTES>), dim3(blocks),
                        dim3(THREADS), 0, s, feat, rois, out, p, ps, static_cast<unsigned>(total),
                        static_cast<unsigned>(work));
+  else if constexpr (G > 1)
+    hipLaunchKernelGGL((roi_resample_kernel<T, TX, TY, TZ, THREADS, LDS_BYTES, KMAX, 1, G>), dim3(blocks),
+                       dim3(THREADS), 0, s, feat, rois, out, p, ps, static_cast<unsigned>(total),
+                       static_cast<unsigned>(work));
   else if (p.order == 0)
     hipLaunchKernelGGL((roi_resample_kernel<T, TX, TY, TZ, THREADS, LDS_BYTES, KMAX, 0>), dim3(blocks),
                        dim3(THREADS), 0, s, feat, rois, out, p, ps, static_cast<unsigned>(total),
@@ -1265,15 +1303,41 @@ __global__ __launch_bounds__(256) void roi_bin_mean_kernel(const T *__restrict__
   out[i] = store_cast<T>(sum / static_cast<float>(gz * g * g));
 }
 
+// Volumes, order 1, a sampling grid of 2 or 4 per axis: the tiled kernel works on the finer grid and
+// sums every bin's samples in registers (fp32, whatever the tensors' type), so nothing but the means is
+// written.  `f` is the problem on the finer grid.
+template <int G>
+static int roi_forward_tiled_means(const void *input, const void *rois, void *output, int dtype, const RoiProblem &f,
+                                   hipStream_t s) {
+  const float *r = static_cast<const float *>(rois);
+  switch (dtype) {
+    case MV_F16:
+      return launch_resample<__half, 16, 16, 16, 512, 74 * 1024, 8, false, G>(
+          static_cast<const __half *>(input), r, static_cast<__half *>(output), f, nullptr, nullptr, s);
+    case MV_BF16:
+      return launch_resample<__hip_bfloat16, 16, 16, 16, 512, 74 * 1024, 8, false, G>(
+          static_cast<const __hip_bfloat16 *>(input), r, static_cast<__hip_bfloat16 *>(output), f, nullptr, nullptr, s);
+    case MV_F32:
+      return launch_resample<float, 16, 16, 8, 512, 74 * 1024, 6, false, G>(
+          static_cast<const float *>(input), r, static_cast<float *>(output), f, nullptr, nullptr, s);
+    default:
+      return -1;
+  }
+}
+
 // A fixed sampling grid of 2..4 per axis on a large output: the bins' samples are exactly the voxels
 // of the same roi resampled at grid 1 onto an output g times finer (start + (cell * g + sub + 0.5) *
-// bin / g), so the tiled kernel writes that finer volume into the workspace and a second pass takes
-// the means.  16-bit samples are rounded before the mean is; fp16's two roundings stay within its
-// tolerance, bf16's would not, so bf16 keeps the general kernel.
+// bin / g).  Volumes at order 1 with a grid of 2 or 4 take the means inside the tiled kernel (above).
+// Otherwise the tiled kernel writes that finer volume into the workspace and a second pass takes
+// the means: 16-bit samples are then rounded before the mean is; fp16's two roundings stay within its
+// tolerance, bf16's would not, so bf16 then keeps the general kernel.  (The workspace query does not
+// know the order and answers for the two passes.)
 static int roi_forward_tiled_grid(const void *input, const void *rois, void *output, int dtype,
                                   const RoiProblem &p, void *workspace, size_t capacity, size_t *need, hipStream_t s) {
   const int g = p.sampling_ratio, gz = p.ndim == 3 ? g : 1;
-  if (dtype != MV_F16 && dtype != MV_F32) return -1;
+  const bool in_kernel = !need && p.ndim == 3 && p.order == 1 && (g == 2 || g == 4) && p.R > 0 &&
+                         (dtype == MV_F16 || dtype == MV_BF16 || dtype == MV_F32);
+  if (dtype != MV_F16 && dtype != MV_F32 && !in_kernel) return -1;
   if (!need && p.order != 1 && p.order != 3) return -1;
   // Outputs that the grid-1 rule sends here, except those of <= 16 cells per axis (the pooled kernels
   // take plain boxes of that size).  Only values that the workspace query also knows may decide.
@@ -1284,6 +1348,13 @@ static int roi_forward_tiled_grid(const void *input, const void *rois, void *out
   f.od = p.od * gz; f.oh = p.oh * g; f.ow = p.ow * g;
   const long cells = static_cast<long>(p.R) * p.C * p.od * p.oh * p.ow;
   const long fine = cells * gz * g * g;
+  // (32-bit byte offsets inside one finer volume, as in the grid-1 rule)
+  if (in_kernel && static_cast<long>(f.od) * f.oh * f.ow * 4 < (1L << 31)) {
+    const int st = g == 2 ? roi_forward_tiled_means<2>(input, rois, output, dtype, f, s)
+                          : roi_forward_tiled_means<4>(input, rois, output, dtype, f, s);
+    if (st != -1) return st;
+  }
+  if (dtype != MV_F16 && dtype != MV_F32) return -1;
   if (fine >= (1L << 31) || (cells + 255) / 256 >= (1L << 31)) return -1;
   size_t inner = 0;
   if (roi_forward_tiled(nullptr, nullptr, nullptr, dtype, f, nullptr, 0, &inner, nullptr) != MV_OK) return -1;

@@ -386,9 +386,12 @@ def test_cubic_affine_vs_oracle(ops, oracle, dtype, ndim, sr):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("sr", [2, 3, 4])
 def test_large_outputs_with_a_sampling_grid(ops, oracle, dtype, sr):
-    """sampling_ratio 2..4 on outputs of resampling size: the tiled kernel writes the samples of the
-    sr times finer grid and a second pass takes the bin means (fp16 / fp32; bf16 stays on the general
-    kernel).  Rotated and plain rois in 3-D and 2-D, order 1, and order 3 through the affine engine."""
+    """sampling_ratio 2..4 on outputs of resampling size: the tiled kernel works on the sr times finer
+    grid of the bins' samples.  Volumes at order 1 with a grid of 2 or 4 (any of the three types) take
+    the means of the bins inside that kernel; a grid of 3, images and order 3 write the finer volume
+    and a second pass takes the means (fp16 / fp32; bf16 then stays on the general kernel).  Rotated
+    and plain rois in 3-D and 2-D, order 1, and order 3 through the affine engine; a second output
+    shape whose finer grid ends inside a tile on every axis."""
     g = wl.gen(700 + sr)
     feat = torch.randn(2, 2, 24, 40, 48, generator=g).to(dtype)
     out = (20, 24, 32) if sr < 4 else (10, 24, 32)
@@ -401,6 +404,10 @@ def test_large_outputs_with_a_sampling_grid(ops, oracle, dtype, sr):
     got = ops.RoIAlign(out, 0.5, sr)(feat.to(DEV), (boxes * torch.tensor([1.] + [2.] * 6)).to(DEV))
     want = oracle.roi_align_forward(feat, boxes * torch.tensor([1.] + [2.] * 6), out, 0.5, sr, True, 1, False)
     assert_close(got, want, FWD_TOL[dtype], "plain 3-D")
+    ragged = (17, 21, 27) if sr < 4 else (9, 21, 27)
+    got = ops.RoIAlignRotated(ragged, 1.0, sr)(feat.to(DEV), rois.to(DEV))
+    want = oracle.roi_align_forward(feat, rois, ragged, 1.0, sr, True, 1, True)
+    assert_close(got, want, FWD_TOL[dtype], "rotated 3-D, tiles cut on every axis")
     img = torch.randn(2, 3, 70, 90, generator=g).to(dtype)
     r2 = torch.tensor([[0, 45.0, 35.0, 80.0, 60.0, 0.4], [1, 40.0, 30.0, 100.0, 50.0, -1.2]])
     got = ops.RoIAlignRotated((64, 80), 1.0, sr)(img.to(DEV), r2.to(DEV))
