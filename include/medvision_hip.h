@@ -114,6 +114,27 @@ size_t mv_roi_align_forward_workspace_bytes_for_input(int dtype, int ndim, int b
                                                       int height, int width, int num_rois, int out_d,
                                                       int out_h, int out_w, int sampling_ratio);
 
+/* Detection heads that pool ONE feature map several times (cascade stages, several batches of rois):
+ * the re-ordered copy that mv_roi_align_2d_forward / _3d_forward make in their workspace on every call
+ * (fp16 features whose width is a multiple of four) can be made once and handed in.
+ * mv_roi_align_prepared_bytes: size of that copy, 0 when the forward pass has no use for one.
+ * mv_roi_align_prepare_features: writes it (8-byte aligned pointers; an error when the size is 0 or
+ * `prepared_bytes` is smaller).  mv_roi_align_forward_prepared: mv_roi_align_{2,3}d_forward (plain
+ * rois; replaces the same reference functions) reading `prepared`, which must have been written from
+ * the very contents `input` has now; outputs equal those of the plain entry points bit for bit.  Its
+ * workspace wants 4 bytes per roi (the order the rois are worked in; without it they run in the given
+ * order).  Heads the copy does not serve (more than 8 cells per axis, order 3, other types) run as
+ * through the plain entry points and then want their workspace.  depth / out_d ignored for ndim 2.
+ * No counterpart in the reference.                                                              */
+size_t mv_roi_align_prepared_bytes(int dtype, int ndim, int batch, int channels, int depth, int height, int width);
+int mv_roi_align_prepare_features(const void *input, int dtype, int ndim, int batch, int channels, int depth,
+                                  int height, int width, void *prepared, size_t prepared_bytes, void *stream);
+int mv_roi_align_forward_prepared(const void *input, const void *prepared, const void *rois, void *output,
+                                  int dtype, int ndim, int batch, int channels, int depth, int height, int width,
+                                  int num_rois, int out_d, int out_h, int out_w, float spatial_scale,
+                                  int sampling_ratio, int order, void *workspace, size_t workspace_bytes,
+                                  void *stream);
+
 /* ---- affine resampling engine (forward only) ----------------------------------------------
  * replaces affine_2d  csrc/affine_2d.h (vision.cpp:74), affine_3d  csrc/affine_3d.h:40 (vision.cpp:75)
  * Same arguments and results as the rotated forward for order 0 / 1 (the reference kernel text

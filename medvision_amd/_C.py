@@ -106,6 +106,61 @@ def _roi_forward(fn_name, what, ndim, cols, input, rois, output, out_sizes, spat
             _lib.ptr(ws), ws_bytes, _lib.stream_of(feats)))
 
 
+def roi_align_prepare(features):
+    """The re-ordered copy of ``features`` that the RoIAlign forward of detection heads reads (made by
+    every call in its workspace otherwise), for callers that pool one feature map several times; None
+    when the forward pass has no use for one (other than fp16, width no multiple of four).  No
+    counterpart in the reference.  Pass it as ``prepared`` to ``roi_align_{2,3}d_forward`` together with
+    the same, unchanged features."""
+    _require_cuda(features, "RoIAlign")
+    _require_contiguous(features, "features")
+    ndim = features.dim() - 2
+    if ndim not in (2, 3):
+        raise RuntimeError(f"expected a 4-d or 5-d feature tensor, got {features.dim()}-d")
+    lib = _lib.load()
+    code = _lib.dtype_code(features)
+    dims = list(features.shape)
+    d5 = dims if ndim == 3 else [dims[0], dims[1], 1, dims[2], dims[3]]
+    nbytes = _cached_bytes("mv_roi_align_prepared_bytes", code, ndim, *d5)
+    if nbytes == 0:
+        return None
+    copy = torch.empty(nbytes, dtype=torch.uint8, device=features.device)
+    with _on_device(features):
+        _lib.check(lib.mv_roi_align_prepare_features(_lib.ptr(features), code, ndim, *d5, _lib.ptr(copy), nbytes,
+                                                     _lib.stream_of(features)))
+    return copy
+
+
+def _roi_forward_prepared(ndim, input, prepared, rois, output, out_sizes, spatial_scale, sampling_ratio, order):
+    _require_cuda(input, "RoIAlign")
+    lib = _lib.load()
+    _same_device(input, output=output, prepared=prepared)
+    _require_contiguous(output, "output")
+    _require_contiguous(input, "input")
+    if output.dtype != input.dtype:
+        raise RuntimeError("output dtype must match input dtype")
+    r = _prep_rois(rois, input, 1 + 2 * ndim)
+    dims = list(input.shape)
+    if len(dims) != ndim + 2:
+        raise RuntimeError(f"expected a {ndim + 2}-d feature tensor, got {len(dims)}-d")
+    want_shape = (r.size(0), dims[1], *out_sizes)
+    if tuple(output.shape) != want_shape:
+        raise RuntimeError(f"output has shape {tuple(output.shape)}, expected {want_shape}")
+    code = _lib.dtype_code(input)
+    d5 = dims if ndim == 3 else [dims[0], dims[1], 1, dims[2], dims[3]]
+    out3 = out_sizes if ndim == 3 else (1, *out_sizes)
+    if prepared.numel() != _cached_bytes("mv_roi_align_prepared_bytes", code, ndim, *d5):
+        raise RuntimeError("prepared copy does not belong to features of this shape")
+    # four bytes per roi for the order the rois are worked in; what heads the copy does not serve need
+    ws_bytes = max(4 * r.size(0), _cached_bytes("mv_roi_align_forward_workspace_bytes", code, ndim, dims[1], r.size(0),
+                                                *out3, int(sampling_ratio)))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=input.device) if ws_bytes else None
+    with _on_device(input):
+        _lib.check(lib.mv_roi_align_forward_prepared(
+            _lib.ptr(input), _lib.ptr(prepared), _lib.ptr(r), _lib.ptr(output), code, ndim, *d5, r.size(0), *out3,
+            float(spatial_scale), int(sampling_ratio), int(order), _lib.ptr(ws), ws_bytes, _lib.stream_of(input)))
+
+
 def _roi_backward(fn_name, what, ndim, cols, top_grad, rois, bottom_grad, out_sizes,
                   spatial_scale, sampling_ratio, extra):
     _require_cuda(top_grad, what)
@@ -133,7 +188,9 @@ def _roi_backward(fn_name, what, ndim, cols, top_grad, rois, bottom_grad, out_si
 
 
 # ---- csrc/roi_align_2d.h, csrc/roi_align_3d.h:71-117 ------------------------------------
-def roi_align_2d_forward(input, rois, output, out_h, out_w, spatial_scale, sampling_ratio, order):
+def roi_align_2d_forward(input, rois, output, out_h, out_w, spatial_scale, sampling_ratio, order, prepared=None):
+    if prepared is not None:
+        return _roi_forward_prepared(2, input, prepared, rois, output, (out_h, out_w), spatial_scale, sampling_ratio, order)
     _roi_forward("mv_roi_align_2d_forward", "RoIAlign", 2, 5, input, rois, output,
                  (out_h, out_w), spatial_scale, sampling_ratio, (int(order),))
 
@@ -145,7 +202,10 @@ def roi_align_2d_backward(top_grad, rois, bottom_grad, out_h, out_w, spatial_sca
 
 
 def roi_align_3d_forward(input, rois, output, out_d, out_h, out_w, spatial_scale, sampling_ratio,
-                         order):
+                         order, prepared=None):
+    if prepared is not None:
+        return _roi_forward_prepared(3, input, prepared, rois, output, (out_d, out_h, out_w), spatial_scale,
+                                     sampling_ratio, order)
     _roi_forward("mv_roi_align_3d_forward", "RoIAlign", 3, 7, input, rois, output,
                  (out_d, out_h, out_w), spatial_scale, sampling_ratio, (int(order),))
 

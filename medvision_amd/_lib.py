@@ -51,6 +51,9 @@ SIGNATURES = {
     "mv_roi_align_backward_workspace_bytes": (_sz, [_i] * 6),
     "mv_roi_align_forward_workspace_bytes": (_sz, [_i] * 8),
     "mv_roi_align_forward_workspace_bytes_for_input": (_sz, [_i] * 12),
+    "mv_roi_align_prepared_bytes": (_sz, [_i] * 7),
+    "mv_roi_align_prepare_features": (_i, [_p, _i] + [_i] * 6 + [_p, _sz, _p]),
+    "mv_roi_align_forward_prepared": (_i, [_p, _p, _p, _p, _i] + [_i] * 10 + [_f, _i, _i, _p, _sz, _p]),
     "mv_affine_2d": (_i, [_p, _p, _p, _i] + [_i] * 7 + [_f, _i, _i, _i, _p, _sz, _p]),
     "mv_affine_3d": (_i, [_p, _p, _p, _i] + [_i] * 9 + [_f, _i, _i, _i, _p, _sz, _p]),
     "mv_dcn3d_output_dims": (_i, [_SHAPE_P, ctypes.POINTER(_i), ctypes.POINTER(_i), ctypes.POINTER(_i)]),

@@ -131,7 +131,11 @@ int roi_backward_tiled(const void *grad_output, const void *rois, float *acc, in
 // roi_pool.hip: separable LDS kernels for plain boxes with small outputs; -1 when not applicable
 size_t roi_pool_forward_workspace(int dtype, const RoiProblem &p);
 int roi_pool_forward(const void *input, const void *rois, void *output, int dtype,
-                     const RoiProblem &p, void *workspace, size_t capacity, hipStream_t s);
+                     const RoiProblem &p, void *workspace, size_t capacity, hipStream_t s,
+                     const void *prepared = nullptr);
+// the re-ordered copy of the features alone (callers that pool one feature map several times)
+size_t roi_pool_prepared_bytes(int dtype, const RoiProblem &p);
+int roi_pool_prepare(const void *input, int dtype, const RoiProblem &p, void *prepared, size_t capacity, hipStream_t s);
 int roi_pool_backward(const void *grad_output, const void *rois, void *acc, int dtype,
                       const RoiProblem &p, hipStream_t s, bool channels_last);
 bool roi_pool_applies(int dtype, const RoiProblem &p);
@@ -178,7 +182,7 @@ int roi_forward(const void *input, const void *rois, void *output, int dtype, in
                 int rotated, int batch, int channels, int depth, int height, int width,
                 int num_rois, int out_d, int out_h, int out_w, float spatial_scale,
                 int sampling_ratio, int aligned, int order, void *workspace, size_t workspace_bytes,
-                void *stream, bool cubic_ok = false) {
+                void *stream, bool cubic_ok = false, const void *prepared = nullptr) {
   RoiProblem p;
   int st = make_problem(p, ndim, rotated, batch, channels, depth, height, width, num_rois, out_d,
                         out_h, out_w, spatial_scale, sampling_ratio, aligned, order, cubic_ok);
@@ -189,6 +193,10 @@ int roi_forward(const void *input, const void *rois, void *output, int dtype, in
   {
     // (a workspace too small for a path selects the kernels that need none)
     const size_t capacity = workspace ? workspace_bytes : 0;
+    if (prepared != nullptr) {   // (a copy the pooled kernels have no use for is left alone)
+      const int pooled = roi_pool_forward(input, rois, output, dtype, p, workspace, capacity, s, prepared);
+      if (pooled >= 0) return pooled;
+    }
     const int tiled = roi_forward_tiled(input, rois, output, dtype, p, workspace, capacity, nullptr, s);
     if (tiled >= 0) return tiled;
     const int pooled = order != 3 ? roi_pool_forward(input, rois, output, dtype, p, workspace, capacity, s) : -1;
@@ -292,6 +300,40 @@ int mv_roi_align_2d_forward(const void *input, const void *rois, void *output, i
                             size_t workspace_bytes, void *stream) {
   return roi_forward(input, rois, output, dtype, 2, 0, batch, channels, 1, height, width, num_rois,
                      1, out_h, out_w, spatial_scale, sampling_ratio, 1, order, workspace, workspace_bytes, stream);
+}
+
+size_t mv_roi_align_prepared_bytes(int dtype, int ndim, int batch, int channels, int depth, int height, int width) {
+  if ((ndim != 2 && ndim != 3) || batch <= 0 || channels <= 0 || depth <= 0 || height <= 0 || width <= 0) return 0;
+  mv::RoiProblem p{};
+  p.ndim = ndim; p.N = batch; p.C = channels; p.D = ndim == 2 ? 1 : depth; p.H = height; p.W = width;
+  return mv::roi_pool_prepared_bytes(dtype, p);
+}
+
+int mv_roi_align_prepare_features(const void *input, int dtype, int ndim, int batch, int channels, int depth,
+                                  int height, int width, void *prepared, size_t prepared_bytes, void *stream) {
+  MV_REQUIRE(ndim == 2 || ndim == 3, "ndim must be 2 or 3");
+  MV_REQUIRE(batch > 0 && channels > 0 && depth > 0 && height > 0 && width > 0,
+             "feature dims must be positive (got %d,%d,%d,%d,%d)", batch, channels, depth, height, width);
+  MV_REQUIRE(input && prepared, "null pointer argument");
+  mv::RoiProblem p{};
+  p.ndim = ndim; p.N = batch; p.C = channels; p.D = ndim == 2 ? 1 : depth; p.H = height; p.W = width;
+  const size_t bytes = mv::roi_pool_prepared_bytes(dtype, p);
+  MV_REQUIRE(bytes > 0, "no prepared copy for these features (mv_roi_align_prepared_bytes is 0)");
+  MV_REQUIRE(prepared_bytes >= bytes, "prepared buffer too small");
+  MV_REQUIRE(reinterpret_cast<uintptr_t>(input) % 8 == 0 && reinterpret_cast<uintptr_t>(prepared) % 8 == 0,
+             "input and prepared must be 8-byte aligned");
+  return mv::roi_pool_prepare(input, dtype, p, prepared, prepared_bytes, static_cast<hipStream_t>(stream));
+}
+
+int mv_roi_align_forward_prepared(const void *input, const void *prepared, const void *rois, void *output,
+                                  int dtype, int ndim, int batch, int channels, int depth, int height, int width,
+                                  int num_rois, int out_d, int out_h, int out_w, float spatial_scale,
+                                  int sampling_ratio, int order, void *workspace, size_t workspace_bytes,
+                                  void *stream) {
+  MV_REQUIRE(ndim == 2 || ndim == 3, "ndim must be 2 or 3");
+  return roi_forward(input, rois, output, dtype, ndim, 0, batch, channels, ndim == 2 ? 1 : depth, height, width,
+                     num_rois, ndim == 2 ? 1 : out_d, out_h, out_w, spatial_scale, sampling_ratio, 1, order,
+                     workspace, workspace_bytes, stream, false, prepared);
 }
 
 int mv_roi_align_2d_backward(const void *grad_output, const void *rois, void *grad_input,

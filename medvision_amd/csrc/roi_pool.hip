@@ -1410,12 +1410,54 @@ size_t roi_pool_forward_workspace(int dtype, const RoiProblem &p) {
   return pool_applies(dtype, p) ? pool_blocked_bytes(dtype, p) : 0;
 }
 
+// The blocked copy alone, for callers that pool one feature map several times: bytes of the copy of
+// these features (0: the forward pass has no use for one; only N, C, D, H, W of `p` are looked at) ...
+size_t roi_pool_prepared_bytes(int dtype, const RoiProblem &p) {
+  if (dtype != MV_F16 || p.W % 4 != 0) return 0;
+  if (static_cast<long>(p.D) * p.H * p.W * p.C * 2 >= (1L << 31)) return 0;   // 32-bit byte offsets inside one image
+  const long rows = static_cast<long>(p.D) * p.H;
+  const int Wb = p.W / 4, ux = std::min(Wb, kBlockUnits);
+  if (p.N * rows * ((Wb + ux - 1) / ux) * ((p.C + 63) / 64) >= (1L << 31)) return 0;
+  return static_cast<size_t>(p.N) * p.D * p.H * p.W * p.C * 2;
+}
+
+// ... and the copy itself.  -1: no copy for these features.
+int roi_pool_prepare(const void *input, int dtype, const RoiProblem &p, void *prepared, size_t capacity, hipStream_t s) {
+  const size_t bytes = roi_pool_prepared_bytes(dtype, p);
+  if (bytes == 0 || capacity < bytes || reinterpret_cast<uintptr_t>(input) % 8 != 0 ||
+      reinterpret_cast<uintptr_t>(prepared) % 8 != 0)
+    return -1;
+  const long rows = static_cast<long>(p.D) * p.H;
+  const int Wb = p.W / 4, ux = std::min(Wb, kBlockUnits);
+  const long copy_blocks = p.N * rows * ((Wb + ux - 1) / ux) * ((p.C + 63) / 64);
+  hipLaunchKernelGGL(pool_block_features_kernel, dim3(static_cast<unsigned>(copy_blocks)), dim3(256), 0, s,
+                     static_cast<const uint2 *>(input), static_cast<uint2 *>(prepared), p.C, rows, Wb,
+                     static_cast<const float *>(nullptr), static_cast<unsigned *>(nullptr), 0, p.ndim, 1.f);
+  return check_launch("pool_block_features_kernel");
+}
+
+// `prepared`: a copy made by roi_pool_prepare from the same features (then only the order of the rois
+// is worked out here, into the workspace when it holds four bytes per roi), or null.
 int roi_pool_forward(const void *input, const void *rois, void *output, int dtype,
-                     const RoiProblem &p, void *workspace, size_t capacity, hipStream_t s) {
+                     const RoiProblem &p, void *workspace, size_t capacity, hipStream_t s, const void *prepared) {
   if (!pool_applies(dtype, p)) return -1;
   const void *blocked = nullptr;
   const unsigned *order = nullptr;
-  if (workspace != nullptr && pool_blocked_bytes(dtype, p) > 0 && capacity >= pool_blocked_bytes(dtype, p) &&
+  if (prepared != nullptr) {
+    // the kernels that read a copy: fp16, up to 8 cells per axis, orders 0 and 1
+    if (roi_pool_prepared_bytes(dtype, p) == 0 || p.order == 3 || p.od > 8 || p.oh > 8 || p.ow > 8 ||
+        reinterpret_cast<uintptr_t>(prepared) % 8 != 0)
+      return -1;
+    blocked = prepared;
+    if (workspace != nullptr && p.R <= kOrderMaxRois && capacity >= static_cast<size_t>(p.R) * 4 &&
+        reinterpret_cast<uintptr_t>(workspace) % 4 == 0) {
+      unsigned *ord = static_cast<unsigned *>(workspace);
+      hipLaunchKernelGGL(pool_block_features_kernel, dim3(1), dim3(256), 0, s, static_cast<const uint2 *>(nullptr),
+                         static_cast<uint2 *>(nullptr), p.C, static_cast<long>(p.D) * p.H, p.W / 4,
+                         static_cast<const float *>(rois), ord, p.R, p.ndim, static_cast<float>(p.scale));
+      order = ord;
+    }
+  } else if (workspace != nullptr && pool_blocked_bytes(dtype, p) > 0 && capacity >= pool_blocked_bytes(dtype, p) &&
       reinterpret_cast<uintptr_t>(input) % 8 == 0 &&
       reinterpret_cast<uintptr_t>(workspace) % 8 == 0) {
     const long rows = static_cast<long>(p.D) * p.H;

@@ -27,14 +27,35 @@ def _kernels(ndim):
     return _C.roi_align_3d_forward, _C.roi_align_3d_backward
 
 
-def _forward(ndim, ctx, features, rois, output_size, spatial_scale, sampling_ratio, order):
+class PreparedFeatures:
+    """Features of a detection head together with the re-ordered copy that the forward pass of
+    ``RoIAlign`` reads (it is made anew by every call otherwise): for heads that pool ONE feature map
+    several times (cascade stages, several batches of rois).  Pass the object to ``RoIAlign`` in place of
+    the features; gradients flow to ``features`` as usual.  The copy follows the contents the features
+    had when the object was made: an in-place change that autograd sees raises, one that it does not see
+    (writes through ``.data``) is the caller's to avoid.  No counterpart in the reference."""
+
+    def __init__(self, features):
+        self.features = features.contiguous()
+        self.copy = _C.roi_align_prepare(self.features.detach())   # None: the forward pass has no use for one
+        self._version = self.features._version
+
+    def check(self):
+        if self.features._version != self._version:
+            raise RuntimeError("the features were changed in place after PreparedFeatures was made")
+
+
+def _forward(ndim, ctx, features, rois, output_size, spatial_scale, sampling_ratio, order, prepared=None):
     out = _parse_output_size(output_size, ndim)
     ctx.spatial_scale, ctx.sampling_ratio, ctx.order = spatial_scale, sampling_ratio, order
     ctx.save_for_backward(rois)
     ctx.feature_size = features.size()
     # every output element is written by the kernel (zeros where a sample is void): no zero fill
     output = features.new_empty(rois.size(0), features.size(1), *out)
-    _kernels(ndim)[0](features, rois, output, *out, spatial_scale, sampling_ratio, order)
+    if prepared is not None:
+        _kernels(ndim)[0](features.contiguous(), rois, output, *out, spatial_scale, sampling_ratio, order, prepared)
+    else:
+        _kernels(ndim)[0](features, rois, output, *out, spatial_scale, sampling_ratio, order)
     return output
 
 
@@ -47,13 +68,13 @@ def _backward(ndim, ctx, grad_output):
         grad_input = grad_output.new_zeros(ctx.feature_size)
         _kernels(ndim)[1](grad_output.contiguous(), rois, grad_input, *grad_output.shape[2:],
                           ctx.spatial_scale, ctx.sampling_ratio, ctx.order)
-    return grad_input, None, None, None, None, None
+    return grad_input, None, None, None, None, None, None
 
 
 class RoIAlign2DFunction(Function):
     @staticmethod
-    def forward(ctx, features, rois, output_size, spatial_scale, sampling_ratio=0, order=1):
-        return _forward(2, ctx, features, rois, output_size, spatial_scale, sampling_ratio, order)
+    def forward(ctx, features, rois, output_size, spatial_scale, sampling_ratio=0, order=1, prepared=None):
+        return _forward(2, ctx, features, rois, output_size, spatial_scale, sampling_ratio, order, prepared)
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -62,8 +83,8 @@ class RoIAlign2DFunction(Function):
 
 class RoIAlign3DFunction(Function):
     @staticmethod
-    def forward(ctx, features, rois, output_size, spatial_scale, sampling_ratio=0, order=1):
-        return _forward(3, ctx, features, rois, output_size, spatial_scale, sampling_ratio, order)
+    def forward(ctx, features, rois, output_size, spatial_scale, sampling_ratio=0, order=1, prepared=None):
+        return _forward(3, ctx, features, rois, output_size, spatial_scale, sampling_ratio, order, prepared)
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -102,6 +123,10 @@ class RoIAlign(nn.Module):
         assert order in [0, 1], "only support order = 0 (nearest) or 1 (linear)"
         # nearest sampling must not average several samples (reference roi_align_nd.py:195)
         sampling_ratio = 1 if order == 0 else self.sampling_ratio
+        if isinstance(features, PreparedFeatures):
+            features.check()
+            return self.roi_align(features.features, rois, self.output_size, self.spatial_scale, sampling_ratio,
+                                  order, features.copy)
         return self.roi_align(features, rois, self.output_size, self.spatial_scale, sampling_ratio,
                               order)
 

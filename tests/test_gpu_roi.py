@@ -509,6 +509,31 @@ def test_pooled_forward_from_blocked_copy(ops, oracle, ndim):
     got = ops.RoIAlign(out, 1.0, 2)(feat.to(DEV), rois.to(DEV))
     want = oracle.roi_align_forward(feat, rois, out, 1.0, 2)
     assert_close(got, want, FWD_TOL[torch.float16], "pooled forward from the blocked copy")
+    # the copy made once and handed in (heads that pool one feature map several times): the same
+    # outputs bit for bit, also for a second, smaller batch of rois and with few rois (no copy would be
+    # made for them inside a call); gradients reach the features
+    x = feat.to(DEV).requires_grad_(True)
+    kept = ops.PreparedFeatures(x)
+    assert kept.copy is not None and kept.copy.numel() == feat.numel() * 2
+    again = ops.RoIAlign(out, 1.0, 2)(kept, rois.to(DEV))
+    assert torch.equal(again, got)
+    few = ops.RoIAlign(out, 1.0, 2)(kept, rois[:5].to(DEV))
+    assert torch.equal(few, got[:5])
+    nearest = ops.RoIAlign(out, 1.0, 2)(kept, rois[:40].to(DEV), order=0)
+    assert torch.equal(nearest, ops.RoIAlign(out, 1.0, 2)(feat.to(DEV), rois[:40].to(DEV), order=0))
+    gy = torch.randn(again.shape, generator=g).half()
+    again.backward(gy.to(DEV))
+    gwant = oracle.roi_align_backward(gy, rois, feat.shape, 1.0, 2)
+    assert_close(x.grad, gwant, BWD_TOL[torch.float16], "backward behind the prepared copy")
+    # heads the copy does not serve run as without it
+    big = tuple(12 for _ in out)
+    assert torch.equal(ops.RoIAlign(big, 1.0, 2)(kept, rois[:50].to(DEV)),
+                       ops.RoIAlign(big, 1.0, 2)(feat.to(DEV), rois[:50].to(DEV)))
+    with torch.no_grad():
+        x.mul_(2.0)
+    with pytest.raises(RuntimeError, match="changed in place"):
+        ops.RoIAlign(out, 1.0, 2)(kept, rois.to(DEV))
+    assert ops.PreparedFeatures(feat.float().to(DEV)).copy is None      # fp16 only
     # few rois: no copy, same kernels from the input itself
     few = rois[:15]
     assert _lib.load().mv_roi_align_forward_workspace_bytes_for_input(_lib.MV_F16, ndim, 2, channels, *in3, 15, *out3, 2) == 0
