@@ -125,8 +125,10 @@ int roi_forward_tiled(const void *input, const void *rois, void *output, int dty
 // roi_resample.hip: backward of the same problems through LDS tiles of the source boxes; `acc` is the
 // fp32 buffer the gradient is added to; -1 when it does not apply
 bool roi_backward_tiled_applies(int dtype, const RoiProblem &p);
-int roi_backward_tiled(const void *grad_output, const void *rois, float *acc, int dtype,
-                       const RoiProblem &p, hipStream_t s);
+int roi_backward_tiled(const void *grad_output, const void *rois, void *acc, int dtype,
+                       const RoiProblem &p, hipStream_t s, bool direct = false);
+// fp16 gradients with even rows: the tiles add to the gradient tensor itself (packed atomics on pairs)
+bool roi_backward_tiled_direct(int dtype, const RoiProblem &p, const void *grad_input);
 
 // roi_pool.hip: separable LDS kernels for plain boxes with small outputs; -1 when not applicable
 size_t roi_pool_forward_workspace(int dtype, const RoiProblem &p);
@@ -234,6 +236,8 @@ int roi_backward(const void *grad_output, const void *rois, void *grad_input, in
   hipStream_t s = static_cast<hipStream_t>(stream);
   const long total = static_cast<long>(batch) * channels * depth * height * width;
   const int fill_blocks = static_cast<int>(std::min<long>((total + 1023) / 1024, 65536));
+  if (roi_backward_tiled_direct(dtype, p, grad_input))
+    return roi_backward_tiled(grad_output, rois, grad_input, dtype, p, s, true);
   if (roi_backward_tiled_applies(dtype, p)) {
     // 16-bit tensors: sums in the fp32 workspace; fp32: sums in grad_input
     float *ws = static_cast<float *>(workspace);

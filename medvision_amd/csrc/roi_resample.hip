@@ -1526,10 +1526,28 @@ constexpr int kScatterLds = MV_SCATTER_LDS;
 constexpr int kScatterWgs = MV_SCATTER_WGS;     // workgroups per compute unit
 constexpr int kTermBits = 19;
 
-template <typename T, int TX, int TY, int TZ>
+// fp16 sums straight into the gradient tensor: one packed atomic adds to the two voxels of an aligned
+// pair (`pair`: the even voxel).  A voxel's sum is then rounded once per tile that reaches it (a few)
+// instead of once at the end.
+__device__ __forceinline__ void atomic_add_pair(__half *pair, float lo, float hi) {
+  typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+  half2_t v;
+  v.x = static_cast<_Float16>(lo); v.y = static_cast<_Float16>(hi);
+  __builtin_amdgcn_global_atomic_fadd_v2f16((__attribute__((address_space(1))) half2_t *)pair, v);
+}
+__device__ __forceinline__ void atomic_add_element(__half *base, long i, float v) {
+  atomic_add_pair(base + (i & ~1L), (i & 1) ? 0.f : v, (i & 1) ? v : 0.f);
+}
+__device__ __forceinline__ void atomic_add_element(float *base, long i, float v) { atomic_add(base + i, v); }
+
+// DIRECT (fp16 only; rows of an even number of voxels, a 4-byte aligned tensor): `acc` is the gradient
+// tensor itself, otherwise an fp32 buffer of its shape.
+template <typename T, int TX, int TY, int TZ, bool DIRECT = false>
 __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward_tiles_kernel(
-    const T *__restrict__ gout, const float *__restrict__ rois, float *__restrict__ acc, const RoiProblem p,
+    const T *__restrict__ gout, const float *__restrict__ rois, void *__restrict__ acc, const RoiProblem p,
     const PlanShape ps, const unsigned total, const unsigned work) {
+  using A = typename std::conditional<DIRECT, T, float>::type;
+  static_assert(!DIRECT || std::is_same<T, __half>::value, "packed atomics of fp16 pairs");
   constexpr int kScatterCells = TX * TY * TZ;   // output voxels per item
   static_assert(kScatterCells % kScatterThreads == 0 && kScatterCells <= (1 << (30 - kTermBits)), "tile shape");
   constexpr int kPerThread = kScatterCells / kScatterThreads, kWaves = kScatterThreads / kWave;
@@ -1564,7 +1582,7 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
     for (int i = 0; i < 12; i++) map[i] = uniform(r.map[i]);
     map[0] += l0; map[4] += l1; map[8] += l2;   // to volume coordinates
     const unsigned chan = p.C > 1 ? ps.by_total.div(item) : 0u;
-    float *const vol = acc + (static_cast<long>(plan_scalar(&r.batch)) * p.C + chan) * plane;
+    A *const vol = static_cast<A *>(acc) + (static_cast<long>(plan_scalar(&r.batch)) * p.C + chan) * plane;
     const T *const gsrc = gout + (static_cast<long>(plan_scalar(&r.roi)) * p.C + chan) * ovol;
     // The item's grad_output, and the largest magnitude in it as the bit pattern of a float (patterns
     // of non-negative floats order like unsigned integers, NaNs above infinity).
@@ -1607,6 +1625,75 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
     const float from_quanta = __uint_as_float(static_cast<unsigned>(254 - ex) << 23);
     // One copy of the loop per (interior, order): a box that is not clipped holds samples in
     // [0, size - 1) only, so the low tap is the floor and neither the void test nor the clamps are needed.
+    // 16-bit tensors at order 1 whose box is in LDS: box-relative fp32 coordinates with the forward
+    // kernel's rules (clipped boxes: the coordinate clamps to [0, cmax], a sample the clamp moves by
+    // more than 1 is void, the low tap is at most top = max(n - 2, 0)); the box's margin covers their
+    // rounding.
+    auto scatter_cells32 = [&](auto interior_tag) {
+    constexpr bool kInterior = decltype(interior_tag)::value;
+    float mf[12], cmax[3], top[3];
+#pragma unroll
+    for (int i = 0; i < 12; i++) mf[i] = uniform(r.mapf[i]);
+#pragma unroll
+    for (int a = 0; a < 3; a++) { cmax[a] = uniform(r.cmaxf[a]); top[a] = uniform(r.topf[a]); }
+    const float gq_scale = to_quanta;
+#pragma unroll
+    for (int k = 0; k < kPerThread; k++) {
+      const int c = threadIdx.x + k * kScatterThreads;
+      const float x = static_cast<float>(c % TX), y = static_cast<float>((c / TX) % TY), z = static_cast<float>(c / (TX * TY));
+      const float g = gv[k];
+      if (g == 0.f) continue;
+      float v[3], f[3];
+      int b0[3];
+#pragma unroll
+      for (int a = 0; a < 3; a++) v[a] = fmaf(mf[4 * a + 3], z, fmaf(mf[4 * a + 2], y, fmaf(mf[4 * a + 1], x, mf[4 * a])));
+      if constexpr (kInterior) {
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+          const float l = floorf(v[a]);
+          f[a] = v[a] - l;
+          b0[a] = static_cast<int>(l);
+        }
+      } else {
+        float moved = 0.f;
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+          const float cl = clamp_ct(v[a], 0.f, cmax[a]);
+          moved = fmaxf(moved, fabsf(v[a] - cl));
+          const float l = fminf(floorf(cl), top[a]);
+          f[a] = cl - l;
+          b0[a] = static_cast<int>(l);
+        }
+        if (!(moved <= 1.f)) continue;
+      }
+      const float wx[2] = {1.f - f[0], f[0]}, wy[2] = {1.f - f[1], f[1]}, wz[2] = {1.f - f[2], f[2]};
+      const float wzy[4] = {wz[0] * wy[0], wz[0] * wy[1], wz[1] * wy[0], wz[1] * wy[1]};
+      // (an axis one voxel thick: both taps are that voxel, the high one with weight 0)
+      const unsigned bx[2] = {static_cast<unsigned>(b0[0]), static_cast<unsigned>(min(b0[0] + 1, kInterior ? b0[0] + 1 : max(n0 - 1, 0)))};
+      const unsigned by[2] = {static_cast<unsigned>(b0[1]), static_cast<unsigned>(min(b0[1] + 1, kInterior ? b0[1] + 1 : max(n1 - 1, 0)))};
+      const unsigned bz[2] = {static_cast<unsigned>(b0[2]), static_cast<unsigned>(min(b0[2] + 1, kInterior ? b0[2] + 1 : max(n2 - 1, 0)))};
+      const bool inside = max(bx[0], bx[1]) < static_cast<unsigned>(n0) && max(by[0], by[1]) < static_cast<unsigned>(n1) &&
+                          max(bz[0], bz[1]) < static_cast<unsigned>(n2);
+      if (inside) {
+        const float gq = g * gq_scale;
+        const int rows[4] = {__mul24(__mul24(bz[0], n1) + by[0], n0), __mul24(__mul24(bz[0], n1) + by[1], n0),
+                             __mul24(__mul24(bz[1], n1) + by[0], n0), __mul24(__mul24(bz[1], n1) + by[1], n0)};
+#pragma unroll
+        for (int n = 0; n < 8; n++)
+          __hip_atomic_fetch_add(tile + rows[n >> 1] + static_cast<int>(bx[n & 1]),
+                                 __float2int_rn(gq * (wzy[n >> 1] * wx[n & 1])), __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_WORKGROUP);
+      } else {   // (rounding beyond the box's margin: not expected; the voxels exist in the volume)
+#pragma unroll 1
+        for (int n = 0; n < 8; n++) {
+          const float w = wzy[n >> 1] * wx[n & 1];
+          const long zi = l2 + static_cast<int>(bz[n >> 2]), yi = l1 + static_cast<int>(by[(n >> 1) & 1]), xi = l0 + static_cast<int>(bx[n & 1]);
+          if (w != 0.f && zi >= 0 && zi < p.D && yi >= 0 && yi < p.H && xi >= 0 && xi < p.W)
+            atomic_add_element(vol, (zi * p.H + yi) * p.W + xi, g * w);
+        }
+      }
+    }
+    };
     auto scatter_cells = [&](auto interior_tag, auto order_tag) {
     constexpr bool kInterior = decltype(interior_tag)::value;
     constexpr int kOrder = decltype(order_tag)::value;
@@ -1657,14 +1744,17 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
         for (int n = 0; n < 8; n++) {
           const float w = wzy[n >> 1] * wx[n & 1];
           if (w != 0.f)
-            atomic_add(vol + (static_cast<long>(zi[n >> 2]) * p.H + yi[(n >> 1) & 1]) * p.W + xi[n & 1], g * w);
+            atomic_add_element(vol, (static_cast<long>(zi[n >> 2]) * p.H + yi[(n >> 1) & 1]) * p.W + xi[n & 1], g * w);
         }
       }
     }
     };
     using Yes = std::true_type;
     using No = std::false_type;
-    if (mode == 3 && p.ndim == 3) {
+    if (sizeof(T) == 2 && p.order == 1 && in_lds) {
+      if (mode == 3 && p.ndim == 3) scatter_cells32(Yes{});
+      else scatter_cells32(No{});
+    } else if (mode == 3 && p.ndim == 3) {
       if (p.order == 0) scatter_cells(Yes{}, std::integral_constant<int, 0>{});
       else scatter_cells(Yes{}, std::integral_constant<int, 1>{});
     } else {
@@ -1678,6 +1768,37 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
       // before the first is looked at.
       constexpr int kAtOnce = 8;
       const int box = n0 * n1 * n2;
+      if constexpr (DIRECT) {
+        // a lane takes an aligned pair of voxels (volume x even): cells first - l0 and first - l0 + 1 of a
+        // box row, either of which may lie outside the row
+        const int first = l0 & ~1, pairs = ((l0 + n0 + 1) >> 1) - (l0 >> 1), rows = n1 * n2;
+        const float inv_pairs = 1.f / static_cast<float>(pairs), inv_rows = 1.f / static_cast<float>(n1);
+        for (int base = threadIdx.x; base < rows * pairs; base += kScatterThreads * kAtOnce) {
+          int q0[kAtOnce], q1[kAtOnce], cell[kAtOnce], row_[kAtOnce];
+#pragma unroll
+          for (int u = 0; u < kAtOnce; u++) {
+            const int i = base + u * kScatterThreads;
+            const int row = div_small(i, inv_pairs), bx = first - l0 + 2 * (i - row * pairs);
+            const bool on = i < rows * pairs;
+            cell[u] = row * n0 + bx;
+            row_[u] = row;
+            q0[u] = (on && bx >= 0) ? tile[cell[u]] : 0;
+            q1[u] = (on && bx + 1 < n0) ? tile[cell[u] + 1] : 0;
+          }
+#pragma unroll
+          for (int u = 0; u < kAtOnce; u++) {
+            if ((q0[u] | q1[u]) == 0) continue;
+            if (q0[u] != 0) tile[cell[u]] = 0;
+            if (q1[u] != 0) tile[cell[u] + 1] = 0;
+            const int row = row_[u], bx = cell[u] - row * n0;
+            const int bz = div_small(row, inv_rows), by = row - bz * n1;
+            atomic_add_pair(vol + (static_cast<long>(bz + l2) * p.H + (by + l1)) * p.W + (l0 + bx),
+                            static_cast<float>(q0[u]) * from_quanta, static_cast<float>(q1[u]) * from_quanta);
+          }
+        }
+        __syncthreads();
+        continue;
+      }
       const float inv_row = 1.f / static_cast<float>(n0), inv_rows = 1.f / static_cast<float>(n1);
       for (int base = threadIdx.x; base < box; base += kScatterThreads * kAtOnce) {
         int q[kAtOnce];
@@ -1693,8 +1814,8 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
           tile[i] = 0;
           const int row = div_small(i, inv_row), bx = i - row * n0;
           const int bz = div_small(row, inv_rows), by = row - bz * n1;
-          atomic_add(vol + (static_cast<long>(bz + l2) * p.H + (by + l1)) * p.W + (l0 + bx),
-                     static_cast<float>(q[u]) * from_quanta);
+          atomic_add_element(vol, (static_cast<long>(bz + l2) * p.H + (by + l1)) * p.W + (l0 + bx),
+                             static_cast<float>(q[u]) * from_quanta);
         }
       }
       __syncthreads();
@@ -1720,11 +1841,19 @@ bool roi_backward_tiled_applies(int dtype, const RoiProblem &p) {
   return scatter_tiling(p).work < (1L << 31) && static_cast<long>(p.D) * p.H * p.W * 4 < (1L << 31);
 }
 
-// `acc`: fp32 gradient buffer [N, C, D, H, W] that the terms are added to.  Returns -1 when the path
-// does not apply.
-int roi_backward_tiled(const void *grad_output, const void *rois, float *acc, int dtype,
-                       const RoiProblem &p, hipStream_t s) {
+// fp16 gradients whose rows hold an even number of voxels need no fp32 buffer: the tiles' sums go
+// straight into the gradient tensor as packed atomics on pairs of voxels.
+bool roi_backward_tiled_direct(int dtype, const RoiProblem &p, const void *grad_input) {
+  return dtype == MV_F16 && p.W % 2 == 0 && reinterpret_cast<uintptr_t>(grad_input) % 4 == 0 &&
+         roi_backward_tiled_applies(dtype, p);
+}
+
+// `acc`: fp32 gradient buffer [N, C, D, H, W] that the terms are added to, or (`direct`, see above) the
+// fp16 gradient tensor itself.  Returns -1 when the path does not apply.
+int roi_backward_tiled(const void *grad_output, const void *rois, void *acc, int dtype,
+                       const RoiProblem &p, hipStream_t s, bool direct) {
   if (!roi_backward_tiled_applies(dtype, p)) return -1;
+  if (direct && !roi_backward_tiled_direct(dtype, p, acc)) return -1;
   const ScatterTiling t = scatter_tiling(p);
   const bool flat = p.ndim == 2;
   const int TX = t.TX, TY = t.TY, TZ = t.TZ;
@@ -1746,6 +1875,19 @@ int roi_backward_tiled(const void *grad_output, const void *rois, float *acc, in
   ps.by_slots.set(1);
   long blocks = std::min<long>(work, static_cast<long>(kScatterWgs) * compute_units());
   blocks = std::max(blocks, (work + kPlanSlots - 1) / kPlanSlots);
+  if (direct) {
+    if (flat)
+      hipLaunchKernelGGL((roi_backward_tiles_kernel<__half, MV_SCATTER_SHAPE_2D, true>), dim3(static_cast<unsigned>(blocks)),
+                         dim3(kScatterThreads), 0, s, static_cast<const __half *>(grad_output),
+                         static_cast<const float *>(rois), acc, p, ps, static_cast<unsigned>(total),
+                         static_cast<unsigned>(work));
+    else
+      hipLaunchKernelGGL((roi_backward_tiles_kernel<__half, MV_SCATTER_SHAPE, true>), dim3(static_cast<unsigned>(blocks)),
+                         dim3(kScatterThreads), 0, s, static_cast<const __half *>(grad_output),
+                         static_cast<const float *>(rois), acc, p, ps, static_cast<unsigned>(total),
+                         static_cast<unsigned>(work));
+    return check_launch("roi_backward_tiles_kernel");
+  }
   MV_DISPATCH(dtype, {
     if constexpr (sizeof(T) <= 4) {
       if (flat)
