@@ -982,13 +982,22 @@ __device__ inline void pool_backward_mfma(const T *__restrict__ src_any, float *
     // the lane's gradient pieces: cells quad * 8 .. + 7 (+ 32) of every pd of its channel
     u32x4 g[8][2];
     const unsigned g0 = cv ? static_cast<unsigned>(c * cells + quad * 8) * 2u : 0x80000000u;
+    // a piece that reaches past its plane of cells brings the next plane's, channel's or roi's values:
+    // their weights are zero, but 0 x inf is not, so they are cleared
+    u32x4 keep[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+      const int c0 = ks * 32 + quad * 8;
+      auto two = [&](int j) { return (c0 + j < ohw ? 0xffffu : 0u) | (c0 + j + 1 < ohw ? 0xffff0000u : 0u); };
+      keep[ks] = u32x4{two(0), two(2), two(4), two(6)};
+    }
 #pragma unroll
     for (int pd = 0; pd < 8; pd++)
 #pragma unroll
       for (int ks = 0; ks < 2; ks++) {
         g[pd][ks] = u32x4{0u, 0u, 0u, 0u};
         if (pd < p.od && ks * 32 + quad * 8 < ohw)
-          g[pd][ks] = __builtin_amdgcn_raw_buffer_load_b128(gr, g0, (pd * ohw + ks * 32) * 2, 0);
+          g[pd][ks] = __builtin_amdgcn_raw_buffer_load_b128(gr, g0, (pd * ohw + ks * 32) * 2, 0) & keep[ks];
       }
     for (int z = 0; z < nz; z++) {
       float wz[8];
@@ -1103,13 +1112,15 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
   if (dense) {   // (the set-up has built the matrices)
     if constexpr (CL && CELLS == 8 && std::is_same<T, __half>::value && std::is_same<G, float>::value) {
       // matrix-core form: 32-bit offsets into the image's accumulation buffer and into this roi's
-      // gradient; its 16-byte loads may reach 14 bytes past a row of cells, so the roi whose rows end
-      // the tensor stays with the form below
+      // gradient; its 16-byte loads may reach 14 bytes past a row of cells (what they bring from there
+      // is masked out), so blocks whose rows end within 16 bytes of the tensor's end stay with the form below
       const int nxp = (nx + 3) & ~3, kt = (ny * nxp + 15) / 16;
       const bool fits = ny * nxp <= kMfmaYx && kt * 16 * kPoolBwdRow * 2 <= kPoolLdsBytes;
       const bool small = plane * p.C * 4 < (1L << 32) && static_cast<long>(c_end - c_begin) * cells * 2 + 64 < (1L << 31);
-      const bool last = n + 1 == static_cast<unsigned>(p.R) && c_end == p.C;
-      if (fits && small && !last) {
+      // (16 bytes of gradient must follow the block's rows: with few cells per roi that rules out more
+      // than the tensor's last block)
+      const long behind = (static_cast<long>(p.R) * p.C - (static_cast<long>(n) * p.C + c_end)) * cells * 2;
+      if (fits && small && behind >= 16) {
         pool_backward_mfma(src, dst_cl, p, sh, wd, lds, c_end - c_begin);
         return;
       }

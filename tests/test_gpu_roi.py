@@ -257,6 +257,37 @@ def test_pooled_kernels_with_large_boxes(ops, oracle, shape, out, sr, extent, dt
                      "backward")
 
 
+@pytest.mark.parametrize("out", [(1, 1, 1), (1, 2, 3), (2, 3, 3)])
+def test_pooled_backward_reads_only_its_own_gradients(ops, oracle, out):
+    """fp16 heads with a few cells per roi: the matrix-core backward loads a plane of cells as 16-byte
+    pieces that reach into the next plane, channel or roi and, for the last rois, past the tensor.
+    What lies there must not matter: grad_output is the front of a buffer that holds NaN behind it, and
+    one roi's gradient is infinite (it reaches that roi's box alone, as in the oracle)."""
+    g = wl.gen(311)
+    n, channels, size = 60, 5, (13, 39, 39)
+    cells = out[0] * out[1] * out[2]
+    feat = torch.randn(3, channels, *size, generator=g).half()
+    lo = torch.rand(n, 3, generator=g) * torch.tensor([30.0, 30.0, 8.0])
+    rois = torch.cat([torch.randint(0, 3, (n, 1), generator=g).float(), lo, lo + 1 + torch.rand(n, 3, generator=g) * 6], 1)
+    rois[7] = torch.tensor([1, 33.0, 33.0, 9.0, 38.0, 38.0, 12.0])      # a corner of its own
+    keep = ~((rois[:, 0] == 1) & (rois[:, 4] > 32) & (rois[:, 5] > 32) & (rois[:, 6] > 8))
+    keep[7] = True
+    rois = rois[keep]
+    n = rois.size(0)
+    buf = torch.full((n * channels * cells + 64,), float("nan"), dtype=torch.float16)
+    gy = buf[:n * channels * cells].view(n, channels, *out)
+    gy.copy_(torch.randn(gy.shape, generator=g))
+    gy[7, 2] = float("inf")
+    x = feat.to(DEV).requires_grad_(True)
+    y = ops.RoIAlign(out, 1.0, 2)(x, rois.to(DEV))
+    y.backward(buf.to(DEV)[:n * channels * cells].view(n, channels, *out))
+    want = oracle.roi_align_backward(gy, rois, feat.shape, 1.0, 2)
+    got = x.grad.cpu().double()
+    assert torch.isinf(want).any() and torch.equal(torch.isfinite(got), torch.isfinite(want))
+    ok = torch.isfinite(want)
+    assert_close(torch.where(ok, got, 0.0), torch.where(ok, want, 0.0), BWD_TOL[torch.float16], "backward")
+
+
 def test_config3_resize_and_crops(ops, oracle):
     """Benchmark configuration 3 at reduced size: CT-like fp16 volume, resize then rotated 3-D crops."""
     g = wl.gen(2)
