@@ -16,6 +16,14 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
+@pytest.fixture(scope="module")
+def ops():
+    import medvision_amd.ops as ops_
+    from medvision_amd import _lib
+    _lib.load()
+    return ops_
+
+
 def make_case(seed):
     rng = random.Random(seed)
     g = torch.Generator().manual_seed(seed)
