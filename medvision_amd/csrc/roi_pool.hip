@@ -997,8 +997,14 @@ __device__ inline void pool_backward_mfma(const T *__restrict__ src_any, float *
       for (int ks = 0; ks < 2; ks++) {
         g[pd][ks] = u32x4{0u, 0u, 0u, 0u};
         if (pd < p.od && ks * 32 + quad * 8 < ohw)
-          g[pd][ks] = __builtin_amdgcn_raw_buffer_load_b128(gr, g0, (pd * ohw + ks * 32) * 2, 0) & keep[ks];
+          g[pd][ks] = __builtin_amdgcn_raw_buffer_load_b128(gr, g0, (pd * ohw + ks * 32) * 2, 0);
       }
+    // (all loads first, then the masks: a mask right behind its load would wait for it there)
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int pd = 0; pd < 8; pd++)
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++) g[pd][ks] &= keep[ks];
     for (int z = 0; z < nz; z++) {
       float wz[8];
       {
