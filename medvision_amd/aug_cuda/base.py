@@ -76,20 +76,24 @@ class CudaAugBase:
     @staticmethod
     def get_range(val_range, bias=0, always_pos=False):
         """bias + U(lo, hi); a single number r means (-r, r), or (0, r) with ``always_pos``."""
-        if isinstance(val_range, (int, float)):
-            val_range = [0, val_range] if always_pos else [-val_range, val_range]
-        assert isinstance(val_range, (list, tuple)) and len(val_range) == 2
-        assert val_range[1] >= val_range[0]
-        return bias + np.random.uniform(*val_range)
+        if isinstance(val_range, (list, tuple)):
+            if len(val_range) != 2 or val_range[0] > val_range[1]:
+                raise AssertionError(f"a range is (low, high) with low <= high, got {val_range}")
+            low, high = val_range
+        elif isinstance(val_range, (int, float)):
+            low, high = (0, val_range) if always_pos else (-val_range, val_range)
+        else:
+            raise AssertionError(f"a range is a number or a (low, high) pair, got {val_range!r}")
+        return bias + np.random.uniform(low, high)
 
     @staticmethod
     def to_tuple(value, length=1):
-        try:
-            value = tuple(value)
-        except TypeError:
-            value = (value,) * length
-        assert len(value) == length, f'Dimension not match. Required is {length}D but value is {len(value)}D'
-        return value
+        """A scalar repeated ``length`` times; an iterable as a tuple, which must have ``length`` entries."""
+        if np.ndim(value) == 0:
+            return (value,) * length
+        entries = tuple(value)
+        assert len(entries) == length, f'Dimension not match. Required is {length}D but value is {len(entries)}D'
+        return entries
 
     def setLatitude(self, val):
         self.latitude = val
