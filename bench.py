@@ -29,7 +29,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense fp16/bf16
 # returns 64 bytes per clock and compute unit at the ~1.97 GHz these kernels run at.
 VALU_NS_PER_WAVE_INSTR = 2.03
 SIMDS, CUS, L1_BYTES_PER_CLK, SHADER_GHZ = 1024, 256, 64, 1.97
-DCN_L1_MISS_REQUESTS = 3.16e7   # config 4 forward, 64-byte requests from the L1s to the L2s per launch
+DCN_L1_MISS_REQUESTS = 2.74e7   # config 4 forward, 64-byte requests from the L1s to the L2s per launch
 L2_GATHER_TBPS = 15.0           # measured line rate of the L2s for scattered 16-byte gathers
 
 
