@@ -220,8 +220,9 @@ def bench_other_configs(args):
     sh = (torch.rand(8, 2, generator=g) * 2 - 1) * 10
     rois = torch.cat([torch.arange(8, dtype=torch.float32)[:, None], 256 + sh, 512 / sc.expand(8, 2), ang], 1).to(dev)
     ms, _ = _events_ms(lambda i: ops.affine_2d(img, rois, (512, 512), 1.0, 1, True, 1), 100, 10)
+    ms3, _ = _events_ms(lambda i: ops.affine_2d(img, rois, (512, 512), 1.0, 1, True, 3), 100, 10)
     res["affine_2d_8x3x512^2_fp16"] = {"ms": round(ms, 4), "gpix_s": round(img.numel() / ms / 1e6, 2),
-                                       "gbps": round(2 * img.numel() * 2 / ms / 1e6, 1)}
+                                       "gbps": round(2 * img.numel() * 2 / ms / 1e6, 1), "order3_ms": round(ms3, 4)}
     return res
 
 

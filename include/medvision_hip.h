@@ -92,7 +92,7 @@ size_t mv_roi_align_backward_workspace_bytes(int dtype, int batch, int channels,
                                              int height, int width);
 /* Workspace of the forward entry points (plain, rotated and affine).  0 for a sampling grid of 1 on
  * volumes (the kernels keep their per-call state in LDS), 40 bytes per roi for images of resampling
- * size (orders 0 / 1: their rois are rewritten for the tiled kernel); for fp16 / fp32 outputs of resampling size with a
+ * size (their rois are rewritten for the tiled kernel); for fp16 / fp32 outputs of resampling size with a
  * fixed sampling_ratio of 2..4 the bytes of the bins' samples (sampling_ratio^ndim per output
  * element), which a second pass averages (volumes at order 1 with a grid of 2 or 4, of any of the three
  * types, take the means inside the kernel and leave the workspace untouched; the query is not told

@@ -396,7 +396,9 @@ __device__ __forceinline__ void catmull_rom(float u, float (&w)[4]) {
   w[3] = 0.5f * u3 - 0.5f * u2;
 }
 
-template <typename T, typename CT, bool INTERIOR, bool WIDE>
+// ONE_ROW: the middle axis is one voxel thick (images as volumes of rows): its four taps are that voxel
+// with weights that sum to 1 (0, 1, 0, 0 at the coordinate the one cell is sampled at), so they are left out.
+template <typename T, typename CT, bool INTERIOR, bool WIDE, bool ONE_ROW = false>
 __device__ __forceinline__ float staged_cubic(const T *__restrict__ tile, CT rx, CT ry, CT rz,
                                               const BoxLimits<CT> &b, int pitch, long slice, int dy, long dz) {
   // void samples: an all-zero bit mask applied to the result (kept as data so that the 64 taps
@@ -443,11 +445,16 @@ __device__ __forceinline__ float staged_cubic(const T *__restrict__ tile, CT rx,
     for (int a = 0; a < 4; a++) {
       const int za = min(max(bz - 1 + a, 0), tz) * sz;
       float plane = 0.f;
+      if constexpr (ONE_ROW) {
+        const T *row = tile + za;
+        plane = wx[0] * load(row + ox[0]) + wx[1] * load(row + ox[1]) + wx[2] * load(row + ox[2]) + wx[3] * load(row + ox[3]);
+      } else {
 #pragma unroll
-      for (int c = 0; c < 4; c++) {
-        const T *row = tile + (za + min(max(by - 1 + c, 0), ty) * sy);
-        plane += wy[c] * (wx[0] * load(row + ox[0]) + wx[1] * load(row + ox[1]) + wx[2] * load(row + ox[2]) +
-                          wx[3] * load(row + ox[3]));
+        for (int c = 0; c < 4; c++) {
+          const T *row = tile + (za + min(max(by - 1 + c, 0), ty) * sy);
+          plane += wy[c] * (wx[0] * load(row + ox[0]) + wx[1] * load(row + ox[1]) + wx[2] * load(row + ox[2]) +
+                            wx[3] * load(row + ox[3]));
+        }
       }
       acc += wz[a] * plane;
     }
@@ -1108,7 +1115,8 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_cubic_kernel(
     bool sep = false;
     if (mode == 1 || mode == 3) {
       const CT *m = plan_map<CT>(rec);
-      sep = m[2] == CT(0) && m[3] == CT(0) && m[5] == CT(0) && m[7] == CT(0) && m[9] == CT(0) && m[10] == CT(0) &&
+      // (images as volumes of rows: 16 taps per pixel are cheaper than three passes of which one copies)
+      sep = TY > 1 && m[2] == CT(0) && m[3] == CT(0) && m[5] == CT(0) && m[7] == CT(0) && m[9] == CT(0) && m[10] == CT(0) &&
             (static_cast<long>(first_f) + bz * by * TX + bz * TY * TX) * 4 + 3 * TS * static_cast<long>(sizeof(AxisTaps3)) <= LDS_BYTES;
       if (sep && tid < TX + TY + TZ) {
         const int a = tid < TX ? 0 : (tid < TX + TY ? 1 : 2), o = tid - (a == 0 ? 0 : (a == 1 ? TX : TX + TY));
@@ -1194,7 +1202,7 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_cubic_kernel(
 #pragma unroll 1
         for (int k = 0; k < count; k++) {
           const CT kk = static_cast<CT>(k);
-          drow[k * zstride] = store_cast<T>(staged_cubic<T, CT, false, true>(
+          drow[k * zstride] = store_cast<T>(staged_cubic<T, CT, false, true, TY == 1>(
               src, b[0] + kk * st[0], b[1] + kk * st[1], b[2] + kk * st[2], lim, W, hw, W, hw));
         }
       } else {
@@ -1202,7 +1210,7 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_cubic_kernel(
 #pragma unroll 1
         for (int k = 0; k < count; k++) {
           const CT kk = static_cast<CT>(k);
-          drow[k * zstride] = store_cast<T>(staged_cubic<T, CT, false, false>(
+          drow[k * zstride] = store_cast<T>(staged_cubic<T, CT, false, false, TY == 1>(
               tile, b[0] + kk * st[0], b[1] + kk * st[1], b[2] + kk * st[2], lim, pitch, slice, dy, dz));
         }
       }
@@ -1404,7 +1412,7 @@ __global__ void roi_rows_as_slices_kernel(const float *__restrict__ flat, float 
 static int roi_forward_tiled_image(const void *input, const void *rois, void *output, int dtype, const RoiProblem &p,
                                    void *workspace, size_t capacity, size_t *need, hipStream_t s) {
   const long vox = static_cast<long>(p.oh) * p.ow;
-  if (p.sampling_ratio != 1 || p.order == 3 || vox < 4096 || p.ow < 16 || p.R == 0) return -1;
+  if (p.sampling_ratio != 1 || vox < 4096 || p.ow < 16 || p.R == 0) return -1;
   if (vox * 4 >= (1L << 31)) return -1;
   if (dtype != MV_F16 && dtype != MV_BF16 && dtype != MV_F32) return -1;
   // (the workspace query does not know whether the rois are rotated: room for the wider rows)
@@ -1420,6 +1428,24 @@ static int roi_forward_tiled_image(const void *input, const void *rois, void *ou
                        vol_rois, p.R, p.rotated, p.aligned, static_cast<float>(p.scale));
   }
   int st;
+  if (p.order == 3) {
+    // (the one cell of the middle axis samples row 0 exactly: its four taps are that row with weights 0, 1, 0, 0)
+    switch (dtype) {
+      case MV_F16:
+        st = launch_resample<__half, 64, 1, 64, 512, 74 * 1024, 8, true>(static_cast<const __half *>(input), vol_rois,
+                                                                          static_cast<__half *>(output), v, nullptr, need, s);
+        break;
+      case MV_BF16:
+        st = launch_resample<__hip_bfloat16, 64, 1, 64, 512, 74 * 1024, 8, true>(
+            static_cast<const __hip_bfloat16 *>(input), vol_rois, static_cast<__hip_bfloat16 *>(output), v, nullptr, need, s);
+        break;
+      default:
+        st = launch_resample<float, 64, 1, 64, 512, 74 * 1024, 6, true>(static_cast<const float *>(input), vol_rois,
+                                                                         static_cast<float *>(output), v, nullptr, need, s);
+    }
+    if (need && st == MV_OK) *need = bytes;
+    return st;
+  }
   switch (dtype) {
     case MV_F16:
       st = launch_resample<__half, 64, 1, 64, 512, 74 * 1024, 8>(static_cast<const __half *>(input), vol_rois,
@@ -1444,8 +1470,7 @@ int roi_forward_tiled(const void *input, const void *rois, void *output, int dty
                       const RoiProblem &p, void *workspace, size_t capacity, size_t *need, hipStream_t s) {
   if (p.sampling_ratio >= 2 && p.sampling_ratio <= 4)
     return roi_forward_tiled_grid(input, rois, output, dtype, p, workspace, capacity, need, s);
-  // images: rows as slices (orders 0 and 1; order 3 stays on the one-thread-per-output kernel, which
-  // took 0.109 against 0.185 ms through depth-1 tiles)
+  // images: rows as slices
   if (p.ndim == 2) return roi_forward_tiled_image(input, rois, output, dtype, p, workspace, capacity, need, s);
   const long vox = static_cast<long>(p.od) * p.oh * p.ow;
   if (p.sampling_ratio != 1 || vox < 4096 || p.ow < 16 || p.R == 0) return -1;

@@ -357,8 +357,8 @@ def test_tiled_resampler_2d(ops, oracle, dtype, width):
     """Images of resampling size run the tiled kernel as volumes whose slices are the image rows (the
     rois are rewritten on the device: one cell on the middle axis that samples row 0, the rotation about
     that axis): rotated rois beyond every border, both `aligned` settings, a spatial scale that is no
-    power of two, orders 0 and 1, rows of whole 16-byte groups and ragged ones, plain boxes, several
-    channels; order 3 stays on the one-thread-per-output kernel."""
+    power of two, orders 0, 1 and 3 (order 3: the four taps of the middle axis are its one row and are
+    left out), rows of whole 16-byte groups and ragged ones, plain boxes, several channels."""
     g = wl.gen(37 + width)
     img = torch.randn(2, 3, 96, width, generator=g).to(dtype)
     rois = torch.tensor([[0, 60.3, 47.1, 130.0, 90.0, 0.4], [1, 50.0, 40.0, 70.0, 110.0, -0.7],
@@ -386,6 +386,11 @@ def test_tiled_resampler_2d(ops, oracle, dtype, width):
     ident = torch.tensor([[b, width / 2, 48, width, 96, 0] for b in range(2)], dtype=torch.float32)
     same = ops.affine_2d(x, ident.to(DEV), (96, width), 1.0, 1, True, 1)
     assert torch.equal(same.cpu(), img)
+    assert torch.equal(ops.affine_2d(x, ident.to(DEV), (96, width), 1.0, 1, True, 3).cpu(), img)
+    # order 3 without rotation (a resize): windows that reach beyond every border
+    got = ops.affine_2d(x, ident.to(DEV), (130, 77), 1.0, 1, True, 3)
+    want = oracle.roi_align_forward(img, ident, (130, 77), 1.0, 1, True, 3, True)
+    assert_close(got, want, FWD_TOL[dtype], "order 3 resize of images")
     # plain boxes with one sample per cell
     boxes = torch.tensor([[0, 3.2, 1.7, 100.4, 80.9], [1, -10.0, 20.0, 60.0, 120.0]], dtype=torch.float32)
     got = ops.RoIAlign(out, 1.0, 1)(x, boxes.to(DEV))
