@@ -715,7 +715,10 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
   constexpr int ZPL = TZ / RZ;             // consecutive output slices per lane
   constexpr int ES = sizeof(T);
   constexpr int ZO = ZPL / G;              // slices a lane stores
-  static_assert(G == 1 || (ZPL % G == 0 && TX % G == 0 && (kWave / TX) % G == 0 && kWave % TX == 0 && TY % (kWave / TX) == 0),
+  // (images as volumes of rows, TY = 1: the middle axis has one cell and takes no part; blocks of G x G)
+  constexpr int GY = TY == 1 ? 1 : G;
+  static_assert(G == 1 || (ZPL % G == 0 && TX % G == 0 && kWave % TX == 0 &&
+                           (TY == 1 || ((kWave / TX) % G == 0 && TY % (kWave / TX) == 0))),
                 "blocks of G x G x G voxels lie inside a wavefront's lanes and a lane's column");
   __shared__ __attribute__((aligned(16))) T tile[kCap];
   __shared__ __attribute__((aligned(16))) TilePlan lplans[kPlanSlots];
@@ -743,11 +746,11 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
   const int lx = tid % TX, ly = (tid / TX) % TY, lz = tid / (TX * TY);
   const CT fx = static_cast<CT>(lx), fy = static_cast<CT>(ly), fz = static_cast<CT>(lz * ZPL);
   const float tid_h = static_cast<float>(tid) + 0.5f;
-  const int oh_o = oh / G, ow_o = ow / G;   // the volume that is written
+  const int oh_o = oh / GY, ow_o = ow / G;   // the volume that is written
   const int zbytes = oh_o * ow_o * ES;
   const int out_bytes = (p.od / G) * zbytes;   // bytes of one output volume (< 2^31, checked by the host)
-  const unsigned lane_out = static_cast<unsigned>(((lz * ZO * oh_o + ly / G) * ow_o + lx / G) * ES);
-  const bool lane_stores = lx % G == 0 && ly % G == 0;
+  const unsigned lane_out = static_cast<unsigned>(((lz * ZO * oh_o + ly / GY) * ow_o + lx / G) * ES);
+  const bool lane_stores = lx % G == 0 && ly % GY == 0;
   const int w_bytes = W * ES;
   const unsigned hw_bytes = static_cast<unsigned>(H) * W * ES;   // < 2^31, checked by the host
   // lane `tid` holds group `tid` of every pass: its place in LDS, slices `gap` bytes apart
@@ -989,13 +992,15 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
         for (int j = 1; j < G; j++) sum += o[kk * G + j];
         sum += __shfl_down(sum, 1);
         if (G == 4) sum += __shfl_down(sum, 2);
-        sum += __shfl_down(sum, TX);
-        if (G == 4) sum += __shfl_down(sum, 2 * TX);
-        held[kk] = sum * (1.f / static_cast<float>(G * G * G));
+        if constexpr (GY > 1) {
+          sum += __shfl_down(sum, TX);
+          if (G == 4) sum += __shfl_down(sum, 2 * TX);
+        }
+        held[kk] = sum * (1.f / static_cast<float>(G * GY * G));
       }
       // the (roi, channel) volume and the tile's first block in it (tile origins are multiples of G)
-      const int bx = plan_scalar(&rec->t0[0]) / G, by0 = plan_scalar(&rec->t0[1]) / G, bz0 = plan_scalar(&rec->t0[2]) / G;
-      pend_base = reinterpret_cast<const char *>(out) + plan.u64(MV_PLAN_DW(out_lo)) / (G * G * G);
+      const int bx = plan_scalar(&rec->t0[0]) / G, by0 = plan_scalar(&rec->t0[1]) / GY, bz0 = plan_scalar(&rec->t0[2]) / G;
+      pend_base = reinterpret_cast<const char *>(out) + plan.u64(MV_PLAN_DW(out_lo)) / (G * GY * G);
       pend_voff = (lane_stores && lx < t.y && ly < t.z)
                       ? lane_out + static_cast<unsigned>(((bz0 * oh_o + by0) * ow_o + bx) * ES) : kOutOfRange;
       pend_bytes = out_bytes;
@@ -1340,12 +1345,16 @@ static int roi_forward_tiled_means(const void *input, const void *rois, void *ou
 // the means: 16-bit samples are then rounded before the mean is; fp16's two roundings stay within its
 // tolerance, bf16's would not, so bf16 then keeps the general kernel.  (The workspace query does not
 // know the order and answers for the two passes.)
+static int roi_forward_tiled_image(const void *input, const void *rois, void *output, int dtype, const RoiProblem &p,
+                                   void *workspace, size_t capacity, size_t *need, hipStream_t s, int pool);
+
 static int roi_forward_tiled_grid(const void *input, const void *rois, void *output, int dtype,
                                   const RoiProblem &p, void *workspace, size_t capacity, size_t *need, hipStream_t s) {
   const int g = p.sampling_ratio, gz = p.ndim == 3 ? g : 1;
-  const bool in_kernel = !need && p.ndim == 3 && p.order == 1 && (g == 2 || g == 4) && p.R > 0 &&
-                         (dtype == MV_F16 || dtype == MV_BF16 || dtype == MV_F32);
-  if (dtype != MV_F16 && dtype != MV_F32 && !in_kernel) return -1;
+  // the means inside the kernel: grids of 2 and 4 at order 1 (images need their rewritten rois in the workspace)
+  const bool means = (g == 2 || g == 4) && p.R > 0 && (dtype == MV_F16 || dtype == MV_BF16 || dtype == MV_F32);
+  const bool in_kernel = !need && means && p.order == 1;
+  if (dtype != MV_F16 && dtype != MV_F32 && !means) return -1;
   if (!need && p.order != 1 && p.order != 3) return -1;
   // Outputs that the grid-1 rule sends here, except those of <= 16 cells per axis (the pooled kernels
   // take plain boxes of that size).  Only values that the workspace query also knows may decide.
@@ -1358,11 +1367,16 @@ static int roi_forward_tiled_grid(const void *input, const void *rois, void *out
   const long fine = cells * gz * g * g;
   // (32-bit byte offsets inside one finer volume, as in the grid-1 rule)
   if (in_kernel && static_cast<long>(f.od) * f.oh * f.ow * 4 < (1L << 31)) {
-    const int st = g == 2 ? roi_forward_tiled_means<2>(input, rois, output, dtype, f, s)
-                          : roi_forward_tiled_means<4>(input, rois, output, dtype, f, s);
+    int st;
+    if (p.ndim == 2) st = roi_forward_tiled_image(input, rois, output, dtype, f, workspace, capacity, nullptr, s, g);
+    else st = g == 2 ? roi_forward_tiled_means<2>(input, rois, output, dtype, f, s)
+                     : roi_forward_tiled_means<4>(input, rois, output, dtype, f, s);
     if (st != -1) return st;
   }
-  if (dtype != MV_F16 && dtype != MV_F32) return -1;
+  if (dtype != MV_F16 && dtype != MV_F32) {   // bf16: the means inside the kernel or nothing
+    if (need && p.ndim == 2) return roi_forward_tiled_image(nullptr, nullptr, nullptr, dtype, f, nullptr, 0, need, nullptr, g);
+    return -1;
+  }
   if (fine >= (1L << 31) || (cells + 255) / 256 >= (1L << 31)) return -1;
   size_t inner = 0;
   if (roi_forward_tiled(nullptr, nullptr, nullptr, dtype, f, nullptr, 0, &inner, nullptr) != MV_OK) return -1;
@@ -1409,10 +1423,13 @@ __global__ void roi_rows_as_slices_kernel(const float *__restrict__ flat, float 
   }
 }
 
+// pool = 2 or 4: `p` is the problem on the finer grid of a fixed sampling grid (order 1) and `output` takes
+// the bins' means (see roi_forward_tiled_grid).
 static int roi_forward_tiled_image(const void *input, const void *rois, void *output, int dtype, const RoiProblem &p,
-                                   void *workspace, size_t capacity, size_t *need, hipStream_t s) {
+                                   void *workspace, size_t capacity, size_t *need, hipStream_t s, int pool) {
   const long vox = static_cast<long>(p.oh) * p.ow;
   if (p.sampling_ratio != 1 || vox < 4096 || p.ow < 16 || p.R == 0) return -1;
+  if (pool != 1 && ((!need && p.order != 1) || (pool != 2 && pool != 4))) return -1;   // (a size query is not told the order)
   if (vox * 4 >= (1L << 31)) return -1;
   if (dtype != MV_F16 && dtype != MV_BF16 && dtype != MV_F32) return -1;
   // (the workspace query does not know whether the rois are rotated: room for the wider rows)
@@ -1446,6 +1463,19 @@ static int roi_forward_tiled_image(const void *input, const void *rois, void *ou
     if (need && st == MV_OK) *need = bytes;
     return st;
   }
+  if (pool != 1) {
+#define MV_IMAGE_MEANS(TYPE, TZV, KMAXV, GV)                                                                         \
+  launch_resample<TYPE, 64, 1, TZV, 512, 74 * 1024, KMAXV, false, GV>(static_cast<const TYPE *>(input), vol_rois, \
+                                                                       static_cast<TYPE *>(output), v, nullptr, need, s)
+    switch (dtype) {
+      case MV_F16: st = pool == 2 ? MV_IMAGE_MEANS(__half, 64, 8, 2) : MV_IMAGE_MEANS(__half, 64, 8, 4); break;
+      case MV_BF16: st = pool == 2 ? MV_IMAGE_MEANS(__hip_bfloat16, 64, 8, 2) : MV_IMAGE_MEANS(__hip_bfloat16, 64, 8, 4); break;
+      default: st = pool == 2 ? MV_IMAGE_MEANS(float, 32, 6, 2) : MV_IMAGE_MEANS(float, 32, 6, 4);
+    }
+#undef MV_IMAGE_MEANS
+    if (need && st == MV_OK) *need = bytes;
+    return st;
+  }
   switch (dtype) {
     case MV_F16:
       st = launch_resample<__half, 64, 1, 64, 512, 74 * 1024, 8>(static_cast<const __half *>(input), vol_rois,
@@ -1471,7 +1501,7 @@ int roi_forward_tiled(const void *input, const void *rois, void *output, int dty
   if (p.sampling_ratio >= 2 && p.sampling_ratio <= 4)
     return roi_forward_tiled_grid(input, rois, output, dtype, p, workspace, capacity, need, s);
   // images: rows as slices
-  if (p.ndim == 2) return roi_forward_tiled_image(input, rois, output, dtype, p, workspace, capacity, need, s);
+  if (p.ndim == 2) return roi_forward_tiled_image(input, rois, output, dtype, p, workspace, capacity, need, s, 1);
   const long vox = static_cast<long>(p.od) * p.oh * p.ow;
   if (p.sampling_ratio != 1 || vox < 4096 || p.ow < 16 || p.R == 0) return -1;
   if (vox * 4 >= (1L << 31)) return -1;   // 32-bit byte offsets inside one output volume

@@ -423,8 +423,8 @@ def test_cubic_affine_vs_oracle(ops, oracle, dtype, ndim, sr):
 @pytest.mark.parametrize("sr", [2, 3, 4])
 def test_large_outputs_with_a_sampling_grid(ops, oracle, dtype, sr):
     """sampling_ratio 2..4 on outputs of resampling size: the tiled kernel works on the sr times finer
-    grid of the bins' samples.  Volumes at order 1 with a grid of 2 or 4 (any of the three types) take
-    the means of the bins inside that kernel; a grid of 3, images and order 3 write the finer volume
+    grid of the bins' samples.  Order 1 with a grid of 2 or 4 (volumes and images, any of the three
+    types) takes the means of the bins inside that kernel; a grid of 3 and order 3 write the finer volume
     and a second pass takes the means (fp16 / fp32; bf16 then stays on the general kernel).  Rotated
     and plain rois in 3-D and 2-D, order 1, and order 3 through the affine engine; a second output
     shape whose finer grid ends inside a tile on every axis."""
