@@ -153,8 +153,7 @@ def bench_other_configs(args):
         nbytes = 3 * vol.numel() * vol.element_size()
         res["config2_backward_" + name] = {"ms": round(ms, 4), "gbps": round(nbytes / ms / 1e6, 1),
                                            "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
-    # config 2 with a sampling grid of 2 per axis (8 samples per output voxel, means taken inside the
-    # tiled kernel)
+    # config 2 with a sampling grid of 2 per axis (8 samples per output voxel, summed inside the tiled kernel)
     g = wl.gen(1)
     r = wl.affine_rois(g, 4, (128, 128, 128)).to(dev)
     for dt, name in ((torch.float16, "fp16"), (torch.bfloat16, "bf16")):

@@ -94,9 +94,9 @@ size_t mv_roi_align_backward_workspace_bytes(int dtype, int batch, int channels,
  * volumes (the kernels keep their per-call state in LDS), 40 bytes per roi for images of resampling
  * size (their rois are rewritten for the tiled kernel); for fp16 / fp32 outputs of resampling size with a
  * fixed sampling_ratio of 2..4 the bytes of the bins' samples (sampling_ratio^ndim per output
- * element), which a second pass averages (order 1 with a grid of 2 or 4, fp16 / bf16 / fp32: the means are
- * taken inside the kernel, volumes leave the workspace untouched and images use 40 bytes per roi of it;
- * the query is not told the order and answers for order 3).  The forward entry points take the workspace together
+ * element), which a second pass averages (orders 0 and 1 sum the samples of a bin inside the
+ * kernel, for any grid, fixed or per roi, and any of the three types: volumes leave the workspace
+ * untouched, images use 40 bytes per roi of it; the query is not told the order and answers for order 3).  The forward entry points take the workspace together
  * with its size in bytes (`workspace_bytes`) and use a path only when the workspace holds what that
  * path needs: NULL, or a workspace that is too small, selects the kernels that need none (same
  * results, slower), never an access beyond `workspace_bytes`.  ndim = 2 or 3 (out_d ignored for 2). */

@@ -62,7 +62,7 @@ struct TilePlan {            // 352 bytes
   int stride;                // bytes between the passes of a lane (span slices)
   unsigned out_lo, out_hi;   // byte offset of the item's (roi, channel) volume in the output tensor
   int zcount;                // output slices from the tile's first one to the end of the volume
-  int pad0[3];
+  int grid[3];               // samples per bin along (x, y, z): the fixed ratio, or ceil(roi extent / cells)
   // dword 48: a lane splits its index into (slice, row, 16-byte group) with two multiplications
   float inv_groups, inv_rows;
   int groups, by;
@@ -113,6 +113,8 @@ struct PlanShape {
   int es;                         // bytes per element
   FastDiv by_per_roi, by_tiles_x, by_tiles_y, by_total, by_slots;
   int halo_lo, halo_hi;           // voxels needed below / above the cell of a sample: 0 / 1, order 3: 1 / 2
+  int grids;                      // 1: the kernel takes every sample of a bin (else items with grids above 1 are void)
+  int flat_axis;                  // 1: the middle axis has one cell sampled once whatever the ratio (images as volumes of rows)
   unsigned warm_groups;           // 16-byte groups of the input to pull into the caches during planning (0: none)
   int pad_slices;                 // 1: LDS slices of a box start 32 bytes past a multiple of 128
 };
@@ -170,6 +172,7 @@ __device__ inline void plan_item_lanes(const float *__restrict__ rois, const Roi
     }
     bin = ext / static_cast<double>(out_cells);
     grid = p.sampling_ratio > 0 ? p.sampling_ratio : static_cast<int>(ceil(ext / static_cast<double>(out_cells)));
+    if (ps.flat_axis && ax == 1) grid = 1;
     sub = bin / static_cast<double>(grid > 0 ? grid : 1);
   }
   const int b = static_cast<int>(roi[0]);
@@ -198,7 +201,8 @@ __device__ inline void plan_item_lanes(const float *__restrict__ rois, const Roi
   const int t0 = tpos * tile_ext;
   const int cells = min(tile_ext, out_cells - t0);
   const double first = live_axis ? start + t0 * bin + static_cast<double>(.5f) * sub : 0.0;
-  const double half = live_axis ? 0.5 * (cells - 1) * bin : 0.0;
+  // (from the first sample of the tile's first cell to the last sample of its last cell)
+  const double half = live_axis ? 0.5 * ((cells - 1) * bin + (grid - 1) * sub) : 0.0;
   double mid = centre, reach = 0.0, pos = centre, inc[3];
   int grids = 1;
 #pragma unroll
@@ -216,7 +220,7 @@ __device__ inline void plan_item_lanes(const float *__restrict__ rois, const Roi
   if (is3d || ax < 2) {
     // widen by more than the rounding of the per-voxel coordinate arithmetic
     const double eps = 4e-5, rmin = mid - reach - eps, rmax = mid + reach + eps;
-    empty = rmax < -1.0 || rmin > S;
+    empty = rmax < -1.0 || rmin > S || grid <= 0;   // (an adaptive grid of a roi without extent: no samples, zeros)
     clipped = rmin < static_cast<double>(ps.halo_lo) || rmax > S - ps.halo_hi;
     int l = static_cast<int>(fmin(fmax(floor(fmax(rmin, 0.0)) - ps.halo_lo, 0.0), static_cast<double>(S - 1)));
     int h = static_cast<int>(fmin(floor(fmax(rmax, 0.0)) + ps.halo_hi, static_cast<double>(S - 1)));
@@ -263,7 +267,7 @@ __device__ inline void plan_item_lanes(const float *__restrict__ rois, const Roi
       }
       const bool fits = static_cast<long>(n2) * slice_e <= ps.cap;
       int mode;
-      if (batch < 0 || any_empty || !grids) mode = 0;   // (grid != 1 cannot happen: ratio is 1)
+      if (batch < 0 || any_empty || (!grids && !ps.grids)) mode = 0;   // (kernels without grids are launched at ratio 1)
       else if (!fits) mode = 2;
       else mode = any_clip ? 1 : 3;
       const int rp = span * n1;
@@ -291,6 +295,7 @@ __device__ inline void plan_item_lanes(const float *__restrict__ rois, const Roi
   }
   dst->lo[a] = lo;
   dst->n[a] = cnt;
+  dst->grid[a] = live_axis ? grid : 1;
   dst->t0[a] = t0;
   dst->cmaxf[a] = static_cast<float>(S - 1 - lo);
   dst->topf[a] = static_cast<float>(max(cnt - 2, 0));
@@ -704,6 +709,9 @@ __device__ __forceinline__ void clipped_column(const T *__restrict__ tile, float
 // G > 1: the problem handed in is the one on the G times finer grid of the bins' samples (cell * G + sub
 // of a fixed sampling grid of G per axis), and every G x G x G block of its voxels leaves as one mean:
 // G slices summed in the lane, the x and y neighbours through lane exchanges, one store per block.
+// G = 0: any sampling grid, fixed or per roi (ceil(roi extent / cells)): the problem is the one asked for,
+// a lane walks the samples of each of its bins in a loop (the plan holds the grid of the item's roi and
+// a box that covers every sample) and keeps their sum in a register.
 template <typename T, int TX, int TY, int TZ, int THREADS, int LDS_BYTES, int KMAX, int ORDER, int G = 1>
 __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
     const T *__restrict__ feat, const float *__restrict__ rois, T *__restrict__ out, const RoiProblem p, const PlanShape ps, const unsigned total, const unsigned work) {
@@ -714,10 +722,11 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
   static_assert((TX * TY) % kWave == 0, "a wavefront's lanes share their z layer");
   constexpr int ZPL = TZ / RZ;             // consecutive output slices per lane
   constexpr int ES = sizeof(T);
-  constexpr int ZO = ZPL / G;              // slices a lane stores
+  constexpr int GO = G > 1 ? G : 1;        // output voxels are means of GO^3 (images: GO^2) voxels of the problem
+  constexpr int ZO = ZPL / GO;             // slices a lane stores
   // (images as volumes of rows, TY = 1: the middle axis has one cell and takes no part; blocks of G x G)
-  constexpr int GY = TY == 1 ? 1 : G;
-  static_assert(G == 1 || (ZPL % G == 0 && TX % G == 0 && kWave % TX == 0 &&
+  constexpr int GY = TY == 1 ? 1 : GO;
+  static_assert(G <= 1 || (ZPL % G == 0 && TX % G == 0 && kWave % TX == 0 &&
                            (TY == 1 || ((kWave / TX) % G == 0 && TY % (kWave / TX) == 0))),
                 "blocks of G x G x G voxels lie inside a wavefront's lanes and a lane's column");
   __shared__ __attribute__((aligned(16))) T tile[kCap];
@@ -746,11 +755,11 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
   const int lx = tid % TX, ly = (tid / TX) % TY, lz = tid / (TX * TY);
   const CT fx = static_cast<CT>(lx), fy = static_cast<CT>(ly), fz = static_cast<CT>(lz * ZPL);
   const float tid_h = static_cast<float>(tid) + 0.5f;
-  const int oh_o = oh / GY, ow_o = ow / G;   // the volume that is written
+  const int oh_o = oh / GY, ow_o = ow / GO;   // the volume that is written
   const int zbytes = oh_o * ow_o * ES;
-  const int out_bytes = (p.od / G) * zbytes;   // bytes of one output volume (< 2^31, checked by the host)
-  const unsigned lane_out = static_cast<unsigned>(((lz * ZO * oh_o + ly / GY) * ow_o + lx / G) * ES);
-  const bool lane_stores = lx % G == 0 && ly % GY == 0;
+  const int out_bytes = (p.od / GO) * zbytes;   // bytes of one output volume (< 2^31, checked by the host)
+  const unsigned lane_out = static_cast<unsigned>(((lz * ZO * oh_o + ly / GY) * ow_o + lx / GO) * ES);
+  const bool lane_stores = lx % GO == 0 && ly % GY == 0;
   const int w_bytes = W * ES;
   const unsigned hw_bytes = static_cast<unsigned>(H) * W * ES;   // < 2^31, checked by the host
   // lane `tid` holds group `tid` of every pass: its place in LDS, slices `gap` bytes apart
@@ -761,7 +770,7 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
   float o[ZPL];      // the previous item's outputs
   [[maybe_unused]] float held[ZO];   // G > 1: the previous item's means (o then belongs to the current item)
   auto pending = [&](int k) -> float {
-    if constexpr (G == 1) return o[k];
+    if constexpr (G <= 1) return o[k];
     else return held[k];
   };
   // outputs waiting to be stored: the (roi, channel) volume, the lane's byte offset in it (out of
@@ -941,7 +950,58 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
         b[a] = m[4 * a] + fx * m[4 * a + 1] + fy * m[4 * a + 2] + fz * m[4 * a + 3];
         st[a] = m[4 * a + 3];
       }
-      if (mode == 3 && sizeof(CT) == 4) {
+      if constexpr (G == 0) {
+        // every sample of the bins: sample (ix, iy, iz) of a bin lies ix / gx, iy / gy, iz / gz of a cell
+        // further along the output axes (the plan's origin is sample (0, 0, 0) of the tile's first cell)
+        const int gx = plan.i32(MV_PLAN_DW(grid)), gy = plan.i32(MV_PLAN_DW(grid) + 1), gz = plan.i32(MV_PLAN_DW(grid) + 2);
+        const CT igx = CT(1) / static_cast<CT>(gx), igy = CT(1) / static_cast<CT>(gy), igz = CT(1) / static_cast<CT>(gz);
+        CT sx[3], sy[3], sz[3];
+#pragma unroll
+        for (int a = 0; a < 3; a++) { sx[a] = m[4 * a + 1] * igx; sy[a] = m[4 * a + 2] * igy; sz[a] = m[4 * a + 3] * igz; }
+        const float inv_count = 1.f / static_cast<float>(gx * gy * gz);
+        const int size[3] = {W, H, p.D};
+        BoxLimits<CT> lim;
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+          const int lo = mode == 2 ? 0 : plan_scalar(&rec->lo[a]);
+          const int n = mode == 2 ? size[a] : plan_scalar(&rec->n[a]);
+          lim.cmax[a] = uniform(static_cast<CT>(size[a] - 1 - lo));
+          lim.top[a] = uniform(static_cast<CT>(max(n - 2, 0)));
+        }
+        auto bins = [&](auto wide_tag, const T *base, int pitch, long slice, int dy, long dz) {
+          constexpr bool kWide = decltype(wide_tag)::value;
+          const float pitch_f = uniform(static_cast<float>(pitch)), slice_f = uniform(static_cast<float>(slice));
+#pragma unroll
+          for (int k = 0; k < ZPL; k++) {
+            before(k);
+            const CT kk = static_cast<CT>(k);
+            const CT c0 = b[0] + kk * st[0], c1 = b[1] + kk * st[1], c2 = b[2] + kk * st[2];
+            float acc = 0.f;
+            for (int iz = 0; iz < gz; iz++)
+              for (int iy = 0; iy < gy; iy++) {
+                const CT fz_ = static_cast<CT>(iz), fy_ = static_cast<CT>(iy);
+                const CT r0 = c0 + fy_ * sy[0] + fz_ * sz[0], r1 = c1 + fy_ * sy[1] + fz_ * sz[1], r2 = c2 + fy_ * sy[2] + fz_ * sz[2];
+                for (int ix = 0; ix < gx; ix++) {
+                  const CT fx_ = static_cast<CT>(ix);
+                  acc += staged_sample<T, CT, false, ORDER, kWide>(base, r0 + fx_ * sx[0], r1 + fx_ * sx[1], r2 + fx_ * sx[2],
+                                                                   lim, pitch, slice, pitch_f, slice_f, dy, dz);
+                }
+              }
+            o[k] = acc * inv_count;
+          }
+        };
+        if (mode == 2) {   // the box does not fit in LDS: taps straight from the feature map
+          for (int a = 0; a < 3; a++) b[a] += static_cast<CT>(plan_scalar(&rec->lo[a]));
+          const T *src = reinterpret_cast<const T *>(
+              reinterpret_cast<const char *>(feat) +
+              ((static_cast<unsigned long>(static_cast<unsigned>(plan_scalar(reinterpret_cast<const int *>(&rec->vol_hi)))) << 32) |
+               static_cast<unsigned>(plan_scalar(reinterpret_cast<const int *>(&rec->vol_lo)))));
+          const long hw = static_cast<long>(H) * W;
+          bins(std::true_type{}, src, W, hw, H > 1 ? W : 0, p.D > 1 ? hw : 0);
+        } else {
+          bins(std::false_type{}, tile, g.x / ES, g.y / ES, g.z / ES, g.w / ES);
+        }
+      } else if (mode == 3 && sizeof(CT) == 4) {
         if constexpr (sizeof(CT) == 4)
           interior_column<T, ORDER, ZPL>(tile, o, b[0], b[1], b[2], st[0], st[1], st[2], g, before);
       } else if (mode == 1 && sizeof(CT) == 4) {
@@ -979,7 +1039,7 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
         }
       }
     }
-    if constexpr (G == 1) {
+    if constexpr (G <= 1) {
       pend_base = reinterpret_cast<const char *>(out) + plan.u64(MV_PLAN_DW(out_lo));
       pend_voff = (lx < t.y && ly < t.z) ? lane_out + static_cast<unsigned>(t.x) : kOutOfRange;
       pend_bytes = out_bytes;
@@ -1254,6 +1314,8 @@ static int launch_resample(const T *feat, const float *rois, T *out, const RoiPr
   ps.cap = LDS_BYTES / sizeof(T);
   ps.threads = THREADS; ps.max_items = KMAX;
   ps.halo_lo = CUBIC ? 1 : 0; ps.halo_hi = CUBIC ? 2 : 1;
+  ps.grids = G == 0 ? 1 : 0;
+  ps.flat_axis = TY == 1 ? 1 : 0;
   {
     // inputs that fit the L2s and are read about once (resampling: no more rois than images)
     const long in_bytes = static_cast<long>(p.N) * p.C * p.D * p.H * p.W * static_cast<long>(sizeof(T));
@@ -1278,7 +1340,16 @@ static int launch_resample(const T *feat, const float *rois, T *out, const RoiPr
     hipLaunchKernelGGL((roi_resample_cubic_kernel<T, TX, TY, TZ, THREADS, LDS_BYTES>), dim3(blocks),
                        dim3(THREADS), 0, s, feat, rois, out, p, ps, static_cast<unsigned>(total),
                        static_cast<unsigned>(work));
-  else if constexpr (G > 1)
+  else if constexpr (G == 0) {
+    if (p.order == 0)
+      hipLaunchKernelGGL((roi_resample_kernel<T, TX, TY, TZ, THREADS, LDS_BYTES, KMAX, 0, 0>), dim3(blocks),
+                         dim3(THREADS), 0, s, feat, rois, out, p, ps, static_cast<unsigned>(total),
+                         static_cast<unsigned>(work));
+    else
+      hipLaunchKernelGGL((roi_resample_kernel<T, TX, TY, TZ, THREADS, LDS_BYTES, KMAX, 1, 0>), dim3(blocks),
+                         dim3(THREADS), 0, s, feat, rois, out, p, ps, static_cast<unsigned>(total),
+                         static_cast<unsigned>(work));
+  } else if constexpr (G > 1)
     hipLaunchKernelGGL((roi_resample_kernel<T, TX, TY, TZ, THREADS, LDS_BYTES, KMAX, 1, G>), dim3(blocks),
                        dim3(THREADS), 0, s, feat, rois, out, p, ps, static_cast<unsigned>(total),
                        static_cast<unsigned>(work));
@@ -1316,44 +1387,27 @@ __global__ __launch_bounds__(256) void roi_bin_mean_kernel(const T *__restrict__
   out[i] = store_cast<T>(sum / static_cast<float>(gz * g * g));
 }
 
-// Volumes, order 1, a sampling grid of 2 or 4 per axis: the tiled kernel works on the finer grid and
-// sums every bin's samples in registers (fp32, whatever the tensors' type), so nothing but the means is
-// written.  `f` is the problem on the finer grid.
-template <int G>
-static int roi_forward_tiled_means(const void *input, const void *rois, void *output, int dtype, const RoiProblem &f,
-                                   hipStream_t s) {
-  const float *r = static_cast<const float *>(rois);
-  switch (dtype) {
-    case MV_F16:
-      return launch_resample<__half, 16, 16, 16, 512, 74 * 1024, 8, false, G>(
-          static_cast<const __half *>(input), r, static_cast<__half *>(output), f, nullptr, nullptr, s);
-    case MV_BF16:
-      return launch_resample<__hip_bfloat16, 16, 16, 16, 512, 74 * 1024, 8, false, G>(
-          static_cast<const __hip_bfloat16 *>(input), r, static_cast<__hip_bfloat16 *>(output), f, nullptr, nullptr, s);
-    case MV_F32:
-      return launch_resample<float, 16, 16, 8, 512, 74 * 1024, 6, false, G>(
-          static_cast<const float *>(input), r, static_cast<float *>(output), f, nullptr, nullptr, s);
-    default:
-      return -1;
-  }
-}
-
 // A fixed sampling grid of 2..4 per axis on a large output: the bins' samples are exactly the voxels
 // of the same roi resampled at grid 1 onto an output g times finer (start + (cell * g + sub + 0.5) *
-// bin / g).  Volumes at order 1 with a grid of 2 or 4 take the means inside the tiled kernel (above).
-// Otherwise the tiled kernel writes that finer volume into the workspace and a second pass takes
-// the means: 16-bit samples are then rounded before the mean is; fp16's two roundings stay within its
-// tolerance, bf16's would not, so bf16 then keeps the general kernel.  (The workspace query does not
-// know the order and answers for the two passes.)
+// bin / g).  Images at order 1 with a grid of 2 or 4 run the tiled kernel on that finer grid and take the
+// means inside it (template argument G).  Order 3, and images with a grid of 3, write the finer volume
+// into the workspace and a second pass takes the means: 16-bit samples are then rounded before the mean
+// is; fp16's two roundings stay within its tolerance, bf16's would not.  Volumes at orders 0 and 1 are
+// not taken here: the kernel that walks the samples of a bin in a loop is as fast or faster for them
+// (config 2, fp16: grid 2 0.111 against 0.130 ms, grid 3 0.314 against 0.524 ms through the two passes,
+// grid 4 0.678 against 0.677 ms), for images it is slower (0.033 / 0.056 / 0.086 against 0.024 / 0.048 /
+// 0.049 ms).  Returns -1 for what it does not take.  (The workspace query does not know the order and
+// answers for the two passes.)
 static int roi_forward_tiled_image(const void *input, const void *rois, void *output, int dtype, const RoiProblem &p,
                                    void *workspace, size_t capacity, size_t *need, hipStream_t s, int pool);
 
 static int roi_forward_tiled_grid(const void *input, const void *rois, void *output, int dtype,
                                   const RoiProblem &p, void *workspace, size_t capacity, size_t *need, hipStream_t s) {
   const int g = p.sampling_ratio, gz = p.ndim == 3 ? g : 1;
-  // the means inside the kernel: grids of 2 and 4 at order 1 (images need their rewritten rois in the workspace)
-  const bool means = (g == 2 || g == 4) && p.R > 0 && (dtype == MV_F16 || dtype == MV_BF16 || dtype == MV_F32);
+  // the means inside the kernel: images, grids of 2 and 4 at order 1 (their rewritten rois are in the workspace)
+  const bool means = p.ndim == 2 && (g == 2 || g == 4) && p.R > 0 && (dtype == MV_F16 || dtype == MV_BF16 || dtype == MV_F32);
   const bool in_kernel = !need && means && p.order == 1;
+  if (!need && p.ndim == 3 && p.order != 3) return -1;   // volumes at orders 0 and 1: the loop over the samples
   if (dtype != MV_F16 && dtype != MV_F32 && !means) return -1;
   if (!need && p.order != 1 && p.order != 3) return -1;
   // Outputs that the grid-1 rule sends here, except those of <= 16 cells per axis (the pooled kernels
@@ -1367,10 +1421,7 @@ static int roi_forward_tiled_grid(const void *input, const void *rois, void *out
   const long fine = cells * gz * g * g;
   // (32-bit byte offsets inside one finer volume, as in the grid-1 rule)
   if (in_kernel && static_cast<long>(f.od) * f.oh * f.ow * 4 < (1L << 31)) {
-    int st;
-    if (p.ndim == 2) st = roi_forward_tiled_image(input, rois, output, dtype, f, workspace, capacity, nullptr, s, g);
-    else st = g == 2 ? roi_forward_tiled_means<2>(input, rois, output, dtype, f, s)
-                     : roi_forward_tiled_means<4>(input, rois, output, dtype, f, s);
+    const int st = roi_forward_tiled_image(input, rois, output, dtype, f, workspace, capacity, nullptr, s, g);
     if (st != -1) return st;
   }
   if (dtype != MV_F16 && dtype != MV_F32) {   // bf16: the means inside the kernel or nothing
@@ -1428,8 +1479,10 @@ __global__ void roi_rows_as_slices_kernel(const float *__restrict__ flat, float 
 static int roi_forward_tiled_image(const void *input, const void *rois, void *output, int dtype, const RoiProblem &p,
                                    void *workspace, size_t capacity, size_t *need, hipStream_t s, int pool) {
   const long vox = static_cast<long>(p.oh) * p.ow;
-  if (p.sampling_ratio != 1 || vox < 4096 || p.ow < 16 || p.R == 0) return -1;
-  if (pool != 1 && ((!need && p.order != 1) || (pool != 2 && pool != 4))) return -1;   // (a size query is not told the order)
+  // pool = 0: `p` is the problem asked for, with any sampling grid, and the kernel walks the samples of a bin
+  if ((pool != 0 && p.sampling_ratio != 1) || vox < 4096 || p.ow < 16 || p.R == 0) return -1;
+  if (pool > 1 && ((!need && p.order != 1) || (pool != 2 && pool != 4))) return -1;   // (a size query is not told the order)
+  if (pool == 0 && !need && p.order == 3) return -1;
   if (vox * 4 >= (1L << 31)) return -1;
   if (dtype != MV_F16 && dtype != MV_BF16 && dtype != MV_F32) return -1;
   // (the workspace query does not know whether the rois are rotated: room for the wider rows)
@@ -1459,6 +1512,23 @@ static int roi_forward_tiled_image(const void *input, const void *rois, void *ou
       default:
         st = launch_resample<float, 64, 1, 64, 512, 74 * 1024, 6, true>(static_cast<const float *>(input), vol_rois,
                                                                          static_cast<float *>(output), v, nullptr, need, s);
+    }
+    if (need && st == MV_OK) *need = bytes;
+    return st;
+  }
+  if (pool == 0) {
+    switch (dtype) {
+      case MV_F16:
+        st = launch_resample<__half, 64, 1, 64, 512, 74 * 1024, 8, false, 0>(static_cast<const __half *>(input), vol_rois,
+                                                                              static_cast<__half *>(output), v, nullptr, need, s);
+        break;
+      case MV_BF16:
+        st = launch_resample<__hip_bfloat16, 64, 1, 64, 512, 74 * 1024, 8, false, 0>(
+            static_cast<const __hip_bfloat16 *>(input), vol_rois, static_cast<__hip_bfloat16 *>(output), v, nullptr, need, s);
+        break;
+      default:
+        st = launch_resample<float, 64, 1, 32, 512, 74 * 1024, 6, false, 0>(static_cast<const float *>(input), vol_rois,
+                                                                             static_cast<float *>(output), v, nullptr, need, s);
     }
     if (need && st == MV_OK) *need = bytes;
     return st;
@@ -1498,14 +1568,35 @@ static int roi_forward_tiled_image(const void *input, const void *rois, void *ou
 // when the path does not apply.
 int roi_forward_tiled(const void *input, const void *rois, void *output, int dtype,
                       const RoiProblem &p, void *workspace, size_t capacity, size_t *need, hipStream_t s) {
-  if (p.sampling_ratio >= 2 && p.sampling_ratio <= 4)
-    return roi_forward_tiled_grid(input, rois, output, dtype, p, workspace, capacity, need, s);
+  if (p.sampling_ratio >= 2 && p.sampling_ratio <= 4) {
+    const int st = roi_forward_tiled_grid(input, rois, output, dtype, p, workspace, capacity, need, s);
+    if (st != -1) return st;
+  }
+  // Every other grid at orders 0 and 1 - volumes with any grid, images with 3 (without a workspace or in
+  // bf16), 5 and more, ceil(roi extent / cells) per roi: the samples of a bin in a loop inside the kernel.
+  const bool any_grid = p.sampling_ratio != 1;
+  if (any_grid && p.order == 3) return -1;
   // images: rows as slices
-  if (p.ndim == 2) return roi_forward_tiled_image(input, rois, output, dtype, p, workspace, capacity, need, s, 1);
+  if (p.ndim == 2) return roi_forward_tiled_image(input, rois, output, dtype, p, workspace, capacity, need, s, any_grid ? 0 : 1);
   const long vox = static_cast<long>(p.od) * p.oh * p.ow;
-  if (p.sampling_ratio != 1 || vox < 4096 || p.ow < 16 || p.R == 0) return -1;
+  if (vox < 4096 || p.ow < 16 || p.R == 0) return -1;
   if (vox * 4 >= (1L << 31)) return -1;   // 32-bit byte offsets inside one output volume
   const float *r = static_cast<const float *>(rois);
+  if (any_grid) {
+    switch (dtype) {
+      case MV_F16:
+        return launch_resample<__half, 16, 16, 16, 512, 74 * 1024, 8, false, 0>(
+            static_cast<const __half *>(input), r, static_cast<__half *>(output), p, workspace, need, s);
+      case MV_BF16:
+        return launch_resample<__hip_bfloat16, 16, 16, 16, 512, 74 * 1024, 8, false, 0>(
+            static_cast<const __hip_bfloat16 *>(input), r, static_cast<__hip_bfloat16 *>(output), p, workspace, need, s);
+      case MV_F32:
+        return launch_resample<float, 16, 16, 8, 512, 74 * 1024, 6, false, 0>(
+            static_cast<const float *>(input), r, static_cast<float *>(output), p, workspace, need, s);
+      default:
+        return -1;
+    }
+  }
   if (p.order == 3) {
     // A source of a few hundred voxels per channel (the control grid of the elastic deformation) needs
     // no 74 KB tile: the instance with a small one keeps twice as many workgroups per compute unit busy.
@@ -1920,6 +2011,7 @@ int roi_backward_tiled(const void *grad_output, const void *rois, void *acc, int
   ps.cap = kScatterLds / 4;
   ps.threads = kScatterThreads; ps.max_items = 0;
   ps.halo_lo = 0; ps.halo_hi = 1;
+  ps.grids = 0; ps.flat_axis = 0;
   ps.warm_groups = 0;
   ps.pad_slices = 0;
   ps.es = 4;

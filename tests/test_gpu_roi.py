@@ -422,12 +422,12 @@ def test_cubic_affine_vs_oracle(ops, oracle, dtype, ndim, sr):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("sr", [2, 3, 4])
 def test_large_outputs_with_a_sampling_grid(ops, oracle, dtype, sr):
-    """sampling_ratio 2..4 on outputs of resampling size: the tiled kernel works on the sr times finer
-    grid of the bins' samples.  Order 1 with a grid of 2 or 4 (volumes and images, any of the three
-    types) takes the means of the bins inside that kernel; a grid of 3 and order 3 write the finer volume
-    and a second pass takes the means (fp16 / fp32; bf16 then stays on the general kernel).  Rotated
-    and plain rois in 3-D and 2-D, order 1, and order 3 through the affine engine; a second output
-    shape whose finer grid ends inside a tile on every axis."""
+    """sampling_ratio 2..4 on outputs of resampling size.  Volumes at orders 0 / 1: the tiled kernel walks
+    the samples of a bin in a loop (any of the three types).  Images at order 1 with a grid of 2 or 4: the
+    kernel works on the sr times finer grid of the bins' samples and takes the means inside; a grid of 3
+    and order 3 write the finer volume and a second pass takes the means (fp16 / fp32).  Rotated and
+    plain rois in 3-D and 2-D, order 1, and order 3 through the affine engine; a second output shape
+    whose tiles are cut on every axis."""
     g = wl.gen(700 + sr)
     feat = torch.randn(2, 2, 24, 40, 48, generator=g).to(dtype)
     out = (20, 24, 32) if sr < 4 else (10, 24, 32)
