@@ -1650,7 +1650,7 @@ int roi_forward_tiled(const void *input, const void *rois, void *output, int dty
 }
 
 // ---------------------------------------------------------------------------------------------
-// Backward of the same problems (grid 1, orders 0 and 1).  The forward's plan is used in reverse: an
+// Backward of the same problems (any sampling grid, orders 0 and 1).  The forward's plan is used in reverse: an
 // item is (output tile, channel), its source box becomes an LDS tile of 32-bit FIXED-POINT sums, every
 // output voxel of the tile adds weight * grad_output to the <= 8 voxels its sample touches, and the
 // tile's non-zero sums go to the fp32 gradient buffer as one atomic per voxel, contiguous along x
@@ -1723,6 +1723,11 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
     const int n0 = plan_scalar(&r.n[0]), n1 = plan_scalar(&r.n[1]), n2 = plan_scalar(&r.n[2]);
     const int l0 = plan_scalar(&r.lo[0]), l1 = plan_scalar(&r.lo[1]), l2 = plan_scalar(&r.lo[2]);
     const int t0x = plan_scalar(&r.t0[0]), t0y = plan_scalar(&r.t0[1]), t0z = plan_scalar(&r.t0[2]);
+    // samples per bin (the fixed ratio, or ceil(roi extent / cells) of this roi); every sample carries
+    // grad_output / count
+    const int gx = plan_scalar(&r.grid[0]), gy = plan_scalar(&r.grid[1]), gz = plan_scalar(&r.grid[2]);
+    const int count = gx * gy * gz;
+    const float inv_count = 1.f / static_cast<float>(count);
     double map[12];
 #pragma unroll
     for (int i = 0; i < 12; i++) map[i] = uniform(r.map[i]);
@@ -1739,7 +1744,7 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
       const int c = threadIdx.x + k * kScatterThreads;
       const int ox = t0x + c % TX, oy = t0y + (c / TX) % TY, oz = t0z + c / (TX * TY);
       const bool in = ox < p.ow && oy < p.oh && oz < p.od;
-      gv[k] = in ? static_cast<float>(load(gsrc + (static_cast<long>(oz) * p.oh + oy) * p.ow + ox)) : 0.f;
+      gv[k] = in ? static_cast<float>(load(gsrc + (static_cast<long>(oz) * p.oh + oy) * p.ow + ox)) * inv_count : 0.f;
       bits = max(bits, __float_as_uint(fabsf(gv[k])));
     }
 #pragma unroll
@@ -1753,19 +1758,23 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
     turn ^= 1;
     bits = __builtin_amdgcn_readfirstlane(bits);
     if (bits == 0) continue;                                  // nothing to add
-    const bool in_lds = bits < 0x7f800000u && mode != 2;      // finite terms, box within the tile
-    // Quanta per unit: a voxel gets at most one term from each output voxel whose sample lies within
-    // one voxel of it on every axis, i.e. inside a ball of radius sqrt(3); along output axis j (bin
-    // b_j = length of column j of the map) that leaves floor(2 sqrt(3) / b_j) + 1 indices.
+    // Quanta per unit: a voxel gets at most one term from each sample that lies within one voxel of it
+    // on every axis, i.e. inside a ball of radius sqrt(3); along output axis j (samples b_j / g_j apart,
+    // b_j = length of column j of the map) that leaves floor(2 sqrt(3) g_j / b_j) + 1 of them.
     int terms = 1;
 #pragma unroll
     for (int j = 0; j < 3; j++) {
       const float c0 = static_cast<float>(map[1 + j]), c1 = static_cast<float>(map[5 + j]), c2 = static_cast<float>(map[9 + j]);
       const float bj = sqrtf(c0 * c0 + c1 * c1 + c2 * c2);
-      const int ext = j == 0 ? TX : (j == 1 ? TY : TZ);
-      terms *= static_cast<int>(fminf(3.4642f / bj * 1.00001f + 1.f, static_cast<float>(ext)));
+      const int ext = j == 0 ? TX : (j == 1 ? TY : TZ), gj = j == 0 ? gx : (j == 1 ? gy : gz);
+      terms *= static_cast<int>(fminf(3.4642f * static_cast<float>(gj) / bj * 1.00001f + 1.f, static_cast<float>(ext * gj)));
     }
-    const int term_bits = 30 - (32 - __clz(terms - 1));   // 30 - ceil(log2 terms) >= kTermBits
+    const int term_bits = 30 - (32 - __clz(terms - 1));   // 30 - ceil(log2 terms); >= kTermBits at one sample per bin
+    // finite terms, box within the tile, enough bits per term: 18 for fp32 tensors (a term is rounded to
+    // 2^-19 of the largest; with more samples per voxel than that leaves room for they go out one by one as
+    // fp32 atomics), 8 for 16-bit ones (a voxel that many terms reach holds a sum that large, and single
+    // terms would be rounded to the tensor's type one by one on the direct path)
+    const bool in_lds = bits < 0x7f800000u && mode != 2 && terms <= (sizeof(T) == 2 ? (1 << 22) : (1 << 12));
     const int ex = min(max(127 + 126 + term_bits - static_cast<int>(bits >> 23), 1), 253);   // 2^(ex - 127) = 2^term_bits / 2^e
     const float to_quanta = __uint_as_float(static_cast<unsigned>(ex) << 23);
     const float from_quanta = __uint_as_float(static_cast<unsigned>(254 - ex) << 23);
@@ -1775,8 +1784,11 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
     // kernel's rules (clipped boxes: the coordinate clamps to [0, cmax], a sample the clamp moves by
     // more than 1 is void, the low tap is at most top = max(n - 2, 0)); the box's margin covers their
     // rounding.
-    auto scatter_cells32 = [&](auto interior_tag) {
+    auto scatter_cells32 = [&](auto interior_tag, auto grids_tag) {
     constexpr bool kInterior = decltype(interior_tag)::value;
+    constexpr bool kGrids = decltype(grids_tag)::value;
+    const int sgx = kGrids ? gx : 1, sgy = kGrids ? gy : 1, sgz = kGrids ? gz : 1;
+    const float igx = 1.f / static_cast<float>(gx), igy = 1.f / static_cast<float>(gy), igz = 1.f / static_cast<float>(gz);
     float mf[12], cmax[3], top[3];
 #pragma unroll
     for (int i = 0; i < 12; i++) mf[i] = uniform(r.mapf[i]);
@@ -1789,10 +1801,17 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
       const float x = static_cast<float>(c % TX), y = static_cast<float>((c / TX) % TY), z = static_cast<float>(c / (TX * TY));
       const float g = gv[k];
       if (g == 0.f) continue;
+      float v0[3];
+#pragma unroll
+      for (int a = 0; a < 3; a++) v0[a] = fmaf(mf[4 * a + 3], z, fmaf(mf[4 * a + 2], y, fmaf(mf[4 * a + 1], x, mf[4 * a])));
+      for (int iz = 0; iz < sgz; iz++)
+      for (int iy = 0; iy < sgy; iy++)
+      for (int ix = 0; ix < sgx; ix++) {
       float v[3], f[3];
       int b0[3];
 #pragma unroll
-      for (int a = 0; a < 3; a++) v[a] = fmaf(mf[4 * a + 3], z, fmaf(mf[4 * a + 2], y, fmaf(mf[4 * a + 1], x, mf[4 * a])));
+      for (int a = 0; a < 3; a++)
+        v[a] = kGrids ? fmaf(mf[4 * a + 3] * igz, static_cast<float>(iz), fmaf(mf[4 * a + 2] * igy, static_cast<float>(iy), fmaf(mf[4 * a + 1] * igx, static_cast<float>(ix), v0[a]))) : v0[a];
       if constexpr (kInterior) {
 #pragma unroll
         for (int a = 0; a < 3; a++) {
@@ -1838,20 +1857,28 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
             atomic_add_element(vol, (zi * p.H + yi) * p.W + xi, g * w);
         }
       }
+      }   // samples of the bin
     }
     };
-    auto scatter_cells = [&](auto interior_tag, auto order_tag) {
+    auto scatter_cells = [&](auto interior_tag, auto order_tag, auto grids_tag) {
     constexpr bool kInterior = decltype(interior_tag)::value;
     constexpr int kOrder = decltype(order_tag)::value;
+    constexpr bool kGrids = decltype(grids_tag)::value;
+    const int sgx = kGrids ? gx : 1, sgy = kGrids ? gy : 1, sgz = kGrids ? gz : 1;
+    const double dgx = 1.0 / gx, dgy = 1.0 / gy, dgz = 1.0 / gz;
 #pragma unroll
     for (int k = 0; k < kPerThread; k++) {
       const int c = threadIdx.x + k * kScatterThreads;
       const int x = c % TX, y = (c / TX) % TY, z = c / (TX * TY);
       const float g = gv[k];
       if (g == 0.f) continue;
-      const double vx = map[0] + map[1] * x + map[2] * y + map[3] * z;
-      const double vy = map[4] + map[5] * x + map[6] * y + map[7] * z;
-      const double vz = map[8] + map[9] * x + map[10] * y + map[11] * z;
+      for (int iz = 0; iz < sgz; iz++)
+      for (int iy = 0; iy < sgy; iy++)
+      for (int ix = 0; ix < sgx; ix++) {
+      const double sx_ = kGrids ? x + ix * dgx : x, sy_ = kGrids ? y + iy * dgy : y, sz_ = kGrids ? z + iz * dgz : z;
+      const double vx = map[0] + map[1] * sx_ + map[2] * sy_ + map[3] * sz_;
+      const double vy = map[4] + map[5] * sx_ + map[6] * sy_ + map[7] * sz_;
+      const double vz = map[8] + map[9] * sx_ + map[10] * sy_ + map[11] * sz_;
       int xi[2], yi[2], zi[2];
       float fx, fy, fz;
       if constexpr (kInterior) {
@@ -1893,19 +1920,24 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
             atomic_add_element(vol, (static_cast<long>(zi[n >> 2]) * p.H + yi[(n >> 1) & 1]) * p.W + xi[n & 1], g * w);
         }
       }
+      }   // samples of the bin
     }
     };
     using Yes = std::true_type;
     using No = std::false_type;
-    if (sizeof(T) == 2 && p.order == 1 && in_lds) {
-      if (mode == 3 && p.ndim == 3) scatter_cells32(Yes{});
-      else scatter_cells32(No{});
+    if (count > 1) {   // (one copy of the loops for grids: the clamped form covers unclipped boxes too)
+      if (sizeof(T) == 2 && p.order == 1 && in_lds) scatter_cells32(No{}, Yes{});
+      else if (p.order == 0) scatter_cells(No{}, std::integral_constant<int, 0>{}, Yes{});
+      else scatter_cells(No{}, std::integral_constant<int, 1>{}, Yes{});
+    } else if (sizeof(T) == 2 && p.order == 1 && in_lds) {
+      if (mode == 3 && p.ndim == 3) scatter_cells32(Yes{}, No{});
+      else scatter_cells32(No{}, No{});
     } else if (mode == 3 && p.ndim == 3) {
-      if (p.order == 0) scatter_cells(Yes{}, std::integral_constant<int, 0>{});
-      else scatter_cells(Yes{}, std::integral_constant<int, 1>{});
+      if (p.order == 0) scatter_cells(Yes{}, std::integral_constant<int, 0>{}, No{});
+      else scatter_cells(Yes{}, std::integral_constant<int, 1>{}, No{});
     } else {
-      if (p.order == 0) scatter_cells(No{}, std::integral_constant<int, 0>{});
-      else scatter_cells(No{}, std::integral_constant<int, 1>{});
+      if (p.order == 0) scatter_cells(No{}, std::integral_constant<int, 0>{}, No{});
+      else scatter_cells(No{}, std::integral_constant<int, 1>{}, No{});
     }
     if (in_lds) {
       __syncthreads();
@@ -1982,7 +2014,7 @@ static ScatterTiling scatter_tiling(const RoiProblem &p) {
 
 bool roi_backward_tiled_applies(int dtype, const RoiProblem &p) {
   const long vox = static_cast<long>(p.od) * p.oh * p.ow;
-  if (p.sampling_ratio != 1 || (p.order != 0 && p.order != 1) || vox < 4096 || p.ow < 16 || p.R == 0) return false;
+  if ((p.order != 0 && p.order != 1) || vox < 4096 || p.ow < 16 || p.R == 0) return false;
   if (dtype != MV_F16 && dtype != MV_BF16 && dtype != MV_F32) return false;
   return scatter_tiling(p).work < (1L << 31) && static_cast<long>(p.D) * p.H * p.W * 4 < (1L << 31);
 }
@@ -2011,7 +2043,7 @@ int roi_backward_tiled(const void *grad_output, const void *rois, void *acc, int
   ps.cap = kScatterLds / 4;
   ps.threads = kScatterThreads; ps.max_items = 0;
   ps.halo_lo = 0; ps.halo_hi = 1;
-  ps.grids = 0; ps.flat_axis = 0;
+  ps.grids = 1; ps.flat_axis = 0;
   ps.warm_groups = 0;
   ps.pad_slices = 0;
   ps.es = 4;
