@@ -41,7 +41,7 @@ int mv_version(void);
  * backward ACCUMULATES into grad_input (callers pass a zero-filled buffer, like the reference's
  * Python wrapper ops/roi_align_nd.py:139 does).  For MV_F16 / MV_BF16 the backward needs an fp32
  * workspace of mv_roi_align_backward_workspace_bytes(); other dtypes accept NULL.  (fp16 outputs of
- * resampling size whose gradient rows hold an even number of voxels leave it untouched: the sums of
+ * resampling size whose gradient rows hold an even number of voxels, at sampling ratios 1..3, leave it untouched: the sums of
  * their tiles go to grad_input as packed fp16 atomics, rounded once per tile that reaches a voxel.) */
 int mv_roi_align_2d_forward(const void *input, const void *rois, void *output, int dtype,
                             int batch, int channels, int height, int width, int num_rois,

@@ -1770,11 +1770,10 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
       terms *= static_cast<int>(fminf(3.4642f * static_cast<float>(gj) / bj * 1.00001f + 1.f, static_cast<float>(ext * gj)));
     }
     const int term_bits = 30 - (32 - __clz(terms - 1));   // 30 - ceil(log2 terms); >= kTermBits at one sample per bin
-    // finite terms, box within the tile, enough bits per term: 18 for fp32 tensors (a term is rounded to
-    // 2^-19 of the largest; with more samples per voxel than that leaves room for they go out one by one as
-    // fp32 atomics), 8 for 16-bit ones (a voxel that many terms reach holds a sum that large, and single
-    // terms would be rounded to the tensor's type one by one on the direct path)
-    const bool in_lds = bits < 0x7f800000u && mode != 2 && terms <= (sizeof(T) == 2 ? (1 << 22) : (1 << 12));
+    // finite terms, box within the tile, enough bits per term: 18 for fp32 tensors, 12 for 16-bit ones (a
+    // term is rounded to 2^-19 / 2^-13 of the largest; grids of many samples over small bins leave less,
+    // and their terms go out one by one as fp32 atomics - the direct fp16 path is not taken for such grids)
+    const bool in_lds = bits < 0x7f800000u && mode != 2 && terms <= (sizeof(T) == 2 ? (1 << 18) : (1 << 12));
     const int ex = min(max(127 + 126 + term_bits - static_cast<int>(bits >> 23), 1), 253);   // 2^(ex - 127) = 2^term_bits / 2^e
     const float to_quanta = __uint_as_float(static_cast<unsigned>(ex) << 23);
     const float from_quanta = __uint_as_float(static_cast<unsigned>(254 - ex) << 23);
@@ -2022,8 +2021,10 @@ bool roi_backward_tiled_applies(int dtype, const RoiProblem &p) {
 // fp16 gradients whose rows hold an even number of voxels need no fp32 buffer: the tiles' sums go
 // straight into the gradient tensor as packed atomics on pairs of voxels.
 bool roi_backward_tiled_direct(int dtype, const RoiProblem &p, const void *grad_input) {
+  // (grids of up to 3 per axis: a tile's voxel then gets at most 48 x 48 x 24 terms, which its 32-bit sums
+  // hold at 14 bits each; larger and adaptive grids may need single terms, which want the fp32 buffer)
   return dtype == MV_F16 && p.W % 2 == 0 && reinterpret_cast<uintptr_t>(grad_input) % 4 == 0 &&
-         roi_backward_tiled_applies(dtype, p);
+         p.sampling_ratio >= 1 && p.sampling_ratio <= 3 && roi_backward_tiled_applies(dtype, p);
 }
 
 // `acc`: fp32 gradient buffer [N, C, D, H, W] that the terms are added to, or (`direct`, see above) the

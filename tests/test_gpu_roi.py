@@ -200,6 +200,41 @@ def test_backward_through_source_box_tiles(ops, oracle, dtype, order):
     check((1, 2, 48, 96, 128), big, (16, 20, 24), True, "boxes beyond the tile")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("sr", [2, 3, 0, 6])
+def test_backward_tiles_with_sampling_grids(ops, oracle, dtype, sr):
+    """Backward of resampling-sized outputs with a sampling grid: fixed ratios, the adaptive grid
+    ceil(roi extent / cells) per roi (rois of different extents on one call), and a ratio whose many
+    samples over small bins leave too few bits per term for fp32 tensors (those tiles add term by term).
+    Rotated and plain rois, volumes and images, forward checked along the way."""
+    g = wl.gen(830 + max(sr, 0))
+
+    def check(feat_shape, rois, out, rotated, what):
+        feat = torch.randn(feat_shape, generator=g).to(dtype)
+        x = feat.to(DEV).requires_grad_(True)
+        mod = (ops.RoIAlignRotated if rotated else ops.RoIAlign)(out, 1.0, sr)
+        y = mod(x, rois.to(DEV))
+        # cells with a sample within coordinate rounding of the edge of [-1, size] prove nothing
+        margin = oracle.roi_decision_margin(feat_shape, rois, out, 1.0, sr, True, rotated)
+        keep = (margin > NEAREST_EPS[dtype])[:, None]
+        want = oracle.roi_align_forward(feat, rois, out, 1.0, sr, True, 1, rotated)
+        assert_close(y.detach().cpu() * keep, want * keep, FWD_TOL[dtype], what + ", forward")
+        gy = (torch.randn(y.shape, generator=g) * keep).to(dtype)
+        y.backward(gy.to(DEV))
+        gwant = oracle.roi_align_backward(gy, rois, feat_shape, 1.0, sr, True, 1, rotated)
+        assert float(gwant.abs().max()) > 0
+        assert_close(x.grad, gwant, BWD_TOL[dtype], what + ", backward")
+
+    rois = wl.affine_rois(g, 2, (48, 40, 24))
+    rois[1, 4:7] *= 2.2                               # a roi that wants more samples per bin than the other
+    check((2, 2, 24, 40, 48), rois, (18, 22, 36), True, "rotated volumes")
+    boxes = torch.tensor([[0, 2.3, 1.2, 0.5, 40.1, 33.3, 20.7], [1, -3.0, 5.0, 2.0, 30.0, 45.0, 30.0],
+                          [1, 10.0, 3.0, 4.0, 14.0, 9.0, 8.0]])       # the last one: bins far below a voxel
+    check((2, 2, 24, 40, 48), boxes, (18, 24, 32), False, "plain volumes")
+    r2 = torch.tensor([[0, 45.0, 35.0, 80.0, 60.0, 0.4], [1, 40.0, 30.0, 160.0, 110.0, -1.2]])
+    check((2, 3, 70, 90), r2, (72, 80), True, "rotated images")
+
+
 def test_backward_tiles_with_zero_and_infinite_gradients(ops, oracle):
     """A grad_output of zeros leaves the gradient untouched; an infinity reaches the voxels the oracle
     sends it to (the tile that holds it adds its terms one by one, the others stay in fixed point)."""
