@@ -1688,7 +1688,9 @@ __device__ __forceinline__ void atomic_add_element(float *base, long i, float v)
 
 // DIRECT (fp16 only; rows of an even number of voxels, a 4-byte aligned tensor): `acc` is the gradient
 // tensor itself, otherwise an fp32 buffer of its shape.
-template <typename T, int TX, int TY, int TZ, bool DIRECT = false>
+// GRIDS: the instance for sampling ratios other than 1 (a lane walks the samples of its bins); the one
+// for ratio 1 is compiled without that code (it has no scalar registers to spare).
+template <typename T, int TX, int TY, int TZ, bool DIRECT = false, bool GRIDS = false>
 __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward_tiles_kernel(
     const T *__restrict__ gout, const float *__restrict__ rois, void *__restrict__ acc, const RoiProblem p,
     const PlanShape ps, const unsigned total, const unsigned work) {
@@ -1725,9 +1727,8 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
     const int t0x = plan_scalar(&r.t0[0]), t0y = plan_scalar(&r.t0[1]), t0z = plan_scalar(&r.t0[2]);
     // samples per bin (the fixed ratio, or ceil(roi extent / cells) of this roi); every sample carries
     // grad_output / count
-    const int gx = plan_scalar(&r.grid[0]), gy = plan_scalar(&r.grid[1]), gz = plan_scalar(&r.grid[2]);
-    const int count = gx * gy * gz;
-    const float inv_count = 1.f / static_cast<float>(count);
+    const int count = GRIDS ? plan_scalar(&r.grid[0]) * plan_scalar(&r.grid[1]) * plan_scalar(&r.grid[2]) : 1;
+    const float inv_count = GRIDS ? 1.f / static_cast<float>(count) : 1.f;
     double map[12];
 #pragma unroll
     for (int i = 0; i < 12; i++) map[i] = uniform(r.map[i]);
@@ -1766,7 +1767,7 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
     for (int j = 0; j < 3; j++) {
       const float c0 = static_cast<float>(map[1 + j]), c1 = static_cast<float>(map[5 + j]), c2 = static_cast<float>(map[9 + j]);
       const float bj = sqrtf(c0 * c0 + c1 * c1 + c2 * c2);
-      const int ext = j == 0 ? TX : (j == 1 ? TY : TZ), gj = j == 0 ? gx : (j == 1 ? gy : gz);
+      const int ext = j == 0 ? TX : (j == 1 ? TY : TZ), gj = GRIDS ? plan_scalar(&r.grid[j]) : 1;
       terms *= static_cast<int>(fminf(3.4642f * static_cast<float>(gj) / bj * 1.00001f + 1.f, static_cast<float>(ext * gj)));
     }
     const int term_bits = 30 - (32 - __clz(terms - 1));   // 30 - ceil(log2 terms); >= kTermBits at one sample per bin
@@ -1786,8 +1787,9 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
     auto scatter_cells32 = [&](auto interior_tag, auto grids_tag) {
     constexpr bool kInterior = decltype(interior_tag)::value;
     constexpr bool kGrids = decltype(grids_tag)::value;
-    const int sgx = kGrids ? gx : 1, sgy = kGrids ? gy : 1, sgz = kGrids ? gz : 1;
-    const float igx = 1.f / static_cast<float>(gx), igy = 1.f / static_cast<float>(gy), igz = 1.f / static_cast<float>(gz);
+    // (the grid is read here, not kept from above: the copy without grids has no scalar registers to spare)
+    const int sgx = kGrids ? plan_scalar(&r.grid[0]) : 1, sgy = kGrids ? plan_scalar(&r.grid[1]) : 1, sgz = kGrids ? plan_scalar(&r.grid[2]) : 1;
+    const float igx = 1.f / static_cast<float>(sgx), igy = 1.f / static_cast<float>(sgy), igz = 1.f / static_cast<float>(sgz);
     float mf[12], cmax[3], top[3];
 #pragma unroll
     for (int i = 0; i < 12; i++) mf[i] = uniform(r.mapf[i]);
@@ -1863,8 +1865,8 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
     constexpr bool kInterior = decltype(interior_tag)::value;
     constexpr int kOrder = decltype(order_tag)::value;
     constexpr bool kGrids = decltype(grids_tag)::value;
-    const int sgx = kGrids ? gx : 1, sgy = kGrids ? gy : 1, sgz = kGrids ? gz : 1;
-    const double dgx = 1.0 / gx, dgy = 1.0 / gy, dgz = 1.0 / gz;
+    const int sgx = kGrids ? plan_scalar(&r.grid[0]) : 1, sgy = kGrids ? plan_scalar(&r.grid[1]) : 1, sgz = kGrids ? plan_scalar(&r.grid[2]) : 1;
+    const double dgx = 1.0 / sgx, dgy = 1.0 / sgy, dgz = 1.0 / sgz;
 #pragma unroll
     for (int k = 0; k < kPerThread; k++) {
       const int c = threadIdx.x + k * kScatterThreads;
@@ -1924,7 +1926,7 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
     };
     using Yes = std::true_type;
     using No = std::false_type;
-    if (count > 1) {   // (one copy of the loops for grids: the clamped form covers unclipped boxes too)
+    if constexpr (GRIDS) {   // (one copy of the loops for grids: the clamped form covers unclipped boxes too)
       if (sizeof(T) == 2 && p.order == 1 && in_lds) scatter_cells32(No{}, Yes{});
       else if (p.order == 0) scatter_cells(No{}, std::integral_constant<int, 0>{}, Yes{});
       else scatter_cells(No{}, std::integral_constant<int, 1>{}, Yes{});
@@ -2055,33 +2057,34 @@ int roi_backward_tiled(const void *grad_output, const void *rois, void *acc, int
   ps.by_slots.set(1);
   long blocks = std::min<long>(work, static_cast<long>(kScatterWgs) * compute_units());
   blocks = std::max(blocks, (work + kPlanSlots - 1) / kPlanSlots);
+  const bool grids = p.sampling_ratio != 1;
+#define MV_SCATTER_LAUNCH(TYPE, DIRECTV, GRIDSV)                                                                       \
+  do {                                                                                                                \
+    if (flat)                                                                                                         \
+      hipLaunchKernelGGL((roi_backward_tiles_kernel<TYPE, MV_SCATTER_SHAPE_2D, DIRECTV, GRIDSV>),                    \
+                         dim3(static_cast<unsigned>(blocks)), dim3(kScatterThreads), 0, s,                            \
+                         static_cast<const TYPE *>(grad_output), static_cast<const float *>(rois), acc, p, ps,        \
+                         static_cast<unsigned>(total), static_cast<unsigned>(work));                                  \
+    else                                                                                                              \
+      hipLaunchKernelGGL((roi_backward_tiles_kernel<TYPE, MV_SCATTER_SHAPE, DIRECTV, GRIDSV>),                       \
+                         dim3(static_cast<unsigned>(blocks)), dim3(kScatterThreads), 0, s,                            \
+                         static_cast<const TYPE *>(grad_output), static_cast<const float *>(rois), acc, p, ps,        \
+                         static_cast<unsigned>(total), static_cast<unsigned>(work));                                  \
+  } while (0)
   if (direct) {
-    if (flat)
-      hipLaunchKernelGGL((roi_backward_tiles_kernel<__half, MV_SCATTER_SHAPE_2D, true>), dim3(static_cast<unsigned>(blocks)),
-                         dim3(kScatterThreads), 0, s, static_cast<const __half *>(grad_output),
-                         static_cast<const float *>(rois), acc, p, ps, static_cast<unsigned>(total),
-                         static_cast<unsigned>(work));
-    else
-      hipLaunchKernelGGL((roi_backward_tiles_kernel<__half, MV_SCATTER_SHAPE, true>), dim3(static_cast<unsigned>(blocks)),
-                         dim3(kScatterThreads), 0, s, static_cast<const __half *>(grad_output),
-                         static_cast<const float *>(rois), acc, p, ps, static_cast<unsigned>(total),
-                         static_cast<unsigned>(work));
-    return check_launch("roi_backward_tiles_kernel");
+    if (grids) MV_SCATTER_LAUNCH(__half, true, true);
+    else MV_SCATTER_LAUNCH(__half, true, false);
+  } else if (dtype == MV_F16) {
+    if (grids) MV_SCATTER_LAUNCH(__half, false, true);
+    else MV_SCATTER_LAUNCH(__half, false, false);
+  } else if (dtype == MV_BF16) {
+    if (grids) MV_SCATTER_LAUNCH(__hip_bfloat16, false, true);
+    else MV_SCATTER_LAUNCH(__hip_bfloat16, false, false);
+  } else {
+    if (grids) MV_SCATTER_LAUNCH(float, false, true);
+    else MV_SCATTER_LAUNCH(float, false, false);
   }
-  MV_DISPATCH(dtype, {
-    if constexpr (sizeof(T) <= 4) {
-      if (flat)
-        hipLaunchKernelGGL((roi_backward_tiles_kernel<T, MV_SCATTER_SHAPE_2D>), dim3(static_cast<unsigned>(blocks)),
-                           dim3(kScatterThreads), 0, s, static_cast<const T *>(grad_output),
-                           static_cast<const float *>(rois), acc, p, ps, static_cast<unsigned>(total),
-                           static_cast<unsigned>(work));
-      else
-        hipLaunchKernelGGL((roi_backward_tiles_kernel<T, MV_SCATTER_SHAPE>), dim3(static_cast<unsigned>(blocks)),
-                           dim3(kScatterThreads), 0, s, static_cast<const T *>(grad_output),
-                           static_cast<const float *>(rois), acc, p, ps, static_cast<unsigned>(total),
-                           static_cast<unsigned>(work));
-    }
-  });
+#undef MV_SCATTER_LAUNCH
   return check_launch("roi_backward_tiles_kernel");
 }
 
