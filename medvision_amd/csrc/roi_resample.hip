@@ -958,7 +958,7 @@ __global__ __launch_bounds__(THREADS, 4) void roi_resample_kernel(
         CT sx[3], sy[3], sz[3];
 #pragma unroll
         for (int a = 0; a < 3; a++) { sx[a] = m[4 * a + 1] * igx; sy[a] = m[4 * a + 2] * igy; sz[a] = m[4 * a + 3] * igz; }
-        const float inv_count = 1.f / static_cast<float>(gx * gy * gz);
+        const float inv_count = 1.f / (static_cast<float>(gx) * static_cast<float>(gy) * static_cast<float>(gz));
         const int size[3] = {W, H, p.D};
         BoxLimits<CT> lim;
 #pragma unroll
@@ -1727,8 +1727,9 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
     const int t0x = plan_scalar(&r.t0[0]), t0y = plan_scalar(&r.t0[1]), t0z = plan_scalar(&r.t0[2]);
     // samples per bin (the fixed ratio, or ceil(roi extent / cells) of this roi); every sample carries
     // grad_output / count
-    const int count = GRIDS ? plan_scalar(&r.grid[0]) * plan_scalar(&r.grid[1]) * plan_scalar(&r.grid[2]) : 1;
-    const float inv_count = GRIDS ? 1.f / static_cast<float>(count) : 1.f;
+    const float inv_count = GRIDS ? 1.f / (static_cast<float>(plan_scalar(&r.grid[0])) * static_cast<float>(plan_scalar(&r.grid[1])) *
+                                          static_cast<float>(plan_scalar(&r.grid[2])))
+                                  : 1.f;
     double map[12];
 #pragma unroll
     for (int i = 0; i < 12; i++) map[i] = uniform(r.map[i]);
