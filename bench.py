@@ -160,6 +160,10 @@ def bench_other_configs(args):
         vol = torch.randn(4, 1, 128, 128, 128, generator=g).to(dt).to(dev)
         ms, _ = _events_ms(lambda i: ops.affine_3d(vol, r, (128, 128, 128), 1.0, 2, True, 1), 50, 5)
         res["config2_sampling_ratio_2_" + name] = {"ms": round(ms, 4), "gsamples_s": round(8 * vol.numel() / ms / 1e6, 1)}
+        gy = torch.randn(4, 1, 128, 128, 128, generator=g).to(dt).to(dev)
+        gi = torch.zeros_like(vol)
+        bms, _ = _events_ms(lambda i: _C.roi_align_rotated_3d_backward(gy, r, gi, 128, 128, 128, 1.0, 2, True, 1), 30, 3)
+        res["config2_sampling_ratio_2_" + name]["backward_ms"] = round(bms, 4)
     g = wl.gen(2)
     vol = wl.ct_like(g, (2, 1, 256, 512, 512)).to(dev)
     full = torch.tensor([[b, 256, 256, 128, 512, 512, 256, 0, 0, 0] for b in range(2)], dtype=torch.float32).to(dev)
