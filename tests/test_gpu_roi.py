@@ -235,6 +235,25 @@ def test_backward_tiles_with_sampling_grids(ops, oracle, dtype, sr):
     check((2, 3, 70, 90), r2, (72, 80), True, "rotated images")
 
 
+def test_backward_tiles_precision_over_a_wide_range_of_gradients(ops, oracle):
+    """fp32 tensors: a tile's terms are rounded to 2^-(t+1) of the tile's largest gradient, t >= 19 at one
+    sample per bin (32-bit fixed-point sums in LDS), so a gradient a million times smaller than its
+    neighbours keeps three digits, not seven: the error is bounded per element against the largest
+    gradient of the volume, and stated here."""
+    g = wl.gen(840)
+    rois = wl.affine_rois(g, 2, (48, 40, 24))
+    shape, out = (2, 1, 24, 40, 48), (20, 24, 40)
+    gy = torch.randn(2, 1, *out, generator=g) * torch.pow(10.0, -6.0 * torch.rand(2, 1, *out, generator=g))
+    x = torch.zeros(shape, device=DEV, requires_grad=True)
+    ops.RoIAlignRotated(out, 1.0, 1)(x, rois.to(DEV)).backward(gy.to(DEV))
+    want = oracle.roi_align_backward(gy, rois, shape, 1.0, 1, True, 1, True)
+    err = (x.grad.cpu().double() - want).abs()
+    bound = 8 * 2.0 ** -20 * float(gy.abs().max())      # eight terms reach a voxel from one output voxel's sample
+    assert float(err.max()) <= bound, f"largest error {float(err.max()):.3e} > {bound:.3e}"
+    small = want.abs() < 1e-3 * float(want.abs().max())
+    assert bool(small.any()) and float(err[small].max()) <= bound
+
+
 def test_backward_tiles_with_zero_and_infinite_gradients(ops, oracle):
     """A grad_output of zeros leaves the gradient untouched; an infinity reaches the voxels the oracle
     sends it to (the tile that holds it adds its terms one by one, the others stay in fixed point)."""
