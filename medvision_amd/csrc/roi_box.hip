@@ -172,10 +172,18 @@ __device__ __forceinline__ BoxSample box_sample(const RoiGeom &g, const RoiProbl
 }
 
 constexpr int kBoxChannels = 16;   // channels a workgroup's tile holds at most (and a workgroup owns at most)
+// Samples per thread whose taps stay in registers while a block's channels pass through the tile: the
+// fp64 geometry of a sample is then worked out once per block, not once per pass.
+constexpr int kBoxKeep = 12;
+// A kept sample in 32 bits: offset of its low corner in the box (14 bits: the tile has 12288 cells), which
+// of the high taps differ from the low ones (x, y, z: bits 14 - 16), its output cell (from bit 17; heads of
+// up to 4096 cells).  Bit 31: the sample touches voxels beyond the box and is worked out again when used.
+constexpr unsigned kKeptVoid = 0xffffffffu, kKeptBeyond = 0x80000000u;
+static_assert(kBoxLds / 4 <= (1 << 14), "a kept sample's box offset has 14 bits");
 
 // ---- backward ------------------------------------------------------------------------------------
 // `per_group` <= kBoxChannels channels per workgroup; the tile holds `cpt` = as many of them as fit
-// side by side, so a sample's taps are worked out once per cpt channels.
+// side by side, so a sample's taps are applied to cpt channels at a time.
 template <typename T, bool ROT>
 __global__ __launch_bounds__(kBoxThreads, 3) void roi_box_backward_kernel(const T *__restrict__ gout,
                                                                           const float *__restrict__ rois,
@@ -186,6 +194,7 @@ __global__ __launch_bounds__(kBoxThreads, 3) void roi_box_backward_kernel(const 
   __shared__ BoxPlan plan;
   __shared__ __attribute__((aligned(16))) int tile[kBoxLds / 4];
   __shared__ unsigned bound[kBoxChannels];
+  __shared__ float to_quanta[kBoxChannels], from_quanta[kBoxChannels];
   const unsigned n = blockIdx.x;
   build_geom_block(gs, trig, rois + static_cast<long>(n) * roi_columns(p.ndim, p.rotated), p);
   // fixed-point sums only where a term keeps 20 binary digits below the channel's bound (fp32 tensors; 12
@@ -205,10 +214,39 @@ __global__ __launch_bounds__(kBoxThreads, 3) void roi_box_backward_kernel(const 
   const int count_shift = 31 - __clz(g.count);   // floor(log2 count): |g| / count < 2^(e - count_shift)
   const int n0 = b.n[0], box = b.n[0] * b.n[1] * b.n[2];
   const int cpt = b.mode == 1 ? min(per_group, (kBoxLds / 4) / box) : per_group;
-  const float inv_row = 1.f / static_cast<float>(n0), inv_rows = 1.f / static_cast<float>(b.n[1]), inv_box = 1.f / static_cast<float>(box);
+  const float inv_row = 1.f / static_cast<float>(n0), inv_rows = 1.f / static_cast<float>(b.n[1]);
   const int blocks = box_blocks(p, b);
   for (int block = 0; block < blocks; block++) {
     const BoxBlock k = box_block(g, p, b, block);
+    const bool few = static_cast<long>(k.cells) * count < (1L << 31);
+    const unsigned total = few ? static_cast<unsigned>(k.cells) * count : 0u;   // sample s = cell * count + sub
+    // several passes over the same samples: keep the first kBoxKeep per thread
+    const bool keep = few && b.mode == 1 && c_end - c_first > cpt;
+    unsigned kept[kBoxKeep];
+    float kfx[kBoxKeep], kfy[kBoxKeep], kfz[kBoxKeep];
+    if (keep) {
+      // worked out last to first, every record moving up one place per round, so that the geometry is
+      // compiled once and the records still sit in registers with fixed names
+#pragma unroll
+      for (int j = 0; j < kBoxKeep; j++) { kept[j] = kKeptVoid; kfx[j] = kfy[j] = kfz[j] = 0.f; }
+#pragma unroll 1
+      for (int round = kBoxKeep - 1; round >= 0; round--) {
+#pragma unroll
+        for (int j = kBoxKeep - 1; j > 0; j--) { kept[j] = kept[j - 1]; kfx[j] = kfx[j - 1]; kfy[j] = kfy[j - 1]; kfz[j] = kfz[j - 1]; }
+        kept[0] = kKeptVoid;
+        const unsigned s = threadIdx.x + static_cast<unsigned>(round) * kBoxThreads;
+        if (s < total) {
+          BoxTaps t;
+          const unsigned cell = block_cell(p, k, s / count);
+          const BoxSample q = box_sample<ROT>(g, p, b, k.lo, cell, s % count, t);
+          if (q.at >= 0)
+            kept[0] = static_cast<unsigned>(q.at) | (q.dx ? 1u << 14 : 0u) | (q.dy ? 1u << 15 : 0u) | (q.dz ? 1u << 16 : 0u) | (cell << 17);
+          else if (q.at == -2)
+            kept[0] = kKeptBeyond | (cell << 17);
+          kfx[0] = t.fx; kfy[0] = t.fy; kfz[0] = t.fz;
+        }
+      }
+    }
     for (int c0 = c_first; c0 < c_end; c0 += cpt) {
       const int nc = min(cpt, c_end - c0);
       const T *gsrc = gout + (static_cast<long>(n) * p.C + c0) * cells;
@@ -220,31 +258,36 @@ __global__ __launch_bounds__(kBoxThreads, 3) void roi_box_backward_kernel(const 
       }
       __syncthreads();
       // |term| <= max |g| / count < 2^(e - 126 - count_shift): quanta of 2^-term_bits of that power of two.
-      // A channel with a NaN or an infinity in its gradient takes the per-sample path.
-      auto channel_scale = [&](int ch, float &to_quanta) -> bool {
-        const unsigned bits = bound[ch];
+      // A channel with a NaN or an infinity in its gradient takes the per-sample path (scale 0).
+      if (threadIdx.x < nc) {
+        const unsigned bits = bound[threadIdx.x];
         const int ex = min(max(127 + 126 + count_shift + b.term_bits - static_cast<int>(bits >> 23), 1), 253);
-        to_quanta = __uint_as_float(static_cast<unsigned>(ex) << 23) * inv_count;
-        return bits < 0x7f800000u;
+        to_quanta[threadIdx.x] = bits < 0x7f800000u ? __uint_as_float(static_cast<unsigned>(ex) << 23) * inv_count : 0.f;
+        from_quanta[threadIdx.x] = __uint_as_float(static_cast<unsigned>(254 - ex) << 23);
+      }
+      __syncthreads();
+      // a sample inside the box: its eight terms per channel into the tile
+      auto into_tile = [&](int at, int dx, int dy, int dz, const float (&w)[8], int ch, float gv, float scale) {
+        const float gq = gv * scale;
+        int *cell0 = tile + ch * box + at;
+#pragma unroll
+        for (int m = 0; m < 8; m++) {
+          const int v = __float2int_rn(gq * w[m]);
+          if (v != 0)
+            __hip_atomic_fetch_add(cell0 + ((m >> 2) ? dz : 0) + (((m >> 1) & 1) ? dy : 0) + ((m & 1) ? dx : 0), v, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
       };
-      auto scatter = [&](unsigned cell, unsigned sub) {
+      auto scatter = [&](unsigned cell, unsigned sub, bool beyond_only) {
         BoxTaps t;
         const BoxSample q = box_sample<ROT>(g, p, b, k.lo, cell, sub, t);
         if (q.at == -1) return;
         for (int ch = 0; ch < nc; ch++) {
           const float gv = static_cast<float>(load(gsrc + static_cast<long>(ch) * cells + cell));
           if (gv == 0.f) continue;
-          float to_quanta;
-          if (channel_scale(ch, to_quanta) && q.at >= 0) {
-            const float gq = gv * to_quanta;
-            int *cell0 = tile + ch * box + q.at;
-#pragma unroll
-            for (int m = 0; m < 8; m++) {
-              const int v = __float2int_rn(gq * q.w[m]);
-              if (v != 0)
-                __hip_atomic_fetch_add(cell0 + ((m >> 2) ? q.dz : 0) + (((m >> 1) & 1) ? q.dy : 0) + ((m & 1) ? q.dx : 0), v,
-                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            }
+          const float scale = to_quanta[ch];
+          if (scale != 0.f && q.at >= 0) {
+            if (!beyond_only) into_tile(q.at, q.dx, q.dy, q.dz, q.w, ch, gv, scale);
           } else {
             const float top = gv * inv_count;
             float *dst = vol + static_cast<long>(ch) * plane;
@@ -255,34 +298,86 @@ __global__ __launch_bounds__(kBoxThreads, 3) void roi_box_backward_kernel(const 
           }
         }
       };
-      if (static_cast<long>(k.cells) * count < (1L << 31)) {
-        // sample s = cell * count + sub: neighbouring lanes take neighbouring samples
-        const unsigned total = static_cast<unsigned>(k.cells) * count;
-        for (unsigned s = threadIdx.x; s < total; s += kBoxThreads) scatter(block_cell(p, k, s / count), s % count);
+      unsigned first = threadIdx.x;
+      unsigned again = 0, apart = 0;   // kept samples to work out again: all their terms / those of channels without a scale
+      if (keep) {
+        // four records per round, then every record moves down four places: after the last round each is
+        // back where the next pass expects it (unrolled over all twelve, the compiler ran out of registers)
+#pragma unroll 1
+        for (int round = 0; round < kBoxKeep / 4; round++) {
+#pragma unroll
+          for (int u = 0; u < 4; u++) {
+            const int j = round * 4 + u;
+            const unsigned rec = kept[u];
+            if (static_cast<unsigned>(j) * kBoxThreads >= total || rec == kKeptVoid) continue;
+            if (rec & kKeptBeyond) { again |= 1u << j; continue; }
+            const unsigned cell = (rec >> 17) & 0x3fffu;
+            const float wx[2] = {1.f - kfx[u], kfx[u]}, wy[2] = {1.f - kfy[u], kfy[u]}, wz[2] = {1.f - kfz[u], kfz[u]};
+            float w[8];
+#pragma unroll
+            for (int m = 0; m < 8; m++) w[m] = wz[m >> 2] * wy[(m >> 1) & 1] * wx[m & 1];
+            const int at = static_cast<int>(rec & 0x3fffu);
+            const int dx = (rec >> 14) & 1, dy = (rec & (1u << 15)) ? n0 : 0, dz = (rec & (1u << 16)) ? n0 * b.n[1] : 0;
+            for (int ch = 0; ch < nc; ch++) {
+              const float gv = static_cast<float>(load(gsrc + static_cast<long>(ch) * cells + cell));
+              if (gv == 0.f) continue;
+              const float scale = to_quanta[ch];
+              if (scale != 0.f) into_tile(at, dx, dy, dz, w, ch, gv, scale);
+              else apart |= 1u << j;   // a channel without a scale: its terms go out one by one
+            }
+          }
+#pragma unroll
+          for (int u = 0; u < 4; u++) {
+            const unsigned r0 = kept[u];
+            const float x0 = kfx[u], y0 = kfy[u], z0 = kfz[u];
+#pragma unroll
+            for (int j = u; j + 4 < kBoxKeep; j += 4) { kept[j] = kept[j + 4]; kfx[j] = kfx[j + 4]; kfy[j] = kfy[j + 4]; kfz[j] = kfz[j + 4]; }
+            kept[kBoxKeep - 4 + u] = r0; kfx[kBoxKeep - 4 + u] = x0; kfy[kBoxKeep - 4 + u] = y0; kfz[kBoxKeep - 4 + u] = z0;
+          }
+        }
+        first += kBoxKeep * kBoxThreads;
+      }
+      if (few) {
+        // neighbouring lanes take neighbouring samples; first what the kept records left over
+        unsigned next = first;
+        while (true) {
+          unsigned s;
+          bool beyond_only = false;
+          if (again | apart) {
+            const int j = __ffs(static_cast<int>(again | apart)) - 1;
+            beyond_only = !((again >> j) & 1u);
+            again &= ~(1u << j); apart &= ~(1u << j);
+            s = threadIdx.x + static_cast<unsigned>(j) * kBoxThreads;
+          } else if (next < total) {
+            s = next; next += kBoxThreads;
+          } else {
+            break;
+          }
+          scatter(block_cell(p, k, s / count), s % count, beyond_only);
+        }
       } else {
         for (unsigned i = threadIdx.x; i < static_cast<unsigned>(k.cells); i += kBoxThreads)
-          for (unsigned sub = 0; sub < count; sub++) scatter(block_cell(p, k, i), sub);
+          for (unsigned sub = 0; sub < count; sub++) scatter(block_cell(p, k, i), sub, false);
       }
       __syncthreads();
       if (b.mode == 1) {
         // lanes along the box's rows: neighbouring lanes add to neighbouring voxels of the buffer
-        for (int i = threadIdx.x; i < nc * box; i += kBoxThreads) {
-          const int q = tile[i];
-          if (q == 0) continue;
-          tile[i] = 0;
-          const int ch = static_cast<int>((static_cast<float>(i) + 0.5f) * inv_box), v = i - ch * box;
-          const int row = static_cast<int>((static_cast<float>(v) + 0.5f) * inv_row), bx = v - row * n0;
-          const int bz = static_cast<int>((static_cast<float>(row) + 0.5f) * inv_rows), by = row - bz * b.n[1];
-          const unsigned bits = bound[ch];
-          const int ex = min(max(127 + 126 + count_shift + b.term_bits - static_cast<int>(bits >> 23), 1), 253);
-          const float from_quanta = __uint_as_float(static_cast<unsigned>(254 - ex) << 23);
-          atomic_add(vol + static_cast<long>(ch) * plane + (static_cast<long>(bz + k.lo[2]) * p.H + (by + k.lo[1])) * p.W + (k.lo[0] + bx),
-                     static_cast<float>(q) * from_quanta);
+        for (int ch = 0; ch < nc; ch++) {
+          const float unit = from_quanta[ch];
+          int *sums = tile + ch * box;
+          float *dst = vol + static_cast<long>(ch) * plane + (static_cast<long>(k.lo[2]) * p.H + k.lo[1]) * p.W + k.lo[0];
+          for (int v = threadIdx.x; v < box; v += kBoxThreads) {
+            const int q = sums[v];
+            if (q == 0) continue;
+            sums[v] = 0;
+            const int row = static_cast<int>((static_cast<float>(v) + 0.5f) * inv_row), bx = v - row * n0;
+            const int bz = static_cast<int>((static_cast<float>(row) + 0.5f) * inv_rows), by = row - bz * b.n[1];
+            atomic_add(dst + static_cast<long>(bz * p.H + by) * p.W + bx, static_cast<float>(q) * unit);
+          }
         }
       }
-      __syncthreads();
       if (threadIdx.x < kBoxChannels) bound[threadIdx.x] = 0;
-      __syncthreads();   // (the next pass takes its maxima behind this barrier)
+      __syncthreads();   // (the next pass takes its maxima and writes its scales behind this barrier)
     }
   }
 }

@@ -983,6 +983,47 @@ def test_rotated_heads_backward_through_box_tiles(ops, oracle, dtype, ndim):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("ndim", [3, 2])
+def test_rotated_heads_backward_with_many_rois_and_channels(ops, oracle, dtype, ndim):
+    """Enough rois x channels for a workgroup to own several channels: a block's samples are worked out
+    once and their taps kept in registers while the channels pass through the LDS tile.  Boxes from one
+    channel per pass (large rois) to all of a workgroup's channels side by side (small ones), more samples
+    per thread than are kept (grid 3, 14^2 cells), a NaN and an infinity in single channels (those
+    channels' terms go out one by one, the others' through the tile), zero gradients."""
+    g = wl.gen(650 + ndim)
+    size = (18, 26, 30)[3 - ndim:]
+    out = (7, 7, 7) if ndim == 3 else (14, 14)
+    C, n = 32, 300
+    feat = torch.randn(2, C, *size, generator=g).to(dtype)
+    xyz = torch.tensor(size[::-1], dtype=torch.float32)
+    ctr = (torch.rand(n, ndim, generator=g) * 1.2 - 0.1) * xyz
+    ext = torch.exp(torch.rand(n, ndim, generator=g) * math.log(40.0)) * 0.6      # 0.6 .. 24 voxels
+    ang = (torch.rand(n, 3 if ndim == 3 else 1, generator=g) * 2 - 1) * math.radians(40)
+    rois = torch.cat([torch.randint(0, 2, (n, 1), generator=g).float(), ctr, ext, ang], 1)
+    for sr in (2, 3, 0):
+        x = feat.to(DEV).requires_grad_(True)
+        y = ops.RoIAlignRotated(out, 1.0, sr, True)(x, rois.to(DEV))
+        gy = torch.randn(y.shape, generator=g).to(dtype)
+        gy[torch.rand(y.shape, generator=g) < 0.05] = 0
+        y.backward(gy.to(DEV))
+        want = oracle.roi_align_backward(gy, rois, feat.shape, 1.0, sr, True, 1, True)
+        assert_close(x.grad, want, BWD_TOL[dtype], f"backward sr={sr}")
+    x = feat.to(DEV).requires_grad_(True)
+    y = ops.RoIAlignRotated(out, 1.0, 2, True)(x, rois.to(DEV))
+    gy = torch.randn(y.shape, generator=g).to(dtype)
+    big = int(torch.argmax(ext.prod(dim=1)))
+    gy[big, 3].view(-1)[gy[big, 3].numel() // 2] = float("nan")
+    gy[(big + 1) % n, 17].view(-1)[5] = float("inf")
+    y.backward(gy.to(DEV))
+    want = oracle.roi_align_backward(gy, rois, feat.shape, 1.0, 2, True, 1, True)
+    got = x.grad.cpu()
+    assert torch.isnan(want).any() and torch.equal(torch.isnan(got), torch.isnan(want))
+    assert torch.equal(torch.isinf(got), torch.isinf(want))
+    ok = torch.isfinite(want)
+    assert_close(got[ok], want[ok], BWD_TOL[dtype], "NaN and infinite gradients")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("ndim,rotated,C,out", [(3, True, 24, (7, 7, 7)), (3, True, 72, (7, 7, 7)),
                                                 (2, True, 520, (14, 14)), (2, False, 32, (20, 20))])
 def test_heads_forward_from_channels_last_copy(ops, oracle, dtype, ndim, rotated, C, out):
