@@ -171,6 +171,92 @@ __device__ __forceinline__ BoxSample box_sample(const RoiGeom &g, const RoiProbl
   return k;
 }
 
+// ---- largest rois first ----------------------------------------------------------------------------
+// A workgroup's time grows with its roi's box, tenfold between the rois of one detection head, and the
+// kernel ends with its slowest workgroup: workgroups therefore take the rois in descending order of size.
+// No sorted list exists anywhere: every workgroup works out by itself which roi has its rank, from a
+// histogram of size classes (four per octave of the extents' product) and a count within its class, in
+// index order -- the same bijection in every workgroup.  Two passes over the roi table (<= kRankRois
+// rows, from the caches) and four barriers, a few microseconds per workgroup.
+constexpr int kRankBuckets = 128;
+constexpr int kRankRois = 4096;   // more rois than this run in index order (the tail of the launch is short then)
+constexpr int kRankPerThread = kRankRois / kBoxThreads;
+__device__ __forceinline__ unsigned roi_size_class(const float *roi, const RoiProblem &p) {
+  float v = 1.f;
+  for (int a = 0; a < p.ndim; a++) {
+    const float e = p.rotated ? roi[1 + p.ndim + a] : roi[1 + p.ndim + a] - roi[1 + a];
+    v *= fmaxf(e * static_cast<float>(p.scale), 1e-3f);
+  }
+  if (!(v == v)) return kRankBuckets - 1;
+  // exponent and two mantissa bits, 2^22 voxels and more in class 0
+  const int cls = (127 + 22) * 4 + 3 - static_cast<int>(__float_as_uint(v) >> 21);
+  return static_cast<unsigned>(min(max(cls, 0), kRankBuckets - 1));
+}
+// Every thread of the workgroup must call it; `lds` holds kRankBuckets + 8 words.
+__device__ inline unsigned roi_of_rank(const float *__restrict__ rois, const RoiProblem &p, unsigned rank, unsigned *lds) {
+  const int cols = roi_columns(p.ndim, p.rotated);
+  const unsigned per = (static_cast<unsigned>(p.R) + kBoxThreads - 1) / kBoxThreads;   // <= kRankPerThread
+  const unsigned first = threadIdx.x * per;
+  unsigned *hist = lds, *wave_total = lds + kRankBuckets, *picked = lds + kRankBuckets + 4;
+  if (threadIdx.x < kRankBuckets) hist[threadIdx.x] = 0;
+  __syncthreads();
+  unsigned cls[kRankPerThread / 4];   // a byte per roi of the thread's run
+#pragma unroll
+  for (int i = 0; i < kRankPerThread / 4; i++) cls[i] = 0;
+#pragma unroll
+  for (int i = 0; i < kRankPerThread; i++) {
+    const unsigned r = first + i;
+    if (static_cast<unsigned>(i) < per && r < static_cast<unsigned>(p.R)) {
+      const unsigned c = roi_size_class(rois + static_cast<long>(r) * cols, p);
+      cls[i / 4] |= c << (8 * (i % 4));
+      atomicAdd(&hist[c], 1u);
+    }
+  }
+  __syncthreads();
+  // the class that holds the rank, and the rank within it: lane l of the first wavefront owns classes 2l, 2l + 1
+  if (threadIdx.x < 64) {
+    const unsigned h0 = hist[2 * threadIdx.x], h1 = hist[2 * threadIdx.x + 1];
+    unsigned incl = h0 + h1;
+#pragma unroll
+    for (int d = 1; d < 64; d *= 2) {
+      const unsigned up = __shfl_up(incl, d);
+      if (threadIdx.x >= static_cast<unsigned>(d)) incl += up;
+    }
+    const unsigned excl = incl - h0 - h1;
+    if (rank >= excl && rank < excl + h0) { picked[0] = 2 * threadIdx.x; picked[1] = rank - excl; }
+    else if (rank >= excl + h0 && rank < incl) { picked[0] = 2 * threadIdx.x + 1; picked[1] = rank - excl - h0; }
+  }
+  __syncthreads();
+  const unsigned want = picked[0], kth = picked[1];
+  unsigned mine = 0;
+#pragma unroll
+  for (int i = 0; i < kRankPerThread; i++)
+    if (static_cast<unsigned>(i) < per && first + i < static_cast<unsigned>(p.R) && ((cls[i / 4] >> (8 * (i % 4))) & 0xffu) == want) mine++;
+  // exclusive sum of `mine` over the workgroup's threads
+  unsigned incl = mine;
+  const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int d = 1; d < 64; d *= 2) {
+    const unsigned up = __shfl_up(incl, d);
+    if (lane >= static_cast<unsigned>(d)) incl += up;
+  }
+  if (lane == 63) wave_total[wave] = incl;
+  __syncthreads();
+  unsigned before = incl - mine;
+  for (unsigned w = 0; w < wave; w++) before += wave_total[w];
+  if (kth >= before && kth < before + mine) {
+    unsigned left = kth - before;
+#pragma unroll
+    for (int i = 0; i < kRankPerThread; i++)
+      if (static_cast<unsigned>(i) < per && first + i < static_cast<unsigned>(p.R) && ((cls[i / 4] >> (8 * (i % 4))) & 0xffu) == want) {
+        if (left == 0) picked[2] = first + i;
+        left--;
+      }
+  }
+  __syncthreads();
+  return picked[2];
+}
+
 constexpr int kBoxChannels = 16;   // channels a workgroup's tile holds at most (and a workgroup owns at most)
 // Samples per thread whose taps stay in registers while a block's channels pass through the tile: the
 // fp64 geometry of a sample is then worked out once per block, not once per pass.
@@ -188,14 +274,19 @@ template <typename T, bool ROT>
 __global__ __launch_bounds__(kBoxThreads, 3) void roi_box_backward_kernel(const T *__restrict__ gout,
                                                                           const float *__restrict__ rois,
                                                                           float *__restrict__ acc, const RoiProblem p,
-                                                                          const int per_group) {
+                                                                          const int per_group, const int groups, const int ranked) {
   __shared__ RoiGeom gs;
   __shared__ double trig[6];
   __shared__ BoxPlan plan;
   __shared__ __attribute__((aligned(16))) int tile[kBoxLds / 4];
   __shared__ unsigned bound[kBoxChannels];
   __shared__ float to_quanta[kBoxChannels], from_quanta[kBoxChannels];
-  const unsigned n = blockIdx.x;
+  __shared__ unsigned rank_scratch[kRankBuckets + 8];
+  // the channel groups of a roi run side by side (they read the same gradient rows and roi), and the
+  // rois in descending order of size where `ranked` says so
+  const unsigned group_index = blockIdx.x % static_cast<unsigned>(groups);
+  unsigned n = blockIdx.x / static_cast<unsigned>(groups);
+  if (ranked) n = roi_of_rank(rois, p, n, rank_scratch);
   build_geom_block(gs, trig, rois + static_cast<long>(n) * roi_columns(p.ndim, p.rotated), p);
   // fixed-point sums only where a term keeps 20 binary digits below the channel's bound (fp32 tensors; 12
   // for 16-bit ones): boxes of a voxel or less, where thousands of samples meet in one voxel, add per sample
@@ -209,13 +300,16 @@ __global__ __launch_bounds__(kBoxThreads, 3) void roi_box_backward_kernel(const 
   const int cells = p.od * p.oh * p.ow;
   const unsigned count = static_cast<unsigned>(g.count);
   const long plane = static_cast<long>(p.D) * p.H * p.W;
-  const int c_first = blockIdx.y * per_group, c_end = min(c_first + per_group, p.C);
+  const int c_first = group_index * per_group, c_end = min(c_first + per_group, p.C);
   const float inv_count = 1.f / static_cast<float>(g.count);
   const int count_shift = 31 - __clz(g.count);   // floor(log2 count): |g| / count < 2^(e - count_shift)
   const int n0 = b.n[0], box = b.n[0] * b.n[1] * b.n[2];
   const int cpt = b.mode == 1 ? min(per_group, (kBoxLds / 4) / box) : per_group;
   const float inv_row = 1.f / static_cast<float>(n0), inv_rows = 1.f / static_cast<float>(b.n[1]);
   const int blocks = box_blocks(p, b);
+  const int row_skip = p.W - n0;
+  const long slice_skip = static_cast<long>(p.H - b.n[1]) * p.W;
+  const bool narrow = plane < (1L << 31);   // offsets within a channel fit 32 bits
   for (int block = 0; block < blocks; block++) {
     const BoxBlock k = box_block(g, p, b, block);
     const bool few = static_cast<long>(k.cells) * count < (1L << 31);
@@ -366,13 +460,23 @@ __global__ __launch_bounds__(kBoxThreads, 3) void roi_box_backward_kernel(const 
           const float unit = from_quanta[ch];
           int *sums = tile + ch * box;
           float *dst = vol + static_cast<long>(ch) * plane + (static_cast<long>(k.lo[2]) * p.H + k.lo[1]) * p.W + k.lo[0];
-          for (int v = threadIdx.x; v < box; v += kBoxThreads) {
-            const int q = sums[v];
-            if (q == 0) continue;
-            sums[v] = 0;
-            const int row = static_cast<int>((static_cast<float>(v) + 0.5f) * inv_row), bx = v - row * n0;
-            const int bz = static_cast<int>((static_cast<float>(row) + 0.5f) * inv_rows), by = row - bz * b.n[1];
-            atomic_add(dst + static_cast<long>(bz * p.H + by) * p.W + bx, static_cast<float>(q) * unit);
+          // four cells per lane and round, read together; a cell's place in the volume from its place in the
+          // box: v + row * (W - n0) + slice * (H - n1) * W
+          for (int v0 = threadIdx.x; v0 < box; v0 += 4 * kBoxThreads) {
+            int q[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) q[u] = v0 + u * kBoxThreads < box ? sums[v0 + u * kBoxThreads] : 0;
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+              if (q[u] == 0) continue;
+              const int v = v0 + u * kBoxThreads;
+              sums[v] = 0;
+              const int row = static_cast<int>((static_cast<float>(v) + 0.5f) * inv_row);
+              const int bz = static_cast<int>((static_cast<float>(row) + 0.5f) * inv_rows);
+              const float add = static_cast<float>(q[u]) * unit;
+              if (narrow) atomic_add(dst + static_cast<unsigned>(v + row * row_skip + bz * static_cast<int>(slice_skip)), add);
+              else atomic_add(dst + (v + static_cast<long>(row) * row_skip + bz * slice_skip), add);
+            }
           }
         }
       }
@@ -405,16 +509,18 @@ int roi_box_backward(const void *grad_output, const void *rois, float *acc, int 
   if (!roi_box_applies(dtype, p)) return -1;
   const int per = box_channels_per_group(p);
   const long groups = (p.C + per - 1) / per;
-  if (groups > 65535) return -1;
-  const dim3 grid(p.R, static_cast<unsigned>(groups)), block(kBoxThreads);
+  if (static_cast<long>(p.R) * groups > 0x7fffffffL) return -1;
+  const dim3 grid(static_cast<unsigned>(p.R * groups)), block(kBoxThreads);
+  // in descending order of size while the launch is a few rounds of workgroups, whose last round the largest rois would stretch
+  const int ranked = p.R > 1 && p.R <= kRankRois ? 1 : 0;
   const float *r = static_cast<const float *>(rois);
 #define MV_BOX_BACKWARD(TYPE)                                                                                              \
   if (p.rotated)                                                                                                           \
     hipLaunchKernelGGL((roi_box_backward_kernel<TYPE, true>), grid, block, 0, s, static_cast<const TYPE *>(grad_output), r, \
-                       acc, p, per);                                                                                       \
+                       acc, p, per, static_cast<int>(groups), ranked);                                                                                       \
   else                                                                                                                     \
     hipLaunchKernelGGL((roi_box_backward_kernel<TYPE, false>), grid, block, 0, s, static_cast<const TYPE *>(grad_output), r, \
-                       acc, p, per)
+                       acc, p, per, static_cast<int>(groups), ranked)
   switch (dtype) {
     case MV_F32: MV_BOX_BACKWARD(float); break;
     case MV_F16: MV_BOX_BACKWARD(__half); break;

@@ -1021,6 +1021,22 @@ def test_rotated_heads_backward_with_many_rois_and_channels(ops, oracle, dtype, 
     assert torch.equal(torch.isinf(got), torch.isinf(want))
     ok = torch.isfinite(want)
     assert_close(got[ok], want[ok], BWD_TOL[dtype], "NaN and infinite gradients")
+    # Workgroups take the rois in descending order of size (every workgroup finds the roi of its rank by
+    # itself), up to 4096 rois; beyond, in index order.  Either way every roi must be taken exactly once:
+    # rois of equal size (one size class, ranks told apart by index), sizes over many octaves.
+    for n in (4096, 4099):
+        small = (2,) * ndim
+        ctr = torch.rand(n, ndim, generator=g) * xyz
+        ext = torch.exp(torch.rand(n, ndim, generator=g) * math.log(3000.0)) * 0.01
+        ext[: n // 4] = 3.0
+        ang = (torch.rand(n, 3 if ndim == 3 else 1, generator=g) * 2 - 1) * math.radians(40)
+        rois = torch.cat([torch.randint(0, 2, (n, 1), generator=g).float(), ctr, ext, ang], 1)
+        x = feat[:, :3].to(DEV).requires_grad_(True)
+        y = ops.RoIAlignRotated(small, 1.0, 2, True)(x, rois.to(DEV))
+        gy = torch.randn(y.shape, generator=g).to(dtype)
+        y.backward(gy.to(DEV))
+        want = oracle.roi_align_backward(gy, rois, x.shape, 1.0, 2, True, 1, True)
+        assert_close(x.grad, want, BWD_TOL[dtype], f"{n} rois")
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
