@@ -10,7 +10,7 @@
 // the tile's non-zero sums then go to the fp32 gradient buffer as one atomic per voxel with lanes along
 // x (one request per 64-byte sector) instead of one scattered atomic per sample corner.  The tile
 // holds as many of the workgroup's channels side by side as fit, so a sample's taps are worked out
-// once for all of them.  Scale per (block, channel): max |grad_output| / count < 2^e is mapped to 2^t
+// once for all of them.  Scale per (roi, channel): max |grad_output| / count < 2^e is mapped to 2^t
 // quanta, t = 30 - ceil(log2(samples that can reach one voxel)); a term is rounded by at most
 // 2^-(t+1) of that bound.  Rois with t < 20 (fp32 tensors; 12 for 16-bit ones: boxes of about a voxel,
 // where thousands of samples meet), blocks of one cell whose box still does not fit, and channels whose
@@ -310,6 +310,25 @@ __global__ __launch_bounds__(kBoxThreads, 3) void roi_box_backward_kernel(const 
   const int row_skip = p.W - n0;
   const long slice_skip = static_cast<long>(p.H - b.n[1]) * p.W;
   const bool narrow = plane < (1L << 31);   // offsets within a channel fit 32 bits
+  // Per channel of the workgroup the largest |grad_output| of the roi, as the bit pattern of a float (NaNs
+  // order above infinity): |term| <= max |g| / count < 2^(e - 126 - count_shift), and a term is counted in
+  // quanta of 2^-term_bits of that power of two.  A channel with a NaN or an infinity in its gradient takes
+  // the per-sample path (scale 0).
+  {
+    const T *gall = gout + (static_cast<long>(n) * p.C + c_first) * cells;
+    const int span = (c_end - c_first) * cells;
+    const float inv_cells = 1.f / static_cast<float>(cells);
+    for (int i = threadIdx.x; i < span; i += kBoxThreads)
+      atomicMax(&bound[static_cast<int>((static_cast<float>(i) + 0.5f) * inv_cells)], __float_as_uint(fabsf(static_cast<float>(load(gall + i)))));
+    __syncthreads();
+    if (static_cast<int>(threadIdx.x) < c_end - c_first) {
+      const unsigned bits = bound[threadIdx.x];
+      const int ex = min(max(127 + 126 + count_shift + b.term_bits - static_cast<int>(bits >> 23), 1), 253);
+      to_quanta[threadIdx.x] = bits < 0x7f800000u ? __uint_as_float(static_cast<unsigned>(ex) << 23) * inv_count : 0.f;
+      from_quanta[threadIdx.x] = __uint_as_float(static_cast<unsigned>(254 - ex) << 23);
+    }
+    __syncthreads();
+  }
   for (int block = 0; block < blocks; block++) {
     const BoxBlock k = box_block(g, p, b, block);
     const bool few = static_cast<long>(k.cells) * count < (1L << 31);
@@ -345,21 +364,7 @@ __global__ __launch_bounds__(kBoxThreads, 3) void roi_box_backward_kernel(const 
       const int nc = min(cpt, c_end - c0);
       const T *gsrc = gout + (static_cast<long>(n) * p.C + c0) * cells;
       float *vol = acc + (static_cast<long>(g.batch) * p.C + c0) * plane;
-      // per channel the largest |grad_output| of the block as the bit pattern of a float (NaNs order above infinity)
-      for (int i = threadIdx.x; i < nc * k.cells; i += kBoxThreads) {
-        const int ch = i / k.cells;
-        atomicMax(&bound[ch], __float_as_uint(fabsf(static_cast<float>(load(gsrc + static_cast<long>(ch) * cells + block_cell(p, k, i - ch * k.cells))))));
-      }
-      __syncthreads();
-      // |term| <= max |g| / count < 2^(e - 126 - count_shift): quanta of 2^-term_bits of that power of two.
-      // A channel with a NaN or an infinity in its gradient takes the per-sample path (scale 0).
-      if (threadIdx.x < nc) {
-        const unsigned bits = bound[threadIdx.x];
-        const int ex = min(max(127 + 126 + count_shift + b.term_bits - static_cast<int>(bits >> 23), 1), 253);
-        to_quanta[threadIdx.x] = bits < 0x7f800000u ? __uint_as_float(static_cast<unsigned>(ex) << 23) * inv_count : 0.f;
-        from_quanta[threadIdx.x] = __uint_as_float(static_cast<unsigned>(254 - ex) << 23);
-      }
-      __syncthreads();
+      const int cq = c0 - c_first;   // the pass's first channel among the workgroup's
       // a sample inside the box: its eight terms per channel into the tile
       auto into_tile = [&](int at, int dx, int dy, int dz, const float (&w)[8], int ch, float gv, float scale) {
         const float gq = gv * scale;
@@ -379,7 +384,7 @@ __global__ __launch_bounds__(kBoxThreads, 3) void roi_box_backward_kernel(const 
         for (int ch = 0; ch < nc; ch++) {
           const float gv = static_cast<float>(load(gsrc + static_cast<long>(ch) * cells + cell));
           if (gv == 0.f) continue;
-          const float scale = to_quanta[ch];
+          const float scale = to_quanta[cq + ch];
           if (scale != 0.f && q.at >= 0) {
             if (!beyond_only) into_tile(q.at, q.dx, q.dy, q.dz, q.w, ch, gv, scale);
           } else {
@@ -415,7 +420,7 @@ __global__ __launch_bounds__(kBoxThreads, 3) void roi_box_backward_kernel(const 
             for (int ch = 0; ch < nc; ch++) {
               const float gv = static_cast<float>(load(gsrc + static_cast<long>(ch) * cells + cell));
               if (gv == 0.f) continue;
-              const float scale = to_quanta[ch];
+              const float scale = to_quanta[cq + ch];
               if (scale != 0.f) into_tile(at, dx, dy, dz, w, ch, gv, scale);
               else apart |= 1u << j;   // a channel without a scale: its terms go out one by one
             }
@@ -457,7 +462,7 @@ __global__ __launch_bounds__(kBoxThreads, 3) void roi_box_backward_kernel(const 
       if (b.mode == 1) {
         // lanes along the box's rows: neighbouring lanes add to neighbouring voxels of the buffer
         for (int ch = 0; ch < nc; ch++) {
-          const float unit = from_quanta[ch];
+          const float unit = from_quanta[cq + ch];
           int *sums = tile + ch * box;
           float *dst = vol + static_cast<long>(ch) * plane + (static_cast<long>(k.lo[2]) * p.H + k.lo[1]) * p.W + k.lo[0];
           // four cells per lane and round, read together; a cell's place in the volume from its place in the
@@ -480,8 +485,7 @@ __global__ __launch_bounds__(kBoxThreads, 3) void roi_box_backward_kernel(const 
           }
         }
       }
-      if (threadIdx.x < kBoxChannels) bound[threadIdx.x] = 0;
-      __syncthreads();   // (the next pass takes its maxima and writes its scales behind this barrier)
+      __syncthreads();   // (the next pass adds to the cells that this one has just cleared)
     }
   }
 }
