@@ -199,6 +199,7 @@ __device__ inline unsigned roi_of_rank(const float *__restrict__ rois, const Roi
   const unsigned first = threadIdx.x * per;
   unsigned *hist = lds, *wave_total = lds + kRankBuckets, *picked = lds + kRankBuckets + 4;
   if (threadIdx.x < kRankBuckets) hist[threadIdx.x] = 0;
+  if (threadIdx.x == 0) { picked[0] = 0; picked[1] = 0; picked[2] = rank; }   // (rank < R: a valid roi whatever follows)
   __syncthreads();
   unsigned cls[kRankPerThread / 4];   // a byte per roi of the thread's run
 #pragma unroll
@@ -254,7 +255,7 @@ __device__ inline unsigned roi_of_rank(const float *__restrict__ rois, const Roi
       }
   }
   __syncthreads();
-  return picked[2];
+  return min(picked[2], static_cast<unsigned>(p.R) - 1u);
 }
 
 constexpr int kBoxChannels = 16;   // channels a workgroup's tile holds at most (and a workgroup owns at most)
