@@ -460,6 +460,36 @@ def resample_timeline(args):
                                                     "second_half_of_each_xcd": round(float(np.median(done[len(done) // 2:])), 2)}}))
 
 
+def lds_tap_reads(args):
+    """The tap reads of the tiled resampler on their own, in four forms (`mv_debug_lds_tap_reads` of the
+    instrumented twin of the library, csrc/roi_resample.hip): clocks of a compute unit per voxel-wavefront."""
+    import ctypes
+    from medvision_amd import build
+    raw = ctypes.CDLL(build.TIMELINE_LIB_PATH)
+    fn = raw.mv_debug_lds_tap_reads
+    fn.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.POINTER(ctypes.c_float), ctypes.c_void_p]
+    props = torch.cuda.get_device_properties(0)
+    cus, mhz = props.multi_processor_count, 1970.0   # (clocks at the shader clock that the profiles' counters showed: 1.97 GHz)
+    out = torch.zeros(1024 * cus, dtype=torch.int32, device="cuda:0")
+    torch.cuda.synchronize()
+    names = ["eight 2-byte reads", "four ds_read2_b32", "four ds_read_b64 at 4-byte alignment",
+             "four aligned dword reads (as from a shifted second copy)"]
+    iters, rows = 400, []
+    for form, name in enumerate(names):
+        best = None
+        for rep in range(4):
+            ms = ctypes.c_float(0)
+            rc = fn(form, iters, 20.0, ctypes.c_void_p(out.data_ptr()), ctypes.byref(ms), None)
+            if rc != 0:
+                sys.exit("mv_debug_lds_tap_reads failed: %d" % rc)
+            best = ms.value if best is None or ms.value < best else best
+        # a compute unit runs two workgroups of eight wavefronts, each wavefront iters x 8 voxels
+        per = best * 1e-3 / (iters * 8 * 8 * 2)
+        rows.append({"form": name, "ms": round(best, 4), "ns_per_voxel_wavefront": round(per * 1e9, 2),
+                     "clocks_per_voxel_wavefront": round(per * mhz * 1e6, 1)})
+    print(json.dumps({"lds_tap_reads": rows, "clock_mhz": mhz, "compute_units": cus}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -473,6 +503,8 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="wall time spent on the CPU oracle")
     ap.add_argument("--timeline", action="store_true",
                     help="only print the in-kernel phase times of the tiled resampler (instrumented library)")
+    ap.add_argument("--lds-taps", action="store_true",
+                    help="only time the resampler's LDS tap reads on their own, in four forms (instrumented library)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a device copy of 4*128^3 fp16 elements (counter calibration)")
     args = ap.parse_args()
@@ -483,6 +515,9 @@ def main():
     from medvision_amd import _lib
     if args.timeline:
         resample_timeline(args)
+        return
+    if args.lds_taps:
+        lds_tap_reads(args)
         return
     _lib.load()
     if args.copy_calibration:

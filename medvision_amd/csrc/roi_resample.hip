@@ -2098,4 +2098,91 @@ extern "C" int mv_debug_resample_timeline(void *host, size_t bytes) {
   const size_t all = sizeof(unsigned long long) * mv::kTimelineGroups * mv::kTimelineSlots;
   return static_cast<int>(hipMemcpyFromSymbol(host, HIP_SYMBOL(mv::mv_timeline), bytes < all ? bytes : all));
 }
+
+// The tap reads of the tiled forward kernel on their own (a measuring aid like the time stamps above): 512
+// threads and two workgroups per compute unit as in the kernel, a 16-bit box in LDS, every lane a column of
+// eight voxels whose low corners follow a rotation by `degrees` about all three axes; the corner addresses
+// are worked out before the timed loop, which holds little besides the reads.  FORM 0: eight 2-byte reads per
+// voxel (what the kernel does); 1: four `ds_read2_b32` (two dwords each, the first at the even voxel at or
+// below the low tap); 2: four `ds_read_b64` at those 4-byte-aligned addresses; 3: four aligned dword reads,
+// as a second copy of the box shifted by one voxel would allow (the odd lanes read elsewhere in the tile).
+namespace mv {
+struct TapReadShape { float m[12]; int n0, n1, n2, pitch, slice, iters, one; };
+template <int FORM>
+__global__ __launch_bounds__(512, 2) void lds_tap_reads_kernel(const TapReadShape p, unsigned *out) {
+  __shared__ __attribute__((aligned(16))) unsigned short box[74 * 1024 / 2];
+  for (int i = threadIdx.x; i < 74 * 1024 / 2; i += 512) box[i] = static_cast<unsigned short>(i * 7 + 1);
+  __syncthreads();
+  const int ox = threadIdx.x % 16, oy = threadIdx.x / 16 % 16, zb = threadIdx.x / 256 * 8;
+  unsigned acc = 0;
+  int base_k[8], x_k[8];
+#pragma unroll
+  for (int k = 0; k < 8; k++) {
+    const float x = ox, y = oy, z = zb + k;
+    const float sx = p.m[0] + p.m[1] * x + p.m[2] * y + p.m[3] * z, sy = p.m[4] + p.m[5] * x + p.m[6] * y + p.m[7] * z;
+    const float sz = p.m[8] + p.m[9] * x + p.m[10] * y + p.m[11] * z;
+    const int x0 = min(max(static_cast<int>(sx), 0), p.n0 - 3), y0 = min(max(static_cast<int>(sy), 0), p.n1 - 3);
+    const int z0 = min(max(static_cast<int>(sz), 0), p.n2 - 3);
+    base_k[k] = z0 * p.slice + y0 * p.pitch;
+    x_k[k] = x0;
+  }
+  for (int it = 0; it < p.iters; it++) {
+    const int shift = (it & 1) * p.pitch;
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+      const int base = base_k[k] + shift, x0 = x_k[k];
+      if (FORM == 0) {
+        const unsigned short *b = box + base + x0;
+        const int o = p.one;   // (a run-time 1: the compiler would merge b[0] and b[1] into one misaligned dword read)
+        acc ^= b[0] ^ b[o] ^ b[p.pitch] ^ b[p.pitch + o] ^ b[p.slice] ^ b[p.slice + o] ^ b[p.slice + p.pitch] ^ b[p.slice + p.pitch + o];
+      } else if (FORM == 3) {
+        const unsigned *w = reinterpret_cast<const unsigned *>(box) + ((base + (x0 & ~1)) >> 1) + (x0 & 1) * 4096;
+        acc ^= w[0] ^ w[p.pitch >> 1] ^ w[p.slice >> 1] ^ w[(p.slice + p.pitch) >> 1];
+      } else {
+        unsigned long long v[4];
+        const int offs[4] = {0, p.pitch, p.slice, p.slice + p.pitch};
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const unsigned addr = static_cast<unsigned>(reinterpret_cast<size_t>(box + base + offs[q] + (x0 & ~1)));
+          if (FORM == 1) asm volatile("ds_read2_b32 %0, %1 offset1:1" : "=v"(v[q]) : "v"(addr));
+          else asm volatile("ds_read_b64 %0, %1" : "=v"(v[q]) : "v"(addr));
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]));
+        acc ^= static_cast<unsigned>(v[0]) ^ static_cast<unsigned>(v[1] >> 32) ^ static_cast<unsigned>(v[2]) ^ static_cast<unsigned>(v[3] >> 32);
+      }
+    }
+  }
+  out[blockIdx.x * 512 + threadIdx.x] = acc;
+}
+}  // namespace mv
+
+// Runs form `form` (0..3) on 2 x the compute units' workgroups, `iters` rounds of eight voxels per lane; `out` holds
+// 1024 x compute units words of device memory.  `*ms`: the launch's duration by HIP events (synchronises the stream).
+extern "C" int mv_debug_lds_tap_reads(int form, int iters, float degrees, unsigned *out, float *ms, void *stream) {
+  mv::TapReadShape p;
+  const double a = degrees * 3.14159265358979323846 / 180.0, ca = cos(a), sa = sin(a);
+  const double rot[9] = {ca * ca, ca * sa * sa - sa * ca, ca * sa * ca + sa * sa, sa * ca, sa * sa * sa + ca * ca,
+                         sa * sa * ca - ca * sa, -sa, ca * sa, ca * ca};
+  for (int r = 0; r < 3; r++) {
+    p.m[4 * r] = 8.f;
+    for (int c = 0; c < 3; c++) p.m[4 * r + 1 + c] = static_cast<float>(rot[3 * r + c]);
+  }
+  p.n0 = 24; p.n1 = 24; p.n2 = 24; p.pitch = 24; p.slice = 24 * 24 + 16; p.iters = iters; p.one = 1;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(2 * mv::compute_units()), block(512);
+  hipEvent_t e0, e1;
+  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return 1;
+  hipEventRecord(e0, s);
+  switch (form) {
+    case 0: hipLaunchKernelGGL(mv::lds_tap_reads_kernel<0>, grid, block, 0, s, p, out); break;
+    case 1: hipLaunchKernelGGL(mv::lds_tap_reads_kernel<1>, grid, block, 0, s, p, out); break;
+    case 2: hipLaunchKernelGGL(mv::lds_tap_reads_kernel<2>, grid, block, 0, s, p, out); break;
+    default: hipLaunchKernelGGL(mv::lds_tap_reads_kernel<3>, grid, block, 0, s, p, out);
+  }
+  hipEventRecord(e1, s);
+  const hipError_t st = hipEventSynchronize(e1);
+  if (st == hipSuccess) hipEventElapsedTime(ms, e0, e1);
+  hipEventDestroy(e0); hipEventDestroy(e1);
+  return st == hipSuccess ? 0 : 1;
+}
 #endif
