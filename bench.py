@@ -253,6 +253,10 @@ def bench_next_rows(args):
     img = vol[:2]
     ms, _ = _events_ms(lambda i: ops.apply_offset_3d(img, field, 1), n, 10)
     res["apply_offset_3d_2x128^3_fp16"] = {"ms": round(ms, 4), "gvox_s": round(2 * 128 ** 3 / ms / 1e6, 2)}
+    img2 = torch.randn(8, 3, 512, 512, generator=g).half().to(dev)
+    field2 = (torch.randn(8, 2, 512, 512, generator=g) * 3).half().to(dev)
+    ms, _ = _events_ms(lambda i: ops.apply_offset_2d(img2, field2, 1), n, 10)
+    res["apply_offset_2d_8x3x512^2_fp16"] = {"ms": round(ms, 4), "gpix_s": round(8 * 3 * 512 ** 2 / ms / 1e6, 2)}
     B, C, H, W = 8, 256, 100, 152
     x = torch.randn(B, C, H, W, generator=g).half().to(dev)
     w = (torch.randn(C, C, 3, 3, generator=g) * 0.02).half().to(dev)
