@@ -214,6 +214,15 @@ def bench_other_configs(args):
     bms, _ = _events_ms(lambda i: _C.roi_align_rotated_3d_backward(gy, rois, gi, 7, 7, 7, 1.0, 2, True, 1), 10, 2)
     res["rotated_head_1000x64x7^3_fp16"] = {"forward_ms": round(ms, 4), "backward_ms": round(bms, 4)}
     del feat, out, gy, gi
+    # a 2-D head with large rois on a fine feature map (bins of 2 - 16 pixels, grid 2: the boxes are read sparsely)
+    feat = torch.randn(2, 256, 200, 304, generator=g).half().to(dev)
+    lo = torch.rand(1000, 2, generator=g) * torch.tensor([250., 160.])
+    ext = 16 + torch.rand(1000, 2, generator=g) * 100
+    rois = torch.cat([torch.randint(0, 2, (1000, 1), generator=g).float(), lo, lo + ext], 1).to(dev)
+    out = torch.empty(1000, 256, 7, 7, dtype=torch.float16, device=dev)
+    ms, _ = _events_ms(lambda i: _C.roi_align_2d_forward(feat, rois, out, 7, 7, 1.0, 2, 1), 20, 3)
+    res["head_2d_1000x256x7^2_rois_16_116px_fp16"] = {"forward_ms": round(ms, 4)}
+    del feat, out
     # RandomAffine on images: fp16 [8,3,512,512], one full-image rotated roi per sample (the tiled kernel with
     # the image rows as slices)
     g = wl.gen(10)

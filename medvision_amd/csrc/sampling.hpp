@@ -82,6 +82,12 @@ __device__ __forceinline__ typename Acc<T>::type sample_clamped(const T *plane, 
   const A hz = A(1) - lz, hy = A(1) - ly, hx = A(1) - lx;
   const T *r00 = plane + (static_cast<long>(z0) * H + y0) * W;
   const T *r01 = plane + (static_cast<long>(z0) * H + y1) * W;
+  if (D == 1) {
+    // an image: the upper slice is the lower one with weight 0 (its four taps are not loaded), as in the
+    // reference's bilinear 2-D kernels (csrc/cuda/interpolation_helpers_2d.h)
+    const A v1 = load(r00 + x0), v2 = load(r00 + x1), v3 = load(r01 + x0), v4 = load(r01 + x1);
+    return hy * (hx * v1 + lx * v2) + ly * (hx * v3 + lx * v4);
+  }
   const T *r10 = plane + (static_cast<long>(z1) * H + y0) * W;
   const T *r11 = plane + (static_cast<long>(z1) * H + y1) * W;
   const A v1 = load(r00 + x0), v2 = load(r00 + x1), v3 = load(r01 + x0), v4 = load(r01 + x1);

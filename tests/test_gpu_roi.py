@@ -311,6 +311,28 @@ def test_pooled_kernels_with_large_boxes(ops, oracle, shape, out, sr, extent, dt
                      "backward")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("ndim", [2, 3])
+def test_pooled_forward_with_dense_and_sparse_rois_in_one_call(ops, oracle, dtype, ndim):
+    """Plain boxes from a fraction of a voxel to most of the feature map, grids of 1 and 2: a roi whose box
+    holds more than half as many voxels as its samples have taps is read sparsely and takes its taps one
+    by one (on images four per sample, the absent slice left out), the others stage their box in LDS;
+    both kinds in one launch, 40 channels (matrix-core blocks and the remainder)."""
+    g = wl.gen(420 + ndim)
+    size = (20, 72, 88)[3 - ndim:]
+    out = (7,) * ndim
+    feat = torch.randn(2, 40, *size, generator=g).to(dtype)
+    xyz = torch.tensor(size[::-1], dtype=torch.float32)
+    n = 48
+    ext = torch.exp(torch.rand(n, ndim, generator=g) * math.log(150.0)) * 0.5          # 0.5 .. 75 voxels
+    ext = torch.minimum(ext, xyz * 1.1)
+    lo = torch.rand(n, ndim, generator=g) * (xyz - ext + 6) - 3
+    rois = torch.cat([torch.randint(0, 2, (n, 1), generator=g).float(), lo, lo + ext], 1)
+    for sr in (1, 2):
+        y = ops.RoIAlign(out, 1.0, sr)(feat.to(DEV), rois.to(DEV))
+        assert_close(y, oracle.roi_align_forward(feat, rois, out, 1.0, sr, True, 1, False), FWD_TOL[dtype], f"forward sr={sr}")
+
+
 @pytest.mark.parametrize("out", [(1, 1, 1), (1, 2, 3), (2, 3, 3)])
 def test_pooled_backward_reads_only_its_own_gradients(ops, oracle, out):
     """fp16 heads with a few cells per roi: the matrix-core backward loads a plane of cells as 16-byte
