@@ -1086,9 +1086,12 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
   if (plan.staged == 1 && !wide) {
     const long bx = sh.ax[0].box_hi - sh.ax[0].box_lo + 1, by = sh.ax[1].box_hi - sh.ax[1].box_lo + 1;
     zs = sh.ax[2].box_hi - sh.ax[2].box_lo + 1;
-    const bool box = !CL;                                  // planar sums: the slab of the box itself is staged
+    const bool box = !CL && dense;                         // planar sums from the dense matrices: the slab of the box itself is staged
     const long per_plane = (box ? by * bx * 4 : 0L) + (by * p.ow + static_cast<long>(p.oh) * p.ow) * 4;
     const int want = min(CL ? 16 : 4, c_end - c_begin);
+    // (the set-up has counted a staged box: planar sums through the tap tables keep none, so that a plane of
+    // an image that is larger than LDS still takes this path and not one atomic per tap of every sample)
+    if (!CL && !dense) plan.chunk = static_cast<int>(min(kPoolLdsBytes / (zs * per_plane + 16), 64L));
     if (plan.chunk < want) {
       zs = static_cast<int>(min(max((kPoolLdsBytes / want - 16) / per_plane, 1L), static_cast<long>(zs)));
       plan.chunk = static_cast<int>(min(kPoolLdsBytes / (zs * per_plane + 16), 64L));
@@ -1232,8 +1235,7 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
     const int nzs = min(zs, nz - z0);
     const int vol_s = nx * ny * nzs;
     const float inv_vol_s = 1.f / vol_s, inv_nzsohw = 1.f / (nzs * ohw);
-    float *gbox = reinterpret_cast<float *>(lds);    // [cs][nzs][ny][nx] (planar accumulation only)
-    float *t1 = gbox + (CL ? 0 : cs * vol_s);          // [cs][nzs][ny][ow]
+    float *t1 = reinterpret_cast<float *>(lds);       // [cs][nzs][ny][ow]
     float *t2 = t1 + cs * nzs * ny * p.ow;            // [cs][nzs][oh][ow]
     const T *go = src + static_cast<long>(cb - c_begin) * cells;
     // Transposed contractions as gathers.  Entries are sorted by coordinate, so the entries whose
@@ -1285,6 +1287,7 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
         }
       }
     } else {
+      G *corner = dst + static_cast<long>(cb - c_begin) * plane + first;
       for (int i = threadIdx.x; i < cs * vol_s; i += kPoolThreads) {  // transpose of "contract x"
         const int row = fdiv(i, inv_nx), x = i - row * nx;
         const float *r = t1 + row * p.ow;
@@ -1294,16 +1297,10 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_backward_kernel(
           const float w = e < mid ? (tx.hi[e] == x ? tx.whi[e] : 0.f) : tx.wlo[e];
           acc += w * r[fdiv(e, inv_gx)];
         }
-        gbox[i] = acc;
-      }
-      __syncthreads();
-      G *corner = dst + static_cast<long>(cb - c_begin) * plane + first;
-      for (int i = threadIdx.x; i < cs * vol_s; i += kPoolThreads) {
-        const float v = gbox[i];
-        if (v == 0.f) continue;
-        const int c = fdiv(i, inv_vol_s), r0 = i - c * vol_s, z = fdiv(r0, inv_nxy), r1 = r0 - z * nx * ny;
-        const int y = fdiv(r1, inv_nx), x = r1 - y * nx;
-        atomic_add(corner + c * plane + (static_cast<long>(z) * p.H + y) * p.W + x, static_cast<G>(v));
+        // (a lane per voxel of a row: the lanes of a wavefront add runs of contiguous elements as they are)
+        if (acc == 0.f) continue;
+        const int c = fdiv(i, inv_vol_s), r0 = i - c * vol_s, z = fdiv(r0, inv_nxy), y = fdiv(r0 - z * nx * ny, inv_nx);
+        atomic_add(corner + c * plane + (static_cast<long>(z) * p.H + y) * p.W + x, static_cast<G>(acc));
       }
     }
     __syncthreads();

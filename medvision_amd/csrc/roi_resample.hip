@@ -2172,17 +2172,17 @@ extern "C" int mv_debug_lds_tap_reads(int form, int iters, float degrees, unsign
   const dim3 grid(2 * mv::compute_units()), block(512);
   hipEvent_t e0, e1;
   if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return 1;
-  hipEventRecord(e0, s);
+  (void)hipEventRecord(e0, s);
   switch (form) {
     case 0: hipLaunchKernelGGL(mv::lds_tap_reads_kernel<0>, grid, block, 0, s, p, out); break;
     case 1: hipLaunchKernelGGL(mv::lds_tap_reads_kernel<1>, grid, block, 0, s, p, out); break;
     case 2: hipLaunchKernelGGL(mv::lds_tap_reads_kernel<2>, grid, block, 0, s, p, out); break;
     default: hipLaunchKernelGGL(mv::lds_tap_reads_kernel<3>, grid, block, 0, s, p, out);
   }
-  hipEventRecord(e1, s);
+  (void)hipEventRecord(e1, s);
   const hipError_t st = hipEventSynchronize(e1);
-  if (st == hipSuccess) hipEventElapsedTime(ms, e0, e1);
-  hipEventDestroy(e0); hipEventDestroy(e1);
+  if (st == hipSuccess) (void)hipEventElapsedTime(ms, e0, e1);
+  (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
   return st == hipSuccess ? 0 : 1;
 }
 #endif

@@ -52,9 +52,11 @@ __global__ __launch_bounds__(256) void deform_warp_kernel(const T *__restrict__ 
           T lo, hi;
           if constexpr (sizeof(T) == 2) {
             if (pairs) {
-              struct __attribute__((packed, aligned(2))) Pair { T a, b; };
-              const Pair two = *reinterpret_cast<const Pair *>(plane + cw.idx[n]);
-              lo = two.a; hi = two.b;
+              unsigned two;
+              __builtin_memcpy(&two, plane + cw.idx[n], sizeof(two));
+              const unsigned short l = static_cast<unsigned short>(two & 0xffffu), h = static_cast<unsigned short>(two >> 16);
+              __builtin_memcpy(&lo, &l, sizeof(l));
+              __builtin_memcpy(&hi, &h, sizeof(h));
             } else {
               lo = plane[cw.idx[n]]; hi = plane[cw.idx[n + 1]];
             }
