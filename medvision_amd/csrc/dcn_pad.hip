@@ -26,7 +26,9 @@ bool dcn_pad_plan(const DcnDims &s, int dtype, DcnPad &pad) {
   if (other % unit != 0) return false;   // groups that do not nest keep the general kernels
   const int unit_p = round_up32(unit), opg_p = round_up32(s.opg);
   if (unit_p == unit && opg_p == s.opg) return false;
-  if (static_cast<long>(s.Cin) * s.Cout < 256) return false;   // tiny layers: the copies would cost more
+  // (Every size: the general kernels take 0.15 - 0.3 ms even for a layer of 8 -> 8 channels on a 4^3 volume, where
+  // the padded layer with its copies takes 0.06 ms; on [2, 8, 64^3] they took 1.9 ms forward and 40 ms backward
+  // against 0.5 and 2.7 ms.)
   DcnDims p = s;
   p.cpg = s.cpg / unit * unit_p;
   p.cpd = s.cpd / unit * unit_p;
