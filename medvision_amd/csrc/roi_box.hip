@@ -77,12 +77,25 @@ __device__ inline void plan_box(BoxPlan &b, const RoiGeom &g, const RoiProblem &
     if (widest < 0) break;
     b.blk[widest] = (b.blk[widest] + 1) / 2;
   }
-  // samples that can reach one voxel: those within a ball of radius sqrt(3) on the lattice of spacing sub
-  long terms = 1;
+  // What the samples can add up to in one voxel, in units of the largest term: the smaller of
+  //  - the number of samples that reach a voxel (those within a ball of radius sqrt(3) on the lattice of spacing
+  //    sub, at most all samples along an axis), and
+  //  - the sum of their WEIGHTS.  A sample's weight is a product of tent functions of its distance to the voxel;
+  //    every sample owns a cell of the lattice (volume sub_x sub_y sub_z, extent e_a = sum_j |rot[a][j]| sub_j along
+  //    voxel axis a), over which the tent widened by e_a / 2 on either side is at least the sample's own, so the
+  //    sum is at most the integral of the widened tents over the cell volume: prod_a (1 + e_a) / prod_j sub_j
+  //    (plain boxes: prod (1 / sub + 1)).  Thousands of samples may reach a voxel of a finely sampled roi, but their
+  //    weights add up to a few hundred.  (The half quantum that each of the reaching terms may be rounded by is
+  //    some tens of quanta per unit of weight, nothing beside the 2^30 quanta that the sums may reach.)
+  double count_bound = 1.0, weight_bound = 1.0;
   for (int j = 0; j < p.ndim; j++) {
-    const double along = static_cast<double>(cells[j]) * g.grid[j];
-    terms *= static_cast<long>(fmin(3.4642 / fmax(g.sub[j], 1e-9) + 1.0, fmax(along, 1.0)));
+    const double along = fmax(static_cast<double>(cells[j]) * g.grid[j], 1.0), sub = fmax(g.sub[j], 1e-9);
+    count_bound *= floor(fmin(3.4642 / sub + 1.0, along));
+    double e = 0.0;
+    for (int k = 0; k < p.ndim; k++) e += fabs(g.rot[3 * j + k]) * fmax(g.sub[k], 1e-9);
+    weight_bound *= (1.0 + e) / sub;
   }
+  const long terms = static_cast<long>(ceil(fmin(fmin(count_bound, weight_bound), 1e15)));
   int bits = 0;
   while ((1L << bits) < terms && bits < 40) bits++;
   b.term_bits = 30 - bits;

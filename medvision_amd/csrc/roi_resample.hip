@@ -1764,12 +1764,28 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
     // on every axis, i.e. inside a ball of radius sqrt(3); along output axis j (samples b_j / g_j apart,
     // b_j = length of column j of the map) that leaves floor(2 sqrt(3) g_j / b_j) + 1 of them.
     int terms = 1;
+    float u[3][3];   // the lattice of the samples: u[j] = step of one sample along output axis j, in source voxels
 #pragma unroll
     for (int j = 0; j < 3; j++) {
       const float c0 = static_cast<float>(map[1 + j]), c1 = static_cast<float>(map[5 + j]), c2 = static_cast<float>(map[9 + j]);
       const float bj = sqrtf(c0 * c0 + c1 * c1 + c2 * c2);
       const int ext = j == 0 ? TX : (j == 1 ? TY : TZ), gj = GRIDS ? plan_scalar(&r.grid[j]) : 1;
       terms *= static_cast<int>(fminf(3.4642f * static_cast<float>(gj) / bj * 1.00001f + 1.f, static_cast<float>(ext * gj)));
+      const float ig = 1.f / static_cast<float>(gj);
+      u[j][0] = c0 * ig; u[j][1] = c1 * ig; u[j][2] = c2 * ig;
+    }
+    // The sum of the WEIGHTS of those terms is smaller still where the samples are dense: every sample owns a cell
+    // of the lattice (volume |det u|, extent e_a = sum_j |u[j][a]| along source axis a), over which the tent
+    // function widened by e_a / 2 on either side is at least the sample's own weight, so the weights that reach a
+    // voxel add up to at most prod_a (1 + e_a) / |det u|.  (Volumes only: an image's middle axis has one sample.)
+    if (TY > 1) {
+      const float det = fabsf(u[0][0] * (u[1][1] * u[2][2] - u[1][2] * u[2][1]) - u[0][1] * (u[1][0] * u[2][2] - u[1][2] * u[2][0]) +
+                              u[0][2] * (u[1][0] * u[2][1] - u[1][1] * u[2][0]));
+      float w = 1.f;
+#pragma unroll
+      for (int a = 0; a < 3; a++) w *= 1.f + fabsf(u[0][a]) + fabsf(u[1][a]) + fabsf(u[2][a]);
+      const float sum = w / fmaxf(det, 1e-30f) * 1.0001f + 1.f;
+      if (sum < static_cast<float>(terms)) terms = max(static_cast<int>(sum), 1);
     }
     const int term_bits = 30 - (32 - __clz(terms - 1));   // 30 - ceil(log2 terms); >= kTermBits at one sample per bin
     // finite terms, box within the tile, enough bits per term: 18 for fp32 tensors, 12 for 16-bit ones (a
