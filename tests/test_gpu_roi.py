@@ -1004,6 +1004,39 @@ def test_rotated_heads_backward_through_box_tiles(ops, oracle, dtype, ndim):
     assert_close(got[ok], want[ok], BWD_TOL[dtype], "a NaN gradient")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("rotated", [False, True])
+@pytest.mark.parametrize("out", [(14, 14, 14), (20, 20, 20)])
+def test_backward_of_finely_sampled_rois_with_gradients_of_one_sign(ops, oracle, dtype, rotated, out):
+    """Grids far finer than the voxels (bins of 0.15 - 0.6 voxels with 2 or 3 samples each): thousands of
+    samples reach a voxel, and the 32-bit fixed-point sums of the box and tile kernels are scaled by a bound
+    on the sum of their weights, not by their number.  Gradients that are all +1 add up without cancelling:
+    a bound that were too small would overflow the sums, and the result would be far off."""
+    g = wl.gen(900 + len(out) + out[0])
+    size = (16, 20, 24)
+    n, C = 10, 3
+    xyz = torch.tensor(size[::-1], dtype=torch.float32)
+    ext = 2.0 + torch.rand(n, 3, generator=g) * 6.0
+    ctr = torch.rand(n, 3, generator=g) * xyz
+    b = torch.randint(0, 2, (n, 1), generator=g).float()
+    if rotated:
+        rois = torch.cat([b, ctr, ext, (torch.rand(n, 3, generator=g) * 2 - 1) * 0.7], 1)
+        mod = lambda sr: ops.RoIAlignRotated(out, 1.0, sr, True)
+    else:
+        rois = torch.cat([b, ctr - ext / 2, ctr + ext / 2], 1)
+        mod = lambda sr: ops.RoIAlign(out, 1.0, sr)
+    shape = (2, C, *size)
+    for sr in (2, 3):
+        x = torch.zeros(shape, dtype=dtype, device=DEV, requires_grad=True)
+        y = mod(sr)(x, rois.to(DEV))
+        gy = torch.ones(y.shape, dtype=dtype)
+        y.backward(gy.to(DEV))
+        want = oracle.roi_align_backward(gy, rois, shape, 1.0, sr, True, 1, rotated)
+        assert_close(x.grad, want, BWD_TOL[dtype], f"backward sr={sr}")
+        # every sample lies in the volume or is void: the mass that arrives is the mass of the valid samples
+        assert abs(float(x.grad.double().sum()) - float(want.sum())) <= 2e-3 * float(want.abs().sum())
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("ndim", [3, 2])
 def test_rotated_heads_backward_with_many_rois_and_channels(ops, oracle, dtype, ndim):
