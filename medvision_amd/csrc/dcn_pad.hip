@@ -26,9 +26,14 @@ bool dcn_pad_plan(const DcnDims &s, int dtype, DcnPad &pad) {
   if (other % unit != 0) return false;   // groups that do not nest keep the general kernels
   const int unit_p = round_up32(unit), opg_p = round_up32(s.opg);
   if (unit_p == unit && opg_p == s.opg) return false;
-  // (Every size: the general kernels take 0.15 - 0.3 ms even for a layer of 8 -> 8 channels on a 4^3 volume, where
-  // the padded layer with its copies takes 0.06 ms; on [2, 8, 64^3] they took 1.9 ms forward and 40 ms backward
-  // against 0.5 and 2.7 ms.)
+  // Which small layers pay for the copies, measured on [2, C, 64^3] .. [2, C, 4^3] with 3^3 taps: the general kernels'
+  // time grows with Cin x Cout (8 -> 8 channels on 64^3: 1.9 ms forward, 40 ms backward, against 0.5 and 2.7 ms padded
+  // to 32 channels; 3 -> 8 on 32^3: 1.9 -> 0.9 ms per training step; even on a 4^3 volume 0.3 -> 0.06 ms forward), and
+  // only below 16 weights per tap are they the faster ones (1 -> 1 and 1 -> 8 channels: 0.35 against 1.1 ms forward
+  // in fp32) -- those stay, which also keeps fp32 columns for layers whose one or two weight gradients are sums
+  // that may nearly cancel.  bf16 layers stay below 256 as before: with 8-bit products such a weight gradient was
+  // off by several per cent of itself in random layers.
+  if (static_cast<long>(s.Cin) * s.Cout < (dtype == MV_BF16 ? 256 : 16)) return false;
   DcnDims p = s;
   p.cpg = s.cpg / unit * unit_p;
   p.cpd = s.cpd / unit * unit_p;
