@@ -657,7 +657,9 @@ __global__ __launch_bounds__(kPoolThreads) void roi_pool_forward_kernel(
     int cs = 0, zs = 0;
     // (measured on 24^3 - 32^3 boxes: the per-output gather below costs about as much as the slabs with
     // 27 samples per output, a third with 8, twice with 64)
-    for (int c = gx * gy * gz > 27 ? 8 : 0; c >= 1 && cs == 0; c >>= 1) {
+    // (one channel per slab, so that a slab holds as many planes as LDS takes: with 8 channels and a plane or two
+    // per slab the passes were 20 - 30 % slower — 200 rois of 24 - 32 voxels x 256 channels, grid 4: 7.0 -> 5.0 ms)
+    for (int c = gx * gy * gz > 27 ? 1 : 0; c >= 1 && cs == 0; c >>= 1) {
       const int cn = min(c, c_end - c_begin);
       const long planes = (kPoolLdsBytes - 32 - cn * static_cast<long>(cells) * 4) / (cn * per_plane);
       if (planes >= 1) { cs = cn; zs = static_cast<int>(min(planes, static_cast<long>(nz))); }
