@@ -554,12 +554,13 @@ def test_channel_counts_padded_for_the_matrix_cores(ops, oracle, dtype, cin, cou
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("cin,cout,groups,dg,modulated", [
-    (24, 40, 1, 1, True), (40, 24, 2, 1, True), (48, 48, 2, 2, False), (48, 80, 2, 4, True), (24, 64, 1, 3, False)])
+    (24, 40, 1, 1, True), (40, 24, 2, 1, True), (48, 48, 2, 2, False), (48, 80, 2, 4, True), (24, 64, 1, 3, False),
+    (8, 8, 1, 1, True), (4, 8, 1, 1, False)])
 def test_raw_abi_with_any_channel_count(oracle, dtype, cin, cout, groups, dg, modulated):
     """mv_dcn3d_forward / mv_dcn3d_backward called straight through ctypes (no shim in between) with
     channel counts that are no multiples of 32, several weight groups and deformable groups that
-    nest either way: results against the oracle, and on the matrix-core kernels (timed against a
-    bound the general kernels miss by an order of magnitude)."""
+    nest either way, layers of a few channels: results against the oracle, and on the matrix-core kernels
+    (timed against a bound the general kernels miss by an order of magnitude)."""
     import ctypes
     from medvision_amd import _lib
     lib = _lib.load()
@@ -574,9 +575,10 @@ def test_raw_abi_with_any_channel_count(oracle, dtype, cin, cout, groups, dg, mo
     code = _lib.DTYPES[dtype]
     xs, offs, ms, ws, bs = _to(DEV, x, off, mask, w, b)
     y = torch.full((2, cout, *size), float("nan"), dtype=dtype, device=DEV)
+    general = dtype == torch.bfloat16 and cin * cout < 256   # (bf16 layers of a few channels: general kernels, no copies)
     nf = lib.mv_dcn3d_forward_workspace_bytes(ctypes.byref(shape), code)
-    assert nf > 0
-    wsf = torch.empty(nf, dtype=torch.uint8, device=DEV)
+    assert nf > 0 or general
+    wsf = torch.empty(max(nf, 16), dtype=torch.uint8, device=DEV)
     stream = _lib.stream_of(xs)
 
     def forward():
@@ -642,6 +644,8 @@ def test_raw_abi_with_any_channel_count(oracle, dtype, cin, cout, groups, dg, mo
         torch.cuda.synchronize()
         return start.elapsed_time(stop) / 10
 
+    if general:
+        return   # (fp32 columns for their few weight gradients)
     for fn, native in ((forward, forward_native), (backward, backward_native)):
         ms_call, ms_native = timed(fn), timed(native)
         print(f"\n{fn.__name__} {dtype} cin={cin} cout={cout} groups={groups} dg={dg}: {ms_call:.3f} ms, "
