@@ -45,6 +45,7 @@ struct BoxPlan {
 __device__ inline void plan_box(BoxPlan &b, const RoiGeom &g, const RoiProblem &p, int cap_voxels, int min_term_bits) {
   const int cells[3] = {p.ow, p.oh, p.od}, size[3] = {p.W, p.H, p.D};
   bool empty = g.batch < 0 || g.grid[0] <= 0 || g.grid[1] <= 0 || (p.ndim == 3 && g.grid[2] <= 0);
+  double edge[3] = {2.0, 2.0, 2.0};
   // the whole roi: void when its samples' bounding box lies outside [-1, size] on some axis
   for (int a = 0; a < p.ndim && !empty; a++) {
     double c = g.centre[a], reach = 0.0;
@@ -55,6 +56,8 @@ __device__ inline void plan_box(BoxPlan &b, const RoiGeom &g, const RoiProblem &
     }
     const double rmin = c - reach - 1e-6, rmax = c + reach + 1e-6;
     if (rmax < -1.0 || rmin > static_cast<double>(size[a]) || !(rmin == rmin) || !(rmax == rmax)) empty = true;
+    // (samples beyond the first or last voxel are moved onto it with their full weight, see the bound below)
+    edge[a] = size[a] == 1 ? 2.0 : ((rmin < 0.0 || rmax > static_cast<double>(size[a] - 1)) ? 1.5 : 1.0);
   }
   for (int j = 0; j < 3; j++) { b.blk[j] = j < p.ndim ? cells[j] : 1; b.n[j] = 1; b.reach[j] = 0.0; }
   bool fits = false;
@@ -84,7 +87,9 @@ __device__ inline void plan_box(BoxPlan &b, const RoiGeom &g, const RoiProblem &
   //    every sample owns a cell of the lattice (volume sub_x sub_y sub_z, extent e_a = sum_j |rot[a][j]| sub_j along
   //    voxel axis a), over which the tent widened by e_a / 2 on either side is at least the sample's own, so the
   //    sum is at most the integral of the widened tents over the cell volume: prod_a (1 + e_a) / prod_j sub_j
-  //    (plain boxes: prod (1 / sub + 1)).  Thousands of samples may reach a voxel of a finely sampled roi, but their
+  //    (plain boxes: prod (1 / sub + 1)).  On an axis where the roi reaches past the volume's first or last voxel the
+  //    samples out there are moved onto that voxel with weight 1: its weight function has the integral 1.5 instead
+  //    of 1 (2 on an axis of one voxel).  Thousands of samples may reach a voxel of a finely sampled roi, but their
   //    weights add up to a few hundred.  (The half quantum that each of the reaching terms may be rounded by is
   //    some tens of quanta per unit of weight, nothing beside the 2^30 quanta that the sums may reach.)
   double count_bound = 1.0, weight_bound = 1.0;
@@ -93,7 +98,7 @@ __device__ inline void plan_box(BoxPlan &b, const RoiGeom &g, const RoiProblem &
     count_bound *= floor(fmin(3.4642 / sub + 1.0, along));
     double e = 0.0;
     for (int k = 0; k < p.ndim; k++) e += fabs(g.rot[3 * j + k]) * fmax(g.sub[k], 1e-9);
-    weight_bound *= (1.0 + e) / sub;
+    weight_bound *= (edge[j] + e) / sub;
   }
   const long terms = static_cast<long>(ceil(fmin(fmin(count_bound, weight_bound), 1e15)));
   int bits = 0;

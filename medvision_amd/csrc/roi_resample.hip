@@ -1777,13 +1777,17 @@ __global__ __launch_bounds__(kScatterThreads, 2 * kScatterWgs) void roi_backward
     // The sum of the WEIGHTS of those terms is smaller still where the samples are dense: every sample owns a cell
     // of the lattice (volume |det u|, extent e_a = sum_j |u[j][a]| along source axis a), over which the tent
     // function widened by e_a / 2 on either side is at least the sample's own weight, so the weights that reach a
-    // voxel add up to at most prod_a (1 + e_a) / |det u|.  (Volumes only: an image's middle axis has one sample.)
+    // voxel add up to at most prod_a (1 + e_a) / |det u| in a box that the volume does not clip.  (Volumes only: an
+    // image's middle axis has one sample.)
     if (TY > 1) {
       const float det = fabsf(u[0][0] * (u[1][1] * u[2][2] - u[1][2] * u[2][1]) - u[0][1] * (u[1][0] * u[2][2] - u[1][2] * u[2][0]) +
                               u[0][2] * (u[1][0] * u[2][1] - u[1][1] * u[2][0]));
       float w = 1.f;
+      // (a box that the volume clips: samples beyond the first or last voxel are moved onto it with weight 1, which
+      // gives that voxel's weight function the integral 1.5 instead of 1, 2 on an axis of one voxel)
+      const float edge = mode == 3 ? 1.f : 2.f;
 #pragma unroll
-      for (int a = 0; a < 3; a++) w *= 1.f + fabsf(u[0][a]) + fabsf(u[1][a]) + fabsf(u[2][a]);
+      for (int a = 0; a < 3; a++) w *= edge + fabsf(u[0][a]) + fabsf(u[1][a]) + fabsf(u[2][a]);
       const float sum = w / fmaxf(det, 1e-30f) * 1.0001f + 1.f;
       if (sum < static_cast<float>(terms)) terms = max(static_cast<int>(sum), 1);
     }

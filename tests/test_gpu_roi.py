@@ -1018,9 +1018,17 @@ def test_backward_of_finely_sampled_rois_with_gradients_of_one_sign(ops, oracle,
     xyz = torch.tensor(size[::-1], dtype=torch.float32)
     ext = 2.0 + torch.rand(n, 3, generator=g) * 6.0
     ctr = torch.rand(n, 3, generator=g) * xyz
+    # rois that start one voxel before the volume or end one voxel behind it: every sample out there is moved onto
+    # the first / last voxel with its full weight, the most that one voxel can collect
+    ctr[0] = ext[0] / 2 - 1.0
+    ctr[1] = xyz - ext[1] / 2 + 1.0
+    ctr[2, 0] = ext[2, 0] / 2 - 1.0
     b = torch.randint(0, 2, (n, 1), generator=g).float()
     if rotated:
-        rois = torch.cat([b, ctr, ext, (torch.rand(n, 3, generator=g) * 2 - 1) * 0.7], 1)
+        ext[:3] = ext[:3].clamp(max=4.0)
+        ang = (torch.rand(n, 3, generator=g) * 2 - 1) * 0.7
+        ang[:3] = 0
+        rois = torch.cat([b, ctr + 0.5, ext, ang], 1)    # (aligned: the centre is taken half a voxel lower)
         mod = lambda sr: ops.RoIAlignRotated(out, 1.0, sr, True)
     else:
         rois = torch.cat([b, ctr - ext / 2, ctr + ext / 2], 1)
