@@ -27,7 +27,7 @@ extern "C" {
 #endif
 
 typedef enum { MV_F32 = 0, MV_F16 = 1, MV_BF16 = 2, MV_F64 = 3,
-               MV_I32 = 4 /* label maps: mv_deform_warp_2d / _3d with order 0 only */ } mv_dtype;
+               MV_I32 = 4 /* label maps: mv_deform_warp_2d / _3d and mv_affine_2d / _3d, order 0 with one sample per cell only */ } mv_dtype;
 typedef enum { MV_OK = 0, MV_INVALID_ARGUMENT = 1, MV_HIP_ERROR = 2 } mv_status;
 
 const char *mv_last_error(void);

@@ -91,7 +91,8 @@ def _roi_forward(fn_name, what, ndim, cols, input, rois, output, out_sizes, spat
     want_shape = (r.size(0), dims[1], *out_sizes)
     if tuple(output.shape) != want_shape:
         raise RuntimeError(f"output has shape {tuple(output.shape)}, expected {want_shape}")
-    code = _lib.dtype_code(feats)
+    # (int32: label maps through the affine engines at order 0, which the library samples as they are)
+    code = _lib.MV_I32 if feats.dtype == torch.int32 and what == "affine" else _lib.dtype_code(feats)
     out3 = out_sizes if ndim == 3 else (1, *out_sizes)
     # the tiled resampler's plans, a re-ordered copy of the features for detection heads with plain
     # boxes, a channels-last copy for heads the separable kernels do not take

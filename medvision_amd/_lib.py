@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libmedvision_hip.so")
 
 MV_F32, MV_F16, MV_BF16, MV_F64 = 0, 1, 2, 3
-MV_I32 = 4   # int32 label maps: the order-0 displacement warp only
+MV_I32 = 4   # int32 label maps: the displacement warp and the affine engines at order 0
 DTYPES = {torch.float32: MV_F32, torch.float16: MV_F16, torch.bfloat16: MV_BF16,
           torch.float64: MV_F64}
 

@@ -47,6 +47,14 @@ class _Resampler:
         out = fn(batch, rois, tuple(int(v) for v in self._out_size()), 1.0, sampling_ratio, True, order)
         return out if self.batched else out.squeeze(0)
 
+    def _labels(self, seg, sampling_ratio):
+        """Order 0 on a label map.  The reference resamples a float copy and converts back
+        (aug_cuda/aug_spatial.py: ``.float()`` ... ``.int()``); int32 maps go to the library as they are,
+        which picks the same voxels and saves the two conversion passes."""
+        if seg.dtype == torch.int32:
+            return self._resample(seg, 0, sampling_ratio)
+        return self._resample(seg.float(), 0, sampling_ratio).int()
+
     def apply_to_img(self, result):
         for key in result.get('img_fields', []):
             if not self._skip():
@@ -56,7 +64,7 @@ class _Resampler:
     def apply_to_seg(self, result):
         for key in result.get('seg_fields', []):
             if not self._skip():
-                result[key] = self._resample(result[key].float(), 0, self.sampling_ratio).int()
+                result[key] = self._labels(result[key], self.sampling_ratio)
 
     def _after_img(self, result, key):
         if key == 'img' and not self.batched:
@@ -119,7 +127,7 @@ class CudaResize(_Resampler, CudaAugBase):
     def apply_to_seg(self, result):   # always a sampling grid of one (nearest)
         for key in result.get('seg_fields', []):
             if not self._skip():
-                result[key] = self._resample(result[key].float(), 0, 1).int()
+                result[key] = self._labels(result[key], 1)
 
     def apply_to_img(self, result):
         for key in result.get('img_fields', []):

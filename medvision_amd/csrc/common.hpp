@@ -68,7 +68,7 @@ template <> __device__ __forceinline__ __hip_bfloat16 store_cast<__hip_bfloat16>
 
 inline size_t dtype_size(int dtype) {
   switch (dtype) {
-    case MV_F32: return 4;
+    case MV_F32: case MV_I32: return 4;
     case MV_F16: case MV_BF16: return 2;
     case MV_F64: return 8;
   }

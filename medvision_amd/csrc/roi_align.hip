@@ -192,6 +192,24 @@ int roi_forward(const void *input, const void *rois, void *output, int dtype, in
   if (num_rois == 0) return MV_OK;
   MV_REQUIRE(input && rois && output, "null pointer argument");
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == MV_I32) {
+    // int32 label maps (the augmentation layer's segmentations): the voxel that order 0 picks, one sample per
+    // cell.  The reference resamples a float copy of the map and converts back
+    // (aug_cuda/aug_spatial.py: `.float()` ... `.int()`); here the two conversion passes happen in the loads
+    // and stores of the kernel.
+    MV_REQUIRE(order == 0 && sampling_ratio == 1 && prepared == nullptr,
+               "int32 label maps are resampled at order 0 with a sampling grid of one");
+    const int tiled = roi_forward_tiled(input, rois, output, dtype, p, workspace, workspace ? workspace_bytes : 0, nullptr, s);
+    if (tiled >= 0) return tiled;
+    const dim3 grid(p.chunks * num_rois), block(kRoiThreads);
+    if (rotated)
+      hipLaunchKernelGGL((roi_forward_kernel<int, float, true>), grid, block, 0, s, static_cast<const int *>(input),
+                         static_cast<const float *>(rois), static_cast<int *>(output), p);
+    else
+      hipLaunchKernelGGL((roi_forward_kernel<int, float, false>), grid, block, 0, s, static_cast<const int *>(input),
+                         static_cast<const float *>(rois), static_cast<int *>(output), p);
+    return check_launch("roi_forward_kernel");
+  }
   {
     // (a workspace too small for a path selects the kernels that need none)
     const size_t capacity = workspace ? workspace_bytes : 0;
@@ -426,7 +444,7 @@ size_t mv_roi_align_forward_workspace_bytes_for_input(int dtype, int ndim, int b
   p.ndim = ndim; p.N = batch; p.C = channels; p.D = ndim == 2 ? 1 : depth; p.H = height; p.W = width; p.R = num_rois;
   p.od = ndim == 2 ? 1 : out_d; p.oh = out_h; p.ow = out_w; p.sampling_ratio = sampling_ratio; p.order = 1;
   if (batch <= 0 || channels <= 0 || p.D <= 0 || height <= 0 || width <= 0 || num_rois <= 0) return basic;
-  if (basic) return basic;   // (the tiled resampler takes the problem)
+  if (basic || dtype == MV_I32) return basic;   // (the tiled resampler takes the problem; label maps have no other path that wants memory)
   const size_t pooled = mv::roi_pool_forward_workspace(dtype, p);
   return pooled ? pooled : mv::roi_forward_cl_workspace(dtype, p);
 }

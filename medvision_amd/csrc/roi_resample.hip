@@ -1555,6 +1555,10 @@ static int roi_forward_tiled_image(const void *input, const void *rois, void *ou
       st = launch_resample<__hip_bfloat16, 64, 1, 64, 512, 74 * 1024, 8>(static_cast<const __hip_bfloat16 *>(input), vol_rois,
                                                                           static_cast<__hip_bfloat16 *>(output), v, nullptr, need, s);
       break;
+    case MV_I32:
+      st = launch_resample<int, 64, 1, 32, 512, 74 * 1024, 6>(static_cast<const int *>(input), vol_rois,
+                                                               static_cast<int *>(output), v, nullptr, need, s);
+      break;
     default:
       st = launch_resample<float, 64, 1, 32, 512, 74 * 1024, 6>(static_cast<const float *>(input), vol_rois,
                                                                  static_cast<float *>(output), v, nullptr, need, s);
@@ -1568,6 +1572,9 @@ static int roi_forward_tiled_image(const void *input, const void *rois, void *ou
 // when the path does not apply.
 int roi_forward_tiled(const void *input, const void *rois, void *output, int dtype,
                       const RoiProblem &p, void *workspace, size_t capacity, size_t *need, hipStream_t s) {
+  // int32 label maps: one sample per cell at order 0 (the voxel's value passes through fp32, which holds
+  // labels below 2^24 exactly, as the float copy did that such maps used to be resampled through)
+  if (dtype == MV_I32 && (p.order != 0 || p.sampling_ratio != 1)) return -1;
   if (p.sampling_ratio >= 2 && p.sampling_ratio <= 4) {
     const int st = roi_forward_tiled_grid(input, rois, output, dtype, p, workspace, capacity, need, s);
     if (st != -1) return st;
@@ -1644,6 +1651,9 @@ int roi_forward_tiled(const void *input, const void *rois, void *output, int dty
     case MV_F32:
       return launch_resample<float, 16, 16, 8, 512, 74 * 1024, 6>(
           static_cast<const float *>(input), r, static_cast<float *>(output), p, workspace, need, s);
+    case MV_I32:
+      return launch_resample<int, 16, 16, 8, 512, 74 * 1024, 6>(
+          static_cast<const int *>(input), r, static_cast<int *>(output), p, workspace, need, s);
     default:
       return -1;
   }

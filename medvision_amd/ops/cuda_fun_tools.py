@@ -13,8 +13,9 @@ from .roi_align_nd import _parse_output_size
 
 def _affine(ndim, features, rois, out_size, spatial_scale, sampling_ratio, aligned, order):
     out = _parse_output_size(out_size, ndim)
-    assert features.dtype in [torch.float32, torch.float16, torch.bfloat16, torch.float64], \
-        f'input must be a floating tensor but got {features.dtype}'
+    # (int32: label maps at order 0, sampled as they are -- the reference resamples a float copy of them)
+    assert features.dtype in [torch.float32, torch.float16, torch.bfloat16, torch.float64] or \
+        (features.dtype == torch.int32 and order == 0), f'input must be a floating tensor but got {features.dtype}'
     assert order in [0, 1, 3], f'order {order} is not supported!'
     if order == 0:
         sampling_ratio = 1  # never average nearest-neighbour samples (reference :72-74)

@@ -263,3 +263,29 @@ def test_batch_crops_around_boxes_and_foreground(aug):
         sz, sy, sx = turns._crop_start({"gt_det": det.to(DEV)}, 0)
         picks.append(0 if sx <= 6 and 11 <= sx + patch[2] else 1)
     assert picks == [0, 1, 0, 1]
+
+
+@pytest.mark.parametrize("dim,size,out", [(3, (40, 48, 56), (40, 48, 56)), (3, (20, 24, 28), (9, 10, 11)),
+                                          (2, (96, 128), (96, 128)), (2, (30, 40), (12, 14))])
+def test_int32_label_maps_are_sampled_as_they_are(dim, size, out):
+    """Order 0 on int32 label maps through the affine engines: the library loads and stores the integers
+    itself (tiled kernel for large outputs, general kernel for small ones) and must pick the very voxels of
+    the float copy that such maps used to be resampled through (the reference's `.float()` ... `.int()`):
+    rotated, shifted and scaled rois that reach past the map, labels from -5 to 2^24 - 1."""
+    import medvision_amd.ops as ops
+    g = wl.gen(77 + dim + out[0])
+    n = 3
+    seg = torch.randint(-5, 40, (n, 2, *size), generator=g, dtype=torch.int32)
+    seg[0, 0].view(-1)[::7] = 2 ** 24 - 1
+    xyz = torch.tensor(size[::-1], dtype=torch.float32)
+    ctr = xyz / 2 + (torch.rand(n, dim, generator=g) * 2 - 1) * 6
+    ext = xyz * (0.7 + torch.rand(n, dim, generator=g) * 0.7)
+    ang = (torch.rand(n, 3 if dim == 3 else 1, generator=g) * 2 - 1) * 0.5
+    rois = torch.cat([torch.arange(n).float().view(n, 1), ctr, ext, ang], 1).to(DEV)
+    fn = ops.affine_3d if dim == 3 else ops.affine_2d
+    got = fn(seg.to(DEV), rois, out, 1.0, 1, True, 0)
+    want = fn(seg.to(DEV).float(), rois, out, 1.0, 1, True, 0).int()
+    assert got.dtype == torch.int32 and torch.equal(got, want)
+    assert int((got != 0).sum()) > got.numel() // 4
+    with pytest.raises((RuntimeError, AssertionError)):
+        fn(seg.to(DEV), rois, out, 1.0, 1, True, 1)    # int32 at order 1
